@@ -1,0 +1,200 @@
+/*
+ * xq.h -- C ABI of libxq_hip.so: the MI355X (gfx950) implementation of xorl's
+ * QLoRA quantized base-linear hot path.
+ *
+ * The reference (togethercomputer/xorl) has no FFI for this path: every
+ * kernel is a Triton function called from Python.  Each entry point below
+ * therefore names the Python function(s) of the reference it replaces
+ * (paths relative to the xorl checkout).  A maintainer binds these with
+ * ctypes; no torch type appears in any signature.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless stated otherwise;
+ *   - `stream` is a hipStream_t passed as void* (0 = the null stream);
+ *   - the library allocates nothing: outputs and workspaces are the caller's;
+ *   - every function validates its arguments on the host and returns
+ *     XQ_OK (0) or a negative error code before launching anything;
+ *     xq_last_error() returns a message for the calling thread's last error;
+ *   - activations are bf16 row-major with an explicit row stride in elements.
+ */
+#ifndef XQ_H
+#define XQ_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define XQ_OK 0
+#define XQ_ERR_ARG (-1)      /* bad argument (shape, alignment, enum, null) */
+#define XQ_ERR_UNSUPPORTED (-2)
+#define XQ_ERR_LAUNCH (-3)   /* hipGetLastError() after a launch was not hipSuccess */
+
+/* weight formats */
+#define XQ_FMT_INT4 0   /* 4-bit offset-binary codes, w = (nib - 8) * scale            */
+#define XQ_FMT_NVFP4 1  /* e2m1 codes, per-16 block scale * fp32 global scale          */
+#define XQ_FMT_FP8 2    /* e4m3fn bytes, fp32 scale per 128x128 block                  */
+
+/* storage layouts of the 4-bit formats (fp8 is symmetric: layout is ignored)
+ *   FLAT: decoded shape [rows, cols]; nibble pairs and scale groups run along
+ *         cols; packed [rows, cols/2], scales [rows, cols/group].  This is the
+ *         dense module's [out_features, in_features] storage.
+ *   GKN : decoded shape [rows, cols]; nibble pairs and scale groups run along
+ *         rows; packed [rows/2, cols], scales [rows/group, cols].  This is the
+ *         expert bank's [in_features, out_features] storage.                 */
+#define XQ_LAYOUT_FLAT 0
+#define XQ_LAYOUT_GKN 1
+
+/* scale element types */
+#define XQ_SCALE_F32 0
+#define XQ_SCALE_BF16 1
+#define XQ_SCALE_E4M3 2
+
+/* element types of outputs / LoRA factors */
+#define XQ_DT_BF16 0
+#define XQ_DT_F32 1
+
+/* A bank of `num_experts` equally shaped quantized matrices (1 for a dense
+ * linear).  Expert e starts at packed + e*packed_bytes, scales + e*scale_bytes
+ * (both derived from the shape), global_scale[e]. */
+typedef struct xq_weight {
+    int32_t format;       /* XQ_FMT_*    */
+    int32_t layout;       /* XQ_LAYOUT_* */
+    int32_t scale_dtype;  /* XQ_SCALE_*  */
+    int32_t group;        /* int4: any even divisor of the grouped dim (128 typical); nvfp4: 16; fp8: 128 */
+    int64_t rows;         /* decoded rows */
+    int64_t cols;         /* decoded cols */
+    int32_t num_experts;
+    int32_t reserved;
+    const void* packed;
+    const void* scales;
+    const float* global_scale; /* nvfp4 only: num_experts floats; else NULL */
+} xq_weight;
+
+/* ---- library ---------------------------------------------------------- */
+const char* xq_version(void);
+const char* xq_last_error(void);
+
+/* ---- decode ------------------------------------------------------------
+ * out[e] = decoded weight of expert e, shape [rows, cols], bf16 or fp32.
+ * Replaces int4_dequantize / int4_dequantize_gkn
+ *   (ops/quantize/int4_quantize.py:113-127, int4_gkn_quantize.py:176-216),
+ * nvfp4_dequantize / nvfp4_dequantize_gkn
+ *   (ops/quantize/nvfp4_quantize.py:157-177, nvfp4_gkn_quantize.py:238-273),
+ * block_fp8_dequantize_gkn (ops/quantize/block_fp8_gkn_quantize.py:157-180;
+ *   XQ_DT_F32 gives that function's fp32 output, XQ_DT_BF16 gives the
+ *   `.to(bf16)` its callers apply, qlora/modules/linear.py:373).
+ * Bit-exact with the reference arithmetic. */
+int xq_decode(const xq_weight* w, void* out, int out_dtype, void* stream);
+
+/* ---- dense QLoRA linear -------------------------------------------------
+ * Replaces QLoRALinear.forward (qlora/modules/linear.py:369-385) and its
+ * autograd backward.  The weight is FLAT [N, K]. */
+
+/* Bytes of scratch the dense entry points need for (M, N, K, r). */
+int64_t xq_linear_workspace_bytes(int64_t M, int64_t N, int64_t K, int r);
+
+/* y[M,N] = x[M,K] . deq(W)^T + bias + s * (x . A^T) . B^T      (bf16 out)
+ *   lora_A [r,K], lora_B [N,r] in lora_dtype (fp32 or bf16), r in {0..64};
+ *   su_out (optional, bf16 [M, r_pad], r_pad = r rounded up to 16) receives
+ *   bf16(s * x . A^T) for reuse by xq_linear_bwd;
+ *   workspace: xq_linear_workspace_bytes(...) bytes, 256-byte aligned. */
+int xq_linear_fwd(const xq_weight* w, const void* x, int64_t ldx, int64_t M,
+                  const void* lora_A, const void* lora_B, int lora_dtype, int r, float scaling,
+                  const void* bias_bf16, void* y, int64_t ldy, void* su_out,
+                  void* workspace, int64_t workspace_bytes, void* stream);
+
+/* dx[M,K] = dy . deq(W) + s * (dy . B) . A   (bf16)
+ * dA[r,K] = s * (dy . B)^T . x               (fp32, overwritten)
+ * dB[N,r] = s * dy^T . (x . A^T)             (fp32, overwritten)
+ *   su: the buffer xq_linear_fwd wrote (or NULL: recomputed from x);
+ *   any of dx / dA / dB may be NULL to skip it. */
+int xq_linear_bwd(const xq_weight* w, const void* x, int64_t ldx, const void* dy, int64_t lddy,
+                  int64_t M, const void* lora_A, const void* lora_B, int lora_dtype, int r,
+                  float scaling, const void* su, void* dx, int64_t lddx, float* dA, float* dB,
+                  void* workspace, int64_t workspace_bytes, void* stream);
+
+/* ---- SwiGLU between gate/up and down ------------------------------------
+ * Replaces fused_silu_and_mul (ops/fused_silu_and_mul.py:22-60 and its
+ * backward): h = bf16(silu_fp32(gate)) * up, two roundings.  With row_w
+ * (fp32 [rows], the routing weight of each expert-ordered row) it is the
+ * routed form of ops/moe/lora.py:639-647, h = bf16(bf16(bf16(silu(g))*u)*w),
+ * and the backward also returns d_row_w[row] = sum_c dh * bf16(bf16(silu(g))*u)
+ * (ops/moe/lora.py:855-917).  row_w / d_row_w may be NULL. */
+int xq_silu_mul_fwd(const void* gate, const void* up, int64_t ld_in, const float* row_w, void* h,
+                    int64_t ld_h, int64_t rows, int64_t cols, void* stream);
+int xq_silu_mul_bwd(const void* gate, const void* up, int64_t ld_in, const void* dh, int64_t ld_dh,
+                    const float* row_w, void* dgate, void* dup, int64_t ld_out, float* d_row_w,
+                    int64_t rows, int64_t cols, void* stream);
+
+/* ---- grouped / routed (MoE experts) --------------------------------------
+ * xq_route_build replaces the dispatch part of _MoeExpertsLoRAFunction.forward
+ * (ops/moe/lora.py:579-583): expert_histogram, stable argsort by expert id,
+ * cumsum.  selected [T*topk] int32 expert ids (row-major [T, topk]).
+ * Outputs: counts [E], offsets [E+1] (exclusive prefix), scatter_index
+ * [T*topk] (row in expert order of routed copy i), tile_offsets [E+1]
+ * (prefix of ceil(count/128), the row-tile schedule of the grouped kernels).
+ * Deterministic and stable.  workspace: xq_route_workspace_bytes() bytes. */
+int64_t xq_route_workspace_bytes(int64_t n_routed, int32_t num_experts);
+int xq_route_build(const int32_t* selected, int64_t n_routed, int32_t num_experts,
+                   int32_t* counts, int32_t* offsets, int32_t* scatter_index,
+                   int32_t* tile_offsets, void* workspace, int64_t workspace_bytes, void* stream);
+
+/* rows_out[scatter_index[i]] = rows_in[i / topk]   (moe_scatter, group_gemm/kernel/moe.py:266-312) */
+int xq_moe_scatter(const void* in, int64_t ld_in, const int32_t* scatter_index, int64_t n_routed,
+                   int32_t topk, int64_t width, void* out, int64_t ld_out, void* stream);
+/* out[t] = sum_j rows[scatter_index[t*topk+j]] (+ rows2[...]), fp32 accumulate
+ * (moe_gather / moe_add_gather, group_gemm/kernel/moe.py:102-141, :178-223) */
+int xq_moe_gather(const void* rows, const void* rows2, int64_t ld_rows, const int32_t* scatter_index,
+                  int64_t n_tokens, int32_t topk, int64_t width, void* out, int64_t ld_out, void* stream);
+/* dst[scatter_index[i]] = float(src[i]) and dst[i] = src[scatter_index[i]]:
+ * the routing-weight permutation of ops/moe/lora.py:644-646 and :857-858. */
+int xq_moe_scatter_scalar(const void* src, int src_dtype, const int32_t* scatter_index, int64_t n,
+                          float* dst, void* stream);
+int xq_moe_gather_scalar(const float* src, const int32_t* scatter_index, int64_t n, void* dst,
+                         int dst_dtype, void* stream);
+
+/* Grouped projection over rows already in expert order:
+ *   for each expert e with rows [offsets[e], offsets[e+1]):
+ *     y[rows] = a[rows] . op(deq(W[e])) + su[rows] . Lr[e]^T
+ * The bank is GKN [E, K_in, N_out]; transpose_w = 0 contracts over the bank's
+ * rows (forward: y = x . W), 1 over its cols (dgrad: dx = dy . W^T).
+ * su bf16 [R, r_pad] (already scaled) and lora_right bf16 [E, n_out, r_pad]
+ * are the low-rank side term (NULL for none).
+ * Replaces group_gemm_same_nk on dequantized banks
+ * (ops/group_gemm/kernel/group_gemm.py:171-256) fused with
+ * dequantize_all_experts (qlora/modules/moe_experts.py:486-498). */
+int xq_grouped_gemm(const xq_weight* w, int transpose_w, const void* a, int64_t lda,
+                    int64_t n_rows, const int32_t* offsets, const int32_t* tile_offsets,
+                    const void* su, const void* lora_right, int r_pad,
+                    void* y, int64_t ldy, void* stream);
+
+/* out[e][i][j] (bf16, zero padded to [rows_out, cols_out]) = in[e][i][j] or
+ * in[e][j][i]: brings fp32/bf16 LoRA factors into the bf16 operand layouts
+ * the kernels above consume (the `.to(compute_dtype)` of ops/moe/lora.py:557-564). */
+int xq_factor_prep(const void* in, int in_dtype, int64_t rows_in, int64_t cols_in, int transpose,
+                   void* out_bf16, int64_t rows_out, int64_t cols_out, int64_t num_experts, void* stream);
+
+/* Grouped low-rank helpers (bf16 in, fp32 accumulate):
+ *   xq_grouped_lora_down: t[rows of e] = bf16(scale * a[rows of e] . F[e]^T),
+ *       F bf16 [E, r_pad, K] (or one shared [r_pad, K]); t is [R, r_pad].
+ *   xq_grouped_lora_wgrad: out[e] = P[rows of e]^T . Q[rows of e], fp32
+ *       [E, p_width, r_out] (or [E, r_out, p_width] with transpose_out); zero
+ *       for empty experts.  With offsets == NULL it is the dense form over all
+ *       n_rows (one output; also the gradient of a factor shared by all
+ *       experts), deterministic, using xq_lora_wgrad_workspace_bytes() scratch.
+ * Replace the small group_gemm_same_nk / group_gemm_same_mn calls of
+ * ops/moe/lora.py:601-660 and :781-960. */
+int xq_grouped_lora_down(const void* a, int64_t lda, int64_t n_rows, const int32_t* offsets,
+                         const int32_t* tile_offsets, int32_t num_experts, const void* F, int shared,
+                         int r_pad, int64_t K, float scale, void* t, void* stream);
+int64_t xq_lora_wgrad_workspace_bytes(int64_t n_rows, int64_t width, int r_pad);
+int xq_grouped_lora_wgrad(const void* P, int64_t ldp, int64_t p_width, const void* Q, int r_pad,
+                          int r_out, int64_t n_rows, const int32_t* offsets, int32_t num_experts,
+                          int transpose_out, float* out, void* workspace, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* XQ_H */

@@ -1,0 +1,112 @@
+"""GPU parity: fused dequant-GEMM + LoRA forward/backward (through the C ABI)
+vs the CPU oracle.  Tolerance: max|got-ref| / max|ref| <= 1e-2 against the
+float64 restatement of the reference recipe (the "fp32-accumulated path")."""
+
+import pytest
+import torch
+
+from oracle import recipe as R
+from tests.util_cases import gen, make_dense_module
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-2
+
+
+def _run(m, x, dy):
+    x = x.clone().requires_grad_(True)
+    y = m(x)
+    y.backward(dy)
+    return y.detach(), x.grad, m.lora_A.grad, m.lora_B.grad
+
+
+@pytest.mark.parametrize("fmt", ["block_fp8", "int4", "nvfp4"])
+@pytest.mark.parametrize("M,K,N,r", [(200, 256, 384, 16), (1, 128, 64, 8), (129, 384, 320, 24), (512, 1024, 512, 64)])
+def test_dense_fwd_bwd_vs_oracle(hip_device, fmt, M, K, N, r):
+    m, w_ref = make_dense_module(fmt, N, K, r, 2 * r, seed=M + K, device=hip_device)
+    x = gen((M, K), 1.0, 11, torch.bfloat16)
+    dy = gen((M, N), 1.0, 12, torch.bfloat16)
+    y, dx, dA, dB = _run(m, x.to(hip_device), dy.to(hip_device))
+    ex = R.linear_fwd_bwd_exact(x, w_ref, m.lora_A.detach().cpu(), m.lora_B.detach().cpu(), m.scaling, dy)
+    assert y.dtype == torch.bfloat16 and dx.dtype == torch.bfloat16
+    assert dA.dtype == torch.float32 and dA.shape == (r, K) and dB.shape == (N, r)
+    for name, got, ref in (("y", y, ex["y"]), ("dx", dx, ex["dx"]), ("dA", dA, ex["dA"]), ("dB", dB, ex["dB"])):
+        err = R.max_rel_err(got.cpu(), ref)
+        assert err <= TOL, f"{fmt} {name}: {err}"
+
+
+def test_config0_int4_full_size(hip_device):
+    """BASELINE config 0: X [512,4096], W [4096,4096] int4 g128 absmax/7 bf16 scales, r=16, alpha=32."""
+    M, K, N, r = 512, 4096, 4096, 16
+    m, w_ref = make_dense_module("int4", N, K, r, 32, seed=0, device=hip_device)
+    x = gen((M, K), 1.0, 1, torch.bfloat16)
+    dy = gen((M, N), 1.0, 2, torch.bfloat16)
+    y, dx, dA, dB = _run(m, x.to(hip_device), dy.to(hip_device))
+    ex = R.linear_fwd_bwd_exact(x, w_ref, m.lora_A.detach().cpu(), m.lora_B.detach().cpu(), 2.0, dy)
+    for name, got, ref in (("y", y, ex["y"]), ("dx", dx, ex["dx"]), ("dA", dA, ex["dA"]), ("dB", dB, ex["dB"])):
+        assert R.max_rel_err(got.cpu(), ref) <= TOL, name
+    # the module's own decode is bit-exact with the oracle
+    assert torch.equal(m._dequantize_weight().cpu(), w_ref)
+
+
+def test_invariants(hip_device):
+    m, w_ref = make_dense_module("block_fp8", 384, 256, 16, 32, seed=5, device=hip_device, bias=True)
+    x = gen((3, 7, 256), 1.0, 13, torch.bfloat16).to(hip_device)        # leading dims are kept
+    with torch.no_grad():
+        y = m(x)
+        assert y.shape == (3, 7, 384)
+        b_saved = m.lora_B.clone()
+        m.lora_B.zero_()
+        y0 = m(x)
+        m.lora_B.copy_(b_saved)
+    base = R.linear_fwd_bwd_exact(x.cpu(), w_ref, m.lora_A.detach().cpu(), torch.zeros(384, 16), 2.0,
+                                  bias=m.bias.detach().cpu())["y"]
+    assert R.max_rel_err(y0.cpu(), base) <= TOL          # lora_B = 0 => base only (+ bias)
+    assert not torch.equal(y, y0)
+    # linearity in x of the whole op (size-independent property)
+    with torch.no_grad():
+        m.bias.zero_()
+        a, b = m(x), m(2 * x)
+    assert R.max_rel_err(b.cpu().float(), 2 * a.cpu().float()) <= TOL
+    # active rank slice (set_runtime_lora_config)
+    m.set_runtime_lora_config(8, 16)
+    with torch.no_grad():
+        y8 = m(x)
+    ex8 = R.linear_fwd_bwd_exact(x.cpu(), w_ref, m.lora_A.detach().cpu()[:8], m.lora_B.detach().cpu()[:, :8], 2.0)["y"]
+    assert R.max_rel_err(y8.cpu(), ex8) <= TOL
+    with pytest.raises(ValueError):
+        m.set_runtime_lora_config(0, 1)
+
+
+def test_errors(hip_device):
+    from xorl_amd.qlora import BlockFP8QLoRALinear, QLoRALinear
+
+    with pytest.raises(TypeError):
+        QLoRALinear(64, 64)
+    m = BlockFP8QLoRALinear(200, 64, device=hip_device)       # K not a multiple of 64
+    with pytest.raises(ValueError):
+        m(torch.zeros(2, 200, dtype=torch.bfloat16, device=hip_device))
+    m2 = BlockFP8QLoRALinear(128, 64, device=hip_device)
+    with pytest.raises(ValueError):
+        m2(torch.zeros(2, 128, dtype=torch.float32, device=hip_device))   # activations must be bf16
+    m2.packed_weight_f32.data = m2.packed_weight_f32.data.to(torch.bfloat16)
+    with pytest.raises(RuntimeError):
+        m2(torch.zeros(2, 128, dtype=torch.bfloat16, device=hip_device))
+
+
+def test_silu_and_mul(hip_device):
+    from xorl_amd.functional import silu_and_mul
+
+    g = (gen((300, 512), 2.0, 20)).to(torch.bfloat16)
+    u = gen((300, 512), 1.0, 21, torch.bfloat16)
+    dh = gen((300, 512), 1.0, 22, torch.bfloat16)
+    gd, ud = g.to(hip_device).requires_grad_(True), u.to(hip_device).requires_grad_(True)
+    h = silu_and_mul(gd, ud)
+    h.backward(dh.to(hip_device))
+    ref = R.silu_and_mul_recipe(g, u)
+    # two-rounding recipe: identical up to 1 bf16 ulp where expf differs in the last bit
+    assert R.max_rel_err(h.cpu(), ref) <= 2 ** -7
+    assert (h.cpu() == ref).float().mean() > 0.99
+    g64, u64 = g.double().requires_grad_(True), u.double().requires_grad_(True)
+    (torch.nn.functional.silu(g64) * u64).backward(dh.double())
+    assert R.max_rel_err(gd.grad.cpu(), g64.grad) <= TOL
+    assert R.max_rel_err(ud.grad.cpu(), u64.grad) <= TOL

@@ -1,0 +1,52 @@
+"""Host logic: the package's torch quantizers emit the same bytes as the C oracle (no GPU)."""
+
+import numpy as np
+import torch
+
+from oracle import cdecode as C
+from xorl_amd import quantize as Q
+
+
+def _w(shape, seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(*shape, generator=g) * 0.02
+
+
+def test_int4_quantizers_match_oracle():
+    w = _w((32, 256), 0)
+    p, s = Q.int4_quantize(w, 128)
+    pc, sc = C.int4_quantize_flat(w.numpy(), 128)
+    assert np.array_equal(p.numpy(), pc) and np.array_equal(s.numpy(), sc)
+    pk, sk = Q.int4_quantize_gkn(w.t().contiguous(), 128)
+    pkc, skc = C.int4_quantize_gkn(w.t().contiguous().numpy(), 128)
+    assert np.array_equal(pk.numpy(), pkc) and np.array_equal(sk.numpy(), skc)
+    ps, ss = Q.int4_quantize_sym(w, 128)
+    psc, ssc = C.int4_quantize_sym_flat(w.numpy(), 128)
+    assert np.array_equal(ps.numpy(), psc)
+    assert np.array_equal(ss.view(torch.int16).numpy().view(np.uint16), ssc)
+
+
+def test_nvfp4_quantizers_match_oracle():
+    w = _w((32, 256), 1)
+    p, bs, g = Q.nvfp4_quantize(w)
+    pc, bsc, gc = C.nvfp4_quantize_flat(w.numpy())
+    assert np.array_equal(p.numpy().reshape(32, 128), pc)
+    assert np.array_equal(bs.view(torch.uint8).numpy().reshape(32, 16), bsc)
+    assert g.item() == gc
+    pk, bk, gk = Q.nvfp4_quantize_gkn(w.t().contiguous())
+    pkc, bkc, gkc = C.nvfp4_quantize_gkn(w.t().contiguous().numpy())
+    assert np.array_equal(pk.numpy(), pkc) and np.array_equal(bk.view(torch.uint8).numpy(), bkc) and gk.item() == gkc
+    # EMA override of the global amax (nvfp4_quantize.py:139-141)
+    p2, bs2, g2 = Q.nvfp4_quantize(w, global_amax=torch.tensor([0.2]))
+    pc2, bsc2, gc2 = C.nvfp4_quantize_flat(w.numpy(), global_amax=0.2)
+    assert np.array_equal(p2.numpy().reshape(32, 128), pc2) and g2.item() == gc2
+    assert np.array_equal(bs2.view(torch.uint8).numpy().reshape(32, 16), bsc2)
+
+
+def test_block_fp8_quantizer_matches_oracle():
+    for shape, seed in (((256, 384), 2), ((200, 300), 3)):
+        w = _w(shape, seed)
+        y, s = Q.block_fp8_quantize_gkn(w)
+        yc, sc = C.fp8_quantize(w.numpy())
+        assert np.array_equal(y.view(torch.uint8).numpy(), yc)
+        assert np.array_equal(s.numpy(), sc)

@@ -1,0 +1,60 @@
+"""Seeded synthetic QLoRA cases shared by the GPU tests, smoke() and bench.py.
+
+Builds quantized weights with the package's torch quantizers (host logic,
+checked byte-for-byte against the oracle in tests/test_quantizers_cpu.py) and
+decodes them with the CPU oracle for the expected values.
+"""
+
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+from oracle import cdecode as C
+from oracle import decode_np as NP
+
+
+def gen(shape, std, seed, dtype=torch.float32):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * std).to(dtype)
+
+
+def bits_to_bf16(bits: np.ndarray) -> torch.Tensor:
+    return torch.from_numpy(bits.view(np.int16).copy()).view(torch.bfloat16)
+
+
+def make_dense_module(fmt: str, N: int, K: int, r: int, alpha: int, seed: int, device, bias=False):
+    """Returns (module on `device`, decoded weight bf16 on CPU from the oracle)."""
+    from xorl_amd.qlora import QLoRALinear
+
+    lin = torch.nn.Linear(K, N, bias=bias)
+    with torch.no_grad():
+        lin.weight.copy_(gen((N, K), 0.02, seed))
+        if bias:
+            lin.bias.copy_(gen((N,), 0.1, seed + 7))
+    m = QLoRALinear.from_module(lin, r=r, lora_alpha=alpha, quant_format=fmt)
+    with torch.no_grad():
+        m.lora_A.copy_(gen((r, K), 0.02, seed + 1))
+        m.lora_B.copy_(gen((N, r), 0.02, seed + 2))
+    w_ref = oracle_decode_dense(m)
+    return m.to(device), w_ref
+
+
+def oracle_decode_dense(m) -> torch.Tensor:
+    """Decode a (CPU) module's packed state with the numpy oracle -> bf16 [N, K]."""
+    N, K = m.out_features, m.in_features
+    packed = m.packed_weight_f32.detach().cpu().contiguous().view(torch.uint8).numpy()
+    if m.quant_format == "block_fp8":
+        s = m.weight_block_scales.cpu().contiguous().view(torch.float32).numpy()
+        return bits_to_bf16(NP.fp8_decode(packed.reshape(N, K), s, N, K)[1])
+    if m.quant_format == "nvfp4":
+        sdt = m._scale_dtypes["weight_block_scales"]
+        sb = m.weight_block_scales.cpu().contiguous()
+        s = C.e4m3_scales_to_f32(sb.numpy()) if sdt == torch.float8_e4m3fn else sb.view(torch.float32).numpy()
+        g = m.weight_global_scale.cpu().contiguous().view(torch.float32).item()
+        return bits_to_bf16(NP.nvfp4_decode_flat(packed, s.reshape(N, K // 16), g, N, K))
+    if m.quant_format == "int4":
+        sdt = m._scale_dtypes["weight_scales"]
+        s = m.weight_scales.cpu().contiguous().view(sdt).float().numpy()
+        return bits_to_bf16(NP.int4_decode_flat(packed, s, N, K, m.quant_group_size))
+    raise ValueError(m.quant_format)

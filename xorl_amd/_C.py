@@ -1,0 +1,168 @@
+"""ctypes binding of libxq_hip.so (the C ABI declared in include/xq.h).
+
+There is no CPU fallback: if the library is missing, or a tensor is not on a
+HIP device, the call raises.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+from typing import Optional
+
+import torch
+
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libxq_hip.so")
+
+XQ_FMT_INT4, XQ_FMT_NVFP4, XQ_FMT_FP8 = 0, 1, 2
+XQ_LAYOUT_FLAT, XQ_LAYOUT_GKN = 0, 1
+XQ_SCALE_F32, XQ_SCALE_BF16, XQ_SCALE_E4M3 = 0, 1, 2
+XQ_DT_BF16, XQ_DT_F32 = 0, 1
+
+FORMATS = {"int4": XQ_FMT_INT4, "nvfp4": XQ_FMT_NVFP4, "block_fp8": XQ_FMT_FP8}
+
+
+class XqWeight(ctypes.Structure):
+    _fields_ = [
+        ("format", ctypes.c_int32),
+        ("layout", ctypes.c_int32),
+        ("scale_dtype", ctypes.c_int32),
+        ("group", ctypes.c_int32),
+        ("rows", ctypes.c_int64),
+        ("cols", ctypes.c_int64),
+        ("num_experts", ctypes.c_int32),
+        ("reserved", ctypes.c_int32),
+        ("packed", ctypes.c_void_p),
+        ("scales", ctypes.c_void_p),
+        ("global_scale", ctypes.c_void_p),
+    ]
+
+
+class XqError(ValueError):
+    """Argument error reported by the library before any launch."""
+
+
+_lib: Optional[ctypes.CDLL] = None
+
+_P, _I64, _I32, _F = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int32, ctypes.c_float
+_W = ctypes.POINTER(XqWeight)
+
+_INT = ctypes.c_int
+_SIGNATURES = {
+    "xq_decode": (_INT, [_W, _P, _INT, _P]),
+    "xq_linear_workspace_bytes": (_I64, [_I64, _I64, _I64, _INT]),
+    # w, x, ldx, M, A, B, lora_dtype, r, scaling, bias, y, ldy, su_out, ws, ws_bytes, stream
+    "xq_linear_fwd": (_INT, [_W, _P, _I64, _I64, _P, _P, _INT, _INT, _F, _P, _P, _I64, _P, _P, _I64, _P]),
+    # w, x, ldx, dy, lddy, M, A, B, lora_dtype, r, scaling, su, dx, lddx, dA, dB, ws, ws_bytes, stream
+    "xq_linear_bwd": (_INT, [_W, _P, _I64, _P, _I64, _I64, _P, _P, _INT, _INT, _F, _P, _P, _I64, _P, _P, _P, _I64,
+                             _P]),
+    # gate, up, ld_in, row_w, h, ld_h, rows, cols, stream
+    "xq_silu_mul_fwd": (_INT, [_P, _P, _I64, _P, _P, _I64, _I64, _I64, _P]),
+    # gate, up, ld_in, dh, ld_dh, row_w, dgate, dup, ld_out, d_row_w, rows, cols, stream
+    "xq_silu_mul_bwd": (_INT, [_P, _P, _I64, _P, _I64, _P, _P, _P, _I64, _P, _I64, _I64, _P]),
+    "xq_route_workspace_bytes": (_I64, [_I64, _I32]),
+    # selected, n_routed, E, counts, offsets, scatter_index, tile_offsets, ws, ws_bytes, stream
+    "xq_route_build": (_INT, [_P, _I64, _I32, _P, _P, _P, _P, _P, _I64, _P]),
+    "xq_moe_scatter": (_INT, [_P, _I64, _P, _I64, _I32, _I64, _P, _I64, _P]),
+    "xq_moe_gather": (_INT, [_P, _P, _I64, _P, _I64, _I32, _I64, _P, _I64, _P]),
+    "xq_moe_scatter_scalar": (_INT, [_P, _INT, _P, _I64, _P, _P]),
+    "xq_moe_gather_scalar": (_INT, [_P, _P, _I64, _P, _INT, _P]),
+    # w, transpose_w, a, lda, n_rows, offsets, tile_offsets, su, lora_right, r_pad, y, ldy, stream
+    "xq_grouped_gemm": (_INT, [_W, _INT, _P, _I64, _I64, _P, _P, _P, _P, _INT, _P, _I64, _P]),
+    # in, in_dtype, rows_in, cols_in, transpose, out, rows_out, cols_out, E, stream
+    "xq_factor_prep": (_INT, [_P, _INT, _I64, _I64, _INT, _P, _I64, _I64, _I64, _P]),
+    # a, lda, n_rows, offsets, tile_offsets, E, F, shared, r_pad, K, scale, t, stream
+    "xq_grouped_lora_down": (_INT, [_P, _I64, _I64, _P, _P, _I32, _P, _INT, _INT, _I64, _F, _P, _P]),
+    "xq_lora_wgrad_workspace_bytes": (_I64, [_I64, _I64, _INT]),
+    # P, ldp, p_width, Q, r_pad, r_out, n_rows, offsets, E, transpose_out, out, ws, stream
+    "xq_grouped_lora_wgrad": (_INT, [_P, _I64, _I64, _P, _INT, _INT, _I64, _P, _I32, _INT, _P, _P, _P]),
+}
+
+EXPORTS = ("xq_version", "xq_last_error") + tuple(_SIGNATURES)
+
+
+def lib() -> ctypes.CDLL:
+    """Load libxq_hip.so; raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with `python -m xorl_amd.csrc.build` "
+                "(there is no CPU or eager fallback for the QLoRA kernels)"
+            )
+        L = ctypes.CDLL(LIB_PATH)
+        L.xq_version.restype = ctypes.c_char_p
+        L.xq_last_error.restype = ctypes.c_char_p
+        for name, (res, args) in _SIGNATURES.items():
+            fn = getattr(L, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = L
+    return _lib
+
+
+def check(rc: int) -> None:
+    if rc != 0:
+        msg = lib().xq_last_error().decode()
+        if rc == -3:
+            raise RuntimeError(msg)
+        raise XqError(msg)
+
+
+def require_hip(*tensors: Optional[torch.Tensor]) -> None:
+    for t in tensors:
+        if t is not None and t.device.type != "cuda":
+            raise RuntimeError(
+                f"xorl_amd kernels run on a HIP device only; got a tensor on {t.device} "
+                "(there is no CPU fallback)"
+            )
+
+
+def ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def stream_ptr(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+_SCALE_DT = {torch.float32: XQ_SCALE_F32, torch.bfloat16: XQ_SCALE_BF16, torch.float8_e4m3fn: XQ_SCALE_E4M3}
+
+
+def make_weight(
+    fmt: str,
+    layout: int,
+    packed: torch.Tensor,
+    scales: torch.Tensor,
+    scale_dtype: torch.dtype,
+    rows: int,
+    cols: int,
+    group: int,
+    global_scale: Optional[torch.Tensor] = None,
+    num_experts: int = 1,
+) -> XqWeight:
+    """Describe a (bank of) quantized matrices.  `packed`/`scales` may be any
+    dtype view of the right bytes (uint8 buffers, fp32-packed parameters);
+    `scale_dtype` is the true element type of the scales."""
+    require_hip(packed, scales, global_scale)
+    if not packed.is_contiguous() or not scales.is_contiguous():
+        raise XqError("packed weights and scales must be contiguous")
+    w = XqWeight()
+    w.format = FORMATS[fmt]
+    w.layout = layout
+    w.scale_dtype = _SCALE_DT[scale_dtype]
+    w.group = group
+    w.rows, w.cols = rows, cols
+    w.num_experts = num_experts
+    w.packed = packed.data_ptr()
+    w.scales = scales.data_ptr()
+    w.global_scale = None if global_scale is None else global_scale.data_ptr()
+    nbytes = rows * cols if fmt == "block_fp8" else rows * cols // 2
+    if packed.numel() * packed.element_size() != nbytes * num_experts:
+        raise XqError(
+            f"packed buffer holds {packed.numel() * packed.element_size()} bytes, "
+            f"expected {nbytes * num_experts} for {num_experts} x [{rows}, {cols}] {fmt}"
+        )
+    return w

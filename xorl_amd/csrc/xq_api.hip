@@ -1,0 +1,61 @@
+// Library-level entry points: version, per-thread error text, weight validation.
+#include <stdarg.h>
+#include <stdio.h>
+
+#include "xq_common.h"
+
+static thread_local char g_err[512] = "";
+
+void xq_set_error(const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+}
+
+extern "C" const char* xq_version(void) { return "xq-hip 0.1 (gfx950)"; }
+extern "C" const char* xq_last_error(void) { return g_err; }
+
+int64_t xq_packed_bytes_per_expert(const xq_weight* w) {
+    int64_t n = w->rows * w->cols;
+    return w->format == XQ_FMT_FP8 ? n : n / 2;
+}
+
+static int scale_elem_bytes(int dt) { return dt == XQ_SCALE_F32 ? 4 : (dt == XQ_SCALE_BF16 ? 2 : 1); }
+
+int64_t xq_scale_bytes_per_expert(const xq_weight* w) {
+    if (w->format == XQ_FMT_FP8) return xq_cdiv(w->rows, 128) * xq_cdiv(w->cols, 128) * 4;
+    return (w->rows * w->cols / w->group) * scale_elem_bytes(w->scale_dtype);
+}
+
+int xq_validate_weight(const xq_weight* w, const char* who) {
+    XQ_REQUIRE(w != nullptr, "%s: weight descriptor is NULL", who);
+    XQ_REQUIRE(w->format >= XQ_FMT_INT4 && w->format <= XQ_FMT_FP8, "%s: unknown format %d", who, w->format);
+    XQ_REQUIRE(w->layout == XQ_LAYOUT_FLAT || w->layout == XQ_LAYOUT_GKN, "%s: unknown layout %d", who, w->layout);
+    XQ_REQUIRE(w->rows >= 0 && w->cols >= 0 && w->num_experts >= 1, "%s: bad shape [%d x %lld x %lld]", who,
+               w->num_experts, (long long)w->rows, (long long)w->cols);
+    XQ_REQUIRE(w->rows < (1ll << 31) && w->cols < (1ll << 31), "%s: dimension exceeds 2^31", who);
+    bool empty = w->rows == 0 || w->cols == 0;
+    XQ_REQUIRE(empty || (w->packed && w->scales), "%s: packed/scales pointer is NULL", who);
+    if (w->format == XQ_FMT_FP8) {
+        XQ_REQUIRE(w->group == 128, "%s: block_fp8 block size must be 128, got %d", who, w->group);
+        XQ_REQUIRE(w->scale_dtype == XQ_SCALE_F32, "%s: block_fp8 scales must be fp32", who);
+        XQ_REQUIRE(empty || xq_aligned(w->scales, 4), "%s: scales not 4-byte aligned", who);
+    } else {
+        XQ_REQUIRE(w->group >= 2 && w->group % 2 == 0, "%s: group size must be even, got %d", who, w->group);
+        int64_t gdim = w->layout == XQ_LAYOUT_FLAT ? w->cols : w->rows;
+        XQ_REQUIRE(gdim % w->group == 0, "%s: grouped dimension %lld not divisible by group %d", who, (long long)gdim,
+                   w->group);
+        XQ_REQUIRE(w->scale_dtype >= XQ_SCALE_F32 && w->scale_dtype <= XQ_SCALE_E4M3, "%s: bad scale dtype %d", who,
+                   w->scale_dtype);
+        if (w->format == XQ_FMT_NVFP4) {
+            XQ_REQUIRE(w->group == 16, "%s: nvfp4 block size must be 16, got %d", who, w->group);
+            XQ_REQUIRE(w->global_scale != nullptr, "%s: nvfp4 needs global_scale", who);
+            XQ_REQUIRE(w->scale_dtype != XQ_SCALE_BF16, "%s: nvfp4 block scales are e4m3 or fp32", who);
+        } else {
+            XQ_REQUIRE(w->scale_dtype != XQ_SCALE_E4M3, "%s: int4 scales are fp32 or bf16", who);
+        }
+        XQ_REQUIRE(empty || xq_aligned(w->scales, scale_elem_bytes(w->scale_dtype)), "%s: scales misaligned", who);
+    }
+    return XQ_OK;
+}

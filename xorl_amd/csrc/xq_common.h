@@ -1,0 +1,90 @@
+// Shared device/host helpers for libxq_hip.so (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/xq.h"
+
+// ---------------------------------------------------------------- host side
+void xq_set_error(const char* fmt, ...);
+
+#define XQ_REQUIRE(cond, ...)            \
+    do {                                 \
+        if (!(cond)) {                   \
+            xq_set_error(__VA_ARGS__);   \
+            return XQ_ERR_ARG;           \
+        }                                \
+    } while (0)
+
+#define XQ_CHECK_LAUNCH(name)                                              \
+    do {                                                                   \
+        hipError_t e__ = hipGetLastError();                                \
+        if (e__ != hipSuccess) {                                           \
+            xq_set_error("%s: launch failed: %s", name, hipGetErrorString(e__)); \
+            return XQ_ERR_LAUNCH;                                          \
+        }                                                                  \
+    } while (0)
+
+int xq_validate_weight(const xq_weight* w, const char* who);
+int64_t xq_packed_bytes_per_expert(const xq_weight* w);
+int64_t xq_scale_bytes_per_expert(const xq_weight* w);
+
+static inline int64_t xq_cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
+static inline bool xq_aligned(const void* p, size_t a) { return ((uintptr_t)p % a) == 0; }
+
+// ---------------------------------------------------------------- vector types
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+
+typedef uint16_t bf16_t;  // raw bf16 bit pattern in memory
+
+// ---------------------------------------------------------------- scalar codecs
+// fp32 -> bf16 bits, round to nearest even (v_cvt_pk_bf16_f32 on gfx950).
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+    bf16x2 v;
+    v[0] = (__bf16)lo;
+    v[1] = (__bf16)hi;
+    return __builtin_bit_cast(uint32_t, v);
+}
+__device__ __forceinline__ bf16_t to_bf16(float f) {
+    __bf16 b = (__bf16)f;
+    return __builtin_bit_cast(bf16_t, b);
+}
+__device__ __forceinline__ float bf16_to_f32(bf16_t h) { return __uint_as_float((uint32_t)h << 16); }
+
+// e4m3fn (OCP) byte pair -> two fp32: v_cvt_pk_f32_fp8.  hi selects the upper
+// 16 bits of the dword.
+__device__ __forceinline__ f32x2 e4m3x2_to_f32(uint32_t word, bool hi) {
+    return hi ? __builtin_amdgcn_cvt_pk_f32_fp8(word, true) : __builtin_amdgcn_cvt_pk_f32_fp8(word, false);
+}
+__device__ __forceinline__ float e4m3_to_f32(uint8_t b) { return __builtin_amdgcn_cvt_pk_f32_fp8((uint32_t)b, false)[0]; }
+
+// e2m1 nibble -> fp32 by bit construction: exponent field c>>1, mantissa bit
+// c&1, exponent 0 is the subnormal {0, 0.5}; bit 3 is the sign.
+__device__ __forceinline__ float e2m1_to_f32(uint32_t nib) {
+    uint32_t c = nib & 7u, e = c >> 1, m = c & 1u;
+    uint32_t bits = e ? (((e + 126u) << 23) | (m << 22)) : m * 0x3f000000u;
+    return __uint_as_float(bits | ((nib & 8u) << 28));
+}
+
+__device__ __forceinline__ float load_scale(const void* p, int64_t idx, int dtype) {
+    if (dtype == XQ_SCALE_F32) return ((const float*)p)[idx];
+    if (dtype == XQ_SCALE_BF16) return bf16_to_f32(((const bf16_t*)p)[idx]);
+    return e4m3_to_f32(((const uint8_t*)p)[idx]);
+}
+
+// int4: w = bf16(fl(fl(nib - 8) * s)), as the reference computes it (the
+// subtraction is exact; sign of zero follows the multiply).  m8s is unused
+// here and kept for the fused form fma(nib, s, -8s), which differs only in
+// the sign of a zero result.
+__device__ __forceinline__ float int4_val(uint32_t nib, float s, float m8s) {
+    (void)m8s;
+    return ((float)nib - 8.0f) * s;
+}

@@ -1,0 +1,216 @@
+// Host entry points of the fused dequant-GEMM + LoRA path (dense and grouped).
+#include "xq_gemm_tile.h"
+#include "xq_lora.h"
+
+namespace xq {
+
+template <int FMT, int LAYOUT>
+static void launch_tile_cc(const TileArgs& g, bool contract_cols, dim3 grid, hipStream_t s) {
+    if (contract_cols) gemm_tile_kernel<FMT, LAYOUT, true><<<grid, 256, 0, s>>>(g);
+    else gemm_tile_kernel<FMT, LAYOUT, false><<<grid, 256, 0, s>>>(g);
+}
+
+// C[rows, Nout] = A . op(deq(W)) (+ su . Lr^T) (+ bias); see xq_gemm_tile.h
+int launch_tile_gemm(const xq_weight* w, bool contract_cols, const bf16_t* A, int64_t lda, int64_t n_rows,
+                     const int32_t* offsets, const int32_t* tile_offsets, const bf16_t* su, const bf16_t* lora_right,
+                     int r_pad, const bf16_t* bias, bf16_t* C, int64_t ldc, hipStream_t stream, const char* who) {
+    TileArgs g;
+    g.A = A; g.lda = lda; g.C = C; g.ldc = ldc;
+    g.packed = (const uint8_t*)w->packed;
+    g.scales = (const uint8_t*)w->scales;
+    g.global_scale = w->global_scale;
+    g.packed_stride = xq_packed_bytes_per_expert(w);
+    g.scale_stride = xq_scale_bytes_per_expert(w);
+    g.wrows = (int32_t)w->rows; g.wcols = (int32_t)w->cols;
+    g.group = w->group; g.scale_dtype = w->scale_dtype;
+    g.Kc = contract_cols ? g.wcols : g.wrows;
+    g.Nout = contract_cols ? g.wrows : g.wcols;
+    g.n_rows = n_rows; g.offsets = offsets; g.tile_offsets = tile_offsets; g.num_experts = w->num_experts;
+    g.su = su; g.lora_right = lora_right; g.r_pad = (su && lora_right) ? r_pad : 0;
+    g.bias = bias;
+    XQ_REQUIRE(g.Kc % BK == 0, "%s: contraction length %d must be a multiple of %d", who, g.Kc, BK);
+    XQ_REQUIRE(g.Nout % 16 == 0, "%s: output width %d must be a multiple of 16", who, g.Nout);
+    XQ_REQUIRE(lda % 8 == 0 && xq_aligned(A, 16), "%s: activation rows must be 16-byte aligned", who);
+    XQ_REQUIRE(xq_aligned(w->packed, 16) && g.packed_stride % 16 == 0, "%s: packed weight must be 16-byte aligned", who);
+    XQ_REQUIRE(g.r_pad == 0 || (g.r_pad % 16 == 0 && g.r_pad <= 64 && xq_aligned(su, 16) && xq_aligned(lora_right, 16)),
+               "%s: bad low-rank side term (r_pad %d)", who, g.r_pad);
+    if (w->format != XQ_FMT_FP8 && w->layout == XQ_LAYOUT_GKN)
+        XQ_REQUIRE(w->rows % 2 == 0, "%s: GKN 4-bit storage needs an even row count", who);
+    if (n_rows == 0) return XQ_OK;
+    unsigned mt = (unsigned)(xq_cdiv(n_rows, BM) + (offsets ? w->num_experts : 0));
+    dim3 grid(mt, (unsigned)xq_cdiv(g.Nout, BN));
+    if (w->format == XQ_FMT_FP8) launch_tile_cc<XQ_FMT_FP8, XQ_LAYOUT_FLAT>(g, contract_cols, grid, stream);
+    else if (w->format == XQ_FMT_INT4 && w->layout == XQ_LAYOUT_FLAT) launch_tile_cc<XQ_FMT_INT4, XQ_LAYOUT_FLAT>(g, contract_cols, grid, stream);
+    else if (w->format == XQ_FMT_INT4) launch_tile_cc<XQ_FMT_INT4, XQ_LAYOUT_GKN>(g, contract_cols, grid, stream);
+    else if (w->layout == XQ_LAYOUT_FLAT) launch_tile_cc<XQ_FMT_NVFP4, XQ_LAYOUT_FLAT>(g, contract_cols, grid, stream);
+    else launch_tile_cc<XQ_FMT_NVFP4, XQ_LAYOUT_GKN>(g, contract_cols, grid, stream);
+    XQ_CHECK_LAUNCH(who);
+    return XQ_OK;
+}
+
+static inline int64_t align256(int64_t b) { return (b + 255) & ~(int64_t)255; }
+static inline int r_pad_of(int r) { return r <= 0 ? 0 : ((r + 15) / 16) * 16; }
+
+struct Carver {
+    uint8_t* base;
+    int64_t used, cap;
+    void* take(int64_t bytes) {
+        void* p = base ? base + used : nullptr;
+        used += align256(bytes);
+        return p;
+    }
+};
+
+}  // namespace xq
+
+using namespace xq;
+
+extern "C" int64_t xq_linear_workspace_bytes(int64_t M, int64_t N, int64_t K, int r) {
+    int rp = r_pad_of(r);
+    if (rp == 0) return 256;
+    int64_t fwd = align256(rp * K * 2) + align256(N * rp * 2) + align256(M * rp * 2);
+    int64_t tnp = tn_partial_bytes(M, N, rp);
+    int64_t tnk = tn_partial_bytes(M, K, rp);
+    int64_t bwd = align256(rp * N * 2) + align256(K * rp * 2) + align256(rp * K * 2) + 2 * align256(M * rp * 2) +
+                  align256(tnp > tnk ? tnp : tnk);
+    return (fwd > bwd ? fwd : bwd) + 256;
+}
+
+static int check_dense(const xq_weight* w, const char* who) {
+    int rc = xq_validate_weight(w, who);
+    if (rc) return rc;
+    XQ_REQUIRE(w->num_experts == 1, "%s: dense entry point takes a single matrix", who);
+    XQ_REQUIRE(w->format == XQ_FMT_FP8 || w->layout == XQ_LAYOUT_FLAT, "%s: dense weights are FLAT [N, K]", who);
+    return XQ_OK;
+}
+
+extern "C" int xq_linear_fwd(const xq_weight* w, const void* x, int64_t ldx, int64_t M, const void* lora_A,
+                             const void* lora_B, int lora_dtype, int r, float scaling, const void* bias_bf16, void* y,
+                             int64_t ldy, void* su_out, void* workspace, int64_t workspace_bytes, void* stream_) {
+    int rc = check_dense(w, "xq_linear_fwd");
+    if (rc) return rc;
+    const int64_t N = w->rows, K = w->cols;
+    XQ_REQUIRE(M >= 0 && x && y, "xq_linear_fwd: NULL activation pointer");
+    XQ_REQUIRE(r >= 0 && r <= 64, "xq_linear_fwd: LoRA rank %d out of range [0, 64]", r);
+    XQ_REQUIRE(r == 0 || (lora_A && lora_B), "xq_linear_fwd: LoRA factors are NULL");
+    XQ_REQUIRE(lora_dtype == XQ_DT_F32 || lora_dtype == XQ_DT_BF16, "xq_linear_fwd: bad lora_dtype");
+    XQ_REQUIRE(ldy % 8 == 0 && xq_aligned(y, 16), "xq_linear_fwd: y rows must be 16-byte aligned");
+    hipStream_t stream = (hipStream_t)stream_;
+    if (M == 0) return XQ_OK;
+    const int rp = r_pad_of(r);
+    bf16_t *A_bf = nullptr, *Bl = nullptr, *su = nullptr;
+    if (rp) {
+        XQ_REQUIRE(workspace && xq_aligned(workspace, 256) && workspace_bytes >= xq_linear_workspace_bytes(M, N, K, r),
+                   "xq_linear_fwd: workspace missing, misaligned or smaller than xq_linear_workspace_bytes()");
+        Carver cv{(uint8_t*)workspace, 0, workspace_bytes};
+        A_bf = (bf16_t*)cv.take(rp * K * 2);
+        Bl = (bf16_t*)cv.take(N * rp * 2);
+        su = su_out ? (bf16_t*)su_out : (bf16_t*)cv.take(M * rp * 2);
+        if ((rc = launch_factor_prep(lora_A, lora_dtype, r, K, false, A_bf, rp, K, 1, stream))) return rc;
+        if ((rc = launch_factor_prep(lora_B, lora_dtype, N, r, false, Bl, N, rp, 1, stream))) return rc;
+        if ((rc = launch_small_nt((const bf16_t*)x, ldx, M, K, A_bf, rp, scaling, su, nullptr, nullptr, 1, true, stream))) return rc;
+    }
+    return launch_tile_gemm(w, true, (const bf16_t*)x, ldx, M, nullptr, nullptr, su, Bl, rp, (const bf16_t*)bias_bf16,
+                            (bf16_t*)y, ldy, stream, "xq_linear_fwd");
+}
+
+extern "C" int xq_linear_bwd(const xq_weight* w, const void* x, int64_t ldx, const void* dy, int64_t lddy, int64_t M,
+                             const void* lora_A, const void* lora_B, int lora_dtype, int r, float scaling,
+                             const void* su_in, void* dx, int64_t lddx, float* dA, float* dB, void* workspace,
+                             int64_t workspace_bytes, void* stream_) {
+    int rc = check_dense(w, "xq_linear_bwd");
+    if (rc) return rc;
+    const int64_t N = w->rows, K = w->cols;
+    XQ_REQUIRE(M >= 0 && dy, "xq_linear_bwd: dy is NULL");
+    XQ_REQUIRE(r >= 0 && r <= 64, "xq_linear_bwd: LoRA rank %d out of range [0, 64]", r);
+    XQ_REQUIRE(r == 0 || (lora_A && lora_B), "xq_linear_bwd: LoRA factors are NULL");
+    XQ_REQUIRE(lora_dtype == XQ_DT_F32 || lora_dtype == XQ_DT_BF16, "xq_linear_bwd: bad lora_dtype");
+    XQ_REQUIRE(!(dA || dB) || r > 0, "xq_linear_bwd: factor gradients requested with r == 0");
+    XQ_REQUIRE(!(dA || dB) || x, "xq_linear_bwd: x is needed for the factor gradients");
+    hipStream_t stream = (hipStream_t)stream_;
+    const int rp = r_pad_of(r);
+    if (M == 0) {
+        if (dA && (rc = launch_zero_fill(dA, (int64_t)r * K * 4, stream))) return rc;
+        if (dB && (rc = launch_zero_fill(dB, N * r * 4, stream))) return rc;
+        return XQ_OK;
+    }
+    bf16_t *Bt = nullptr, *At = nullptr, *v = nullptr;
+    const bf16_t* su = (const bf16_t*)su_in;
+    float* partial = nullptr;
+    if (rp) {
+        XQ_REQUIRE(workspace && xq_aligned(workspace, 256) && workspace_bytes >= xq_linear_workspace_bytes(M, N, K, r),
+                   "xq_linear_bwd: workspace missing, misaligned or smaller than xq_linear_workspace_bytes()");
+        Carver cv{(uint8_t*)workspace, 0, workspace_bytes};
+        Bt = (bf16_t*)cv.take(rp * N * 2);
+        At = (bf16_t*)cv.take(K * rp * 2);
+        bf16_t* A_bf = (bf16_t*)cv.take(rp * K * 2);
+        v = (bf16_t*)cv.take(M * rp * 2);
+        bf16_t* su_ws = (bf16_t*)cv.take(M * rp * 2);
+        partial = (float*)cv.take(0);
+        // v = bf16(s * dy . B)   [M, rp]
+        if ((rc = launch_factor_prep(lora_B, lora_dtype, N, r, true, Bt, rp, N, 1, stream))) return rc;
+        if ((rc = launch_small_nt((const bf16_t*)dy, lddy, M, N, Bt, rp, scaling, v, nullptr, nullptr, 1, true, stream))) return rc;
+        if (dx && (rc = launch_factor_prep(lora_A, lora_dtype, r, K, true, At, K, rp, 1, stream))) return rc;
+        if (dB && !su) {
+            if ((rc = launch_factor_prep(lora_A, lora_dtype, r, K, false, A_bf, rp, K, 1, stream))) return rc;
+            if ((rc = launch_small_nt((const bf16_t*)x, ldx, M, K, A_bf, rp, scaling, su_ws, nullptr, nullptr, 1, true, stream))) return rc;
+            su = su_ws;
+        }
+    }
+    if (dx) {
+        XQ_REQUIRE(lddx % 8 == 0 && xq_aligned(dx, 16), "xq_linear_bwd: dx rows must be 16-byte aligned");
+        if ((rc = launch_tile_gemm(w, false, (const bf16_t*)dy, lddy, M, nullptr, nullptr, v, At, rp, nullptr, (bf16_t*)dx,
+                                   lddx, stream, "xq_linear_bwd(dx)")))
+            return rc;
+    }
+    // dB[N, r] = dy^T . su ; dA[r, K] = (x^T . v)^T
+    if (dB && (rc = launch_tn((const bf16_t*)dy, lddy, N, su, rp, r, M, false, dB, partial, nullptr, 1, stream))) return rc;
+    if (dA && (rc = launch_tn((const bf16_t*)x, ldx, K, v, rp, r, M, true, dA, partial, nullptr, 1, stream))) return rc;
+    return XQ_OK;
+}
+
+extern "C" int xq_grouped_gemm(const xq_weight* w, int transpose_w, const void* a, int64_t lda, int64_t n_rows,
+                               const int32_t* offsets, const int32_t* tile_offsets, const void* su,
+                               const void* lora_right, int r_pad, void* y, int64_t ldy, void* stream) {
+    int rc = xq_validate_weight(w, "xq_grouped_gemm");
+    if (rc) return rc;
+    XQ_REQUIRE(offsets && tile_offsets, "xq_grouped_gemm: offsets / tile_offsets are NULL");
+    XQ_REQUIRE(n_rows == 0 || (a && y), "xq_grouped_gemm: NULL activation pointer");
+    XQ_REQUIRE(ldy % 8 == 0 && xq_aligned(y, 16), "xq_grouped_gemm: y rows must be 16-byte aligned");
+    // bank is [E, K_in, N_out]: forward contracts over W rows, dgrad over W cols
+    return launch_tile_gemm(w, transpose_w != 0, (const bf16_t*)a, lda, n_rows, offsets, tile_offsets, (const bf16_t*)su,
+                            (const bf16_t*)lora_right, r_pad, nullptr, (bf16_t*)y, ldy, (hipStream_t)stream,
+                            "xq_grouped_gemm");
+}
+
+extern "C" int xq_factor_prep(const void* in, int in_dtype, int64_t rows_in, int64_t cols_in, int transpose,
+                              void* out_bf16, int64_t rows_out, int64_t cols_out, int64_t num_experts, void* stream) {
+    XQ_REQUIRE(in_dtype == XQ_DT_F32 || in_dtype == XQ_DT_BF16, "xq_factor_prep: bad dtype");
+    XQ_REQUIRE(num_experts == 0 || rows_out * cols_out == 0 || (in && out_bf16), "xq_factor_prep: NULL pointer");
+    int64_t need_r = transpose ? cols_in : rows_in, need_c = transpose ? rows_in : cols_in;
+    XQ_REQUIRE(rows_out >= need_r && cols_out >= need_c, "xq_factor_prep: output [%lld, %lld] smaller than source", (long long)rows_out, (long long)cols_out);
+    return launch_factor_prep(in, in_dtype, rows_in, cols_in, transpose != 0, (bf16_t*)out_bf16, rows_out, cols_out,
+                              num_experts, (hipStream_t)stream);
+}
+
+extern "C" int xq_grouped_lora_down(const void* a, int64_t lda, int64_t n_rows, const int32_t* offsets,
+                                    const int32_t* tile_offsets, int32_t num_experts, const void* F, int shared,
+                                    int r_pad, int64_t K, float scale, void* t, void* stream) {
+    XQ_REQUIRE(offsets && tile_offsets && num_experts >= 1, "xq_grouped_lora_down: offsets / tile_offsets are NULL");
+    XQ_REQUIRE(n_rows == 0 || (a && F && t), "xq_grouped_lora_down: NULL pointer");
+    return launch_small_nt((const bf16_t*)a, lda, n_rows, K, (const bf16_t*)F, r_pad, scale, (bf16_t*)t, offsets,
+                           tile_offsets, num_experts, shared != 0, (hipStream_t)stream);
+}
+
+extern "C" int64_t xq_lora_wgrad_workspace_bytes(int64_t n_rows, int64_t width, int r_pad) {
+    return tn_partial_bytes(n_rows, width, r_pad) + 256;
+}
+
+extern "C" int xq_grouped_lora_wgrad(const void* P, int64_t ldp, int64_t p_width, const void* Q, int r_pad, int r_out,
+                                     int64_t n_rows, const int32_t* offsets, int32_t num_experts, int transpose_out,
+                                     float* out, void* workspace, void* stream) {
+    XQ_REQUIRE(out && (n_rows == 0 || (P && Q)), "xq_grouped_lora_wgrad: NULL pointer");
+    if (n_rows == 0 && !offsets) return launch_zero_fill(out, p_width * r_out * 4, (hipStream_t)stream);
+    return launch_tn((const bf16_t*)P, ldp, p_width, (const bf16_t*)Q, r_pad, r_out, n_rows, transpose_out != 0, out,
+                     (float*)workspace, offsets, num_experts, (hipStream_t)stream);
+}

@@ -1,0 +1,34 @@
+// Low-rank (LoRA) helper kernels: factor preparation, the skinny "down"
+// products (x.A^T, dy.B) and the weight-gradient products (dy^T.u, v^T.x).
+// All are HBM-bound: they stream one large bf16 activation matrix once.
+#pragma once
+
+#include "xq_common.h"
+
+namespace xq {
+
+// out[i][j] (bf16, [R_out, C_out], zero padded) = in[i][j] or in[j][i];  `in` is
+// fp32 or bf16 with shape [R_in, C_in] per expert.
+int launch_factor_prep(const void* in, int in_dtype, int64_t R_in, int64_t C_in, bool transpose,
+                       bf16_t* out, int64_t R_out, int64_t C_out, int64_t num_experts, hipStream_t stream);
+
+// T[rows, r_pad] = bf16(scale * In[rows, Kc] . F[r_pad, Kc]^T).
+//   dense (offsets == NULL): rows = n_rows, one F;
+//   grouped: rows in expert order, F[e] = F + e*r_pad*Kc (or shared).
+int launch_small_nt(const bf16_t* In, int64_t ld_in, int64_t n_rows, int64_t Kc, const bf16_t* F,
+                    int r_pad, float scale, bf16_t* T, const int32_t* offsets,
+                    const int32_t* tile_offsets, int32_t num_experts, bool shared_f, hipStream_t stream);
+
+// out[c][j] (or out[j][c] when transpose_out) = sum_m P[m][c] * Q[m][j], fp32.
+//   dense: all rows, split over `splits` row ranges, partials in `partial`
+//          ([splits][width][r_pad] fp32) reduced in fixed order (deterministic);
+//   grouped: out[e] over rows [offsets[e], offsets[e+1]); zero for empty experts.
+// r_out is the number of valid columns of Q (<= r_pad) written.
+int64_t tn_partial_bytes(int64_t n_rows, int64_t width, int r_pad);
+int launch_tn(const bf16_t* P, int64_t ldp, int64_t width, const bf16_t* Q, int r_pad, int r_out,
+              int64_t n_rows, bool transpose_out, float* out, float* partial,
+              const int32_t* offsets, int32_t num_experts, hipStream_t stream);
+
+int launch_zero_fill(void* p, int64_t bytes, hipStream_t stream);
+
+}  // namespace xq

@@ -1,0 +1,224 @@
+"""PyTorch-ROCm custom ops and autograd functions over the C ABI.
+
+Ops are registered for the HIP ("cuda") dispatch key only: calling them with
+CPU tensors raises from the dispatcher -- there is no CPU or eager fallback.
+Outputs and workspaces are allocated here with torch (device memory is
+plumbing); the kernels allocate nothing.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from dataclasses import dataclass
+from typing import List, Optional, Tuple
+
+import torch
+from torch import Tensor
+
+from . import _C
+
+
+_CODE_TO_DT = {0: torch.float32, 1: torch.bfloat16, 2: torch.float8_e4m3fn}
+_DT_TO_CODE = {v: k for k, v in _CODE_TO_DT.items()}
+
+
+@dataclass
+class QuantWeight:
+    """Host-side description of a (bank of) quantized matrices.
+
+    packed / scales are tensors holding the right BYTES (uint8 buffers or the
+    bytes-in-fp32 parameter the modules keep for FSDP2); scale_dtype is the
+    true element type of the scales.  rows x cols is the decoded shape:
+    [out, in] for dense (FLAT), [in, out] per expert for banks (GKN)."""
+
+    fmt: str
+    layout: int
+    packed: Tensor
+    scales: Tensor
+    scale_dtype: torch.dtype
+    rows: int
+    cols: int
+    group: int
+    global_scale: Optional[Tensor] = None
+    num_experts: int = 1
+
+    def c(self) -> _C.XqWeight:
+        return _C.make_weight(self.fmt, self.layout, self.packed, self.scales, self.scale_dtype, self.rows,
+                              self.cols, self.group, self.global_scale, self.num_experts)
+
+
+def _r_pad(r: int) -> int:
+    return 0 if r <= 0 else ((r + 15) // 16) * 16
+
+
+def _lora_dt(t: Optional[Tensor]) -> int:
+    if t is None or t.dtype == torch.float32:
+        return _C.XQ_DT_F32
+    if t.dtype == torch.bfloat16:
+        return _C.XQ_DT_BF16
+    raise _C.XqError(f"LoRA factors must be fp32 or bf16, got {t.dtype}")
+
+
+def _as_2d(x: Tensor) -> Tensor:
+    x2 = x.reshape(-1, x.shape[-1])
+    if x2.stride(-1) != 1 or (x2.shape[0] > 1 and x2.stride(0) % 8 != 0) or x2.data_ptr() % 16 != 0:
+        x2 = x2.contiguous()
+    return x2
+
+
+def _ld(x2: Tensor) -> int:
+    return x2.stride(0) if x2.shape[0] > 1 else x2.shape[1]
+
+
+# ---------------------------------------------------------------------------
+# dense: custom ops
+# ---------------------------------------------------------------------------
+@torch.library.custom_op("xq::linear_fwd", mutates_args=(), device_types="cuda")
+def _linear_fwd_op(x: Tensor, packed: Tensor, scales: Tensor, global_scale: Optional[Tensor],
+                   lora_A: Optional[Tensor], lora_B: Optional[Tensor], bias: Optional[Tensor],
+                   fmt: str, scale_code: int, group: int, N: int, K: int, r: int,
+                   scaling: float) -> Tuple[Tensor, Tensor]:
+    if x.dtype != torch.bfloat16:
+        raise _C.XqError(f"activations must be bf16, got {x.dtype}")
+    x2 = _as_2d(x)
+    M = x2.shape[0]
+    if x2.shape[1] != K:
+        raise _C.XqError(f"input width {x2.shape[1]} != in_features {K}")
+    w = _C.make_weight(fmt, _C.XQ_LAYOUT_FLAT, packed, scales, _CODE_TO_DT[scale_code], N, K, group, global_scale)
+    dev = x.device
+    y = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+    rp = _r_pad(r)
+    su = torch.empty(M, rp, dtype=torch.bfloat16, device=dev)
+    L = _C.lib()
+    ws_bytes = L.xq_linear_workspace_bytes(M, N, K, r)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    A = lora_A.contiguous() if lora_A is not None else None
+    B = lora_B.contiguous() if lora_B is not None else None
+    b = bias.to(torch.bfloat16).contiguous() if bias is not None else None
+    _C.check(L.xq_linear_fwd(ctypes.byref(w), x2.data_ptr(), _ld(x2), M, _C.ptr(A), _C.ptr(B), _lora_dt(A), r,
+                             scaling, _C.ptr(b), y.data_ptr(), N, su.data_ptr() if rp else None, ws.data_ptr(),
+                             ws_bytes, _C.stream_ptr(dev)))
+    return y.reshape(*x.shape[:-1], N), su
+
+
+@_linear_fwd_op.register_fake
+def _(x, packed, scales, global_scale, lora_A, lora_B, bias, fmt, scale_code, group, N, K, r, scaling):
+    M = x.numel() // max(x.shape[-1], 1)
+    return x.new_empty(*x.shape[:-1], N), x.new_empty(M, _r_pad(r))
+
+
+@torch.library.custom_op("xq::linear_bwd", mutates_args=(), device_types="cuda")
+def _linear_bwd_op(dy: Tensor, x: Tensor, su: Tensor, packed: Tensor, scales: Tensor,
+                   global_scale: Optional[Tensor], lora_A: Optional[Tensor], lora_B: Optional[Tensor],
+                   fmt: str, scale_code: int, group: int, N: int, K: int, r: int, scaling: float,
+                   need_dx: bool, need_dA: bool, need_dB: bool) -> Tuple[Tensor, Tensor, Tensor]:
+    dy2 = _as_2d(dy.to(torch.bfloat16))
+    x2 = _as_2d(x)
+    M = dy2.shape[0]
+    w = _C.make_weight(fmt, _C.XQ_LAYOUT_FLAT, packed, scales, _CODE_TO_DT[scale_code], N, K, group, global_scale)
+    dev = dy.device
+    dx = torch.empty(M, K, dtype=torch.bfloat16, device=dev) if need_dx else torch.empty(0, dtype=torch.bfloat16, device=dev)
+    dA = torch.empty(r, K, dtype=torch.float32, device=dev) if need_dA else torch.empty(0, device=dev)
+    dB = torch.empty(N, r, dtype=torch.float32, device=dev) if need_dB else torch.empty(0, device=dev)
+    L = _C.lib()
+    ws_bytes = L.xq_linear_workspace_bytes(M, N, K, r)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    A = lora_A.contiguous() if lora_A is not None else None
+    B = lora_B.contiguous() if lora_B is not None else None
+    _C.check(L.xq_linear_bwd(ctypes.byref(w), x2.data_ptr(), _ld(x2), dy2.data_ptr(), _ld(dy2), M, _C.ptr(A),
+                             _C.ptr(B), _lora_dt(A), r, scaling, su.data_ptr() if su.numel() else None,
+                             dx.data_ptr() if need_dx else None, K, dA.data_ptr() if need_dA else None,
+                             dB.data_ptr() if need_dB else None, ws.data_ptr(), ws_bytes, _C.stream_ptr(dev)))
+    if need_dx:
+        dx = dx.reshape(x.shape)
+    return dx, dA, dB
+
+
+@_linear_bwd_op.register_fake
+def _(dy, x, su, packed, scales, global_scale, lora_A, lora_B, fmt, scale_code, group, N, K, r, scaling,
+      need_dx, need_dA, need_dB):
+    return (x.new_empty(x.shape) if need_dx else x.new_empty(0),
+            x.new_empty(r, K, dtype=torch.float32) if need_dA else x.new_empty(0, dtype=torch.float32),
+            x.new_empty(N, r, dtype=torch.float32) if need_dB else x.new_empty(0, dtype=torch.float32))
+
+
+class QLoRALinearFunction(torch.autograd.Function):
+    """y = x . deq(W)^T + bias + s * (x . A^T) . B^T with the packed weight decoded inside the GEMM.
+
+    Backward returns (dx, dA, dB); the frozen packed weight gets no gradient
+    (qlora/modules/block_fp8_linear.py:48-51).  Nothing but x and the small
+    [M, r] LoRA intermediate is saved -- no decoded weight."""
+
+    @staticmethod
+    def forward(ctx, x, lora_A, lora_B, bias, qw: QuantWeight, r: int, scaling: float):
+        A = lora_A[:r] if lora_A is not None else None
+        B = lora_B[:, :r] if lora_B is not None else None
+        y, su = _linear_fwd_op(x, qw.packed, qw.scales, qw.global_scale, A, B, bias, qw.fmt,
+                               _DT_TO_CODE[qw.scale_dtype], qw.group, qw.rows, qw.cols, r, float(scaling))
+        ctx.qw, ctx.r, ctx.scaling = qw, r, float(scaling)
+        ctx.save_for_backward(x, su, lora_A, lora_B)
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, su, lora_A, lora_B = ctx.saved_tensors
+        qw, r = ctx.qw, ctx.r
+        need_dx, need_dA, need_dB = ctx.needs_input_grad[0], ctx.needs_input_grad[1], ctx.needs_input_grad[2]
+        A = lora_A[:r] if lora_A is not None else None
+        B = lora_B[:, :r] if lora_B is not None else None
+        dx, dA, dB = _linear_bwd_op(dy, x, su, qw.packed, qw.scales, qw.global_scale, A, B, qw.fmt,
+                                    _DT_TO_CODE[qw.scale_dtype], qw.group, qw.rows, qw.cols, r, ctx.scaling,
+                                    need_dx, need_dA, need_dB)
+        gA = gB = None
+        if need_dA:
+            gA = dA if lora_A.shape[0] == r else torch.cat([dA, dA.new_zeros(lora_A.shape[0] - r, dA.shape[1])], 0)
+            gA = gA.to(lora_A.dtype)
+        if need_dB:
+            gB = dB if lora_B.shape[1] == r else torch.cat([dB, dB.new_zeros(dB.shape[0], lora_B.shape[1] - r)], 1)
+            gB = gB.to(lora_B.dtype)
+        gbias = None
+        if ctx.needs_input_grad[3]:
+            gbias = dy.reshape(-1, dy.shape[-1]).sum(0)
+        return (dx if need_dx else None), gA, gB, gbias, None, None, None
+
+
+def qlora_linear(x: Tensor, qw: QuantWeight, lora_A: Optional[Tensor], lora_B: Optional[Tensor], r: int,
+                 scaling: float, bias: Optional[Tensor] = None) -> Tensor:
+    return QLoRALinearFunction.apply(x, lora_A, lora_B, bias, qw, r, scaling)
+
+
+# ---------------------------------------------------------------------------
+# SwiGLU
+# ---------------------------------------------------------------------------
+class SiluAndMulFunction(torch.autograd.Function):
+    """fused_silu_and_mul (ops/fused_silu_and_mul.py): h = bf16(silu(gate)) * up."""
+
+    @staticmethod
+    def forward(ctx, gate: Tensor, up: Tensor):
+        _C.require_hip(gate, up)
+        g2, u2 = _as_2d(gate), _as_2d(up)
+        if _ld(g2) != _ld(u2):
+            g2, u2 = g2.contiguous(), u2.contiguous()
+        rows, cols = g2.shape
+        h = torch.empty(rows, cols, dtype=torch.bfloat16, device=gate.device)
+        _C.check(_C.lib().xq_silu_mul_fwd(g2.data_ptr(), u2.data_ptr(), _ld(g2), None, h.data_ptr(), cols, rows, cols,
+                                          _C.stream_ptr(gate.device)))
+        ctx.save_for_backward(g2, u2)
+        ctx.shape = gate.shape
+        return h.reshape(gate.shape)
+
+    @staticmethod
+    def backward(ctx, dh):
+        g2, u2 = ctx.saved_tensors
+        rows, cols = g2.shape
+        d2 = _as_2d(dh.to(torch.bfloat16))
+        dg = torch.empty(rows, cols, dtype=torch.bfloat16, device=dh.device)
+        du = torch.empty(rows, cols, dtype=torch.bfloat16, device=dh.device)
+        _C.check(_C.lib().xq_silu_mul_bwd(g2.data_ptr(), u2.data_ptr(), _ld(g2), d2.data_ptr(), _ld(d2), None,
+                                          dg.data_ptr(), du.data_ptr(), cols, None, rows, cols,
+                                          _C.stream_ptr(dh.device)))
+        return dg.reshape(ctx.shape), du.reshape(ctx.shape)
+
+
+def silu_and_mul(gate: Tensor, up: Tensor) -> Tensor:
+    return SiluAndMulFunction.apply(gate, up)

@@ -1,0 +1,19 @@
+"""Drop-in counterparts of ``xorl.qlora.modules`` backed by the HIP kernels."""
+
+from .linear import (
+    BlockFP8QLoRALinear,
+    Int4QLoRALinear,
+    LoraModule,
+    NvFP4QLoRALinear,
+    QLoRALinear,
+    deregister_qlora_weights_from_fsdp,
+)
+
+__all__ = [
+    "LoraModule",
+    "QLoRALinear",
+    "BlockFP8QLoRALinear",
+    "NvFP4QLoRALinear",
+    "Int4QLoRALinear",
+    "deregister_qlora_weights_from_fsdp",
+]

@@ -1,0 +1,607 @@
+"""QLoRA linear modules: quantized frozen base weight + trainable LoRA, on HIP kernels.
+
+These classes keep the constructor signatures, parameter / buffer names,
+shapes, dtypes and helper methods of the reference modules so that trainer
+code, checkpoint code and FSDP2 wrapping written against the reference keep
+working:
+
+  QLoRALinear              xorl/qlora/modules/linear.py:29-412
+  BlockFP8QLoRALinear      xorl/qlora/modules/block_fp8_linear.py
+  NvFP4QLoRALinear         xorl/qlora/modules/nvfp4_linear.py
+  Int4QLoRALinear          no counterpart class in the reference (its int4 is a
+                           stand-alone codec, ops/quantize/int4_quantize.py);
+                           follows the same subclass pattern, buffer name
+                           ``weight_scales`` as the reference's NF4 module.
+
+What differs is forward(): instead of materialising the decoded weight and
+calling F.linear plus two LoRA GEMMs, it runs one fused dequant-GEMM (the
+packed bytes are decoded inside the kernel) and the backward never sees a
+decoded weight either.
+"""
+
+from __future__ import annotations
+
+import math
+from typing import Dict, Iterator, Optional, Tuple
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+from torch import Tensor
+
+from .. import _C
+from .. import quantize as Q
+from ..functional import QuantWeight, qlora_linear
+
+
+class LoraModule:
+    """Interface shared by LoRA-carrying modules (xorl/lora/modules/base.py:18-157)."""
+
+    r: int
+    lora_alpha: int
+    scaling: float
+    exact_merged_forward: bool = False
+
+    @classmethod
+    def from_module(cls, module: nn.Module, r: int, lora_alpha: int, **kwargs):
+        raise NotImplementedError
+
+    def reset_lora_parameters(self) -> None:
+        raise NotImplementedError
+
+    def get_delta_weight(self) -> Tensor:
+        raise NotImplementedError(
+            f"{type(self).__name__} does not implement get_delta_weight(). "
+            "For MoE modules, use merge_weights() directly."
+        )
+
+    def merge_weights(self) -> None:
+        raise NotImplementedError
+
+    def get_lora_parameters(self) -> Iterator[nn.Parameter]:
+        if not isinstance(self, nn.Module):
+            raise TypeError("LoraModule must be mixed with nn.Module")
+        for name, p in self.named_parameters():
+            if "lora_" in name:
+                yield p
+
+    def get_lora_state_dict(self) -> Dict[str, Tensor]:
+        if not isinstance(self, nn.Module):
+            raise TypeError("LoraModule must be mixed with nn.Module")
+        return {n: p.detach() for n, p in self.named_parameters() if "lora_" in n}
+
+
+def _is_dtensor(t) -> bool:
+    return hasattr(t, "_local_tensor") and hasattr(t, "full_tensor")
+
+
+class QLoRALinear(LoraModule, nn.Module):
+    """Abstract base.  Subclasses register ``packed_weight_f32`` (the packed bytes
+    viewed four per fp32 so FSDP2 can shard them without a dtype cast) and the
+    uint8 scale buffers, then call ``reset_lora_parameters()``."""
+
+    adapter_gradient_producer_family = "module_managed"
+    # FSDP2 must not apply a parameter-cast policy to this module: the fp32
+    # parameter holds raw bytes and the LoRA masters stay fp32.
+    fsdp_requires_full_precision = True
+
+    _is_prequantized: bool = False
+    _inline_loaded: bool = False
+    _merge_sources: Optional[Tuple[str, ...]] = None
+    _source_fqn: Optional[str] = None
+    _source_quant_format: Optional[str] = None
+
+    def __init__(self, in_features: int, out_features: int, r: int = 16, lora_alpha: int = 16,
+                 quant_format: str = "nvfp4", quant_group_size: int = 16, bias: bool = False,
+                 device: Optional[torch.device] = None, enable_aqn: bool = False, aqn_alpha: float = 1.0):
+        if type(self) is QLoRALinear:
+            raise TypeError(
+                "QLoRALinear is abstract. Use NvFP4QLoRALinear, BlockFP8QLoRALinear or Int4QLoRALinear."
+            )
+        if r <= 0 or r > 64:
+            raise ValueError(f"LoRA rank must be in [1, 64] for the fused kernels, got {r}")
+        super().__init__()
+        self.in_features, self.out_features = in_features, out_features
+        self.quant_format, self.quant_group_size = quant_format, quant_group_size
+        self.enable_aqn, self.aqn_alpha = enable_aqn, aqn_alpha
+        self._aqn_step_cache: Optional[Tensor] = None
+        self._aqn_stream = None
+        self._aqn_noise_buf: Optional[Tensor] = None
+        self._aqn_noise_ready = False
+        self.r, self.lora_alpha = r, lora_alpha
+        self.active_r, self.active_lora_alpha = r, lora_alpha
+        self.scaling = lora_alpha / r
+        self.lora_A = nn.Parameter(torch.empty(r, in_features, dtype=torch.float32, device=device))
+        self.lora_B = nn.Parameter(torch.empty(out_features, r, dtype=torch.float32, device=device))
+        if bias:
+            self.bias = nn.Parameter(torch.zeros(out_features, device=device), requires_grad=False)
+        else:
+            self.register_parameter("bias", None)
+        self.register_parameter("weight", None)   # only used by deferred (meta-init) quantization
+        self._ema_amax: Optional[Tensor] = None
+        self._scale_dtypes: Dict[str, torch.dtype] = {}
+
+    # ------------------------------------------------------------------ LoRA
+    def reset_lora_parameters(self) -> None:
+        nn.init.kaiming_uniform_(self.lora_A, a=math.sqrt(5))
+        nn.init.zeros_(self.lora_B)
+
+    def set_runtime_lora_config(self, lora_rank: int, lora_alpha: int) -> None:
+        if lora_rank <= 0 or lora_rank > self.r:
+            raise ValueError(f"Active LoRA rank must be in [1, {self.r}], got {lora_rank}")
+        self.active_r, self.active_lora_alpha = lora_rank, lora_alpha
+
+    def _active_scaling(self) -> float:
+        return self.active_lora_alpha / self.active_r
+
+    @staticmethod
+    def _to_regular_tensor(t: Tensor) -> Tensor:
+        return t.full_tensor() if hasattr(t, "full_tensor") else t
+
+    def get_delta_weight(self) -> Tensor:
+        A = self._to_regular_tensor(self.lora_A[: self.active_r])
+        B = self._to_regular_tensor(self.lora_B[:, : self.active_r])
+        return (B @ A) * self._active_scaling()
+
+    # ------------------------------------------------------------------ factories
+    @classmethod
+    def _class_for(cls, quant_format: str):
+        table = {"block_fp8": BlockFP8QLoRALinear, "nvfp4": NvFP4QLoRALinear, "int4": Int4QLoRALinear}
+        if quant_format not in table:
+            raise ValueError(f"unsupported quant_format {quant_format!r}; expected one of {sorted(table)}")
+        return table[quant_format]
+
+    @classmethod
+    def from_module(cls, module: nn.Module, r: int = 16, lora_alpha: int = 16, **kwargs) -> "QLoRALinear":
+        if cls is QLoRALinear:
+            fmt = kwargs.pop("quant_format", "nvfp4")
+            kwargs.pop("quant_group_size", None)
+            return cls._class_for(fmt).from_module(module, r=r, lora_alpha=lora_alpha, **kwargs)
+        q = cls(in_features=module.in_features, out_features=module.out_features, r=r, lora_alpha=lora_alpha,
+                bias=module.bias is not None, device=module.weight.device,
+                enable_aqn=kwargs.get("enable_aqn", False), aqn_alpha=kwargs.get("aqn_alpha", 1.0))
+        if module.bias is not None:
+            with torch.no_grad():
+                q.bias.copy_(module.bias.detach())
+        q._init_from_weight(module.weight.detach())
+        return q
+
+    def _init_from_weight(self, w: Tensor) -> None:
+        self._quantize_and_store(w)
+
+    @classmethod
+    def from_quantized(cls, packed_weight: Tensor, weight_scales: Optional[Tensor] = None,
+                       weight_block_scales: Optional[Tensor] = None, weight_global_scale: Optional[Tensor] = None,
+                       in_features: int = 0, out_features: int = 0, r: int = 16, lora_alpha: int = 16,
+                       quant_format: str = "nvfp4", quant_group_size: int = 16, bias: bool = False,
+                       device: Optional[torch.device] = None, **kwargs) -> "QLoRALinear":
+        if cls is QLoRALinear:
+            cls = cls._class_for(quant_format)
+        q = cls(in_features=in_features, out_features=out_features, r=r, lora_alpha=lora_alpha, bias=bias,
+                device=device)
+        q.packed_weight_f32 = nn.Parameter(cls._to_uint8(packed_weight).contiguous().view(torch.float32),
+                                           requires_grad=False)
+        q._scale_dtypes = {}
+        for name, t in (("weight_scales", weight_scales), ("weight_block_scales", weight_block_scales),
+                        ("weight_global_scale", weight_global_scale)):
+            if t is not None:
+                q._scale_dtypes[name] = t.dtype
+                setattr(q, name, cls._to_uint8(t))
+        q._is_prequantized = True
+        return q
+
+    # ------------------------------------------------------------------ byte storage
+    @staticmethod
+    def _to_uint8(t: Tensor) -> Tensor:
+        """uint8 view: scales and codes are stored as bytes so that no mixed
+        precision policy can cast them (the true dtype lives in _scale_dtypes)."""
+        return t.contiguous() if t.dtype == torch.uint8 else t.contiguous().view(torch.uint8)
+
+    def _recover_tensor(self, buf: Tensor, original_dtype: torch.dtype) -> Tensor:
+        return buf if original_dtype == torch.uint8 else buf.contiguous().view(original_dtype)
+
+    def _write_packed_weight(self, uint8_data: Tensor) -> None:
+        """Store packed bytes into packed_weight_f32 (plain, meta or DTensor shard)."""
+        f32 = uint8_data.contiguous().view(torch.float32)
+        cur = self.packed_weight_f32
+        if cur is None or cur.device.type == "meta":
+            if cur is not None:
+                f32 = f32.reshape(cur.shape)
+            self.packed_weight_f32 = nn.Parameter(f32, requires_grad=False)
+            return
+        if _is_dtensor(cur):
+            from torch.distributed._tensor import Shard
+
+            f32 = f32.reshape(cur.shape)
+            dim = next((p.dim for p in cur.placements if isinstance(p, Shard)), None)
+            local = cur._local_tensor
+            if dim is None:
+                local.copy_(f32)
+                return
+            mesh = cur.device_mesh
+            chunk = f32.shape[dim] // mesh.size()
+            start = mesh.get_local_rank() * chunk
+            local.copy_(f32.narrow(dim, start, chunk))
+            return
+        if cur.numel() == f32.numel():
+            cur.data.copy_(f32.reshape(cur.shape))
+        else:
+            self.packed_weight_f32 = nn.Parameter(f32, requires_grad=False)
+
+    @torch.compiler.disable
+    def _read_packed_weight_uint8(self) -> Tensor:
+        f32 = self.packed_weight_f32.data
+        if _is_dtensor(f32):
+            f32 = f32.full_tensor()
+        elif f32.dtype != torch.float32:
+            raise RuntimeError(
+                f"QLoRA packed_weight_f32 has dtype {f32.dtype} (expected float32). "
+                "FSDP2 mixed precision likely cast it, corrupting packed weight data. "
+                "Ensure packed_weight_f32 is deregistered from FSDP param groups."
+            )
+        return f32.contiguous().view(torch.uint8)
+
+    def _apply(self, fn, recurse: bool = True):
+        """model.to(bf16) must not touch the packed bytes or the fp32 LoRA masters."""
+        probe = fn(torch.empty(0, dtype=torch.float32, device=self.lora_A.device))
+        names = [n for n in ("lora_A", "lora_B", "packed_weight_f32") if self._parameters.get(n) is not None]
+        held = {n: self._parameters.pop(n) for n in names}
+        try:
+            out = super()._apply(fn, recurse=recurse)
+        finally:
+            for n, p in held.items():
+                if p.is_meta:
+                    p = nn.Parameter(torch.empty_like(p, dtype=torch.float32, device=probe.device),
+                                     requires_grad=p.requires_grad)
+                else:
+                    with torch.no_grad():
+                        p.data = p.data.to(device=probe.device, dtype=torch.float32)
+                        if p.grad is not None:
+                            p.grad.data = p.grad.data.to(device=probe.device, dtype=torch.float32)
+                self._parameters[n] = p
+        return out
+
+    # ------------------------------------------------------------------ checkpoint loading
+    def load_prequantized_weights(self, weight_map: dict, shard_cache: dict, weights_path: str) -> None:
+        import os
+
+        import safetensors.torch
+
+        def _load(key: str) -> Tensor:
+            shard = weight_map.get(key)
+            if shard is None:
+                raise RuntimeError(f"Key {key} not found in checkpoint index")
+            if shard not in shard_cache:
+                path = os.path.join(weights_path, shard)
+                if not os.path.exists(path):
+                    from transformers.utils import cached_file
+
+                    path = cached_file(weights_path, shard)
+                shard_cache[shard] = safetensors.torch.load_file(path, device="cpu")
+            return shard_cache[shard][key]
+
+        self._load_prequantized(_load)
+
+    def _load_prequantized(self, _load_tensor) -> None:
+        raise NotImplementedError
+
+    def quantize_weight(self) -> None:
+        """Deferred quantization: turn the (FSDP-loaded) `weight` into packed form."""
+        if self.weight is None:
+            return
+        w = self.weight.data
+        if _is_dtensor(w):
+            w = w.full_tensor()
+        self._quantize_and_store(w)
+        self.weight = None
+
+    def _quantize_and_store(self, w: Tensor, global_amax: Optional[Tensor] = None) -> None:
+        raise NotImplementedError
+
+    def _quant_weight(self) -> QuantWeight:
+        """Describe the packed state for the kernels (no copies)."""
+        raise NotImplementedError
+
+    @torch.compiler.disable
+    def _dequantize_weight(self) -> Tensor:
+        raise NotImplementedError
+
+    @torch.compiler.disable
+    def _compute_aqn_step(self) -> Tensor:
+        raise NotImplementedError
+
+    def merge_weights(self, ema_decay: float = 0.1) -> None:
+        """W' = Q(deq(W) + dW); re-initialise A, zero B (block_fp8_linear.py:111-119)."""
+        with torch.no_grad():
+            w = self._dequantize_weight()
+            merged = w + self.get_delta_weight().to(w.dtype)
+            self._requantize_merged(merged, ema_decay)
+            nn.init.kaiming_uniform_(self.lora_A, a=math.sqrt(5))
+            self.lora_B.zero_()
+
+    def _requantize_merged(self, merged: Tensor, ema_decay: float) -> None:
+        self._quantize_and_store(merged)
+
+    # ------------------------------------------------------------------ AQN (optional, off by default)
+    @torch.compiler.disable
+    def _aqn_start_noise(self, device: torch.device, dtype: torch.dtype) -> None:
+        shape = (self.out_features, self.in_features)
+        if self._aqn_stream is None:
+            self._aqn_stream = torch.cuda.Stream(device=device)
+        buf = self._aqn_noise_buf
+        if buf is None or buf.shape != shape or buf.dtype != dtype or buf.device != device:
+            self._aqn_noise_buf = torch.empty(*shape, device=device, dtype=dtype)
+        self._aqn_stream.wait_stream(torch.cuda.current_stream(device))
+        with torch.cuda.stream(self._aqn_stream):
+            self._aqn_noise_buf.normal_()
+        self._aqn_noise_ready = True
+
+    @torch.compiler.disable
+    def _aqn_apply_noise(self, w: Tensor) -> Tensor:
+        torch.cuda.current_stream(w.device).wait_stream(self._aqn_stream)
+        if self._aqn_step_cache is None:
+            self._aqn_step_cache = self._compute_aqn_step()
+        step = self._aqn_step_cache.to(dtype=w.dtype, device=w.device)
+        self._aqn_noise_ready = False
+        return torch.addcmul(w, self._aqn_noise_buf, step, value=self.aqn_alpha)
+
+    def _forward_with_noise(self, x: Tensor) -> Tensor:
+        """AQN perturbs the decoded weight, so this training-time regulariser needs
+        the weight materialised (qlora/modules/linear.py:369-385 as written)."""
+        if not self._aqn_noise_ready:
+            self._aqn_start_noise(x.device, x.dtype)
+        w = self._aqn_apply_noise(self._dequantize_weight().to(x.dtype))
+        base = F.linear(x, w, self.bias)
+        A, B = self.lora_A[: self.active_r], self.lora_B[:, : self.active_r]
+        lo = F.linear(F.linear(x.to(A.dtype), A), B) * self._active_scaling()
+        return base + lo.to(base.dtype)
+
+    # ------------------------------------------------------------------ forward
+    def forward(self, x: Tensor) -> Tensor:
+        if self.enable_aqn and self.training:
+            return self._forward_with_noise(x)
+        return qlora_linear(x, self._quant_weight(), self.lora_A, self.lora_B, self.active_r,
+                            self._active_scaling(), self.bias)
+
+    # ------------------------------------------------------------------ checkpoint helpers
+    def get_quantized_state_dict(self) -> Dict[str, Tensor]:
+        state = {"packed_weight_f32": self.packed_weight_f32}
+        for name in ("weight_scales", "weight_block_scales", "weight_global_scale"):
+            t = getattr(self, name, None)
+            if t is not None:
+                state[name] = t
+        return state
+
+    def extra_repr(self) -> str:
+        s = (f"in_features={self.in_features}, out_features={self.out_features}, bias={self.bias is not None}, "
+             f"r={self.r}, lora_alpha={self.lora_alpha}, quant_format={self.quant_format}, "
+             f"quant_group_size={self.quant_group_size}")
+        return s + (f", aqn=True(alpha={self.aqn_alpha})" if self.enable_aqn else "")
+
+
+# =============================================================================
+class BlockFP8QLoRALinear(QLoRALinear):
+    """e4m3 bytes + fp32 scale per 128x128 block (block_fp8_linear.py:14-144)."""
+
+    def __init__(self, in_features: int, out_features: int, r: int = 16, lora_alpha: int = 16, bias: bool = False,
+                 device: Optional[torch.device] = None, enable_aqn: bool = False, aqn_alpha: float = 1.0):
+        super().__init__(in_features, out_features, r=r, lora_alpha=lora_alpha, quant_format="block_fp8",
+                         quant_group_size=128, bias=bias, device=device, enable_aqn=enable_aqn, aqn_alpha=aqn_alpha)
+        if in_features % 4:
+            raise ValueError(f"block_fp8 needs in_features % 4 == 0, got {in_features}")
+        self.packed_weight_f32 = nn.Parameter(
+            torch.empty(out_features, in_features // 4, dtype=torch.float32, device=device), requires_grad=False)
+        self.register_buffer("weight_block_scales", torch.empty(
+            math.ceil(out_features / 128), math.ceil(in_features / 128) * 4, dtype=torch.uint8, device=device))
+        self._scale_dtypes = {"weight_block_scales": torch.float32}
+        self.reset_lora_parameters()
+
+    def _quantize_and_store(self, w: Tensor, global_amax: Optional[Tensor] = None) -> None:
+        fp8_w, scales = Q.block_fp8_quantize_gkn(w.float().contiguous(), self.quant_group_size)
+        self._write_packed_weight(self._to_uint8(fp8_w))
+        self._scale_dtypes = {"weight_block_scales": scales.dtype}
+        self.weight_block_scales = self._to_uint8(scales)
+        self._aqn_step_cache = None
+
+    def _quant_weight(self) -> QuantWeight:
+        return QuantWeight("block_fp8", _C.XQ_LAYOUT_FLAT, self._read_packed_weight_uint8(),
+                           self.weight_block_scales, torch.float32, self.out_features, self.in_features, 128)
+
+    @torch.compiler.disable
+    def _dequantize_weight(self) -> Tensor:
+        """fp32 [out, in], as block_fp8_dequantize_gkn returns it (callers cast to bf16)."""
+        fp8 = self._read_packed_weight_uint8().view(torch.float8_e4m3fn).reshape(self.out_features, self.in_features)
+        scales = self._recover_tensor(self.weight_block_scales, self._scale_dtypes["weight_block_scales"])
+        return Q.block_fp8_dequantize_gkn(fp8, scales, self.quant_group_size)
+
+    @torch.compiler.disable
+    def _compute_aqn_step(self) -> Tensor:
+        """0.125 * block scale: the e4m3 ulp at unit magnitude (block_fp8_linear.py:102-109)."""
+        s = self._recover_tensor(self.weight_block_scales, self._scale_dtypes["weight_block_scales"]).float()
+        step = s.repeat_interleave(128, 0).repeat_interleave(128, 1)[: self.out_features, : self.in_features]
+        return (0.125 * step).contiguous()
+
+    def _load_prequantized(self, _load_tensor) -> None:
+        """HF fp8 checkpoints: `{m}.weight` (e4m3) + `{m}.weight_scale_inv` (fp32)."""
+        if self._merge_sources is not None:
+            parts = [(f"{self._source_fqn}.{p}") for p in self._merge_sources]
+            packed = torch.cat([_load_tensor(f"{q}.weight") for q in parts], 0)
+            scales = torch.cat([_load_tensor(f"{q}.weight_scale_inv") for q in parts], 0)
+        else:
+            packed = _load_tensor(f"{self._source_fqn}.weight")
+            scales = _load_tensor(f"{self._source_fqn}.weight_scale_inv")
+        dev = self.lora_A.device if self.lora_A.device.type != "meta" else torch.device("cuda")
+        self._write_packed_weight(self._to_uint8(packed).to(dev))
+        self._scale_dtypes = {"weight_block_scales": torch.float32}
+        self.weight_block_scales = self._to_uint8(scales.float()).to(dev)
+        self._ema_amax = None
+        self._aqn_step_cache = None
+
+
+# =============================================================================
+class NvFP4QLoRALinear(QLoRALinear):
+    """e2m1 codes, per-16 e4m3 block scales, fp32 global scale (nvfp4_linear.py:14-175)."""
+
+    def __init__(self, in_features: int, out_features: int, r: int = 16, lora_alpha: int = 16, bias: bool = False,
+                 device: Optional[torch.device] = None, enable_aqn: bool = False, aqn_alpha: float = 1.0):
+        super().__init__(in_features, out_features, r=r, lora_alpha=lora_alpha, quant_format="nvfp4",
+                         quant_group_size=16, bias=bias, device=device, enable_aqn=enable_aqn, aqn_alpha=aqn_alpha)
+        if in_features % 16:
+            raise ValueError(f"nvfp4 needs in_features % 16 == 0, got {in_features}")
+        self.packed_weight_f32 = nn.Parameter(
+            torch.empty(out_features, in_features // 8, dtype=torch.float32, device=device), requires_grad=False)
+        self.register_buffer("weight_block_scales", torch.empty(
+            out_features, (in_features // 16) * 4, dtype=torch.uint8, device=device))
+        self.register_buffer("weight_global_scale", torch.empty(4, dtype=torch.uint8, device=device))
+        self._scale_dtypes = {"weight_block_scales": torch.float32, "weight_global_scale": torch.float32}
+        self.reset_lora_parameters()
+
+    def _init_from_weight(self, w: Tensor) -> None:
+        self._ema_amax = w.float().abs().max().reshape(1).to(w.device)
+        self._quantize_and_store(w, global_amax=self._ema_amax)
+
+    def _quantize_and_store(self, w: Tensor, global_amax: Optional[Tensor] = None) -> None:
+        packed, block_scales, global_scale = Q.nvfp4_quantize(w, self.quant_group_size, global_amax=global_amax)
+        self._write_packed_weight(self._to_uint8(packed))
+        self._scale_dtypes = {"weight_block_scales": block_scales.dtype, "weight_global_scale": global_scale.dtype}
+        self.weight_block_scales = self._to_uint8(block_scales)
+        self.weight_global_scale = self._to_uint8(global_scale)
+        self._aqn_step_cache = None
+
+    def _scales(self) -> Tuple[Tensor, torch.dtype, Tensor]:
+        sdt = self._scale_dtypes["weight_block_scales"]
+        g = self._recover_tensor(self.weight_global_scale, self._scale_dtypes["weight_global_scale"]).float()
+        return self.weight_block_scales, sdt, g
+
+    def _quant_weight(self) -> QuantWeight:
+        s, sdt, g = self._scales()
+        return QuantWeight("nvfp4", _C.XQ_LAYOUT_FLAT, self._read_packed_weight_uint8(), s, sdt,
+                           self.out_features, self.in_features, 16, global_scale=g)
+
+    @torch.compiler.disable
+    def _dequantize_weight(self) -> Tensor:
+        s, sdt, g = self._scales()
+        n = self.out_features * self.in_features
+        w = Q.nvfp4_dequantize(self._read_packed_weight_uint8(), self._recover_tensor(s, sdt), g, n, 16)
+        return w.reshape(self.out_features, self.in_features)
+
+    @torch.compiler.disable
+    def _compute_aqn_step(self) -> Tensor:
+        """0.5 * block scale * global scale: the smallest e2m1 step (nvfp4_linear.py:115-124)."""
+        s, sdt, g = self._scales()
+        eff = self._recover_tensor(s, sdt).float() * g
+        return (0.5 * eff.reshape(self.out_features, -1).repeat_interleave(16, 1)).contiguous()
+
+    def _requantize_merged(self, merged: Tensor, ema_decay: float) -> None:
+        fresh = merged.float().abs().max().reshape(1)
+        if self._ema_amax is not None:
+            self._ema_amax.lerp_(fresh.to(self._ema_amax.device), ema_decay)
+        else:
+            self._ema_amax = fresh
+        self._quantize_and_store(merged, global_amax=self._ema_amax)
+
+    def _load_prequantized(self, _load_tensor) -> None:
+        """modelopt nvfp4 checkpoints: `.weight`, `.weight_scale` (e4m3), `.weight_scale_2` (fp32);
+        the global scale is folded into fp32 block scales and stored as 1.0."""
+        srcs = ([f"{self._source_fqn}.{p}" for p in self._merge_sources]
+                if self._merge_sources is not None else [self._source_fqn])
+        packed, scales, amaxes = [], [], []
+        for q in srcs:
+            g = _load_tensor(f"{q}.weight_scale_2").float()
+            packed.append(_load_tensor(f"{q}.weight"))
+            scales.append(_load_tensor(f"{q}.weight_scale").float() * g)
+            amaxes.append(g.item() * 6.0 * 448.0)
+        dev = self.lora_A.device if self.lora_A.device.type != "meta" else torch.device("cuda")
+        self._write_packed_weight(self._to_uint8(torch.cat(packed, 0)).to(dev))
+        self._scale_dtypes = {"weight_block_scales": torch.float32, "weight_global_scale": torch.float32}
+        self.weight_block_scales = self._to_uint8(torch.cat(scales, 0)).to(dev)
+        self.weight_global_scale = self._to_uint8(torch.tensor([1.0], dtype=torch.float32)).to(dev)
+        self._ema_amax = torch.tensor([max(amaxes)], dtype=torch.float32, device=dev)
+        self._aqn_step_cache = None
+
+
+# =============================================================================
+class Int4QLoRALinear(QLoRALinear):
+    """Group-scaled int4: w = (nib - 8) * scale, one scale per `quant_group_size`
+    consecutive input features; scales bf16 (symmetric absmax/7 rule) or fp32
+    (the reference codec's amax*2/15 rule)."""
+
+    def __init__(self, in_features: int, out_features: int, r: int = 16, lora_alpha: int = 16, bias: bool = False,
+                 device: Optional[torch.device] = None, enable_aqn: bool = False, aqn_alpha: float = 1.0,
+                 quant_group_size: int = 128, symmetric: bool = True):
+        super().__init__(in_features, out_features, r=r, lora_alpha=lora_alpha, quant_format="int4",
+                         quant_group_size=quant_group_size, bias=bias, device=device, enable_aqn=enable_aqn,
+                         aqn_alpha=aqn_alpha)
+        if in_features % quant_group_size or in_features % 8:
+            raise ValueError(f"int4 needs in_features divisible by 8 and by the group size {quant_group_size}")
+        self.symmetric = symmetric
+        self.packed_weight_f32 = nn.Parameter(
+            torch.empty(out_features, in_features // 8, dtype=torch.float32, device=device), requires_grad=False)
+        sdt = torch.bfloat16 if symmetric else torch.float32
+        nbytes = (in_features // quant_group_size) * (2 if symmetric else 4)
+        self.register_buffer("weight_scales", torch.empty(out_features, nbytes, dtype=torch.uint8, device=device))
+        self._scale_dtypes = {"weight_scales": sdt}
+        self.reset_lora_parameters()
+
+    @classmethod
+    def from_module(cls, module: nn.Module, r: int = 16, lora_alpha: int = 16, **kwargs) -> "Int4QLoRALinear":
+        q = cls(in_features=module.in_features, out_features=module.out_features, r=r, lora_alpha=lora_alpha,
+                bias=module.bias is not None, device=module.weight.device,
+                quant_group_size=kwargs.get("quant_group_size", 128), symmetric=kwargs.get("symmetric", True),
+                enable_aqn=kwargs.get("enable_aqn", False), aqn_alpha=kwargs.get("aqn_alpha", 1.0))
+        if module.bias is not None:
+            with torch.no_grad():
+                q.bias.copy_(module.bias.detach())
+        q._quantize_and_store(module.weight.detach())
+        return q
+
+    def _quantize_and_store(self, w: Tensor, global_amax: Optional[Tensor] = None) -> None:
+        fn = Q.int4_quantize_sym if self.symmetric else Q.int4_quantize
+        packed, scales = fn(w.float(), self.quant_group_size)
+        self._write_packed_weight(self._to_uint8(packed))
+        self._scale_dtypes = {"weight_scales": scales.dtype}
+        self.weight_scales = self._to_uint8(scales)
+        self._aqn_step_cache = None
+
+    def _quant_weight(self) -> QuantWeight:
+        return QuantWeight("int4", _C.XQ_LAYOUT_FLAT, self._read_packed_weight_uint8(), self.weight_scales,
+                           self._scale_dtypes["weight_scales"], self.out_features, self.in_features,
+                           self.quant_group_size)
+
+    @torch.compiler.disable
+    def _dequantize_weight(self) -> Tensor:
+        s = self._recover_tensor(self.weight_scales, self._scale_dtypes["weight_scales"])
+        return Q.int4_dequantize(self._read_packed_weight_uint8(), s, self.out_features, self.in_features,
+                                 self.quant_group_size)
+
+    @torch.compiler.disable
+    def _compute_aqn_step(self) -> Tensor:
+        s = self._recover_tensor(self.weight_scales, self._scale_dtypes["weight_scales"]).float()
+        return (0.5 * s.repeat_interleave(self.quant_group_size, 1)).contiguous()
+
+
+# =============================================================================
+def deregister_qlora_weights_from_fsdp(model: nn.Module, param_names: tuple = ("weight",)) -> int:
+    """Drop QLoRALinear parameters from FSDP2 parameter groups so no mixed
+    precision cast ever touches the packed bytes; they stay sharded DTensors
+    and forward gathers them in fp32 (qlora/utils.py:490-542)."""
+    wanted = set(param_names)
+    ours = {id(m) for m in model.modules() if isinstance(m, QLoRALinear)}
+    removed = 0
+    for m in model.modules():
+        get_state = getattr(m, "_get_fsdp_state", None)
+        if get_state is None:
+            continue
+        try:
+            group = get_state()._fsdp_param_group
+        except Exception:
+            continue
+        if group is None:
+            continue
+        drop = [fp for fp in group.fsdp_params
+                if hasattr(fp, "_module_info") and fp._module_info.param_name in wanted
+                and id(fp._module_info.module) in ours]
+        for fp in drop:
+            group.fsdp_params.remove(fp)
+            removed += 1
+    return removed

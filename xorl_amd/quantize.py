@@ -1,0 +1,200 @@
+"""Codec functions with the names and signatures of ``xorl.ops.quantize``.
+
+Dequantizers launch the HIP decode kernels (``xq_decode``); they are bit-exact
+with the reference's Triton decoders.  Quantizers run once at load / merge
+time, are plain torch ops (IEEE fp32) on whatever device the tensor lives on,
+and restate the reference quantizers' arithmetic:
+
+  int4_quantize[_gkn]        ops/quantize/int4_quantize.py:97-110, int4_gkn_quantize.py:137-173
+  int4_quantize_sym          the symmetric absmax/7 bf16-scale rule (not in the reference)
+  nvfp4_quantize[_gkn]       ops/quantize/nvfp4_quantize.py:114-154, nvfp4_gkn_quantize.py:176-235
+  block_fp8_quantize_gkn     ops/quantize/block_fp8_gkn_quantize.py:73-121
+"""
+
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+from torch import Tensor
+
+from . import _C
+
+
+FP4_E2M1_MAX = 6.0
+FP8_E4M3_MAX = 448.0
+
+
+# ---------------------------------------------------------------------------
+# decode (HIP)
+# ---------------------------------------------------------------------------
+def _decode(w: _C.XqWeight, out: Tensor, out_dtype: int) -> Tensor:
+    import ctypes
+
+    _C.check(_C.lib().xq_decode(ctypes.byref(w), out.data_ptr(), out_dtype, _C.stream_ptr(out.device)))
+    return out
+
+
+def int4_dequantize(packed: Tensor, scales: Tensor, M: int, K: int, group_size: int = -1,
+                    out_dtype: torch.dtype = torch.bfloat16) -> Tensor:
+    """[M, K/2] u8 + [M, K/gs] scales (fp32 or bf16) -> [M, K] bf16."""
+    gs = K if group_size == -1 else group_size
+    w = _C.make_weight("int4", _C.XQ_LAYOUT_FLAT, packed, scales, scales.dtype, M, K, gs)
+    out = _decode(w, torch.empty(M, K, dtype=torch.bfloat16, device=packed.device), _C.XQ_DT_BF16)
+    return out if out_dtype == torch.bfloat16 else out.to(out_dtype)
+
+
+def int4_dequantize_gkn(packed: Tensor, scales: Tensor, K: int, N: int, group_size: int = -1,
+                        out_dtype: torch.dtype = torch.bfloat16) -> Tensor:
+    """[K/2, N] u8 + [K/gs, N] scales -> [K, N] bf16 (groups and nibble pairs along K)."""
+    gs = K if group_size == -1 else group_size
+    w = _C.make_weight("int4", _C.XQ_LAYOUT_GKN, packed, scales, scales.dtype, K, N, gs)
+    out = _decode(w, torch.empty(K, N, dtype=torch.bfloat16, device=packed.device), _C.XQ_DT_BF16)
+    return out if out_dtype == torch.bfloat16 else out.to(out_dtype)
+
+
+def nvfp4_dequantize(packed: Tensor, block_scales: Tensor, global_scale: Tensor, num_elements: int,
+                     block_size: int = 16) -> Tensor:
+    """Flat decode of `num_elements` values -> 1-D bf16 (caller reshapes)."""
+    assert num_elements % block_size == 0
+    gs = global_scale.reshape(1) if global_scale.numel() == 1 else global_scale
+    w = _C.make_weight("nvfp4", _C.XQ_LAYOUT_FLAT, packed, block_scales, block_scales.dtype,
+                       1, num_elements, block_size, global_scale=gs.float())
+    return _decode(w, torch.empty(num_elements, dtype=torch.bfloat16, device=packed.device), _C.XQ_DT_BF16)
+
+
+def nvfp4_dequantize_gkn(packed: Tensor, block_scales: Tensor, global_scale: Tensor, K: int, N: int,
+                         block_size: int = 16) -> Tensor:
+    gs = global_scale.reshape(1) if global_scale.numel() == 1 else global_scale
+    w = _C.make_weight("nvfp4", _C.XQ_LAYOUT_GKN, packed, block_scales, block_scales.dtype,
+                       K, N, block_size, global_scale=gs.float())
+    return _decode(w, torch.empty(K, N, dtype=torch.bfloat16, device=packed.device), _C.XQ_DT_BF16)
+
+
+def block_fp8_dequantize_gkn(x: Tensor, s: Tensor, block_size: int = 128,
+                             out_dtype: Optional[torch.dtype] = None) -> Tensor:
+    """e4m3 [R, C] * fp32 scale [ceil(R/128), ceil(C/128)].  Like the reference
+    the result is fp32 (the default dtype) unless out_dtype=torch.bfloat16,
+    which fuses the `.to(bf16)` every caller applies."""
+    assert x.dim() == 2 and s.dim() == 2 and x.is_contiguous() and s.is_contiguous()
+    R, Cc = x.shape
+    dt = out_dtype or torch.float32
+    w = _C.make_weight("block_fp8", _C.XQ_LAYOUT_FLAT, x, s, torch.float32, R, Cc, block_size)
+    out = torch.empty(R, Cc, dtype=dt, device=x.device)
+    return _decode(w, out, _C.XQ_DT_F32 if dt == torch.float32 else _C.XQ_DT_BF16)
+
+
+# ---------------------------------------------------------------------------
+# quantizers (torch, load-time)
+# ---------------------------------------------------------------------------
+def _pack_nibbles_last(q: Tensor) -> Tensor:
+    """[..., 2n] codes -> [..., n] bytes, even element in the low nibble."""
+    q = q.to(torch.uint8)
+    return q[..., 0::2] | (q[..., 1::2] << 4)
+
+
+def _pack_nibbles_first(q: Tensor) -> Tensor:
+    """[2k, N] codes -> [k, N] bytes, even K-row in the low nibble."""
+    q = q.to(torch.uint8)
+    return q[0::2] | (q[1::2] << 4)
+
+
+def int4_quantize(x: Tensor, group_size: int = -1) -> Tuple[Tensor, Tensor]:
+    assert x.dim() == 2
+    M, K = x.shape
+    gs = K if group_size == -1 else group_size
+    assert K % gs == 0 and gs % 2 == 0
+    xf = x.float().reshape(M, K // gs, gs)
+    scale = xf.abs().amax(-1).clamp_min(1e-12) * torch.tensor(2.0 / 15.0, dtype=torch.float32, device=x.device)
+    inv = 1.0 / scale
+    q = (xf * inv.unsqueeze(-1) + 8.5).to(torch.int32).clamp_(0, 15)
+    return _pack_nibbles_last(q.reshape(M, K)), scale
+
+
+def int4_quantize_gkn(x: Tensor, group_size: int = -1) -> Tuple[Tensor, Tensor]:
+    assert x.dim() == 2
+    K, N = x.shape
+    gs = K if group_size == -1 else group_size
+    assert K % gs == 0 and gs % 2 == 0
+    xf = x.float().reshape(K // gs, gs, N)
+    scale = xf.abs().amax(1).clamp_min(1e-12) * torch.tensor(2.0 / 15.0, dtype=torch.float32, device=x.device)
+    inv = 1.0 / scale
+    q = (xf * inv.unsqueeze(1) + 8.5).to(torch.int32).clamp_(0, 15)
+    return _pack_nibbles_first(q.reshape(K, N)), scale
+
+
+def int4_quantize_sym(x: Tensor, group_size: int = 128) -> Tuple[Tensor, Tensor]:
+    """Symmetric int4: scale = bf16(absmax/7), q = clamp(rne(w/scale), -7, 7) + 8."""
+    M, K = x.shape
+    assert K % group_size == 0
+    xf = x.float().reshape(M, K // group_size, group_size)
+    scale = (xf.abs().amax(-1) / 7.0).to(torch.bfloat16)
+    sf = scale.float().unsqueeze(-1)
+    q = torch.where(sf > 0, torch.round(xf / sf).clamp_(-7, 7), torch.zeros_like(xf)).to(torch.int32) + 8
+    return _pack_nibbles_last(q.reshape(M, K)), scale
+
+
+def _fp4_encode(v: Tensor) -> Tensor:
+    """ops/quantize/fp4_codec.py:12-19 (ties up in magnitude)."""
+    sign = (v < 0).to(torch.int32) * 8
+    a = v.abs()
+    lo = (a * 2.0 + 0.5).to(torch.int32).clamp_max(3)
+    hi = 4 + (a >= 2.5).to(torch.int32) + (a >= 3.5).to(torch.int32) + (a >= 5.0).to(torch.int32)
+    return torch.where(a >= 1.75, hi, lo) + sign
+
+
+def _e4m3_satfinite(t: Tensor) -> Tensor:
+    return t.clamp(-FP8_E4M3_MAX, FP8_E4M3_MAX).to(torch.float8_e4m3fn)
+
+
+def _nvfp4_scales(amax: Tensor, global_amax: Optional[Tensor]):
+    gamax = amax.max().reshape(1) if global_amax is None else global_amax.float().reshape(1).to(amax.device)
+    gamax = gamax.clamp_min(1e-12)
+    block_scales = _e4m3_satfinite(amax / gamax * FP8_E4M3_MAX)
+    global_scale = gamax * torch.tensor(1.0 / FP4_E2M1_MAX, dtype=torch.float32, device=amax.device) / FP8_E4M3_MAX
+    return block_scales, global_scale
+
+
+def nvfp4_quantize(x: Tensor, block_size: int = 16, global_amax: Optional[Tensor] = None):
+    """-> packed u8 [n/2] (flat), e4m3 block scales [n/block], global scale fp32 [1]."""
+    assert x.dim() == 2
+    n = x.numel()
+    assert n % block_size == 0 and block_size % 2 == 0
+    xf = x.float().reshape(-1, block_size)
+    amax = xf.abs().amax(-1).clamp_min(1e-12)
+    scaled = (xf * (6.0 / amax).unsqueeze(-1)).clamp_(-6.0, 6.0)
+    packed = _pack_nibbles_last(_fp4_encode(scaled).reshape(-1))
+    block_scales, global_scale = _nvfp4_scales(amax, global_amax)
+    return packed, block_scales, global_scale
+
+
+def nvfp4_quantize_gkn(x: Tensor, block_size: int = 16, global_amax: Optional[Tensor] = None):
+    """[K, N] -> packed [K/2, N], e4m3 block scales [K/block, N], global [1]."""
+    assert x.dim() == 2
+    K, N = x.shape
+    assert K % block_size == 0 and block_size % 2 == 0
+    xf = x.float().reshape(K // block_size, block_size, N)
+    amax = xf.abs().amax(1).clamp_min(1e-12)
+    scaled = (xf * (6.0 / amax).unsqueeze(1)).clamp_(-6.0, 6.0)
+    packed = _pack_nibbles_first(_fp4_encode(scaled).reshape(K, N))
+    block_scales, global_scale = _nvfp4_scales(amax.reshape(-1), global_amax)
+    return packed, block_scales.reshape(K // block_size, N), global_scale
+
+
+def block_fp8_quantize_gkn(x: Tensor, block_size: int = 128, amax_scale: float = 1.0):
+    """[R, C] -> e4m3 [R, C], fp32 scales [ceil(R/bs), ceil(C/bs)] (edge tiles partial)."""
+    assert x.is_contiguous() and x.dim() == 2
+    if amax_scale <= 0.0:
+        raise ValueError(f"amax_scale must be positive, got {amax_scale}")
+    R, Cc = x.shape
+    bs = block_size
+    pr, pc = (-R) % bs, (-Cc) % bs
+    xf = x.float()
+    if pr or pc:
+        xf = torch.nn.functional.pad(xf, (0, pc, 0, pr))
+    nr, nc = xf.shape[0] // bs, xf.shape[1] // bs
+    blocks = xf.reshape(nr, bs, nc, bs)
+    s = (blocks.abs().amax(dim=(1, 3)) * amax_scale / FP8_E4M3_MAX).clamp_min(1e-12)
+    y = (blocks / s[:, None, :, None]).clamp_(-FP8_E4M3_MAX, FP8_E4M3_MAX).to(torch.float8_e4m3fn)
+    y = y.reshape(nr * bs, nc * bs)[:R, :Cc].contiguous()
+    return y, s
