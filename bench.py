@@ -1,0 +1,180 @@
+#!/usr/bin/env python3
+"""Benchmark of the QLoRA quantized base-linear hot path on one MI355X.
+
+Workload (BASELINE.json configs[1]): block_fp8 QLoRA on the Qwen3-8B MLP --
+M = 8192 tokens, hidden 4096, intermediate 12288, gate/up [12288, 4096] and
+down [4096, 12288] quantized to e4m3 with 128x128 fp32 block scales, LoRA
+r = 32 on all three projections, SwiGLU in between, full forward + backward.
+One "step" is one forward + backward of that MLP on synthetic inputs that are
+resident in HBM before the timed region starts.
+
+Prints ONE JSON line (see the keys at the bottom).  `value` is algorithmic
+TFLOP/s of the whole step (4MKN + 6Mr(K+N) per projection); `roofline` is the
+fused dequant-GEMM kernel alone, timed per launch with HIP events on the launch
+stream; `cpu_baseline` is the reference recipe (decode -> bf16 F.linear -> fp32
+LoRA -> autograd) on the host cores over a bounded row sample.
+"""
+
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+METRIC = "QLoRA dequant-GEMM+LoRA fwd/bwd TFLOP/s & % MFMA/HBM peak, 1 GPU"
+M, H, I, R, ALPHA = 8192, 4096, 12288, 32, 64
+BF16_MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense bf16, published
+
+
+def step_flops(m: int) -> float:
+    per = lambda K, N: 4.0 * m * K * N + 6.0 * m * R * (K + N)
+    return 2 * per(H, I) + per(I, H)
+
+
+def gen(shape, std, seed, dtype=torch.float32):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * std).to(dtype)
+
+
+def build_modules():
+    """Three BlockFP8QLoRALinear modules built on the CPU (so the CPU baseline can
+    decode the very same bytes)."""
+    from xorl_amd.qlora import QLoRALinear
+
+    mods = {}
+    for i, (name, (N, K)) in enumerate({"gate": (I, H), "up": (I, H), "down": (H, I)}.items()):
+        lin = torch.nn.Linear(K, N, bias=False)
+        with torch.no_grad():
+            lin.weight.copy_(gen((N, K), 0.02, 100 + i))
+        m = QLoRALinear.from_module(lin, r=R, lora_alpha=ALPHA, quant_format="block_fp8")
+        with torch.no_grad():
+            m.lora_A.copy_(gen((R, K), 0.02, 200 + i))
+            m.lora_B.copy_(gen((N, R), 0.02, 300 + i))
+        mods[name] = m
+    return mods
+
+
+def cpu_baseline(mods, rows: int):
+    """Reference recipe on host cores over `rows` tokens of the same workload."""
+    from oracle import decode_np as NP
+    from oracle import recipe as RC
+
+    torch.set_num_threads(os.cpu_count())
+    x = gen((rows, H), 1.0, 1, torch.bfloat16)
+    dy = gen((rows, H), 1.0, 2, torch.bfloat16)
+
+    def run():
+        w = {}
+        for k, m in mods.items():    # the reference decodes every weight in every forward
+            packed = m.packed_weight_f32.detach().contiguous().view(torch.uint8).numpy()
+            s = m.weight_block_scales.contiguous().view(torch.float32).numpy()
+            w[k] = torch.from_numpy(NP.fp8_decode(packed, s, m.out_features, m.in_features)[0])   # fp32, as the reference
+        xx = x.clone().requires_grad_(True)
+        P = {k: (m.lora_A.detach().clone().requires_grad_(True), m.lora_B.detach().clone().requires_grad_(True))
+             for k, m in mods.items()}
+        g = RC.linear_forward_recipe(xx, w["gate"], *P["gate"], ALPHA / R)
+        u = RC.linear_forward_recipe(xx, w["up"], *P["up"], ALPHA / R)
+        h = RC.silu_and_mul_recipe(g, u)
+        y = RC.linear_forward_recipe(h, w["down"], *P["down"], ALPHA / R)
+        y.backward(dy)
+        return y
+
+    t0 = time.perf_counter()
+    run()
+    dt = time.perf_counter() - t0
+    return {
+        "value": step_flops(rows) / dt / 1e12,
+        "unit": "TFLOP/s",
+        "cores": os.cpu_count(),
+        "kind": "port",
+        "sample": f"{rows} of {M} token rows of the same MLP, decode+fwd+bwd, torch CPU ops on the oracle decode, "
+                  f"{dt:.1f} s",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--cpu-rows", type=int, default=256, help="token rows of the CPU baseline sample (0 = skip)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs the QLoRA path on ONE GPU; --gpus must be 1 "
+                 "(no collectives or sharding are part of it)")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no HIP device visible")
+
+    from xorl_amd import _C
+    from xorl_amd.functional import silu_and_mul
+
+    dev = torch.device("cuda:0")
+    mods_cpu = build_modules()
+    cpu = cpu_baseline(mods_cpu, args.cpu_rows) if args.cpu_rows > 0 else None
+    mods = {k: m.to(dev) for k, m in mods_cpu.items()}
+    x = gen((M, H), 1.0, 1, torch.bfloat16).to(dev).requires_grad_(True)
+    dy = gen((M, H), 1.0, 2, torch.bfloat16).to(dev)
+    params = [p for m in mods.values() for p in (m.lora_A, m.lora_B)]
+
+    def step():
+        x.grad = None
+        for p in params:
+            p.grad = None
+        g = mods["gate"](x)
+        u = mods["up"](x)
+        h = silu_and_mul(g, u)
+        y = mods["down"](h)
+        y.backward(dy)
+
+    L = _C.lib()
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    L.xq_profile_enable(1)
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    n, ms, fl = ctypes.c_int(0), ctypes.c_double(0), ctypes.c_double(0)
+    _C.check(L.xq_profile_collect(ctypes.byref(n), ctypes.byref(ms), ctypes.byref(fl)))
+    L.xq_profile_enable(0)
+
+    ms_per_step = dt / args.steps * 1e3
+    value = step_flops(M) / (dt / args.steps) / 1e12
+    achieved = fl.value / (ms.value * 1e-3) / 1e12 if ms.value > 0 else 0.0
+    out = {
+        "metric": METRIC,
+        "value": value,
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "configs[1]: block_fp8 QLoRA Qwen3-8B MLP fwd+bwd, M=8192, hidden 4096, "
+                               "intermediate 12288, LoRA r=32 on gate/up/down, SwiGLU",
+                   "tokens": M, "hidden": H, "intermediate": I, "lora_r": R, "format": "block_fp8"},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": BF16_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": achieved / BF16_MFMA_PEAK_TFLOPS, "traffic": None,
+                     "kernel": "gemm_tile_kernel<fp8> (fused dequant-GEMM, fwd and dgrad launches)",
+                     "launches": n.value, "avg_launch_ms": ms.value / max(n.value, 1)},
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -76,6 +76,15 @@ typedef struct xq_weight {
 const char* xq_version(void);
 const char* xq_last_error(void);
 
+/* Per-launch timing of the fused dequant-GEMM kernel (the dominant kernel)
+ * with HIP events on the launch stream; used by the benchmark's roofline
+ * figure.  No counterpart in the reference.  xq_profile_enable(1) starts
+ * recording (at most 8192 launches), xq_profile_collect waits for the
+ * recorded launches and returns their count, summed duration and summed
+ * algorithmic FLOPs (2*rows*Nout*(Kc + r_pad) each), then resets. */
+int xq_profile_enable(int on);
+int xq_profile_collect(int* n_launches, double* total_ms, double* total_flops);
+
 /* ---- decode ------------------------------------------------------------
  * out[e] = decoded weight of expert e, shape [rows, cols], bf16 or fp32.
  * Replaces int4_dequantize / int4_dequantize_gkn

@@ -51,6 +51,8 @@ _W = ctypes.POINTER(XqWeight)
 
 _INT = ctypes.c_int
 _SIGNATURES = {
+    "xq_profile_enable": (_INT, [_INT]),
+    "xq_profile_collect": (_INT, [_P, _P, _P]),
     "xq_decode": (_INT, [_W, _P, _INT, _P]),
     "xq_linear_workspace_bytes": (_I64, [_I64, _I64, _I64, _INT]),
     # w, x, ldx, M, A, B, lora_dtype, r, scaling, bias, y, ldy, su_out, ws, ws_bytes, stream

@@ -59,3 +59,58 @@ int xq_validate_weight(const xq_weight* w, const char* who) {
     }
     return XQ_OK;
 }
+
+// ---------------------------------------------------------------- launch timing
+// Optional per-launch timing of the fused dequant-GEMM kernel with HIP events
+// recorded on the launch stream.  Off by default; the benchmark turns it on for
+// its timed region.  Events are created once (no device memory is allocated).
+namespace {
+constexpr int kMaxProfiled = 8192;
+struct ProfileState {
+    bool enabled = false;
+    int count = 0;
+    hipEvent_t start[kMaxProfiled], stop[kMaxProfiled];
+    double flops[kMaxProfiled];
+    int created = 0;
+} g_prof;
+}  // namespace
+
+bool xq_profile_mark_begin(hipStream_t s, double flops) {
+    if (!g_prof.enabled || g_prof.count >= kMaxProfiled) return false;
+    int i = g_prof.count;
+    if (i >= g_prof.created) {
+        if (hipEventCreate(&g_prof.start[i]) != hipSuccess || hipEventCreate(&g_prof.stop[i]) != hipSuccess) return false;
+        g_prof.created = i + 1;
+    }
+    g_prof.flops[i] = flops;
+    return hipEventRecord(g_prof.start[i], s) == hipSuccess;
+}
+void xq_profile_mark_end(hipStream_t s) {
+    hipEventRecord(g_prof.stop[g_prof.count], s);
+    ++g_prof.count;
+}
+
+extern "C" int xq_profile_enable(int on) {
+    g_prof.enabled = on != 0;
+    g_prof.count = 0;
+    return XQ_OK;
+}
+
+extern "C" int xq_profile_collect(int* n_launches, double* total_ms, double* total_flops) {
+    double ms = 0.0, fl = 0.0;
+    for (int i = 0; i < g_prof.count; ++i) {
+        if (hipEventSynchronize(g_prof.stop[i]) != hipSuccess) {
+            xq_set_error("xq_profile_collect: event synchronize failed");
+            return XQ_ERR_LAUNCH;
+        }
+        float t = 0.0f;
+        hipEventElapsedTime(&t, g_prof.start[i], g_prof.stop[i]);
+        ms += t;
+        fl += g_prof.flops[i];
+    }
+    if (n_launches) *n_launches = g_prof.count;
+    if (total_ms) *total_ms = ms;
+    if (total_flops) *total_flops = fl;
+    g_prof.count = 0;
+    return XQ_OK;
+}

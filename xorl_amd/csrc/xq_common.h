@@ -27,6 +27,8 @@ void xq_set_error(const char* fmt, ...);
     } while (0)
 
 int xq_validate_weight(const xq_weight* w, const char* who);
+bool xq_profile_mark_begin(hipStream_t s, double flops);
+void xq_profile_mark_end(hipStream_t s);
 int64_t xq_packed_bytes_per_expert(const xq_weight* w);
 int64_t xq_scale_bytes_per_expert(const xq_weight* w);
 

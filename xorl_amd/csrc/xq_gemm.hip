@@ -39,11 +39,13 @@ int launch_tile_gemm(const xq_weight* w, bool contract_cols, const bf16_t* A, in
     if (n_rows == 0) return XQ_OK;
     unsigned mt = (unsigned)(xq_cdiv(n_rows, BM) + (offsets ? w->num_experts : 0));
     dim3 grid(mt, (unsigned)xq_cdiv(g.Nout, BN));
+    const bool timed = xq_profile_mark_begin(stream, 2.0 * (double)n_rows * g.Nout * ((double)g.Kc + g.r_pad));
     if (w->format == XQ_FMT_FP8) launch_tile_cc<XQ_FMT_FP8, XQ_LAYOUT_FLAT>(g, contract_cols, grid, stream);
     else if (w->format == XQ_FMT_INT4 && w->layout == XQ_LAYOUT_FLAT) launch_tile_cc<XQ_FMT_INT4, XQ_LAYOUT_FLAT>(g, contract_cols, grid, stream);
     else if (w->format == XQ_FMT_INT4) launch_tile_cc<XQ_FMT_INT4, XQ_LAYOUT_GKN>(g, contract_cols, grid, stream);
     else if (w->layout == XQ_LAYOUT_FLAT) launch_tile_cc<XQ_FMT_NVFP4, XQ_LAYOUT_FLAT>(g, contract_cols, grid, stream);
     else launch_tile_cc<XQ_FMT_NVFP4, XQ_LAYOUT_GKN>(g, contract_cols, grid, stream);
+    if (timed) xq_profile_mark_end(stream);
     XQ_CHECK_LAUNCH(who);
     return XQ_OK;
 }
