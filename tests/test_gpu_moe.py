@@ -1,0 +1,132 @@
+"""GPU parity: routing kernels (bit-exact vs the oracle's stable sort) and the grouped
+routed QLoRA expert MLP (forward + backward) vs the float64 per-expert oracle program."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import cdecode as C
+from oracle import decode_np as NP
+from oracle import recipe as R
+from tests.util_cases import bits_to_bf16, gen
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-2
+
+
+def _zipf_routing(T, E, topk, seed, empty=1):
+    """Seeded logits: Zipf(1.1) popularity over a permutation of experts, the last `empty` never chosen."""
+    g = torch.Generator().manual_seed(seed)
+    perm = torch.randperm(E, generator=g)
+    pmf = 1.0 / torch.arange(1, E + 1, dtype=torch.float64) ** 1.1
+    logits = torch.log(pmf / pmf.sum())[perm.argsort()].float()
+    gumbel = -torch.log(-torch.log(torch.rand(T, E, generator=g).clamp_min(1e-9)))
+    z = logits[None, :] + gumbel
+    if empty:
+        z[:, perm[-empty:]] = -1e9
+    rw, sel = torch.topk(torch.softmax(z, -1), topk, dim=-1)
+    rw = rw / rw.sum(-1, keepdim=True)
+    return rw, sel.int()
+
+
+@pytest.mark.parametrize("T,E,topk", [(64, 8, 2), (1000, 128, 8), (5, 4, 1), (16384, 128, 8)])
+def test_route_scatter_gather_exact(hip_device, T, E, topk):
+    from xorl_amd import moe_functional as MF
+
+    rw, sel = _zipf_routing(T, E, topk, seed=T)
+    splits, sidx_ref = R.route_build(sel, E)
+    counts, offsets, sidx, tile_offsets = MF.route_build(sel.to(hip_device), E)
+    assert torch.equal(counts.cpu().long(), splits)
+    assert torch.equal(sidx.cpu().view(T, topk), sidx_ref)
+    assert torch.equal(offsets.cpu().long(), torch.cat([torch.zeros(1, dtype=torch.long), splits.cumsum(0)]))
+    tiles = (splits + 127) // 128
+    assert torch.equal(tile_offsets.cpu().long(), torch.cat([torch.zeros(1, dtype=torch.long), tiles.cumsum(0)]))
+    assert (splits == 0).any() or E <= 4
+    # scatter then gather: out[t] = sum_j x[t] = topk * x[t] (exact in bf16 for power-of-two topk)
+    x = gen((T, 64), 1.0, 3, torch.bfloat16).to(hip_device)
+    xs = MF.moe_scatter(x, sidx, topk)
+    ref = torch.empty(T * topk, 64, dtype=torch.bfloat16)
+    ref[sidx_ref.flatten().long()] = x.cpu().repeat_interleave(topk, 0)
+    assert torch.equal(xs.cpu(), ref)
+    back = MF.moe_gather(xs, None, sidx, T, topk)
+    assert torch.equal(back.cpu(), (x.cpu().float() * topk).to(torch.bfloat16))
+
+
+def _make_experts(fmt, E, H, I, r, hybrid, seed, device):
+    from xorl_amd.qlora import BlockFP8QLoRAMoeExperts, NvFP4QLoRAMoeExperts
+
+    cls = BlockFP8QLoRAMoeExperts if fmt == "block_fp8" else NvFP4QLoRAMoeExperts
+    m = cls(E, E, I, H, r=r, lora_alpha=2 * r, hybrid_shared=hybrid)
+    m.load_weights(gen((E, H, I), 0.05, seed), gen((E, H, I), 0.05, seed + 1), gen((E, I, H), 0.05, seed + 2))
+    with torch.no_grad():
+        for i, name in enumerate(("gate_proj", "up_proj", "down_proj")):
+            A, B = getattr(m, f"{name}_lora_A"), getattr(m, f"{name}_lora_B")
+            A.copy_(gen(tuple(A.shape), 0.05, seed + 10 + i))
+            B.copy_(gen(tuple(B.shape), 0.05, seed + 20 + i))
+    # oracle decode of the banks (CPU)
+    banks = {}
+    for p in ("gate", "up", "down"):
+        K, N = m._proj_dims(p)
+        packed = getattr(m, f"{p}_packed").numpy()
+        per = []
+        for e in range(E):
+            if fmt == "block_fp8":
+                s = getattr(m, f"{p}_block_scales")[e].contiguous().view(torch.float32).numpy()
+                per.append(bits_to_bf16(NP.fp8_decode(packed[e].reshape(K, N), s, K, N)[1]))
+            else:
+                sb = getattr(m, f"{p}_block_scales")[e].numpy()
+                g = getattr(m, f"{p}_global_scale")[e].contiguous().view(torch.float32).item()
+                per.append(bits_to_bf16(NP.nvfp4_decode_gkn(packed[e], C.e4m3_scales_to_f32(sb), g, K, N)))
+        banks[p] = torch.stack(per)
+    return m.to(device), banks
+
+
+@pytest.mark.parametrize("fmt", ["block_fp8", "nvfp4"])
+@pytest.mark.parametrize("E,T,H,I,r,topk,hybrid", [(6, 300, 128, 192, 8, 2, True), (16, 700, 256, 128, 16, 4, False)])
+def test_moe_fwd_bwd_vs_oracle(hip_device, fmt, E, T, H, I, r, topk, hybrid):
+    m, banks = _make_experts(fmt, E, H, I, r, hybrid, seed=E + T, device=hip_device)
+    # the module's own bank decode is bit-exact with the oracle
+    for p in ("gate", "up", "down"):
+        K, N = m._proj_dims(p)
+        assert torch.equal(m.dequantize_all_experts(p, K, N).to(torch.bfloat16).cpu(), banks[p]), p
+    rw, sel = _zipf_routing(T, E, topk, seed=7)
+    rw = rw.to(torch.bfloat16)
+    x = gen((T, H), 1.0, 8, torch.bfloat16)
+    dy = gen((T, H), 1.0, 9, torch.bfloat16)
+    xd = x.to(hip_device).requires_grad_(True)
+    rwd = rw.to(hip_device).requires_grad_(True)
+    y = m(xd, rwd, sel.to(hip_device))
+    y.backward(dy.to(hip_device))
+    lora = {k: (getattr(m, f"{k}_proj_lora_A").detach().cpu(), getattr(m, f"{k}_proj_lora_B").detach().cpu())
+            for k in ("gate", "up", "down")}
+    ex = R.moe_fwd_bwd(x, rw, sel, banks["gate"], banks["up"], banks["down"], lora, m.scaling, dy)
+    assert R.max_rel_err(y.cpu(), ex["y"]) <= TOL
+    assert R.max_rel_err(xd.grad.cpu(), ex["dx"]) <= TOL
+    # routing-weight grads pass through bf16 intermediates (ops/moe/lora.py:855-861): 2e-2
+    assert R.max_rel_err(rwd.grad.cpu(), ex["d_routing"]) <= 2e-2
+    for k in ("gate", "up", "down"):
+        gA, gB = getattr(m, f"{k}_proj_lora_A").grad.cpu(), getattr(m, f"{k}_proj_lora_B").grad.cpu()
+        assert gA.shape == lora[k][0].shape and gB.shape == lora[k][1].shape
+        assert R.max_rel_err(gA, ex[f"dA_{k}"]) <= TOL, f"dA_{k}"
+        assert R.max_rel_err(gB, ex[f"dB_{k}"]) <= TOL, f"dB_{k}"
+    # experts without rows: exact-zero factor gradients (structural zeros)
+    empty = (torch.bincount(sel.flatten().long(), minlength=E) == 0).nonzero().flatten()
+    assert empty.numel() >= 1
+    for k in ("gate", "up", "down"):
+        for t in (getattr(m, f"{k}_proj_lora_A").grad, getattr(m, f"{k}_proj_lora_B").grad):
+            if t.shape[0] == E:
+                assert torch.count_nonzero(t[empty.to(t.device)]) == 0
+
+
+def test_moe_zero_lora_equals_base(hip_device):
+    m, banks = _make_experts("block_fp8", 8, 128, 128, 8, True, seed=40, device=hip_device)
+    rw, sel = _zipf_routing(200, 8, 2, seed=41)
+    x = gen((200, 128), 1.0, 42, torch.bfloat16)
+    with torch.no_grad():
+        for k in ("gate", "up", "down"):
+            getattr(m, f"{k}_proj_lora_B").zero_()
+        y = m(x.to(hip_device), rw.to(torch.bfloat16).to(hip_device), sel.to(hip_device))
+    zero = {k: (getattr(m, f"{k}_proj_lora_A").detach().cpu(), getattr(m, f"{k}_proj_lora_B").detach().cpu())
+            for k in ("gate", "up", "down")}
+    ex = R.moe_fwd_bwd(x, rw.to(torch.bfloat16), sel, banks["gate"], banks["up"], banks["down"], zero, m.scaling)
+    assert R.max_rel_err(y.cpu(), ex["y"]) <= TOL

@@ -17,3 +17,7 @@ __all__ = [
     "Int4QLoRALinear",
     "deregister_qlora_weights_from_fsdp",
 ]
+
+from .moe_experts import BlockFP8QLoRAMoeExperts, NvFP4QLoRAMoeExperts, QLoRAMoeExperts  # noqa: E402
+
+__all__ += ["QLoRAMoeExperts", "BlockFP8QLoRAMoeExperts", "NvFP4QLoRAMoeExperts"]

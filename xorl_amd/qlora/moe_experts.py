@@ -1,0 +1,331 @@
+"""QLoRA MoE experts on packed expert banks (drop-in for xorl/qlora/modules/moe_experts.py).
+
+Keeps the reference module's constructor, buffer / parameter names and shapes
+(`{gate,up,down}_packed` uint8 `[E, K(/2), N]`, `{...}_block_scales` uint8 views,
+`{...}_global_scale`, `{gate,up,down}_proj_lora_{A,B}` fp32 in GKN form, the
+hybrid-shared factor layout) and its helper methods.  forward() differs: the
+banks are never dequantized; the grouped kernels decode weight tiles in place.
+Only the local (single-GPU) path exists here: expert parallelism is out of scope.
+"""
+
+from __future__ import annotations
+
+import math
+from typing import Dict, Optional, Tuple
+
+import torch
+import torch.nn as nn
+from torch import Tensor
+
+from .. import _C
+from .. import quantize as Q
+from ..functional import QuantWeight
+from ..moe_functional import moe_experts_qlora_forward
+from .linear import LoraModule
+
+
+EXPERT_PROJECTION_ROLES = frozenset({"gate_proj", "up_proj", "down_proj"})
+
+
+def compute_lora_scaling(lora_alpha: float, r: int, use_rslora: bool = False) -> float:
+    return lora_alpha / math.sqrt(r) if use_rslora else lora_alpha / r
+
+
+class QLoRAMoeExperts(LoraModule, nn.Module):
+    """Base class; use BlockFP8QLoRAMoeExperts or NvFP4QLoRAMoeExperts."""
+
+    adapter_gradient_producer_family = "fused_managed"
+
+    def __init__(self, num_local_experts: int, num_experts: int, intermediate_size: int, hidden_size: int,
+                 r: int = 16, lora_alpha: int = 16, quant_format: str = "nvfp4", quant_group_size: int = 16,
+                 act_fn: Optional[nn.Module] = None, hidden_act: Optional[str] = None, expert_offset: int = 0,
+                 device: Optional[torch.device] = None, moe_implementation: str = "hip", hybrid_shared: bool = True,
+                 use_rslora: bool = False, ep_dispatch: str = "alltoall", deepep_buffer_size_gb: float = 2.0,
+                 deepep_num_sms: int = 20, deepep_async_combine: bool = False,
+                 alltoall_combine_hidden_chunk_size: int = 0, target_modules: Optional[list] = None):
+        if type(self) is QLoRAMoeExperts:
+            raise TypeError("QLoRAMoeExperts is abstract. Use BlockFP8QLoRAMoeExperts or NvFP4QLoRAMoeExperts.")
+        super().__init__()
+        if num_local_experts != num_experts or expert_offset != 0:
+            raise ValueError("this build holds all experts on one GPU (num_local_experts == num_experts, offset 0)")
+        if r <= 0 or r > 64:
+            raise ValueError(f"LoRA rank must be in [1, 64] for the fused kernels, got {r}")
+        self.num_local_experts, self.num_experts = num_local_experts, num_experts
+        self.intermediate_size, self.hidden_size = intermediate_size, hidden_size
+        self.hidden_dim = hidden_size
+        self.r, self.lora_alpha = r, lora_alpha
+        self.active_r, self.active_lora_alpha = r, lora_alpha
+        self.use_rslora = use_rslora
+        self.scaling = compute_lora_scaling(lora_alpha, r, use_rslora)
+        self.quant_format, self.quant_group_size = quant_format, quant_group_size
+        self.act_fn = act_fn or nn.SiLU()
+        if hidden_act is None:
+            plain = act_fn is None or isinstance(act_fn, nn.SiLU) or type(act_fn).__name__ == "SiLUActivation"
+            hidden_act = "silu" if plain else f"custom:{type(act_fn).__qualname__}"
+        if hidden_act != "silu":
+            raise ValueError(f"the fused expert path implements SiLU gating only, got {hidden_act!r}")
+        self.hidden_act = hidden_act
+        self.gated = True
+        self.swiglu_limit = 0.0
+        self.gate_up_bias = None
+        self.down_bias = None
+        self.expert_offset = expert_offset
+        self.moe_implementation = moe_implementation
+        self.hybrid_shared = hybrid_shared
+        targets = tuple(("gate_proj", "up_proj", "down_proj") if target_modules is None else target_modules)
+        if not targets or len(set(targets)) != len(targets) or set(targets) - EXPERT_PROJECTION_ROLES:
+            raise ValueError("QLoRA expert target_modules must be a non-empty subset of "
+                             f"{sorted(EXPERT_PROJECTION_ROLES)}; got {list(targets)!r}")
+        self.target_modules = targets
+        self.ep_dispatch = ep_dispatch
+        self.deepep_buffer_size_gb, self.deepep_num_sms = deepep_buffer_size_gb, deepep_num_sms
+        self.deepep_async_combine = deepep_async_combine
+        self.alltoall_combine_hidden_chunk_size = alltoall_combine_hidden_chunk_size
+        self._source_fqn: Optional[str] = None
+        self._source_quant_format: Optional[str] = None
+        self._weights_loaded = False
+        self._ema_amax: Dict[str, Optional[Tensor]] = {"gate": None, "up": None, "down": None}
+
+        # hybrid-shared layout: gate/up share A across experts, down shares B
+        # (qlora/modules/moe_experts.py:205-238)
+        shared = 1 if hybrid_shared else num_experts
+        self._create_lora_params("gate_proj", shared, num_experts, r, hidden_size, intermediate_size, device)
+        self._create_lora_params("up_proj", shared, num_experts, r, hidden_size, intermediate_size, device)
+        self._create_lora_params("down_proj", num_experts, shared, r, intermediate_size, hidden_size, device)
+        self._scale_dtypes: Dict[str, Dict[str, torch.dtype]] = {"gate": {}, "up": {}, "down": {}}
+        self._skip_fsdp = True
+        self._qlora_expected_skip_keys = {"gate_proj", "up_proj", "down_proj"}
+
+    # ------------------------------------------------------------------ LoRA params
+    def _create_lora_params(self, name, A_experts, B_experts, r, in_features, out_features, device=None):
+        A = torch.empty(A_experts, in_features, r, dtype=torch.float32, device=device)
+        B = torch.empty(B_experts, r, out_features, dtype=torch.float32, device=device)
+        if name in self.target_modules:
+            setattr(self, f"{name}_lora_A", nn.Parameter(A))
+            setattr(self, f"{name}_lora_B", nn.Parameter(B))
+        else:   # untargeted projections carry frozen zero factors
+            self.register_buffer(f"{name}_lora_A", torch.zeros_like(A), persistent=False)
+            self.register_buffer(f"{name}_lora_B", torch.zeros_like(B), persistent=False)
+
+    def reset_lora_parameters(self) -> None:
+        for proj in self.target_modules:
+            A, B = getattr(self, f"{proj}_lora_A"), getattr(self, f"{proj}_lora_B")
+            for i in range(A.shape[0]):
+                nn.init.kaiming_uniform_(A.data[i], a=math.sqrt(5))
+            nn.init.zeros_(B.data)
+
+    def set_runtime_lora_config(self, lora_rank: int, lora_alpha: int) -> None:
+        if lora_rank <= 0 or lora_rank > self.r:
+            raise ValueError(f"Active LoRA rank must be in [1, {self.r}], got {lora_rank}")
+        self.active_r, self.active_lora_alpha = lora_rank, lora_alpha
+
+    def _active_scaling(self) -> float:
+        return compute_lora_scaling(self.active_lora_alpha, self.active_r, self.use_rslora)
+
+    def _active_lora_views(self, proj_name: str) -> Tuple[Tensor, Tensor]:
+        A = getattr(self, f"{proj_name}_lora_A")[..., : self.active_r].contiguous()
+        B = getattr(self, f"{proj_name}_lora_B")[:, : self.active_r, ...].contiguous()
+        return A, B
+
+    def _compute_proj_delta(self, proj_name: str) -> Tensor:
+        A, B = self._active_lora_views(proj_name)
+        E = max(A.shape[0], B.shape[0])
+        return torch.bmm(A.expand(E, -1, -1), B.expand(E, -1, -1)) * self._active_scaling()
+
+    # ------------------------------------------------------------------ storage helpers
+    @staticmethod
+    def _to_uint8(t: Tensor) -> Tensor:
+        return t.contiguous() if t.dtype == torch.uint8 else t.contiguous().view(torch.uint8)
+
+    def _recover_tensor(self, buf: Tensor, original_dtype: torch.dtype) -> Tensor:
+        return buf if original_dtype == torch.uint8 else buf.contiguous().view(original_dtype)
+
+    def _quantize_2d(self, w: Tensor, global_amax=None):
+        raise NotImplementedError
+
+    def _dequantize_2d(self, packed: Tensor, scales_dict: dict, K: int, N: int) -> Tensor:
+        raise NotImplementedError
+
+    def _quantize_proj(self, proj_name: str, w3d: Tensor, global_amax_per_expert: Optional[Tensor] = None) -> None:
+        """Quantize [E, K, N] expert by expert and stack the buffers."""
+        res = []
+        for i in range(w3d.shape[0]):
+            ga = global_amax_per_expert[i: i + 1] if global_amax_per_expert is not None else None
+            res.append(self._quantize_2d(w3d[i], global_amax=ga))
+        setattr(self, f"{proj_name}_packed", torch.stack([p for p, _ in res]))
+        self._scale_dtypes[proj_name] = {}
+        suffix = {"weight_block_scales": "block_scales", "weight_global_scale": "global_scale",
+                  "weight_scales": "scales"}
+        for key in res[0][1]:
+            self._scale_dtypes[proj_name][key] = res[0][1][key][1]
+            setattr(self, f"{proj_name}_{suffix[key]}", torch.stack([sd[key][0] for _, sd in res]))
+
+    def _build_scales_dict(self, proj_name: str, expert_idx: int) -> dict:
+        suffix = {"weight_block_scales": "block_scales", "weight_global_scale": "global_scale",
+                  "weight_scales": "scales"}
+        out = {}
+        for key, dt in self._scale_dtypes[proj_name].items():
+            buf = getattr(self, f"{proj_name}_{suffix[key]}", None)
+            if buf is not None:
+                out[key] = (buf[expert_idx], dt)
+        return out
+
+    def _proj_dims(self, proj_name: str) -> Tuple[int, int]:
+        return ((self.intermediate_size, self.hidden_size) if proj_name == "down"
+                else (self.hidden_size, self.intermediate_size))
+
+    def load_weights(self, gate: Tensor, up: Tensor, down: Tensor) -> None:
+        """Quantize full-precision GKN banks ([E, H, I], [E, H, I], [E, I, H]) into the packed buffers."""
+        with torch.no_grad():
+            for name, w in (("gate", gate), ("up", up), ("down", down)):
+                self._quantize_proj(name, w.float())
+        self._weights_loaded = True
+
+    def _bank(self, proj_name: str) -> QuantWeight:
+        raise NotImplementedError
+
+    @torch.compiler.disable
+    def dequantize_all_experts(self, proj_name: str, K: int, N: int) -> Tensor:
+        """[E, K, N] decoded bank in one launch (the reference loops over experts)."""
+        raise NotImplementedError
+
+    def dequantize_expert(self, proj_name: str, expert_idx: int, K: int, N: int) -> Tensor:
+        packed = getattr(self, f"{proj_name}_packed")
+        return self._dequantize_2d(packed[expert_idx], self._build_scales_dict(proj_name, expert_idx), K, N)
+
+    @property
+    def gate_proj(self) -> Tensor:
+        return self.dequantize_all_experts("gate", self.hidden_size, self.intermediate_size)
+
+    @property
+    def up_proj(self) -> Tensor:
+        return self.dequantize_all_experts("up", self.hidden_size, self.intermediate_size)
+
+    @property
+    def down_proj(self) -> Tensor:
+        return self.dequantize_all_experts("down", self.intermediate_size, self.hidden_size)
+
+    @property
+    def gate_up_proj(self) -> Tensor:
+        return torch.cat([self.gate_proj, self.up_proj], dim=2)
+
+    # ------------------------------------------------------------------ forward
+    def forward(self, hidden_states: Tensor, routing_weights: Tensor = None, selected_experts: Tensor = None,
+                expert_idx: int = None) -> Tensor:
+        if expert_idx is not None or self.moe_implementation == "eager":
+            raise NotImplementedError("per-expert eager calls are not part of the fused packed-bank path")
+        gA, gB = self._active_lora_views("gate_proj")
+        uA, uB = self._active_lora_views("up_proj")
+        dA, dB = self._active_lora_views("down_proj")
+        return moe_experts_qlora_forward(
+            num_experts=self.num_experts, routing_weights=routing_weights, selected_experts=selected_experts,
+            hidden_states=hidden_states, gate_proj=self._bank("gate"), up_proj=self._bank("up"),
+            down_proj=self._bank("down"), gate_proj_lora_A=gA, gate_proj_lora_B=gB, up_proj_lora_A=uA,
+            up_proj_lora_B=uB, down_proj_lora_A=dA, down_proj_lora_B=dB, scaling=self._active_scaling())
+
+    def merge_weights(self, ema_decay: float = 0.1) -> None:
+        with torch.no_grad():
+            for name in ("gate", "up", "down"):
+                K, N = self._proj_dims(name)
+                w = self.dequantize_all_experts(name, K, N).float()
+                merged = w + self._compute_proj_delta(f"{name}_proj").to(w.dtype)
+                self._requantize_proj(name, merged, ema_decay)
+        self.reset_lora_parameters()
+
+    def _requantize_proj(self, name: str, merged: Tensor, ema_decay: float) -> None:
+        self._quantize_proj(name, merged)
+
+    def extra_repr(self) -> str:
+        return (f"num_local_experts={self.num_local_experts}, num_experts={self.num_experts}, "
+                f"expert_offset={self.expert_offset}, intermediate_size={self.intermediate_size}, "
+                f"hidden_size={self.hidden_size}, r={self.active_r}, max_r={self.r}, "
+                f"quant_format={self.quant_format}, moe_implementation={self.moe_implementation}, "
+                f"hybrid_shared={self.hybrid_shared}, target_modules={list(self.target_modules)}")
+
+
+class BlockFP8QLoRAMoeExperts(QLoRAMoeExperts):
+    """e4m3 banks with fp32 128x128 block scales; buffers {gate,up,down}_{packed,block_scales}."""
+
+    def __init__(self, num_local_experts, num_experts, intermediate_size, hidden_size, r=16, lora_alpha=16, **kw):
+        kw.pop("quant_format", None)
+        kw.pop("quant_group_size", None)
+        super().__init__(num_local_experts, num_experts, intermediate_size, hidden_size, r=r, lora_alpha=lora_alpha,
+                         quant_format="block_fp8", quant_group_size=128, **kw)
+        for p in ("gate", "up", "down"):
+            self.register_buffer(f"{p}_packed", None)
+            self.register_buffer(f"{p}_block_scales", None)
+        self.reset_lora_parameters()
+
+    def _quantize_2d(self, w: Tensor, global_amax=None):
+        fp8, scales = Q.block_fp8_quantize_gkn(w.float().contiguous(), 128)
+        return self._to_uint8(fp8), {"weight_block_scales": (self._to_uint8(scales), scales.dtype)}
+
+    def _dequantize_2d(self, packed: Tensor, scales_dict: dict, K: int, N: int) -> Tensor:
+        scales = self._recover_tensor(*scales_dict["weight_block_scales"])
+        return Q.block_fp8_dequantize_gkn(packed.view(torch.float8_e4m3fn).reshape(K, N), scales, 128)
+
+    def _bank(self, proj_name: str) -> QuantWeight:
+        K, N = self._proj_dims(proj_name)
+        return QuantWeight("block_fp8", _C.XQ_LAYOUT_GKN, getattr(self, f"{proj_name}_packed"),
+                           getattr(self, f"{proj_name}_block_scales"), torch.float32, K, N, 128,
+                           num_experts=self.num_local_experts)
+
+    @torch.compiler.disable
+    def dequantize_all_experts(self, proj_name: str, K: int, N: int) -> Tensor:
+        import ctypes
+
+        w = self._bank(proj_name).c()
+        out = torch.empty(self.num_local_experts, K, N, dtype=torch.float32, device=getattr(self, f"{proj_name}_packed").device)
+        _C.check(_C.lib().xq_decode(ctypes.byref(w), out.data_ptr(), _C.XQ_DT_F32, _C.stream_ptr(out.device)))
+        return out
+
+
+class NvFP4QLoRAMoeExperts(QLoRAMoeExperts):
+    """e2m1 banks, per-16 block scales along K, fp32 global scale per expert;
+    buffers {gate,up,down}_{packed,block_scales,global_scale}."""
+
+    def __init__(self, num_local_experts, num_experts, intermediate_size, hidden_size, r=16, lora_alpha=16, **kw):
+        kw.pop("quant_format", None)
+        kw.pop("quant_group_size", None)
+        super().__init__(num_local_experts, num_experts, intermediate_size, hidden_size, r=r, lora_alpha=lora_alpha,
+                         quant_format="nvfp4", quant_group_size=16, **kw)
+        for p in ("gate", "up", "down"):
+            self.register_buffer(f"{p}_packed", None)
+            self.register_buffer(f"{p}_block_scales", None)
+            self.register_buffer(f"{p}_global_scale", None)
+        self.reset_lora_parameters()
+
+    def _quantize_2d(self, w: Tensor, global_amax=None):
+        packed, bs, g = Q.nvfp4_quantize_gkn(w, 16, global_amax=global_amax)
+        return self._to_uint8(packed), {"weight_block_scales": (self._to_uint8(bs), bs.dtype),
+                                        "weight_global_scale": (self._to_uint8(g), g.dtype)}
+
+    def _dequantize_2d(self, packed: Tensor, scales_dict: dict, K: int, N: int) -> Tensor:
+        bs = self._recover_tensor(*scales_dict["weight_block_scales"])
+        g = self._recover_tensor(*scales_dict["weight_global_scale"])
+        return Q.nvfp4_dequantize_gkn(packed, bs, g, K, N, 16)
+
+    def _bank(self, proj_name: str) -> QuantWeight:
+        K, N = self._proj_dims(proj_name)
+        sd = self._scale_dtypes[proj_name]
+        g = self._recover_tensor(getattr(self, f"{proj_name}_global_scale"), sd["weight_global_scale"])
+        return QuantWeight("nvfp4", _C.XQ_LAYOUT_GKN, getattr(self, f"{proj_name}_packed"),
+                           getattr(self, f"{proj_name}_block_scales"), sd["weight_block_scales"], K, N, 16,
+                           global_scale=g.float().reshape(-1).contiguous(), num_experts=self.num_local_experts)
+
+    @torch.compiler.disable
+    def dequantize_all_experts(self, proj_name: str, K: int, N: int) -> Tensor:
+        import ctypes
+
+        w = self._bank(proj_name).c()
+        out = torch.empty(self.num_local_experts, K, N, dtype=torch.bfloat16, device=getattr(self, f"{proj_name}_packed").device)
+        _C.check(_C.lib().xq_decode(ctypes.byref(w), out.data_ptr(), _C.XQ_DT_BF16, _C.stream_ptr(out.device)))
+        return out
+
+    def _requantize_proj(self, name: str, merged: Tensor, ema_decay: float) -> None:
+        fresh = merged.float().abs().amax(dim=(1, 2))
+        if self._ema_amax[name] is not None:
+            self._ema_amax[name].lerp_(fresh.to(self._ema_amax[name].device), ema_decay)
+        else:
+            self._ema_amax[name] = fresh
+        self._quantize_proj(name, merged, global_amax_per_expert=self._ema_amax[name])
