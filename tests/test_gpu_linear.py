@@ -20,7 +20,7 @@ def _run(m, x, dy):
 
 
 @pytest.mark.parametrize("fmt", ["block_fp8", "int4", "nvfp4"])
-@pytest.mark.parametrize("M,K,N,r", [(200, 256, 384, 16), (1, 128, 64, 8), (129, 384, 320, 24), (512, 1024, 512, 64)])
+@pytest.mark.parametrize("M,K,N,r", [(200, 256, 384, 16), (1, 128, 64, 8), (129, 384, 320, 24), (512, 1024, 512, 64), (1100, 512, 768, 32)])
 def test_dense_fwd_bwd_vs_oracle(hip_device, fmt, M, K, N, r):
     m, w_ref = make_dense_module(fmt, N, K, r, 2 * r, seed=M + K, device=hip_device)
     x = gen((M, K), 1.0, 11, torch.bfloat16)

@@ -86,7 +86,7 @@ bool xq_profile_mark_begin(hipStream_t s, double flops) {
     return hipEventRecord(g_prof.start[i], s) == hipSuccess;
 }
 void xq_profile_mark_end(hipStream_t s) {
-    hipEventRecord(g_prof.stop[g_prof.count], s);
+    (void)hipEventRecord(g_prof.stop[g_prof.count], s);
     ++g_prof.count;
 }
 
@@ -104,7 +104,7 @@ extern "C" int xq_profile_collect(int* n_launches, double* total_ms, double* tot
             return XQ_ERR_LAUNCH;
         }
         float t = 0.0f;
-        hipEventElapsedTime(&t, g_prof.start[i], g_prof.stop[i]);
+        (void)hipEventElapsedTime(&t, g_prof.start[i], g_prof.stop[i]);
         ms += t;
         fl += g_prof.flops[i];
     }

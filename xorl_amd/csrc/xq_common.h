@@ -90,3 +90,19 @@ __device__ __forceinline__ float int4_val(uint32_t nib, float s, float m8s) {
     (void)m8s;
     return ((float)nib - 8.0f) * s;
 }
+
+// ---------------------------------------------------------------- transposing LDS fragment read
+// MFMA 32x32x16 operand fragment from a row-major [k][col] bf16 LDS tile:
+__device__ __forceinline__ bf16x8 lds_tr_frag(const bf16_t* tile, int pitch, int krow0, int col0, int lane) {
+    // 8 consecutive k (rows krow0 + 8*(lane/32) + 0..7) of column col0 + lane%32,
+    // from a row-major [k][col] LDS tile, via two ds_read_b64_tr_b16.
+    const int i = lane & 15, g = lane >> 4;
+    const bf16_t* base = tile + (krow0 + 8 * (g >> 1) + (i >> 2)) * pitch + col0 + 16 * (g & 1) + 4 * (i & 3);
+    typedef __attribute__((ext_vector_type(4))) short s16x4;
+    s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(base));
+    s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(base + 4 * pitch));
+    typedef __attribute__((ext_vector_type(8))) short s16x8;
+    s16x8 v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    return __builtin_bit_cast(bf16x8, v);
+}
+

@@ -1,5 +1,7 @@
 // Host entry points of the fused dequant-GEMM + LoRA path (dense and grouped).
 #include "xq_gemm_tile.h"
+#include "xq_gemm_fp8.h"
+#include <stdlib.h>
 #include "xq_lora.h"
 
 namespace xq {
@@ -9,6 +11,9 @@ static void launch_tile_cc(const TileArgs& g, bool contract_cols, dim3 grid, hip
     if (contract_cols) gemm_tile_kernel<FMT, LAYOUT, true><<<grid, 256, 0, s>>>(g);
     else gemm_tile_kernel<FMT, LAYOUT, false><<<grid, 256, 0, s>>>(g);
 }
+
+// 1 = use the 256x256 block-fp8 kernel for large dense problems (default); 0 = generic tile kernel only
+static int g_fp8_variant = [] { const char* e = getenv("XQ_FP8_KERNEL"); return e ? atoi(e) : 1; }();
 
 // C[rows, Nout] = A . op(deq(W)) (+ su . Lr^T) (+ bias); see xq_gemm_tile.h
 int launch_tile_gemm(const xq_weight* w, bool contract_cols, const bf16_t* A, int64_t lda, int64_t n_rows,
@@ -37,6 +42,34 @@ int launch_tile_gemm(const xq_weight* w, bool contract_cols, const bf16_t* A, in
     if (w->format != XQ_FMT_FP8 && w->layout == XQ_LAYOUT_GKN)
         XQ_REQUIRE(w->rows % 2 == 0, "%s: GKN 4-bit storage needs an even row count", who);
     if (n_rows == 0) return XQ_OK;
+    // dense block-fp8 with enough rows: the 256x256 kernel
+    if (w->format == XQ_FMT_FP8 && !offsets && n_rows >= 1024 && g_fp8_variant != 0) {
+        Fp8Args f;
+        f.A = A; f.lda = lda; f.C = C; f.ldc = ldc;
+        f.W = (const uint8_t*)w->packed; f.scales = (const float*)w->scales;
+        f.wrows = g.wrows; f.wcols = g.wcols; f.Kc = g.Kc; f.Nout = g.Nout; f.M = n_rows;
+        f.su = g.r_pad ? su : nullptr; f.lora_right = g.r_pad ? lora_right : nullptr; f.r_pad = g.r_pad;
+        f.bias = bias;
+        f.tiles_m = (int32_t)xq_cdiv(n_rows, F8_BM); f.tiles_n = (int32_t)xq_cdiv(g.Nout, F8_BN);
+        const size_t lds = (size_t)(2 * F8_A_STAGE + 2 * (contract_cols ? F8_B_STAGE_NT : F8_B_STAGE_NN)) * 2;
+        static bool attr_set = false;
+        if (!attr_set) {
+            hipError_t e1 = hipFuncSetAttribute((const void*)gemm_fp8_256_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            hipError_t e2 = hipFuncSetAttribute((const void*)gemm_fp8_256_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            if (e1 != hipSuccess || e2 != hipSuccess) {
+                xq_set_error("%s: cannot raise the dynamic LDS limit: %s", who, hipGetErrorString(e1 != hipSuccess ? e1 : e2));
+                return XQ_ERR_LAUNCH;
+            }
+            attr_set = true;
+        }
+        dim3 grid((unsigned)(f.tiles_m * f.tiles_n));
+        const bool timed = xq_profile_mark_begin(stream, 2.0 * (double)n_rows * g.Nout * ((double)g.Kc + g.r_pad));
+        if (contract_cols) gemm_fp8_256_kernel<true><<<grid, 512, lds, stream>>>(f);
+        else gemm_fp8_256_kernel<false><<<grid, 512, lds, stream>>>(f);
+        if (timed) xq_profile_mark_end(stream);
+        XQ_CHECK_LAUNCH(who);
+        return XQ_OK;
+    }
     unsigned mt = (unsigned)(xq_cdiv(n_rows, BM) + (offsets ? w->num_experts : 0));
     dim3 grid(mt, (unsigned)xq_cdiv(g.Nout, BN));
     const bool timed = xq_profile_mark_begin(stream, 2.0 * (double)n_rows * g.Nout * ((double)g.Kc + g.r_pad));

@@ -212,19 +212,6 @@ struct TnArgs {
 constexpr int TN_PP = 128 + 16;  // Ps pitch (bf16 elements): 288 B rows
 constexpr int TN_QP = 80;        // Qs pitch: 160 B rows
 
-__device__ __forceinline__ bf16x8 lds_tr_frag(const bf16_t* tile, int pitch, int krow0, int col0, int lane) {
-    // 8 consecutive k (rows krow0 + 8*(lane/32) + 0..7) of column col0 + lane%32,
-    // from a row-major [k][col] LDS tile, via two ds_read_b64_tr_b16.
-    const int i = lane & 15, g = lane >> 4;
-    const bf16_t* base = tile + (krow0 + 8 * (g >> 1) + (i >> 2)) * pitch + col0 + 16 * (g & 1) + 4 * (i & 3);
-    typedef __attribute__((ext_vector_type(4))) short s16x4;
-    s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(base));
-    s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(base + 4 * pitch));
-    typedef __attribute__((ext_vector_type(8))) short s16x8;
-    s16x8 v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-    return __builtin_bit_cast(bf16x8, v);
-}
-
 template <int NT>
 __global__ void __launch_bounds__(256) tn_kernel(TnArgs g) {
     __shared__ __attribute__((aligned(16))) bf16_t Ps[32 * TN_PP];
