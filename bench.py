@@ -169,7 +169,7 @@ def main():
                    "tokens": M, "hidden": H, "intermediate": I, "lora_r": R, "format": "block_fp8"},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": BF16_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / BF16_MFMA_PEAK_TFLOPS, "traffic": None,
-                     "kernel": "gemm_tile_kernel<fp8> (fused dequant-GEMM, fwd and dgrad launches)",
+                     "kernel": "gemm_fp8_256_kernel<true|false> (fused fp8 dequant-GEMM, forward and dgrad launches)",
                      "launches": n.value, "avg_launch_ms": ms.value / max(n.value, 1)},
         "cpu_baseline": cpu,
     }
