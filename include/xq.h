@@ -107,7 +107,8 @@ int64_t xq_linear_workspace_bytes(int64_t M, int64_t N, int64_t K, int r);
 /* y[M,N] = x[M,K] . deq(W)^T + bias + s * (x . A^T) . B^T      (bf16 out)
  *   lora_A [r,K], lora_B [N,r] in lora_dtype (fp32 or bf16), r in {0..64};
  *   su_out (optional, bf16 [M, r_pad], r_pad = r rounded up to 16) receives
- *   bf16(s * x . A^T) for reuse by xq_linear_bwd;
+ *   bf16(s * x . A^T) for reuse by xq_linear_bwd; with su_out == NULL and
+ *   M <= 64 (K % 128 == 0) the weight-streaming skinny kernel is used;
  *   workspace: xq_linear_workspace_bytes(...) bytes, 256-byte aligned. */
 int xq_linear_fwd(const xq_weight* w, const void* x, int64_t ldx, int64_t M,
                   const void* lora_A, const void* lora_B, int lora_dtype, int r, float scaling,

@@ -13,6 +13,7 @@ static void launch_tile_cc(const TileArgs& g, bool contract_cols, dim3 grid, hip
 }
 
 // 1 = use the 256x256 block-fp8 kernel for large dense problems (default); 0 = generic tile kernel only
+static int g_skinny_enabled = [] { const char* e = getenv("XQ_SKINNY"); return e ? atoi(e) : 1; }();
 static int g_fp8_variant = [] { const char* e = getenv("XQ_FP8_KERNEL"); return e ? atoi(e) : 1; }();
 
 // C[rows, Nout] = A . op(deq(W)) (+ su . Lr^T) (+ bias); see xq_gemm_tile.h
@@ -102,13 +103,15 @@ using namespace xq;
 
 extern "C" int64_t xq_linear_workspace_bytes(int64_t M, int64_t N, int64_t K, int r) {
     int rp = r_pad_of(r);
-    if (rp == 0) return 256;
+    int64_t skinny = M <= 64 ? skinny_workspace_bytes(M, N, K, rp) : 0;
+    if (rp == 0) return skinny > 256 ? skinny : 256;
     int64_t fwd = align256(rp * K * 2) + align256(N * rp * 2) + align256(M * rp * 2);
     int64_t tnp = tn_partial_bytes(M, N, rp);
     int64_t tnk = tn_partial_bytes(M, K, rp);
     int64_t bwd = align256(rp * N * 2) + align256(K * rp * 2) + align256(rp * K * 2) + 2 * align256(M * rp * 2) +
                   align256(tnp > tnk ? tnp : tnk);
-    return (fwd > bwd ? fwd : bwd) + 256;
+    int64_t need = (fwd > bwd ? fwd : bwd) + 256;
+    return need > skinny ? need : skinny;
 }
 
 static int check_dense(const xq_weight* w, const char* who) {
@@ -133,6 +136,10 @@ extern "C" int xq_linear_fwd(const xq_weight* w, const void* x, int64_t ldx, int
     hipStream_t stream = (hipStream_t)stream_;
     if (M == 0) return XQ_OK;
     const int rp = r_pad_of(r);
+    // decode / rollout shapes: stream the packed weight once (HBM-bound kernel); forward only
+    if (!su_out && g_skinny_enabled && skinny_supported(w, M))
+        return launch_skinny(w, (const bf16_t*)x, ldx, M, lora_A, lora_B, lora_dtype, r, scaling,
+                             (const bf16_t*)bias_bf16, (bf16_t*)y, ldy, workspace, workspace_bytes, stream);
     bf16_t *A_bf = nullptr, *Bl = nullptr, *su = nullptr;
     if (rp) {
         XQ_REQUIRE(workspace && xq_aligned(workspace, 256) && workspace_bytes >= xq_linear_workspace_bytes(M, N, K, r),

@@ -31,4 +31,11 @@ int launch_tn(const bf16_t* P, int64_t ldp, int64_t width, const bf16_t* Q, int 
 
 int launch_zero_fill(void* p, int64_t bytes, hipStream_t stream);
 
+// skinny-M (M <= 64) forward path, xq_skinny.hip
+bool skinny_supported(const xq_weight* w, int64_t M);
+int64_t skinny_workspace_bytes(int64_t M, int64_t N, int64_t K, int r_pad);
+int launch_skinny(const xq_weight* w, const bf16_t* x, int64_t ldx, int64_t M, const void* lora_A, const void* lora_B,
+                  int lora_dtype, int r, float scaling, const bf16_t* bias, bf16_t* y, int64_t ldy, void* workspace,
+                  int64_t workspace_bytes, hipStream_t stream);
+
 }  // namespace xq

@@ -77,7 +77,7 @@ def _ld(x2: Tensor) -> int:
 def _linear_fwd_op(x: Tensor, packed: Tensor, scales: Tensor, global_scale: Optional[Tensor],
                    lora_A: Optional[Tensor], lora_B: Optional[Tensor], bias: Optional[Tensor],
                    fmt: str, scale_code: int, group: int, N: int, K: int, r: int,
-                   scaling: float) -> Tuple[Tensor, Tensor]:
+                   scaling: float, want_su: bool) -> Tuple[Tensor, Tensor]:
     if x.dtype != torch.bfloat16:
         raise _C.XqError(f"activations must be bf16, got {x.dtype}")
     x2 = _as_2d(x)
@@ -88,7 +88,7 @@ def _linear_fwd_op(x: Tensor, packed: Tensor, scales: Tensor, global_scale: Opti
     dev = x.device
     y = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
     rp = _r_pad(r)
-    su = torch.empty(M, rp, dtype=torch.bfloat16, device=dev)
+    su = torch.empty(M if want_su else 0, rp, dtype=torch.bfloat16, device=dev)
     L = _C.lib()
     ws_bytes = L.xq_linear_workspace_bytes(M, N, K, r)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
@@ -96,15 +96,15 @@ def _linear_fwd_op(x: Tensor, packed: Tensor, scales: Tensor, global_scale: Opti
     B = lora_B.contiguous() if lora_B is not None else None
     b = bias.to(torch.bfloat16).contiguous() if bias is not None else None
     _C.check(L.xq_linear_fwd(ctypes.byref(w), x2.data_ptr(), _ld(x2), M, _C.ptr(A), _C.ptr(B), _lora_dt(A), r,
-                             scaling, _C.ptr(b), y.data_ptr(), N, su.data_ptr() if rp else None, ws.data_ptr(),
+                             scaling, _C.ptr(b), y.data_ptr(), N, su.data_ptr() if (rp and want_su) else None, ws.data_ptr(),
                              ws_bytes, _C.stream_ptr(dev)))
     return y.reshape(*x.shape[:-1], N), su
 
 
 @_linear_fwd_op.register_fake
-def _(x, packed, scales, global_scale, lora_A, lora_B, bias, fmt, scale_code, group, N, K, r, scaling):
+def _(x, packed, scales, global_scale, lora_A, lora_B, bias, fmt, scale_code, group, N, K, r, scaling, want_su):
     M = x.numel() // max(x.shape[-1], 1)
-    return x.new_empty(*x.shape[:-1], N), x.new_empty(M, _r_pad(r))
+    return x.new_empty(*x.shape[:-1], N), x.new_empty(M if want_su else 0, _r_pad(r))
 
 
 @torch.library.custom_op("xq::linear_bwd", mutates_args=(), device_types="cuda")
@@ -150,11 +150,11 @@ class QLoRALinearFunction(torch.autograd.Function):
     [M, r] LoRA intermediate is saved -- no decoded weight."""
 
     @staticmethod
-    def forward(ctx, x, lora_A, lora_B, bias, qw: QuantWeight, r: int, scaling: float):
+    def forward(ctx, x, lora_A, lora_B, bias, qw: QuantWeight, r: int, scaling: float, want_su: bool = True):
         A = lora_A[:r] if lora_A is not None else None
         B = lora_B[:, :r] if lora_B is not None else None
         y, su = _linear_fwd_op(x, qw.packed, qw.scales, qw.global_scale, A, B, bias, qw.fmt,
-                               _DT_TO_CODE[qw.scale_dtype], qw.group, qw.rows, qw.cols, r, float(scaling))
+                               _DT_TO_CODE[qw.scale_dtype], qw.group, qw.rows, qw.cols, r, float(scaling), want_su)
         ctx.qw, ctx.r, ctx.scaling = qw, r, float(scaling)
         ctx.save_for_backward(x, su, lora_A, lora_B)
         return y
@@ -179,12 +179,16 @@ class QLoRALinearFunction(torch.autograd.Function):
         gbias = None
         if ctx.needs_input_grad[3]:
             gbias = dy.reshape(-1, dy.shape[-1]).sum(0)
-        return (dx if need_dx else None), gA, gB, gbias, None, None, None
+        return (dx if need_dx else None), gA, gB, gbias, None, None, None, None
 
 
 def qlora_linear(x: Tensor, qw: QuantWeight, lora_A: Optional[Tensor], lora_B: Optional[Tensor], r: int,
                  scaling: float, bias: Optional[Tensor] = None) -> Tensor:
-    return QLoRALinearFunction.apply(x, lora_A, lora_B, bias, qw, r, scaling)
+    # Without a backward (inference / rollout) nothing needs the saved LoRA intermediate, which
+    # also lets small batches take the weight-streaming kernel.
+    training = torch.is_grad_enabled() and any(
+        t is not None and t.requires_grad for t in (x, lora_A, lora_B, bias))
+    return QLoRALinearFunction.apply(x, lora_A, lora_B, bias, qw, r, scaling, training)
 
 
 # ---------------------------------------------------------------------------
