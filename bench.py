@@ -106,6 +106,12 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--cpu-rows", type=int, default=256, help="token rows of the CPU baseline sample (0 = skip)")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="before the warmup, run one plain 256 MiB -> 256 MiB elementwise copy so that a counter "
+                         "run (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE) holds a kernel of known traffic to scale by")
+    ap.add_argument("--traffic-bytes", type=float, default=None,
+                    help="HBM bytes per launch of the roofline kernel from such counter runs (reported as "
+                         "roofline.traffic; null when not given)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs the QLoRA path on ONE GPU; --gpus must be 1 "
@@ -135,6 +141,12 @@ def main():
         y.backward(dy)
 
     L = _C.lib()
+    if args.calibrate_copy:
+        src = torch.ones(64 << 20, dtype=torch.float32, device=dev)      # 256 MiB read + 256 MiB written
+        dst = torch.empty_like(src)
+        torch.mul(src, 1.0, out=dst)
+        torch.cuda.synchronize()
+        del src, dst
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -168,7 +180,7 @@ def main():
                                "intermediate 12288, LoRA r=32 on gate/up/down, SwiGLU",
                    "tokens": M, "hidden": H, "intermediate": I, "lora_r": R, "format": "block_fp8"},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": BF16_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / BF16_MFMA_PEAK_TFLOPS, "traffic": None,
+                     "frac": achieved / BF16_MFMA_PEAK_TFLOPS, "traffic": args.traffic_bytes,
                      "kernel": "gemm_fp8_256_kernel<true|false> (fused fp8 dequant-GEMM, forward and dgrad launches)",
                      "launches": n.value, "avg_launch_ms": ms.value / max(n.value, 1)},
         "cpu_baseline": cpu,

@@ -184,16 +184,19 @@ __global__ void __launch_bounds__(512, 2) gemm_fp8_256_kernel(Fp8Args g) {
 
     // Pipeline: at the top of iteration kt the registers hold tile kt+1 (loaded one
     // whole iteration earlier, so the global latency is covered by a full tile of
-    // MFMAs).  They are stored/decoded into the other LDS stage, the loads of tile
-    // kt+2 are issued, and tile kt is multiplied out of the current stage.
+    // MFMAs) and the operand fragments of k16-step 0 of tile kt.  Tile kt+1 is
+    // stored/decoded into the other LDS stage and the loads of tile kt+2 are issued
+    // while steps 0..2 are multiplied; the single barrier of the iteration sits before
+    // the last step, whose MFMAs then cover both the barrier skew and the fetch of the
+    // next tile's first fragments.  (Every read of a stage completes before the barrier
+    // that precedes the next stores into it.)
     const int nk = g.Kc / F8_BK;
+    bf16x8 af0[4], bf0[2], af1[4], bf1[2];
     auto iteration = [&](int kt, bool have_next, bool have_next2) {
         const bf16_t* a = As + (kt & 1) * F8_A_STAGE;
         const bf16_t* b = Bs + (kt & 1) * B_STAGE;
         bf16_t* an = As + ((kt + 1) & 1) * F8_A_STAGE;
         bf16_t* bn = Bs + ((kt + 1) & 1) * B_STAGE;
-        bf16x8 af0[4], bf0[2], af1[4], bf1[2];
-        load_frags(a, b, 0, false, af0, bf0);
         load_frags(a, b, 1, false, af1, bf1);
         if (have_next) store_a(an);
         if (have_next2) load_a(kt + 2);
@@ -206,8 +209,9 @@ __global__ void __launch_bounds__(512, 2) gemm_fp8_256_kernel(Fp8Args g) {
         mma(af1, bf1);
         load_frags(a, b, 3, false, af1, bf1);
         mma(af0, bf0);
-        mma(af1, bf1);
         __syncthreads();
+        if (have_next) load_frags(an, bn, 0, false, af0, bf0);
+        mma(af1, bf1);
     };
     load_a(0);
     load_w(0);
@@ -216,6 +220,7 @@ __global__ void __launch_bounds__(512, 2) gemm_fp8_256_kernel(Fp8Args g) {
     store_w(Bs, 1);
     if (nk > 1) { load_a(1); load_w(1); }
     __syncthreads();
+    load_frags(As, Bs, 0, false, af0, bf0);
     int kt = 0;
     for (; kt + 2 < nk; ++kt) iteration(kt, true, true);
     if (kt + 1 < nk) { iteration(kt, true, false); ++kt; }
