@@ -100,12 +100,126 @@ def cpu_baseline(mods, rows: int):
     }
 
 
+def zipf_routing(T, E, topk, seed, empty=2, device="cpu"):
+    """Seeded router output whose per-expert token counts follow Zipf(s=1.1) over a random
+    permutation of the experts; the `empty` least popular experts are never chosen."""
+    g = torch.Generator().manual_seed(seed)
+    perm = torch.randperm(E, generator=g)
+    pmf = 1.0 / torch.arange(1, E + 1, dtype=torch.float64) ** 1.1
+    logits = torch.log(pmf / pmf.sum())[perm.argsort()].float()
+    gumbel = -torch.log(-torch.log(torch.rand(T, E, generator=g).clamp_min(1e-9)))
+    z = logits[None, :] + gumbel
+    z[:, perm[-empty:]] = -1e9
+    rw, sel = torch.topk(torch.softmax(z, -1), topk, dim=-1)
+    rw = rw / rw.sum(-1, keepdim=True)
+    return rw.to(torch.bfloat16).to(device), sel.int().to(device)
+
+
+def dense_module(fmt, N, K, r, alpha, seed, dev):
+    from xorl_amd.qlora import QLoRALinear
+
+    lin = torch.nn.Linear(K, N, bias=False, device=dev)
+    g = torch.Generator(device=dev).manual_seed(seed)
+    with torch.no_grad():
+        lin.weight.copy_(torch.randn(N, K, generator=g, device=dev) * 0.02)
+    m = QLoRALinear.from_module(lin, r=r, lora_alpha=alpha, quant_format=fmt)
+    with torch.no_grad():
+        m.lora_A.copy_(torch.randn(r, K, generator=g, device=dev) * 0.02)
+        m.lora_B.copy_(torch.randn(N, r, generator=g, device=dev) * 0.02)
+    return m
+
+
+def other_config(cfg: int, dev):
+    """Builds BASELINE.json configs[0], [2], [3] or [4] on the device.  Returns
+    (step_fn, work_per_step, unit_is_bytes, workload_text, kernel_text)."""
+    lin_flops = lambda m, K, N, r: 4.0 * m * K * N + 6.0 * m * r * (K + N)
+    rnd = lambda *shape, seed: torch.randn(*shape, generator=torch.Generator(device=dev).manual_seed(seed),
+                                           device=dev).to(torch.bfloat16)
+    if cfg == 0:
+        m = dense_module("int4", 4096, 4096, 16, 32, 10, dev)
+        x, dy = rnd(512, 4096, seed=1).requires_grad_(True), rnd(512, 4096, seed=2)
+
+        def step():
+            x.grad = m.lora_A.grad = m.lora_B.grad = None
+            m(x).backward(dy)
+        return (step, lin_flops(512, 4096, 4096, 16), False,
+                "configs[0]: int4 (group 128, bf16 absmax/7 scales) QLoRA linear 4096->4096, M=512, r=16, fwd+bwd",
+                "gemm_tile_kernel<int4> (fused dequant-GEMM, forward and dgrad launches)")
+    if cfg == 2:
+        Mtok, Hd = 4096, 5120
+        shapes = {"q": (8192, Hd), "k": (1024, Hd), "v": (1024, Hd), "o": (Hd, 8192)}
+        mods = {k: dense_module("nvfp4", N, K, 16, 32, 20 + i, dev) for i, (k, (N, K)) in enumerate(shapes.items())}
+        xs = {k: rnd(Mtok, K, seed=30 + i).requires_grad_(True) for i, (k, (N, K)) in enumerate(shapes.items())}
+        dys = {k: rnd(Mtok, N, seed=40 + i) for i, (k, (N, K)) in enumerate(shapes.items())}
+
+        def step():
+            for k, m in mods.items():
+                xs[k].grad = m.lora_A.grad = m.lora_B.grad = None
+                m(xs[k]).backward(dys[k])
+        return (step, sum(lin_flops(Mtok, K, N, 16) for (N, K) in shapes.values()), False,
+                "configs[2]: nvfp4 QLoRA Qwen3-32B attention projections q/k/v/o, hidden 5120, M=4096, r=16, fwd+bwd",
+                "gemm_tile_kernel<nvfp4> (fused dequant-GEMM, forward and dgrad launches)")
+    if cfg == 3:
+        from xorl_amd.qlora import BlockFP8QLoRAMoeExperts
+
+        E, Hd, I, T, topk, r = 128, 2048, 768, 16384, 8, 16
+        m = BlockFP8QLoRAMoeExperts(E, E, I, Hd, r=r, lora_alpha=2 * r, hybrid_shared=False).to(dev)
+        g = torch.Generator(device=dev).manual_seed(50)
+        w = lambda *shape: torch.randn(*shape, generator=g, device=dev) * 0.02
+        m.load_weights(w(E, Hd, I), w(E, Hd, I), w(E, I, Hd))
+        m = m.to(dev)
+        with torch.no_grad():
+            for name in ("gate_proj", "up_proj", "down_proj"):
+                getattr(m, f"{name}_lora_A").copy_(w(*getattr(m, f"{name}_lora_A").shape))
+                getattr(m, f"{name}_lora_B").copy_(w(*getattr(m, f"{name}_lora_B").shape))
+        rw, sel = zipf_routing(T, E, topk, seed=3, device=dev)
+        counts = torch.bincount(sel.flatten().long(), minlength=E)
+        assert int((counts == 0).sum()) >= 1, "the routing must leave some experts empty"
+        x, dy = rnd(T, Hd, seed=51).requires_grad_(True), rnd(T, Hd, seed=52)
+        params = [p for p in m.parameters() if p.requires_grad]
+
+        def step():
+            x.grad = None
+            for p in params:
+                p.grad = None
+            m(x, rw, sel).backward(dy)
+        R = T * topk
+        return (step, R * (12.0 * Hd * I + 18.0 * r * (Hd + I)), False,
+                f"configs[3]: grouped block_fp8 QLoRA Qwen3-30B-A3B experts, E=128, hidden 2048, intermediate 768, "
+                f"top-8 of 16384 tokens, Zipf(1.1) counts (max {int(counts.max())}, {int((counts == 0).sum())} empty), "
+                f"per-expert r=16, fwd+bwd",
+                "gemm_tile_kernel<fp8, grouped> (fused dequant grouped GEMM, forward and dgrad launches)")
+    if cfg == 4:
+        shapes = {"q": (4096, 4096), "kv": (1024, 4096), "gate_up": (12288, 4096), "down": (4096, 12288)}
+        cases, total = [], 0.0
+        for fmt in ("int4", "block_fp8"):
+            for i, (k, (N, K)) in enumerate(shapes.items()):
+                m = dense_module(fmt, N, K, 16, 32, 60 + i, dev)
+                wbytes = (K * N / 2 + 2 * K * N / 128) if fmt == "int4" else (K * N + 4 * ((K + 127) // 128) * ((N + 127) // 128))
+                for Mtok in (1, 8, 32, 64):
+                    cases.append((m, rnd(Mtok, K, seed=70 + Mtok)))
+                    total += wbytes + 2 * Mtok * K + 2 * Mtok * N + 4 * 16 * (K + N)
+
+        def step():
+            with torch.no_grad():
+                for m, x in cases:
+                    m(x)
+        return (step, total, True,
+                "configs[4]: skinny-M forward, M in {1,8,32,64} x {q 4096->4096, kv 4096->1024, gate/up 4096->12288, "
+                "down 12288->4096} x {int4, block_fp8}, r=16 (32 launches per step)",
+                "skinny_kernel<int4|fp8> (weight-streaming fused dequant-GEMV/GEMM)")
+    raise SystemExit(f"bench.py: unknown --config {cfg}")
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--cpu-rows", type=int, default=256, help="token rows of the CPU baseline sample (0 = skip)")
+    ap.add_argument("--config", type=int, default=1,
+                    help="BASELINE.json configs index; 1 (default) is the headline workload, the others report the "
+                         "same JSON for their own workload (no CPU baseline)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="before the warmup, run one plain 256 MiB -> 256 MiB elementwise copy so that a counter "
                          "run (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE) holds a kernel of known traffic to scale by")
@@ -123,6 +237,8 @@ def main():
     from xorl_amd.functional import silu_and_mul
 
     dev = torch.device("cuda:0")
+    if args.config != 1:
+        return run_other(args, dev)
     mods_cpu = build_modules()
     cpu = cpu_baseline(mods_cpu, args.cpu_rows) if args.cpu_rows > 0 else None
     mods = {k: m.to(dev) for k, m in mods_cpu.items()}
@@ -186,6 +302,35 @@ def main():
         "cpu_baseline": cpu,
     }
     print(json.dumps(out))
+
+
+def run_other(args, dev):
+    from xorl_amd import _C
+
+    step, work, is_bytes, workload, kernel = other_config(args.config, dev)
+    L = _C.lib()
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    L.xq_profile_enable(1)
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / args.steps
+    n, ms, fl = ctypes.c_int(0), ctypes.c_double(0), ctypes.c_double(0)
+    _C.check(L.xq_profile_collect(ctypes.byref(n), ctypes.byref(ms), ctypes.byref(fl)))
+    L.xq_profile_enable(0)
+    scale, unit, peak = (1e9, "GB/s", 8000.0) if is_bytes else (1e12, "TFLOP/s", BF16_MFMA_PEAK_TFLOPS)
+    achieved = fl.value / (ms.value * 1e-3) / scale if ms.value > 0 else 0.0
+    print(json.dumps({
+        "metric": METRIC, "value": work / dt / scale, "unit": unit, "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": dt * 1e3, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic", "config": {"workload": workload},
+        "roofline": {"bound": "hbm" if is_bytes else "mfma", "achieved": achieved, "peak": peak, "unit": unit,
+                     "frac": achieved / peak, "traffic": args.traffic_bytes, "kernel": kernel,
+                     "launches": n.value, "avg_launch_ms": ms.value / max(n.value, 1)},
+        "cpu_baseline": None}))
 
 
 if __name__ == "__main__":

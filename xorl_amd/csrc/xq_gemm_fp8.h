@@ -197,21 +197,36 @@ __global__ void __launch_bounds__(512, 2) gemm_fp8_256_kernel(Fp8Args g) {
         const bf16_t* b = Bs + (kt & 1) * B_STAGE;
         bf16_t* an = As + ((kt + 1) & 1) * F8_A_STAGE;
         bf16_t* bn = Bs + ((kt + 1) & 1) * B_STAGE;
+        // region 1: MFMAs of step 0 over the step-1 fragment reads, the A-tile stores and the next A loads
+        mma(af0, bf0);
         load_frags(a, b, 1, false, af1, bf1);
         if (have_next) store_a(an);
         if (have_next2) load_a(kt + 2);
-        __builtin_amdgcn_sched_barrier(0);   // pin the global loads early: a full tile of MFMAs covers their latency
-        mma(af0, bf0);
+        // interleave: one LDS read behind each of the first six MFMAs, then the stores and global loads
+        for (int q = 0; q < 6; ++q) { __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); }
+        for (int q = 0; q < 2; ++q) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x200, 2, 0);
+            __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        // region 2: MFMAs of step 1 over the weight decode + stores, the next weight loads, step-2 fragment reads
+        mma(af1, bf1);
         if (have_next) { store_w(bn, 0); store_w(bn, 1); }
         if (have_next2) load_w(kt + 2);
-        __builtin_amdgcn_sched_barrier(0);
         load_frags(a, b, 2, false, af0, bf0);
-        mma(af1, bf1);
-        load_frags(a, b, 3, false, af1, bf1);
+        __builtin_amdgcn_sched_barrier(0);
+        // region 3: MFMAs of step 2 over the step-3 fragment reads
         mma(af0, bf0);
+        load_frags(a, b, 3, false, af1, bf1);
+        __builtin_amdgcn_sched_barrier(0);
         __syncthreads();
+        // region 4: MFMAs of step 3 over the next tile's first fragment reads, which must have
+        // landed before the next iteration starts multiplying
         if (have_next) load_frags(an, bn, 0, false, af0, bf0);
         mma(af1, bf1);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
     };
     load_a(0);
     load_w(0);
