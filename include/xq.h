@@ -85,6 +85,15 @@ const char* xq_last_error(void);
 int xq_profile_enable(int on);
 int xq_profile_collect(int* n_launches, double* total_ms, double* total_flops);
 
+/* Kernel selection of the fused dequant-GEMM entry points (dense and grouped),
+ * for tests and A/B measurements; no counterpart in the reference.
+ *   0 (default): by problem size -- the 256x256 tile kernel when its tiles fill
+ *      the chip (block-fp8, and FLAT int4/nvfp4 with a power-of-two group >= 16),
+ *      else the generic 128x128 tile kernel;
+ *   1: always the generic 128x128 tile kernel;
+ *   2: the 256x256 kernel whenever the format allows it, whatever the size. */
+int xq_set_tile_policy(int policy);
+
 /* ---- decode ------------------------------------------------------------
  * out[e] = decoded weight of expert e, shape [rows, cols], bf16 or fp32.
  * Replaces int4_dequantize / int4_dequantize_gkn
@@ -143,8 +152,9 @@ int xq_silu_mul_bwd(const void* gate, const void* up, int64_t ld_in, const void*
  * (ops/moe/lora.py:579-583): expert_histogram, stable argsort by expert id,
  * cumsum.  selected [T*topk] int32 expert ids (row-major [T, topk]).
  * Outputs: counts [E], offsets [E+1] (exclusive prefix), scatter_index
- * [T*topk] (row in expert order of routed copy i), tile_offsets [E+1]
- * (prefix of ceil(count/128), the row-tile schedule of the grouped kernels).
+ * [T*topk] (row in expert order of routed copy i), tile_offsets [2*(E+1)]:
+ * two row-tile schedules of the grouped kernels back to back, the prefix of
+ * ceil(count/128) in [0, E] and the prefix of ceil(count/256) in [E+1, 2E+1].
  * Deterministic and stable.  workspace: xq_route_workspace_bytes() bytes. */
 int64_t xq_route_workspace_bytes(int64_t n_routed, int32_t num_experts);
 int xq_route_build(const int32_t* selected, int64_t n_routed, int32_t num_experts,

@@ -19,3 +19,13 @@ def hip_device():
     if not torch.cuda.is_available():
         pytest.skip("no GPU")
     return torch.device("cuda:0")
+
+
+@pytest.fixture
+def tile_policy(request):
+    """Selects the fused dequant-GEMM kernel for one test: 0 = by size, 1 = 128x128 tiles, 2 = 256x256 tiles."""
+    from xorl_amd import _C
+
+    _C.check(_C.lib().xq_set_tile_policy(int(request.param)))
+    yield int(request.param)
+    _C.check(_C.lib().xq_set_tile_policy(0))

@@ -19,9 +19,10 @@ def _run(m, x, dy):
     return y.detach(), x.grad, m.lora_A.grad, m.lora_B.grad
 
 
+@pytest.mark.parametrize("tile_policy", [0, 2], indirect=True)
 @pytest.mark.parametrize("fmt", ["block_fp8", "int4", "nvfp4"])
 @pytest.mark.parametrize("M,K,N,r", [(200, 256, 384, 16), (1, 128, 64, 8), (129, 384, 320, 24), (512, 1024, 512, 64), (1100, 512, 768, 32)])
-def test_dense_fwd_bwd_vs_oracle(hip_device, fmt, M, K, N, r):
+def test_dense_fwd_bwd_vs_oracle(hip_device, tile_policy, fmt, M, K, N, r):
     m, w_ref = make_dense_module(fmt, N, K, r, 2 * r, seed=M + K, device=hip_device)
     x = gen((M, K), 1.0, 11, torch.bfloat16)
     dy = gen((M, N), 1.0, 12, torch.bfloat16)
@@ -34,7 +35,8 @@ def test_dense_fwd_bwd_vs_oracle(hip_device, fmt, M, K, N, r):
         assert err <= TOL, f"{fmt} {name}: {err}"
 
 
-def test_config0_int4_full_size(hip_device):
+@pytest.mark.parametrize("tile_policy", [0, 2], indirect=True)
+def test_config0_int4_full_size(hip_device, tile_policy):
     """BASELINE config 0: X [512,4096], W [4096,4096] int4 g128 absmax/7 bf16 scales, r=16, alpha=32."""
     M, K, N, r = 512, 4096, 4096, 16
     m, w_ref = make_dense_module("int4", N, K, r, 32, seed=0, device=hip_device)

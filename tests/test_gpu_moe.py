@@ -40,7 +40,9 @@ def test_route_scatter_gather_exact(hip_device, T, E, topk):
     assert torch.equal(sidx.cpu().view(T, topk), sidx_ref)
     assert torch.equal(offsets.cpu().long(), torch.cat([torch.zeros(1, dtype=torch.long), splits.cumsum(0)]))
     tiles = (splits + 127) // 128
-    assert torch.equal(tile_offsets.cpu().long(), torch.cat([torch.zeros(1, dtype=torch.long), tiles.cumsum(0)]))
+    assert torch.equal(tile_offsets.cpu().long()[: E + 1], torch.cat([torch.zeros(1, dtype=torch.long), tiles.cumsum(0)]))
+    tiles2 = (counts.cpu().long() + 255) // 256
+    assert torch.equal(tile_offsets.cpu().long()[E + 1 :], torch.cat([torch.zeros(1, dtype=torch.long), tiles2.cumsum(0)]))
     assert (splits == 0).any() or E <= 4
     # scatter then gather: out[t] = sum_j x[t] = topk * x[t] (exact in bf16 for power-of-two topk)
     x = gen((T, 64), 1.0, 3, torch.bfloat16).to(hip_device)
@@ -81,9 +83,10 @@ def _make_experts(fmt, E, H, I, r, hybrid, seed, device):
     return m.to(device), banks
 
 
+@pytest.mark.parametrize("tile_policy", [0, 2], indirect=True)
 @pytest.mark.parametrize("fmt", ["block_fp8", "nvfp4"])
 @pytest.mark.parametrize("E,T,H,I,r,topk,hybrid", [(6, 300, 128, 192, 8, 2, True), (16, 700, 256, 128, 16, 4, False)])
-def test_moe_fwd_bwd_vs_oracle(hip_device, fmt, E, T, H, I, r, topk, hybrid):
+def test_moe_fwd_bwd_vs_oracle(hip_device, tile_policy, fmt, E, T, H, I, r, topk, hybrid):
     m, banks = _make_experts(fmt, E, H, I, r, hybrid, seed=E + T, device=hip_device)
     # the module's own bank decode is bit-exact with the oracle
     for p in ("gate", "up", "down"):

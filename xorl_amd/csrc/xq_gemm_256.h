@@ -1,0 +1,436 @@
+// Large-M fused dequant-GEMM: 256x256x64 tiles, 8 waves (2 along M x 4 along N, two
+// per SIMD so one wave's LDS/VALU work hides under the other's MFMAs), each wave a
+// 128x64 sub-tile of 4x2 v_mfma_f32_32x32x16_bf16 (128 fp32 accumulators).
+//
+//   C[rows, Nout] = A[rows, Kc] . Wop (+ su[rows, r] . Lr[Nout, r]^T) (+ bias)
+//
+// W is a quantized [wrows, wcols] matrix: block-fp8 (e4m3 bytes, fp32 scale per
+// 128x128 block) or a 4-bit FLAT matrix (int4 / nvfp4: two codes per byte along
+// the columns, one scale per `group` consecutive columns).
+//   CONTRACT_COLS (dense forward, expert-bank dgrad):  Wop[kc][n] = W[n][kc]; the
+//     decoded tile is stored in LDS as [n][kc] (kc contiguous, XOR-swizzled 16-byte
+//     chunks) and read with ds_read_b128 in MFMA operand order.
+//   !CONTRACT_COLS (dense dgrad, expert-bank forward): Wop[kc][n] = W[kc][n]; the
+//     decoded tile is stored as it lies in memory, [kc][n], and the operand
+//     fragments are read with the transposing LDS load ds_read_b64_tr_b16 -- no
+//     transposed copy of the weight exists anywhere.
+// Every packed code is decoded exactly once per tile, in registers, to the bf16
+// value the reference decoder produces.  LDS is double buffered; the next tile's
+// global loads are issued one iteration ahead, its LDS stores and decode are spread
+// between the four k16 MFMA groups of the current tile, and operand fragments are
+// fetched one k16 step ahead.  Operands are swapped in the MFMA (D = W_frag x
+// A_frag) so that each lane ends up with 4 consecutive output columns and the
+// epilogue writes 8-byte packed bf16.
+//
+// GROUPED: rows are in expert order; a block works on one 256-row tile of one
+// expert (found from the 256-row tile prefix that xq_route_build emits) against
+// that expert's matrix of the bank.
+#pragma once
+
+#include "xq_common.h"
+
+namespace xq {
+
+constexpr int F8_BM = 256, F8_BN = 256, F8_BK = 64;
+constexpr int F8_A_STAGE = F8_BM * F8_BK;             // bf16 elements (32 KB)
+constexpr int F8_NN_PITCH = F8_BN + 32;               // [kc][n] rows of 576 B
+constexpr int F8_B_STAGE_NT = F8_BN * F8_BK;          // 32 KB
+constexpr int F8_B_STAGE_NN = F8_BK * F8_NN_PITCH;    // 36 KB
+
+// element offset of 16-byte chunk `c` (0..7) of row `r` in a [rows][64] bf16 tile.
+// gfx950 LDS has 64 banks (256 B/clk) and serves a ds_read_b128 sixteen lanes at a
+// time: 16 consecutive rows (128 B each, so even/odd rows sit in different bank
+// halves) must land on 8 distinct chunk slots per parity -> XOR with (r >> 1) & 7.
+__device__ __forceinline__ int swz(int r, int c) { return r * 64 + ((c ^ ((r >> 1) & 7)) << 3); }
+
+struct G256Args {
+    const bf16_t* A;
+    int64_t lda;
+    bf16_t* C;
+    int64_t ldc;
+    const uint8_t* W;          // packed codes (expert 0)
+    const uint8_t* scales;     // scales (expert 0)
+    const float* global_scale; // nvfp4: one per expert
+    int64_t packed_stride, scale_stride;  // bytes per expert
+    int32_t wrows, wcols;
+    int32_t gshift;            // 4-bit: log2(group)
+    int32_t scale_dtype;
+    int32_t Kc, Nout;
+    int64_t M;                 // total rows
+    const int32_t* offsets;    // grouped: [E+1] row offsets in expert order
+    const int32_t* tiles256;   // grouped: [E+1] prefix of ceil(count/256)
+    int32_t num_experts;
+    const bf16_t* su;          // [M, r_pad] or NULL
+    const bf16_t* lora_right;  // [E][Nout, r_pad] or NULL
+    int32_t r_pad;
+    const bf16_t* bias;
+    int32_t tiles_m, tiles_n;  // grouped: tiles_m is an upper bound
+};
+
+// ---------------------------------------------------------------- weight-tile loaders
+// A 256(n) x 64(kc) tile is split over 512 threads as 2 runs of 16 consecutive codes
+// each: run u = tid + p*512.  CONTRACT_COLS: W row n0 + (u >> 2), columns k0 + (u&3)*16
+// .. +16; otherwise W row k0 + (u >> 4), columns n0 + (u&15)*16 .. +16.  load()
+// fetches the packed bytes and scale(s) of K-step kt into registers; store() decodes
+// one run and writes its 16 bf16 values (two 16-byte LDS stores) to the stage.
+
+template <bool CC>
+__device__ __forceinline__ void store_run16(bf16_t* b, int u, const u32x4& lo, const u32x4& hi) {
+    if (CC) {
+        const int r = u >> 2, c = (u & 3) * 2;
+        *(u32x4*)(b + swz(r, c)) = lo;
+        *(u32x4*)(b + swz(r, c + 1)) = hi;
+    } else {
+        bf16_t* d = b + (u >> 4) * F8_NN_PITCH + (u & 15) * 16;
+        *(u32x4*)d = lo;
+        *(u32x4*)(d + 8) = hi;
+    }
+}
+
+template <bool CC>
+struct W256Fp8 {
+    const uint8_t* src[2];
+    const float* s_src[2];
+    int64_t kstep;
+    int scols, tid;
+    u32x4 raw[2];
+    float s[2];
+    __device__ __forceinline__ void init(const G256Args& g, const uint8_t* pk, const uint8_t* sc, float, int n0, int tid_) {
+        tid = tid_;
+        scols = (g.wcols + 127) >> 7;
+#pragma unroll
+        for (int p = 0; p < 2; ++p) {
+            const int u = tid + p * 512;
+            int wr, wc;
+            if (CC) { wr = min(n0 + (u >> 2), g.wrows - 1); wc = (u & 3) * 16; }
+            else { wr = u >> 4; wc = min(n0 + (u & 15) * 16, g.wcols - 16); }
+            src[p] = pk + (int64_t)wr * g.wcols + wc;
+            s_src[p] = (const float*)sc + (CC ? (wr >> 7) * scols : (wc >> 7));
+        }
+        kstep = CC ? F8_BK : (int64_t)F8_BK * g.wcols;
+    }
+    __device__ __forceinline__ void load(int kt) {
+        const int k0 = kt * F8_BK;
+#pragma unroll
+        for (int p = 0; p < 2; ++p) {
+            raw[p] = *(const u32x4*)(src[p] + kt * kstep);
+            s[p] = CC ? s_src[p][k0 >> 7] : s_src[p][(k0 >> 7) * scols];
+        }
+    }
+    __device__ __forceinline__ void store(bf16_t* b, int p) {
+        const float sc = s[p];
+        u32x4 lo, hi;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            f32x2 x0 = e4m3x2_to_f32(raw[p][i], false), x1 = e4m3x2_to_f32(raw[p][i], true);
+            uint32_t v0 = pack_bf16x2(x0[0] * sc, x0[1] * sc), v1 = pack_bf16x2(x1[0] * sc, x1[1] * sc);
+            if (i < 2) { lo[2 * i] = v0; lo[2 * i + 1] = v1; }
+            else { hi[2 * (i - 2)] = v0; hi[2 * (i - 2) + 1] = v1; }
+        }
+        store_run16<CC>(b, tid + p * 512, lo, hi);
+    }
+};
+
+__device__ __forceinline__ uint32_t load_scale_raw(const uint8_t* p, int64_t idx, int dtype) {
+    if (dtype == XQ_SCALE_F32) return ((const uint32_t*)p)[idx];
+    if (dtype == XQ_SCALE_BF16) return ((const uint16_t*)p)[idx];
+    return p[idx];
+}
+__device__ __forceinline__ float scale_from_raw(uint32_t raw, int dtype) {
+    if (dtype == XQ_SCALE_F32) return __uint_as_float(raw);
+    if (dtype == XQ_SCALE_BF16) return __uint_as_float(raw << 16);
+    return e4m3_to_f32((uint8_t)raw);
+}
+
+// value of 8 e2m1 codes: the magnitude code c = nib & 7 indexes the table
+// {0, .5, 1, 1.5, 2, 3, 4, 6}; built as fp32 bits, sign from bit 3.
+template <int FMT>
+__device__ __forceinline__ void decode8_4bit(uint32_t w, float s, uint32_t* out4) {
+    float v[8];
+    if (FMT == XQ_FMT_INT4) {
+        // (nib - 8) * s with a single rounding: fma(nib, s, -8s) is the same real number
+        // (-8s is exact), so it rounds identically; only the sign of an exact zero can
+        // differ from the two-step form, which no sum can see.
+        const float m8s = -8.0f * s;
+        const uint32_t even = w & 0x0f0f0f0fu, odd = (w >> 4) & 0x0f0f0f0fu;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            v[2 * i] = __builtin_fmaf((float)((even >> (8 * i)) & 0xffu), s, m8s);
+            v[2 * i + 1] = __builtin_fmaf((float)((odd >> (8 * i)) & 0xffu), s, m8s);
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = e2m1_to_f32((w >> (4 * i)) & 0xfu) * s;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) out4[i] = pack_bf16x2(v[2 * i], v[2 * i + 1]);
+}
+
+template <int FMT, bool CC>
+struct W256Flat4 {
+    const uint8_t* src[2];
+    const uint8_t* sc_base;
+    int64_t s_idx[2];    // scale index at K-step 0
+    int64_t kstep;       // bytes per K-step
+    int32_t s_kstep;     // !CC: scale entries per K-step
+    int32_t col0[2];     // CC: first column of the run at K-step 0
+    int gshift, sdt, tid;
+    float gs;
+    u32x2 raw[2];
+    uint32_t sraw[2];
+    __device__ __forceinline__ void init(const G256Args& g, const uint8_t* pk, const uint8_t* sc, float gscale, int n0, int tid_) {
+        tid = tid_; gshift = g.gshift; sdt = g.scale_dtype; gs = gscale; sc_base = sc;
+        const int spr = g.wcols >> gshift;  // scales per W row
+#pragma unroll
+        for (int p = 0; p < 2; ++p) {
+            const int u = tid + p * 512;
+            int wr, wc;
+            if (CC) { wr = min(n0 + (u >> 2), g.wrows - 1); wc = (u & 3) * 16; }
+            else { wr = u >> 4; wc = min(n0 + (u & 15) * 16, g.wcols - 16); }
+            src[p] = pk + (((int64_t)wr * g.wcols + wc) >> 1);
+            s_idx[p] = (int64_t)wr * spr + (CC ? 0 : (wc >> gshift));
+            col0[p] = wc;
+        }
+        kstep = CC ? F8_BK / 2 : (int64_t)F8_BK * g.wcols / 2;
+        s_kstep = F8_BK * spr;
+    }
+    __device__ __forceinline__ void load(int kt) {
+#pragma unroll
+        for (int p = 0; p < 2; ++p) {
+            raw[p] = *(const u32x2*)(src[p] + kt * kstep);
+            const int64_t si = CC ? s_idx[p] + ((col0[p] + kt * F8_BK) >> gshift) : s_idx[p] + (int64_t)kt * s_kstep;
+            sraw[p] = load_scale_raw(sc_base, si, sdt);
+        }
+    }
+    __device__ __forceinline__ void store(bf16_t* b, int p) {
+        float s = scale_from_raw(sraw[p], sdt);
+        if (FMT == XQ_FMT_NVFP4) s = s * gs;
+        uint32_t lo[4], hi[4];
+        decode8_4bit<FMT>(raw[p][0], s, lo);
+        decode8_4bit<FMT>(raw[p][1], s, hi);
+        store_run16<CC>(b, tid + p * 512, u32x4{lo[0], lo[1], lo[2], lo[3]}, u32x4{hi[0], hi[1], hi[2], hi[3]});
+    }
+};
+
+template <int FMT, bool CC> struct W256Sel { using type = W256Flat4<FMT, CC>; };
+template <bool CC> struct W256Sel<XQ_FMT_FP8, CC> { using type = W256Fp8<CC>; };
+
+// ---------------------------------------------------------------- the kernel
+template <int FMT, bool CC, bool GROUPED>
+__global__ void __launch_bounds__(512, 2) gemm_256_kernel(G256Args g) {
+    extern __shared__ __attribute__((aligned(16))) bf16_t smem[];
+    constexpr int B_STAGE = CC ? F8_B_STAGE_NT : F8_B_STAGE_NN;
+    bf16_t* As = smem;                    // 2 stages
+    bf16_t* Bs = smem + 2 * F8_A_STAGE;   // 2 stages
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 2, wn = wave & 3;   // wave tile: rows wm*128.., cols wn*64..
+
+    // ---- XCD-aware tile mapping: consecutive workgroup ids land on different XCDs, so
+    // give each XCD a contiguous range of logical tiles.  Dense: walk the logical tiles
+    // in groups of 4 row-tiles so concurrent tiles share operands in L2.  Grouped: walk
+    // row-tile by row-tile (all column tiles of a row tile, then the next row tile of the
+    // same expert) so an XCD stays on one expert's matrix.
+    int pid_m, pid_n;
+    {
+        const int nb = g.tiles_m * g.tiles_n;
+        int b = blockIdx.x;
+        const int per = nb >> 3;
+        int logical = (b < per * 8) ? (b & 7) * per + (b >> 3) : b;
+        if (GROUPED) {
+            pid_m = logical / g.tiles_n;
+            pid_n = logical - pid_m * g.tiles_n;
+        } else {
+            constexpr int GM = 4;
+            const int width = GM * g.tiles_n;
+            const int grp = logical / width, first_m = grp * GM;
+            const int gsz = min(g.tiles_m - first_m, GM);
+            const int in = logical - grp * width;
+            pid_m = first_m + in % gsz;
+            pid_n = in / gsz;
+        }
+    }
+    int e = 0;
+    int64_t row0, row_end;
+    if (GROUPED) {
+        int* sh_info = (int*)smem;
+        if (tid == 0) {
+            const int E = g.num_experts;
+            if (pid_m >= g.tiles256[E]) sh_info[0] = -1;
+            else {
+                int lo = 0, hi = E;  // tiles256[lo] <= pid_m < tiles256[lo + 1]
+                while (hi - lo > 1) { int mid = (lo + hi) >> 1; if (g.tiles256[mid] <= pid_m) lo = mid; else hi = mid; }
+                sh_info[0] = lo;
+                sh_info[1] = g.offsets[lo] + (pid_m - g.tiles256[lo]) * F8_BM;
+                sh_info[2] = g.offsets[lo + 1];
+            }
+        }
+        __syncthreads();
+        e = sh_info[0];
+        const int r0 = sh_info[1], r1 = sh_info[2];
+        __syncthreads();
+        if (e < 0) return;
+        row0 = r0;
+        row_end = r1;
+    } else {
+        row0 = (int64_t)pid_m * F8_BM;
+        row_end = g.M;
+    }
+    const int n0 = pid_n * F8_BN;
+
+    // ---- per-thread global addresses (fixed across K-steps except for the k offset)
+    const bf16_t* a_src[4];
+    int a_dst[4];
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        const int u = tid + p * 512;
+        int64_t r = row0 + (u >> 3);
+        r = r < row_end ? r : row_end - 1;
+        a_src[p] = g.A + r * g.lda + (u & 7) * 8;
+        a_dst[p] = swz(u >> 3, u & 7);
+    }
+    typename W256Sel<FMT, CC>::type wl;
+    wl.init(g, g.W + (int64_t)e * g.packed_stride, g.scales + (int64_t)e * g.scale_stride,
+            FMT == XQ_FMT_NVFP4 ? g.global_scale[e] : 1.0f, n0, tid);
+
+    u32x4 areg[4];
+    auto load_a = [&](int kt) {
+        const int k0 = kt * F8_BK;
+#pragma unroll
+        for (int p = 0; p < 4; ++p) areg[p] = *(const u32x4*)(a_src[p] + k0);
+    };
+    auto store_a = [&](bf16_t* a) {
+#pragma unroll
+        for (int p = 0; p < 4; ++p) *(u32x4*)(a + a_dst[p]) = areg[p];
+    };
+
+    f32x16 acc[4][2];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int q = 0; q < 16; ++q) acc[i][j][q] = 0.0f;
+
+    const int fr = lane & 31, fh = lane >> 5;
+    auto load_frags = [&](const bf16_t* a, const bf16_t* b, int ks, bool b_is_nt, bf16x8* af, bf16x8* bfr) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) af[i] = *(const bf16x8*)(a + swz(wm * 128 + i * 32 + fr, ks * 2 + fh));
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            if (CC || b_is_nt) bfr[j] = *(const bf16x8*)(b + swz(wn * 64 + j * 32 + fr, ks * 2 + fh));
+            else bfr[j] = lds_tr_frag(b, F8_NN_PITCH, ks * 16, wn * 64 + j * 32, lane);
+        }
+    };
+    auto mma = [&](const bf16x8* af, const bf16x8* bfr) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[j], af[i], acc[i][j], 0, 0, 0);
+    };
+
+    // Pipeline: at the top of iteration kt the registers hold tile kt+1 (loaded one
+    // whole iteration earlier, so the global latency is covered by a full tile of
+    // MFMAs) and the operand fragments of k16-step 0 of tile kt.  Tile kt+1 is
+    // stored/decoded into the other LDS stage and the loads of tile kt+2 are issued
+    // while steps 0..2 are multiplied; the single barrier of the iteration sits before
+    // the last step, whose MFMAs then cover both the barrier skew and the fetch of the
+    // next tile's first fragments.  (Every read of a stage completes before the barrier
+    // that precedes the next stores into it.)
+    const int nk = g.Kc / F8_BK;
+    bf16x8 af0[4], bf0[2], af1[4], bf1[2];
+    auto iteration = [&](int kt, bool have_next, bool have_next2) {
+        const bf16_t* a = As + (kt & 1) * F8_A_STAGE;
+        const bf16_t* b = Bs + (kt & 1) * B_STAGE;
+        bf16_t* an = As + ((kt + 1) & 1) * F8_A_STAGE;
+        bf16_t* bn = Bs + ((kt + 1) & 1) * B_STAGE;
+        // region 1: MFMAs of step 0 over the step-1 fragment reads, the A-tile stores and the next A loads
+        mma(af0, bf0);
+        load_frags(a, b, 1, false, af1, bf1);
+        if (have_next) store_a(an);
+        if (have_next2) load_a(kt + 2);
+        // interleave: one LDS read behind each of the first six MFMAs, then the stores and global loads
+        for (int q = 0; q < 6; ++q) { __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); }
+        for (int q = 0; q < 2; ++q) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x200, 2, 0);
+            __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        // region 2: MFMAs of step 1 over the weight decode + stores, the next weight loads, step-2 fragment reads
+        mma(af1, bf1);
+        if (have_next) { wl.store(bn, 0); wl.store(bn, 1); }
+        if (have_next2) wl.load(kt + 2);
+        load_frags(a, b, 2, false, af0, bf0);
+        __builtin_amdgcn_sched_barrier(0);
+        // region 3: MFMAs of step 2 over the step-3 fragment reads
+        mma(af0, bf0);
+        load_frags(a, b, 3, false, af1, bf1);
+        __builtin_amdgcn_sched_barrier(0);
+        __syncthreads();
+        // region 4: MFMAs of step 3 over the next tile's first fragment reads, which must have
+        // landed before the next iteration starts multiplying
+        if (have_next) load_frags(an, bn, 0, false, af0, bf0);
+        mma(af1, bf1);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    load_a(0);
+    wl.load(0);
+    store_a(As);
+    wl.store(Bs, 0);
+    wl.store(Bs, 1);
+    if (nk > 1) { load_a(1); wl.load(1); }
+    __syncthreads();
+    load_frags(As, Bs, 0, false, af0, bf0);
+    int kt = 0;
+    for (; kt + 2 < nk; ++kt) iteration(kt, true, true);
+    if (kt + 1 < nk) { iteration(kt, true, false); ++kt; }
+    iteration(kt, false, false);
+
+    // ---- low-rank side term: su[rows, rp] x lora_right[n, rp], both [row][k] tiles in stage 0
+    if (g.r_pad > 0) {
+        const int rp = g.r_pad, cpr = rp >> 3;  // 16-byte chunks per row
+        const bf16_t* lr = g.lora_right + (int64_t)e * g.Nout * rp;
+        for (int idx = tid; idx < 256 * cpr; idx += 512) {
+            const int r = idx / cpr, c = idx - r * cpr;
+            int64_t row = row0 + r;
+            row = row < row_end ? row : row_end - 1;
+            *(u32x4*)(As + swz(r, c)) = *(const u32x4*)(g.su + row * rp + c * 8);
+            int n = n0 + r;
+            n = n < g.Nout ? n : g.Nout - 1;
+            *(u32x4*)(Bs + swz(r, c)) = *(const u32x4*)(lr + (int64_t)n * rp + c * 8);
+        }
+        __syncthreads();
+        for (int ks = 0; ks < (rp >> 4); ++ks) {
+            bf16x8 af[4], bfr[2];
+            load_frags(As, Bs, ks, true, af, bfr);
+            mma(af, bfr);
+        }
+    }
+
+    // ---- epilogue: lane holds, per (i, j) tile, row m = fr and 4 x 4 consecutive columns
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int64_t row = row0 + wm * 128 + i * 32 + fr;
+        if (row >= row_end) continue;
+        bf16_t* crow = g.C + row * g.ldc;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+#pragma unroll
+            for (int q4 = 0; q4 < 4; ++q4) {
+                const int n = n0 + wn * 64 + j * 32 + 8 * q4 + 4 * fh;
+                if (n >= g.Nout) continue;  // Nout % 16 == 0: groups of 4 are all in or all out
+                float v0 = acc[i][j][4 * q4], v1 = acc[i][j][4 * q4 + 1], v2 = acc[i][j][4 * q4 + 2], v3 = acc[i][j][4 * q4 + 3];
+                if (g.bias) {
+                    v0 += bf16_to_f32(g.bias[n]); v1 += bf16_to_f32(g.bias[n + 1]);
+                    v2 += bf16_to_f32(g.bias[n + 2]); v3 += bf16_to_f32(g.bias[n + 3]);
+                }
+                *(u32x2*)(crow + n) = u32x2{pack_bf16x2(v0, v1), pack_bf16x2(v2, v3)};
+            }
+        }
+    }
+}
+
+}  // namespace xq

@@ -119,15 +119,19 @@ __global__ void __launch_bounds__(256) route_scan_kernel(int32_t* chunk_counts, 
     }
     __syncthreads();
     if (threadIdx.x == 0) {
-        int32_t o = 0, t = 0;
+        int32_t o = 0, t = 0, t2 = 0;
+        int32_t* tiles256 = tile_offsets + (E + 1);
         for (int e = 0; e < E; ++e) {
             offsets[e] = o;
             tile_offsets[e] = t;
+            tiles256[e] = t2;
             o += tot[e];
             t += (tot[e] + 127) / 128;
+            t2 += (tot[e] + 255) / 256;
         }
         offsets[E] = o;
         tile_offsets[E] = t;
+        tiles256[E] = t2;
     }
 }
 

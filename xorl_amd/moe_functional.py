@@ -27,7 +27,10 @@ def _s(dev):
 
 
 def route_build(selected_experts: Tensor, num_experts: int):
-    """-> counts [E], offsets [E+1], scatter_index [T*topk], tile_offsets [E+1] (all int32, device)."""
+    """-> counts [E], offsets [E+1], scatter_index [T*topk], tile_offsets [2*(E+1)] (all int32, device).
+
+    tile_offsets holds two row-tile schedules back to back: the prefix of ceil(count/128) and the
+    prefix of ceil(count/256)."""
     _C.require_hip(selected_experts)
     dev = selected_experts.device
     sel = selected_experts.reshape(-1).to(torch.int32).contiguous()
@@ -35,7 +38,7 @@ def route_build(selected_experts: Tensor, num_experts: int):
     L = _C.lib()
     counts = torch.empty(num_experts, dtype=torch.int32, device=dev)
     offsets = torch.empty(num_experts + 1, dtype=torch.int32, device=dev)
-    tile_offsets = torch.empty(num_experts + 1, dtype=torch.int32, device=dev)
+    tile_offsets = torch.empty(2 * (num_experts + 1), dtype=torch.int32, device=dev)
     sidx = torch.empty(n, dtype=torch.int32, device=dev)
     wsb = L.xq_route_workspace_bytes(n, num_experts)
     ws = torch.empty(wsb, dtype=torch.uint8, device=dev)
