@@ -203,7 +203,9 @@ int xq_factor_prep(const void* in, int in_dtype, int64_t rows_in, int64_t cols_i
  *       [E, p_width, r_out] (or [E, r_out, p_width] with transpose_out); zero
  *       for empty experts.  With offsets == NULL it is the dense form over all
  *       n_rows (one output; also the gradient of a factor shared by all
- *       experts), deterministic, using xq_lora_wgrad_workspace_bytes() scratch.
+ *       experts).  Both forms split the rows over blocks and add the pieces in
+ *       a fixed order (deterministic), in xq_lora_wgrad_workspace_bytes() bytes
+ *       of scratch (256-byte aligned, required).
  * Replace the small group_gemm_same_nk / group_gemm_same_mn calls of
  * ops/moe/lora.py:601-660 and :781-960. */
 int xq_grouped_lora_down(const void* a, int64_t lda, int64_t n_rows, const int32_t* offsets,

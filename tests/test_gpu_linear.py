@@ -50,6 +50,33 @@ def test_config0_int4_full_size(hip_device, tile_policy):
     assert torch.equal(m._dequantize_weight().cpu(), w_ref)
 
 
+@pytest.mark.parametrize("tile_policy", [1, 2], indirect=True)
+@pytest.mark.parametrize("fmt", ["block_fp8", "int4", "nvfp4"])
+def test_gemm_decode_bit_exact(hip_device, tile_policy, fmt):
+    """With X = I (and lora_B = 0) every output is a single product 1 * w, so the forward returns the
+    decoded weight itself and the dgrad of dY = I returns it transposed: the in-kernel decode of both
+    fused kernels, in both contraction directions, must equal the oracle's decode bit for bit."""
+    N = K = 512
+    m, w_ref = make_dense_module(fmt, N, K, 16, 32, seed=77, device=hip_device)
+    with torch.no_grad():
+        m.lora_B.zero_()
+    eye = torch.eye(K, dtype=torch.bfloat16, device=hip_device)
+    x = eye.clone().requires_grad_(True)
+    y = m(x)                                   # y[m, n] = w[n, m]
+    y.backward(eye)                            # dx[m, k] = sum_n I[m, n] w[n, k] = w[m, k]
+    wd = w_ref.to(hip_device)
+    assert torch.equal(y.detach().view(torch.int16), wd.t().contiguous().view(torch.int16)) or \
+        _equal_mod_zero_sign(y.detach(), wd.t())
+    assert torch.equal(x.grad.view(torch.int16), wd.view(torch.int16)) or _equal_mod_zero_sign(x.grad, wd)
+
+
+def _equal_mod_zero_sign(a, b):
+    """Bitwise equality except that a sum may return +0 where the decoded weight is -0."""
+    a16, b16 = a.contiguous().view(torch.int16), b.contiguous().view(torch.int16)
+    diff = a16 != b16
+    return bool(((a.float() == 0) & (b.float() == 0))[diff].all())
+
+
 def test_invariants(hip_device):
     m, w_ref = make_dense_module("block_fp8", 384, 256, 16, 32, seed=5, device=hip_device, bias=True)
     x = gen((3, 7, 256), 1.0, 13, torch.bfloat16).to(hip_device)        # leading dims are kept

@@ -142,21 +142,33 @@ __device__ __forceinline__ float scale_from_raw(uint32_t raw, int dtype) {
     return e4m3_to_f32((uint8_t)raw);
 }
 
-// value of 8 e2m1 codes: the magnitude code c = nib & 7 indexes the table
-// {0, .5, 1, 1.5, 2, 3, 4, 6}; built as fp32 bits, sign from bit 3.
+// 8 codes of one dword -> 8 bf16 (4 packed dwords), each bf16(fl(value(code) * s)).
+//   int4:  value = nib - 8.  fma(nib, s, -8s) is the same real number as (nib - 8) * s
+//          (-8s is exact), so it rounds identically; only the sign of an exact zero can
+//          differ from the two-step form, which no sum can see.
+//   nvfp4: the 3 magnitude bits placed at fp32 bits 22..24 form a float (subnormal for
+//          codes 0 and 1) equal to e2m1(code) * 2^-126 -- e2m1 is a tiny IEEE format, so
+//          one exact multiply by 2^126 decodes it, subnormals included; that factor is
+//          folded into the scale (s126 = s * 2^126, exact while |s| < 2) and the product
+//          is rounded once, like the reference's fl(e2m1 * s).  Bit 3 is the sign.
 template <int FMT>
 __device__ __forceinline__ void decode8_4bit(uint32_t w, float s, uint32_t* out4) {
     float v[8];
     if (FMT == XQ_FMT_INT4) {
-        // (nib - 8) * s with a single rounding: fma(nib, s, -8s) is the same real number
-        // (-8s is exact), so it rounds identically; only the sign of an exact zero can
-        // differ from the two-step form, which no sum can see.
         const float m8s = -8.0f * s;
         const uint32_t even = w & 0x0f0f0f0fu, odd = (w >> 4) & 0x0f0f0f0fu;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             v[2 * i] = __builtin_fmaf((float)((even >> (8 * i)) & 0xffu), s, m8s);
             v[2 * i + 1] = __builtin_fmaf((float)((odd >> (8 * i)) & 0xffu), s, m8s);
+        }
+    } else if (__builtin_fabsf(s) < 2.0f) {
+        const float s126 = s * 0x1p126f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const uint32_t mag = (4 * i <= 22 ? (w << (22 - 4 * i)) : (w >> (4 * i - 22))) & 0x01c00000u;
+            const uint32_t sgn = (w << (28 - 4 * i)) & 0x80000000u;
+            v[i] = __uint_as_float(mag | sgn) * s126;
         }
     } else {
 #pragma unroll

@@ -212,49 +212,37 @@ struct TnArgs {
 constexpr int TN_PP = 128 + 16;  // Ps pitch (bf16 elements): 288 B rows
 constexpr int TN_QP = 80;        // Qs pitch: 160 B rows
 
-template <int NT>
-__global__ void __launch_bounds__(256) tn_kernel(TnArgs g) {
-    __shared__ __attribute__((aligned(16))) bf16_t Ps[32 * TN_PP];
-    __shared__ __attribute__((aligned(16))) bf16_t Qs[32 * TN_QP];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int64_t c0 = (int64_t)blockIdx.x * 128;
-    int64_t m_begin, m_end;
-    float* out;
-    if (g.offsets) {
-        m_begin = g.offsets[blockIdx.y];
-        m_end = g.offsets[blockIdx.y + 1];
-        out = g.out + (int64_t)blockIdx.y * g.width * g.r_out;
-    } else {
-        m_begin = (int64_t)blockIdx.y * g.rows_per_split;
-        m_end = m_begin + g.rows_per_split;
-        m_end = m_end < g.n_rows ? m_end : g.n_rows;
-        out = g.out + (int64_t)blockIdx.y * g.width * g.r_pad;
-    }
-    f32x16 acc[NT];
-#pragma unroll
-    for (int n = 0; n < NT; ++n)
-#pragma unroll
-        for (int q = 0; q < 16; ++q) acc[n][q] = 0.0f;
+constexpr int TN_CHUNK = 1024;   // grouped: rows per block (global row chunks, cut at expert boundaries)
 
+// acc += P[m_begin:m_end, c0 + wave*32 .. +32]^T . Q[m_begin:m_end, :]; the next 32-row tile is
+// fetched into registers while the current one is multiplied out of LDS.
+template <int NT>
+__device__ __forceinline__ void tn_accumulate(const TnArgs& g, int64_t c0, int64_t m_begin, int64_t m_end, bf16_t* Ps,
+                                              bf16_t* Qs, f32x16* acc) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int pr = tid >> 4, pc = (tid & 15) * 8;  // P tile: rows pr, pr+16; 8 cols at pc
     const bool pcol_ok = c0 + pc < g.width;        // width % 8 == 0
     const int qchunks = g.r_pad / 8;
     const int qr = tid / qchunks, qc = (tid % qchunks) * 8;
     const bool q_thread = tid < 32 * qchunks;
     const u32x4 z = {0, 0, 0, 0};
-
-    for (int64_t m = m_begin; m < m_end; m += 32) {
-        u32x4 p0 = z, p1 = z, qv = z;
+    u32x4 p0 = z, p1 = z, qv = z;
+    auto fetch = [&](int64_t m) {
+        p0 = z; p1 = z; qv = z;
         if (pcol_ok) {
             if (m + pr < m_end) p0 = *(const u32x4*)(g.P + (m + pr) * g.ldp + c0 + pc);
             if (m + pr + 16 < m_end) p1 = *(const u32x4*)(g.P + (m + pr + 16) * g.ldp + c0 + pc);
         }
         if (q_thread && m + qr < m_end) qv = *(const u32x4*)(g.Q + (m + qr) * g.r_pad + qc);
-        __syncthreads();  // previous iteration's fragment reads are done
+    };
+    if (m_begin < m_end) fetch(m_begin);
+    for (int64_t m = m_begin; m < m_end; m += 32) {
+        __syncthreads();  // previous tile's fragment reads are done
         *(u32x4*)(Ps + pr * TN_PP + pc) = p0;
         *(u32x4*)(Ps + (pr + 16) * TN_PP + pc) = p1;
         if (q_thread) *(u32x4*)(Qs + qr * TN_QP + qc) = qv;
         __syncthreads();
+        if (m + 32 < m_end) fetch(m + 32);
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) {
             bf16x8 a = lds_tr_frag(Ps, TN_PP, ks * 16, wave * 32, lane);
@@ -265,24 +253,109 @@ __global__ void __launch_bounds__(256) tn_kernel(TnArgs g) {
             }
         }
     }
+}
+
+// out[c][j] (pitch = row length of the destination) or, transposed, out[j][c]; j < r_lim
+template <int NT>
+__device__ __forceinline__ void tn_write(const f32x16* acc, float* out, int64_t c0, int64_t width, int r_lim, int pitch,
+                                         bool transposed) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int rgrp = (lane >> 5) * 4;
 #pragma unroll
     for (int n = 0; n < NT; ++n) {
-        int j = n * 32 + (lane & 31);
+        const int j = n * 32 + (lane & 31);
+        if (j >= r_lim) continue;
 #pragma unroll
         for (int q = 0; q < 16; ++q) {
-            int64_t c = c0 + wave * 32 + (q & 3) + rgrp + 8 * (q >> 2);
-            if (c >= g.width) continue;
-            if (g.offsets) {
-                if (j < g.r_out) {
-                    if (g.transpose_out) out[(int64_t)j * g.width + c] = acc[n][q];
-                    else out[c * g.r_out + j] = acc[n][q];
-                }
-            } else if (j < g.r_pad) {
-                out[c * g.r_pad + j] = acc[n][q];
-            }
+            const int64_t c = c0 + wave * 32 + (q & 3) + rgrp + 8 * (q >> 2);
+            if (c >= width) continue;
+            if (transposed) out[(int64_t)j * width + c] = acc[n][q];
+            else out[c * pitch + j] = acc[n][q];
         }
     }
+}
+
+// dense: block (col tile, row split) -> partial[split][width][r_pad]
+template <int NT>
+__global__ void __launch_bounds__(256) tn_kernel(TnArgs g) {
+    __shared__ __attribute__((aligned(16))) bf16_t Ps[32 * TN_PP];
+    __shared__ __attribute__((aligned(16))) bf16_t Qs[32 * TN_QP];
+    const int64_t c0 = (int64_t)blockIdx.x * 128;
+    const int64_t m_begin = (int64_t)blockIdx.y * g.rows_per_split;
+    int64_t m_end = m_begin + g.rows_per_split;
+    m_end = m_end < g.n_rows ? m_end : g.n_rows;
+    f32x16 acc[NT];
+#pragma unroll
+    for (int n = 0; n < NT; ++n)
+#pragma unroll
+        for (int q = 0; q < 16; ++q) acc[n][q] = 0.0f;
+    tn_accumulate<NT>(g, c0, m_begin, m_end, Ps, Qs, acc);
+    tn_write<NT>(acc, g.out + (int64_t)blockIdx.y * g.width * g.r_pad, c0, g.width, g.r_pad, g.r_pad, false);
+}
+
+// grouped: block (col tile, chunk of TN_CHUNK global rows).  The chunk is walked expert by expert;
+// an expert that lies wholly inside the chunk is written to out[e] directly, a piece of an expert
+// that continues from the previous chunk goes to partial[chunk][0], one that continues into the
+// next chunk to partial[chunk][1] (tn_grouped_reduce_kernel adds the pieces in chunk order).
+template <int NT>
+__global__ void __launch_bounds__(256) tn_grouped_kernel(TnArgs g, int32_t num_experts, float* partial) {
+    __shared__ __attribute__((aligned(16))) bf16_t Ps[32 * TN_PP];
+    __shared__ __attribute__((aligned(16))) bf16_t Qs[32 * TN_QP];
+    __shared__ int sh_e;
+    const int64_t c0 = (int64_t)blockIdx.x * 128;
+    const int64_t r_begin = (int64_t)blockIdx.y * TN_CHUNK;
+    int64_t r_end = r_begin + TN_CHUNK;
+    r_end = r_end < g.n_rows ? r_end : g.n_rows;
+    if (threadIdx.x == 0) {
+        int lo = 0, hi = num_experts;  // last e with offsets[e] <= r_begin
+        while (hi - lo > 1) { int mid = (lo + hi) >> 1; if (g.offsets[mid] <= r_begin) lo = mid; else hi = mid; }
+        sh_e = lo;
+    }
+    __syncthreads();
+    int e = sh_e;
+    int64_t m = r_begin;
+    while (m < r_end && e < num_experts) {
+        const int64_t eb = g.offsets[e], ee = g.offsets[e + 1];
+        const int64_t seg_end = ee < r_end ? ee : r_end;
+        if (seg_end <= m) { ++e; continue; }   // expert without rows (or already passed)
+        f32x16 acc[NT];
+#pragma unroll
+        for (int n = 0; n < NT; ++n)
+#pragma unroll
+            for (int q = 0; q < 16; ++q) acc[n][q] = 0.0f;
+        tn_accumulate<NT>(g, c0, m, seg_end, Ps, Qs, acc);
+        if (eb >= r_begin && ee <= r_end)
+            tn_write<NT>(acc, g.out + (int64_t)e * g.width * g.r_out, c0, g.width, g.r_out, g.r_out, g.transpose_out != 0);
+        else
+            tn_write<NT>(acc, partial + ((int64_t)blockIdx.y * 2 + (eb < r_begin ? 0 : 1)) * g.width * g.r_pad, c0, g.width,
+                         g.r_pad, g.r_pad, false);
+        m = seg_end;
+        ++e;
+    }
+}
+
+// out[e] for the experts the chunk walk did not finish: zero for an expert without rows, the sum of
+// its pieces in chunk order for one that spans several chunks.
+__global__ void __launch_bounds__(256) tn_grouped_reduce_kernel(const float* partial, const int32_t* offsets, int64_t width,
+                                                                int r_pad, int r_out, int transpose_out, float* out) {
+    const int e = blockIdx.y;
+    const int64_t b = offsets[e], en = offsets[e + 1];
+    const int64_t ch0 = b / TN_CHUNK, ch1 = en > b ? (en - 1) / TN_CHUNK : ch0;
+    if (en > b && ch0 == ch1) return;   // written directly
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (t >= width * r_pad) return;
+    const int64_t c = t / r_pad;
+    const int j = (int)(t - c * r_pad);
+    if (j >= r_out) return;
+    float s = 0.0f;
+    if (en > b) {
+        const int64_t per = width * r_pad;
+        s = partial[(ch0 * 2 + 1) * per + t];
+        for (int64_t ch = ch0 + 1; ch <= ch1; ++ch) s += partial[(ch * 2) * per + t];
+    }
+    float* o = out + (int64_t)e * width * r_out;
+    if (transpose_out) o[(int64_t)j * width + c] = s;
+    else o[c * r_out + j] = s;
 }
 
 // sums the dense partials in split order: out[c][j] or out[j][c], j < r_out
@@ -309,7 +382,9 @@ static int tn_splits(int64_t n_rows, int64_t width) {
 }
 
 int64_t tn_partial_bytes(int64_t n_rows, int64_t width, int r_pad) {
-    return (int64_t)tn_splits(n_rows, width) * width * r_pad * 4;
+    const int64_t dense = (int64_t)tn_splits(n_rows, width) * width * r_pad * 4;
+    const int64_t grouped = xq_cdiv(n_rows > 0 ? n_rows : 1, TN_CHUNK) * 2 * width * r_pad * 4;
+    return dense > grouped ? dense : grouped;
 }
 
 int launch_tn(const bf16_t* P, int64_t ldp, int64_t width, const bf16_t* Q, int r_pad, int r_out, int64_t n_rows,
@@ -320,14 +395,19 @@ int launch_tn(const bf16_t* P, int64_t ldp, int64_t width, const bf16_t* Q, int 
     if (width == 0 || r_out == 0) return XQ_OK;
     TnArgs g{P, ldp, width, Q, r_pad, r_out, n_rows, 0, transpose_out ? 1 : 0, out, offsets};
     unsigned col_tiles = (unsigned)xq_cdiv(width, 128);
+    XQ_REQUIRE(partial != nullptr, "tn: partial workspace is NULL");
     if (offsets) {
-        dim3 grid(col_tiles, (unsigned)num_experts);
-        if (r_pad <= 32) tn_kernel<1><<<grid, 256, 0, stream>>>(g);
-        else tn_kernel<2><<<grid, 256, 0, stream>>>(g);
-        XQ_CHECK_LAUNCH("tn(grouped)");
+        if (n_rows > 0) {
+            dim3 grid(col_tiles, (unsigned)xq_cdiv(n_rows, TN_CHUNK));
+            if (r_pad <= 32) tn_grouped_kernel<1><<<grid, 256, 0, stream>>>(g, num_experts, partial);
+            else tn_grouped_kernel<2><<<grid, 256, 0, stream>>>(g, num_experts, partial);
+            XQ_CHECK_LAUNCH("tn(grouped)");
+        }
+        dim3 rgrid((unsigned)xq_cdiv(width * r_pad, 256), (unsigned)num_experts);
+        tn_grouped_reduce_kernel<<<rgrid, 256, 0, stream>>>(partial, offsets, width, r_pad, r_out, transpose_out ? 1 : 0, out);
+        XQ_CHECK_LAUNCH("tn(grouped reduce)");
         return XQ_OK;
     }
-    XQ_REQUIRE(partial != nullptr, "tn: partial workspace is NULL");
     int S = tn_splits(n_rows, width);
     int64_t rps = xq_cdiv(xq_cdiv(n_rows, S), 32) * 32;
     g.rows_per_split = rps;

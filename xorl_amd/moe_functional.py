@@ -110,9 +110,7 @@ def _wgrad(P: Tensor, Q: Tensor, r: int, offsets: Optional[Tensor], E: int, tran
     n_out = E if offsets is not None else 1
     shape = (n_out, r, width) if transpose_out else (n_out, width, r)
     out = torch.empty(*shape, dtype=torch.float32, device=P.device)
-    ws = None
-    if offsets is None:
-        ws = torch.empty(L.xq_lora_wgrad_workspace_bytes(R, width, rp), dtype=torch.uint8, device=P.device)
+    ws = torch.empty(L.xq_lora_wgrad_workspace_bytes(R, width, rp), dtype=torch.uint8, device=P.device)
     _C.check(L.xq_grouped_lora_wgrad(P.data_ptr(), P.stride(0), width, Q.data_ptr(), rp, r, R, _C.ptr(offsets), E,
                                      int(transpose_out), out.data_ptr(), _C.ptr(ws), _s(P.device)))
     return out
