@@ -33,6 +33,14 @@ METRIC = "QLoRA dequant-GEMM+LoRA fwd/bwd TFLOP/s & % MFMA/HBM peak, 1 GPU"
 M, H, I, R, ALPHA = 8192, 4096, 12288, 32, 64
 BF16_MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense bf16, published
 
+# HBM-side bytes per launch of each config's roofline kernel, from the committed counter runs
+# (rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE, each scaled by what the same counter reads for a plain
+# 256 MiB -> 256 MiB copy; the files under profiles/ hold the figures and the commands).  A config that
+# has no counter run reports null.  --traffic-bytes overrides.
+MEASURED_TRAFFIC_BYTES = {
+    1: 904.9 * 2 ** 20,   # gemm_256_kernel<fp8>: mean of the forward (927.9 MiB) and dgrad (882.0 MiB) launches
+}
+
 
 def step_flops(m: int) -> float:
     per = lambda K, N: 4.0 * m * K * N + 6.0 * m * R * (K + N)
@@ -158,7 +166,7 @@ def other_config(cfg: int, dev):
                 m(xs[k]).backward(dys[k])
         return (step, sum(lin_flops(Mtok, K, N, 16) for (N, K) in shapes.values()), False,
                 "configs[2]: nvfp4 QLoRA Qwen3-32B attention projections q/k/v/o, hidden 5120, M=4096, r=16, fwd+bwd",
-                "gemm_tile_kernel<nvfp4> (fused dequant-GEMM, forward and dgrad launches)")
+                "gemm_256_kernel<nvfp4> (q/o and the k/v dgrad) and gemm_tile_kernel<nvfp4> (k/v forward): fused dequant-GEMM, forward and dgrad launches")
     if cfg == 3:
         from xorl_amd.qlora import BlockFP8QLoRAMoeExperts
 
@@ -188,7 +196,7 @@ def other_config(cfg: int, dev):
                 f"configs[3]: grouped block_fp8 QLoRA Qwen3-30B-A3B experts, E=128, hidden 2048, intermediate 768, "
                 f"top-8 of 16384 tokens, Zipf(1.1) counts (max {int(counts.max())}, {int((counts == 0).sum())} empty), "
                 f"per-expert r=16, fwd+bwd",
-                "gemm_tile_kernel<fp8, grouped> (fused dequant grouped GEMM, forward and dgrad launches)")
+                "gemm_256_kernel<fp8, grouped> (fused dequant grouped GEMM, forward and dgrad launches)")
     if cfg == 4:
         shapes = {"q": (4096, 4096), "kv": (1024, 4096), "gate_up": (12288, 4096), "down": (4096, 12288)}
         cases, total = [], 0.0
@@ -211,6 +219,19 @@ def other_config(cfg: int, dev):
     raise SystemExit(f"bench.py: unknown --config {cfg}")
 
 
+def calibrate_copy(dev):
+    """One plain elementwise copy of known traffic: 256 MiB read + 256 MiB written."""
+    src = torch.ones(64 << 20, dtype=torch.float32, device=dev)
+    dst = torch.empty_like(src)
+    torch.mul(src, 1.0, out=dst)
+    torch.cuda.synchronize()
+    del src, dst
+
+
+def traffic_of(args):
+    return args.traffic_bytes if args.traffic_bytes is not None else MEASURED_TRAFFIC_BYTES.get(args.config)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -225,7 +246,7 @@ def main():
                          "run (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE) holds a kernel of known traffic to scale by")
     ap.add_argument("--traffic-bytes", type=float, default=None,
                     help="HBM bytes per launch of the roofline kernel from such counter runs (reported as "
-                         "roofline.traffic; null when not given)")
+                         "roofline.traffic; default: the committed measurement of that config, else null)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs the QLoRA path on ONE GPU; --gpus must be 1 "
@@ -258,11 +279,7 @@ def main():
 
     L = _C.lib()
     if args.calibrate_copy:
-        src = torch.ones(64 << 20, dtype=torch.float32, device=dev)      # 256 MiB read + 256 MiB written
-        dst = torch.empty_like(src)
-        torch.mul(src, 1.0, out=dst)
-        torch.cuda.synchronize()
-        del src, dst
+        calibrate_copy(dev)
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -296,8 +313,9 @@ def main():
                                "intermediate 12288, LoRA r=32 on gate/up/down, SwiGLU",
                    "tokens": M, "hidden": H, "intermediate": I, "lora_r": R, "format": "block_fp8"},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": BF16_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / BF16_MFMA_PEAK_TFLOPS, "traffic": args.traffic_bytes,
-                     "kernel": "gemm_fp8_256_kernel<true|false> (fused fp8 dequant-GEMM, forward and dgrad launches)",
+                     "frac": achieved / BF16_MFMA_PEAK_TFLOPS, "traffic": traffic_of(args),
+                     "kernel": "gemm_256_kernel<fp8, contract_cols true|false, dense> (fused fp8 dequant-GEMM, "
+                               "forward and dgrad launches)",
                      "launches": n.value, "avg_launch_ms": ms.value / max(n.value, 1)},
         "cpu_baseline": cpu,
     }
@@ -309,6 +327,8 @@ def run_other(args, dev):
 
     step, work, is_bytes, workload, kernel = other_config(args.config, dev)
     L = _C.lib()
+    if args.calibrate_copy:
+        calibrate_copy(dev)
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -328,7 +348,7 @@ def run_other(args, dev):
         "warmup": args.warmup, "ms_per_step": dt * 1e3, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic", "config": {"workload": workload},
         "roofline": {"bound": "hbm" if is_bytes else "mfma", "achieved": achieved, "peak": peak, "unit": unit,
-                     "frac": achieved / peak, "traffic": args.traffic_bytes, "kernel": kernel,
+                     "frac": achieved / peak, "traffic": traffic_of(args), "kernel": kernel,
                      "launches": n.value, "avg_launch_ms": ms.value / max(n.value, 1)},
         "cpu_baseline": None}))
 
