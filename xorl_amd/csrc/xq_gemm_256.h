@@ -146,11 +146,9 @@ __device__ __forceinline__ float scale_from_raw(uint32_t raw, int dtype) {
 //   int4:  value = nib - 8.  fma(nib, s, -8s) is the same real number as (nib - 8) * s
 //          (-8s is exact), so it rounds identically; only the sign of an exact zero can
 //          differ from the two-step form, which no sum can see.
-//   nvfp4: the 3 magnitude bits placed at fp32 bits 22..24 form a float (subnormal for
-//          codes 0 and 1) equal to e2m1(code) * 2^-126 -- e2m1 is a tiny IEEE format, so
-//          one exact multiply by 2^126 decodes it, subnormals included; that factor is
-//          folded into the scale (s126 = s * 2^126, exact while |s| < 2) and the product
-//          is rounded once, like the reference's fl(e2m1 * s).  Bit 3 is the sign.
+//   nvfp4: v_cvt_scalef32_pk_f32_fp4 with scale 1.0 returns the exact e2m1 values of the two
+//          codes of a byte (low nibble first); each is multiplied by s in fp32 and rounded
+//          once, like the reference's fl(e2m1 * s).
 template <int FMT>
 __device__ __forceinline__ void decode8_4bit(uint32_t w, float s, uint32_t* out4) {
     float v[8];
@@ -162,17 +160,16 @@ __device__ __forceinline__ void decode8_4bit(uint32_t w, float s, uint32_t* out4
             v[2 * i] = __builtin_fmaf((float)((even >> (8 * i)) & 0xffu), s, m8s);
             v[2 * i + 1] = __builtin_fmaf((float)((odd >> (8 * i)) & 0xffu), s, m8s);
         }
-    } else if (__builtin_fabsf(s) < 2.0f) {
-        const float s126 = s * 0x1p126f;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const uint32_t mag = (4 * i <= 22 ? (w << (22 - 4 * i)) : (w >> (4 * i - 22))) & 0x01c00000u;
-            const uint32_t sgn = (w << (28 - 4 * i)) & 0x80000000u;
-            v[i] = __uint_as_float(mag | sgn) * s126;
-        }
     } else {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) v[i] = e2m1_to_f32((w >> (4 * i)) & 0xfu) * s;
+        for (int i = 0; i < 4; ++i) {
+            f32x2 x = i == 0 ? __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 0)
+                    : i == 1 ? __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 1)
+                    : i == 2 ? __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 2)
+                             : __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 3);
+            v[2 * i] = x[0] * s;
+            v[2 * i + 1] = x[1] * s;
+        }
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) out4[i] = pack_bf16x2(v[2 * i], v[2 * i + 1]);

@@ -8,10 +8,20 @@
 // lane issues per chunk (two for 4-bit formats) cover whole 128-byte lines and
 // every line is used once.  The bytes are decoded in registers to the exact bf16
 // value of the reference decoder and fed to v_mfma_f32_32x32x16_bf16 against x
-// fragments read straight from global memory (x is small and stays in L2).
-// A block owns 32 weight rows and all of K; its eight waves each stream one
-// eighth of K and the partial sums meet in LDS in a fixed order (no atomics
-// on the output, no device-scope fences).
+// fragments.  x is small and L2 resident, but every block needs all of it: it is
+// fetched with coalesced 16-byte loads (16 lanes per 256-byte row piece) and turned
+// into operand fragments through a wave-private, padded LDS tile -- per-lane
+// row-strided loads of x would cost more address-unit cycles than the whole weight
+// stream.
+// A block owns 32 weight rows and all of K; its NW waves (8, or 4 when there are
+// more slabs than CUs) each stream 1/NW of K and the partial sums meet in LDS
+// in a fixed order (no atomics, no device-scope fences: deterministic).  Loads are
+// issued a whole batch at a time -- packed codes, scales and the x fragments of
+// the batch together -- into one of two register sets, so the next batch is in
+// flight while the current one is decoded and multiplied.
+// The low-rank term needs one small launch before it: su = x . A^T (fp32), one
+// block whose 16 waves split K; both kernels read the LoRA factors in their own
+// dtype (fp32 or bf16), so nothing is repacked or zeroed per call.
 #include "xq_common.h"
 #include "xq_lora.h"
 
@@ -27,8 +37,8 @@ struct SkinnyArgs {
     int32_t group, scale_dtype;
     const float* su_f32;       // [M, r_pad] fp32 sums of x . A^T (unscaled) or NULL
     float su_scale;
-    const bf16_t* lora_right;  // [N, r_pad]
-    int32_t r_pad;
+    const void* lora_B;        // [N, r] fp32 or bf16
+    int32_t lora_f32, r, r_pad;
     const bf16_t* bias;
     bf16_t* y;
     int64_t ldy;
@@ -68,38 +78,51 @@ __device__ __forceinline__ bf16x8 decode8(uint32_t w0, uint32_t w1, float s0, fl
     return __builtin_bit_cast(bf16x8, r);
 }
 
-// One block = 32*NT weight rows x the whole K, SK_NW waves each streaming 1/SK_NW of K
-// (in-block split-K: no atomics, no fences, fixed summation order).  x fragments are read
-// straight from global memory (it is small and L2 resident); rows >= M are never touched.
-constexpr int SK_NW = 8;   // waves per block; each streams 1/SK_NW of K
+// 8 consecutive LoRA factor entries (fp32 or bf16 storage) -> one MFMA operand; entries at or
+// beyond `limit` (counted from the first) are zero
+__device__ __forceinline__ bf16x8 factor_frag(const void* base, int64_t idx, bool f32, int limit) {
+    uint32_t o[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        float lo = 0.0f, hi = 0.0f;
+        if (2 * e < limit) lo = f32 ? ((const float*)base)[idx + 2 * e] : bf16_to_f32(((const bf16_t*)base)[idx + 2 * e]);
+        if (2 * e + 1 < limit) hi = f32 ? ((const float*)base)[idx + 2 * e + 1] : bf16_to_f32(((const bf16_t*)base)[idx + 2 * e + 1]);
+        o[e] = pack_bf16x2(lo, hi);
+    }
+    u32x4 r = {o[0], o[1], o[2], o[3]};
+    return __builtin_bit_cast(bf16x8, r);
+}
 
-// One block = 32 weight rows x the whole K, SK_NW waves each streaming 1/SK_NW of K
-// (in-block split-K: no atomics, no fences, fixed summation order).  A wave fetches its
-// codes in batches of 8 KB (all loads of a batch are issued before any is used) and reads
-// its x fragments from global memory just in time (x is small and L1/L2 resident).
-template <int FMT, int MT>
-__global__ void __launch_bounds__(SK_NW * 64) skinny_kernel(SkinnyArgs g) {
-    extern __shared__ __attribute__((aligned(16))) float red[];   // [SK_NW waves][MT*16 regs][64 lanes]
+// One block = 32 weight rows x the whole K, NW waves each streaming 1/NW of K (in-block
+// split-K: no atomics, no fences, fixed summation order).  x fragments are read from global
+// memory (coalesced, see the top of the file) together with the codes of the same batch.
+template <int FMT, int MT, int NW>
+__global__ void __launch_bounds__(NW * 64) skinny_kernel(SkinnyArgs g) {
+    extern __shared__ __attribute__((aligned(16))) float red[];   // [NW waves][MT*16 regs][64 lanes]
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: keeps the K-range loop on scalar branches
     const int fr = lane & 31, fh = lane >> 5;
     const int n0 = blockIdx.x * 32;
     constexpr int EB = FMT == XQ_FMT_FP8 ? 1 : 2;      // elements per byte
     constexpr int NLOAD = FMT == XQ_FMT_FP8 ? 4 : 2;   // 16-byte loads per lane per 128-k chunk
-    constexpr int BC = FMT == XQ_FMT_FP8 ? 2 : 4;      // chunks per batch (8 x 16 B per lane)
+    constexpr int BC = 2 / MT;                         // chunks per batch (per register set)
+    constexpr int NSC = FMT == XQ_FMT_NVFP4 ? 4 : 1;   // scale registers per chunk
     const float gsc = FMT == XQ_FMT_NVFP4 ? g.global_scale[0] : 1.0f;
+    // int4 groups shorter than a lane's 64-element run are looked up per 8 elements at use
+    const bool int4_small_group = FMT == XQ_FMT_INT4 && g.group < 64;
 
     int n = n0 + fr;
     n = n < g.N ? n : g.N - 1;
     const uint8_t* wrow = g.packed + ((int64_t)n * g.K + fh * 64) / EB;
-    // Lanes whose row m is >= M read x row 0 instead (no per-lane branches): column m of the
-    // product depends only on x row m, and columns >= M are never stored.
-    const bf16_t* xg[MT];
-#pragma unroll
-    for (int i = 0; i < MT; ++i) {
-        const int m = i * 32 + fr;
-        xg[i] = g.x + (int64_t)(m < g.M ? m : 0) * g.ldx + fh * 64;
-    }
+    // x chunk tile of this wave: [MT*32 rows][128 k] bf16, rows padded to 272 B so that the 16 lanes
+    // of a b128 read phase (consecutive rows, same column piece) fall on distinct banks.  Rows >= M are
+    // never written: they feed only output columns >= M, which are never stored.
+    constexpr int XP = 136;                                     // row pitch in bf16 elements
+    bf16_t* xs = (bf16_t*)red + wave * (MT * 32 * XP);
+    const int xrow = lane >> 4, xpiece = lane & 15;             // coalesced fetch: 4 rows x 16 pieces per instruction
+    const bf16_t* xg = g.x + (int64_t)xrow * g.ldx + xpiece * 8;
+    const int64_t xstep = 4 * g.ldx;
+    const int mrows = g.M;
 
     f32x16 acc[MT];
 #pragma unroll
@@ -107,99 +130,127 @@ __global__ void __launch_bounds__(SK_NW * 64) skinny_kernel(SkinnyArgs g) {
 #pragma unroll
         for (int q = 0; q < 16; ++q) acc[i][q] = 0.0f;
 
-    // low-rank operands (last wave only), loaded now so their latency hides under the weight stream
-    const bool lora_wave = g.r_pad > 0 && wave == SK_NW - 1;
-    bf16x8 lb[4], ls[MT][4];
-    if (lora_wave) {
-#pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
-            if (ks < (g.r_pad >> 4)) {
-                lb[ks] = *(const bf16x8*)(g.lora_right + (int64_t)n * g.r_pad + ks * 16 + fh * 8);
-#pragma unroll
-                for (int i = 0; i < MT; ++i) {
-                    const int m = i * 32 + fr;
-                    const float* sp = g.su_f32 + (int64_t)(m < g.M ? m : 0) * g.r_pad + ks * 16 + fh * 8;
-                    uint32_t o[4];
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) o[e] = pack_bf16x2(sp[2 * e] * g.su_scale, sp[2 * e + 1] * g.su_scale);
-                    u32x4 r = {o[0], o[1], o[2], o[3]};
-                    ls[i][ks] = __builtin_bit_cast(bf16x8, r);
-                }
-            }
-        }
-    }
-
     const int ct = g.K >> 7;                                   // 128-element chunks in K
-    const int c_begin = (ct * wave) / SK_NW, c_end = (ct * (wave + 1)) / SK_NW;
+    const int c_begin = (ct * wave) / NW, c_end = (ct * (wave + 1)) / NW;
 
-    for (int c0 = c_begin; c0 < c_end; c0 += BC) {
+    struct Batch {
         u32x4 w[BC][NLOAD];
-        float sc[BC];
-        // ---- issue every load of the batch
+        uint32_t sc[BC][NSC];
+        u32x4 xr[BC][MT * 8];
+    };
+    auto issue = [&](Batch& B, int c0) {
 #pragma unroll
         for (int b = 0; b < BC; ++b) {
             if (c0 + b < c_end) {
                 const int c = c0 + b, k0 = c * 128 + fh * 64;
 #pragma unroll
-                for (int i = 0; i < NLOAD; ++i) w[b][i] = *(const u32x4*)(wrow + (int64_t)c * (128 / EB) + i * 16);
-                sc[b] = 0.0f;
-                if (FMT == XQ_FMT_FP8) sc[b] = ((const float*)g.scales)[(n >> 7) * ((g.K + 127) >> 7) + (k0 >> 7)];
-                else if (FMT == XQ_FMT_INT4 && g.group >= 64) sc[b] = load_scale(g.scales, ((int64_t)n * g.K + k0) / g.group, g.scale_dtype);
+                for (int i = 0; i < NLOAD; ++i) B.w[b][i] = *(const u32x4*)(wrow + (int64_t)c * (128 / EB) + i * 16);
+                if (FMT == XQ_FMT_FP8) B.sc[b][0] = ((const uint32_t*)g.scales)[(n >> 7) * ((g.K + 127) >> 7) + (k0 >> 7)];
+                else if (FMT == XQ_FMT_INT4) {
+                    if (!int4_small_group) {
+                        const int64_t si = ((int64_t)n * g.K + k0) / g.group;
+                        B.sc[b][0] = g.scale_dtype == XQ_SCALE_F32 ? ((const uint32_t*)g.scales)[si] : ((const uint16_t*)g.scales)[si];
+                    }
+                } else {
+                    const int64_t si = ((int64_t)n * g.K + k0) >> 4;   // 4 scales of the 64-element run
+                    if (g.scale_dtype == XQ_SCALE_E4M3) B.sc[b][0] = *(const uint32_t*)(g.scales + si);
+                    else {
+                        const u32x4 t = *(const u32x4*)((const float*)g.scales + si);
+#pragma unroll
+                        for (int j = 0; j < NSC; ++j) B.sc[b][j] = t[j];
+                    }
+                }
+#pragma unroll
+                for (int j = 0; j < MT * 8; ++j)
+                    if (j * 4 + xrow < mrows) B.xr[b][j] = *(const u32x4*)(xg + j * xstep + c * 128);   // lanes of rows >= M keep stale data
             }
         }
-        // ---- decode + multiply
+    };
+    auto compute = [&](Batch& B, int c0) {
 #pragma unroll
         for (int b = 0; b < BC; ++b) {
             if (c0 + b < c_end) {
                 const int c = c0 + b, k0 = c * 128 + fh * 64;
-                bf16x8 xf[MT][8];
+                // x tile -> LDS (LDS operations of one wave execute in order: the previous chunk's fragment
+                // reads are ahead of these writes)
 #pragma unroll
-                for (int i = 0; i < MT; ++i)
-#pragma unroll
-                    for (int t = 0; t < 8; ++t) xf[i][t] = *(const bf16x8*)(xg[i] + c * 128 + t * 8);
+                for (int j = 0; j < MT * 8; ++j)
+                    if (j * 4 < mrows) *(u32x4*)(xs + (j * 4 + xrow) * XP + xpiece * 8) = B.xr[b][j];
 #pragma unroll
                 for (int t = 0; t < 8; ++t) {
                     bf16x8 wf;
                     if (FMT == XQ_FMT_FP8) {
-                        wf = decode8<FMT>(w[b][t >> 1][(t & 1) * 2], w[b][t >> 1][(t & 1) * 2 + 1], sc[b], 0.0f);
+                        wf = decode8<FMT>(B.w[b][t >> 1][(t & 1) * 2], B.w[b][t >> 1][(t & 1) * 2 + 1], __uint_as_float(B.sc[b][0]), 0.0f);
                     } else if (FMT == XQ_FMT_INT4) {
-                        float s = g.group >= 64 ? sc[b] : load_scale(g.scales, ((int64_t)n * g.K + k0 + t * 8) / g.group, g.scale_dtype);
-                        wf = decode8<FMT>(w[b][t >> 2][t & 3], 0u, s, -8.0f * s);
+                        float s;
+                        if (int4_small_group) s = load_scale(g.scales, ((int64_t)n * g.K + k0 + t * 8) / g.group, g.scale_dtype);
+                        else s = g.scale_dtype == XQ_SCALE_F32 ? __uint_as_float(B.sc[b][0]) : __uint_as_float(B.sc[b][0] << 16);
+                        wf = decode8<FMT>(B.w[b][t >> 2][t & 3], 0u, s, -8.0f * s);
                     } else {
-                        float s = load_scale(g.scales, ((int64_t)n * g.K + k0 + t * 8) >> 4, g.scale_dtype) * gsc;
-                        wf = decode8<FMT>(w[b][t >> 2][t & 3], 0u, s, 0.0f);
+                        float s;
+                        if (g.scale_dtype == XQ_SCALE_E4M3) s = e4m3_to_f32((uint8_t)(B.sc[b][0] >> (8 * (t >> 1))));
+                        else s = __uint_as_float(B.sc[b][(t >> 1) % NSC]);
+                        wf = decode8<FMT>(B.w[b][t >> 2][t & 3], 0u, s * gsc, 0.0f);
                     }
 #pragma unroll
-                    for (int i = 0; i < MT; ++i) acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf, xf[i][t], acc[i], 0, 0, 0);
+                    for (int i = 0; i < MT; ++i) {
+                        const bf16x8 xf = *(const bf16x8*)(xs + (i * 32 + fr) * XP + fh * 64 + t * 8);
+                        acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf, xf, acc[i], 0, 0, 0);
+                    }
+                }
+            }
+        }
+    };
+
+    // two register sets: the next batch is in flight while the current one is multiplied
+    Batch B0, B1;
+    int c = c_begin;
+    if (c < c_end) issue(B0, c);
+    while (c < c_end) {
+        if (c + BC < c_end) issue(B1, c + BC);
+        compute(B0, c);
+        c += BC;
+        if (c >= c_end) break;
+        if (c + BC < c_end) issue(B0, c + BC);
+        compute(B1, c);
+        c += BC;
+    }
+
+    // ---- low-rank side term (last wave): y += (s * su) . B^T with su = x . A^T from skinny_su_kernel
+    if (g.r_pad > 0 && wave == NW - 1) {
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            if (ks < (g.r_pad >> 4)) {
+                const int j0 = ks * 16 + fh * 8;   // first rank index of this lane's 8
+                const bf16x8 lb = factor_frag(g.lora_B, (int64_t)n * g.r + j0, g.lora_f32 != 0, g.r - j0);
+#pragma unroll
+                for (int i = 0; i < MT; ++i) {
+                    const int m = i * 32 + fr;
+                    const float* sp = g.su_f32 + (int64_t)(m < g.M ? m : 0) * g.r_pad + j0;
+                    uint32_t o[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) o[e] = pack_bf16x2(sp[2 * e] * g.su_scale, sp[2 * e + 1] * g.su_scale);
+                    u32x4 r = {o[0], o[1], o[2], o[3]};
+                    acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lb, __builtin_bit_cast(bf16x8, r), acc[i], 0, 0, 0);
                 }
             }
         }
     }
 
-    // ---- low-rank side term: its operands were fetched before the stream started
-    if (lora_wave) {
-#pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
-            if (ks < (g.r_pad >> 4)) {
-#pragma unroll
-                for (int i = 0; i < MT; ++i) acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lb[ks], ls[i][ks], acc[i], 0, 0, 0);
-            }
-        }
-    }
-
-    // ---- cross-wave reduction through LDS, summed in wave order
+    // ---- cross-wave reduction through LDS, summed in wave order (the x tiles are dead by now)
     constexpr int R = MT * 16;
+    __syncthreads();
 #pragma unroll
     for (int i = 0; i < MT; ++i)
 #pragma unroll
         for (int q = 0; q < 16; ++q) red[(wave * R + i * 16 + q) * 64 + lane] = acc[i][q];
     __syncthreads();
-    // quads of 4 consecutive output columns: quad id = (i, q4); wave w takes quads w, w+SK_NW, ...
-    for (int quad = wave; quad < MT * 4; quad += SK_NW) {
+    // quads of 4 consecutive output columns: quad id = (i, q4); wave w takes quads w, w+NW, ...
+    for (int quad = wave; quad < MT * 4; quad += NW) {
         const int i = quad >> 2, q4 = quad & 3;
         float v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-        for (int w = 0; w < SK_NW; ++w)
+        for (int w = 0; w < NW; ++w)
 #pragma unroll
             for (int e = 0; e < 4; ++e) v[e] += red[(w * R + i * 16 + q4 * 4 + e) * 64 + lane];
         const int m = i * 32 + fr, nn = n0 + 8 * q4 + 4 * fh;
@@ -213,39 +264,50 @@ __global__ void __launch_bounds__(SK_NW * 64) skinny_kernel(SkinnyArgs g) {
     }
 }
 
-// partial sums of x . A^T over one 256-wide K range, added with atomics to su_f32 [M, r_pad] (zeroed)
+// su_f32[M, r_pad] = x[M, K] . A[r, K]^T (fp32, unscaled; columns r..r_pad-1 are zero).  One block;
+// its SU_NW waves split K, partial sums meet in LDS and are added in wave order (deterministic).
+constexpr int SU_NW = 8;
 template <int MT>
-__global__ void __launch_bounds__(64) skinny_su_kernel(const bf16_t* x, int64_t ldx, int M, int K, const bf16_t* A_bf,
-                                                       int r_pad, float* su_f32) {
-    const int lane = threadIdx.x, fr = lane & 31, fh = lane >> 5;
-    const int kb = blockIdx.x * 256;
+__global__ void __launch_bounds__(SU_NW * 64) skinny_su_kernel(const bf16_t* x, int64_t ldx, int M, int K, const void* A,
+                                                              int a_f32, int r, int r_pad, float* su_f32) {
+    extern __shared__ __attribute__((aligned(16))) float red[];   // [SU_NW][MT*16][64]
+    const int tid = threadIdx.x, lane = tid & 63, fr = lane & 31, fh = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int steps = K >> 4;
+    const int s_begin = (steps * wave) / SU_NW, s_end = (steps * (wave + 1)) / SU_NW;
     const int nt = (r_pad + 31) >> 5;
     for (int j = 0; j < nt; ++j) {
         const int rrow = j * 32 + fr;
+        const bool rvalid = rrow < r;
         f32x16 acc[MT];
 #pragma unroll
         for (int i = 0; i < MT; ++i)
 #pragma unroll
             for (int q = 0; q < 16; ++q) acc[i][q] = 0.0f;
-        const bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
-        for (int k = kb; k < kb + 256 && k < K; k += 16) {
-            bf16x8 af = rrow < r_pad ? *(const bf16x8*)(A_bf + (int64_t)rrow * K + k + fh * 8) : z;
+        for (int st = s_begin; st < s_end; ++st) {
+            const int k = st * 16 + fh * 8;
+            const bf16x8 af = factor_frag(A, (int64_t)(rvalid ? rrow : 0) * K + k, a_f32 != 0, rvalid ? 8 : 0);
 #pragma unroll
             for (int i = 0; i < MT; ++i) {
                 const int m = i * 32 + fr;
-                bf16x8 xf = m < M ? *(const bf16x8*)(x + (int64_t)m * ldx + k + fh * 8) : z;
+                const bf16x8 xf = *(const bf16x8*)(x + (int64_t)(m < M ? m : 0) * ldx + k);
                 acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, xf, acc[i], 0, 0, 0);   // D[rank][m]
             }
         }
+        constexpr int R = MT * 16;
+        __syncthreads();   // the previous rank tile's sums have been read
 #pragma unroll
-        for (int i = 0; i < MT; ++i) {
-            const int m = i * 32 + fr;
-            if (m >= M) continue;
+        for (int i = 0; i < MT; ++i)
 #pragma unroll
-            for (int q = 0; q < 16; ++q) {
-                const int rr = j * 32 + (q & 3) + 4 * fh + 8 * (q >> 2);
-                if (rr < r_pad) atomicAdd(su_f32 + (int64_t)m * r_pad + rr, acc[i][q]);
-            }
+            for (int q = 0; q < 16; ++q) red[(wave * R + i * 16 + q) * 64 + lane] = acc[i][q];
+        __syncthreads();
+        for (int idx = wave; idx < R; idx += SU_NW) {   // register idx = (i, q) of every lane
+            float v = 0.0f;
+#pragma unroll
+            for (int w = 0; w < SU_NW; ++w) v += red[(w * R + idx) * 64 + lane];
+            const int i = idx >> 4, q = idx & 15;
+            const int m = i * 32 + fr, rr = j * 32 + (q & 3) + 4 * fh + 8 * (q >> 2);
+            if (m < M && rr < r_pad) su_f32[(int64_t)m * r_pad + rr] = v;
         }
     }
 }
@@ -253,7 +315,8 @@ __global__ void __launch_bounds__(64) skinny_su_kernel(const bf16_t* x, int64_t 
 static inline int64_t al256(int64_t b) { return (b + 255) & ~(int64_t)255; }
 
 int64_t skinny_workspace_bytes(int64_t M, int64_t N, int64_t K, int r_pad) {
-    return al256(M * (r_pad ? r_pad : 16) * 4) + al256((int64_t)r_pad * K * 2) + al256(N * (int64_t)r_pad * 2) + 256;
+    (void)N; (void)K;
+    return al256(M * (r_pad ? r_pad : 16) * 4) + 256;
 }
 
 bool skinny_supported(const xq_weight* w, int64_t M) {
@@ -264,12 +327,31 @@ bool skinny_supported(const xq_weight* w, int64_t M) {
     return true;
 }
 
+template <int FMT, int MT, int NW>
+static int launch_skinny_one(const SkinnyArgs& g, dim3 grid, hipStream_t s) {
+    // LDS: the wave-private x tiles (MT*32 rows of 272 B per wave); the reduction buffer reuses them
+    constexpr size_t lds = (size_t)NW * MT * 32 * 136 * 2;
+    static_assert(lds >= (size_t)NW * MT * 16 * 64 * 4, "reduction buffer must fit in the x tiles");
+    static bool attr_set = false;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute((const void*)skinny_kernel<FMT, MT, NW>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e != hipSuccess) {
+            xq_set_error("xq_linear_fwd: cannot raise the dynamic LDS limit: %s", hipGetErrorString(e));
+            return XQ_ERR_LAUNCH;
+        }
+        attr_set = true;
+    }
+    skinny_kernel<FMT, MT, NW><<<grid, NW * 64, lds, s>>>(g);
+    return XQ_OK;
+}
+
 template <int FMT>
 static int launch_skinny_cfg(const SkinnyArgs& g, hipStream_t s) {
     dim3 grid((unsigned)xq_cdiv(g.N, 32));
-    if (g.M <= 32) skinny_kernel<FMT, 1><<<grid, SK_NW * 64, (size_t)SK_NW * 16 * 64 * 4, s>>>(g);
-    else skinny_kernel<FMT, 2><<<grid, SK_NW * 64, (size_t)SK_NW * 32 * 64 * 4, s>>>(g);
-    return XQ_OK;
+    // more slabs than CUs: 4 waves per slab so that two blocks share a CU; else 8 waves per slab
+    const bool many = grid.x > 256;
+    if (g.M <= 32) return many ? launch_skinny_one<FMT, 1, 4>(g, grid, s) : launch_skinny_one<FMT, 1, 8>(g, grid, s);
+    return many ? launch_skinny_one<FMT, 2, 4>(g, grid, s) : launch_skinny_one<FMT, 2, 8>(g, grid, s);
 }
 
 int launch_skinny(const xq_weight* w, const bf16_t* x, int64_t ldx, int64_t M, const void* lora_A, const void* lora_B,
@@ -280,26 +362,22 @@ int launch_skinny(const xq_weight* w, const bf16_t* x, int64_t ldx, int64_t M, c
     XQ_REQUIRE(workspace && xq_aligned(workspace, 256) && workspace_bytes >= skinny_workspace_bytes(M, N, K, rp),
                "xq_linear_fwd: workspace missing, misaligned or too small for the skinny path");
     XQ_REQUIRE(ldx % 8 == 0 && xq_aligned(x, 16) && xq_aligned(w->packed, 16), "xq_linear_fwd: operands must be 16-byte aligned");
-    uint8_t* p = (uint8_t*)workspace;
-    float* su_f32 = (float*)p; p += al256(M * (rp ? rp : 16) * 4);
-    bf16_t* A_bf = (bf16_t*)p; p += al256((int64_t)rp * K * 2);
-    bf16_t* Bl = (bf16_t*)p;
+    XQ_REQUIRE(rp == 0 || xq_aligned(lora_A, 4) && xq_aligned(lora_B, 4), "xq_linear_fwd: LoRA factors must be 4-byte aligned");
+    float* su_f32 = (float*)workspace;
 
     int rc;
     if (rp) {
-        if ((rc = launch_zero_fill(su_f32, M * rp * 4, stream))) return rc;
-        if ((rc = launch_factor_prep(lora_A, lora_dtype, r, K, false, A_bf, rp, K, 1, stream))) return rc;
-        if ((rc = launch_factor_prep(lora_B, lora_dtype, N, r, false, Bl, N, rp, 1, stream))) return rc;
-        dim3 sg((unsigned)xq_cdiv(K, 256));
-        if (M <= 32) skinny_su_kernel<1><<<sg, 64, 0, stream>>>(x, ldx, (int)M, (int)K, A_bf, rp, su_f32);
-        else skinny_su_kernel<2><<<sg, 64, 0, stream>>>(x, ldx, (int)M, (int)K, A_bf, rp, su_f32);
+        const int f32 = lora_dtype == XQ_DT_F32;
+        if (M <= 32) skinny_su_kernel<1><<<dim3(1), SU_NW * 64, (size_t)SU_NW * 16 * 64 * 4, stream>>>(x, ldx, (int)M, (int)K, lora_A, f32, r, rp, su_f32);
+        else skinny_su_kernel<2><<<dim3(1), SU_NW * 64, (size_t)SU_NW * 32 * 64 * 4, stream>>>(x, ldx, (int)M, (int)K, lora_A, f32, r, rp, su_f32);
         XQ_CHECK_LAUNCH("skinny_su");
     }
     SkinnyArgs g;
     g.x = x; g.ldx = ldx; g.M = (int)M; g.N = (int)N; g.K = (int)K;
     g.packed = (const uint8_t*)w->packed; g.scales = (const uint8_t*)w->scales; g.global_scale = w->global_scale;
     g.group = w->group; g.scale_dtype = w->scale_dtype;
-    g.su_f32 = rp ? su_f32 : nullptr; g.su_scale = scaling; g.lora_right = rp ? Bl : nullptr; g.r_pad = rp;
+    g.su_f32 = rp ? su_f32 : nullptr; g.su_scale = scaling; g.lora_B = rp ? lora_B : nullptr;
+    g.lora_f32 = lora_dtype == XQ_DT_F32; g.r = r; g.r_pad = rp;
     g.bias = bias; g.y = y; g.ldy = ldy;
     // algorithmic bytes: packed weight + scales + x + y (+ LoRA factors), for the roofline figure
     const double wbytes = (double)xq_packed_bytes_per_expert(w) + (double)xq_scale_bytes_per_expert(w);
