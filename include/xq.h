@@ -87,11 +87,13 @@ int xq_profile_collect(int* n_launches, double* total_ms, double* total_flops);
 
 /* Kernel selection of the fused dequant-GEMM entry points (dense and grouped),
  * for tests and A/B measurements; no counterpart in the reference.
- *   0 (default): by problem size -- the 256x256 tile kernel when its tiles fill
- *      the chip (block-fp8, and FLAT int4/nvfp4 with a power-of-two group >= 16),
- *      else the generic 128x128 tile kernel;
- *   1: always the generic 128x128 tile kernel;
- *   2: the 256x256 kernel whenever the format allows it, whatever the size. */
+ *   0 (default): by problem size.  Block-fp8 and FLAT int4/nvfp4 weights with a
+ *      power-of-two group >= 16 use the pipelined tile kernel, with 256x256 tiles
+ *      when those fill the chip and 128x128 tiles otherwise; other weights (GKN
+ *      4-bit banks, odd groups) use the generic single-buffered 128x128 kernel;
+ *   1: always the generic kernel;
+ *   2 / 3: the pipelined kernel with 256x256 / 128x128 tiles whenever the format
+ *      allows it, whatever the size. */
 int xq_set_tile_policy(int policy);
 
 /* ---- decode ------------------------------------------------------------

@@ -23,7 +23,7 @@ def hip_device():
 
 @pytest.fixture
 def tile_policy(request):
-    """Selects the fused dequant-GEMM kernel for one test: 0 = by size, 1 = 128x128 tiles, 2 = 256x256 tiles."""
+    """Selects the fused dequant-GEMM kernel for one test: 0 = by size, 1 = generic kernel, 2 / 3 = pipelined kernel with 256x256 / 128x128 tiles."""
     from xorl_amd import _C
 
     _C.check(_C.lib().xq_set_tile_policy(int(request.param)))

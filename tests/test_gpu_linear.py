@@ -19,7 +19,7 @@ def _run(m, x, dy):
     return y.detach(), x.grad, m.lora_A.grad, m.lora_B.grad
 
 
-@pytest.mark.parametrize("tile_policy", [0, 2], indirect=True)
+@pytest.mark.parametrize("tile_policy", [0, 1, 2], indirect=True)
 @pytest.mark.parametrize("fmt", ["block_fp8", "int4", "nvfp4"])
 @pytest.mark.parametrize("M,K,N,r", [(200, 256, 384, 16), (1, 128, 64, 8), (129, 384, 320, 24), (512, 1024, 512, 64), (1100, 512, 768, 32)])
 def test_dense_fwd_bwd_vs_oracle(hip_device, tile_policy, fmt, M, K, N, r):
@@ -35,7 +35,7 @@ def test_dense_fwd_bwd_vs_oracle(hip_device, tile_policy, fmt, M, K, N, r):
         assert err <= TOL, f"{fmt} {name}: {err}"
 
 
-@pytest.mark.parametrize("tile_policy", [0, 2], indirect=True)
+@pytest.mark.parametrize("tile_policy", [0, 1, 2], indirect=True)
 def test_config0_int4_full_size(hip_device, tile_policy):
     """BASELINE config 0: X [512,4096], W [4096,4096] int4 g128 absmax/7 bf16 scales, r=16, alpha=32."""
     M, K, N, r = 512, 4096, 4096, 16
@@ -50,7 +50,7 @@ def test_config0_int4_full_size(hip_device, tile_policy):
     assert torch.equal(m._dequantize_weight().cpu(), w_ref)
 
 
-@pytest.mark.parametrize("tile_policy", [1, 2], indirect=True)
+@pytest.mark.parametrize("tile_policy", [1, 2, 3], indirect=True)
 @pytest.mark.parametrize("fmt", ["block_fp8", "int4", "nvfp4"])
 def test_gemm_decode_bit_exact(hip_device, tile_policy, fmt):
     """With X = I (and lora_B = 0) every output is a single product 1 * w, so the forward returns the

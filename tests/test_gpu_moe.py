@@ -83,7 +83,7 @@ def _make_experts(fmt, E, H, I, r, hybrid, seed, device):
     return m.to(device), banks
 
 
-@pytest.mark.parametrize("tile_policy", [0, 2], indirect=True)
+@pytest.mark.parametrize("tile_policy", [0, 1, 2], indirect=True)
 @pytest.mark.parametrize("fmt", ["block_fp8", "nvfp4"])
 @pytest.mark.parametrize("E,T,H,I,r,topk,hybrid", [(6, 300, 128, 192, 8, 2, True), (16, 700, 256, 128, 16, 4, False)])
 def test_moe_fwd_bwd_vs_oracle(hip_device, tile_policy, fmt, E, T, H, I, r, topk, hybrid):

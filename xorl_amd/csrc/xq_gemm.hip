@@ -12,8 +12,9 @@ static void launch_tile_cc(const TileArgs& g, bool contract_cols, dim3 grid, hip
     else gemm_tile_kernel<FMT, LAYOUT, false><<<grid, 256, 0, s>>>(g);
 }
 
-// kernel-selection policy (xq_set_tile_policy): 0 = by problem size, 1 = always the generic 128x128 tile
-// kernel, 2 = the 256x256 kernel whenever the format allows it.  XQ_SKINNY=0 disables the M <= 64 path.
+// kernel-selection policy (xq_set_tile_policy): 0 = by problem size, 1 = always the generic single-buffered
+// tile kernel, 2 / 3 = the pipelined kernel with 256x256 / 128x128 tiles whenever the format allows it.
+// XQ_SKINNY=0 disables the M <= 64 path.
 static int g_skinny_enabled = [] { const char* e = getenv("XQ_SKINNY"); return e ? atoi(e) : 1; }();
 static int g_tile_policy = [] { const char* e = getenv("XQ_TILE_POLICY"); return e ? atoi(e) : 0; }();
 
@@ -27,22 +28,27 @@ static int raise_lds_limit(K kernel, const char* who) {
     return XQ_OK;
 }
 
-template <int FMT, bool CC, bool GROUPED>
-static int launch_256_one(const G256Args& f, dim3 grid, size_t lds, hipStream_t s, const char* who) {
+template <int FMT, bool CC, bool GROUPED, int T>
+static int launch_256_one(const G256Args& f, dim3 grid, hipStream_t s, const char* who) {
     static bool attr_set = false;  // per instantiation
     if (!attr_set) {
-        int rc = raise_lds_limit(gemm_256_kernel<FMT, CC, GROUPED>, who);
+        int rc = raise_lds_limit(gemm_256_kernel<FMT, CC, GROUPED, T>, who);
         if (rc) return rc;
         attr_set = true;
     }
-    gemm_256_kernel<FMT, CC, GROUPED><<<grid, 512, lds, s>>>(f);
+    gemm_256_kernel<FMT, CC, GROUPED, T><<<grid, Geo<T>::NT, Geo<T>::lds_bytes(CC), s>>>(f);
     return XQ_OK;
 }
 
+template <int FMT, bool CC, bool GROUPED>
+static int launch_256_t(const G256Args& f, int T, dim3 grid, hipStream_t s, const char* who) {
+    return T == 256 ? launch_256_one<FMT, CC, GROUPED, 256>(f, grid, s, who) : launch_256_one<FMT, CC, GROUPED, 128>(f, grid, s, who);
+}
+
 template <int FMT>
-static int launch_256(const G256Args& f, bool cc, bool grouped, dim3 grid, size_t lds, hipStream_t s, const char* who) {
-    if (cc) return grouped ? launch_256_one<FMT, true, true>(f, grid, lds, s, who) : launch_256_one<FMT, true, false>(f, grid, lds, s, who);
-    return grouped ? launch_256_one<FMT, false, true>(f, grid, lds, s, who) : launch_256_one<FMT, false, false>(f, grid, lds, s, who);
+static int launch_256(const G256Args& f, bool cc, bool grouped, int T, dim3 grid, hipStream_t s, const char* who) {
+    if (cc) return grouped ? launch_256_t<FMT, true, true>(f, T, grid, s, who) : launch_256_t<FMT, true, false>(f, T, grid, s, who);
+    return grouped ? launch_256_t<FMT, false, true>(f, T, grid, s, who) : launch_256_t<FMT, false, false>(f, T, grid, s, who);
 }
 
 // C[rows, Nout] = A . op(deq(W)) (+ su . Lr^T) (+ bias); see xq_gemm_tile.h
@@ -72,36 +78,38 @@ int launch_tile_gemm(const xq_weight* w, bool contract_cols, const bf16_t* A, in
     if (w->format != XQ_FMT_FP8 && w->layout == XQ_LAYOUT_GKN)
         XQ_REQUIRE(w->rows % 2 == 0, "%s: GKN 4-bit storage needs an even row count", who);
     if (n_rows == 0) return XQ_OK;
-    // enough 256x256 tiles to occupy the chip: the 256x256 kernel (block-fp8 and FLAT 4-bit; dense or grouped)
+    // block-fp8 and FLAT 4-bit weights: the pipelined tile kernel, 256x256 tiles when they fill the chip,
+    // 128x128 tiles otherwise (dense or grouped)
     {
         const bool grouped = offsets != nullptr;
-        const int64_t tiles_m = xq_cdiv(n_rows, F8_BM) + (grouped ? w->num_experts : 0);
-        const int64_t tiles_n = xq_cdiv(g.Nout, F8_BN);
         int gshift = 0;
         while ((1 << gshift) < g.group) ++gshift;
         const bool fmt_ok = w->format == XQ_FMT_FP8 ||
                             (w->layout == XQ_LAYOUT_FLAT && (1 << gshift) == g.group && g.group >= 16);
         const bool big = grouped ? (n_rows >= 128ll * w->num_experts && n_rows >= 8192)
-                                 : (xq_cdiv(n_rows, F8_BM) * tiles_n >= 96);
-        if (fmt_ok && (g_tile_policy == 2 || (big && g_tile_policy == 0)) && tiles_m * tiles_n < (1ll << 31)) {
+                                 : (xq_cdiv(n_rows, 256) * xq_cdiv(g.Nout, 256) >= 96);
+        const int T = g_tile_policy == 2 ? 256 : g_tile_policy == 3 ? 128 : (big ? 256 : 128);
+        const int64_t tiles_m = xq_cdiv(n_rows, T) + (grouped ? w->num_experts : 0);
+        const int64_t tiles_n = xq_cdiv(g.Nout, T);
+        if (fmt_ok && g_tile_policy != 1 && tiles_m * tiles_n < (1ll << 31)) {
             G256Args f;
             f.A = A; f.lda = lda; f.C = C; f.ldc = ldc;
             f.W = g.packed; f.scales = g.scales; f.global_scale = g.global_scale;
             f.packed_stride = g.packed_stride; f.scale_stride = g.scale_stride;
             f.wrows = g.wrows; f.wcols = g.wcols; f.gshift = gshift; f.scale_dtype = g.scale_dtype;
             f.Kc = g.Kc; f.Nout = g.Nout; f.M = n_rows;
-            f.offsets = offsets; f.tiles256 = grouped ? tile_offsets + (w->num_experts + 1) : nullptr;
+            f.offsets = offsets;
+            f.tile_prefix = !grouped ? nullptr : (T == 256 ? tile_offsets + (w->num_experts + 1) : tile_offsets);
             f.num_experts = w->num_experts;
             f.su = g.r_pad ? su : nullptr; f.lora_right = g.r_pad ? lora_right : nullptr; f.r_pad = g.r_pad;
             f.bias = bias;
             f.tiles_m = (int32_t)tiles_m; f.tiles_n = (int32_t)tiles_n;
-            const size_t lds = (size_t)(2 * F8_A_STAGE + 2 * (contract_cols ? F8_B_STAGE_NT : F8_B_STAGE_NN)) * 2;
             dim3 grid((unsigned)(tiles_m * tiles_n));
             const bool timed = xq_profile_mark_begin(stream, 2.0 * (double)n_rows * g.Nout * ((double)g.Kc + g.r_pad));
             int rc;
-            if (w->format == XQ_FMT_FP8) rc = launch_256<XQ_FMT_FP8>(f, contract_cols, grouped, grid, lds, stream, who);
-            else if (w->format == XQ_FMT_INT4) rc = launch_256<XQ_FMT_INT4>(f, contract_cols, grouped, grid, lds, stream, who);
-            else rc = launch_256<XQ_FMT_NVFP4>(f, contract_cols, grouped, grid, lds, stream, who);
+            if (w->format == XQ_FMT_FP8) rc = launch_256<XQ_FMT_FP8>(f, contract_cols, grouped, T, grid, stream, who);
+            else if (w->format == XQ_FMT_INT4) rc = launch_256<XQ_FMT_INT4>(f, contract_cols, grouped, T, grid, stream, who);
+            else rc = launch_256<XQ_FMT_NVFP4>(f, contract_cols, grouped, T, grid, stream, who);
             if (timed) xq_profile_mark_end(stream);
             if (rc) return rc;
             XQ_CHECK_LAUNCH(who);
@@ -139,7 +147,7 @@ struct Carver {
 using namespace xq;
 
 extern "C" int xq_set_tile_policy(int policy) {
-    XQ_REQUIRE(policy >= 0 && policy <= 2, "xq_set_tile_policy: policy %d not in {0, 1, 2}", policy);
+    XQ_REQUIRE(policy >= 0 && policy <= 3, "xq_set_tile_policy: policy %d not in {0, 1, 2, 3}", policy);
     g_tile_policy = policy;
     return XQ_OK;
 }

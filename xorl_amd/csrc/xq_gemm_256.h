@@ -1,6 +1,8 @@
-// Large-M fused dequant-GEMM: 256x256x64 tiles, 8 waves (2 along M x 4 along N, two
-// per SIMD so one wave's LDS/VALU work hides under the other's MFMAs), each wave a
-// 128x64 sub-tile of 4x2 v_mfma_f32_32x32x16_bf16 (128 fp32 accumulators).
+// Fused dequant-GEMM tile kernel.  T = 256: 256x256x64 tiles, 8 waves (2 along M x 4
+// along N, two per SIMD so one wave's LDS/VALU work hides under the other's MFMAs), each
+// wave a 128x64 sub-tile of 4x2 v_mfma_f32_32x32x16_bf16 (128 fp32 accumulators) -- the
+// large-M kernel.  T = 128: the same program on 128x128x64 tiles with 4 waves of 64x64
+// (two blocks per CU), for problems that do not fill the chip with 256x256 tiles.
 //
 //   C[rows, Nout] = A[rows, Kc] . Wop (+ su[rows, r] . Lr[Nout, r]^T) (+ bias)
 //
@@ -22,8 +24,8 @@
 // A_frag) so that each lane ends up with 4 consecutive output columns and the
 // epilogue writes 8-byte packed bf16.
 //
-// GROUPED: rows are in expert order; a block works on one 256-row tile of one
-// expert (found from the 256-row tile prefix that xq_route_build emits) against
+// GROUPED: rows are in expert order; a block works on one T-row tile of one
+// expert (found from the T-row tile prefix that xq_route_build emits) against
 // that expert's matrix of the bank.
 #pragma once
 
@@ -31,11 +33,20 @@
 
 namespace xq {
 
-constexpr int F8_BM = 256, F8_BN = 256, F8_BK = 64;
-constexpr int F8_A_STAGE = F8_BM * F8_BK;             // bf16 elements (32 KB)
-constexpr int F8_NN_PITCH = F8_BN + 32;               // [kc][n] rows of 576 B
-constexpr int F8_B_STAGE_NT = F8_BN * F8_BK;          // 32 KB
-constexpr int F8_B_STAGE_NN = F8_BK * F8_NN_PITCH;    // 36 KB
+constexpr int F8_BK = 64;
+// geometry of a T x T tile (T = 256: 8 waves, 2 x 4; T = 128: 4 waves, 2 x 2; wave tile (T/2) x 64)
+template <int T>
+struct Geo {
+    static constexpr int BM = T, BN = T, NT = 2 * T;      // tile rows / cols, threads
+    static constexpr int TM = T / 64, TN = 2;              // 32x32 MFMA tiles per wave
+    static constexpr int WN = T / 64;                      // waves along N
+    static constexpr int A_STAGE = BM * F8_BK;             // bf16 elements
+    static constexpr int NN_PITCH = BN + 32;               // [kc][n] row pitch (T = 256: 576 B)
+    static constexpr int B_STAGE_NT = BN * F8_BK;
+    static constexpr int B_STAGE_NN = F8_BK * NN_PITCH;
+    static constexpr int RPR = BN / 16;                    // 16-code runs per [kc] row of the tile
+    static constexpr size_t lds_bytes(bool cc) { return (size_t)(2 * A_STAGE + 2 * (cc ? B_STAGE_NT : B_STAGE_NN)) * 2; }
+};
 
 // element offset of 16-byte chunk `c` (0..7) of row `r` in a [rows][64] bf16 tile.
 // gfx950 LDS has 64 banks (256 B/clk) and serves a ds_read_b128 sixteen lanes at a
@@ -58,7 +69,7 @@ struct G256Args {
     int32_t Kc, Nout;
     int64_t M;                 // total rows
     const int32_t* offsets;    // grouped: [E+1] row offsets in expert order
-    const int32_t* tiles256;   // grouped: [E+1] prefix of ceil(count/256)
+    const int32_t* tile_prefix;// grouped: [E+1] prefix of ceil(count / tile rows)
     int32_t num_experts;
     const bf16_t* su;          // [M, r_pad] or NULL
     const bf16_t* lora_right;  // [E][Nout, r_pad] or NULL
@@ -68,26 +79,26 @@ struct G256Args {
 };
 
 // ---------------------------------------------------------------- weight-tile loaders
-// A 256(n) x 64(kc) tile is split over 512 threads as 2 runs of 16 consecutive codes
-// each: run u = tid + p*512.  CONTRACT_COLS: W row n0 + (u >> 2), columns k0 + (u&3)*16
-// .. +16; otherwise W row k0 + (u >> 4), columns n0 + (u&15)*16 .. +16.  load()
+// A T(n) x 64(kc) tile is split over the 2T threads as 2 runs of 16 consecutive codes
+// each: run u = tid + p*2T.  CONTRACT_COLS: W row n0 + (u >> 2), columns k0 + (u&3)*16
+// .. +16; otherwise W row k0 + u / (T/16), columns n0 + (u % (T/16))*16 .. +16.  load()
 // fetches the packed bytes and scale(s) of K-step kt into registers; store() decodes
 // one run and writes its 16 bf16 values (two 16-byte LDS stores) to the stage.
 
-template <bool CC>
+template <bool CC, int T>
 __device__ __forceinline__ void store_run16(bf16_t* b, int u, const u32x4& lo, const u32x4& hi) {
     if (CC) {
         const int r = u >> 2, c = (u & 3) * 2;
         *(u32x4*)(b + swz(r, c)) = lo;
         *(u32x4*)(b + swz(r, c + 1)) = hi;
     } else {
-        bf16_t* d = b + (u >> 4) * F8_NN_PITCH + (u & 15) * 16;
+        bf16_t* d = b + (u / Geo<T>::RPR) * Geo<T>::NN_PITCH + (u % Geo<T>::RPR) * 16;
         *(u32x4*)d = lo;
         *(u32x4*)(d + 8) = hi;
     }
 }
 
-template <bool CC>
+template <bool CC, int T>
 struct W256Fp8 {
     const uint8_t* src[2];
     const float* s_src[2];
@@ -100,10 +111,10 @@ struct W256Fp8 {
         scols = (g.wcols + 127) >> 7;
 #pragma unroll
         for (int p = 0; p < 2; ++p) {
-            const int u = tid + p * 512;
+            const int u = tid + p * Geo<T>::NT;
             int wr, wc;
             if (CC) { wr = min(n0 + (u >> 2), g.wrows - 1); wc = (u & 3) * 16; }
-            else { wr = u >> 4; wc = min(n0 + (u & 15) * 16, g.wcols - 16); }
+            else { wr = u / Geo<T>::RPR; wc = min(n0 + (u % Geo<T>::RPR) * 16, g.wcols - 16); }
             src[p] = pk + (int64_t)wr * g.wcols + wc;
             s_src[p] = (const float*)sc + (CC ? (wr >> 7) * scols : (wc >> 7));
         }
@@ -127,7 +138,7 @@ struct W256Fp8 {
             if (i < 2) { lo[2 * i] = v0; lo[2 * i + 1] = v1; }
             else { hi[2 * (i - 2)] = v0; hi[2 * (i - 2) + 1] = v1; }
         }
-        store_run16<CC>(b, tid + p * 512, lo, hi);
+        store_run16<CC, T>(b, tid + p * Geo<T>::NT, lo, hi);
     }
 };
 
@@ -175,7 +186,7 @@ __device__ __forceinline__ void decode8_4bit(uint32_t w, float s, uint32_t* out4
     for (int i = 0; i < 4; ++i) out4[i] = pack_bf16x2(v[2 * i], v[2 * i + 1]);
 }
 
-template <int FMT, bool CC>
+template <int FMT, bool CC, int T>
 struct W256Flat4 {
     const uint8_t* src[2];
     const uint8_t* sc_base;
@@ -192,10 +203,10 @@ struct W256Flat4 {
         const int spr = g.wcols >> gshift;  // scales per W row
 #pragma unroll
         for (int p = 0; p < 2; ++p) {
-            const int u = tid + p * 512;
+            const int u = tid + p * Geo<T>::NT;
             int wr, wc;
             if (CC) { wr = min(n0 + (u >> 2), g.wrows - 1); wc = (u & 3) * 16; }
-            else { wr = u >> 4; wc = min(n0 + (u & 15) * 16, g.wcols - 16); }
+            else { wr = u / Geo<T>::RPR; wc = min(n0 + (u % Geo<T>::RPR) * 16, g.wcols - 16); }
             src[p] = pk + (((int64_t)wr * g.wcols + wc) >> 1);
             s_idx[p] = (int64_t)wr * spr + (CC ? 0 : (wc >> gshift));
             col0[p] = wc;
@@ -217,23 +228,26 @@ struct W256Flat4 {
         uint32_t lo[4], hi[4];
         decode8_4bit<FMT>(raw[p][0], s, lo);
         decode8_4bit<FMT>(raw[p][1], s, hi);
-        store_run16<CC>(b, tid + p * 512, u32x4{lo[0], lo[1], lo[2], lo[3]}, u32x4{hi[0], hi[1], hi[2], hi[3]});
+        store_run16<CC, T>(b, tid + p * Geo<T>::NT, u32x4{lo[0], lo[1], lo[2], lo[3]}, u32x4{hi[0], hi[1], hi[2], hi[3]});
     }
 };
 
-template <int FMT, bool CC> struct W256Sel { using type = W256Flat4<FMT, CC>; };
-template <bool CC> struct W256Sel<XQ_FMT_FP8, CC> { using type = W256Fp8<CC>; };
+template <int FMT, bool CC, int T> struct W256Sel { using type = W256Flat4<FMT, CC, T>; };
+template <bool CC, int T> struct W256Sel<XQ_FMT_FP8, CC, T> { using type = W256Fp8<CC, T>; };
 
 // ---------------------------------------------------------------- the kernel
-template <int FMT, bool CC, bool GROUPED>
-__global__ void __launch_bounds__(512, 2) gemm_256_kernel(G256Args g) {
+template <int FMT, bool CC, bool GROUPED, int T>
+__global__ void __launch_bounds__(2 * T, 2) gemm_256_kernel(G256Args g) {
+    using G = Geo<T>;
+    constexpr int F8_BM = G::BM, F8_BN = G::BN, F8_A_STAGE = G::A_STAGE, F8_NN_PITCH = G::NN_PITCH;
+    constexpr int TM = G::TM, TN = G::TN, NT = G::NT;
     extern __shared__ __attribute__((aligned(16))) bf16_t smem[];
-    constexpr int B_STAGE = CC ? F8_B_STAGE_NT : F8_B_STAGE_NN;
+    constexpr int B_STAGE = CC ? G::B_STAGE_NT : G::B_STAGE_NN;
     bf16_t* As = smem;                    // 2 stages
     bf16_t* Bs = smem + 2 * F8_A_STAGE;   // 2 stages
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 2, wn = wave & 3;   // wave tile: rows wm*128.., cols wn*64..
+    const int wm = wave / G::WN, wn = wave % G::WN;   // wave tile: rows wm*(T/2).., cols wn*64..
 
     // ---- XCD-aware tile mapping: consecutive workgroup ids land on different XCDs, so
     // give each XCD a contiguous range of logical tiles.  Dense: walk the logical tiles
@@ -265,12 +279,12 @@ __global__ void __launch_bounds__(512, 2) gemm_256_kernel(G256Args g) {
         int* sh_info = (int*)smem;
         if (tid == 0) {
             const int E = g.num_experts;
-            if (pid_m >= g.tiles256[E]) sh_info[0] = -1;
+            if (pid_m >= g.tile_prefix[E]) sh_info[0] = -1;
             else {
-                int lo = 0, hi = E;  // tiles256[lo] <= pid_m < tiles256[lo + 1]
-                while (hi - lo > 1) { int mid = (lo + hi) >> 1; if (g.tiles256[mid] <= pid_m) lo = mid; else hi = mid; }
+                int lo = 0, hi = E;  // tile_prefix[lo] <= pid_m < tile_prefix[lo + 1]
+                while (hi - lo > 1) { int mid = (lo + hi) >> 1; if (g.tile_prefix[mid] <= pid_m) lo = mid; else hi = mid; }
                 sh_info[0] = lo;
-                sh_info[1] = g.offsets[lo] + (pid_m - g.tiles256[lo]) * F8_BM;
+                sh_info[1] = g.offsets[lo] + (pid_m - g.tile_prefix[lo]) * F8_BM;
                 sh_info[2] = g.offsets[lo + 1];
             }
         }
@@ -292,13 +306,13 @@ __global__ void __launch_bounds__(512, 2) gemm_256_kernel(G256Args g) {
     int a_dst[4];
 #pragma unroll
     for (int p = 0; p < 4; ++p) {
-        const int u = tid + p * 512;
+        const int u = tid + p * NT;
         int64_t r = row0 + (u >> 3);
         r = r < row_end ? r : row_end - 1;
         a_src[p] = g.A + r * g.lda + (u & 7) * 8;
         a_dst[p] = swz(u >> 3, u & 7);
     }
-    typename W256Sel<FMT, CC>::type wl;
+    typename W256Sel<FMT, CC, T>::type wl;
     wl.init(g, g.W + (int64_t)e * g.packed_stride, g.scales + (int64_t)e * g.scale_stride,
             FMT == XQ_FMT_NVFP4 ? g.global_scale[e] : 1.0f, n0, tid);
 
@@ -313,29 +327,29 @@ __global__ void __launch_bounds__(512, 2) gemm_256_kernel(G256Args g) {
         for (int p = 0; p < 4; ++p) *(u32x4*)(a + a_dst[p]) = areg[p];
     };
 
-    f32x16 acc[4][2];
+    f32x16 acc[TM][TN];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < TN; ++j)
 #pragma unroll
             for (int q = 0; q < 16; ++q) acc[i][j][q] = 0.0f;
 
     const int fr = lane & 31, fh = lane >> 5;
     auto load_frags = [&](const bf16_t* a, const bf16_t* b, int ks, bool b_is_nt, bf16x8* af, bf16x8* bfr) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) af[i] = *(const bf16x8*)(a + swz(wm * 128 + i * 32 + fr, ks * 2 + fh));
+        for (int i = 0; i < TM; ++i) af[i] = *(const bf16x8*)(a + swz(wm * (T / 2) + i * 32 + fr, ks * 2 + fh));
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
+        for (int j = 0; j < TN; ++j) {
             if (CC || b_is_nt) bfr[j] = *(const bf16x8*)(b + swz(wn * 64 + j * 32 + fr, ks * 2 + fh));
             else bfr[j] = lds_tr_frag(b, F8_NN_PITCH, ks * 16, wn * 64 + j * 32, lane);
         }
     };
     auto mma = [&](const bf16x8* af, const bf16x8* bfr) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < TM; ++i)
 #pragma unroll
-            for (int j = 0; j < 2; ++j)
+            for (int j = 0; j < TN; ++j)
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[j], af[i], acc[i][j], 0, 0, 0);
     };
 
@@ -348,7 +362,7 @@ __global__ void __launch_bounds__(512, 2) gemm_256_kernel(G256Args g) {
     // next tile's first fragments.  (Every read of a stage completes before the barrier
     // that precedes the next stores into it.)
     const int nk = g.Kc / F8_BK;
-    bf16x8 af0[4], bf0[2], af1[4], bf1[2];
+    bf16x8 af0[TM], bf0[TN], af1[TM], bf1[TN];
     auto iteration = [&](int kt, bool have_next, bool have_next2) {
         const bf16_t* a = As + (kt & 1) * F8_A_STAGE;
         const bf16_t* b = Bs + (kt & 1) * B_STAGE;
@@ -359,12 +373,14 @@ __global__ void __launch_bounds__(512, 2) gemm_256_kernel(G256Args g) {
         load_frags(a, b, 1, false, af1, bf1);
         if (have_next) store_a(an);
         if (have_next2) load_a(kt + 2);
-        // interleave: one LDS read behind each of the first six MFMAs, then the stores and global loads
-        for (int q = 0; q < 6; ++q) { __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); }
-        for (int q = 0; q < 2; ++q) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x200, 2, 0);
-            __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
+        // interleave: one LDS read behind each of the first MFMAs, then the stores and global loads
+        if (T == 256) {
+            for (int q = 0; q < 6; ++q) { __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); }
+            for (int q = 0; q < 2; ++q) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x200, 2, 0);
+                __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
+            }
         }
         __builtin_amdgcn_sched_barrier(0);
         // region 2: MFMAs of step 1 over the weight decode + stores, the next weight loads, step-2 fragment reads
@@ -402,7 +418,7 @@ __global__ void __launch_bounds__(512, 2) gemm_256_kernel(G256Args g) {
     if (g.r_pad > 0) {
         const int rp = g.r_pad, cpr = rp >> 3;  // 16-byte chunks per row
         const bf16_t* lr = g.lora_right + (int64_t)e * g.Nout * rp;
-        for (int idx = tid; idx < 256 * cpr; idx += 512) {
+        for (int idx = tid; idx < F8_BM * cpr; idx += NT) {
             const int r = idx / cpr, c = idx - r * cpr;
             int64_t row = row0 + r;
             row = row < row_end ? row : row_end - 1;
@@ -413,7 +429,7 @@ __global__ void __launch_bounds__(512, 2) gemm_256_kernel(G256Args g) {
         }
         __syncthreads();
         for (int ks = 0; ks < (rp >> 4); ++ks) {
-            bf16x8 af[4], bfr[2];
+            bf16x8 af[TM], bfr[TN];
             load_frags(As, Bs, ks, true, af, bfr);
             mma(af, bfr);
         }
@@ -421,12 +437,12 @@ __global__ void __launch_bounds__(512, 2) gemm_256_kernel(G256Args g) {
 
     // ---- epilogue: lane holds, per (i, j) tile, row m = fr and 4 x 4 consecutive columns
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int64_t row = row0 + wm * 128 + i * 32 + fr;
+    for (int i = 0; i < TM; ++i) {
+        const int64_t row = row0 + wm * (T / 2) + i * 32 + fr;
         if (row >= row_end) continue;
         bf16_t* crow = g.C + row * g.ldc;
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
+        for (int j = 0; j < TN; ++j) {
 #pragma unroll
             for (int q4 = 0; q4 < 4; ++q4) {
                 const int n = n0 + wn * 64 + j * 32 + 8 * q4 + 4 * fh;
