@@ -35,7 +35,8 @@ struct SkinnyArgs {
     const uint8_t* scales;
     const float* global_scale;
     int32_t group, scale_dtype;
-    const float* su_f32;       // [M, r_pad] fp32 sums of x . A^T (unscaled) or NULL
+    const float* su_part;      // [su_parts][M, r_pad] fp32 partial sums of x . A^T (unscaled) or NULL
+    int32_t su_parts;
     float su_scale;
     const void* lora_B;        // [N, r] fp32 or bf16
     int32_t lora_f32, r, r_pad;
@@ -206,17 +207,9 @@ __global__ void __launch_bounds__(NW * 64) skinny_kernel(SkinnyArgs g) {
     Batch B0, B1;
     int c = c_begin;
     if (c < c_end) issue(B0, c);
-    while (c < c_end) {
-        if (c + BC < c_end) issue(B1, c + BC);
-        compute(B0, c);
-        c += BC;
-        if (c >= c_end) break;
-        if (c + BC < c_end) issue(B0, c + BC);
-        compute(B1, c);
-        c += BC;
-    }
 
-    // ---- low-rank side term (last wave): y += (s * su) . B^T with su = x . A^T from skinny_su_kernel
+    // ---- low-rank side term (last wave), under the latency of the first batch: acc = (s * su) . B^T with
+    // su = x . A^T summed from skinny_su_kernel's parts
     if (g.r_pad > 0 && wave == NW - 1) {
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
@@ -226,15 +219,34 @@ __global__ void __launch_bounds__(NW * 64) skinny_kernel(SkinnyArgs g) {
 #pragma unroll
                 for (int i = 0; i < MT; ++i) {
                     const int m = i * 32 + fr;
-                    const float* sp = g.su_f32 + (int64_t)(m < g.M ? m : 0) * g.r_pad + j0;
+                    const float* sp = g.su_part + (int64_t)(m < g.M ? m : 0) * g.r_pad + j0;
+                    f32x4 s0 = {0.0f, 0.0f, 0.0f, 0.0f}, s1 = s0;
+#pragma unroll 4
+                    for (int kb = 0; kb < g.su_parts; ++kb) {   // fixed order
+                        s0 += *(const f32x4*)(sp + (int64_t)kb * g.M * g.r_pad);
+                        s1 += *(const f32x4*)(sp + (int64_t)kb * g.M * g.r_pad + 4);
+                    }
                     uint32_t o[4];
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) o[e] = pack_bf16x2(sp[2 * e] * g.su_scale, sp[2 * e + 1] * g.su_scale);
+                    for (int e = 0; e < 2; ++e) {
+                        o[e] = pack_bf16x2(s0[2 * e] * g.su_scale, s0[2 * e + 1] * g.su_scale);
+                        o[2 + e] = pack_bf16x2(s1[2 * e] * g.su_scale, s1[2 * e + 1] * g.su_scale);
+                    }
                     u32x4 r = {o[0], o[1], o[2], o[3]};
                     acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lb, __builtin_bit_cast(bf16x8, r), acc[i], 0, 0, 0);
                 }
             }
         }
+    }
+
+    while (c < c_end) {
+        if (c + BC < c_end) issue(B1, c + BC);
+        compute(B0, c);
+        c += BC;
+        if (c >= c_end) break;
+        if (c + BC < c_end) issue(B0, c + BC);
+        compute(B1, c);
+        c += BC;
     }
 
     // ---- cross-wave reduction through LDS, summed in wave order (the x tiles are dead by now)
@@ -264,18 +276,22 @@ __global__ void __launch_bounds__(NW * 64) skinny_kernel(SkinnyArgs g) {
     }
 }
 
-// su_f32[M, r_pad] = x[M, K] . A[r, K]^T (fp32, unscaled; columns r..r_pad-1 are zero).  One block;
-// its SU_NW waves split K, partial sums meet in LDS and are added in wave order (deterministic).
-constexpr int SU_NW = 8;
+// Partial sums of su = x[M, K] . A[r, K]^T (fp32, unscaled): block kb covers K range
+// [kb*SU_KB, (kb+1)*SU_KB) with its 8 waves (one eighth each, summed through LDS in wave order) and
+// writes part[kb][M][r_pad]; columns r..r_pad-1 are zero.  skinny_kernel adds the parts in block
+// order, so the low-rank term is deterministic and needs no zeroed buffer and no atomics.
+constexpr int SU_KB = 512, SU_NW = 8;
 template <int MT>
 __global__ void __launch_bounds__(SU_NW * 64) skinny_su_kernel(const bf16_t* x, int64_t ldx, int M, int K, const void* A,
-                                                              int a_f32, int r, int r_pad, float* su_f32) {
+                                                              int a_f32, int r, int r_pad, float* part) {
     extern __shared__ __attribute__((aligned(16))) float red[];   // [SU_NW][MT*16][64]
     const int tid = threadIdx.x, lane = tid & 63, fr = lane & 31, fh = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int steps = K >> 4;
-    const int s_begin = (steps * wave) / SU_NW, s_end = (steps * (wave + 1)) / SU_NW;
+    const int kb0 = blockIdx.x * SU_KB;
+    constexpr int SPW = SU_KB / 16 / SU_NW;   // k16 steps per wave
+    float* out = part + (int64_t)blockIdx.x * M * r_pad;
     const int nt = (r_pad + 31) >> 5;
+    const bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
     for (int j = 0; j < nt; ++j) {
         const int rrow = j * 32 + fr;
         const bool rvalid = rrow < r;
@@ -284,15 +300,25 @@ __global__ void __launch_bounds__(SU_NW * 64) skinny_su_kernel(const bf16_t* x, 
         for (int i = 0; i < MT; ++i)
 #pragma unroll
             for (int q = 0; q < 16; ++q) acc[i][q] = 0.0f;
-        for (int st = s_begin; st < s_end; ++st) {
-            const int k = st * 16 + fh * 8;
-            const bf16x8 af = factor_frag(A, (int64_t)(rvalid ? rrow : 0) * K + k, a_f32 != 0, rvalid ? 8 : 0);
 #pragma unroll
-            for (int i = 0; i < MT; ++i) {
-                const int m = i * 32 + fr;
-                const bf16x8 xf = *(const bf16x8*)(x + (int64_t)(m < M ? m : 0) * ldx + k);
-                acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, xf, acc[i], 0, 0, 0);   // D[rank][m]
+        for (int s0 = 0; s0 < SPW; s0 += 4) {
+            bf16x8 af[4], xf[MT][4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {     // the loads of four steps are issued together
+                const int kk = kb0 + (wave * SPW + s0 + u) * 16;
+                const bool kvalid = kk < K;   // wave-uniform (K % 16 == 0)
+                const int k = kk + fh * 8;
+                af[u] = kvalid ? factor_frag(A, (int64_t)(rvalid ? rrow : 0) * K + k, a_f32 != 0, rvalid ? 8 : 0) : z;
+#pragma unroll
+                for (int i = 0; i < MT; ++i) {
+                    const int m = i * 32 + fr;
+                    xf[i][u] = kvalid ? *(const bf16x8*)(x + (int64_t)(m < M ? m : 0) * ldx + k) : z;
+                }
             }
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+#pragma unroll
+                for (int i = 0; i < MT; ++i) acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[u], xf[i][u], acc[i], 0, 0, 0);   // D[rank][m]
         }
         constexpr int R = MT * 16;
         __syncthreads();   // the previous rank tile's sums have been read
@@ -307,7 +333,7 @@ __global__ void __launch_bounds__(SU_NW * 64) skinny_su_kernel(const bf16_t* x, 
             for (int w = 0; w < SU_NW; ++w) v += red[(w * R + idx) * 64 + lane];
             const int i = idx >> 4, q = idx & 15;
             const int m = i * 32 + fr, rr = j * 32 + (q & 3) + 4 * fh + 8 * (q >> 2);
-            if (m < M && rr < r_pad) su_f32[(int64_t)m * r_pad + rr] = v;
+            if (m < M && rr < r_pad) out[(int64_t)m * r_pad + rr] = v;
         }
     }
 }
@@ -315,8 +341,8 @@ __global__ void __launch_bounds__(SU_NW * 64) skinny_su_kernel(const bf16_t* x, 
 static inline int64_t al256(int64_t b) { return (b + 255) & ~(int64_t)255; }
 
 int64_t skinny_workspace_bytes(int64_t M, int64_t N, int64_t K, int r_pad) {
-    (void)N; (void)K;
-    return al256(M * (r_pad ? r_pad : 16) * 4) + 256;
+    (void)N;
+    return al256(xq_cdiv(K, SU_KB) * M * (r_pad ? r_pad : 16) * 4) + 256;
 }
 
 bool skinny_supported(const xq_weight* w, int64_t M) {
@@ -363,20 +389,21 @@ int launch_skinny(const xq_weight* w, const bf16_t* x, int64_t ldx, int64_t M, c
                "xq_linear_fwd: workspace missing, misaligned or too small for the skinny path");
     XQ_REQUIRE(ldx % 8 == 0 && xq_aligned(x, 16) && xq_aligned(w->packed, 16), "xq_linear_fwd: operands must be 16-byte aligned");
     XQ_REQUIRE(rp == 0 || xq_aligned(lora_A, 4) && xq_aligned(lora_B, 4), "xq_linear_fwd: LoRA factors must be 4-byte aligned");
-    float* su_f32 = (float*)workspace;
+    float* su_part = (float*)workspace;
+    const int su_parts = (int)xq_cdiv(K, SU_KB);
 
     int rc;
     if (rp) {
         const int f32 = lora_dtype == XQ_DT_F32;
-        if (M <= 32) skinny_su_kernel<1><<<dim3(1), SU_NW * 64, (size_t)SU_NW * 16 * 64 * 4, stream>>>(x, ldx, (int)M, (int)K, lora_A, f32, r, rp, su_f32);
-        else skinny_su_kernel<2><<<dim3(1), SU_NW * 64, (size_t)SU_NW * 32 * 64 * 4, stream>>>(x, ldx, (int)M, (int)K, lora_A, f32, r, rp, su_f32);
+        if (M <= 32) skinny_su_kernel<1><<<dim3(su_parts), SU_NW * 64, (size_t)SU_NW * 16 * 64 * 4, stream>>>(x, ldx, (int)M, (int)K, lora_A, f32, r, rp, su_part);
+        else skinny_su_kernel<2><<<dim3(su_parts), SU_NW * 64, (size_t)SU_NW * 32 * 64 * 4, stream>>>(x, ldx, (int)M, (int)K, lora_A, f32, r, rp, su_part);
         XQ_CHECK_LAUNCH("skinny_su");
     }
     SkinnyArgs g;
     g.x = x; g.ldx = ldx; g.M = (int)M; g.N = (int)N; g.K = (int)K;
     g.packed = (const uint8_t*)w->packed; g.scales = (const uint8_t*)w->scales; g.global_scale = w->global_scale;
     g.group = w->group; g.scale_dtype = w->scale_dtype;
-    g.su_f32 = rp ? su_f32 : nullptr; g.su_scale = scaling; g.lora_B = rp ? lora_B : nullptr;
+    g.su_part = rp ? su_part : nullptr; g.su_parts = su_parts; g.su_scale = scaling; g.lora_B = rp ? lora_B : nullptr;
     g.lora_f32 = lora_dtype == XQ_DT_F32; g.r = r; g.r_pad = rp;
     g.bias = bias; g.y = y; g.ldy = ldy;
     // algorithmic bytes: packed weight + scales + x + y (+ LoRA factors), for the roofline figure
