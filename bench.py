@@ -237,7 +237,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--cpu-rows", type=int, default=2048, help="token rows of the CPU baseline sample (0 = skip)")
+    ap.add_argument("--cpu-rows", type=int, default=8192, help="token rows of the CPU baseline sample (0 = skip)")
     ap.add_argument("--config", type=int, default=1,
                     help="BASELINE.json configs index; 1 (default) is the headline workload, the others report the "
                          "same JSON for their own workload (no CPU baseline)")
