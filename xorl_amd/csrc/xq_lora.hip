@@ -67,10 +67,16 @@ struct SmallNtArgs {
 };
 
 // TR rows per block: 32 (dense; the 4 waves split K) or 128 (grouped; one wave per 32 rows).
+// Both operands are fetched with coalesced 16-byte loads (16 lanes per 256-byte row piece, 4 rows
+// per instruction) and reach the MFMA operand layout through wave-private LDS tiles of 128 k per
+// row (row pitch 272 B: the 16 lanes of a b128 read phase hit distinct banks); per-lane row-strided
+// loads would touch 64 cache lines per instruction and leave the kernel address-unit bound.
+constexpr int SN_P = 136;   // LDS row pitch in bf16 elements
 template <int TR, int NT>
 __global__ void __launch_bounds__(256) small_nt_kernel(SmallNtArgs g) {
     constexpr int RG = TR / 32, KS = 4 / RG;
-    __shared__ float red[KS > 1 ? (KS - 1) * NT * 64 * 16 : 1];
+    constexpr int WTILE = (32 + NT * 32) * SN_P;   // bf16 elements per wave: In tile + F tile
+    extern __shared__ __attribute__((aligned(16))) bf16_t sn_lds[];
     __shared__ int sh_info[3];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int rg = wave % RG, ks = wave / RG;
@@ -99,18 +105,13 @@ __global__ void __launch_bounds__(256) small_nt_kernel(SmallNtArgs g) {
         if (row0 >= row_end) return;
     }
     const bf16_t* F = g.F + (int64_t)e * g.f_stride;
+    bf16_t* xs = sn_lds + wave * WTILE;          // [32][SN_P]
+    bf16_t* fs = xs + 32 * SN_P;                 // [NT*32][SN_P]
     const int fr = lane & 31, fk = (lane >> 5) * 8;
-    int64_t arow = row0 + rg * 32 + fr;
-    arow = arow < row_end ? arow : row_end - 1;
-    const bf16_t* ap = g.In + arow * g.ld_in + fk;
-    const bf16_t* fp[NT];
-    bool fvalid[NT];
-#pragma unroll
-    for (int n = 0; n < NT; ++n) {
-        int j = n * 32 + fr;
-        fvalid[n] = j < g.r_pad;
-        fp[n] = F + (int64_t)(fvalid[n] ? j : 0) * g.Kc + fk;
-    }
+    const int crow = lane >> 4, cpiece = (lane & 15) * 8;   // coalesced fetch: row within a group of 4, k offset
+    const int64_t wrow0 = row0 + rg * 32;
+    const int frows = g.r_pad;                   // rows of F in use (multiple of 16)
+
     f32x16 acc[NT];
 #pragma unroll
     for (int n = 0; n < NT; ++n)
@@ -119,31 +120,42 @@ __global__ void __launch_bounds__(256) small_nt_kernel(SmallNtArgs g) {
 
     const int64_t kspan = g.Kc / KS;  // multiple of 16
     const int64_t kbeg = ks * kspan, kend = kbeg + kspan;
-    const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
-    int64_t k = kbeg;
-    for (; k + 64 <= kend; k += 64) {
-        bf16x8 a[4], b[NT][4];
+    u32x4 xr[8], fq[NT * 8];
+    auto fetch = [&](int64_t k) {     // chunk [k, k+128) clipped to kend; rows clamped to the segment / to F
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            a[u] = *(const bf16x8*)(ap + k + u * 16);
-#pragma unroll
-            for (int n = 0; n < NT; ++n) b[n][u] = fvalid[n] ? *(const bf16x8*)(fp[n] + k + u * 16) : zero8;
+        for (int j = 0; j < 8; ++j) {
+            int64_t r = wrow0 + j * 4 + crow;
+            r = r < row_end ? r : row_end - 1;
+            if (k + cpiece < kend) xr[j] = *(const u32x4*)(g.In + r * g.ld_in + k + cpiece);
         }
 #pragma unroll
-        for (int u = 0; u < 4; ++u)
+        for (int j = 0; j < NT * 8; ++j)
+            if (j * 4 < frows && k + cpiece < kend) fq[j] = *(const u32x4*)(F + (int64_t)(j * 4 + crow) * g.Kc + k + cpiece);
+    };
+    if (kbeg < kend) fetch(kbeg);
+    for (int64_t k = kbeg; k < kend; k += 128) {
+        // LDS operations of one wave execute in order: the previous chunk's fragment reads are ahead of these writes
 #pragma unroll
-            for (int n = 0; n < NT; ++n) acc[n] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[u], b[n][u], acc[n], 0, 0, 0);
-    }
-    for (; k < kend; k += 16) {
-        bf16x8 a = *(const bf16x8*)(ap + k);
+        for (int j = 0; j < 8; ++j) *(u32x4*)(xs + (j * 4 + crow) * SN_P + cpiece) = xr[j];
 #pragma unroll
-        for (int n = 0; n < NT; ++n) {
-            bf16x8 b = fvalid[n] ? *(const bf16x8*)(fp[n] + k) : zero8;
-            acc[n] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[n], 0, 0, 0);
+        for (int j = 0; j < NT * 8; ++j)
+            if (j * 4 < frows) *(u32x4*)(fs + (j * 4 + crow) * SN_P + cpiece) = fq[j];
+        if (k + 128 < kend) fetch(k + 128);
+        const int nsteps = (int)((kend - k < 128 ? kend - k : 128) >> 4);
+        for (int st = 0; st < nsteps; ++st) {
+            const bf16x8 a = *(const bf16x8*)(xs + fr * SN_P + st * 16 + fk);
+#pragma unroll
+            for (int n = 0; n < NT; ++n) {
+                const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+                const bf16x8 b = (n * 32 + fr < frows) ? *(const bf16x8*)(fs + (n * 32 + fr) * SN_P + st * 16 + fk) : zero8;
+                acc[n] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[n], 0, 0, 0);
+            }
         }
     }
 
     if (KS > 1) {
+        float* red = (float*)sn_lds;   // [(KS-1)][NT][16][64] floats, over the (now dead) tiles
+        __syncthreads();
         if (ks > 0) {
 #pragma unroll
             for (int n = 0; n < NT; ++n)
@@ -172,6 +184,22 @@ __global__ void __launch_bounds__(256) small_nt_kernel(SmallNtArgs g) {
     }
 }
 
+template <int TR, int NT>
+static int launch_small_nt_one(const SmallNtArgs& g, unsigned blocks, hipStream_t stream) {
+    constexpr size_t lds = (size_t)4 * (32 + NT * 32) * SN_P * 2;
+    static bool attr_set = false;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute((const void*)small_nt_kernel<TR, NT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) {
+            xq_set_error("small_nt: cannot raise the dynamic LDS limit: %s", hipGetErrorString(e));
+            return XQ_ERR_LAUNCH;
+        }
+        attr_set = true;
+    }
+    small_nt_kernel<TR, NT><<<dim3(blocks), 256, lds, stream>>>(g);
+    return XQ_OK;
+}
+
 int launch_small_nt(const bf16_t* In, int64_t ld_in, int64_t n_rows, int64_t Kc, const bf16_t* F, int r_pad,
                     float scale, bf16_t* T, const int32_t* offsets, const int32_t* tile_offsets,
                     int32_t num_experts, bool shared_f, hipStream_t stream) {
@@ -181,16 +209,16 @@ int launch_small_nt(const bf16_t* In, int64_t ld_in, int64_t n_rows, int64_t Kc,
     if (n_rows == 0) return XQ_OK;
     SmallNtArgs g{In, ld_in, n_rows, Kc, F, shared_f ? 0 : (int64_t)r_pad * Kc, r_pad, scale, T, offsets, tile_offsets,
                   num_experts};
+    int rc;
     if (offsets) {
         unsigned blocks = (unsigned)(xq_cdiv(n_rows, 128) + num_experts);
-        if (r_pad <= 32) small_nt_kernel<128, 1><<<dim3(blocks), 256, 0, stream>>>(g);
-        else small_nt_kernel<128, 2><<<dim3(blocks), 256, 0, stream>>>(g);
+        rc = r_pad <= 32 ? launch_small_nt_one<128, 1>(g, blocks, stream) : launch_small_nt_one<128, 2>(g, blocks, stream);
     } else {
         g.f_stride = 0;
         unsigned blocks = (unsigned)xq_cdiv(n_rows, 32);
-        if (r_pad <= 32) small_nt_kernel<32, 1><<<dim3(blocks), 256, 0, stream>>>(g);
-        else small_nt_kernel<32, 2><<<dim3(blocks), 256, 0, stream>>>(g);
+        rc = r_pad <= 32 ? launch_small_nt_one<32, 1>(g, blocks, stream) : launch_small_nt_one<32, 2>(g, blocks, stream);
     }
+    if (rc) return rc;
     XQ_CHECK_LAUNCH("small_nt");
     return XQ_OK;
 }
