@@ -138,7 +138,7 @@ def dense_module(fmt, N, K, r, alpha, seed, dev):
 
 
 def other_config(cfg: int, dev):
-    """Builds BASELINE.json configs[0], [2], [3] or [4] on the device.  Returns
+    """Builds BASELINE.json configs[0], [2], [3] or [4] (or the merge pass, 5) on the device.  Returns
     (step_fn, work_per_step, unit_is_bytes, workload_text, kernel_text)."""
     lin_flops = lambda m, K, N, r: 4.0 * m * K * N + 6.0 * m * r * (K + N)
     rnd = lambda *shape, seed: torch.randn(*shape, generator=torch.Generator(device=dev).manual_seed(seed),
@@ -216,6 +216,29 @@ def other_config(cfg: int, dev):
                 "configs[4]: skinny-M forward, M in {1,8,32,64} x {q 4096->4096, kv 4096->1024, gate/up 4096->12288, "
                 "down 12288->4096} x {int4, block_fp8}, r=16 (32 launches per step)",
                 "skinny_kernel<int4|fp8> (weight-streaming fused dequant-GEMV/GEMM)")
+    if cfg == 5:
+        # not a BASELINE config: the merge / re-quantise pass over configs[1]'s three block_fp8 weights (r = 32)
+        from xorl_amd.functional import merge_dense, merge_requant_fp8
+
+        mods = [dense_module("block_fp8", N, K, 32, 64, 80 + i, dev) for i, (N, K) in
+                enumerate(((12288, 4096), (12288, 4096), (4096, 12288)))]
+        outs = [(torch.empty(m.out_features, m.in_features, dtype=torch.uint8, device=dev),
+                 torch.empty((m.out_features + 127) // 128, (m.in_features + 127) // 128, dtype=torch.float32, device=dev))
+                for m in mods]
+        total = 0.0
+        for m in mods:
+            nk = m.out_features * m.in_features
+            total += 2 * (nk + 4 * ((m.out_features + 127) // 128) * ((m.in_features + 127) // 128)) + (nk + 2 * nk)
+
+        def step():
+            with torch.no_grad():
+                for m, (po, so) in zip(mods, outs):
+                    merge_requant_fp8(m._quant_weight(), m.lora_A, m.lora_B, 32, 2.0, po, so)
+                    merge_dense(m._quant_weight(), m.lora_A, m.lora_B, 32, 2.0, torch.bfloat16)
+        return (step, total, True,
+                "merge pass (not a BASELINE config): decode + LoRA update + re-encode (block_fp8 -> block_fp8) and "
+                "decode + update -> bf16, for gate/up [12288,4096] and down [4096,12288], r=32",
+                "merge_kernel<fp8> (fused decode + low-rank update + re-quantise / publish)")
     raise SystemExit(f"bench.py: unknown --config {cfg}")
 
 

@@ -136,6 +136,29 @@ int xq_linear_bwd(const xq_weight* w, const void* x, int64_t ldx, const void* dy
                   float scaling, const void* su, void* dx, int64_t lddx, float* dA, float* dB,
                   void* workspace, int64_t workspace_bytes, void* stream);
 
+/* ---- merging the LoRA update into the base weight ------------------------
+ * W'[n,k] = deq(W)[n,k] + scaling * sum_j B[n,j] * A[j,k], W FLAT [N, K]
+ * (in_features % 16 == 0), factors fp32 or bf16, r in {0..64}; the low-rank
+ * product is evaluated to ~16 significant bits per factor (hi/lo bf16 split).
+ *
+ * xq_merge_dense writes W' as bf16 or fp32 [N, K] without materialising
+ * deq(W).  bf16: bf16(bf16(deq) + bf16(delta)), the arithmetic of the
+ * reference's weight-sync merge (server/weight_sync/handler.py:2119-2131:
+ * `_dequantize_weight().to(bf16) + get_delta_weight().to(bf16)`).  fp32: the
+ * sum merge_weights forms before it re-quantises (qlora/modules/
+ * block_fp8_linear.py:111-115; for the 4-bit formats, whose decoders return
+ * bf16, the bf16 sum widened to fp32).
+ *
+ * xq_merge_requant_fp8 (block_fp8 only) is merge_weights + _quantize_and_store
+ * in one pass (block_fp8_linear.py:111-119 with block_fp8_quantize_gkn,
+ * ops/quantize/block_fp8_gkn_quantize.py:40-121): per 128x128 block
+ * s = max(amax(W') / 448, 1e-12), bytes = e4m3(clamp(W' / s, +-448)).
+ * packed_out / scales_out may be the weight's own buffers (in-place). */
+int xq_merge_dense(const xq_weight* w, const void* lora_A, const void* lora_B, int lora_dtype, int r,
+                   float scaling, void* out, int out_dtype, void* stream);
+int xq_merge_requant_fp8(const xq_weight* w, const void* lora_A, const void* lora_B, int lora_dtype, int r,
+                         float scaling, void* packed_out, float* scales_out, void* stream);
+
 /* ---- SwiGLU between gate/up and down ------------------------------------
  * Replaces fused_silu_and_mul (ops/fused_silu_and_mul.py:22-60 and its
  * backward): h = bf16(silu_fp32(gate)) * up, two roundings.  With row_w

@@ -199,3 +199,23 @@ def max_rel_err(got: torch.Tensor, ref: torch.Tensor) -> float:
     if denom == 0.0:
         return float((got.double() - ref).abs().max().item())
     return float((got.double() - ref).abs().max().item() / denom)
+
+
+# ---------------------------------------------------------------------------
+# merging the LoRA update into the base weight
+# ---------------------------------------------------------------------------
+def merge_delta_exact(lora_A: torch.Tensor, lora_B: torch.Tensor, scaling: float) -> torch.Tensor:
+    """get_delta_weight (qlora/modules/linear.py:397-400): (B @ A) * scaling, here with the product in
+    float64 and one rounding to fp32 at the end (the reference's fp32 matmul has an unspecified
+    summation order; any order is within a few fp32 ulps of this)."""
+    return ((lora_B.double() @ lora_A.double()) * scaling).float()
+
+
+def merge_publish_recipe(w_deq: torch.Tensor, lora_A, lora_B, scaling: float) -> torch.Tensor:
+    """server/weight_sync/handler.py:2119-2131: `deq.to(bf16) + delta.to(bf16)` (a bf16 add)."""
+    return w_deq.to(torch.bfloat16) + merge_delta_exact(lora_A, lora_B, scaling).to(torch.bfloat16)
+
+
+def merge_fp32_recipe(w_deq_f32: torch.Tensor, lora_A, lora_B, scaling: float) -> torch.Tensor:
+    """block_fp8 merge_weights before re-quantisation (block_fp8_linear.py:111-115): fp32 deq + fp32 delta."""
+    return w_deq_f32.float() + merge_delta_exact(lora_A, lora_B, scaling)

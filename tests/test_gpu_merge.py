@@ -1,0 +1,121 @@
+"""GPU parity: merging the LoRA update into the quantized base weight (through the C ABI)
+vs the CPU oracle.
+
+publish  : bf16(bf16(deq) + bf16(delta)) -- the reference's weight-sync arithmetic.  Expected bit-exact
+           except where the fp32 value of delta lies within the kernel's product error (2^-16 relative per
+           factor) of a bf16 rounding boundary; the test allows one bf16 step at operand magnitude on at
+           most 1e-3 of the elements.
+requant  : block_fp8 decode -> add -> re-encode.  With the LoRA update switched off the kernel must
+           reproduce the oracle quantizer byte for byte on the decoded weight (the e4m3 encoder, the
+           division and the block absmax are then the only arithmetic); with a large update on, scales match
+           to 5e-5 relative and bytes differ by at most one code on at most 5e-3 of the elements.
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import cdecode as C
+from oracle import recipe as R
+from tests.util_cases import gen, make_dense_module
+
+pytestmark = pytest.mark.gpu
+
+
+def _deq_f32(m, w_ref_bf16):
+    """fp32 decode of a block_fp8 module from the oracle (fl(e4m3 * scale)); bf16 decode for the others."""
+    if m.quant_format != "block_fp8":
+        return w_ref_bf16.float()
+    N, K = m.out_features, m.in_features
+    packed = m.packed_weight_f32.detach().cpu().contiguous().view(torch.uint8).numpy().reshape(N, K)
+    s = m.weight_block_scales.cpu().contiguous().view(torch.float32).numpy()
+    from oracle import decode_np as NP
+
+    return torch.from_numpy(NP.fp8_decode(packed, s, N, K)[0].copy())
+
+
+@pytest.mark.parametrize("fmt", ["block_fp8", "int4", "nvfp4"])
+@pytest.mark.parametrize("N,K,r", [(384, 256, 16), (200, 320, 24), (1024, 512, 64), (128, 128, 0)])
+def test_merge_publish_bf16(hip_device, fmt, N, K, r):
+    if fmt != "block_fp8" and N % 16:
+        N = 208
+    if fmt == "int4" and K % 128:
+        K = 384
+    m, w_ref = make_dense_module(fmt, N, K, max(r, 8), 32, seed=N + K, device=hip_device)
+    if r == 0:
+        with torch.no_grad():
+            m.lora_B.zero_()
+    else:
+        m.set_runtime_lora_config(r, 2 * r) if r != m.r else None
+    got = m.merged_weight(torch.bfloat16).cpu()
+    A, B = m.lora_A.detach().cpu()[: m.active_r], m.lora_B.detach().cpu()[:, : m.active_r]
+    want = R.merge_publish_recipe(_deq_f32(m, w_ref), A, B, m._active_scaling())
+    assert got.shape == (N, K) and got.dtype == torch.bfloat16
+    mism = got.view(torch.int16) != want.view(torch.int16)
+    assert float(mism.float().mean()) <= 1e-3
+    # where they differ it is by one bf16 step of the update (its own rounding may flip) plus one of the result
+    a = _deq_f32(m, w_ref).to(torch.bfloat16).float().abs()
+    # the low-rank product carries ~2^-16 relative error per TERM, i.e. relative to sum_j |B||A|, not to a
+    # sum that cancels
+    terms = (B.abs().double() @ A.abs().double()).float() * abs(m._active_scaling())
+    delta_bf16 = R.merge_delta_exact(A, B, m._active_scaling()).to(torch.bfloat16).float().abs()
+    tol = 2.0 ** -7 * (torch.maximum(a, want.float().abs()) + delta_bf16) + 2.0 ** -14 * terms
+    assert bool(((got.float() - want.float()).abs() <= tol).all())
+    if r == 0:
+        assert not bool(mism.any())           # no update: the decoded weight itself
+
+
+@pytest.mark.parametrize("N,K", [(384, 256), (200, 320), (1024, 1024)])
+def test_requant_identity_matches_oracle_quantizer(hip_device, N, K):
+    """LoRA off: requant(deq(W)) must equal the oracle quantizer applied to the oracle decode, byte for byte."""
+    from xorl_amd.functional import merge_requant_fp8
+
+    m, w_ref = make_dense_module("block_fp8", N, K, 8, 16, seed=3 * N + K, device=hip_device)
+    deq = _deq_f32(m, w_ref).numpy()
+    want_b, want_s = C.fp8_quantize(deq, 128, 1.0)
+    packed, scales = merge_requant_fp8(m._quant_weight(), None, None, 0, 1.0)
+    got_b, want_b = packed.cpu().numpy(), want_b.reshape(N, K)
+    # a decoded -0 plus the (+0) update is +0, as in the reference's `w + delta`: byte 0x00 where the
+    # quantizer alone would keep 0x80
+    neg_zero = (want_b == 0x80) & (deq == 0)
+    assert np.array_equal(np.where(neg_zero, 0, want_b), got_b)
+    assert np.array_equal(scales.cpu().numpy().view(np.uint32).ravel(), want_s.view(np.uint32).ravel())
+
+
+@pytest.mark.parametrize("N,K,r", [(384, 256, 16), (200, 320, 32), (1024, 512, 64)])
+def test_merge_requant_fp8(hip_device, N, K, r):
+    from xorl_amd.functional import merge_dense, merge_requant_fp8
+
+    m, w_ref = make_dense_module("block_fp8", N, K, r, 4 * r, seed=N - K, device=hip_device)
+    with torch.no_grad():                      # a visible update: |delta| comparable to the e4m3 step
+        m.lora_A.mul_(8.0)
+        m.lora_B.mul_(8.0)
+    A, B, s = m.lora_A.detach().cpu(), m.lora_B.detach().cpu(), m._active_scaling()
+    merged = R.merge_fp32_recipe(_deq_f32(m, w_ref), A, B, s)
+    # fp32 sum from the kernel: within the product error of the oracle's
+    got32 = merge_dense(m._quant_weight(), m.lora_A, m.lora_B, r, s, torch.float32).cpu()
+    assert R.max_rel_err(got32, merged) <= 1e-5
+    want_b, want_s = C.fp8_quantize(merged.numpy(), 128, 1.0)
+    packed, scales = merge_requant_fp8(m._quant_weight(), m.lora_A, m.lora_B, r, s)
+    sc = scales.cpu().numpy()
+    assert np.allclose(sc, want_s.reshape(sc.shape), rtol=5e-5, atol=0)
+    gb, wb = packed.cpu().numpy().astype(np.int32), want_b.reshape(N, K).astype(np.int32)
+    assert float((gb != wb).mean()) <= 5e-3
+    sg, sw = np.where(gb & 0x80, -(gb & 0x7f), gb & 0x7f), np.where(wb & 0x80, -(wb & 0x7f), wb & 0x7f)
+    assert bool(((np.abs(sg - sw) <= 1) | ((np.abs(sg) <= 1) & (np.abs(sw) <= 1))).all())   # neighbouring codes only
+    # the module method: in place, LoRA reset, and the new weight decodes to ~merged (e4m3 step: 2^-4 relative)
+    m.merge_weights()
+    assert torch.count_nonzero(m.lora_B) == 0
+    w_new = m._dequantize_weight().cpu().float()
+    assert R.max_rel_err(w_new, merged) <= 2 ** -4
+
+
+def test_merge_errors(hip_device):
+    from xorl_amd import _C
+    from xorl_amd.functional import merge_requant_fp8
+
+    m, _ = make_dense_module("int4", 256, 256, 8, 16, seed=1, device=hip_device)
+    with pytest.raises(ValueError):
+        merge_requant_fp8(m._quant_weight(), m.lora_A, m.lora_B, 8, 2.0)      # block_fp8 only
+    with pytest.raises(ValueError):
+        m.merged_weight(torch.float16)

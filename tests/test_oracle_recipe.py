@@ -182,3 +182,21 @@ def test_grouped_bf16_recipe_close_to_exact():
     lo = R.moe_fwd_bwd(hidden, rw, sel, wg, wu, wd, lora, 0.5, dy, dtype=torch.bfloat16)
     assert R.max_rel_err(lo["y"], ex["y"]) < 3e-2
     assert R.max_rel_err(lo["dx"], ex["dx"]) < 3e-2
+
+
+def test_merge_recipes():
+    """merge_delta_exact against a per-element brute force; the publish recipe is a bf16 add of two bf16
+    tensors; zero B leaves the decoded weight; the fp32 recipe is linear in the scaling."""
+    N, K, r = 24, 40, 5
+    g = torch.Generator().manual_seed(5)
+    A, B = torch.randn(r, K, generator=g) * 0.1, torch.randn(N, r, generator=g) * 0.1
+    w = torch.randn(N, K, generator=g) * 0.02
+    d = R.merge_delta_exact(A, B, 1.7)
+    brute = torch.tensor([[1.7 * sum(float(B[n, j]) * float(A[j, k]) for j in range(r)) for k in range(K)] for n in range(N)])
+    assert torch.allclose(d.double(), brute.double(), rtol=1e-6, atol=1e-12)
+    pub = R.merge_publish_recipe(w, A, B, 1.7)
+    assert pub.dtype == torch.bfloat16
+    assert torch.equal(pub, (w.to(torch.bfloat16).float() + d.to(torch.bfloat16).float()).to(torch.bfloat16))
+    assert torch.equal(R.merge_publish_recipe(w, A, torch.zeros_like(B), 1.7), w.to(torch.bfloat16))
+    m1, m2 = R.merge_fp32_recipe(w, A, B, 1.0), R.merge_fp32_recipe(w, A, B, 2.0)
+    assert torch.allclose((m2 - w).double(), 2 * (m1 - w).double(), rtol=1e-5, atol=1e-7)

@@ -226,3 +226,46 @@ class SiluAndMulFunction(torch.autograd.Function):
 
 def silu_and_mul(gate: Tensor, up: Tensor) -> Tensor:
     return SiluAndMulFunction.apply(gate, up)
+
+
+# ---------------------------------------------------------------------------
+# merging the LoRA update into the base weight
+# ---------------------------------------------------------------------------
+def merge_dense(qw: QuantWeight, lora_A: Optional[Tensor], lora_B: Optional[Tensor], r: int, scaling: float,
+                out_dtype: torch.dtype = torch.bfloat16) -> Tensor:
+    """deq(W) + scaling * B[:, :r] @ A[:r] as bf16 (weight-sync arithmetic, server/weight_sync/handler.py:2119-2131)
+    or fp32 (the sum merge_weights re-quantises, qlora/modules/block_fp8_linear.py:111-115), [N, K]; deq(W) is
+    never materialised."""
+    _C.require_hip(qw.packed, lora_A, lora_B)
+    if out_dtype not in (torch.bfloat16, torch.float32):
+        raise _C.XqError(f"merge_dense: out_dtype must be bf16 or fp32, got {out_dtype}")
+    dev = qw.packed.device
+    A = lora_A[:r].contiguous() if r > 0 else None
+    B = lora_B[:, :r].contiguous() if r > 0 else None
+    out = torch.empty(qw.rows, qw.cols, dtype=out_dtype, device=dev)
+    w = qw.c()
+    _C.check(_C.lib().xq_merge_dense(ctypes.byref(w), _C.ptr(A), _C.ptr(B), _lora_dt(A), r, float(scaling),
+                                     out.data_ptr(), _C.XQ_DT_BF16 if out_dtype == torch.bfloat16 else _C.XQ_DT_F32,
+                                     _C.stream_ptr(dev)))
+    return out
+
+
+def merge_requant_fp8(qw: QuantWeight, lora_A: Optional[Tensor], lora_B: Optional[Tensor], r: int, scaling: float,
+                      packed_out: Optional[Tensor] = None, scales_out: Optional[Tensor] = None) -> Tuple[Tensor, Tensor]:
+    """block_fp8 only: Q(deq(W) + scaling * B @ A) with fresh 128x128 block scales in one pass
+    (merge_weights + _quantize_and_store, qlora/modules/block_fp8_linear.py:111-119).  Returns (e4m3 bytes as
+    uint8 [N, K], fp32 scales [ceil(N/128), ceil(K/128)]); pass the weight's own buffers to update in place."""
+    _C.require_hip(qw.packed, lora_A, lora_B)
+    if qw.fmt != "block_fp8":
+        raise _C.XqError(f"merge_requant_fp8: the weight must be block_fp8, got {qw.fmt}")
+    dev = qw.packed.device
+    A = lora_A[:r].contiguous() if r > 0 else None
+    B = lora_B[:, :r].contiguous() if r > 0 else None
+    if packed_out is None:
+        packed_out = torch.empty(qw.rows, qw.cols, dtype=torch.uint8, device=dev)
+    if scales_out is None:
+        scales_out = torch.empty((qw.rows + 127) // 128, (qw.cols + 127) // 128, dtype=torch.float32, device=dev)
+    w = qw.c()
+    _C.check(_C.lib().xq_merge_requant_fp8(ctypes.byref(w), _C.ptr(A), _C.ptr(B), _lora_dt(A), r, float(scaling),
+                                           packed_out.data_ptr(), scales_out.data_ptr(), _C.stream_ptr(dev)))
+    return packed_out, scales_out

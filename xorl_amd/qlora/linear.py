@@ -319,6 +319,15 @@ class QLoRALinear(LoraModule, nn.Module):
             nn.init.kaiming_uniform_(self.lora_A, a=math.sqrt(5))
             self.lora_B.zero_()
 
+    def merged_weight(self, dtype: torch.dtype = torch.bfloat16) -> Tensor:
+        """deq(W).to(bf16) + get_delta_weight().to(bf16): the tensor the weight-sync path publishes
+        (server/weight_sync/handler.py:2119-2131), produced by one fused kernel."""
+        from ..functional import merge_dense
+
+        with torch.no_grad():
+            return merge_dense(self._quant_weight(), self._to_regular_tensor(self.lora_A),
+                               self._to_regular_tensor(self.lora_B), self.active_r, self._active_scaling(), dtype)
+
     def _requantize_merged(self, merged: Tensor, ema_decay: float) -> None:
         self._quantize_and_store(merged)
 
@@ -406,6 +415,23 @@ class BlockFP8QLoRALinear(QLoRALinear):
     def _quant_weight(self) -> QuantWeight:
         return QuantWeight("block_fp8", _C.XQ_LAYOUT_FLAT, self._read_packed_weight_uint8(),
                            self.weight_block_scales, torch.float32, self.out_features, self.in_features, 128)
+
+    def merge_weights(self, ema_decay: float = 0.1) -> None:
+        """Decode, add the LoRA update and re-encode with fresh block scales in one fused pass over the
+        bytes (block_fp8_linear.py:111-119); falls back to the generic path for sharded (DTensor) state."""
+        from ..functional import merge_requant_fp8
+
+        if _is_dtensor(self.packed_weight_f32) or _is_dtensor(self.lora_A):
+            return super().merge_weights(ema_decay)
+        with torch.no_grad():
+            packed, scales = merge_requant_fp8(self._quant_weight(), self.lora_A, self.lora_B, self.active_r,
+                                               self._active_scaling())
+            self._write_packed_weight(packed.reshape(-1))
+            self._scale_dtypes = {"weight_block_scales": torch.float32}
+            self.weight_block_scales = self._to_uint8(scales)
+            self._aqn_step_cache = None
+            nn.init.kaiming_uniform_(self.lora_A, a=math.sqrt(5))
+            self.lora_B.zero_()
 
     @torch.compiler.disable
     def _dequantize_weight(self) -> Tensor:
