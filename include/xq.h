@@ -35,6 +35,7 @@ extern "C" {
 #define XQ_FMT_INT4 0   /* 4-bit offset-binary codes, w = (nib - 8) * scale            */
 #define XQ_FMT_NVFP4 1  /* e2m1 codes, per-16 block scale * fp32 global scale          */
 #define XQ_FMT_FP8 2    /* e4m3fn bytes, fp32 scale per 128x128 block                  */
+#define XQ_FMT_NF4 3    /* NormalFloat4 codes, w = level[nib] * scale (fp32/bf16 scale) */
 
 /* storage layouts of the 4-bit formats (fp8 is symmetric: layout is ignored)
  *   FLAT: decoded shape [rows, cols]; nibble pairs and scale groups run along
@@ -62,7 +63,7 @@ typedef struct xq_weight {
     int32_t format;       /* XQ_FMT_*    */
     int32_t layout;       /* XQ_LAYOUT_* */
     int32_t scale_dtype;  /* XQ_SCALE_*  */
-    int32_t group;        /* int4: any even divisor of the grouped dim (128 typical); nvfp4: 16; fp8: 128 */
+    int32_t group;        /* int4 / nf4: any even divisor of the grouped dim (128 / 64 typical); nvfp4: 16; fp8: 128 */
     int64_t rows;         /* decoded rows */
     int64_t cols;         /* decoded cols */
     int32_t num_experts;
@@ -102,6 +103,8 @@ int xq_set_tile_policy(int policy);
  *   (ops/quantize/int4_quantize.py:113-127, int4_gkn_quantize.py:176-216),
  * nvfp4_dequantize / nvfp4_dequantize_gkn
  *   (ops/quantize/nvfp4_quantize.py:157-177, nvfp4_gkn_quantize.py:238-273),
+ * nf4_dequantize / nf4_dequantize_gkn
+ *   (ops/quantize/nf4_quantize.py:154-185, nf4_gkn_quantize.py:182-, levels nf4_codec.py:18-35),
  * block_fp8_dequantize_gkn (ops/quantize/block_fp8_gkn_quantize.py:157-180;
  *   XQ_DT_F32 gives that function's fp32 output, XQ_DT_BF16 gives the
  *   `.to(bf16)` its callers apply, qlora/modules/linear.py:373).

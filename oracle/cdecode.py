@@ -53,6 +53,14 @@ def lib() -> ctypes.CDLL:
         L.xqo_int4_quantize_flat.argtypes = [p, p, p, i64, i64]
         L.xqo_int4_quantize_gkn.argtypes = [p, p, p, i64, i64, i64]
         L.xqo_int4_quantize_sym_flat.argtypes = [p, p, p, i64, i64]
+        L.xqo_nf4_decode_flat.argtypes = [p, p, p, i64, i64]
+        L.xqo_nf4_decode_gkn.argtypes = [p, p, p, i64, i64, i64]
+        L.xqo_nf4_quantize_flat.argtypes = [p, p, p, i64, i64]
+        L.xqo_nf4_quantize_gkn.argtypes = [p, p, p, i64, i64, i64]
+        L.xqo_nf4_level.argtypes = [ctypes.c_int]
+        L.xqo_nf4_level.restype = ctypes.c_float
+        L.xqo_nf4_encode.argtypes = [ctypes.c_float]
+        L.xqo_nf4_encode.restype = ctypes.c_uint8
         L.xqo_nvfp4_decode_flat.argtypes = [p, p, f32, p, i64, i64]
         L.xqo_nvfp4_decode_gkn.argtypes = [p, p, f32, p, i64, i64, i64]
         L.xqo_nvfp4_quantize_flat.restype = f32
@@ -64,6 +72,7 @@ def lib() -> ctypes.CDLL:
         for name in (
             "xqo_int4_decode_flat", "xqo_int4_decode_gkn", "xqo_int4_quantize_flat",
             "xqo_int4_quantize_gkn", "xqo_int4_quantize_sym_flat", "xqo_nvfp4_decode_flat",
+            "xqo_nf4_decode_flat", "xqo_nf4_decode_gkn", "xqo_nf4_quantize_flat", "xqo_nf4_quantize_gkn",
             "xqo_nvfp4_decode_gkn", "xqo_fp8_decode", "xqo_fp8_quantize",
         ):
             getattr(L, name).restype = None
@@ -133,6 +142,51 @@ def int4_quantize_gkn(x, group):
     packed = np.zeros((K // 2, N), dtype=np.uint8)
     scales = np.empty((K // group, N), dtype=np.float32)
     lib().xqo_int4_quantize_gkn(_p(x), _p(packed), _p(scales), K, N, group)
+    return packed, scales
+
+
+# ---------------------------------------------------------------- nf4
+def nf4_table() -> np.ndarray:
+    L = lib()
+    return np.array([L.xqo_nf4_level(c) for c in range(16)], dtype=np.float32)
+
+
+def nf4_encode(v: np.ndarray) -> np.ndarray:
+    L = lib()
+    return np.array([L.xqo_nf4_encode(float(t)) for t in np.asarray(v, dtype=np.float32).ravel()], dtype=np.uint8)
+
+
+def nf4_decode_flat(packed, scales_f32, rows, cols, group) -> np.ndarray:
+    packed, scales = _c(packed, np.uint8), _c(scales_f32, np.float32)
+    assert packed.size == rows * cols // 2 and scales.size == rows * cols // group
+    out = np.empty((rows, cols), dtype=np.uint16)
+    lib().xqo_nf4_decode_flat(_p(packed), _p(scales), _p(out), rows * cols, group)
+    return out
+
+
+def nf4_decode_gkn(packed, scales_f32, K, N, group) -> np.ndarray:
+    packed, scales = _c(packed, np.uint8), _c(scales_f32, np.float32)
+    assert packed.size == K * N // 2 and scales.size == (K // group) * N
+    out = np.empty((K, N), dtype=np.uint16)
+    lib().xqo_nf4_decode_gkn(_p(packed), _p(scales), _p(out), K, N, group)
+    return out
+
+
+def nf4_quantize_flat(x, group):
+    x = _c(x, np.float32)
+    rows, cols = x.shape
+    packed = np.zeros((rows, cols // 2), dtype=np.uint8)
+    scales = np.empty((rows, cols // group), dtype=np.float32)
+    lib().xqo_nf4_quantize_flat(_p(x), _p(packed), _p(scales), rows * cols, group)
+    return packed, scales
+
+
+def nf4_quantize_gkn(x, group):
+    x = _c(x, np.float32)
+    K, N = x.shape
+    packed = np.zeros((K // 2, N), dtype=np.uint8)
+    scales = np.empty((K // group, N), dtype=np.float32)
+    lib().xqo_nf4_quantize_gkn(_p(x), _p(packed), _p(scales), K, N, group)
     return packed, scales
 
 

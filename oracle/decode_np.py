@@ -10,6 +10,8 @@ Reference arithmetic restated (paths relative to the xorl checkout):
   nvfp4  ops/quantize/nvfp4_quantize.py:64-98, nvfp4_gkn_quantize.py:112-169,
          fp4_codec.py:22-30
   fp8    ops/quantize/block_fp8_gkn_quantize.py:131-180
+  nf4    ops/quantize/nf4_quantize.py:62-105, nf4_gkn_quantize.py:84-142,
+         nf4_codec.py:18-35
 """
 
 from __future__ import annotations
@@ -21,6 +23,13 @@ import numpy as np
 # ops/quantize/nvfp4_fake_quant.py:40.
 E2M1_ABS = np.array([0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0], dtype=np.float32)
 E2M1 = np.concatenate([E2M1_ABS, -E2M1_ABS]).astype(np.float32)  # code 8 = -0.0
+
+
+# NormalFloat4 levels as fp32 bit patterns (the fp32 roundings of the sixteen
+# constants at ops/quantize/nf4_codec.py:18-35).
+NF4 = np.array([0xBF800000, 0xBF3239B1, 0xBF066B30, 0xBECA32A0, 0xBE91A24D, 0xBE3D353F, 0xBDBA7871, 0x00000000,
+                0x3DA2FAFF, 0x3E24CAE3, 0x3E7C04DD, 0x3EAD033A, 0x3EE1A4B8, 0x3F1007AB, 0x3F3913B3, 0x3F800000],
+               dtype=np.uint32).view(np.float32)
 
 
 def _e4m3_table() -> np.ndarray:
@@ -79,6 +88,18 @@ def int4_decode_gkn(packed, scales_f32, K, N, group):
     nib = _unpack_gkn(packed, K, N).astype(np.float32)
     s = np.repeat(np.asarray(scales_f32, dtype=np.float32).reshape(K // group, N), group, axis=0)
     return bf16_rne_bits((nib - np.float32(8.0)) * s)
+
+
+def nf4_decode_flat(packed, scales_f32, rows, cols, group):
+    v = NF4[_unpack_flat(packed, rows, cols)]
+    s = np.repeat(np.asarray(scales_f32, dtype=np.float32).reshape(rows, cols // group), group, axis=1)
+    return bf16_rne_bits(v * s)
+
+
+def nf4_decode_gkn(packed, scales_f32, K, N, group):
+    v = NF4[_unpack_gkn(packed, K, N)]
+    s = np.repeat(np.asarray(scales_f32, dtype=np.float32).reshape(K // group, N), group, axis=0)
+    return bf16_rne_bits(v * s)
 
 
 def nvfp4_decode_flat(packed, scales_f32, global_scale, rows, cols, block=16):

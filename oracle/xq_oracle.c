@@ -12,11 +12,13 @@
  * one round-to-nearest-even cast to bfloat16".
  *
  * Pin status (see tests/test_oracle_*.py):
- *   decode  int4 / nvfp4 / block_fp8, flat and GKN ........ pinned
+ *   decode  int4 / nvfp4 / block_fp8 / nf4, flat and GKN .. pinned
  *       (exhaustive code enumeration vs torch.float8_e4m3fn / torch.bfloat16
  *        library casts, the e2m1 table, the reference-held block-fp8
- *        restatement, layout transposition identities, a numpy twin)
- *   quantizers (int4 A2, nvfp4 A4, block_fp8 A6) .......... pinned for IEEE
+ *        restatement, layout transposition identities, a numpy twin; nf4:
+ *        the level table against the normal-quantile construction it is
+ *        published with, decision points = fp32 mean of neighbouring levels)
+ *   quantizers (int4 A2, nvfp4 A4, block_fp8 A6, nf4) ..... pinned for IEEE
  *        arithmetic; byte parity with a GPU-run Triton quantizer is UNPINNED
  *        (Triton's fp32 division / fma contraction / fp8 saturation are not
  *        fixed by the reference text).  Not required: oracle and kernels
@@ -211,6 +213,104 @@ XQO_API void xqo_int4_quantize_sym_flat(const float* x, uint8_t* packed, uint16_
             else packed[i >> 1] = (uint8_t)q;
         }
     }
+}
+
+/* ------------------------------------------------------------------ */
+/* nf4                                                                  */
+/* ------------------------------------------------------------------ */
+
+/* The sixteen NormalFloat4 levels, ops/quantize/nf4_codec.py:18-35 (the
+ * reference holds them as doubles and builds its fp32 LUT from them, :82-87). */
+static const double kNf4Levels[16] = {
+    -1.0, -0.6961928009986877, -0.5250730514526367, -0.39491748809814453,
+    -0.28444138169288635, -0.18477343022823334, -0.09105003625154495, 0.0,
+    0.07958029955625534, 0.16093020141124725, 0.24611230194568634, 0.33791524171829224,
+    0.44070982933044434, 0.5626170039176941, 0.7229568362236023, 1.0};
+
+/* The fifteen decision points of the encoder, nf4_codec.py:48-62. */
+static const double kNf4Cuts[15] = {
+    -0.8480964004993439, -0.6106329262256622, -0.4599952697753906, -0.3396794348955154,
+    -0.2346074059605598, -0.1379117332398891, -0.0455250181257725, 0.0397901497781277,
+    0.1202552504837513, 0.2035212516784668, 0.2920137718319893, 0.3893125355243683,
+    0.5016634166240692, 0.6427869200706482, 0.8614784181118012};
+
+XQO_API float xqo_nf4_level(int code) { return (float)kNf4Levels[code & 15]; }
+
+/* code = how many decision points lie strictly below v (nf4_codec.py:42-64). */
+XQO_API uint8_t xqo_nf4_encode(float v) {
+    int code = 0;
+    for (int i = 0; i < 15; ++i) code += v > (float)kNf4Cuts[i];
+    return (uint8_t)code;
+}
+
+/* flat: _nf4_dequantize_kernel, ops/quantize/nf4_quantize.py:62-105: byte i
+ * holds element 2i (low nibble) and 2i+1 (high) (:89-90), w =
+ * bf16(fl(level[nib] * scale)) with one scale per `group` consecutive elements
+ * (:95-103). */
+XQO_API void xqo_nf4_decode_flat(const uint8_t* packed, const float* scales,
+                                 uint16_t* out, int64_t n_elems, int64_t group) {
+    for (int64_t i = 0; i < n_elems; ++i) {
+        uint8_t b = packed[i >> 1];
+        uint8_t nib = (i & 1) ? (b >> 4) : (b & 0xf);
+        float v = (float)kNf4Levels[nib] * scales[i / group];
+        out[i] = xqo_bf16_rne(v);
+    }
+}
+
+/* GKN [K, N]: packed [K/2, N], nibble pairs and groups along K
+ * (ops/quantize/nf4_gkn_quantize.py:84-142). */
+XQO_API void xqo_nf4_decode_gkn(const uint8_t* packed, const float* scales,
+                                uint16_t* out, int64_t K, int64_t N, int64_t group) {
+    for (int64_t k = 0; k < K; ++k)
+        for (int64_t n = 0; n < N; ++n) {
+            uint8_t b = packed[(k >> 1) * N + n];
+            uint8_t nib = (k & 1) ? (b >> 4) : (b & 0xf);
+            float v = (float)kNf4Levels[nib] * scales[(k / group) * N + n];
+            out[k * N + n] = xqo_bf16_rne(v);
+        }
+}
+
+/* Quantizer, _nf4_quantize_kernel nf4_quantize.py:20-59: scale = max(amax,
+ * 1e-12) (:42-43); code = encode(clamp(x * (1/scale), -1, 1)) (:48-52). */
+XQO_API void xqo_nf4_quantize_flat(const float* x, uint8_t* packed, float* scales,
+                                   int64_t n_elems, int64_t group) {
+    for (int64_t g = 0; g < n_elems / group; ++g) {
+        float amax = 0.0f;
+        for (int64_t j = 0; j < group; ++j) amax = fmaxf(amax, fabsf(x[g * group + j]));
+        float scale = fmaxf(amax, 1e-12f);
+        scales[g] = scale;
+        float inv = 1.0f / scale;
+        for (int64_t j = 0; j < group; ++j) {
+            int64_t i = g * group + j;
+            float t = x[i] * inv;
+            t = fminf(fmaxf(t, -1.0f), 1.0f);
+            int q = xqo_nf4_encode(t);
+            if (i & 1) packed[i >> 1] = (uint8_t)((packed[i >> 1] & 0x0f) | (q << 4));
+            else packed[i >> 1] = (uint8_t)q;
+        }
+    }
+}
+
+/* GKN twin, nf4_gkn_quantize.py:22-81. */
+XQO_API void xqo_nf4_quantize_gkn(const float* x, uint8_t* packed, float* scales,
+                                  int64_t K, int64_t N, int64_t group) {
+    for (int64_t g = 0; g < K / group; ++g)
+        for (int64_t n = 0; n < N; ++n) {
+            float amax = 0.0f;
+            for (int64_t j = 0; j < group; ++j) amax = fmaxf(amax, fabsf(x[(g * group + j) * N + n]));
+            float scale = fmaxf(amax, 1e-12f);
+            scales[g * N + n] = scale;
+            float inv = 1.0f / scale;
+            for (int64_t j = 0; j < group; ++j) {
+                int64_t k = g * group + j;
+                float t = x[k * N + n] * inv;
+                t = fminf(fmaxf(t, -1.0f), 1.0f);
+                int q = xqo_nf4_encode(t);
+                uint8_t* p = &packed[(k >> 1) * N + n];
+                if (k & 1) *p = (uint8_t)((*p & 0x0f) | (q << 4));
+                else *p = (uint8_t)q;
+            }
+        }
 }
 
 /* ------------------------------------------------------------------ */

@@ -56,6 +56,28 @@ def decode_int4(rng):
     return out
 
 
+def decode_nf4(rng):
+    out = {}
+    packed = rng.integers(0, 256, size=(ROWS, COLS // 2), dtype=np.uint8)
+    packed[0, :8] = [0x10, 0x32, 0x54, 0x76, 0x98, 0xBA, 0xDC, 0xFE]      # element i == code i
+    for group in (32, 64):
+        # absmax scales are positive; a wide range of magnitudes and the 1e-12 floor
+        s = np.abs(rng.standard_normal((ROWS, COLS // group))) * np.exp2(rng.integers(-14, 4, size=(ROWS, COLS // group)))
+        s = s.astype(np.float32)
+        s[0, 0], s[1, 0] = 1.0, 1e-12
+        flat = C.nf4_decode_flat(packed, s, ROWS, COLS, group)
+        assert _same(flat, NP.nf4_decode_flat(packed, s, ROWS, COLS, group))
+        out[f"scales_g{group}"] = s
+        out[f"flat_g{group}"] = flat
+    K, N = COLS, ROWS
+    pg = rng.integers(0, 256, size=(K // 2, N), dtype=np.uint8)
+    sg = (np.abs(rng.standard_normal((K // 64, N))) * 0.05).astype(np.float32)
+    gkn = C.nf4_decode_gkn(pg, sg, K, N, 64)
+    assert _same(gkn, NP.nf4_decode_gkn(pg, sg, K, N, 64))
+    out.update(packed=packed, packed_gkn=pg, scales_gkn=sg, gkn=gkn)
+    return out
+
+
 def decode_nvfp4(rng):
     packed = rng.integers(0, 256, size=(ROWS, COLS // 2), dtype=np.uint8)
     # every finite e4m3 byte appears as a block scale (0x7f / 0xff are NaN and excluded)
@@ -126,6 +148,7 @@ def main():
     np.savez_compressed(os.path.join(HERE, "decode_nvfp4.npz"), **decode_nvfp4(rng))
     np.savez_compressed(os.path.join(HERE, "decode_fp8.npz"), **decode_fp8(rng))
     np.savez_compressed(os.path.join(HERE, "fp8_closed_form.npz"), **fp8_closed_form())
+    np.savez_compressed(os.path.join(HERE, "decode_nf4.npz"), **decode_nf4(np.random.default_rng(20240608)))
     for f in sorted(os.listdir(HERE)):
         if f.endswith(".npz"):
             print(f, os.path.getsize(os.path.join(HERE, f)), "bytes")

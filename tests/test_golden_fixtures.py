@@ -53,6 +53,19 @@ def test_oracle_int4_fixture():
         assert np.array_equal(impl.int4_decode_gkn(f["packed_gkn"], f["scales_gkn"], K, N, 128), f["gkn"])
 
 
+def test_oracle_nf4_fixture():
+    f = _load("decode_nf4.npz")
+    R, Cc = f["packed"].shape[0], f["packed"].shape[1] * 2
+    for g in (32, 64):
+        for impl in (C, NP):
+            assert np.array_equal(impl.nf4_decode_flat(f["packed"], f[f"scales_g{g}"], R, Cc, g), f[f"flat_g{g}"])
+    # with scale 1.0 the first sixteen elements are the bf16 roundings of the level table
+    assert np.array_equal(f["flat_g64"][0, :16], NP.bf16_rne_bits(NP.NF4))
+    K, N = f["packed_gkn"].shape[0] * 2, f["packed_gkn"].shape[1]
+    for impl in (C, NP):
+        assert np.array_equal(impl.nf4_decode_gkn(f["packed_gkn"], f["scales_gkn"], K, N, 64), f["gkn"])
+
+
 def test_oracle_nvfp4_fixture():
     f = _load("decode_nvfp4.npz")
     R, Cc = f["packed"].shape[0], f["packed"].shape[1] * 2
@@ -110,6 +123,15 @@ def test_hip_decode_fixtures(hip_device):
         assert np.array_equal(_bits(got), f[f"flat_g{g}"])          # the stored scales are bf16-representable
     K, N = f["packed_gkn"].shape[0] * 2, f["packed_gkn"].shape[1]
     got = Q.int4_dequantize_gkn(torch.from_numpy(f["packed_gkn"]).to(dev), torch.from_numpy(f["scales_gkn"]).to(dev), K, N, 128)
+    assert np.array_equal(_bits(got), f["gkn"])
+
+    f = _load("decode_nf4.npz")
+    R, Cc = f["packed"].shape[0], f["packed"].shape[1] * 2
+    for g in (32, 64):
+        got = Q.nf4_dequantize(torch.from_numpy(f["packed"]).to(dev), torch.from_numpy(f[f"scales_g{g}"]).to(dev), R * Cc, g)
+        assert np.array_equal(_bits(got).reshape(R, Cc), f[f"flat_g{g}"])
+    K, N = f["packed_gkn"].shape[0] * 2, f["packed_gkn"].shape[1]
+    got = Q.nf4_dequantize_gkn(torch.from_numpy(f["packed_gkn"]).to(dev), torch.from_numpy(f["scales_gkn"]).to(dev), K, N, 64)
     assert np.array_equal(_bits(got), f["gkn"])
 
     f = _load("decode_nvfp4.npz")

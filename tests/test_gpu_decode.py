@@ -50,6 +50,48 @@ def test_int4_gkn(hip_device, K, N, group):
     assert np.array_equal(_bits(got), NP.int4_decode_gkn(packed, scales, K, N, group))
 
 
+@pytest.mark.parametrize("rows,cols,group,sdt", [
+    (64, 256, 64, "f32"), (64, 256, 64, "bf16"), (8, 96, 32, "f32"), (5, 30, 6, "f32"), (4096, 4096, 64, "f32"),
+])
+def test_nf4_flat(hip_device, rows, cols, group, sdt):
+    from xorl_amd import quantize as Q
+
+    rng = np.random.default_rng(rows + cols + 1)
+    packed = _codes(rng, (rows, cols // 2))
+    scales = np.abs(rng.normal(0, 0.05, (rows, cols // group))).astype(np.float32)
+    st = torch.from_numpy(scales)
+    if sdt == "bf16":
+        st = st.to(torch.bfloat16)
+        scales = st.float().numpy()
+    got = Q.nf4_dequantize(torch.from_numpy(packed).to(hip_device), st.to(hip_device), rows * cols, group)
+    ref = NP.nf4_decode_flat(packed, scales, rows, cols, group)
+    assert np.array_equal(_bits(got).reshape(rows, cols), ref)
+    if rows * cols <= 1 << 16:
+        assert np.array_equal(ref, C.nf4_decode_flat(packed, scales, rows, cols, group))
+
+
+@pytest.mark.parametrize("K,N,group", [(256, 64, 64), (64, 48, 32), (6, 5, 2), (2048, 768, 64)])
+def test_nf4_gkn(hip_device, K, N, group):
+    from xorl_amd import quantize as Q
+
+    rng = np.random.default_rng(K + N + 1)
+    packed = _codes(rng, (K // 2, N))
+    scales = np.abs(rng.normal(0, 0.05, (K // group, N))).astype(np.float32)
+    got = Q.nf4_dequantize_gkn(torch.from_numpy(packed).to(hip_device), torch.from_numpy(scales).to(hip_device), K, N, group)
+    assert np.array_equal(_bits(got), NP.nf4_decode_gkn(packed, scales, K, N, group))
+
+
+def test_nf4_quantize_on_device_matches_oracle(hip_device):
+    # the package's torch quantizer run on the GPU emits the oracle's bytes
+    from xorl_amd import quantize as Q
+
+    g = torch.Generator().manual_seed(9)
+    w = torch.randn(64, 512, generator=g) * 0.02
+    p, s = Q.nf4_quantize(w.to(hip_device), 64)
+    pc, sc = C.nf4_quantize_flat(w.numpy(), 64)
+    assert np.array_equal(p.cpu().numpy(), pc.reshape(-1)) and np.array_equal(s.cpu().numpy(), sc.reshape(-1))
+
+
 @pytest.mark.parametrize("rows,cols,e4m3", [(64, 256, True), (64, 256, False), (3, 48, True), (8192, 5120, True)])
 def test_nvfp4_flat(hip_device, rows, cols, e4m3):
     from xorl_amd import quantize as Q

@@ -20,7 +20,7 @@ def _run(m, x, dy):
 
 
 @pytest.mark.parametrize("tile_policy", [0, 1, 2], indirect=True)
-@pytest.mark.parametrize("fmt", ["block_fp8", "int4", "nvfp4"])
+@pytest.mark.parametrize("fmt", ["block_fp8", "int4", "nvfp4", "nf4"])
 @pytest.mark.parametrize("M,K,N,r", [(200, 256, 384, 16), (1, 128, 64, 8), (129, 384, 320, 24), (512, 1024, 512, 64), (1100, 512, 768, 32)])
 def test_dense_fwd_bwd_vs_oracle(hip_device, tile_policy, fmt, M, K, N, r):
     m, w_ref = make_dense_module(fmt, N, K, r, 2 * r, seed=M + K, device=hip_device)
@@ -51,7 +51,7 @@ def test_config0_int4_full_size(hip_device, tile_policy):
 
 
 @pytest.mark.parametrize("tile_policy", [1, 2, 3], indirect=True)
-@pytest.mark.parametrize("fmt", ["block_fp8", "int4", "nvfp4"])
+@pytest.mark.parametrize("fmt", ["block_fp8", "int4", "nvfp4", "nf4"])
 def test_gemm_decode_bit_exact(hip_device, tile_policy, fmt):
     """With X = I (and lora_B = 0) every output is a single product 1 * w, so the forward returns the
     decoded weight itself and the dgrad of dY = I returns it transposed: the in-kernel decode of both

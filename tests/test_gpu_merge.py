@@ -34,7 +34,7 @@ def _deq_f32(m, w_ref_bf16):
     return torch.from_numpy(NP.fp8_decode(packed, s, N, K)[0].copy())
 
 
-@pytest.mark.parametrize("fmt", ["block_fp8", "int4", "nvfp4"])
+@pytest.mark.parametrize("fmt", ["block_fp8", "int4", "nvfp4", "nf4"])
 @pytest.mark.parametrize("N,K,r", [(384, 256, 16), (200, 320, 24), (1024, 512, 64), (128, 128, 0)])
 def test_merge_publish_bf16(hip_device, fmt, N, K, r):
     if fmt != "block_fp8" and N % 16:

@@ -55,9 +55,9 @@ def test_route_scatter_gather_exact(hip_device, T, E, topk):
 
 
 def _make_experts(fmt, E, H, I, r, hybrid, seed, device):
-    from xorl_amd.qlora import BlockFP8QLoRAMoeExperts, NvFP4QLoRAMoeExperts
+    from xorl_amd.qlora import BlockFP8QLoRAMoeExperts, NF4QLoRAMoeExperts, NvFP4QLoRAMoeExperts
 
-    cls = BlockFP8QLoRAMoeExperts if fmt == "block_fp8" else NvFP4QLoRAMoeExperts
+    cls = {"block_fp8": BlockFP8QLoRAMoeExperts, "nvfp4": NvFP4QLoRAMoeExperts, "nf4": NF4QLoRAMoeExperts}[fmt]
     m = cls(E, E, I, H, r=r, lora_alpha=2 * r, hybrid_shared=hybrid)
     m.load_weights(gen((E, H, I), 0.05, seed), gen((E, H, I), 0.05, seed + 1), gen((E, I, H), 0.05, seed + 2))
     with torch.no_grad():
@@ -75,6 +75,9 @@ def _make_experts(fmt, E, H, I, r, hybrid, seed, device):
             if fmt == "block_fp8":
                 s = getattr(m, f"{p}_block_scales")[e].contiguous().view(torch.float32).numpy()
                 per.append(bits_to_bf16(NP.fp8_decode(packed[e].reshape(K, N), s, K, N)[1]))
+            elif fmt == "nf4":
+                s = getattr(m, f"{p}_scales")[e].contiguous().view(torch.float32).numpy()
+                per.append(bits_to_bf16(NP.nf4_decode_gkn(packed[e], s, K, N, 64)))
             else:
                 sb = getattr(m, f"{p}_block_scales")[e].numpy()
                 g = getattr(m, f"{p}_global_scale")[e].contiguous().view(torch.float32).item()
@@ -84,7 +87,7 @@ def _make_experts(fmt, E, H, I, r, hybrid, seed, device):
 
 
 @pytest.mark.parametrize("tile_policy", [0, 1, 2], indirect=True)
-@pytest.mark.parametrize("fmt", ["block_fp8", "nvfp4"])
+@pytest.mark.parametrize("fmt", ["block_fp8", "nvfp4", "nf4"])
 @pytest.mark.parametrize("E,T,H,I,r,topk,hybrid", [(6, 300, 128, 192, 8, 2, True), (16, 700, 256, 128, 16, 4, False)])
 def test_moe_fwd_bwd_vs_oracle(hip_device, tile_policy, fmt, E, T, H, I, r, topk, hybrid):
     m, banks = _make_experts(fmt, E, H, I, r, hybrid, seed=E + T, device=hip_device)

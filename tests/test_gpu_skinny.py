@@ -11,7 +11,7 @@ pytestmark = pytest.mark.gpu
 TOL = 1e-2
 
 
-@pytest.mark.parametrize("fmt", ["block_fp8", "int4", "nvfp4"])
+@pytest.mark.parametrize("fmt", ["block_fp8", "int4", "nvfp4", "nf4"])
 @pytest.mark.parametrize("M", [1, 8, 32, 64, 5, 33])
 def test_skinny_forward_vs_oracle(hip_device, fmt, M):
     K, N, r = 1024, 384, 16

@@ -34,7 +34,7 @@ def test_product_never_imports_the_oracle():
 
 
 def test_dense_module_state_matches_reference_contract():
-    from xorl_amd.qlora import BlockFP8QLoRALinear, Int4QLoRALinear, NvFP4QLoRALinear, QLoRALinear
+    from xorl_amd.qlora import BlockFP8QLoRALinear, Int4QLoRALinear, NF4QLoRALinear, NvFP4QLoRALinear, QLoRALinear
 
     with pytest.raises(TypeError):
         QLoRALinear(8, 8)
@@ -54,6 +54,11 @@ def test_dense_module_state_matches_reference_contract():
     assert tuple(n.weight_block_scales.shape) == (32, 16)
     i4 = Int4QLoRALinear(256, 32)
     assert tuple(i4.weight_scales.shape) == (32, 4) and i4._scale_dtypes["weight_scales"] == torch.bfloat16
+    n4 = NF4QLoRALinear(256, 32)
+    assert n4.quant_group_size == 64 and tuple(n4.packed_weight_f32.shape) == (32, 32)
+    assert tuple(n4.weight_scales.shape) == (32, 16) and n4._scale_dtypes["weight_scales"] == torch.float32
+    with pytest.raises(NotImplementedError):
+        n4._load_prequantized(lambda k: None)
     with pytest.raises(ValueError):
         m.set_runtime_lora_config(17, 1)
 
@@ -62,7 +67,7 @@ def test_from_module_roundtrip_and_model_dtype_move():
     from xorl_amd.qlora import QLoRALinear
 
     lin = torch.nn.Linear(256, 128, bias=True)
-    for fmt in ("block_fp8", "nvfp4", "int4"):
+    for fmt in ("block_fp8", "nvfp4", "int4", "nf4"):
         q = QLoRALinear.from_module(lin, r=8, lora_alpha=16, quant_format=fmt)
         assert q.quant_format == fmt and torch.equal(q.bias, lin.bias)
         packed = q.packed_weight_f32.detach().clone()
@@ -75,7 +80,7 @@ def test_from_module_roundtrip_and_model_dtype_move():
         with pytest.raises(RuntimeError, match="expected float32"):
             q._read_packed_weight_uint8()
     with pytest.raises(ValueError):
-        QLoRALinear.from_module(lin, quant_format="nf4")
+        QLoRALinear.from_module(lin, quant_format="mxfp4")
 
 
 def test_from_quantized_and_delta_weight():

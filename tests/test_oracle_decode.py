@@ -148,6 +148,92 @@ def test_int4_sym_quantizer_rule():
     assert np.array_equal(codes, ref.astype(np.int32))
 
 
+def test_nf4_level_table_is_the_normal_quantile_map():
+    # The levels are published as a construction, not only as numbers: eight
+    # standard-normal quantiles on the positive side, seven on the negative,
+    # zero, normalised by the largest (offset 0.9677083, Dettmers et al. 2023).
+    from scipy.stats import norm
+
+    off = 0.9677083
+    pos = norm.ppf(np.linspace(off, 0.5, 9)[:-1])
+    neg = -norm.ppf(np.linspace(off, 0.5, 8)[:-1])
+    want = np.sort(np.concatenate([pos, [0.0], neg]))
+    want /= want.max()
+    t = C.nf4_table()
+    assert t.dtype == np.float32 and np.array_equal(t.view(np.uint32), NP.NF4.view(np.uint32))
+    assert np.max(np.abs(t - want)) < 5e-7
+    assert np.all(np.diff(t) > 0) and t[0] == -1.0 and t[7] == 0.0 and t[15] == 1.0
+    # asymmetric by construction: 7 negative and 8 positive non-zero levels
+    assert (t < 0).sum() == 7 and (t > 0).sum() == 8
+
+
+def test_nf4_encoder_is_nearest_level():
+    # Decision points are the means of neighbouring levels, so the encoder is
+    # nearest-level; check against a brute-force argmin away from the cuts and
+    # the strict ">" at them (nf4_codec.py:42-64).
+    t = C.nf4_table().astype(np.float64)
+    v = np.linspace(-1, 1, 4001).astype(np.float32)
+    got = C.nf4_encode(v)
+    d = np.abs(v.astype(np.float64)[:, None] - t[None, :])
+    near = d.argmin(1)
+    srt = np.sort(d, 1)
+    clear = (srt[:, 1] - srt[:, 0]) > 1e-6
+    assert np.array_equal(got[clear], near[clear].astype(np.uint8))
+    cuts = ((t[1:] + t[:-1]) / 2).astype(np.float32)
+    assert np.array_equal(C.nf4_encode(cuts), np.arange(15, dtype=np.uint8))               # not above the cut
+    assert np.array_equal(C.nf4_encode(np.nextafter(cuts, np.float32(2))), np.arange(1, 16, dtype=np.uint8))
+    assert np.array_equal(C.nf4_encode(t.astype(np.float32)), np.arange(16, dtype=np.uint8))
+
+
+def test_nf4_decode_flat_and_gkn():
+    rng = np.random.default_rng(11)
+    rows, cols, group = 16, 256, 64
+    packed = rng.integers(0, 256, (rows, cols // 2), dtype=np.uint8)
+    packed[0, :8] = [0x10, 0x32, 0x54, 0x76, 0x98, 0xBA, 0xDC, 0xFE]   # element i == code i
+    scales = np.abs(rng.normal(0, 0.05, (rows, cols // group))).astype(np.float32)
+    scales[0, 0] = 1.0
+    got_c = C.nf4_decode_flat(packed, scales, rows, cols, group)
+    assert np.array_equal(got_c, NP.nf4_decode_flat(packed, scales, rows, cols, group))
+    # torch restatement: LUT gather, low nibble = even element (nf4_quantize.py:89-103)
+    p = torch.from_numpy(packed).long()
+    nib = torch.stack([p & 0xF, p >> 4], dim=-1).reshape(rows, cols)
+    w = (torch.from_numpy(C.nf4_table())[nib] * torch.from_numpy(scales).repeat_interleave(group, dim=1)).to(torch.bfloat16)
+    assert np.array_equal(got_c, _bf16_bits(w))
+    assert np.array_equal(got_c[0, :16], _bf16_bits(torch.from_numpy(C.nf4_table())))
+    # GKN of the transposed codes decodes to the transpose
+    codes = nib.numpy().astype(np.uint8)
+    ct = codes.T.copy()
+    gkn_packed = (ct[0::2] | (ct[1::2] << 4)).astype(np.uint8)
+    b = C.nf4_decode_gkn(gkn_packed, scales.T.copy(), cols, rows, group)
+    assert np.array_equal(got_c.T, b)
+    assert np.array_equal(NP.nf4_decode_gkn(gkn_packed, scales.T.copy(), cols, rows, group), b)
+
+
+def test_nf4_quantizer_rule_and_roundtrip():
+    # scale = absmax (so +-absmax land exactly on codes 15 / 0), zeros on code 7,
+    # an all-zero group keeps the 1e-12 floor; round-trip error under the
+    # 0.10 the reference's own round-trip test allows.
+    rng = np.random.default_rng(12)
+    x = rng.normal(0, 0.02, (8, 256)).astype(np.float32)
+    x[0, :64] = 0.0
+    x[1, 0], x[1, 1], x[1, 2] = 0.5, -0.5, 0.0
+    packed, scales = C.nf4_quantize_flat(x, 64)
+    assert np.array_equal(scales, np.maximum(np.abs(x.reshape(8, 4, 64)).max(-1), np.float32(1e-12)))
+    codes = np.stack([packed & 0xF, packed >> 4], -1).reshape(8, 256)
+    assert set(codes[0, :64]) == {7} and scales[0, 0] == np.float32(1e-12)
+    assert list(codes[1, :3]) == [15, 0, 7] and scales[1, 0] == np.float32(0.5)
+    w = NP.bf16_bits_to_f32(C.nf4_decode_flat(packed, scales, 8, 256, 64))
+    assert np.abs(w - x)[2:].mean() / np.abs(x)[2:].mean() < 0.10  # the metric of tests/qlora/test_qlora.py:151-152
+    # every element sits on the level nearest to x/scale
+    norm = x / np.repeat(scales, 64, 1)
+    t = C.nf4_table()
+    assert np.all(np.abs(t[codes] - norm) <= np.abs(t[None, None, :] - norm[..., None]).min(-1) + 1e-6)
+    # GKN twin: transposed input -> transposed codes, same scales
+    pk, sk = C.nf4_quantize_gkn(x.T.copy(), 64)
+    ck = np.stack([pk & 0xF, pk >> 4], 1).reshape(256, 8)
+    assert np.array_equal(ck, codes.T) and np.array_equal(sk, scales.T)
+
+
 def test_nvfp4_decode_flat_and_gkn():
     rng = np.random.default_rng(5)
     N, K = 16, 128

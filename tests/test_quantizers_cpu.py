@@ -26,6 +26,19 @@ def test_int4_quantizers_match_oracle():
     assert np.array_equal(ss.view(torch.int16).numpy().view(np.uint16), ssc)
 
 
+def test_nf4_quantizers_match_oracle():
+    w = _w((32, 256), 5)
+    w[3, :64] = 0.0
+    p, s = Q.nf4_quantize(w, 64)
+    pc, sc = C.nf4_quantize_flat(w.numpy(), 64)
+    assert np.array_equal(p.numpy(), pc.reshape(-1)) and np.array_equal(s.numpy(), sc.reshape(-1))
+    pk, sk = Q.nf4_quantize_gkn(w.t().contiguous(), 64)
+    pkc, skc = C.nf4_quantize_gkn(w.t().contiguous().numpy(), 64)
+    assert np.array_equal(pk.numpy(), pkc) and np.array_equal(sk.numpy(), skc)
+    assert np.array_equal(np.array(Q.NF4_TABLE, dtype=np.float32), C.nf4_table())
+    assert Q.NF4_MIN_STEP == min(b - a for a, b in zip(Q.NF4_TABLE, Q.NF4_TABLE[1:]))
+
+
 def test_nvfp4_quantizers_match_oracle():
     w = _w((32, 256), 1)
     p, bs, g = Q.nvfp4_quantize(w)

@@ -57,4 +57,7 @@ def oracle_decode_dense(m) -> torch.Tensor:
         sdt = m._scale_dtypes["weight_scales"]
         s = m.weight_scales.cpu().contiguous().view(sdt).float().numpy()
         return bits_to_bf16(NP.int4_decode_flat(packed, s, N, K, m.quant_group_size))
+    if m.quant_format == "nf4":
+        s = m.weight_scales.cpu().contiguous().view(torch.float32).numpy()
+        return bits_to_bf16(NP.nf4_decode_flat(packed, s, N, K, m.quant_group_size))
     raise ValueError(m.quant_format)

@@ -16,12 +16,12 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libxq_hip.so")
 
-XQ_FMT_INT4, XQ_FMT_NVFP4, XQ_FMT_FP8 = 0, 1, 2
+XQ_FMT_INT4, XQ_FMT_NVFP4, XQ_FMT_FP8, XQ_FMT_NF4 = 0, 1, 2, 3
 XQ_LAYOUT_FLAT, XQ_LAYOUT_GKN = 0, 1
 XQ_SCALE_F32, XQ_SCALE_BF16, XQ_SCALE_E4M3 = 0, 1, 2
 XQ_DT_BF16, XQ_DT_F32 = 0, 1
 
-FORMATS = {"int4": XQ_FMT_INT4, "nvfp4": XQ_FMT_NVFP4, "block_fp8": XQ_FMT_FP8}
+FORMATS = {"int4": XQ_FMT_INT4, "nvfp4": XQ_FMT_NVFP4, "block_fp8": XQ_FMT_FP8, "nf4": XQ_FMT_NF4}
 
 
 class XqWeight(ctypes.Structure):

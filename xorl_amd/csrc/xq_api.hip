@@ -30,7 +30,7 @@ int64_t xq_scale_bytes_per_expert(const xq_weight* w) {
 
 int xq_validate_weight(const xq_weight* w, const char* who) {
     XQ_REQUIRE(w != nullptr, "%s: weight descriptor is NULL", who);
-    XQ_REQUIRE(w->format >= XQ_FMT_INT4 && w->format <= XQ_FMT_FP8, "%s: unknown format %d", who, w->format);
+    XQ_REQUIRE(w->format >= XQ_FMT_INT4 && w->format <= XQ_FMT_NF4, "%s: unknown format %d", who, w->format);
     XQ_REQUIRE(w->layout == XQ_LAYOUT_FLAT || w->layout == XQ_LAYOUT_GKN, "%s: unknown layout %d", who, w->layout);
     XQ_REQUIRE(w->rows >= 0 && w->cols >= 0 && w->num_experts >= 1, "%s: bad shape [%d x %lld x %lld]", who,
                w->num_experts, (long long)w->rows, (long long)w->cols);
@@ -53,7 +53,7 @@ int xq_validate_weight(const xq_weight* w, const char* who) {
             XQ_REQUIRE(w->global_scale != nullptr, "%s: nvfp4 needs global_scale", who);
             XQ_REQUIRE(w->scale_dtype != XQ_SCALE_BF16, "%s: nvfp4 block scales are e4m3 or fp32", who);
         } else {
-            XQ_REQUIRE(w->scale_dtype != XQ_SCALE_E4M3, "%s: int4 scales are fp32 or bf16", who);
+            XQ_REQUIRE(w->scale_dtype != XQ_SCALE_E4M3, "%s: int4 / nf4 scales are fp32 or bf16", who);
         }
         XQ_REQUIRE(empty || xq_aligned(w->scales, scale_elem_bytes(w->scale_dtype)), "%s: scales misaligned", who);
     }

@@ -91,6 +91,23 @@ __device__ __forceinline__ float int4_val(uint32_t nib, float s, float m8s) {
     return ((float)nib - 8.0f) * s;
 }
 
+// NF4 (NormalFloat4) levels, ops/quantize/nf4_codec.py:18-35: w = bf16(fl(level[nib] * scale)).
+// A per-lane index into this 64-byte table is a vector load that stays in L1.
+static __device__ __constant__ float kNf4Level[16] = {
+    -1.0f, -0.6961928009986877f, -0.5250730514526367f, -0.39491748809814453f,
+    -0.28444138169288635f, -0.18477343022823334f, -0.09105003625154495f, 0.0f,
+    0.07958029955625534f, 0.16093020141124725f, 0.24611230194568634f, 0.33791524171829224f,
+    0.44070982933044434f, 0.5626170039176941f, 0.7229568362236023f, 1.0f};
+
+// decoded fp32 value of one 4-bit code, before the bf16 rounding; for nvfp4 `s` is already
+// fl(block_scale * global_scale)
+template <int FMT>
+__device__ __forceinline__ float val4(uint32_t nib, float s) {
+    if (FMT == XQ_FMT_INT4) return int4_val(nib, s, 0.0f);
+    if (FMT == XQ_FMT_NVFP4) return e2m1_to_f32(nib) * s;
+    return kNf4Level[nib & 0xfu] * s;
+}
+
 // ---------------------------------------------------------------- transposing LDS fragment read
 // MFMA 32x32x16 operand fragment from a row-major [k][col] bf16 LDS tile:
 __device__ __forceinline__ bf16x8 lds_tr_frag(const bf16_t* tile, int pitch, int krow0, int col0, int lane) {

@@ -1,8 +1,9 @@
-// Stand-alone weight decode: packed int4 / nvfp4 / block-fp8 -> bf16 (or fp32).
+// Stand-alone weight decode: packed int4 / nvfp4 / nf4 / block-fp8 -> bf16 (or fp32).
 // HBM-bound: every thread moves 16 B of packed codes and writes the decoded
 // run with 16 B stores.  Bit-exact with the reference decoders:
 //   int4   (nib-8)*scale                    ops/quantize/int4_quantize.py:45-76, int4_gkn_quantize.py:79-130
 //   nvfp4  e2m1(nib)*(block_scale*global)   ops/quantize/nvfp4_quantize.py:64-98, nvfp4_gkn_quantize.py:112-169
+//   nf4    level[nib]*scale                 ops/quantize/nf4_quantize.py:61-105, nf4_gkn_quantize.py:84-138
 //   fp8    float(e4m3)*s[i/128][j/128]      ops/quantize/block_fp8_gkn_quantize.py:131-154
 #include "xq_common.h"
 
@@ -87,15 +88,9 @@ __global__ void __launch_bounds__(256) decode_4bit_flat_vec(DecodeArgs a, int64_
     int64_t gidx = (row * a.cols + c0) / a.group;
     float s = load_scale(a.scales + e * a.scale_stride, gidx, a.scale_dtype);
     float v[16];
-    if (FMT == XQ_FMT_INT4) {
-        float m8s = -8.0f * s;
+    if (FMT == XQ_FMT_NVFP4) s = s * a.global_scale[e];
 #pragma unroll
-        for (int i = 0; i < 16; ++i) v[i] = int4_val((w[i >> 3] >> (4 * (i & 7))) & 0xfu, s, m8s);
-    } else {
-        s = s * a.global_scale[e];
-#pragma unroll
-        for (int i = 0; i < 16; ++i) v[i] = e2m1_to_f32((w[i >> 3] >> (4 * (i & 7))) & 0xfu) * s;
-    }
+    for (int i = 0; i < 16; ++i) v[i] = val4<FMT>((w[i >> 3] >> (4 * (i & 7))) & 0xfu, s);
     store_run16<false>(a.out, (e * a.rows + row) * a.cols + c0, v);
 }
 
@@ -108,16 +103,8 @@ __global__ void __launch_bounds__(256) decode_4bit_flat_scalar(DecodeArgs a, int
     int64_t e = t / per_expert, rem = t - e * per_expert;
     uint32_t b = a.packed[e * a.packed_stride + rem];
     float s = load_scale(a.scales + e * a.scale_stride, (rem * 2) / a.group, a.scale_dtype);
-    float lo, hi;
-    if (FMT == XQ_FMT_INT4) {
-        float m8s = -8.0f * s;
-        lo = int4_val(b & 0xfu, s, m8s);
-        hi = int4_val(b >> 4, s, m8s);
-    } else {
-        s = s * a.global_scale[e];
-        lo = e2m1_to_f32(b & 0xfu) * s;
-        hi = e2m1_to_f32(b >> 4) * s;
-    }
+    if (FMT == XQ_FMT_NVFP4) s = s * a.global_scale[e];
+    const float lo = val4<FMT>(b & 0xfu, s), hi = val4<FMT>(b >> 4, s);
     ((uint32_t*)a.out)[t] = pack_bf16x2(lo, hi);
 }
 
@@ -139,15 +126,9 @@ __global__ void __launch_bounds__(256) decode_4bit_gkn_vec(DecodeArgs a, int64_t
     for (int i = 0; i < 16; ++i) {
         uint32_t b = (w[i >> 2] >> (8 * (i & 3))) & 0xffu;
         float s = load_scale(sp, g * a.cols + c0 + i, a.scale_dtype);
-        if (FMT == XQ_FMT_INT4) {
-            float m8s = -8.0f * s;
-            ve[i] = int4_val(b & 0xfu, s, m8s);
-            vo[i] = int4_val(b >> 4, s, m8s);
-        } else {
-            s = s * gs;
-            ve[i] = e2m1_to_f32(b & 0xfu) * s;
-            vo[i] = e2m1_to_f32(b >> 4) * s;
-        }
+        if (FMT == XQ_FMT_NVFP4) s = s * gs;
+        ve[i] = val4<FMT>(b & 0xfu, s);
+        vo[i] = val4<FMT>(b >> 4, s);
     }
     int64_t base = (e * a.rows + 2 * r2) * a.cols + c0;
     store_run16<false>(a.out, base, ve);
@@ -163,16 +144,8 @@ __global__ void __launch_bounds__(256) decode_4bit_gkn_scalar(DecodeArgs a, int6
     int64_t r2 = rem / a.cols, c = rem - r2 * a.cols;
     uint32_t b = a.packed[e * a.packed_stride + rem];
     float s = load_scale(a.scales + e * a.scale_stride, ((2 * r2) / a.group) * a.cols + c, a.scale_dtype);
-    float lo, hi;
-    if (FMT == XQ_FMT_INT4) {
-        float m8s = -8.0f * s;
-        lo = int4_val(b & 0xfu, s, m8s);
-        hi = int4_val(b >> 4, s, m8s);
-    } else {
-        s = s * a.global_scale[e];
-        lo = e2m1_to_f32(b & 0xfu) * s;
-        hi = e2m1_to_f32(b >> 4) * s;
-    }
+    if (FMT == XQ_FMT_NVFP4) s = s * a.global_scale[e];
+    const float lo = val4<FMT>(b & 0xfu, s), hi = val4<FMT>(b >> 4, s);
     bf16_t* o = (bf16_t*)a.out + (e * a.rows + 2 * r2) * a.cols + c;
     o[0] = to_bf16(lo);
     o[a.cols] = to_bf16(hi);
@@ -222,23 +195,27 @@ extern "C" int xq_decode(const xq_weight* w, void* out, int out_dtype, void* str
         if (vec) {
             int64_t cpr = w->cols / 16, total = E * w->rows * cpr;
             if (w->format == XQ_FMT_INT4) decode_4bit_flat_vec<XQ_FMT_INT4><<<grid_for(total), 256, 0, stream>>>(a, cpr, total);
-            else decode_4bit_flat_vec<XQ_FMT_NVFP4><<<grid_for(total), 256, 0, stream>>>(a, cpr, total);
+            else if (w->format == XQ_FMT_NVFP4) decode_4bit_flat_vec<XQ_FMT_NVFP4><<<grid_for(total), 256, 0, stream>>>(a, cpr, total);
+            else decode_4bit_flat_vec<XQ_FMT_NF4><<<grid_for(total), 256, 0, stream>>>(a, cpr, total);
         } else {
             int64_t total = elems / 2;
             XQ_REQUIRE(xq_aligned(out, 4), "xq_decode: out must be 4-byte aligned");
             if (w->format == XQ_FMT_INT4) decode_4bit_flat_scalar<XQ_FMT_INT4><<<grid_for(total), 256, 0, stream>>>(a, total);
-            else decode_4bit_flat_scalar<XQ_FMT_NVFP4><<<grid_for(total), 256, 0, stream>>>(a, total);
+            else if (w->format == XQ_FMT_NVFP4) decode_4bit_flat_scalar<XQ_FMT_NVFP4><<<grid_for(total), 256, 0, stream>>>(a, total);
+            else decode_4bit_flat_scalar<XQ_FMT_NF4><<<grid_for(total), 256, 0, stream>>>(a, total);
         }
     } else {
         bool vec = (w->cols % 16 == 0) && xq_aligned(w->packed, 16) && xq_aligned(out, 16) && (a.packed_stride % 16 == 0);
         if (vec) {
             int64_t cpr = w->cols / 16, total = E * (w->rows / 2) * cpr;
             if (w->format == XQ_FMT_INT4) decode_4bit_gkn_vec<XQ_FMT_INT4><<<grid_for(total), 256, 0, stream>>>(a, cpr, total);
-            else decode_4bit_gkn_vec<XQ_FMT_NVFP4><<<grid_for(total), 256, 0, stream>>>(a, cpr, total);
+            else if (w->format == XQ_FMT_NVFP4) decode_4bit_gkn_vec<XQ_FMT_NVFP4><<<grid_for(total), 256, 0, stream>>>(a, cpr, total);
+            else decode_4bit_gkn_vec<XQ_FMT_NF4><<<grid_for(total), 256, 0, stream>>>(a, cpr, total);
         } else {
             int64_t total = elems / 2;
             if (w->format == XQ_FMT_INT4) decode_4bit_gkn_scalar<XQ_FMT_INT4><<<grid_for(total), 256, 0, stream>>>(a, total);
-            else decode_4bit_gkn_scalar<XQ_FMT_NVFP4><<<grid_for(total), 256, 0, stream>>>(a, total);
+            else if (w->format == XQ_FMT_NVFP4) decode_4bit_gkn_scalar<XQ_FMT_NVFP4><<<grid_for(total), 256, 0, stream>>>(a, total);
+            else decode_4bit_gkn_scalar<XQ_FMT_NF4><<<grid_for(total), 256, 0, stream>>>(a, total);
         }
     }
     XQ_CHECK_LAUNCH("xq_decode");

@@ -109,6 +109,7 @@ int launch_tile_gemm(const xq_weight* w, bool contract_cols, const bf16_t* A, in
             int rc;
             if (w->format == XQ_FMT_FP8) rc = launch_256<XQ_FMT_FP8>(f, contract_cols, grouped, T, grid, stream, who);
             else if (w->format == XQ_FMT_INT4) rc = launch_256<XQ_FMT_INT4>(f, contract_cols, grouped, T, grid, stream, who);
+            else if (w->format == XQ_FMT_NF4) rc = launch_256<XQ_FMT_NF4>(f, contract_cols, grouped, T, grid, stream, who);
             else rc = launch_256<XQ_FMT_NVFP4>(f, contract_cols, grouped, T, grid, stream, who);
             if (timed) xq_profile_mark_end(stream);
             if (rc) return rc;
@@ -122,6 +123,8 @@ int launch_tile_gemm(const xq_weight* w, bool contract_cols, const bf16_t* A, in
     if (w->format == XQ_FMT_FP8) launch_tile_cc<XQ_FMT_FP8, XQ_LAYOUT_FLAT>(g, contract_cols, grid, stream);
     else if (w->format == XQ_FMT_INT4 && w->layout == XQ_LAYOUT_FLAT) launch_tile_cc<XQ_FMT_INT4, XQ_LAYOUT_FLAT>(g, contract_cols, grid, stream);
     else if (w->format == XQ_FMT_INT4) launch_tile_cc<XQ_FMT_INT4, XQ_LAYOUT_GKN>(g, contract_cols, grid, stream);
+    else if (w->format == XQ_FMT_NF4 && w->layout == XQ_LAYOUT_FLAT) launch_tile_cc<XQ_FMT_NF4, XQ_LAYOUT_FLAT>(g, contract_cols, grid, stream);
+    else if (w->format == XQ_FMT_NF4) launch_tile_cc<XQ_FMT_NF4, XQ_LAYOUT_GKN>(g, contract_cols, grid, stream);
     else if (w->layout == XQ_LAYOUT_FLAT) launch_tile_cc<XQ_FMT_NVFP4, XQ_LAYOUT_FLAT>(g, contract_cols, grid, stream);
     else launch_tile_cc<XQ_FMT_NVFP4, XQ_LAYOUT_GKN>(g, contract_cols, grid, stream);
     if (timed) xq_profile_mark_end(stream);

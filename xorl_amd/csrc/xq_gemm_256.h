@@ -7,7 +7,7 @@
 //   C[rows, Nout] = A[rows, Kc] . Wop (+ su[rows, r] . Lr[Nout, r]^T) (+ bias)
 //
 // W is a quantized [wrows, wcols] matrix: block-fp8 (e4m3 bytes, fp32 scale per
-// 128x128 block) or a 4-bit FLAT matrix (int4 / nvfp4: two codes per byte along
+// 128x128 block) or a 4-bit FLAT matrix (int4 / nvfp4 / nf4: two codes per byte along
 // the columns, one scale per `group` consecutive columns).
 //   CONTRACT_COLS (dense forward, expert-bank dgrad):  Wop[kc][n] = W[n][kc]; the
 //     decoded tile is stored in LDS as [n][kc] (kc contiguous, XOR-swizzled 16-byte
@@ -157,6 +157,7 @@ __device__ __forceinline__ float scale_from_raw(uint32_t raw, int dtype) {
 //   int4:  value = nib - 8.  fma(nib, s, -8s) is the same real number as (nib - 8) * s
 //          (-8s is exact), so it rounds identically; only the sign of an exact zero can
 //          differ from the two-step form, which no sum can see.
+//   nf4:   level[nib] * s, the level read from a 64-byte constant table (one L1-resident line).
 //   nvfp4: v_cvt_scalef32_pk_f32_fp4 with scale 1.0 returns the exact e2m1 values of the two
 //          codes of a byte (low nibble first); each is multiplied by s in fp32 and rounded
 //          once, like the reference's fl(e2m1 * s).
@@ -171,6 +172,9 @@ __device__ __forceinline__ void decode8_4bit(uint32_t w, float s, uint32_t* out4
             v[2 * i] = __builtin_fmaf((float)((even >> (8 * i)) & 0xffu), s, m8s);
             v[2 * i + 1] = __builtin_fmaf((float)((odd >> (8 * i)) & 0xffu), s, m8s);
         }
+    } else if (FMT == XQ_FMT_NF4) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = kNf4Level[(w >> (4 * i)) & 0xfu] * s;
     } else {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {

@@ -48,15 +48,9 @@ struct TileArgs {
 
 template <int FMT>
 __device__ __forceinline__ void decode16_4bit(const u32x2 w, float s, float gs, float* v) {
-    if (FMT == XQ_FMT_INT4) {
-        float m8s = -8.0f * s;
+    if (FMT == XQ_FMT_NVFP4) s = s * gs;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) v[i] = int4_val((w[i >> 3] >> (4 * (i & 7))) & 0xfu, s, m8s);
-    } else {
-        s = s * gs;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) v[i] = e2m1_to_f32((w[i >> 3] >> (4 * (i & 7))) & 0xfu) * s;
-    }
+    for (int i = 0; i < 16; ++i) v[i] = val4<FMT>((w[i >> 3] >> (4 * (i & 7))) & 0xfu, s);
 }
 
 __device__ __forceinline__ void lds_store_run16(bf16_t* dst, const float* v) {
@@ -163,15 +157,9 @@ struct Loader4Gkn {
         for (int i = 0; i < 16; ++i) {
             uint32_t b = (raw[i >> 2] >> (8 * (i & 3))) & 0xffu;
             float sc = s[i];
-            if (FMT == XQ_FMT_INT4) {
-                float m8s = -8.0f * sc;
-                ve[i] = int4_val(b & 0xfu, sc, m8s);
-                vo[i] = int4_val(b >> 4, sc, m8s);
-            } else {
-                sc = sc * gs;
-                ve[i] = e2m1_to_f32(b & 0xfu) * sc;
-                vo[i] = e2m1_to_f32(b >> 4) * sc;
-            }
+            if (FMT == XQ_FMT_NVFP4) sc = sc * gs;
+            ve[i] = val4<FMT>(b & 0xfu, sc);
+            vo[i] = val4<FMT>(b >> 4, sc);
         }
         if (CONTRACT_COLS) {
             int n = 2 * (tid >> 2), kc = (tid & 3) * 16;
@@ -191,6 +179,8 @@ template <bool CC> struct LoaderSel<XQ_FMT_INT4, XQ_LAYOUT_FLAT, CC> { using typ
 template <bool CC> struct LoaderSel<XQ_FMT_NVFP4, XQ_LAYOUT_FLAT, CC> { using type = Loader4Flat<XQ_FMT_NVFP4, CC>; };
 template <bool CC> struct LoaderSel<XQ_FMT_INT4, XQ_LAYOUT_GKN, CC> { using type = Loader4Gkn<XQ_FMT_INT4, CC>; };
 template <bool CC> struct LoaderSel<XQ_FMT_NVFP4, XQ_LAYOUT_GKN, CC> { using type = Loader4Gkn<XQ_FMT_NVFP4, CC>; };
+template <bool CC> struct LoaderSel<XQ_FMT_NF4, XQ_LAYOUT_FLAT, CC> { using type = Loader4Flat<XQ_FMT_NF4, CC>; };
+template <bool CC> struct LoaderSel<XQ_FMT_NF4, XQ_LAYOUT_GKN, CC> { using type = Loader4Gkn<XQ_FMT_NF4, CC>; };
 
 // ------------------------------------------------------------------ the kernel
 template <int FMT, int LAYOUT, bool CONTRACT_COLS>

@@ -64,7 +64,7 @@ __device__ __forceinline__ void decode_run16(const MergeArgs& g, int64_t n, int 
             const uint32_t nib = (w[i >> 3] >> (4 * (i & 7))) & 0xfu;
             // one scale per `group` elements; group is even, so a pair never straddles two groups
             const float s = load_scale(g.scales, (n * g.K + k + i) / g.group, g.scale_dtype);
-            v[i] = FMT == XQ_FMT_INT4 ? int4_val(nib, s, 0.0f) : e2m1_to_f32(nib) * (s * gs);
+            v[i] = val4<FMT>(nib, FMT == XQ_FMT_NVFP4 ? s * gs : s);
         }
     }
 }
@@ -288,6 +288,7 @@ static int launch_merge(const xq_weight* w, const void* A, const void* B, int lo
     const bool timed = xq_profile_mark_begin(stream, merge_bytes(w, mode));
     if (w->format == XQ_FMT_FP8) rc = launch_merge_fmt<XQ_FMT_FP8>(g, grid, lds, stream, who);
     else if (w->format == XQ_FMT_INT4) rc = launch_merge_fmt<XQ_FMT_INT4>(g, grid, lds, stream, who);
+    else if (w->format == XQ_FMT_NF4) rc = launch_merge_fmt<XQ_FMT_NF4>(g, grid, lds, stream, who);
     else rc = launch_merge_fmt<XQ_FMT_NVFP4>(g, grid, lds, stream, who);
     if (timed) xq_profile_mark_end(stream);
     if (rc) return rc;

@@ -347,6 +347,7 @@ int64_t skinny_workspace_bytes(int64_t M, int64_t N, int64_t K, int r_pad) {
 
 bool skinny_supported(const xq_weight* w, int64_t M) {
     if (M < 1 || M > 64 || w->num_experts != 1) return false;
+    if (w->format == XQ_FMT_NF4) return false;   // nf4 takes the tile kernels
     if (w->format != XQ_FMT_FP8 && w->layout != XQ_LAYOUT_FLAT) return false;
     if (w->cols % 128 != 0 || w->cols < 1024 || w->rows % 16 != 0) return false;
     if (w->format == XQ_FMT_INT4 && (w->group % 8 != 0)) return false;

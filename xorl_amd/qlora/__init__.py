@@ -4,6 +4,7 @@ from .linear import (
     BlockFP8QLoRALinear,
     Int4QLoRALinear,
     LoraModule,
+    NF4QLoRALinear,
     NvFP4QLoRALinear,
     QLoRALinear,
     deregister_qlora_weights_from_fsdp,
@@ -15,9 +16,10 @@ __all__ = [
     "BlockFP8QLoRALinear",
     "NvFP4QLoRALinear",
     "Int4QLoRALinear",
+    "NF4QLoRALinear",
     "deregister_qlora_weights_from_fsdp",
 ]
 
-from .moe_experts import BlockFP8QLoRAMoeExperts, NvFP4QLoRAMoeExperts, QLoRAMoeExperts  # noqa: E402
+from .moe_experts import BlockFP8QLoRAMoeExperts, NF4QLoRAMoeExperts, NvFP4QLoRAMoeExperts, QLoRAMoeExperts  # noqa: E402
 
-__all__ += ["QLoRAMoeExperts", "BlockFP8QLoRAMoeExperts", "NvFP4QLoRAMoeExperts"]
+__all__ += ["QLoRAMoeExperts", "BlockFP8QLoRAMoeExperts", "NvFP4QLoRAMoeExperts", "NF4QLoRAMoeExperts"]

@@ -146,7 +146,8 @@ class QLoRALinear(LoraModule, nn.Module):
     # ------------------------------------------------------------------ factories
     @classmethod
     def _class_for(cls, quant_format: str):
-        table = {"block_fp8": BlockFP8QLoRALinear, "nvfp4": NvFP4QLoRALinear, "int4": Int4QLoRALinear}
+        table = {"block_fp8": BlockFP8QLoRALinear, "nvfp4": NvFP4QLoRALinear, "int4": Int4QLoRALinear,
+                 "nf4": NF4QLoRALinear}
         if quant_format not in table:
             raise ValueError(f"unsupported quant_format {quant_format!r}; expected one of {sorted(table)}")
         return table[quant_format]
@@ -604,6 +605,72 @@ class Int4QLoRALinear(QLoRALinear):
     def _compute_aqn_step(self) -> Tensor:
         s = self._recover_tensor(self.weight_scales, self._scale_dtypes["weight_scales"]).float()
         return (0.5 * s.repeat_interleave(self.quant_group_size, 1)).contiguous()
+
+
+# =============================================================================
+class NF4QLoRALinear(QLoRALinear):
+    """NormalFloat4: w = level[nib] * absmax, one fp32 absmax per 64 consecutive
+    elements of the row-major weight (qlora/modules/nf4_linear.py:15-136).  State:
+    `packed_weight_f32 [N, K/8]`, `weight_scales` u8 view of fp32 `[N, K/64]`."""
+
+    def __init__(self, in_features: int, out_features: int, r: int = 16, lora_alpha: int = 16, bias: bool = False,
+                 device: Optional[torch.device] = None, enable_aqn: bool = False, aqn_alpha: float = 1.0):
+        super().__init__(in_features, out_features, r=r, lora_alpha=lora_alpha, quant_format="nf4",
+                         quant_group_size=64, bias=bias, device=device, enable_aqn=enable_aqn, aqn_alpha=aqn_alpha)
+        if in_features % self.quant_group_size:
+            raise ValueError(f"nf4 needs in_features divisible by the group size {self.quant_group_size}")
+        self.packed_weight_f32 = nn.Parameter(
+            torch.empty(out_features, in_features // 8, dtype=torch.float32, device=device), requires_grad=False)
+        self.register_buffer("weight_scales", torch.empty(out_features, (in_features // self.quant_group_size) * 4,
+                                                          dtype=torch.uint8, device=device))
+        self._scale_dtypes = {"weight_scales": torch.float32}
+        self.reset_lora_parameters()
+
+    @classmethod
+    def from_module(cls, module: nn.Module, r: int = 16, lora_alpha: int = 16, enable_aqn: bool = False,
+                    aqn_alpha: float = 1.0, **kwargs) -> "NF4QLoRALinear":
+        """Quantize a bf16 nn.Linear; on the meta device keep `weight` for a later
+        `quantize_weight()` (nf4_linear.py:64-96)."""
+        q = cls(in_features=module.in_features, out_features=module.out_features, r=r, lora_alpha=lora_alpha,
+                bias=module.bias is not None, device=module.weight.device, enable_aqn=enable_aqn,
+                aqn_alpha=aqn_alpha)
+        if module.weight.device.type == "meta":
+            q.weight = nn.Parameter(module.weight.detach(), requires_grad=False)
+            return q
+        if module.bias is not None:
+            with torch.no_grad():
+                q.bias.copy_(module.bias.detach())
+        q._quantize_and_store(module.weight.detach())
+        return q
+
+    def _quantize_and_store(self, w: Tensor, global_amax: Optional[Tensor] = None) -> None:
+        packed, scales = Q.nf4_quantize(w.reshape(self.out_features, self.in_features), self.quant_group_size)
+        self._write_packed_weight(self._to_uint8(packed))
+        self._scale_dtypes = {"weight_scales": scales.dtype}
+        self.weight_scales = self._to_uint8(scales.reshape(self.out_features, -1))
+        self._aqn_step_cache = None
+
+    def _quant_weight(self) -> QuantWeight:
+        return QuantWeight("nf4", _C.XQ_LAYOUT_FLAT, self._read_packed_weight_uint8(), self.weight_scales,
+                           self._scale_dtypes["weight_scales"], self.out_features, self.in_features,
+                           self.quant_group_size)
+
+    @torch.compiler.disable
+    def _dequantize_weight(self) -> Tensor:
+        s = self._recover_tensor(self.weight_scales, self._scale_dtypes["weight_scales"])
+        n = self.out_features * self.in_features
+        return Q.nf4_dequantize(self._read_packed_weight_uint8(), s, n, self.quant_group_size).reshape(
+            self.out_features, self.in_features)
+
+    @torch.compiler.disable
+    def _compute_aqn_step(self) -> Tensor:
+        """Half the narrowest gap between levels times the group's absmax (nf4_linear.py:113-120)."""
+        s = self._recover_tensor(self.weight_scales, self._scale_dtypes["weight_scales"]).float()
+        s = s.reshape(self.out_features, self.in_features // self.quant_group_size)
+        return (0.5 * Q.NF4_MIN_STEP * s.repeat_interleave(self.quant_group_size, 1)).contiguous()
+
+    def _load_prequantized(self, _load_tensor) -> None:
+        raise NotImplementedError("NF4 has no pre-quantized checkpoint format; use from_module() on bf16 weights")
 
 
 # =============================================================================

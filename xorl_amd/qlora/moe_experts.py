@@ -32,7 +32,7 @@ def compute_lora_scaling(lora_alpha: float, r: int, use_rslora: bool = False) ->
 
 
 class QLoRAMoeExperts(LoraModule, nn.Module):
-    """Base class; use BlockFP8QLoRAMoeExperts or NvFP4QLoRAMoeExperts."""
+    """Base class; use BlockFP8QLoRAMoeExperts, NvFP4QLoRAMoeExperts or NF4QLoRAMoeExperts."""
 
     adapter_gradient_producer_family = "fused_managed"
 
@@ -329,3 +329,41 @@ class NvFP4QLoRAMoeExperts(QLoRAMoeExperts):
         else:
             self._ema_amax[name] = fresh
         self._quantize_proj(name, merged, global_amax_per_expert=self._ema_amax[name])
+
+
+class NF4QLoRAMoeExperts(QLoRAMoeExperts):
+    """NormalFloat4 banks, one fp32 absmax per 64 elements along K; buffers
+    {gate,up,down}_{packed,scales} (qlora/modules/moe_experts.py:1149-1260)."""
+
+    def __init__(self, num_local_experts, num_experts, intermediate_size, hidden_size, r=16, lora_alpha=16, **kw):
+        kw.pop("quant_format", None)
+        kw.pop("quant_group_size", None)
+        super().__init__(num_local_experts, num_experts, intermediate_size, hidden_size, r=r, lora_alpha=lora_alpha,
+                         quant_format="nf4", quant_group_size=64, **kw)
+        for p in ("gate", "up", "down"):
+            self.register_buffer(f"{p}_packed", None)
+            self.register_buffer(f"{p}_scales", None)
+        self.reset_lora_parameters()
+
+    def _quantize_2d(self, w: Tensor, global_amax=None):
+        packed, scales = Q.nf4_quantize_gkn(w, self.quant_group_size)
+        return self._to_uint8(packed), {"weight_scales": (self._to_uint8(scales), scales.dtype)}
+
+    def _dequantize_2d(self, packed: Tensor, scales_dict: dict, K: int, N: int) -> Tensor:
+        scales = self._recover_tensor(*scales_dict["weight_scales"])
+        return Q.nf4_dequantize_gkn(packed, scales, K, N, self.quant_group_size)
+
+    def _bank(self, proj_name: str) -> QuantWeight:
+        K, N = self._proj_dims(proj_name)
+        return QuantWeight("nf4", _C.XQ_LAYOUT_GKN, getattr(self, f"{proj_name}_packed"),
+                           getattr(self, f"{proj_name}_scales"), self._scale_dtypes[proj_name]["weight_scales"],
+                           K, N, self.quant_group_size, num_experts=self.num_local_experts)
+
+    @torch.compiler.disable
+    def dequantize_all_experts(self, proj_name: str, K: int, N: int) -> Tensor:
+        import ctypes
+
+        w = self._bank(proj_name).c()
+        out = torch.empty(self.num_local_experts, K, N, dtype=torch.bfloat16, device=getattr(self, f"{proj_name}_packed").device)
+        _C.check(_C.lib().xq_decode(ctypes.byref(w), out.data_ptr(), _C.XQ_DT_BF16, _C.stream_ptr(out.device)))
+        return out

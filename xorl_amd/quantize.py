@@ -9,6 +9,7 @@ and restate the reference quantizers' arithmetic:
   int4_quantize_sym          the symmetric absmax/7 bf16-scale rule (not in the reference)
   nvfp4_quantize[_gkn]       ops/quantize/nvfp4_quantize.py:114-154, nvfp4_gkn_quantize.py:176-235
   block_fp8_quantize_gkn     ops/quantize/block_fp8_gkn_quantize.py:73-121
+  nf4_quantize[_gkn], nf4_dequantize[_gkn]   ops/quantize/nf4_quantize.py, nf4_gkn_quantize.py, nf4_codec.py
 """
 
 from __future__ import annotations
@@ -51,6 +52,21 @@ def int4_dequantize_gkn(packed: Tensor, scales: Tensor, K: int, N: int, group_si
     w = _C.make_weight("int4", _C.XQ_LAYOUT_GKN, packed, scales, scales.dtype, K, N, gs)
     out = _decode(w, torch.empty(K, N, dtype=torch.bfloat16, device=packed.device), _C.XQ_DT_BF16)
     return out if out_dtype == torch.bfloat16 else out.to(out_dtype)
+
+
+def nf4_dequantize(packed: Tensor, scales: Tensor, num_elements: int, group_size: int = 64) -> Tensor:
+    """Flat decode of `num_elements` NF4 values -> 1-D bf16 (ops/quantize/nf4_quantize.py:154-185)."""
+    assert num_elements % group_size == 0
+    sc = scales if scales.dtype in (torch.float32, torch.bfloat16) else scales.float()
+    w = _C.make_weight("nf4", _C.XQ_LAYOUT_FLAT, packed.reshape(-1), sc.reshape(-1), sc.dtype, 1, num_elements, group_size)
+    return _decode(w, torch.empty(num_elements, dtype=torch.bfloat16, device=packed.device), _C.XQ_DT_BF16)
+
+
+def nf4_dequantize_gkn(packed: Tensor, scales: Tensor, K: int, N: int, group_size: int = 64) -> Tensor:
+    """[K/2, N] u8 + [K/gs, N] scales -> [K, N] bf16 (ops/quantize/nf4_gkn_quantize.py:182-)."""
+    sc = scales if scales.dtype in (torch.float32, torch.bfloat16) else scales.float()
+    w = _C.make_weight("nf4", _C.XQ_LAYOUT_GKN, packed, sc, sc.dtype, K, N, group_size)
+    return _decode(w, torch.empty(K, N, dtype=torch.bfloat16, device=packed.device), _C.XQ_DT_BF16)
 
 
 def nvfp4_dequantize(packed: Tensor, block_scales: Tensor, global_scale: Tensor, num_elements: int,
@@ -97,6 +113,50 @@ def _pack_nibbles_first(q: Tensor) -> Tensor:
     """[2k, N] codes -> [k, N] bytes, even K-row in the low nibble."""
     q = q.to(torch.uint8)
     return q[0::2] | (q[1::2] << 4)
+
+
+# NF4 levels and the midpoints between neighbours (ops/quantize/nf4_codec.py:18-35, :42-64)
+NF4_TABLE = (-1.0, -0.6961928009986877, -0.5250730514526367, -0.39491748809814453, -0.28444138169288635,
+             -0.18477343022823334, -0.09105003625154495, 0.0, 0.07958029955625534, 0.16093020141124725,
+             0.24611230194568634, 0.33791524171829224, 0.44070982933044434, 0.5626170039176941,
+             0.7229568362236023, 1.0)
+NF4_MIN_STEP = 0.07958029955625534
+_NF4_MIDPOINTS = (-0.8480964004993439, -0.6106329262256622, -0.4599952697753906, -0.3396794348955154,
+                  -0.2346074059605598, -0.1379117332398891, -0.0455250181257725, 0.0397901497781277,
+                  0.1202552504837513, 0.2035212516784668, 0.2920137718319893, 0.3893125355243683,
+                  0.5016634166240692, 0.6427869200706482, 0.8614784181118012)
+
+
+def _nf4_encode(norm: Tensor) -> Tensor:
+    """code = number of midpoints strictly below the value (nf4_codec.py:42-64)."""
+    mid = torch.tensor(_NF4_MIDPOINTS, dtype=torch.float32, device=norm.device)
+    return (norm.unsqueeze(-1) > mid).sum(-1).to(torch.uint8)
+
+
+def nf4_quantize(x: Tensor, group_size: int = 64) -> Tuple[Tensor, Tensor]:
+    """[M, K] -> flat (M*K/2,) u8, flat (M*K/gs,) fp32 absmax scales (nf4_quantize.py:20-56, :118-151):
+    scale = max(amax, 1e-12); code = encode(clamp(x * (1/scale), -1, 1)); even element in the low nibble."""
+    assert x.dim() == 2
+    n = x.numel()
+    assert n % group_size == 0 and group_size % 2 == 0
+    xf = x.float().reshape(n // group_size, group_size)
+    scale = xf.abs().amax(-1).clamp_min(1e-12)
+    norm = (xf * (1.0 / scale).unsqueeze(-1)).clamp_(-1.0, 1.0)
+    codes = _nf4_encode(norm).reshape(-1)
+    return (codes[0::2] | (codes[1::2] << 4)).contiguous(), scale.contiguous()
+
+
+def nf4_quantize_gkn(x: Tensor, group_size: int = 64) -> Tuple[Tensor, Tensor]:
+    """[K, N] -> [K/2, N] u8, [K/gs, N] fp32 scales; groups and nibble pairs along K
+    (nf4_gkn_quantize.py:22-81, :145-179)."""
+    assert x.dim() == 2
+    K, N = x.shape
+    assert K % group_size == 0 and group_size % 2 == 0
+    xf = x.float().reshape(K // group_size, group_size, N)
+    scale = xf.abs().amax(1).clamp_min(1e-12)
+    norm = (xf * (1.0 / scale).unsqueeze(1)).clamp_(-1.0, 1.0)
+    codes = _nf4_encode(norm).reshape(K, N)
+    return _pack_nibbles_first(codes).contiguous(), scale.contiguous()
 
 
 def int4_quantize(x: Tensor, group_size: int = -1) -> Tuple[Tensor, Tensor]:
