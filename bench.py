@@ -138,7 +138,8 @@ def dense_module(fmt, N, K, r, alpha, seed, dev):
 
 
 def other_config(cfg: int, dev):
-    """Builds BASELINE.json configs[0], [2], [3] or [4] (or the merge pass, 5) on the device.  Returns
+    """Builds BASELINE.json configs[0], [2], [3] or [4] (or the merge pass, 5, or the NF4 variant of configs[1], 6)
+    on the device.  Returns
     (step_fn, work_per_step, unit_is_bytes, workload_text, kernel_text)."""
     lin_flops = lambda m, K, N, r: 4.0 * m * K * N + 6.0 * m * r * (K + N)
     rnd = lambda *shape, seed: torch.randn(*shape, generator=torch.Generator(device=dev).manual_seed(seed),
@@ -239,6 +240,22 @@ def other_config(cfg: int, dev):
                 "merge pass (not a BASELINE config): decode + LoRA update + re-encode (block_fp8 -> block_fp8) and "
                 "decode + update -> bf16, for gate/up [12288,4096] and down [4096,12288], r=32",
                 "merge_kernel<fp8> (fused decode + low-rank update + re-quantise / publish)")
+    if cfg == 6:
+        # not a BASELINE config: configs[1]'s three projections held as NF4 (group 64, fp32 absmax scales)
+        Mtok = 8192
+        shapes = {"gate": (12288, 4096), "up": (12288, 4096), "down": (4096, 12288)}
+        mods = {k: dense_module("nf4", N, K, 32, 64, 90 + i, dev) for i, (k, (N, K)) in enumerate(shapes.items())}
+        xs = {k: rnd(Mtok, K, seed=94 + i).requires_grad_(True) for i, (k, (N, K)) in enumerate(shapes.items())}
+        dys = {k: rnd(Mtok, N, seed=97 + i) for i, (k, (N, K)) in enumerate(shapes.items())}
+
+        def step():
+            for k, m in mods.items():
+                xs[k].grad = m.lora_A.grad = m.lora_B.grad = None
+                m(xs[k]).backward(dys[k])
+        return (step, sum(lin_flops(Mtok, K, N, 32) for (N, K) in shapes.values()), False,
+                "NF4 (not a BASELINE config): QLoRA Qwen3-8B MLP projections gate/up 4096->12288, down 12288->4096 "
+                "as NF4 group 64, M=8192, r=32, fwd+bwd of each linear",
+                "gemm_256_kernel<nf4> (fused dequant-GEMM, forward and dgrad launches)")
     raise SystemExit(f"bench.py: unknown --config {cfg}")
 
 

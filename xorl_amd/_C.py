@@ -132,7 +132,9 @@ def ptr(t: Optional[torch.Tensor]) -> Optional[int]:
 
 
 def stream_ptr(device: torch.device) -> int:
-    return torch.cuda.current_stream(device).cuda_stream
+    """Raw handle of torch's current stream on `device` (what every kernel is launched on)."""
+    idx = device.index
+    return torch._C._cuda_getCurrentRawStream(torch.cuda.current_device() if idx is None else idx)
 
 
 _SCALE_DT = {torch.float32: XQ_SCALE_F32, torch.bfloat16: XQ_SCALE_BF16, torch.float8_e4m3fn: XQ_SCALE_E4M3}

@@ -73,18 +73,17 @@ def _ld(x2: Tensor) -> int:
 # ---------------------------------------------------------------------------
 # dense: custom ops
 # ---------------------------------------------------------------------------
-@torch.library.custom_op("xq::linear_fwd", mutates_args=(), device_types="cuda")
-def _linear_fwd_op(x: Tensor, packed: Tensor, scales: Tensor, global_scale: Optional[Tensor],
-                   lora_A: Optional[Tensor], lora_B: Optional[Tensor], bias: Optional[Tensor],
-                   fmt: str, scale_code: int, group: int, N: int, K: int, r: int,
-                   scaling: float, want_su: bool) -> Tuple[Tensor, Tensor]:
+def _linear_fwd_impl(x: Tensor, packed: Tensor, scales: Tensor, global_scale: Optional[Tensor],
+                     lora_A: Optional[Tensor], lora_B: Optional[Tensor], bias: Optional[Tensor],
+                     fmt: str, scale_dt: torch.dtype, group: int, N: int, K: int, r: int,
+                     scaling: float, want_su: bool) -> Tuple[Tensor, Tensor]:
     if x.dtype != torch.bfloat16:
         raise _C.XqError(f"activations must be bf16, got {x.dtype}")
     x2 = _as_2d(x)
     M = x2.shape[0]
     if x2.shape[1] != K:
         raise _C.XqError(f"input width {x2.shape[1]} != in_features {K}")
-    w = _C.make_weight(fmt, _C.XQ_LAYOUT_FLAT, packed, scales, _CODE_TO_DT[scale_code], N, K, group, global_scale)
+    w = _C.make_weight(fmt, _C.XQ_LAYOUT_FLAT, packed, scales, scale_dt, N, K, group, global_scale)
     dev = x.device
     y = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
     rp = _r_pad(r)
@@ -99,6 +98,15 @@ def _linear_fwd_op(x: Tensor, packed: Tensor, scales: Tensor, global_scale: Opti
                              scaling, _C.ptr(b), y.data_ptr(), N, su.data_ptr() if (rp and want_su) else None, ws.data_ptr(),
                              ws_bytes, _C.stream_ptr(dev)))
     return y.reshape(*x.shape[:-1], N), su
+
+
+@torch.library.custom_op("xq::linear_fwd", mutates_args=(), device_types="cuda")
+def _linear_fwd_op(x: Tensor, packed: Tensor, scales: Tensor, global_scale: Optional[Tensor],
+                   lora_A: Optional[Tensor], lora_B: Optional[Tensor], bias: Optional[Tensor],
+                   fmt: str, scale_code: int, group: int, N: int, K: int, r: int,
+                   scaling: float, want_su: bool) -> Tuple[Tensor, Tensor]:
+    return _linear_fwd_impl(x, packed, scales, global_scale, lora_A, lora_B, bias, fmt, _CODE_TO_DT[scale_code],
+                            group, N, K, r, scaling, want_su)
 
 
 @_linear_fwd_op.register_fake
@@ -188,6 +196,14 @@ def qlora_linear(x: Tensor, qw: QuantWeight, lora_A: Optional[Tensor], lora_B: O
     # also lets small batches take the weight-streaming kernel.
     training = torch.is_grad_enabled() and any(
         t is not None and t.requires_grad for t in (x, lora_A, lora_B, bias))
+    if not training and not torch.compiler.is_compiling():
+        # decode-regime calls are launch-bound: go straight to the library, skipping the autograd and
+        # custom-op dispatch layers (tens of microseconds of host time per call)
+        A = lora_A.detach()[:r] if lora_A is not None else None
+        B = lora_B.detach()[:, :r] if lora_B is not None else None
+        return _linear_fwd_impl(x.detach(), qw.packed, qw.scales, qw.global_scale, A, B,
+                                None if bias is None else bias.detach(), qw.fmt, qw.scale_dtype, qw.group,
+                                qw.rows, qw.cols, r, float(scaling), False)[0]
     return QLoRALinearFunction.apply(x, lora_A, lora_B, bias, qw, r, scaling, training)
 
 
