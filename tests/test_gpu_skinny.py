@@ -43,3 +43,36 @@ def test_skinny_projection_shapes(hip_device, fmt, N, K):
         with torch.no_grad():
             y_again = m(x.to(hip_device))
         assert R.max_rel_err(y_again.cpu(), ex["y"]) <= TOL
+
+
+@pytest.mark.parametrize("fmt,N,K,M,r,bf16_factors", [
+    ("block_fp8", 21888, 1280, 3, 16, False),    # 10 chunks over 3 splits: 4 + 3 + 3 chunks per block
+    ("int4", 21888, 1280, 16, 16, False),
+    ("nvfp4", 208, 1024, 16, 6, False),          # ragged last row block, rank not a multiple of 4
+    ("block_fp8", 384, 2048, 17, 64, True),      # four 16-rank tiles, bf16 factors
+    ("int4", 1024, 4096, 32, 40, False),         # rank padded to 48
+    ("nvfp4", 4096, 4096, 9, 16, True),
+])
+def test_skinny_split_plans(hip_device, fmt, N, K, M, r, bf16_factors):
+    """K-split organisation: uneven splits, ragged row blocks, every rank-tile count, both factor dtypes."""
+    from xorl_amd.functional import qlora_linear
+
+    m, w_ref = make_dense_module(fmt, N, K, r, 2 * r, seed=N + K + M, device=hip_device, bias=(M == 16))
+    x = gen((M, K), 1.0, 300 + M, torch.bfloat16)
+    A, B = m.lora_A.detach(), m.lora_B.detach()
+    if bf16_factors:
+        A, B = A.to(torch.bfloat16), B.to(torch.bfloat16)
+    with torch.no_grad():
+        y = qlora_linear(x.to(hip_device), m._quant_weight(), A, B, r, m.scaling, m.bias)
+    ex = R.linear_fwd_bwd_exact(x, w_ref, A.float().cpu(), B.float().cpu(), m.scaling,
+                                bias=None if m.bias is None else m.bias.detach().cpu())
+    assert y.shape == (M, N) and R.max_rel_err(y.cpu(), ex["y"]) <= TOL
+    # deterministic: a second call returns the same bits
+    with torch.no_grad():
+        y2 = qlora_linear(x.to(hip_device), m._quant_weight(), A, B, r, m.scaling, m.bias)
+    assert torch.equal(y, y2)
+    # no low-rank term at all
+    with torch.no_grad():
+        y0 = qlora_linear(x.to(hip_device), m._quant_weight(), None, None, 0, 0.0, None)
+    ex0 = R.linear_fwd_bwd_exact(x, w_ref, torch.zeros(1, K), torch.zeros(N, 1), 0.0)
+    assert R.max_rel_err(y0.cpu(), ex0["y"]) <= TOL

@@ -1,33 +1,65 @@
 // Skinny-M (M <= 64) fused dequant-GEMM forward: the HBM-bound decode/rollout regime.
 //
-//   y[M, N] = x[M, K] . deq(W)^T + bias + su[M, r] . Lr[N, r]^T          (W FLAT [N, K])
+//   y[M, N] = x[M, K] . deq(W)^T + bias + s * (x . A^T) . B^T          (W FLAT [N, K])
 //
-// The packed weight is streamed from HBM exactly once, straight into the MFMA
-// operand registers: lane (n, h) of a wave owns row n of a 32-row slab and the
-// h-th 64-element half of each 128-element K chunk, so the four 16-byte loads a
-// lane issues per chunk (two for 4-bit formats) cover whole 128-byte lines and
-// every line is used once.  The bytes are decoded in registers to the exact bf16
-// value of the reference decoder and fed to v_mfma_f32_32x32x16_bf16 against x
-// fragments.  x is small and L2 resident, but every block needs all of it: it is
-// fetched with coalesced 16-byte loads (16 lanes per 256-byte row piece) and turned
-// into operand fragments through a wave-private, padded LDS tile -- per-lane
-// row-strided loads of x would cost more address-unit cycles than the whole weight
-// stream.
-// A block owns 32 weight rows and all of K; its NW waves (8, or 4 when there are
-// more slabs than CUs) each stream 1/NW of K and the partial sums meet in LDS
-// in a fixed order (no atomics, no device-scope fences: deterministic).  Loads are
-// issued a whole batch at a time -- packed codes, scales and the x fragments of
-// the batch together -- into one of two register sets, so the next batch is in
-// flight while the current one is decoded and multiplied.
-// The low-rank term needs one small launch before it: su = x . A^T (fp32), one
-// block whose 16 waves split K; both kernels read the LoRA factors in their own
-// dtype (fp32 or bf16), so nothing is repacked or zeroed per call.
+// Every byte of the packed weight is read from HBM exactly once, decoded in registers to the exact bf16
+// value of the reference decoder and fed to v_mfma_f32_32x32x16_bf16 against x fragments.  Two launches per
+// forward, no atomics, no zeroed buffers, fixed summation orders (deterministic).  Two organisations:
+//
+//  M <= 32 -- K split across blocks (skinny_split_kernel + skinny_epilogue_kernel).  Partial outputs are
+//     tiny at these M, so the grid is (128-row block) x (K split): a block's four waves own 32 weight rows
+//     each and the same K range of at most four 128-element chunks.  ALL loads of a block -- its x slice and
+//     its whole weight tile -- are issued before anything is waited for, so the kernel is one memory round
+//     trip deep, and the number of K splits is chosen so that the whole grid is resident at once (four blocks
+//     per CU at M <= 16, three above).  Weight loads are coalesced (a load instruction covers whole rows of a
+//     chunk) and reach the MFMA layout through a wave-private XOR-swizzled LDS slab; the x slice
+//     [M, K range] goes through LDS once per block and is shared by the four waves.  Each block stores its fp32 partial tile to
+//     part[split][M][N]; the first `su_blocks` blocks carry no weight rows and compute the low-rank
+//     intermediate su = x . A^T for one K split each.  The epilogue sums the splits in order, adds bias and
+//     s * su . B^T in fp32 and rounds once to bf16.
+//
+//  32 < M <= 64 -- K split across the waves of a block (skinny_su_kernel + skinny_rows_kernel).  Partial
+//     tiles would cost as much traffic as the weights here, so a block owns 32 weight rows and all of K; its
+//     waves (8, or 4 when there are more slabs than CUs) each stream 1/NW of K in batches through two
+//     register sets and the partial sums meet in LDS in wave order.  x is fetched with coalesced loads into
+//     wave-private padded LDS tiles.  The low-rank term needs one small launch before it (partial sums of
+//     x . A^T over K ranges of 512) and is added by the last wave under the latency of its first batch.
 #include "xq_common.h"
 #include "xq_lora.h"
 
 namespace xq {
 
 struct SkinnyArgs {
+    const bf16_t* x;
+    int64_t ldx;
+    int32_t M, N, K;
+    const uint8_t* packed;
+    const uint8_t* scales;
+    const float* global_scale;
+    int32_t group, scale_dtype;
+    int32_t splits;            // K splits
+    int32_t su_blocks;         // leading grid rows (0 or 1) whose blocks compute the su part of their split
+    int32_t chunk_q, chunk_rem; // 128-element chunks per split: chunk_q, one more in the first chunk_rem splits
+    int32_t xp;                // LDS row pitch of the x slice in bf16 elements (longest split + 8)
+    float* partial;            // [splits][M][N]
+    float* su_part;            // [splits * 4][M][r_pad]
+    const void* lora_A;        // [r, K] fp32 or bf16
+    int32_t lora_f32, r, r_pad;
+};
+
+struct SkinnyEpiArgs {
+    const float* partial;
+    const float* su_part;
+    int32_t splits, su_parts, M, N;
+    const void* lora_B;        // [N, r] fp32 or bf16
+    int32_t lora_f32, r, r_pad;
+    float su_scale;
+    const bf16_t* bias;
+    bf16_t* y;
+    int64_t ldy;
+};
+
+struct SkinnyRowsArgs {
     const bf16_t* x;
     int64_t ldx;
     int32_t M, N, K;
@@ -94,11 +126,361 @@ __device__ __forceinline__ bf16x8 factor_frag(const void* base, int64_t idx, boo
     return __builtin_bit_cast(bf16x8, r);
 }
 
+// One block = 128 weight rows x one K split (or, for the leading su blocks, the x . A^T part of one split).
+template <int FMT, int MR, int NCH>
+__global__ void __launch_bounds__(256, MR == 16 ? 4 : 3) skinny_split_kernel(SkinnyArgs g) {
+    constexpr int MT = 1;                              // one 32-column MFMA tile of x rows (M <= MR <= 32)
+    // Pin every argument in scalar registers here: otherwise the argument loads are placed lazily, each batch
+    // with its own wait, and several memory round trips pass before the first weight load is issued.
+    asm volatile("" ::"s"(g.x), "s"(g.ldx), "s"(g.M), "s"(g.N), "s"(g.K), "s"(g.packed), "s"(g.scales), "s"(g.global_scale),
+                 "s"(g.group), "s"(g.scale_dtype), "s"(g.splits), "s"(g.su_blocks), "s"(g.chunk_q), "s"(g.chunk_rem),
+                 "s"(g.xp), "s"(g.partial), "s"(g.su_part), "s"(g.lora_A), "s"(g.lora_f32), "s"(g.r), "s"(g.r_pad));
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    bf16_t* xs = (bf16_t*)smem;                                  // [M rows][xp]; fragment rows >= M read row 0: they feed
+    const int XP = g.xp;                                         // only output columns >= M, which are never stored
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int fr = lane & 31, fh = lane >> 5;
+    constexpr int EB = FMT == XQ_FMT_FP8 ? 1 : 2;      // elements per byte
+    constexpr int NLOAD = FMT == XQ_FMT_FP8 ? 4 : 2;   // 16-byte loads per lane per 128-k chunk
+    constexpr int NSC = FMT == XQ_FMT_NVFP4 ? 4 : 1;   // scale registers per chunk
+
+    // grid: x = K split, y = 128-row block, preceded by one row of su blocks when there is a low-rank term
+    const int split = blockIdx.x;
+    const bool su_block = (int)blockIdx.y < g.su_blocks;
+    const int rb = su_block ? 0 : (int)blockIdx.y - g.su_blocks;
+    // the first `chunk_rem` splits hold chunk_q + 1 chunks of 128 elements, the others chunk_q (no divisions here:
+    // nothing is in flight until the loads below are issued)
+    const int c_begin = split * g.chunk_q + (split < g.chunk_rem ? split : g.chunk_rem);
+    const int nch = g.chunk_q + (split < g.chunk_rem ? 1 : 0);   // 1 .. NCH (the launcher guarantees it)
+    const int c_end = c_begin + nch;
+    const int k_begin = c_begin << 7;
+
+    // ---- x slice [M][nch*128]: coalesced 16-byte pieces, row-major over the block's threads.  Every load below
+    // is unconditional (rows and chunks past the end are clamped onto valid ones and their data ignored): with
+    // no branches between the loads and their uses the waits count exactly, so the x slice is staged and each
+    // weight chunk decoded while the chunks behind it are still in flight.
+    constexpr int XL = MR * NCH / 16;                            // pieces per thread at most: MR rows x NCH*16 / 256
+    const int ppr = nch << 4;                                    // pieces per row: 16, 32, 48 or 64
+    const int q256 = nch == 3 ? 5 : 16 >> (nch >> 1), r256 = nch == 3 ? 16 : 0;   // 256 = q256 * ppr + r256
+    const int row0 = nch == 3 ? ((tid >> 4) * 11) >> 5 : tid >> (4 + (nch >> 1)); // tid / ppr
+    const int col0 = tid - row0 * ppr;
+    u32x4 xr[XL];
+    {
+        int row = row0, col = col0;
+#pragma unroll
+        for (int i = 0; i < XL; ++i) {
+            const int rc = row < g.M ? row : g.M - 1;
+            xr[i] = *(const u32x4*)(g.x + (int64_t)rc * g.ldx + k_begin + col * 8);
+            col += r256;
+            row += q256;
+            if (col >= ppr) { col -= ppr; ++row; }
+        }
+    }
+    int xrow[MT];                                                // LDS row of this lane's x fragments
+#pragma unroll
+    for (int i = 0; i < MT; ++i) xrow[i] = i * 32 + fr < g.M ? i * 32 + fr : 0;
+    auto stage_x = [&]() {
+        int row = row0, col = col0;
+#pragma unroll
+        for (int i = 0; i < XL; ++i) {
+            if (row < g.M) *(u32x4*)(xs + row * XP + col * 8) = xr[i];
+            col += r256;
+            row += q256;
+            if (col >= ppr) { col -= ppr; ++row; }
+        }
+        // block barrier on the LDS writes only: __syncthreads() would also wait for every weight load in flight
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    };
+
+    if (su_block) {
+        // su part of this split, D[rank][m] (ranks >= r are zero): wave w takes the k16 steps t = w, w+4, ...; the
+        // four sums meet in LDS (behind the x slice) in wave order.  The factor rows are fetched with unconditional
+        // 16-byte loads (rows and steps past the end clamped, their values masked), the first rank tile's together
+        // with the x slice.
+        const int steps = nch << 3;
+        float* out = g.su_part + (int64_t)split * g.M * g.r_pad;
+        float* red = (float*)(smem + (size_t)g.M * XP * 2);        // [4 waves][16 regs][64 lanes]
+        u32x4 ar[2 * NCH][2];
+        auto load_a = [&](int jt) {
+            const int rrow = jt * 32 + fr;
+            const int64_t base = (int64_t)(rrow < g.r ? rrow : 0) * g.K + k_begin + fh * 8;
+#pragma unroll
+            for (int u = 0; u < 2 * NCH; ++u) {
+                const int t = wave + 4 * u < steps ? wave + 4 * u : steps - 1;
+                if (g.lora_f32) {
+                    ar[u][0] = *(const u32x4*)((const float*)g.lora_A + base + t * 16);
+                    ar[u][1] = *(const u32x4*)((const float*)g.lora_A + base + t * 16 + 4);
+                } else {
+                    ar[u][0] = *(const u32x4*)((const bf16_t*)g.lora_A + base + t * 16);
+                }
+            }
+        };
+        load_a(0);
+        stage_x();
+        for (int jt = 0; jt < ((g.r_pad + 31) >> 5); ++jt) {
+            if (jt > 0) load_a(jt);
+            const bool rvalid = jt * 32 + fr < g.r;
+            bf16x8 af[2 * NCH];
+#pragma unroll
+            for (int u = 0; u < 2 * NCH; ++u) {
+                u32x4 v = ar[u][0];
+                if (g.lora_f32) {
+                    v = u32x4{pack_bf16x2(__uint_as_float(ar[u][0][0]), __uint_as_float(ar[u][0][1])),
+                              pack_bf16x2(__uint_as_float(ar[u][0][2]), __uint_as_float(ar[u][0][3])),
+                              pack_bf16x2(__uint_as_float(ar[u][1][0]), __uint_as_float(ar[u][1][1])),
+                              pack_bf16x2(__uint_as_float(ar[u][1][2]), __uint_as_float(ar[u][1][3]))};
+                }
+                if (!rvalid || wave + 4 * u >= steps) v = u32x4{0, 0, 0, 0};
+                af[u] = __builtin_bit_cast(bf16x8, v);
+            }
+            f32x16 sacc;
+#pragma unroll
+            for (int q = 0; q < 16; ++q) sacc[q] = 0.0f;
+#pragma unroll
+            for (int u = 0; u < 2 * NCH; ++u) {
+                const int t = wave + 4 * u;
+                if (t < steps) {
+                    const bf16x8 xf = *(const bf16x8*)(xs + xrow[0] * XP + t * 16 + fh * 8);
+                    sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[u], xf, sacc, 0, 0, 0);
+                }
+            }
+            __syncthreads();   // the previous rank tile's sums have been read
+#pragma unroll
+            for (int q = 0; q < 16; ++q) red[(wave * 16 + q) * 64 + lane] = sacc[q];
+            __syncthreads();
+            // wave w sums register quad w of every lane: ranks jt*32 + 8w + 4*fh .. +3 of row m = fr
+            f32x4 v = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int ww = 0; ww < 4; ++ww)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] += red[(ww * 16 + wave * 4 + e) * 64 + lane];
+            const int j0 = jt * 32 + 8 * wave + 4 * fh;
+            if (fr < g.M && j0 < g.r_pad) *(f32x4*)(out + (int64_t)fr * g.r_pad + j0) = v;
+        }
+        return;
+    }
+
+    // ---- the block's whole weight tile -> registers, fetched coalesced: a load instruction covers whole
+    // rows of the chunk (lane l: row l / PPR of the instruction's rows, 16-byte piece l % PPR)
+    constexpr int PPR = FMT == XQ_FMT_FP8 ? 8 : 4;     // 16-byte pieces per row per 128-k chunk
+    constexpr int RPI = 64 / PPR;                      // rows per load instruction
+    const int lrow = lane / PPR, lpiece = lane % PPR;
+    const int nbase = rb * 128 + wave * 32;
+    int n = nbase + fr;                                 // the row this lane feeds to the MFMA
+    n = n < g.N ? n : g.N - 1;
+    u32x4 w[NCH][NLOAD];
+    uint32_t sc[NCH][NSC];
+    const bool int4_small_group = FMT == XQ_FMT_INT4 && (g.group & 127) != 0;   // looked up per 8 elements at use
+    {
+        const uint8_t* wp[NLOAD];
+#pragma unroll
+        for (int i = 0; i < NLOAD; ++i) {
+            int nl = nbase + RPI * i + lrow;
+            nl = nl < g.N ? nl : g.N - 1;
+            wp[i] = g.packed + ((int64_t)nl * g.K) / EB + lpiece * 16;
+        }
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) {
+            const int cc = c_begin + c < c_end ? c_begin + c : c_end - 1;
+#pragma unroll
+            for (int i = 0; i < NLOAD; ++i) w[c][i] = *(const u32x4*)(wp[i] + (int64_t)cc * (128 / EB));
+            if (FMT == XQ_FMT_FP8) sc[c][0] = ((const uint32_t*)g.scales)[(n >> 7) * ((g.K + 127) >> 7) + cc];
+            else if (FMT == XQ_FMT_INT4) {
+                const int64_t si = int4_small_group ? 0 : ((int64_t)n * g.K + cc * 128) / g.group;
+                sc[c][0] = g.scale_dtype == XQ_SCALE_F32 ? ((const uint32_t*)g.scales)[si] : ((const uint16_t*)g.scales)[si];
+            } else {
+                const int64_t si = ((int64_t)n * g.K + cc * 128) >> 4;   // the 8 block scales of this row's chunk
+                if (g.scale_dtype == XQ_SCALE_E4M3) {
+                    const u32x2 t = *(const u32x2*)(g.scales + si);
+                    sc[c][0] = t[0];
+                    sc[c][1] = t[1];
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) sc[c][j] = ((const uint32_t*)g.scales)[si + 2 * j + fh];   // this lane's four
+                }
+            }
+        }
+    }
+    stage_x();
+
+    // ---- decode + multiply: D[n][m] += deq(W)[n][k] x[m][k].  Each chunk's slab goes through a wave-private LDS
+    // staging area (XOR-swizzled 16-byte pieces: writes and fragment reads are conflict free) to reach the
+    // MFMA layout: lane (row fr, half fh) reads piece 2u+fh of its row for the k16 steps 2u and 2u+1, i.e. step
+    // t = 2u+v covers k = 32u + 16*fh + 8v .. +7 of the chunk; the x fragments use the same map.  LDS operations
+    // of one wave execute in order, so the slab is reused chunk after chunk without barriers.
+    const float gsc = FMT == XQ_FMT_NVFP4 ? g.global_scale[0] : 1.0f;
+    unsigned char* wst = smem + (size_t)g.M * XP * 2 + wave * (PPR * 32 * 16);
+    f32x16 acc[MT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int q = 0; q < 16; ++q) acc[i][q] = 0.0f;
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+        if (c < nch) {
+#pragma unroll
+            for (int i = 0; i < NLOAD; ++i) {
+                const int rl = RPI * i + lrow;
+                const int sw = FMT == XQ_FMT_FP8 ? (rl >> 1) & 7 : (rl >> 2) & 3;
+                *(u32x4*)(wst + (rl * PPR + (lpiece ^ sw)) * 16) = w[c][i];
+            }
+            __builtin_amdgcn_wave_barrier();
+            const int kc = (c_begin + c) * 128;
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                uint32_t f[4];
+                if (FMT == XQ_FMT_FP8) {
+                    const u32x4 t = *(const u32x4*)(wst + (fr * 8 + ((2 * u + fh) ^ ((fr >> 1) & 7))) * 16);
+                    f[0] = t[0]; f[1] = t[1]; f[2] = t[2]; f[3] = t[3];
+                } else {
+                    const u32x2 t = *(const u32x2*)(wst + (fr * 4 + (u ^ ((fr >> 2) & 3))) * 16 + fh * 8);
+                    f[0] = t[0]; f[1] = t[1];
+                }
+#pragma unroll
+                for (int v = 0; v < 2; ++v) {
+                    bf16x8 wf;
+                    if (FMT == XQ_FMT_FP8) {
+                        wf = decode8<FMT>(f[2 * v], f[2 * v + 1], __uint_as_float(sc[c][0]), 0.0f);
+                    } else if (FMT == XQ_FMT_INT4) {
+                        float sv;
+                        if (int4_small_group) sv = load_scale(g.scales, ((int64_t)n * g.K + kc + 32 * u + 16 * fh + 8 * v) / g.group, g.scale_dtype);
+                        else sv = g.scale_dtype == XQ_SCALE_F32 ? __uint_as_float(sc[c][0]) : __uint_as_float(sc[c][0] << 16);
+                        wf = decode8<FMT>(f[v], 0u, sv, -8.0f * sv);
+                    } else {
+                        float sv;   // block scale 2u + fh of the chunk
+                        if (g.scale_dtype == XQ_SCALE_E4M3) sv = e4m3_to_f32((uint8_t)(sc[c][u >> 1] >> (8 * (2 * (u & 1) + fh))));
+                        else sv = __uint_as_float(sc[c][u]);
+                        wf = decode8<FMT>(f[v], 0u, sv * gsc, 0.0f);
+                    }
+#pragma unroll
+                    for (int i = 0; i < MT; ++i) {
+                        const bf16x8 xf = *(const bf16x8*)(xs + xrow[i] * XP + c * 128 + 32 * u + 16 * fh + 8 * v);
+                        acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf, xf, acc[i], 0, 0, 0);
+                    }
+                }
+            }
+            __builtin_amdgcn_wave_barrier();
+        }
+    }
+
+    // ---- fp32 partial tile: lane (m = fr) holds 4 consecutive weight rows per register quad
+    float* out = g.partial + (int64_t)split * g.M * g.N;
+    const int nb = nbase;
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+        const int m = i * 32 + fr;
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) {
+            const int nn = nb + 8 * q4 + 4 * fh;
+            if (m < g.M && nn < g.N)   // N % 16 == 0: groups of 4 columns are all in or all out
+                *(f32x4*)(out + (int64_t)m * g.N + nn) = f32x4{acc[i][q4 * 4], acc[i][q4 * 4 + 1], acc[i][q4 * 4 + 2], acc[i][q4 * 4 + 3]};
+        }
+    }
+}
+
+// y[m][n..n+3] = sum_s part[s][m][n..] + bias + su_scale * sum_j su[m][j] * B[n][j], su = sum of the su parts.
+// One wave per output row m (up to four rows per block), a lane per 4 consecutive columns; nothing is shared
+// between waves.  Loads are unconditional (indices past the end are clamped, their values masked to zero), so
+// that a wave's su parts, partial tiles and B rows are all in flight together.  Every sum runs in a fixed
+// order: parts p = g, g+4, ... per lane group g, then the four groups; splits ascending.
+// RT = 16-rank tiles of the low-rank term (0 = none); VEC = B is fp32 with r % 4 == 0 (16-byte row pieces).
+template <int RT, bool VEC>
+__global__ void __launch_bounds__(256) skinny_epilogue_kernel(SkinnyEpiArgs g) {
+    // all arguments in scalar registers after one round trip (see skinny_split_kernel)
+    asm volatile("" ::"s"(g.partial), "s"(g.su_part), "s"(g.splits), "s"(g.su_parts), "s"(g.M), "s"(g.N), "s"(g.lora_B),
+                 "s"(g.lora_f32), "s"(g.r), "s"(g.r_pad), "s"(g.su_scale), "s"(g.bias), "s"(g.y), "s"(g.ldy));
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int m = blockIdx.y * 4 + wave;
+    if (m >= g.M) return;                                        // wave-uniform
+    int n = (blockIdx.x * 64 + lane) * 4;
+    const bool nvalid = n < g.N;                                 // N % 4 == 0: a lane's 4 columns are all in or all out
+    n = nvalid ? n : 0;
+    const int j = lane & 15, pg = lane >> 4;
+
+    // su parts: lane (j, pg) sums parts pg, pg+4, ... of rank j of each tile
+    float sv[RT > 0 ? RT : 1];
+#pragma unroll
+    for (int jt = 0; jt < RT; ++jt) sv[jt] = 0.0f;
+    const int64_t pstride = (int64_t)g.M * g.r_pad;
+    for (int p0 = 0; p0 < g.su_parts; p0 += 32) {
+        float t[RT > 0 ? RT : 1][8];
+#pragma unroll
+        for (int jt = 0; jt < RT; ++jt)
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int pi = p0 + pg + 4 * u;
+                t[jt][u] = g.su_part[(int64_t)(pi < g.su_parts ? pi : g.su_parts - 1) * pstride + (int64_t)m * g.r_pad + jt * 16 + j];
+            }
+#pragma unroll
+        for (int jt = 0; jt < RT; ++jt)
+#pragma unroll
+            for (int u = 0; u < 8; ++u) sv[jt] += p0 + pg + 4 * u < g.su_parts ? t[jt][u] : 0.0f;
+    }
+    // partial tiles
+    f32x4 o = {0.0f, 0.0f, 0.0f, 0.0f};
+    const float* pp = g.partial + (int64_t)m * g.N + n;
+    const int64_t sstride = (int64_t)g.M * g.N;
+    for (int s0 = 0; s0 < g.splits; s0 += 16) {
+        f32x4 t[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) t[u] = *(const f32x4*)(pp + (int64_t)(s0 + u < g.splits ? s0 + u : g.splits - 1) * sstride);
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+            if (s0 + u < g.splits) o += t[u];                     // wave-uniform
+        }
+    }
+    // low-rank term, 16 ranks at a time
+#pragma unroll
+    for (int jt = 0; jt < RT; ++jt) {
+        float bv[4][16];
+        if (VEC) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int jr = jt * 16 + 4 * q;              // r % 4 == 0: a group of 4 ranks is all in or all out
+                    const f32x4 t = *(const f32x4*)((const float*)g.lora_B + (int64_t)(n + e) * g.r + (jr < g.r ? jr : 0));
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) bv[e][4 * q + c] = jr < g.r ? t[c] : 0.0f;
+                }
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+#pragma unroll
+                for (int jj = 0; jj < 16; ++jj) {
+                    const int jr = jt * 16 + jj;
+                    const int64_t idx = (int64_t)(n + e) * g.r + (jr < g.r ? jr : 0);
+                    const float t = g.lora_f32 ? ((const float*)g.lora_B)[idx] : bf16_to_f32(((const bf16_t*)g.lora_B)[idx]);
+                    bv[e][jj] = jr < g.r ? t : 0.0f;
+                }
+        }
+        float tot = __shfl(sv[jt], j, 64);
+        tot += __shfl(sv[jt], 16 + j, 64);
+        tot += __shfl(sv[jt], 32 + j, 64);
+        tot += __shfl(sv[jt], 48 + j, 64);
+        tot *= g.su_scale;                                        // lane l holds su[m][jt*16 + (l & 15)], zero for ranks >= r
+#pragma unroll
+        for (int jj = 0; jj < 16; ++jj) {
+            const float sj = __shfl(tot, jj, 64);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o[e] = __builtin_fmaf(sj, bv[e][jj], o[e]);
+        }
+    }
+    if (!nvalid) return;
+    if (g.bias) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] += bf16_to_f32(g.bias[n + e]);
+    }
+    *(u32x2*)(g.y + (int64_t)m * g.ldy + n) = u32x2{pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3])};
+}
+
 // One block = 32 weight rows x the whole K, NW waves each streaming 1/NW of K (in-block
 // split-K: no atomics, no fences, fixed summation order).  x fragments are read from global
 // memory (coalesced, see the top of the file) together with the codes of the same batch.
 template <int FMT, int MT, int NW>
-__global__ void __launch_bounds__(NW * 64) skinny_kernel(SkinnyArgs g) {
+__global__ void __launch_bounds__(NW * 64) skinny_rows_kernel(SkinnyRowsArgs g) {
     extern __shared__ __attribute__((aligned(16))) float red[];   // [NW waves][MT*16 regs][64 lanes]
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: keeps the K-range loop on scalar branches
@@ -278,7 +660,7 @@ __global__ void __launch_bounds__(NW * 64) skinny_kernel(SkinnyArgs g) {
 
 // Partial sums of su = x[M, K] . A[r, K]^T (fp32, unscaled): block kb covers K range
 // [kb*SU_KB, (kb+1)*SU_KB) with its 8 waves (one eighth each, summed through LDS in wave order) and
-// writes part[kb][M][r_pad]; columns r..r_pad-1 are zero.  skinny_kernel adds the parts in block
+// writes part[kb][M][r_pad]; columns r..r_pad-1 are zero.  skinny_rows_kernel adds the parts in block
 // order, so the low-rank term is deterministic and needs no zeroed buffer and no atomics.
 constexpr int SU_KB = 512, SU_NW = 8;
 template <int MT>
@@ -338,11 +720,32 @@ __global__ void __launch_bounds__(SU_NW * 64) skinny_su_kernel(const bf16_t* x, 
     }
 }
 
+
 static inline int64_t al256(int64_t b) { return (b + 255) & ~(int64_t)255; }
 
+constexpr int kSplitMaxM = 32;   // rows up to which the K-split-across-blocks organisation is used
+
+// K splits for the split organisation: at most four chunks per split; more splits until the grid holds
+// about two blocks per CU, never more than the 1024 blocks that are resident at once (four per CU).
+struct SkinnyPlan { int splits, nch, row_blocks; };
+static SkinnyPlan skinny_plan(int64_t N, int64_t K) {
+    const int ct = (int)(K >> 7), rb = (int)xq_cdiv(N, 128);
+    int splits = (int)xq_cdiv(ct, 4);
+    while (splits < ct && (int64_t)(rb + 1) * splits < 512 && (int64_t)(rb + 1) * (splits + 1) <= 1024) ++splits;
+    SkinnyPlan p;
+    p.splits = splits;
+    p.nch = (int)xq_cdiv(ct, splits);   // the longest split
+    p.row_blocks = rb;
+    return p;
+}
+
 int64_t skinny_workspace_bytes(int64_t M, int64_t N, int64_t K, int r_pad) {
-    (void)N;
-    return al256(xq_cdiv(K, SU_KB) * M * (r_pad ? r_pad : 16) * 4) + 256;
+    const int rp = r_pad ? r_pad : 16;
+    if (M <= kSplitMaxM) {
+        const SkinnyPlan p = skinny_plan(N, K);
+        return al256((int64_t)p.splits * M * N * 4) + al256((int64_t)p.splits * M * rp * 4) + 256;
+    }
+    return al256(xq_cdiv(K, SU_KB) * M * rp * 4) + 256;
 }
 
 bool skinny_supported(const xq_weight* w, int64_t M) {
@@ -354,31 +757,117 @@ bool skinny_supported(const xq_weight* w, int64_t M) {
     return true;
 }
 
+// ---------------------------------------------------------------- M <= 32
+template <int FMT, int NCH>
+static int launch_split_one(const SkinnyArgs& g, dim3 grid, size_t lds, hipStream_t s) {
+    // at most 32 rows of 1040 B + the slabs = 49 KB: below the default dynamic LDS limit
+    if (g.M <= 16) skinny_split_kernel<FMT, 16, NCH><<<grid, 256, lds, s>>>(g);
+    else skinny_split_kernel<FMT, 32, NCH><<<grid, 256, lds, s>>>(g);
+    return XQ_OK;
+}
+
+template <int FMT>
+static int launch_split_cfg(const SkinnyArgs& g, int nch, dim3 grid, size_t lds, hipStream_t s) {
+    if (nch <= 1) return launch_split_one<FMT, 1>(g, grid, lds, s);
+    if (nch <= 2) return launch_split_one<FMT, 2>(g, grid, lds, s);
+    return launch_split_one<FMT, 4>(g, grid, lds, s);
+}
+
+static int launch_skinny_split(const xq_weight* w, const bf16_t* x, int64_t ldx, int64_t M, const void* lora_A, const void* lora_B,
+                               int lora_dtype, int r, int rp, float scaling, const bf16_t* bias, bf16_t* y, int64_t ldy,
+                               void* workspace, hipStream_t stream) {
+    const int64_t N = w->rows, K = w->cols;
+    const SkinnyPlan p = skinny_plan(N, K);
+    XQ_REQUIRE(p.nch <= 4, "xq_linear_fwd: internal error: K split too long (%d chunks)", p.nch);
+    XQ_REQUIRE(rp == 0 || xq_aligned(lora_A, 16), "xq_linear_fwd: lora_A must be 16-byte aligned");
+    SkinnyArgs g;
+    g.x = x; g.ldx = ldx; g.M = (int)M; g.N = (int)N; g.K = (int)K;
+    g.packed = (const uint8_t*)w->packed; g.scales = (const uint8_t*)w->scales; g.global_scale = w->global_scale;
+    g.group = w->group; g.scale_dtype = w->scale_dtype;
+    g.splits = p.splits; g.su_blocks = rp ? 1 : 0; g.xp = p.nch * 128 + 8;
+    g.chunk_q = (int)(K >> 7) / p.splits; g.chunk_rem = (int)(K >> 7) % p.splits;
+    g.partial = (float*)workspace;
+    g.su_part = (float*)((char*)workspace + al256((int64_t)p.splits * M * N * 4));
+    g.lora_A = rp ? lora_A : nullptr; g.lora_f32 = lora_dtype == XQ_DT_F32; g.r = r; g.r_pad = rp;
+    const dim3 grid((unsigned)p.splits, (unsigned)(p.row_blocks + g.su_blocks));
+    const size_t lds = (size_t)M * g.xp * 2 + 4 * 4096;   // x slice + the four weight slabs (or the su reduction buffer)
+
+    SkinnyEpiArgs e;
+    e.partial = g.partial; e.su_part = g.su_part; e.splits = p.splits; e.su_parts = rp ? p.splits : 0;
+    e.M = (int)M; e.N = (int)N; e.lora_B = rp ? lora_B : nullptr; e.lora_f32 = g.lora_f32; e.r = r; e.r_pad = rp;
+    e.su_scale = scaling; e.bias = bias; e.y = y; e.ldy = ldy;
+
+    int rc;
+    if (w->format == XQ_FMT_FP8) rc = launch_split_cfg<XQ_FMT_FP8>(g, p.nch, grid, lds, stream);
+    else if (w->format == XQ_FMT_INT4) rc = launch_split_cfg<XQ_FMT_INT4>(g, p.nch, grid, lds, stream);
+    else rc = launch_split_cfg<XQ_FMT_NVFP4>(g, p.nch, grid, lds, stream);
+    if (rc) return rc;
+    const int waves = M < 4 ? (int)M : 4;
+    const dim3 egrid((unsigned)xq_cdiv(N, 256), (unsigned)xq_cdiv(M, 4));
+    const bool vec = g.lora_f32 && r % 4 == 0 && xq_aligned(lora_B, 16);
+#define XQ_EPI(RT)                                                                                      \
+    do {                                                                                                \
+        if (vec) skinny_epilogue_kernel<RT, true><<<egrid, waves * 64, 0, stream>>>(e);                 \
+        else skinny_epilogue_kernel<RT, false><<<egrid, waves * 64, 0, stream>>>(e);                    \
+    } while (0)
+    switch (rp >> 4) {
+        case 0: skinny_epilogue_kernel<0, false><<<egrid, waves * 64, 0, stream>>>(e); break;
+        case 1: XQ_EPI(1); break;
+        case 2: XQ_EPI(2); break;
+        case 3: XQ_EPI(3); break;
+        default: XQ_EPI(4); break;
+    }
+#undef XQ_EPI
+    return XQ_OK;
+}
+
+// ---------------------------------------------------------------- 32 < M <= 64
 template <int FMT, int MT, int NW>
-static int launch_skinny_one(const SkinnyArgs& g, dim3 grid, hipStream_t s) {
+static int launch_rows_one(const SkinnyRowsArgs& g, dim3 grid, hipStream_t s) {
     // LDS: the wave-private x tiles (MT*32 rows of 272 B per wave); the reduction buffer reuses them
     constexpr size_t lds = (size_t)NW * MT * 32 * 136 * 2;
     static_assert(lds >= (size_t)NW * MT * 16 * 64 * 4, "reduction buffer must fit in the x tiles");
     static bool attr_set = false;
     if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute((const void*)skinny_kernel<FMT, MT, NW>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        hipError_t e = hipFuncSetAttribute((const void*)skinny_rows_kernel<FMT, MT, NW>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) {
             xq_set_error("xq_linear_fwd: cannot raise the dynamic LDS limit: %s", hipGetErrorString(e));
             return XQ_ERR_LAUNCH;
         }
         attr_set = true;
     }
-    skinny_kernel<FMT, MT, NW><<<grid, NW * 64, lds, s>>>(g);
+    skinny_rows_kernel<FMT, MT, NW><<<grid, NW * 64, lds, s>>>(g);
     return XQ_OK;
 }
 
 template <int FMT>
-static int launch_skinny_cfg(const SkinnyArgs& g, hipStream_t s) {
+static int launch_rows_cfg(const SkinnyRowsArgs& g, hipStream_t s) {
     dim3 grid((unsigned)xq_cdiv(g.N, 32));
     // more slabs than CUs: 4 waves per slab so that two blocks share a CU; else 8 waves per slab
     const bool many = grid.x > 256;
-    if (g.M <= 32) return many ? launch_skinny_one<FMT, 1, 4>(g, grid, s) : launch_skinny_one<FMT, 1, 8>(g, grid, s);
-    return many ? launch_skinny_one<FMT, 2, 4>(g, grid, s) : launch_skinny_one<FMT, 2, 8>(g, grid, s);
+    return many ? launch_rows_one<FMT, 2, 4>(g, grid, s) : launch_rows_one<FMT, 2, 8>(g, grid, s);
+}
+
+static int launch_skinny_rows(const xq_weight* w, const bf16_t* x, int64_t ldx, int64_t M, const void* lora_A, const void* lora_B,
+                              int lora_dtype, int r, int rp, float scaling, const bf16_t* bias, bf16_t* y, int64_t ldy,
+                              void* workspace, hipStream_t stream) {
+    const int64_t N = w->rows, K = w->cols;
+    float* su_part = (float*)workspace;
+    const int su_parts = (int)xq_cdiv(K, SU_KB);
+    if (rp) {
+        const int f32 = lora_dtype == XQ_DT_F32;
+        skinny_su_kernel<2><<<dim3(su_parts), SU_NW * 64, (size_t)SU_NW * 32 * 64 * 4, stream>>>(x, ldx, (int)M, (int)K, lora_A, f32, r, rp, su_part);
+    }
+    SkinnyRowsArgs g;
+    g.x = x; g.ldx = ldx; g.M = (int)M; g.N = (int)N; g.K = (int)K;
+    g.packed = (const uint8_t*)w->packed; g.scales = (const uint8_t*)w->scales; g.global_scale = w->global_scale;
+    g.group = w->group; g.scale_dtype = w->scale_dtype;
+    g.su_part = rp ? su_part : nullptr; g.su_parts = su_parts; g.su_scale = scaling; g.lora_B = rp ? lora_B : nullptr;
+    g.lora_f32 = lora_dtype == XQ_DT_F32; g.r = r; g.r_pad = rp;
+    g.bias = bias; g.y = y; g.ldy = ldy;
+    if (w->format == XQ_FMT_FP8) return launch_rows_cfg<XQ_FMT_FP8>(g, stream);
+    if (w->format == XQ_FMT_INT4) return launch_rows_cfg<XQ_FMT_INT4>(g, stream);
+    return launch_rows_cfg<XQ_FMT_NVFP4>(g, stream);
 }
 
 int launch_skinny(const xq_weight* w, const bf16_t* x, int64_t ldx, int64_t M, const void* lora_A, const void* lora_B,
@@ -389,33 +878,18 @@ int launch_skinny(const xq_weight* w, const bf16_t* x, int64_t ldx, int64_t M, c
     XQ_REQUIRE(workspace && xq_aligned(workspace, 256) && workspace_bytes >= skinny_workspace_bytes(M, N, K, rp),
                "xq_linear_fwd: workspace missing, misaligned or too small for the skinny path");
     XQ_REQUIRE(ldx % 8 == 0 && xq_aligned(x, 16) && xq_aligned(w->packed, 16), "xq_linear_fwd: operands must be 16-byte aligned");
+    XQ_REQUIRE(ldy % 4 == 0 && xq_aligned(y, 8), "xq_linear_fwd: output rows must be 8-byte aligned");
     XQ_REQUIRE(rp == 0 || xq_aligned(lora_A, 4) && xq_aligned(lora_B, 4), "xq_linear_fwd: LoRA factors must be 4-byte aligned");
-    float* su_part = (float*)workspace;
-    const int su_parts = (int)xq_cdiv(K, SU_KB);
-
-    int rc;
-    if (rp) {
-        const int f32 = lora_dtype == XQ_DT_F32;
-        if (M <= 32) skinny_su_kernel<1><<<dim3(su_parts), SU_NW * 64, (size_t)SU_NW * 16 * 64 * 4, stream>>>(x, ldx, (int)M, (int)K, lora_A, f32, r, rp, su_part);
-        else skinny_su_kernel<2><<<dim3(su_parts), SU_NW * 64, (size_t)SU_NW * 32 * 64 * 4, stream>>>(x, ldx, (int)M, (int)K, lora_A, f32, r, rp, su_part);
-        XQ_CHECK_LAUNCH("skinny_su");
-    }
-    SkinnyArgs g;
-    g.x = x; g.ldx = ldx; g.M = (int)M; g.N = (int)N; g.K = (int)K;
-    g.packed = (const uint8_t*)w->packed; g.scales = (const uint8_t*)w->scales; g.global_scale = w->global_scale;
-    g.group = w->group; g.scale_dtype = w->scale_dtype;
-    g.su_part = rp ? su_part : nullptr; g.su_parts = su_parts; g.su_scale = scaling; g.lora_B = rp ? lora_B : nullptr;
-    g.lora_f32 = lora_dtype == XQ_DT_F32; g.r = r; g.r_pad = rp;
-    g.bias = bias; g.y = y; g.ldy = ldy;
-    // algorithmic bytes: packed weight + scales + x + y (+ LoRA factors), for the roofline figure
+    // algorithmic bytes: packed weight + scales + x + y (+ LoRA factors), for the roofline figure; the timed
+    // region is the whole forward (both launches)
     const double wbytes = (double)xq_packed_bytes_per_expert(w) + (double)xq_scale_bytes_per_expert(w);
     const bool timed = xq_profile_mark_begin(stream, wbytes + 2.0 * M * K + 2.0 * M * N + 4.0 * r * (K + N));
-    if (w->format == XQ_FMT_FP8) rc = launch_skinny_cfg<XQ_FMT_FP8>(g, stream);
-    else if (w->format == XQ_FMT_INT4) rc = launch_skinny_cfg<XQ_FMT_INT4>(g, stream);
-    else rc = launch_skinny_cfg<XQ_FMT_NVFP4>(g, stream);
+    const int rc = M <= kSplitMaxM
+        ? launch_skinny_split(w, x, ldx, M, lora_A, lora_B, lora_dtype, r, rp, scaling, bias, y, ldy, workspace, stream)
+        : launch_skinny_rows(w, x, ldx, M, lora_A, lora_B, lora_dtype, r, rp, scaling, bias, y, ldy, workspace, stream);
     if (timed) xq_profile_mark_end(stream);
     if (rc) return rc;
-    XQ_CHECK_LAUNCH("skinny_kernel");
+    XQ_CHECK_LAUNCH("skinny forward");
     return XQ_OK;
 }
 
