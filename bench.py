@@ -216,7 +216,8 @@ def other_config(cfg: int, dev):
         return (step, total, True,
                 "configs[4]: skinny-M forward, M in {1,8,32,64} x {q 4096->4096, kv 4096->1024, gate/up 4096->12288, "
                 "down 12288->4096} x {int4, block_fp8}, r=16 (32 launches per step)",
-                "skinny_kernel<int4|fp8> (weight-streaming fused dequant-GEMV/GEMM)")
+                "skinny_split_kernel<int4|fp8> + skinny_epilogue_kernel (weight-streaming fused dequant-GEMV/GEMM; the "
+                "timed region is the whole forward, both launches)")
     if cfg == 5:
         # not a BASELINE config: the merge / re-quantise pass over configs[1]'s three block_fp8 weights (r = 32)
         from xorl_amd.functional import merge_dense, merge_requant_fp8
@@ -281,6 +282,8 @@ def main():
     ap.add_argument("--config", type=int, default=1,
                     help="BASELINE.json configs index; 1 (default) is the headline workload, the others report the "
                          "same JSON for their own workload (no CPU baseline)")
+    ap.add_argument("--no-graph", action="store_true",
+                    help="config 4 only: issue the 32 forwards of a step eagerly instead of replaying them as one HIP graph")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="before the warmup, run one plain 256 MiB -> 256 MiB elementwise copy so that a counter "
                          "run (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE) holds a kernel of known traffic to scale by")
@@ -369,15 +372,41 @@ def run_other(args, dev):
     L = _C.lib()
     if args.calibrate_copy:
         calibrate_copy(dev)
+    use_graph = args.config == 4 and not args.no_graph
+    if use_graph:
+        # the decode-regime step is 32 launch-bound forwards: replay it as one HIP graph (what a serving loop
+        # does).  Captured after an eager warm-up on a side stream; every replay runs the same kernels on the
+        # same buffers.  The per-forward roofline figure is taken from eager steps after the timed region,
+        # because event records inside a graph cannot be read back.
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(3):
+                step()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            step()
+        run = graph.replay
+        workload += "; the step is replayed as one HIP graph"
+    else:
+        run = step
     for _ in range(args.warmup):
-        step()
+        run()
     torch.cuda.synchronize()
-    L.xq_profile_enable(1)
+    if not use_graph:
+        L.xq_profile_enable(1)
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        step()
+        run()
     torch.cuda.synchronize()
     dt = (time.perf_counter() - t0) / args.steps
+    if use_graph:
+        L.xq_profile_enable(1)
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
     n, ms, fl = ctypes.c_int(0), ctypes.c_double(0), ctypes.c_double(0)
     _C.check(L.xq_profile_collect(ctypes.byref(n), ctypes.byref(ms), ctypes.byref(fl)))
     L.xq_profile_enable(0)

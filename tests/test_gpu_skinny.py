@@ -76,3 +76,37 @@ def test_skinny_split_plans(hip_device, fmt, N, K, M, r, bf16_factors):
         y0 = qlora_linear(x.to(hip_device), m._quant_weight(), None, None, 0, 0.0, None)
     ex0 = R.linear_fwd_bwd_exact(x, w_ref, torch.zeros(1, K), torch.zeros(N, 1), 0.0)
     assert R.max_rel_err(y0.cpu(), ex0["y"]) <= TOL
+
+
+def test_skinny_forward_under_hip_graph(hip_device):
+    """A captured decode step (several skinny forwards) replays to the eager result bit for bit, also with
+    eager work and synchronisations between replays."""
+    mods = [make_dense_module(fmt, N, K, 16, 32, seed=i, device=hip_device)[0]
+            for i, (fmt, N, K) in enumerate((("block_fp8", 1024, 4096), ("int4", 4096, 4096), ("nvfp4", 1024, 1024)))]
+    xs = [gen((M, m.in_features), 1.0, 500 + M, torch.bfloat16).to(hip_device) for M, m in zip((1, 8, 48), mods)]
+
+    def step():
+        with torch.no_grad():
+            return [m(x) for m, x in zip(mods, xs)]
+
+    eager = [y.clone() for y in step()]
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = step()
+    for rep in range(4):
+        for y in outs:
+            y.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        for y, e in zip(outs, eager):
+            assert torch.equal(y, e), rep
+        again = step()                      # eager work between replays
+        torch.cuda.synchronize()
+        for y, e in zip(again, eager):
+            assert torch.equal(y, e)

@@ -4,26 +4,24 @@
 //
 // Every byte of the packed weight is read from HBM exactly once, decoded in registers to the exact bf16
 // value of the reference decoder and fed to v_mfma_f32_32x32x16_bf16 against x fragments.  Two launches per
-// forward, no atomics, no zeroed buffers, fixed summation orders (deterministic).  Two organisations:
+// forward, no atomics, no zeroed buffers, fixed summation orders (deterministic):
 //
-//  M <= 32 -- K split across blocks (skinny_split_kernel + skinny_epilogue_kernel).  Partial outputs are
-//     tiny at these M, so the grid is (128-row block) x (K split): a block's four waves own 32 weight rows
-//     each and the same K range of at most four 128-element chunks.  ALL loads of a block -- its x slice and
-//     its whole weight tile -- are issued before anything is waited for, so the kernel is one memory round
+//  1. skinny_split_kernel: a grid of (128-row block) x (K split) tiles.  A block's four waves own 32 weight
+//     rows each and the same K range of at most four 128-element chunks.  ALL loads of a block -- its x slice
+//     and its whole weight tile -- are issued before anything is waited for, so the kernel is one memory round
 //     trip deep, and the number of K splits is chosen so that the whole grid is resident at once (four blocks
 //     per CU at M <= 16, three above).  Weight loads are coalesced (a load instruction covers whole rows of a
 //     chunk) and reach the MFMA layout through a wave-private XOR-swizzled LDS slab; the x slice
-//     [M, K range] goes through LDS once per block and is shared by the four waves.  Each block stores its fp32 partial tile to
-//     part[split][M][N]; the first `su_blocks` blocks carry no weight rows and compute the low-rank
-//     intermediate su = x . A^T for one K split each.  The epilogue sums the splits in order, adds bias and
-//     s * su . B^T in fp32 and rounds once to bf16.
+//     [rows, K range] goes through LDS once per block and is shared by the four waves, 32 rows at a time
+//     (M > 32 makes a second pass over the weight registers).  Each block stores its fp32 partial tile to
+//     part[split][M][N]; the first row of blocks carries no weight rows and computes the low-rank
+//     intermediate su = x . A^T for one K split each.
+//  2. skinny_epilogue_kernel: sums the splits in order, adds bias and s * su . B^T in fp32 and rounds once
+//     to bf16.
 //
-//  32 < M <= 64 -- K split across the waves of a block (skinny_su_kernel + skinny_rows_kernel).  Partial
-//     tiles would cost as much traffic as the weights here, so a block owns 32 weight rows and all of K; its
-//     waves (8, or 4 when there are more slabs than CUs) each stream 1/NW of K in batches through two
-//     register sets and the partial sums meet in LDS in wave order.  x is fetched with coalesced loads into
-//     wave-private padded LDS tiles.  The low-rank term needs one small launch before it (partial sums of
-//     x . A^T over K ranges of 512) and is added by the last wave under the latency of its first batch.
+// Measured per forward on an MI355X, launches back to back (block_fp8, r = 16): 4096->12288 (48 MiB) 15.5 us
+// at M = 1, 22 us at M = 32, 35 us at M = 64; 4096->1024 (4 MiB) 7.3 us at M = 1.  A kernel that only reads
+// the 48 MiB takes 8-9 us.
 #include "xq_common.h"
 #include "xq_lora.h"
 
@@ -54,24 +52,6 @@ struct SkinnyEpiArgs {
     const void* lora_B;        // [N, r] fp32 or bf16
     int32_t lora_f32, r, r_pad;
     float su_scale;
-    const bf16_t* bias;
-    bf16_t* y;
-    int64_t ldy;
-};
-
-struct SkinnyRowsArgs {
-    const bf16_t* x;
-    int64_t ldx;
-    int32_t M, N, K;
-    const uint8_t* packed;
-    const uint8_t* scales;
-    const float* global_scale;
-    int32_t group, scale_dtype;
-    const float* su_part;      // [su_parts][M, r_pad] fp32 partial sums of x . A^T (unscaled) or NULL
-    int32_t su_parts;
-    float su_scale;
-    const void* lora_B;        // [N, r] fp32 or bf16
-    int32_t lora_f32, r, r_pad;
     const bf16_t* bias;
     bf16_t* y;
     int64_t ldy;
@@ -127,17 +107,21 @@ __device__ __forceinline__ bf16x8 factor_frag(const void* base, int64_t idx, boo
 }
 
 // One block = 128 weight rows x one K split (or, for the leading su blocks, the x . A^T part of one split).
+// MR = 16, 32 or 64 bounds M; at MR = 64 the x rows go through LDS 32 at a time (two passes over the weight
+// registers), so that three blocks still fit a CU.
 template <int FMT, int MR, int NCH>
 __global__ void __launch_bounds__(256, MR == 16 ? 4 : 3) skinny_split_kernel(SkinnyArgs g) {
-    constexpr int MT = 1;                              // one 32-column MFMA tile of x rows (M <= MR <= 32)
+    constexpr int TR = MR < 32 ? MR : 32;              // x rows staged at a time
+    constexpr int NPASS = MR / TR;
     // Pin every argument in scalar registers here: otherwise the argument loads are placed lazily, each batch
     // with its own wait, and several memory round trips pass before the first weight load is issued.
     asm volatile("" ::"s"(g.x), "s"(g.ldx), "s"(g.M), "s"(g.N), "s"(g.K), "s"(g.packed), "s"(g.scales), "s"(g.global_scale),
                  "s"(g.group), "s"(g.scale_dtype), "s"(g.splits), "s"(g.su_blocks), "s"(g.chunk_q), "s"(g.chunk_rem),
                  "s"(g.xp), "s"(g.partial), "s"(g.su_part), "s"(g.lora_A), "s"(g.lora_f32), "s"(g.r), "s"(g.r_pad));
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    bf16_t* xs = (bf16_t*)smem;                                  // [M rows][xp]; fragment rows >= M read row 0: they feed
-    const int XP = g.xp;                                         // only output columns >= M, which are never stored
+    bf16_t* xs = (bf16_t*)smem;                                  // [min(M, 32) rows][xp]; fragment rows past M read row 0:
+    const int XP = g.xp;                                         // they feed only output columns >= M, which are never stored
+    const int xrows = g.M < 32 ? g.M : 32;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int fr = lane & 31, fh = lane >> 5;
@@ -156,42 +140,39 @@ __global__ void __launch_bounds__(256, MR == 16 ? 4 : 3) skinny_split_kernel(Ski
     const int c_end = c_begin + nch;
     const int k_begin = c_begin << 7;
 
-    // ---- x slice [M][nch*128]: coalesced 16-byte pieces, row-major over the block's threads.  Every load below
-    // is unconditional (rows and chunks past the end are clamped onto valid ones and their data ignored): with
-    // no branches between the loads and their uses the waits count exactly, so the x slice is staged and each
-    // weight chunk decoded while the chunks behind it are still in flight.
-    constexpr int XL = MR * NCH / 16;                            // pieces per thread at most: MR rows x NCH*16 / 256
-    const int ppr = nch << 4;                                    // pieces per row: 16, 32, 48 or 64
-    const int q256 = nch == 3 ? 5 : 16 >> (nch >> 1), r256 = nch == 3 ? 16 : 0;   // 256 = q256 * ppr + r256
-    const int row0 = nch == 3 ? ((tid >> 4) * 11) >> 5 : tid >> (4 + (nch >> 1)); // tid / ppr
-    const int col0 = tid - row0 * ppr;
+    // ---- x slice [rows of pass h][nch*128]: coalesced 16-byte pieces, row-major over the block's threads.  Every
+    // load of this kernel is unconditional (rows and chunks past the end are clamped onto valid ones and their
+    // data ignored): with no branches between the loads and their uses the waits count exactly, so the x slice
+    // is staged and each weight chunk decoded while the chunks behind it are still in flight.
+    // Thread t owns column piece t % (NCH*16) of rows t / (NCH*16) + i * (16/NCH); pieces past the split's own
+    // nch*16 columns (a split shorter than NCH chunks) are loaded clamped and never stored.
+    constexpr int XL = TR * NCH / 16;                            // pieces per thread: TR rows x NCH*16 / 256
+    constexpr int CPR = NCH * 16, RSTEP = 16 / NCH;              // column pieces per row, rows per step
+    const int ppr = nch << 4;                                    // pieces of a row that belong to this split
     u32x4 xr[XL];
-    {
-        int row = row0, col = col0;
+    auto load_x = [&](int h, int t) {
+        const int col = t % CPR < ppr ? t % CPR : ppr - 1;
 #pragma unroll
         for (int i = 0; i < XL; ++i) {
-            const int rc = row < g.M ? row : g.M - 1;
-            xr[i] = *(const u32x4*)(g.x + (int64_t)rc * g.ldx + k_begin + col * 8);
-            col += r256;
-            row += q256;
-            if (col >= ppr) { col -= ppr; ++row; }
+            const int row = h * 32 + t / CPR + i * RSTEP;
+            xr[i] = *(const u32x4*)(g.x + (int64_t)(row < g.M ? row : g.M - 1) * g.ldx + k_begin + col * 8);
         }
-    }
-    int xrow[MT];                                                // LDS row of this lane's x fragments
-#pragma unroll
-    for (int i = 0; i < MT; ++i) xrow[i] = i * 32 + fr < g.M ? i * 32 + fr : 0;
-    auto stage_x = [&]() {
-        int row = row0, col = col0;
-#pragma unroll
-        for (int i = 0; i < XL; ++i) {
-            if (row < g.M) *(u32x4*)(xs + row * XP + col * 8) = xr[i];
-            col += r256;
-            row += q256;
-            if (col >= ppr) { col -= ppr; ++row; }
-        }
-        // block barrier on the LDS writes only: __syncthreads() would also wait for every weight load in flight
-        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     };
+    // block barrier on LDS traffic only: __syncthreads() would also wait for every weight load in flight
+    auto lds_barrier = [&]() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+    auto stage_x = [&](int h, int t) {
+        const int col = t % CPR;
+#pragma unroll
+        for (int i = 0; i < XL; ++i) {
+            const int row = t / CPR + i * RSTEP;
+            if (col < ppr && h * 32 + row < g.M) *(u32x4*)(xs + row * XP + col * 8) = xr[i];
+        }
+        lds_barrier();
+    };
+    // a value the optimiser cannot see through: index arithmetic derived from it inside a loop is redone per
+    // iteration instead of being hoisted into (and spilling) registers held across the whole loop
+    auto opaque = [](int v) { asm volatile("" : "+v"(v)); return v; };
+    load_x(0, tid);
 
     if (su_block) {
         // su part of this split, D[rank][m] (ranks >= r are zero): wave w takes the k16 steps t = w, w+4, ...; the
@@ -200,7 +181,7 @@ __global__ void __launch_bounds__(256, MR == 16 ? 4 : 3) skinny_split_kernel(Ski
         // with the x slice.
         const int steps = nch << 3;
         float* out = g.su_part + (int64_t)split * g.M * g.r_pad;
-        float* red = (float*)(smem + (size_t)g.M * XP * 2);        // [4 waves][16 regs][64 lanes]
+        float* red = (float*)(smem + (size_t)xrows * XP * 2);      // [4 waves][16 regs][64 lanes]
         u32x4 ar[2 * NCH][2];
         auto load_a = [&](int jt) {
             const int rrow = jt * 32 + fr;
@@ -217,7 +198,6 @@ __global__ void __launch_bounds__(256, MR == 16 ? 4 : 3) skinny_split_kernel(Ski
             }
         };
         load_a(0);
-        stage_x();
         for (int jt = 0; jt < ((g.r_pad + 31) >> 5); ++jt) {
             if (jt > 0) load_a(jt);
             const bool rvalid = jt * 32 + fr < g.r;
@@ -234,29 +214,40 @@ __global__ void __launch_bounds__(256, MR == 16 ? 4 : 3) skinny_split_kernel(Ski
                 if (!rvalid || wave + 4 * u >= steps) v = u32x4{0, 0, 0, 0};
                 af[u] = __builtin_bit_cast(bf16x8, v);
             }
-            f32x16 sacc;
+#pragma unroll 1
+            for (int h = 0; h < NPASS; ++h) {
+                if (h * 32 < g.M) {
+                    // the x tile in LDS is current only for a single pass and the first rank tile
+                    if (NPASS > 1 || jt == 0) {
+                        if (h > 0 || jt > 0) load_x(h, tid);       // earlier reads of the tile are behind two barriers
+                        stage_x(h, tid);
+                    }
+                    const int xrow = h * 32 + fr < g.M ? fr : 0;
+                    f32x16 sacc;
 #pragma unroll
-            for (int q = 0; q < 16; ++q) sacc[q] = 0.0f;
+                    for (int q = 0; q < 16; ++q) sacc[q] = 0.0f;
 #pragma unroll
-            for (int u = 0; u < 2 * NCH; ++u) {
-                const int t = wave + 4 * u;
-                if (t < steps) {
-                    const bf16x8 xf = *(const bf16x8*)(xs + xrow[0] * XP + t * 16 + fh * 8);
-                    sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[u], xf, sacc, 0, 0, 0);
+                    for (int u = 0; u < 2 * NCH; ++u) {
+                        const int t = wave + 4 * u;
+                        if (t < steps) {
+                            const bf16x8 xf = *(const bf16x8*)(xs + xrow * XP + t * 16 + fh * 8);
+                            sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[u], xf, sacc, 0, 0, 0);
+                        }
+                    }
+                    __syncthreads();   // the previous sums have been read
+#pragma unroll
+                    for (int q = 0; q < 16; ++q) red[(wave * 16 + q) * 64 + lane] = sacc[q];
+                    __syncthreads();
+                    // wave w sums register quad w of every lane: ranks jt*32 + 8w + 4*fh .. +3 of row m = 32h + fr
+                    f32x4 v = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                    for (int ww = 0; ww < 4; ++ww)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) v[e] += red[(ww * 16 + wave * 4 + e) * 64 + lane];
+                    const int j0 = jt * 32 + 8 * wave + 4 * fh, m = h * 32 + fr;
+                    if (m < g.M && j0 < g.r_pad) *(f32x4*)(out + (int64_t)m * g.r_pad + j0) = v;
                 }
             }
-            __syncthreads();   // the previous rank tile's sums have been read
-#pragma unroll
-            for (int q = 0; q < 16; ++q) red[(wave * 16 + q) * 64 + lane] = sacc[q];
-            __syncthreads();
-            // wave w sums register quad w of every lane: ranks jt*32 + 8w + 4*fh .. +3 of row m = fr
-            f32x4 v = {0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-            for (int ww = 0; ww < 4; ++ww)
-#pragma unroll
-                for (int e = 0; e < 4; ++e) v[e] += red[(ww * 16 + wave * 4 + e) * 64 + lane];
-            const int j0 = jt * 32 + 8 * wave + 4 * fh;
-            if (fr < g.M && j0 < g.r_pad) *(f32x4*)(out + (int64_t)fr * g.r_pad + j0) = v;
         }
         return;
     }
@@ -302,7 +293,6 @@ __global__ void __launch_bounds__(256, MR == 16 ? 4 : 3) skinny_split_kernel(Ski
             }
         }
     }
-    stage_x();
 
     // ---- decode + multiply: D[n][m] += deq(W)[n][k] x[m][k].  Each chunk's slab goes through a wave-private LDS
     // staging area (XOR-swizzled 16-byte pieces: writes and fragment reads are conflict free) to reach the
@@ -310,71 +300,74 @@ __global__ void __launch_bounds__(256, MR == 16 ? 4 : 3) skinny_split_kernel(Ski
     // t = 2u+v covers k = 32u + 16*fh + 8v .. +7 of the chunk; the x fragments use the same map.  LDS operations
     // of one wave execute in order, so the slab is reused chunk after chunk without barriers.
     const float gsc = FMT == XQ_FMT_NVFP4 ? g.global_scale[0] : 1.0f;
-    unsigned char* wst = smem + (size_t)g.M * XP * 2 + wave * (PPR * 32 * 16);
-    f32x16 acc[MT];
+    unsigned char* wst = smem + (size_t)xrows * XP * 2 + wave * (PPR * 32 * 16);
 #pragma unroll
-    for (int i = 0; i < MT; ++i)
-#pragma unroll
-        for (int q = 0; q < 16; ++q) acc[i][q] = 0.0f;
-#pragma unroll
-    for (int c = 0; c < NCH; ++c) {
-        if (c < nch) {
-#pragma unroll
-            for (int i = 0; i < NLOAD; ++i) {
-                const int rl = RPI * i + lrow;
-                const int sw = FMT == XQ_FMT_FP8 ? (rl >> 1) & 7 : (rl >> 2) & 3;
-                *(u32x4*)(wst + (rl * PPR + (lpiece ^ sw)) * 16) = w[c][i];
+    for (int h = 0; h < NPASS; ++h) {
+        if (h * 32 < g.M) {
+            const int tv = h > 0 ? opaque(tid) : tid;
+            if (h > 0) {
+                lds_barrier();                         // every wave has read its fragments of the previous pass
+                load_x(h, tv);
             }
-            __builtin_amdgcn_wave_barrier();
-            const int kc = (c_begin + c) * 128;
+            stage_x(h, tv);
+            const int lv = tv & 63, fr = lv & 31, fh = lv >> 5, lrow = lv / PPR, lpiece = lv % PPR;
+            const int xrow = h * 32 + fr < g.M ? fr : 0;
+            f32x16 acc;
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                uint32_t f[4];
-                if (FMT == XQ_FMT_FP8) {
-                    const u32x4 t = *(const u32x4*)(wst + (fr * 8 + ((2 * u + fh) ^ ((fr >> 1) & 7))) * 16);
-                    f[0] = t[0]; f[1] = t[1]; f[2] = t[2]; f[3] = t[3];
-                } else {
-                    const u32x2 t = *(const u32x2*)(wst + (fr * 4 + (u ^ ((fr >> 2) & 3))) * 16 + fh * 8);
-                    f[0] = t[0]; f[1] = t[1];
-                }
+            for (int q = 0; q < 16; ++q) acc[q] = 0.0f;
 #pragma unroll
-                for (int v = 0; v < 2; ++v) {
-                    bf16x8 wf;
-                    if (FMT == XQ_FMT_FP8) {
-                        wf = decode8<FMT>(f[2 * v], f[2 * v + 1], __uint_as_float(sc[c][0]), 0.0f);
-                    } else if (FMT == XQ_FMT_INT4) {
-                        float sv;
-                        if (int4_small_group) sv = load_scale(g.scales, ((int64_t)n * g.K + kc + 32 * u + 16 * fh + 8 * v) / g.group, g.scale_dtype);
-                        else sv = g.scale_dtype == XQ_SCALE_F32 ? __uint_as_float(sc[c][0]) : __uint_as_float(sc[c][0] << 16);
-                        wf = decode8<FMT>(f[v], 0u, sv, -8.0f * sv);
-                    } else {
-                        float sv;   // block scale 2u + fh of the chunk
-                        if (g.scale_dtype == XQ_SCALE_E4M3) sv = e4m3_to_f32((uint8_t)(sc[c][u >> 1] >> (8 * (2 * (u & 1) + fh))));
-                        else sv = __uint_as_float(sc[c][u]);
-                        wf = decode8<FMT>(f[v], 0u, sv * gsc, 0.0f);
+            for (int c = 0; c < NCH; ++c) {
+                if (c < nch) {
+#pragma unroll
+                    for (int i = 0; i < NLOAD; ++i) {
+                        const int rl = RPI * i + lrow;
+                        const int sw = FMT == XQ_FMT_FP8 ? (rl >> 1) & 7 : (rl >> 2) & 3;
+                        *(u32x4*)(wst + (rl * PPR + (lpiece ^ sw)) * 16) = w[c][i];
                     }
+                    __builtin_amdgcn_wave_barrier();
+                    const int kc = (c_begin + c) * 128;
 #pragma unroll
-                    for (int i = 0; i < MT; ++i) {
-                        const bf16x8 xf = *(const bf16x8*)(xs + xrow[i] * XP + c * 128 + 32 * u + 16 * fh + 8 * v);
-                        acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf, xf, acc[i], 0, 0, 0);
+                    for (int u = 0; u < 4; ++u) {
+                        uint32_t f[4];
+                        if (FMT == XQ_FMT_FP8) {
+                            const u32x4 t = *(const u32x4*)(wst + (fr * 8 + ((2 * u + fh) ^ ((fr >> 1) & 7))) * 16);
+                            f[0] = t[0]; f[1] = t[1]; f[2] = t[2]; f[3] = t[3];
+                        } else {
+                            const u32x2 t = *(const u32x2*)(wst + (fr * 4 + (u ^ ((fr >> 2) & 3))) * 16 + fh * 8);
+                            f[0] = t[0]; f[1] = t[1];
+                        }
+#pragma unroll
+                        for (int v = 0; v < 2; ++v) {
+                            bf16x8 wf;
+                            if (FMT == XQ_FMT_FP8) {
+                                wf = decode8<FMT>(f[2 * v], f[2 * v + 1], __uint_as_float(sc[c][0]), 0.0f);
+                            } else if (FMT == XQ_FMT_INT4) {
+                                float sv;
+                                if (int4_small_group) sv = load_scale(g.scales, ((int64_t)n * g.K + kc + 32 * u + 16 * fh + 8 * v) / g.group, g.scale_dtype);
+                                else sv = g.scale_dtype == XQ_SCALE_F32 ? __uint_as_float(sc[c][0]) : __uint_as_float(sc[c][0] << 16);
+                                wf = decode8<FMT>(f[v], 0u, sv, -8.0f * sv);
+                            } else {
+                                float sv;   // block scale 2u + fh of the chunk
+                                if (g.scale_dtype == XQ_SCALE_E4M3) sv = e4m3_to_f32((uint8_t)(sc[c][u >> 1] >> (8 * (2 * (u & 1) + fh))));
+                                else sv = __uint_as_float(sc[c][u]);
+                                wf = decode8<FMT>(f[v], 0u, sv * gsc, 0.0f);
+                            }
+                            const bf16x8 xf = *(const bf16x8*)(xs + xrow * XP + c * 128 + 32 * u + 16 * fh + 8 * v);
+                            acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf, xf, acc, 0, 0, 0);
+                        }
                     }
+                    __builtin_amdgcn_wave_barrier();
                 }
             }
-            __builtin_amdgcn_wave_barrier();
-        }
-    }
-
-    // ---- fp32 partial tile: lane (m = fr) holds 4 consecutive weight rows per register quad
-    float* out = g.partial + (int64_t)split * g.M * g.N;
-    const int nb = nbase;
+            // fp32 partial tile: lane (m = 32h + fr) holds 4 consecutive weight rows per register quad
+            float* out = g.partial + (int64_t)split * g.M * g.N;
+            const int m = h * 32 + fr;
 #pragma unroll
-    for (int i = 0; i < MT; ++i) {
-        const int m = i * 32 + fr;
-#pragma unroll
-        for (int q4 = 0; q4 < 4; ++q4) {
-            const int nn = nb + 8 * q4 + 4 * fh;
-            if (m < g.M && nn < g.N)   // N % 16 == 0: groups of 4 columns are all in or all out
-                *(f32x4*)(out + (int64_t)m * g.N + nn) = f32x4{acc[i][q4 * 4], acc[i][q4 * 4 + 1], acc[i][q4 * 4 + 2], acc[i][q4 * 4 + 3]};
+            for (int q4 = 0; q4 < 4; ++q4) {
+                const int nn = nbase + 8 * q4 + 4 * fh;
+                if (m < g.M && nn < g.N)   // N % 16 == 0: groups of 4 columns are all in or all out
+                    *(f32x4*)(out + (int64_t)m * g.N + nn) = f32x4{acc[q4 * 4], acc[q4 * 4 + 1], acc[q4 * 4 + 2], acc[q4 * 4 + 3]};
+            }
         }
     }
 }
@@ -476,254 +469,7 @@ __global__ void __launch_bounds__(256) skinny_epilogue_kernel(SkinnyEpiArgs g) {
     *(u32x2*)(g.y + (int64_t)m * g.ldy + n) = u32x2{pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3])};
 }
 
-// One block = 32 weight rows x the whole K, NW waves each streaming 1/NW of K (in-block
-// split-K: no atomics, no fences, fixed summation order).  x fragments are read from global
-// memory (coalesced, see the top of the file) together with the codes of the same batch.
-template <int FMT, int MT, int NW>
-__global__ void __launch_bounds__(NW * 64) skinny_rows_kernel(SkinnyRowsArgs g) {
-    extern __shared__ __attribute__((aligned(16))) float red[];   // [NW waves][MT*16 regs][64 lanes]
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: keeps the K-range loop on scalar branches
-    const int fr = lane & 31, fh = lane >> 5;
-    const int n0 = blockIdx.x * 32;
-    constexpr int EB = FMT == XQ_FMT_FP8 ? 1 : 2;      // elements per byte
-    constexpr int NLOAD = FMT == XQ_FMT_FP8 ? 4 : 2;   // 16-byte loads per lane per 128-k chunk
-    constexpr int BC = 2 / MT;                         // chunks per batch (per register set)
-    constexpr int NSC = FMT == XQ_FMT_NVFP4 ? 4 : 1;   // scale registers per chunk
-    const float gsc = FMT == XQ_FMT_NVFP4 ? g.global_scale[0] : 1.0f;
-    // int4 groups shorter than a lane's 64-element run are looked up per 8 elements at use
-    const bool int4_small_group = FMT == XQ_FMT_INT4 && g.group < 64;
-
-    int n = n0 + fr;
-    n = n < g.N ? n : g.N - 1;
-    const uint8_t* wrow = g.packed + ((int64_t)n * g.K + fh * 64) / EB;
-    // x chunk tile of this wave: [MT*32 rows][128 k] bf16, rows padded to 272 B so that the 16 lanes
-    // of a b128 read phase (consecutive rows, same column piece) fall on distinct banks.  Rows >= M are
-    // never written: they feed only output columns >= M, which are never stored.
-    constexpr int XP = 136;                                     // row pitch in bf16 elements
-    bf16_t* xs = (bf16_t*)red + wave * (MT * 32 * XP);
-    const int xrow = lane >> 4, xpiece = lane & 15;             // coalesced fetch: 4 rows x 16 pieces per instruction
-    const bf16_t* xg = g.x + (int64_t)xrow * g.ldx + xpiece * 8;
-    const int64_t xstep = 4 * g.ldx;
-    const int mrows = g.M;
-
-    f32x16 acc[MT];
-#pragma unroll
-    for (int i = 0; i < MT; ++i)
-#pragma unroll
-        for (int q = 0; q < 16; ++q) acc[i][q] = 0.0f;
-
-    const int ct = g.K >> 7;                                   // 128-element chunks in K
-    const int c_begin = (ct * wave) / NW, c_end = (ct * (wave + 1)) / NW;
-
-    struct Batch {
-        u32x4 w[BC][NLOAD];
-        uint32_t sc[BC][NSC];
-        u32x4 xr[BC][MT * 8];
-    };
-    auto issue = [&](Batch& B, int c0) {
-#pragma unroll
-        for (int b = 0; b < BC; ++b) {
-            if (c0 + b < c_end) {
-                const int c = c0 + b, k0 = c * 128 + fh * 64;
-#pragma unroll
-                for (int i = 0; i < NLOAD; ++i) B.w[b][i] = *(const u32x4*)(wrow + (int64_t)c * (128 / EB) + i * 16);
-                if (FMT == XQ_FMT_FP8) B.sc[b][0] = ((const uint32_t*)g.scales)[(n >> 7) * ((g.K + 127) >> 7) + (k0 >> 7)];
-                else if (FMT == XQ_FMT_INT4) {
-                    if (!int4_small_group) {
-                        const int64_t si = ((int64_t)n * g.K + k0) / g.group;
-                        B.sc[b][0] = g.scale_dtype == XQ_SCALE_F32 ? ((const uint32_t*)g.scales)[si] : ((const uint16_t*)g.scales)[si];
-                    }
-                } else {
-                    const int64_t si = ((int64_t)n * g.K + k0) >> 4;   // 4 scales of the 64-element run
-                    if (g.scale_dtype == XQ_SCALE_E4M3) B.sc[b][0] = *(const uint32_t*)(g.scales + si);
-                    else {
-                        const u32x4 t = *(const u32x4*)((const float*)g.scales + si);
-#pragma unroll
-                        for (int j = 0; j < NSC; ++j) B.sc[b][j] = t[j];
-                    }
-                }
-#pragma unroll
-                for (int j = 0; j < MT * 8; ++j)
-                    if (j * 4 + xrow < mrows) B.xr[b][j] = *(const u32x4*)(xg + j * xstep + c * 128);   // lanes of rows >= M keep stale data
-            }
-        }
-    };
-    auto compute = [&](Batch& B, int c0) {
-#pragma unroll
-        for (int b = 0; b < BC; ++b) {
-            if (c0 + b < c_end) {
-                const int c = c0 + b, k0 = c * 128 + fh * 64;
-                // x tile -> LDS (LDS operations of one wave execute in order: the previous chunk's fragment
-                // reads are ahead of these writes)
-#pragma unroll
-                for (int j = 0; j < MT * 8; ++j)
-                    if (j * 4 < mrows) *(u32x4*)(xs + (j * 4 + xrow) * XP + xpiece * 8) = B.xr[b][j];
-#pragma unroll
-                for (int t = 0; t < 8; ++t) {
-                    bf16x8 wf;
-                    if (FMT == XQ_FMT_FP8) {
-                        wf = decode8<FMT>(B.w[b][t >> 1][(t & 1) * 2], B.w[b][t >> 1][(t & 1) * 2 + 1], __uint_as_float(B.sc[b][0]), 0.0f);
-                    } else if (FMT == XQ_FMT_INT4) {
-                        float s;
-                        if (int4_small_group) s = load_scale(g.scales, ((int64_t)n * g.K + k0 + t * 8) / g.group, g.scale_dtype);
-                        else s = g.scale_dtype == XQ_SCALE_F32 ? __uint_as_float(B.sc[b][0]) : __uint_as_float(B.sc[b][0] << 16);
-                        wf = decode8<FMT>(B.w[b][t >> 2][t & 3], 0u, s, -8.0f * s);
-                    } else {
-                        float s;
-                        if (g.scale_dtype == XQ_SCALE_E4M3) s = e4m3_to_f32((uint8_t)(B.sc[b][0] >> (8 * (t >> 1))));
-                        else s = __uint_as_float(B.sc[b][(t >> 1) % NSC]);
-                        wf = decode8<FMT>(B.w[b][t >> 2][t & 3], 0u, s * gsc, 0.0f);
-                    }
-#pragma unroll
-                    for (int i = 0; i < MT; ++i) {
-                        const bf16x8 xf = *(const bf16x8*)(xs + (i * 32 + fr) * XP + fh * 64 + t * 8);
-                        acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf, xf, acc[i], 0, 0, 0);
-                    }
-                }
-            }
-        }
-    };
-
-    // two register sets: the next batch is in flight while the current one is multiplied
-    Batch B0, B1;
-    int c = c_begin;
-    if (c < c_end) issue(B0, c);
-
-    // ---- low-rank side term (last wave), under the latency of the first batch: acc = (s * su) . B^T with
-    // su = x . A^T summed from skinny_su_kernel's parts
-    if (g.r_pad > 0 && wave == NW - 1) {
-#pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
-            if (ks < (g.r_pad >> 4)) {
-                const int j0 = ks * 16 + fh * 8;   // first rank index of this lane's 8
-                const bf16x8 lb = factor_frag(g.lora_B, (int64_t)n * g.r + j0, g.lora_f32 != 0, g.r - j0);
-#pragma unroll
-                for (int i = 0; i < MT; ++i) {
-                    const int m = i * 32 + fr;
-                    const float* sp = g.su_part + (int64_t)(m < g.M ? m : 0) * g.r_pad + j0;
-                    f32x4 s0 = {0.0f, 0.0f, 0.0f, 0.0f}, s1 = s0;
-#pragma unroll 4
-                    for (int kb = 0; kb < g.su_parts; ++kb) {   // fixed order
-                        s0 += *(const f32x4*)(sp + (int64_t)kb * g.M * g.r_pad);
-                        s1 += *(const f32x4*)(sp + (int64_t)kb * g.M * g.r_pad + 4);
-                    }
-                    uint32_t o[4];
-#pragma unroll
-                    for (int e = 0; e < 2; ++e) {
-                        o[e] = pack_bf16x2(s0[2 * e] * g.su_scale, s0[2 * e + 1] * g.su_scale);
-                        o[2 + e] = pack_bf16x2(s1[2 * e] * g.su_scale, s1[2 * e + 1] * g.su_scale);
-                    }
-                    u32x4 r = {o[0], o[1], o[2], o[3]};
-                    acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lb, __builtin_bit_cast(bf16x8, r), acc[i], 0, 0, 0);
-                }
-            }
-        }
-    }
-
-    while (c < c_end) {
-        if (c + BC < c_end) issue(B1, c + BC);
-        compute(B0, c);
-        c += BC;
-        if (c >= c_end) break;
-        if (c + BC < c_end) issue(B0, c + BC);
-        compute(B1, c);
-        c += BC;
-    }
-
-    // ---- cross-wave reduction through LDS, summed in wave order (the x tiles are dead by now)
-    constexpr int R = MT * 16;
-    __syncthreads();
-#pragma unroll
-    for (int i = 0; i < MT; ++i)
-#pragma unroll
-        for (int q = 0; q < 16; ++q) red[(wave * R + i * 16 + q) * 64 + lane] = acc[i][q];
-    __syncthreads();
-    // quads of 4 consecutive output columns: quad id = (i, q4); wave w takes quads w, w+NW, ...
-    for (int quad = wave; quad < MT * 4; quad += NW) {
-        const int i = quad >> 2, q4 = quad & 3;
-        float v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-        for (int w = 0; w < NW; ++w)
-#pragma unroll
-            for (int e = 0; e < 4; ++e) v[e] += red[(w * R + i * 16 + q4 * 4 + e) * 64 + lane];
-        const int m = i * 32 + fr, nn = n0 + 8 * q4 + 4 * fh;
-        if (m < g.M && nn < g.N) {   // N % 16 == 0: groups of 4 columns are all in or all out
-            if (g.bias) {
-#pragma unroll
-                for (int e = 0; e < 4; ++e) v[e] += bf16_to_f32(g.bias[nn + e]);
-            }
-            *(u32x2*)(g.y + (int64_t)m * g.ldy + nn) = u32x2{pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
-        }
-    }
-}
-
-// Partial sums of su = x[M, K] . A[r, K]^T (fp32, unscaled): block kb covers K range
-// [kb*SU_KB, (kb+1)*SU_KB) with its 8 waves (one eighth each, summed through LDS in wave order) and
-// writes part[kb][M][r_pad]; columns r..r_pad-1 are zero.  skinny_rows_kernel adds the parts in block
-// order, so the low-rank term is deterministic and needs no zeroed buffer and no atomics.
-constexpr int SU_KB = 512, SU_NW = 8;
-template <int MT>
-__global__ void __launch_bounds__(SU_NW * 64) skinny_su_kernel(const bf16_t* x, int64_t ldx, int M, int K, const void* A,
-                                                              int a_f32, int r, int r_pad, float* part) {
-    extern __shared__ __attribute__((aligned(16))) float red[];   // [SU_NW][MT*16][64]
-    const int tid = threadIdx.x, lane = tid & 63, fr = lane & 31, fh = lane >> 5;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int kb0 = blockIdx.x * SU_KB;
-    constexpr int SPW = SU_KB / 16 / SU_NW;   // k16 steps per wave
-    float* out = part + (int64_t)blockIdx.x * M * r_pad;
-    const int nt = (r_pad + 31) >> 5;
-    const bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
-    for (int j = 0; j < nt; ++j) {
-        const int rrow = j * 32 + fr;
-        const bool rvalid = rrow < r;
-        f32x16 acc[MT];
-#pragma unroll
-        for (int i = 0; i < MT; ++i)
-#pragma unroll
-            for (int q = 0; q < 16; ++q) acc[i][q] = 0.0f;
-#pragma unroll
-        for (int s0 = 0; s0 < SPW; s0 += 4) {
-            bf16x8 af[4], xf[MT][4];
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {     // the loads of four steps are issued together
-                const int kk = kb0 + (wave * SPW + s0 + u) * 16;
-                const bool kvalid = kk < K;   // wave-uniform (K % 16 == 0)
-                const int k = kk + fh * 8;
-                af[u] = kvalid ? factor_frag(A, (int64_t)(rvalid ? rrow : 0) * K + k, a_f32 != 0, rvalid ? 8 : 0) : z;
-#pragma unroll
-                for (int i = 0; i < MT; ++i) {
-                    const int m = i * 32 + fr;
-                    xf[i][u] = kvalid ? *(const bf16x8*)(x + (int64_t)(m < M ? m : 0) * ldx + k) : z;
-                }
-            }
-#pragma unroll
-            for (int u = 0; u < 4; ++u)
-#pragma unroll
-                for (int i = 0; i < MT; ++i) acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[u], xf[i][u], acc[i], 0, 0, 0);   // D[rank][m]
-        }
-        constexpr int R = MT * 16;
-        __syncthreads();   // the previous rank tile's sums have been read
-#pragma unroll
-        for (int i = 0; i < MT; ++i)
-#pragma unroll
-            for (int q = 0; q < 16; ++q) red[(wave * R + i * 16 + q) * 64 + lane] = acc[i][q];
-        __syncthreads();
-        for (int idx = wave; idx < R; idx += SU_NW) {   // register idx = (i, q) of every lane
-            float v = 0.0f;
-#pragma unroll
-            for (int w = 0; w < SU_NW; ++w) v += red[(w * R + idx) * 64 + lane];
-            const int i = idx >> 4, q = idx & 15;
-            const int m = i * 32 + fr, rr = j * 32 + (q & 3) + 4 * fh + 8 * (q >> 2);
-            if (m < M && rr < r_pad) out[(int64_t)m * r_pad + rr] = v;
-        }
-    }
-}
-
-
 static inline int64_t al256(int64_t b) { return (b + 255) & ~(int64_t)255; }
-
-constexpr int kSplitMaxM = 32;   // rows up to which the K-split-across-blocks organisation is used
 
 // K splits for the split organisation: at most four chunks per split; more splits until the grid holds
 // about two blocks per CU, never more than the 1024 blocks that are resident at once (four per CU).
@@ -741,11 +487,8 @@ static SkinnyPlan skinny_plan(int64_t N, int64_t K) {
 
 int64_t skinny_workspace_bytes(int64_t M, int64_t N, int64_t K, int r_pad) {
     const int rp = r_pad ? r_pad : 16;
-    if (M <= kSplitMaxM) {
-        const SkinnyPlan p = skinny_plan(N, K);
-        return al256((int64_t)p.splits * M * N * 4) + al256((int64_t)p.splits * M * rp * 4) + 256;
-    }
-    return al256(xq_cdiv(K, SU_KB) * M * rp * 4) + 256;
+    const SkinnyPlan p = skinny_plan(N, K);
+    return al256((int64_t)p.splits * M * N * 4) + al256((int64_t)p.splits * M * rp * 4) + 256;
 }
 
 bool skinny_supported(const xq_weight* w, int64_t M) {
@@ -757,12 +500,12 @@ bool skinny_supported(const xq_weight* w, int64_t M) {
     return true;
 }
 
-// ---------------------------------------------------------------- M <= 32
 template <int FMT, int NCH>
 static int launch_split_one(const SkinnyArgs& g, dim3 grid, size_t lds, hipStream_t s) {
     // at most 32 rows of 1040 B + the slabs = 49 KB: below the default dynamic LDS limit
     if (g.M <= 16) skinny_split_kernel<FMT, 16, NCH><<<grid, 256, lds, s>>>(g);
-    else skinny_split_kernel<FMT, 32, NCH><<<grid, 256, lds, s>>>(g);
+    else if (g.M <= 32) skinny_split_kernel<FMT, 32, NCH><<<grid, 256, lds, s>>>(g);
+    else skinny_split_kernel<FMT, 64, NCH><<<grid, 256, lds, s>>>(g);
     return XQ_OK;
 }
 
@@ -790,7 +533,7 @@ static int launch_skinny_split(const xq_weight* w, const bf16_t* x, int64_t ldx,
     g.su_part = (float*)((char*)workspace + al256((int64_t)p.splits * M * N * 4));
     g.lora_A = rp ? lora_A : nullptr; g.lora_f32 = lora_dtype == XQ_DT_F32; g.r = r; g.r_pad = rp;
     const dim3 grid((unsigned)p.splits, (unsigned)(p.row_blocks + g.su_blocks));
-    const size_t lds = (size_t)M * g.xp * 2 + 4 * 4096;   // x slice + the four weight slabs (or the su reduction buffer)
+    const size_t lds = (size_t)(M < 32 ? M : 32) * g.xp * 2 + 4 * 4096;   // x slice + the four weight slabs (or the su reduction buffer)
 
     SkinnyEpiArgs e;
     e.partial = g.partial; e.su_part = g.su_part; e.splits = p.splits; e.su_parts = rp ? p.splits : 0;
@@ -821,55 +564,6 @@ static int launch_skinny_split(const xq_weight* w, const bf16_t* x, int64_t ldx,
     return XQ_OK;
 }
 
-// ---------------------------------------------------------------- 32 < M <= 64
-template <int FMT, int MT, int NW>
-static int launch_rows_one(const SkinnyRowsArgs& g, dim3 grid, hipStream_t s) {
-    // LDS: the wave-private x tiles (MT*32 rows of 272 B per wave); the reduction buffer reuses them
-    constexpr size_t lds = (size_t)NW * MT * 32 * 136 * 2;
-    static_assert(lds >= (size_t)NW * MT * 16 * 64 * 4, "reduction buffer must fit in the x tiles");
-    static bool attr_set = false;
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute((const void*)skinny_rows_kernel<FMT, MT, NW>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        if (e != hipSuccess) {
-            xq_set_error("xq_linear_fwd: cannot raise the dynamic LDS limit: %s", hipGetErrorString(e));
-            return XQ_ERR_LAUNCH;
-        }
-        attr_set = true;
-    }
-    skinny_rows_kernel<FMT, MT, NW><<<grid, NW * 64, lds, s>>>(g);
-    return XQ_OK;
-}
-
-template <int FMT>
-static int launch_rows_cfg(const SkinnyRowsArgs& g, hipStream_t s) {
-    dim3 grid((unsigned)xq_cdiv(g.N, 32));
-    // more slabs than CUs: 4 waves per slab so that two blocks share a CU; else 8 waves per slab
-    const bool many = grid.x > 256;
-    return many ? launch_rows_one<FMT, 2, 4>(g, grid, s) : launch_rows_one<FMT, 2, 8>(g, grid, s);
-}
-
-static int launch_skinny_rows(const xq_weight* w, const bf16_t* x, int64_t ldx, int64_t M, const void* lora_A, const void* lora_B,
-                              int lora_dtype, int r, int rp, float scaling, const bf16_t* bias, bf16_t* y, int64_t ldy,
-                              void* workspace, hipStream_t stream) {
-    const int64_t N = w->rows, K = w->cols;
-    float* su_part = (float*)workspace;
-    const int su_parts = (int)xq_cdiv(K, SU_KB);
-    if (rp) {
-        const int f32 = lora_dtype == XQ_DT_F32;
-        skinny_su_kernel<2><<<dim3(su_parts), SU_NW * 64, (size_t)SU_NW * 32 * 64 * 4, stream>>>(x, ldx, (int)M, (int)K, lora_A, f32, r, rp, su_part);
-    }
-    SkinnyRowsArgs g;
-    g.x = x; g.ldx = ldx; g.M = (int)M; g.N = (int)N; g.K = (int)K;
-    g.packed = (const uint8_t*)w->packed; g.scales = (const uint8_t*)w->scales; g.global_scale = w->global_scale;
-    g.group = w->group; g.scale_dtype = w->scale_dtype;
-    g.su_part = rp ? su_part : nullptr; g.su_parts = su_parts; g.su_scale = scaling; g.lora_B = rp ? lora_B : nullptr;
-    g.lora_f32 = lora_dtype == XQ_DT_F32; g.r = r; g.r_pad = rp;
-    g.bias = bias; g.y = y; g.ldy = ldy;
-    if (w->format == XQ_FMT_FP8) return launch_rows_cfg<XQ_FMT_FP8>(g, stream);
-    if (w->format == XQ_FMT_INT4) return launch_rows_cfg<XQ_FMT_INT4>(g, stream);
-    return launch_rows_cfg<XQ_FMT_NVFP4>(g, stream);
-}
-
 int launch_skinny(const xq_weight* w, const bf16_t* x, int64_t ldx, int64_t M, const void* lora_A, const void* lora_B,
                   int lora_dtype, int r, float scaling, const bf16_t* bias, bf16_t* y, int64_t ldy, void* workspace,
                   int64_t workspace_bytes, hipStream_t stream) {
@@ -884,9 +578,7 @@ int launch_skinny(const xq_weight* w, const bf16_t* x, int64_t ldx, int64_t M, c
     // region is the whole forward (both launches)
     const double wbytes = (double)xq_packed_bytes_per_expert(w) + (double)xq_scale_bytes_per_expert(w);
     const bool timed = xq_profile_mark_begin(stream, wbytes + 2.0 * M * K + 2.0 * M * N + 4.0 * r * (K + N));
-    const int rc = M <= kSplitMaxM
-        ? launch_skinny_split(w, x, ldx, M, lora_A, lora_B, lora_dtype, r, rp, scaling, bias, y, ldy, workspace, stream)
-        : launch_skinny_rows(w, x, ldx, M, lora_A, lora_B, lora_dtype, r, rp, scaling, bias, y, ldy, workspace, stream);
+    const int rc = launch_skinny_split(w, x, ldx, M, lora_A, lora_B, lora_dtype, r, rp, scaling, bias, y, ldy, workspace, stream);
     if (timed) xq_profile_mark_end(stream);
     if (rc) return rc;
     XQ_CHECK_LAUNCH("skinny forward");

@@ -41,10 +41,14 @@ class QuantWeight:
     group: int
     global_scale: Optional[Tensor] = None
     num_experts: int = 1
+    _cw: Optional[_C.XqWeight] = None
 
     def c(self) -> _C.XqWeight:
-        return _C.make_weight(self.fmt, self.layout, self.packed, self.scales, self.scale_dtype, self.rows,
-                              self.cols, self.group, self.global_scale, self.num_experts)
+        """The C descriptor (built once per QuantWeight: it holds raw pointers into the tensors above)."""
+        if self._cw is None:
+            self._cw = _C.make_weight(self.fmt, self.layout, self.packed, self.scales, self.scale_dtype, self.rows,
+                                      self.cols, self.group, self.global_scale, self.num_experts)
+        return self._cw
 
 
 def _r_pad(r: int) -> int:
@@ -73,30 +77,46 @@ def _ld(x2: Tensor) -> int:
 # ---------------------------------------------------------------------------
 # dense: custom ops
 # ---------------------------------------------------------------------------
+_WS_BYTES: dict = {}
+_EMPTY: dict = {}
+
+
+def _workspace_bytes(M: int, N: int, K: int, r: int) -> int:
+    key = (M, N, K, r)
+    v = _WS_BYTES.get(key)
+    if v is None:
+        v = _WS_BYTES[key] = _C.lib().xq_linear_workspace_bytes(M, N, K, r)
+    return v
+
+
 def _linear_fwd_impl(x: Tensor, packed: Tensor, scales: Tensor, global_scale: Optional[Tensor],
                      lora_A: Optional[Tensor], lora_B: Optional[Tensor], bias: Optional[Tensor],
                      fmt: str, scale_dt: torch.dtype, group: int, N: int, K: int, r: int,
-                     scaling: float, want_su: bool) -> Tuple[Tensor, Tensor]:
+                     scaling: float, want_su: bool, cw: Optional[_C.XqWeight] = None) -> Tuple[Tensor, Tensor]:
     if x.dtype != torch.bfloat16:
         raise _C.XqError(f"activations must be bf16, got {x.dtype}")
     x2 = _as_2d(x)
     M = x2.shape[0]
     if x2.shape[1] != K:
         raise _C.XqError(f"input width {x2.shape[1]} != in_features {K}")
-    w = _C.make_weight(fmt, _C.XQ_LAYOUT_FLAT, packed, scales, scale_dt, N, K, group, global_scale)
+    w = cw if cw is not None else _C.make_weight(fmt, _C.XQ_LAYOUT_FLAT, packed, scales, scale_dt, N, K, group, global_scale)
     dev = x.device
     y = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
     rp = _r_pad(r)
-    su = torch.empty(M if want_su else 0, rp, dtype=torch.bfloat16, device=dev)
-    L = _C.lib()
-    ws_bytes = L.xq_linear_workspace_bytes(M, N, K, r)
+    if want_su:
+        su = torch.empty(M, rp, dtype=torch.bfloat16, device=dev)
+    else:
+        su = _EMPTY.get(dev)
+        if su is None:
+            su = _EMPTY[dev] = torch.empty(0, dtype=torch.bfloat16, device=dev)
+    ws_bytes = _workspace_bytes(M, N, K, r)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     A = lora_A.contiguous() if lora_A is not None else None
     B = lora_B.contiguous() if lora_B is not None else None
     b = bias.to(torch.bfloat16).contiguous() if bias is not None else None
-    _C.check(L.xq_linear_fwd(ctypes.byref(w), x2.data_ptr(), _ld(x2), M, _C.ptr(A), _C.ptr(B), _lora_dt(A), r,
-                             scaling, _C.ptr(b), y.data_ptr(), N, su.data_ptr() if (rp and want_su) else None, ws.data_ptr(),
-                             ws_bytes, _C.stream_ptr(dev)))
+    _C.check(_C.lib().xq_linear_fwd(ctypes.byref(w), x2.data_ptr(), _ld(x2), M, _C.ptr(A), _C.ptr(B), _lora_dt(A), r,
+                                    scaling, _C.ptr(b), y.data_ptr(), N, su.data_ptr() if (rp and want_su) else None,
+                                    ws.data_ptr(), ws_bytes, _C.stream_ptr(dev)))
     return y.reshape(*x.shape[:-1], N), su
 
 
@@ -203,7 +223,7 @@ def qlora_linear(x: Tensor, qw: QuantWeight, lora_A: Optional[Tensor], lora_B: O
         B = lora_B.detach()[:, :r] if lora_B is not None else None
         return _linear_fwd_impl(x.detach(), qw.packed, qw.scales, qw.global_scale, A, B,
                                 None if bias is None else bias.detach(), qw.fmt, qw.scale_dtype, qw.group,
-                                qw.rows, qw.cols, r, float(scaling), False)[0]
+                                qw.rows, qw.cols, r, float(scaling), False, qw.c())[0]
     return QLoRALinearFunction.apply(x, lora_A, lora_B, bias, qw, r, scaling, training)
 
 

@@ -370,8 +370,24 @@ class QLoRALinear(LoraModule, nn.Module):
     def forward(self, x: Tensor) -> Tensor:
         if self.enable_aqn and self.training:
             return self._forward_with_noise(x)
-        return qlora_linear(x, self._quant_weight(), self.lora_A, self.lora_B, self.active_r,
+        return qlora_linear(x, self._forward_quant_weight(), self.lora_A, self.lora_B, self.active_r,
                             self._active_scaling(), self.bias)
+
+    def _forward_quant_weight(self) -> QuantWeight:
+        """`_quant_weight()` memoised on the addresses of the packed state: the description (and its C
+        descriptor) is rebuilt only when a buffer has been replaced.  Sharded state is gathered every call."""
+        p = self.packed_weight_f32
+        if _is_dtensor(p.data):
+            return self._quant_weight()
+        key = (p.data_ptr(), p.dtype) + tuple(
+            t.data_ptr() for t in (getattr(self, "weight_scales", None), getattr(self, "weight_block_scales", None),
+                                   getattr(self, "weight_global_scale", None)) if t is not None)
+        key += tuple(self._scale_dtypes.values())
+        cached = self.__dict__.get("_qw_cache")
+        if cached is None or cached[0] != key:
+            cached = (key, self._quant_weight())
+            self.__dict__["_qw_cache"] = cached
+        return cached[1]
 
     # ------------------------------------------------------------------ checkpoint helpers
     def get_quantized_state_dict(self) -> Dict[str, Tensor]:
