@@ -156,11 +156,18 @@ int xq_linear_bwd(const xq_weight* w, const void* x, int64_t ldx, const void* dy
  * in one pass (block_fp8_linear.py:111-119 with block_fp8_quantize_gkn,
  * ops/quantize/block_fp8_gkn_quantize.py:40-121): per 128x128 block
  * s = max(amax(W') / 448, 1e-12), bytes = e4m3(clamp(W' / s, +-448)).
- * packed_out / scales_out may be the weight's own buffers (in-place). */
+ * packed_out / scales_out may be the weight's own buffers (in-place).
+ *
+ * Both take a workspace of xq_merge_workspace_bytes(N, K, r) bytes (256-byte
+ * aligned; may be NULL when r == 0): the factors are split once per call
+ * into bf16 hi/lo panels there. */
+int64_t xq_merge_workspace_bytes(int64_t N, int64_t K, int r);
 int xq_merge_dense(const xq_weight* w, const void* lora_A, const void* lora_B, int lora_dtype, int r,
-                   float scaling, void* out, int out_dtype, void* stream);
+                   float scaling, void* out, int out_dtype, void* workspace, int64_t workspace_bytes,
+                   void* stream);
 int xq_merge_requant_fp8(const xq_weight* w, const void* lora_A, const void* lora_B, int lora_dtype, int r,
-                         float scaling, void* packed_out, float* scales_out, void* stream);
+                         float scaling, void* packed_out, float* scales_out, void* workspace,
+                         int64_t workspace_bytes, void* stream);
 
 /* ---- SwiGLU between gate/up and down ------------------------------------
  * Replaces fused_silu_and_mul (ops/fused_silu_and_mul.py:22-60 and its

@@ -61,9 +61,10 @@ _SIGNATURES = {
     "xq_linear_bwd": (_INT, [_W, _P, _I64, _P, _I64, _I64, _P, _P, _INT, _INT, _F, _P, _P, _I64, _P, _P, _P, _I64,
                              _P]),
     # w, A, B, lora_dtype, r, scaling, out, out_dtype, stream
-    "xq_merge_dense": (_INT, [_W, _P, _P, _INT, _INT, _F, _P, _INT, _P]),
+    "xq_merge_workspace_bytes": (_I64, [_I64, _I64, _INT]),
+    "xq_merge_dense": (_INT, [_W, _P, _P, _INT, _INT, _F, _P, _INT, _P, _I64, _P]),
     # w, A, B, lora_dtype, r, scaling, packed_out, scales_out, stream
-    "xq_merge_requant_fp8": (_INT, [_W, _P, _P, _INT, _INT, _F, _P, _P, _P]),
+    "xq_merge_requant_fp8": (_INT, [_W, _P, _P, _INT, _INT, _F, _P, _P, _P, _I64, _P]),
     # gate, up, ld_in, row_w, h, ld_h, rows, cols, stream
     "xq_silu_mul_fwd": (_INT, [_P, _P, _I64, _P, _P, _I64, _I64, _I64, _P]),
     # gate, up, ld_in, dh, ld_dh, row_w, dgate, dup, ld_out, d_row_w, rows, cols, stream

@@ -2,28 +2,32 @@
 //
 //   W'[n, k] = deq(W)[n, k] + scaling * sum_j B[n, j] * A[j, k]          (W FLAT [N, K])
 //
-// One block owns a 128 x 128 tile -- exactly one block-fp8 scale block -- and
-//   1. computes the tile of the low-rank product on the matrix cores.  The reference
-//      multiplies the fp32 factors in fp32; here each factor is split into two bf16
-//      terms (hi + lo, 16 significant bits) and the product is the three bf16 MFMA
-//      products hi*hi + hi*lo + lo*hi with fp32 accumulation (relative error ~2^-16
-//      per term instead of 2^-9 with plain bf16 factors);
-//   2. parks it in LDS, then walks the tile row-contiguously: every thread owns 64
-//      consecutive columns of one row, loads the packed codes with 16-byte loads,
-//      decodes them to the reference decoder's value and adds the update;
-//   3a. (publish) rounds to bf16 -- bf16(bf16(deq) + bf16(delta)), the arithmetic of the
-//      reference's weight-sync merge -- or writes the fp32 sum; or
+// One block owns a 128 x 128 tile -- exactly one block-fp8 scale block.  It
+//   0. issues every load it will need before waiting for any: the tile's packed codes (16-element runs,
+//      coalesced: consecutive lanes walk a row) and scales, then its MFMA operands.  All loads are
+//      unconditional (indices past the end are clamped, values masked), so the waits count exactly and the
+//      codes arrive while the low-rank product is computed;
+//   1. computes the tile of the low-rank product on the matrix cores.  The reference multiplies the fp32
+//      factors in fp32; here each factor is split into two bf16 terms (hi + lo, 16 significant bits) and the
+//      product is the three bf16 MFMA products hi*hi + hi*lo + lo*hi with fp32 accumulation (relative error
+//      ~2^-16 per term instead of 2^-9 with plain bf16 factors).  A small launch before it (merge_prep_kernel)
+//      splits scaling * B and A^T once into zero-padded bf16 panels in the caller's workspace, laid out so
+//      that a tile's rows are one contiguous run of each panel: the tile kernel copies them to LDS with 16-byte
+//      pieces and multiplies while its codes are still in flight;
+//   2. hands it to the row-contiguous pass through LDS, 64 columns at a time: every thread decodes its runs
+//      to the reference decoder's value and adds the update;
+//   3a. (publish) rounds to bf16 -- bf16(bf16(deq) + bf16(delta)), the arithmetic of the reference's
+//      weight-sync merge -- or writes the fp32 sum; or
 //   3b. (requantise, block-fp8) reduces the tile's absmax, derives the new block scale
-//      s = max(amax / 448, 1e-12) and writes e4m3(clamp(x / s)) bytes and the scale:
-//      decode -> add -> re-encode in one pass over 1 byte per weight each way.
+//      s = max(amax / 448, 1e-12) and writes e4m3(clamp(x / s)) bytes and the scale: decode -> add ->
+//      re-encode in one pass over 1 byte per weight each way.
 #include "xq_common.h"
 #include "xq_lora.h"
 
 namespace xq {
 
 constexpr int MG_T = 128;           // tile edge
-constexpr int MG_FP = 64 + 8;       // factor tile row pitch (bf16 elements): 144 B
-constexpr int MG_DP = MG_T + 4;     // delta tile row pitch (floats)
+constexpr int MG_HP = 64 + 4;       // delta half-tile row pitch (floats)
 
 struct MergeArgs {
     const uint8_t* packed;
@@ -31,193 +35,233 @@ struct MergeArgs {
     const float* global_scale;
     int32_t fmt, group, scale_dtype;
     int32_t N, K;
-    const void* A;       // [r, K]
-    const void* B;       // [N, r]
+    const void* A;       // [r, K]   } read by merge_prep_kernel only
+    const void* B;       // [N, r]   }
     int32_t lora_f32, r, r_pad;
     float scaling;
+    const bf16_t* Bh;    // factor panels written by merge_prep_kernel: hi and lo bf16 parts of scaling * B, rows
+    const bf16_t* Bl;    // padded to a multiple of 128 ([Npad][r_pad], zero beyond N and r), and of A transposed
+    const bf16_t* Ah;    // ([Kpad][r_pad], row = k)
+    const bf16_t* Al;
     int32_t mode;        // 0: bf16 out (publish arithmetic), 1: fp32 out, 2: block-fp8 requantise
     void* out;           // mode 0/1: [N, K]
     uint8_t* packed_out; // mode 2: [N, K] e4m3 bytes    } both may alias the inputs: a block reads its tile and its
     float* scales_out;   // mode 2: [ceil(N/128), ceil(K/128)] } scale before it writes them, and touches no other
 };
 
-__device__ __forceinline__ float factor_at(const void* p, int64_t idx, bool f32) {
-    return f32 ? ((const float*)p)[idx] : bf16_to_f32(((const bf16_t*)p)[idx]);
-}
-
-// decode 16 consecutive elements of row n starting at column k (k % 16 == 0) to fp32, exactly as xq_decode does
-template <int FMT>
-__device__ __forceinline__ void decode_run16(const MergeArgs& g, int64_t n, int k, float* v) {
-    if (FMT == XQ_FMT_FP8) {
-        const u32x4 w = *(const u32x4*)(g.packed + n * g.K + k);
-        const float s = ((const float*)g.scales)[(n >> 7) * ((g.K + 127) >> 7) + (k >> 7)];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const f32x2 lo = e4m3x2_to_f32(w[i], false), hi = e4m3x2_to_f32(w[i], true);
-            v[4 * i] = lo[0] * s; v[4 * i + 1] = lo[1] * s; v[4 * i + 2] = hi[0] * s; v[4 * i + 3] = hi[1] * s;
-        }
-    } else {
-        const u32x2 w = *(const u32x2*)(g.packed + ((n * g.K + k) >> 1));
-        const float gs = FMT == XQ_FMT_NVFP4 ? g.global_scale[0] : 1.0f;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const uint32_t nib = (w[i >> 3] >> (4 * (i & 7))) & 0xfu;
-            // one scale per `group` elements; group is even, so a pair never straddles two groups
-            const float s = load_scale(g.scales, (n * g.K + k + i) / g.group, g.scale_dtype);
-            v[i] = val4<FMT>(nib, FMT == XQ_FMT_NVFP4 ? s * gs : s);
-        }
+// hi/lo bf16 split of the factors, once per call instead of once per tile: Bh/Bl[n][j] from scaling * B[n][j],
+// Ah/Al[k][j] from A[j][k] (transposed so that a tile's MFMA operand rows are contiguous 16-byte pieces).
+// Rows beyond N / K (up to the next multiple of 128) and ranks beyond r are zero, so the tile kernel reads the
+// panels without bounds checks.
+__global__ void __launch_bounds__(256) merge_prep_kernel(MergeArgs g, int npad, int kpad) {
+    const int rp = g.r_pad;
+    const int64_t nb = (int64_t)npad * rp, na = (int64_t)kpad * rp;
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const bool f32 = g.lora_f32 != 0;
+    if (idx < nb) {
+        const int64_t n = idx / rp;
+        const int j = (int)(idx - n * rp);
+        float v = 0.0f;
+        if (n < g.N && j < g.r) v = g.scaling * (f32 ? ((const float*)g.B)[n * g.r + j] : bf16_to_f32(((const bf16_t*)g.B)[n * g.r + j]));
+        const bf16_t hi = to_bf16(v);
+        ((bf16_t*)g.Bh)[idx] = hi;
+        ((bf16_t*)g.Bl)[idx] = to_bf16(v - bf16_to_f32(hi));
+    } else if (idx < nb + na) {
+        const int64_t t = idx - nb;           // k fastest: coalesced reads of A's rows
+        const int j = (int)(t / kpad);
+        const int64_t k = t - (int64_t)j * kpad;
+        float v = 0.0f;
+        if (k < g.K && j < g.r) v = f32 ? ((const float*)g.A)[(int64_t)j * g.K + k] : bf16_to_f32(((const bf16_t*)g.A)[(int64_t)j * g.K + k]);
+        const bf16_t hi = to_bf16(v);
+        ((bf16_t*)g.Ah)[k * rp + j] = hi;
+        ((bf16_t*)g.Al)[k * rp + j] = to_bf16(v - bf16_to_f32(hi));
     }
 }
 
-template <int FMT, int RP>
-__global__ void __launch_bounds__(256) merge_kernel(MergeArgs g) {
+// REQ: the block-fp8 re-quantise mode (results are held in registers until the tile's absmax is known).
+// 512 threads per tile: 32 result registers per thread in that mode, so that two blocks (16 waves) fit a CU.
+template <int FMT, int RP, bool REQ>
+__global__ void __launch_bounds__(512, 4) merge_kernel(MergeArgs g) {
+    asm volatile("" ::"s"(g.packed), "s"(g.scales), "s"(g.global_scale), "s"(g.group), "s"(g.scale_dtype), "s"(g.N), "s"(g.K),
+                 "s"(g.Bh), "s"(g.Bl), "s"(g.Ah), "s"(g.Al), "s"(g.mode), "s"(g.out), "s"(g.packed_out), "s"(g.scales_out));
+    // (all arguments in scalar registers after one round trip)
     extern __shared__ __attribute__((aligned(16))) uint8_t mg_lds[];
-    __shared__ float sh_amax[4];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    __shared__ float sh_amax[8];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int k0 = blockIdx.x * MG_T, n0 = blockIdx.y * MG_T;
-    constexpr int rp = RP;        // LoRA rank rounded up to 16 (0: no update)
-    float* dt = (float*)mg_lds;   // delta tile [128][MG_DP] (used after the factor tiles are dead)
+    constexpr bool FP8 = FMT == XQ_FMT_FP8;
+    auto lds_barrier = [&]() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
 
-    if (rp > 0) {
-        // ---- 1. factor tiles, split hi/lo, both [row][j]: Bt rows = n, At rows = k
-        bf16_t* Bh = (bf16_t*)mg_lds;
-        bf16_t* Bl = Bh + MG_T * MG_FP;
-        bf16_t* Ah = Bl + MG_T * MG_FP;
-        bf16_t* Al = Ah + MG_T * MG_FP;
-        const bool f32 = g.lora_f32 != 0;
-        // every load of a factor tile is issued before its first use (compile-time trip counts)
-        {
-            constexpr int H = RP / 2;                     // thread -> row tid >> 1, ranks (tid & 1) * H .. +H
-            const int row = tid >> 1, j0 = (tid & 1) * H;
-            const int64_t n = n0 + row;
-            float v[H > 0 ? H : 1];
+    // ---- 0a. this tile's rows of the four factor panels -> registers (16-byte pieces, each tile one contiguous
+    // run of its panel), issued before the codes so that they can be waited for on their own
+    constexpr int FP = RP + 8;                        // LDS row pitch (bf16 elements): fragment reads are conflict free
+    constexpr int PPRW = RP / 8;                      // 16-byte pieces per panel row
+    constexpr int NP = RP / 8;                        // pieces per thread: 4 tiles x 128 rows x PPRW / 512
+    u32x4 fp[NP > 0 ? NP : 1];
+    if (RP > 0) {
 #pragma unroll
-            for (int jj = 0; jj < H; ++jj) v[jj] = (j0 + jj < g.r && n < g.N) ? factor_at(g.B, n * g.r + j0 + jj, f32) : 0.0f;
-#pragma unroll
-            for (int jj = 0; jj < H; jj += 2) {
-                const bf16_t h0 = to_bf16(v[jj]), h1 = to_bf16(v[jj + 1]);
-                *(uint32_t*)(Bh + row * MG_FP + j0 + jj) = (uint32_t)h0 | ((uint32_t)h1 << 16);
-                *(uint32_t*)(Bl + row * MG_FP + j0 + jj) = pack_bf16x2(v[jj] - bf16_to_f32(h0), v[jj + 1] - bf16_to_f32(h1));
-            }
+        for (int i = 0; i < NP; ++i) {
+            const int p = tid + 512 * i, tile = p / (128 * PPRW), q = p % (128 * PPRW);
+            const bf16_t* base = tile == 0 ? g.Bh + (int64_t)n0 * RP : tile == 1 ? g.Bl + (int64_t)n0 * RP
+                               : tile == 2 ? g.Ah + (int64_t)k0 * RP : g.Al + (int64_t)k0 * RP;
+            fp[i] = *(const u32x4*)(base + q * 8);
         }
-        {
-            constexpr int H = RP / 2;                     // thread -> column tid & 127, ranks (tid >> 7) * H .. +H
-            const int kk = tid & 127, j0 = (tid >> 7) * H;   // consecutive threads along k: coalesced rows of A
-            const int64_t k = k0 + kk;
-            float v[H > 0 ? H : 1];
-#pragma unroll
-            for (int jj = 0; jj < H; ++jj) v[jj] = (j0 + jj < g.r && k < g.K) ? factor_at(g.A, (int64_t)(j0 + jj) * g.K + k, f32) : 0.0f;
-#pragma unroll
-            for (int jj = 0; jj < H; jj += 2) {
-                const bf16_t h0 = to_bf16(v[jj]), h1 = to_bf16(v[jj + 1]);
-                *(uint32_t*)(Ah + kk * MG_FP + j0 + jj) = (uint32_t)h0 | ((uint32_t)h1 << 16);
-                *(uint32_t*)(Al + kk * MG_FP + j0 + jj) = pack_bf16x2(v[jj] - bf16_to_f32(h0), v[jj + 1] - bf16_to_f32(h1));
-            }
-        }
-        __syncthreads();
-        // ---- 2. delta tile on the matrix cores: wave (wm, wn) owns rows wm*64.., cols wn*64..
-        const int wm = wave >> 1, wn = wave & 1, fr = lane & 31, fk = (lane >> 5) * 8;
-        f32x16 acc[2][2];
-#pragma unroll
-        for (int i = 0; i < 2; ++i)
-#pragma unroll
-            for (int j = 0; j < 2; ++j)
-#pragma unroll
-                for (int q = 0; q < 16; ++q) acc[i][j][q] = 0.0f;
-        for (int ks = 0; ks < (rp >> 4); ++ks) {
-            bf16x8 bh[2], bl[2], ah[2], al[2];
-#pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                const int ro = (wm * 64 + i * 32 + fr) * MG_FP + ks * 16 + fk;
-                const int co = (wn * 64 + i * 32 + fr) * MG_FP + ks * 16 + fk;
-                bh[i] = *(const bf16x8*)(Bh + ro); bl[i] = *(const bf16x8*)(Bl + ro);
-                ah[i] = *(const bf16x8*)(Ah + co); al[i] = *(const bf16x8*)(Al + co);
-            }
-#pragma unroll
-            for (int i = 0; i < 2; ++i)
-#pragma unroll
-                for (int j = 0; j < 2; ++j) {
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bl[i], ah[j], acc[i][j], 0, 0, 0);
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bh[i], al[j], acc[i][j], 0, 0, 0);
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bh[i], ah[j], acc[i][j], 0, 0, 0);
-                }
-        }
-        __syncthreads();   // factor tiles are dead: the delta tile takes their place
-        const int rgrp = (lane >> 5) * 4;
-#pragma unroll
-        for (int i = 0; i < 2; ++i)
-#pragma unroll
-            for (int j = 0; j < 2; ++j)
-#pragma unroll
-                for (int q = 0; q < 16; ++q) {
-                    const int row = wm * 64 + i * 32 + (q & 3) + rgrp + 8 * (q >> 2), col = wn * 64 + j * 32 + fr;
-                    dt[row * MG_DP + col] = acc[i][j][q] * g.scaling;
-                }
-        __syncthreads();
     }
 
-    // ---- 3. row-contiguous pass: thread -> row tid >> 1, columns (tid & 1) * 64 .. +64
-    const int row = tid >> 1, c0 = (tid & 1) * 64;
-    const int64_t n = n0 + row;
-    const bool row_ok = n < g.N;
-    float m[64];
+    // ---- 0b. the tile's codes: run h of this thread = row tid >> 2, columns h*64 + (tid & 3)*16 .. +15
+    const int rrow = tid >> 2, rcol = (tid & 3) * 16;
+    u32x4 wr[2];                                      // fp8: 16 bytes; 4-bit: 8 bytes (first two words)
+    uint32_t sraw[2];                                 // 4-bit: the run's scale (group % 16 == 0), raw
+    const bool run_scale = !FP8 && (g.group & 15) == 0;
+    float tile_scale = 1.0f;
+    if (FP8) tile_scale = ((const float*)g.scales)[(int64_t)blockIdx.y * ((g.K + 127) >> 7) + blockIdx.x];
+    const int64_t nrow = n0 + rrow < g.N ? n0 + rrow : g.N - 1;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const int k = k0 + h * 64 + rcol < g.K ? k0 + h * 64 + rcol : g.K - 16;   // K % 16 == 0
+        if (FP8) wr[h] = *(const u32x4*)(g.packed + nrow * g.K + k);
+        else {
+            const u32x2 t = *(const u32x2*)(g.packed + ((nrow * g.K + k) >> 1));
+            wr[h] = u32x4{t[0], t[1], 0u, 0u};
+            const int64_t si = run_scale ? (nrow * g.K + k) / g.group : 0;
+            sraw[h] = g.scale_dtype == XQ_SCALE_F32 ? ((const uint32_t*)g.scales)[si]
+                    : g.scale_dtype == XQ_SCALE_BF16 ? ((const uint16_t*)g.scales)[si] : g.scales[si];
+        }
+    }
+    const float gs = FMT == XQ_FMT_NVFP4 ? g.global_scale[0] : 1.0f;
+
+    float* dt = (float*)mg_lds;   // delta half tile [128][MG_HP] (takes the place of the factor tiles)
+    f32x16 acc[2];                // wave (wq, wh): rows wq*32 .. +31, columns wh*64 + j*32 .. +31
+    const int wq = wave & 3, wh = wave >> 2, fr = lane & 31, fk = (lane >> 5) * 8;
+    if (RP > 0) {
+        // ---- 1. factor tiles -> LDS ([tile][128][FP]); the delta tile on the matrix cores while the codes are
+        // still in flight
+        bf16_t* ft = (bf16_t*)mg_lds;
+#pragma unroll
+        for (int i = 0; i < NP; ++i) {
+            const int p = tid + 512 * i, tile = p / (128 * PPRW), q = p % (128 * PPRW);
+            *(u32x4*)(ft + (tile * 128 + q / PPRW) * FP + (q % PPRW) * 8) = fp[i];
+        }
+        lds_barrier();
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int q = 0; q < 16; ++q) acc[j][q] = 0.0f;
+        const bf16_t* pb = ft + (wq * 32 + fr) * FP + fk;                    // Bh rows of this wave; Bl one tile further
+        const bf16_t* pa = ft + (2 * 128 + wh * 64 + fr) * FP + fk;          // Ah rows of this wave's columns; Al one tile further
+#pragma unroll
+        for (int ks = 0; ks < (RP >> 4); ++ks) {
+            const bf16x8 bh = *(const bf16x8*)(pb + ks * 16), bl = *(const bf16x8*)(pb + 128 * FP + ks * 16);
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const bf16x8 ah = *(const bf16x8*)(pa + j * 32 * FP + ks * 16), al = *(const bf16x8*)(pa + (128 + j * 32) * FP + ks * 16);
+                acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bl, ah, acc[j], 0, 0, 0);
+                acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bh, al, acc[j], 0, 0, 0);
+                acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bh, ah, acc[j], 0, 0, 0);
+            }
+        }
+    }
+
+    // ---- 2./3. per 64-column half: delta half tile -> LDS (the four waves that own it), row-contiguous pass
+    float m[REQ ? 32 : 1];
     float amax = 0.0f;
+    const int64_t n = n0 + rrow;
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-        const int k = k0 + c0 + u * 16;
-        const bool ok = row_ok && k < g.K;   // K % 16 == 0: runs are all in or all out
-        float v[16];
-        if (ok) decode_run16<FMT>(g, n, k, v);
+    for (int h = 0; h < 2; ++h) {
+        if (RP > 0) {
+            lds_barrier();   // h = 0: the factor tiles are dead; h = 1: the first half has been read
+            if (wh == h) {
+                const int rgrp = (lane >> 5) * 4;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const float d = rp > 0 ? dt[row * MG_DP + c0 + u * 16 + i] : 0.0f;
-            float x;
-            if (g.mode == 0) x = bf16_to_f32(to_bf16(bf16_to_f32(to_bf16(v[i])) + bf16_to_f32(to_bf16(d))));
-            else if (FMT == XQ_FMT_FP8) x = v[i] + d;
-            else x = bf16_to_f32(to_bf16(bf16_to_f32(to_bf16(v[i])) + bf16_to_f32(to_bf16(d))));   // 4-bit decoders return bf16
-            x = ok ? x : 0.0f;
-            m[u * 16 + i] = x;
-            amax = fmaxf(amax, fabsf(x));
+                for (int j = 0; j < 2; ++j)
+#pragma unroll
+                    for (int q = 0; q < 16; ++q) {
+                        const int row = wq * 32 + (q & 3) + rgrp + 8 * (q >> 2), col = j * 32 + fr;
+                        dt[row * MG_HP + col] = acc[j][q];
+                    }
+            }
+            lds_barrier();
         }
-    }
-    if (g.mode != 2) {
+        const int k = k0 + h * 64 + rcol;
+        const bool ok = n < g.N && k < g.K;               // K % 16 == 0: runs are all in or all out
+        float v[16];
+        if (FP8) {
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int k = k0 + c0 + u * 16;
-            if (!(row_ok && k < g.K)) continue;
+            for (int i = 0; i < 4; ++i) {
+                const f32x2 lo = e4m3x2_to_f32(wr[h][i], false), hi = e4m3x2_to_f32(wr[h][i], true);
+                v[4 * i] = lo[0] * tile_scale; v[4 * i + 1] = lo[1] * tile_scale;
+                v[4 * i + 2] = hi[0] * tile_scale; v[4 * i + 3] = hi[1] * tile_scale;
+            }
+        } else {
+            const uint32_t sr = sraw[h];
+            const float srun = g.scale_dtype == XQ_SCALE_F32 ? __uint_as_float(sr)
+                             : g.scale_dtype == XQ_SCALE_BF16 ? __uint_as_float(sr << 16) : e4m3_to_f32((uint8_t)sr);
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const uint32_t nib = (wr[h][i >> 3] >> (4 * (i & 7))) & 0xfu;
+                // groups that are not multiples of 16 (never with the reference's formats): per-element lookup
+                const float sc = run_scale ? srun : load_scale(g.scales, (nrow * g.K + (k < g.K ? k : 0) + i) / g.group, g.scale_dtype);
+                v[i] = val4<FMT>(nib, FMT == XQ_FMT_NVFP4 ? sc * gs : sc);
+            }
+        }
+        float x[16];
+#pragma unroll
+        for (int i = 0; i < 16; i += 4) {
+            f32x4 d = {0.0f, 0.0f, 0.0f, 0.0f};
+            if (RP > 0) d = *(const f32x4*)(dt + rrow * MG_HP + rcol + i);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                float t;
+                if (g.mode == 0 || !FP8) t = bf16_to_f32(to_bf16(bf16_to_f32(to_bf16(v[i + e])) + bf16_to_f32(to_bf16(d[e]))));   // 4-bit decoders return bf16
+                else t = v[i + e] + d[e];
+                x[i + e] = ok ? t : 0.0f;
+            }
+        }
+        if (REQ) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                m[h * 16 + i] = x[i];
+                amax = fmaxf(amax, fabsf(x[i]));
+            }
+        } else if (ok) {
             if (g.mode == 0) {
                 bf16_t* o = (bf16_t*)g.out + n * g.K + k;
                 uint32_t pk[8];
 #pragma unroll
-                for (int i = 0; i < 8; ++i) pk[i] = pack_bf16x2(m[u * 16 + 2 * i], m[u * 16 + 2 * i + 1]);
+                for (int i = 0; i < 8; ++i) pk[i] = pack_bf16x2(x[2 * i], x[2 * i + 1]);
                 *(u32x4*)o = u32x4{pk[0], pk[1], pk[2], pk[3]};
                 *(u32x4*)(o + 8) = u32x4{pk[4], pk[5], pk[6], pk[7]};
             } else {
                 float* o = (float*)g.out + n * g.K + k;
 #pragma unroll
-                for (int i = 0; i < 4; ++i) *(f32x4*)(o + 4 * i) = f32x4{m[u * 16 + 4 * i], m[u * 16 + 4 * i + 1], m[u * 16 + 4 * i + 2], m[u * 16 + 4 * i + 3]};
+                for (int i = 0; i < 4; ++i) *(f32x4*)(o + 4 * i) = f32x4{x[4 * i], x[4 * i + 1], x[4 * i + 2], x[4 * i + 3]};
             }
         }
-        return;
     }
+    if (!REQ) return;
     // ---- 3b. block absmax -> new scale -> e4m3 bytes
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
     if (lane == 0) sh_amax[wave] = amax;
     __syncthreads();
-    amax = fmaxf(fmaxf(sh_amax[0], sh_amax[1]), fmaxf(sh_amax[2], sh_amax[3]));
+    amax = fmaxf(fmaxf(fmaxf(sh_amax[0], sh_amax[1]), fmaxf(sh_amax[2], sh_amax[3])),
+                 fmaxf(fmaxf(sh_amax[4], sh_amax[5]), fmaxf(sh_amax[6], sh_amax[7])));
     const float s = fmaxf(amax / 448.0f, 1e-12f);
+    // one division per block; x * (1/s) is within 1.5 ulp of x / s, far inside an e4m3 rounding interval except
+    // for quotients within that distance of a rounding boundary
+    const float rs = 1.0f / s;
     if (tid == 0) g.scales_out[(int64_t)blockIdx.y * gridDim.x + blockIdx.x] = s;
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-        const int k = k0 + c0 + u * 16;
-        if (!(row_ok && k < g.K)) continue;
+    for (int h = 0; h < 2; ++h) {
+        const int k = k0 + h * 64 + rcol;
+        if (!(n < g.N && k < g.K)) continue;
         uint32_t pk[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             float y[4];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) y[e] = fminf(fmaxf(m[u * 16 + 4 * i + e] / s, -448.0f), 448.0f);
+            for (int e = 0; e < 4; ++e) y[e] = __builtin_amdgcn_fmed3f(m[h * 16 + 4 * i + e] * rs, -448.0f, 448.0f);
             uint32_t w = 0;
             w = __builtin_amdgcn_cvt_pk_fp8_f32(y[0], y[1], w, false);
             w = __builtin_amdgcn_cvt_pk_fp8_f32(y[2], y[3], w, true);
@@ -238,34 +282,45 @@ static double merge_bytes(const xq_weight* w, int mode) {
     return in + (mode == 0 ? 2.0 * n : mode == 1 ? 4.0 * n : in);
 }
 
-template <int FMT, int RP>
-static int launch_merge_one(const MergeArgs& g, dim3 grid, size_t lds, hipStream_t s, const char* who) {
+template <int FMT, int RP, bool REQ>
+static int launch_merge_one(const MergeArgs& g, dim3 grid, hipStream_t s, const char* who) {
+    // LDS: the four factor tiles, then the delta half tile in their place
+    constexpr size_t lds_f = (size_t)4 * MG_T * (RP + 8) * 2, lds_d = (size_t)MG_T * MG_HP * 4;
+    constexpr size_t lds = RP == 0 ? 16 : (lds_f > lds_d ? lds_f : lds_d);
     static bool attr_set = false;   // per instantiation
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute((const void*)merge_kernel<FMT, RP>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (!attr_set && lds > 64 * 1024) {
+        hipError_t e = hipFuncSetAttribute((const void*)merge_kernel<FMT, RP, REQ>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) {
             xq_set_error("%s: cannot raise the dynamic LDS limit: %s", who, hipGetErrorString(e));
             return XQ_ERR_LAUNCH;
         }
         attr_set = true;
     }
-    merge_kernel<FMT, RP><<<grid, 256, lds, s>>>(g);
+    merge_kernel<FMT, RP, REQ><<<grid, 512, lds, s>>>(g);
     return XQ_OK;
 }
 
-template <int FMT>
-static int launch_merge_fmt(const MergeArgs& g, dim3 grid, size_t lds, hipStream_t s, const char* who) {
+template <int FMT, bool REQ>
+static int launch_merge_fmt(const MergeArgs& g, dim3 grid, hipStream_t s, const char* who) {
     switch (g.r_pad) {
-        case 0: return launch_merge_one<FMT, 0>(g, grid, lds, s, who);
-        case 16: return launch_merge_one<FMT, 16>(g, grid, lds, s, who);
-        case 32: return launch_merge_one<FMT, 32>(g, grid, lds, s, who);
-        case 48: return launch_merge_one<FMT, 48>(g, grid, lds, s, who);
-        default: return launch_merge_one<FMT, 64>(g, grid, lds, s, who);
+        case 0: return launch_merge_one<FMT, 0, REQ>(g, grid, s, who);
+        case 16: return launch_merge_one<FMT, 16, REQ>(g, grid, s, who);
+        case 32: return launch_merge_one<FMT, 32, REQ>(g, grid, s, who);
+        case 48: return launch_merge_one<FMT, 48, REQ>(g, grid, s, who);
+        default: return launch_merge_one<FMT, 64, REQ>(g, grid, s, who);
     }
 }
 
+static int64_t merge_ws_bytes(int64_t N, int64_t K, int r) {
+    const int64_t rp = r <= 0 ? 0 : ((r + 15) / 16) * 16;
+    return 256 + 4 * (xq_cdiv(N, MG_T) + xq_cdiv(K, MG_T)) * MG_T * rp;   // four bf16 panels
+}
+
+extern "C" int64_t xq_merge_workspace_bytes(int64_t N, int64_t K, int r) { return merge_ws_bytes(N, K, r); }
+
 static int launch_merge(const xq_weight* w, const void* A, const void* B, int lora_dtype, int r, float scaling, int mode,
-                        void* out, void* packed_out, float* scales_out, hipStream_t stream, const char* who) {
+                        void* out, void* packed_out, float* scales_out, void* workspace, int64_t workspace_bytes,
+                        hipStream_t stream, const char* who) {
     int rc = xq_validate_weight(w, who);
     if (rc) return rc;
     XQ_REQUIRE(w->num_experts == 1, "%s: takes a single matrix", who);
@@ -282,14 +337,23 @@ static int launch_merge(const xq_weight* w, const void* A, const void* B, int lo
     g.N = (int32_t)w->rows; g.K = (int32_t)w->cols;
     g.A = A; g.B = B; g.lora_f32 = lora_dtype == XQ_DT_F32; g.r = r; g.r_pad = r <= 0 ? 0 : ((r + 15) / 16) * 16;
     g.scaling = scaling; g.mode = mode; g.out = out; g.packed_out = (uint8_t*)packed_out; g.scales_out = scales_out;
-    const size_t lds_f = (size_t)4 * MG_T * MG_FP * 2, lds_d = (size_t)MG_T * MG_DP * 4;
-    const size_t lds = lds_f > lds_d ? lds_f : lds_d;
+    const int64_t npad = xq_cdiv(w->rows, MG_T) * MG_T, kpad = xq_cdiv(w->cols, MG_T) * MG_T;
+    g.Bh = g.Bl = g.Ah = g.Al = nullptr;
+    if (g.r_pad > 0) {
+        XQ_REQUIRE(workspace && xq_aligned(workspace, 256) && workspace_bytes >= merge_ws_bytes(w->rows, w->cols, r),
+                   "%s: workspace missing, misaligned or smaller than xq_merge_workspace_bytes()", who);
+        bf16_t* p = (bf16_t*)workspace;
+        g.Bh = p; g.Bl = p + npad * g.r_pad; g.Ah = p + 2 * npad * g.r_pad; g.Al = g.Ah + kpad * g.r_pad;
+    }
     dim3 grid((unsigned)xq_cdiv(w->cols, MG_T), (unsigned)xq_cdiv(w->rows, MG_T));
     const bool timed = xq_profile_mark_begin(stream, merge_bytes(w, mode));
-    if (w->format == XQ_FMT_FP8) rc = launch_merge_fmt<XQ_FMT_FP8>(g, grid, lds, stream, who);
-    else if (w->format == XQ_FMT_INT4) rc = launch_merge_fmt<XQ_FMT_INT4>(g, grid, lds, stream, who);
-    else if (w->format == XQ_FMT_NF4) rc = launch_merge_fmt<XQ_FMT_NF4>(g, grid, lds, stream, who);
-    else rc = launch_merge_fmt<XQ_FMT_NVFP4>(g, grid, lds, stream, who);
+    if (g.r_pad > 0)
+        merge_prep_kernel<<<dim3((unsigned)xq_cdiv((npad + kpad) * g.r_pad, 256)), 256, 0, stream>>>(g, (int)npad, (int)kpad);
+    if (w->format == XQ_FMT_FP8) rc = mode == 2 ? launch_merge_fmt<XQ_FMT_FP8, true>(g, grid, stream, who)
+                                                : launch_merge_fmt<XQ_FMT_FP8, false>(g, grid, stream, who);
+    else if (w->format == XQ_FMT_INT4) rc = launch_merge_fmt<XQ_FMT_INT4, false>(g, grid, stream, who);
+    else if (w->format == XQ_FMT_NF4) rc = launch_merge_fmt<XQ_FMT_NF4, false>(g, grid, stream, who);
+    else rc = launch_merge_fmt<XQ_FMT_NVFP4, false>(g, grid, stream, who);
     if (timed) xq_profile_mark_end(stream);
     if (rc) return rc;
     XQ_CHECK_LAUNCH(who);
@@ -297,17 +361,19 @@ static int launch_merge(const xq_weight* w, const void* A, const void* B, int lo
 }
 
 extern "C" int xq_merge_dense(const xq_weight* w, const void* lora_A, const void* lora_B, int lora_dtype, int r,
-                              float scaling, void* out, int out_dtype, void* stream) {
+                              float scaling, void* out, int out_dtype, void* workspace, int64_t workspace_bytes,
+                              void* stream) {
     XQ_REQUIRE(out_dtype == XQ_DT_BF16 || out_dtype == XQ_DT_F32, "xq_merge_dense: bad out_dtype");
     XQ_REQUIRE(out && xq_aligned(out, 16), "xq_merge_dense: out is NULL or not 16-byte aligned");
     return launch_merge(w, lora_A, lora_B, lora_dtype, r, scaling, out_dtype == XQ_DT_BF16 ? 0 : 1, out, nullptr, nullptr,
-                        (hipStream_t)stream, "xq_merge_dense");
+                        workspace, workspace_bytes, (hipStream_t)stream, "xq_merge_dense");
 }
 
 extern "C" int xq_merge_requant_fp8(const xq_weight* w, const void* lora_A, const void* lora_B, int lora_dtype, int r,
-                                    float scaling, void* packed_out, float* scales_out, void* stream) {
+                                    float scaling, void* packed_out, float* scales_out, void* workspace,
+                                    int64_t workspace_bytes, void* stream) {
     XQ_REQUIRE(w && w->format == XQ_FMT_FP8, "xq_merge_requant_fp8: the weight must be block_fp8");
     XQ_REQUIRE(packed_out && scales_out && xq_aligned(packed_out, 16), "xq_merge_requant_fp8: NULL or misaligned output");
-    return launch_merge(w, lora_A, lora_B, lora_dtype, r, scaling, 2, nullptr, packed_out, scales_out, (hipStream_t)stream,
-                        "xq_merge_requant_fp8");
+    return launch_merge(w, lora_A, lora_B, lora_dtype, r, scaling, 2, nullptr, packed_out, scales_out, workspace, workspace_bytes,
+                        (hipStream_t)stream, "xq_merge_requant_fp8");
 }

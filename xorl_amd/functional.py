@@ -280,9 +280,11 @@ def merge_dense(qw: QuantWeight, lora_A: Optional[Tensor], lora_B: Optional[Tens
     B = lora_B[:, :r].contiguous() if r > 0 else None
     out = torch.empty(qw.rows, qw.cols, dtype=out_dtype, device=dev)
     w = qw.c()
+    ws_bytes = _C.lib().xq_merge_workspace_bytes(qw.rows, qw.cols, r)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     _C.check(_C.lib().xq_merge_dense(ctypes.byref(w), _C.ptr(A), _C.ptr(B), _lora_dt(A), r, float(scaling),
                                      out.data_ptr(), _C.XQ_DT_BF16 if out_dtype == torch.bfloat16 else _C.XQ_DT_F32,
-                                     _C.stream_ptr(dev)))
+                                     ws.data_ptr(), ws_bytes, _C.stream_ptr(dev)))
     return out
 
 
@@ -302,6 +304,9 @@ def merge_requant_fp8(qw: QuantWeight, lora_A: Optional[Tensor], lora_B: Optiona
     if scales_out is None:
         scales_out = torch.empty((qw.rows + 127) // 128, (qw.cols + 127) // 128, dtype=torch.float32, device=dev)
     w = qw.c()
+    ws_bytes = _C.lib().xq_merge_workspace_bytes(qw.rows, qw.cols, r)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     _C.check(_C.lib().xq_merge_requant_fp8(ctypes.byref(w), _C.ptr(A), _C.ptr(B), _lora_dt(A), r, float(scaling),
-                                           packed_out.data_ptr(), scales_out.data_ptr(), _C.stream_ptr(dev)))
+                                           packed_out.data_ptr(), scales_out.data_ptr(), ws.data_ptr(), ws_bytes,
+                                           _C.stream_ptr(dev)))
     return packed_out, scales_out
