@@ -136,3 +136,36 @@ def test_moe_zero_lora_equals_base(hip_device):
             for k in ("gate", "up", "down")}
     ex = R.moe_fwd_bwd(x, rw.to(torch.bfloat16), sel, banks["gate"], banks["up"], banks["down"], zero, m.scaling)
     assert R.max_rel_err(y.cpu(), ex["y"]) <= TOL
+
+
+def test_prequantized_checkpoint_load_on_device_matches_direct_quantisation(hip_device):
+    """HF-layout block-fp8 experts ([out, in] bytes + [out/128, in/128] scales) loaded through `_load_experts` on
+    the GPU give the same banks as quantizing the transposed weights directly, and the module then runs."""
+    from xorl_amd import quantize as Q
+    from xorl_amd.qlora import BlockFP8QLoRAMoeExperts
+
+    E, H, I, r = 4, 256, 384, 8
+    hf = {(e, p): gen((H, I) if p == "down_proj" else (I, H), 0.05, 900 + 7 * e + i)
+          for e in range(E) for i, p in enumerate(("gate_proj", "up_proj", "down_proj"))}
+    data = {}
+    for (e, p), w in hf.items():
+        b, s = Q.block_fp8_quantize_gkn(w.float().contiguous(), 128)      # per-128x128-block rule: layout agnostic
+        data[f"experts.{e}.{p}.weight"] = b
+        data[f"experts.{e}.{p}.weight_scale_inv"] = s
+    m = BlockFP8QLoRAMoeExperts(E, E, I, H, r=r, lora_alpha=2 * r).to(hip_device)
+    m._source_fqn = "experts"
+    m._load_experts(lambda k: data[k], {})
+    d = BlockFP8QLoRAMoeExperts(E, E, I, H, r=r, lora_alpha=2 * r)
+    d.load_weights(torch.stack([hf[(e, "gate_proj")].t() for e in range(E)]),
+                   torch.stack([hf[(e, "up_proj")].t() for e in range(E)]),
+                   torch.stack([hf[(e, "down_proj")].t() for e in range(E)]))
+    for p in ("gate", "up", "down"):
+        assert getattr(m, f"{p}_packed").device.type == "cuda"
+        assert torch.equal(getattr(m, f"{p}_packed").cpu(), getattr(d, f"{p}_packed")), p
+        assert torch.equal(getattr(m, f"{p}_block_scales").cpu(), getattr(d, f"{p}_block_scales")), p
+    rw, sel = _zipf_routing(64, E, 2, seed=3, empty=0)
+    x = gen((64, H), 1.0, 4, torch.bfloat16).to(hip_device)
+    with torch.no_grad():
+        y = m(x, rw.to(torch.bfloat16).to(hip_device), sel.to(hip_device))
+        y2 = d.to(hip_device)(x, rw.to(torch.bfloat16).to(hip_device), sel.to(hip_device))
+    assert torch.equal(y, y2)

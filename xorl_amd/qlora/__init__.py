@@ -23,3 +23,7 @@ __all__ = [
 from .moe_experts import BlockFP8QLoRAMoeExperts, NF4QLoRAMoeExperts, NvFP4QLoRAMoeExperts, QLoRAMoeExperts  # noqa: E402
 
 __all__ += ["QLoRAMoeExperts", "BlockFP8QLoRAMoeExperts", "NvFP4QLoRAMoeExperts", "NF4QLoRAMoeExperts"]
+
+from .utils import maybe_load_prequantized_qlora, maybe_requant_qlora  # noqa: E402
+
+__all__ += ["maybe_load_prequantized_qlora", "maybe_requant_qlora"]

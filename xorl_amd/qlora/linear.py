@@ -196,7 +196,10 @@ class QLoRALinear(LoraModule, nn.Module):
     def _to_uint8(t: Tensor) -> Tensor:
         """uint8 view: scales and codes are stored as bytes so that no mixed
         precision policy can cast them (the true dtype lives in _scale_dtypes)."""
-        return t.contiguous() if t.dtype == torch.uint8 else t.contiguous().view(torch.uint8)
+        t = t.contiguous()
+        if t.dim() and t.stride(-1) != 1:      # a size-1 last dimension may keep a foreign stride
+            t = t.clone(memory_format=torch.contiguous_format)
+        return t if t.dtype == torch.uint8 else t.view(torch.uint8)
 
     def _recover_tensor(self, buf: Tensor, original_dtype: torch.dtype) -> Tensor:
         return buf if original_dtype == torch.uint8 else buf.contiguous().view(original_dtype)

@@ -135,7 +135,10 @@ class QLoRAMoeExperts(LoraModule, nn.Module):
     # ------------------------------------------------------------------ storage helpers
     @staticmethod
     def _to_uint8(t: Tensor) -> Tensor:
-        return t.contiguous() if t.dtype == torch.uint8 else t.contiguous().view(torch.uint8)
+        t = t.contiguous()
+        if t.dim() and t.stride(-1) != 1:      # a size-1 last dimension may keep a foreign stride
+            t = t.clone(memory_format=torch.contiguous_format)
+        return t if t.dtype == torch.uint8 else t.view(torch.uint8)
 
     def _recover_tensor(self, buf: Tensor, original_dtype: torch.dtype) -> Tensor:
         return buf if original_dtype == torch.uint8 else buf.contiguous().view(original_dtype)
@@ -180,6 +183,59 @@ class QLoRAMoeExperts(LoraModule, nn.Module):
             for name, w in (("gate", gate), ("up", up), ("down", down)):
                 self._quantize_proj(name, w.float())
         self._weights_loaded = True
+
+    # ------------------------------------------------------------------ loading from a HF checkpoint
+    _HF_PROJ = (("gate", "gate_proj"), ("up", "up_proj"), ("down", "down_proj"))
+
+    def load_and_quantize_weights(self, weights_path: str, weight_map: Optional[dict] = None,
+                                  shard_cache: Optional[dict] = None) -> None:
+        """Fill the packed banks from the per-expert tensors `<_source_fqn>.<i>.<proj>.*` of a safetensors
+        checkpoint (qlora/modules/moe_experts.py:514-546).  `weights_path` is a local directory (or a hub id
+        resolvable by transformers' cache); `weight_map` is the index's key -> shard-file map; `shard_cache`
+        lets several modules share loaded shards.  Each subclass reads its own checkpoint format."""
+        if self._weights_loaded or self._source_fqn is None:
+            return
+        import os
+
+        import safetensors.torch
+
+        cache = shard_cache if shard_cache is not None else {}
+
+        def _load_tensor(key: str) -> Tensor:
+            if weight_map is not None:
+                shard = weight_map.get(key)
+                if shard is None:
+                    raise RuntimeError(f"Key {key} not found in checkpoint index")
+            else:
+                shard = "model.safetensors"
+            if shard not in cache:
+                path = os.path.join(weights_path, shard)
+                if not os.path.exists(path):
+                    from transformers.utils import cached_file
+
+                    path = cached_file(weights_path, shard)
+                cache[shard] = safetensors.torch.load_file(path, device="cpu")
+            tensors = cache[shard]
+            if key not in tensors:
+                raise RuntimeError(f"Key {key} not found in {shard}")
+            return tensors[key]
+
+        with torch.no_grad():
+            self._load_experts(_load_tensor, cache)
+        self._weights_loaded = True
+
+    def _load_experts(self, _load_tensor, _shard_cache) -> None:
+        raise NotImplementedError
+
+    def _load_device(self) -> torch.device:
+        """Where loaded banks go: the module's device, or the GPU for a module still on the meta device."""
+        dev = self.gate_proj_lora_B.device
+        if dev.type in ("meta",):
+            dev = torch.device("cuda") if torch.cuda.is_available() else torch.device("cpu")
+        return dev
+
+    def _expert_range(self):
+        return range(self.expert_offset, self.expert_offset + self.num_local_experts)
 
     def _bank(self, proj_name: str) -> QuantWeight:
         raise NotImplementedError
@@ -264,6 +320,24 @@ class BlockFP8QLoRAMoeExperts(QLoRAMoeExperts):
         scales = self._recover_tensor(*scales_dict["weight_block_scales"])
         return Q.block_fp8_dequantize_gkn(packed.view(torch.float8_e4m3fn).reshape(K, N), scales, 128)
 
+    def _load_experts(self, _load_tensor, _shard_cache) -> None:
+        """Pre-quantized block-fp8 experts (moe_experts.py:1074-1119).  Checkpoint: `weight` [N, K] e4m3 and
+        `weight_scale_inv` [N/128, K/128] per expert; bank: bytes [E, K, N] and fp32 scales [E, K/128, N/128] --
+        a pure transpose of bytes and scales, done once per projection on the device after one bulk copy."""
+        dev = self._load_device()
+        for proj, hf in self._HF_PROJ:
+            w8, sc = [], []
+            for i in self._expert_range():
+                prefix = f"{self._source_fqn}.{i}.{hf}"
+                w8.append(_load_tensor(f"{prefix}.weight").view(torch.uint8))
+                sc.append(_load_tensor(f"{prefix}.weight_scale_inv").float())
+            bank = torch.stack(w8).to(dev).transpose(1, 2).contiguous()
+            scales = torch.stack(sc).to(dev).transpose(1, 2).contiguous()
+            setattr(self, f"{proj}_packed", self._to_uint8(bank))
+            setattr(self, f"{proj}_block_scales", self._to_uint8(scales))
+            self._scale_dtypes[proj] = {"weight_block_scales": torch.float32}
+            _shard_cache.clear()
+
     def _bank(self, proj_name: str) -> QuantWeight:
         K, N = self._proj_dims(proj_name)
         return QuantWeight("block_fp8", _C.XQ_LAYOUT_GKN, getattr(self, f"{proj_name}_packed"),
@@ -304,6 +378,52 @@ class NvFP4QLoRAMoeExperts(QLoRAMoeExperts):
         bs = self._recover_tensor(*scales_dict["weight_block_scales"])
         g = self._recover_tensor(*scales_dict["weight_global_scale"])
         return Q.nvfp4_dequantize_gkn(packed, bs, g, K, N, 16)
+
+    def _load_experts(self, _load_tensor, _shard_cache) -> None:
+        """nvfp4 experts from a modelopt checkpoint (`weight` [N, K/2] u8, `weight_scale` [N, K/16] e4m3,
+        `weight_scale_2` fp32 scalar) or, when the first expert has no `weight_scale`, from a bf16 checkpoint
+        quantized here (moe_experts.py:869-971).  Either way the global scale is folded into fp32 block scales
+        (stored global = 1) and the per-expert amax seeds the EMA used by re-quantisation."""
+        dev = self._load_device()
+        E = self.num_local_experts
+        try:
+            _load_tensor(f"{self._source_fqn}.{self.expert_offset}.gate_proj.weight_scale")
+            prequantized = True
+        except RuntimeError:
+            prequantized = False
+        for proj, hf in self._HF_PROJ:
+            amax = []
+            if prequantized:
+                codes, bs, gs = [], [], []
+                for i in self._expert_range():
+                    prefix = f"{self._source_fqn}.{i}.{hf}"
+                    codes.append(_load_tensor(f"{prefix}.weight"))
+                    bs.append(_load_tensor(f"{prefix}.weight_scale").view(torch.uint8))
+                    g = _load_tensor(f"{prefix}.weight_scale_2").float().item()
+                    gs.append(g)
+                    amax.append(g * Q.FP4_E2M1_MAX * Q.FP8_E4M3_MAX)
+                g_dev = torch.tensor(gs, dtype=torch.float32, device=dev)
+                folded = torch.stack(bs).to(dev).view(torch.float8_e4m3fn).float() * g_dev[:, None, None]
+                bank = torch.stack(codes).to(dev).transpose(1, 2).contiguous()      # [E, K/2, N]: byte (k2, n) = K pair of column n
+                scales = folded.transpose(1, 2).contiguous()                        # [E, K/16, N] fp32
+            else:
+                codes, sc = [], []
+                for i in self._expert_range():
+                    w = _load_tensor(f"{self._source_fqn}.{i}.{hf}.weight").to(device=dev, dtype=torch.bfloat16).t().contiguous()
+                    a = w.float().abs().max().reshape(1)
+                    amax.append(a.item())
+                    packed, block_scales, global_scale = Q.nvfp4_quantize_gkn(w, self.quant_group_size, global_amax=a)
+                    codes.append(self._to_uint8(packed))
+                    sc.append((block_scales.float() * global_scale.float()).contiguous())
+                    _shard_cache.clear()
+                bank, scales = torch.stack(codes), torch.stack(sc)
+            setattr(self, f"{proj}_packed", self._to_uint8(bank))
+            setattr(self, f"{proj}_block_scales", self._to_uint8(scales))
+            setattr(self, f"{proj}_global_scale", self._to_uint8(torch.ones(E, 1, dtype=torch.float32, device=dev)))
+            self._scale_dtypes[proj] = {"weight_block_scales": torch.float32, "weight_global_scale": torch.float32}
+            self._ema_amax[proj] = torch.tensor(amax, dtype=torch.float32, device=dev)
+            if prequantized:
+                _shard_cache.clear()
 
     def _bank(self, proj_name: str) -> QuantWeight:
         K, N = self._proj_dims(proj_name)
@@ -352,6 +472,15 @@ class NF4QLoRAMoeExperts(QLoRAMoeExperts):
     def _dequantize_2d(self, packed: Tensor, scales_dict: dict, K: int, N: int) -> Tensor:
         scales = self._recover_tensor(*scales_dict["weight_scales"])
         return Q.nf4_dequantize_gkn(packed, scales, K, N, self.quant_group_size)
+
+    def _load_experts(self, _load_tensor, _shard_cache) -> None:
+        """bf16 experts `[out, in]` -> transposed to `[in, out]` and quantized to NF4 along K
+        (moe_experts.py:1213-1236); there is no pre-quantized NF4 checkpoint format."""
+        dev = self._load_device()
+        for proj, hf in self._HF_PROJ:
+            w = [_load_tensor(f"{self._source_fqn}.{i}.{hf}.weight").t().contiguous().float() for i in self._expert_range()]
+            self._quantize_proj(proj, torch.stack(w).to(dev))
+            _shard_cache.clear()
 
     def _bank(self, proj_name: str) -> QuantWeight:
         K, N = self._proj_dims(proj_name)
