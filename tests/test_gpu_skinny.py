@@ -5,7 +5,8 @@ import pytest
 import torch
 
 from oracle import recipe as R
-from tests.util_cases import gen, make_dense_module
+from oracle import decode_np as NP
+from tests.util_cases import bits_to_bf16, gen, make_dense_module
 
 pytestmark = pytest.mark.gpu
 TOL = 1e-2
@@ -110,3 +111,44 @@ def test_skinny_forward_under_hip_graph(hip_device):
         torch.cuda.synchronize()
         for y, e in zip(again, eager):
             assert torch.equal(y, e)
+
+
+@pytest.mark.parametrize("M", [1, 24, 40])
+def test_skinny_scale_storage_variants(hip_device, M):
+    """Scale storages the default modules do not produce: nvfp4 with fp32 block scales and a folded global scale
+    (pre-quantized checkpoints), int4 with fp32 scales and with groups shorter than a 128-element chunk."""
+    from xorl_amd import quantize as Q
+    from xorl_amd.qlora import Int4QLoRALinear, QLoRALinear
+
+    N, K, r = 384, 1024, 16
+    x = gen((M, K), 1.0, 700 + M, torch.bfloat16)
+    w = gen((N, K), 0.02, 701)
+    A, B = gen((r, K), 0.02, 702), gen((N, r), 0.02, 703)
+
+    def check(m, w_ref):
+        m = m.to(hip_device)
+        with torch.no_grad():
+            m.lora_A.copy_(A)
+            m.lora_B.copy_(B)
+            y = m(x.to(hip_device))
+        ex = R.linear_fwd_bwd_exact(x, w_ref, A, B, m.scaling)
+        assert R.max_rel_err(y.cpu(), ex["y"]) <= TOL
+        assert torch.equal(m._dequantize_weight().cpu().reshape(N, K), w_ref)      # same bytes, same decode
+
+    # nvfp4: fold the global scale into fp32 block scales, as the checkpoint loaders do
+    packed, bs, g = Q.nvfp4_quantize(w, 16)
+    folded = (bs.float() * g.float()).reshape(N, K // 16).contiguous()
+    m = QLoRALinear.from_quantized(packed.reshape(N, K // 2), weight_block_scales=folded,
+                                   weight_global_scale=torch.ones(1), in_features=K, out_features=N, r=r,
+                                   lora_alpha=2 * r, quant_format="nvfp4")
+    check(m, bits_to_bf16(NP.nvfp4_decode_flat(packed.numpy().reshape(N, K // 2), folded.numpy(), 1.0, N, K)))
+
+    # int4, reference codec (fp32 scales), group 128 and group 32
+    for group in (128, 32):
+        lin = torch.nn.Linear(K, N, bias=False)
+        with torch.no_grad():
+            lin.weight.copy_(w)
+        m = Int4QLoRALinear.from_module(lin, r=r, lora_alpha=2 * r, quant_group_size=group, symmetric=False)
+        pk = m.packed_weight_f32.detach().contiguous().view(torch.uint8).numpy()
+        sc = m.weight_scales.contiguous().view(torch.float32).numpy()
+        check(m, bits_to_bf16(NP.int4_decode_flat(pk, sc, N, K, group)))
