@@ -38,7 +38,13 @@ BF16_MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense bf16, published
 # 256 MiB -> 256 MiB copy; the files under profiles/ hold the figures and the commands).  A config that
 # has no counter run reports null.  --traffic-bytes overrides.
 MEASURED_TRAFFIC_BYTES = {
-    1: 904.9 * 2 ** 20,   # gemm_256_kernel<fp8>: mean of the forward (927.9 MiB) and dgrad (882.0 MiB) launches
+    0: 45.6 * 2 ** 20,     # gemm_256_kernel<int4, T=128>: mean of the forward and dgrad launches
+    1: 905.4 * 2 ** 20,    # gemm_256_kernel<fp8>: mean of the forward and dgrad launches
+    2: 227.8 * 2 ** 20,    # gemm_256_kernel<nvfp4> / gemm_tile_kernel<nvfp4>: mean over the 8 launches of a step
+    3: 1032.2 * 2 ** 20,   # gemm_256_kernel<fp8, grouped>: mean over the 6 launches of a step
+    4: 41.0 * 2 ** 20,     # skinny_split_kernel + skinny_epilogue_kernel: mean per forward over the 32 cases (includes
+                           # the fp32 partial tiles written and read back: 23.3 MiB of it are algorithmic)
+    5: 134.4 * 2 ** 20,    # merge_prep_kernel + merge_kernel<fp8>: mean per call (re-quantise 96 MiB, publish 144 MiB algorithmic)
 }
 
 
