@@ -51,10 +51,12 @@ static int launch_256(const G256Args& f, bool cc, bool grouped, int T, dim3 grid
     return grouped ? launch_256_t<FMT, false, true>(f, T, grid, s, who) : launch_256_t<FMT, false, false>(f, T, grid, s, who);
 }
 
-// C[rows, Nout] = A . op(deq(W)) (+ su . Lr^T) (+ bias); see xq_gemm_tile.h
-int launch_tile_gemm(const xq_weight* w, bool contract_cols, const bf16_t* A, int64_t lda, int64_t n_rows,
-                     const int32_t* offsets, const int32_t* tile_offsets, const bf16_t* su, const bf16_t* lora_right,
-                     int r_pad, const bf16_t* bias, bf16_t* C, int64_t ldc, hipStream_t stream, const char* who) {
+// C[rows, Nout] = A . op(deq(W)) (+ su . Lr^T) (+ bias); see xq_gemm_tile.h.  force_T = 256 / 128 fixes the tile
+// size of the pipelined kernel, 0 leaves it to the selection policy.
+static int launch_tile_gemm_t(const xq_weight* w, bool contract_cols, const bf16_t* A, int64_t lda, int64_t n_rows,
+                              const int32_t* offsets, const int32_t* tile_offsets, const bf16_t* su, const bf16_t* lora_right,
+                              int r_pad, const bf16_t* bias, bf16_t* C, int64_t ldc, hipStream_t stream, const char* who,
+                              int force_T) {
     TileArgs g;
     g.A = A; g.lda = lda; g.C = C; g.ldc = ldc;
     g.packed = (const uint8_t*)w->packed;
@@ -88,7 +90,30 @@ int launch_tile_gemm(const xq_weight* w, bool contract_cols, const bf16_t* A, in
                             (w->layout == XQ_LAYOUT_FLAT && (1 << gshift) == g.group && g.group >= 16);
         const bool big = grouped ? (n_rows >= 128ll * w->num_experts && n_rows >= 8192)
                                  : (xq_cdiv(n_rows, 256) * xq_cdiv(g.Nout, 256) >= 96);
-        const int T = g_tile_policy == 2 ? 256 : g_tile_policy == 3 ? 128 : (big ? 256 : 128);
+        const int T = force_T ? force_T : g_tile_policy == 2 ? 256 : g_tile_policy == 3 ? 128 : (big ? 256 : 128);
+        // A dense launch of 256x256 tiles whose last round would fill only part of the chip: the leading tile rows
+        // that make whole rounds keep the large tiles, the remaining rows run as a second launch of 128x128 tiles
+        // (two of those blocks share a CU).  Costs in units of one round of large tiles: a launch of small tiles
+        // takes about 0.54 (up to one block per CU) or 0.7 (up to two per CU) of it.
+        if (!grouped && fmt_ok && g_tile_policy == 0 && force_T == 0 && T == 256) {
+            const int64_t tr = xq_cdiv(n_rows, 256), tc = xq_cdiv(g.Nout, 256), cus = 256;
+            const int64_t full = tr * tc / cus, rem = tr * tc - full * cus;
+            const int64_t keep = full * cus / tc;                  // tile rows that stay on large tiles
+            if (rem > 0 && keep > 0 && keep < tr) {
+                const int64_t tail_rows = n_rows - keep * 256;
+                const int64_t n128 = xq_cdiv(tail_rows, 128) * xq_cdiv(g.Nout, 128);
+                const double tail = n128 <= cus ? 0.54 : 0.7 * (double)xq_cdiv(n128, 2 * cus);
+                if ((double)xq_cdiv(keep * tc, cus) + tail < (double)(full + 1) - 0.2) {
+                    const int64_t head = keep * 256;
+                    const int rc = launch_tile_gemm_t(w, contract_cols, A, lda, head, nullptr, nullptr, su, lora_right, r_pad,
+                                                      bias, C, ldc, stream, who, 256);
+                    if (rc) return rc;
+                    return launch_tile_gemm_t(w, contract_cols, A + head * lda, lda, tail_rows, nullptr, nullptr,
+                                              su ? su + head * r_pad : nullptr, lora_right, r_pad, bias, C + head * ldc, ldc,
+                                              stream, who, 128);
+                }
+            }
+        }
         const int64_t tiles_m = xq_cdiv(n_rows, T) + (grouped ? w->num_experts : 0);
         const int64_t tiles_n = xq_cdiv(g.Nout, T);
         if (fmt_ok && g_tile_policy != 1 && tiles_m * tiles_n < (1ll << 31)) {
@@ -130,6 +155,13 @@ int launch_tile_gemm(const xq_weight* w, bool contract_cols, const bf16_t* A, in
     if (timed) xq_profile_mark_end(stream);
     XQ_CHECK_LAUNCH(who);
     return XQ_OK;
+}
+
+int launch_tile_gemm(const xq_weight* w, bool contract_cols, const bf16_t* A, int64_t lda, int64_t n_rows,
+                     const int32_t* offsets, const int32_t* tile_offsets, const bf16_t* su, const bf16_t* lora_right,
+                     int r_pad, const bf16_t* bias, bf16_t* C, int64_t ldc, hipStream_t stream, const char* who) {
+    return launch_tile_gemm_t(w, contract_cols, A, lda, n_rows, offsets, tile_offsets, su, lora_right, r_pad, bias, C, ldc,
+                              stream, who, 0);
 }
 
 static inline int64_t align256(int64_t b) { return (b + 255) & ~(int64_t)255; }
