@@ -81,15 +81,37 @@ def test_nf4_gkn(hip_device, K, N, group):
     assert np.array_equal(_bits(got), NP.nf4_decode_gkn(packed, scales, K, N, group))
 
 
-def test_nf4_quantize_on_device_matches_oracle(hip_device):
-    # the package's torch quantizer run on the GPU emits the oracle's bytes
+def test_quantizers_on_device_match_oracle(hip_device):
+    """The package's torch quantizers run on the GPU (bank loading, re-quantisation, format conversion do that) emit
+    the oracle's bytes: every quotient in them is a tensor-by-tensor IEEE division, not the reciprocal
+    multiplication torch substitutes for Python-scalar operands."""
     from xorl_amd import quantize as Q
 
     g = torch.Generator().manual_seed(9)
-    w = torch.randn(64, 512, generator=g) * 0.02
-    p, s = Q.nf4_quantize(w.to(hip_device), 64)
+    w = torch.randn(256, 512, generator=g) * 0.02
+    wd = w.to(hip_device)
+    p, s = Q.nf4_quantize(wd, 64)
     pc, sc = C.nf4_quantize_flat(w.numpy(), 64)
     assert np.array_equal(p.cpu().numpy(), pc.reshape(-1)) and np.array_equal(s.cpu().numpy(), sc.reshape(-1))
+    p, s = Q.int4_quantize(wd, 128)
+    pc, sc = C.int4_quantize_flat(w.numpy(), 128)
+    assert np.array_equal(p.cpu().numpy(), pc) and np.array_equal(s.cpu().numpy(), sc)
+    p, s = Q.int4_quantize_sym(wd, 128)
+    pc, sc = C.int4_quantize_sym_flat(w.numpy(), 128)
+    assert np.array_equal(p.cpu().numpy(), pc)
+    assert np.array_equal(s.cpu().view(torch.int16).numpy().view(np.uint16), sc)
+    p, bs, gs = Q.nvfp4_quantize(wd)
+    pc, bsc, gc = C.nvfp4_quantize_flat(w.numpy())
+    assert np.array_equal(p.cpu().numpy().reshape(pc.shape), pc)
+    assert np.array_equal(bs.cpu().view(torch.uint8).numpy().reshape(bsc.shape), bsc) and gs.item() == gc
+    p, bs, gs = Q.nvfp4_quantize_gkn(wd.t().contiguous())
+    pc, bsc, gc = C.nvfp4_quantize_gkn(w.t().contiguous().numpy())
+    assert np.array_equal(p.cpu().numpy(), pc) and np.array_equal(bs.cpu().view(torch.uint8).numpy(), bsc) and gs.item() == gc
+    for shape in ((256, 512), (200, 300)):
+        x = w[: shape[0], : shape[1]].contiguous()
+        y, s = Q.block_fp8_quantize_gkn(x.to(hip_device))
+        yc, sc = C.fp8_quantize(x.numpy())
+        assert np.array_equal(y.cpu().view(torch.uint8).numpy(), yc) and np.array_equal(s.cpu().numpy(), sc)
 
 
 @pytest.mark.parametrize("rows,cols,e4m3", [(64, 256, True), (64, 256, False), (3, 48, True), (8192, 5120, True)])

@@ -169,3 +169,50 @@ def test_prequantized_checkpoint_load_on_device_matches_direct_quantisation(hip_
         y = m(x, rw.to(torch.bfloat16).to(hip_device), sel.to(hip_device))
         y2 = d.to(hip_device)(x, rw.to(torch.bfloat16).to(hip_device), sel.to(hip_device))
     assert torch.equal(y, y2)
+
+
+@pytest.mark.parametrize("src,dst", [("block_fp8", "nvfp4"), ("nvfp4", "block_fp8")])
+def test_inline_buffer_converts_between_checkpoint_and_module_format(hip_device, src, dst):
+    """A checkpoint in one format streamed into modules of the other: the buffer decodes with the source format's
+    kernel and re-quantizes; the pairs it hands back equal the CPU quantizer run on the oracle's decode."""
+    from xorl_amd import quantize as Q
+    from xorl_amd.qlora import BlockFP8QLoRALinear, NvFP4QLoRALinear
+    from xorl_amd.qlora.inline_buffers import QLoRAWeightBuffer
+
+    N, K = 256, 384
+    w = gen((N, K), 0.05, 77)
+    tensors = {}
+    if src == "block_fp8":
+        b, s = Q.block_fp8_quantize_gkn(w, 128)
+        tensors = {"m.proj.weight": b, "m.proj.weight_scale_inv": s}
+        deq = torch.from_numpy(NP.fp8_decode(b.view(torch.uint8).numpy(), s.numpy(), N, K)[0])     # fp32, as decoded
+    else:
+        codes, bs, g = Q.nvfp4_quantize(w, 16)
+        tensors = {"m.proj.weight": codes.reshape(N, K // 2), "m.proj.weight_scale": bs.reshape(N, K // 16),
+                   "m.proj.weight_scale_2": g.reshape(())}
+        folded = (bs.reshape(N, K // 16).float() * g.float()).numpy()           # what the buffer folds before decoding
+        deq = bits_to_bf16(NP.nvfp4_decode_flat(codes.reshape(N, K // 2).numpy(), folded, 1.0, N, K))
+
+    class Holder(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.proj = (NvFP4QLoRALinear if dst == "nvfp4" else BlockFP8QLoRALinear)(K, N, r=4, lora_alpha=4)
+            self.proj._is_prequantized, self.proj._source_fqn, self.proj._source_quant_format = True, "m.proj", src
+
+    model = Holder()
+    buf = QLoRAWeightBuffer(model)
+    assert buf.source_format == src
+    pairs = None
+    for k, t in tensors.items():
+        pairs = buf.try_consume(k, t)
+    got = dict(pairs)
+    if dst == "nvfp4":
+        codes, bs, g = Q.nvfp4_quantize(deq, 16, global_amax=deq.float().abs().max().reshape(1))
+        assert torch.equal(got["proj.packed_weight_f32"].contiguous().view(torch.uint8).flatten(), codes.flatten())
+        assert torch.equal(got["proj.weight_block_scales"].contiguous().view(torch.float32).flatten(), bs.float().flatten())
+        assert torch.equal(got["proj.weight_global_scale"].contiguous().view(torch.float32), g.float().reshape(-1))
+    else:
+        b, s = Q.block_fp8_quantize_gkn(deq.float(), 128)
+        assert torch.equal(got["proj.packed_weight_f32"].contiguous().view(torch.uint8).flatten(), b.view(torch.uint8).flatten())
+        assert torch.equal(got["proj.weight_block_scales"].contiguous().view(torch.float32).flatten(), s.flatten())
+    assert got["proj.packed_weight_f32"].shape == model.proj.packed_weight_f32.shape

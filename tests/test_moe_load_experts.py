@@ -224,3 +224,152 @@ def test_model_level_prequantized_load_and_requant(tmp_path):
         maybe_load_prequantized_qlora(model, str(tmp_path))
     with pytest.raises(RuntimeError, match="model.safetensors.index.json"):
         maybe_load_prequantized_qlora(model, str(tmp_path / "nowhere"))
+
+
+# ---------------------------------------------------------------------------------------------------------
+# streaming ("inline") buffers: the same packed state as the module-at-a-time loader, whatever order the keys
+# arrive in (the reference's contracts: checkpoint_handlers/buffers.py:617-776 dense, :925-1200 experts)
+def _dense_model(K):
+    from xorl_amd.qlora import BlockFP8QLoRALinear, NvFP4QLoRALinear
+
+    class Layer(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.o_proj = BlockFP8QLoRALinear(K, 256, r=4, lora_alpha=4)
+            self.o_proj._is_prequantized, self.o_proj._source_fqn = True, "model.layers.0.self_attn.o_proj"
+            self.o_proj._source_quant_format = "block_fp8"
+            self.qkv_proj = NvFP4QLoRALinear(K, 256, r=4, lora_alpha=4)
+            self.qkv_proj._is_prequantized, self.qkv_proj._source_fqn = True, "model.layers.0.self_attn"
+            self.qkv_proj._merge_sources = ("q_proj", "k_proj", "v_proj")
+            self.qkv_proj._source_quant_format = "nvfp4"
+
+    return Layer()
+
+
+@pytest.mark.parametrize("order_seed", [0, 1, 2])
+def test_inline_dense_buffers_match_the_deferred_loader(order_seed):
+    from xorl_amd.qlora.inline_buffers import BlockFP8WeightBuffer, NvFP4WeightBuffer, QLoRAWeightBuffer
+
+    K = 256
+    tensors = {}
+    wo, so = _fp8_tensors(1, 256, K, seed=21)
+    tensors["model.layers.0.self_attn.o_proj.weight"] = wo[0]
+    tensors["model.layers.0.self_attn.o_proj.weight_scale_inv"] = so[0]
+    for name, n in {"q_proj": 128, "k_proj": 64, "v_proj": 64}.items():
+        codes, bs, gs = _nvfp4_tensors(1, n, K, seed=len(name) + n)
+        tensors[f"model.layers.0.self_attn.{name}.weight"] = codes[0]
+        tensors[f"model.layers.0.self_attn.{name}.weight_scale"] = bs[0]
+        tensors[f"model.layers.0.self_attn.{name}.weight_scale_2"] = gs[0]
+        tensors[f"model.layers.0.self_attn.{name}.input_scale"] = torch.ones(1)      # not a piece of the format
+    tensors["model.norm.weight"] = torch.ones(4)
+
+    # expected: the module-at-a-time loader on a twin model
+    twin = _dense_model(K)
+    for mod in (twin.o_proj, twin.qkv_proj):
+        mod._load_prequantized(lambda k: tensors[k])
+
+    model = _dense_model(K)
+    # the factory picks the format of the first pre-quantized module; each format gets its own buffer
+    assert isinstance(QLoRAWeightBuffer(model), BlockFP8WeightBuffer)
+    bufs = [BlockFP8WeightBuffer(model), NvFP4WeightBuffer(model)]
+    keys = list(tensors)
+    order = torch.randperm(len(keys), generator=torch.Generator().manual_seed(order_seed)).tolist()
+    got, complete = {}, 0
+    for i in order:
+        key = keys[i]
+        claimed = [b.try_consume(key, tensors[key]) for b in bufs if b.is_qlora_key(key)]
+        if key.endswith("input_scale") or key == "model.norm.weight":
+            assert claimed == [] and all(b.try_consume(key, tensors[key]) is None for b in bufs)
+            continue
+        assert len(claimed) == 1                      # exactly one buffer owns a quantized key
+        if claimed[0]:
+            complete += 1
+            got.update(dict(claimed[0]))
+    assert complete == 2
+    assert set(got) == {"o_proj.packed_weight_f32", "o_proj.weight_block_scales", "qkv_proj.packed_weight_f32",
+                        "qkv_proj.weight_block_scales", "qkv_proj.weight_global_scale"}
+    sd = dict(twin.named_parameters()) | dict(twin.named_buffers())
+    for name, t in got.items():
+        want = sd[name]
+        assert t.dtype == want.dtype and t.shape == want.shape, name
+        assert torch.equal(t.contiguous().view(torch.uint8), want.detach().contiguous().view(torch.uint8)), name
+    # a reader dispatches the pairs into the module, then the buffers record what the bytes mean
+    with torch.no_grad():
+        for name, t in got.items():
+            mod, attr = name.split(".")
+            tgt = getattr(getattr(model, mod), attr)
+            if tgt.shape == t.shape:
+                tgt.copy_(t)
+            else:
+                setattr(getattr(model, mod), attr, t)
+    for b in bufs:
+        b.set_inline_metadata()
+    assert model.qkv_proj._inline_loaded and not model.o_proj._inline_loaded       # block_fp8 is filled again from disk
+    assert model.qkv_proj._scale_dtypes == twin.qkv_proj._scale_dtypes
+    assert torch.equal(model.qkv_proj._ema_amax, twin.qkv_proj._ema_amax) and model.o_proj._ema_amax is None
+
+
+@pytest.mark.parametrize("fmt", ["block_fp8", "nvfp4"])
+def test_inline_expert_buffer_fills_the_local_range(fmt):
+    """Two ranks' worth of experts stream by in a shuffled order; rank 1 keeps experts [2, 4), counts the others
+    (some offered as tensors, some reported as skipped) and ends with the bank the module-at-a-time loader builds."""
+    from xorl_amd.qlora.inline_buffers import QLoRAExpertBuffer, parse_expert_full_key
+
+    E, I, H = 4, 128, 256
+    cls = BlockFP8QLoRAMoeExperts if fmt == "block_fp8" else NvFP4QLoRAMoeExperts
+    tensors = {}
+    for hf in HF:
+        N, K = (H, I) if hf == "down_proj" else (I, H)
+        if fmt == "block_fp8":
+            w, sc = _fp8_tensors(E, N, K, seed=len(hf))
+            for e in range(E):
+                tensors[f"model.layers.3.mlp.experts.{e}.{hf}.weight"] = w[e]
+                tensors[f"model.layers.3.mlp.experts.{e}.{hf}.weight_scale_inv"] = sc[e]
+        else:
+            codes, bs, gs = _nvfp4_tensors(E, N, K, seed=len(hf))
+            for e in range(E):
+                tensors[f"model.layers.3.mlp.experts.{e}.{hf}.weight"] = codes[e]
+                tensors[f"model.layers.3.mlp.experts.{e}.{hf}.weight_scale"] = bs[e]
+                tensors[f"model.layers.3.mlp.experts.{e}.{hf}.weight_scale_2"] = gs[e]
+                tensors[f"model.layers.3.mlp.experts.{e}.{hf}.input_scale"] = torch.ones(1)
+    assert parse_expert_full_key("model.layers.3.mlp.experts.2.up_proj.weight_scale") == (3, 2, "up", "weight_scale")
+    assert parse_expert_full_key("model.layers.3.mlp.gate.weight") is None
+
+    def make():
+        class Model(torch.nn.Module):
+            def __init__(self):
+                super().__init__()
+                self.layers = torch.nn.ModuleList([torch.nn.Identity() for _ in range(4)])
+                m = cls(2, 2, I, H, r=4, lora_alpha=4)      # this rank's two experts
+                m.expert_offset, m._source_fqn = 2, "model.layers.3.mlp.experts"
+                self.layers[3] = m
+        return Model()
+
+    twin = make()
+    twin.layers[3]._load_experts(lambda k: tensors[k], {})
+    model = make()
+    buf = QLoRAExpertBuffer(model, ep_rank=1, ep_size=2, num_experts=E)
+    assert buf is not None and (buf.expert_start, buf.expert_end) == (2, 4)
+    keys = list(tensors)
+    order = torch.randperm(len(keys), generator=torch.Generator().manual_seed(5)).tolist()
+    assert buf.try_consume("model.layers.0.mlp.experts.0.gate_proj.weight", torch.zeros(1)) is None   # no module there
+    for n, i in enumerate(order):
+        key = keys[i]
+        expert = parse_expert_full_key(key)[1]
+        if expert < 2 and n % 2:
+            assert buf.count_skipped(key) == []                   # the reader never loaded this tensor
+        else:
+            assert buf.try_consume(key, tensors[key]) == []
+        if n == len(order) // 2:
+            assert buf.get_pending() and not model.layers[3]._weights_loaded
+    assert buf.get_pending() == [] and model.layers[3]._weights_loaded
+    got, want = model.layers[3], twin.layers[3]
+    for p in ("gate", "up", "down"):
+        assert torch.equal(getattr(got, f"{p}_packed"), getattr(want, f"{p}_packed")), p
+        assert torch.equal(getattr(got, f"{p}_block_scales"), getattr(want, f"{p}_block_scales")), p
+        assert got._scale_dtypes[p] == want._scale_dtypes[p]
+        if fmt == "nvfp4":
+            assert torch.equal(getattr(got, f"{p}_global_scale"), getattr(want, f"{p}_global_scale"))
+            assert torch.equal(got._ema_amax[p], want._ema_amax[p])
+    # a model whose expert modules are all loaded needs no buffer
+    assert QLoRAExpertBuffer(model, 1, 2, E) is None

@@ -63,3 +63,32 @@ def test_block_fp8_quantizer_matches_oracle():
         yc, sc = C.fp8_quantize(w.numpy())
         assert np.array_equal(y.view(torch.uint8).numpy(), yc)
         assert np.array_equal(s.numpy(), sc)
+
+
+def test_nvfp4_multiplier_is_one_ieee_division():
+    """The codes are taken from x * fl(6 / amax): ONE division.  `6.0 / tensor` in torch is reciprocal-then-multiply
+    (two roundings, a different multiplier for about a third of all amax values), which moves an element across an
+    encode threshold only once in millions of random draws -- so the cases are constructed: for blocks whose two
+    multipliers differ, an element is placed where the products fall on opposite sides of a threshold."""
+    rng = np.random.default_rng(3)
+    amax = (rng.random(200000, dtype=np.float32) * 4 + 0.5).astype(np.float32)
+    m1 = (np.float32(6.0) / amax).astype(np.float32)
+    m2 = ((np.float32(1.0) / amax).astype(np.float32) * np.float32(6.0)).astype(np.float32)
+    idx = np.nonzero(m1 != m2)[0]
+    assert idx.size > 1000
+    thresholds = np.array([0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0], dtype=np.float32)
+    blocks = []
+    for i in idx[:20000]:
+        t = thresholds[i % 7]
+        x0 = np.float32(t / m1[i])
+        for x in (x0, np.nextafter(x0, np.float32(0)), np.nextafter(x0, np.float32(8))):
+            if x < amax[i] and (np.float32(x * m1[i]) >= t) != (np.float32(x * m2[i]) >= t):
+                b = np.zeros(16, dtype=np.float32)
+                b[0], b[1] = amax[i], x
+                blocks.append(b)
+                break
+    assert len(blocks) >= 20, len(blocks)
+    x = torch.from_numpy(np.stack(blocks))
+    packed, bs, g = Q.nvfp4_quantize(x, 16)
+    po, so, go = C.nvfp4_quantize_flat(x.numpy())
+    assert np.array_equal(packed.numpy().reshape(po.shape), po)

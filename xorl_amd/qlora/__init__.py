@@ -27,3 +27,16 @@ __all__ += ["QLoRAMoeExperts", "BlockFP8QLoRAMoeExperts", "NvFP4QLoRAMoeExperts"
 from .utils import maybe_load_prequantized_qlora, maybe_requant_qlora  # noqa: E402
 
 __all__ += ["maybe_load_prequantized_qlora", "maybe_requant_qlora"]
+
+from .inline_buffers import (  # noqa: E402
+    BlockFP8QLoRAExpertBuffer,
+    BlockFP8WeightBuffer,
+    NvFP4QLoRAExpertBuffer,
+    NvFP4WeightBuffer,
+    QLoRAExpertBuffer,
+    QLoRAWeightBuffer,
+    parse_expert_full_key,
+)
+
+__all__ += ["QLoRAWeightBuffer", "NvFP4WeightBuffer", "BlockFP8WeightBuffer", "QLoRAExpertBuffer",
+            "NvFP4QLoRAExpertBuffer", "BlockFP8QLoRAExpertBuffer", "parse_expert_full_key"]

@@ -286,8 +286,36 @@ class QLoRALinear(LoraModule, nn.Module):
 
         self._load_prequantized(_load)
 
+    # suffixes of the checkpoint tensors one source projection contributes (empty: no pre-quantized format)
+    _prequant_suffixes: Tuple[str, ...] = ()
+
+    def _prequant_sources(self) -> Tuple[str, ...]:
+        """Checkpoint prefixes this module is assembled from: its own, or one per merged projection."""
+        if self._merge_sources is not None:
+            return tuple(f"{self._source_fqn}.{p}" for p in self._merge_sources)
+        return (self._source_fqn,)
+
     def _load_prequantized(self, _load_tensor) -> None:
+        """Fetch this module's checkpoint tensors through `_load_tensor(key)` and install them."""
+        if not self._prequant_suffixes:
+            raise NotImplementedError
+        pieces = [{sfx: _load_tensor(f"{q}.{sfx}") for sfx in self._prequant_suffixes} for q in self._prequant_sources()]
+        self._install_prequantized(self._pack_prequantized(pieces))
+
+    def _pack_prequantized(self, pieces) -> dict:
+        """`pieces`: one {suffix: tensor} mapping per source projection, in row order.  Returns the module state
+        they make: "packed" (uint8 rows), one entry per scale buffer (true dtype), "scale_dtypes", "ema_amax"."""
         raise NotImplementedError
+
+    def _install_prequantized(self, state: dict) -> None:
+        dev = self.lora_A.device if self.lora_A.device.type != "meta" else torch.device("cuda")
+        self._write_packed_weight(state["packed"].to(dev))
+        self._scale_dtypes = dict(state["scale_dtypes"])
+        for name in self._scale_dtypes:
+            setattr(self, name, self._to_uint8(state[name]).to(dev))
+        ema = state.get("ema_amax")
+        self._ema_amax = None if ema is None else ema.to(dev)
+        self._aqn_step_cache = None
 
     def quantize_weight(self) -> None:
         """Deferred quantization: turn the (FSDP-loaded) `weight` into packed form."""
@@ -467,21 +495,17 @@ class BlockFP8QLoRALinear(QLoRALinear):
         step = s.repeat_interleave(128, 0).repeat_interleave(128, 1)[: self.out_features, : self.in_features]
         return (0.125 * step).contiguous()
 
-    def _load_prequantized(self, _load_tensor) -> None:
-        """HF fp8 checkpoints: `{m}.weight` (e4m3) + `{m}.weight_scale_inv` (fp32)."""
-        if self._merge_sources is not None:
-            parts = [(f"{self._source_fqn}.{p}") for p in self._merge_sources]
-            packed = torch.cat([_load_tensor(f"{q}.weight") for q in parts], 0)
-            scales = torch.cat([_load_tensor(f"{q}.weight_scale_inv") for q in parts], 0)
-        else:
-            packed = _load_tensor(f"{self._source_fqn}.weight")
-            scales = _load_tensor(f"{self._source_fqn}.weight_scale_inv")
-        dev = self.lora_A.device if self.lora_A.device.type != "meta" else torch.device("cuda")
-        self._write_packed_weight(self._to_uint8(packed).to(dev))
-        self._scale_dtypes = {"weight_block_scales": torch.float32}
-        self.weight_block_scales = self._to_uint8(scales.float()).to(dev)
-        self._ema_amax = None
-        self._aqn_step_cache = None
+    _prequant_suffixes = ("weight", "weight_scale_inv")
+
+    def _pack_prequantized(self, pieces) -> dict:
+        """HF fp8 checkpoints: `{m}.weight` (e4m3 [N, K]) + `{m}.weight_scale_inv` (fp32 [N/128, K/128]); merged
+        projections are row-wise concatenations of bytes and of scale rows (checkpoint_handlers/buffers.py:878-901)."""
+        return {
+            "packed": torch.cat([self._to_uint8(p["weight"]) for p in pieces], 0),
+            "weight_block_scales": torch.cat([p["weight_scale_inv"].float() for p in pieces], 0),
+            "scale_dtypes": {"weight_block_scales": torch.float32},
+            "ema_amax": None,
+        }
 
 
 # =============================================================================
@@ -546,24 +570,25 @@ class NvFP4QLoRALinear(QLoRALinear):
             self._ema_amax = fresh
         self._quantize_and_store(merged, global_amax=self._ema_amax)
 
-    def _load_prequantized(self, _load_tensor) -> None:
-        """modelopt nvfp4 checkpoints: `.weight`, `.weight_scale` (e4m3), `.weight_scale_2` (fp32);
-        the global scale is folded into fp32 block scales and stored as 1.0."""
-        srcs = ([f"{self._source_fqn}.{p}" for p in self._merge_sources]
-                if self._merge_sources is not None else [self._source_fqn])
-        packed, scales, amaxes = [], [], []
-        for q in srcs:
-            g = _load_tensor(f"{q}.weight_scale_2").float()
-            packed.append(_load_tensor(f"{q}.weight"))
-            scales.append(_load_tensor(f"{q}.weight_scale").float() * g)
-            amaxes.append(g.item() * 6.0 * 448.0)
-        dev = self.lora_A.device if self.lora_A.device.type != "meta" else torch.device("cuda")
-        self._write_packed_weight(self._to_uint8(torch.cat(packed, 0)).to(dev))
-        self._scale_dtypes = {"weight_block_scales": torch.float32, "weight_global_scale": torch.float32}
-        self.weight_block_scales = self._to_uint8(torch.cat(scales, 0)).to(dev)
-        self.weight_global_scale = self._to_uint8(torch.tensor([1.0], dtype=torch.float32)).to(dev)
-        self._ema_amax = torch.tensor([max(amaxes)], dtype=torch.float32, device=dev)
-        self._aqn_step_cache = None
+    _prequant_suffixes = ("weight", "weight_scale", "weight_scale_2")
+
+    def _pack_prequantized(self, pieces) -> dict:
+        """modelopt nvfp4 checkpoints: `.weight` (codes [N, K/2]), `.weight_scale` (e4m3 [N, K/16]), `.weight_scale_2`
+        (fp32 scalar).  Each source's global scale is folded into fp32 block scales and the stored global is 1.0, so
+        that merged projections with different globals share one module; the largest source amax
+        (global * 6 * 448) seeds the EMA used by re-quantisation (checkpoint_handlers/buffers.py:827-865)."""
+        scales, amax = [], []
+        for p in pieces:
+            g = p["weight_scale_2"].float()
+            scales.append(p["weight_scale"].float() * g)
+            amax.append(g.item() * 6.0 * 448.0)
+        return {
+            "packed": torch.cat([self._to_uint8(p["weight"]) for p in pieces], 0),
+            "weight_block_scales": torch.cat(scales, 0),
+            "weight_global_scale": torch.tensor([1.0], dtype=torch.float32),
+            "scale_dtypes": {"weight_block_scales": torch.float32, "weight_global_scale": torch.float32},
+            "ema_amax": torch.tensor([max(amax)], dtype=torch.float32),
+        }
 
 
 # =============================================================================

@@ -320,23 +320,26 @@ class BlockFP8QLoRAMoeExperts(QLoRAMoeExperts):
         scales = self._recover_tensor(*scales_dict["weight_block_scales"])
         return Q.block_fp8_dequantize_gkn(packed.view(torch.float8_e4m3fn).reshape(K, N), scales, 128)
 
+    _prequant_suffixes = ("weight", "weight_scale_inv")
+
     def _load_experts(self, _load_tensor, _shard_cache) -> None:
-        """Pre-quantized block-fp8 experts (moe_experts.py:1074-1119).  Checkpoint: `weight` [N, K] e4m3 and
-        `weight_scale_inv` [N/128, K/128] per expert; bank: bytes [E, K, N] and fp32 scales [E, K/128, N/128] --
-        a pure transpose of bytes and scales, done once per projection on the device after one bulk copy."""
-        dev = self._load_device()
+        """Pre-quantized block-fp8 experts (moe_experts.py:1074-1119): one projection at a time."""
         for proj, hf in self._HF_PROJ:
-            w8, sc = [], []
-            for i in self._expert_range():
-                prefix = f"{self._source_fqn}.{i}.{hf}"
-                w8.append(_load_tensor(f"{prefix}.weight").view(torch.uint8))
-                sc.append(_load_tensor(f"{prefix}.weight_scale_inv").float())
-            bank = torch.stack(w8).to(dev).transpose(1, 2).contiguous()
-            scales = torch.stack(sc).to(dev).transpose(1, 2).contiguous()
-            setattr(self, f"{proj}_packed", self._to_uint8(bank))
-            setattr(self, f"{proj}_block_scales", self._to_uint8(scales))
-            self._scale_dtypes[proj] = {"weight_block_scales": torch.float32}
+            pieces = [{sfx: _load_tensor(f"{self._source_fqn}.{i}.{hf}.{sfx}") for sfx in self._prequant_suffixes}
+                      for i in self._expert_range()]
+            self._install_prequantized_bank(proj, pieces)
             _shard_cache.clear()
+
+    def _install_prequantized_bank(self, proj: str, pieces) -> None:
+        """`pieces[i]`: local expert i's checkpoint tensors, `weight` [N, K] e4m3 and `weight_scale_inv`
+        [N/128, K/128].  Bank: bytes [E, K, N] and fp32 scales [E, K/128, N/128] -- a pure transpose of bytes and
+        scales, done once per projection on the device after one bulk copy."""
+        dev = self._load_device()
+        bank = torch.stack([p["weight"].view(torch.uint8) for p in pieces]).to(dev).transpose(1, 2).contiguous()
+        scales = torch.stack([p["weight_scale_inv"].float() for p in pieces]).to(dev).transpose(1, 2).contiguous()
+        setattr(self, f"{proj}_packed", self._to_uint8(bank))
+        setattr(self, f"{proj}_block_scales", self._to_uint8(scales))
+        self._scale_dtypes[proj] = {"weight_block_scales": torch.float32}
 
     def _bank(self, proj_name: str) -> QuantWeight:
         K, N = self._proj_dims(proj_name)
@@ -379,6 +382,8 @@ class NvFP4QLoRAMoeExperts(QLoRAMoeExperts):
         g = self._recover_tensor(*scales_dict["weight_global_scale"])
         return Q.nvfp4_dequantize_gkn(packed, bs, g, K, N, 16)
 
+    _prequant_suffixes = ("weight", "weight_scale", "weight_scale_2")
+
     def _load_experts(self, _load_tensor, _shard_cache) -> None:
         """nvfp4 experts from a modelopt checkpoint (`weight` [N, K/2] u8, `weight_scale` [N, K/16] e4m3,
         `weight_scale_2` fp32 scalar) or, when the first expert has no `weight_scale`, from a bf16 checkpoint
@@ -392,38 +397,43 @@ class NvFP4QLoRAMoeExperts(QLoRAMoeExperts):
         except RuntimeError:
             prequantized = False
         for proj, hf in self._HF_PROJ:
-            amax = []
             if prequantized:
-                codes, bs, gs = [], [], []
-                for i in self._expert_range():
-                    prefix = f"{self._source_fqn}.{i}.{hf}"
-                    codes.append(_load_tensor(f"{prefix}.weight"))
-                    bs.append(_load_tensor(f"{prefix}.weight_scale").view(torch.uint8))
-                    g = _load_tensor(f"{prefix}.weight_scale_2").float().item()
-                    gs.append(g)
-                    amax.append(g * Q.FP4_E2M1_MAX * Q.FP8_E4M3_MAX)
-                g_dev = torch.tensor(gs, dtype=torch.float32, device=dev)
-                folded = torch.stack(bs).to(dev).view(torch.float8_e4m3fn).float() * g_dev[:, None, None]
-                bank = torch.stack(codes).to(dev).transpose(1, 2).contiguous()      # [E, K/2, N]: byte (k2, n) = K pair of column n
-                scales = folded.transpose(1, 2).contiguous()                        # [E, K/16, N] fp32
-            else:
-                codes, sc = [], []
-                for i in self._expert_range():
-                    w = _load_tensor(f"{self._source_fqn}.{i}.{hf}.weight").to(device=dev, dtype=torch.bfloat16).t().contiguous()
-                    a = w.float().abs().max().reshape(1)
-                    amax.append(a.item())
-                    packed, block_scales, global_scale = Q.nvfp4_quantize_gkn(w, self.quant_group_size, global_amax=a)
-                    codes.append(self._to_uint8(packed))
-                    sc.append((block_scales.float() * global_scale.float()).contiguous())
-                    _shard_cache.clear()
-                bank, scales = torch.stack(codes), torch.stack(sc)
-            setattr(self, f"{proj}_packed", self._to_uint8(bank))
-            setattr(self, f"{proj}_block_scales", self._to_uint8(scales))
-            setattr(self, f"{proj}_global_scale", self._to_uint8(torch.ones(E, 1, dtype=torch.float32, device=dev)))
-            self._scale_dtypes[proj] = {"weight_block_scales": torch.float32, "weight_global_scale": torch.float32}
-            self._ema_amax[proj] = torch.tensor(amax, dtype=torch.float32, device=dev)
-            if prequantized:
+                pieces = [{sfx: _load_tensor(f"{self._source_fqn}.{i}.{hf}.{sfx}") for sfx in self._prequant_suffixes}
+                          for i in self._expert_range()]
+                self._install_prequantized_bank(proj, pieces)
                 _shard_cache.clear()
+                continue
+            amax, codes, sc = [], [], []
+            for i in self._expert_range():
+                w = _load_tensor(f"{self._source_fqn}.{i}.{hf}.weight").to(device=dev, dtype=torch.bfloat16).t().contiguous()
+                a = w.float().abs().max().reshape(1)
+                amax.append(a.item())
+                packed, block_scales, global_scale = Q.nvfp4_quantize_gkn(w, self.quant_group_size, global_amax=a)
+                codes.append(self._to_uint8(packed))
+                sc.append((block_scales.float() * global_scale.float()).contiguous())
+                _shard_cache.clear()
+            self._set_folded_bank(proj, torch.stack(codes), torch.stack(sc), amax)
+
+    def _install_prequantized_bank(self, proj: str, pieces) -> None:
+        """`pieces[i]`: local expert i's modelopt tensors.  Codes and block scales are transposed to K-major on the
+        device after one bulk copy: byte (k2, n) of the bank holds the K pair of column n."""
+        dev = self._load_device()
+        gs = [p["weight_scale_2"].float().item() for p in pieces]
+        g_dev = torch.tensor(gs, dtype=torch.float32, device=dev)
+        bs = torch.stack([p["weight_scale"].view(torch.uint8) for p in pieces]).to(dev)
+        folded = bs.view(torch.float8_e4m3fn).float() * g_dev[:, None, None]
+        bank = torch.stack([p["weight"] for p in pieces]).to(dev).transpose(1, 2).contiguous()      # [E, K/2, N]
+        self._set_folded_bank(proj, bank, folded.transpose(1, 2).contiguous(),                     # [E, K/16, N] fp32
+                              [g * Q.FP4_E2M1_MAX * Q.FP8_E4M3_MAX for g in gs])
+
+    def _set_folded_bank(self, proj: str, bank: Tensor, scales: Tensor, amax) -> None:
+        dev = bank.device
+        setattr(self, f"{proj}_packed", self._to_uint8(bank))
+        setattr(self, f"{proj}_block_scales", self._to_uint8(scales))
+        setattr(self, f"{proj}_global_scale",
+                self._to_uint8(torch.ones(self.num_local_experts, 1, dtype=torch.float32, device=dev)))
+        self._scale_dtypes[proj] = {"weight_block_scales": torch.float32, "weight_global_scale": torch.float32}
+        self._ema_amax[proj] = torch.tensor(amax, dtype=torch.float32, device=dev)
 
     def _bank(self, proj_name: str) -> QuantWeight:
         K, N = self._proj_dims(proj_name)

@@ -127,6 +127,13 @@ _NF4_MIDPOINTS = (-0.8480964004993439, -0.6106329262256622, -0.4599952697753906,
                   0.5016634166240692, 0.6427869200706482, 0.8614784181118012)
 
 
+def _const(like: Tensor, v: float) -> Tensor:
+    """`v` as a 0-dim fp32 tensor on `like`'s device.  Quotients are taken between tensors so that they are one
+    IEEE division on every device: torch turns a Python-scalar divisor into a multiplication by its rounded
+    reciprocal on the GPU, and a Python-scalar numerator into reciprocal-then-multiply everywhere (two roundings)."""
+    return torch.tensor(v, dtype=torch.float32, device=like.device)
+
+
 def _nf4_encode(norm: Tensor) -> Tensor:
     """code = number of midpoints strictly below the value (nf4_codec.py:42-64)."""
     mid = torch.tensor(_NF4_MIDPOINTS, dtype=torch.float32, device=norm.device)
@@ -141,7 +148,7 @@ def nf4_quantize(x: Tensor, group_size: int = 64) -> Tuple[Tensor, Tensor]:
     assert n % group_size == 0 and group_size % 2 == 0
     xf = x.float().reshape(n // group_size, group_size)
     scale = xf.abs().amax(-1).clamp_min(1e-12)
-    norm = (xf * (1.0 / scale).unsqueeze(-1)).clamp_(-1.0, 1.0)
+    norm = (xf * (_const(scale, 1.0) / scale).unsqueeze(-1)).clamp_(-1.0, 1.0)
     codes = _nf4_encode(norm).reshape(-1)
     return (codes[0::2] | (codes[1::2] << 4)).contiguous(), scale.contiguous()
 
@@ -154,7 +161,7 @@ def nf4_quantize_gkn(x: Tensor, group_size: int = 64) -> Tuple[Tensor, Tensor]:
     assert K % group_size == 0 and group_size % 2 == 0
     xf = x.float().reshape(K // group_size, group_size, N)
     scale = xf.abs().amax(1).clamp_min(1e-12)
-    norm = (xf * (1.0 / scale).unsqueeze(1)).clamp_(-1.0, 1.0)
+    norm = (xf * (_const(scale, 1.0) / scale).unsqueeze(1)).clamp_(-1.0, 1.0)
     codes = _nf4_encode(norm).reshape(K, N)
     return _pack_nibbles_first(codes).contiguous(), scale.contiguous()
 
@@ -166,7 +173,7 @@ def int4_quantize(x: Tensor, group_size: int = -1) -> Tuple[Tensor, Tensor]:
     assert K % gs == 0 and gs % 2 == 0
     xf = x.float().reshape(M, K // gs, gs)
     scale = xf.abs().amax(-1).clamp_min(1e-12) * torch.tensor(2.0 / 15.0, dtype=torch.float32, device=x.device)
-    inv = 1.0 / scale
+    inv = _const(scale, 1.0) / scale
     q = (xf * inv.unsqueeze(-1) + 8.5).to(torch.int32).clamp_(0, 15)
     return _pack_nibbles_last(q.reshape(M, K)), scale
 
@@ -178,7 +185,7 @@ def int4_quantize_gkn(x: Tensor, group_size: int = -1) -> Tuple[Tensor, Tensor]:
     assert K % gs == 0 and gs % 2 == 0
     xf = x.float().reshape(K // gs, gs, N)
     scale = xf.abs().amax(1).clamp_min(1e-12) * torch.tensor(2.0 / 15.0, dtype=torch.float32, device=x.device)
-    inv = 1.0 / scale
+    inv = _const(scale, 1.0) / scale
     q = (xf * inv.unsqueeze(1) + 8.5).to(torch.int32).clamp_(0, 15)
     return _pack_nibbles_first(q.reshape(K, N)), scale
 
@@ -188,7 +195,7 @@ def int4_quantize_sym(x: Tensor, group_size: int = 128) -> Tuple[Tensor, Tensor]
     M, K = x.shape
     assert K % group_size == 0
     xf = x.float().reshape(M, K // group_size, group_size)
-    scale = (xf.abs().amax(-1) / 7.0).to(torch.bfloat16)
+    scale = (xf.abs().amax(-1) / _const(xf, 7.0)).to(torch.bfloat16)
     sf = scale.float().unsqueeze(-1)
     q = torch.where(sf > 0, torch.round(xf / sf).clamp_(-7, 7), torch.zeros_like(xf)).to(torch.int32) + 8
     return _pack_nibbles_last(q.reshape(M, K)), scale
@@ -211,7 +218,7 @@ def _nvfp4_scales(amax: Tensor, global_amax: Optional[Tensor]):
     gamax = amax.max().reshape(1) if global_amax is None else global_amax.float().reshape(1).to(amax.device)
     gamax = gamax.clamp_min(1e-12)
     block_scales = _e4m3_satfinite(amax / gamax * FP8_E4M3_MAX)
-    global_scale = gamax * torch.tensor(1.0 / FP4_E2M1_MAX, dtype=torch.float32, device=amax.device) / FP8_E4M3_MAX
+    global_scale = gamax * torch.tensor(1.0 / FP4_E2M1_MAX, dtype=torch.float32, device=amax.device) / _const(amax, FP8_E4M3_MAX)
     return block_scales, global_scale
 
 
@@ -222,7 +229,7 @@ def nvfp4_quantize(x: Tensor, block_size: int = 16, global_amax: Optional[Tensor
     assert n % block_size == 0 and block_size % 2 == 0
     xf = x.float().reshape(-1, block_size)
     amax = xf.abs().amax(-1).clamp_min(1e-12)
-    scaled = (xf * (6.0 / amax).unsqueeze(-1)).clamp_(-6.0, 6.0)
+    scaled = (xf * (_const(amax, 6.0) / amax).unsqueeze(-1)).clamp_(-6.0, 6.0)
     packed = _pack_nibbles_last(_fp4_encode(scaled).reshape(-1))
     block_scales, global_scale = _nvfp4_scales(amax, global_amax)
     return packed, block_scales, global_scale
@@ -235,7 +242,7 @@ def nvfp4_quantize_gkn(x: Tensor, block_size: int = 16, global_amax: Optional[Te
     assert K % block_size == 0 and block_size % 2 == 0
     xf = x.float().reshape(K // block_size, block_size, N)
     amax = xf.abs().amax(1).clamp_min(1e-12)
-    scaled = (xf * (6.0 / amax).unsqueeze(1)).clamp_(-6.0, 6.0)
+    scaled = (xf * (_const(amax, 6.0) / amax).unsqueeze(1)).clamp_(-6.0, 6.0)
     packed = _pack_nibbles_first(_fp4_encode(scaled).reshape(K, N))
     block_scales, global_scale = _nvfp4_scales(amax.reshape(-1), global_amax)
     return packed, block_scales.reshape(K // block_size, N), global_scale
@@ -254,7 +261,7 @@ def block_fp8_quantize_gkn(x: Tensor, block_size: int = 128, amax_scale: float =
         xf = torch.nn.functional.pad(xf, (0, pc, 0, pr))
     nr, nc = xf.shape[0] // bs, xf.shape[1] // bs
     blocks = xf.reshape(nr, bs, nc, bs)
-    s = (blocks.abs().amax(dim=(1, 3)) * amax_scale / FP8_E4M3_MAX).clamp_min(1e-12)
+    s = (blocks.abs().amax(dim=(1, 3)) * amax_scale / _const(xf, FP8_E4M3_MAX)).clamp_min(1e-12)
     y = (blocks / s[:, None, :, None]).clamp_(-FP8_E4M3_MAX, FP8_E4M3_MAX).to(torch.float8_e4m3fn)
     y = y.reshape(nr * bs, nc * bs)[:R, :Cc].contiguous()
     return y, s
