@@ -66,14 +66,20 @@ struct SmallNtArgs {
     int32_t num_experts;
 };
 
-// TR rows per block: 32 (dense; the 4 waves split K) or 128 (grouped; one wave per 32 rows).
+// TR rows per block: 32 (dense; the 4 waves split K) or 128 (grouped; one wave per 32 rows).  FJ = rows of F in
+// use / 4 (4, 8, 12 or 16).
 // Both operands are fetched with coalesced 16-byte loads (16 lanes per 256-byte row piece, 4 rows
 // per instruction) and reach the MFMA operand layout through wave-private LDS tiles of 128 k per
 // row (row pitch 272 B: the 16 lanes of a b128 read phase hit distinct banks); per-lane row-strided
 // loads would touch 64 cache lines per instruction and leave the kernel address-unit bound.
+// A wave keeps two 128-k chunks of its activation rows in flight (the factor chunk, which comes from L2, one):
+// every load is unconditional -- rows past the segment and columns past the wave's K range are clamped onto
+// valid ones and their values never used -- so the waits count exactly and the loads of chunk k+2 stay in
+// flight while chunk k is multiplied.
 constexpr int SN_P = 136;   // LDS row pitch in bf16 elements
-template <int TR, int NT>
+template <int TR, int FJ>
 __global__ void __launch_bounds__(256) small_nt_kernel(SmallNtArgs g) {
+    constexpr int NT = (FJ + 7) / 8;
     constexpr int RG = TR / 32, KS = 4 / RG;
     constexpr int WTILE = (32 + NT * 32) * SN_P;   // bf16 elements per wave: In tile + F tile
     extern __shared__ __attribute__((aligned(16))) bf16_t sn_lds[];
@@ -110,7 +116,7 @@ __global__ void __launch_bounds__(256) small_nt_kernel(SmallNtArgs g) {
     const int fr = lane & 31, fk = (lane >> 5) * 8;
     const int crow = lane >> 4, cpiece = (lane & 15) * 8;   // coalesced fetch: row within a group of 4, k offset
     const int64_t wrow0 = row0 + rg * 32;
-    const int frows = g.r_pad;                   // rows of F in use (multiple of 16)
+    const int frows = g.r_pad;                   // rows of F in use (= 4 * FJ)
 
     f32x16 acc[NT];
 #pragma unroll
@@ -120,37 +126,56 @@ __global__ void __launch_bounds__(256) small_nt_kernel(SmallNtArgs g) {
 
     const int64_t kspan = g.Kc / KS;  // multiple of 16
     const int64_t kbeg = ks * kspan, kend = kbeg + kspan;
-    u32x4 xr[8], fq[NT * 8];
-    auto fetch = [&](int64_t k) {     // chunk [k, k+128) clipped to kend; rows clamped to the segment / to F
+    const bf16_t* xp[8];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            int64_t r = wrow0 + j * 4 + crow;
-            r = r < row_end ? r : row_end - 1;
-            if (k + cpiece < kend) xr[j] = *(const u32x4*)(g.In + r * g.ld_in + k + cpiece);
-        }
+    for (int j = 0; j < 8; ++j) {
+        int64_t r = wrow0 + j * 4 + crow;
+        r = r < row_end ? r : row_end - 1;       // wrow0 may lie past a short segment's end: still a valid row
+        r = r < 0 ? 0 : r;
+        xp[j] = g.In + r * g.ld_in;
+    }
+    u32x4 xr[2][8], fq[FJ];
+    auto fetch_x = [&](u32x4* dst, int64_t k) {  // chunk [k, k+128); pieces past kend come from the range's last piece
+        int64_t kc = k + cpiece;
+        kc = kc < kend ? kc : kend - 8;
 #pragma unroll
-        for (int j = 0; j < NT * 8; ++j)
-            if (j * 4 < frows && k + cpiece < kend) fq[j] = *(const u32x4*)(F + (int64_t)(j * 4 + crow) * g.Kc + k + cpiece);
+        for (int j = 0; j < 8; ++j) dst[j] = *(const u32x4*)(xp[j] + kc);
     };
-    if (kbeg < kend) fetch(kbeg);
-    for (int64_t k = kbeg; k < kend; k += 128) {
+    auto fetch_f = [&](int64_t k) {
+        int64_t kc = k + cpiece;
+        kc = kc < kend ? kc : kend - 8;
+#pragma unroll
+        for (int j = 0; j < FJ; ++j) fq[j] = *(const u32x4*)(F + (int64_t)(j * 4 + crow) * g.Kc + kc);
+    };
+    auto chunk = [&](u32x4* cur, int64_t k) {    // multiply chunk k out of `cur`; refill it with chunk k + 256
         // LDS operations of one wave execute in order: the previous chunk's fragment reads are ahead of these writes
 #pragma unroll
-        for (int j = 0; j < 8; ++j) *(u32x4*)(xs + (j * 4 + crow) * SN_P + cpiece) = xr[j];
+        for (int j = 0; j < 8; ++j) *(u32x4*)(xs + (j * 4 + crow) * SN_P + cpiece) = cur[j];
 #pragma unroll
-        for (int j = 0; j < NT * 8; ++j)
-            if (j * 4 < frows) *(u32x4*)(fs + (j * 4 + crow) * SN_P + cpiece) = fq[j];
-        if (k + 128 < kend) fetch(k + 128);
-        const int nsteps = (int)((kend - k < 128 ? kend - k : 128) >> 4);
-        for (int st = 0; st < nsteps; ++st) {
-            const bf16x8 a = *(const bf16x8*)(xs + fr * SN_P + st * 16 + fk);
+        for (int j = 0; j < FJ; ++j) *(u32x4*)(fs + (j * 4 + crow) * SN_P + cpiece) = fq[j];
+        fetch_f(k + 128);
+        fetch_x(cur, k + 256);
+        const int64_t left = kend - k;           // <= 0 for the idle second half of the last pair
+        const int nsteps = (int)((left < 128 ? (left < 0 ? 0 : left) : 128) >> 4);
 #pragma unroll
-            for (int n = 0; n < NT; ++n) {
-                const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
-                const bf16x8 b = (n * 32 + fr < frows) ? *(const bf16x8*)(fs + (n * 32 + fr) * SN_P + st * 16 + fk) : zero8;
-                acc[n] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[n], 0, 0, 0);
+        for (int st = 0; st < 8; ++st) {
+            if (st < nsteps) {                   // uniform
+                const bf16x8 a = *(const bf16x8*)(xs + fr * SN_P + st * 16 + fk);
+#pragma unroll
+                for (int n = 0; n < NT; ++n) {
+                    const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+                    const bf16x8 b = (n * 32 + fr < frows) ? *(const bf16x8*)(fs + (n * 32 + fr) * SN_P + st * 16 + fk) : zero8;
+                    acc[n] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[n], 0, 0, 0);
+                }
             }
         }
+    };
+    fetch_x(xr[0], kbeg);
+    fetch_f(kbeg);
+    fetch_x(xr[1], kbeg + 128);
+    for (int64_t k = kbeg; k < kend; k += 256) {
+        chunk(xr[0], k);
+        chunk(xr[1], k + 128);
     }
 
     if (KS > 1) {
@@ -184,20 +209,31 @@ __global__ void __launch_bounds__(256) small_nt_kernel(SmallNtArgs g) {
     }
 }
 
-template <int TR, int NT>
+template <int TR, int FJ>
 static int launch_small_nt_one(const SmallNtArgs& g, unsigned blocks, hipStream_t stream) {
+    constexpr int NT = (FJ + 7) / 8;
     constexpr size_t lds = (size_t)4 * (32 + NT * 32) * SN_P * 2;
     static bool attr_set = false;
     if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute((const void*)small_nt_kernel<TR, NT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        hipError_t e = hipFuncSetAttribute((const void*)small_nt_kernel<TR, FJ>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) {
             xq_set_error("small_nt: cannot raise the dynamic LDS limit: %s", hipGetErrorString(e));
             return XQ_ERR_LAUNCH;
         }
         attr_set = true;
     }
-    small_nt_kernel<TR, NT><<<dim3(blocks), 256, lds, stream>>>(g);
+    small_nt_kernel<TR, FJ><<<dim3(blocks), 256, lds, stream>>>(g);
     return XQ_OK;
+}
+
+template <int TR>
+static int launch_small_nt_rows(const SmallNtArgs& g, unsigned blocks, hipStream_t stream) {
+    switch (g.r_pad) {
+        case 16: return launch_small_nt_one<TR, 4>(g, blocks, stream);
+        case 32: return launch_small_nt_one<TR, 8>(g, blocks, stream);
+        case 48: return launch_small_nt_one<TR, 12>(g, blocks, stream);
+        default: return launch_small_nt_one<TR, 16>(g, blocks, stream);
+    }
 }
 
 int launch_small_nt(const bf16_t* In, int64_t ld_in, int64_t n_rows, int64_t Kc, const bf16_t* F, int r_pad,
@@ -211,12 +247,10 @@ int launch_small_nt(const bf16_t* In, int64_t ld_in, int64_t n_rows, int64_t Kc,
                   num_experts};
     int rc;
     if (offsets) {
-        unsigned blocks = (unsigned)(xq_cdiv(n_rows, 128) + num_experts);
-        rc = r_pad <= 32 ? launch_small_nt_one<128, 1>(g, blocks, stream) : launch_small_nt_one<128, 2>(g, blocks, stream);
+        rc = launch_small_nt_rows<128>(g, (unsigned)(xq_cdiv(n_rows, 128) + num_experts), stream);
     } else {
         g.f_stride = 0;
-        unsigned blocks = (unsigned)xq_cdiv(n_rows, 32);
-        rc = r_pad <= 32 ? launch_small_nt_one<32, 1>(g, blocks, stream) : launch_small_nt_one<32, 2>(g, blocks, stream);
+        rc = launch_small_nt_rows<32>(g, (unsigned)xq_cdiv(n_rows, 32), stream);
     }
     if (rc) return rc;
     XQ_CHECK_LAUNCH("small_nt");

@@ -165,13 +165,24 @@ __global__ void __launch_bounds__(64) route_place_kernel(const int32_t* sel, int
     }
 }
 
-// out[scatter_index[i]] = in[i / topk]  (rows of `width` bf16; width % 8 == 0)
+// out[scatter_index[t * topk + j]] = in[t] for j < topk (rows of `width` bf16; width % 8 == 0).  One block per
+// token: the source row is read once and stored topk times, so the kernel runs at the rate of its writes.
 __global__ void __launch_bounds__(256) moe_scatter_kernel(const bf16_t* in, int64_t ld_in, const int32_t* sidx,
                                                           int32_t topk, int64_t width8, bf16_t* out, int64_t ld_out) {
-    int64_t i = blockIdx.x;
-    const bf16_t* src = in + (i / topk) * ld_in;
-    bf16_t* dst = out + (int64_t)sidx[i] * ld_out;
-    for (int64_t c = threadIdx.x; c < width8; c += 256) ((u32x4*)dst)[c] = ((const u32x4*)src)[c];
+    const int64_t t = blockIdx.x;
+    const u32x4* src = (const u32x4*)(in + t * ld_in);
+    const int32_t* dst_rows = sidx + t * topk;             // uniform: scalar loads
+    for (int64_t c = threadIdx.x; c < width8; c += 256) {
+        const u32x4 v = src[c];
+        for (int j0 = 0; j0 < topk; j0 += 8) {
+            int64_t r[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) r[u] = dst_rows[j0 + u < topk ? j0 + u : topk - 1];
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (j0 + u < topk) ((u32x4*)(out + r[u] * ld_out))[c] = v;     // uniform
+        }
+    }
 }
 
 // dst[scatter_index[i]] = src[i] (fp32 scalars; routing weights bf16/fp32 -> fp32)
@@ -191,27 +202,40 @@ __global__ void __launch_bounds__(256) moe_gather_scalar_kernel(const float* src
     else ((bf16_t*)dst)[i] = to_bf16(v);
 }
 
-// out[t] = sum_j rows[sidx[t*topk+j]] (+ rows2[...]); fp32 accumulate in slot order
+// out[t] = sum_j rows[sidx[t*topk+j]] (+ rows2[...]); fp32 accumulate in slot order.  One block per token; the row
+// indices of up to 8 slots are fetched first and their loads issued together (slots past topk are clamped onto
+// the last one and their values left out), so a token costs one memory round trip instead of one per slot.
+template <bool TWO>
 __global__ void __launch_bounds__(256) moe_gather_kernel(const bf16_t* rows, const bf16_t* rows2, int64_t ld_rows,
                                                          const int32_t* sidx, int32_t topk, int64_t width8,
                                                          bf16_t* out, int64_t ld_out) {
-    int64_t t = blockIdx.x;
+    const int64_t t = blockIdx.x;
+    const int32_t* src_rows = sidx + t * topk;             // uniform: scalar loads
     for (int64_t c = threadIdx.x; c < width8; c += 256) {
         float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-        for (int j = 0; j < topk; ++j) {
-            int64_t r = sidx[t * topk + j];
-            u32x4 v = ((const u32x4*)(rows + r * ld_rows))[c];
+        for (int j0 = 0; j0 < topk; j0 += 8) {
+            u32x4 v[8], v2[8];
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                acc[2 * q] += bf16_to_f32((bf16_t)(v[q] & 0xffffu));
-                acc[2 * q + 1] += bf16_to_f32((bf16_t)(v[q] >> 16));
+            for (int u = 0; u < 8; ++u) {
+                const int64_t r = src_rows[j0 + u < topk ? j0 + u : topk - 1];
+                v[u] = ((const u32x4*)(rows + r * ld_rows))[c];
+                if (TWO) v2[u] = ((const u32x4*)(rows2 + r * ld_rows))[c];
             }
-            if (rows2) {
-                u32x4 v2 = ((const u32x4*)(rows2 + r * ld_rows))[c];
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    acc[2 * q] += bf16_to_f32((bf16_t)(v2[q] & 0xffffu));
-                    acc[2 * q + 1] += bf16_to_f32((bf16_t)(v2[q] >> 16));
+            for (int u = 0; u < 8; ++u) {
+                if (j0 + u < topk) {                       // uniform
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        acc[2 * q] += bf16_to_f32((bf16_t)(v[u][q] & 0xffffu));
+                        acc[2 * q + 1] += bf16_to_f32((bf16_t)(v[u][q] >> 16));
+                    }
+                    if (TWO) {
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) {
+                            acc[2 * q] += bf16_to_f32((bf16_t)(v2[u][q] & 0xffffu));
+                            acc[2 * q + 1] += bf16_to_f32((bf16_t)(v2[u][q] >> 16));
+                        }
+                    }
                 }
             }
         }
@@ -280,8 +304,9 @@ extern "C" int xq_moe_scatter(const void* in, int64_t ld_in, const int32_t* scat
     XQ_REQUIRE(topk >= 1 && width % 8 == 0 && ld_in % 8 == 0 && ld_out % 8 == 0, "xq_moe_scatter: width/strides must be multiples of 8");
     if (n_routed == 0 || width == 0) return XQ_OK;
     XQ_REQUIRE(in && out && scatter_index && xq_aligned(in, 16) && xq_aligned(out, 16), "xq_moe_scatter: bad pointer");
-    moe_scatter_kernel<<<dim3((unsigned)n_routed), 256, 0, (hipStream_t)stream>>>((const bf16_t*)in, ld_in, scatter_index,
-                                                                                  topk, width / 8, (bf16_t*)out, ld_out);
+    XQ_REQUIRE(n_routed % topk == 0, "xq_moe_scatter: n_routed %lld is not a multiple of topk %d", (long long)n_routed, topk);
+    moe_scatter_kernel<<<dim3((unsigned)(n_routed / topk)), 256, 0, (hipStream_t)stream>>>((const bf16_t*)in, ld_in, scatter_index,
+                                                                                           topk, width / 8, (bf16_t*)out, ld_out);
     XQ_CHECK_LAUNCH("xq_moe_scatter");
     return XQ_OK;
 }
@@ -312,8 +337,12 @@ extern "C" int xq_moe_gather(const void* rows, const void* rows2, int64_t ld_row
     if (n_tokens == 0 || width == 0) return XQ_OK;
     XQ_REQUIRE(rows && out && scatter_index && xq_aligned(rows, 16) && xq_aligned(out, 16) && (!rows2 || xq_aligned(rows2, 16)),
                "xq_moe_gather: bad pointer");
-    moe_gather_kernel<<<dim3((unsigned)n_tokens), 256, 0, (hipStream_t)stream>>>(
-        (const bf16_t*)rows, (const bf16_t*)rows2, ld_rows, scatter_index, topk, width / 8, (bf16_t*)out, ld_out);
+    if (rows2)
+        moe_gather_kernel<true><<<dim3((unsigned)n_tokens), 256, 0, (hipStream_t)stream>>>(
+            (const bf16_t*)rows, (const bf16_t*)rows2, ld_rows, scatter_index, topk, width / 8, (bf16_t*)out, ld_out);
+    else
+        moe_gather_kernel<false><<<dim3((unsigned)n_tokens), 256, 0, (hipStream_t)stream>>>(
+            (const bf16_t*)rows, nullptr, ld_rows, scatter_index, topk, width / 8, (bf16_t*)out, ld_out);
     XQ_CHECK_LAUNCH("xq_moe_gather");
     return XQ_OK;
 }
