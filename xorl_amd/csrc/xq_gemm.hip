@@ -19,8 +19,8 @@ static int g_skinny_enabled = [] { const char* e = getenv("XQ_SKINNY"); return e
 static int g_tile_policy = [] { const char* e = getenv("XQ_TILE_POLICY"); return e ? atoi(e) : 0; }();
 
 template <typename K>
-static int raise_lds_limit(K kernel, const char* who) {
-    hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+static int raise_lds_limit(K kernel, size_t bytes, const char* who) {
+    hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
     if (e != hipSuccess) {
         xq_set_error("%s: cannot raise the dynamic LDS limit: %s", who, hipGetErrorString(e));
         return XQ_ERR_LAUNCH;
@@ -32,7 +32,7 @@ template <int FMT, bool CC, bool GROUPED, int T>
 static int launch_256_one(const G256Args& f, dim3 grid, hipStream_t s, const char* who) {
     static bool attr_set = false;  // per instantiation
     if (!attr_set) {
-        int rc = raise_lds_limit(gemm_256_kernel<FMT, CC, GROUPED, T>, who);
+        int rc = raise_lds_limit(gemm_256_kernel<FMT, CC, GROUPED, T>, Geo<T>::lds_bytes(CC), who);
         if (rc) return rc;
         attr_set = true;
     }

@@ -157,12 +157,14 @@ __device__ __forceinline__ float scale_from_raw(uint32_t raw, int dtype) {
 //   int4:  value = nib - 8.  fma(nib, s, -8s) is the same real number as (nib - 8) * s
 //          (-8s is exact), so it rounds identically; only the sign of an exact zero can
 //          differ from the two-step form, which no sum can see.
-//   nf4:   level[nib] * s, the level read from a 64-byte constant table (one L1-resident line).
+//   nf4:   level[nib] * s, the level read from a 64-byte copy of the table in LDS (16 banks: any mix of
+//          codes in a wave is conflict free).  The copy in constant memory would be a vector memory load per
+//          code, which returns in order behind the next K-step's prefetch loads and so waits for them.
 //   nvfp4: v_cvt_scalef32_pk_f32_fp4 with scale 1.0 returns the exact e2m1 values of the two
 //          codes of a byte (low nibble first); each is multiplied by s in fp32 and rounded
 //          once, like the reference's fl(e2m1 * s).
 template <int FMT>
-__device__ __forceinline__ void decode8_4bit(uint32_t w, float s, uint32_t* out4) {
+__device__ __forceinline__ void decode8_4bit(uint32_t w, float s, uint32_t* out4, const float* nf4_lds) {
     float v[8];
     if (FMT == XQ_FMT_INT4) {
         const float m8s = -8.0f * s;
@@ -174,7 +176,7 @@ __device__ __forceinline__ void decode8_4bit(uint32_t w, float s, uint32_t* out4
         }
     } else if (FMT == XQ_FMT_NF4) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) v[i] = kNf4Level[(w >> (4 * i)) & 0xfu] * s;
+        for (int i = 0; i < 8; ++i) v[i] = nf4_lds[(w >> (4 * i)) & 0xfu] * s;
     } else {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -200,10 +202,11 @@ struct W256Flat4 {
     int32_t col0[2];     // CC: first column of the run at K-step 0
     int gshift, sdt, tid;
     float gs;
+    const float* nf4_lds;   // nf4: the 16 levels in LDS
     u32x2 raw[2];
     uint32_t sraw[2];
     __device__ __forceinline__ void init(const G256Args& g, const uint8_t* pk, const uint8_t* sc, float gscale, int n0, int tid_) {
-        tid = tid_; gshift = g.gshift; sdt = g.scale_dtype; gs = gscale; sc_base = sc;
+        tid = tid_; gshift = g.gshift; sdt = g.scale_dtype; gs = gscale; sc_base = sc; nf4_lds = nullptr;
         const int spr = g.wcols >> gshift;  // scales per W row
 #pragma unroll
         for (int p = 0; p < 2; ++p) {
@@ -230,8 +233,8 @@ struct W256Flat4 {
         float s = scale_from_raw(sraw[p], sdt);
         if (FMT == XQ_FMT_NVFP4) s = s * gs;
         uint32_t lo[4], hi[4];
-        decode8_4bit<FMT>(raw[p][0], s, lo);
-        decode8_4bit<FMT>(raw[p][1], s, hi);
+        decode8_4bit<FMT>(raw[p][0], s, lo, nf4_lds);
+        decode8_4bit<FMT>(raw[p][1], s, hi, nf4_lds);
         store_run16<CC, T>(b, tid + p * Geo<T>::NT, u32x4{lo[0], lo[1], lo[2], lo[3]}, u32x4{hi[0], hi[1], hi[2], hi[3]});
     }
 };
@@ -319,6 +322,12 @@ __global__ void __launch_bounds__(2 * T, 2) gemm_256_kernel(G256Args g) {
     typename W256Sel<FMT, CC, T>::type wl;
     wl.init(g, g.W + (int64_t)e * g.packed_stride, g.scales + (int64_t)e * g.scale_stride,
             FMT == XQ_FMT_NVFP4 ? g.global_scale[e] : 1.0f, n0, tid);
+    if constexpr (FMT == XQ_FMT_NF4) {
+        __shared__ float s_nf4[16];
+        if (tid < 16) s_nf4[tid] = kNf4Level[tid];
+        __syncthreads();
+        wl.nf4_lds = s_nf4;
+    }
 
     u32x4 areg[4];
     auto load_a = [&](int kt) {
