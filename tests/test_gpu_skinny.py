@@ -30,7 +30,7 @@ def test_skinny_forward_vs_oracle(hip_device, fmt, M):
 
 
 @pytest.mark.parametrize("fmt,N,K", [("block_fp8", 1024, 4096), ("int4", 1024, 4096), ("block_fp8", 4096, 12288),
-                                     ("int4", 12288, 4096)])
+                                     ("int4", 12288, 4096), ("nf4", 4096, 12288), ("nf4", 12288, 4096)])
 def test_skinny_projection_shapes(hip_device, fmt, N, K):
     """Qwen3-8B projection shapes of BASELINE config 4 at M = 8 and 64 (oracle in float64 on CPU)."""
     m, w_ref = make_dense_module(fmt, N, K, 16, 32, seed=N + K, device=hip_device)
@@ -53,6 +53,8 @@ def test_skinny_projection_shapes(hip_device, fmt, N, K):
     ("block_fp8", 384, 2048, 17, 64, True),      # four 16-rank tiles, bf16 factors
     ("int4", 1024, 4096, 32, 40, False),         # rank padded to 48
     ("nvfp4", 4096, 4096, 9, 16, True),
+    ("nf4", 21888, 1280, 5, 16, False),          # uneven splits with two scales per chunk
+    ("nf4", 208, 1024, 40, 24, True),
 ])
 def test_skinny_split_plans(hip_device, fmt, N, K, M, r, bf16_factors):
     """K-split organisation: uneven splits, ragged row blocks, every rank-tile count, both factor dtypes."""
@@ -152,3 +154,25 @@ def test_skinny_scale_storage_variants(hip_device, M):
         pk = m.packed_weight_f32.detach().contiguous().view(torch.uint8).numpy()
         sc = m.weight_scales.contiguous().view(torch.float32).numpy()
         check(m, bits_to_bf16(NP.int4_decode_flat(pk, sc, N, K, group)))
+
+
+@pytest.mark.parametrize("fmt", ["block_fp8", "int4", "nvfp4", "nf4"])
+@pytest.mark.parametrize("M", [16, 64])
+def test_skinny_decode_bit_exact(hip_device, fmt, M):
+    """Rows of X that are unit vectors (and no low-rank term) make every output a single product 1 * w: the
+    forward returns columns of the decoded weight, which must equal the oracle's decode bit for bit (up to the sign
+    of zero: a sum of zeros is +0).  The columns cover every K split and both halves of a scale group."""
+    from xorl_amd.functional import qlora_linear
+
+    N, K = 384, 2048
+    m, w_ref = make_dense_module(fmt, N, K, 8, 16, seed=31 + M, device=hip_device)
+    cols = torch.tensor([(37 * i * i + 11 * i) % K for i in range(M)])
+    cols[0], cols[1] = 0, K - 1
+    x = torch.zeros(M, K, dtype=torch.bfloat16)
+    x[torch.arange(M), cols] = 1.0
+    with torch.no_grad():
+        y = qlora_linear(x.to(hip_device), m._quant_weight(), None, None, 0, 0.0, None).cpu()
+    want = w_ref[:, cols].t().contiguous()                       # [M, N]
+    same = y.view(torch.int16) == want.view(torch.int16)
+    both_zero = (y.float() == 0) & (want.float() == 0)
+    assert bool((same | both_zero).all())

@@ -59,7 +59,7 @@ struct SkinnyEpiArgs {
 
 // decode 8 consecutive K elements (one MFMA operand) of this lane's row
 template <int FMT>
-__device__ __forceinline__ bf16x8 decode8(uint32_t w0, uint32_t w1, float s0, float s1) {
+__device__ __forceinline__ bf16x8 decode8(uint32_t w0, uint32_t w1, float s0, float s1, const float* nf4_lds = nullptr) {
     uint32_t o[4];
     if (FMT == XQ_FMT_FP8) {
         f32x2 a = e4m3x2_to_f32(w0, false), b = e4m3x2_to_f32(w0, true);
@@ -76,6 +76,11 @@ __device__ __forceinline__ bf16x8 decode8(uint32_t w0, uint32_t w1, float s0, fl
             float hi = __builtin_fmaf((float)((w0 >> (8 * i + 4)) & 0xfu), s0, s1);
             o[i] = pack_bf16x2(lo, hi);
         }
+    } else if (FMT == XQ_FMT_NF4) {
+        // level[nib] * scale, the levels read from a 64-byte copy of the table in LDS (conflict free for any mix of codes)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            o[i] = pack_bf16x2(nf4_lds[(w0 >> (8 * i)) & 0xfu] * s0, nf4_lds[(w0 >> (8 * i + 4)) & 0xfu] * s0);
     } else {
         // v_cvt_scalef32_pk_f32_fp4 with scale 1.0 yields the exact e2m1 values of byte i (low nibble first)
         f32x2 v0 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w0, 1.0f, 0);
@@ -127,7 +132,7 @@ __global__ void __launch_bounds__(256, MR == 16 ? 4 : 3) skinny_split_kernel(Ski
     const int fr = lane & 31, fh = lane >> 5;
     constexpr int EB = FMT == XQ_FMT_FP8 ? 1 : 2;      // elements per byte
     constexpr int NLOAD = FMT == XQ_FMT_FP8 ? 4 : 2;   // 16-byte loads per lane per 128-k chunk
-    constexpr int NSC = FMT == XQ_FMT_NVFP4 ? 4 : 1;   // scale registers per chunk
+    constexpr int NSC = FMT == XQ_FMT_NVFP4 ? 4 : FMT == XQ_FMT_NF4 ? 2 : 1;   // scale registers per chunk
 
     // grid: x = K split, y = 128-row block, preceded by one row of su blocks when there is a low-rank term
     const int split = blockIdx.x;
@@ -280,6 +285,10 @@ __global__ void __launch_bounds__(256, MR == 16 ? 4 : 3) skinny_split_kernel(Ski
             else if (FMT == XQ_FMT_INT4) {
                 const int64_t si = int4_small_group ? 0 : ((int64_t)n * g.K + cc * 128) / g.group;
                 sc[c][0] = g.scale_dtype == XQ_SCALE_F32 ? ((const uint32_t*)g.scales)[si] : ((const uint16_t*)g.scales)[si];
+            } else if (FMT == XQ_FMT_NF4) {
+                const u32x2 t = *(const u32x2*)((const uint32_t*)g.scales + (((int64_t)n * g.K + cc * 128) >> 6));   // fp32, group 64
+                sc[c][0] = t[0];
+                sc[c][1] = t[1];
             } else {
                 const int64_t si = ((int64_t)n * g.K + cc * 128) >> 4;   // the 8 block scales of this row's chunk
                 if (g.scale_dtype == XQ_SCALE_E4M3) {
@@ -301,6 +310,8 @@ __global__ void __launch_bounds__(256, MR == 16 ? 4 : 3) skinny_split_kernel(Ski
     // of one wave execute in order, so the slab is reused chunk after chunk without barriers.
     const float gsc = FMT == XQ_FMT_NVFP4 ? g.global_scale[0] : 1.0f;
     unsigned char* wst = smem + (size_t)xrows * XP * 2 + wave * (PPR * 32 * 16);
+    float* nf4_lds = (float*)(smem + (size_t)xrows * XP * 2 + 4 * 4096);    // 16 levels behind the slabs
+    if (FMT == XQ_FMT_NF4 && tid < 16) nf4_lds[tid] = kNf4Level[tid];        // ordered before its use by stage_x's barrier
 #pragma unroll
     for (int h = 0; h < NPASS; ++h) {
         if (h * 32 < g.M) {
@@ -341,6 +352,8 @@ __global__ void __launch_bounds__(256, MR == 16 ? 4 : 3) skinny_split_kernel(Ski
                             bf16x8 wf;
                             if (FMT == XQ_FMT_FP8) {
                                 wf = decode8<FMT>(f[2 * v], f[2 * v + 1], __uint_as_float(sc[c][0]), 0.0f);
+                            } else if (FMT == XQ_FMT_NF4) {
+                                wf = decode8<FMT>(f[v], 0u, __uint_as_float(sc[c][u >> 1]), 0.0f, nf4_lds);   // group 64: k = 32u + ..
                             } else if (FMT == XQ_FMT_INT4) {
                                 float sv;
                                 if (int4_small_group) sv = load_scale(g.scales, ((int64_t)n * g.K + kc + 32 * u + 16 * fh + 8 * v) / g.group, g.scale_dtype);
@@ -493,7 +506,7 @@ int64_t skinny_workspace_bytes(int64_t M, int64_t N, int64_t K, int r_pad) {
 
 bool skinny_supported(const xq_weight* w, int64_t M) {
     if (M < 1 || M > 64 || w->num_experts != 1) return false;
-    if (w->format == XQ_FMT_NF4) return false;   // nf4 takes the tile kernels
+    if (w->format == XQ_FMT_NF4 && (w->group != 64 || w->scale_dtype != XQ_SCALE_F32)) return false;   // other nf4 storages take the tile kernels
     if (w->format != XQ_FMT_FP8 && w->layout != XQ_LAYOUT_FLAT) return false;
     if (w->cols % 128 != 0 || w->cols < 1024 || w->rows % 16 != 0) return false;
     if (w->format == XQ_FMT_INT4 && (w->group % 8 != 0)) return false;
@@ -533,7 +546,7 @@ static int launch_skinny_split(const xq_weight* w, const bf16_t* x, int64_t ldx,
     g.su_part = (float*)((char*)workspace + al256((int64_t)p.splits * M * N * 4));
     g.lora_A = rp ? lora_A : nullptr; g.lora_f32 = lora_dtype == XQ_DT_F32; g.r = r; g.r_pad = rp;
     const dim3 grid((unsigned)p.splits, (unsigned)(p.row_blocks + g.su_blocks));
-    const size_t lds = (size_t)(M < 32 ? M : 32) * g.xp * 2 + 4 * 4096;   // x slice + the four weight slabs (or the su reduction buffer)
+    const size_t lds = (size_t)(M < 32 ? M : 32) * g.xp * 2 + 4 * 4096 + 64;   // x slice + the four weight slabs (or the su reduction buffer) + nf4 levels
 
     SkinnyEpiArgs e;
     e.partial = g.partial; e.su_part = g.su_part; e.splits = p.splits; e.su_parts = rp ? p.splits : 0;
@@ -543,6 +556,7 @@ static int launch_skinny_split(const xq_weight* w, const bf16_t* x, int64_t ldx,
     int rc;
     if (w->format == XQ_FMT_FP8) rc = launch_split_cfg<XQ_FMT_FP8>(g, p.nch, grid, lds, stream);
     else if (w->format == XQ_FMT_INT4) rc = launch_split_cfg<XQ_FMT_INT4>(g, p.nch, grid, lds, stream);
+    else if (w->format == XQ_FMT_NF4) rc = launch_split_cfg<XQ_FMT_NF4>(g, p.nch, grid, lds, stream);
     else rc = launch_split_cfg<XQ_FMT_NVFP4>(g, p.nch, grid, lds, stream);
     if (rc) return rc;
     const int waves = M < 4 ? (int)M : 4;
