@@ -40,10 +40,11 @@ BF16_MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense bf16, published
 MEASURED_TRAFFIC_BYTES = {
     0: 45.6 * 2 ** 20,     # gemm_256_kernel<int4, T=128>: mean of the forward and dgrad launches
     1: 905.4 * 2 ** 20,    # gemm_256_kernel<fp8>: mean of the forward and dgrad launches
-    2: 227.8 * 2 ** 20,    # gemm_256_kernel<nvfp4> / gemm_tile_kernel<nvfp4>: mean over the 8 launches of a step
+    2: 153.2 * 2 ** 20,    # gemm_256_kernel<nvfp4>, 256x256 and 128x128 tiles: mean over the 12 launches of a step
     3: 1032.2 * 2 ** 20,   # gemm_256_kernel<fp8, grouped>: mean over the 6 launches of a step
     4: 41.0 * 2 ** 20,     # skinny_split_kernel + skinny_epilogue_kernel: mean per forward over the 32 cases (includes
                            # the fp32 partial tiles written and read back: 23.3 MiB of it are algorithmic)
+    6: 737.0 * 2 ** 20,    # gemm_256_kernel<nf4>: mean of the forward and dgrad launches
     5: 134.4 * 2 ** 20,    # merge_prep_kernel + merge_kernel<fp8>: mean per call (re-quantise 96 MiB, publish 144 MiB algorithmic)
 }
 
@@ -173,7 +174,7 @@ def other_config(cfg: int, dev):
                 m(xs[k]).backward(dys[k])
         return (step, sum(lin_flops(Mtok, K, N, 16) for (N, K) in shapes.values()), False,
                 "configs[2]: nvfp4 QLoRA Qwen3-32B attention projections q/k/v/o, hidden 5120, M=4096, r=16, fwd+bwd",
-                "gemm_256_kernel<nvfp4> (q/o and the k/v dgrad) and gemm_tile_kernel<nvfp4> (k/v forward): fused dequant-GEMM, forward and dgrad launches")
+                "gemm_256_kernel<nvfp4> with 256x256 tiles (whole rounds of the chip) and 128x128 tiles (k/v forward, trailing rows): fused dequant-GEMM, forward and dgrad launches")
     if cfg == 3:
         from xorl_amd.qlora import BlockFP8QLoRAMoeExperts
 
