@@ -216,3 +216,29 @@ def test_inline_buffer_converts_between_checkpoint_and_module_format(hip_device,
         assert torch.equal(got["proj.packed_weight_f32"].contiguous().view(torch.uint8).flatten(), b.view(torch.uint8).flatten())
         assert torch.equal(got["proj.weight_block_scales"].contiguous().view(torch.float32).flatten(), s.flatten())
     assert got["proj.packed_weight_f32"].shape == model.proj.packed_weight_f32.shape
+
+
+@pytest.mark.parametrize("tile_policy", [1, 2, 3], indirect=True)
+@pytest.mark.parametrize("fmt", ["block_fp8", "nvfp4", "nf4"])
+def test_grouped_gemm_decode_bit_exact(hip_device, tile_policy, fmt):
+    """Every expert gets the rows of an identity matrix, so the grouped forward product (contraction along the
+    bank's rows) returns the expert's decoded [K, N] matrix and the dgrad product (contraction along its columns)
+    returns the transpose: the in-kernel decode of each grouped kernel, in both directions, must equal the oracle's
+    bank decode bit for bit (up to the sign of zero)."""
+    from xorl_amd import moe_functional as MF
+
+    E, H, I = 3, 256, 384
+    m, banks = _make_experts(fmt, E, H, I, 8, False, seed=60, device=hip_device)
+    for proj, (K, N) in (("gate", (H, I)), ("down", (I, H))):
+        qw = m._bank(proj)
+        ref = banks[proj].to(hip_device)                                   # [E, K, N] bf16
+        for transpose_w, rows in ((False, K), (True, N)):
+            sel = torch.arange(E, dtype=torch.int32).repeat_interleave(rows).reshape(-1, 1).to(hip_device)
+            counts, offsets, sidx, tile_offsets = MF.route_build(sel, E)
+            assert torch.equal(sidx.cpu().flatten(), torch.arange(E * rows, dtype=torch.int32))   # already in expert order
+            a = torch.eye(rows, dtype=torch.bfloat16, device=hip_device).repeat(E, 1)
+            y = MF._grouped_gemm(qw, transpose_w, a, offsets, tile_offsets, None, None)
+            want = (ref.transpose(1, 2) if transpose_w else ref).reshape(E * rows, -1).contiguous()
+            same = y.view(torch.int16) == want.view(torch.int16)
+            both_zero = (y.float() == 0) & (want.float() == 0)
+            assert bool((same | both_zero).all()), (proj, transpose_w)

@@ -86,8 +86,13 @@ static int launch_tile_gemm_t(const xq_weight* w, bool contract_cols, const bf16
         const bool grouped = offsets != nullptr;
         int gshift = 0;
         while ((1 << gshift) < g.group) ++gshift;
+        // 4-bit: power-of-two groups of at least 16; dense matrices FLAT, expert banks GKN (16-byte pieces of codes
+        // and of scales: columns in multiples of 16, 16-byte aligned scale storage)
         const bool fmt_ok = w->format == XQ_FMT_FP8 ||
-                            (w->layout == XQ_LAYOUT_FLAT && (1 << gshift) == g.group && g.group >= 16);
+                            ((1 << gshift) == g.group && g.group >= 16 &&
+                             (grouped ? w->layout == XQ_LAYOUT_GKN && g.wcols % 16 == 0 && g.wrows >= 2 &&
+                                            xq_aligned(w->scales, 16) && g.scale_stride % 16 == 0
+                                      : w->layout == XQ_LAYOUT_FLAT));
         const bool big = grouped ? (n_rows >= 128ll * w->num_experts && n_rows >= 8192)
                                  : (xq_cdiv(n_rows, 256) * xq_cdiv(g.Nout, 256) >= 96);
         const int T = force_T ? force_T : g_tile_policy == 2 ? 256 : g_tile_policy == 3 ? 128 : (big ? 256 : 128);

@@ -7,8 +7,9 @@
 //   C[rows, Nout] = A[rows, Kc] . Wop (+ su[rows, r] . Lr[Nout, r]^T) (+ bias)
 //
 // W is a quantized [wrows, wcols] matrix: block-fp8 (e4m3 bytes, fp32 scale per
-// 128x128 block) or a 4-bit FLAT matrix (int4 / nvfp4 / nf4: two codes per byte along
-// the columns, one scale per `group` consecutive columns).
+// 128x128 block), a dense 4-bit FLAT matrix (int4 / nvfp4 / nf4: two codes per byte along
+// the columns, one scale per `group` consecutive columns) or, GROUPED, a 4-bit GKN matrix of an
+// expert bank (two codes per byte along the rows, one scale per `group` rows of a column).
 //   CONTRACT_COLS (dense forward, expert-bank dgrad):  Wop[kc][n] = W[n][kc]; the
 //     decoded tile is stored in LDS as [n][kc] (kc contiguous, XOR-swizzled 16-byte
 //     chunks) and read with ds_read_b128 in MFMA operand order.
@@ -239,8 +240,128 @@ struct W256Flat4 {
     }
 };
 
-template <int FMT, bool CC, int T> struct W256Sel { using type = W256Flat4<FMT, CC, T>; };
-template <bool CC, int T> struct W256Sel<XQ_FMT_FP8, CC, T> { using type = W256Fp8<CC, T>; };
+// 4-bit GKN matrix of an expert bank, [wrows = K, wcols = N]: byte (k / 2, n) holds rows k (low nibble) and
+// k + 1 (high nibble) of column n; one scale per `group` rows per column, [K / group][N].  A thread owns one
+// 16-byte piece per K-step -- 16 consecutive columns of one row pair, i.e. two 16-code runs that share their bytes
+// and their 16 scales.
+//   !CC (bank forward, contraction along K): pair t / RPR of the K-step's 32 row pairs, columns n0 + (t % RPR) * 16;
+//   CC (bank dgrad, contraction along N): rows n0 + 2 * (t >> 2), columns k0 + (t & 3) * 16.
+template <int FMT, bool CC, int T>
+struct W256Gkn4 {
+    const uint8_t* src;
+    const uint8_t* sc_base;
+    int64_t kstep;           // bytes per K-step
+    int32_t wcols, row, col; // !CC: first row of the pair within the K-step; CC: global row of the pair; first column at K-step 0
+    int gshift, sdt, tid;
+    float gs;
+    const float* nf4_lds;
+    u32x4 raw;
+    u32x4 s0, s1, s2, s3;    // 16 scales: 4 / 2 / 1 registers of them for fp32 / bf16 / e4m3 storage
+    __device__ __forceinline__ void init(const G256Args& g, const uint8_t* pk, const uint8_t* sc, float gscale, int n0, int tid_) {
+        tid = tid_; gshift = g.gshift; sdt = g.scale_dtype; gs = gscale; sc_base = sc; nf4_lds = nullptr; wcols = g.wcols;
+        if (CC) {
+            row = min(n0 + 2 * (tid >> 2), g.wrows - 2);
+            col = (tid & 3) * 16;
+            src = pk + (int64_t)(row >> 1) * g.wcols + col;
+            kstep = F8_BK;
+        } else {
+            row = 2 * (tid / Geo<T>::RPR);
+            col = min(n0 + (tid % Geo<T>::RPR) * 16, g.wcols - 16);
+            src = pk + (int64_t)(row >> 1) * g.wcols + col;
+            kstep = (int64_t)(F8_BK / 2) * g.wcols;
+        }
+    }
+    __device__ __forceinline__ void load(int kt) {
+        raw = *(const u32x4*)(src + kt * kstep);
+        const int64_t si = CC ? (int64_t)(row >> gshift) * wcols + col + kt * F8_BK
+                              : (int64_t)((kt * F8_BK + row) >> gshift) * wcols + col;
+        // unconditional loads of what the widest storage needs (narrower storages read the same piece again:
+        // cache hits), so that the four registers are plain values and the waits count exactly
+        const int esz = sdt == XQ_SCALE_F32 ? 4 : sdt == XQ_SCALE_BF16 ? 2 : 1;
+        const uint8_t* sp = sc_base + si * esz;
+        const int q1 = esz >= 2 ? 16 : 0, q2 = esz == 4 ? 32 : 0, q3 = esz == 4 ? 48 : 0;
+        s0 = *(const u32x4*)sp;
+        s1 = *(const u32x4*)(sp + q1);
+        s2 = *(const u32x4*)(sp + q2);
+        s3 = *(const u32x4*)(sp + q3);
+    }
+    // both rows of the pair in one pass over the 16 columns, four at a time: scales and decoded values live only
+    // until they are packed
+    template <int SDT>
+    __device__ __forceinline__ void store_both(bf16_t* b) {
+        uint32_t ev[8], od[8];                       // packed bf16 pairs of the even / the odd row
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {                // code dword q: columns 4q .. 4q + 3
+            float sc[4];
+            if (SDT == XQ_SCALE_F32) {
+                const u32x4& f = q == 0 ? s0 : q == 1 ? s1 : q == 2 ? s2 : s3;
+#pragma unroll
+                for (int c = 0; c < 4; ++c) sc[c] = __uint_as_float(f[c]);
+            } else if (SDT == XQ_SCALE_BF16) {
+                const u32x4& h = q < 2 ? s0 : s1;
+                const uint32_t d0 = h[(2 * q) & 3], d1 = h[((2 * q) & 3) + 1];
+                sc[0] = __uint_as_float(d0 << 16); sc[1] = __uint_as_float(d0 & 0xffff0000u);
+                sc[2] = __uint_as_float(d1 << 16); sc[3] = __uint_as_float(d1 & 0xffff0000u);
+            } else {
+                const f32x2 lo = e4m3x2_to_f32(s0[q], false), hi = e4m3x2_to_f32(s0[q], true);
+                sc[0] = lo[0]; sc[1] = lo[1]; sc[2] = hi[0]; sc[3] = hi[1];
+            }
+            if (FMT == XQ_FMT_NVFP4) {
+#pragma unroll
+                for (int c = 0; c < 4; ++c) sc[c] = sc[c] * gs;
+            }
+            const uint32_t w = raw[q];
+            float e[4], o[4];
+            if (FMT == XQ_FMT_NVFP4) {
+                const f32x2 x0 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 0), x1 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 1);
+                const f32x2 x2 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 2), x3 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 3);
+                e[0] = x0[0] * sc[0]; o[0] = x0[1] * sc[0]; e[1] = x1[0] * sc[1]; o[1] = x1[1] * sc[1];
+                e[2] = x2[0] * sc[2]; o[2] = x2[1] * sc[2]; e[3] = x3[0] * sc[3]; o[3] = x3[1] * sc[3];
+            } else if (FMT == XQ_FMT_INT4) {
+                const uint32_t lo = w & 0x0f0f0f0fu, hi = (w >> 4) & 0x0f0f0f0fu;
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    const float m8s = -8.0f * sc[c];
+                    e[c] = __builtin_fmaf((float)((lo >> (8 * c)) & 0xffu), sc[c], m8s);
+                    o[c] = __builtin_fmaf((float)((hi >> (8 * c)) & 0xffu), sc[c], m8s);
+                }
+            } else {
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    e[c] = nf4_lds[(w >> (8 * c)) & 0xfu] * sc[c];
+                    o[c] = nf4_lds[(w >> (8 * c + 4)) & 0xfu] * sc[c];
+                }
+            }
+            ev[2 * q] = pack_bf16x2(e[0], e[1]); ev[2 * q + 1] = pack_bf16x2(e[2], e[3]);
+            od[2 * q] = pack_bf16x2(o[0], o[1]); od[2 * q + 1] = pack_bf16x2(o[2], o[3]);
+        }
+        const u32x4 elo = {ev[0], ev[1], ev[2], ev[3]}, ehi = {ev[4], ev[5], ev[6], ev[7]};
+        const u32x4 olo = {od[0], od[1], od[2], od[3]}, ohi = {od[4], od[5], od[6], od[7]};
+        if (CC) {
+            const int u = 2 * (tid >> 2) * 4 + (tid & 3);
+            store_run16<true, T>(b, u, elo, ehi);
+            store_run16<true, T>(b, u + 4, olo, ohi);
+        } else {
+            bf16_t* d = b + row * Geo<T>::NN_PITCH + (tid % Geo<T>::RPR) * 16;
+            *(u32x4*)d = elo;
+            *(u32x4*)(d + 8) = ehi;
+            *(u32x4*)(d + Geo<T>::NN_PITCH) = olo;
+            *(u32x4*)(d + Geo<T>::NN_PITCH + 8) = ohi;
+        }
+    }
+    // the kernel stores a thread's two runs one after the other: the first call does both
+    __device__ __forceinline__ void store(bf16_t* b, int p) {
+        if (p != 0) return;
+        if (sdt == XQ_SCALE_F32) store_both<XQ_SCALE_F32>(b);
+        else if (sdt == XQ_SCALE_BF16) store_both<XQ_SCALE_BF16>(b);
+        else store_both<XQ_SCALE_E4M3>(b);
+    }
+};
+
+template <int FMT, bool CC, bool GROUPED, int T> struct W256Sel { using type = W256Flat4<FMT, CC, T>; };
+template <int FMT, bool CC, int T> struct W256Sel<FMT, CC, true, T> { using type = W256Gkn4<FMT, CC, T>; };   // expert banks
+template <bool CC, bool GROUPED, int T> struct W256Sel<XQ_FMT_FP8, CC, GROUPED, T> { using type = W256Fp8<CC, T>; };
+template <bool CC, int T> struct W256Sel<XQ_FMT_FP8, CC, true, T> { using type = W256Fp8<CC, T>; };
 
 // ---------------------------------------------------------------- the kernel
 template <int FMT, bool CC, bool GROUPED, int T>
@@ -319,7 +440,7 @@ __global__ void __launch_bounds__(2 * T, 2) gemm_256_kernel(G256Args g) {
         a_src[p] = g.A + r * g.lda + (u & 7) * 8;
         a_dst[p] = swz(u >> 3, u & 7);
     }
-    typename W256Sel<FMT, CC, T>::type wl;
+    typename W256Sel<FMT, CC, GROUPED, T>::type wl;
     wl.init(g, g.W + (int64_t)e * g.packed_stride, g.scales + (int64_t)e * g.scale_stride,
             FMT == XQ_FMT_NVFP4 ? g.global_scale[e] : 1.0f, n0, tid);
     if constexpr (FMT == XQ_FMT_NF4) {
