@@ -175,11 +175,14 @@ def other_config(cfg: int, dev):
         return (step, sum(lin_flops(Mtok, K, N, 16) for (N, K) in shapes.values()), False,
                 "configs[2]: nvfp4 QLoRA Qwen3-32B attention projections q/k/v/o, hidden 5120, M=4096, r=16, fwd+bwd",
                 "gemm_256_kernel<nvfp4> with 256x256 tiles (whole rounds of the chip) and 128x128 tiles (k/v forward, trailing rows): fused dequant-GEMM, forward and dgrad launches")
-    if cfg == 3:
-        from xorl_amd.qlora import BlockFP8QLoRAMoeExperts
+    if cfg in (3, 7, 8):
+        # 7 / 8 are not BASELINE configs: configs[3] with the banks held as nvfp4 / NF4 (4-bit GKN storage)
+        from xorl_amd.qlora import BlockFP8QLoRAMoeExperts, NF4QLoRAMoeExperts, NvFP4QLoRAMoeExperts
 
         E, Hd, I, T, topk, r = 128, 2048, 768, 16384, 8, 16
-        m = BlockFP8QLoRAMoeExperts(E, E, I, Hd, r=r, lora_alpha=2 * r, hybrid_shared=False).to(dev)
+        cls, fmt_name, kfmt = {3: (BlockFP8QLoRAMoeExperts, "block_fp8", "fp8"), 7: (NvFP4QLoRAMoeExperts, "nvfp4", "nvfp4 GKN"),
+                               8: (NF4QLoRAMoeExperts, "NF4", "nf4 GKN")}[cfg]
+        m = cls(E, E, I, Hd, r=r, lora_alpha=2 * r, hybrid_shared=False).to(dev)
         g = torch.Generator(device=dev).manual_seed(50)
         w = lambda *shape: torch.randn(*shape, generator=g, device=dev) * 0.02
         m.load_weights(w(E, Hd, I), w(E, Hd, I), w(E, I, Hd))
@@ -201,10 +204,11 @@ def other_config(cfg: int, dev):
             m(x, rw, sel).backward(dy)
         R = T * topk
         return (step, R * (12.0 * Hd * I + 18.0 * r * (Hd + I)), False,
-                f"configs[3]: grouped block_fp8 QLoRA Qwen3-30B-A3B experts, E=128, hidden 2048, intermediate 768, "
+                f"{'configs[3]' if cfg == 3 else 'configs[3] shapes with ' + fmt_name + ' banks (not a BASELINE config)'}: "
+                f"grouped {fmt_name} QLoRA Qwen3-30B-A3B experts, E=128, hidden 2048, intermediate 768, "
                 f"top-8 of 16384 tokens, Zipf(1.1) counts (max {int(counts.max())}, {int((counts == 0).sum())} empty), "
                 f"per-expert r=16, fwd+bwd",
-                "gemm_256_kernel<fp8, grouped> (fused dequant grouped GEMM, forward and dgrad launches)")
+                f"gemm_256_kernel<{kfmt}, grouped> (fused dequant grouped GEMM, forward and dgrad launches)")
     if cfg == 4:
         shapes = {"q": (4096, 4096), "kv": (1024, 4096), "gate_up": (12288, 4096), "down": (4096, 12288)}
         cases, total = [], 0.0
