@@ -83,7 +83,7 @@ __global__ void __launch_bounds__(256) silu_mul_bwd_kernel(const bf16_t* gate, c
 }
 
 // ------------------------------------------------------------------ routing
-constexpr int RB_CHUNK = 1024;  // routed entries per block (one wave walks them in order)
+constexpr int RB_CHUNK = 256;   // routed entries per block (one wave walks them in order)
 constexpr int RB_MAX_E = 1024;
 
 // pass 1: per-chunk histogram
@@ -103,64 +103,119 @@ __global__ void __launch_bounds__(64) route_hist_kernel(const int32_t* sel, int6
     for (int e = threadIdx.x; e < E; e += 64) chunk_counts[(int64_t)blockIdx.x * E + e] = cnt[e];
 }
 
-// pass 2 (one block): totals, expert offsets, tile offsets, and per-chunk bases (exclusive scan over chunks)
-__global__ void __launch_bounds__(256) route_scan_kernel(int32_t* chunk_counts, int32_t n_chunks, int32_t E,
-                                                         int32_t* counts, int32_t* offsets, int32_t* tile_offsets) {
-    __shared__ int32_t tot[RB_MAX_E];
-    for (int e = threadIdx.x; e < E; e += 256) {
-        int32_t run = 0;
-        for (int c = 0; c < n_chunks; ++c) {
-            int32_t v = chunk_counts[(int64_t)c * E + e];
-            chunk_counts[(int64_t)c * E + e] = run;  // becomes the chunk's base within the expert
-            run += v;
+// pass 2 (one block of 16 waves): totals, expert offsets, tile offsets, and per-chunk bases (exclusive scan over
+// chunks).  The counts are a [chunk][expert] matrix; wave w owns the chunk rows [w * cpw, (w + 1) * cpw) and its
+// lanes the experts (a row is read with coalesced loads, eight rows in flight): column sums of the wave's rows,
+// then, through LDS, each wave's base = the sums of the waves before it, then the running base written back over
+// the counts.  The prefixes over experts are one wave's scans, 64 experts at a time.
+__device__ __forceinline__ int32_t wave_inclusive_scan(int32_t v, int lane) {
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const int32_t u = __shfl_up(v, o, 64);
+        if (lane >= o) v += u;
+    }
+    return v;
+}
+
+__global__ void __launch_bounds__(1024) route_scan_kernel(int32_t* chunk_counts, int32_t n_chunks, int32_t E,
+                                                          int32_t* counts, int32_t* offsets, int32_t* tile_offsets) {
+    extern __shared__ int32_t scan_lds[];
+    int32_t* part = scan_lds;            // [16][E]
+    int32_t* tot = scan_lds + 16 * E;    // [E]
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int cpw = (n_chunks + 15) >> 4;
+    const int c_begin = wave * cpw, c_end = c_begin + cpw < n_chunks ? c_begin + cpw : n_chunks;
+    const int c_last = n_chunks - 1;
+    for (int e = lane; e < E; e += 64) {
+        int32_t sum = 0;
+        for (int c = c_begin; c < c_end; c += 8) {
+            int32_t v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = chunk_counts[(int64_t)(c + u < c_end ? c + u : c_last) * E + e];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) sum += c + u < c_end ? v[u] : 0;
         }
-        tot[e] = run;
-        counts[e] = run;
+        part[wave * E + e] = sum;
     }
     __syncthreads();
-    if (threadIdx.x == 0) {
+    for (int e = lane; e < E; e += 64) {
+        int32_t run = 0, total = 0;
+        for (int w = 0; w < 16; ++w) {
+            const int32_t v = part[w * E + e];
+            run += w < wave ? v : 0;
+            total += v;
+        }
+        if (wave == 0) {
+            tot[e] = total;
+            counts[e] = total;
+        }
+        for (int c = c_begin; c < c_end; c += 8) {
+            int32_t v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = chunk_counts[(int64_t)(c + u < c_end ? c + u : c_last) * E + e];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                if (c + u < c_end) {
+                    chunk_counts[(int64_t)(c + u) * E + e] = run;   // becomes the chunk's base within the expert
+                    run += v[u];
+                }
+            }
+        }
+    }
+    __syncthreads();
+    if (wave == 0) {
         int32_t o = 0, t = 0, t2 = 0;
         int32_t* tiles256 = tile_offsets + (E + 1);
-        for (int e = 0; e < E; ++e) {
-            offsets[e] = o;
-            tile_offsets[e] = t;
-            tiles256[e] = t2;
-            o += tot[e];
-            t += (tot[e] + 127) / 128;
-            t2 += (tot[e] + 255) / 256;
+        for (int e0 = 0; e0 < E; e0 += 64) {
+            const int e = e0 + lane;
+            const int32_t c = e < E ? tot[e] : 0;
+            const int32_t c128 = (c + 127) / 128, c256 = (c + 255) / 256;
+            const int32_t io = wave_inclusive_scan(c, lane), it = wave_inclusive_scan(c128, lane), it2 = wave_inclusive_scan(c256, lane);
+            if (e < E) {
+                offsets[e] = o + io - c;
+                tile_offsets[e] = t + it - c128;
+                tiles256[e] = t2 + it2 - c256;
+            }
+            o += __shfl(io, 63, 64);
+            t += __shfl(it, 63, 64);
+            t2 += __shfl(it2, 63, 64);
         }
-        offsets[E] = o;
-        tile_offsets[E] = t;
-        tiles256[E] = t2;
+        if (lane == 0) {
+            offsets[E] = o;
+            tile_offsets[E] = t;
+            tiles256[E] = t2;
+        }
     }
 }
 
-// pass 3: stable position of every routed entry (one wave per chunk, in order)
-__global__ void __launch_bounds__(64) route_place_kernel(const int32_t* sel, int64_t n, int32_t E,
+// pass 3: stable position of every routed entry (one wave per chunk, in order).  The lanes of a 64-entry segment that
+// hold the same expert are found by intersecting, over the bits of the expert id, the ballots of "my value of
+// this bit"; a lane's position is the expert's running base plus the number of such lanes below it.
+__global__ void __launch_bounds__(64) route_place_kernel(const int32_t* sel, int64_t n, int32_t E, int32_t id_bits,
                                                          const int32_t* chunk_base, const int32_t* offsets,
                                                          int32_t* scatter_index) {
     __shared__ int32_t run[RB_MAX_E];
     for (int e = threadIdx.x; e < E; e += 64) run[e] = offsets[e] + chunk_base[(int64_t)blockIdx.x * E + e];
     __syncthreads();
     const int lane = threadIdx.x;
+    const uint64_t below = (1ull << lane) - 1ull;
     int64_t base = (int64_t)blockIdx.x * RB_CHUNK;
     for (int seg = 0; seg < RB_CHUNK; seg += 64) {
         int64_t idx = base + seg + lane;
         bool valid = idx < n;
         int e = valid ? sel[idx] : -1;
         if (e >= E) e = -1;
-        int before = 0, after = 0;
-        for (int j = 0; j < 64; ++j) {
-            int ej = __shfl(e, j, 64);
-            bool same = (ej == e) && (e >= 0);
-            before += (same && j < lane) ? 1 : 0;
-            after += (same && j > lane) ? 1 : 0;
+        uint64_t same = __ballot(e >= 0);
+        for (int b = 0; b < id_bits; ++b) {
+            const bool bit = (e >> b) & 1;
+            const uint64_t m = __ballot(bit);
+            same &= bit ? m : ~m;
         }
-        if (e >= 0) {
-            scatter_index[idx] = run[e] + before;
-        }
+        const int before = __popcll(same & below);
+        const bool last = (same & ~below & ~(1ull << lane)) == 0;   // no higher lane holds this expert
+        if (e >= 0) scatter_index[idx] = run[e] + before;
         __syncthreads();
-        if (e >= 0 && after == 0) run[e] += before + 1;  // last lane of this expert in the segment
+        if (e >= 0 && last) run[e] += before + 1;
         __syncthreads();
     }
 }
@@ -290,10 +345,20 @@ extern "C" int xq_route_build(const int32_t* selected, int64_t n_routed, int32_t
     int32_t* cc = (int32_t*)workspace;
     route_hist_kernel<<<dim3(n_chunks), 64, 0, stream>>>(selected, n_routed, num_experts, cc);
     XQ_CHECK_LAUNCH("route_hist");
-    route_scan_kernel<<<dim3(1), 256, 0, stream>>>(cc, n_chunks, num_experts, counts, offsets, tile_offsets);
+    static bool scan_attr_set = false;
+    if (!scan_attr_set) {
+        if (hipFuncSetAttribute((const void*)route_scan_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 17 * RB_MAX_E * 4) != hipSuccess) {
+            xq_set_error("xq_route_build: cannot raise the dynamic LDS limit");
+            return XQ_ERR_LAUNCH;
+        }
+        scan_attr_set = true;
+    }
+    route_scan_kernel<<<dim3(1), 1024, (size_t)17 * num_experts * 4, stream>>>(cc, n_chunks, num_experts, counts, offsets, tile_offsets);
     XQ_CHECK_LAUNCH("route_scan");
     if (n_routed > 0) {
-        route_place_kernel<<<dim3(n_chunks), 64, 0, stream>>>(selected, n_routed, num_experts, cc, offsets, scatter_index);
+        int id_bits = 0;
+        while ((1 << id_bits) < num_experts) ++id_bits;
+        route_place_kernel<<<dim3(n_chunks), 64, 0, stream>>>(selected, n_routed, num_experts, id_bits, cc, offsets, scatter_index);
         XQ_CHECK_LAUNCH("route_place");
     }
     return XQ_OK;
