@@ -276,45 +276,57 @@ constexpr int TN_QP = 80;        // Qs pitch: 160 B rows
 
 constexpr int TN_CHUNK = 1024;   // grouped: rows per block (global row chunks, cut at expert boundaries)
 
-// acc += P[m_begin:m_end, c0 + wave*32 .. +32]^T . Q[m_begin:m_end, :]; the next 32-row tile is
-// fetched into registers while the current one is multiplied out of LDS.
+// acc += P[m_begin:m_end, c0 + wave*32 .. +32]^T . Q[m_begin:m_end, :]  (m_begin < m_end).  Rows go through LDS 32 at
+// a time, in two alternating buffers (Ps, Qs hold both), so one block barrier per tile is enough; the tiles m + 64
+// and m + 96 are in flight in registers while tiles m and m + 32 are multiplied.  Every load is unconditional:
+// rows past m_end are clamped onto the last row and their Q values replaced by zero, columns past the width are
+// clamped onto column 0 and never written.
 template <int NT>
 __device__ __forceinline__ void tn_accumulate(const TnArgs& g, int64_t c0, int64_t m_begin, int64_t m_end, bf16_t* Ps,
                                               bf16_t* Qs, f32x16* acc) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int pr = tid >> 4, pc = (tid & 15) * 8;  // P tile: rows pr, pr+16; 8 cols at pc
-    const bool pcol_ok = c0 + pc < g.width;        // width % 8 == 0
+    const int64_t pcol = c0 + pc < g.width ? c0 + pc : 0;   // width % 8 == 0
     const int qchunks = g.r_pad / 8;
-    const int qr = tid / qchunks, qc = (tid % qchunks) * 8;
     const bool q_thread = tid < 32 * qchunks;
+    const int qr = q_thread ? tid / qchunks : 0, qc = q_thread ? (tid % qchunks) * 8 : 0;
     const u32x4 z = {0, 0, 0, 0};
-    u32x4 p0 = z, p1 = z, qv = z;
-    auto fetch = [&](int64_t m) {
-        p0 = z; p1 = z; qv = z;
-        if (pcol_ok) {
-            if (m + pr < m_end) p0 = *(const u32x4*)(g.P + (m + pr) * g.ldp + c0 + pc);
-            if (m + pr + 16 < m_end) p1 = *(const u32x4*)(g.P + (m + pr + 16) * g.ldp + c0 + pc);
-        }
-        if (q_thread && m + qr < m_end) qv = *(const u32x4*)(g.Q + (m + qr) * g.r_pad + qc);
+    const int64_t last = m_end - 1;
+    struct Tile { u32x4 p0, p1, q; };
+    auto fetch = [&](Tile& t, int64_t m) {
+        const int64_t r0 = m + pr < m_end ? m + pr : last, r1 = m + pr + 16 < m_end ? m + pr + 16 : last;
+        const int64_t rq = m + qr < m_end ? m + qr : last;
+        t.p0 = *(const u32x4*)(g.P + r0 * g.ldp + pcol);
+        t.p1 = *(const u32x4*)(g.P + r1 * g.ldp + pcol);
+        t.q = *(const u32x4*)(g.Q + rq * g.r_pad + qc);
     };
-    if (m_begin < m_end) fetch(m_begin);
-    for (int64_t m = m_begin; m < m_end; m += 32) {
-        __syncthreads();  // previous tile's fragment reads are done
-        *(u32x4*)(Ps + pr * TN_PP + pc) = p0;
-        *(u32x4*)(Ps + (pr + 16) * TN_PP + pc) = p1;
-        if (q_thread) *(u32x4*)(Qs + qr * TN_QP + qc) = qv;
-        __syncthreads();
-        if (m + 32 < m_end) fetch(m + 32);
+    auto tile = [&](Tile& t, int64_t m, int buf) {     // multiply tile m out of LDS buffer `buf`, refill t with tile m + 64
+        bf16_t* ps = Ps + buf * (32 * TN_PP);
+        bf16_t* qs = Qs + buf * (32 * TN_QP);
+        *(u32x4*)(ps + pr * TN_PP + pc) = t.p0;
+        *(u32x4*)(ps + (pr + 16) * TN_PP + pc) = t.p1;
+        if (q_thread) *(u32x4*)(qs + qr * TN_QP + qc) = m + qr < m_end ? t.q : z;
+        fetch(t, m + 64);
+        // the other buffer's fragment reads lie before this barrier in every wave, its next stores after the next one
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) {
-            bf16x8 a = lds_tr_frag(Ps, TN_PP, ks * 16, wave * 32, lane);
+            bf16x8 a = lds_tr_frag(ps, TN_PP, ks * 16, wave * 32, lane);
 #pragma unroll
             for (int n = 0; n < NT; ++n) {
-                bf16x8 b = lds_tr_frag(Qs, TN_QP, ks * 16, n * 32, lane);
+                bf16x8 b = lds_tr_frag(qs, TN_QP, ks * 16, n * 32, lane);
                 acc[n] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[n], 0, 0, 0);
             }
         }
+    };
+    Tile ta, tb;
+    fetch(ta, m_begin);
+    fetch(tb, m_begin + 32);
+    for (int64_t m = m_begin; m < m_end; m += 64) {
+        tile(ta, m, 0);
+        tile(tb, m + 32, 1);        // past m_end: all-zero Q rows, no contribution
     }
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");   // the buffers are free again when this returns
 }
 
 // out[c][j] (pitch = row length of the destination) or, transposed, out[j][c]; j < r_lim
@@ -340,8 +352,8 @@ __device__ __forceinline__ void tn_write(const f32x16* acc, float* out, int64_t 
 // dense: block (col tile, row split) -> partial[split][width][r_pad]
 template <int NT>
 __global__ void __launch_bounds__(256) tn_kernel(TnArgs g) {
-    __shared__ __attribute__((aligned(16))) bf16_t Ps[32 * TN_PP];
-    __shared__ __attribute__((aligned(16))) bf16_t Qs[32 * TN_QP];
+    __shared__ __attribute__((aligned(16))) bf16_t Ps[2 * 32 * TN_PP];
+    __shared__ __attribute__((aligned(16))) bf16_t Qs[2 * 32 * TN_QP];
     const int64_t c0 = (int64_t)blockIdx.x * 128;
     const int64_t m_begin = (int64_t)blockIdx.y * g.rows_per_split;
     int64_t m_end = m_begin + g.rows_per_split;
@@ -361,8 +373,8 @@ __global__ void __launch_bounds__(256) tn_kernel(TnArgs g) {
 // next chunk to partial[chunk][1] (tn_grouped_reduce_kernel adds the pieces in chunk order).
 template <int NT>
 __global__ void __launch_bounds__(256) tn_grouped_kernel(TnArgs g, int32_t num_experts, float* partial) {
-    __shared__ __attribute__((aligned(16))) bf16_t Ps[32 * TN_PP];
-    __shared__ __attribute__((aligned(16))) bf16_t Qs[32 * TN_QP];
+    __shared__ __attribute__((aligned(16))) bf16_t Ps[2 * 32 * TN_PP];
+    __shared__ __attribute__((aligned(16))) bf16_t Qs[2 * 32 * TN_QP];
     __shared__ int sh_e;
     const int64_t c0 = (int64_t)blockIdx.x * 128;
     const int64_t r_begin = (int64_t)blockIdx.y * TN_CHUNK;
