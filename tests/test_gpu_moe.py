@@ -242,3 +242,61 @@ def test_grouped_gemm_decode_bit_exact(hip_device, tile_policy, fmt):
             same = y.view(torch.int16) == want.view(torch.int16)
             both_zero = (y.float() == 0) & (want.float() == 0)
             assert bool((same | both_zero).all()), (proj, transpose_w)
+
+
+@pytest.mark.parametrize("tile_policy", [1, 2, 3], indirect=True)
+@pytest.mark.parametrize("scale_dtype,group", [(torch.float32, 128), (torch.bfloat16, 32), (torch.float32, 16)])
+def test_grouped_gemm_int4_gkn_bank_bit_exact(hip_device, tile_policy, scale_dtype, group):
+    """int4 banks have no module of their own; through the C ABI they take the same grouped kernels (and, with bf16
+    scales, the one scale storage the modules do not produce).  Identity rows again: both products must return the
+    oracle's bank decode bit for bit."""
+    from xorl_amd import _C, moe_functional as MF
+    from xorl_amd import quantize as Q
+    from xorl_amd.functional import QuantWeight
+
+    E, K, N = 3, 256, 320
+    packed, scales, ref = [], [], []
+    for e in range(E):
+        p, s = Q.int4_quantize_gkn(gen((K, N), 0.05, 80 + e), group)
+        s = s.to(scale_dtype)
+        packed.append(p)
+        scales.append(s)
+        ref.append(bits_to_bf16(NP.int4_decode_gkn(p.numpy(), s.float().numpy(), K, N, group)))
+    qw = QuantWeight("int4", _C.XQ_LAYOUT_GKN, torch.stack(packed).to(hip_device), torch.stack(scales).to(hip_device),
+                     scale_dtype, K, N, group, num_experts=E)
+    ref = torch.stack(ref).to(hip_device)
+    for transpose_w, rows in ((False, K), (True, N)):
+        sel = torch.arange(E, dtype=torch.int32).repeat_interleave(rows).reshape(-1, 1).to(hip_device)
+        counts, offsets, sidx, tile_offsets = MF.route_build(sel, E)
+        a = torch.eye(rows, dtype=torch.bfloat16, device=hip_device).repeat(E, 1)
+        y = MF._grouped_gemm(qw, transpose_w, a, offsets, tile_offsets, None, None)
+        want = (ref.transpose(1, 2) if transpose_w else ref).reshape(E * rows, -1).contiguous()
+        same = y.view(torch.int16) == want.view(torch.int16)
+        both_zero = (y.float() == 0) & (want.float() == 0)
+        assert bool((same | both_zero).all()), transpose_w
+
+
+def test_nvfp4_bank_with_folded_fp32_scales_matches_e4m3_storage(hip_device):
+    """A modelopt checkpoint loads as fp32 block scales with the global scale folded in (stored global = 1); the
+    same codes with e4m3 block scales and a separate global decode to the same values, so both storages must give
+    identical outputs and gradients through the grouped kernels."""
+    E, H, I, r = 4, 256, 384, 8
+    m1, _ = _make_experts("nvfp4", E, H, I, r, False, seed=90, device=hip_device)
+    m2, _ = _make_experts("nvfp4", E, H, I, r, False, seed=90, device=hip_device)
+    for p in ("gate", "up", "down"):
+        bs = getattr(m1, f"{p}_block_scales").view(torch.float8_e4m3fn).float()             # [E, K/16, N]
+        g = getattr(m1, f"{p}_global_scale").contiguous().view(torch.float32).reshape(E, 1, 1)
+        setattr(m2, f"{p}_block_scales", m2._to_uint8((bs * g).contiguous()))
+        setattr(m2, f"{p}_global_scale", m2._to_uint8(torch.ones(E, 1, dtype=torch.float32, device=hip_device)))
+        m2._scale_dtypes[p] = {"weight_block_scales": torch.float32, "weight_global_scale": torch.float32}
+    rw, sel = _zipf_routing(500, E, 2, seed=5, empty=0)
+    x = gen((500, H), 1.0, 6, torch.bfloat16).to(hip_device)
+    dy = gen((500, H), 1.0, 7, torch.bfloat16).to(hip_device)
+    outs = []
+    for m in (m1, m2):
+        xd = x.clone().requires_grad_(True)
+        y = m(xd, rw.to(torch.bfloat16).to(hip_device), sel.to(hip_device))
+        y.backward(dy)
+        outs.append((y.detach(), xd.grad, m.gate_proj_lora_A.grad.clone(), m.down_proj_lora_B.grad.clone()))
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
