@@ -6,7 +6,7 @@
  * kernel is a Triton function called from Python.  Each entry point below
  * therefore names the Python function(s) of the reference it replaces
  * (paths relative to the xorl checkout).  A maintainer binds these with
- * ctypes; no torch type appears in any signature.
+ * ctypes (xorl_amd/_C.py holds every signature); no torch type appears in any signature.
  *
  * Conventions
  *   - every pointer is a DEVICE pointer unless stated otherwise;
