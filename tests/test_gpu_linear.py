@@ -139,3 +139,23 @@ def test_silu_and_mul(hip_device):
     (torch.nn.functional.silu(g64) * u64).backward(dh.double())
     assert R.max_rel_err(gd.grad.cpu(), g64.grad) <= TOL
     assert R.max_rel_err(ud.grad.cpu(), u64.grad) <= TOL
+
+
+@pytest.mark.parametrize("fmt,M,K,N", [("block_fp8", 4100, 256, 4096), ("int4", 4352, 384, 5120), ("nvfp4", 4099, 256, 4352)])
+def test_dense_split_launch_tail_rows(hip_device, fmt, M, K, N):
+    """Shapes whose 256x256 tiling leaves a partly filled last round of the chip: the launcher runs the leading
+    tile rows on large tiles and the trailing rows (here 4, 256 and 3 + 256 of them) as a second launch of small
+    tiles.  Forward, dgrad and both factor gradients against the float64 form, with particular attention to the
+    rows on either side of the seam."""
+    r = 16
+    m, w_ref = make_dense_module(fmt, N, K, r, 32, seed=M + N, device=hip_device, bias=True)
+    x = gen((M, K), 1.0, 31, torch.bfloat16)
+    dy = gen((M, N), 1.0, 32, torch.bfloat16)
+    y, dx, dA, dB = _run(m, x.to(hip_device), dy.to(hip_device))
+    ex = R.linear_fwd_bwd_exact(x, w_ref, m.lora_A.detach().cpu(), m.lora_B.detach().cpu(), m.scaling, dy,
+                                bias=m.bias.detach().cpu())
+    for name, got, ref in (("y", y, ex["y"]), ("dx", dx, ex["dx"]), ("dA", dA, ex["dA"]), ("dB", dB, ex["dB"])):
+        assert R.max_rel_err(got.cpu(), ref) <= TOL, f"{fmt} {name}"
+    seam = slice((M // 256) * 256 - 300, M)
+    assert R.max_rel_err(y.cpu()[seam], ex["y"][seam]) <= TOL
+    assert R.max_rel_err(dx.cpu()[seam], ex["dx"][seam]) <= TOL
