@@ -159,3 +159,27 @@ def test_dense_split_launch_tail_rows(hip_device, fmt, M, K, N):
     seam = slice((M // 256) * 256 - 300, M)
     assert R.max_rel_err(y.cpu()[seam], ex["y"][seam]) <= TOL
     assert R.max_rel_err(dx.cpu()[seam], ex["dx"][seam]) <= TOL
+
+
+@pytest.mark.parametrize("fmt", ["block_fp8", "nvfp4"])
+@pytest.mark.parametrize("M", [8, 300])
+def test_row_strided_activations(hip_device, fmt, M):
+    """x and dY that are column windows of wider tensors (row stride > width, 16-byte aligned) are consumed in
+    place through their leading dimension: skinny forward (M = 8, no grad), tile forward and backward."""
+    K, N, r = 1024, 384, 16
+    m, w_ref = make_dense_module(fmt, N, K, r, 32, seed=M, device=hip_device)
+    xw = gen((M, K + 64), 1.0, 41, torch.bfloat16).to(hip_device)
+    dyw = gen((M, N + 128), 1.0, 42, torch.bfloat16).to(hip_device)
+    x, dy = xw[:, 32:32 + K], dyw[:, 64:64 + N]
+    assert not x.is_contiguous() and not dy.is_contiguous()
+    A, B = m.lora_A.detach().cpu(), m.lora_B.detach().cpu()
+    ex = R.linear_fwd_bwd_exact(x.cpu(), w_ref, A, B, m.scaling, dy.cpu())
+    with torch.no_grad():
+        assert R.max_rel_err(m(x).cpu(), ex["y"]) <= TOL
+    xg = x.detach().requires_grad_(True)
+    y = m(xg)
+    y.backward(dy)
+    assert R.max_rel_err(y.detach().cpu(), ex["y"]) <= TOL
+    assert R.max_rel_err(xg.grad.cpu(), ex["dx"]) <= TOL
+    assert R.max_rel_err(m.lora_A.grad.cpu(), ex["dA"]) <= TOL
+    assert R.max_rel_err(m.lora_B.grad.cpu(), ex["dB"]) <= TOL
