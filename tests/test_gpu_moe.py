@@ -300,3 +300,27 @@ def test_nvfp4_bank_with_folded_fp32_scales_matches_e4m3_storage(hip_device):
         outs.append((y.detach(), xd.grad, m.gate_proj_lora_A.grad.clone(), m.down_proj_lora_B.grad.clone()))
     for a, b in zip(*outs):
         assert torch.equal(a, b)
+
+
+def test_empty_batches(hip_device):
+    """No tokens at all: the dense module and the expert module return empty outputs, and a backward pass leaves
+    exact-zero factor gradients (the reference's zero-size guards, ops/moe/lora.py:566-570)."""
+    m, _ = _make_experts("block_fp8", 4, 128, 128, 8, True, seed=70, device=hip_device)
+    x = torch.zeros(0, 128, dtype=torch.bfloat16, device=hip_device, requires_grad=True)
+    rw = torch.zeros(0, 2, dtype=torch.bfloat16, device=hip_device)
+    sel = torch.zeros(0, 2, dtype=torch.int32, device=hip_device)
+    y = m(x, rw, sel)
+    assert y.shape == (0, 128)
+    y.sum().backward()
+    for k in ("gate", "up", "down"):
+        for f in ("A", "B"):
+            g = getattr(m, f"{k}_proj_lora_{f}").grad
+            assert g is not None and torch.count_nonzero(g) == 0
+    from tests.util_cases import make_dense_module
+
+    d, _ = make_dense_module("nvfp4", 128, 256, 8, 16, seed=71, device=hip_device)
+    xd = torch.zeros(0, 256, dtype=torch.bfloat16, device=hip_device, requires_grad=True)
+    yd = d(xd)
+    assert yd.shape == (0, 128)
+    yd.sum().backward()
+    assert torch.count_nonzero(d.lora_A.grad) == 0 and torch.count_nonzero(d.lora_B.grad) == 0

@@ -219,13 +219,13 @@ extern "C" int xq_linear_fwd(const xq_weight* w, const void* x, int64_t ldx, int
     int rc = check_dense(w, "xq_linear_fwd");
     if (rc) return rc;
     const int64_t N = w->rows, K = w->cols;
-    XQ_REQUIRE(M >= 0 && x && y, "xq_linear_fwd: NULL activation pointer");
+    XQ_REQUIRE(M >= 0 && (M == 0 || (x && y)), "xq_linear_fwd: NULL activation pointer");   // an empty batch has no storage
     XQ_REQUIRE(r >= 0 && r <= 64, "xq_linear_fwd: LoRA rank %d out of range [0, 64]", r);
     XQ_REQUIRE(r == 0 || (lora_A && lora_B), "xq_linear_fwd: LoRA factors are NULL");
     XQ_REQUIRE(lora_dtype == XQ_DT_F32 || lora_dtype == XQ_DT_BF16, "xq_linear_fwd: bad lora_dtype");
-    XQ_REQUIRE(ldy % 8 == 0 && xq_aligned(y, 16), "xq_linear_fwd: y rows must be 16-byte aligned");
     hipStream_t stream = (hipStream_t)stream_;
     if (M == 0) return XQ_OK;
+    XQ_REQUIRE(ldy % 8 == 0 && xq_aligned(y, 16), "xq_linear_fwd: y rows must be 16-byte aligned");
     const int rp = r_pad_of(r);
     // decode / rollout shapes: stream the packed weight once (HBM-bound kernel); forward only
     if (!su_out && g_skinny_enabled && skinny_supported(w, M))
@@ -254,12 +254,12 @@ extern "C" int xq_linear_bwd(const xq_weight* w, const void* x, int64_t ldx, con
     int rc = check_dense(w, "xq_linear_bwd");
     if (rc) return rc;
     const int64_t N = w->rows, K = w->cols;
-    XQ_REQUIRE(M >= 0 && dy, "xq_linear_bwd: dy is NULL");
+    XQ_REQUIRE(M >= 0 && (M == 0 || dy), "xq_linear_bwd: dy is NULL");
     XQ_REQUIRE(r >= 0 && r <= 64, "xq_linear_bwd: LoRA rank %d out of range [0, 64]", r);
     XQ_REQUIRE(r == 0 || (lora_A && lora_B), "xq_linear_bwd: LoRA factors are NULL");
     XQ_REQUIRE(lora_dtype == XQ_DT_F32 || lora_dtype == XQ_DT_BF16, "xq_linear_bwd: bad lora_dtype");
     XQ_REQUIRE(!(dA || dB) || r > 0, "xq_linear_bwd: factor gradients requested with r == 0");
-    XQ_REQUIRE(!(dA || dB) || x, "xq_linear_bwd: x is needed for the factor gradients");
+    XQ_REQUIRE(!(dA || dB) || M == 0 || x, "xq_linear_bwd: x is needed for the factor gradients");
     hipStream_t stream = (hipStream_t)stream_;
     const int rp = r_pad_of(r);
     if (M == 0) {

@@ -303,10 +303,10 @@ __global__ void __launch_bounds__(256) moe_gather_kernel(const bf16_t* rows, con
 
 extern "C" int xq_silu_mul_fwd(const void* gate, const void* up, int64_t ld_in, const float* row_w, void* h,
                                int64_t ld_h, int64_t rows, int64_t cols, void* stream) {
-    XQ_REQUIRE(gate && up && h, "xq_silu_mul_fwd: NULL pointer");
     XQ_REQUIRE(cols % 8 == 0 && ld_in % 8 == 0 && ld_h % 8 == 0, "xq_silu_mul_fwd: cols and strides must be multiples of 8");
+    if (rows == 0 || cols == 0) return XQ_OK;   // an empty batch has no storage to point at
+    XQ_REQUIRE(gate && up && h, "xq_silu_mul_fwd: NULL pointer");
     XQ_REQUIRE(xq_aligned(gate, 16) && xq_aligned(up, 16) && xq_aligned(h, 16), "xq_silu_mul_fwd: pointers must be 16-byte aligned");
-    if (rows == 0 || cols == 0) return XQ_OK;
     int64_t total = rows * (cols / 8);
     silu_mul_fwd_kernel<<<dim3((unsigned)xq_cdiv(total, 256)), 256, 0, (hipStream_t)stream>>>(
         (const bf16_t*)gate, (const bf16_t*)up, ld_in, row_w, (bf16_t*)h, ld_h, rows, cols / 8);
@@ -317,11 +317,11 @@ extern "C" int xq_silu_mul_fwd(const void* gate, const void* up, int64_t ld_in, 
 extern "C" int xq_silu_mul_bwd(const void* gate, const void* up, int64_t ld_in, const void* dh, int64_t ld_dh,
                                const float* row_w, void* dgate, void* dup, int64_t ld_out, float* d_row_w,
                                int64_t rows, int64_t cols, void* stream) {
-    XQ_REQUIRE(gate && up && dh && dgate && dup, "xq_silu_mul_bwd: NULL pointer");
     XQ_REQUIRE(cols % 8 == 0 && ld_in % 8 == 0 && ld_dh % 8 == 0 && ld_out % 8 == 0, "xq_silu_mul_bwd: cols and strides must be multiples of 8");
+    if (rows == 0 || cols == 0) return XQ_OK;   // an empty batch has no storage to point at
+    XQ_REQUIRE(gate && up && dh && dgate && dup, "xq_silu_mul_bwd: NULL pointer");
     XQ_REQUIRE(xq_aligned(gate, 16) && xq_aligned(up, 16) && xq_aligned(dh, 16) && xq_aligned(dgate, 16) && xq_aligned(dup, 16),
                "xq_silu_mul_bwd: pointers must be 16-byte aligned");
-    if (rows == 0 || cols == 0) return XQ_OK;
     silu_mul_bwd_kernel<<<dim3((unsigned)rows), 256, 0, (hipStream_t)stream>>>(
         (const bf16_t*)gate, (const bf16_t*)up, ld_in, (const bf16_t*)dh, ld_dh, row_w, (bf16_t*)dgate, (bf16_t*)dup,
         ld_out, d_row_w, rows, cols);
