@@ -183,3 +183,33 @@ def test_row_strided_activations(hip_device, fmt, M):
     assert R.max_rel_err(xg.grad.cpu(), ex["dx"]) <= TOL
     assert R.max_rel_err(m.lora_A.grad.cpu(), ex["dA"]) <= TOL
     assert R.max_rel_err(m.lora_B.grad.cpu(), ex["dB"]) <= TOL
+
+
+@pytest.mark.parametrize("fmt,r", [("block_fp8", 96), ("nvfp4", 128), ("int4", 72)])
+def test_ranks_above_the_fused_limit(hip_device, fmt, r):
+    """Ranks above 64: the first 64 ride in the fused kernel, the rest as library GEMMs.  Forward (tile and skinny
+    paths), all gradients, the published merged weight and merge_weights against the float64 forms."""
+    M, K, N = 300, 512, 384
+    m, w_ref = make_dense_module(fmt, N, K, r, 2 * r, seed=r, device=hip_device)
+    x = gen((M, K), 1.0, 51, torch.bfloat16)
+    dy = gen((M, N), 1.0, 52, torch.bfloat16)
+    y, dx, dA, dB = _run(m, x.to(hip_device), dy.to(hip_device))
+    A, B = m.lora_A.detach().cpu(), m.lora_B.detach().cpu()
+    ex = R.linear_fwd_bwd_exact(x, w_ref, A, B, m.scaling, dy)
+    assert dA.shape == (r, K) and dB.shape == (N, r)
+    for name, got, ref in (("y", y, ex["y"]), ("dx", dx, ex["dx"]), ("dA", dA, ex["dA"]), ("dB", dB, ex["dB"])):
+        assert R.max_rel_err(got.cpu(), ref) <= TOL, f"{fmt} {name}"
+    # every rank contributes: the tail ranks' gradients are not zero
+    assert float(dA[64:].abs().max()) > 0 and float(dB[:, 64:].abs().max()) > 0
+    with torch.no_grad():
+        ys = m(x[:4].to(hip_device))                                        # skinny path
+    assert R.max_rel_err(ys.cpu(), ex["y"][:4]) <= TOL
+    # publish and merge
+    pub = m.merged_weight().cpu()
+    want = R.merge_publish_recipe(w_ref, A, B, m.scaling)
+    assert R.max_rel_err(pub, want) <= 2 ** -7
+    m.merge_weights()
+    assert torch.count_nonzero(m.lora_B) == 0
+    merged = w_ref.double() + R.merge_delta_exact(A, B, m.scaling)
+    step = {"block_fp8": 2 ** -3, "nvfp4": 0.3, "int4": 0.2}[fmt]             # one quantization step of the format
+    assert R.max_rel_err(m._dequantize_weight().cpu().float(), merged) <= step

@@ -210,8 +210,20 @@ class QLoRALinearFunction(torch.autograd.Function):
         return (dx if need_dx else None), gA, gB, gbias, None, None, None, None
 
 
+MAX_FUSED_RANK = 64     # ranks the fused kernels carry as one extra K-step
+
+
 def qlora_linear(x: Tensor, qw: QuantWeight, lora_A: Optional[Tensor], lora_B: Optional[Tensor], r: int,
                  scaling: float, bias: Optional[Tensor] = None) -> Tensor:
+    if r > MAX_FUSED_RANK and lora_A is not None:
+        # The first 64 ranks ride in the fused kernel; the others are two plain library GEMMs on the bf16-rounded
+        # factors (fp32 accumulation), added in bf16 the way the reference adds its whole LoRA branch
+        # (qlora/modules/linear.py:376-385).  Autograd differentiates the tail; the factor slices are views, so
+        # both parts' gradients land in the same parameters.
+        y = qlora_linear(x, qw, lora_A[:MAX_FUSED_RANK], lora_B[:, :MAX_FUSED_RANK], MAX_FUSED_RANK, scaling, bias)
+        A_t, B_t = lora_A[MAX_FUSED_RANK:r].to(x.dtype), lora_B[:, MAX_FUSED_RANK:r].to(x.dtype)
+        su = (torch.nn.functional.linear(x, A_t).float() * scaling).to(x.dtype)
+        return y + torch.nn.functional.linear(su, B_t)
     # Without a backward (inference / rollout) nothing needs the saved LoRA intermediate, which
     # also lets small batches take the weight-streaming kernel.
     training = torch.is_grad_enabled() and any(

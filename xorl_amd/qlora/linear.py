@@ -31,7 +31,7 @@ from torch import Tensor
 
 from .. import _C
 from .. import quantize as Q
-from ..functional import QuantWeight, qlora_linear
+from ..functional import MAX_FUSED_RANK, QuantWeight, qlora_linear
 
 
 class LoraModule:
@@ -98,8 +98,8 @@ class QLoRALinear(LoraModule, nn.Module):
             raise TypeError(
                 "QLoRALinear is abstract. Use NvFP4QLoRALinear, BlockFP8QLoRALinear or Int4QLoRALinear."
             )
-        if r <= 0 or r > 64:
-            raise ValueError(f"LoRA rank must be in [1, 64] for the fused kernels, got {r}")
+        if r <= 0:
+            raise ValueError(f"LoRA rank must be positive, got {r}")
         super().__init__()
         self.in_features, self.out_features = in_features, out_features
         self.quant_format, self.quant_group_size = quant_format, quant_group_size
@@ -357,6 +357,9 @@ class QLoRALinear(LoraModule, nn.Module):
         from ..functional import merge_dense
 
         with torch.no_grad():
+            if self.active_r > MAX_FUSED_RANK:      # beyond the fused kernel's rank: decode kernel + the update as written there
+                w = self._dequantize_weight().to(torch.bfloat16) + self.get_delta_weight().to(torch.bfloat16)
+                return w.to(dtype)
             return merge_dense(self._quant_weight(), self._to_regular_tensor(self.lora_A),
                                self._to_regular_tensor(self.lora_B), self.active_r, self._active_scaling(), dtype)
 
@@ -469,7 +472,7 @@ class BlockFP8QLoRALinear(QLoRALinear):
         bytes (block_fp8_linear.py:111-119); falls back to the generic path for sharded (DTensor) state."""
         from ..functional import merge_requant_fp8
 
-        if _is_dtensor(self.packed_weight_f32) or _is_dtensor(self.lora_A):
+        if _is_dtensor(self.packed_weight_f32) or _is_dtensor(self.lora_A) or self.active_r > MAX_FUSED_RANK:
             return super().merge_weights(ema_decay)
         with torch.no_grad():
             packed, scales = merge_requant_fp8(self._quant_weight(), self.lora_A, self.lora_B, self.active_r,
