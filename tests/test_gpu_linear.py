@@ -213,3 +213,44 @@ def test_ranks_above_the_fused_limit(hip_device, fmt, r):
     merged = w_ref.double() + R.merge_delta_exact(A, B, m.scaling)
     step = {"block_fp8": 2 ** -3, "nvfp4": 0.3, "int4": 0.2}[fmt]             # one quantization step of the format
     assert R.max_rel_err(m._dequantize_weight().cpu().float(), merged) <= step
+
+
+@pytest.mark.parametrize("tile_policy", [0, 2], indirect=True)
+def test_dense_seeded_shape_sweep(hip_device, tile_policy):
+    """Sixteen seeded draws of (format, M, K, N, r, bias): K and N any multiple of 64, ragged M,
+    every rank 1..64 -- forward and all three gradients against the float64 form, by size-selected tiles and with
+    256x256 tiles forced."""
+    import numpy as np
+
+    rng = np.random.default_rng(7)
+    fmts = ["block_fp8", "int4", "nvfp4", "nf4"]
+    for case in range(16):
+        fmt = fmts[case % 4]
+        M = int(rng.integers(1, 700))
+        K = int(rng.integers(1, 17)) * 64
+        N = int(rng.integers(1, 13)) * 64           # the backward contracts over N: multiples of 64
+        r = int(rng.integers(1, 65))
+        if fmt == "int4" and K % 128:
+            K += 64
+        m, w_ref = make_dense_module(fmt, N, K, r, 2 * r, seed=3000 + case, device=hip_device, bias=bool(case % 2))
+        x = gen((M, K), 1.0, 4000 + case, torch.bfloat16)
+        dy = gen((M, N), 1.0, 5000 + case, torch.bfloat16)
+        y, dx, dA, dB = _run(m, x.to(hip_device), dy.to(hip_device))
+        ex = R.linear_fwd_bwd_exact(x, w_ref, m.lora_A.detach().cpu(), m.lora_B.detach().cpu(), m.scaling, dy,
+                                    bias=None if m.bias is None else m.bias.detach().cpu())
+        for name, got, ref in (("y", y, ex["y"]), ("dx", dx, ex["dx"]), ("dA", dA, ex["dA"]), ("dB", dB, ex["dB"])):
+            err = R.max_rel_err(got.cpu(), ref)
+            assert err <= TOL, (case, fmt, M, K, N, r, name, err)
+
+
+def test_training_shape_rule_is_reported_at_the_forward(hip_device):
+    """out_features = 48 is fine for a forward-only call; with gradients enabled the call says at once that the
+    backward product needs out_features % 64 == 0."""
+    m, w_ref = make_dense_module("block_fp8", 48, 128, 8, 16, seed=9, device=hip_device)
+    x = gen((5, 128), 1.0, 61, torch.bfloat16).to(hip_device)
+    with torch.no_grad():
+        y = m(x)
+    ex = R.linear_fwd_bwd_exact(x.cpu(), w_ref, m.lora_A.detach().cpu(), m.lora_B.detach().cpu(), m.scaling)
+    assert R.max_rel_err(y.cpu(), ex["y"]) <= TOL
+    with pytest.raises(ValueError, match="out_features % 64"):
+        m(x.requires_grad_(True))

@@ -176,3 +176,33 @@ def test_skinny_decode_bit_exact(hip_device, fmt, M):
     same = y.view(torch.int16) == want.view(torch.int16)
     both_zero = (y.float() == 0) & (want.float() == 0)
     assert bool((same | both_zero).all())
+
+
+def test_skinny_seeded_shape_sweep(hip_device):
+    """Twenty-four seeded draws of (format, N, K, M, r, bias, factor dtype) within the path's shape rules --
+    N any multiple of 16 (ragged last row block), K any multiple of 128 from 1024 (every split / chunk
+    combination the planner makes), M 1..64, r 1..64 -- against the float64 form."""
+    import numpy as np
+
+    from xorl_amd.functional import qlora_linear
+
+    rng = np.random.default_rng(2024)
+    fmts = ["block_fp8", "int4", "nvfp4", "nf4"]
+    for case in range(24):
+        fmt = fmts[case % 4]
+        N = int(rng.integers(1, 40)) * 16 * int(rng.choice([1, 1, 3, 8]))
+        K = int(rng.integers(8, 41)) * 128
+        M = int(rng.integers(1, 65))
+        r = int(rng.integers(1, 65))
+        bf16_factors = bool(rng.integers(0, 2))
+        m, w_ref = make_dense_module(fmt, N, K, r, 2 * r, seed=1000 + case, device=hip_device, bias=bool(case % 3 == 0))
+        x = gen((M, K), 1.0, 2000 + case, torch.bfloat16)
+        A, B = m.lora_A.detach(), m.lora_B.detach()
+        if bf16_factors:
+            A, B = A.to(torch.bfloat16), B.to(torch.bfloat16)
+        with torch.no_grad():
+            y = qlora_linear(x.to(hip_device), m._quant_weight(), A, B, r, m.scaling, m.bias)
+        ex = R.linear_fwd_bwd_exact(x, w_ref, A.float().cpu(), B.float().cpu(), m.scaling,
+                                    bias=None if m.bias is None else m.bias.detach().cpu())
+        err = R.max_rel_err(y.cpu(), ex["y"])
+        assert y.shape == (M, N) and err <= TOL, (case, fmt, N, K, M, r, bf16_factors, err)

@@ -236,6 +236,10 @@ def qlora_linear(x: Tensor, qw: QuantWeight, lora_A: Optional[Tensor], lora_B: O
         return _linear_fwd_impl(x.detach(), qw.packed, qw.scales, qw.global_scale, A, B,
                                 None if bias is None else bias.detach(), qw.fmt, qw.scale_dtype, qw.group,
                                 qw.rows, qw.cols, r, float(scaling), False, qw.c())[0]
+    if qw.rows % 64 != 0:
+        # the backward pass contracts over the output features; say so now rather than in the middle of backward()
+        raise _C.XqError(f"qlora_linear: training needs out_features % 64 == 0 (the input-gradient product contracts "
+                         f"over them), got {qw.rows}; forward-only calls need out_features % 16 == 0")
     return QLoRALinearFunction.apply(x, lora_A, lora_B, bias, qw, r, scaling, training)
 
 
