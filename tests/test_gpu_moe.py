@@ -324,3 +324,47 @@ def test_empty_batches(hip_device):
     assert yd.shape == (0, 128)
     yd.sum().backward()
     assert torch.count_nonzero(d.lora_A.grad) == 0 and torch.count_nonzero(d.lora_B.grad) == 0
+
+
+def test_moe_seeded_shape_sweep(hip_device):
+    """Nine seeded draws of (format, E, T, H, I, r, top-k, shared / per-expert factors): forward and every
+    gradient against the float64 per-expert program."""
+    rng = np.random.default_rng(11)
+    fmts = ["block_fp8", "nvfp4", "nf4"]
+    for case in range(9):
+        fmt = fmts[case % 3]
+        E = int(rng.integers(2, 21))
+        T = int(rng.integers(1, 500))
+        H = int(rng.integers(1, 5)) * 128 if fmt == "block_fp8" else int(rng.integers(1, 7)) * 64
+        I = int(rng.integers(1, 5)) * 128 if fmt == "block_fp8" else int(rng.integers(1, 7)) * 64
+        r = int(rng.integers(1, 65))
+        topk = int(rng.integers(1, min(E, 8) + 1))
+        hybrid = bool(rng.integers(0, 2))
+        m, banks = _make_experts(fmt, E, H, I, r, hybrid, seed=200 + case, device=hip_device)
+        rw, sel = _zipf_routing(T, E, topk, seed=300 + case, empty=1 if E > topk else 0)
+        rw = rw.to(torch.bfloat16)
+        x = gen((T, H), 1.0, 400 + case, torch.bfloat16)
+        dy = gen((T, H), 1.0, 500 + case, torch.bfloat16)
+        xd = x.to(hip_device).requires_grad_(True)
+        rwd = rw.to(hip_device).requires_grad_(True)
+        y = m(xd, rwd, sel.to(hip_device))
+        y.backward(dy.to(hip_device))
+        lora = {k: (getattr(m, f"{k}_proj_lora_A").detach().cpu(), getattr(m, f"{k}_proj_lora_B").detach().cpu())
+                for k in ("gate", "up", "down")}
+        ex = R.moe_fwd_bwd(x, rw, sel, banks["gate"], banks["up"], banks["down"], lora, m.scaling, dy)
+        tag = (case, fmt, E, T, H, I, r, topk, hybrid)
+        assert R.max_rel_err(y.cpu(), ex["y"]) <= TOL, tag
+        assert R.max_rel_err(xd.grad.cpu(), ex["dx"]) <= TOL, tag
+        assert R.max_rel_err(rwd.grad.cpu(), ex["d_routing"]) <= 2e-2, tag
+        # factor gradients pass through bf16 intermediates in the reference too (ops/moe/lora.py:557-564): where
+        # the float64 distance exceeds the tolerance, it must not exceed what the reference's own rounding points
+        # (the oracle's bf16 mode) leave
+        rec = None
+        for k in ("gate", "up", "down"):
+            for f in ("A", "B"):
+                err = R.max_rel_err(getattr(m, f"{k}_proj_lora_{f}").grad.cpu(), ex[f"d{f}_{k}"])
+                if err > TOL:
+                    if rec is None:
+                        rec = R.moe_fwd_bwd(x, rw, sel, banks["gate"], banks["up"], banks["down"], lora, m.scaling, dy,
+                                            dtype=torch.bfloat16)
+                    assert err <= 1.5 * R.max_rel_err(rec[f"d{f}_{k}"].float(), ex[f"d{f}_{k}"]), tag + (k, f, err)
