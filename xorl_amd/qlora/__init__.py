@@ -24,9 +24,22 @@ from .moe_experts import BlockFP8QLoRAMoeExperts, NF4QLoRAMoeExperts, NvFP4QLoRA
 
 __all__ += ["QLoRAMoeExperts", "BlockFP8QLoRAMoeExperts", "NvFP4QLoRAMoeExperts", "NF4QLoRAMoeExperts"]
 
-from .utils import maybe_load_prequantized_qlora, maybe_requant_qlora  # noqa: E402
+from .utils import (  # noqa: E402
+    detect_prequantized_block_fp8,
+    detect_prequantized_nvfp4,
+    inject_qlora_into_model,
+    maybe_load_and_quantize_moe_qlora,
+    maybe_load_prequantized_qlora,
+    maybe_merge_lora,
+    maybe_quantize_qlora,
+    maybe_requant_qlora,
+    reset_lora_optimizer_states,
+    save_qlora_checkpoint,
+)
 
-__all__ += ["maybe_load_prequantized_qlora", "maybe_requant_qlora"]
+__all__ += ["inject_qlora_into_model", "maybe_load_prequantized_qlora", "maybe_load_and_quantize_moe_qlora",
+            "maybe_quantize_qlora", "maybe_requant_qlora", "save_qlora_checkpoint", "detect_prequantized_nvfp4",
+            "detect_prequantized_block_fp8", "maybe_merge_lora", "reset_lora_optimizer_states"]
 
 from .inline_buffers import (  # noqa: E402
     BlockFP8QLoRAExpertBuffer,

@@ -96,6 +96,45 @@ class QLoRAMoeExperts(LoraModule, nn.Module):
         self._skip_fsdp = True
         self._qlora_expected_skip_keys = {"gate_proj", "up_proj", "down_proj"}
 
+    # ------------------------------------------------------------------ factory
+    @classmethod
+    def from_module(cls, module: nn.Module, r: int = 16, lora_alpha: int = 16, quant_format: str = "nvfp4",
+                    quant_group_size: int = 16, num_local_experts: Optional[int] = None, expert_offset: int = 0,
+                    hybrid_shared: bool = True, target_modules: Optional[list] = None, use_rslora: bool = False,
+                    **kwargs) -> "QLoRAMoeExperts":
+        """An empty packed-bank module shaped like `module`, an experts container whose weights are
+        [num_experts, in, out] parameters (`gate_proj` / `up_proj` / `down_proj`, or a fused `gate_up_proj`);
+        the banks are filled later by load_weights() or load_and_quantize_weights()
+        (qlora/modules/moe_experts.py:354-427)."""
+        gate = getattr(module, "gate_proj", None)
+        if isinstance(gate, Tensor) and gate.dim() == 3:
+            total, hidden, inter = gate.shape
+        else:
+            fused = getattr(module, "gate_up_proj", None)
+            if not (isinstance(fused, Tensor) and fused.dim() == 3):
+                raise TypeError(f"{type(module).__name__} holds no [num_experts, in, out] expert weights")
+            gate = fused
+            total, hidden, inter = fused.shape[0], fused.shape[1], fused.shape[2] // 2
+        for attr, want in (("gated", True), ("swiglu_limit", 0.0), ("gate_up_bias", None), ("down_bias", None)):
+            have = getattr(module, attr, want)
+            if have is not None and have != want and not (attr == "swiglu_limit" and not have):
+                raise ValueError(f"expert adapters need gated SiLU experts without clamping or biases; "
+                                 f"{type(module).__name__}.{attr} = {have!r}")
+        required = {"nvfp4": 16, "block_fp8": 128, "nf4": 64}
+        if quant_format not in required:
+            raise ValueError(f"Expert QLoRA formats: {sorted(required)}; got {quant_format!r}")
+        if quant_group_size != required[quant_format]:
+            raise ValueError(f"Expert {quant_format} QLoRA requires quant_group_size={required[quant_format]}; "
+                             f"got {quant_group_size}")
+        if cls is QLoRAMoeExperts:
+            cls = {"block_fp8": BlockFP8QLoRAMoeExperts, "nf4": NF4QLoRAMoeExperts, "nvfp4": NvFP4QLoRAMoeExperts}[quant_format]
+        return cls(num_local_experts=total if num_local_experts is None else num_local_experts, num_experts=total,
+                   intermediate_size=getattr(module, "intermediate_size", inter),
+                   hidden_size=getattr(module, "hidden_dim", hidden), r=r, lora_alpha=lora_alpha,
+                   act_fn=getattr(module, "act_fn", None), hidden_act=getattr(module, "hidden_act", "silu"),
+                   expert_offset=expert_offset, device=gate.device, hybrid_shared=hybrid_shared,
+                   target_modules=target_modules, use_rslora=use_rslora)
+
     # ------------------------------------------------------------------ LoRA params
     def _create_lora_params(self, name, A_experts, B_experts, r, in_features, out_features, device=None):
         A = torch.empty(A_experts, in_features, r, dtype=torch.float32, device=device)
