@@ -38,9 +38,10 @@ BF16_MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense bf16, published
 # 256 MiB -> 256 MiB copy; the files under profiles/ hold the figures and the commands).  A config that
 # has no counter run reports null.  --traffic-bytes overrides.
 MEASURED_TRAFFIC_BYTES = {
-    0: 45.6 * 2 ** 20,     # gemm_256_kernel<int4, T=128>: mean of the forward and dgrad launches
+    0: 109.6 * 2 ** 20,    # gemm_256_kernel<int4, T=128> in 4 K splits + splitk_reduce_kernel: mean of the forward and dgrad
+                           # launches (64 MiB of it are the fp32 partial sums written and read back)
     1: 905.4 * 2 ** 20,    # gemm_256_kernel<fp8>: mean of the forward and dgrad launches
-    2: 153.2 * 2 ** 20,    # gemm_256_kernel<nvfp4>, 256x256 and 128x128 tiles: mean over the 12 launches of a step
+    2: 160.4 * 2 ** 20,    # gemm_256_kernel<nvfp4>, 256x256 and 128x128 tiles: mean over the 12 launches of a step
     3: 1032.2 * 2 ** 20,   # gemm_256_kernel<fp8, grouped>: mean over the 6 launches of a step
     4: 41.0 * 2 ** 20,     # skinny_split_kernel + skinny_epilogue_kernel: mean per forward over the 32 cases (includes
                            # the fp32 partial tiles written and read back: 23.3 MiB of it are algorithmic)
@@ -161,7 +162,7 @@ def other_config(cfg: int, dev):
             m(x).backward(dy)
         return (step, lin_flops(512, 4096, 4096, 16), False,
                 "configs[0]: int4 (group 128, bf16 absmax/7 scales) QLoRA linear 4096->4096, M=512, r=16, fwd+bwd",
-                "gemm_tile_kernel<int4> (fused dequant-GEMM, forward and dgrad launches)")
+                "gemm_256_kernel<int4> with 128x128 tiles in 4 K splits + splitk_reduce_kernel (fused dequant-GEMM, forward and dgrad launches)")
     if cfg == 2:
         Mtok, Hd = 4096, 5120
         shapes = {"q": (8192, Hd), "k": (1024, Hd), "v": (1024, Hd), "o": (Hd, 8192)}

@@ -115,7 +115,11 @@ int xq_decode(const xq_weight* w, void* out, int out_dtype, void* stream);
  * Replaces QLoRALinear.forward (qlora/modules/linear.py:369-385) and its
  * autograd backward.  The weight is FLAT [N, K]. */
 
-/* Bytes of scratch the dense entry points need for (M, N, K, r). */
+/* Bytes of scratch the dense entry points need for (M, N, K, r): the prepared
+ * LoRA panels and partial sums of the factor gradients (r > 0) and, for row
+ * counts that leave most of the chip without a tile, the fp32 partial sums of
+ * the split-K product.  With r == 0 the workspace is optional: a call without
+ * it (or with fewer bytes) runs the product unsplit. */
 int64_t xq_linear_workspace_bytes(int64_t M, int64_t N, int64_t K, int r);
 
 /* y[M,N] = x[M,K] . deq(W)^T + bias + s * (x . A^T) . B^T      (bf16 out)

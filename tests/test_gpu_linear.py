@@ -70,6 +70,58 @@ def test_gemm_decode_bit_exact(hip_device, tile_policy, fmt):
     assert torch.equal(x.grad.view(torch.int16), wd.view(torch.int16)) or _equal_mod_zero_sign(x.grad, wd)
 
 
+@pytest.mark.parametrize("fmt", ["block_fp8", "int4", "nvfp4", "nf4"])
+def test_split_k_decode_bit_exact(hip_device, fmt):
+    """N = K = M = 1024 under the default policy: 64 tiles of 128 x 128 leave most of the chip idle, so the 16
+    K-steps are divided over two blocks per tile whose fp32 sums a second kernel adds.  With X = I every sum has
+    one non-zero term, so forward and dgrad must still return the oracle's decode bit for bit."""
+    from xorl_amd import _C
+
+    N = K = 1024
+    assert _C.lib().xq_linear_workspace_bytes(K, N, K, 0) >= 2 * K * N * 4       # the plan does split
+    m, w_ref = make_dense_module(fmt, N, K, 16, 32, seed=78, device=hip_device)
+    with torch.no_grad():
+        m.lora_B.zero_()
+    eye = torch.eye(K, dtype=torch.bfloat16, device=hip_device)
+    x = eye.clone().requires_grad_(True)
+    y = m(x)
+    y.backward(eye)
+    wd = w_ref.to(hip_device)
+    assert _equal_mod_zero_sign(y.detach(), wd.t()) and _equal_mod_zero_sign(x.grad, wd)
+
+
+@pytest.mark.parametrize("fmt,M,N,K,r,bias", [
+    ("block_fp8", 512, 1024, 4096, 16, True),     # 32 tiles -> 8 splits forward, 2 in the dgrad (contraction 1024)
+    ("int4", 192, 320, 2048, 8, False),           # ragged tiles in both directions, 4 splits
+    ("nvfp4", 320, 512, 1536, 32, False),         # 24 K-steps -> 3 splits of 8
+    ("nf4", 130, 256, 1088, 16, True),            # 17 K-steps -> 2 splits of 9 and 8
+])
+def test_split_k_fwd_bwd_vs_oracle(hip_device, fmt, M, N, K, r, bias):
+    from xorl_amd import _C
+
+    assert _C.lib().xq_linear_workspace_bytes(M, N, K, 0) >= 2 * M * N * 4
+    m, w_ref = make_dense_module(fmt, N, K, r, 2 * r, seed=M + K, device=hip_device, bias=bias)
+    x = gen((M, K), 1.0, 31, torch.bfloat16)
+    dy = gen((M, N), 1.0, 32, torch.bfloat16)
+    y, dx, dA, dB = _run(m, x.to(hip_device), dy.to(hip_device))
+    ex = R.linear_fwd_bwd_exact(x, w_ref, m.lora_A.detach().cpu(), m.lora_B.detach().cpu(), m.scaling, dy,
+                                bias=m.bias.detach().cpu() if bias else None)
+    for name, got, ref in (("y", y, ex["y"]), ("dx", dx, ex["dx"]), ("dA", dA, ex["dA"]), ("dB", dB, ex["dB"])):
+        err = R.max_rel_err(got.cpu(), ref)
+        assert err <= TOL, f"{fmt} {name}: {err}"
+    # the same call again gives the same bits (fixed summation order, no atomics)
+    y2, dx2, _, _ = _run(m, x.to(hip_device), dy.to(hip_device))
+    assert torch.equal(y, y2) and torch.equal(dx, dx2)
+    # and the unsplit kernel agrees to rounding
+    _C.check(_C.lib().xq_set_tile_policy(1))
+    try:
+        with torch.no_grad():
+            y1 = m(x.to(hip_device))
+    finally:
+        _C.check(_C.lib().xq_set_tile_policy(0))
+    assert R.max_rel_err(y.cpu(), y1.cpu().double()) <= 4e-3
+
+
 def _equal_mod_zero_sign(a, b):
     """Bitwise equality except that a sum may return +0 where the decoded weight is -0."""
     a16, b16 = a.contiguous().view(torch.int16), b.contiguous().view(torch.int16)

@@ -51,12 +51,38 @@ static int launch_256(const G256Args& f, bool cc, bool grouped, int T, dim3 grid
     return grouped ? launch_256_t<FMT, false, true>(f, T, grid, s, who) : launch_256_t<FMT, false, false>(f, T, grid, s, who);
 }
 
+// Tile size of a dense launch under the default policy: large tiles from the point where they fill more than
+// half the chip (up to 512 small tiles are resident at once, two per CU, and finish sooner than one round of up
+// to 128 large ones).
+static inline int dense_tile_size(int64_t n_rows, int64_t Nout) {
+    return xq_cdiv(n_rows, 256) * xq_cdiv(Nout, 256) > 128 ? 256 : 128;
+}
+
+// K splits of a dense launch of `blocks` small tiles over nk K-steps (1 = none): used when the tiles fill at most
+// half of the block slots of the chip; every split keeps at least 8 K-steps.
+static inline int ksplit_for(int64_t blocks, int T, int64_t nk) {
+    const int64_t slots = 512;                       // small tiles only: two blocks per CU
+    if (T != 128 || blocks <= 0 || blocks * 2 > slots) return 1;
+    int64_t s = slots / blocks;
+    if (s > nk / 8) s = nk / 8;
+    if (s > 8) s = 8;
+    return s < 2 ? 1 : (int)s;
+}
+
+// fp32 partial-sum bytes the split-K form of a dense [n_rows, Nout] product over Kc wants, under any tile policy
+int64_t tile_gemm_partial_bytes(int64_t n_rows, int64_t Nout, int64_t Kc) {
+    if (n_rows <= 0 || Kc % BK) return 0;
+    const int s = ksplit_for(xq_cdiv(n_rows, 128) * xq_cdiv(Nout, 128), 128, Kc / BK);
+    return s > 1 ? (int64_t)s * n_rows * Nout * 4 : 0;
+}
+
 // C[rows, Nout] = A . op(deq(W)) (+ su . Lr^T) (+ bias); see xq_gemm_tile.h.  force_T = 256 / 128 fixes the tile
-// size of the pipelined kernel, 0 leaves it to the selection policy.
+// size of the pipelined kernel, 0 leaves it to the selection policy.  `partial` (may be NULL) is scratch for
+// split-K sums; a launch that would split but finds less than tile_gemm_partial_bytes() there runs unsplit.
 static int launch_tile_gemm_t(const xq_weight* w, bool contract_cols, const bf16_t* A, int64_t lda, int64_t n_rows,
                               const int32_t* offsets, const int32_t* tile_offsets, const bf16_t* su, const bf16_t* lora_right,
                               int r_pad, const bf16_t* bias, bf16_t* C, int64_t ldc, hipStream_t stream, const char* who,
-                              int force_T) {
+                              int force_T, float* partial, int64_t partial_bytes) {
     TileArgs g;
     g.A = A; g.lda = lda; g.C = C; g.ldc = ldc;
     g.packed = (const uint8_t*)w->packed;
@@ -94,7 +120,7 @@ static int launch_tile_gemm_t(const xq_weight* w, bool contract_cols, const bf16
                                             xq_aligned(w->scales, 16) && g.scale_stride % 16 == 0
                                       : w->layout == XQ_LAYOUT_FLAT));
         const bool big = grouped ? (n_rows >= 128ll * w->num_experts && n_rows >= 8192)
-                                 : (xq_cdiv(n_rows, 256) * xq_cdiv(g.Nout, 256) >= 96);
+                                 : dense_tile_size(n_rows, g.Nout) == 256;
         const int T = force_T ? force_T : g_tile_policy == 2 ? 256 : g_tile_policy == 3 ? 128 : (big ? 256 : 128);
         // A dense launch of 256x256 tiles whose last round would fill only part of the chip: the leading tile rows
         // that make whole rounds keep the large tiles, the remaining rows run as a second launch of 128x128 tiles
@@ -111,11 +137,11 @@ static int launch_tile_gemm_t(const xq_weight* w, bool contract_cols, const bf16
                 if ((double)xq_cdiv(keep * tc, cus) + tail < (double)(full + 1) - 0.2) {
                     const int64_t head = keep * 256;
                     const int rc = launch_tile_gemm_t(w, contract_cols, A, lda, head, nullptr, nullptr, su, lora_right, r_pad,
-                                                      bias, C, ldc, stream, who, 256);
+                                                      bias, C, ldc, stream, who, 256, nullptr, 0);
                     if (rc) return rc;
                     return launch_tile_gemm_t(w, contract_cols, A + head * lda, lda, tail_rows, nullptr, nullptr,
                                               su ? su + head * r_pad : nullptr, lora_right, r_pad, bias, C + head * ldc, ldc,
-                                              stream, who, 128);
+                                              stream, who, 128, nullptr, 0);
                 }
             }
         }
@@ -134,16 +160,24 @@ static int launch_tile_gemm_t(const xq_weight* w, bool contract_cols, const bf16
             f.su = g.r_pad ? su : nullptr; f.lora_right = g.r_pad ? lora_right : nullptr; f.r_pad = g.r_pad;
             f.bias = bias;
             f.tiles_m = (int32_t)tiles_m; f.tiles_n = (int32_t)tiles_n;
-            dim3 grid((unsigned)(tiles_m * tiles_n));
+            int ksplit = (grouped || force_T) ? 1 : ksplit_for(tiles_m * tiles_n, T, g.Kc / BK);
+            if (ksplit > 1 && (!partial || !xq_aligned(partial, 16) || partial_bytes < (int64_t)ksplit * n_rows * g.Nout * 4)) ksplit = 1;
+            f.ksplit = ksplit; f.partial = ksplit > 1 ? partial : nullptr;
+            dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)ksplit);
             const bool timed = xq_profile_mark_begin(stream, 2.0 * (double)n_rows * g.Nout * ((double)g.Kc + g.r_pad));
             int rc;
             if (w->format == XQ_FMT_FP8) rc = launch_256<XQ_FMT_FP8>(f, contract_cols, grouped, T, grid, stream, who);
             else if (w->format == XQ_FMT_INT4) rc = launch_256<XQ_FMT_INT4>(f, contract_cols, grouped, T, grid, stream, who);
             else if (w->format == XQ_FMT_NF4) rc = launch_256<XQ_FMT_NF4>(f, contract_cols, grouped, T, grid, stream, who);
             else rc = launch_256<XQ_FMT_NVFP4>(f, contract_cols, grouped, T, grid, stream, who);
-            if (timed) xq_profile_mark_end(stream);
             if (rc) return rc;
             XQ_CHECK_LAUNCH(who);
+            if (ksplit > 1) {
+                const int64_t quads = n_rows * (g.Nout >> 2);
+                splitk_reduce_kernel<<<(unsigned)xq_cdiv(quads, 256), 256, 0, stream>>>(partial, ksplit, n_rows, g.Nout, C, ldc);
+                XQ_CHECK_LAUNCH(who);
+            }
+            if (timed) xq_profile_mark_end(stream);
             return XQ_OK;
         }
     }
@@ -164,9 +198,10 @@ static int launch_tile_gemm_t(const xq_weight* w, bool contract_cols, const bf16
 
 int launch_tile_gemm(const xq_weight* w, bool contract_cols, const bf16_t* A, int64_t lda, int64_t n_rows,
                      const int32_t* offsets, const int32_t* tile_offsets, const bf16_t* su, const bf16_t* lora_right,
-                     int r_pad, const bf16_t* bias, bf16_t* C, int64_t ldc, hipStream_t stream, const char* who) {
+                     int r_pad, const bf16_t* bias, bf16_t* C, int64_t ldc, hipStream_t stream, const char* who,
+                     float* partial, int64_t partial_bytes) {
     return launch_tile_gemm_t(w, contract_cols, A, lda, n_rows, offsets, tile_offsets, su, lora_right, r_pad, bias, C, ldc,
-                              stream, who, 0);
+                              stream, who, 0, partial, partial_bytes);
 }
 
 static inline int64_t align256(int64_t b) { return (b + 255) & ~(int64_t)255; }
@@ -195,13 +230,19 @@ extern "C" int xq_set_tile_policy(int policy) {
 extern "C" int64_t xq_linear_workspace_bytes(int64_t M, int64_t N, int64_t K, int r) {
     int rp = r_pad_of(r);
     int64_t skinny = M <= 64 ? skinny_workspace_bytes(M, N, K, rp) : 0;
-    if (rp == 0) return skinny > 256 ? skinny : 256;
-    int64_t fwd = align256(rp * K * 2) + align256(N * rp * 2) + align256(M * rp * 2);
-    int64_t tnp = tn_partial_bytes(M, N, rp);
-    int64_t tnk = tn_partial_bytes(M, K, rp);
-    int64_t bwd = align256(rp * N * 2) + align256(K * rp * 2) + align256(rp * K * 2) + 2 * align256(M * rp * 2) +
-                  align256(tnp > tnk ? tnp : tnk);
-    int64_t need = (fwd > bwd ? fwd : bwd) + 256;
+    // split-K partial sums of the forward (output N, contraction K) and of the dgrad (output K, contraction N)
+    const int64_t pf = align256(tile_gemm_partial_bytes(M, N, K));
+    const int64_t pb = align256(tile_gemm_partial_bytes(M, K, N));
+    int64_t need = (pf > pb ? pf : pb) + 256;
+    if (rp) {
+        int64_t fwd = align256(rp * K * 2) + align256(N * rp * 2) + align256(M * rp * 2) + pf;
+        int64_t tnp = tn_partial_bytes(M, N, rp);
+        int64_t tnk = tn_partial_bytes(M, K, rp);
+        int64_t tn = align256(tnp > tnk ? tnp : tnk);     // the weight-gradient partials reuse the dgrad's region
+        int64_t bwd = align256(rp * N * 2) + align256(K * rp * 2) + align256(rp * K * 2) + 2 * align256(M * rp * 2) +
+                      (tn > pb ? tn : pb);
+        need = (fwd > bwd ? fwd : bwd) + 256;
+    }
     return need > skinny ? need : skinny;
 }
 
@@ -232,10 +273,10 @@ extern "C" int xq_linear_fwd(const xq_weight* w, const void* x, int64_t ldx, int
         return launch_skinny(w, (const bf16_t*)x, ldx, M, lora_A, lora_B, lora_dtype, r, scaling,
                              (const bf16_t*)bias_bf16, (bf16_t*)y, ldy, workspace, workspace_bytes, stream);
     bf16_t *A_bf = nullptr, *Bl = nullptr, *su = nullptr;
+    Carver cv{(workspace && xq_aligned(workspace, 256)) ? (uint8_t*)workspace : nullptr, 0, workspace_bytes};
     if (rp) {
         XQ_REQUIRE(workspace && xq_aligned(workspace, 256) && workspace_bytes >= xq_linear_workspace_bytes(M, N, K, r),
                    "xq_linear_fwd: workspace missing, misaligned or smaller than xq_linear_workspace_bytes()");
-        Carver cv{(uint8_t*)workspace, 0, workspace_bytes};
         A_bf = (bf16_t*)cv.take(rp * K * 2);
         Bl = (bf16_t*)cv.take(N * rp * 2);
         su = su_out ? (bf16_t*)su_out : (bf16_t*)cv.take(M * rp * 2);
@@ -243,8 +284,10 @@ extern "C" int xq_linear_fwd(const xq_weight* w, const void* x, int64_t ldx, int
         if ((rc = launch_factor_prep(lora_B, lora_dtype, N, r, false, Bl, N, rp, 1, stream))) return rc;
         if ((rc = launch_small_nt((const bf16_t*)x, ldx, M, K, A_bf, rp, scaling, su, nullptr, nullptr, 1, true, stream))) return rc;
     }
+    // what is left of the workspace holds split-K partial sums (small row counts); without it the launch is unsplit
+    float* partial = (float*)cv.take(0);
     return launch_tile_gemm(w, true, (const bf16_t*)x, ldx, M, nullptr, nullptr, su, Bl, rp, (const bf16_t*)bias_bf16,
-                            (bf16_t*)y, ldy, stream, "xq_linear_fwd");
+                            (bf16_t*)y, ldy, stream, "xq_linear_fwd", partial, partial ? workspace_bytes - cv.used : 0);
 }
 
 extern "C" int xq_linear_bwd(const xq_weight* w, const void* x, int64_t ldx, const void* dy, int64_t lddy, int64_t M,
@@ -270,16 +313,15 @@ extern "C" int xq_linear_bwd(const xq_weight* w, const void* x, int64_t ldx, con
     bf16_t *Bt = nullptr, *At = nullptr, *v = nullptr;
     const bf16_t* su = (const bf16_t*)su_in;
     float* partial = nullptr;
+    Carver cv{(workspace && xq_aligned(workspace, 256)) ? (uint8_t*)workspace : nullptr, 0, workspace_bytes};
     if (rp) {
         XQ_REQUIRE(workspace && xq_aligned(workspace, 256) && workspace_bytes >= xq_linear_workspace_bytes(M, N, K, r),
                    "xq_linear_bwd: workspace missing, misaligned or smaller than xq_linear_workspace_bytes()");
-        Carver cv{(uint8_t*)workspace, 0, workspace_bytes};
         Bt = (bf16_t*)cv.take(rp * N * 2);
         At = (bf16_t*)cv.take(K * rp * 2);
         bf16_t* A_bf = (bf16_t*)cv.take(rp * K * 2);
         v = (bf16_t*)cv.take(M * rp * 2);
         bf16_t* su_ws = (bf16_t*)cv.take(M * rp * 2);
-        partial = (float*)cv.take(0);
         // v = bf16(s * dy . B)   [M, rp]
         if ((rc = launch_factor_prep(lora_B, lora_dtype, N, r, true, Bt, rp, N, 1, stream))) return rc;
         if ((rc = launch_small_nt((const bf16_t*)dy, lddy, M, N, Bt, rp, scaling, v, nullptr, nullptr, 1, true, stream))) return rc;
@@ -290,10 +332,13 @@ extern "C" int xq_linear_bwd(const xq_weight* w, const void* x, int64_t ldx, con
             su = su_ws;
         }
     }
+    // one region after the carved buffers: split-K partial sums of the dgrad first, then (stream order) the
+    // partial sums of the factor gradients
+    partial = (float*)cv.take(0);
     if (dx) {
         XQ_REQUIRE(lddx % 8 == 0 && xq_aligned(dx, 16), "xq_linear_bwd: dx rows must be 16-byte aligned");
         if ((rc = launch_tile_gemm(w, false, (const bf16_t*)dy, lddy, M, nullptr, nullptr, v, At, rp, nullptr, (bf16_t*)dx,
-                                   lddx, stream, "xq_linear_bwd(dx)")))
+                                   lddx, stream, "xq_linear_bwd(dx)", partial, partial ? workspace_bytes - cv.used : 0)))
             return rc;
     }
     // dB[N, r] = dy^T . su ; dA[r, K] = (x^T . v)^T
@@ -313,7 +358,7 @@ extern "C" int xq_grouped_gemm(const xq_weight* w, int transpose_w, const void* 
     // bank is [E, K_in, N_out]: forward contracts over W rows, dgrad over W cols
     return launch_tile_gemm(w, transpose_w != 0, (const bf16_t*)a, lda, n_rows, offsets, tile_offsets, (const bf16_t*)su,
                             (const bf16_t*)lora_right, r_pad, nullptr, (bf16_t*)y, ldy, (hipStream_t)stream,
-                            "xq_grouped_gemm");
+                            "xq_grouped_gemm", nullptr, 0);
 }
 
 extern "C" int xq_factor_prep(const void* in, int in_dtype, int64_t rows_in, int64_t cols_in, int transpose,

@@ -35,6 +35,9 @@
 namespace xq {
 
 constexpr int F8_BK = 64;
+#ifndef XQ_SMALL_TILE_DEPTH
+#define XQ_SMALL_TILE_DEPTH 2
+#endif
 // geometry of a T x T tile (T = 256: 8 waves, 2 x 4; T = 128: 4 waves, 2 x 2; wave tile (T/2) x 64)
 template <int T>
 struct Geo {
@@ -46,6 +49,7 @@ struct Geo {
     static constexpr int B_STAGE_NT = BN * F8_BK;
     static constexpr int B_STAGE_NN = F8_BK * NN_PITCH;
     static constexpr int RPR = BN / 16;                    // 16-code runs per [kc] row of the tile
+    static constexpr int PD = T == 256 ? 1 : XQ_SMALL_TILE_DEPTH;   // tiles in flight from global memory
     static constexpr size_t lds_bytes(bool cc) { return (size_t)(2 * A_STAGE + 2 * (cc ? B_STAGE_NT : B_STAGE_NN)) * 2; }
 };
 
@@ -77,6 +81,10 @@ struct G256Args {
     int32_t r_pad;
     const bf16_t* bias;
     int32_t tiles_m, tiles_n;  // grouped: tiles_m is an upper bound
+    // dense launches of the small tile only: ksplit > 1 divides the K-steps over gridDim.y blocks per tile; split s then writes its fp32
+    // sums to partial + s * M * Nout (row pitch Nout) instead of C, and split 0 carries the low-rank term and bias
+    int32_t ksplit;
+    float* partial;
 };
 
 // ---------------------------------------------------------------- weight-tile loaders
@@ -428,6 +436,15 @@ __global__ void __launch_bounds__(2 * T, 2) gemm_256_kernel(G256Args g) {
         row_end = g.M;
     }
     const int n0 = pid_n * F8_BN;
+    // K-steps of this block: all of them, or the split's share (every split has at least one)
+    constexpr bool CAN_SPLIT = !GROUPED && T == 128;      // only the small tile is used on part-filled chips
+    int kt0 = 0, nk = g.Kc / F8_BK;
+    const int split = CAN_SPLIT ? (int)blockIdx.y : 0;
+    if (CAN_SPLIT && g.ksplit > 1) {
+        const int per = (nk + g.ksplit - 1) / g.ksplit;
+        kt0 = split * per;
+        nk = min(per, nk - kt0);
+    }
 
     // ---- per-thread global addresses (fixed across K-steps except for the k offset)
     const bf16_t* a_src[4];
@@ -437,26 +454,34 @@ __global__ void __launch_bounds__(2 * T, 2) gemm_256_kernel(G256Args g) {
         const int u = tid + p * NT;
         int64_t r = row0 + (u >> 3);
         r = r < row_end ? r : row_end - 1;
-        a_src[p] = g.A + r * g.lda + (u & 7) * 8;
+        a_src[p] = g.A + r * g.lda + (u & 7) * 8 + kt0 * F8_BK;
         a_dst[p] = swz(u >> 3, u & 7);
     }
-    typename W256Sel<FMT, CC, GROUPED, T>::type wl;
-    wl.init(g, g.W + (int64_t)e * g.packed_stride, g.scales + (int64_t)e * g.scale_stride,
-            FMT == XQ_FMT_NVFP4 ? g.global_scale[e] : 1.0f, n0, tid);
+    // PD register sets hold the tiles in flight from global memory: tile j lives in set j % PD.  The large tile has
+    // one (two waves per SIMD and an iteration longer than the memory latency cover it); the small tile, whose
+    // iteration is a fraction of the latency, keeps PD tiles in flight.
+    constexpr int PD = (GROUPED && FMT != XQ_FMT_FP8) ? 1 : Geo<T>::PD;   // the GKN 4-bit loader has no registers to spare
+    using WL = typename W256Sel<FMT, CC, GROUPED, T>::type;
+    WL wls[PD];
+#pragma unroll
+    for (int d = 0; d < PD; ++d)
+        wls[d].init(g, g.W + (int64_t)e * g.packed_stride, g.scales + (int64_t)e * g.scale_stride,
+                    FMT == XQ_FMT_NVFP4 ? g.global_scale[e] : 1.0f, n0, tid);
     if constexpr (FMT == XQ_FMT_NF4) {
         __shared__ float s_nf4[16];
         if (tid < 16) s_nf4[tid] = kNf4Level[tid];
         __syncthreads();
-        wl.nf4_lds = s_nf4;
+#pragma unroll
+        for (int d = 0; d < PD; ++d) wls[d].nf4_lds = s_nf4;
     }
 
-    u32x4 areg[4];
-    auto load_a = [&](int kt) {
+    u32x4 aregs[PD][4];
+    auto load_a = [&](u32x4* areg, int kt) {
         const int k0 = kt * F8_BK;
 #pragma unroll
         for (int p = 0; p < 4; ++p) areg[p] = *(const u32x4*)(a_src[p] + k0);
     };
-    auto store_a = [&](bf16_t* a) {
+    auto store_a = [&](bf16_t* a, const u32x4* areg) {
 #pragma unroll
         for (int p = 0; p < 4; ++p) *(u32x4*)(a + a_dst[p]) = areg[p];
     };
@@ -495,9 +520,8 @@ __global__ void __launch_bounds__(2 * T, 2) gemm_256_kernel(G256Args g) {
     // the last step, whose MFMAs then cover both the barrier skew and the fetch of the
     // next tile's first fragments.  (Every read of a stage completes before the barrier
     // that precedes the next stores into it.)
-    const int nk = g.Kc / F8_BK;
     bf16x8 af0[TM], bf0[TN], af1[TM], bf1[TN];
-    auto iteration = [&](int kt, bool have_next, bool have_next2) {
+    auto iteration = [&](int kt, bool have_next, bool have_next2, u32x4* areg, WL& wl, int kload) {
         const bf16_t* a = As + (kt & 1) * F8_A_STAGE;
         const bf16_t* b = Bs + (kt & 1) * B_STAGE;
         bf16_t* an = As + ((kt + 1) & 1) * F8_A_STAGE;
@@ -505,8 +529,8 @@ __global__ void __launch_bounds__(2 * T, 2) gemm_256_kernel(G256Args g) {
         // region 1: MFMAs of step 0 over the step-1 fragment reads, the A-tile stores and the next A loads
         mma(af0, bf0);
         load_frags(a, b, 1, false, af1, bf1);
-        if (have_next) store_a(an);
-        if (have_next2) load_a(kt + 2);
+        if (have_next) store_a(an, areg);
+        if (have_next2) load_a(areg, kload);
         // interleave: one LDS read behind each of the first MFMAs, then the stores and global loads
         if (T == 256) {
             for (int q = 0; q < 6; ++q) { __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); }
@@ -520,7 +544,7 @@ __global__ void __launch_bounds__(2 * T, 2) gemm_256_kernel(G256Args g) {
         // region 2: MFMAs of step 1 over the weight decode + stores, the next weight loads, step-2 fragment reads
         mma(af1, bf1);
         if (have_next) { wl.store(bn, 0); wl.store(bn, 1); }
-        if (have_next2) wl.load(kt + 2);
+        if (have_next2) wl.load(kt0 + kload);
         load_frags(a, b, 2, false, af0, bf0);
         __builtin_amdgcn_sched_barrier(0);
         // region 3: MFMAs of step 2 over the step-3 fragment reads
@@ -535,21 +559,41 @@ __global__ void __launch_bounds__(2 * T, 2) gemm_256_kernel(G256Args g) {
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         __builtin_amdgcn_sched_barrier(0);
     };
-    load_a(0);
-    wl.load(0);
-    store_a(As);
-    wl.store(Bs, 0);
-    wl.store(Bs, 1);
-    if (nk > 1) { load_a(1); wl.load(1); }
-    __syncthreads();
-    load_frags(As, Bs, 0, false, af0, bf0);
-    int kt = 0;
-    for (; kt + 2 < nk; ++kt) iteration(kt, true, true);
-    if (kt + 1 < nk) { iteration(kt, true, false); ++kt; }
-    iteration(kt, false, false);
+    load_a(aregs[0], 0);
+    wls[0].load(kt0);
+    store_a(As, aregs[0]);
+    wls[0].store(Bs, 0);
+    wls[0].store(Bs, 1);
+    if constexpr (PD == 1) {
+        if (nk > 1) { load_a(aregs[0], 1); wls[0].load(kt0 + 1); }
+        __syncthreads();
+        load_frags(As, Bs, 0, false, af0, bf0);
+        int kt = 0;
+        for (; kt + 2 < nk; ++kt) iteration(kt, true, true, aregs[0], wls[0], kt + 2);
+        if (kt + 1 < nk) { iteration(kt, true, false, aregs[0], wls[0], 0); ++kt; }
+        iteration(kt, false, false, aregs[0], wls[0], 0);
+    } else {
+        // Tiles 1 .. PD are requested in this order, so that they also arrive in it.  Every iteration stores the
+        // set of tile kt+1 and refills it with tile kt+1+PD; past the end the tile index is clamped (the last tile
+        // is fetched again and stored into the stage nobody reads any more), which keeps every load unconditional.
+        const int last = nk - 1;
+#pragma unroll
+        for (int d = 1; d <= PD; ++d) { load_a(aregs[d % PD], min(d, last)); wls[d % PD].load(kt0 + min(d, last)); }
+        __syncthreads();
+        load_frags(As, Bs, 0, false, af0, bf0);
+        int kt = 0;
+        for (; kt + PD <= nk; kt += PD) {
+#pragma unroll
+            for (int d = 0; d < PD; ++d)
+                iteration(kt + d, true, true, aregs[(d + 1) % PD], wls[(d + 1) % PD], min(kt + d + 1 + PD, last));
+        }
+#pragma unroll
+        for (int d = 0; d < PD - 1; ++d)
+            if (kt + d < nk) iteration(kt + d, true, true, aregs[(d + 1) % PD], wls[(d + 1) % PD], last);
+    }
 
     // ---- low-rank side term: su[rows, rp] x lora_right[n, rp], both [row][k] tiles in stage 0
-    if (g.r_pad > 0) {
+    if (g.r_pad > 0 && split == 0) {
         const int rp = g.r_pad, cpr = rp >> 3;  // 16-byte chunks per row
         const bf16_t* lr = g.lora_right + (int64_t)e * g.Nout * rp;
         for (int idx = tid; idx < F8_BM * cpr; idx += NT) {
@@ -575,6 +619,7 @@ __global__ void __launch_bounds__(2 * T, 2) gemm_256_kernel(G256Args g) {
         const int64_t row = row0 + wm * (T / 2) + i * 32 + fr;
         if (row >= row_end) continue;
         bf16_t* crow = g.C + row * g.ldc;
+        float* prow = (CAN_SPLIT && g.ksplit > 1) ? g.partial + ((int64_t)split * g.M + row) * g.Nout : nullptr;
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
 #pragma unroll
@@ -582,14 +627,30 @@ __global__ void __launch_bounds__(2 * T, 2) gemm_256_kernel(G256Args g) {
                 const int n = n0 + wn * 64 + j * 32 + 8 * q4 + 4 * fh;
                 if (n >= g.Nout) continue;  // Nout % 16 == 0: groups of 4 are all in or all out
                 float v0 = acc[i][j][4 * q4], v1 = acc[i][j][4 * q4 + 1], v2 = acc[i][j][4 * q4 + 2], v3 = acc[i][j][4 * q4 + 3];
-                if (g.bias) {
+                if (g.bias && split == 0) {
                     v0 += bf16_to_f32(g.bias[n]); v1 += bf16_to_f32(g.bias[n + 1]);
                     v2 += bf16_to_f32(g.bias[n + 2]); v3 += bf16_to_f32(g.bias[n + 3]);
                 }
-                *(u32x2*)(crow + n) = u32x2{pack_bf16x2(v0, v1), pack_bf16x2(v2, v3)};
+                if (prow) *(f32x4*)(prow + n) = f32x4{v0, v1, v2, v3};
+                else *(u32x2*)(crow + n) = u32x2{pack_bf16x2(v0, v1), pack_bf16x2(v2, v3)};
             }
         }
     }
+}
+
+// C[row][n] = bf16(partial[0][row][n] + partial[1][row][n] + ...), splits added in index order; a thread per 4 columns
+__global__ void __launch_bounds__(256) splitk_reduce_kernel(const float* __restrict__ partial, int ksplit, int64_t M, int Nout,
+                                                            bf16_t* __restrict__ C, int64_t ldc) {
+    const int64_t quads = (int64_t)(Nout >> 2), idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= M * quads) return;
+    const int64_t row = idx / quads, n = (idx - row * quads) << 2;
+    const float* p = partial + row * Nout + n;
+    f32x4 acc = *(const f32x4*)p;
+    for (int s = 1; s < ksplit; ++s) {
+        const f32x4 v = *(const f32x4*)(p + (int64_t)s * M * Nout);
+        acc[0] += v[0]; acc[1] += v[1]; acc[2] += v[2]; acc[3] += v[3];
+    }
+    *(u32x2*)(C + row * ldc + n) = u32x2{pack_bf16x2(acc[0], acc[1]), pack_bf16x2(acc[2], acc[3])};
 }
 
 }  // namespace xq
