@@ -368,3 +368,56 @@ def test_moe_seeded_shape_sweep(hip_device):
                         rec = R.moe_fwd_bwd(x, rw, sel, banks["gate"], banks["up"], banks["down"], lora, m.scaling, dy,
                                             dtype=torch.bfloat16)
                     assert err <= 1.5 * R.max_rel_err(rec[f"d{f}_{k}"].float(), ex[f"d{f}_{k}"]), tag + (k, f, err)
+
+
+@pytest.mark.parametrize("fmt,hybrid", [("block_fp8", False), ("nvfp4", True)])
+def test_dispatched_rows_compute_and_single_expert_calls(hip_device, fmt, hybrid):
+    """The compute step of an expert-parallel forward (rows already grouped by expert + inclusive cumsum, no routing
+    weight) and the per-expert call of the eager implementation, against the float64 per-expert program."""
+    from xorl_amd.moe_functional import EP_EXPERT_COMPUTE_QLORA_PACKED
+
+    E, H, I, r = 6, 128, 192, 8
+    m, banks = _make_experts(fmt, E, H, I, r, hybrid, seed=61, device=hip_device)
+    counts = torch.tensor([37, 0, 130, 1, 0, 64])
+    R_ = int(counts.sum())
+    cumsum = counts.cumsum(0)
+    expert = torch.repeat_interleave(torch.arange(E), counts).int()
+    x = gen((R_, H), 1.0, 62, torch.bfloat16)
+    dy = gen((R_, H), 1.0, 63, torch.bfloat16)
+    lora = {k: (getattr(m, f"{k}_proj_lora_A").detach().cpu(), getattr(m, f"{k}_proj_lora_B").detach().cpu())
+            for k in ("gate", "up", "down")}
+    ex = R.moe_fwd_bwd(x, torch.ones(R_, 1), expert.unsqueeze(1), banks["gate"], banks["up"], banks["down"], lora,
+                       m.scaling, dy)
+
+    xd = x.to(hip_device).requires_grad_(True)
+    y = m.compute_dispatched(xd, cumsum.to(hip_device))
+    y.backward(dy.to(hip_device))
+    assert y.shape == (R_, H) and R.max_rel_err(y.cpu(), ex["y"]) <= TOL
+    assert R.max_rel_err(xd.grad.cpu(), ex["dx"]) <= TOL
+    for k in ("gate", "up", "down"):
+        assert R.max_rel_err(getattr(m, f"{k}_proj_lora_A").grad.cpu(), ex[f"dA_{k}"]) <= TOL, k
+        assert R.max_rel_err(getattr(m, f"{k}_proj_lora_B").grad.cpu(), ex[f"dB_{k}"]) <= TOL, k
+    # the registry callable is the same program; scores multiply afterwards
+    gA, gB = m._active_lora_views("gate_proj")
+    uA, uB = m._active_lora_views("up_proj")
+    dA, dB = m._active_lora_views("down_proj")
+    with torch.no_grad():
+        y2 = EP_EXPERT_COMPUTE_QLORA_PACKED["hip"](x.to(hip_device), cumsum.to(hip_device), m._bank("gate"), m._bank("up"),
+                                                   m._bank("down"), gA, gB, uA, uB, dA, dB, m._active_scaling())
+        assert torch.equal(y2, y.detach())
+        scores = torch.rand(R_, device=hip_device)
+        y3 = m.compute_dispatched(x.to(hip_device), cumsum.to(hip_device), expert_scores=scores)
+        assert torch.equal(y3, y.detach() * scores.unsqueeze(1).to(torch.bfloat16))
+        # one expert at a time: the same rows give the same values as inside the grouped call
+        lo = int(cumsum[1])
+        y_e2 = m(x[lo:lo + 130].to(hip_device), expert_idx=2)
+        assert R.max_rel_err(y_e2.cpu(), ex["y"][lo:lo + 130]) <= TOL
+        assert torch.count_nonzero(m(x[:4].to(hip_device), expert_idx=E + 3)) == 0       # lives on another rank
+        # a rank that received no rows
+        empty = m.compute_dispatched(x[:0].to(hip_device), torch.zeros(E, dtype=torch.int64, device=hip_device))
+        assert empty.shape == (0, H)
+    with pytest.raises(ValueError):
+        m.compute_dispatched(x.to(hip_device), (cumsum - 1).clamp_min(0).to(hip_device))   # cumsum must end at the row count
+    m.moe_implementation = "eager"
+    with pytest.raises(ValueError, match="expert_idx"):
+        m(x.to(hip_device), torch.ones(R_, 1, device=hip_device), expert.unsqueeze(1).to(hip_device))

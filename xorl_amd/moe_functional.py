@@ -251,5 +251,39 @@ def moe_experts_qlora_forward(num_experts: int, routing_weights: Tensor, selecte
                                          down_proj_lora_B, gate_proj, up_proj, down_proj, num_experts, scaling)
 
 
-# registry entry a maintainer adds beside "triton" / "native" / "quack"
+def moe_experts_qlora_ep_compute(permute_tokens: Tensor, cumsum: Tensor, gate_proj: QuantWeight, up_proj: QuantWeight,
+                                 down_proj: QuantWeight, gate_proj_lora_A: Tensor, gate_proj_lora_B: Tensor,
+                                 up_proj_lora_A: Tensor, up_proj_lora_B: Tensor, down_proj_lora_A: Tensor,
+                                 down_proj_lora_B: Tensor, scaling: float, swiglu_limit: float = 0.0) -> Tensor:
+    """The expert MLP on rows that are already in expert order: `permute_tokens` [R, H] holds expert 0's rows, then
+    expert 1's, ...; `cumsum` [E] is the inclusive running count.  Returns [R, H] in the same order, with no routing
+    score applied (the caller multiplies afterwards).  Argument order of the reference's EP_EXPERT_COMPUTE_LORA
+    callables (models/layers/moe/backend/__init__.py:377-408; stated per expert in backend/eager.py:187-242), the
+    three banks as packed QuantWeight descriptors.
+
+    The rows run through the routed program as a top-1 problem with unit weights: the stable sort by expert is
+    then the identity and the weight multiplication exact."""
+    if swiglu_limit:
+        raise NotImplementedError("swiglu_limit clamping is not part of the packed-bank expert path")
+    E = gate_proj.num_experts
+    R = permute_tokens.shape[0]
+    if cumsum.numel() < E:
+        raise _C.XqError(f"cumsum has {cumsum.numel()} entries for {E} experts")
+    factors = (gate_proj_lora_A, gate_proj_lora_B, up_proj_lora_A, up_proj_lora_B, down_proj_lora_A, down_proj_lora_B)
+    if R == 0:
+        # no rows on this rank: an empty output that still reaches every factor, so their gradients are zeros
+        anchor = sum(f.sum() for f in factors) * 0.0
+        return permute_tokens.new_zeros((0, down_proj.cols)) + anchor.to(permute_tokens.dtype)
+    dev = permute_tokens.device
+    ends = cumsum[:E].to(device=dev, dtype=torch.int64)
+    expert_of_row = torch.searchsorted(ends, torch.arange(R, device=dev), right=True)
+    if int(ends[-1]) != R:
+        raise _C.XqError(f"cumsum ends at {int(ends[-1])} but {R} rows were passed")
+    ones = torch.ones(R, 1, dtype=torch.float32, device=dev)
+    return MoeExpertsQLoRAFunction.apply(permute_tokens, ones, expert_of_row.to(torch.int32).unsqueeze(1), *factors,
+                                         gate_proj, up_proj, down_proj, E, scaling)
+
+
+# registry entries a maintainer adds beside "triton" / "native" / "quack"
 MOE_EXPERT_BACKENDS_QLORA_PACKED: Dict[str, object] = {"hip": moe_experts_qlora_forward}
+EP_EXPERT_COMPUTE_QLORA_PACKED: Dict[str, object] = {"hip": moe_experts_qlora_ep_compute}

@@ -20,7 +20,7 @@ from torch import Tensor
 from .. import _C
 from .. import quantize as Q
 from ..functional import QuantWeight
-from ..moe_functional import moe_experts_qlora_forward
+from ..moe_functional import moe_experts_qlora_ep_compute, moe_experts_qlora_forward
 from .linear import LoraModule
 
 
@@ -307,8 +307,19 @@ class QLoRAMoeExperts(LoraModule, nn.Module):
     # ------------------------------------------------------------------ forward
     def forward(self, hidden_states: Tensor, routing_weights: Tensor = None, selected_experts: Tensor = None,
                 expert_idx: int = None) -> Tensor:
-        if expert_idx is not None or self.moe_implementation == "eager":
-            raise NotImplementedError("per-expert eager calls are not part of the fused packed-bank path")
+        """Routed call (hidden [T, H], routing_weights / selected_experts [T, top-k]) or, with `expert_idx`, the
+        MLP of one expert on the rows passed (moe_experts.py:576-620, :738-786): `expert_idx` is a global index,
+        an expert that lives on another rank returns zeros."""
+        if self.moe_implementation == "eager" and expert_idx is None:
+            raise ValueError("moe_implementation='eager' calls the experts one at a time: pass expert_idx")
+        if expert_idx is not None:
+            local = expert_idx - self.expert_offset
+            if local < 0 or local >= self.num_local_experts:
+                return torch.zeros_like(hidden_states[..., : self.hidden_size])
+            rows = hidden_states.reshape(-1, hidden_states.shape[-1])
+            cumsum = torch.zeros(self.num_local_experts, dtype=torch.int64, device=rows.device)
+            cumsum[local:] = rows.shape[0]
+            return self.compute_dispatched(rows, cumsum).reshape(*hidden_states.shape[:-1], self.hidden_size)
         gA, gB = self._active_lora_views("gate_proj")
         uA, uB = self._active_lora_views("up_proj")
         dA, dB = self._active_lora_views("down_proj")
@@ -317,6 +328,19 @@ class QLoRAMoeExperts(LoraModule, nn.Module):
             hidden_states=hidden_states, gate_proj=self._bank("gate"), up_proj=self._bank("up"),
             down_proj=self._bank("down"), gate_proj_lora_A=gA, gate_proj_lora_B=gB, up_proj_lora_A=uA,
             up_proj_lora_B=uB, down_proj_lora_A=dA, down_proj_lora_B=dB, scaling=self._active_scaling())
+
+    def compute_dispatched(self, permute_tokens: Tensor, cumsum: Tensor, expert_scores: Tensor = None) -> Tensor:
+        """The compute step of an expert-parallel forward (moe_experts.py:652-698): rows already grouped by local
+        expert (`cumsum` inclusive per local expert) -> their MLP outputs in the same order; `expert_scores` [R],
+        when given, multiply the output rows afterwards, as the reference does between compute and combine."""
+        gA, gB = self._active_lora_views("gate_proj")
+        uA, uB = self._active_lora_views("up_proj")
+        dA, dB = self._active_lora_views("down_proj")
+        out = moe_experts_qlora_ep_compute(permute_tokens, cumsum, self._bank("gate"), self._bank("up"),
+                                           self._bank("down"), gA, gB, uA, uB, dA, dB, self._active_scaling())
+        if expert_scores is not None:
+            out = out * expert_scores.unsqueeze(1).to(out.dtype)
+        return out
 
     def merge_weights(self, ema_decay: float = 0.1) -> None:
         with torch.no_grad():
