@@ -135,21 +135,21 @@ def _(x, packed, scales, global_scale, lora_A, lora_B, bias, fmt, scale_code, gr
     return x.new_empty(*x.shape[:-1], N), x.new_empty(M if want_su else 0, _r_pad(r))
 
 
-@torch.library.custom_op("xq::linear_bwd", mutates_args=(), device_types="cuda")
-def _linear_bwd_op(dy: Tensor, x: Tensor, su: Tensor, packed: Tensor, scales: Tensor,
-                   global_scale: Optional[Tensor], lora_A: Optional[Tensor], lora_B: Optional[Tensor],
-                   fmt: str, scale_code: int, group: int, N: int, K: int, r: int, scaling: float,
-                   need_dx: bool, need_dA: bool, need_dB: bool) -> Tuple[Tensor, Tensor, Tensor]:
+def _linear_bwd_impl(dy: Tensor, x: Tensor, su: Tensor, packed: Tensor, scales: Tensor,
+                     global_scale: Optional[Tensor], lora_A: Optional[Tensor], lora_B: Optional[Tensor],
+                     fmt: str, scale_dt: torch.dtype, group: int, N: int, K: int, r: int, scaling: float,
+                     need_dx: bool, need_dA: bool, need_dB: bool,
+                     cw: Optional[_C.XqWeight] = None) -> Tuple[Tensor, Tensor, Tensor]:
     dy2 = _as_2d(dy.to(torch.bfloat16))
     x2 = _as_2d(x)
     M = dy2.shape[0]
-    w = _C.make_weight(fmt, _C.XQ_LAYOUT_FLAT, packed, scales, _CODE_TO_DT[scale_code], N, K, group, global_scale)
+    w = cw if cw is not None else _C.make_weight(fmt, _C.XQ_LAYOUT_FLAT, packed, scales, scale_dt, N, K, group, global_scale)
     dev = dy.device
     dx = torch.empty(M, K, dtype=torch.bfloat16, device=dev) if need_dx else torch.empty(0, dtype=torch.bfloat16, device=dev)
     dA = torch.empty(r, K, dtype=torch.float32, device=dev) if need_dA else torch.empty(0, device=dev)
     dB = torch.empty(N, r, dtype=torch.float32, device=dev) if need_dB else torch.empty(0, device=dev)
     L = _C.lib()
-    ws_bytes = L.xq_linear_workspace_bytes(M, N, K, r)
+    ws_bytes = _workspace_bytes(M, N, K, r)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     A = lora_A.contiguous() if lora_A is not None else None
     B = lora_B.contiguous() if lora_B is not None else None
@@ -160,6 +160,15 @@ def _linear_bwd_op(dy: Tensor, x: Tensor, su: Tensor, packed: Tensor, scales: Te
     if need_dx:
         dx = dx.reshape(x.shape)
     return dx, dA, dB
+
+
+@torch.library.custom_op("xq::linear_bwd", mutates_args=(), device_types="cuda")
+def _linear_bwd_op(dy: Tensor, x: Tensor, su: Tensor, packed: Tensor, scales: Tensor,
+                   global_scale: Optional[Tensor], lora_A: Optional[Tensor], lora_B: Optional[Tensor],
+                   fmt: str, scale_code: int, group: int, N: int, K: int, r: int, scaling: float,
+                   need_dx: bool, need_dA: bool, need_dB: bool) -> Tuple[Tensor, Tensor, Tensor]:
+    return _linear_bwd_impl(dy, x, su, packed, scales, global_scale, lora_A, lora_B, fmt, _CODE_TO_DT[scale_code],
+                            group, N, K, r, scaling, need_dx, need_dA, need_dB)
 
 
 @_linear_bwd_op.register_fake
@@ -181,8 +190,12 @@ class QLoRALinearFunction(torch.autograd.Function):
     def forward(ctx, x, lora_A, lora_B, bias, qw: QuantWeight, r: int, scaling: float, want_su: bool = True):
         A = lora_A[:r] if lora_A is not None else None
         B = lora_B[:, :r] if lora_B is not None else None
-        y, su = _linear_fwd_op(x, qw.packed, qw.scales, qw.global_scale, A, B, bias, qw.fmt,
-                               _DT_TO_CODE[qw.scale_dtype], qw.group, qw.rows, qw.cols, r, float(scaling), want_su)
+        if torch.compiler.is_compiling():
+            y, su = _linear_fwd_op(x, qw.packed, qw.scales, qw.global_scale, A, B, bias, qw.fmt,
+                                   _DT_TO_CODE[qw.scale_dtype], qw.group, qw.rows, qw.cols, r, float(scaling), want_su)
+        else:       # eager: straight to the library (the custom-op layer costs tens of microseconds of host time per call)
+            y, su = _linear_fwd_impl(x, qw.packed, qw.scales, qw.global_scale, A, B, bias, qw.fmt, qw.scale_dtype,
+                                     qw.group, qw.rows, qw.cols, r, float(scaling), want_su, qw.c())
         ctx.qw, ctx.r, ctx.scaling = qw, r, float(scaling)
         ctx.save_for_backward(x, su, lora_A, lora_B)
         return y
@@ -194,9 +207,14 @@ class QLoRALinearFunction(torch.autograd.Function):
         need_dx, need_dA, need_dB = ctx.needs_input_grad[0], ctx.needs_input_grad[1], ctx.needs_input_grad[2]
         A = lora_A[:r] if lora_A is not None else None
         B = lora_B[:, :r] if lora_B is not None else None
-        dx, dA, dB = _linear_bwd_op(dy, x, su, qw.packed, qw.scales, qw.global_scale, A, B, qw.fmt,
-                                    _DT_TO_CODE[qw.scale_dtype], qw.group, qw.rows, qw.cols, r, ctx.scaling,
-                                    need_dx, need_dA, need_dB)
+        if torch.compiler.is_compiling():
+            dx, dA, dB = _linear_bwd_op(dy, x, su, qw.packed, qw.scales, qw.global_scale, A, B, qw.fmt,
+                                        _DT_TO_CODE[qw.scale_dtype], qw.group, qw.rows, qw.cols, r, ctx.scaling,
+                                        need_dx, need_dA, need_dB)
+        else:
+            dx, dA, dB = _linear_bwd_impl(dy, x, su, qw.packed, qw.scales, qw.global_scale, A, B, qw.fmt,
+                                          qw.scale_dtype, qw.group, qw.rows, qw.cols, r, ctx.scaling,
+                                          need_dx, need_dA, need_dB, qw.c())
         gA = gB = None
         if need_dA:
             gA = dA if lora_A.shape[0] == r else torch.cat([dA, dA.new_zeros(lora_A.shape[0] - r, dA.shape[1])], 0)
