@@ -306,3 +306,27 @@ def test_training_shape_rule_is_reported_at_the_forward(hip_device):
     assert R.max_rel_err(y.cpu(), ex["y"]) <= TOL
     with pytest.raises(ValueError, match="out_features % 64"):
         m(x.requires_grad_(True))
+
+
+@pytest.mark.parametrize("backend", ["eager", "aot_eager"])
+def test_module_under_torch_compile(hip_device, backend):
+    """Traced by torch.compile the module reaches the library through the registered custom ops (fake tensors for
+    shapes); forward and all gradients equal the eager call bit for bit."""
+    from torch.library import opcheck
+
+    from xorl_amd import functional as Fn
+
+    m, _ = make_dense_module("block_fp8", 512, 256, 16, 32, seed=1, device=hip_device)
+    x = gen((200, 256), 1.0, 3, torch.bfloat16).to(hip_device)
+    dy = gen((200, 512), 1.0, 4, torch.bfloat16).to(hip_device)
+    ref = _run(m, x, dy)
+    ref = tuple(t.clone() for t in ref)
+    m.lora_A.grad = m.lora_B.grad = None
+    torch._dynamo.reset()
+    got = _run(torch.compile(m, backend=backend), x, dy)
+    for a, b in zip(ref, got):
+        assert torch.equal(a, b)
+    qw = m._forward_quant_weight()
+    args = (x, qw.packed, qw.scales, qw.global_scale, m.lora_A.detach(), m.lora_B.detach(), None, qw.fmt,
+            Fn._DT_TO_CODE[qw.scale_dtype], qw.group, qw.rows, qw.cols, 16, 2.0, True)
+    assert set(opcheck(Fn._linear_fwd_op, args, test_utils=("test_schema", "test_faketensor")).values()) == {"SUCCESS"}
