@@ -41,7 +41,8 @@ MEASURED_TRAFFIC_BYTES = {
     0: 109.6 * 2 ** 20,    # gemm_256_kernel<int4, T=128> in 4 K splits + splitk_reduce_kernel: mean of the forward and dgrad
                            # launches (64 MiB of it are the fp32 partial sums written and read back)
     1: 905.4 * 2 ** 20,    # gemm_256_kernel<fp8>: mean of the forward and dgrad launches
-    2: 160.4 * 2 ** 20,    # gemm_256_kernel<nvfp4>, 256x256 and 128x128 tiles: mean over the 12 launches of a step
+    2: 187.2 * 2 ** 20,    # gemm_256_kernel<nvfp4>, 256x256 tiles (whole rounds; trailing rows in K splits) and 128x128 tiles
+                           # (+ splitk_reduce_kernel): mean over the 12 launches of a step, fp32 partial sums included
     3: 1032.2 * 2 ** 20,   # gemm_256_kernel<fp8, grouped>: mean over the 6 launches of a step
     4: 41.0 * 2 ** 20,     # skinny_split_kernel + skinny_epilogue_kernel: mean per forward over the 32 cases (includes
                            # the fp32 partial tiles written and read back: 23.3 MiB of it are algorithmic)
@@ -176,7 +177,7 @@ def other_config(cfg: int, dev):
                 m(xs[k]).backward(dys[k])
         return (step, sum(lin_flops(Mtok, K, N, 16) for (N, K) in shapes.values()), False,
                 "configs[2]: nvfp4 QLoRA Qwen3-32B attention projections q/k/v/o, hidden 5120, M=4096, r=16, fwd+bwd",
-                "gemm_256_kernel<nvfp4> with 256x256 tiles (whole rounds of the chip) and 128x128 tiles (k/v forward, trailing rows): fused dequant-GEMM, forward and dgrad launches")
+                "gemm_256_kernel<nvfp4> with 256x256 tiles (whole rounds of the chip; trailing tile rows in K splits + splitk_reduce_kernel) and 128x128 tiles (k/v forward and dgrad): fused dequant-GEMM, forward and dgrad launches")
     if cfg in (3, 7, 8):
         # 7 / 8 are not BASELINE configs: configs[3] with the banks held as nvfp4 / NF4 (4-bit GKN storage)
         from xorl_amd.qlora import BlockFP8QLoRAMoeExperts, NF4QLoRAMoeExperts, NvFP4QLoRAMoeExperts

@@ -193,13 +193,20 @@ def test_silu_and_mul(hip_device):
     assert R.max_rel_err(ud.grad.cpu(), u64.grad) <= TOL
 
 
-@pytest.mark.parametrize("fmt,M,K,N", [("block_fp8", 4100, 256, 4096), ("int4", 4352, 384, 5120), ("nvfp4", 4099, 256, 4352)])
+@pytest.mark.parametrize("fmt,M,K,N", [("block_fp8", 4100, 256, 4096), ("int4", 4352, 384, 5120), ("nvfp4", 4099, 256, 4352),
+                                       ("block_fp8", 4352, 2048, 4096), ("nvfp4", 4200, 2048, 4096)])
 def test_dense_split_launch_tail_rows(hip_device, fmt, M, K, N):
     """Shapes whose 256x256 tiling leaves a partly filled last round of the chip: the launcher runs the leading
-    tile rows on large tiles and the trailing rows (here 4, 256 and 3 + 256 of them) as a second launch of small
-    tiles.  Forward, dgrad and both factor gradients against the float64 form, with particular attention to the
-    rows on either side of the seam."""
+    tile rows on large tiles and the trailing rows (here 4, 256, 3 + 256, 256 and 104 of them) as a second launch:
+    of small tiles when the contraction is short, of large tiles in K splits (fp32 partial sums added by a reduce
+    kernel) when it has at least 16 K-steps -- the last two cases.  Forward, dgrad and both factor gradients
+    against the float64 form, with particular attention to the rows on either side of the seam."""
     r = 16
+    if K >= 1024:
+        from xorl_amd import _C
+
+        tail = M - (M // 256) * 256 if M % 256 else 256
+        assert _C.lib().xq_linear_workspace_bytes(M, N, K, 0) >= 2 * tail * N * 4      # the plan splits the tail
     m, w_ref = make_dense_module(fmt, N, K, r, 32, seed=M + N, device=hip_device, bias=True)
     x = gen((M, K), 1.0, 31, torch.bfloat16)
     dy = gen((M, N), 1.0, 32, torch.bfloat16)

@@ -28,20 +28,22 @@ static int raise_lds_limit(K kernel, size_t bytes, const char* who) {
     return XQ_OK;
 }
 
-template <int FMT, bool CC, bool GROUPED, int T>
+template <int FMT, bool CC, bool GROUPED, int T, bool SPLIT256 = false>
 static int launch_256_one(const G256Args& f, dim3 grid, hipStream_t s, const char* who) {
     static bool attr_set = false;  // per instantiation
     if (!attr_set) {
-        int rc = raise_lds_limit(gemm_256_kernel<FMT, CC, GROUPED, T>, Geo<T>::lds_bytes(CC), who);
+        int rc = raise_lds_limit(gemm_256_kernel<FMT, CC, GROUPED, T, SPLIT256>, Geo<T>::lds_bytes(CC), who);
         if (rc) return rc;
         attr_set = true;
     }
-    gemm_256_kernel<FMT, CC, GROUPED, T><<<grid, Geo<T>::NT, Geo<T>::lds_bytes(CC), s>>>(f);
+    gemm_256_kernel<FMT, CC, GROUPED, T, SPLIT256><<<grid, Geo<T>::NT, Geo<T>::lds_bytes(CC), s>>>(f);
     return XQ_OK;
 }
 
 template <int FMT, bool CC, bool GROUPED>
 static int launch_256_t(const G256Args& f, int T, dim3 grid, hipStream_t s, const char* who) {
+    if constexpr (!GROUPED)
+        if (T == 256 && f.ksplit > 1) return launch_256_one<FMT, CC, false, 256, true>(f, grid, s, who);
     return T == 256 ? launch_256_one<FMT, CC, GROUPED, 256>(f, grid, s, who) : launch_256_one<FMT, CC, GROUPED, 128>(f, grid, s, who);
 }
 
@@ -58,31 +60,77 @@ static inline int dense_tile_size(int64_t n_rows, int64_t Nout) {
     return xq_cdiv(n_rows, 256) * xq_cdiv(Nout, 256) > 128 ? 256 : 128;
 }
 
-// K splits of a dense launch of `blocks` small tiles over nk K-steps (1 = none): used when the tiles fill at most
-// half of the block slots of the chip; every split keeps at least 8 K-steps.
+// K splits of a dense launch of `blocks` tiles of size T over nk K-steps (1 = none): used when the tiles fill at
+// most half of the block slots of the chip (256 large tiles, 512 small ones); every split keeps at least 8 K-steps.
 static inline int ksplit_for(int64_t blocks, int T, int64_t nk) {
-    const int64_t slots = 512;                       // small tiles only: two blocks per CU
-    if (T != 128 || blocks <= 0 || blocks * 2 > slots) return 1;
+    const int64_t slots = T == 256 ? 256 : 512;
+    if (blocks <= 0 || blocks * 2 > slots) return 1;
     int64_t s = slots / blocks;
     if (s > nk / 8) s = nk / 8;
     if (s > 8) s = 8;
     return s < 2 ? 1 : (int)s;
 }
 
-// fp32 partial-sum bytes the split-K form of a dense [n_rows, Nout] product over Kc wants, under any tile policy
+// How the default policy runs a dense [n_rows, Nout] product over nk K-steps: `head_rows` leading rows on tiles of
+// size T in `split` K splits, and, when head_rows < n_rows, the trailing rows as a second launch.  A launch of large
+// tiles whose last round would fill only part of the chip keeps the tile rows that make whole rounds and hands the
+// others either to small tiles (two of those blocks share a CU) or to large tiles in K splits, whichever the
+// estimates below make cheaper; the whole launch stays as it is unless that saves a fifth of a round.
+struct DensePlan {
+    int T, split;
+    int64_t head_rows;
+    int tail_T, tail_split;
+};
+static DensePlan plan_dense(int64_t n_rows, int64_t Nout, int64_t nk) {
+    DensePlan p{dense_tile_size(n_rows, Nout), 1, n_rows, 0, 1};
+    if (p.T == 128) {
+        p.split = ksplit_for(xq_cdiv(n_rows, 128) * xq_cdiv(Nout, 128), 128, nk);
+        return p;
+    }
+    const int64_t tr = xq_cdiv(n_rows, 256), tc = xq_cdiv(Nout, 256), cus = 256;
+    const int64_t full = tr * tc / cus, rem = tr * tc - full * cus;
+    const int64_t keep = full * cus / tc;                  // tile rows that stay on whole rounds of large tiles
+    if (rem == 0 || keep == 0 || keep >= tr) return p;
+    const int64_t tail_rows = n_rows - keep * 256;
+    // costs in units of one round of large tiles (measured: small tiles take 0.54 of it with up to one block per
+    // CU, 0.7 with up to two; a split large tile 1/S of it plus the pass over its fp32 partial sums at ~4 TB/s,
+    // a round lasting ~1.9 us per K-step)
+    const int64_t n128 = xq_cdiv(tail_rows, 128) * xq_cdiv(Nout, 128);
+    const double small_cost = n128 <= cus ? 0.54 : 0.7 * (double)xq_cdiv(n128, 2 * cus);
+    const int s256 = ksplit_for((tr - keep) * tc, 256, nk);
+    const double round_us = 1.9 * (double)nk;
+    const double split_cost = s256 > 1 ? 1.0 / s256 + (3.0 + (4.0 * s256 + 2.0) * (double)tail_rows * (double)Nout / 4.0e6) / round_us : 1e9;
+    const double tail_cost = small_cost < split_cost ? small_cost : split_cost;
+    if ((double)xq_cdiv(keep * tc, cus) + tail_cost < (double)(full + 1) - 0.2) {
+        p.head_rows = keep * 256;
+        if (split_cost < small_cost) { p.tail_T = 256; p.tail_split = s256; }
+        else { p.tail_T = 128; p.tail_split = 1; }
+    }
+    return p;
+}
+
+// fp32 partial-sum bytes the split-K forms of a dense [n_rows, Nout] product over Kc may want, under any tile policy
 int64_t tile_gemm_partial_bytes(int64_t n_rows, int64_t Nout, int64_t Kc) {
     if (n_rows <= 0 || Kc % BK) return 0;
-    const int s = ksplit_for(xq_cdiv(n_rows, 128) * xq_cdiv(Nout, 128), 128, Kc / BK);
-    return s > 1 ? (int64_t)s * n_rows * Nout * 4 : 0;
+    const int64_t nk = Kc / BK;
+    int64_t elems = 0;
+    for (int T : {128, 256}) {         // a whole launch on either tile size (default or forced policy)
+        const int s = ksplit_for(xq_cdiv(n_rows, T) * xq_cdiv(Nout, T), T, nk);
+        if (s > 1 && s * n_rows > elems) elems = s * n_rows;
+    }
+    const DensePlan p = plan_dense(n_rows, Nout, nk);
+    if (p.head_rows < n_rows && p.tail_split > 1 && p.tail_split * (n_rows - p.head_rows) > elems)
+        elems = p.tail_split * (n_rows - p.head_rows);
+    return elems * Nout * 4;
 }
 
 // C[rows, Nout] = A . op(deq(W)) (+ su . Lr^T) (+ bias); see xq_gemm_tile.h.  force_T = 256 / 128 fixes the tile
-// size of the pipelined kernel, 0 leaves it to the selection policy.  `partial` (may be NULL) is scratch for
+// size of the pipelined kernel (and force_split its K splits), 0 leaves both to the selection policy.  `partial` (may be NULL) is scratch for
 // split-K sums; a launch that would split but finds less than tile_gemm_partial_bytes() there runs unsplit.
 static int launch_tile_gemm_t(const xq_weight* w, bool contract_cols, const bf16_t* A, int64_t lda, int64_t n_rows,
                               const int32_t* offsets, const int32_t* tile_offsets, const bf16_t* su, const bf16_t* lora_right,
                               int r_pad, const bf16_t* bias, bf16_t* C, int64_t ldc, hipStream_t stream, const char* who,
-                              int force_T, float* partial, int64_t partial_bytes) {
+                              int force_T, int force_split, float* partial, int64_t partial_bytes) {
     TileArgs g;
     g.A = A; g.lda = lda; g.C = C; g.ldc = ldc;
     g.packed = (const uint8_t*)w->packed;
@@ -119,31 +167,18 @@ static int launch_tile_gemm_t(const xq_weight* w, bool contract_cols, const bf16
                              (grouped ? w->layout == XQ_LAYOUT_GKN && g.wcols % 16 == 0 && g.wrows >= 2 &&
                                             xq_aligned(w->scales, 16) && g.scale_stride % 16 == 0
                                       : w->layout == XQ_LAYOUT_FLAT));
-        const bool big = grouped ? (n_rows >= 128ll * w->num_experts && n_rows >= 8192)
-                                 : dense_tile_size(n_rows, g.Nout) == 256;
-        const int T = force_T ? force_T : g_tile_policy == 2 ? 256 : g_tile_policy == 3 ? 128 : (big ? 256 : 128);
-        // A dense launch of 256x256 tiles whose last round would fill only part of the chip: the leading tile rows
-        // that make whole rounds keep the large tiles, the remaining rows run as a second launch of 128x128 tiles
-        // (two of those blocks share a CU).  Costs in units of one round of large tiles: a launch of small tiles
-        // takes about 0.54 (up to one block per CU) or 0.7 (up to two per CU) of it.
-        if (!grouped && fmt_ok && g_tile_policy == 0 && force_T == 0 && T == 256) {
-            const int64_t tr = xq_cdiv(n_rows, 256), tc = xq_cdiv(g.Nout, 256), cus = 256;
-            const int64_t full = tr * tc / cus, rem = tr * tc - full * cus;
-            const int64_t keep = full * cus / tc;                  // tile rows that stay on large tiles
-            if (rem > 0 && keep > 0 && keep < tr) {
-                const int64_t tail_rows = n_rows - keep * 256;
-                const int64_t n128 = xq_cdiv(tail_rows, 128) * xq_cdiv(g.Nout, 128);
-                const double tail = n128 <= cus ? 0.54 : 0.7 * (double)xq_cdiv(n128, 2 * cus);
-                if ((double)xq_cdiv(keep * tc, cus) + tail < (double)(full + 1) - 0.2) {
-                    const int64_t head = keep * 256;
-                    const int rc = launch_tile_gemm_t(w, contract_cols, A, lda, head, nullptr, nullptr, su, lora_right, r_pad,
-                                                      bias, C, ldc, stream, who, 256, nullptr, 0);
-                    if (rc) return rc;
-                    return launch_tile_gemm_t(w, contract_cols, A + head * lda, lda, tail_rows, nullptr, nullptr,
-                                              su ? su + head * r_pad : nullptr, lora_right, r_pad, bias, C + head * ldc, ldc,
-                                              stream, who, 128, nullptr, 0);
-                }
-            }
+        const bool big = grouped && n_rows >= 128ll * w->num_experts && n_rows >= 8192;   // grouped: large tiles
+        const DensePlan plan = plan_dense(n_rows, g.Nout, g.Kc / BK);
+        const bool planned = !grouped && fmt_ok && g_tile_policy == 0 && force_T == 0;
+        const int T = force_T ? force_T : g_tile_policy == 2 ? 256 : g_tile_policy == 3 ? 128 : grouped ? (big ? 256 : 128) : plan.T;
+        if (planned && plan.head_rows < n_rows) {
+            const int64_t head = plan.head_rows;
+            const int rc = launch_tile_gemm_t(w, contract_cols, A, lda, head, nullptr, nullptr, su, lora_right, r_pad,
+                                              bias, C, ldc, stream, who, 256, 1, nullptr, 0);
+            if (rc) return rc;
+            return launch_tile_gemm_t(w, contract_cols, A + head * lda, lda, n_rows - head, nullptr, nullptr,
+                                      su ? su + head * r_pad : nullptr, lora_right, r_pad, bias, C + head * ldc, ldc,
+                                      stream, who, plan.tail_T, plan.tail_split, partial, partial_bytes);
         }
         const int64_t tiles_m = xq_cdiv(n_rows, T) + (grouped ? w->num_experts : 0);
         const int64_t tiles_n = xq_cdiv(g.Nout, T);
@@ -160,7 +195,7 @@ static int launch_tile_gemm_t(const xq_weight* w, bool contract_cols, const bf16
             f.su = g.r_pad ? su : nullptr; f.lora_right = g.r_pad ? lora_right : nullptr; f.r_pad = g.r_pad;
             f.bias = bias;
             f.tiles_m = (int32_t)tiles_m; f.tiles_n = (int32_t)tiles_n;
-            int ksplit = (grouped || force_T) ? 1 : ksplit_for(tiles_m * tiles_n, T, g.Kc / BK);
+            int ksplit = grouped ? 1 : force_T ? force_split : planned ? plan.split : ksplit_for(tiles_m * tiles_n, T, g.Kc / BK);
             if (ksplit > 1 && (!partial || !xq_aligned(partial, 16) || partial_bytes < (int64_t)ksplit * n_rows * g.Nout * 4)) ksplit = 1;
             f.ksplit = ksplit; f.partial = ksplit > 1 ? partial : nullptr;
             dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)ksplit);
@@ -201,7 +236,7 @@ int launch_tile_gemm(const xq_weight* w, bool contract_cols, const bf16_t* A, in
                      int r_pad, const bf16_t* bias, bf16_t* C, int64_t ldc, hipStream_t stream, const char* who,
                      float* partial, int64_t partial_bytes) {
     return launch_tile_gemm_t(w, contract_cols, A, lda, n_rows, offsets, tile_offsets, su, lora_right, r_pad, bias, C, ldc,
-                              stream, who, 0, partial, partial_bytes);
+                              stream, who, 0, 1, partial, partial_bytes);
 }
 
 static inline int64_t align256(int64_t b) { return (b + 255) & ~(int64_t)255; }

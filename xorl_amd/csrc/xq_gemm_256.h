@@ -81,7 +81,7 @@ struct G256Args {
     int32_t r_pad;
     const bf16_t* bias;
     int32_t tiles_m, tiles_n;  // grouped: tiles_m is an upper bound
-    // dense launches of the small tile only: ksplit > 1 divides the K-steps over gridDim.y blocks per tile; split s then writes its fp32
+    // dense launches: ksplit > 1 divides the K-steps over gridDim.y blocks per tile; split s then writes its fp32
     // sums to partial + s * M * Nout (row pitch Nout) instead of C, and split 0 carries the low-rank term and bias
     int32_t ksplit;
     float* partial;
@@ -372,7 +372,7 @@ template <bool CC, bool GROUPED, int T> struct W256Sel<XQ_FMT_FP8, CC, GROUPED, 
 template <bool CC, int T> struct W256Sel<XQ_FMT_FP8, CC, true, T> { using type = W256Fp8<CC, T>; };
 
 // ---------------------------------------------------------------- the kernel
-template <int FMT, bool CC, bool GROUPED, int T>
+template <int FMT, bool CC, bool GROUPED, int T, bool SPLIT256 = false>
 __global__ void __launch_bounds__(2 * T, 2) gemm_256_kernel(G256Args g) {
     using G = Geo<T>;
     constexpr int F8_BM = G::BM, F8_BN = G::BN, F8_A_STAGE = G::A_STAGE, F8_NN_PITCH = G::NN_PITCH;
@@ -437,7 +437,9 @@ __global__ void __launch_bounds__(2 * T, 2) gemm_256_kernel(G256Args g) {
     }
     const int n0 = pid_n * F8_BN;
     // K-steps of this block: all of them, or the split's share (every split has at least one)
-    constexpr bool CAN_SPLIT = !GROUPED && T == 128;      // only the small tile is used on part-filled chips
+    // K splits: the small tile always knows them; the large tile has an instantiation of its own for them
+    // (trailing rows of a launch that fill part of a round), so the unsplit one carries nothing extra
+    constexpr bool CAN_SPLIT = !GROUPED && (T == 128 || SPLIT256);
     int kt0 = 0, nk = g.Kc / F8_BK;
     const int split = CAN_SPLIT ? (int)blockIdx.y : 0;
     if (CAN_SPLIT && g.ksplit > 1) {
