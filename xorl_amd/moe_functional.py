@@ -158,6 +158,8 @@ class MoeExpertsQLoRAFunction(torch.autograd.Function):
         F_dA = _prep(dA, True, rp, I)                                             # [E|1, rp, I]
         Lr_dB = _prep(_expand(dB, E), True, H, rp)                                # [E, H, rp]
 
+        # (one pass over xs with both panels side by side takes as long as these two: the product is bound by its
+        # fp32 multiply-adds, not by reading the rows)
         su_g = _lora_down(xs, F_gA, offsets, tile_offsets, E, s)
         su_u = _lora_down(xs, F_uA, offsets, tile_offsets, E, s)
         gate_out = _grouped_gemm(qw_gate, False, xs, offsets, tile_offsets, su_g, Lr_gB)    # [R, I]
@@ -224,11 +226,18 @@ class MoeExpertsQLoRAFunction(torch.autograd.Function):
             Lr_A = _prep(_expand(A, E), False, H, rp)                                        # [E, H, rp]
             dx = _grouped_gemm(qw, True, g_out, offsets, tile_offsets, v, Lr_A)              # [R, H]
             gB_ = _wgrad(g_out, su, r, None if B.shape[0] == 1 else offsets, E, True)        # [E|1, r, I]
-            gA_ = _wgrad(xs, v, r, None if A.shape[0] == 1 else offsets, E, False)           # [E|1, H, r]
-            return dx, gA_, gB_
+            return dx, v, gB_
 
-        dx_u, grad_uA, grad_uB = proj_bwd(dup, qw_up, uA, uB, su_u)
-        dx_g, grad_gA, grad_gB = proj_bwd(dgate, qw_gate, gA, gB, su_g)
+        dx_u, v_u, grad_uB = proj_bwd(dup, qw_up, uA, uB, su_u)
+        dx_g, v_g, grad_gB = proj_bwd(dgate, qw_gate, gA, gB, su_g)
+        # gradients of the two A factors, [E|1, H, r] = x^T . v: both contract the same rows of x, so they share
+        # one pass over them (v_g | v_u side by side) when the panels fit
+        if gA.shape[0] == uA.shape[0] and 2 * rp <= 32:
+            both = _wgrad(xs, torch.cat([v_g, v_u], dim=1), rp + r, None if gA.shape[0] == 1 else offsets, E, False)
+            grad_gA, grad_uA = both[..., :r], both[..., rp:rp + r]
+        else:
+            grad_gA = _wgrad(xs, v_g, r, None if gA.shape[0] == 1 else offsets, E, False)
+            grad_uA = _wgrad(xs, v_u, r, None if uA.shape[0] == 1 else offsets, E, False)
         dx = moe_gather(dx_g, dx_u, sidx, T, topk).reshape(shape) if ctx.needs_input_grad[0] else None
 
         cast = lambda g, p: g.to(p.dtype)
