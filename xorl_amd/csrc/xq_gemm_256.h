@@ -412,16 +412,19 @@ __global__ void __launch_bounds__(2 * T, 2) gemm_256_kernel(G256Args g) {
     int e = 0;
     int64_t row0, row_end;
     if (GROUPED) {
+        // The expert whose tile range holds this row tile: thread t looks at expert t (and t + NT, ...), all loads
+        // issued together -- one memory round trip for the block instead of the chain of dependent loads a
+        // binary search by one thread makes.  Exactly one expert matches, or none beyond the last tile.
         int* sh_info = (int*)smem;
-        if (tid == 0) {
-            const int E = g.num_experts;
-            if (pid_m >= g.tile_prefix[E]) sh_info[0] = -1;
-            else {
-                int lo = 0, hi = E;  // tile_prefix[lo] <= pid_m < tile_prefix[lo + 1]
-                while (hi - lo > 1) { int mid = (lo + hi) >> 1; if (g.tile_prefix[mid] <= pid_m) lo = mid; else hi = mid; }
-                sh_info[0] = lo;
-                sh_info[1] = g.offsets[lo] + (pid_m - g.tile_prefix[lo]) * F8_BM;
-                sh_info[2] = g.offsets[lo + 1];
+        if (tid == 0) sh_info[0] = -1;
+        __syncthreads();
+        for (int t = tid; t < g.num_experts; t += NT) {
+            const int lo = g.tile_prefix[t], hi = g.tile_prefix[t + 1];
+            const int o0 = g.offsets[t], o1 = g.offsets[t + 1];
+            if (lo <= pid_m && pid_m < hi) {
+                sh_info[0] = t;
+                sh_info[1] = o0 + (pid_m - lo) * F8_BM;
+                sh_info[2] = o1;
             }
         }
         __syncthreads();

@@ -90,14 +90,18 @@ __global__ void __launch_bounds__(256) small_nt_kernel(SmallNtArgs g) {
     int e = 0;
     int64_t row0, row_end;
     if (g.offsets) {
-        if (tid == 0) {
-            int t = blockIdx.x, lo = 0, hi = g.num_experts;
-            if (t >= g.tile_offsets[g.num_experts]) sh_info[0] = -1;
-            else {
-                while (hi - lo > 1) { int mid = (lo + hi) >> 1; if (g.tile_offsets[mid] <= t) lo = mid; else hi = mid; }
-                sh_info[0] = lo;
-                sh_info[1] = g.offsets[lo] + (t - g.tile_offsets[lo]) * TR;
-                sh_info[2] = g.offsets[lo + 1];
+        // the expert whose tile range holds this block's tile: one look per thread, all loads in flight together
+        // (a binary search by one thread is a chain of dependent memory round trips)
+        if (tid == 0) sh_info[0] = -1;
+        __syncthreads();
+        const int t = blockIdx.x;
+        for (int x = tid; x < g.num_experts; x += blockDim.x) {
+            const int lo = g.tile_offsets[x], hi = g.tile_offsets[x + 1];
+            const int o0 = g.offsets[x], o1 = g.offsets[x + 1];
+            if (lo <= t && t < hi) {
+                sh_info[0] = x;
+                sh_info[1] = o0 + (t - lo) * TR;
+                sh_info[2] = o1;
             }
         }
         __syncthreads();
@@ -380,10 +384,13 @@ __global__ void __launch_bounds__(256) tn_grouped_kernel(TnArgs g, int32_t num_e
     const int64_t r_begin = (int64_t)blockIdx.y * TN_CHUNK;
     int64_t r_end = r_begin + TN_CHUNK;
     r_end = r_end < g.n_rows ? r_end : g.n_rows;
-    if (threadIdx.x == 0) {
-        int lo = 0, hi = num_experts;  // last e with offsets[e] <= r_begin
-        while (hi - lo > 1) { int mid = (lo + hi) >> 1; if (g.offsets[mid] <= r_begin) lo = mid; else hi = mid; }
-        sh_e = lo;
+    // the expert that owns row r_begin (offsets[e] <= r_begin < offsets[e + 1]; r_begin < n_rows = offsets[E], so
+    // exactly one does): one look per thread instead of a chain of dependent loads
+    if (threadIdx.x == 0) sh_e = num_experts;      // rows beyond the last expert's: nothing to do
+    __syncthreads();
+    for (int x = threadIdx.x; x < num_experts; x += 256) {
+        const int64_t o0 = g.offsets[x], o1 = g.offsets[x + 1];
+        if (o0 <= r_begin && r_begin < o1) sh_e = x;
     }
     __syncthreads();
     int e = sh_e;
