@@ -357,12 +357,16 @@ extern "C" int xq_linear_bwd(const xq_weight* w, const void* x, int64_t ldx, con
         bf16_t* A_bf = (bf16_t*)cv.take(rp * K * 2);
         v = (bf16_t*)cv.take(M * rp * 2);
         bf16_t* su_ws = (bf16_t*)cv.take(M * rp * 2);
+        // every factor layout this call needs, in one launch
+        FactorPrepJobs jobs{};
+        jobs.in_f32 = lora_dtype == XQ_DT_F32;
+        jobs.add(lora_B, N, r, true, Bt, rp, N);
+        if (dx) jobs.add(lora_A, r, K, true, At, K, rp);
+        if (dB && !su) jobs.add(lora_A, r, K, false, A_bf, rp, K);
+        if ((rc = launch_factor_prep_multi(jobs, stream))) return rc;
         // v = bf16(s * dy . B)   [M, rp]
-        if ((rc = launch_factor_prep(lora_B, lora_dtype, N, r, true, Bt, rp, N, 1, stream))) return rc;
         if ((rc = launch_small_nt((const bf16_t*)dy, lddy, M, N, Bt, rp, scaling, v, nullptr, nullptr, 1, true, stream))) return rc;
-        if (dx && (rc = launch_factor_prep(lora_A, lora_dtype, r, K, true, At, K, rp, 1, stream))) return rc;
         if (dB && !su) {
-            if ((rc = launch_factor_prep(lora_A, lora_dtype, r, K, false, A_bf, rp, K, 1, stream))) return rc;
             if ((rc = launch_small_nt((const bf16_t*)x, ldx, M, K, A_bf, rp, scaling, su_ws, nullptr, nullptr, 1, true, stream))) return rc;
             su = su_ws;
         }

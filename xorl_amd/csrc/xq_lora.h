@@ -9,6 +9,19 @@ namespace xq {
 
 // out[i][j] (bf16, [R_out, C_out], zero padded) = in[i][j] or in[j][i];  `in` is
 // fp32 or bf16 with shape [R_in, C_in] per expert.
+// up to three single-matrix conversions (same source dtype) done by one launch
+struct FactorPrepJobs {
+    const void* in[3];
+    bf16_t* out[3];
+    int64_t R_in[3], C_in[3], R_out[3], C_out[3];
+    int transpose[3];
+    int in_f32, n;
+    void add(const void* src, int64_t r_in, int64_t c_in, bool tr, bf16_t* dst, int64_t r_out, int64_t c_out) {
+        in[n] = src; out[n] = dst; R_in[n] = r_in; C_in[n] = c_in; R_out[n] = r_out; C_out[n] = c_out; transpose[n] = tr ? 1 : 0;
+        ++n;
+    }
+};
+int launch_factor_prep_multi(const FactorPrepJobs& jobs, hipStream_t stream);
 int launch_factor_prep(const void* in, int in_dtype, int64_t R_in, int64_t C_in, bool transpose,
                        bf16_t* out, int64_t R_out, int64_t C_out, int64_t num_experts, hipStream_t stream);
 

@@ -50,6 +50,32 @@ int launch_factor_prep(const void* in, int in_dtype, int64_t R_in, int64_t C_in,
     return XQ_OK;
 }
 
+// Two or three dense factor conversions in one launch (blockIdx.y = job): the linear entry points prepare both
+// factors of a call together, which matters where a step is a dozen short launches.
+__global__ void __launch_bounds__(256) factor_prep_multi_kernel(FactorPrepJobs j) {
+    const int k = blockIdx.y;
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t R_out = j.R_out[k], C_out = j.C_out[k], R_in = j.R_in[k], C_in = j.C_in[k];
+    if (t >= R_out * C_out) return;
+    const int64_t i = t / C_out, c = t - i * C_out;
+    const int64_t si = j.transpose[k] ? c : i, sj = j.transpose[k] ? i : c;
+    float v = 0.0f;
+    if (si < R_in && sj < C_in) {
+        const int64_t idx = si * C_in + sj;
+        v = j.in_f32 ? ((const float*)j.in[k])[idx] : bf16_to_f32(((const bf16_t*)j.in[k])[idx]);
+    }
+    j.out[k][t] = to_bf16(v);
+}
+
+int launch_factor_prep_multi(const FactorPrepJobs& j, hipStream_t stream) {
+    int64_t most = 0;
+    for (int k = 0; k < j.n; ++k) most = j.R_out[k] * j.C_out[k] > most ? j.R_out[k] * j.C_out[k] : most;
+    if (j.n == 0 || most == 0) return XQ_OK;
+    factor_prep_multi_kernel<<<dim3((unsigned)xq_cdiv(most, 256), (unsigned)j.n), 256, 0, stream>>>(j);
+    XQ_CHECK_LAUNCH("factor_prep_multi");
+    return XQ_OK;
+}
+
 // ------------------------------------------------------------------ small_nt
 struct SmallNtArgs {
     const bf16_t* In;
