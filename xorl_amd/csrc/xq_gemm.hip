@@ -315,8 +315,11 @@ extern "C" int xq_linear_fwd(const xq_weight* w, const void* x, int64_t ldx, int
         A_bf = (bf16_t*)cv.take(rp * K * 2);
         Bl = (bf16_t*)cv.take(N * rp * 2);
         su = su_out ? (bf16_t*)su_out : (bf16_t*)cv.take(M * rp * 2);
-        if ((rc = launch_factor_prep(lora_A, lora_dtype, r, K, false, A_bf, rp, K, 1, stream))) return rc;
-        if ((rc = launch_factor_prep(lora_B, lora_dtype, N, r, false, Bl, N, rp, 1, stream))) return rc;
+        FactorPrepJobs jobs{};
+        jobs.in_f32 = lora_dtype == XQ_DT_F32;
+        jobs.add(lora_A, r, K, false, A_bf, rp, K);
+        jobs.add(lora_B, N, r, false, Bl, N, rp);
+        if ((rc = launch_factor_prep_multi(jobs, stream))) return rc;
         if ((rc = launch_small_nt((const bf16_t*)x, ldx, M, K, A_bf, rp, scaling, su, nullptr, nullptr, 1, true, stream))) return rc;
     }
     // what is left of the workspace holds split-K partial sums (small row counts); without it the launch is unsplit
