@@ -148,7 +148,7 @@ def dense_module(fmt, N, K, r, alpha, seed, dev):
 
 
 def other_config(cfg: int, dev):
-    """Builds BASELINE.json configs[0], [2], [3] or [4] (or the merge pass, 5, or the NF4 variant of configs[1], 6)
+    """Builds BASELINE.json configs[0], [2], [3] or [4] (or the merge passes, 5 and 9, or the NF4 variant of configs[1], 6)
     on the device.  Returns
     (step_fn, work_per_step, unit_is_bytes, workload_text, kernel_text)."""
     lin_flops = lambda m, K, N, r: 4.0 * m * K * N + 6.0 * m * r * (K + N)
@@ -255,6 +255,30 @@ def other_config(cfg: int, dev):
                 "merge pass (not a BASELINE config): decode + LoRA update + re-encode (block_fp8 -> block_fp8) and "
                 "decode + update -> bf16, for gate/up [12288,4096] and down [4096,12288], r=32",
                 "merge_kernel<fp8> (fused decode + low-rank update + re-quantise / publish)")
+    if cfg == 9:
+        # not a BASELINE config: the nvfp4 merge / re-quantise pass over configs[2]'s four weights (r = 16): tensor amax
+        # of the merged weight, re-encode against it, and the bf16 publish
+        from xorl_amd.functional import merge_amax, merge_dense, merge_requant_nvfp4
+
+        mods = [dense_module("nvfp4", N, K, 16, 32, 120 + i, dev) for i, (N, K) in
+                enumerate(((8192, 5120), (1024, 5120), (1024, 5120), (5120, 8192)))]
+        total = 0.0
+        for m in mods:
+            nk = m.out_features * m.in_features
+            packed = nk / 2 + nk / 16
+            total += packed + 2 * packed + (packed + 2 * nk)       # amax pass reads; requant reads + writes; publish
+
+        def step():
+            with torch.no_grad():
+                for m in mods:
+                    qw = m._quant_weight()
+                    amax = merge_amax(qw, m.lora_A, m.lora_B, 16, 2.0)
+                    merge_requant_nvfp4(qw, m.lora_A, m.lora_B, 16, 2.0, amax)
+                    merge_dense(qw, m.lora_A, m.lora_B, 16, 2.0, torch.bfloat16)
+        return (step, total, True,
+                "nvfp4 merge pass (not a BASELINE config): tensor amax of decode + LoRA update, re-encode (nvfp4 -> nvfp4) "
+                "and decode + update -> bf16, for q [8192,5120], k/v [1024,5120], o [5120,8192], r=16",
+                "merge_kernel<nvfp4> (fused decode + low-rank update + amax / re-quantise / publish)")
     if cfg == 6:
         # not a BASELINE config: configs[1]'s three projections held as NF4 (group 64, fp32 absmax scales)
         Mtok = 8192

@@ -173,6 +173,24 @@ int xq_merge_requant_fp8(const xq_weight* w, const void* lora_A, const void* lor
                          float scaling, void* packed_out, float* scales_out, void* workspace,
                          int64_t workspace_bytes, void* stream);
 
+/* nvfp4 counterpart, in two launches because the scales hang on a tensor-wide
+ * quantity (qlora/modules/nvfp4_linear.py:126-139 with nvfp4_quantize,
+ * ops/quantize/nvfp4_quantize.py:25-60,102-154).  The merged values are those
+ * xq_merge_dense writes as bf16.
+ *   xq_merge_amax: amax_out[0] = max |W'| over the matrix (any format), which
+ *     the module blends into its running amax (`_ema_amax.lerp_`).
+ *   xq_merge_requant_nvfp4: with global_amax[0] (device memory) as the tensor
+ *     amax, per 16-element block: codes = e2m1(clamp(W' * (6 / amax_b), +-6)),
+ *     block scale = e4m3(amax_b / global_amax * 448); global_scale_out[0] =
+ *     global_amax / 6 / 448.  codes_out [N, K/2] and block_scales_out
+ *     [N, K/16] may be the weight's own buffers when its block scales are stored
+ *     as e4m3; global_scale_out must be other memory than w->global_scale. */
+int xq_merge_amax(const xq_weight* w, const void* lora_A, const void* lora_B, int lora_dtype, int r, float scaling,
+                  float* amax_out, void* workspace, int64_t workspace_bytes, void* stream);
+int xq_merge_requant_nvfp4(const xq_weight* w, const void* lora_A, const void* lora_B, int lora_dtype, int r,
+                           float scaling, const float* global_amax, void* codes_out, void* block_scales_out,
+                           float* global_scale_out, void* workspace, int64_t workspace_bytes, void* stream);
+
 /* ---- SwiGLU between gate/up and down ------------------------------------
  * Replaces fused_silu_and_mul (ops/fused_silu_and_mul.py:22-60 and its
  * backward): h = bf16(silu_fp32(gate)) * up, two roundings.  With row_w

@@ -110,6 +110,47 @@ def test_merge_requant_fp8(hip_device, N, K, r):
     assert R.max_rel_err(w_new, merged) <= 2 ** -4
 
 
+@pytest.mark.parametrize("N,K,r", [(384, 256, 0), (384, 256, 16), (200, 320, 32), (1024, 512, 64)])
+def test_merge_requant_nvfp4(hip_device, N, K, r):
+    """Fused nvfp4 merge + re-quantise: the tensor amax pass and the encode pass against the oracle's C quantizer
+    applied to the merged values the publish kernel writes (same decode, same update), byte for byte: codes, e4m3
+    block scales and the global scale; then the module method (running amax, scale convention, LoRA reset)."""
+    from xorl_amd.functional import merge_amax, merge_dense, merge_requant_nvfp4
+
+    m, w_ref = make_dense_module("nvfp4", N, K, max(r, 8), 4 * max(r, 8), seed=N + 3 * K, device=hip_device)
+    with torch.no_grad():
+        m.lora_A.mul_(8.0)
+        m.lora_B.mul_(8.0)
+        if r == 0:
+            m.lora_B.zero_()                      # the module below then merges a zero update as well
+    s = m._active_scaling()
+    qw = m._quant_weight()
+    merged = merge_dense(qw, m.lora_A, m.lora_B, r, s, torch.bfloat16).cpu()          # bf16(bf16(deq) + bf16(delta))
+    if r == 0:
+        assert torch.equal(merged, w_ref) or bool(((merged.float() == 0) & (w_ref.float() == 0))[merged != w_ref].all())
+    fresh = merge_amax(qw, m.lora_A, m.lora_B, r, s)
+    assert fresh.shape == (1,) and fresh.item() == merged.float().abs().max().item()
+    gamax = torch.tensor([0.9 * m._ema_amax.item() + 0.1 * fresh.item()])
+    codes, bscales, gscale = merge_requant_nvfp4(qw, m.lora_A, m.lora_B, r, s, gamax.to(hip_device))
+    want_codes, want_bs, want_g = C.nvfp4_quantize_flat(merged.float().numpy(), 16, global_amax=gamax.item())
+    assert np.array_equal(codes.cpu().numpy(), np.asarray(want_codes).reshape(-1))
+    assert np.array_equal(bscales.cpu().view(torch.uint8).numpy(), np.asarray(want_bs).reshape(-1).view(np.uint8))
+    assert np.float32(gscale.item()) == np.float32(np.asarray(want_g).reshape(-1)[0])
+    # the module method
+    ema0 = m._ema_amax.clone()
+    # (decay 1: the running amax jumps to the fresh one -- with this test's exaggerated update a slowly moving
+    # amax would leave the block scales saturated, which is the recipe's behaviour, not the kernel's)
+    m.merge_weights(ema_decay=1.0)
+    assert torch.count_nonzero(m.lora_B) == 0 and not torch.all(m.lora_A == 0)
+    want_ema = torch.lerp(ema0.cpu(), fresh.cpu(), 1.0)
+    assert abs(m._ema_amax.item() - want_ema.item()) <= 1e-6 * want_ema.item()
+    assert torch.equal(m._read_packed_weight_uint8().reshape(-1).cpu(), codes.cpu())
+    gs_new = m._recover_tensor(m.weight_global_scale, m._scale_dtypes["weight_global_scale"]).item()
+    assert abs(gs_new - m._ema_amax.item() / (6.0 * 448.0)) / gs_new < 1e-6
+    w_new = m._dequantize_weight().cpu().float()
+    assert (w_new - merged.float()).abs().mean() / merged.float().abs().mean() < 0.15    # e2m1 round trip
+
+
 def test_merge_errors(hip_device):
     from xorl_amd import _C
     from xorl_amd.functional import merge_requant_fp8

@@ -43,11 +43,26 @@ struct MergeArgs {
     const bf16_t* Bl;    // padded to a multiple of 128 ([Npad][r_pad], zero beyond N and r), and of A transposed
     const bf16_t* Ah;    // ([Kpad][r_pad], row = k)
     const bf16_t* Al;
-    int32_t mode;        // 0: bf16 out (publish arithmetic), 1: fp32 out, 2: block-fp8 requantise
+    int32_t mode;        // 0: bf16 out (publish arithmetic), 1: fp32 out, 2: block-fp8 requantise,
+                         // 3: absmax of the mode-0 values only, 4: nvfp4 requantise of the mode-0 values
     void* out;           // mode 0/1: [N, K]
     uint8_t* packed_out; // mode 2: [N, K] e4m3 bytes    } both may alias the inputs: a block reads its tile and its
     float* scales_out;   // mode 2: [ceil(N/128), ceil(K/128)] } scale before it writes them, and touches no other
+    float* amax_out;     // mode 3: one float, zeroed before the launch; receives max |value| over the matrix
+    const float* gamax;  // mode 4: the tensor-level amax the scales are derived from (one float on the device)
+    uint8_t* codes_out;  // mode 4: [N, K/2] e2m1 code pairs  } may alias the inputs (tile-local, read before written);
+    uint8_t* bscale_out; // mode 4: [N, K/16] e4m3 block scales } the global scale output may not
+    float* gscale_out;   // mode 4: one float
 };
+
+// e2m1 code of a value already scaled into [-6, 6] (ops/quantize/fp4_codec.py:12-19: ties go up in magnitude)
+__device__ __forceinline__ uint32_t fp4_encode(float v) {
+    const float a = fabsf(v);
+    int lo = (int)(a * 2.0f + 0.5f);
+    lo = lo > 3 ? 3 : lo;
+    const int hi = 4 + (a >= 2.5f) + (a >= 3.5f) + (a >= 5.0f);
+    return (uint32_t)(a >= 1.75f ? hi : lo) + (v < 0.0f ? 8u : 0u);
+}
 
 // hi/lo bf16 split of the factors, once per call instead of once per tile: Bh/Bl[n][j] from scaling * B[n][j],
 // Ah/Al[k][j] from A[j][k] (transposed so that a tile's MFMA operand rows are contiguous 16-byte pieces).
@@ -213,7 +228,7 @@ __global__ void __launch_bounds__(512, 4) merge_kernel(MergeArgs g) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 float t;
-                if (g.mode == 0 || !FP8) t = bf16_to_f32(to_bf16(bf16_to_f32(to_bf16(v[i + e])) + bf16_to_f32(to_bf16(d[e]))));   // 4-bit decoders return bf16
+                if (g.mode == 0 || g.mode >= 3 || !FP8) t = bf16_to_f32(to_bf16(bf16_to_f32(to_bf16(v[i + e])) + bf16_to_f32(to_bf16(d[e]))));   // 4-bit decoders return bf16
                 else t = v[i + e] + d[e];
                 x[i + e] = ok ? t : 0.0f;
             }
@@ -223,6 +238,29 @@ __global__ void __launch_bounds__(512, 4) merge_kernel(MergeArgs g) {
             for (int i = 0; i < 16; ++i) {
                 m[h * 16 + i] = x[i];
                 amax = fmaxf(amax, fabsf(x[i]));
+            }
+        } else if (g.mode == 3) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) amax = fmaxf(amax, fabsf(x[i]));
+        } else if (g.mode == 4) {
+            // one nvfp4 block per run (ops/quantize/nvfp4_quantize.py:25-60,102-111): codes against the raw block
+            // amax, block scale = e4m3(amax / global amax * 448)
+            if (ok) {
+                float bmax = 0.0f;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) bmax = fmaxf(bmax, fabsf(x[i]));
+                bmax = fmaxf(bmax, 1e-12f);
+                const float q = 6.0f / bmax;
+                uint32_t lo = 0, hi = 0;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    lo |= fp4_encode(__builtin_amdgcn_fmed3f(x[i] * q, -6.0f, 6.0f)) << (4 * i);
+                    hi |= fp4_encode(__builtin_amdgcn_fmed3f(x[8 + i] * q, -6.0f, 6.0f)) << (4 * i);
+                }
+                *(u32x2*)(g.codes_out + ((n * g.K + k) >> 1)) = u32x2{lo, hi};
+                const float gm = fmaxf(g.gamax[0], 1e-12f);
+                const float bs = __builtin_amdgcn_fmed3f(bmax / gm * 448.0f, -448.0f, 448.0f);
+                g.bscale_out[(n * g.K + k) >> 4] = (uint8_t)(__builtin_amdgcn_cvt_pk_fp8_f32(bs, 0.0f, 0u, false) & 0xffu);
             }
         } else if (ok) {
             if (g.mode == 0) {
@@ -239,7 +277,23 @@ __global__ void __launch_bounds__(512, 4) merge_kernel(MergeArgs g) {
             }
         }
     }
-    if (!REQ) return;
+    if (!REQ) {
+        if (g.mode == 3) {       // tile absmax -> one atomic per block (values are non-negative: integer order = float order)
+#pragma unroll
+            for (int off = 32; off >= 1; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+            if (lane == 0) sh_amax[wave] = amax;
+            __syncthreads();
+            if (tid == 0) {
+                float t = 0.0f;
+                for (int i = 0; i < 8; ++i) t = fmaxf(t, sh_amax[i]);
+                atomicMax((unsigned int*)g.amax_out, __float_as_uint(t));
+            }
+        } else if (g.mode == 4 && tid == 0 && blockIdx.x == 0 && blockIdx.y == 0) {
+            // global scale = amax / 6 / 448 in the quantizer's operation order
+            g.gscale_out[0] = fmaxf(g.gamax[0], 1e-12f) * (1.0f / 6.0f) / 448.0f;
+        }
+        return;
+    }
     // ---- 3b. block absmax -> new scale -> e4m3 bytes
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
@@ -279,7 +333,7 @@ using namespace xq;
 static double merge_bytes(const xq_weight* w, int mode) {
     const double n = (double)w->rows * w->cols;
     const double in = (double)xq_packed_bytes_per_expert(w) + (double)xq_scale_bytes_per_expert(w);
-    return in + (mode == 0 ? 2.0 * n : mode == 1 ? 4.0 * n : in);
+    return in + (mode == 0 ? 2.0 * n : mode == 1 ? 4.0 * n : mode == 3 ? 0.0 : in);
 }
 
 template <int FMT, int RP, bool REQ>
@@ -318,9 +372,17 @@ static int64_t merge_ws_bytes(int64_t N, int64_t K, int r) {
 
 extern "C" int64_t xq_merge_workspace_bytes(int64_t N, int64_t K, int r) { return merge_ws_bytes(N, K, r); }
 
+struct Nvfp4Out {      // outputs of modes 3 and 4
+    float* amax_out = nullptr;
+    const float* gamax = nullptr;
+    uint8_t* codes_out = nullptr;
+    uint8_t* bscale_out = nullptr;
+    float* gscale_out = nullptr;
+};
+
 static int launch_merge(const xq_weight* w, const void* A, const void* B, int lora_dtype, int r, float scaling, int mode,
                         void* out, void* packed_out, float* scales_out, void* workspace, int64_t workspace_bytes,
-                        hipStream_t stream, const char* who) {
+                        hipStream_t stream, const char* who, const Nvfp4Out& nv = Nvfp4Out()) {
     int rc = xq_validate_weight(w, who);
     if (rc) return rc;
     XQ_REQUIRE(w->num_experts == 1, "%s: takes a single matrix", who);
@@ -337,6 +399,7 @@ static int launch_merge(const xq_weight* w, const void* A, const void* B, int lo
     g.N = (int32_t)w->rows; g.K = (int32_t)w->cols;
     g.A = A; g.B = B; g.lora_f32 = lora_dtype == XQ_DT_F32; g.r = r; g.r_pad = r <= 0 ? 0 : ((r + 15) / 16) * 16;
     g.scaling = scaling; g.mode = mode; g.out = out; g.packed_out = (uint8_t*)packed_out; g.scales_out = scales_out;
+    g.amax_out = nv.amax_out; g.gamax = nv.gamax; g.codes_out = nv.codes_out; g.bscale_out = nv.bscale_out; g.gscale_out = nv.gscale_out;
     const int64_t npad = xq_cdiv(w->rows, MG_T) * MG_T, kpad = xq_cdiv(w->cols, MG_T) * MG_T;
     g.Bh = g.Bl = g.Ah = g.Al = nullptr;
     if (g.r_pad > 0) {
@@ -376,4 +439,29 @@ extern "C" int xq_merge_requant_fp8(const xq_weight* w, const void* lora_A, cons
     XQ_REQUIRE(packed_out && scales_out && xq_aligned(packed_out, 16), "xq_merge_requant_fp8: NULL or misaligned output");
     return launch_merge(w, lora_A, lora_B, lora_dtype, r, scaling, 2, nullptr, packed_out, scales_out, workspace, workspace_bytes,
                         (hipStream_t)stream, "xq_merge_requant_fp8");
+}
+
+extern "C" int xq_merge_amax(const xq_weight* w, const void* lora_A, const void* lora_B, int lora_dtype, int r, float scaling,
+                             float* amax_out, void* workspace, int64_t workspace_bytes, void* stream) {
+    XQ_REQUIRE(amax_out, "xq_merge_amax: amax_out is NULL");
+    int rc = launch_zero_fill(amax_out, 4, (hipStream_t)stream);
+    if (rc) return rc;
+    Nvfp4Out nv;
+    nv.amax_out = amax_out;
+    return launch_merge(w, lora_A, lora_B, lora_dtype, r, scaling, 3, nullptr, nullptr, nullptr, workspace, workspace_bytes,
+                        (hipStream_t)stream, "xq_merge_amax", nv);
+}
+
+extern "C" int xq_merge_requant_nvfp4(const xq_weight* w, const void* lora_A, const void* lora_B, int lora_dtype, int r,
+                                      float scaling, const float* global_amax, void* codes_out, void* block_scales_out,
+                                      float* global_scale_out, void* workspace, int64_t workspace_bytes, void* stream) {
+    XQ_REQUIRE(w && w->format == XQ_FMT_NVFP4 && w->group == 16, "xq_merge_requant_nvfp4: the weight must be nvfp4 with 16-element blocks");
+    XQ_REQUIRE(global_amax && codes_out && block_scales_out && global_scale_out && xq_aligned(codes_out, 8),
+               "xq_merge_requant_nvfp4: NULL or misaligned output");
+    XQ_REQUIRE((const void*)global_scale_out != (const void*)w->global_scale,
+               "xq_merge_requant_nvfp4: the new global scale may not overwrite the one the kernel decodes with");
+    Nvfp4Out nv;
+    nv.gamax = global_amax; nv.codes_out = (uint8_t*)codes_out; nv.bscale_out = (uint8_t*)block_scales_out; nv.gscale_out = global_scale_out;
+    return launch_merge(w, lora_A, lora_B, lora_dtype, r, scaling, 4, nullptr, nullptr, nullptr, workspace, workspace_bytes,
+                        (hipStream_t)stream, "xq_merge_requant_nvfp4", nv);
 }

@@ -344,3 +344,45 @@ def merge_requant_fp8(qw: QuantWeight, lora_A: Optional[Tensor], lora_B: Optiona
                                            packed_out.data_ptr(), scales_out.data_ptr(), ws.data_ptr(), ws_bytes,
                                            _C.stream_ptr(dev)))
     return packed_out, scales_out
+
+
+def merge_amax(qw: QuantWeight, lora_A: Optional[Tensor], lora_B: Optional[Tensor], r: int, scaling: float) -> Tensor:
+    """max |bf16(bf16(deq(W)) + bf16(scaling * B @ A))| over the matrix, fp32 [1]: the fresh tensor amax an nvfp4
+    module blends into its running one before it re-quantises (qlora/modules/nvfp4_linear.py:126-139), without
+    materialising the merged weight."""
+    _C.require_hip(qw.packed, lora_A, lora_B)
+    dev = qw.packed.device
+    A = lora_A[:r].contiguous() if r > 0 else None
+    B = lora_B[:, :r].contiguous() if r > 0 else None
+    out = torch.empty(1, dtype=torch.float32, device=dev)
+    ws_bytes = _C.lib().xq_merge_workspace_bytes(qw.rows, qw.cols, r)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    w = qw.c()
+    _C.check(_C.lib().xq_merge_amax(ctypes.byref(w), _C.ptr(A), _C.ptr(B), _lora_dt(A), r, float(scaling), out.data_ptr(),
+                                    ws.data_ptr(), ws_bytes, _C.stream_ptr(dev)))
+    return out
+
+
+def merge_requant_nvfp4(qw: QuantWeight, lora_A: Optional[Tensor], lora_B: Optional[Tensor], r: int, scaling: float,
+                        global_amax: Tensor) -> Tuple[Tensor, Tensor, Tensor]:
+    """nvfp4 only: nvfp4_quantize(deq(W) + scaling * B @ A, global_amax) in one pass over the packed bytes
+    (merge_weights + _quantize_and_store, qlora/modules/nvfp4_linear.py:126-139).  Returns (codes uint8 [N*K/2],
+    e4m3 block scales [N*K/16], fp32 global scale [1]) in fresh tensors."""
+    _C.require_hip(qw.packed, lora_A, lora_B)
+    if qw.fmt != "nvfp4":
+        raise _C.XqError(f"merge_requant_nvfp4: the weight must be nvfp4, got {qw.fmt}")
+    dev = qw.packed.device
+    A = lora_A[:r].contiguous() if r > 0 else None
+    B = lora_B[:, :r].contiguous() if r > 0 else None
+    n = qw.rows * qw.cols
+    codes = torch.empty(n // 2, dtype=torch.uint8, device=dev)
+    bscales = torch.empty(n // 16, dtype=torch.uint8, device=dev)
+    gscale = torch.empty(1, dtype=torch.float32, device=dev)
+    gamax = global_amax.to(device=dev, dtype=torch.float32).reshape(1).contiguous()
+    ws_bytes = _C.lib().xq_merge_workspace_bytes(qw.rows, qw.cols, r)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    w = qw.c()
+    _C.check(_C.lib().xq_merge_requant_nvfp4(ctypes.byref(w), _C.ptr(A), _C.ptr(B), _lora_dt(A), r, float(scaling),
+                                             gamax.data_ptr(), codes.data_ptr(), bscales.data_ptr(), gscale.data_ptr(),
+                                             ws.data_ptr(), ws_bytes, _C.stream_ptr(dev)))
+    return codes, bscales.view(torch.float8_e4m3fn), gscale

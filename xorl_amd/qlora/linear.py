@@ -565,6 +565,32 @@ class NvFP4QLoRALinear(QLoRALinear):
         eff = self._recover_tensor(s, sdt).float() * g
         return (0.5 * eff.reshape(self.out_features, -1).repeat_interleave(16, 1)).contiguous()
 
+    def merge_weights(self, ema_decay: float = 0.1) -> None:
+        """Decode, add the LoRA update, blend the fresh tensor amax into the running one and re-encode with it, in
+        two fused passes over the packed bytes (nvfp4_linear.py:126-139); sharded (DTensor) state and ranks beyond
+        the fused kernels' take the generic path."""
+        from ..functional import merge_amax, merge_requant_nvfp4
+
+        if (_is_dtensor(self.packed_weight_f32) or _is_dtensor(self.lora_A) or self.active_r > MAX_FUSED_RANK
+                or not self.packed_weight_f32.is_cuda):
+            return super().merge_weights(ema_decay)
+        with torch.no_grad():
+            qw = self._quant_weight()
+            fresh = merge_amax(qw, self.lora_A, self.lora_B, self.active_r, self._active_scaling())
+            if self._ema_amax is not None:
+                self._ema_amax.lerp_(fresh.to(self._ema_amax.device), ema_decay)
+            else:
+                self._ema_amax = fresh
+            codes, bscales, gscale = merge_requant_nvfp4(qw, self.lora_A, self.lora_B, self.active_r,
+                                                         self._active_scaling(), self._ema_amax)
+            self._write_packed_weight(codes)
+            self._scale_dtypes = {"weight_block_scales": bscales.dtype, "weight_global_scale": gscale.dtype}
+            self.weight_block_scales = self._to_uint8(bscales)
+            self.weight_global_scale = self._to_uint8(gscale)
+            self._aqn_step_cache = None
+            nn.init.kaiming_uniform_(self.lora_A, a=math.sqrt(5))
+            self.lora_B.zero_()
+
     def _requantize_merged(self, merged: Tensor, ema_decay: float) -> None:
         fresh = merged.float().abs().max().reshape(1)
         if self._ema_amax is not None:
