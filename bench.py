@@ -48,6 +48,7 @@ MEASURED_TRAFFIC_BYTES = {
                            # the fp32 partial tiles written and read back: 23.3 MiB of it are algorithmic)
     6: 737.0 * 2 ** 20,    # gemm_256_kernel<nf4>: mean of the forward and dgrad launches
     7: 889.1 * 2 ** 20,    # gemm_256_kernel<nvfp4 GKN, grouped>: mean over the 6 launches of a step
+    9: 59.0 * 2 ** 20,     # merge_prep_kernel + merge_kernel<nvfp4>: mean per call over amax / re-quantise / publish of the four weights
     5: 134.4 * 2 ** 20,    # merge_prep_kernel + merge_kernel<fp8>: mean per call (re-quantise 96 MiB, publish 144 MiB algorithmic)
 }
 
