@@ -191,6 +191,16 @@ int xq_merge_requant_nvfp4(const xq_weight* w, const void* lora_A, const void* l
                            float scaling, const float* global_amax, void* codes_out, void* block_scales_out,
                            float* global_scale_out, void* workspace, int64_t workspace_bytes, void* stream);
 
+/* NF4 counterpart (qlora/modules/nf4_linear.py merge_weights with nf4_quantize,
+ * ops/quantize/nf4_quantize.py:20-56): one pass; per 64-element group
+ * scale = max(absmax, 1e-12) (fp32), code = nearest-level code of
+ * clamp(W' / scale, +-1) by the midpoint rule.  The weight must hold fp32
+ * scales per 64 elements; in_features % 64 == 0.  codes_out [N, K/2] and
+ * scales_out [N*K/64] may be the weight's own buffers. */
+int xq_merge_requant_nf4(const xq_weight* w, const void* lora_A, const void* lora_B, int lora_dtype, int r,
+                         float scaling, void* codes_out, float* scales_out, void* workspace,
+                         int64_t workspace_bytes, void* stream);
+
 /* ---- SwiGLU between gate/up and down ------------------------------------
  * Replaces fused_silu_and_mul (ops/fused_silu_and_mul.py:22-60 and its
  * backward): h = bf16(silu_fp32(gate)) * up, two roundings.  With row_w

@@ -151,6 +151,32 @@ def test_merge_requant_nvfp4(hip_device, N, K, r):
     assert (w_new - merged.float()).abs().mean() / merged.float().abs().mean() < 0.15    # e2m1 round trip
 
 
+@pytest.mark.parametrize("N,K,r", [(384, 256, 0), (200, 320, 16), (1024, 512, 64)])
+def test_merge_requant_nf4(hip_device, N, K, r):
+    """Fused NF4 merge + re-quantise against the oracle's C quantizer applied to the merged values the publish
+    kernel writes: codes and fp32 group scales byte for byte; then the module method, in place."""
+    from xorl_amd.functional import merge_dense, merge_requant_nf4
+
+    m, w_ref = make_dense_module("nf4", N, K, max(r, 8), 4 * max(r, 8), seed=2 * N + K, device=hip_device)
+    with torch.no_grad():
+        m.lora_A.mul_(8.0)
+        m.lora_B.mul_(8.0)
+        if r == 0:
+            m.lora_B.zero_()
+    s = m._active_scaling()
+    qw = m._quant_weight()
+    merged = merge_dense(qw, m.lora_A, m.lora_B, r, s, torch.bfloat16).cpu()
+    codes, scales = merge_requant_nf4(qw, m.lora_A, m.lora_B, r, s)
+    want_codes, want_scales = C.nf4_quantize_flat(merged.float().numpy(), 64)
+    assert np.array_equal(codes.cpu().numpy(), np.asarray(want_codes).reshape(-1))
+    assert np.array_equal(scales.cpu().numpy().view(np.uint32), np.asarray(want_scales).reshape(-1).view(np.uint32))
+    m.merge_weights()
+    assert torch.count_nonzero(m.lora_B) == 0
+    assert torch.equal(m._read_packed_weight_uint8().reshape(-1).cpu(), codes.cpu())
+    w_new = m._dequantize_weight().cpu().float()
+    assert (w_new - merged.float()).abs().mean() / merged.float().abs().mean() < 0.10
+
+
 def test_merge_errors(hip_device):
     from xorl_amd import _C
     from xorl_amd.functional import merge_requant_fp8

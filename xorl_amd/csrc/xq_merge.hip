@@ -44,16 +44,30 @@ struct MergeArgs {
     const bf16_t* Ah;    // ([Kpad][r_pad], row = k)
     const bf16_t* Al;
     int32_t mode;        // 0: bf16 out (publish arithmetic), 1: fp32 out, 2: block-fp8 requantise,
-                         // 3: absmax of the mode-0 values only, 4: nvfp4 requantise of the mode-0 values
+                         // 3: absmax of the mode-0 values only, 4 / 5: nvfp4 / nf4 requantise of the mode-0 values
     void* out;           // mode 0/1: [N, K]
     uint8_t* packed_out; // mode 2: [N, K] e4m3 bytes    } both may alias the inputs: a block reads its tile and its
     float* scales_out;   // mode 2: [ceil(N/128), ceil(K/128)] } scale before it writes them, and touches no other
     float* amax_out;     // mode 3: one float, zeroed before the launch; receives max |value| over the matrix
     const float* gamax;  // mode 4: the tensor-level amax the scales are derived from (one float on the device)
-    uint8_t* codes_out;  // mode 4: [N, K/2] e2m1 code pairs  } may alias the inputs (tile-local, read before written);
+    uint8_t* codes_out;  // mode 4 / 5: [N, K/2] code pairs     } may alias the inputs (tile-local, read before written);
     uint8_t* bscale_out; // mode 4: [N, K/16] e4m3 block scales } the global scale output may not
     float* gscale_out;   // mode 4: one float
 };
+
+// NF4 code of a value already normalised into [-1, 1]: the number of midpoints between neighbouring levels that lie
+// strictly below it (ops/quantize/nf4_codec.py:42-64)
+__device__ __forceinline__ uint32_t nf4_encode(float v) {
+    constexpr float kMid[15] = {(float)-0.8480964004993439, (float)-0.6106329262256622, (float)-0.4599952697753906,
+                                (float)-0.3396794348955154, (float)-0.2346074059605598, (float)-0.1379117332398891,
+                                (float)-0.0455250181257725, (float)0.0397901497781277,  (float)0.1202552504837513,
+                                (float)0.2035212516784668,  (float)0.2920137718319893,  (float)0.3893125355243683,
+                                (float)0.5016634166240692,  (float)0.6427869200706482,  (float)0.8614784181118012};
+    uint32_t c = 0;
+#pragma unroll
+    for (int i = 0; i < 15; ++i) c += v > kMid[i] ? 1u : 0u;
+    return c;
+}
 
 // e2m1 code of a value already scaled into [-6, 6] (ops/quantize/fp4_codec.py:12-19: ties go up in magnitude)
 __device__ __forceinline__ uint32_t fp4_encode(float v) {
@@ -262,6 +276,25 @@ __global__ void __launch_bounds__(512, 4) merge_kernel(MergeArgs g) {
                 const float bs = __builtin_amdgcn_fmed3f(bmax / gm * 448.0f, -448.0f, 448.0f);
                 g.bscale_out[(n * g.K + k) >> 4] = (uint8_t)(__builtin_amdgcn_cvt_pk_fp8_f32(bs, 0.0f, 0u, false) & 0xffu);
             }
+        } else if (g.mode == 5) {
+            // NF4 (ops/quantize/nf4_quantize.py:20-56): a 64-element group is the four runs of four neighbouring lanes;
+            // scale = max(absmax, 1e-12), code = encode(clamp(x * (1 / scale), +-1))
+            float bmax = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) bmax = fmaxf(bmax, fabsf(x[i]));
+            bmax = fmaxf(bmax, __shfl_xor(bmax, 1, 64));
+            bmax = fmaxf(bmax, __shfl_xor(bmax, 2, 64));
+            const float sc = fmaxf(bmax, 1e-12f), inv = 1.0f / sc;
+            if (ok) {
+                uint32_t lo = 0, hi = 0;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    lo |= nf4_encode(__builtin_amdgcn_fmed3f(x[i] * inv, -1.0f, 1.0f)) << (4 * i);
+                    hi |= nf4_encode(__builtin_amdgcn_fmed3f(x[8 + i] * inv, -1.0f, 1.0f)) << (4 * i);
+                }
+                *(u32x2*)(g.codes_out + ((n * g.K + k) >> 1)) = u32x2{lo, hi};
+                if ((tid & 3) == 0) g.scales_out[(n * g.K + k) >> 6] = sc;
+            }
         } else if (ok) {
             if (g.mode == 0) {
                 bf16_t* o = (bf16_t*)g.out + n * g.K + k;
@@ -464,4 +497,16 @@ extern "C" int xq_merge_requant_nvfp4(const xq_weight* w, const void* lora_A, co
     nv.gamax = global_amax; nv.codes_out = (uint8_t*)codes_out; nv.bscale_out = (uint8_t*)block_scales_out; nv.gscale_out = global_scale_out;
     return launch_merge(w, lora_A, lora_B, lora_dtype, r, scaling, 4, nullptr, nullptr, nullptr, workspace, workspace_bytes,
                         (hipStream_t)stream, "xq_merge_requant_nvfp4", nv);
+}
+
+extern "C" int xq_merge_requant_nf4(const xq_weight* w, const void* lora_A, const void* lora_B, int lora_dtype, int r,
+                                    float scaling, void* codes_out, float* scales_out, void* workspace,
+                                    int64_t workspace_bytes, void* stream) {
+    XQ_REQUIRE(w && w->format == XQ_FMT_NF4 && w->group == 64 && w->scale_dtype == XQ_SCALE_F32 && w->cols % 64 == 0,
+               "xq_merge_requant_nf4: the weight must be NF4 with fp32 scales per 64 elements and in_features %% 64 == 0");
+    XQ_REQUIRE(codes_out && scales_out && xq_aligned(codes_out, 8), "xq_merge_requant_nf4: NULL or misaligned output");
+    Nvfp4Out nv;
+    nv.codes_out = (uint8_t*)codes_out;
+    return launch_merge(w, lora_A, lora_B, lora_dtype, r, scaling, 5, nullptr, nullptr, scales_out, workspace, workspace_bytes,
+                        (hipStream_t)stream, "xq_merge_requant_nf4", nv);
 }

@@ -386,3 +386,28 @@ def merge_requant_nvfp4(qw: QuantWeight, lora_A: Optional[Tensor], lora_B: Optio
                                              gamax.data_ptr(), codes.data_ptr(), bscales.data_ptr(), gscale.data_ptr(),
                                              ws.data_ptr(), ws_bytes, _C.stream_ptr(dev)))
     return codes, bscales.view(torch.float8_e4m3fn), gscale
+
+
+def merge_requant_nf4(qw: QuantWeight, lora_A: Optional[Tensor], lora_B: Optional[Tensor], r: int, scaling: float,
+                      codes_out: Optional[Tensor] = None, scales_out: Optional[Tensor] = None) -> Tuple[Tensor, Tensor]:
+    """NF4 only: nf4_quantize(deq(W) + scaling * B @ A) in one pass over the packed bytes (merge_weights +
+    _quantize_and_store of qlora/modules/nf4_linear.py).  Returns (codes uint8 [N*K/2], fp32 scales [N*K/64]); pass
+    the weight's own buffers to update in place."""
+    _C.require_hip(qw.packed, lora_A, lora_B)
+    if qw.fmt != "nf4":
+        raise _C.XqError(f"merge_requant_nf4: the weight must be nf4, got {qw.fmt}")
+    dev = qw.packed.device
+    A = lora_A[:r].contiguous() if r > 0 else None
+    B = lora_B[:, :r].contiguous() if r > 0 else None
+    n = qw.rows * qw.cols
+    if codes_out is None:
+        codes_out = torch.empty(n // 2, dtype=torch.uint8, device=dev)
+    if scales_out is None:
+        scales_out = torch.empty(n // 64, dtype=torch.float32, device=dev)
+    ws_bytes = _C.lib().xq_merge_workspace_bytes(qw.rows, qw.cols, r)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    w = qw.c()
+    _C.check(_C.lib().xq_merge_requant_nf4(ctypes.byref(w), _C.ptr(A), _C.ptr(B), _lora_dt(A), r, float(scaling),
+                                           codes_out.data_ptr(), scales_out.data_ptr(), ws.data_ptr(), ws_bytes,
+                                           _C.stream_ptr(dev)))
+    return codes_out, scales_out

@@ -723,6 +723,24 @@ class NF4QLoRALinear(QLoRALinear):
         self.weight_scales = self._to_uint8(scales.reshape(self.out_features, -1))
         self._aqn_step_cache = None
 
+    def merge_weights(self, ema_decay: float = 0.1) -> None:
+        """Decode, add the LoRA update and re-encode with fresh group scales in one fused pass over the bytes;
+        sharded (DTensor) state, other group sizes and ranks beyond the fused kernels' take the generic path."""
+        from ..functional import merge_requant_nf4
+
+        if (_is_dtensor(self.packed_weight_f32) or _is_dtensor(self.lora_A) or self.active_r > MAX_FUSED_RANK
+                or not self.packed_weight_f32.is_cuda or self.quant_group_size != 64 or self.in_features % 64
+                or self._scale_dtypes.get("weight_scales") != torch.float32):
+            return super().merge_weights(ema_decay)
+        with torch.no_grad():
+            codes, scales = merge_requant_nf4(self._quant_weight(), self.lora_A, self.lora_B, self.active_r,
+                                              self._active_scaling())
+            self._write_packed_weight(codes)
+            self.weight_scales = self._to_uint8(scales.reshape(self.out_features, -1))
+            self._aqn_step_cache = None
+            nn.init.kaiming_uniform_(self.lora_A, a=math.sqrt(5))
+            self.lora_B.zero_()
+
     def _quant_weight(self) -> QuantWeight:
         return QuantWeight("nf4", _C.XQ_LAYOUT_FLAT, self._read_packed_weight_uint8(), self.weight_scales,
                            self._scale_dtypes["weight_scales"], self.out_features, self.in_features,
