@@ -133,6 +133,25 @@ int xq_linear_fwd(const xq_weight* w, const void* x, int64_t ldx, int64_t M,
                   const void* bias_bf16, void* y, int64_t ldy, void* su_out,
                   void* workspace, int64_t workspace_bytes, void* stream);
 
+/* xq_linear_fwd for callers that cannot allocate device memory or be handed a
+ * workspace: code under HIP-graph capture, tight rollout / serving loops,
+ * harnesses that forbid allocation.  No counterpart in the reference (its
+ * forward allocates through torch).  Same arguments and results as
+ * xq_linear_fwd with su_out == NULL (bit-identical: the same kernels run), but
+ * the scratch is a buffer of XQ_STATIC_SCRATCH_BYTES built into the library's
+ * code object, one copy per device, resolved once per device at the first call
+ * made with that device current.  The call allocates and frees nothing.
+ * Shapes whose xq_linear_workspace_bytes(M, N, K, r) exceeds the buffer are
+ * rejected with XQ_ERR_ARG.  All calls on one device share that device's
+ * buffer: calls that overlap in time on one device (two streams, two host
+ * threads) race; calls on one stream, or ordered by events, do not.  Nothing in
+ * the buffer has to start at zero, so nothing is cleared between calls. */
+#define XQ_STATIC_SCRATCH_BYTES (32ll << 20)
+int64_t xq_static_scratch_bytes(void);
+int xq_linear_fwd_static(const xq_weight* w, const void* x, int64_t ldx, int64_t M,
+                         const void* lora_A, const void* lora_B, int lora_dtype, int r, float scaling,
+                         const void* bias_bf16, void* y, int64_t ldy, void* stream);
+
 /* dx[M,K] = dy . deq(W) + s * (dy . B) . A   (bf16)
  * dA[r,K] = s * (dy . B)^T . x               (fp32, overwritten)
  * dB[N,r] = s * dy^T . (x . A^T)             (fp32, overwritten)

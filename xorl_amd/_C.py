@@ -57,6 +57,9 @@ _SIGNATURES = {
     "xq_linear_workspace_bytes": (_I64, [_I64, _I64, _I64, _INT]),
     # w, x, ldx, M, A, B, lora_dtype, r, scaling, bias, y, ldy, su_out, ws, ws_bytes, stream
     "xq_linear_fwd": (_INT, [_W, _P, _I64, _I64, _P, _P, _INT, _INT, _F, _P, _P, _I64, _P, _P, _I64, _P]),
+    "xq_static_scratch_bytes": (_I64, []),
+    # w, x, ldx, M, A, B, lora_dtype, r, scaling, bias, y, ldy, stream
+    "xq_linear_fwd_static": (_INT, [_W, _P, _I64, _I64, _P, _P, _INT, _INT, _F, _P, _P, _I64, _P]),
     # w, x, ldx, dy, lddy, M, A, B, lora_dtype, r, scaling, su, dx, lddx, dA, dB, ws, ws_bytes, stream
     "xq_linear_bwd": (_INT, [_W, _P, _I64, _P, _I64, _I64, _P, _P, _INT, _INT, _F, _P, _P, _I64, _P, _P, _P, _I64,
                              _P]),

@@ -2,6 +2,7 @@
 #include "xq_gemm_tile.h"
 #include "xq_gemm_256.h"
 #include <stdlib.h>
+#include <mutex>
 #include "xq_lora.h"
 
 namespace xq {
@@ -326,6 +327,64 @@ extern "C" int xq_linear_fwd(const xq_weight* w, const void* x, int64_t ldx, int
     float* partial = (float*)cv.take(0);
     return launch_tile_gemm(w, true, (const bf16_t*)x, ldx, M, nullptr, nullptr, su, Bl, rp, (const bf16_t*)bias_bf16,
                             (bf16_t*)y, ldy, stream, "xq_linear_fwd", partial, partial ? workspace_bytes - cv.used : 0);
+}
+
+// ---- forward for callers that cannot allocate ------------------------------------------------------------------
+// The scratch of xq_linear_fwd (prepared LoRA panels, the [M, r_pad] intermediate, split-K partial sums) in an
+// array that is part of the loaded code object: each device the library runs on holds its own copy at its own
+// address until the process ends.  Host code reaches it only through the address hipGetSymbolAddress returns with
+// that device current; the array's name is a host-side handle, never a device address.
+static __device__ __align__(256) unsigned char scratch[XQ_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mu;
+void* g_scratch_ptr[kMaxDevices] = {};
+}  // namespace
+
+// device address of this device's copy of `scratch` (resolved once per device, with that device current)
+static int static_scratch(void** out, const char* who) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        xq_set_error("%s: cannot identify the current device: %s", who, hipGetErrorString(e));
+        return XQ_ERR_LAUNCH;
+    }
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) {
+            xq_set_error("%s: hipGetSymbolAddress(scratch) failed on device %d: %s", who, dev, hipGetErrorString(e));
+            return XQ_ERR_LAUNCH;
+        }
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return XQ_OK;
+}
+
+extern "C" int64_t xq_static_scratch_bytes(void) { return XQ_STATIC_SCRATCH_BYTES; }
+
+extern "C" int xq_linear_fwd_static(const xq_weight* w, const void* x, int64_t ldx, int64_t M, const void* lora_A,
+                                    const void* lora_B, int lora_dtype, int r, float scaling, const void* bias_bf16,
+                                    void* y, int64_t ldy, void* stream_) {
+    int rc = check_dense(w, "xq_linear_fwd_static");
+    if (rc) return rc;
+    XQ_REQUIRE(M >= 0, "xq_linear_fwd_static: negative row count");
+    XQ_REQUIRE(r >= 0 && r <= 64, "xq_linear_fwd_static: LoRA rank %d out of range [0, 64]", r);
+    const int64_t need = xq_linear_workspace_bytes(M, w->rows, w->cols, r);
+    XQ_REQUIRE(need <= XQ_STATIC_SCRATCH_BYTES,
+               "xq_linear_fwd_static: M=%lld, N=%lld, K=%lld, r=%d needs %lld bytes of scratch, the built-in buffer "
+               "holds %lld; use xq_linear_fwd with a caller workspace",
+               (long long)M, (long long)w->rows, (long long)w->cols, r, (long long)need,
+               (long long)XQ_STATIC_SCRATCH_BYTES);
+    void* ws = nullptr;
+    if ((rc = static_scratch(&ws, "xq_linear_fwd_static"))) return rc;
+    // nothing in the forward reads scratch it has not written in the same call (no counters, no accumulation into
+    // memory), so the previous call's contents need no clearing
+    return xq_linear_fwd(w, x, ldx, M, lora_A, lora_B, lora_dtype, r, scaling, bias_bf16, y, ldy, nullptr, ws,
+                         XQ_STATIC_SCRATCH_BYTES, stream_);
 }
 
 extern "C" int xq_linear_bwd(const xq_weight* w, const void* x, int64_t ldx, const void* dy, int64_t lddy, int64_t M,
