@@ -247,6 +247,10 @@ int xq_route_build(const int32_t* selected, int64_t n_routed, int32_t num_expert
                    int32_t* counts, int32_t* offsets, int32_t* scatter_index,
                    int32_t* tile_offsets, void* workspace, int64_t workspace_bytes, void* stream);
 
+/* An expert id outside [0, num_experts) (the reference asserts on these on the device) drops that routed copy:
+ * it is not counted, gets scatter_index -1, and the row movers below skip it -- xq_moe_scatter stores nothing for
+ * it, xq_moe_gather adds nothing, xq_moe_scatter_scalar skips it, xq_moe_gather_scalar returns 0.  offsets[E] is
+ * then smaller than n_routed and the rows [offsets[E], n_routed) of expert-ordered buffers belong to no expert. */
 /* rows_out[scatter_index[i]] = rows_in[i / topk]   (moe_scatter, group_gemm/kernel/moe.py:266-312) */
 int xq_moe_scatter(const void* in, int64_t ld_in, const int32_t* scatter_index, int64_t n_routed,
                    int32_t topk, int64_t width, void* out, int64_t ld_out, void* stream);
@@ -291,7 +295,9 @@ int xq_factor_prep(const void* in, int in_dtype, int64_t rows_in, int64_t cols_i
  *       n_rows (one output; also the gradient of a factor shared by all
  *       experts).  Both forms split the rows over blocks and add the pieces in
  *       a fixed order (deterministic), in xq_lora_wgrad_workspace_bytes() bytes
- *       of scratch (256-byte aligned, required).
+ *       of scratch (256-byte aligned, required).  row_limit (device, may be NULL) restricts the dense form to
+ *       the rows below *row_limit: offsets + E of xq_route_build, so that rows no expert owns (routed
+ *       copies whose expert id was out of range) are left out.
  * Replace the small group_gemm_same_nk / group_gemm_same_mn calls of
  * ops/moe/lora.py:601-660 and :781-960. */
 int xq_grouped_lora_down(const void* a, int64_t lda, int64_t n_rows, const int32_t* offsets,
@@ -300,7 +306,7 @@ int xq_grouped_lora_down(const void* a, int64_t lda, int64_t n_rows, const int32
 int64_t xq_lora_wgrad_workspace_bytes(int64_t n_rows, int64_t width, int r_pad);
 int xq_grouped_lora_wgrad(const void* P, int64_t ldp, int64_t p_width, const void* Q, int r_pad,
                           int r_out, int64_t n_rows, const int32_t* offsets, int32_t num_experts,
-                          int transpose_out, float* out, void* workspace, void* stream);
+                          int transpose_out, float* out, void* workspace, const int32_t* row_limit, void* stream);
 
 #ifdef __cplusplus
 }

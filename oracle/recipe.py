@@ -84,27 +84,30 @@ def silu_and_mul_recipe(gate, up):
     return act * up
 
 
-def mlp_fwd_bwd_exact(x, w_gate, w_up, w_down, loras, scaling, dy=None):
-    """SwiGLU MLP of three QLoRA linears in float64 (Qwen3MLP.forward,
-    models/transformers/qwen3/modeling_qwen3.py:60-81).  ``loras`` maps
-    'gate'/'up'/'down' to (A [r,K], B [N,r]).  Returns y and grads by autograd."""
-    X = x.double().detach().clone().requires_grad_(dy is not None)
+def mlp_fwd_bwd_exact(x, w_gate, w_up, w_down, loras, scaling, dy=None, dtype=torch.float64):
+    """SwiGLU MLP of three QLoRA linears without intermediate rounding (Qwen3MLP.forward,
+    models/transformers/qwen3/modeling_qwen3.py:60-81: down(act(gate(x)) * up(x))).  ``loras`` maps
+    'gate'/'up'/'down' to (A [r,K], B [N,r]).  Returns y and grads by autograd.
+
+    dtype=float64 is the yardstick; dtype=float32 is the same program with fp32 accumulation (its own
+    error, ~1e-6 relative, is far below the 1e-2 tolerance) for sizes float64 cannot finish in seconds."""
+    need = dy is not None
+    X = x.to(dtype).detach().clone().requires_grad_(need)
     P = {}
     for k, (A, B) in loras.items():
-        P[k] = (A.double().detach().clone().requires_grad_(dy is not None),
-                B.double().detach().clone().requires_grad_(dy is not None))
+        P[k] = (A.to(dtype).detach().clone().requires_grad_(need), B.to(dtype).detach().clone().requires_grad_(need))
 
     def lin(inp, w, key):
         A, B = P[key]
-        return inp @ w.to(torch.bfloat16).double().t() + scaling * ((inp @ A.t()) @ B.t())
+        return inp @ w.to(torch.bfloat16).to(dtype).t() + scaling * ((inp @ A.t()) @ B.t())
 
     g = lin(X, w_gate, "gate")
     u = lin(X, w_up, "up")
     h = F.silu(g) * u
     y = lin(h, w_down, "down")
     out = {"y": y.detach(), "gate": g.detach(), "up": u.detach(), "h": h.detach()}
-    if dy is not None:
-        y.backward(dy.double())
+    if need:
+        y.backward(dy.to(dtype))
         out["dx"] = X.grad
         for k, (A, B) in P.items():
             out[f"dA_{k}"], out[f"dB_{k}"] = A.grad, B.grad
@@ -199,6 +202,23 @@ def max_rel_err(got: torch.Tensor, ref: torch.Tensor) -> float:
     if denom == 0.0:
         return float((got.double() - ref).abs().max().item())
     return float((got.double() - ref).abs().max().item() / denom)
+
+
+def row_rel_err(got: torch.Tensor, ref: torch.Tensor) -> float:
+    """max over rows of  max |got_row - ref_row| / max |ref_row|  (rows = the last dimension's vectors).
+
+    Stricter than max_rel_err: a systematic error confined to rows of small magnitude (which the
+    tensor-wide maximum hides) shows up here.  Rows whose reference is all zero must be exactly zero."""
+    ref = ref.double().reshape(-1, ref.shape[-1]) if ref.dim() > 1 else ref.double().reshape(1, -1)
+    got = got.double().reshape(ref.shape)
+    err = (got - ref).abs().amax(dim=1)
+    den = ref.abs().amax(dim=1)
+    zero = den == 0
+    if bool((err[zero] != 0).any()):
+        return float("inf")
+    if bool(zero.all()):
+        return 0.0
+    return float((err[~zero] / den[~zero]).max().item())
 
 
 # ---------------------------------------------------------------------------

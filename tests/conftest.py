@@ -29,3 +29,16 @@ def tile_policy(request):
     _C.check(_C.lib().xq_set_tile_policy(int(request.param)))
     yield int(request.param)
     _C.check(_C.lib().xq_set_tile_policy(0))
+
+
+def pytest_sessionfinish(session, exitstatus):
+    """Worst tolerance metrics per test (tensor-wide and per-row), for the parity table of the design notes."""
+    import json
+
+    from tests.util_cases import PARITY_WORST
+
+    if PARITY_WORST:
+        out = os.path.join(ROOT, "gpurun_out")
+        os.makedirs(out, exist_ok=True)
+        with open(os.path.join(out, "parity_worst.json"), "w") as f:
+            json.dump({k: {"tensor": v[0], "row": v[1]} for k, v in sorted(PARITY_WORST.items())}, f, indent=1)

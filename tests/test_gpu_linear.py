@@ -6,7 +6,7 @@ import pytest
 import torch
 
 from oracle import recipe as R
-from tests.util_cases import gen, make_dense_module
+from tests.util_cases import close, gen, make_dense_module
 
 pytestmark = pytest.mark.gpu
 TOL = 1e-2
@@ -31,8 +31,7 @@ def test_dense_fwd_bwd_vs_oracle(hip_device, tile_policy, fmt, M, K, N, r):
     assert y.dtype == torch.bfloat16 and dx.dtype == torch.bfloat16
     assert dA.dtype == torch.float32 and dA.shape == (r, K) and dB.shape == (N, r)
     for name, got, ref in (("y", y, ex["y"]), ("dx", dx, ex["dx"]), ("dA", dA, ex["dA"]), ("dB", dB, ex["dB"])):
-        err = R.max_rel_err(got.cpu(), ref)
-        assert err <= TOL, f"{fmt} {name}: {err}"
+        close(got.cpu(), ref, TOL)
 
 
 @pytest.mark.parametrize("tile_policy", [0, 1, 2], indirect=True)
@@ -45,7 +44,7 @@ def test_config0_int4_full_size(hip_device, tile_policy):
     y, dx, dA, dB = _run(m, x.to(hip_device), dy.to(hip_device))
     ex = R.linear_fwd_bwd_exact(x, w_ref, m.lora_A.detach().cpu(), m.lora_B.detach().cpu(), 2.0, dy)
     for name, got, ref in (("y", y, ex["y"]), ("dx", dx, ex["dx"]), ("dA", dA, ex["dA"]), ("dB", dB, ex["dB"])):
-        assert R.max_rel_err(got.cpu(), ref) <= TOL, name
+        close(got.cpu(), ref, TOL)
     # the module's own decode is bit-exact with the oracle
     assert torch.equal(m._dequantize_weight().cpu(), w_ref)
 
@@ -107,8 +106,7 @@ def test_split_k_fwd_bwd_vs_oracle(hip_device, fmt, M, N, K, r, bias):
     ex = R.linear_fwd_bwd_exact(x, w_ref, m.lora_A.detach().cpu(), m.lora_B.detach().cpu(), m.scaling, dy,
                                 bias=m.bias.detach().cpu() if bias else None)
     for name, got, ref in (("y", y, ex["y"]), ("dx", dx, ex["dx"]), ("dA", dA, ex["dA"]), ("dB", dB, ex["dB"])):
-        err = R.max_rel_err(got.cpu(), ref)
-        assert err <= TOL, f"{fmt} {name}: {err}"
+        close(got.cpu(), ref, TOL)
     # the same call again gives the same bits (fixed summation order, no atomics)
     y2, dx2, _, _ = _run(m, x.to(hip_device), dy.to(hip_device))
     assert torch.equal(y, y2) and torch.equal(dx, dx2)
@@ -141,19 +139,19 @@ def test_invariants(hip_device):
         m.lora_B.copy_(b_saved)
     base = R.linear_fwd_bwd_exact(x.cpu(), w_ref, m.lora_A.detach().cpu(), torch.zeros(384, 16), 2.0,
                                   bias=m.bias.detach().cpu())["y"]
-    assert R.max_rel_err(y0.cpu(), base) <= TOL          # lora_B = 0 => base only (+ bias)
+    close(y0.cpu(), base, TOL)          # lora_B = 0 => base only (+ bias)
     assert not torch.equal(y, y0)
     # linearity in x of the whole op (size-independent property)
     with torch.no_grad():
         m.bias.zero_()
         a, b = m(x), m(2 * x)
-    assert R.max_rel_err(b.cpu().float(), 2 * a.cpu().float()) <= TOL
+    close(b.cpu().float(), 2 * a.cpu().float(), TOL)
     # active rank slice (set_runtime_lora_config)
     m.set_runtime_lora_config(8, 16)
     with torch.no_grad():
         y8 = m(x)
     ex8 = R.linear_fwd_bwd_exact(x.cpu(), w_ref, m.lora_A.detach().cpu()[:8], m.lora_B.detach().cpu()[:, :8], 2.0)["y"]
-    assert R.max_rel_err(y8.cpu(), ex8) <= TOL
+    close(y8.cpu(), ex8, TOL)
     with pytest.raises(ValueError):
         m.set_runtime_lora_config(0, 1)
 
@@ -189,8 +187,8 @@ def test_silu_and_mul(hip_device):
     assert (h.cpu() == ref).float().mean() > 0.99
     g64, u64 = g.double().requires_grad_(True), u.double().requires_grad_(True)
     (torch.nn.functional.silu(g64) * u64).backward(dh.double())
-    assert R.max_rel_err(gd.grad.cpu(), g64.grad) <= TOL
-    assert R.max_rel_err(ud.grad.cpu(), u64.grad) <= TOL
+    close(gd.grad.cpu(), g64.grad, TOL)
+    close(ud.grad.cpu(), u64.grad, TOL)
 
 
 @pytest.mark.parametrize("fmt,M,K,N", [("block_fp8", 4100, 256, 4096), ("int4", 4352, 384, 5120), ("nvfp4", 4099, 256, 4352),
@@ -214,10 +212,10 @@ def test_dense_split_launch_tail_rows(hip_device, fmt, M, K, N):
     ex = R.linear_fwd_bwd_exact(x, w_ref, m.lora_A.detach().cpu(), m.lora_B.detach().cpu(), m.scaling, dy,
                                 bias=m.bias.detach().cpu())
     for name, got, ref in (("y", y, ex["y"]), ("dx", dx, ex["dx"]), ("dA", dA, ex["dA"]), ("dB", dB, ex["dB"])):
-        assert R.max_rel_err(got.cpu(), ref) <= TOL, f"{fmt} {name}"
+        close(got.cpu(), ref, TOL)
     seam = slice((M // 256) * 256 - 300, M)
-    assert R.max_rel_err(y.cpu()[seam], ex["y"][seam]) <= TOL
-    assert R.max_rel_err(dx.cpu()[seam], ex["dx"][seam]) <= TOL
+    close(y.cpu()[seam], ex["y"][seam], TOL)
+    close(dx.cpu()[seam], ex["dx"][seam], TOL)
 
 
 @pytest.mark.parametrize("fmt", ["block_fp8", "nvfp4"])
@@ -234,14 +232,14 @@ def test_row_strided_activations(hip_device, fmt, M):
     A, B = m.lora_A.detach().cpu(), m.lora_B.detach().cpu()
     ex = R.linear_fwd_bwd_exact(x.cpu(), w_ref, A, B, m.scaling, dy.cpu())
     with torch.no_grad():
-        assert R.max_rel_err(m(x).cpu(), ex["y"]) <= TOL
+        close(m(x).cpu(), ex["y"], TOL)
     xg = x.detach().requires_grad_(True)
     y = m(xg)
     y.backward(dy)
-    assert R.max_rel_err(y.detach().cpu(), ex["y"]) <= TOL
-    assert R.max_rel_err(xg.grad.cpu(), ex["dx"]) <= TOL
-    assert R.max_rel_err(m.lora_A.grad.cpu(), ex["dA"]) <= TOL
-    assert R.max_rel_err(m.lora_B.grad.cpu(), ex["dB"]) <= TOL
+    close(y.detach().cpu(), ex["y"], TOL)
+    close(xg.grad.cpu(), ex["dx"], TOL)
+    close(m.lora_A.grad.cpu(), ex["dA"], TOL)
+    close(m.lora_B.grad.cpu(), ex["dB"], TOL)
 
 
 @pytest.mark.parametrize("fmt,r", [("block_fp8", 96), ("nvfp4", 128), ("int4", 72)])
@@ -257,12 +255,12 @@ def test_ranks_above_the_fused_limit(hip_device, fmt, r):
     ex = R.linear_fwd_bwd_exact(x, w_ref, A, B, m.scaling, dy)
     assert dA.shape == (r, K) and dB.shape == (N, r)
     for name, got, ref in (("y", y, ex["y"]), ("dx", dx, ex["dx"]), ("dA", dA, ex["dA"]), ("dB", dB, ex["dB"])):
-        assert R.max_rel_err(got.cpu(), ref) <= TOL, f"{fmt} {name}"
+        close(got.cpu(), ref, TOL)
     # every rank contributes: the tail ranks' gradients are not zero
     assert float(dA[64:].abs().max()) > 0 and float(dB[:, 64:].abs().max()) > 0
     with torch.no_grad():
         ys = m(x[:4].to(hip_device))                                        # skinny path
-    assert R.max_rel_err(ys.cpu(), ex["y"][:4]) <= TOL
+    close(ys.cpu(), ex["y"][:4], TOL)
     # publish and merge
     pub = m.merged_weight().cpu()
     want = R.merge_publish_recipe(w_ref, A, B, m.scaling)
@@ -298,8 +296,7 @@ def test_dense_seeded_shape_sweep(hip_device, tile_policy):
         ex = R.linear_fwd_bwd_exact(x, w_ref, m.lora_A.detach().cpu(), m.lora_B.detach().cpu(), m.scaling, dy,
                                     bias=None if m.bias is None else m.bias.detach().cpu())
         for name, got, ref in (("y", y, ex["y"]), ("dx", dx, ex["dx"]), ("dA", dA, ex["dA"]), ("dB", dB, ex["dB"])):
-            err = R.max_rel_err(got.cpu(), ref)
-            assert err <= TOL, (case, fmt, M, K, N, r, name, err)
+            close(got.cpu(), ref, TOL)
 
 
 def test_training_shape_rule_is_reported_at_the_forward(hip_device):
@@ -310,7 +307,7 @@ def test_training_shape_rule_is_reported_at_the_forward(hip_device):
     with torch.no_grad():
         y = m(x)
     ex = R.linear_fwd_bwd_exact(x.cpu(), w_ref, m.lora_A.detach().cpu(), m.lora_B.detach().cpu(), m.scaling)
-    assert R.max_rel_err(y.cpu(), ex["y"]) <= TOL
+    close(y.cpu(), ex["y"], TOL)
     with pytest.raises(ValueError, match="out_features % 64"):
         m(x.requires_grad_(True))
 
@@ -337,3 +334,101 @@ def test_module_under_torch_compile(hip_device, backend):
     args = (x, qw.packed, qw.scales, qw.global_scale, m.lora_A.detach(), m.lora_B.detach(), None, qw.fmt,
             Fn._DT_TO_CODE[qw.scale_dtype], qw.group, qw.rows, qw.cols, 16, 2.0, True)
     assert set(opcheck(Fn._linear_fwd_op, args, test_utils=("test_schema", "test_faketensor")).values()) == {"SUCCESS"}
+
+
+_ZERO_CODE = {"block_fp8": 0x00, "int4": 0x88, "nvfp4": 0x00, "nf4": 0x77}    # bytes whose codes all decode to 0.0
+
+
+@pytest.mark.parametrize("tile_policy", [0, 1, 2], indirect=True)
+@pytest.mark.parametrize("fmt", ["block_fp8", "int4", "nvfp4", "nf4"])
+@pytest.mark.parametrize("M", [16, 640])
+def test_lora_term_alone(hip_device, tile_policy, fmt, M):
+    """Base codes that decode to zero (e4m3 byte 0x00, int4 code 8, e2m1 code 0, NF4 level 7), so that y and dx
+    are the low-rank term alone and are judged on ITS scale, not the base product's: the kernels round the factors
+    and the [M, r] intermediate to bf16 where the reference runs this branch in fp32
+    (qlora/modules/linear.py:378-382); y, dx, dA, dB must stay within 1e-2 of the fp64 program all the same.
+    M = 16 without grad takes the skinny path, M = 640 the tile kernels."""
+    K, N, r = 1024, 768, 16
+    m, _ = make_dense_module(fmt, N, K, r, 32, seed=M, device=hip_device)
+    nbytes = N * K if fmt == "block_fp8" else N * K // 2
+    with torch.no_grad():
+        m._write_packed_weight(torch.full((nbytes,), _ZERO_CODE[fmt], dtype=torch.uint8, device=hip_device))
+    assert torch.count_nonzero(m._dequantize_weight()) == 0
+    w0 = torch.zeros(N, K, dtype=torch.bfloat16)
+    x = gen((M, K), 1.0, 61, torch.bfloat16)
+    dy = gen((M, N), 1.0, 62, torch.bfloat16)
+    A, B = m.lora_A.detach().cpu(), m.lora_B.detach().cpu()
+    ex = R.linear_fwd_bwd_exact(x, w0, A, B, m.scaling, dy)
+    assert float(ex["y"].abs().max()) > 0
+    with torch.no_grad():
+        close(m(x.to(hip_device)).cpu(), ex["y"], TOL)
+    y, dx, dA, dB = _run(m, x.to(hip_device), dy.to(hip_device))
+    for got, ref in ((y, ex["y"]), (dx, ex["dx"]), (dA, ex["dA"]), (dB, ex["dB"])):
+        close(got.cpu(), ref, TOL)
+
+
+@pytest.mark.parametrize("fmt", ["block_fp8", "nvfp4", "nf4", "int4"])
+def test_aqn_forward(hip_device, fmt):
+    """Adaptive quantization noise (qlora/modules/linear.py:337-363): in training the decoded weight is perturbed by
+    aqn_alpha * N(0, 1) * step, step = 0.125 * block scale (block_fp8_linear.py:102-109), 0.5 * block scale * global
+    scale (nvfp4_linear.py:115-124), 0.5 * NF4_MIN_STEP * group absmax (nf4_linear.py:113-120).  With alpha = 0 the
+    noisy forward is the plain recipe and must agree with the fused kernels; with alpha > 0 the perturbation of the
+    weight, recovered through X = I, has the stated per-element standard deviation; eval mode never adds noise."""
+    from xorl_amd import quantize as Q
+
+    N = K = 512
+    r = 16
+    m, w_ref = make_dense_module(fmt, N, K, r, 32, seed=91, device=hip_device)
+    x = gen((96, K), 1.0, 92, torch.bfloat16).to(hip_device)
+    m.eval()
+    with torch.no_grad():
+        y_fused = m(x)
+    m.enable_aqn, m.aqn_alpha = True, 0.0
+    with torch.no_grad():
+        assert torch.equal(m(x), y_fused)                    # eval: the fused path whatever enable_aqn says
+    m.train()
+    ex = R.linear_fwd_bwd_exact(x.cpu(), w_ref, m.lora_A.detach().cpu(), m.lora_B.detach().cpu(), m.scaling)
+    with torch.no_grad():
+        y0 = m(x)
+    close(y0.cpu(), ex["y"], TOL)                            # alpha = 0: same function as the fused kernels
+    assert R.max_rel_err(y0.cpu(), y_fused.cpu().double()) <= TOL
+
+    # the step tensor against the oracle's decode of the scales
+    step = m._compute_aqn_step().cpu()
+    assert step.shape == (N, K) and step.dtype == torch.float32
+    if fmt == "block_fp8":
+        s = m.weight_block_scales.cpu().contiguous().view(torch.float32).reshape(N // 128, K // 128)
+        want = 0.125 * s.repeat_interleave(128, 0).repeat_interleave(128, 1)
+    elif fmt == "nvfp4":
+        bs = m.weight_block_scales.cpu().contiguous().view(torch.float8_e4m3fn).float().reshape(N, K // 16)
+        gs = m.weight_global_scale.cpu().contiguous().view(torch.float32)
+        want = 0.5 * (bs * gs).repeat_interleave(16, 1)
+    elif fmt == "nf4":
+        s = m.weight_scales.cpu().contiguous().view(torch.float32).reshape(N, K // 64)
+        want = 0.5 * Q.NF4_MIN_STEP * s.repeat_interleave(64, 1)
+    else:
+        s = m.weight_scales.cpu().contiguous().view(m._scale_dtypes["weight_scales"]).float().reshape(N, K // 128)
+        want = 0.5 * s.repeat_interleave(128, 1)
+    assert torch.equal(step, want)
+
+    # alpha > 0: y(I) - y0(I) = (alpha * noise * step)^T up to the bf16 rounding of the perturbed weight, which a
+    # large alpha makes negligible against the perturbation (a step is a fraction of the weight's own bf16 ulp)
+    alpha = 64.0
+    eye = torch.eye(K, dtype=torch.bfloat16, device=hip_device)
+    with torch.no_grad():
+        m.lora_B.zero_()
+        m.aqn_alpha = 0.0
+        base = m(eye).float()
+        m.aqn_alpha = alpha
+        pert = (m(eye).float() - base).t().cpu()             # [N, K] perturbation of w
+        pert2 = (m(eye).float() - base).t().cpu()            # a fresh draw every forward
+    z = pert / (alpha * step)
+    assert abs(float(z.mean())) < 0.02 and abs(float(z.std()) - 1.0) < 0.05, (float(z.mean()), float(z.std()))
+    assert not torch.equal(pert, pert2)
+    # gradients flow to the factors and to x through the noisy weight
+    m.aqn_alpha = 1.0
+    with torch.no_grad():
+        m.lora_B.copy_(gen((N, r), 0.02, 93).to(hip_device))
+    xg = x.clone().requires_grad_(True)
+    m(xg).sum().backward()
+    assert xg.grad is not None and m.lora_A.grad is not None and float(m.lora_B.grad.abs().max()) > 0

@@ -6,7 +6,7 @@ import torch
 
 from oracle import recipe as R
 from oracle import decode_np as NP
-from tests.util_cases import bits_to_bf16, gen, make_dense_module
+from tests.util_cases import close, bits_to_bf16, gen, make_dense_module
 
 pytestmark = pytest.mark.gpu
 TOL = 1e-2
@@ -23,27 +23,39 @@ def test_skinny_forward_vs_oracle(hip_device, fmt, M):
     ex = R.linear_fwd_bwd_exact(x, w_ref, m.lora_A.detach().cpu(), m.lora_B.detach().cpu(), m.scaling,
                                 bias=None if m.bias is None else m.bias.detach().cpu())
     assert y.shape == (M, N) and y.dtype == torch.bfloat16
-    assert R.max_rel_err(y.cpu(), ex["y"]) <= TOL
+    close(y.cpu(), ex["y"], TOL)
     # the training path (tile kernel; needs grad) gives the same answer within bf16
     y2 = m(x.to(hip_device).requires_grad_(True))
-    assert R.max_rel_err(y2.detach().cpu(), ex["y"]) <= TOL
+    close(y2.detach().cpu(), ex["y"], TOL)
 
 
-@pytest.mark.parametrize("fmt,N,K", [("block_fp8", 1024, 4096), ("int4", 1024, 4096), ("block_fp8", 4096, 12288),
-                                     ("int4", 12288, 4096), ("nf4", 4096, 12288), ("nf4", 12288, 4096)])
-def test_skinny_projection_shapes(hip_device, fmt, N, K):
-    """Qwen3-8B projection shapes of BASELINE config 4 at M = 8 and 64 (oracle in float64 on CPU)."""
+@pytest.mark.parametrize("fmt", ["int4", "block_fp8"])
+@pytest.mark.parametrize("proj,N,K", [("q", 4096, 4096), ("kv", 1024, 4096), ("gate_up", 12288, 4096), ("down", 4096, 12288)])
+def test_config4_full_grid(hip_device, fmt, proj, N, K):
+    """BASELINE configs[4] in full: {int4, block_fp8} x the Qwen3-8B projection set x M in {1, 8, 32, 64}, r = 16,
+    forward only, every cell against the float64 program on the oracle's decode of the module's bytes."""
     m, w_ref = make_dense_module(fmt, N, K, 16, 32, seed=N + K, device=hip_device)
+    A, B = m.lora_A.detach().cpu(), m.lora_B.detach().cpu()
+    for M in (1, 8, 32, 64):
+        x = gen((M, K), 1.0, M, torch.bfloat16)
+        with torch.no_grad():
+            y = m(x.to(hip_device))
+        ex = R.linear_fwd_bwd_exact(x, w_ref, A, B, m.scaling)
+        assert y.shape == (M, N) and y.dtype == torch.bfloat16
+        close(y.cpu(), ex["y"], TOL)
+        with torch.no_grad():                     # the same bits from a second call on fresh scratch
+            assert torch.equal(m(x.to(hip_device)), y)
+
+
+@pytest.mark.parametrize("N,K", [(4096, 12288), (12288, 4096)])
+def test_skinny_projection_shapes_nf4(hip_device, N, K):
+    m, w_ref = make_dense_module("nf4", N, K, 16, 32, seed=N + K, device=hip_device)
     for M in (8, 64):
         x = gen((M, K), 1.0, M, torch.bfloat16)
         with torch.no_grad():
             y = m(x.to(hip_device))
         ex = R.linear_fwd_bwd_exact(x, w_ref, m.lora_A.detach().cpu(), m.lora_B.detach().cpu(), m.scaling)
-        assert R.max_rel_err(y.cpu(), ex["y"]) <= TOL, (fmt, N, K, M)
-        # repeated calls reuse the zeroed scratch correctly
-        with torch.no_grad():
-            y_again = m(x.to(hip_device))
-        assert R.max_rel_err(y_again.cpu(), ex["y"]) <= TOL
+        close(y.cpu(), ex["y"], TOL)
 
 
 @pytest.mark.parametrize("fmt,N,K,M,r,bf16_factors", [
@@ -69,7 +81,8 @@ def test_skinny_split_plans(hip_device, fmt, N, K, M, r, bf16_factors):
         y = qlora_linear(x.to(hip_device), m._quant_weight(), A, B, r, m.scaling, m.bias)
     ex = R.linear_fwd_bwd_exact(x, w_ref, A.float().cpu(), B.float().cpu(), m.scaling,
                                 bias=None if m.bias is None else m.bias.detach().cpu())
-    assert y.shape == (M, N) and R.max_rel_err(y.cpu(), ex["y"]) <= TOL
+    assert y.shape == (M, N)
+    close(y.cpu(), ex["y"], TOL)
     # deterministic: a second call returns the same bits
     with torch.no_grad():
         y2 = qlora_linear(x.to(hip_device), m._quant_weight(), A, B, r, m.scaling, m.bias)
@@ -78,7 +91,7 @@ def test_skinny_split_plans(hip_device, fmt, N, K, M, r, bf16_factors):
     with torch.no_grad():
         y0 = qlora_linear(x.to(hip_device), m._quant_weight(), None, None, 0, 0.0, None)
     ex0 = R.linear_fwd_bwd_exact(x, w_ref, torch.zeros(1, K), torch.zeros(N, 1), 0.0)
-    assert R.max_rel_err(y0.cpu(), ex0["y"]) <= TOL
+    close(y0.cpu(), ex0["y"], TOL)
 
 
 def test_skinny_forward_under_hip_graph(hip_device):
@@ -134,7 +147,7 @@ def test_skinny_scale_storage_variants(hip_device, M):
             m.lora_B.copy_(B)
             y = m(x.to(hip_device))
         ex = R.linear_fwd_bwd_exact(x, w_ref, A, B, m.scaling)
-        assert R.max_rel_err(y.cpu(), ex["y"]) <= TOL
+        close(y.cpu(), ex["y"], TOL)
         assert torch.equal(m._dequantize_weight().cpu().reshape(N, K), w_ref)      # same bytes, same decode
 
     # nvfp4: fold the global scale into fp32 block scales, as the checkpoint loaders do
@@ -204,5 +217,5 @@ def test_skinny_seeded_shape_sweep(hip_device):
             y = qlora_linear(x.to(hip_device), m._quant_weight(), A, B, r, m.scaling, m.bias)
         ex = R.linear_fwd_bwd_exact(x, w_ref, A.float().cpu(), B.float().cpu(), m.scaling,
                                     bias=None if m.bias is None else m.bias.detach().cpu())
-        err = R.max_rel_err(y.cpu(), ex["y"])
-        assert y.shape == (M, N) and err <= TOL, (case, fmt, N, K, M, r, bf16_factors, err)
+        assert y.shape == (M, N), (case, fmt, N, K, M, r, bf16_factors)
+        close(y.cpu(), ex["y"], TOL)

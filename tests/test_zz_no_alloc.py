@@ -8,7 +8,7 @@ import pytest
 import torch
 
 from oracle import recipe as R
-from tests.util_cases import gen, make_dense_module
+from tests.util_cases import close, gen, make_dense_module
 from xorl_amd import _C
 
 pytestmark = pytest.mark.gpu
@@ -74,7 +74,7 @@ def test_static_scratch_forward_matches_workspace_forward(hip_device, fmt, N, K,
         A = m.lora_A.detach().cpu() if r else torch.zeros(1, K)
         B = m.lora_B.detach().cpu() if r else torch.zeros(N, 1)
         ex = R.linear_fwd_bwd_exact(x, w_ref, A, B, m.scaling if r else 0.0, bias=bias)
-        assert R.max_rel_err(y_st.cpu(), ex["y"]) <= TOL
+        close(y_st.cpu(), ex["y"], TOL)
 
 
 def test_static_scratch_rejects_oversized_shapes(hip_device):

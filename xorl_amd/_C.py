@@ -93,8 +93,8 @@ _SIGNATURES = {
     # a, lda, n_rows, offsets, tile_offsets, E, F, shared, r_pad, K, scale, t, stream
     "xq_grouped_lora_down": (_INT, [_P, _I64, _I64, _P, _P, _I32, _P, _INT, _INT, _I64, _F, _P, _P]),
     "xq_lora_wgrad_workspace_bytes": (_I64, [_I64, _I64, _INT]),
-    # P, ldp, p_width, Q, r_pad, r_out, n_rows, offsets, E, transpose_out, out, ws, stream
-    "xq_grouped_lora_wgrad": (_INT, [_P, _I64, _I64, _P, _INT, _INT, _I64, _P, _I32, _INT, _P, _P, _P]),
+    # P, ldp, p_width, Q, r_pad, r_out, n_rows, offsets, E, transpose_out, out, ws, row_limit, stream
+    "xq_grouped_lora_wgrad": (_INT, [_P, _I64, _I64, _P, _INT, _INT, _I64, _P, _I32, _INT, _P, _P, _P, _P]),
 }
 
 EXPORTS = ("xq_version", "xq_last_error") + tuple(_SIGNATURES)

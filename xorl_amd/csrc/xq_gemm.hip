@@ -487,9 +487,9 @@ extern "C" int64_t xq_lora_wgrad_workspace_bytes(int64_t n_rows, int64_t width, 
 
 extern "C" int xq_grouped_lora_wgrad(const void* P, int64_t ldp, int64_t p_width, const void* Q, int r_pad, int r_out,
                                      int64_t n_rows, const int32_t* offsets, int32_t num_experts, int transpose_out,
-                                     float* out, void* workspace, void* stream) {
+                                     float* out, void* workspace, const int32_t* row_limit, void* stream) {
     XQ_REQUIRE(out && (n_rows == 0 || (P && Q)), "xq_grouped_lora_wgrad: NULL pointer");
     if (n_rows == 0 && !offsets) return launch_zero_fill(out, p_width * r_out * 4, (hipStream_t)stream);
     return launch_tn((const bf16_t*)P, ldp, p_width, (const bf16_t*)Q, r_pad, r_out, n_rows, transpose_out != 0, out,
-                     (float*)workspace, offsets, num_experts, (hipStream_t)stream);
+                     (float*)workspace, offsets, num_experts, (hipStream_t)stream, row_limit);
 }

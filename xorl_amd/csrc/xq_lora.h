@@ -40,7 +40,8 @@ int launch_small_nt(const bf16_t* In, int64_t ld_in, int64_t n_rows, int64_t Kc,
 int64_t tn_partial_bytes(int64_t n_rows, int64_t width, int r_pad);
 int launch_tn(const bf16_t* P, int64_t ldp, int64_t width, const bf16_t* Q, int r_pad, int r_out,
               int64_t n_rows, bool transpose_out, float* out, float* partial,
-              const int32_t* offsets, int32_t num_experts, hipStream_t stream);
+              const int32_t* offsets, int32_t num_experts, hipStream_t stream,
+              const int32_t* row_limit = nullptr);   // dense form: contract only rows below *row_limit (device value)
 
 int launch_zero_fill(void* p, int64_t bytes, hipStream_t stream);
 

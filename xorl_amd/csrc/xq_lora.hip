@@ -299,6 +299,7 @@ struct TnArgs {
     int transpose_out;
     float* out;              // dense: partial [S][width][r_pad]; grouped: out [E][...]
     const int32_t* offsets;  // grouped
+    const int32_t* row_limit;  // dense, optional (device): only rows below *row_limit are contracted
 };
 
 constexpr int TN_PP = 128 + 16;  // Ps pitch (bf16 elements): 288 B rows
@@ -388,12 +389,16 @@ __global__ void __launch_bounds__(256) tn_kernel(TnArgs g) {
     const int64_t m_begin = (int64_t)blockIdx.y * g.rows_per_split;
     int64_t m_end = m_begin + g.rows_per_split;
     m_end = m_end < g.n_rows ? m_end : g.n_rows;
+    if (g.row_limit) {
+        const int64_t lim = *g.row_limit;
+        m_end = m_end < lim ? m_end : lim;
+    }
     f32x16 acc[NT];
 #pragma unroll
     for (int n = 0; n < NT; ++n)
 #pragma unroll
         for (int q = 0; q < 16; ++q) acc[n][q] = 0.0f;
-    tn_accumulate<NT>(g, c0, m_begin, m_end, Ps, Qs, acc);
+    if (m_begin < m_end) tn_accumulate<NT>(g, c0, m_begin, m_end, Ps, Qs, acc);     // uniform over the block
     tn_write<NT>(acc, g.out + (int64_t)blockIdx.y * g.width * g.r_pad, c0, g.width, g.r_pad, g.r_pad, false);
 }
 
@@ -496,11 +501,11 @@ int64_t tn_partial_bytes(int64_t n_rows, int64_t width, int r_pad) {
 
 int launch_tn(const bf16_t* P, int64_t ldp, int64_t width, const bf16_t* Q, int r_pad, int r_out, int64_t n_rows,
               bool transpose_out, float* out, float* partial, const int32_t* offsets, int32_t num_experts,
-              hipStream_t stream) {
+              hipStream_t stream, const int32_t* row_limit) {
     XQ_REQUIRE(r_pad > 0 && r_pad <= 64 && r_pad % 16 == 0 && r_out <= r_pad, "tn: bad rank (r_pad %d, r_out %d)", r_pad, r_out);
     XQ_REQUIRE(width % 8 == 0 && ldp % 8 == 0 && xq_aligned(P, 16) && xq_aligned(Q, 16), "tn: operands must be 16-byte aligned, width %% 8 == 0");
     if (width == 0 || r_out == 0) return XQ_OK;
-    TnArgs g{P, ldp, width, Q, r_pad, r_out, n_rows, 0, transpose_out ? 1 : 0, out, offsets};
+    TnArgs g{P, ldp, width, Q, r_pad, r_out, n_rows, 0, transpose_out ? 1 : 0, out, offsets, offsets ? nullptr : row_limit};
     unsigned col_tiles = (unsigned)xq_cdiv(width, 128);
     XQ_REQUIRE(partial != nullptr, "tn: partial workspace is NULL");
     if (offsets) {

@@ -214,6 +214,7 @@ __global__ void __launch_bounds__(64) route_place_kernel(const int32_t* sel, int
         const int before = __popcll(same & below);
         const bool last = (same & ~below & ~(1ull << lane)) == 0;   // no higher lane holds this expert
         if (e >= 0) scatter_index[idx] = run[e] + before;
+        else if (valid) scatter_index[idx] = -1;          // id outside [0, E): the copy is dropped by every consumer
         __syncthreads();
         if (e >= 0 && last) run[e] += before + 1;
         __syncthreads();
@@ -235,7 +236,7 @@ __global__ void __launch_bounds__(256) moe_scatter_kernel(const bf16_t* in, int6
             for (int u = 0; u < 8; ++u) r[u] = dst_rows[j0 + u < topk ? j0 + u : topk - 1];
 #pragma unroll
             for (int u = 0; u < 8; ++u)
-                if (j0 + u < topk) ((u32x4*)(out + r[u] * ld_out))[c] = v;     // uniform
+                if (j0 + u < topk && r[u] >= 0) ((u32x4*)(out + r[u] * ld_out))[c] = v;     // uniform; -1 = dropped copy
         }
     }
 }
@@ -245,14 +246,17 @@ __global__ void __launch_bounds__(256) moe_scatter_scalar_kernel(const void* src
                                                                  int64_t n, float* dst) {
     int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= n) return;
-    dst[sidx[i]] = src_f32 ? ((const float*)src)[i] : bf16_to_f32(((const bf16_t*)src)[i]);
+    const int32_t d = sidx[i];
+    if (d < 0) return;                                   // dropped copy
+    dst[d] = src_f32 ? ((const float*)src)[i] : bf16_to_f32(((const bf16_t*)src)[i]);
 }
 // dst[i] = src[scatter_index[i]]
 __global__ void __launch_bounds__(256) moe_gather_scalar_kernel(const float* src, const int32_t* sidx, int64_t n,
                                                                 void* dst, int dst_f32) {
     int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= n) return;
-    float v = src[sidx[i]];
+    const int32_t d = sidx[i];
+    float v = d < 0 ? 0.0f : src[d];                     // a dropped copy has no row: zero
     if (dst_f32) ((float*)dst)[i] = v;
     else ((bf16_t*)dst)[i] = to_bf16(v);
 }
@@ -270,15 +274,18 @@ __global__ void __launch_bounds__(256) moe_gather_kernel(const bf16_t* rows, con
         float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
         for (int j0 = 0; j0 < topk; j0 += 8) {
             u32x4 v[8], v2[8];
+            bool keep[8];
 #pragma unroll
             for (int u = 0; u < 8; ++u) {
-                const int64_t r = src_rows[j0 + u < topk ? j0 + u : topk - 1];
+                const int64_t r0 = src_rows[j0 + u < topk ? j0 + u : topk - 1];
+                keep[u] = r0 >= 0;                         // -1 = dropped copy: row 0 is read in its place and left out
+                const int64_t r = keep[u] ? r0 : 0;
                 v[u] = ((const u32x4*)(rows + r * ld_rows))[c];
                 if (TWO) v2[u] = ((const u32x4*)(rows2 + r * ld_rows))[c];
             }
 #pragma unroll
             for (int u = 0; u < 8; ++u) {
-                if (j0 + u < topk) {                       // uniform
+                if (j0 + u < topk && keep[u]) {            // uniform
 #pragma unroll
                     for (int q = 0; q < 4; ++q) {
                         acc[2 * q] += bf16_to_f32((bf16_t)(v[u][q] & 0xffffu));

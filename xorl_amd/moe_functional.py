@@ -101,9 +101,11 @@ def _grouped_gemm(qw: QuantWeight, transpose_w: bool, a: Tensor, offsets, tile_o
     return y
 
 
-def _wgrad(P: Tensor, Q: Tensor, r: int, offsets: Optional[Tensor], E: int, transpose_out: bool) -> Tensor:
+def _wgrad(P: Tensor, Q: Tensor, r: int, offsets: Optional[Tensor], E: int, transpose_out: bool,
+           row_limit: Optional[Tensor] = None) -> Tensor:
     """Per expert (offsets given): out[e] = P[rows e]^T . Q[rows e] -> [E, width, r] or [E, r, width];
-    offsets None: one product over all rows -> [1, ...] (gradient of a factor shared by all experts)."""
+    offsets None: one product over all rows (below row_limit[0], a device int32, when given) -> [1, ...]
+    (gradient of a factor shared by all experts)."""
     R, width = P.shape
     rp = Q.shape[1]
     L = _C.lib()
@@ -112,7 +114,8 @@ def _wgrad(P: Tensor, Q: Tensor, r: int, offsets: Optional[Tensor], E: int, tran
     out = torch.empty(*shape, dtype=torch.float32, device=P.device)
     ws = torch.empty(L.xq_lora_wgrad_workspace_bytes(R, width, rp), dtype=torch.uint8, device=P.device)
     _C.check(L.xq_grouped_lora_wgrad(P.data_ptr(), P.stride(0), width, Q.data_ptr(), rp, r, R, _C.ptr(offsets), E,
-                                     int(transpose_out), out.data_ptr(), _C.ptr(ws), _s(P.device)))
+                                     int(transpose_out), out.data_ptr(), _C.ptr(ws),
+                                     _C.ptr(row_limit) if offsets is None else None, _s(P.device)))
     return out
 
 
@@ -137,6 +140,9 @@ class MoeExpertsQLoRAFunction(torch.autograd.Function):
         if hidden.dtype != torch.bfloat16:
             raise _C.XqError(f"hidden states must be bf16, got {hidden.dtype}")
         E = num_experts
+        for qw in (qw_gate, qw_up, qw_down):
+            if qw.num_experts != E:          # the tile schedules route_build emits are laid out for E experts
+                raise _C.XqError(f"routing over {E} experts but a bank holds {qw.num_experts}")
         shape = hidden.shape
         H = shape[-1]
         hidden2 = hidden.reshape(-1, H)
@@ -202,8 +208,9 @@ class MoeExpertsQLoRAFunction(torch.autograd.Function):
         Lr_dA = _prep(_expand(dA, E), False, I, rp)                                          # [E, I, rp]
         dh = _grouped_gemm(qw_down, True, g_down, offsets, tile_offsets, v_d, Lr_dA)         # [R, I]
         shared_dB = dB.shape[0] == 1
-        grad_dB = _wgrad(g_down, su_d, r, None if shared_dB else offsets, E, True)           # [E|1, r, H]
-        grad_dA = _wgrad(h, v_d, r, None if dA.shape[0] == 1 else offsets, E, False)         # [E|1, I, r]
+        n_valid = offsets[E:]            # rows that belong to an expert (all of them unless an id was out of range)
+        grad_dB = _wgrad(g_down, su_d, r, None if shared_dB else offsets, E, True, n_valid)  # [E|1, r, H]
+        grad_dA = _wgrad(h, v_d, r, None if dA.shape[0] == 1 else offsets, E, False, n_valid)   # [E|1, I, r]
 
         # ---- SwiGLU + routing weight
         dgate = torch.empty(R, I, dtype=torch.bfloat16, device=dev)
@@ -225,7 +232,7 @@ class MoeExpertsQLoRAFunction(torch.autograd.Function):
             v = _lora_down(g_out, F_B, offsets, tile_offsets, E, s)
             Lr_A = _prep(_expand(A, E), False, H, rp)                                        # [E, H, rp]
             dx = _grouped_gemm(qw, True, g_out, offsets, tile_offsets, v, Lr_A)              # [R, H]
-            gB_ = _wgrad(g_out, su, r, None if B.shape[0] == 1 else offsets, E, True)        # [E|1, r, I]
+            gB_ = _wgrad(g_out, su, r, None if B.shape[0] == 1 else offsets, E, True, n_valid)   # [E|1, r, I]
             return dx, v, gB_
 
         dx_u, v_u, grad_uB = proj_bwd(dup, qw_up, uA, uB, su_u)
@@ -233,11 +240,11 @@ class MoeExpertsQLoRAFunction(torch.autograd.Function):
         # gradients of the two A factors, [E|1, H, r] = x^T . v: both contract the same rows of x, so they share
         # one pass over them (v_g | v_u side by side) when the panels fit
         if gA.shape[0] == uA.shape[0] and 2 * rp <= 32:
-            both = _wgrad(xs, torch.cat([v_g, v_u], dim=1), rp + r, None if gA.shape[0] == 1 else offsets, E, False)
+            both = _wgrad(xs, torch.cat([v_g, v_u], dim=1), rp + r, None if gA.shape[0] == 1 else offsets, E, False, n_valid)
             grad_gA, grad_uA = both[..., :r], both[..., rp:rp + r]
         else:
-            grad_gA = _wgrad(xs, v_g, r, None if gA.shape[0] == 1 else offsets, E, False)
-            grad_uA = _wgrad(xs, v_u, r, None if uA.shape[0] == 1 else offsets, E, False)
+            grad_gA = _wgrad(xs, v_g, r, None if gA.shape[0] == 1 else offsets, E, False, n_valid)
+            grad_uA = _wgrad(xs, v_u, r, None if uA.shape[0] == 1 else offsets, E, False, n_valid)
         dx = moe_gather(dx_g, dx_u, sidx, T, topk).reshape(shape) if ctx.needs_input_grad[0] else None
 
         cast = lambda g, p: g.to(p.dtype)

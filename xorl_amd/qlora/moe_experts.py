@@ -320,11 +320,15 @@ class QLoRAMoeExperts(LoraModule, nn.Module):
             cumsum = torch.zeros(self.num_local_experts, dtype=torch.int64, device=rows.device)
             cumsum[local:] = rows.shape[0]
             return self.compute_dispatched(rows, cumsum).reshape(*hidden_states.shape[:-1], self.hidden_size)
+        if self.num_local_experts != self.num_experts:
+            raise ValueError(
+                f"the routed call needs every expert on this rank (num_local_experts={self.num_local_experts}, "
+                f"num_experts={self.num_experts}); an expert-parallel caller dispatches rows and uses compute_dispatched()")
         gA, gB = self._active_lora_views("gate_proj")
         uA, uB = self._active_lora_views("up_proj")
         dA, dB = self._active_lora_views("down_proj")
         return moe_experts_qlora_forward(
-            num_experts=self.num_experts, routing_weights=routing_weights, selected_experts=selected_experts,
+            num_experts=self.num_local_experts, routing_weights=routing_weights, selected_experts=selected_experts,
             hidden_states=hidden_states, gate_proj=self._bank("gate"), up_proj=self._bank("up"),
             down_proj=self._bank("down"), gate_proj_lora_A=gA, gate_proj_lora_B=gB, up_proj_lora_A=uA,
             up_proj_lora_B=uB, down_proj_lora_A=dA, down_proj_lora_B=dB, scaling=self._active_scaling())
@@ -342,13 +346,23 @@ class QLoRAMoeExperts(LoraModule, nn.Module):
             out = out * expert_scores.unsqueeze(1).to(out.dtype)
         return out
 
-    def merge_weights(self, ema_decay: float = 0.1) -> None:
+    def merge_weights(self, ema_decay: float = 0.1, experts_per_step: int = 16) -> None:
+        """W' = Q(deq(W) + delta.to(deq dtype)), then fresh LoRA factors (moe_experts.py:987-1008, :1134-1146,
+        :1249-1261).  The sum is formed in the dtype the bank decodes to, as the reference does: bf16 for nvfp4 and
+        nf4 (a bf16 add of two bf16 tensors), fp32 for block_fp8.  The update is added to the decoded bank in place,
+        `experts_per_step` experts at a time, so the peak is the decoded bank plus one step's update."""
         with torch.no_grad():
             for name in ("gate", "up", "down"):
                 K, N = self._proj_dims(name)
-                w = self.dequantize_all_experts(name, K, N).float()
-                merged = w + self._compute_proj_delta(f"{name}_proj").to(w.dtype)
-                self._requantize_proj(name, merged, ema_decay)
+                w = self.dequantize_all_experts(name, K, N)
+                A, B = self._active_lora_views(f"{name}_proj")
+                E = w.shape[0]
+                A, B = A.expand(E, -1, -1), B.expand(E, -1, -1)
+                for e0 in range(0, E, experts_per_step):
+                    e1 = min(E, e0 + experts_per_step)
+                    delta = torch.bmm(A[e0:e1], B[e0:e1]) * self._active_scaling()
+                    w[e0:e1] += delta.to(w.dtype)
+                self._requantize_proj(name, w, ema_decay)
         self.reset_lora_parameters()
 
     def _requantize_proj(self, name: str, merged: Tensor, ema_decay: float) -> None:
