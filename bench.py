@@ -35,21 +35,33 @@ BF16_MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense bf16, published
 
 # HBM-side bytes per launch of each config's roofline kernel, from the committed counter runs
 # (rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE, each scaled by what the same counter reads for a plain
-# 256 MiB -> 256 MiB copy; the files under profiles/ hold the figures and the commands).  A config that
-# has no counter run reports null.  --traffic-bytes overrides.
-MEASURED_TRAFFIC_BYTES = {
-    0: 109.6 * 2 ** 20,    # gemm_256_kernel<int4, T=128> in 4 K splits + splitk_reduce_kernel: mean of the forward and dgrad
-                           # launches (64 MiB of it are the fp32 partial sums written and read back)
-    1: 905.4 * 2 ** 20,    # gemm_256_kernel<fp8>: mean of the forward and dgrad launches
-    2: 187.2 * 2 ** 20,    # gemm_256_kernel<nvfp4>, 256x256 tiles (whole rounds; trailing rows in K splits) and 128x128 tiles
-                           # (+ splitk_reduce_kernel): mean over the 12 launches of a step, fp32 partial sums included
-    3: 1032.2 * 2 ** 20,   # gemm_256_kernel<fp8, grouped>: mean over the 6 launches of a step
-    4: 41.0 * 2 ** 20,     # skinny_split_kernel + skinny_epilogue_kernel: mean per forward over the 32 cases (includes
-                           # the fp32 partial tiles written and read back: 23.3 MiB of it are algorithmic)
-    6: 737.0 * 2 ** 20,    # gemm_256_kernel<nf4>: mean of the forward and dgrad launches
-    7: 889.1 * 2 ** 20,    # gemm_256_kernel<nvfp4 GKN, grouped>: mean over the 6 launches of a step
-    9: 59.0 * 2 ** 20,     # merge_prep_kernel + merge_kernel<nvfp4>: mean per call over amax / re-quantise / publish of the four weights
-    5: 134.4 * 2 ** 20,    # merge_prep_kernel + merge_kernel<fp8>: mean per call (re-quantise 96 MiB, publish 144 MiB algorithmic)
+# 256 MiB -> 256 MiB copy).  Each entry names the profile file that holds the figures and the commands, and the
+# average launch duration of the roofline kernel in that profile's own bench line: a run whose live average differs
+# from it by more than 10 % is timing another kernel build (or another machine state) than the counters saw, and
+# reports traffic null with the reason instead of a stale constant.  A config that has no counter run reports null.
+# --traffic-bytes overrides.
+MEASURED_TRAFFIC = {
+    # gemm_256_kernel<int4, T=128> in 4 K splits + splitk_reduce_kernel: mean of the forward and dgrad launches
+    # (64 MiB of it are the fp32 partial sums written and read back)
+    0: (109.6 * 2 ** 20, "profiles/gemm_128_int4_linear_m512.txt", 0.04478),
+    # gemm_256_kernel<fp8>: mean of the forward and dgrad launches
+    1: (905.4 * 2 ** 20, "profiles/gemm_256_fp8_mlp_m8192.txt", 0.73747),
+    # gemm_256_kernel<nvfp4>, 256x256 tiles (whole rounds; trailing rows in K splits) and 128x128 tiles
+    # (+ splitk_reduce_kernel): mean over the 12 launches of a step, fp32 partial sums included
+    2: (187.2 * 2 ** 20, "profiles/gemm_256_nvfp4_attn_m4096.txt", 0.14518),
+    # gemm_256_kernel<fp8, grouped>: mean over the 6 launches of a step
+    3: (1032.2 * 2 ** 20, "profiles/gemm_256_fp8_grouped_moe_e128.txt", 0.57350),
+    # skinny_split_kernel + skinny_epilogue_kernel: mean per forward over the 32 cases (includes the fp32 partial
+    # tiles written and read back: 23.3 MiB of it are algorithmic)
+    4: (41.0 * 2 ** 20, "profiles/skinny_split_kernel_decode_shapes.txt", 0.02006),
+    # merge_prep_kernel + merge_kernel<fp8>: mean per call (re-quantise 96 MiB, publish 144 MiB algorithmic)
+    5: (134.4 * 2 ** 20, "profiles/merge_kernel_fp8_mlp_weights.txt", 0.04168),
+    # gemm_256_kernel<nf4>: mean of the forward and dgrad launches
+    6: (737.0 * 2 ** 20, "profiles/gemm_256_nf4_mlp_m8192.txt", 0.85447),
+    # gemm_256_kernel<nvfp4 GKN, grouped>: mean over the 6 launches of a step
+    7: (889.1 * 2 ** 20, "profiles/gemm_256_nvfp4_gkn_grouped_moe_e128.txt", 0.58278),
+    # merge_prep_kernel + merge_kernel<nvfp4>: mean per call over amax / re-quantise / publish of the four weights
+    9: (59.0 * 2 ** 20, "profiles/merge_kernel_nvfp4_attn_weights.txt", 0.03500),
 }
 
 
@@ -81,7 +93,7 @@ def build_modules():
     return mods
 
 
-def cpu_baseline(mods, rows: int):
+def cpu_baseline(mods, rows: int, warmups: int = 2, runs: int = 5):
     """Reference recipe on host cores over `rows` tokens of the same workload."""
     from oracle import decode_np as NP
     from oracle import recipe as RC
@@ -106,16 +118,22 @@ def cpu_baseline(mods, rows: int):
         y.backward(dy)
         return y
 
-    t0 = time.perf_counter()
-    run()
-    dt = time.perf_counter() - t0
+    for _ in range(warmups):
+        run()
+    times = []
+    for _ in range(runs):
+        t0 = time.perf_counter()
+        run()
+        times.append(time.perf_counter() - t0)
+    dt = sorted(times)[len(times) // 2]
     return {
         "value": step_flops(rows) / dt / 1e12,
         "unit": "TFLOP/s",
         "cores": os.cpu_count(),
         "kind": "port",
-        "sample": f"{rows} of {M} token rows of the same MLP, decode+fwd+bwd, torch CPU ops on the oracle decode, "
-                  f"{dt:.1f} s",
+        "sample": f"{rows} of {M} token rows of the same MLP, decode+fwd+bwd, torch CPU ops on the oracle decode: "
+                  f"median of {runs} runs after {warmups} warm-ups, {dt:.2f} s per run "
+                  f"(min {min(times):.2f}, max {max(times):.2f})",
     }
 
 
@@ -308,8 +326,19 @@ def calibrate_copy(dev):
     del src, dst
 
 
-def traffic_of(args):
-    return args.traffic_bytes if args.traffic_bytes is not None else MEASURED_TRAFFIC_BYTES.get(args.config)
+def traffic_of(args, live_avg_launch_ms):
+    """-> (traffic bytes or None, provenance text).  The committed counter figure of this config, unless the run's
+    own average launch duration says that it times something else than the counters measured."""
+    if args.traffic_bytes is not None:
+        return args.traffic_bytes, "--traffic-bytes"
+    entry = MEASURED_TRAFFIC.get(args.config)
+    if entry is None:
+        return None, "no counter run committed for this config"
+    nbytes, profile, ref_ms = entry
+    if live_avg_launch_ms <= 0 or abs(live_avg_launch_ms / ref_ms - 1.0) > 0.10:
+        return None, (f"stale: {profile} measured its counters at {ref_ms:.4f} ms per launch, this run averages "
+                      f"{live_avg_launch_ms:.4f} ms; re-run the --pmc passes named in that file")
+    return nbytes, f"{profile} ({ref_ms:.4f} ms per launch there, {live_avg_launch_ms:.4f} ms here)"
 
 
 def main():
@@ -317,7 +346,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--cpu-rows", type=int, default=8192, help="token rows of the CPU baseline sample (0 = skip)")
+    ap.add_argument("--cpu-rows", type=int, default=4096,
+                    help="token rows of the CPU baseline sample (0 = skip); 2 warm-ups + 5 timed runs, ~12 s at 4096 rows")
     ap.add_argument("--config", type=int, default=1,
                     help="BASELINE.json configs index; 1 (default) is the headline workload, the others report the "
                          "same JSON for their own workload (no CPU baseline)")
@@ -378,6 +408,8 @@ def main():
     ms_per_step = dt / args.steps * 1e3
     value = step_flops(M) / (dt / args.steps) / 1e12
     achieved = fl.value / (ms.value * 1e-3) / 1e12 if ms.value > 0 else 0.0
+    avg_launch_ms = ms.value / max(n.value, 1)
+    traffic, traffic_source = traffic_of(args, avg_launch_ms)
     out = {
         "metric": METRIC,
         "value": value,
@@ -395,10 +427,10 @@ def main():
                                "intermediate 12288, LoRA r=32 on gate/up/down, SwiGLU",
                    "tokens": M, "hidden": H, "intermediate": I, "lora_r": R, "format": "block_fp8"},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": BF16_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / BF16_MFMA_PEAK_TFLOPS, "traffic": traffic_of(args),
+                     "frac": achieved / BF16_MFMA_PEAK_TFLOPS, "traffic": traffic, "traffic_source": traffic_source,
                      "kernel": "gemm_256_kernel<fp8, contract_cols true|false, dense> (fused fp8 dequant-GEMM, "
                                "forward and dgrad launches)",
-                     "launches": n.value, "avg_launch_ms": ms.value / max(n.value, 1)},
+                     "launches": n.value, "avg_launch_ms": avg_launch_ms},
         "cpu_baseline": cpu,
     }
     print(json.dumps(out))
@@ -451,13 +483,15 @@ def run_other(args, dev):
     L.xq_profile_enable(0)
     scale, unit, peak = (1e9, "GB/s", 8000.0) if is_bytes else (1e12, "TFLOP/s", BF16_MFMA_PEAK_TFLOPS)
     achieved = fl.value / (ms.value * 1e-3) / scale if ms.value > 0 else 0.0
+    avg_launch_ms = ms.value / max(n.value, 1)
+    traffic, traffic_source = traffic_of(args, avg_launch_ms)
     print(json.dumps({
         "metric": METRIC, "value": work / dt / scale, "unit": unit, "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": dt * 1e3, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic", "config": {"workload": workload},
         "roofline": {"bound": "hbm" if is_bytes else "mfma", "achieved": achieved, "peak": peak, "unit": unit,
-                     "frac": achieved / peak, "traffic": traffic_of(args), "kernel": kernel,
-                     "launches": n.value, "avg_launch_ms": ms.value / max(n.value, 1)},
+                     "frac": achieved / peak, "traffic": traffic, "traffic_source": traffic_source, "kernel": kernel,
+                     "launches": n.value, "avg_launch_ms": avg_launch_ms},
         "cpu_baseline": None}))
 
 

@@ -432,3 +432,28 @@ def test_aqn_forward(hip_device, fmt):
     xg = x.clone().requires_grad_(True)
     m(xg).sum().backward()
     assert xg.grad is not None and m.lora_A.grad is not None and float(m.lora_B.grad.abs().max()) > 0
+
+
+def test_weight_descriptor_checks_scale_storage(hip_device):
+    """The kernels index scales by shape alone, so the descriptor refuses a scale buffer whose size or element type
+    does not match what it says, and an nvfp4 weight without a proper fp32 global scale."""
+    from xorl_amd import _C
+
+    N, K = 256, 512
+    packed8 = torch.zeros(N, K, dtype=torch.uint8, device=hip_device)
+    packed4 = torch.zeros(N, K // 2, dtype=torch.uint8, device=hip_device)
+    ok = _C.make_weight("block_fp8", _C.XQ_LAYOUT_FLAT, packed8, torch.ones(2, 4, device=hip_device), torch.float32, N, K, 128)
+    assert ok.rows == N
+    with pytest.raises(_C.XqError, match="scale buffer"):
+        _C.make_weight("block_fp8", _C.XQ_LAYOUT_FLAT, packed8, torch.ones(2, 3, device=hip_device), torch.float32, N, K, 128)
+    with pytest.raises(_C.XqError, match="scale buffer"):       # bf16 storage announced as fp32
+        _C.make_weight("int4", _C.XQ_LAYOUT_FLAT, packed4, torch.ones(N, K // 128, dtype=torch.bfloat16, device=hip_device),
+                       torch.float32, N, K, 128)
+    e4 = torch.zeros(N * K // 16, dtype=torch.uint8, device=hip_device)
+    with pytest.raises(_C.XqError, match="global_scale"):
+        _C.make_weight("nvfp4", _C.XQ_LAYOUT_FLAT, packed4, e4, torch.float8_e4m3fn, N, K, 16,
+                       global_scale=torch.ones(1, dtype=torch.bfloat16, device=hip_device))
+    with pytest.raises(_C.XqError, match="global_scale"):
+        _C.make_weight("nvfp4", _C.XQ_LAYOUT_GKN, torch.zeros(4, K // 2, N, dtype=torch.uint8, device=hip_device),
+                       torch.zeros(4, K // 16, N, dtype=torch.uint8, device=hip_device), torch.float8_e4m3fn, K, N, 16,
+                       global_scale=torch.ones(3, device=hip_device), num_experts=4)

@@ -184,4 +184,23 @@ def make_weight(
             f"packed buffer holds {packed.numel() * packed.element_size()} bytes, "
             f"expected {nbytes * num_experts} for {num_experts} x [{rows}, {cols}] {fmt}"
         )
+    # the kernels index the scales by shape alone: a buffer of another size or element type than `scale_dtype`
+    # says (a state_dict load into differently typed storage, say) would be read out of bounds
+    esz = {XQ_SCALE_F32: 4, XQ_SCALE_BF16: 2, XQ_SCALE_E4M3: 1}[w.scale_dtype]
+    if fmt == "block_fp8":
+        if scale_dtype != torch.float32:
+            raise XqError(f"block_fp8 scales are fp32, got {scale_dtype}")
+        sbytes = -(-rows // 128) * -(-cols // 128) * 4
+    else:
+        if group <= 0 or (rows * cols) % group:
+            raise XqError(f"group {group} does not divide [{rows}, {cols}]")
+        sbytes = rows * cols // group * esz
+    have = scales.numel() * scales.element_size()
+    if have != sbytes * num_experts:
+        raise XqError(f"scale buffer holds {have} bytes, expected {sbytes * num_experts} for {num_experts} x "
+                      f"[{rows}, {cols}] {fmt} with {scale_dtype} scales (group {group})")
+    if fmt == "nvfp4":
+        if global_scale is None or global_scale.dtype != torch.float32 or global_scale.numel() < num_experts \
+                or not global_scale.is_contiguous():
+            raise XqError(f"nvfp4 needs a contiguous fp32 global_scale with {num_experts} element(s)")
     return w

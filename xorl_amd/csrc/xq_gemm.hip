@@ -1,5 +1,6 @@
 // Host entry points of the fused dequant-GEMM + LoRA path (dense and grouped).
 #include "xq_gemm_tile.h"
+#include <atomic>
 #include "xq_gemm_256.h"
 #include <stdlib.h>
 #include <mutex>
@@ -15,7 +16,8 @@ static void launch_tile_cc(const TileArgs& g, bool contract_cols, dim3 grid, hip
 
 // kernel-selection policy (xq_set_tile_policy): 0 = by problem size, 1 = always the generic single-buffered
 // tile kernel, 2 / 3 = the pipelined kernel with 256x256 / 128x128 tiles whenever the format allows it.
-// XQ_SKINNY=0 disables the M <= 64 path.
+// XQ_SKINNY=0 disables the M <= 64 path.  Both are process-wide test switches: set them while no other thread is
+// inside the library.
 static int g_skinny_enabled = [] { const char* e = getenv("XQ_SKINNY"); return e ? atoi(e) : 1; }();
 static int g_tile_policy = [] { const char* e = getenv("XQ_TILE_POLICY"); return e ? atoi(e) : 0; }();
 
@@ -31,7 +33,7 @@ static int raise_lds_limit(K kernel, size_t bytes, const char* who) {
 
 template <int FMT, bool CC, bool GROUPED, int T, bool SPLIT256 = false>
 static int launch_256_one(const G256Args& f, dim3 grid, hipStream_t s, const char* who) {
-    static bool attr_set = false;  // per instantiation
+    static std::atomic<bool> attr_set{false};   // per instantiation; the attribute call is idempotent: a race only repeats it
     if (!attr_set) {
         int rc = raise_lds_limit(gemm_256_kernel<FMT, CC, GROUPED, T, SPLIT256>, Geo<T>::lds_bytes(CC), who);
         if (rc) return rc;
@@ -54,17 +56,29 @@ static int launch_256(const G256Args& f, bool cc, bool grouped, int T, dim3 grid
     return grouped ? launch_256_t<FMT, false, true>(f, T, grid, s, who) : launch_256_t<FMT, false, false>(f, T, grid, s, who);
 }
 
+// compute units of the current device (256 on MI355X), asked once
+static int num_cus() {
+    static std::atomic<int> cached{0};
+    int c = cached.load(std::memory_order_relaxed);
+    if (c > 0) return c;
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+        n = 256;
+    cached.store(n, std::memory_order_relaxed);
+    return n;
+}
+
 // Tile size of a dense launch under the default policy: large tiles from the point where they fill more than
-// half the chip (up to 512 small tiles are resident at once, two per CU, and finish sooner than one round of up
-// to 128 large ones).
+// half the chip (two small tiles are resident per compute unit, and finish sooner than a half-empty round of
+// large ones).
 static inline int dense_tile_size(int64_t n_rows, int64_t Nout) {
-    return xq_cdiv(n_rows, 256) * xq_cdiv(Nout, 256) > 128 ? 256 : 128;
+    return xq_cdiv(n_rows, 256) * xq_cdiv(Nout, 256) > num_cus() / 2 ? 256 : 128;
 }
 
 // K splits of a dense launch of `blocks` tiles of size T over nk K-steps (1 = none): used when the tiles fill at
 // most half of the block slots of the chip (256 large tiles, 512 small ones); every split keeps at least 8 K-steps.
 static inline int ksplit_for(int64_t blocks, int T, int64_t nk) {
-    const int64_t slots = T == 256 ? 256 : 512;
+    const int64_t slots = T == 256 ? num_cus() : 2 * num_cus();   // one large or two small tiles per compute unit
     if (blocks <= 0 || blocks * 2 > slots) return 1;
     int64_t s = slots / blocks;
     if (s > nk / 8) s = nk / 8;
@@ -88,7 +102,7 @@ static DensePlan plan_dense(int64_t n_rows, int64_t Nout, int64_t nk) {
         p.split = ksplit_for(xq_cdiv(n_rows, 128) * xq_cdiv(Nout, 128), 128, nk);
         return p;
     }
-    const int64_t tr = xq_cdiv(n_rows, 256), tc = xq_cdiv(Nout, 256), cus = 256;
+    const int64_t tr = xq_cdiv(n_rows, 256), tc = xq_cdiv(Nout, 256), cus = num_cus();
     const int64_t full = tr * tc / cus, rem = tr * tc - full * cus;
     const int64_t keep = full * cus / tc;                  // tile rows that stay on whole rounds of large tiles
     if (rem == 0 || keep == 0 || keep >= tr) return p;

@@ -1,5 +1,6 @@
 // Low-rank helper kernels (see xq_lora.h).  bf16 MFMA, fp32 accumulate.
 #include "xq_lora.h"
+#include <atomic>
 
 namespace xq {
 
@@ -243,7 +244,7 @@ template <int TR, int FJ>
 static int launch_small_nt_one(const SmallNtArgs& g, unsigned blocks, hipStream_t stream) {
     constexpr int NT = (FJ + 7) / 8;
     constexpr size_t lds = (size_t)4 * (32 + NT * 32) * SN_P * 2;
-    static bool attr_set = false;
+    static std::atomic<bool> attr_set{false};   // the attribute call is idempotent: a race only repeats it
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute((const void*)small_nt_kernel<TR, FJ>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) {

@@ -22,6 +22,7 @@
 //      s = max(amax / 448, 1e-12) and writes e4m3(clamp(x / s)) bytes and the scale: decode -> add ->
 //      re-encode in one pass over 1 byte per weight each way.
 #include "xq_common.h"
+#include <atomic>
 #include "xq_lora.h"
 
 namespace xq {
@@ -374,7 +375,7 @@ static int launch_merge_one(const MergeArgs& g, dim3 grid, hipStream_t s, const 
     // LDS: the four factor tiles, then the delta half tile in their place
     constexpr size_t lds_f = (size_t)4 * MG_T * (RP + 8) * 2, lds_d = (size_t)MG_T * MG_HP * 4;
     constexpr size_t lds = RP == 0 ? 16 : (lds_f > lds_d ? lds_f : lds_d);
-    static bool attr_set = false;   // per instantiation
+    static std::atomic<bool> attr_set{false};   // per instantiation; the attribute call is idempotent: a race only repeats it
     if (!attr_set && lds > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute((const void*)merge_kernel<FMT, RP, REQ>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) {

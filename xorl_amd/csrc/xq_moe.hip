@@ -5,6 +5,7 @@
 //   scatter     ops/group_gemm/kernel/moe.py:266-312
 //   gather      ops/group_gemm/kernel/moe.py:102-141 (fp32 accumulate), :178-223 (add_gather)
 #include "xq_common.h"
+#include <atomic>
 
 namespace {
 
@@ -352,7 +353,7 @@ extern "C" int xq_route_build(const int32_t* selected, int64_t n_routed, int32_t
     int32_t* cc = (int32_t*)workspace;
     route_hist_kernel<<<dim3(n_chunks), 64, 0, stream>>>(selected, n_routed, num_experts, cc);
     XQ_CHECK_LAUNCH("route_hist");
-    static bool scan_attr_set = false;
+    static std::atomic<bool> scan_attr_set{false};   // the attribute call is idempotent: a race only repeats it
     if (!scan_attr_set) {
         if (hipFuncSetAttribute((const void*)route_scan_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 17 * RB_MAX_E * 4) != hipSuccess) {
             xq_set_error("xq_route_build: cannot raise the dynamic LDS limit");

@@ -22,6 +22,9 @@ import torch.nn as nn
 
 from .linear import (BlockFP8QLoRALinear, LoraModule, NF4QLoRALinear, NvFP4QLoRALinear, QLoRALinear,
                      deregister_qlora_weights_from_fsdp)
+
+# the name the reference's callers and tests import (qlora/utils.py:490-542)
+_deregister_qlora_weights_from_fsdp = deregister_qlora_weights_from_fsdp
 from .moe_experts import QLoRAMoeExperts
 
 SAFE_WEIGHTS_INDEX_NAME = "model.safetensors.index.json"
