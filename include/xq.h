@@ -308,6 +308,69 @@ int xq_grouped_lora_wgrad(const void* P, int64_t ldp, int64_t p_width, const voi
                           int r_out, int64_t n_rows, const int32_t* offsets, int32_t num_experts,
                           int transpose_out, float* out, void* workspace, const int32_t* row_limit, void* stream);
 
+/* ---- the routed expert MLP in two calls ------------------------------------
+ * xq_grouped_fwd / xq_grouped_bwd run the whole program of the reference's local LoRA expert compute
+ * (_MoeExpertsLoRAFunction.forward / .backward, ops/moe/lora.py:525-713 and :715-1007; registry entry
+ * MOE_EXPERT_BACKENDS_LORA, models/layers/moe/backend/__init__.py:421-445) on packed banks, composed from the entry
+ * points above on the caller's stream: route build, scatter, gate / up projections with LoRA, SwiGLU with the
+ * routing weight applied before the down projection, down projection with LoRA, top-k gather-sum; and its
+ * backward (dX, routing-weight gradients, the six factor gradients; the frozen banks get none).  A host without
+ * Python gets the routed MLP from these two calls.
+ *
+ * Banks are GKN: gate and up [E, H, I], down [E, I, H] (H, I multiples of 64).  LoRA factors in GKN form,
+ * A[p] [A_experts[p], in, r] and B[p] [B_experts[p], r, out] for p = 0 gate, 1 up, 2 down, each held once
+ * (shared by all experts: 1) or per expert (E); fp32 or bf16; r in 1..64.
+ *
+ * xq_grouped_saved names caller buffers the forward fills and the backward reads (R = n_tokens * topk routed
+ * rows, r_pad = r rounded up to 16): xs bf16 [R, H] (token rows in expert order), gate_out / up_out / h bf16
+ * [R, I], w_row fp32 [R], su_gate / su_up / su_down bf16 [R, r_pad], scatter_index int32 [R], offsets int32
+ * [E + 1], tile_offsets int32 [2 (E + 1)], counts int32 [E].  A forward-only caller passes scratch for them.
+ * Factor gradients are fp32, shaped like the factors, overwritten (exact zeros for experts without rows).
+ * hidden, out, dy, dx are bf16 [n_tokens, H] with row strides in elements; routing_w [n_tokens, topk] fp32 or
+ * bf16, selected int32 [n_tokens, topk]; dx / d_routing may be NULL.  Expert ids outside [0, E) drop their copy.
+ * workspace: xq_grouped_workspace_bytes(..., backward) bytes, 256-byte aligned. */
+typedef struct xq_grouped_lora {
+    const void* A[3];
+    const void* B[3];
+    int32_t A_experts[3];
+    int32_t B_experts[3];
+    int32_t dtype;      /* XQ_DT_* of all six factors */
+    int32_t r;
+    float scaling;
+    int32_t reserved;
+} xq_grouped_lora;
+
+typedef struct xq_grouped_saved {
+    void* xs;
+    void* gate_out;
+    void* up_out;
+    void* h;
+    float* w_row;
+    void* su_gate;
+    void* su_up;
+    void* su_down;
+    int32_t* scatter_index;
+    int32_t* offsets;
+    int32_t* tile_offsets;
+    int32_t* counts;
+} xq_grouped_saved;
+
+typedef struct xq_grouped_grads {
+    float* dA[3];
+    float* dB[3];
+} xq_grouped_grads;
+
+int64_t xq_grouped_workspace_bytes(int64_t n_tokens, int32_t topk, int32_t num_experts, int64_t hidden,
+                                   int64_t intermediate, int r, int backward);
+int xq_grouped_fwd(const xq_weight* gate, const xq_weight* up, const xq_weight* down, const xq_grouped_lora* lora,
+                   const void* hidden, int64_t ld_hidden, int64_t n_tokens, const void* routing_w, int rw_dtype,
+                   const int32_t* selected, int32_t topk, void* out, int64_t ld_out,
+                   const xq_grouped_saved* saved, void* workspace, int64_t workspace_bytes, void* stream);
+int xq_grouped_bwd(const xq_weight* gate, const xq_weight* up, const xq_weight* down, const xq_grouped_lora* lora,
+                   const void* dy, int64_t ld_dy, int64_t n_tokens, int32_t topk, const xq_grouped_saved* saved,
+                   void* dx, int64_t ld_dx, void* d_routing, int rw_dtype, const xq_grouped_grads* grads,
+                   void* workspace, int64_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

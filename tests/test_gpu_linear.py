@@ -327,7 +327,7 @@ def test_module_under_torch_compile(hip_device, backend):
     ref = tuple(t.clone() for t in ref)
     m.lora_A.grad = m.lora_B.grad = None
     torch._dynamo.reset()
-    got = _run(torch.compile(m, backend=backend), x, dy)
+    got = _run(torch.compile(m, backend=backend, fullgraph=True), x, dy)
     for a, b in zip(ref, got):
         assert torch.equal(a, b)
     qw = m._forward_quant_weight()

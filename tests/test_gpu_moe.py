@@ -582,3 +582,98 @@ def test_expert_merge_weights_matches_reference_arithmetic(hip_device, fmt, hybr
                     assert g.view(np.uint32).item() == np.float32(per[e][2]).view(np.uint32).item(), (round_, p, e)
             if fmt == "nvfp4":
                 assert torch.equal(m._ema_amax[p].cpu(), ema), (round_, p)
+
+
+@pytest.mark.parametrize("backend", ["eager", "aot_eager"])
+def test_expert_module_and_swiglu_under_torch_compile(hip_device, backend):
+    """Traced by torch.compile, the expert module and SwiGLU reach the library through registered custom ops
+    (xq::moe_fwd / moe_bwd, xq::silu_mul_fwd / silu_mul_bwd) with fake-tensor shape functions: outputs and every
+    gradient equal the eager call bit for bit, and the ops pass torch's schema and fake-tensor checks."""
+    from torch.library import opcheck
+
+    from xorl_amd import functional as Fn
+    from xorl_amd import moe_functional as MF
+
+    E, T, H, I, r, topk = 6, 200, 128, 192, 8, 2
+    m, _ = _make_experts("block_fp8", E, H, I, r, True, seed=90, device=hip_device)
+    rw, sel = _zipf_routing(T, E, topk, seed=91)
+    rw, sel = rw.to(torch.bfloat16).to(hip_device), sel.to(hip_device)
+    x = gen((T, H), 1.0, 92, torch.bfloat16).to(hip_device)
+    dy = gen((T, H), 1.0, 93, torch.bfloat16).to(hip_device)
+    names = [f"{k}_proj_lora_{f}" for k in ("gate", "up", "down") for f in ("A", "B")]
+
+    def run(mod):
+        for n in names:
+            getattr(m, n).grad = None
+        xd, rwd = x.clone().requires_grad_(True), rw.clone().requires_grad_(True)
+        y = mod(xd, rwd, sel)
+        y.backward(dy)
+        return [y.detach().clone(), xd.grad.clone(), rwd.grad.clone()] + [getattr(m, n).grad.clone() for n in names]
+
+    ref = run(m)
+    torch._dynamo.reset()
+    got = run(torch.compile(m, backend=backend, fullgraph=True))
+    for a, b in zip(ref, got):
+        assert torch.equal(a, b)
+
+    # SwiGLU
+    g = gen((T, I), 2.0, 94).to(torch.bfloat16).to(hip_device)
+    u = gen((T, I), 1.0, 95, torch.bfloat16).to(hip_device)
+    dh = gen((T, I), 1.0, 96, torch.bfloat16).to(hip_device)
+
+    def run_silu(fn):
+        gd, ud = g.clone().requires_grad_(True), u.clone().requires_grad_(True)
+        h = fn(gd, ud)
+        h.backward(dh)
+        return h.detach(), gd.grad, ud.grad
+
+    ref = run_silu(Fn.silu_and_mul)
+    torch._dynamo.reset()
+    got = run_silu(torch.compile(Fn.silu_and_mul, backend=backend, fullgraph=True))
+    for a, b in zip(ref, got):
+        assert torch.equal(a, b)
+
+    if backend == "eager":
+        ok = {"SUCCESS"}
+        assert set(opcheck(Fn._silu_fwd_op, (g, u), test_utils=("test_schema", "test_faketensor")).values()) == ok
+        assert set(opcheck(Fn._silu_bwd_op, (g, u, dh), test_utils=("test_schema", "test_faketensor")).values()) == ok
+        qg, qu, qd = m._bank("gate"), m._bank("up"), m._bank("down")
+        f = [getattr(m, n).detach().contiguous() for n in names]
+        args = (x, rw, sel, *f, qg.packed, qg.scales, qg.global_scale, qu.packed, qu.scales, qu.global_scale, qd.packed,
+                qd.scales, qd.global_scale, qg.fmt, qg.layout, Fn._DT_TO_CODE[qg.scale_dtype], qg.group, E, H, I, r, 2.0)
+        assert set(opcheck(MF._moe_fwd_op, args, test_utils=("test_schema", "test_faketensor")).values()) == ok
+
+
+def test_grouped_low_rank_entry_points(hip_device):
+    """xq_factor_prep, xq_grouped_lora_down and xq_grouped_lora_wgrad one at a time against plain torch arithmetic
+    on the same bf16 operands (fp32 accumulation; the products are small enough for float64 to be the yardstick)."""
+    from xorl_amd import moe_functional as MF
+
+    E, K, r, rp, width = 5, 256, 12, 16, 192
+    counts = torch.tensor([70, 0, 300, 1, 129])
+    R_ = int(counts.sum())
+    sel = torch.arange(E, dtype=torch.int32).repeat_interleave(counts).reshape(-1, 1).to(hip_device)
+    _, offsets, _, tile_offsets = MF.route_build(sel, E)
+    F32 = gen((E, K, r), 0.1, 1)                                            # a per-expert A factor [E, in, r]
+    F = MF._prep(F32.to(hip_device), True, rp, K)                           # -> bf16 [E, rp, K], zero padded
+    want = torch.zeros(E, rp, K)
+    want[:, :r] = F32.transpose(1, 2).to(torch.bfloat16).float()
+    assert torch.equal(F.float().cpu(), want)
+    a = gen((R_, K), 1.0, 2, torch.bfloat16)
+    t = MF._lora_down(a.to(hip_device), F, offsets, tile_offsets, E, 0.5).cpu()        # [R, rp] = bf16(0.5 * a . F[e]^T)
+    ends = counts.cumsum(0)
+    e_of = torch.searchsorted(ends, torch.arange(R_), right=True)
+    ref_t = 0.5 * torch.einsum("rk,rjk->rj", a.double(), want.double()[e_of])
+    close(t, ref_t, 1e-2, rows="none")
+    assert torch.count_nonzero(t[:, r:]) == 0
+    P = gen((R_, width), 1.0, 3, torch.bfloat16)
+    g = MF._wgrad(P.to(hip_device), t.to(hip_device), r, offsets, E, False).cpu()       # [E, width, r]
+    for e in range(E):
+        lo, hi = int(ends[e] - counts[e]), int(ends[e])
+        ref = P[lo:hi].double().t() @ t[lo:hi, :r].double()
+        if hi == lo:
+            assert torch.count_nonzero(g[e]) == 0
+        else:
+            close(g[e], ref, 1e-2, rows="none")
+    g1 = MF._wgrad(P.to(hip_device), t.to(hip_device), r, None, E, True).cpu()          # one product over all rows, [1, r, width]
+    close(g1[0], t[:, :r].double().t() @ P.double(), 1e-2, rows="none")

@@ -40,6 +40,21 @@ class XqWeight(ctypes.Structure):
     ]
 
 
+class XqGroupedLora(ctypes.Structure):
+    _fields_ = [("A", ctypes.c_void_p * 3), ("B", ctypes.c_void_p * 3), ("A_experts", ctypes.c_int32 * 3),
+                ("B_experts", ctypes.c_int32 * 3), ("dtype", ctypes.c_int32), ("r", ctypes.c_int32),
+                ("scaling", ctypes.c_float), ("reserved", ctypes.c_int32)]
+
+
+class XqGroupedSaved(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_void_p) for n in ("xs", "gate_out", "up_out", "h", "w_row", "su_gate", "su_up", "su_down",
+                                               "scatter_index", "offsets", "tile_offsets", "counts")]
+
+
+class XqGroupedGrads(ctypes.Structure):
+    _fields_ = [("dA", ctypes.c_void_p * 3), ("dB", ctypes.c_void_p * 3)]
+
+
 class XqError(ValueError):
     """Argument error reported by the library before any launch."""
 
@@ -95,6 +110,14 @@ _SIGNATURES = {
     "xq_lora_wgrad_workspace_bytes": (_I64, [_I64, _I64, _INT]),
     # P, ldp, p_width, Q, r_pad, r_out, n_rows, offsets, E, transpose_out, out, ws, row_limit, stream
     "xq_grouped_lora_wgrad": (_INT, [_P, _I64, _I64, _P, _INT, _INT, _I64, _P, _I32, _INT, _P, _P, _P, _P]),
+    "xq_grouped_workspace_bytes": (_I64, [_I64, _I32, _I32, _I64, _I64, _INT, _INT]),
+    # gate, up, down, lora, hidden, ld_hidden, n_tokens, routing_w, rw_dtype, selected, topk, out, ld_out, saved, ws, ws_bytes, stream
+    "xq_grouped_fwd": (_INT, [_W, _W, _W, ctypes.POINTER(XqGroupedLora), _P, _I64, _I64, _P, _INT, _P, _I32, _P, _I64,
+                              ctypes.POINTER(XqGroupedSaved), _P, _I64, _P]),
+    # gate, up, down, lora, dy, ld_dy, n_tokens, topk, saved, dx, ld_dx, d_routing, rw_dtype, grads, ws, ws_bytes, stream
+    "xq_grouped_bwd": (_INT, [_W, _W, _W, ctypes.POINTER(XqGroupedLora), _P, _I64, _I64, _I32,
+                              ctypes.POINTER(XqGroupedSaved), _P, _I64, _P, _INT, ctypes.POINTER(XqGroupedGrads), _P, _I64,
+                              _P]),
 }
 
 EXPORTS = ("xq_version", "xq_last_error") + tuple(_SIGNATURES)

@@ -1,0 +1,282 @@
+// xq_grouped_fwd / xq_grouped_bwd: the routed SwiGLU expert MLP with LoRA on packed expert banks as two calls.
+// Host code only: the program of the reference's _MoeExpertsLoRAFunction (ops/moe/lora.py:525-1007) composed from
+// this library's kernels on the caller's stream -- routing, row movement, the fused dequant-GEMMs on the packed
+// banks, the low-rank helpers and SwiGLU.  Nothing is allocated: temporaries are carved from the caller's workspace,
+// tensors the backward needs live in caller buffers named by xq_grouped_saved.
+#include "xq_lora.h"
+
+namespace xq {
+int launch_tile_gemm(const xq_weight* w, bool contract_cols, const bf16_t* A, int64_t lda, int64_t n_rows,
+                     const int32_t* offsets, const int32_t* tile_offsets, const bf16_t* su, const bf16_t* lora_right,
+                     int r_pad, const bf16_t* bias, bf16_t* C, int64_t ldc, hipStream_t stream, const char* who,
+                     float* partial, int64_t partial_bytes);
+
+namespace {
+
+inline int64_t al256(int64_t b) { return (b + 255) & ~(int64_t)255; }
+inline int r_pad_of(int r) { return ((r + 15) / 16) * 16; }
+
+struct Carve {
+    uint8_t* base;
+    int64_t used;
+    template <typename T>
+    T* take(int64_t bytes) {
+        T* p = (T*)(base + used);
+        used += al256(bytes);
+        return p;
+    }
+};
+
+// ---- every LoRA panel of a call in one launch: job k converts a [n_src, R_in, C_in] fp32 / bf16 factor (n_src = 1
+// or the expert count) into bf16 [n_out, R_out, C_out], optionally transposed, zero padded; n_src == 1 < n_out
+// repeats the one source matrix for every expert (a factor shared by all experts, handed to a kernel that indexes
+// panels by expert).
+constexpr int MAX_PREP_JOBS = 6;
+struct PrepJobs {
+    const void* in[MAX_PREP_JOBS];
+    bf16_t* out[MAX_PREP_JOBS];
+    int64_t R_in[MAX_PREP_JOBS], C_in[MAX_PREP_JOBS], R_out[MAX_PREP_JOBS], C_out[MAX_PREP_JOBS];
+    int32_t n_src[MAX_PREP_JOBS], n_out[MAX_PREP_JOBS], transpose[MAX_PREP_JOBS];
+    int32_t in_f32, n;
+    bf16_t* add(const void* src, int n_src_, int64_t r_in, int64_t c_in, bool tr, bf16_t* dst, int n_out_, int64_t r_out, int64_t c_out) {
+        in[n] = src; out[n] = dst; R_in[n] = r_in; C_in[n] = c_in; R_out[n] = r_out; C_out[n] = c_out;
+        n_src[n] = n_src_; n_out[n] = n_out_; transpose[n] = tr ? 1 : 0;
+        ++n;
+        return dst;
+    }
+};
+
+__global__ void __launch_bounds__(256) grouped_prep_kernel(PrepJobs j) {
+    const int k = blockIdx.y;
+    const int64_t per = j.R_out[k] * j.C_out[k], total = per * j.n_out[k];
+    const int64_t R_in = j.R_in[k], C_in = j.C_in[k], C_out = j.C_out[k];
+    const bool tr = j.transpose[k] != 0, shared = j.n_src[k] == 1;
+    for (int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x; t < total; t += (int64_t)gridDim.x * 256) {
+        const int64_t e = t / per, rem = t - e * per;
+        const int64_t i = rem / C_out, c = rem - i * C_out;
+        const int64_t si = tr ? c : i, sj = tr ? i : c;
+        float v = 0.0f;
+        if (si < R_in && sj < C_in) {
+            const int64_t idx = (shared ? 0 : e) * R_in * C_in + si * C_in + sj;
+            v = j.in_f32 ? ((const float*)j.in[k])[idx] : bf16_to_f32(((const bf16_t*)j.in[k])[idx]);
+        }
+        j.out[k][t] = to_bf16(v);
+    }
+}
+
+int launch_prep(const PrepJobs& j, hipStream_t stream) {
+    int64_t most = 0;
+    for (int k = 0; k < j.n; ++k) {
+        const int64_t t = j.R_out[k] * j.C_out[k] * j.n_out[k];
+        most = t > most ? t : most;
+    }
+    if (j.n == 0 || most == 0) return XQ_OK;
+    int64_t blocks = xq_cdiv(most, 256);
+    if (blocks > 4096) blocks = 4096;
+    grouped_prep_kernel<<<dim3((unsigned)blocks, (unsigned)j.n), 256, 0, stream>>>(j);
+    XQ_CHECK_LAUNCH("grouped_prep");
+    return XQ_OK;
+}
+
+struct Dims {
+    int32_t E, topk, r, rp;
+    int64_t T, R, H, I;
+};
+
+int check_call(const xq_weight* gate, const xq_weight* up, const xq_weight* down, const xq_grouped_lora* lora,
+               int64_t n_tokens, int32_t topk, const xq_grouped_saved* saved, const char* who, Dims* d) {
+    XQ_REQUIRE(gate && up && down && lora && saved, "%s: NULL descriptor", who);
+    int rc;
+    if ((rc = xq_validate_weight(gate, who)) || (rc = xq_validate_weight(up, who)) || (rc = xq_validate_weight(down, who))) return rc;
+    const int32_t E = gate->num_experts;
+    XQ_REQUIRE(up->num_experts == E && down->num_experts == E, "%s: the three banks hold %d / %d / %d experts", who, E,
+               up->num_experts, down->num_experts);
+    const int64_t H = gate->rows, I = gate->cols;
+    XQ_REQUIRE(up->rows == H && up->cols == I && down->rows == I && down->cols == H,
+               "%s: bank shapes do not make an MLP (gate [%lld, %lld], up [%lld, %lld], down [%lld, %lld])", who,
+               (long long)H, (long long)I, (long long)up->rows, (long long)up->cols, (long long)down->rows, (long long)down->cols);
+    XQ_REQUIRE(H % 64 == 0 && I % 64 == 0, "%s: hidden size %lld and intermediate size %lld must be multiples of 64", who,
+               (long long)H, (long long)I);
+    XQ_REQUIRE(n_tokens >= 0 && topk >= 1 && n_tokens * topk < (1ll << 31), "%s: bad token count / top-k", who);
+    XQ_REQUIRE(lora->r >= 1 && lora->r <= 64, "%s: LoRA rank %d out of range [1, 64]", who, lora->r);
+    XQ_REQUIRE(lora->dtype == XQ_DT_F32 || lora->dtype == XQ_DT_BF16, "%s: bad lora dtype", who);
+    for (int p = 0; p < 3; ++p) {
+        XQ_REQUIRE(lora->A[p] && lora->B[p], "%s: LoRA factor %d is NULL", who, p);
+        XQ_REQUIRE((lora->A_experts[p] == 1 || lora->A_experts[p] == E) && (lora->B_experts[p] == 1 || lora->B_experts[p] == E),
+                   "%s: a LoRA factor holds 1 (shared) or %d matrices", who, E);
+    }
+    d->E = E; d->topk = topk; d->r = lora->r; d->rp = r_pad_of(lora->r);
+    d->T = n_tokens; d->R = n_tokens * topk; d->H = H; d->I = I;
+    if (d->R > 0)
+        XQ_REQUIRE(saved->xs && saved->gate_out && saved->up_out && saved->h && saved->w_row && saved->su_gate && saved->su_up &&
+                       saved->su_down && saved->scatter_index,
+                   "%s: a buffer of xq_grouped_saved is NULL", who);
+    XQ_REQUIRE(saved->offsets && saved->tile_offsets && saved->counts, "%s: a routing buffer of xq_grouped_saved is NULL", who);
+    return XQ_OK;
+}
+
+int64_t fwd_workspace(const Dims& d) {
+    const int64_t panels = 2 * al256((int64_t)d.E * d.rp * d.H * 2) + 2 * al256((int64_t)d.E * d.I * d.rp * 2) +
+                           al256((int64_t)d.E * d.rp * d.I * 2) + al256((int64_t)d.E * d.H * d.rp * 2);
+    return al256(xq_route_workspace_bytes(d.R, d.E)) + panels + al256(d.R * d.H * 2) + 256;
+}
+
+int64_t bwd_workspace(const Dims& d) {
+    const int64_t EH = al256((int64_t)d.E * d.rp * d.H * 2), EI = al256((int64_t)d.E * d.rp * d.I * 2);
+    const int64_t panels = 3 * EH + 3 * EI;     // F_dB, Lr_gA, Lr_uA over H; Lr_dA, F_gB, F_uB over I
+    const int64_t wide = d.H > d.I ? d.H : d.I;
+    const int64_t wg = al256(xq_lora_wgrad_workspace_bytes(d.R, wide, d.rp));
+    return panels + 3 * al256(d.R * d.H * 2) + 3 * al256(d.R * d.I * 2) + al256(d.R * 4) + 3 * al256(d.R * d.rp * 2) + wg + 256;
+}
+
+}  // namespace
+}  // namespace xq
+
+using namespace xq;
+
+extern "C" int64_t xq_grouped_workspace_bytes(int64_t n_tokens, int32_t topk, int32_t num_experts, int64_t hidden,
+                                              int64_t intermediate, int r, int backward) {
+    if (n_tokens < 0 || topk < 1 || num_experts < 1 || r < 1) return 0;
+    Dims d{num_experts, topk, r, r_pad_of(r), n_tokens, n_tokens * topk, hidden, intermediate};
+    return backward ? bwd_workspace(d) : fwd_workspace(d);
+}
+
+extern "C" int xq_grouped_fwd(const xq_weight* gate, const xq_weight* up, const xq_weight* down, const xq_grouped_lora* lora,
+                              const void* hidden, int64_t ld_hidden, int64_t n_tokens, const void* routing_w, int rw_dtype,
+                              const int32_t* selected, int32_t topk, void* out, int64_t ld_out,
+                              const xq_grouped_saved* saved, void* workspace, int64_t workspace_bytes, void* stream_) {
+    static const char* who = "xq_grouped_fwd";
+    Dims d;
+    int rc = check_call(gate, up, down, lora, n_tokens, topk, saved, who, &d);
+    if (rc) return rc;
+    XQ_REQUIRE(rw_dtype == XQ_DT_F32 || rw_dtype == XQ_DT_BF16, "%s: routing weights are fp32 or bf16", who);
+    XQ_REQUIRE(workspace && xq_aligned(workspace, 256) && workspace_bytes >= fwd_workspace(d),
+               "%s: workspace missing, misaligned or smaller than xq_grouped_workspace_bytes()", who);
+    XQ_REQUIRE(d.T == 0 || (hidden && routing_w && selected && out), "%s: NULL tensor", who);
+    hipStream_t stream = (hipStream_t)stream_;
+    const int E = d.E, rp = d.rp;
+    const int64_t R = d.R, H = d.H, I = d.I;
+    const float s = lora->scaling;
+    Carve cv{(uint8_t*)workspace, 0};
+    void* route_ws = cv.take<uint8_t>(xq_route_workspace_bytes(R, E));
+    const int64_t route_ws_bytes = al256(xq_route_workspace_bytes(R, E));
+
+    if ((rc = xq_route_build(selected, R, E, saved->counts, saved->offsets, saved->scatter_index, saved->tile_offsets,
+                             route_ws, route_ws_bytes, stream)))
+        return rc;
+    if (R == 0) return XQ_OK;
+    bf16_t* xs = (bf16_t*)saved->xs;
+    if ((rc = xq_moe_scatter(hidden, ld_hidden, saved->scatter_index, R, topk, H, xs, H, stream))) return rc;
+
+    // bf16 operand layouts of the six factors, one launch.  A factors [E|1, in, r] become the "down" panels
+    // [E|1, rp, in] of x . A; B factors [E|1, r, out] become the per-expert right-hand panels [E, out, rp].
+    PrepJobs jobs{};
+    jobs.in_f32 = lora->dtype == XQ_DT_F32;
+    const int gAe = lora->A_experts[0], uAe = lora->A_experts[1], dAe = lora->A_experts[2];
+    bf16_t* F_gA = jobs.add(lora->A[0], gAe, H, d.r, true, cv.take<bf16_t>((int64_t)gAe * rp * H * 2), gAe, rp, H);
+    bf16_t* F_uA = jobs.add(lora->A[1], uAe, H, d.r, true, cv.take<bf16_t>((int64_t)uAe * rp * H * 2), uAe, rp, H);
+    bf16_t* Lr_gB = jobs.add(lora->B[0], lora->B_experts[0], d.r, I, true, cv.take<bf16_t>((int64_t)E * I * rp * 2), E, I, rp);
+    bf16_t* Lr_uB = jobs.add(lora->B[1], lora->B_experts[1], d.r, I, true, cv.take<bf16_t>((int64_t)E * I * rp * 2), E, I, rp);
+    bf16_t* F_dA = jobs.add(lora->A[2], dAe, I, d.r, true, cv.take<bf16_t>((int64_t)dAe * rp * I * 2), dAe, rp, I);
+    bf16_t* Lr_dB = jobs.add(lora->B[2], lora->B_experts[2], d.r, H, true, cv.take<bf16_t>((int64_t)E * H * rp * 2), E, H, rp);
+    if ((rc = launch_prep(jobs, stream))) return rc;
+    bf16_t* down_out = cv.take<bf16_t>(R * H * 2);
+
+    const int32_t *off = saved->offsets, *toff = saved->tile_offsets;
+    bf16_t *su_g = (bf16_t*)saved->su_gate, *su_u = (bf16_t*)saved->su_up, *su_d = (bf16_t*)saved->su_down;
+    bf16_t *gate_out = (bf16_t*)saved->gate_out, *up_out = (bf16_t*)saved->up_out, *h = (bf16_t*)saved->h;
+    if ((rc = launch_small_nt(xs, H, R, H, F_gA, rp, s, su_g, off, toff, E, gAe == 1, stream))) return rc;
+    if ((rc = launch_small_nt(xs, H, R, H, F_uA, rp, s, su_u, off, toff, E, uAe == 1, stream))) return rc;
+    if ((rc = launch_tile_gemm(gate, false, xs, H, R, off, toff, su_g, Lr_gB, rp, nullptr, gate_out, I, stream, who, nullptr, 0))) return rc;
+    if ((rc = launch_tile_gemm(up, false, xs, H, R, off, toff, su_u, Lr_uB, rp, nullptr, up_out, I, stream, who, nullptr, 0))) return rc;
+    if ((rc = xq_moe_scatter_scalar(routing_w, rw_dtype, saved->scatter_index, R, saved->w_row, stream))) return rc;
+    if ((rc = xq_silu_mul_fwd(gate_out, up_out, I, saved->w_row, h, I, R, I, stream))) return rc;
+    if ((rc = launch_small_nt(h, I, R, I, F_dA, rp, s, su_d, off, toff, E, dAe == 1, stream))) return rc;
+    if ((rc = launch_tile_gemm(down, false, h, I, R, off, toff, su_d, Lr_dB, rp, nullptr, down_out, H, stream, who, nullptr, 0))) return rc;
+    return xq_moe_gather(down_out, nullptr, H, saved->scatter_index, d.T, topk, H, out, ld_out, stream);
+}
+
+extern "C" int xq_grouped_bwd(const xq_weight* gate, const xq_weight* up, const xq_weight* down, const xq_grouped_lora* lora,
+                              const void* dy, int64_t ld_dy, int64_t n_tokens, int32_t topk, const xq_grouped_saved* saved,
+                              void* dx, int64_t ld_dx, void* d_routing, int rw_dtype, const xq_grouped_grads* grads,
+                              void* workspace, int64_t workspace_bytes, void* stream_) {
+    static const char* who = "xq_grouped_bwd";
+    Dims d;
+    int rc = check_call(gate, up, down, lora, n_tokens, topk, saved, who, &d);
+    if (rc) return rc;
+    XQ_REQUIRE(grads, "%s: grads is NULL", who);
+    for (int p = 0; p < 3; ++p) XQ_REQUIRE(grads->dA[p] && grads->dB[p], "%s: a factor gradient buffer is NULL", who);
+    XQ_REQUIRE(!d_routing || rw_dtype == XQ_DT_F32 || rw_dtype == XQ_DT_BF16, "%s: routing-weight gradients are fp32 or bf16", who);
+    XQ_REQUIRE(workspace && xq_aligned(workspace, 256) && workspace_bytes >= bwd_workspace(d),
+               "%s: workspace missing, misaligned or smaller than xq_grouped_workspace_bytes()", who);
+    hipStream_t stream = (hipStream_t)stream_;
+    const int E = d.E, r = d.r, rp = d.rp;
+    const int64_t R = d.R, H = d.H, I = d.I;
+    const float s = lora->scaling;
+    if (R == 0) {      // no rows: every factor gradient is zero
+        for (int p = 0; p < 3; ++p) {
+            const int64_t in = p == 2 ? I : H, outw = p == 2 ? H : I;
+            if ((rc = launch_zero_fill(grads->dA[p], (int64_t)lora->A_experts[p] * in * r * 4, stream))) return rc;
+            if ((rc = launch_zero_fill(grads->dB[p], (int64_t)lora->B_experts[p] * r * outw * 4, stream))) return rc;
+        }
+        return XQ_OK;
+    }
+    XQ_REQUIRE(dy, "%s: dy is NULL", who);
+    Carve cv{(uint8_t*)workspace, 0};
+    const int32_t *off = saved->offsets, *toff = saved->tile_offsets, *sidx = saved->scatter_index;
+    const int32_t* n_valid = off + E;     // rows that belong to an expert (all of them unless an id was out of range)
+    const bf16_t *xs = (const bf16_t*)saved->xs, *gate_out = (const bf16_t*)saved->gate_out, *up_out = (const bf16_t*)saved->up_out;
+    const bf16_t *h = (const bf16_t*)saved->h, *su_g = (const bf16_t*)saved->su_gate, *su_u = (const bf16_t*)saved->su_up;
+    const bf16_t* su_d = (const bf16_t*)saved->su_down;
+
+    // every panel of the call in one launch: B factors [E|1, r, out] as the "down" panels [E|1, rp, out] of g . B^T,
+    // A factors [E|1, in, r] as the per-expert right-hand panels [E, in, rp] of the dgrads
+    PrepJobs jobs{};
+    jobs.in_f32 = lora->dtype == XQ_DT_F32;
+    const int gBe = lora->B_experts[0], uBe = lora->B_experts[1], dBe = lora->B_experts[2];
+    const int gAe = lora->A_experts[0], uAe = lora->A_experts[1], dAe = lora->A_experts[2];
+    bf16_t* F_dB = jobs.add(lora->B[2], dBe, r, H, false, cv.take<bf16_t>((int64_t)dBe * rp * H * 2), dBe, rp, H);
+    bf16_t* Lr_dA = jobs.add(lora->A[2], dAe, I, r, false, cv.take<bf16_t>((int64_t)E * I * rp * 2), E, I, rp);
+    bf16_t* F_uB = jobs.add(lora->B[1], uBe, r, I, false, cv.take<bf16_t>((int64_t)uBe * rp * I * 2), uBe, rp, I);
+    bf16_t* Lr_uA = jobs.add(lora->A[1], uAe, H, r, false, cv.take<bf16_t>((int64_t)E * H * rp * 2), E, H, rp);
+    bf16_t* F_gB = jobs.add(lora->B[0], gBe, r, I, false, cv.take<bf16_t>((int64_t)gBe * rp * I * 2), gBe, rp, I);
+    bf16_t* Lr_gA = jobs.add(lora->A[0], gAe, H, r, false, cv.take<bf16_t>((int64_t)E * H * rp * 2), E, H, rp);
+    if ((rc = launch_prep(jobs, stream))) return rc;
+
+    bf16_t* g_down = cv.take<bf16_t>(R * H * 2);
+    bf16_t* dx_g = cv.take<bf16_t>(R * H * 2);
+    bf16_t* dx_u = cv.take<bf16_t>(R * H * 2);
+    bf16_t* dh = cv.take<bf16_t>(R * I * 2);
+    bf16_t* dgate = cv.take<bf16_t>(R * I * 2);
+    bf16_t* dup = cv.take<bf16_t>(R * I * 2);
+    float* d_w_row = cv.take<float>(R * 4);
+    bf16_t* v_d = cv.take<bf16_t>(R * rp * 2);
+    bf16_t* v_g = cv.take<bf16_t>(R * rp * 2);
+    bf16_t* v_u = cv.take<bf16_t>(R * rp * 2);
+    float* wg = cv.take<float>(0);
+
+    if ((rc = xq_moe_scatter(dy, ld_dy, sidx, R, topk, H, g_down, H, stream))) return rc;
+
+    // ---- down projection: y = h.W + s*(h.A).B
+    if ((rc = launch_small_nt(g_down, H, R, H, F_dB, rp, s, v_d, off, toff, E, dBe == 1, stream))) return rc;        // s * g . B^T
+    if ((rc = launch_tile_gemm(down, true, g_down, H, R, off, toff, v_d, Lr_dA, rp, nullptr, dh, I, stream, who, nullptr, 0))) return rc;
+    if ((rc = launch_tn(g_down, H, H, su_d, rp, r, R, true, grads->dB[2], wg, dBe == 1 ? nullptr : off, E, stream, n_valid))) return rc;   // [E|1, r, H]
+    if ((rc = launch_tn(h, I, I, v_d, rp, r, R, false, grads->dA[2], wg, dAe == 1 ? nullptr : off, E, stream, n_valid))) return rc;        // [E|1, I, r]
+
+    // ---- SwiGLU + routing weight
+    if ((rc = xq_silu_mul_bwd(gate_out, up_out, I, dh, I, saved->w_row, dgate, dup, I, d_w_row, R, I, stream))) return rc;
+    if (d_routing && (rc = xq_moe_gather_scalar(d_w_row, sidx, R, d_routing, rw_dtype, stream))) return rc;
+
+    // ---- up / gate projections: y = x.W + s*(x.A).B
+    if ((rc = launch_small_nt(dup, I, R, I, F_uB, rp, s, v_u, off, toff, E, uBe == 1, stream))) return rc;
+    if ((rc = launch_tile_gemm(up, true, dup, I, R, off, toff, v_u, Lr_uA, rp, nullptr, dx_u, H, stream, who, nullptr, 0))) return rc;
+    if ((rc = launch_tn(dup, I, I, su_u, rp, r, R, true, grads->dB[1], wg, uBe == 1 ? nullptr : off, E, stream, n_valid))) return rc;      // [E|1, r, I]
+    if ((rc = launch_small_nt(dgate, I, R, I, F_gB, rp, s, v_g, off, toff, E, gBe == 1, stream))) return rc;
+    if ((rc = launch_tile_gemm(gate, true, dgate, I, R, off, toff, v_g, Lr_gA, rp, nullptr, dx_g, H, stream, who, nullptr, 0))) return rc;
+    if ((rc = launch_tn(dgate, I, I, su_g, rp, r, R, true, grads->dB[0], wg, gBe == 1 ? nullptr : off, E, stream, n_valid))) return rc;
+    // gradients of the two A factors, [E|1, H, r] = x^T . v
+    if ((rc = launch_tn(xs, H, H, v_g, rp, r, R, false, grads->dA[0], wg, gAe == 1 ? nullptr : off, E, stream, n_valid))) return rc;
+    if ((rc = launch_tn(xs, H, H, v_u, rp, r, R, false, grads->dA[1], wg, uAe == 1 ? nullptr : off, E, stream, n_valid))) return rc;
+    if (dx) return xq_moe_gather(dx_g, dx_u, H, sidx, d.T, topk, H, dx, ld_dx, stream);
+    return XQ_OK;
+}

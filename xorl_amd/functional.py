@@ -65,6 +65,8 @@ def _lora_dt(t: Optional[Tensor]) -> int:
 
 def _as_2d(x: Tensor) -> Tensor:
     x2 = x.reshape(-1, x.shape[-1])
+    if torch.compiler.is_compiling():      # addresses are not traceable: a traced call always takes a packed copy
+        return x2.contiguous()
     if x2.stride(-1) != 1 or (x2.shape[0] > 1 and x2.stride(0) % 8 != 0) or x2.data_ptr() % 16 != 0:
         x2 = x2.contiguous()
     return x2
@@ -264,19 +266,55 @@ def qlora_linear(x: Tensor, qw: QuantWeight, lora_A: Optional[Tensor], lora_B: O
 # ---------------------------------------------------------------------------
 # SwiGLU
 # ---------------------------------------------------------------------------
+def _silu_fwd_impl(g2: Tensor, u2: Tensor) -> Tensor:
+    rows, cols = g2.shape
+    h = torch.empty(rows, cols, dtype=torch.bfloat16, device=g2.device)
+    _C.check(_C.lib().xq_silu_mul_fwd(g2.data_ptr(), u2.data_ptr(), _ld(g2), None, h.data_ptr(), cols, rows, cols,
+                                      _C.stream_ptr(g2.device)))
+    return h
+
+
+def _silu_bwd_impl(g2: Tensor, u2: Tensor, d2: Tensor) -> Tuple[Tensor, Tensor]:
+    rows, cols = g2.shape
+    dg = torch.empty(rows, cols, dtype=torch.bfloat16, device=g2.device)
+    du = torch.empty(rows, cols, dtype=torch.bfloat16, device=g2.device)
+    _C.check(_C.lib().xq_silu_mul_bwd(g2.data_ptr(), u2.data_ptr(), _ld(g2), d2.data_ptr(), _ld(d2), None,
+                                      dg.data_ptr(), du.data_ptr(), cols, None, rows, cols, _C.stream_ptr(g2.device)))
+    return dg, du
+
+
+@torch.library.custom_op("xq::silu_mul_fwd", mutates_args=(), device_types="cuda")
+def _silu_fwd_op(gate: Tensor, up: Tensor) -> Tensor:
+    return _silu_fwd_impl(gate, up)
+
+
+@_silu_fwd_op.register_fake
+def _(gate, up):
+    return gate.new_empty(gate.shape)
+
+
+@torch.library.custom_op("xq::silu_mul_bwd", mutates_args=(), device_types="cuda")
+def _silu_bwd_op(gate: Tensor, up: Tensor, dh: Tensor) -> Tuple[Tensor, Tensor]:
+    return _silu_bwd_impl(gate, up, dh)
+
+
+@_silu_bwd_op.register_fake
+def _(gate, up, dh):
+    return gate.new_empty(gate.shape), gate.new_empty(gate.shape)
+
+
 class SiluAndMulFunction(torch.autograd.Function):
     """fused_silu_and_mul (ops/fused_silu_and_mul.py): h = bf16(silu(gate)) * up."""
 
     @staticmethod
     def forward(ctx, gate: Tensor, up: Tensor):
         _C.require_hip(gate, up)
+        if gate.dtype != torch.bfloat16 or up.dtype != torch.bfloat16:
+            raise _C.XqError(f"silu_and_mul takes bf16 tensors, got {gate.dtype} and {up.dtype}")
         g2, u2 = _as_2d(gate), _as_2d(up)
-        if _ld(g2) != _ld(u2):
+        if _ld(g2) != _ld(u2) or torch.compiler.is_compiling():
             g2, u2 = g2.contiguous(), u2.contiguous()
-        rows, cols = g2.shape
-        h = torch.empty(rows, cols, dtype=torch.bfloat16, device=gate.device)
-        _C.check(_C.lib().xq_silu_mul_fwd(g2.data_ptr(), u2.data_ptr(), _ld(g2), None, h.data_ptr(), cols, rows, cols,
-                                          _C.stream_ptr(gate.device)))
+        h = _silu_fwd_op(g2, u2) if torch.compiler.is_compiling() else _silu_fwd_impl(g2, u2)
         ctx.save_for_backward(g2, u2)
         ctx.shape = gate.shape
         return h.reshape(gate.shape)
@@ -284,13 +322,11 @@ class SiluAndMulFunction(torch.autograd.Function):
     @staticmethod
     def backward(ctx, dh):
         g2, u2 = ctx.saved_tensors
-        rows, cols = g2.shape
         d2 = _as_2d(dh.to(torch.bfloat16))
-        dg = torch.empty(rows, cols, dtype=torch.bfloat16, device=dh.device)
-        du = torch.empty(rows, cols, dtype=torch.bfloat16, device=dh.device)
-        _C.check(_C.lib().xq_silu_mul_bwd(g2.data_ptr(), u2.data_ptr(), _ld(g2), d2.data_ptr(), _ld(d2), None,
-                                          dg.data_ptr(), du.data_ptr(), cols, None, rows, cols,
-                                          _C.stream_ptr(dh.device)))
+        if torch.compiler.is_compiling():
+            dg, du = _silu_bwd_op(g2, u2, d2.contiguous())
+        else:
+            dg, du = _silu_bwd_impl(g2, u2, d2)
         return dg.reshape(ctx.shape), du.reshape(ctx.shape)
 
 

@@ -13,13 +13,13 @@ qlora/modules/moe_experts.py:486-498).
 from __future__ import annotations
 
 import ctypes
-from typing import Dict, Optional, Tuple
+from typing import Dict, List, Optional, Tuple
 
 import torch
 from torch import Tensor
 
 from . import _C
-from .functional import QuantWeight, _r_pad
+from .functional import _CODE_TO_DT, _DT_TO_CODE, QuantWeight, _as_2d, _r_pad
 
 
 def _s(dev):
@@ -123,8 +123,148 @@ def _expand(t: Tensor, E: int) -> Tensor:
     return t.expand(E, -1, -1).contiguous() if t.shape[0] == 1 else t
 
 
+# ---------------------------------------------------------------------------
+# the routed expert MLP: two library calls behind two custom ops
+# ---------------------------------------------------------------------------
+_PROJ = ("gate", "up", "down")
+_WS: dict = {}
+
+
+def _bank_args(qw: QuantWeight):
+    return qw.packed, qw.scales, qw.global_scale
+
+
+def _rebuild_bank(packed, scales, gs, fmt, layout, scale_dt, rows, cols, group, E) -> QuantWeight:
+    return QuantWeight(fmt, layout, packed, scales, scale_dt, rows, cols, group, global_scale=gs, num_experts=E)
+
+
+def _lora_struct(factors, r: int, scaling: float) -> _C.XqGroupedLora:
+    gA, gB, uA, uB, dA, dB = factors
+    dt = gA.dtype
+    if dt not in (torch.float32, torch.bfloat16) or any(f.dtype != dt for f in factors):
+        raise _C.XqError(f"LoRA factors must all be fp32 or all be bf16, got {[f.dtype for f in factors]}")
+    L = _C.XqGroupedLora()
+    for p, (A, B) in enumerate(((gA, gB), (uA, uB), (dA, dB))):
+        L.A[p], L.B[p] = A.data_ptr(), B.data_ptr()
+        L.A_experts[p], L.B_experts[p] = A.shape[0], B.shape[0]
+    L.dtype = _C.XQ_DT_F32 if dt == torch.float32 else _C.XQ_DT_BF16
+    L.r, L.scaling = r, scaling
+    return L
+
+
+def _saved_struct(saved) -> _C.XqGroupedSaved:
+    S = _C.XqGroupedSaved()
+    for name, t in zip(("xs", "gate_out", "up_out", "h", "w_row", "su_gate", "su_up", "su_down", "scatter_index",
+                        "offsets", "tile_offsets", "counts"), saved):
+        setattr(S, name, t.data_ptr())
+    return S
+
+
+def _workspace(dev, T: int, topk: int, E: int, H: int, I: int, r: int, backward: bool) -> Tensor:
+    key = (T, topk, E, H, I, r, backward)
+    n = _WS.get(key)
+    if n is None:
+        n = _WS[key] = _C.lib().xq_grouped_workspace_bytes(T, topk, E, H, I, r, int(backward))
+    return torch.empty(n, dtype=torch.uint8, device=dev)
+
+
+def _moe_fwd_impl(hidden2: Tensor, rw: Tensor, sel: Tensor, factors, banks, r: int, scaling: float):
+    """xq_grouped_fwd.  hidden2 bf16 [T, H]; rw [T, topk] fp32 / bf16; sel int32 [T, topk]; factors the six active
+    LoRA views, contiguous; banks three QuantWeight.  -> (out [T, H], the twelve tensors the backward reads)."""
+    qg, qu, qd = banks
+    E, H, I = qg.num_experts, qg.rows, qg.cols
+    T, topk = sel.shape
+    R, rp, dev = T * topk, _r_pad(r), hidden2.device
+    bf = lambda *shape: torch.empty(*shape, dtype=torch.bfloat16, device=dev)
+    i32 = lambda n: torch.empty(n, dtype=torch.int32, device=dev)
+    saved = (bf(R, H), bf(R, I), bf(R, I), bf(R, I), torch.empty(R, dtype=torch.float32, device=dev), bf(R, rp), bf(R, rp),
+             bf(R, rp), i32(R), i32(E + 1), i32(2 * (E + 1)), i32(E))
+    out = bf(T, H)
+    ws = _workspace(dev, T, topk, E, H, I, r, False)
+    lora, S = _lora_struct(factors, r, scaling), _saved_struct(saved)
+    wg, wu, wd = qg.c(), qu.c(), qd.c()
+    _C.check(_C.lib().xq_grouped_fwd(ctypes.byref(wg), ctypes.byref(wu), ctypes.byref(wd), ctypes.byref(lora),
+                                     hidden2.data_ptr(), hidden2.stride(0) if T > 1 else H, T, rw.data_ptr(),
+                                     _C.XQ_DT_F32 if rw.dtype == torch.float32 else _C.XQ_DT_BF16, sel.data_ptr(), topk,
+                                     out.data_ptr(), H, ctypes.byref(S), ws.data_ptr(), ws.numel(), _s(dev)))
+    return out, saved
+
+
+def _moe_bwd_impl(dy2: Tensor, saved, factors, banks, r: int, scaling: float, T: int, topk: int, rw_dtype: torch.dtype,
+                  need_dx: bool, need_drw: bool):
+    """xq_grouped_bwd -> (dx [T, H] or empty, d_routing [T, topk] or empty, six fp32 factor gradients)."""
+    qg, qu, qd = banks
+    E, H, I = qg.num_experts, qg.rows, qg.cols
+    dev = dy2.device
+    dx = torch.empty(T, H, dtype=torch.bfloat16, device=dev) if need_dx else torch.empty(0, dtype=torch.bfloat16, device=dev)
+    out_dt = rw_dtype if rw_dtype in (torch.float32, torch.bfloat16) else torch.float32
+    drw = torch.empty(T, topk, dtype=out_dt, device=dev) if need_drw else torch.empty(0, dtype=out_dt, device=dev)
+    grads = [torch.empty(f.shape, dtype=torch.float32, device=dev) for f in factors]
+    G = _C.XqGroupedGrads()
+    for p in range(3):
+        G.dA[p], G.dB[p] = grads[2 * p].data_ptr(), grads[2 * p + 1].data_ptr()
+    ws = _workspace(dev, T, topk, E, H, I, r, True)
+    lora, S = _lora_struct(factors, r, scaling), _saved_struct(saved)
+    wg, wu, wd = qg.c(), qu.c(), qd.c()
+    _C.check(_C.lib().xq_grouped_bwd(ctypes.byref(wg), ctypes.byref(wu), ctypes.byref(wd), ctypes.byref(lora),
+                                     dy2.data_ptr(), dy2.stride(0) if T > 1 else H, T, topk, ctypes.byref(S),
+                                     dx.data_ptr() if need_dx else None, H, drw.data_ptr() if need_drw else None,
+                                     _C.XQ_DT_F32 if out_dt == torch.float32 else _C.XQ_DT_BF16, ctypes.byref(G),
+                                     ws.data_ptr(), ws.numel(), _s(dev)))
+    return dx, drw, grads
+
+
+@torch.library.custom_op("xq::moe_fwd", mutates_args=(), device_types="cuda")
+def _moe_fwd_op(hidden: Tensor, rw: Tensor, sel: Tensor, gA: Tensor, gB: Tensor, uA: Tensor, uB: Tensor, dA: Tensor,
+                dB: Tensor, g_packed: Tensor, g_scales: Tensor, g_gs: Optional[Tensor], u_packed: Tensor,
+                u_scales: Tensor, u_gs: Optional[Tensor], d_packed: Tensor, d_scales: Tensor, d_gs: Optional[Tensor],
+                fmt: str, layout: int, scale_code: int, group: int, E: int, H: int, I: int, r: int,
+                scaling: float) -> List[Tensor]:
+    sd = _CODE_TO_DT[scale_code]
+    banks = (_rebuild_bank(g_packed, g_scales, g_gs, fmt, layout, sd, H, I, group, E),
+             _rebuild_bank(u_packed, u_scales, u_gs, fmt, layout, sd, H, I, group, E),
+             _rebuild_bank(d_packed, d_scales, d_gs, fmt, layout, sd, I, H, group, E))
+    out, saved = _moe_fwd_impl(hidden, rw, sel, (gA, gB, uA, uB, dA, dB), banks, r, scaling)
+    return [out, *saved]
+
+
+@_moe_fwd_op.register_fake
+def _(hidden, rw, sel, gA, gB, uA, uB, dA, dB, g_packed, g_scales, g_gs, u_packed, u_scales, u_gs, d_packed, d_scales,
+      d_gs, fmt, layout, scale_code, group, E, H, I, r, scaling):
+    T, topk = sel.shape
+    R, rp = T * topk, _r_pad(r)
+    bf = lambda *shape: hidden.new_empty(*shape, dtype=torch.bfloat16)
+    i32 = lambda n: hidden.new_empty(n, dtype=torch.int32)
+    return [bf(T, H), bf(R, H), bf(R, I), bf(R, I), bf(R, I), hidden.new_empty(R, dtype=torch.float32), bf(R, rp),
+            bf(R, rp), bf(R, rp), i32(R), i32(E + 1), i32(2 * (E + 1)), i32(E)]
+
+
+@torch.library.custom_op("xq::moe_bwd", mutates_args=(), device_types="cuda")
+def _moe_bwd_op(dy: Tensor, saved: List[Tensor], gA: Tensor, gB: Tensor, uA: Tensor, uB: Tensor, dA: Tensor, dB: Tensor,
+                g_packed: Tensor, g_scales: Tensor, g_gs: Optional[Tensor], u_packed: Tensor, u_scales: Tensor,
+                u_gs: Optional[Tensor], d_packed: Tensor, d_scales: Tensor, d_gs: Optional[Tensor], fmt: str,
+                layout: int, scale_code: int, group: int, E: int, H: int, I: int, r: int, scaling: float, T: int,
+                topk: int, rw_code: int, need_dx: bool, need_drw: bool) -> List[Tensor]:
+    sd = _CODE_TO_DT[scale_code]
+    banks = (_rebuild_bank(g_packed, g_scales, g_gs, fmt, layout, sd, H, I, group, E),
+             _rebuild_bank(u_packed, u_scales, u_gs, fmt, layout, sd, H, I, group, E),
+             _rebuild_bank(d_packed, d_scales, d_gs, fmt, layout, sd, I, H, group, E))
+    dx, drw, grads = _moe_bwd_impl(dy, tuple(saved), (gA, gB, uA, uB, dA, dB), banks, r, scaling, T, topk,
+                                   _CODE_TO_DT[rw_code], need_dx, need_drw)
+    return [dx, drw, *grads]
+
+
+@_moe_bwd_op.register_fake
+def _(dy, saved, gA, gB, uA, uB, dA, dB, g_packed, g_scales, g_gs, u_packed, u_scales, u_gs, d_packed, d_scales, d_gs,
+      fmt, layout, scale_code, group, E, H, I, r, scaling, T, topk, rw_code, need_dx, need_drw):
+    rw_dt = _CODE_TO_DT[rw_code]
+    return [dy.new_empty((T, H) if need_dx else (0,), dtype=torch.bfloat16),
+            dy.new_empty((T, topk) if need_drw else (0,), dtype=rw_dt),
+            *[dy.new_empty(f.shape, dtype=torch.float32) for f in (gA, gB, uA, uB, dA, dB)]]
+
+
 class MoeExpertsQLoRAFunction(torch.autograd.Function):
-    """Routed SwiGLU expert MLP with LoRA on packed banks.
+    """Routed SwiGLU expert MLP with LoRA on packed banks (xq_grouped_fwd / xq_grouped_bwd).
 
     inputs: hidden [T, H] bf16, routing_weights [T, topk], selected_experts
     [T, topk], three QuantWeight banks (GKN: gate/up [E, H, I], down [E, I, H]),
@@ -140,116 +280,55 @@ class MoeExpertsQLoRAFunction(torch.autograd.Function):
         if hidden.dtype != torch.bfloat16:
             raise _C.XqError(f"hidden states must be bf16, got {hidden.dtype}")
         E = num_experts
-        for qw in (qw_gate, qw_up, qw_down):
-            if qw.num_experts != E:          # the tile schedules route_build emits are laid out for E experts
+        banks = (qw_gate, qw_up, qw_down)
+        for qw in banks:
+            if qw.num_experts != E:          # the tile schedules of the routing are laid out for E experts
                 raise _C.XqError(f"routing over {E} experts but a bank holds {qw.num_experts}")
         shape = hidden.shape
-        H = shape[-1]
+        H, I = qw_gate.rows, qw_gate.cols
         hidden2 = hidden.reshape(-1, H)
+        hidden2 = _as_2d(hidden2)
         T = hidden2.shape[0]
         topk = selected_experts.shape[-1]
-        dev = hidden.device
-        r = gA.shape[-1]
-        rp = _r_pad(r)
-        I = qw_gate.cols
-        s = float(scaling)
-
-        counts, offsets, sidx, tile_offsets = route_build(selected_experts, E)
-        xs = moe_scatter(hidden2, sidx, topk)                                     # [R, H] expert order
-        # bf16 operand layouts of the factors
-        F_gA = _prep(gA, True, rp, H)                                             # [E|1, rp, H]
-        F_uA = _prep(uA, True, rp, H)
-        Lr_gB = _prep(_expand(gB, E), True, I, rp)                                # [E, I, rp]
-        Lr_uB = _prep(_expand(uB, E), True, I, rp)
-        F_dA = _prep(dA, True, rp, I)                                             # [E|1, rp, I]
-        Lr_dB = _prep(_expand(dB, E), True, H, rp)                                # [E, H, rp]
-
-        # (one pass over xs with both panels side by side takes as long as these two: the product is bound by its
-        # fp32 multiply-adds, not by reading the rows)
-        su_g = _lora_down(xs, F_gA, offsets, tile_offsets, E, s)
-        su_u = _lora_down(xs, F_uA, offsets, tile_offsets, E, s)
-        gate_out = _grouped_gemm(qw_gate, False, xs, offsets, tile_offsets, su_g, Lr_gB)    # [R, I]
-        up_out = _grouped_gemm(qw_up, False, xs, offsets, tile_offsets, su_u, Lr_uB)
-        L = _C.lib()
-        R = xs.shape[0]
-        rw = routing_weights.reshape(-1).contiguous()
+        sel = selected_experts.reshape(T, topk).to(torch.int32).contiguous()
+        rw = routing_weights.reshape(T, topk)
         if rw.dtype not in (torch.float32, torch.bfloat16):
             rw = rw.float()
-        w_row = torch.empty(R, dtype=torch.float32, device=dev)
-        _C.check(L.xq_moe_scatter_scalar(rw.data_ptr(), _C.XQ_DT_F32 if rw.dtype == torch.float32 else _C.XQ_DT_BF16,
-                                         sidx.data_ptr(), R, w_row.data_ptr(), _s(dev)))
-        h = torch.empty(R, I, dtype=torch.bfloat16, device=dev)
-        _C.check(L.xq_silu_mul_fwd(gate_out.data_ptr(), up_out.data_ptr(), I, w_row.data_ptr(), h.data_ptr(), I, R, I,
-                                   _s(dev)))
-        su_d = _lora_down(h, F_dA, offsets, tile_offsets, E, s)
-        down_out = _grouped_gemm(qw_down, False, h, offsets, tile_offsets, su_d, Lr_dB)     # [R, H]
-        out = moe_gather(down_out, None, sidx, T, topk)
-
-        ctx.qw = (qw_gate, qw_up, qw_down)
-        ctx.meta = (E, T, topk, H, I, r, rp, s, shape, routing_weights.dtype, routing_weights.shape)
-        ctx.save_for_backward(xs, gate_out, up_out, h, w_row, su_g, su_u, su_d, sidx, offsets, tile_offsets,
-                              gA, gB, uA, uB, dA, dB)
+        rw = rw.contiguous()
+        r = gA.shape[-1]
+        factors = tuple(f.contiguous() for f in (gA, gB, uA, uB, dA, dB))
+        s = float(scaling)
+        if torch.compiler.is_compiling():
+            res = _moe_fwd_op(hidden2, rw, sel, *factors, *_bank_args(qw_gate), *_bank_args(qw_up), *_bank_args(qw_down),
+                              qw_gate.fmt, qw_gate.layout, _DT_TO_CODE[qw_gate.scale_dtype], qw_gate.group, E, H, I, r, s)
+            out, saved = res[0], tuple(res[1:])
+        else:
+            out, saved = _moe_fwd_impl(hidden2, rw, sel, factors, banks, r, s)
+        ctx.qw = banks
+        ctx.meta = (E, T, topk, H, I, r, s, shape, routing_weights.dtype, routing_weights.shape)
+        ctx.save_for_backward(*saved, *factors)
         return out.reshape(shape)
 
     @staticmethod
     def backward(ctx, dy):
-        (xs, gate_out, up_out, h, w_row, su_g, su_u, su_d, sidx, offsets, tile_offsets,
-         gA, gB, uA, uB, dA, dB) = ctx.saved_tensors
+        saved, factors = ctx.saved_tensors[:12], ctx.saved_tensors[12:]
         qw_gate, qw_up, qw_down = ctx.qw
-        E, T, topk, H, I, r, rp, s, shape, rw_dtype, rw_shape = ctx.meta
-        dev = dy.device
-        L = _C.lib()
-        R = xs.shape[0]
-        g_down = moe_scatter(dy.reshape(-1, H).to(torch.bfloat16), sidx, topk)               # [R, H]
-
-        # ---- down projection: y = h.W + s*(h.A).B
-        F_dB = _prep(dB, False, rp, H)                                                       # [E|1, rp, H]
-        v_d = _lora_down(g_down, F_dB, offsets, tile_offsets, E, s)                          # s * g . B^T
-        Lr_dA = _prep(_expand(dA, E), False, I, rp)                                          # [E, I, rp]
-        dh = _grouped_gemm(qw_down, True, g_down, offsets, tile_offsets, v_d, Lr_dA)         # [R, I]
-        shared_dB = dB.shape[0] == 1
-        n_valid = offsets[E:]            # rows that belong to an expert (all of them unless an id was out of range)
-        grad_dB = _wgrad(g_down, su_d, r, None if shared_dB else offsets, E, True, n_valid)  # [E|1, r, H]
-        grad_dA = _wgrad(h, v_d, r, None if dA.shape[0] == 1 else offsets, E, False, n_valid)   # [E|1, I, r]
-
-        # ---- SwiGLU + routing weight
-        dgate = torch.empty(R, I, dtype=torch.bfloat16, device=dev)
-        dup = torch.empty(R, I, dtype=torch.bfloat16, device=dev)
-        d_w_row = torch.empty(R, dtype=torch.float32, device=dev)
-        _C.check(L.xq_silu_mul_bwd(gate_out.data_ptr(), up_out.data_ptr(), I, dh.data_ptr(), I, w_row.data_ptr(),
-                                   dgate.data_ptr(), dup.data_ptr(), I, d_w_row.data_ptr(), R, I, _s(dev)))
-        d_rw = None
-        if ctx.needs_input_grad[1]:
-            out_dt = rw_dtype if rw_dtype in (torch.float32, torch.bfloat16) else torch.float32
-            d_rw = torch.empty(R, dtype=out_dt, device=dev)
-            _C.check(L.xq_moe_gather_scalar(d_w_row.data_ptr(), sidx.data_ptr(), R, d_rw.data_ptr(),
-                                            _C.XQ_DT_F32 if out_dt == torch.float32 else _C.XQ_DT_BF16, _s(dev)))
-            d_rw = d_rw.reshape(rw_shape).to(rw_dtype)
-
-        # ---- up / gate projections: y = x.W + s*(x.A).B
-        def proj_bwd(g_out, qw, A, B, su):
-            F_B = _prep(B, False, rp, I)                                                     # [E|1, rp, I]
-            v = _lora_down(g_out, F_B, offsets, tile_offsets, E, s)
-            Lr_A = _prep(_expand(A, E), False, H, rp)                                        # [E, H, rp]
-            dx = _grouped_gemm(qw, True, g_out, offsets, tile_offsets, v, Lr_A)              # [R, H]
-            gB_ = _wgrad(g_out, su, r, None if B.shape[0] == 1 else offsets, E, True, n_valid)   # [E|1, r, I]
-            return dx, v, gB_
-
-        dx_u, v_u, grad_uB = proj_bwd(dup, qw_up, uA, uB, su_u)
-        dx_g, v_g, grad_gB = proj_bwd(dgate, qw_gate, gA, gB, su_g)
-        # gradients of the two A factors, [E|1, H, r] = x^T . v: both contract the same rows of x, so they share
-        # one pass over them (v_g | v_u side by side) when the panels fit
-        if gA.shape[0] == uA.shape[0] and 2 * rp <= 32:
-            both = _wgrad(xs, torch.cat([v_g, v_u], dim=1), rp + r, None if gA.shape[0] == 1 else offsets, E, False, n_valid)
-            grad_gA, grad_uA = both[..., :r], both[..., rp:rp + r]
+        E, T, topk, H, I, r, s, shape, rw_dtype, rw_shape = ctx.meta
+        dy2 = dy.reshape(-1, H).to(torch.bfloat16)
+        dy2 = _as_2d(dy2)
+        need_dx, need_drw = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        kernel_rw_dt = rw_dtype if rw_dtype in (torch.float32, torch.bfloat16) else torch.float32
+        if torch.compiler.is_compiling():
+            res = _moe_bwd_op(dy2, list(saved), *factors, *_bank_args(qw_gate), *_bank_args(qw_up), *_bank_args(qw_down),
+                              qw_gate.fmt, qw_gate.layout, _DT_TO_CODE[qw_gate.scale_dtype], qw_gate.group, E, H, I, r, s,
+                              T, topk, _DT_TO_CODE[kernel_rw_dt], need_dx, need_drw)
+            dx, drw, grads = res[0], res[1], res[2:]
         else:
-            grad_gA = _wgrad(xs, v_g, r, None if gA.shape[0] == 1 else offsets, E, False, n_valid)
-            grad_uA = _wgrad(xs, v_u, r, None if uA.shape[0] == 1 else offsets, E, False, n_valid)
-        dx = moe_gather(dx_g, dx_u, sidx, T, topk).reshape(shape) if ctx.needs_input_grad[0] else None
-
-        cast = lambda g, p: g.to(p.dtype)
-        return (dx, d_rw, None, cast(grad_gA, gA), cast(grad_gB, gB), cast(grad_uA, uA), cast(grad_uB, uB),
-                cast(grad_dA, dA), cast(grad_dB, dB), None, None, None, None, None)
+            dx, drw, grads = _moe_bwd_impl(dy2, saved, factors, ctx.qw, r, s, T, topk, kernel_rw_dt, need_dx, need_drw)
+        dx = dx.reshape(shape) if need_dx else None
+        drw = drw.reshape(rw_shape).to(rw_dtype) if need_drw else None
+        gs = [g.to(f.dtype) for g, f in zip(grads, factors)]
+        return (dx, drw, None, *gs, None, None, None, None, None)
 
 
 def moe_experts_qlora_forward(num_experts: int, routing_weights: Tensor, selected_experts: Tensor,

@@ -233,10 +233,15 @@ class QLoRALinear(LoraModule, nn.Module):
             self.packed_weight_f32 = nn.Parameter(f32, requires_grad=False)
 
     @torch.compiler.disable
+    def _gather_packed_weight(self, f32: Tensor) -> Tensor:
+        return f32.full_tensor()
+
     def _read_packed_weight_uint8(self) -> Tensor:
+        """The packed bytes as a uint8 view (qlora/modules/linear.py:268-280).  Only the gather of sharded state is
+        kept out of traced graphs; the plain view traces, so that a compiled module is one graph."""
         f32 = self.packed_weight_f32.data
         if _is_dtensor(f32):
-            f32 = f32.full_tensor()
+            f32 = self._gather_packed_weight(f32)
         elif f32.dtype != torch.float32:
             raise RuntimeError(
                 f"QLoRA packed_weight_f32 has dtype {f32.dtype} (expected float32). "
@@ -411,7 +416,7 @@ class QLoRALinear(LoraModule, nn.Module):
         """`_quant_weight()` memoised on the addresses of the packed state: the description (and its C
         descriptor) is rebuilt only when a buffer has been replaced.  Sharded state is gathered every call."""
         p = self.packed_weight_f32
-        if _is_dtensor(p.data):
+        if torch.compiler.is_compiling() or _is_dtensor(p.data):     # addresses are not traceable
             return self._quant_weight()
         key = (p.data_ptr(), p.dtype) + tuple(
             t.data_ptr() for t in (getattr(self, "weight_scales", None), getattr(self, "weight_block_scales", None),
