@@ -322,8 +322,8 @@ int xq_grouped_lora_wgrad(const void* P, int64_t ldp, int64_t p_width, const voi
  * (shared by all experts: 1) or per expert (E); fp32 or bf16; r in 1..64.
  *
  * xq_grouped_saved names caller buffers the forward fills and the backward reads (R = n_tokens * topk routed
- * rows, r_pad = r rounded up to 16): xs bf16 [R, H] (token rows in expert order), gate_out / up_out / h bf16
- * [R, I], w_row fp32 [R], su_gate / su_up / su_down bf16 [R, r_pad], scatter_index int32 [R], offsets int32
+ * rows, r_pad = r rounded up to 16): xs bf16 [R, H] (token rows in expert order), gate_up bf16 [R, 2 I] (the
+ * gate projection in columns [0, I), the up projection in [I, 2 I)), h bf16 [R, I], w_row fp32 [R], su_gate / su_up / su_down bf16 [R, r_pad], scatter_index int32 [R], offsets int32
  * [E + 1], tile_offsets int32 [2 (E + 1)], counts int32 [E].  A forward-only caller passes scratch for them.
  * Factor gradients are fp32, shaped like the factors, overwritten (exact zeros for experts without rows).
  * hidden, out, dy, dx are bf16 [n_tokens, H] with row strides in elements; routing_w [n_tokens, topk] fp32 or
@@ -342,8 +342,7 @@ typedef struct xq_grouped_lora {
 
 typedef struct xq_grouped_saved {
     void* xs;
-    void* gate_out;
-    void* up_out;
+    void* gate_up;
     void* h;
     float* w_row;
     void* su_gate;

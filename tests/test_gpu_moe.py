@@ -88,7 +88,10 @@ def _make_experts(fmt, E, H, I, r, hybrid, seed, device):
 
 @pytest.mark.parametrize("tile_policy", [0, 1, 2], indirect=True)
 @pytest.mark.parametrize("fmt", ["block_fp8", "nvfp4", "nf4"])
-@pytest.mark.parametrize("E,T,H,I,r,topk,hybrid", [(6, 300, 128, 192, 8, 2, True), (16, 700, 256, 128, 16, 4, False)])
+@pytest.mark.parametrize("E,T,H,I,r,topk,hybrid", [(6, 300, 128, 192, 8, 2, True), (16, 700, 256, 128, 16, 4, False),
+                                                   # intermediate sizes of whole 256-column tiles: block-fp8 banks run gate
+                                                   # and up as one forward launch and their dgrads as one sum
+                                                   (4, 900, 256, 512, 16, 2, False), (5, 600, 128, 768, 24, 3, True)])
 def test_moe_fwd_bwd_vs_oracle(hip_device, tile_policy, fmt, E, T, H, I, r, topk, hybrid):
     m, banks = _make_experts(fmt, E, H, I, r, hybrid, seed=E + T, device=hip_device)
     # the module's own bank decode is bit-exact with the oracle

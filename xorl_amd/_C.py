@@ -47,7 +47,7 @@ class XqGroupedLora(ctypes.Structure):
 
 
 class XqGroupedSaved(ctypes.Structure):
-    _fields_ = [(n, ctypes.c_void_p) for n in ("xs", "gate_out", "up_out", "h", "w_row", "su_gate", "su_up", "su_down",
+    _fields_ = [(n, ctypes.c_void_p) for n in ("xs", "gate_up", "h", "w_row", "su_gate", "su_up", "su_down",
                                                "scatter_index", "offsets", "tile_offsets", "counts")]
 
 

@@ -139,13 +139,21 @@ int64_t tile_gemm_partial_bytes(int64_t n_rows, int64_t Nout, int64_t Kc) {
     return elems * Nout * 4;
 }
 
+// Whether a grouped launch on this bank may take a second bank of the same shape (see G256Args::W2): block-fp8 on the
+// pipelined kernel, whole 256-column tiles per bank (which also keeps the K-step where the dgrad changes banks on a
+// scale-block boundary and away from the pipeline's prologue).
+bool two_banks_supported(const xq_weight* w) {
+    return w->format == XQ_FMT_FP8 && g_tile_policy != 1 && w->cols % 256 == 0 && w->cols >= 512 && w->num_experts >= 1;
+}
+
 // C[rows, Nout] = A . op(deq(W)) (+ su . Lr^T) (+ bias); see xq_gemm_tile.h.  force_T = 256 / 128 fixes the tile
 // size of the pipelined kernel (and force_split its K splits), 0 leaves both to the selection policy.  `partial` (may be NULL) is scratch for
 // split-K sums; a launch that would split but finds less than tile_gemm_partial_bytes() there runs unsplit.
 static int launch_tile_gemm_t(const xq_weight* w, bool contract_cols, const bf16_t* A, int64_t lda, int64_t n_rows,
                               const int32_t* offsets, const int32_t* tile_offsets, const bf16_t* su, const bf16_t* lora_right,
                               int r_pad, const bf16_t* bias, bf16_t* C, int64_t ldc, hipStream_t stream, const char* who,
-                              int force_T, int force_split, float* partial, int64_t partial_bytes) {
+                              int force_T, int force_split, float* partial, int64_t partial_bytes,
+                              const TwoBanks* two = nullptr) {
     TileArgs g;
     g.A = A; g.lda = lda; g.C = C; g.ldc = ldc;
     g.packed = (const uint8_t*)w->packed;
@@ -157,6 +165,13 @@ static int launch_tile_gemm_t(const xq_weight* w, bool contract_cols, const bf16
     g.group = w->group; g.scale_dtype = w->scale_dtype;
     g.Kc = contract_cols ? g.wcols : g.wrows;
     g.Nout = contract_cols ? g.wrows : g.wcols;
+    if (two) {       // a second bank of the same shape: twice the contraction (dgrad) or twice the output columns (forward)
+        XQ_REQUIRE(offsets && two_banks_supported(w) && two->w2 && two_banks_supported(two->w2) && two->w2->rows == w->rows &&
+                       two->w2->cols == w->cols && two->w2->num_experts == w->num_experts,
+                   "%s: a two-bank launch takes two block-fp8 expert banks of one shape (columns a multiple of 256)", who);
+        if (contract_cols) g.Kc *= 2;
+        else g.Nout *= 2;
+    }
     g.n_rows = n_rows; g.offsets = offsets; g.tile_offsets = tile_offsets; g.num_experts = w->num_experts;
     g.su = su; g.lora_right = lora_right; g.r_pad = (su && lora_right) ? r_pad : 0;
     g.bias = bias;
@@ -213,6 +228,12 @@ static int launch_tile_gemm_t(const xq_weight* w, bool contract_cols, const bf16
             int ksplit = grouped ? 1 : force_T ? force_split : planned ? plan.split : ksplit_for(tiles_m * tiles_n, T, g.Kc / BK);
             if (ksplit > 1 && (!partial || !xq_aligned(partial, 16) || partial_bytes < (int64_t)ksplit * n_rows * g.Nout * 4)) ksplit = 1;
             f.ksplit = ksplit; f.partial = ksplit > 1 ? partial : nullptr;
+            f.W2 = nullptr; f.scales2 = nullptr; f.su2 = nullptr; f.lora_right2 = nullptr; f.ncols1 = 0; f.nk1 = 0;
+            if (two) {
+                f.W2 = (const uint8_t*)two->w2->packed; f.scales2 = (const uint8_t*)two->w2->scales;
+                f.su2 = g.r_pad ? two->su2 : nullptr; f.lora_right2 = g.r_pad ? two->lora_right2 : nullptr;
+                f.ncols1 = g.wcols; f.nk1 = g.wcols / BK;
+            }
             dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)ksplit);
             const bool timed = xq_profile_mark_begin(stream, 2.0 * (double)n_rows * g.Nout * ((double)g.Kc + g.r_pad));
             int rc;
@@ -249,9 +270,9 @@ static int launch_tile_gemm_t(const xq_weight* w, bool contract_cols, const bf16
 int launch_tile_gemm(const xq_weight* w, bool contract_cols, const bf16_t* A, int64_t lda, int64_t n_rows,
                      const int32_t* offsets, const int32_t* tile_offsets, const bf16_t* su, const bf16_t* lora_right,
                      int r_pad, const bf16_t* bias, bf16_t* C, int64_t ldc, hipStream_t stream, const char* who,
-                     float* partial, int64_t partial_bytes) {
+                     float* partial, int64_t partial_bytes, const TwoBanks* two) {
     return launch_tile_gemm_t(w, contract_cols, A, lda, n_rows, offsets, tile_offsets, su, lora_right, r_pad, bias, C, ldc,
-                              stream, who, 0, 1, partial, partial_bytes);
+                              stream, who, 0, 1, partial, partial_bytes, two);
 }
 
 static inline int64_t align256(int64_t b) { return (b + 255) & ~(int64_t)255; }

@@ -85,6 +85,16 @@ struct G256Args {
     // sums to partial + s * M * Nout (row pitch Nout) instead of C, and split 0 carries the low-rank term and bias
     int32_t ksplit;
     float* partial;
+    // grouped block-fp8 launches over two banks of equal shape (gate and up of an expert MLP), W2 == NULL for one bank:
+    //   bank forward (!CONTRACT_COLS): the output is [rows, 2 * wcols]; column tiles from ncols1 on take the second
+    //     bank, its side term (su2, lora_right2) and write at their own columns -- both projections in one launch;
+    //   bank dgrad (CONTRACT_COLS): the contraction runs over 2 * wcols -- the first nk1 K-steps against the first
+    //     bank, the others against the second -- so dX = [dgate | dup] . [Wg ; Wu]^T leaves the kernel as one sum.
+    const uint8_t* W2;
+    const uint8_t* scales2;
+    const bf16_t* su2;
+    const bf16_t* lora_right2;
+    int32_t ncols1, nk1;
 };
 
 // ---------------------------------------------------------------- weight-tile loaders
@@ -136,6 +146,11 @@ struct W256Fp8 {
             raw[p] = *(const u32x4*)(src[p] + kt * kstep);
             s[p] = CC ? s_src[p][k0 >> 7] : s_src[p][(k0 >> 7) * scols];
         }
+    }
+    // continue on another matrix of the same shape: byte and scale offsets between the two, both uniform
+    __device__ __forceinline__ void rebase(int64_t wdelta, int64_t sdelta) {
+#pragma unroll
+        for (int p = 0; p < 2; ++p) { src[p] += wdelta; s_src[p] += sdelta; }
     }
     __device__ __forceinline__ void store(bf16_t* b, int p) {
         const float sc = s[p];
@@ -238,6 +253,7 @@ struct W256Flat4 {
             sraw[p] = load_scale_raw(sc_base, si, sdt);
         }
     }
+    __device__ __forceinline__ void rebase(int64_t, int64_t) {}
     __device__ __forceinline__ void store(bf16_t* b, int p) {
         float s = scale_from_raw(sraw[p], sdt);
         if (FMT == XQ_FMT_NVFP4) s = s * gs;
@@ -357,6 +373,7 @@ struct W256Gkn4 {
             *(u32x4*)(d + Geo<T>::NN_PITCH + 8) = ohi;
         }
     }
+    __device__ __forceinline__ void rebase(int64_t, int64_t) {}
     // the kernel stores a thread's two runs one after the other: the first call does both
     __device__ __forceinline__ void store(bf16_t* b, int p) {
         if (p != 0) return;
@@ -439,6 +456,20 @@ __global__ void __launch_bounds__(2 * T, 2) gemm_256_kernel(G256Args g) {
         row_end = g.M;
     }
     const int n0 = pid_n * F8_BN;
+    // two banks (grouped block-fp8 only): a forward block past the first bank's columns works on the second bank
+    constexpr bool TWO_OK = GROUPED && FMT == XQ_FMT_FP8;
+    const uint8_t* Wb = g.W;
+    const uint8_t* Sb = g.scales;
+    const bf16_t* su_b = g.su;
+    const bf16_t* lr_b = g.lora_right;
+    int n0w = n0;                                   // first column of the tile within its bank
+    int bank_width = g.Nout;                        // output columns one bank provides
+    if constexpr (TWO_OK) {
+        if (g.W2 != nullptr && !CC) {
+            bank_width = g.ncols1;
+            if (n0 >= g.ncols1) { Wb = g.W2; Sb = g.scales2; su_b = g.su2; lr_b = g.lora_right2; n0w = n0 - g.ncols1; }
+        }
+    }
     // K-steps of this block: all of them, or the split's share (every split has at least one)
     // K splits: the small tile always knows them; the large tile has an instantiation of its own for them
     // (trailing rows of a launch that fill part of a round), so the unsplit one carries nothing extra
@@ -470,8 +501,18 @@ __global__ void __launch_bounds__(2 * T, 2) gemm_256_kernel(G256Args g) {
     WL wls[PD];
 #pragma unroll
     for (int d = 0; d < PD; ++d)
-        wls[d].init(g, g.W + (int64_t)e * g.packed_stride, g.scales + (int64_t)e * g.scale_stride,
-                    FMT == XQ_FMT_NVFP4 ? g.global_scale[e] : 1.0f, n0, tid);
+        wls[d].init(g, Wb + (int64_t)e * g.packed_stride, Sb + (int64_t)e * g.scale_stride,
+                    FMT == XQ_FMT_NVFP4 ? g.global_scale[e] : 1.0f, n0w, tid);
+    // dgrad over two banks: the K-steps from nk1 on read the second bank (same expert offset in both)
+    int64_t wdelta = 0, sdelta = 0;
+    int nk1 = 1 << 30;
+    if constexpr (TWO_OK && CC) {
+        if (g.W2 != nullptr) {
+            nk1 = g.nk1;
+            wdelta = (g.W2 - g.W) - (int64_t)nk1 * F8_BK;
+            sdelta = ((const float*)g.scales2 - (const float*)g.scales) - (nk1 >> 1);
+        }
+    }
     if constexpr (FMT == XQ_FMT_NF4) {
         __shared__ float s_nf4[16];
         if (tid < 16) s_nf4[tid] = kNf4Level[tid];
@@ -549,6 +590,9 @@ __global__ void __launch_bounds__(2 * T, 2) gemm_256_kernel(G256Args g) {
         // region 2: MFMAs of step 1 over the weight decode + stores, the next weight loads, step-2 fragment reads
         mma(af1, bf1);
         if (have_next) { wl.store(bn, 0); wl.store(bn, 1); }
+        if constexpr (TWO_OK && CC) {
+            if (kload >= nk1 && kload - PD < nk1) wl.rebase(wdelta, sdelta);     // uniform; once per loader and tile
+        }
         if (have_next2) wl.load(kt0 + kload);
         load_frags(a, b, 2, false, af0, bf0);
         __builtin_amdgcn_sched_barrier(0);
@@ -600,14 +644,14 @@ __global__ void __launch_bounds__(2 * T, 2) gemm_256_kernel(G256Args g) {
     // ---- low-rank side term: su[rows, rp] x lora_right[n, rp], both [row][k] tiles in stage 0
     if (g.r_pad > 0 && split == 0) {
         const int rp = g.r_pad, cpr = rp >> 3;  // 16-byte chunks per row
-        const bf16_t* lr = g.lora_right + (int64_t)e * g.Nout * rp;
+        const bf16_t* lr = lr_b + (int64_t)e * bank_width * rp;
         for (int idx = tid; idx < F8_BM * cpr; idx += NT) {
             const int r = idx / cpr, c = idx - r * cpr;
             int64_t row = row0 + r;
             row = row < row_end ? row : row_end - 1;
-            *(u32x4*)(As + swz(r, c)) = *(const u32x4*)(g.su + row * rp + c * 8);
-            int n = n0 + r;
-            n = n < g.Nout ? n : g.Nout - 1;
+            *(u32x4*)(As + swz(r, c)) = *(const u32x4*)(su_b + row * rp + c * 8);
+            int n = n0w + r;
+            n = n < bank_width ? n : bank_width - 1;
             *(u32x4*)(Bs + swz(r, c)) = *(const u32x4*)(lr + (int64_t)n * rp + c * 8);
         }
         __syncthreads();

@@ -6,11 +6,6 @@
 #include "xq_lora.h"
 
 namespace xq {
-int launch_tile_gemm(const xq_weight* w, bool contract_cols, const bf16_t* A, int64_t lda, int64_t n_rows,
-                     const int32_t* offsets, const int32_t* tile_offsets, const bf16_t* su, const bf16_t* lora_right,
-                     int r_pad, const bf16_t* bias, bf16_t* C, int64_t ldc, hipStream_t stream, const char* who,
-                     float* partial, int64_t partial_bytes);
-
 namespace {
 
 inline int64_t al256(int64_t b) { return (b + 255) & ~(int64_t)255; }
@@ -35,11 +30,14 @@ constexpr int MAX_PREP_JOBS = 6;
 struct PrepJobs {
     const void* in[MAX_PREP_JOBS];
     bf16_t* out[MAX_PREP_JOBS];
-    int64_t R_in[MAX_PREP_JOBS], C_in[MAX_PREP_JOBS], R_out[MAX_PREP_JOBS], C_out[MAX_PREP_JOBS];
+    int64_t R_in[MAX_PREP_JOBS], C_in[MAX_PREP_JOBS], R_out[MAX_PREP_JOBS], C_out[MAX_PREP_JOBS], pitch[MAX_PREP_JOBS];
     int32_t n_src[MAX_PREP_JOBS], n_out[MAX_PREP_JOBS], transpose[MAX_PREP_JOBS];
     int32_t in_f32, n;
-    bf16_t* add(const void* src, int n_src_, int64_t r_in, int64_t c_in, bool tr, bf16_t* dst, int n_out_, int64_t r_out, int64_t c_out) {
+    // `pitch` (0: c_out) is the row length of the destination, for a panel that is a column band of a wider one
+    bf16_t* add(const void* src, int n_src_, int64_t r_in, int64_t c_in, bool tr, bf16_t* dst, int n_out_, int64_t r_out,
+                int64_t c_out, int64_t pitch_ = 0) {
         in[n] = src; out[n] = dst; R_in[n] = r_in; C_in[n] = c_in; R_out[n] = r_out; C_out[n] = c_out;
+        pitch[n] = pitch_ ? pitch_ : c_out;
         n_src[n] = n_src_; n_out[n] = n_out_; transpose[n] = tr ? 1 : 0;
         ++n;
         return dst;
@@ -49,7 +47,7 @@ struct PrepJobs {
 __global__ void __launch_bounds__(256) grouped_prep_kernel(PrepJobs j) {
     const int k = blockIdx.y;
     const int64_t per = j.R_out[k] * j.C_out[k], total = per * j.n_out[k];
-    const int64_t R_in = j.R_in[k], C_in = j.C_in[k], C_out = j.C_out[k];
+    const int64_t R_in = j.R_in[k], C_in = j.C_in[k], C_out = j.C_out[k], R_out = j.R_out[k], pitch = j.pitch[k];
     const bool tr = j.transpose[k] != 0, shared = j.n_src[k] == 1;
     for (int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x; t < total; t += (int64_t)gridDim.x * 256) {
         const int64_t e = t / per, rem = t - e * per;
@@ -60,7 +58,7 @@ __global__ void __launch_bounds__(256) grouped_prep_kernel(PrepJobs j) {
             const int64_t idx = (shared ? 0 : e) * R_in * C_in + si * C_in + sj;
             v = j.in_f32 ? ((const float*)j.in[k])[idx] : bf16_to_f32(((const bf16_t*)j.in[k])[idx]);
         }
-        j.out[k][t] = to_bf16(v);
+        j.out[k][(e * R_out + i) * pitch + c] = to_bf16(v);
     }
 }
 
@@ -76,6 +74,17 @@ int launch_prep(const PrepJobs& j, hipStream_t stream) {
     grouped_prep_kernel<<<dim3((unsigned)blocks, (unsigned)j.n), 256, 0, stream>>>(j);
     XQ_CHECK_LAUNCH("grouped_prep");
     return XQ_OK;
+}
+
+// dst0[m][i][j] = src[m][i][j], dst1[m][i][j] = src[m][i][half + j] for j < r: the two factor gradients that one
+// pass over the rows produced side by side
+__global__ void __launch_bounds__(256) split_pair_kernel(const float* src, int64_t rows, int half, int r, float* dst0, float* dst1) {
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (t >= rows * r) return;
+    const int64_t i = t / r;
+    const int j = (int)(t - i * r);
+    dst0[t] = src[i * 2 * half + j];
+    dst1[t] = src[i * 2 * half + half + j];
 }
 
 struct Dims {
@@ -108,7 +117,7 @@ int check_call(const xq_weight* gate, const xq_weight* up, const xq_weight* down
     d->E = E; d->topk = topk; d->r = lora->r; d->rp = r_pad_of(lora->r);
     d->T = n_tokens; d->R = n_tokens * topk; d->H = H; d->I = I;
     if (d->R > 0)
-        XQ_REQUIRE(saved->xs && saved->gate_out && saved->up_out && saved->h && saved->w_row && saved->su_gate && saved->su_up &&
+        XQ_REQUIRE(saved->xs && saved->gate_up && saved->h && saved->w_row && saved->su_gate && saved->su_up &&
                        saved->su_down && saved->scatter_index,
                    "%s: a buffer of xq_grouped_saved is NULL", who);
     XQ_REQUIRE(saved->offsets && saved->tile_offsets && saved->counts, "%s: a routing buffer of xq_grouped_saved is NULL", who);
@@ -125,9 +134,14 @@ int64_t bwd_workspace(const Dims& d) {
     const int64_t EH = al256((int64_t)d.E * d.rp * d.H * 2), EI = al256((int64_t)d.E * d.rp * d.I * 2);
     const int64_t panels = 3 * EH + 3 * EI;     // F_dB, Lr_gA, Lr_uA over H; Lr_dA, F_gB, F_uB over I
     const int64_t wide = d.H > d.I ? d.H : d.I;
-    const int64_t wg = al256(xq_lora_wgrad_workspace_bytes(d.R, wide, d.rp));
-    return panels + 3 * al256(d.R * d.H * 2) + 3 * al256(d.R * d.I * 2) + al256(d.R * 4) + 3 * al256(d.R * d.rp * 2) + wg + 256;
+    const int64_t wg = al256(xq_lora_wgrad_workspace_bytes(d.R, wide, 2 * d.rp <= 64 ? 2 * d.rp : d.rp));
+    const int64_t pair = al256((int64_t)d.E * d.H * 2 * d.rp * 4);      // the two A gradients side by side
+    return panels + 3 * al256(d.R * d.H * 2) + al256(d.R * d.I * 2) + al256(d.R * 2 * d.I * 2) + al256(d.R * 4) +
+           al256(d.R * d.rp * 2) + al256(d.R * 2 * d.rp * 2) + pair + wg + 256;
 }
+
+// one launch for gate and up (forward) / one sum for their two dgrads: block-fp8 banks on the pipelined kernel
+bool fuse_gate_up(const xq_weight* gate, const xq_weight* up) { return two_banks_supported(gate) && two_banks_supported(up); }
 
 }  // namespace
 }  // namespace xq
@@ -184,13 +198,18 @@ extern "C" int xq_grouped_fwd(const xq_weight* gate, const xq_weight* up, const 
 
     const int32_t *off = saved->offsets, *toff = saved->tile_offsets;
     bf16_t *su_g = (bf16_t*)saved->su_gate, *su_u = (bf16_t*)saved->su_up, *su_d = (bf16_t*)saved->su_down;
-    bf16_t *gate_out = (bf16_t*)saved->gate_out, *up_out = (bf16_t*)saved->up_out, *h = (bf16_t*)saved->h;
+    bf16_t *gu = (bf16_t*)saved->gate_up, *h = (bf16_t*)saved->h;       // gu [R, 2I]: gate | up
     if ((rc = launch_small_nt(xs, H, R, H, F_gA, rp, s, su_g, off, toff, E, gAe == 1, stream))) return rc;
     if ((rc = launch_small_nt(xs, H, R, H, F_uA, rp, s, su_u, off, toff, E, uAe == 1, stream))) return rc;
-    if ((rc = launch_tile_gemm(gate, false, xs, H, R, off, toff, su_g, Lr_gB, rp, nullptr, gate_out, I, stream, who, nullptr, 0))) return rc;
-    if ((rc = launch_tile_gemm(up, false, xs, H, R, off, toff, su_u, Lr_uB, rp, nullptr, up_out, I, stream, who, nullptr, 0))) return rc;
+    if (fuse_gate_up(gate, up)) {       // both projections in one launch: column tiles past I take the up bank
+        const TwoBanks two{up, su_u, Lr_uB};
+        if ((rc = launch_tile_gemm(gate, false, xs, H, R, off, toff, su_g, Lr_gB, rp, nullptr, gu, 2 * I, stream, who, nullptr, 0, &two))) return rc;
+    } else {
+        if ((rc = launch_tile_gemm(gate, false, xs, H, R, off, toff, su_g, Lr_gB, rp, nullptr, gu, 2 * I, stream, who, nullptr, 0))) return rc;
+        if ((rc = launch_tile_gemm(up, false, xs, H, R, off, toff, su_u, Lr_uB, rp, nullptr, gu + I, 2 * I, stream, who, nullptr, 0))) return rc;
+    }
     if ((rc = xq_moe_scatter_scalar(routing_w, rw_dtype, saved->scatter_index, R, saved->w_row, stream))) return rc;
-    if ((rc = xq_silu_mul_fwd(gate_out, up_out, I, saved->w_row, h, I, R, I, stream))) return rc;
+    if ((rc = xq_silu_mul_fwd(gu, gu + I, 2 * I, saved->w_row, h, I, R, I, stream))) return rc;
     if ((rc = launch_small_nt(h, I, R, I, F_dA, rp, s, su_d, off, toff, E, dAe == 1, stream))) return rc;
     if ((rc = launch_tile_gemm(down, false, h, I, R, off, toff, su_d, Lr_dB, rp, nullptr, down_out, H, stream, who, nullptr, 0))) return rc;
     return xq_moe_gather(down_out, nullptr, H, saved->scatter_index, d.T, topk, H, out, ld_out, stream);
@@ -225,35 +244,46 @@ extern "C" int xq_grouped_bwd(const xq_weight* gate, const xq_weight* up, const 
     Carve cv{(uint8_t*)workspace, 0};
     const int32_t *off = saved->offsets, *toff = saved->tile_offsets, *sidx = saved->scatter_index;
     const int32_t* n_valid = off + E;     // rows that belong to an expert (all of them unless an id was out of range)
-    const bf16_t *xs = (const bf16_t*)saved->xs, *gate_out = (const bf16_t*)saved->gate_out, *up_out = (const bf16_t*)saved->up_out;
+    const bf16_t *xs = (const bf16_t*)saved->xs, *gu = (const bf16_t*)saved->gate_up;
     const bf16_t *h = (const bf16_t*)saved->h, *su_g = (const bf16_t*)saved->su_gate, *su_u = (const bf16_t*)saved->su_up;
     const bf16_t* su_d = (const bf16_t*)saved->su_down;
-
-    // every panel of the call in one launch: B factors [E|1, r, out] as the "down" panels [E|1, rp, out] of g . B^T,
-    // A factors [E|1, in, r] as the per-expert right-hand panels [E, in, rp] of the dgrads
-    PrepJobs jobs{};
-    jobs.in_f32 = lora->dtype == XQ_DT_F32;
     const int gBe = lora->B_experts[0], uBe = lora->B_experts[1], dBe = lora->B_experts[2];
     const int gAe = lora->A_experts[0], uAe = lora->A_experts[1], dAe = lora->A_experts[2];
+    // one dgrad launch for gate and up: dX = [dgate | dup] . [Wg ; Wu]^T + [v_g | v_u] . [Lr_gA | Lr_uA]^T (the two
+    // low-rank terms ride as one side term of width 2 * rp)
+    // (the A gradients then come from one pass over the rows too, which wants both A factors held the same way)
+    const bool fused = fuse_gate_up(gate, up) && 2 * rp <= 64 && gAe == uAe;
+    const int rp2 = 2 * rp;
+
+    // every panel of the call in one launch: B factors [E|1, r, out] as the "down" panels [E|1, rp, out] of g . B^T,
+    // A factors [E|1, in, r] as the per-expert right-hand panels [E, in, rp] of the dgrads (gate's and up's side by
+    // side in one [E, H, 2 rp] panel when their dgrads share a launch)
+    PrepJobs jobs{};
+    jobs.in_f32 = lora->dtype == XQ_DT_F32;
     bf16_t* F_dB = jobs.add(lora->B[2], dBe, r, H, false, cv.take<bf16_t>((int64_t)dBe * rp * H * 2), dBe, rp, H);
     bf16_t* Lr_dA = jobs.add(lora->A[2], dAe, I, r, false, cv.take<bf16_t>((int64_t)E * I * rp * 2), E, I, rp);
     bf16_t* F_uB = jobs.add(lora->B[1], uBe, r, I, false, cv.take<bf16_t>((int64_t)uBe * rp * I * 2), uBe, rp, I);
-    bf16_t* Lr_uA = jobs.add(lora->A[1], uAe, H, r, false, cv.take<bf16_t>((int64_t)E * H * rp * 2), E, H, rp);
     bf16_t* F_gB = jobs.add(lora->B[0], gBe, r, I, false, cv.take<bf16_t>((int64_t)gBe * rp * I * 2), gBe, rp, I);
-    bf16_t* Lr_gA = jobs.add(lora->A[0], gAe, H, r, false, cv.take<bf16_t>((int64_t)E * H * rp * 2), E, H, rp);
+    bf16_t* Lr_guA = cv.take<bf16_t>((int64_t)E * H * rp2 * 2);       // fused: [E, H, 2 rp]; else gate's [E, H, rp] then up's
+    bf16_t* Lr_uA = fused ? Lr_guA + rp : Lr_guA + (int64_t)E * H * rp;
+    jobs.add(lora->A[0], gAe, H, r, false, Lr_guA, E, H, rp, fused ? rp2 : rp);
+    jobs.add(lora->A[1], uAe, H, r, false, Lr_uA, E, H, rp, fused ? rp2 : rp);
     if ((rc = launch_prep(jobs, stream))) return rc;
 
     bf16_t* g_down = cv.take<bf16_t>(R * H * 2);
     bf16_t* dx_g = cv.take<bf16_t>(R * H * 2);
     bf16_t* dx_u = cv.take<bf16_t>(R * H * 2);
     bf16_t* dh = cv.take<bf16_t>(R * I * 2);
-    bf16_t* dgate = cv.take<bf16_t>(R * I * 2);
-    bf16_t* dup = cv.take<bf16_t>(R * I * 2);
+    bf16_t* dgu = cv.take<bf16_t>(R * 2 * I * 2);         // [R, 2I]: dgate | dup
     float* d_w_row = cv.take<float>(R * 4);
     bf16_t* v_d = cv.take<bf16_t>(R * rp * 2);
-    bf16_t* v_g = cv.take<bf16_t>(R * rp * 2);
-    bf16_t* v_u = cv.take<bf16_t>(R * rp * 2);
+    bf16_t* v_gu = cv.take<bf16_t>(R * rp2 * 2);          // fused: [R, 2 rp] = v_g | v_u; else v_g [R, rp] then v_u [R, rp]
+    float* pair = cv.take<float>((int64_t)E * H * rp2 * 4);
     float* wg = cv.take<float>(0);
+    bf16_t *dgate = dgu, *dup = dgu + I;
+    bf16_t* v_g = v_gu;
+    bf16_t* v_u = fused ? v_gu + rp : v_gu + R * rp;
+    const int64_t ld_v = fused ? rp2 : rp;
 
     if ((rc = xq_moe_scatter(dy, ld_dy, sidx, R, topk, H, g_down, H, stream))) return rc;
 
@@ -264,19 +294,32 @@ extern "C" int xq_grouped_bwd(const xq_weight* gate, const xq_weight* up, const 
     if ((rc = launch_tn(h, I, I, v_d, rp, r, R, false, grads->dA[2], wg, dAe == 1 ? nullptr : off, E, stream, n_valid))) return rc;        // [E|1, I, r]
 
     // ---- SwiGLU + routing weight
-    if ((rc = xq_silu_mul_bwd(gate_out, up_out, I, dh, I, saved->w_row, dgate, dup, I, d_w_row, R, I, stream))) return rc;
+    if ((rc = xq_silu_mul_bwd(gu, gu + I, 2 * I, dh, I, saved->w_row, dgate, dup, 2 * I, d_w_row, R, I, stream))) return rc;
     if (d_routing && (rc = xq_moe_gather_scalar(d_w_row, sidx, R, d_routing, rw_dtype, stream))) return rc;
 
     // ---- up / gate projections: y = x.W + s*(x.A).B
-    if ((rc = launch_small_nt(dup, I, R, I, F_uB, rp, s, v_u, off, toff, E, uBe == 1, stream))) return rc;
-    if ((rc = launch_tile_gemm(up, true, dup, I, R, off, toff, v_u, Lr_uA, rp, nullptr, dx_u, H, stream, who, nullptr, 0))) return rc;
-    if ((rc = launch_tn(dup, I, I, su_u, rp, r, R, true, grads->dB[1], wg, uBe == 1 ? nullptr : off, E, stream, n_valid))) return rc;      // [E|1, r, I]
-    if ((rc = launch_small_nt(dgate, I, R, I, F_gB, rp, s, v_g, off, toff, E, gBe == 1, stream))) return rc;
-    if ((rc = launch_tile_gemm(gate, true, dgate, I, R, off, toff, v_g, Lr_gA, rp, nullptr, dx_g, H, stream, who, nullptr, 0))) return rc;
-    if ((rc = launch_tn(dgate, I, I, su_g, rp, r, R, true, grads->dB[0], wg, gBe == 1 ? nullptr : off, E, stream, n_valid))) return rc;
-    // gradients of the two A factors, [E|1, H, r] = x^T . v
-    if ((rc = launch_tn(xs, H, H, v_g, rp, r, R, false, grads->dA[0], wg, gAe == 1 ? nullptr : off, E, stream, n_valid))) return rc;
-    if ((rc = launch_tn(xs, H, H, v_u, rp, r, R, false, grads->dA[1], wg, uAe == 1 ? nullptr : off, E, stream, n_valid))) return rc;
-    if (dx) return xq_moe_gather(dx_g, dx_u, H, sidx, d.T, topk, H, dx, ld_dx, stream);
-    return XQ_OK;
+    if ((rc = launch_small_nt(dup, 2 * I, R, I, F_uB, rp, s, v_u, off, toff, E, uBe == 1, stream, ld_v))) return rc;
+    if ((rc = launch_small_nt(dgate, 2 * I, R, I, F_gB, rp, s, v_g, off, toff, E, gBe == 1, stream, ld_v))) return rc;
+    if (fused) {
+        const TwoBanks two{up, nullptr, nullptr};
+        if ((rc = launch_tile_gemm(gate, true, dgu, 2 * I, R, off, toff, v_gu, Lr_guA, rp2, nullptr, dx_g, H, stream, who, nullptr, 0, &two))) return rc;
+    } else {
+        if ((rc = launch_tile_gemm(up, true, dup, 2 * I, R, off, toff, v_u, Lr_uA, rp, nullptr, dx_u, H, stream, who, nullptr, 0))) return rc;
+        if ((rc = launch_tile_gemm(gate, true, dgate, 2 * I, R, off, toff, v_g, Lr_guA, rp, nullptr, dx_g, H, stream, who, nullptr, 0))) return rc;
+    }
+    if ((rc = launch_tn(dup, 2 * I, I, su_u, rp, r, R, true, grads->dB[1], wg, uBe == 1 ? nullptr : off, E, stream, n_valid))) return rc;      // [E|1, r, I]
+    if ((rc = launch_tn(dgate, 2 * I, I, su_g, rp, r, R, true, grads->dB[0], wg, gBe == 1 ? nullptr : off, E, stream, n_valid))) return rc;
+    // gradients of the two A factors, [E|1, H, r] = x^T . v: both contract the same rows of x, so with v_g | v_u side
+    // by side they share one pass over them
+    if (fused) {
+        if ((rc = launch_tn(xs, H, H, v_gu, rp2, rp2, R, false, pair, wg, gAe == 1 ? nullptr : off, E, stream, n_valid))) return rc;
+        const int64_t rows = (int64_t)gAe * H;
+        split_pair_kernel<<<dim3((unsigned)xq_cdiv(rows * r, 256)), 256, 0, stream>>>(pair, rows, rp, r, grads->dA[0], grads->dA[1]);
+        XQ_CHECK_LAUNCH(who);
+    } else {
+        if ((rc = launch_tn(xs, H, H, v_g, rp, r, R, false, grads->dA[0], wg, gAe == 1 ? nullptr : off, E, stream, n_valid))) return rc;
+        if ((rc = launch_tn(xs, H, H, v_u, rp, r, R, false, grads->dA[1], wg, uAe == 1 ? nullptr : off, E, stream, n_valid))) return rc;
+    }
+    if (!dx) return XQ_OK;
+    return xq_moe_gather(dx_g, fused ? nullptr : dx_u, H, sidx, d.T, topk, H, dx, ld_dx, stream);
 }

@@ -30,7 +30,8 @@ int launch_factor_prep(const void* in, int in_dtype, int64_t R_in, int64_t C_in,
 //   grouped: rows in expert order, F[e] = F + e*r_pad*Kc (or shared).
 int launch_small_nt(const bf16_t* In, int64_t ld_in, int64_t n_rows, int64_t Kc, const bf16_t* F,
                     int r_pad, float scale, bf16_t* T, const int32_t* offsets,
-                    const int32_t* tile_offsets, int32_t num_experts, bool shared_f, hipStream_t stream);
+                    const int32_t* tile_offsets, int32_t num_experts, bool shared_f, hipStream_t stream,
+                    int64_t ld_t = 0);      // row pitch of T in elements (0: r_pad), to write a column band of a wider matrix
 
 // out[c][j] (or out[j][c] when transpose_out) = sum_m P[m][c] * Q[m][j], fp32.
 //   dense: all rows, split over `splits` row ranges, partials in `partial`
@@ -44,6 +45,20 @@ int launch_tn(const bf16_t* P, int64_t ldp, int64_t width, const bf16_t* Q, int 
               const int32_t* row_limit = nullptr);   // dense form: contract only rows below *row_limit (device value)
 
 int launch_zero_fill(void* p, int64_t bytes, hipStream_t stream);
+
+// fused dequant-GEMM launcher (xq_gemm.hip).  `two`: a grouped launch over two block-fp8 banks of one shape -- the
+// forward (contract_cols false) writes [rows, 2 * cols] with the second bank's columns, side term su2 / lora_right2,
+// after the first's; the dgrad (contract_cols true) contracts A [rows, 2 * cols] against both banks into one sum.
+struct TwoBanks {
+    const xq_weight* w2;
+    const bf16_t* su2;
+    const bf16_t* lora_right2;
+};
+bool two_banks_supported(const xq_weight* w);
+int launch_tile_gemm(const xq_weight* w, bool contract_cols, const bf16_t* A, int64_t lda, int64_t n_rows,
+                     const int32_t* offsets, const int32_t* tile_offsets, const bf16_t* su, const bf16_t* lora_right,
+                     int r_pad, const bf16_t* bias, bf16_t* C, int64_t ldc, hipStream_t stream, const char* who,
+                     float* partial, int64_t partial_bytes, const TwoBanks* two = nullptr);
 
 // skinny-M (M <= 64) forward path, xq_skinny.hip
 bool skinny_supported(const xq_weight* w, int64_t M);

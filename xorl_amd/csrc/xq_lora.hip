@@ -88,6 +88,7 @@ struct SmallNtArgs {
     int r_pad;
     float scale;
     bf16_t* T;
+    int64_t ld_t;      // row pitch of T in elements (>= r_pad)
     const int32_t* offsets;
     const int32_t* tile_offsets;
     int32_t num_experts;
@@ -235,7 +236,7 @@ __global__ void __launch_bounds__(256) small_nt_kernel(SmallNtArgs g) {
 #pragma unroll
         for (int q = 0; q < 16; ++q) {
             int64_t row = row0 + rg * 32 + (q & 3) + rgrp + 8 * (q >> 2);
-            if (row < row_end) g.T[row * g.r_pad + j] = to_bf16(acc[n][q] * g.scale);
+            if (row < row_end) g.T[row * g.ld_t + j] = to_bf16(acc[n][q] * g.scale);
         }
     }
 }
@@ -269,12 +270,14 @@ static int launch_small_nt_rows(const SmallNtArgs& g, unsigned blocks, hipStream
 
 int launch_small_nt(const bf16_t* In, int64_t ld_in, int64_t n_rows, int64_t Kc, const bf16_t* F, int r_pad,
                     float scale, bf16_t* T, const int32_t* offsets, const int32_t* tile_offsets,
-                    int32_t num_experts, bool shared_f, hipStream_t stream) {
+                    int32_t num_experts, bool shared_f, hipStream_t stream, int64_t ld_t) {
+    if (ld_t <= 0) ld_t = r_pad;
+    XQ_REQUIRE(ld_t >= r_pad, "small_nt: output pitch %lld below r_pad %d", (long long)ld_t, r_pad);
     XQ_REQUIRE(r_pad > 0 && r_pad <= 64 && r_pad % 16 == 0, "small_nt: r_pad must be 16/32/48/64, got %d", r_pad);
     XQ_REQUIRE(Kc % 64 == 0, "small_nt: contraction length %lld must be a multiple of 64", (long long)Kc);
     XQ_REQUIRE(ld_in % 8 == 0 && xq_aligned(In, 16) && xq_aligned(F, 16), "small_nt: operands must be 16-byte aligned");
     if (n_rows == 0) return XQ_OK;
-    SmallNtArgs g{In, ld_in, n_rows, Kc, F, shared_f ? 0 : (int64_t)r_pad * Kc, r_pad, scale, T, offsets, tile_offsets,
+    SmallNtArgs g{In, ld_in, n_rows, Kc, F, shared_f ? 0 : (int64_t)r_pad * Kc, r_pad, scale, T, ld_t, offsets, tile_offsets,
                   num_experts};
     int rc;
     if (offsets) {

@@ -154,8 +154,8 @@ def _lora_struct(factors, r: int, scaling: float) -> _C.XqGroupedLora:
 
 def _saved_struct(saved) -> _C.XqGroupedSaved:
     S = _C.XqGroupedSaved()
-    for name, t in zip(("xs", "gate_out", "up_out", "h", "w_row", "su_gate", "su_up", "su_down", "scatter_index",
-                        "offsets", "tile_offsets", "counts"), saved):
+    for name, t in zip(("xs", "gate_up", "h", "w_row", "su_gate", "su_up", "su_down", "scatter_index", "offsets",
+                        "tile_offsets", "counts"), saved):
         setattr(S, name, t.data_ptr())
     return S
 
@@ -170,14 +170,14 @@ def _workspace(dev, T: int, topk: int, E: int, H: int, I: int, r: int, backward:
 
 def _moe_fwd_impl(hidden2: Tensor, rw: Tensor, sel: Tensor, factors, banks, r: int, scaling: float):
     """xq_grouped_fwd.  hidden2 bf16 [T, H]; rw [T, topk] fp32 / bf16; sel int32 [T, topk]; factors the six active
-    LoRA views, contiguous; banks three QuantWeight.  -> (out [T, H], the twelve tensors the backward reads)."""
+    LoRA views, contiguous; banks three QuantWeight.  -> (out [T, H], the eleven tensors the backward reads)."""
     qg, qu, qd = banks
     E, H, I = qg.num_experts, qg.rows, qg.cols
     T, topk = sel.shape
     R, rp, dev = T * topk, _r_pad(r), hidden2.device
     bf = lambda *shape: torch.empty(*shape, dtype=torch.bfloat16, device=dev)
     i32 = lambda n: torch.empty(n, dtype=torch.int32, device=dev)
-    saved = (bf(R, H), bf(R, I), bf(R, I), bf(R, I), torch.empty(R, dtype=torch.float32, device=dev), bf(R, rp), bf(R, rp),
+    saved = (bf(R, H), bf(R, 2 * I), bf(R, I), torch.empty(R, dtype=torch.float32, device=dev), bf(R, rp), bf(R, rp),
              bf(R, rp), i32(R), i32(E + 1), i32(2 * (E + 1)), i32(E))
     out = bf(T, H)
     ws = _workspace(dev, T, topk, E, H, I, r, False)
@@ -235,7 +235,7 @@ def _(hidden, rw, sel, gA, gB, uA, uB, dA, dB, g_packed, g_scales, g_gs, u_packe
     R, rp = T * topk, _r_pad(r)
     bf = lambda *shape: hidden.new_empty(*shape, dtype=torch.bfloat16)
     i32 = lambda n: hidden.new_empty(n, dtype=torch.int32)
-    return [bf(T, H), bf(R, H), bf(R, I), bf(R, I), bf(R, I), hidden.new_empty(R, dtype=torch.float32), bf(R, rp),
+    return [bf(T, H), bf(R, H), bf(R, 2 * I), bf(R, I), hidden.new_empty(R, dtype=torch.float32), bf(R, rp),
             bf(R, rp), bf(R, rp), i32(R), i32(E + 1), i32(2 * (E + 1)), i32(E)]
 
 
@@ -311,7 +311,7 @@ class MoeExpertsQLoRAFunction(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, dy):
-        saved, factors = ctx.saved_tensors[:12], ctx.saved_tensors[12:]
+        saved, factors = ctx.saved_tensors[:11], ctx.saved_tensors[11:]
         qw_gate, qw_up, qw_down = ctx.qw
         E, T, topk, H, I, r, s, shape, rw_dtype, rw_shape = ctx.meta
         dy2 = dy.reshape(-1, H).to(torch.bfloat16)
