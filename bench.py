@@ -351,6 +351,9 @@ def main():
     ap.add_argument("--config", type=int, default=1,
                     help="BASELINE.json configs index; 1 (default) is the headline workload, the others report the "
                          "same JSON for their own workload (no CPU baseline)")
+    ap.add_argument("--unfused", action="store_true",
+                    help="config 1 only: call the three QLoRA linears and the SwiGLU kernel one by one instead of the "
+                         "fused MLP entry points (same arithmetic; for A/B timing)")
     ap.add_argument("--no-graph", action="store_true",
                     help="config 4 only: issue the 32 forwards of a step eagerly instead of replaying them as one HIP graph")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -379,14 +382,16 @@ def main():
     dy = gen((M, H), 1.0, 2, torch.bfloat16).to(dev)
     params = [p for m in mods.values() for p in (m.lora_A, m.lora_B)]
 
+    from xorl_amd.qlora import qlora_mlp_forward
+
     def step():
         x.grad = None
         for p in params:
             p.grad = None
-        g = mods["gate"](x)
-        u = mods["up"](x)
-        h = silu_and_mul(g, u)
-        y = mods["down"](h)
+        if args.unfused:          # the three modules and the SwiGLU kernel one by one
+            y = mods["down"](silu_and_mul(mods["gate"](x), mods["up"](x)))
+        else:                     # the same MLP through the library's fused forward / backward (xq_mlp_fwd / xq_mlp_bwd)
+            y = qlora_mlp_forward(mods["gate"], mods["up"], mods["down"], x)
         y.backward(dy)
 
     L = _C.lib()
@@ -428,7 +433,10 @@ def main():
                    "tokens": M, "hidden": H, "intermediate": I, "lora_r": R, "format": "block_fp8"},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": BF16_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / BF16_MFMA_PEAK_TFLOPS, "traffic": traffic, "traffic_source": traffic_source,
-                     "kernel": "gemm_256_kernel<fp8, contract_cols true|false, dense> (fused fp8 dequant-GEMM, "
+                     "kernel": "gemm_256_kernel<fp8, contract_cols true|false, dense> (fused fp8 dequant-GEMM: gate|up "
+                               "forward with the SwiGLU epilogue, down forward, down dgrad, gate+up dgrad as one sum)"
+                               if not args.unfused else
+                               "gemm_256_kernel<fp8, contract_cols true|false, dense> (fused fp8 dequant-GEMM, "
                                "forward and dgrad launches)",
                      "launches": n.value, "avg_launch_ms": avg_launch_ms},
         "cpu_baseline": cpu,

@@ -370,6 +370,51 @@ int xq_grouped_bwd(const xq_weight* gate, const xq_weight* up, const xq_weight* 
                    void* dx, int64_t ld_dx, void* d_routing, int rw_dtype, const xq_grouped_grads* grads,
                    void* workspace, int64_t workspace_bytes, void* stream);
 
+/* ---- the dense SwiGLU MLP in two calls ---------------------------------------
+ * y = down(silu(gate(x)) * up(x)) over three QLoRA linears: the reference's Qwen3MLP.forward
+ * (models/transformers/qwen3/modeling_qwen3.py:60-81) on QLoRALinear modules (qlora/modules/linear.py:369-385) with
+ * fused_silu_and_mul between them (ops/fused_silu_and_mul.py:22-60), and its autograd backward.  Same arithmetic
+ * and rounding points as three xq_linear_fwd calls around xq_silu_mul_fwd; what the separate calls repeat is
+ * shared (one pass over x for both low-rank intermediates; block-fp8 gate / up as one launch that also writes the
+ * SwiGLU output; the two input-gradient products as one launch; one pass over x for the two A gradients).
+ *
+ * Weights FLAT: gate, up [I, H], down [H, I] (H, I multiples of 64), any format.  LoRA factors in the dense module
+ * layout, A[p] [r, in], B[p] [out, r] for p = 0 gate, 1 up, 2 down, fp32 or bf16, r in 0..64; bias[p] bf16 or NULL.
+ * xq_mlp_saved names caller buffers the forward fills and the backward reads (r_pad = r rounded up to 16):
+ * gate_up bf16 [M, 2 I] (gate | up), h bf16 [M, I], su_gate_up bf16 M * 2 * r_pad elements, su_down bf16
+ * [M, r_pad]; the backward also reads x.  Factor gradients fp32, shaped like the factors, overwritten; dx may be
+ * NULL.  workspace: xq_mlp_workspace_bytes(..., backward) bytes, 256-byte aligned. */
+typedef struct xq_mlp_lora {
+    const void* A[3];
+    const void* B[3];
+    const void* bias[3];
+    int32_t dtype;      /* XQ_DT_* of all six factors */
+    int32_t r;
+    float scaling;
+    int32_t reserved;
+} xq_mlp_lora;
+
+typedef struct xq_mlp_saved {
+    void* gate_up;
+    void* h;
+    void* su_gate_up;
+    void* su_down;
+} xq_mlp_saved;
+
+typedef struct xq_mlp_grads {
+    float* dA[3];
+    float* dB[3];
+} xq_mlp_grads;
+
+int64_t xq_mlp_workspace_bytes(int64_t M, int64_t hidden, int64_t intermediate, int r, int backward);
+int xq_mlp_fwd(const xq_weight* gate, const xq_weight* up, const xq_weight* down, const xq_mlp_lora* lora,
+               const void* x, int64_t ldx, int64_t M, void* y, int64_t ldy, const xq_mlp_saved* saved,
+               void* workspace, int64_t workspace_bytes, void* stream);
+int xq_mlp_bwd(const xq_weight* gate, const xq_weight* up, const xq_weight* down, const xq_mlp_lora* lora,
+               const void* x, int64_t ldx, const void* dy, int64_t lddy, int64_t M, const xq_mlp_saved* saved,
+               void* dx, int64_t lddx, const xq_mlp_grads* grads, void* workspace, int64_t workspace_bytes,
+               void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -101,6 +101,34 @@ def test_config1_mlp_chain_full_size(hip_device):
     assert R.max_rel_err(full["y"][rows], ex["y"]) <= 1e-4
 
 
+def test_config1_fused_mlp_full_size(hip_device):
+    """configs[1] through the fused MLP entry points (what the benchmark times): y and dX on a seeded sample of rows
+    against the float64 program, the six factor gradients in full against the fp32 host program."""
+    from xorl_amd.qlora import qlora_mlp_forward
+
+    M, H, I, r = 8192, 4096, 12288, 32
+    dev = hip_device
+    mods, w_ref = {}, {}
+    for i, (k, (N, K)) in enumerate({"gate": (I, H), "up": (I, H), "down": (H, I)}.items()):
+        mods[k], w_ref[k] = make_dense_module("block_fp8", N, K, r, 2 * r, seed=100 + i, device=dev)
+    x = gen((M, H), 1.0, 1, torch.bfloat16)
+    dy = gen((M, H), 1.0, 2, torch.bfloat16)
+    xd = x.to(dev).requires_grad_(True)
+    y = qlora_mlp_forward(mods["gate"], mods["up"], mods["down"], xd)
+    y.backward(dy.to(dev))
+    loras = {k: (m.lora_A.detach().cpu(), m.lora_B.detach().cpu()) for k, m in mods.items()}
+    s = mods["gate"].scaling
+    rows = torch.from_numpy(np.random.default_rng(82).choice(M, NROWS, replace=False)).long()
+    rows[0], rows[1] = 0, M - 1
+    ex = R.mlp_fwd_bwd_exact(x[rows], w_ref["gate"], w_ref["up"], w_ref["down"], loras, s, dy[rows])
+    close(y.detach().cpu()[rows], ex["y"], TOL)
+    close(xd.grad.cpu()[rows], ex["dx"], TOL)
+    full = R.mlp_fwd_bwd_exact(x, w_ref["gate"], w_ref["up"], w_ref["down"], loras, s, dy, dtype=torch.float32)
+    for k, m in mods.items():
+        close(m.lora_A.grad.cpu(), full[f"dA_{k}"], TOL)
+        close(m.lora_B.grad.cpu(), full[f"dB_{k}"], TOL)
+
+
 def test_silu_and_mul_full_size(hip_device):
     """SwiGLU kernels on the [8192, 12288] intermediate of configs[1] against the two-rounding recipe and the
     float64 derivative."""

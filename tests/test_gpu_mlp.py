@@ -1,0 +1,124 @@
+"""GPU parity of the fused dense SwiGLU MLP (xq_mlp_fwd / xq_mlp_bwd through qlora_mlp_forward) against the float64
+program of the oracle and against the three modules called one by one (same rounding points: the base products
+are the same kernels' sums, so the two ways agree to bf16 rounding of reordered fp32 sums)."""
+
+import pytest
+import torch
+
+from oracle import recipe as R
+from tests.util_cases import close, gen, make_dense_module
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-2
+
+
+def _mods(fmt, H, I, r, dev, bias=False, seed=0):
+    mods, w_ref = {}, {}
+    for i, (k, (N, K)) in enumerate({"gate": (I, H), "up": (I, H), "down": (H, I)}.items()):
+        mods[k], w_ref[k] = make_dense_module(fmt, N, K, r, 2 * r, seed=seed + 10 * i, device=dev, bias=bias)
+    return mods, w_ref
+
+
+def _grads(mods):
+    return {f"d{f}_{k}": getattr(m, f"lora_{f}").grad.clone() for k, m in mods.items() for f in ("A", "B")}
+
+
+def _zero(mods):
+    for m in mods.values():
+        m.lora_A.grad = m.lora_B.grad = None
+
+
+@pytest.mark.parametrize("tile_policy", [0, 1, 2], indirect=True)
+@pytest.mark.parametrize("fmt,M,H,I,r", [
+    ("block_fp8", 300, 256, 512, 16),      # fused gate/up/SwiGLU launch, fused dgrad (T = 128 tiles under policy 0)
+    ("block_fp8", 1100, 512, 1024, 32),    # 2 rp = 64: both intermediates from one 64-row panel
+    ("block_fp8", 130, 128, 192, 8),       # intermediate size not a multiple of 128: dgrads launch by launch
+    ("block_fp8", 64, 256, 512, 40),       # 2 rp > 64: separate low-rank passes and dgrads
+    ("nvfp4", 260, 256, 512, 16),          # 4-bit formats: the same program launch by launch
+    ("int4", 200, 256, 384, 16),
+    ("nf4", 200, 256, 384, 16),
+])
+def test_fused_mlp_vs_oracle_and_modules(hip_device, tile_policy, fmt, M, H, I, r):
+    from xorl_amd.functional import silu_and_mul
+    from xorl_amd.qlora import qlora_mlp_forward
+
+    mods, w_ref = _mods(fmt, H, I, r, hip_device, seed=M)
+    x = gen((M, H), 1.0, 71, torch.bfloat16)
+    dy = gen((M, H), 1.0, 72, torch.bfloat16)
+    loras = {k: (m.lora_A.detach().cpu(), m.lora_B.detach().cpu()) for k, m in mods.items()}
+    ex = R.mlp_fwd_bwd_exact(x, w_ref["gate"], w_ref["up"], w_ref["down"], loras, mods["gate"].scaling, dy)
+
+    xd = x.to(hip_device).requires_grad_(True)
+    y = qlora_mlp_forward(mods["gate"], mods["up"], mods["down"], xd)
+    y.backward(dy.to(hip_device))
+    fused = {"y": y.detach().clone(), "dx": xd.grad.clone(), **_grads(mods)}
+    close(fused["y"].cpu(), ex["y"], TOL)
+    close(fused["dx"].cpu(), ex["dx"], TOL)
+    for k in ("gate", "up", "down"):
+        close(fused[f"dA_{k}"].cpu(), ex[f"dA_{k}"], TOL)
+        close(fused[f"dB_{k}"].cpu(), ex[f"dB_{k}"], TOL)
+
+    _zero(mods)
+    xs = x.to(hip_device).requires_grad_(True)
+    ys = mods["down"](silu_and_mul(mods["gate"](xs), mods["up"](xs)))
+    ys.backward(dy.to(hip_device))
+    sep = {"y": ys.detach(), "dx": xs.grad, **_grads(mods)}
+    for name in fused:
+        assert R.max_rel_err(fused[name].float().cpu(), sep[name].double().cpu()) <= 2 ** -7, name     # a bf16 step of the largest entry: dX is one rounded sum here, the sum of two rounded products there
+    # a forward without grad (inference) gives the training forward's bits
+    with torch.no_grad():
+        assert torch.equal(qlora_mlp_forward(mods["gate"], mods["up"], mods["down"], x.to(hip_device)), fused["y"])
+
+
+def test_fused_mlp_bias_no_lora_and_fallbacks(hip_device):
+    from xorl_amd.qlora import qlora_mlp_forward
+
+    H, I, M = 256, 512, 200
+    mods, w_ref = _mods("block_fp8", H, I, 16, hip_device, bias=True, seed=3)
+    x = gen((M, H), 1.0, 81, torch.bfloat16)
+    dy = gen((M, H), 1.0, 82, torch.bfloat16)
+    # biases on all three projections, against the float64 program
+    Wg, Wu, Wd = (w_ref[k].double() for k in ("gate", "up", "down"))
+    s = mods["gate"].scaling
+    lin = lambda inp, W, m: inp @ W.t() + m.bias.detach().cpu().double() + s * ((inp @ m.lora_A.detach().cpu().double().t()) @ m.lora_B.detach().cpu().double().t())
+    X = x.double()
+    want = lin(torch.nn.functional.silu(lin(X, Wg, mods["gate"])) * lin(X, Wu, mods["up"]), Wd, mods["down"])
+    with torch.no_grad():
+        y = qlora_mlp_forward(mods["gate"], mods["up"], mods["down"], x.to(hip_device))
+    close(y.cpu(), want, TOL)
+    # frozen biases: the backward still returns dx and the factor gradients
+    xd = x.to(hip_device).requires_grad_(True)
+    qlora_mlp_forward(mods["gate"], mods["up"], mods["down"], xd).backward(dy.to(hip_device))
+    assert xd.grad is not None and mods["down"].lora_B.grad is not None
+    # different active ranks: the helper calls the modules one by one and still agrees
+    mods["up"].set_runtime_lora_config(8, 16)
+    with torch.no_grad():
+        y2 = qlora_mlp_forward(mods["gate"], mods["up"], mods["down"], x.to(hip_device))
+    assert y2.shape == y.shape and bool(torch.isfinite(y2.float()).all())
+    # empty batch
+    with torch.no_grad():
+        y0 = qlora_mlp_forward(mods["gate"], mods["down"].__class__(H, I, device=hip_device) if False else mods["up"], mods["down"],
+                               torch.zeros(0, H, dtype=torch.bfloat16, device=hip_device))
+    assert y0.shape == (0, H)
+
+
+@pytest.mark.parametrize("backend", ["eager", "aot_eager"])
+def test_fused_mlp_under_torch_compile(hip_device, backend):
+    from xorl_amd.qlora import qlora_mlp_forward
+
+    mods, _ = _mods("block_fp8", 256, 512, 16, hip_device, seed=9)
+    x = gen((300, 256), 1.0, 91, torch.bfloat16).to(hip_device)
+    dy = gen((300, 256), 1.0, 92, torch.bfloat16).to(hip_device)
+
+    def run(fn):
+        _zero(mods)
+        xd = x.clone().requires_grad_(True)
+        y = fn(mods["gate"], mods["up"], mods["down"], xd)
+        y.backward(dy)
+        return [y.detach().clone(), xd.grad.clone()] + list(_grads(mods).values())
+
+    ref = run(qlora_mlp_forward)
+    torch._dynamo.reset()
+    got = run(torch.compile(qlora_mlp_forward, backend=backend, fullgraph=True))
+    for a, b in zip(ref, got):
+        assert torch.equal(a, b)

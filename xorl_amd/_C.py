@@ -55,6 +55,19 @@ class XqGroupedGrads(ctypes.Structure):
     _fields_ = [("dA", ctypes.c_void_p * 3), ("dB", ctypes.c_void_p * 3)]
 
 
+class XqMlpLora(ctypes.Structure):
+    _fields_ = [("A", ctypes.c_void_p * 3), ("B", ctypes.c_void_p * 3), ("bias", ctypes.c_void_p * 3),
+                ("dtype", ctypes.c_int32), ("r", ctypes.c_int32), ("scaling", ctypes.c_float), ("reserved", ctypes.c_int32)]
+
+
+class XqMlpSaved(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_void_p) for n in ("gate_up", "h", "su_gate_up", "su_down")]
+
+
+class XqMlpGrads(ctypes.Structure):
+    _fields_ = [("dA", ctypes.c_void_p * 3), ("dB", ctypes.c_void_p * 3)]
+
+
 class XqError(ValueError):
     """Argument error reported by the library before any launch."""
 
@@ -118,6 +131,13 @@ _SIGNATURES = {
     "xq_grouped_bwd": (_INT, [_W, _W, _W, ctypes.POINTER(XqGroupedLora), _P, _I64, _I64, _I32,
                               ctypes.POINTER(XqGroupedSaved), _P, _I64, _P, _INT, ctypes.POINTER(XqGroupedGrads), _P, _I64,
                               _P]),
+    "xq_mlp_workspace_bytes": (_I64, [_I64, _I64, _I64, _INT, _INT]),
+    # gate, up, down, lora, x, ldx, M, y, ldy, saved, ws, ws_bytes, stream
+    "xq_mlp_fwd": (_INT, [_W, _W, _W, ctypes.POINTER(XqMlpLora), _P, _I64, _I64, _P, _I64, ctypes.POINTER(XqMlpSaved), _P,
+                          _I64, _P]),
+    # gate, up, down, lora, x, ldx, dy, lddy, M, saved, dx, lddx, grads, ws, ws_bytes, stream
+    "xq_mlp_bwd": (_INT, [_W, _W, _W, ctypes.POINTER(XqMlpLora), _P, _I64, _P, _I64, _I64, ctypes.POINTER(XqMlpSaved), _P,
+                          _I64, ctypes.POINTER(XqMlpGrads), _P, _I64, _P]),
 }
 
 EXPORTS = ("xq_version", "xq_last_error") + tuple(_SIGNATURES)

@@ -61,6 +61,11 @@ __device__ __forceinline__ bf16_t to_bf16(float f) {
 }
 __device__ __forceinline__ float bf16_to_f32(bf16_t h) { return __uint_as_float((uint32_t)h << 16); }
 
+// SwiGLU arithmetic shared by the elementwise kernels and the fused GEMM epilogues (ops/fused_silu_and_mul.py:22-60):
+// sigmoid in fp32, the activation rounded to bf16 before it meets `up`
+__device__ __forceinline__ float sigmoid_f32(float x) { return 1.0f / (1.0f + __expf(-x)); }
+__device__ __forceinline__ float round_bf16(float x) { return bf16_to_f32(to_bf16(x)); }
+
 // e4m3fn (OCP) byte pair -> two fp32: v_cvt_pk_f32_fp8.  hi selects the upper
 // 16 bits of the dword.
 __device__ __forceinline__ f32x2 e4m3x2_to_f32(uint32_t word, bool hi) {

@@ -146,6 +146,12 @@ bool two_banks_supported(const xq_weight* w) {
     return w->format == XQ_FMT_FP8 && g_tile_policy != 1 && w->cols % 256 == 0 && w->cols >= 512 && w->num_experts >= 1;
 }
 
+// Whether the dgrad of two dense [N, K] weights of one shape may run as one launch (see launch_tile_gemm): block-fp8 on
+// the pipelined kernel, the change of matrix on a scale-block boundary and past the pipeline's prologue.
+bool two_dense_supported(const xq_weight* w) {
+    return w->format == XQ_FMT_FP8 && g_tile_policy != 1 && w->num_experts == 1 && w->rows % 128 == 0 && w->rows >= 512;
+}
+
 // C[rows, Nout] = A . op(deq(W)) (+ su . Lr^T) (+ bias); see xq_gemm_tile.h.  force_T = 256 / 128 fixes the tile
 // size of the pipelined kernel (and force_split its K splits), 0 leaves both to the selection policy.  `partial` (may be NULL) is scratch for
 // split-K sums; a launch that would split but finds less than tile_gemm_partial_bytes() there runs unsplit.
@@ -165,12 +171,22 @@ static int launch_tile_gemm_t(const xq_weight* w, bool contract_cols, const bf16
     g.group = w->group; g.scale_dtype = w->scale_dtype;
     g.Kc = contract_cols ? g.wcols : g.wrows;
     g.Nout = contract_cols ? g.wrows : g.wcols;
-    if (two) {       // a second bank of the same shape: twice the contraction (dgrad) or twice the output columns (forward)
-        XQ_REQUIRE(offsets && two_banks_supported(w) && two->w2 && two_banks_supported(two->w2) && two->w2->rows == w->rows &&
-                       two->w2->cols == w->cols && two->w2->num_experts == w->num_experts,
-                   "%s: a two-bank launch takes two block-fp8 expert banks of one shape (columns a multiple of 256)", who);
-        if (contract_cols) g.Kc *= 2;
-        else g.Nout *= 2;
+    const bool two_dense = two && !offsets;
+    if (two) {
+        // a second matrix of the same shape.  Expert banks: twice the contraction (dgrad) or twice the output columns
+        // (forward).  Dense [N, K] weights: the dgrad contracts over the rows of both, dX = [dY1 | dY2] . [W1 ; W2].
+        XQ_REQUIRE(two->w2 && two->w2->rows == w->rows && two->w2->cols == w->cols && two->w2->num_experts == w->num_experts,
+                   "%s: a two-matrix launch takes two weights of one shape", who);
+        if (two_dense) {
+            XQ_REQUIRE(!contract_cols && two_dense_supported(w) && two_dense_supported(two->w2),
+                       "%s: the dense two-matrix form is the dgrad of two block-fp8 weights (out_features %% 128 == 0, >= 512)", who);
+            g.Kc *= 2;
+        } else {
+            XQ_REQUIRE(two_banks_supported(w) && two_banks_supported(two->w2),
+                       "%s: a two-bank launch takes two block-fp8 expert banks (columns a multiple of 256)", who);
+            if (contract_cols) g.Kc *= 2;
+            else g.Nout *= 2;
+        }
     }
     g.n_rows = n_rows; g.offsets = offsets; g.tile_offsets = tile_offsets; g.num_experts = w->num_experts;
     g.su = su; g.lora_right = lora_right; g.r_pad = (su && lora_right) ? r_pad : 0;
@@ -199,7 +215,7 @@ static int launch_tile_gemm_t(const xq_weight* w, bool contract_cols, const bf16
                                       : w->layout == XQ_LAYOUT_FLAT));
         const bool big = grouped && n_rows >= 128ll * w->num_experts && n_rows >= 8192;   // grouped: large tiles
         const DensePlan plan = plan_dense(n_rows, g.Nout, g.Kc / BK);
-        const bool planned = !grouped && fmt_ok && g_tile_policy == 0 && force_T == 0;
+        const bool planned = !grouped && fmt_ok && g_tile_policy == 0 && force_T == 0 && !two_dense;   // two matrices: one unsplit launch
         const int T = force_T ? force_T : g_tile_policy == 2 ? 256 : g_tile_policy == 3 ? 128 : grouped ? (big ? 256 : 128) : plan.T;
         if (planned && plan.head_rows < n_rows) {
             const int64_t head = plan.head_rows;
@@ -225,14 +241,15 @@ static int launch_tile_gemm_t(const xq_weight* w, bool contract_cols, const bf16
             f.su = g.r_pad ? su : nullptr; f.lora_right = g.r_pad ? lora_right : nullptr; f.r_pad = g.r_pad;
             f.bias = bias;
             f.tiles_m = (int32_t)tiles_m; f.tiles_n = (int32_t)tiles_n;
-            int ksplit = grouped ? 1 : force_T ? force_split : planned ? plan.split : ksplit_for(tiles_m * tiles_n, T, g.Kc / BK);
+            int ksplit = grouped || two_dense ? 1 : force_T ? force_split : planned ? plan.split : ksplit_for(tiles_m * tiles_n, T, g.Kc / BK);
             if (ksplit > 1 && (!partial || !xq_aligned(partial, 16) || partial_bytes < (int64_t)ksplit * n_rows * g.Nout * 4)) ksplit = 1;
             f.ksplit = ksplit; f.partial = ksplit > 1 ? partial : nullptr;
             f.W2 = nullptr; f.scales2 = nullptr; f.su2 = nullptr; f.lora_right2 = nullptr; f.ncols1 = 0; f.nk1 = 0;
+            f.ld_su = g.r_pad; f.H = nullptr; f.ldh = 0; f.bias2 = nullptr;
             if (two) {
                 f.W2 = (const uint8_t*)two->w2->packed; f.scales2 = (const uint8_t*)two->w2->scales;
                 f.su2 = g.r_pad ? two->su2 : nullptr; f.lora_right2 = g.r_pad ? two->lora_right2 : nullptr;
-                f.ncols1 = g.wcols; f.nk1 = g.wcols / BK;
+                f.ncols1 = g.wcols; f.nk1 = (two_dense ? g.wrows : g.wcols) / BK;
             }
             dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)ksplit);
             const bool timed = xq_profile_mark_begin(stream, 2.0 * (double)n_rows * g.Nout * ((double)g.Kc + g.r_pad));
@@ -264,6 +281,53 @@ static int launch_tile_gemm_t(const xq_weight* w, bool contract_cols, const bf16
     else launch_tile_cc<XQ_FMT_NVFP4, XQ_LAYOUT_GKN>(g, contract_cols, grid, stream);
     if (timed) xq_profile_mark_end(stream);
     XQ_CHECK_LAUNCH(who);
+    return XQ_OK;
+}
+
+// gate | up | SwiGLU of a dense block-fp8 MLP in one launch: gu[M, 2I] = (x . deq(Wg)^T + side term | x . deq(Wu)^T +
+// side term) and h[M, I] = bf16(silu(gate)) * up from the rounded projections.  Both weights [I, K] block-fp8.
+int launch_gate_up_swiglu(const xq_weight* wg, const xq_weight* wu, const bf16_t* x, int64_t ldx, int64_t M,
+                          const bf16_t* su_g, const bf16_t* su_u, int64_t ld_su, const bf16_t* lr_g, const bf16_t* lr_u,
+                          int r_pad, const bf16_t* bias_g, const bf16_t* bias_u, bf16_t* gu, int64_t ldgu, bf16_t* h,
+                          int64_t ldh, hipStream_t stream) {
+    static const char* who = "gate_up_swiglu";
+    XQ_REQUIRE(wg->format == XQ_FMT_FP8 && wu->format == XQ_FMT_FP8 && wg->rows == wu->rows && wg->cols == wu->cols,
+               "%s: two block-fp8 weights of one shape", who);
+    const int64_t I = wg->rows, K = wg->cols;
+    XQ_REQUIRE(K % BK == 0 && I % 16 == 0, "%s: in_features %% 64 == 0 and out_features %% 16 == 0", who);
+    XQ_REQUIRE(ldx % 8 == 0 && xq_aligned(x, 16) && xq_aligned(wg->packed, 16) && xq_aligned(wu->packed, 16),
+               "%s: operands must be 16-byte aligned", who);
+    XQ_REQUIRE(ldgu % 4 == 0 && ldh % 4 == 0 && xq_aligned(gu, 8) && xq_aligned(h, 8), "%s: output rows must be 8-byte aligned", who);
+    const bool side = su_g && su_u && lr_g && lr_u && r_pad > 0;
+    XQ_REQUIRE(!side || (r_pad % 16 == 0 && r_pad <= 64 && ld_su >= r_pad && ld_su % 8 == 0 && xq_aligned(su_g, 16) &&
+                         xq_aligned(su_u, 16) && xq_aligned(lr_g, 16) && xq_aligned(lr_u, 16)),
+               "%s: bad low-rank side term", who);
+    if (M == 0) return XQ_OK;
+    G256Args f{};
+    f.A = x; f.lda = ldx; f.C = gu; f.ldc = ldgu;
+    f.W = (const uint8_t*)wg->packed; f.scales = (const uint8_t*)wg->scales;
+    f.W2 = (const uint8_t*)wu->packed; f.scales2 = (const uint8_t*)wu->scales;
+    f.wrows = (int32_t)I; f.wcols = (int32_t)K; f.scale_dtype = XQ_SCALE_F32;
+    f.Kc = (int32_t)K; f.Nout = (int32_t)I; f.M = M;
+    f.num_experts = 1;
+    f.su = side ? su_g : nullptr; f.su2 = side ? su_u : nullptr; f.ld_su = ld_su;
+    f.lora_right = side ? lr_g : nullptr; f.lora_right2 = side ? lr_u : nullptr; f.r_pad = side ? r_pad : 0;
+    f.bias = bias_g; f.bias2 = bias_u;
+    f.tiles_m = (int32_t)xq_cdiv(M, 256); f.tiles_n = (int32_t)xq_cdiv(I, 128);
+    f.ksplit = 1;
+    f.H = h; f.ldh = ldh;
+    static std::atomic<bool> attr_set{false};
+    if (!attr_set) {
+        int rc = raise_lds_limit(gemm_256_kernel<XQ_FMT_FP8, true, false, 256, false, true>, Geo<256>::lds_bytes(true), who);
+        if (rc) return rc;
+        attr_set = true;
+    }
+    // flops of the two projections and their side terms
+    const bool timed = xq_profile_mark_begin(stream, 2.0 * (double)M * (2.0 * I) * ((double)K + f.r_pad));
+    gemm_256_kernel<XQ_FMT_FP8, true, false, 256, false, true>
+        <<<dim3((unsigned)(f.tiles_m * f.tiles_n)), Geo<256>::NT, Geo<256>::lds_bytes(true), stream>>>(f);
+    XQ_CHECK_LAUNCH(who);
+    if (timed) xq_profile_mark_end(stream);
     return XQ_OK;
 }
 

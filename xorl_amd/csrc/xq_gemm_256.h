@@ -95,6 +95,13 @@ struct G256Args {
     const bf16_t* su2;
     const bf16_t* lora_right2;
     int32_t ncols1, nk1;
+    int64_t ld_su;             // row pitch of su / su2 in elements (>= r_pad)
+    // gate / up / SwiGLU launch (template flag GU, dense block-fp8 forward): W is the gate weight, W2 the up weight, both
+    // [Nout, Kc]; a tile holds 128 gate columns and the same 128 up columns, C is [M, 2 * Nout] (gate | up) and
+    // H [M, Nout] receives bf16(silu(gate)) * up computed from the rounded outputs in the epilogue
+    bf16_t* H;
+    int64_t ldh;
+    const bf16_t* bias2;
 };
 
 // ---------------------------------------------------------------- weight-tile loaders
@@ -146,6 +153,18 @@ struct W256Fp8 {
             raw[p] = *(const u32x4*)(src[p] + kt * kstep);
             s[p] = CC ? s_src[p][k0 >> 7] : s_src[p][(k0 >> 7) * scols];
         }
+    }
+    // gate / up tile: run 0 of a thread is a row of the gate weight, run 1 the same row of the up weight (LDS rows
+    // tid >> 2 and 128 + (tid >> 2) of the [n][kc] tile)
+    __device__ __forceinline__ void init_gu(const G256Args& g, int n0, int tid_) {
+        tid = tid_;
+        scols = (g.wcols + 127) >> 7;
+        const int wr = min(n0 + (tid >> 2), g.wrows - 1), wc = (tid & 3) * 16;
+        src[0] = g.W + (int64_t)wr * g.wcols + wc;
+        src[1] = g.W2 + (int64_t)wr * g.wcols + wc;
+        s_src[0] = (const float*)g.scales + (wr >> 7) * scols;
+        s_src[1] = (const float*)g.scales2 + (wr >> 7) * scols;
+        kstep = F8_BK;
     }
     // continue on another matrix of the same shape: byte and scale offsets between the two, both uniform
     __device__ __forceinline__ void rebase(int64_t wdelta, int64_t sdelta) {
@@ -389,8 +408,9 @@ template <bool CC, bool GROUPED, int T> struct W256Sel<XQ_FMT_FP8, CC, GROUPED, 
 template <bool CC, int T> struct W256Sel<XQ_FMT_FP8, CC, true, T> { using type = W256Fp8<CC, T>; };
 
 // ---------------------------------------------------------------- the kernel
-template <int FMT, bool CC, bool GROUPED, int T, bool SPLIT256 = false>
+template <int FMT, bool CC, bool GROUPED, int T, bool SPLIT256 = false, bool GU = false>
 __global__ void __launch_bounds__(2 * T, 2) gemm_256_kernel(G256Args g) {
+    static_assert(!GU || (FMT == XQ_FMT_FP8 && CC && !GROUPED && T == 256 && !SPLIT256), "gate / up tiles: dense block-fp8 forward");
     using G = Geo<T>;
     constexpr int F8_BM = G::BM, F8_BN = G::BN, F8_A_STAGE = G::A_STAGE, F8_NN_PITCH = G::NN_PITCH;
     constexpr int TM = G::TM, TN = G::TN, NT = G::NT;
@@ -455,7 +475,7 @@ __global__ void __launch_bounds__(2 * T, 2) gemm_256_kernel(G256Args g) {
         row0 = (int64_t)pid_m * F8_BM;
         row_end = g.M;
     }
-    const int n0 = pid_n * F8_BN;
+    const int n0 = GU ? pid_n * (F8_BN / 2) : pid_n * F8_BN;      // GU: first gate (= up) column of the tile
     // two banks (grouped block-fp8 only): a forward block past the first bank's columns works on the second bank
     constexpr bool TWO_OK = GROUPED && FMT == XQ_FMT_FP8;
     const uint8_t* Wb = g.W;
@@ -500,17 +520,22 @@ __global__ void __launch_bounds__(2 * T, 2) gemm_256_kernel(G256Args g) {
     using WL = typename W256Sel<FMT, CC, GROUPED, T>::type;
     WL wls[PD];
 #pragma unroll
-    for (int d = 0; d < PD; ++d)
-        wls[d].init(g, Wb + (int64_t)e * g.packed_stride, Sb + (int64_t)e * g.scale_stride,
-                    FMT == XQ_FMT_NVFP4 ? g.global_scale[e] : 1.0f, n0w, tid);
-    // dgrad over two banks: the K-steps from nk1 on read the second bank (same expert offset in both)
+    for (int d = 0; d < PD; ++d) {
+        if constexpr (GU) wls[d].init_gu(g, n0, tid);
+        else wls[d].init(g, Wb + (int64_t)e * g.packed_stride, Sb + (int64_t)e * g.scale_stride,
+                         FMT == XQ_FMT_NVFP4 ? g.global_scale[e] : 1.0f, n0w, tid);
+    }
+    // contraction over two matrices of one shape (expert-bank dgrad of gate and up; dense dgrad of gate and up): the
+    // K-steps from nk1 on read the second one (same expert offset in both)
+    constexpr bool TWO_K = FMT == XQ_FMT_FP8 && !GU && ((GROUPED && CC) || (!GROUPED && !CC && !SPLIT256));
     int64_t wdelta = 0, sdelta = 0;
     int nk1 = 1 << 30;
-    if constexpr (TWO_OK && CC) {
+    if constexpr (TWO_K) {
         if (g.W2 != nullptr) {
             nk1 = g.nk1;
-            wdelta = (g.W2 - g.W) - (int64_t)nk1 * F8_BK;
-            sdelta = ((const float*)g.scales2 - (const float*)g.scales) - (nk1 >> 1);
+            const int64_t scols = (g.wcols + 127) >> 7;
+            wdelta = (g.W2 - g.W) - (int64_t)nk1 * (CC ? F8_BK : (int64_t)F8_BK * g.wcols);
+            sdelta = ((const float*)g.scales2 - (const float*)g.scales) - (int64_t)(nk1 >> 1) * (CC ? 1 : scols);
         }
     }
     if constexpr (FMT == XQ_FMT_NF4) {
@@ -546,7 +571,8 @@ __global__ void __launch_bounds__(2 * T, 2) gemm_256_kernel(G256Args g) {
         for (int i = 0; i < TM; ++i) af[i] = *(const bf16x8*)(a + swz(wm * (T / 2) + i * 32 + fr, ks * 2 + fh));
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
-            if (CC || b_is_nt) bfr[j] = *(const bf16x8*)(b + swz(wn * 64 + j * 32 + fr, ks * 2 + fh));
+            if (GU) bfr[j] = *(const bf16x8*)(b + swz(j * 128 + wn * 32 + fr, ks * 2 + fh));    // j = 0 gate, 1 up: same columns
+            else if (CC || b_is_nt) bfr[j] = *(const bf16x8*)(b + swz(wn * 64 + j * 32 + fr, ks * 2 + fh));
             else bfr[j] = lds_tr_frag(b, F8_NN_PITCH, ks * 16, wn * 64 + j * 32, lane);
         }
     };
@@ -590,7 +616,7 @@ __global__ void __launch_bounds__(2 * T, 2) gemm_256_kernel(G256Args g) {
         // region 2: MFMAs of step 1 over the weight decode + stores, the next weight loads, step-2 fragment reads
         mma(af1, bf1);
         if (have_next) { wl.store(bn, 0); wl.store(bn, 1); }
-        if constexpr (TWO_OK && CC) {
+        if constexpr (TWO_K) {
             if (kload >= nk1 && kload - PD < nk1) wl.rebase(wdelta, sdelta);     // uniform; once per loader and tile
         }
         if (have_next2) wl.load(kt0 + kload);
@@ -649,17 +675,66 @@ __global__ void __launch_bounds__(2 * T, 2) gemm_256_kernel(G256Args g) {
             const int r = idx / cpr, c = idx - r * cpr;
             int64_t row = row0 + r;
             row = row < row_end ? row : row_end - 1;
-            *(u32x4*)(As + swz(r, c)) = *(const u32x4*)(su_b + row * rp + c * 8);
-            int n = n0w + r;
-            n = n < bank_width ? n : bank_width - 1;
-            *(u32x4*)(Bs + swz(r, c)) = *(const u32x4*)(lr + (int64_t)n * rp + c * 8);
+            *(u32x4*)(As + swz(r, c)) = *(const u32x4*)(su_b + row * g.ld_su + c * 8);
+            if constexpr (GU) {
+                // the up projection's intermediate in the second activation stage; factor rows: 128 of gate's, 128 of up's
+                *(u32x4*)(As + F8_A_STAGE + swz(r, c)) = *(const u32x4*)(g.su2 + row * g.ld_su + c * 8);
+                int n = n0 + (r & 127);
+                n = n < g.Nout ? n : g.Nout - 1;
+                *(u32x4*)(Bs + swz(r, c)) = *(const u32x4*)((r < 128 ? g.lora_right : g.lora_right2) + (int64_t)n * rp + c * 8);
+            } else {
+                int n = n0w + r;
+                n = n < bank_width ? n : bank_width - 1;
+                *(u32x4*)(Bs + swz(r, c)) = *(const u32x4*)(lr + (int64_t)n * rp + c * 8);
+            }
         }
         __syncthreads();
         for (int ks = 0; ks < (rp >> 4); ++ks) {
             bf16x8 af[TM], bfr[TN];
             load_frags(As, Bs, ks, true, af, bfr);
-            mma(af, bfr);
+            if constexpr (GU) {
+                bf16x8 af2[TM], unused[TN];
+                load_frags(As + F8_A_STAGE, Bs, ks, true, af2, unused);
+#pragma unroll
+                for (int i = 0; i < TM; ++i) {
+                    acc[i][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[0], af[i], acc[i][0], 0, 0, 0);
+                    acc[i][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[1], af2[i], acc[i][1], 0, 0, 0);
+                }
+            } else {
+                mma(af, bfr);
+            }
         }
+    }
+
+    // ---- gate / up epilogue: acc[i][0] is the gate, acc[i][1] the up projection of the same 4 x 4 columns
+    if constexpr (GU) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            const int64_t row = row0 + wm * (T / 2) + i * 32 + fr;
+            if (row >= row_end) continue;
+            bf16_t* crow = g.C + row * g.ldc;
+            bf16_t* hrow = g.H + row * g.ldh;
+#pragma unroll
+            for (int q4 = 0; q4 < 4; ++q4) {
+                const int n = n0 + wn * 32 + 8 * q4 + 4 * fh;
+                if (n >= g.Nout) continue;
+                float gv[4], uv[4], hv[4];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    gv[c] = acc[i][0][4 * q4 + c];
+                    uv[c] = acc[i][1][4 * q4 + c];
+                    if (g.bias) gv[c] += bf16_to_f32(g.bias[n + c]);
+                    if (g.bias2) uv[c] += bf16_to_f32(g.bias2[n + c]);
+                    gv[c] = round_bf16(gv[c]);                       // the two projections as their bf16 outputs
+                    uv[c] = round_bf16(uv[c]);
+                    hv[c] = round_bf16(gv[c] * sigmoid_f32(gv[c])) * uv[c];
+                }
+                *(u32x2*)(crow + n) = u32x2{pack_bf16x2(gv[0], gv[1]), pack_bf16x2(gv[2], gv[3])};
+                *(u32x2*)(crow + g.Nout + n) = u32x2{pack_bf16x2(uv[0], uv[1]), pack_bf16x2(uv[2], uv[3])};
+                *(u32x2*)(hrow + n) = u32x2{pack_bf16x2(hv[0], hv[1]), pack_bf16x2(hv[2], hv[3])};
+            }
+        }
+        return;
     }
 
     // ---- epilogue: lane holds, per (i, j) tile, row m = fr and 4 x 4 consecutive columns

@@ -22,60 +22,6 @@ struct Carve {
     }
 };
 
-// ---- every LoRA panel of a call in one launch: job k converts a [n_src, R_in, C_in] fp32 / bf16 factor (n_src = 1
-// or the expert count) into bf16 [n_out, R_out, C_out], optionally transposed, zero padded; n_src == 1 < n_out
-// repeats the one source matrix for every expert (a factor shared by all experts, handed to a kernel that indexes
-// panels by expert).
-constexpr int MAX_PREP_JOBS = 6;
-struct PrepJobs {
-    const void* in[MAX_PREP_JOBS];
-    bf16_t* out[MAX_PREP_JOBS];
-    int64_t R_in[MAX_PREP_JOBS], C_in[MAX_PREP_JOBS], R_out[MAX_PREP_JOBS], C_out[MAX_PREP_JOBS], pitch[MAX_PREP_JOBS];
-    int32_t n_src[MAX_PREP_JOBS], n_out[MAX_PREP_JOBS], transpose[MAX_PREP_JOBS];
-    int32_t in_f32, n;
-    // `pitch` (0: c_out) is the row length of the destination, for a panel that is a column band of a wider one
-    bf16_t* add(const void* src, int n_src_, int64_t r_in, int64_t c_in, bool tr, bf16_t* dst, int n_out_, int64_t r_out,
-                int64_t c_out, int64_t pitch_ = 0) {
-        in[n] = src; out[n] = dst; R_in[n] = r_in; C_in[n] = c_in; R_out[n] = r_out; C_out[n] = c_out;
-        pitch[n] = pitch_ ? pitch_ : c_out;
-        n_src[n] = n_src_; n_out[n] = n_out_; transpose[n] = tr ? 1 : 0;
-        ++n;
-        return dst;
-    }
-};
-
-__global__ void __launch_bounds__(256) grouped_prep_kernel(PrepJobs j) {
-    const int k = blockIdx.y;
-    const int64_t per = j.R_out[k] * j.C_out[k], total = per * j.n_out[k];
-    const int64_t R_in = j.R_in[k], C_in = j.C_in[k], C_out = j.C_out[k], R_out = j.R_out[k], pitch = j.pitch[k];
-    const bool tr = j.transpose[k] != 0, shared = j.n_src[k] == 1;
-    for (int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x; t < total; t += (int64_t)gridDim.x * 256) {
-        const int64_t e = t / per, rem = t - e * per;
-        const int64_t i = rem / C_out, c = rem - i * C_out;
-        const int64_t si = tr ? c : i, sj = tr ? i : c;
-        float v = 0.0f;
-        if (si < R_in && sj < C_in) {
-            const int64_t idx = (shared ? 0 : e) * R_in * C_in + si * C_in + sj;
-            v = j.in_f32 ? ((const float*)j.in[k])[idx] : bf16_to_f32(((const bf16_t*)j.in[k])[idx]);
-        }
-        j.out[k][(e * R_out + i) * pitch + c] = to_bf16(v);
-    }
-}
-
-int launch_prep(const PrepJobs& j, hipStream_t stream) {
-    int64_t most = 0;
-    for (int k = 0; k < j.n; ++k) {
-        const int64_t t = j.R_out[k] * j.C_out[k] * j.n_out[k];
-        most = t > most ? t : most;
-    }
-    if (j.n == 0 || most == 0) return XQ_OK;
-    int64_t blocks = xq_cdiv(most, 256);
-    if (blocks > 4096) blocks = 4096;
-    grouped_prep_kernel<<<dim3((unsigned)blocks, (unsigned)j.n), 256, 0, stream>>>(j);
-    XQ_CHECK_LAUNCH("grouped_prep");
-    return XQ_OK;
-}
-
 // dst0[m][i][j] = src[m][i][j], dst1[m][i][j] = src[m][i][half + j] for j < r: the two factor gradients that one
 // pass over the rows produced side by side
 __global__ void __launch_bounds__(256) split_pair_kernel(const float* src, int64_t rows, int half, int r, float* dst0, float* dst1) {
@@ -184,7 +130,7 @@ extern "C" int xq_grouped_fwd(const xq_weight* gate, const xq_weight* up, const 
 
     // bf16 operand layouts of the six factors, one launch.  A factors [E|1, in, r] become the "down" panels
     // [E|1, rp, in] of x . A; B factors [E|1, r, out] become the per-expert right-hand panels [E, out, rp].
-    PrepJobs jobs{};
+    PanelJobs jobs{};
     jobs.in_f32 = lora->dtype == XQ_DT_F32;
     const int gAe = lora->A_experts[0], uAe = lora->A_experts[1], dAe = lora->A_experts[2];
     bf16_t* F_gA = jobs.add(lora->A[0], gAe, H, d.r, true, cv.take<bf16_t>((int64_t)gAe * rp * H * 2), gAe, rp, H);
@@ -193,7 +139,7 @@ extern "C" int xq_grouped_fwd(const xq_weight* gate, const xq_weight* up, const 
     bf16_t* Lr_uB = jobs.add(lora->B[1], lora->B_experts[1], d.r, I, true, cv.take<bf16_t>((int64_t)E * I * rp * 2), E, I, rp);
     bf16_t* F_dA = jobs.add(lora->A[2], dAe, I, d.r, true, cv.take<bf16_t>((int64_t)dAe * rp * I * 2), dAe, rp, I);
     bf16_t* Lr_dB = jobs.add(lora->B[2], lora->B_experts[2], d.r, H, true, cv.take<bf16_t>((int64_t)E * H * rp * 2), E, H, rp);
-    if ((rc = launch_prep(jobs, stream))) return rc;
+    if ((rc = launch_panel_prep(jobs, stream))) return rc;
     bf16_t* down_out = cv.take<bf16_t>(R * H * 2);
 
     const int32_t *off = saved->offsets, *toff = saved->tile_offsets;
@@ -258,7 +204,7 @@ extern "C" int xq_grouped_bwd(const xq_weight* gate, const xq_weight* up, const 
     // every panel of the call in one launch: B factors [E|1, r, out] as the "down" panels [E|1, rp, out] of g . B^T,
     // A factors [E|1, in, r] as the per-expert right-hand panels [E, in, rp] of the dgrads (gate's and up's side by
     // side in one [E, H, 2 rp] panel when their dgrads share a launch)
-    PrepJobs jobs{};
+    PanelJobs jobs{};
     jobs.in_f32 = lora->dtype == XQ_DT_F32;
     bf16_t* F_dB = jobs.add(lora->B[2], dBe, r, H, false, cv.take<bf16_t>((int64_t)dBe * rp * H * 2), dBe, rp, H);
     bf16_t* Lr_dA = jobs.add(lora->A[2], dAe, I, r, false, cv.take<bf16_t>((int64_t)E * I * rp * 2), E, I, rp);
@@ -268,7 +214,7 @@ extern "C" int xq_grouped_bwd(const xq_weight* gate, const xq_weight* up, const 
     bf16_t* Lr_uA = fused ? Lr_guA + rp : Lr_guA + (int64_t)E * H * rp;
     jobs.add(lora->A[0], gAe, H, r, false, Lr_guA, E, H, rp, fused ? rp2 : rp);
     jobs.add(lora->A[1], uAe, H, r, false, Lr_uA, E, H, rp, fused ? rp2 : rp);
-    if ((rc = launch_prep(jobs, stream))) return rc;
+    if ((rc = launch_panel_prep(jobs, stream))) return rc;
 
     bf16_t* g_down = cv.take<bf16_t>(R * H * 2);
     bf16_t* dx_g = cv.take<bf16_t>(R * H * 2);

@@ -22,6 +22,29 @@ struct FactorPrepJobs {
     }
 };
 int launch_factor_prep_multi(const FactorPrepJobs& jobs, hipStream_t stream);
+
+// Every LoRA panel of a call in one launch: job k converts a [n_src, R_in, C_in] fp32 / bf16 factor (n_src = 1 or
+// the expert count) into bf16 [n_out, R_out, C_out], optionally transposed, zero padded; n_src == 1 < n_out repeats
+// the one source matrix for every expert (a factor shared by all experts, handed to a kernel that indexes panels
+// by expert).  `pitch` (0: C_out) is the row length of the destination, for a panel that is a column band of a
+// wider one.
+constexpr int MAX_PANEL_JOBS = 6;
+struct PanelJobs {
+    const void* in[MAX_PANEL_JOBS];
+    bf16_t* out[MAX_PANEL_JOBS];
+    int64_t R_in[MAX_PANEL_JOBS], C_in[MAX_PANEL_JOBS], R_out[MAX_PANEL_JOBS], C_out[MAX_PANEL_JOBS], pitch[MAX_PANEL_JOBS];
+    int32_t n_src[MAX_PANEL_JOBS], n_out[MAX_PANEL_JOBS], transpose[MAX_PANEL_JOBS];
+    int32_t in_f32, n;
+    bf16_t* add(const void* src, int n_src_, int64_t r_in, int64_t c_in, bool tr, bf16_t* dst, int n_out_, int64_t r_out,
+                int64_t c_out, int64_t pitch_ = 0) {
+        in[n] = src; out[n] = dst; R_in[n] = r_in; C_in[n] = c_in; R_out[n] = r_out; C_out[n] = c_out;
+        pitch[n] = pitch_ ? pitch_ : c_out;
+        n_src[n] = n_src_; n_out[n] = n_out_; transpose[n] = tr ? 1 : 0;
+        ++n;
+        return dst;
+    }
+};
+int launch_panel_prep(const PanelJobs& jobs, hipStream_t stream);
 int launch_factor_prep(const void* in, int in_dtype, int64_t R_in, int64_t C_in, bool transpose,
                        bf16_t* out, int64_t R_out, int64_t C_out, int64_t num_experts, hipStream_t stream);
 
@@ -42,7 +65,8 @@ int64_t tn_partial_bytes(int64_t n_rows, int64_t width, int r_pad);
 int launch_tn(const bf16_t* P, int64_t ldp, int64_t width, const bf16_t* Q, int r_pad, int r_out,
               int64_t n_rows, bool transpose_out, float* out, float* partial,
               const int32_t* offsets, int32_t num_experts, hipStream_t stream,
-              const int32_t* row_limit = nullptr);   // dense form: contract only rows below *row_limit (device value)
+              const int32_t* row_limit = nullptr,    // dense form: contract only rows below *row_limit (device value)
+              int64_t ldq = 0);                      // row pitch of Q in elements (0: r_pad), for a column band of a wider matrix
 
 int launch_zero_fill(void* p, int64_t bytes, hipStream_t stream);
 
@@ -54,7 +78,13 @@ struct TwoBanks {
     const bf16_t* su2;
     const bf16_t* lora_right2;
 };
+int64_t tile_gemm_partial_bytes(int64_t n_rows, int64_t Nout, int64_t Kc);   // split-K scratch a dense launch may want
 bool two_banks_supported(const xq_weight* w);
+bool two_dense_supported(const xq_weight* w);   // dense [N, K] pair: one dgrad launch, dX = [dY1 | dY2] . [W1 ; W2]
+int launch_gate_up_swiglu(const xq_weight* wg, const xq_weight* wu, const bf16_t* x, int64_t ldx, int64_t M,
+                          const bf16_t* su_g, const bf16_t* su_u, int64_t ld_su, const bf16_t* lr_g, const bf16_t* lr_u,
+                          int r_pad, const bf16_t* bias_g, const bf16_t* bias_u, bf16_t* gu, int64_t ldgu, bf16_t* h,
+                          int64_t ldh, hipStream_t stream);
 int launch_tile_gemm(const xq_weight* w, bool contract_cols, const bf16_t* A, int64_t lda, int64_t n_rows,
                      const int32_t* offsets, const int32_t* tile_offsets, const bf16_t* su, const bf16_t* lora_right,
                      int r_pad, const bf16_t* bias, bf16_t* C, int64_t ldc, hipStream_t stream, const char* who,

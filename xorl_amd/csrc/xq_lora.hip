@@ -77,6 +77,38 @@ int launch_factor_prep_multi(const FactorPrepJobs& j, hipStream_t stream) {
     return XQ_OK;
 }
 
+__global__ void __launch_bounds__(256) panel_prep_kernel(PanelJobs j) {
+    const int k = blockIdx.y;
+    const int64_t per = j.R_out[k] * j.C_out[k], total = per * j.n_out[k];
+    const int64_t R_in = j.R_in[k], C_in = j.C_in[k], C_out = j.C_out[k], R_out = j.R_out[k], pitch = j.pitch[k];
+    const bool tr = j.transpose[k] != 0, shared = j.n_src[k] == 1;
+    for (int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x; t < total; t += (int64_t)gridDim.x * 256) {
+        const int64_t e = t / per, rem = t - e * per;
+        const int64_t i = rem / C_out, c = rem - i * C_out;
+        const int64_t si = tr ? c : i, sj = tr ? i : c;
+        float v = 0.0f;
+        if (si < R_in && sj < C_in) {
+            const int64_t idx = (shared ? 0 : e) * R_in * C_in + si * C_in + sj;
+            v = j.in_f32 ? ((const float*)j.in[k])[idx] : bf16_to_f32(((const bf16_t*)j.in[k])[idx]);
+        }
+        j.out[k][(e * R_out + i) * pitch + c] = to_bf16(v);
+    }
+}
+
+int launch_panel_prep(const PanelJobs& j, hipStream_t stream) {
+    int64_t most = 0;
+    for (int k = 0; k < j.n; ++k) {
+        const int64_t t = j.R_out[k] * j.C_out[k] * j.n_out[k];
+        most = t > most ? t : most;
+    }
+    if (j.n == 0 || most == 0) return XQ_OK;
+    int64_t blocks = xq_cdiv(most, 256);
+    if (blocks > 4096) blocks = 4096;
+    panel_prep_kernel<<<dim3((unsigned)blocks, (unsigned)j.n), 256, 0, stream>>>(j);
+    XQ_CHECK_LAUNCH("panel_prep");
+    return XQ_OK;
+}
+
 // ------------------------------------------------------------------ small_nt
 struct SmallNtArgs {
     const bf16_t* In;
@@ -304,6 +336,7 @@ struct TnArgs {
     float* out;              // dense: partial [S][width][r_pad]; grouped: out [E][...]
     const int32_t* offsets;  // grouped
     const int32_t* row_limit;  // dense, optional (device): only rows below *row_limit are contracted
+    int64_t ldq;               // row pitch of Q in elements
 };
 
 constexpr int TN_PP = 128 + 16;  // Ps pitch (bf16 elements): 288 B rows
@@ -333,7 +366,7 @@ __device__ __forceinline__ void tn_accumulate(const TnArgs& g, int64_t c0, int64
         const int64_t rq = m + qr < m_end ? m + qr : last;
         t.p0 = *(const u32x4*)(g.P + r0 * g.ldp + pcol);
         t.p1 = *(const u32x4*)(g.P + r1 * g.ldp + pcol);
-        t.q = *(const u32x4*)(g.Q + rq * g.r_pad + qc);
+        t.q = *(const u32x4*)(g.Q + rq * g.ldq + qc);
     };
     auto tile = [&](Tile& t, int64_t m, int buf) {     // multiply tile m out of LDS buffer `buf`, refill t with tile m + 64
         bf16_t* ps = Ps + buf * (32 * TN_PP);
@@ -505,11 +538,13 @@ int64_t tn_partial_bytes(int64_t n_rows, int64_t width, int r_pad) {
 
 int launch_tn(const bf16_t* P, int64_t ldp, int64_t width, const bf16_t* Q, int r_pad, int r_out, int64_t n_rows,
               bool transpose_out, float* out, float* partial, const int32_t* offsets, int32_t num_experts,
-              hipStream_t stream, const int32_t* row_limit) {
+              hipStream_t stream, const int32_t* row_limit, int64_t ldq) {
+    if (ldq <= 0) ldq = r_pad;
+    XQ_REQUIRE(ldq >= r_pad && ldq % 8 == 0, "tn: Q pitch %lld must be a multiple of 8 and at least r_pad", (long long)ldq);
     XQ_REQUIRE(r_pad > 0 && r_pad <= 64 && r_pad % 16 == 0 && r_out <= r_pad, "tn: bad rank (r_pad %d, r_out %d)", r_pad, r_out);
     XQ_REQUIRE(width % 8 == 0 && ldp % 8 == 0 && xq_aligned(P, 16) && xq_aligned(Q, 16), "tn: operands must be 16-byte aligned, width %% 8 == 0");
     if (width == 0 || r_out == 0) return XQ_OK;
-    TnArgs g{P, ldp, width, Q, r_pad, r_out, n_rows, 0, transpose_out ? 1 : 0, out, offsets, offsets ? nullptr : row_limit};
+    TnArgs g{P, ldp, width, Q, r_pad, r_out, n_rows, 0, transpose_out ? 1 : 0, out, offsets, offsets ? nullptr : row_limit, ldq};
     unsigned col_tiles = (unsigned)xq_cdiv(width, 128);
     XQ_REQUIRE(partial != nullptr, "tn: partial workspace is NULL");
     if (offsets) {

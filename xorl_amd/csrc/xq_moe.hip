@@ -9,9 +9,6 @@
 
 namespace {
 
-__device__ __forceinline__ float sigmoid_f32(float x) { return 1.0f / (1.0f + __expf(-x)); }
-__device__ __forceinline__ float round_bf16(float x) { return bf16_to_f32(to_bf16(x)); }
-
 // h = bf16(bf16(bf16(silu(g)) * u) * w_row)
 __global__ void __launch_bounds__(256) silu_mul_fwd_kernel(const bf16_t* gate, const bf16_t* up, int64_t ld_in,
                                                            const float* row_w, bf16_t* h, int64_t ld_h, int64_t rows,

@@ -264,6 +264,206 @@ def qlora_linear(x: Tensor, qw: QuantWeight, lora_A: Optional[Tensor], lora_B: O
 
 
 # ---------------------------------------------------------------------------
+# dense SwiGLU MLP of three QLoRA linears (xq_mlp_fwd / xq_mlp_bwd)
+# ---------------------------------------------------------------------------
+_MLP_WS: dict = {}
+
+
+def _mlp_lora_struct(factors, biases, r: int, scaling: float) -> _C.XqMlpLora:
+    L = _C.XqMlpLora()
+    for p in range(3):
+        A, B = factors[2 * p], factors[2 * p + 1]
+        L.A[p], L.B[p] = _C.ptr(A), _C.ptr(B)
+        L.bias[p] = _C.ptr(biases[p])
+    L.dtype = _lora_dt(factors[0])
+    L.r, L.scaling = r, scaling
+    return L
+
+
+def _mlp_saved_struct(saved) -> _C.XqMlpSaved:
+    S = _C.XqMlpSaved()
+    S.gate_up, S.h, S.su_gate_up, S.su_down = (t.data_ptr() for t in saved)
+    return S
+
+
+def _mlp_workspace(dev, M: int, H: int, I: int, r: int, backward: bool) -> Tensor:
+    key = (M, H, I, r, backward)
+    n = _MLP_WS.get(key)
+    if n is None:
+        n = _MLP_WS[key] = _C.lib().xq_mlp_workspace_bytes(M, H, I, r, int(backward))
+    return torch.empty(n, dtype=torch.uint8, device=dev)
+
+
+def _mlp_fwd_impl(x2: Tensor, factors, biases, banks, r: int, scaling: float):
+    """xq_mlp_fwd.  x2 bf16 [M, H]; factors (gA, gB, uA, uB, dA, dB) active views, contiguous (None at r == 0);
+    biases three bf16 vectors or None; banks (gate, up, down) QuantWeight.  -> (y [M, H], four saved tensors)."""
+    qg, qu, qd = banks
+    I, H = qg.rows, qg.cols
+    M, dev, rp = x2.shape[0], x2.device, max(_r_pad(r), 16)
+    bf = lambda *shape: torch.empty(*shape, dtype=torch.bfloat16, device=dev)
+    saved = (bf(M, 2 * I), bf(M, I), bf(M, 2 * rp), bf(M, rp))
+    y = bf(M, H)
+    ws = _mlp_workspace(dev, M, H, I, r, False)
+    lora, S = _mlp_lora_struct(factors, biases, r, scaling), _mlp_saved_struct(saved)
+    wg, wu, wd = qg.c(), qu.c(), qd.c()
+    _C.check(_C.lib().xq_mlp_fwd(ctypes.byref(wg), ctypes.byref(wu), ctypes.byref(wd), ctypes.byref(lora), x2.data_ptr(),
+                                 _ld(x2), M, y.data_ptr(), H, ctypes.byref(S), ws.data_ptr(), ws.numel(),
+                                 _C.stream_ptr(dev)))
+    return y, saved
+
+
+def _mlp_bwd_impl(dy2: Tensor, x2: Tensor, saved, factors, banks, r: int, scaling: float, need_dx: bool):
+    """xq_mlp_bwd -> (dx [M, H] or empty, six fp32 factor gradients (empty at r == 0))."""
+    qg, qu, qd = banks
+    I, H = qg.rows, qg.cols
+    M, dev = x2.shape[0], x2.device
+    dx = torch.empty(M, H, dtype=torch.bfloat16, device=dev) if need_dx else torch.empty(0, dtype=torch.bfloat16, device=dev)
+    grads = [torch.empty(f.shape if f is not None else (0,), dtype=torch.float32, device=dev) for f in factors]
+    G = _C.XqMlpGrads()
+    for p in range(3):
+        G.dA[p], G.dB[p] = (grads[2 * p].data_ptr(), grads[2 * p + 1].data_ptr()) if r else (None, None)
+    ws = _mlp_workspace(dev, M, H, I, r, True)
+    lora, S = _mlp_lora_struct(factors, (None, None, None), r, scaling), _mlp_saved_struct(saved)
+    wg, wu, wd = qg.c(), qu.c(), qd.c()
+    _C.check(_C.lib().xq_mlp_bwd(ctypes.byref(wg), ctypes.byref(wu), ctypes.byref(wd), ctypes.byref(lora), x2.data_ptr(),
+                                 _ld(x2), dy2.data_ptr(), _ld(dy2), M, ctypes.byref(S), dx.data_ptr() if need_dx else None,
+                                 H, ctypes.byref(G), ws.data_ptr(), ws.numel(), _C.stream_ptr(dev)))
+    return dx, grads
+
+
+def _qw_args(qw: QuantWeight):
+    return qw.packed, qw.scales, qw.global_scale, qw.fmt, _DT_TO_CODE[qw.scale_dtype], qw.group
+
+
+def _qw_from(packed, scales, gs, fmt, scale_code, group, rows, cols) -> QuantWeight:
+    return QuantWeight(fmt, _C.XQ_LAYOUT_FLAT, packed, scales, _CODE_TO_DT[scale_code], rows, cols, group, global_scale=gs)
+
+
+@torch.library.custom_op("xq::mlp_fwd", mutates_args=(), device_types="cuda")
+def _mlp_fwd_op(x: Tensor, factors: List[Tensor], biases: List[Optional[Tensor]],
+                g_packed: Tensor, g_scales: Tensor, g_gs: Optional[Tensor], g_fmt: str, g_code: int, g_group: int,
+                u_packed: Tensor, u_scales: Tensor, u_gs: Optional[Tensor], u_fmt: str, u_code: int, u_group: int,
+                d_packed: Tensor, d_scales: Tensor, d_gs: Optional[Tensor], d_fmt: str, d_code: int, d_group: int,
+                H: int, I: int, r: int, scaling: float) -> List[Tensor]:
+    banks = (_qw_from(g_packed, g_scales, g_gs, g_fmt, g_code, g_group, I, H),
+             _qw_from(u_packed, u_scales, u_gs, u_fmt, u_code, u_group, I, H),
+             _qw_from(d_packed, d_scales, d_gs, d_fmt, d_code, d_group, H, I))
+    y, saved = _mlp_fwd_impl(x, tuple(factors) if r else (None,) * 6, tuple(biases), banks, r, scaling)
+    return [y, *saved]
+
+
+@_mlp_fwd_op.register_fake
+def _(x, factors, biases, g_packed, g_scales, g_gs, g_fmt, g_code, g_group, u_packed, u_scales, u_gs, u_fmt, u_code, u_group,
+      d_packed, d_scales, d_gs, d_fmt, d_code, d_group, H, I, r, scaling):
+    M, rp = x.shape[0], max(_r_pad(r), 16)
+    return [x.new_empty(M, H), x.new_empty(M, 2 * I), x.new_empty(M, I), x.new_empty(M, 2 * rp), x.new_empty(M, rp)]
+
+
+@torch.library.custom_op("xq::mlp_bwd", mutates_args=(), device_types="cuda")
+def _mlp_bwd_op(dy: Tensor, x: Tensor, saved: List[Tensor], factors: List[Tensor],
+                g_packed: Tensor, g_scales: Tensor, g_gs: Optional[Tensor], g_fmt: str, g_code: int, g_group: int,
+                u_packed: Tensor, u_scales: Tensor, u_gs: Optional[Tensor], u_fmt: str, u_code: int, u_group: int,
+                d_packed: Tensor, d_scales: Tensor, d_gs: Optional[Tensor], d_fmt: str, d_code: int, d_group: int,
+                H: int, I: int, r: int, scaling: float, need_dx: bool) -> List[Tensor]:
+    banks = (_qw_from(g_packed, g_scales, g_gs, g_fmt, g_code, g_group, I, H),
+             _qw_from(u_packed, u_scales, u_gs, u_fmt, u_code, u_group, I, H),
+             _qw_from(d_packed, d_scales, d_gs, d_fmt, d_code, d_group, H, I))
+    dx, grads = _mlp_bwd_impl(dy, x, tuple(saved), tuple(factors) if r else (None,) * 6, banks, r, scaling, need_dx)
+    return [dx, *grads]
+
+
+@_mlp_bwd_op.register_fake
+def _(dy, x, saved, factors, g_packed, g_scales, g_gs, g_fmt, g_code, g_group, u_packed, u_scales, u_gs, u_fmt, u_code,
+      u_group, d_packed, d_scales, d_gs, d_fmt, d_code, d_group, H, I, r, scaling, need_dx):
+    out = [x.new_empty(x.shape if need_dx else (0,))]
+    if r:
+        out += [x.new_empty(f.shape, dtype=torch.float32) for f in factors]
+    else:
+        out += [x.new_empty(0, dtype=torch.float32) for _ in range(6)]
+    return out
+
+
+class QLoRAMLPFunction(torch.autograd.Function):
+    """y = down(silu(gate(x)) * up(x)) over three QLoRA linears with packed weights (xq_mlp_fwd / xq_mlp_bwd).
+    Gradients: x and the six factors (full parameter shapes: ranks beyond the active one get zeros)."""
+
+    @staticmethod
+    def forward(ctx, x, gA, gB, uA, uB, dA, dB, bias_g, bias_u, bias_d, qg: QuantWeight, qu: QuantWeight, qd: QuantWeight,
+                r: int, scaling: float):
+        _C.require_hip(x)
+        if x.dtype != torch.bfloat16:
+            raise _C.XqError(f"activations must be bf16, got {x.dtype}")
+        I, H = qg.rows, qg.cols
+        x2 = _as_2d(x)
+        if x2.shape[1] != H:
+            raise _C.XqError(f"input width {x2.shape[1]} != in_features {H}")
+        params = (gA, gB, uA, uB, dA, dB)
+        if r:
+            factors = tuple((p[:r] if i % 2 == 0 else p[:, :r]).contiguous() for i, p in enumerate(params))
+        else:
+            factors = (None,) * 6
+        biases = tuple(None if b is None else b.to(torch.bfloat16).contiguous() for b in (bias_g, bias_u, bias_d))
+        s = float(scaling)
+        if torch.compiler.is_compiling():
+            res = _mlp_fwd_op(x2, list(factors) if r else [], list(biases), *_qw_args(qg), *_qw_args(qu), *_qw_args(qd), H, I, r, s)
+            y, saved = res[0], tuple(res[1:])
+        else:
+            y, saved = _mlp_fwd_impl(x2, factors, biases, (qg, qu, qd), r, s)
+        ctx.banks, ctx.r, ctx.s, ctx.shape = (qg, qu, qd), r, s, x.shape
+        ctx.param_shapes = tuple(None if p is None else p.shape for p in params)
+        ctx.param_dtypes = tuple(None if p is None else p.dtype for p in params)
+        ctx.n_factors = 6 if r else 0
+        ctx.save_for_backward(x2, *saved, *(factors if r else ()))
+        return y.reshape(*x.shape[:-1], H)
+
+    @staticmethod
+    def backward(ctx, dy):
+        x2, saved = ctx.saved_tensors[0], ctx.saved_tensors[1:5]
+        factors = tuple(ctx.saved_tensors[5:]) if ctx.n_factors else (None,) * 6
+        qg, qu, qd = ctx.banks
+        I, H, r = qg.rows, qg.cols, ctx.r
+        dy2 = _as_2d(dy.to(torch.bfloat16))
+        need_dx = ctx.needs_input_grad[0]
+        if torch.compiler.is_compiling():
+            res = _mlp_bwd_op(dy2, x2, list(saved), list(factors) if r else [], *_qw_args(qg), *_qw_args(qu), *_qw_args(qd),
+                              H, I, r, ctx.s, need_dx)
+            dx, grads = res[0], res[1:]
+        else:
+            dx, grads = _mlp_bwd_impl(dy2, x2, saved, factors, ctx.banks, r, ctx.s, need_dx)
+        out = []
+        for i, (g, shape, dt) in enumerate(zip(grads, ctx.param_shapes, ctx.param_dtypes)):
+            if shape is None or not r or not ctx.needs_input_grad[1 + i]:
+                out.append(None)
+                continue
+            if tuple(g.shape) != tuple(shape):        # ranks beyond the active one: zero gradient
+                full = g.new_zeros(shape)
+                if i % 2 == 0:
+                    full[:r] = g
+                else:
+                    full[:, :r] = g
+                g = full
+            out.append(g.to(dt))
+        gb = [None, None, None]
+        if ctx.needs_input_grad[9]:        # the down projection's bias sees dy itself
+            gb[2] = dy2.float().sum(0).to(dy.dtype)
+        if ctx.needs_input_grad[7] or ctx.needs_input_grad[8]:
+            raise NotImplementedError("trainable gate / up biases are not part of the fused MLP path (frozen in QLoRA)")
+        return (dx.reshape(ctx.shape) if need_dx else None, *out, *gb, None, None, None, None, None)
+
+
+def qlora_mlp(x: Tensor, qw_gate: QuantWeight, qw_up: QuantWeight, qw_down: QuantWeight, gate_A: Optional[Tensor],
+              gate_B: Optional[Tensor], up_A: Optional[Tensor], up_B: Optional[Tensor], down_A: Optional[Tensor],
+              down_B: Optional[Tensor], r: int, scaling: float, bias_gate: Optional[Tensor] = None,
+              bias_up: Optional[Tensor] = None, bias_down: Optional[Tensor] = None) -> Tensor:
+    """down(silu(gate(x)) * up(x)) of three QLoRA linears that share LoRA rank and scaling, in two library calls
+    (forward, backward) instead of seven.  Same rounding points as the separate modules."""
+    if r > MAX_FUSED_RANK:
+        raise _C.XqError(f"the fused MLP takes LoRA ranks up to {MAX_FUSED_RANK}, got {r}")
+    return QLoRAMLPFunction.apply(x, gate_A, gate_B, up_A, up_B, down_A, down_B, bias_gate, bias_up, bias_down, qw_gate,
+                                  qw_up, qw_down, r, scaling)
+
+
+# ---------------------------------------------------------------------------
 # SwiGLU
 # ---------------------------------------------------------------------------
 def _silu_fwd_impl(g2: Tensor, u2: Tensor) -> Tensor:

@@ -8,6 +8,7 @@ from .linear import (
     NvFP4QLoRALinear,
     QLoRALinear,
     deregister_qlora_weights_from_fsdp,
+    qlora_mlp_forward,
 )
 
 __all__ = [
@@ -18,6 +19,7 @@ __all__ = [
     "Int4QLoRALinear",
     "NF4QLoRALinear",
     "deregister_qlora_weights_from_fsdp",
+    "qlora_mlp_forward",
 ]
 
 from .moe_experts import BlockFP8QLoRAMoeExperts, NF4QLoRAMoeExperts, NvFP4QLoRAMoeExperts, QLoRAMoeExperts  # noqa: E402

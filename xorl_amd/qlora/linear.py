@@ -770,6 +770,31 @@ class NF4QLoRALinear(QLoRALinear):
 
 
 # =============================================================================
+def qlora_mlp_forward(gate_proj: "QLoRALinear", up_proj: "QLoRALinear", down_proj: "QLoRALinear", x: Tensor) -> Tensor:
+    """`down_proj(silu(gate_proj(x)) * up_proj(x))` -- the body of the reference's Qwen3MLP.forward
+    (models/transformers/qwen3/modeling_qwen3.py:60-81) on three QLoRA linears -- as one fused forward and one fused
+    backward of the library when the three modules allow it: same active LoRA rank (<= 64) and scaling, plain
+    (unsharded) state, no quantization noise.  Otherwise the three modules and the SwiGLU kernel are called one by
+    one; both ways give the same rounding points."""
+    from ..functional import qlora_mlp, silu_and_mul
+
+    mods = (gate_proj, up_proj, down_proj)
+    r, s = gate_proj.active_r, gate_proj._active_scaling()
+    fusable = (all(isinstance(m, QLoRALinear) for m in mods)
+               and all(m.active_r == r and m._active_scaling() == s for m in mods) and r <= MAX_FUSED_RANK
+               and not any(m.enable_aqn and m.training for m in mods)
+               and not any(_is_dtensor(m.packed_weight_f32.data) or _is_dtensor(m.lora_A) for m in mods)
+               and gate_proj.out_features == up_proj.out_features == down_proj.in_features
+               and gate_proj.in_features == up_proj.in_features == down_proj.out_features
+               and gate_proj.in_features % 64 == 0 and gate_proj.out_features % 64 == 0
+               and x.dtype == torch.bfloat16 and x.is_cuda)
+    if not fusable:
+        return down_proj(silu_and_mul(gate_proj(x), up_proj(x)))
+    return qlora_mlp(x, gate_proj._forward_quant_weight(), up_proj._forward_quant_weight(), down_proj._forward_quant_weight(),
+                     gate_proj.lora_A, gate_proj.lora_B, up_proj.lora_A, up_proj.lora_B, down_proj.lora_A, down_proj.lora_B,
+                     r, s, gate_proj.bias, up_proj.bias, down_proj.bias)
+
+
 def deregister_qlora_weights_from_fsdp(model: nn.Module, param_names: tuple = ("weight",)) -> int:
     """Drop QLoRALinear parameters from FSDP2 parameter groups so no mixed
     precision cast ever touches the packed bytes; they stay sharded DTensors
