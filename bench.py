@@ -44,13 +44,15 @@ MEASURED_TRAFFIC = {
     # gemm_256_kernel<int4, T=128> in 4 K splits + splitk_reduce_kernel: mean of the forward and dgrad launches
     # (64 MiB of it are the fp32 partial sums written and read back)
     0: (109.6 * 2 ** 20, "profiles/gemm_128_int4_linear_m512.txt", 0.04478),
-    # gemm_256_kernel<fp8>: mean of the forward and dgrad launches
-    1: (905.4 * 2 ** 20, "profiles/gemm_256_fp8_mlp_m8192.txt", 0.73747),
+    # gemm_256_kernel<fp8>: mean over the 4 launches of a step (gate|up forward with the SwiGLU epilogue, down
+    # forward, d_h, dx as one sum over the gate and up weights)
+    1: (1457.8 * 2 ** 20, "profiles/gemm_256_fp8_mlp_m8192.txt", 1.13390),
     # gemm_256_kernel<nvfp4>, 256x256 tiles (whole rounds; trailing rows in K splits) and 128x128 tiles
     # (+ splitk_reduce_kernel): mean over the 12 launches of a step, fp32 partial sums included
     2: (187.2 * 2 ** 20, "profiles/gemm_256_nvfp4_attn_m4096.txt", 0.14518),
-    # gemm_256_kernel<fp8, grouped>: mean over the 6 launches of a step
-    3: (1032.2 * 2 ** 20, "profiles/gemm_256_fp8_grouped_moe_e128.txt", 0.57350),
+    # gemm_256_kernel<fp8, grouped>: mean over the 4 launches of a step (gate|up forward over two banks, down
+    # forward, d_h, dx as one sum over both banks)
+    3: (1351.6 * 2 ** 20, "profiles/gemm_256_fp8_grouped_moe_e128.txt", 0.83854),
     # skinny_split_kernel + skinny_epilogue_kernel: mean per forward over the 32 cases (includes the fp32 partial
     # tiles written and read back: 23.3 MiB of it are algorithmic)
     4: (41.0 * 2 ** 20, "profiles/skinny_split_kernel_decode_shapes.txt", 0.02006),
