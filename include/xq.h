@@ -97,6 +97,13 @@ int xq_profile_collect(int* n_launches, double* total_ms, double* total_flops);
  *      allows it, whatever the size. */
 int xq_set_tile_policy(int policy);
 
+/* The 256x256 tile kernel (unsplit launches) is a persistent program: one block per compute unit walks the
+ * tiles b, b + grid, ... and requests its next tile's first operands before it stores the finished tile.
+ * enabled = 0 launches one block per tile instead -- the same kernel and, bit for bit, the same results; a
+ * process-wide switch for tests and A/B measurements (XQ_PERSIST=0 in the environment sets it at load time);
+ * no counterpart in the reference. */
+int xq_set_persistent_tiles(int enabled);
+
 /* ---- decode ------------------------------------------------------------
  * out[e] = decoded weight of expert e, shape [rows, cols], bf16 or fp32.
  * Replaces int4_dequantize / int4_dequantize_gkn

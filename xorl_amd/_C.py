@@ -107,6 +107,7 @@ _SIGNATURES = {
     # gate, up, ld_in, dh, ld_dh, row_w, dgate, dup, ld_out, d_row_w, rows, cols, stream
     "xq_silu_mul_bwd": (_INT, [_P, _P, _I64, _P, _I64, _P, _P, _P, _I64, _P, _I64, _I64, _P]),
     "xq_set_tile_policy": (_INT, [_INT]),
+    "xq_set_persistent_tiles": (_INT, [_INT]),
     "xq_route_workspace_bytes": (_I64, [_I64, _I32]),
     # selected, n_routed, E, counts, offsets, scatter_index, tile_offsets, ws, ws_bytes, stream
     "xq_route_build": (_INT, [_P, _I64, _I32, _P, _P, _P, _P, _P, _I64, _P]),

@@ -63,7 +63,9 @@ __device__ __forceinline__ float bf16_to_f32(bf16_t h) { return __uint_as_float(
 
 // SwiGLU arithmetic shared by the elementwise kernels and the fused GEMM epilogues (ops/fused_silu_and_mul.py:22-60):
 // sigmoid in fp32, the activation rounded to bf16 before it meets `up`
-__device__ __forceinline__ float sigmoid_f32(float x) { return 1.0f / (1.0f + __expf(-x)); }
+// 1 / (1 + e^-x) with the hardware reciprocal (1 ulp) in place of an IEEE division sequence: the quotient feeds a
+// product that is rounded to bf16, and the SwiGLU epilogue of the gate / up launch pays for every instruction here
+__device__ __forceinline__ float sigmoid_f32(float x) { return __builtin_amdgcn_rcpf(1.0f + __expf(-x)); }
 __device__ __forceinline__ float round_bf16(float x) { return bf16_to_f32(to_bf16(x)); }
 
 // e4m3fn (OCP) byte pair -> two fp32: v_cvt_pk_f32_fp8.  hi selects the upper

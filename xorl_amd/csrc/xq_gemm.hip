@@ -1,5 +1,6 @@
 // Host entry points of the fused dequant-GEMM + LoRA path (dense and grouped).
 #include "xq_gemm_tile.h"
+#include <algorithm>
 #include <atomic>
 #include "xq_gemm_256.h"
 #include <stdlib.h>
@@ -66,6 +67,17 @@ static int num_cus() {
         n = 256;
     cached.store(n, std::memory_order_relaxed);
     return n;
+}
+
+// Grid of the persistent program (large unsplit tiles): one block per compute unit, a multiple of 8 so that every
+// tile of a block falls into the same XCD's range of the tile order; more blocks when a block would otherwise walk
+// more tiles than it keeps a table for.  XQ_PERSIST=0 launches one block per tile (same kernel, same results).
+static int g_persist = [] { const char* e = getenv("XQ_PERSIST"); return e ? atoi(e) : 1; }();
+static inline unsigned persistent_grid(int64_t tiles) {
+    if (!g_persist) return (unsigned)tiles;
+    int64_t blocks = std::max<int64_t>((num_cus() / 8) * 8, 8);
+    blocks = std::max(blocks, (xq_cdiv(tiles, G256_MAX_ROUNDS) + 7) / 8 * 8);
+    return (unsigned)std::min(tiles, blocks);
 }
 
 // Tile size of a dense launch under the default policy: large tiles from the point where they fill more than
@@ -246,12 +258,15 @@ static int launch_tile_gemm_t(const xq_weight* w, bool contract_cols, const bf16
             f.ksplit = ksplit; f.partial = ksplit > 1 ? partial : nullptr;
             f.W2 = nullptr; f.scales2 = nullptr; f.su2 = nullptr; f.lora_right2 = nullptr; f.ncols1 = 0; f.nk1 = 0;
             f.ld_su = g.r_pad; f.H = nullptr; f.ldh = 0; f.bias2 = nullptr;
+            f.wide_rows = xq_aligned(C, 16) && ldc % 8 == 0 && xq_aligned(bias, 8);
             if (two) {
                 f.W2 = (const uint8_t*)two->w2->packed; f.scales2 = (const uint8_t*)two->w2->scales;
                 f.su2 = g.r_pad ? two->su2 : nullptr; f.lora_right2 = g.r_pad ? two->lora_right2 : nullptr;
                 f.ncols1 = g.wcols; f.nk1 = (two_dense ? g.wrows : g.wcols) / BK;
             }
-            dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)ksplit);
+            // (the kernel's own rule: large unsplit tiles, except the 4-bit expert banks)
+            const bool persistent = T == 256 && ksplit == 1 && !(grouped && w->format != XQ_FMT_FP8);
+            dim3 grid(persistent ? persistent_grid(tiles_m * tiles_n) : (unsigned)(tiles_m * tiles_n), (unsigned)ksplit);
             const bool timed = xq_profile_mark_begin(stream, 2.0 * (double)n_rows * g.Nout * ((double)g.Kc + g.r_pad));
             int rc;
             if (w->format == XQ_FMT_FP8) rc = launch_256<XQ_FMT_FP8>(f, contract_cols, grouped, T, grid, stream, who);
@@ -297,7 +312,8 @@ int launch_gate_up_swiglu(const xq_weight* wg, const xq_weight* wu, const bf16_t
     XQ_REQUIRE(K % BK == 0 && I % 16 == 0, "%s: in_features %% 64 == 0 and out_features %% 16 == 0", who);
     XQ_REQUIRE(ldx % 8 == 0 && xq_aligned(x, 16) && xq_aligned(wg->packed, 16) && xq_aligned(wu->packed, 16),
                "%s: operands must be 16-byte aligned", who);
-    XQ_REQUIRE(ldgu % 4 == 0 && ldh % 4 == 0 && xq_aligned(gu, 8) && xq_aligned(h, 8), "%s: output rows must be 8-byte aligned", who);
+    XQ_REQUIRE(ldgu % 8 == 0 && ldh % 8 == 0 && xq_aligned(gu, 16) && xq_aligned(h, 16), "%s: output rows must be 16-byte aligned", who);
+    XQ_REQUIRE(xq_aligned(bias_g, 8) && xq_aligned(bias_u, 8), "%s: bias vectors must be 8-byte aligned", who);
     const bool side = su_g && su_u && lr_g && lr_u && r_pad > 0;
     XQ_REQUIRE(!side || (r_pad % 16 == 0 && r_pad <= 64 && ld_su >= r_pad && ld_su % 8 == 0 && xq_aligned(su_g, 16) &&
                          xq_aligned(su_u, 16) && xq_aligned(lr_g, 16) && xq_aligned(lr_u, 16)),
@@ -316,6 +332,7 @@ int launch_gate_up_swiglu(const xq_weight* wg, const xq_weight* wu, const bf16_t
     f.tiles_m = (int32_t)xq_cdiv(M, 256); f.tiles_n = (int32_t)xq_cdiv(I, 128);
     f.ksplit = 1;
     f.H = h; f.ldh = ldh;
+    f.wide_rows = 1;
     static std::atomic<bool> attr_set{false};
     if (!attr_set) {
         int rc = raise_lds_limit(gemm_256_kernel<XQ_FMT_FP8, true, false, 256, false, true>, Geo<256>::lds_bytes(true), who);
@@ -325,7 +342,7 @@ int launch_gate_up_swiglu(const xq_weight* wg, const xq_weight* wu, const bf16_t
     // flops of the two projections and their side terms
     const bool timed = xq_profile_mark_begin(stream, 2.0 * (double)M * (2.0 * I) * ((double)K + f.r_pad));
     gemm_256_kernel<XQ_FMT_FP8, true, false, 256, false, true>
-        <<<dim3((unsigned)(f.tiles_m * f.tiles_n)), Geo<256>::NT, Geo<256>::lds_bytes(true), stream>>>(f);
+        <<<dim3(persistent_grid((int64_t)f.tiles_m * f.tiles_n)), Geo<256>::NT, Geo<256>::lds_bytes(true), stream>>>(f);
     XQ_CHECK_LAUNCH(who);
     if (timed) xq_profile_mark_end(stream);
     return XQ_OK;
@@ -359,6 +376,11 @@ using namespace xq;
 extern "C" int xq_set_tile_policy(int policy) {
     XQ_REQUIRE(policy >= 0 && policy <= 3, "xq_set_tile_policy: policy %d not in {0, 1, 2, 3}", policy);
     g_tile_policy = policy;
+    return XQ_OK;
+}
+
+extern "C" int xq_set_persistent_tiles(int enabled) {
+    g_persist = enabled != 0;
     return XQ_OK;
 }
 

@@ -35,6 +35,7 @@
 namespace xq {
 
 constexpr int F8_BK = 64;
+constexpr int G256_MAX_ROUNDS = 64;   // tiles one block of the persistent program may walk (the launcher sizes the grid for it)
 #ifndef XQ_SMALL_TILE_DEPTH
 #define XQ_SMALL_TILE_DEPTH 2
 #endif
@@ -102,6 +103,9 @@ struct G256Args {
     bf16_t* H;
     int64_t ldh;
     const bf16_t* bias2;
+    // C rows start 16-byte aligned: the finished tile then leaves through LDS as whole 128-byte row pieces (the gate / up
+    // launch requires it of C and H)
+    int32_t wide_rows;
 };
 
 // ---------------------------------------------------------------- weight-tile loaders
@@ -422,17 +426,24 @@ __global__ void __launch_bounds__(2 * T, 2) gemm_256_kernel(G256Args g) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / G::WN, wn = wave % G::WN;   // wave tile: rows wm*(T/2).., cols wn*64..
 
+    // The large unsplit tile is a persistent program: block b works on the tiles b, b + gridDim.x, ... and fetches
+    // the first K-step of its next tile before it multiplies the low-rank term and stores the current one, so that a
+    // tile's drain and the next tile's first memory round trip overlap.  (A grid that covers every tile runs each
+    // block once: the same program.)
+    constexpr bool CAN_SPLIT = !GROUPED && (T == 128 || SPLIT256);
+    constexpr bool PERSIST = T == 256 && !SPLIT256 && !(GROUPED && FMT != XQ_FMT_FP8);   // the GKN 4-bit loader has no registers to spare
+    constexpr int MAX_ROUNDS = G256_MAX_ROUNDS;
+
     // ---- XCD-aware tile mapping: consecutive workgroup ids land on different XCDs, so
     // give each XCD a contiguous range of logical tiles.  Dense: walk the logical tiles
     // in groups of 4 row-tiles so concurrent tiles share operands in L2.  Grouped: walk
     // row-tile by row-tile (all column tiles of a row tile, then the next row tile of the
-    // same expert) so an XCD stays on one expert's matrix.
-    int pid_m, pid_n;
-    {
-        const int nb = g.tiles_m * g.tiles_n;
-        int b = blockIdx.x;
+    // same expert) so an XCD stays on one expert's matrix.  (gridDim.x is a multiple of 8 whenever a block
+    // walks more than one tile, so every tile of a block lies in the same XCD's range.)
+    const int nb = g.tiles_m * g.tiles_n;
+    auto tile_of = [&](int b, int& pid_m, int& pid_n) {
         const int per = nb >> 3;
-        int logical = (b < per * 8) ? (b & 7) * per + (b >> 3) : b;
+        const int logical = (b < per * 8) ? (b & 7) * per + (b >> 3) : b;
         if (GROUPED) {
             pid_m = logical / g.tiles_n;
             pid_n = logical - pid_m * g.tiles_n;
@@ -445,55 +456,74 @@ __global__ void __launch_bounds__(2 * T, 2) gemm_256_kernel(G256Args g) {
             pid_m = first_m + in % gsz;
             pid_n = in / gsz;
         }
-    }
-    int e = 0;
-    int64_t row0, row_end;
-    if (GROUPED) {
-        // The expert whose tile range holds this row tile: thread t looks at expert t (and t + NT, ...), all loads
-        // issued together -- one memory round trip for the block instead of the chain of dependent loads a
-        // binary search by one thread makes.  Exactly one expert matches, or none beyond the last tile.
-        int* sh_info = (int*)smem;
-        if (tid == 0) sh_info[0] = -1;
+    };
+    // Grouped: (expert, first row, end row) of every tile this block will work on, found once: thread t looks at
+    // expert t (and t + NT, ...) with all loads issued together -- one memory round trip for the block instead of
+    // the chain of dependent loads a binary search makes, and none per tile.  A row tile belongs to exactly one
+    // expert, or to none beyond the last tile.
+    __shared__ int sh_tab[GROUPED ? 3 * MAX_ROUNDS : 1];
+    if constexpr (GROUPED) {
+        const int first = (int)blockIdx.x, stride = (int)gridDim.x;
+        const int rounds = PERSIST ? min((nb - first + stride - 1) / stride, MAX_ROUNDS) : 1;
+        for (int j = tid; j < rounds; j += NT) sh_tab[3 * j] = -1;
         __syncthreads();
         for (int t = tid; t < g.num_experts; t += NT) {
             const int lo = g.tile_prefix[t], hi = g.tile_prefix[t + 1];
             const int o0 = g.offsets[t], o1 = g.offsets[t + 1];
-            if (lo <= pid_m && pid_m < hi) {
-                sh_info[0] = t;
-                sh_info[1] = o0 + (pid_m - lo) * F8_BM;
-                sh_info[2] = o1;
+            if (lo < hi) {
+                for (int j = 0; j < rounds; ++j) {
+                    int pm, pn;
+                    tile_of(first + j * stride, pm, pn);
+                    if (lo <= pm && pm < hi) {
+                        sh_tab[3 * j] = t;
+                        sh_tab[3 * j + 1] = o0 + (pm - lo) * F8_BM;
+                        sh_tab[3 * j + 2] = o1;
+                    }
+                }
             }
         }
         __syncthreads();
-        e = sh_info[0];
-        const int r0 = sh_info[1], r1 = sh_info[2];
-        __syncthreads();
-        if (e < 0) return;
-        row0 = r0;
-        row_end = r1;
-    } else {
-        row0 = (int64_t)pid_m * F8_BM;
-        row_end = g.M;
     }
-    const int n0 = GU ? pid_n * (F8_BN / 2) : pid_n * F8_BN;      // GU: first gate (= up) column of the tile
     // two banks (grouped block-fp8 only): a forward block past the first bank's columns works on the second bank
     constexpr bool TWO_OK = GROUPED && FMT == XQ_FMT_FP8;
-    const uint8_t* Wb = g.W;
-    const uint8_t* Sb = g.scales;
-    const bf16_t* su_b = g.su;
-    const bf16_t* lr_b = g.lora_right;
-    int n0w = n0;                                   // first column of the tile within its bank
-    int bank_width = g.Nout;                        // output columns one bank provides
-    if constexpr (TWO_OK) {
-        if (g.W2 != nullptr && !CC) {
-            bank_width = g.ncols1;
-            if (n0 >= g.ncols1) { Wb = g.W2; Sb = g.scales2; su_b = g.su2; lr_b = g.lora_right2; n0w = n0 - g.ncols1; }
+    struct TileDesc {
+        int e;                                          // expert (0 for a dense launch)
+        int64_t row0, row_end;                          // first row of the tile, end of the rows it may read and write
+        int n0, n0w, bank_width;                        // first output column; the same within its bank; columns of a bank
+        const uint8_t* Wb;
+        const uint8_t* Sb;
+        const bf16_t* su_b;
+        const bf16_t* lr_b;
+    };
+    auto describe = [&](int b, int round, TileDesc& t) -> bool {      // false: there is no such tile
+        if (b >= nb || round >= MAX_ROUNDS) return false;
+        int pid_m, pid_n;
+        tile_of(b, pid_m, pid_n);
+        t.e = 0;
+        if constexpr (GROUPED) {
+            t.e = __builtin_amdgcn_readfirstlane(sh_tab[3 * round]);
+            if (t.e < 0) return false;
+            t.row0 = __builtin_amdgcn_readfirstlane(sh_tab[3 * round + 1]);
+            t.row_end = __builtin_amdgcn_readfirstlane(sh_tab[3 * round + 2]);
+        } else {
+            t.row0 = (int64_t)pid_m * F8_BM;
+            t.row_end = g.M;
         }
-    }
+        t.n0 = GU ? pid_n * (F8_BN / 2) : pid_n * F8_BN;      // GU: first gate (= up) column of the tile
+        t.Wb = g.W; t.Sb = g.scales; t.su_b = g.su; t.lr_b = g.lora_right;
+        t.n0w = t.n0;
+        t.bank_width = g.Nout;
+        if constexpr (TWO_OK) {
+            if (g.W2 != nullptr && !CC) {
+                t.bank_width = g.ncols1;
+                if (t.n0 >= g.ncols1) { t.Wb = g.W2; t.Sb = g.scales2; t.su_b = g.su2; t.lr_b = g.lora_right2; t.n0w = t.n0 - g.ncols1; }
+            }
+        }
+        return true;
+    };
     // K-steps of this block: all of them, or the split's share (every split has at least one)
     // K splits: the small tile always knows them; the large tile has an instantiation of its own for them
     // (trailing rows of a launch that fill part of a round), so the unsplit one carries nothing extra
-    constexpr bool CAN_SPLIT = !GROUPED && (T == 128 || SPLIT256);
     int kt0 = 0, nk = g.Kc / F8_BK;
     const int split = CAN_SPLIT ? (int)blockIdx.y : 0;
     if (CAN_SPLIT && g.ksplit > 1) {
@@ -502,29 +532,47 @@ __global__ void __launch_bounds__(2 * T, 2) gemm_256_kernel(G256Args g) {
         nk = min(per, nk - kt0);
     }
 
-    // ---- per-thread global addresses (fixed across K-steps except for the k offset)
-    const bf16_t* a_src[4];
-    int a_dst[4];
-#pragma unroll
-    for (int p = 0; p < 4; ++p) {
-        const int u = tid + p * NT;
-        int64_t r = row0 + (u >> 3);
-        r = r < row_end ? r : row_end - 1;
-        a_src[p] = g.A + r * g.lda + (u & 7) * 8 + kt0 * F8_BK;
-        a_dst[p] = swz(u >> 3, u & 7);
-    }
     // PD register sets hold the tiles in flight from global memory: tile j lives in set j % PD.  The large tile has
     // one (two waves per SIMD and an iteration longer than the memory latency cover it); the small tile, whose
     // iteration is a fraction of the latency, keeps PD tiles in flight.
     constexpr int PD = (GROUPED && FMT != XQ_FMT_FP8) ? 1 : Geo<T>::PD;   // the GKN 4-bit loader has no registers to spare
+    static_assert(!PERSIST || PD == 1, "the persistent loop refills one register set");
     using WL = typename W256Sel<FMT, CC, GROUPED, T>::type;
     WL wls[PD];
-#pragma unroll
-    for (int d = 0; d < PD; ++d) {
-        if constexpr (GU) wls[d].init_gu(g, n0, tid);
-        else wls[d].init(g, Wb + (int64_t)e * g.packed_stride, Sb + (int64_t)e * g.scale_stride,
-                         FMT == XQ_FMT_NVFP4 ? g.global_scale[e] : 1.0f, n0w, tid);
+    const float* nf4_levels = nullptr;
+    if constexpr (FMT == XQ_FMT_NF4) {
+        __shared__ float s_nf4[16];
+        if (tid < 16) s_nf4[tid] = kNf4Level[tid];
+        __syncthreads();
+        nf4_levels = s_nf4;
     }
+    // ---- per-thread global addresses of a tile (fixed across its K-steps except for the k offset)
+    const bf16_t* a_src[4];
+    int a_dst[4];
+#pragma unroll
+    for (int p = 0; p < 4; ++p) a_dst[p] = swz((tid + p * NT) >> 3, (tid + p * NT) & 7);
+    auto aim = [&](const TileDesc& t) {
+        // the thread index as a value the optimiser cannot see through: the address arithmetic below is then done
+        // per tile, where it is needed, instead of being split into tile-independent parts that would have to stay
+        // in registers (or spill) across the whole main loop
+        int tv = tid;
+        if constexpr (PERSIST) asm volatile("" : "+v"(tv));
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            const int u = tv + p * NT;
+            int64_t r = t.row0 + (u >> 3);
+            r = r < t.row_end ? r : t.row_end - 1;
+            a_src[p] = g.A + r * g.lda + (u & 7) * 8 + kt0 * F8_BK;
+        }
+#pragma unroll
+        for (int d = 0; d < PD; ++d) {
+            if constexpr (GU) wls[d].init_gu(g, t.n0, tv);
+            else wls[d].init(g, t.Wb + (int64_t)t.e * g.packed_stride, t.Sb + (int64_t)t.e * g.scale_stride,
+                             FMT == XQ_FMT_NVFP4 ? g.global_scale[t.e] : 1.0f, t.n0w, tv);
+            wls[d].tid = tid;            // the LDS addresses of its stores do not change from tile to tile
+            if constexpr (FMT == XQ_FMT_NF4) wls[d].nf4_lds = nf4_levels;
+        }
+    };
     // contraction over two matrices of one shape (expert-bank dgrad of gate and up; dense dgrad of gate and up): the
     // K-steps from nk1 on read the second one (same expert offset in both)
     constexpr bool TWO_K = FMT == XQ_FMT_FP8 && !GU && ((GROUPED && CC) || (!GROUPED && !CC && !SPLIT256));
@@ -537,13 +585,6 @@ __global__ void __launch_bounds__(2 * T, 2) gemm_256_kernel(G256Args g) {
             wdelta = (g.W2 - g.W) - (int64_t)nk1 * (CC ? F8_BK : (int64_t)F8_BK * g.wcols);
             sdelta = ((const float*)g.scales2 - (const float*)g.scales) - (int64_t)(nk1 >> 1) * (CC ? 1 : scols);
         }
-    }
-    if constexpr (FMT == XQ_FMT_NF4) {
-        __shared__ float s_nf4[16];
-        if (tid < 16) s_nf4[tid] = kNf4Level[tid];
-        __syncthreads();
-#pragma unroll
-        for (int d = 0; d < PD; ++d) wls[d].nf4_lds = s_nf4;
     }
 
     u32x4 aregs[PD][4];
@@ -558,13 +599,6 @@ __global__ void __launch_bounds__(2 * T, 2) gemm_256_kernel(G256Args g) {
     };
 
     f32x16 acc[TM][TN];
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-            for (int q = 0; q < 16; ++q) acc[i][j][q] = 0.0f;
-
     const int fr = lane & 31, fh = lane >> 5;
     auto load_frags = [&](const bf16_t* a, const bf16_t* b, int ks, bool b_is_nt, bf16x8* af, bf16x8* bfr) {
 #pragma unroll
@@ -634,131 +668,246 @@ __global__ void __launch_bounds__(2 * T, 2) gemm_256_kernel(G256Args g) {
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         __builtin_amdgcn_sched_barrier(0);
     };
+    TileDesc cur;
+    int vb = (int)blockIdx.x, round = 0;
+    if (!describe(vb, 0, cur)) return;
+    aim(cur);
     load_a(aregs[0], 0);
     wls[0].load(kt0);
-    store_a(As, aregs[0]);
-    wls[0].store(Bs, 0);
-    wls[0].store(Bs, 1);
-    if constexpr (PD == 1) {
-        if (nk > 1) { load_a(aregs[0], 1); wls[0].load(kt0 + 1); }
-        __syncthreads();
-        load_frags(As, Bs, 0, false, af0, bf0);
-        int kt = 0;
-        for (; kt + 2 < nk; ++kt) iteration(kt, true, true, aregs[0], wls[0], kt + 2);
-        if (kt + 1 < nk) { iteration(kt, true, false, aregs[0], wls[0], 0); ++kt; }
-        iteration(kt, false, false, aregs[0], wls[0], 0);
-    } else {
-        // Tiles 1 .. PD are requested in this order, so that they also arrive in it.  Every iteration stores the
-        // set of tile kt+1 and refills it with tile kt+1+PD; past the end the tile index is clamped (the last tile
-        // is fetched again and stored into the stage nobody reads any more), which keeps every load unconditional.
-        const int last = nk - 1;
+    for (;;) {
 #pragma unroll
-        for (int d = 1; d <= PD; ++d) { load_a(aregs[d % PD], min(d, last)); wls[d % PD].load(kt0 + min(d, last)); }
-        __syncthreads();
-        load_frags(As, Bs, 0, false, af0, bf0);
-        int kt = 0;
-        for (; kt + PD <= nk; kt += PD) {
+        for (int i = 0; i < TM; ++i)
 #pragma unroll
-            for (int d = 0; d < PD; ++d)
-                iteration(kt + d, true, true, aregs[(d + 1) % PD], wls[(d + 1) % PD], min(kt + d + 1 + PD, last));
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int q = 0; q < 16; ++q) acc[i][j][q] = 0.0f;
+        store_a(As, aregs[0]);
+        wls[0].store(Bs, 0);
+        wls[0].store(Bs, 1);
+        if constexpr (PD == 1) {
+            if (nk > 1) { load_a(aregs[0], 1); wls[0].load(kt0 + 1); }
+            __syncthreads();
+            load_frags(As, Bs, 0, false, af0, bf0);
+            int kt = 0;
+            for (; kt + 2 < nk; ++kt) iteration(kt, true, true, aregs[0], wls[0], kt + 2);
+            if (kt + 1 < nk) { iteration(kt, true, false, aregs[0], wls[0], 0); ++kt; }
+            iteration(kt, false, false, aregs[0], wls[0], 0);
+        } else {
+            // Tiles 1 .. PD are requested in this order, so that they also arrive in it.  Every iteration stores the
+            // set of tile kt+1 and refills it with tile kt+1+PD; past the end the tile index is clamped (the last tile
+            // is fetched again and stored into the stage nobody reads any more), which keeps every load unconditional.
+            const int last = nk - 1;
+#pragma unroll
+            for (int d = 1; d <= PD; ++d) { load_a(aregs[d % PD], min(d, last)); wls[d % PD].load(kt0 + min(d, last)); }
+            __syncthreads();
+            load_frags(As, Bs, 0, false, af0, bf0);
+            int kt = 0;
+            for (; kt + PD <= nk; kt += PD) {
+#pragma unroll
+                for (int d = 0; d < PD; ++d)
+                    iteration(kt + d, true, true, aregs[(d + 1) % PD], wls[(d + 1) % PD], min(kt + d + 1 + PD, last));
+            }
+#pragma unroll
+            for (int d = 0; d < PD - 1; ++d)
+                if (kt + d < nk) iteration(kt + d, true, true, aregs[(d + 1) % PD], wls[(d + 1) % PD], last);
         }
-#pragma unroll
-        for (int d = 0; d < PD - 1; ++d)
-            if (kt + d < nk) iteration(kt + d, true, true, aregs[(d + 1) % PD], wls[(d + 1) % PD], last);
-    }
 
-    // ---- low-rank side term: su[rows, rp] x lora_right[n, rp], both [row][k] tiles in stage 0
-    if (g.r_pad > 0 && split == 0) {
-        const int rp = g.r_pad, cpr = rp >> 3;  // 16-byte chunks per row
-        const bf16_t* lr = lr_b + (int64_t)e * bank_width * rp;
-        for (int idx = tid; idx < F8_BM * cpr; idx += NT) {
-            const int r = idx / cpr, c = idx - r * cpr;
-            int64_t row = row0 + r;
-            row = row < row_end ? row : row_end - 1;
-            *(u32x4*)(As + swz(r, c)) = *(const u32x4*)(su_b + row * g.ld_su + c * 8);
-            if constexpr (GU) {
-                // the up projection's intermediate in the second activation stage; factor rows: 128 of gate's, 128 of up's
-                *(u32x4*)(As + F8_A_STAGE + swz(r, c)) = *(const u32x4*)(g.su2 + row * g.ld_su + c * 8);
-                int n = n0 + (r & 127);
-                n = n < g.Nout ? n : g.Nout - 1;
-                *(u32x4*)(Bs + swz(r, c)) = *(const u32x4*)((r < 128 ? g.lora_right : g.lora_right2) + (int64_t)n * rp + c * 8);
-            } else {
-                int n = n0w + r;
-                n = n < bank_width ? n : bank_width - 1;
-                *(u32x4*)(Bs + swz(r, c)) = *(const u32x4*)(lr + (int64_t)n * rp + c * 8);
+        // ---- the block's next tile: its first K-step is requested now and arrives while the low-rank term is
+        // multiplied and the finished tile is stored (the register set and the loader are free: the pipeline is drained)
+        TileDesc nx;
+        bool has_next = false;
+        if constexpr (PERSIST) {
+            has_next = describe(vb + (int)gridDim.x, round + 1, nx);
+            if (has_next) {
+                aim(nx);
+                load_a(aregs[0], 0);
+                wls[0].load(kt0);
             }
         }
-        __syncthreads();
-        for (int ks = 0; ks < (rp >> 4); ++ks) {
-            bf16x8 af[TM], bfr[TN];
-            load_frags(As, Bs, ks, true, af, bfr);
-            if constexpr (GU) {
-                bf16x8 af2[TM], unused[TN];
-                load_frags(As + F8_A_STAGE, Bs, ks, true, af2, unused);
-#pragma unroll
-                for (int i = 0; i < TM; ++i) {
-                    acc[i][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[0], af[i], acc[i][0], 0, 0, 0);
-                    acc[i][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[1], af2[i], acc[i][1], 0, 0, 0);
+
+        // ---- low-rank side term: su[rows, rp] x lora_right[n, rp], both [row][k] tiles in stage 0
+        if (g.r_pad > 0 && split == 0) {
+            const int rp = g.r_pad, cpr = rp >> 3;  // 16-byte chunks per row
+            const bf16_t* lr = cur.lr_b + (int64_t)cur.e * cur.bank_width * rp;
+            for (int idx = tid; idx < F8_BM * cpr; idx += NT) {
+                const int r = idx / cpr, c = idx - r * cpr;
+                int64_t row = cur.row0 + r;
+                row = row < cur.row_end ? row : cur.row_end - 1;
+                *(u32x4*)(As + swz(r, c)) = *(const u32x4*)(cur.su_b + row * g.ld_su + c * 8);
+                if constexpr (GU) {
+                    // the up projection's intermediate in the second activation stage; factor rows: 128 of gate's, 128 of up's
+                    *(u32x4*)(As + F8_A_STAGE + swz(r, c)) = *(const u32x4*)(g.su2 + row * g.ld_su + c * 8);
+                    int n = cur.n0 + (r & 127);
+                    n = n < g.Nout ? n : g.Nout - 1;
+                    *(u32x4*)(Bs + swz(r, c)) = *(const u32x4*)((r < 128 ? g.lora_right : g.lora_right2) + (int64_t)n * rp + c * 8);
+                } else {
+                    int n = cur.n0w + r;
+                    n = n < cur.bank_width ? n : cur.bank_width - 1;
+                    *(u32x4*)(Bs + swz(r, c)) = *(const u32x4*)(lr + (int64_t)n * rp + c * 8);
                 }
-            } else {
-                mma(af, bfr);
             }
-        }
-    }
-
-    // ---- gate / up epilogue: acc[i][0] is the gate, acc[i][1] the up projection of the same 4 x 4 columns
-    if constexpr (GU) {
+            __syncthreads();
+            for (int ks = 0; ks < (rp >> 4); ++ks) {
+                bf16x8 af[TM], bfr[TN];
+                load_frags(As, Bs, ks, true, af, bfr);
+                if constexpr (GU) {
+                    bf16x8 af2[TM], unused[TN];
+                    load_frags(As + F8_A_STAGE, Bs, ks, true, af2, unused);
 #pragma unroll
-        for (int i = 0; i < TM; ++i) {
-            const int64_t row = row0 + wm * (T / 2) + i * 32 + fr;
-            if (row >= row_end) continue;
-            bf16_t* crow = g.C + row * g.ldc;
-            bf16_t* hrow = g.H + row * g.ldh;
+                    for (int i = 0; i < TM; ++i) {
+                        acc[i][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[0], af[i], acc[i][0], 0, 0, 0);
+                        acc[i][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[1], af2[i], acc[i][1], 0, 0, 0);
+                    }
+                } else {
+                    mma(af, bfr);
+                }
+            }
+            if (GU || g.wide_rows) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");   // the stages become staging areas
+        }
+
+        // ---- the finished tile.  A lane holds, per 32 x 32 MFMA tile, row fr and 4 x 4 consecutive columns; stored from
+        // there, an instruction writes 16-byte pieces of 32 different rows and the memory system sees the tile as 8192
+        // partial-line writes (measured: 13 % of a launch).  Instead each wave passes its (T/2) x 64 sub-tile through a
+        // private LDS area ([row][64] bf16, the operand tiles' chunk swizzle; LDS operations of a wave execute in order,
+        // so no barrier) and writes whole 128-byte row pieces, 8 rows per instruction.  Lanes fr and fr + 32 first swap
+        // 8-byte halves (v_permlane32_swap) so that each holds 16 consecutive bytes.
+        bf16_t* stg = smem + wave * (TM * 32 * 64);
+        // (the lane index as a value the optimiser cannot see through: the staging addresses are then worked out here,
+        // per tile, instead of being carried -- spilled -- across the main loop)
+        int lv = lane;
+        asm volatile("" : "+v"(lv));
+        const int sfr = lv & 31, sfh = lv >> 5;
+        auto stage_pair = [&](int row, int chunk, uint32_t y0, uint32_t y1, uint32_t x0, uint32_t x1) {
+            // in: columns 4 fh .. + 3 of the 8-column groups 2p (y) and 2p + 1 (x); out: 8 consecutive columns of group 2p + fh
+            const auto s0 = __builtin_amdgcn_permlane32_swap(y0, x0, false, false);
+            const auto s1 = __builtin_amdgcn_permlane32_swap(y1, x1, false, false);
+            *(u32x4*)(stg + swz(row, chunk)) = u32x4{s0[0], s1[0], s0[1], s1[1]};
+        };
+
+        if constexpr (GU) {
+            // ---- gate / up epilogue: acc[i][0] is the gate, acc[i][1] the up projection of the same 4 x 4 columns
+            // per 32-row band: the two projections as their bf16 outputs (a staged row = 32 gate columns | the same 32
+            // up columns) are staged and written, then h from the rounded values goes through the same rows
+            uint32_t bg[4][2] = {}, bu[4][2] = {};       // this lane's 16 bias values of either projection, packed bf16
 #pragma unroll
             for (int q4 = 0; q4 < 4; ++q4) {
-                const int n = n0 + wn * 32 + 8 * q4 + 4 * fh;
-                if (n >= g.Nout) continue;
-                float gv[4], uv[4], hv[4];
+                const int n = min(cur.n0 + wn * 32 + 8 * q4 + 4 * sfh, g.Nout - 4);
+                if (g.bias) { const u32x2 b = *(const u32x2*)(g.bias + n); bg[q4][0] = b[0]; bg[q4][1] = b[1]; }
+                if (g.bias2) { const u32x2 b = *(const u32x2*)(g.bias2 + n); bu[q4][0] = b[0]; bu[q4][1] = b[1]; }
+            }
 #pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    gv[c] = acc[i][0][4 * q4 + c];
-                    uv[c] = acc[i][1][4 * q4 + c];
-                    if (g.bias) gv[c] += bf16_to_f32(g.bias[n + c]);
-                    if (g.bias2) uv[c] += bf16_to_f32(g.bias2[n + c]);
-                    gv[c] = round_bf16(gv[c]);                       // the two projections as their bf16 outputs
-                    uv[c] = round_bf16(uv[c]);
-                    hv[c] = round_bf16(gv[c] * sigmoid_f32(gv[c])) * uv[c];
+            for (int i = 0; i < TM; ++i) {
+                uint32_t gp[4][2], up[4][2], hp[4][2];
+#pragma unroll
+                for (int q4 = 0; q4 < 4; ++q4) {
+                    float gv[4], uv[4], hv[4];
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        gv[c] = acc[i][0][4 * q4 + c];
+                        uv[c] = acc[i][1][4 * q4 + c];
+                        if (g.bias) gv[c] += __uint_as_float((c & 1) ? (bg[q4][c >> 1] & 0xffff0000u) : (bg[q4][c >> 1] << 16));
+                        if (g.bias2) uv[c] += __uint_as_float((c & 1) ? (bu[q4][c >> 1] & 0xffff0000u) : (bu[q4][c >> 1] << 16));
+                        gv[c] = round_bf16(gv[c]);
+                        uv[c] = round_bf16(uv[c]);
+                        hv[c] = round_bf16(gv[c] * sigmoid_f32(gv[c])) * uv[c];
+                    }
+                    gp[q4][0] = pack_bf16x2(gv[0], gv[1]); gp[q4][1] = pack_bf16x2(gv[2], gv[3]);
+                    up[q4][0] = pack_bf16x2(uv[0], uv[1]); up[q4][1] = pack_bf16x2(uv[2], uv[3]);
+                    hp[q4][0] = pack_bf16x2(hv[0], hv[1]); hp[q4][1] = pack_bf16x2(hv[2], hv[3]);
                 }
-                *(u32x2*)(crow + n) = u32x2{pack_bf16x2(gv[0], gv[1]), pack_bf16x2(gv[2], gv[3])};
-                *(u32x2*)(crow + g.Nout + n) = u32x2{pack_bf16x2(uv[0], uv[1]), pack_bf16x2(uv[2], uv[3])};
-                *(u32x2*)(hrow + n) = u32x2{pack_bf16x2(hv[0], hv[1]), pack_bf16x2(hv[2], hv[3])};
+#pragma unroll
+                for (int p = 0; p < 2; ++p) {
+                    stage_pair(i * 32 + sfr, 2 * p + sfh, gp[2 * p][0], gp[2 * p][1], gp[2 * p + 1][0], gp[2 * p + 1][1]);
+                    stage_pair(i * 32 + sfr, 4 + 2 * p + sfh, up[2 * p][0], up[2 * p][1], up[2 * p + 1][0], up[2 * p + 1][1]);
+                }
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    const int rl = i * 32 + t * 8 + (lv >> 3), ch = lv & 7;
+                    const u32x4 v = *(const u32x4*)(stg + swz(rl, ch));
+                    const int64_t row = cur.row0 + wm * (T / 2) + rl;
+                    const int n = cur.n0 + wn * 32 + (ch & 3) * 8;
+                    if (row < cur.row_end && n < g.Nout) *(u32x4*)(g.C + row * g.ldc + (ch >> 2) * g.Nout + n) = v;
+                }
+#pragma unroll
+                for (int p = 0; p < 2; ++p)
+                    stage_pair(i * 32 + sfr, 2 * p + sfh, hp[2 * p][0], hp[2 * p][1], hp[2 * p + 1][0], hp[2 * p + 1][1]);
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    const int rl = i * 32 + t * 16 + (lv >> 2), ch = lv & 3;
+                    const u32x4 v = *(const u32x4*)(stg + swz(rl, ch));
+                    const int64_t row = cur.row0 + wm * (T / 2) + rl;
+                    const int n = cur.n0 + wn * 32 + ch * 8;
+                    if (row < cur.row_end && n < g.Nout) *(u32x4*)(g.H + row * g.ldh + n) = v;
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        } else {
+            // ---- epilogue: lane holds, per (i, j) tile, row m = fr and 4 x 4 consecutive columns
+            if (g.wide_rows && !(CAN_SPLIT && g.ksplit > 1)) {
+#pragma unroll
+                for (int j = 0; j < TN; ++j) {
+                    uint32_t bw[4][2] = {};          // this lane's 16 bias values of the column tile, packed bf16
+                    if (g.bias) {
+#pragma unroll
+                        for (int q4 = 0; q4 < 4; ++q4) {
+                            const u32x2 b = *(const u32x2*)(g.bias + min(cur.n0 + wn * 64 + j * 32 + 8 * q4 + 4 * sfh, g.Nout - 4));
+                            bw[q4][0] = b[0]; bw[q4][1] = b[1];
+                        }
+                    }
+#pragma unroll
+                    for (int i = 0; i < TM; ++i) {
+                        uint32_t pk[4][2];
+#pragma unroll
+                        for (int q4 = 0; q4 < 4; ++q4) {
+                            float v0 = acc[i][j][4 * q4], v1 = acc[i][j][4 * q4 + 1], v2 = acc[i][j][4 * q4 + 2], v3 = acc[i][j][4 * q4 + 3];
+                            if (g.bias) {
+                                v0 += __uint_as_float(bw[q4][0] << 16); v1 += __uint_as_float(bw[q4][0] & 0xffff0000u);
+                                v2 += __uint_as_float(bw[q4][1] << 16); v3 += __uint_as_float(bw[q4][1] & 0xffff0000u);
+                            }
+                            pk[q4][0] = pack_bf16x2(v0, v1); pk[q4][1] = pack_bf16x2(v2, v3);
+                        }
+#pragma unroll
+                        for (int p = 0; p < 2; ++p)
+                            stage_pair(i * 32 + sfr, j * 4 + 2 * p + sfh, pk[2 * p][0], pk[2 * p][1], pk[2 * p + 1][0], pk[2 * p + 1][1]);
+                    }
+                }
+#pragma unroll
+                for (int t = 0; t < TM * 4; ++t) {
+                    const int rl = t * 8 + (lv >> 3), ch = lv & 7;
+                    const u32x4 v = *(const u32x4*)(stg + swz(rl, ch));
+                    const int64_t row = cur.row0 + wm * (T / 2) + rl;
+                    const int n = cur.n0 + wn * 64 + ch * 8;
+                    if (row < cur.row_end && n < g.Nout) *(u32x4*)(g.C + row * g.ldc + n) = v;
+                }
+            } else
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+                const int64_t row = cur.row0 + wm * (T / 2) + i * 32 + fr;
+                if (row >= cur.row_end) continue;
+                bf16_t* crow = g.C + row * g.ldc;
+                float* prow = (CAN_SPLIT && g.ksplit > 1) ? g.partial + ((int64_t)split * g.M + row) * g.Nout : nullptr;
+#pragma unroll
+                for (int j = 0; j < TN; ++j) {
+#pragma unroll
+                    for (int q4 = 0; q4 < 4; ++q4) {
+                        const int n = cur.n0 + wn * 64 + j * 32 + 8 * q4 + 4 * fh;
+                        if (n >= g.Nout) continue;  // Nout % 16 == 0: groups of 4 are all in or all out
+                        float v0 = acc[i][j][4 * q4], v1 = acc[i][j][4 * q4 + 1], v2 = acc[i][j][4 * q4 + 2], v3 = acc[i][j][4 * q4 + 3];
+                        if (g.bias && split == 0) {
+                            v0 += bf16_to_f32(g.bias[n]); v1 += bf16_to_f32(g.bias[n + 1]);
+                            v2 += bf16_to_f32(g.bias[n + 2]); v3 += bf16_to_f32(g.bias[n + 3]);
+                        }
+                        if (prow) *(f32x4*)(prow + n) = f32x4{v0, v1, v2, v3};
+                        else *(u32x2*)(crow + n) = u32x2{pack_bf16x2(v0, v1), pack_bf16x2(v2, v3)};
+                    }
+                }
             }
         }
-        return;
-    }
-
-    // ---- epilogue: lane holds, per (i, j) tile, row m = fr and 4 x 4 consecutive columns
-#pragma unroll
-    for (int i = 0; i < TM; ++i) {
-        const int64_t row = row0 + wm * (T / 2) + i * 32 + fr;
-        if (row >= row_end) continue;
-        bf16_t* crow = g.C + row * g.ldc;
-        float* prow = (CAN_SPLIT && g.ksplit > 1) ? g.partial + ((int64_t)split * g.M + row) * g.Nout : nullptr;
-#pragma unroll
-        for (int j = 0; j < TN; ++j) {
-#pragma unroll
-            for (int q4 = 0; q4 < 4; ++q4) {
-                const int n = n0 + wn * 64 + j * 32 + 8 * q4 + 4 * fh;
-                if (n >= g.Nout) continue;  // Nout % 16 == 0: groups of 4 are all in or all out
-                float v0 = acc[i][j][4 * q4], v1 = acc[i][j][4 * q4 + 1], v2 = acc[i][j][4 * q4 + 2], v3 = acc[i][j][4 * q4 + 3];
-                if (g.bias && split == 0) {
-                    v0 += bf16_to_f32(g.bias[n]); v1 += bf16_to_f32(g.bias[n + 1]);
-                    v2 += bf16_to_f32(g.bias[n + 2]); v3 += bf16_to_f32(g.bias[n + 3]);
-                }
-                if (prow) *(f32x4*)(prow + n) = f32x4{v0, v1, v2, v3};
-                else *(u32x2*)(crow + n) = u32x2{pack_bf16x2(v0, v1), pack_bf16x2(v2, v3)};
-            }
-        }
+        if (!has_next) break;
+        cur = nx;
+        vb += (int)gridDim.x;
+        ++round;
+        __syncthreads();      // the low-rank fragments of stage 0 have been read before the next tile is stored there
     }
 }
 

@@ -87,6 +87,8 @@ int check_call(const xq_weight* gate, const xq_weight* up, const xq_weight* down
         for (int p = 0; p < 3; ++p) XQ_REQUIRE(lora->A[p] && lora->B[p], "%s: LoRA factor %d is NULL", who, p);
     d->M = M; d->H = H; d->I = I; d->r = lora->r; d->rp = r_pad_of(lora->r);
     if (M > 0) XQ_REQUIRE(saved->gate_up && saved->h && (d->rp == 0 || (saved->su_gate_up && saved->su_down)), "%s: a buffer of xq_mlp_saved is NULL", who);
+    XQ_REQUIRE(xq_aligned(saved->gate_up, 16) && xq_aligned(saved->h, 16), "%s: gate_up and h of xq_mlp_saved must be 16-byte aligned", who);
+    for (int p = 0; p < 3; ++p) XQ_REQUIRE(xq_aligned(lora->bias[p], 8), "%s: bias vectors must be 8-byte aligned", who);
     return XQ_OK;
 }
 
