@@ -43,25 +43,25 @@ BF16_MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense bf16, published
 MEASURED_TRAFFIC = {
     # gemm_256_kernel<int4, T=128> in 4 K splits + splitk_reduce_kernel: mean of the forward and dgrad launches
     # (64 MiB of it are the fp32 partial sums written and read back)
-    0: (109.6 * 2 ** 20, "profiles/gemm_128_int4_linear_m512.txt", 0.04478),
+    0: (109.6 * 2 ** 20, "profiles/gemm_128_int4_linear_m512.txt", 0.04486),
     # gemm_256_kernel<fp8>: mean over the 4 launches of a step (gate|up forward with the SwiGLU epilogue, down
     # forward, d_h, dx as one sum over the gate and up weights)
-    1: (1457.8 * 2 ** 20, "profiles/gemm_256_fp8_mlp_m8192.txt", 1.13390),
+    1: (1461.2 * 2 ** 20, "profiles/gemm_256_fp8_mlp_m8192.txt", 1.08942),
     # gemm_256_kernel<nvfp4>, 256x256 tiles (whole rounds; trailing rows in K splits) and 128x128 tiles
     # (+ splitk_reduce_kernel): mean over the 12 launches of a step, fp32 partial sums included
-    2: (187.2 * 2 ** 20, "profiles/gemm_256_nvfp4_attn_m4096.txt", 0.14518),
+    2: (185.7 * 2 ** 20, "profiles/gemm_256_nvfp4_attn_m4096.txt", 0.14304),
     # gemm_256_kernel<fp8, grouped>: mean over the 4 launches of a step (gate|up forward over two banks, down
     # forward, d_h, dx as one sum over both banks)
-    3: (1351.6 * 2 ** 20, "profiles/gemm_256_fp8_grouped_moe_e128.txt", 0.83854),
+    3: (1345.0 * 2 ** 20, "profiles/gemm_256_fp8_grouped_moe_e128.txt", 0.72525),
     # skinny_split_kernel + skinny_epilogue_kernel: mean per forward over the 32 cases (includes the fp32 partial
     # tiles written and read back: 23.3 MiB of it are algorithmic)
     4: (41.0 * 2 ** 20, "profiles/skinny_split_kernel_decode_shapes.txt", 0.02006),
     # merge_prep_kernel + merge_kernel<fp8>: mean per call (re-quantise 96 MiB, publish 144 MiB algorithmic)
     5: (134.4 * 2 ** 20, "profiles/merge_kernel_fp8_mlp_weights.txt", 0.04168),
     # gemm_256_kernel<nf4>: mean of the forward and dgrad launches
-    6: (737.0 * 2 ** 20, "profiles/gemm_256_nf4_mlp_m8192.txt", 0.85447),
+    6: (748.2 * 2 ** 20, "profiles/gemm_256_nf4_mlp_m8192.txt", 0.84180),
     # gemm_256_kernel<nvfp4 GKN, grouped>: mean over the 6 launches of a step
-    7: (889.1 * 2 ** 20, "profiles/gemm_256_nvfp4_gkn_grouped_moe_e128.txt", 0.58278),
+    7: (900.4 * 2 ** 20, "profiles/gemm_256_nvfp4_gkn_grouped_moe_e128.txt", 0.54453),
     # merge_prep_kernel + merge_kernel<nvfp4>: mean per call over amax / re-quantise / publish of the four weights
     9: (59.0 * 2 ** 20, "profiles/merge_kernel_nvfp4_attn_weights.txt", 0.03500),
 }
