@@ -133,8 +133,19 @@ extern "C" int xq_grouped_fwd(const xq_weight* gate, const xq_weight* up, const 
     PanelJobs jobs{};
     jobs.in_f32 = lora->dtype == XQ_DT_F32;
     const int gAe = lora->A_experts[0], uAe = lora->A_experts[1], dAe = lora->A_experts[2];
-    bf16_t* F_gA = jobs.add(lora->A[0], gAe, H, d.r, true, cv.take<bf16_t>((int64_t)gAe * rp * H * 2), gAe, rp, H);
-    bf16_t* F_uA = jobs.add(lora->A[1], uAe, H, d.r, true, cv.take<bf16_t>((int64_t)uAe * rp * H * 2), uAe, rp, H);
+    // gate's and up's A panels as the row bands [0, rp) and [rp, 2 rp) of one [2 rp, H] panel per expert when both are
+    // held the same way: both low-rank intermediates then come from one pass over the routed rows
+    const bool one_pass = gAe == uAe && 2 * rp <= 64;
+    bf16_t *F_gA, *F_uA;
+    if (one_pass) {
+        F_gA = cv.take<bf16_t>((int64_t)gAe * 2 * rp * H * 2);
+        F_uA = F_gA + (int64_t)rp * H;
+        jobs.add(lora->A[0], gAe, H, d.r, true, F_gA, gAe, rp, H, 0, 2 * (int64_t)rp * H);
+        jobs.add(lora->A[1], uAe, H, d.r, true, F_uA, uAe, rp, H, 0, 2 * (int64_t)rp * H);
+    } else {
+        F_gA = jobs.add(lora->A[0], gAe, H, d.r, true, cv.take<bf16_t>((int64_t)gAe * rp * H * 2), gAe, rp, H);
+        F_uA = jobs.add(lora->A[1], uAe, H, d.r, true, cv.take<bf16_t>((int64_t)uAe * rp * H * 2), uAe, rp, H);
+    }
     bf16_t* Lr_gB = jobs.add(lora->B[0], lora->B_experts[0], d.r, I, true, cv.take<bf16_t>((int64_t)E * I * rp * 2), E, I, rp);
     bf16_t* Lr_uB = jobs.add(lora->B[1], lora->B_experts[1], d.r, I, true, cv.take<bf16_t>((int64_t)E * I * rp * 2), E, I, rp);
     bf16_t* F_dA = jobs.add(lora->A[2], dAe, I, d.r, true, cv.take<bf16_t>((int64_t)dAe * rp * I * 2), dAe, rp, I);
@@ -145,8 +156,12 @@ extern "C" int xq_grouped_fwd(const xq_weight* gate, const xq_weight* up, const 
     const int32_t *off = saved->offsets, *toff = saved->tile_offsets;
     bf16_t *su_g = (bf16_t*)saved->su_gate, *su_u = (bf16_t*)saved->su_up, *su_d = (bf16_t*)saved->su_down;
     bf16_t *gu = (bf16_t*)saved->gate_up, *h = (bf16_t*)saved->h;       // gu [R, 2I]: gate | up
-    if ((rc = launch_small_nt(xs, H, R, H, F_gA, rp, s, su_g, off, toff, E, gAe == 1, stream))) return rc;
-    if ((rc = launch_small_nt(xs, H, R, H, F_uA, rp, s, su_u, off, toff, E, uAe == 1, stream))) return rc;
+    if (one_pass) {
+        if ((rc = launch_small_nt(xs, H, R, H, F_gA, 2 * rp, s, su_g, off, toff, E, gAe == 1, stream, rp, su_u, rp))) return rc;
+    } else {
+        if ((rc = launch_small_nt(xs, H, R, H, F_gA, rp, s, su_g, off, toff, E, gAe == 1, stream))) return rc;
+        if ((rc = launch_small_nt(xs, H, R, H, F_uA, rp, s, su_u, off, toff, E, uAe == 1, stream))) return rc;
+    }
     if (fuse_gate_up(gate, up)) {       // both projections in one launch: column tiles past I take the up bank
         const TwoBanks two{up, su_u, Lr_uB};
         if ((rc = launch_tile_gemm(gate, false, xs, H, R, off, toff, su_g, Lr_gB, rp, nullptr, gu, 2 * I, stream, who, nullptr, 0, &two))) return rc;

@@ -27,18 +27,21 @@ int launch_factor_prep_multi(const FactorPrepJobs& jobs, hipStream_t stream);
 // the expert count) into bf16 [n_out, R_out, C_out], optionally transposed, zero padded; n_src == 1 < n_out repeats
 // the one source matrix for every expert (a factor shared by all experts, handed to a kernel that indexes panels
 // by expert).  `pitch` (0: C_out) is the row length of the destination, for a panel that is a column band of a
-// wider one.
+// wider one; `e_stride` (0: R_out * pitch) the distance between two experts' panels in the destination, for a panel
+// that is a row band of a taller one.
 constexpr int MAX_PANEL_JOBS = 6;
 struct PanelJobs {
     const void* in[MAX_PANEL_JOBS];
     bf16_t* out[MAX_PANEL_JOBS];
     int64_t R_in[MAX_PANEL_JOBS], C_in[MAX_PANEL_JOBS], R_out[MAX_PANEL_JOBS], C_out[MAX_PANEL_JOBS], pitch[MAX_PANEL_JOBS];
+    int64_t e_stride[MAX_PANEL_JOBS];
     int32_t n_src[MAX_PANEL_JOBS], n_out[MAX_PANEL_JOBS], transpose[MAX_PANEL_JOBS];
     int32_t in_f32, n;
     bf16_t* add(const void* src, int n_src_, int64_t r_in, int64_t c_in, bool tr, bf16_t* dst, int n_out_, int64_t r_out,
-                int64_t c_out, int64_t pitch_ = 0) {
+                int64_t c_out, int64_t pitch_ = 0, int64_t e_stride_ = 0) {
         in[n] = src; out[n] = dst; R_in[n] = r_in; C_in[n] = c_in; R_out[n] = r_out; C_out[n] = c_out;
         pitch[n] = pitch_ ? pitch_ : c_out;
+        e_stride[n] = e_stride_ ? e_stride_ : r_out * pitch[n];
         n_src[n] = n_src_; n_out[n] = n_out_; transpose[n] = tr ? 1 : 0;
         ++n;
         return dst;
@@ -54,7 +57,8 @@ int launch_factor_prep(const void* in, int in_dtype, int64_t R_in, int64_t C_in,
 int launch_small_nt(const bf16_t* In, int64_t ld_in, int64_t n_rows, int64_t Kc, const bf16_t* F,
                     int r_pad, float scale, bf16_t* T, const int32_t* offsets,
                     const int32_t* tile_offsets, int32_t num_experts, bool shared_f, hipStream_t stream,
-                    int64_t ld_t = 0);      // row pitch of T in elements (0: r_pad), to write a column band of a wider matrix
+                    int64_t ld_t = 0,       // row pitch of T in elements (0: r_pad), to write a column band of a wider matrix
+                    bf16_t* T2 = nullptr, int split = 0);   // result columns from `split` on go to T2 (same pitch): two panels' products from one pass
 
 // out[c][j] (or out[j][c] when transpose_out) = sum_m P[m][c] * Q[m][j], fp32.
 //   dense: all rows, split over `splits` row ranges, partials in `partial`

@@ -77,34 +77,73 @@ int launch_factor_prep_multi(const FactorPrepJobs& j, hipStream_t stream) {
     return XQ_OK;
 }
 
+// A block converts one tile of a destination panel through LDS -- 16 x 256 (rows x columns) of a wide panel, 256 x 16
+// of a tall one -- so that both the source and the destination are touched in whole row pieces whichever way the job
+// transposes: e.g. a transposing job into a wide panel reads 256 source rows of 16 entries (one contiguous run when
+// the factor is 16 wide) and writes 16 destination rows of 512 bytes.  (Element by element, the transposing jobs of
+// an expert bank read 4 bytes of every 64-byte row piece per instruction: 61 us for the panels of 128 experts.)
+// Every load is unconditional (indices past the source clamped onto it, the value replaced by zero afterwards): with a
+// branch around them the compiler waits for each load before it issues the next, sixteen round trips per tile.
+constexpr int PP_S = 16, PP_L = 256;
+template <bool F32>
 __global__ void __launch_bounds__(256) panel_prep_kernel(PanelJobs j) {
-    const int k = blockIdx.y;
-    const int64_t per = j.R_out[k] * j.C_out[k], total = per * j.n_out[k];
+    __shared__ float tile[PP_L][PP_S + 1];      // [index along the tile's long side][along its short side]
+    const int k = blockIdx.y, tid = threadIdx.x;
     const int64_t R_in = j.R_in[k], C_in = j.C_in[k], C_out = j.C_out[k], R_out = j.R_out[k], pitch = j.pitch[k];
     const bool tr = j.transpose[k] != 0, shared = j.n_src[k] == 1;
-    for (int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x; t < total; t += (int64_t)gridDim.x * 256) {
-        const int64_t e = t / per, rem = t - e * per;
-        const int64_t i = rem / C_out, c = rem - i * C_out;
-        const int64_t si = tr ? c : i, sj = tr ? i : c;
-        float v = 0.0f;
-        if (si < R_in && sj < C_in) {
-            const int64_t idx = (shared ? 0 : e) * R_in * C_in + si * C_in + sj;
-            v = j.in_f32 ? ((const float*)j.in[k])[idx] : bf16_to_f32(((const bf16_t*)j.in[k])[idx]);
+    const void* in = j.in[k];
+    bf16_t* out = j.out[k];
+    const int64_t e_stride = j.e_stride[k];
+    const bool wide = C_out >= R_out;           // the long side runs along the destination's columns
+    const int64_t TRW = wide ? PP_S : PP_L, TCW = wide ? PP_L : PP_S;
+    const int64_t tiles_r = (R_out + TRW - 1) / TRW, tiles_c = (C_out + TCW - 1) / TCW;
+    const int64_t total = tiles_r * tiles_c * j.n_out[k];
+    const bool load_long_first = wide != tr;    // consecutive threads walk along the source's rows
+    for (int64_t t = blockIdx.x; t < total; t += gridDim.x) {
+        const int64_t e = t / (tiles_r * tiles_c), rem = t - e * (tiles_r * tiles_c);
+        const int64_t i0 = (rem / tiles_c) * TRW, c0 = (rem % tiles_c) * TCW;
+        const int64_t base = (shared ? 0 : e) * R_in * C_in;
+        float val[PP_S];
+        uint32_t keep = 0xffffu;
+#pragma unroll
+        for (int u = 0; u < PP_S; ++u) {
+            const int idx = u * 256 + tid;
+            const int l = load_long_first ? idx % PP_L : idx / PP_S, sh = load_long_first ? idx / PP_L : idx % PP_S;
+            const int64_t i = i0 + (wide ? sh : l), c = c0 + (wide ? l : sh);
+            const int64_t si = tr ? c : i, sj = tr ? i : c;
+            const int64_t src = base + (si < R_in ? si : R_in - 1) * C_in + (sj < C_in ? sj : C_in - 1);
+            val[u] = F32 ? ((const float*)in)[src] : bf16_to_f32(((const bf16_t*)in)[src]);
+            if (!(si < R_in && sj < C_in)) keep &= ~(1u << u);
         }
-        j.out[k][(e * R_out + i) * pitch + c] = to_bf16(v);
+#pragma unroll
+        for (int u = 0; u < PP_S; ++u) {
+            const int idx = u * 256 + tid;
+            const int l = load_long_first ? idx % PP_L : idx / PP_S, sh = load_long_first ? idx / PP_L : idx % PP_S;
+            tile[l][sh] = (keep >> u) & 1u ? val[u] : 0.0f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int u = 0; u < PP_S; ++u) {
+            const int idx = u * 256 + tid;      // consecutive threads walk along the destination's rows
+            const int l = wide ? idx % PP_L : idx / PP_S, sh = wide ? idx / PP_L : idx % PP_S;
+            const int64_t i = i0 + (wide ? sh : l), c = c0 + (wide ? l : sh);
+            if (i < R_out && c < C_out) out[e * e_stride + i * pitch + c] = to_bf16(tile[l][sh]);
+        }
+        __syncthreads();
     }
 }
 
 int launch_panel_prep(const PanelJobs& j, hipStream_t stream) {
     int64_t most = 0;
     for (int k = 0; k < j.n; ++k) {
-        const int64_t t = j.R_out[k] * j.C_out[k] * j.n_out[k];
+        const bool wide = j.C_out[k] >= j.R_out[k];
+        const int64_t t = xq_cdiv(j.R_out[k], wide ? PP_S : PP_L) * xq_cdiv(j.C_out[k], wide ? PP_L : PP_S) * j.n_out[k];
         most = t > most ? t : most;
     }
     if (j.n == 0 || most == 0) return XQ_OK;
-    int64_t blocks = xq_cdiv(most, 256);
-    if (blocks > 4096) blocks = 4096;
-    panel_prep_kernel<<<dim3((unsigned)blocks, (unsigned)j.n), 256, 0, stream>>>(j);
+    if (most > 16384) most = 16384;
+    if (j.in_f32) panel_prep_kernel<true><<<dim3((unsigned)most, (unsigned)j.n), 256, 0, stream>>>(j);
+    else panel_prep_kernel<false><<<dim3((unsigned)most, (unsigned)j.n), 256, 0, stream>>>(j);
     XQ_CHECK_LAUNCH("panel_prep");
     return XQ_OK;
 }
@@ -120,7 +159,9 @@ struct SmallNtArgs {
     int r_pad;
     float scale;
     bf16_t* T;
-    int64_t ld_t;      // row pitch of T in elements (>= r_pad)
+    int64_t ld_t;      // row pitch of T (and T2) in elements
+    bf16_t* T2;        // optional: result columns from `split` on go to T2 (as its columns 0 ..) instead of T
+    int split;
     const int32_t* offsets;
     const int32_t* tile_offsets;
     int32_t num_experts;
@@ -265,10 +306,13 @@ __global__ void __launch_bounds__(256) small_nt_kernel(SmallNtArgs g) {
     for (int n = 0; n < NT; ++n) {
         int j = n * 32 + fr;
         if (j >= g.r_pad) continue;
+        bf16_t* dst = g.T;
+        int jj = j;
+        if (g.T2 && j >= g.split) { dst = g.T2; jj = j - g.split; }
 #pragma unroll
         for (int q = 0; q < 16; ++q) {
             int64_t row = row0 + rg * 32 + (q & 3) + rgrp + 8 * (q >> 2);
-            if (row < row_end) g.T[row * g.ld_t + j] = to_bf16(acc[n][q] * g.scale);
+            if (row < row_end) dst[row * g.ld_t + jj] = to_bf16(acc[n][q] * g.scale);
         }
     }
 }
@@ -302,15 +346,16 @@ static int launch_small_nt_rows(const SmallNtArgs& g, unsigned blocks, hipStream
 
 int launch_small_nt(const bf16_t* In, int64_t ld_in, int64_t n_rows, int64_t Kc, const bf16_t* F, int r_pad,
                     float scale, bf16_t* T, const int32_t* offsets, const int32_t* tile_offsets,
-                    int32_t num_experts, bool shared_f, hipStream_t stream, int64_t ld_t) {
+                    int32_t num_experts, bool shared_f, hipStream_t stream, int64_t ld_t, bf16_t* T2, int split) {
     if (ld_t <= 0) ld_t = r_pad;
-    XQ_REQUIRE(ld_t >= r_pad, "small_nt: output pitch %lld below r_pad %d", (long long)ld_t, r_pad);
+    if (T2) XQ_REQUIRE(split > 0 && split < r_pad && ld_t >= split && ld_t >= r_pad - split, "small_nt: bad split of the result columns");
+    else XQ_REQUIRE(ld_t >= r_pad, "small_nt: output pitch %lld below r_pad %d", (long long)ld_t, r_pad);
     XQ_REQUIRE(r_pad > 0 && r_pad <= 64 && r_pad % 16 == 0, "small_nt: r_pad must be 16/32/48/64, got %d", r_pad);
     XQ_REQUIRE(Kc % 64 == 0, "small_nt: contraction length %lld must be a multiple of 64", (long long)Kc);
     XQ_REQUIRE(ld_in % 8 == 0 && xq_aligned(In, 16) && xq_aligned(F, 16), "small_nt: operands must be 16-byte aligned");
     if (n_rows == 0) return XQ_OK;
-    SmallNtArgs g{In, ld_in, n_rows, Kc, F, shared_f ? 0 : (int64_t)r_pad * Kc, r_pad, scale, T, ld_t, offsets, tile_offsets,
-                  num_experts};
+    SmallNtArgs g{In, ld_in, n_rows, Kc, F, shared_f ? 0 : (int64_t)r_pad * Kc, r_pad, scale, T, ld_t, T2, split, offsets,
+                  tile_offsets, num_experts};
     int rc;
     if (offsets) {
         rc = launch_small_nt_rows<128>(g, (unsigned)(xq_cdiv(n_rows, 128) + num_experts), stream);
