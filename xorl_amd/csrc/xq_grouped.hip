@@ -33,6 +33,15 @@ __global__ void __launch_bounds__(256) split_pair_kernel(const float* src, int64
     dst1[t] = src[i * 2 * half + half + j];
 }
 
+// token_of_row[scatter_index[i]] = i / topk: the token whose copy sits in row r of the expert order (routed copies
+// with an invalid expert id have no row)
+__global__ void __launch_bounds__(256) invert_scatter_kernel(const int32_t* scatter_index, int64_t n, int topk, int32_t* token_of_row) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const int32_t r = scatter_index[i];
+    if (r >= 0) token_of_row[r] = (int32_t)(i / topk);
+}
+
 struct Dims {
     int32_t E, topk, r, rp;
     int64_t T, R, H, I;
@@ -73,7 +82,7 @@ int check_call(const xq_weight* gate, const xq_weight* up, const xq_weight* down
 int64_t fwd_workspace(const Dims& d) {
     const int64_t panels = 2 * al256((int64_t)d.E * d.rp * d.H * 2) + 2 * al256((int64_t)d.E * d.I * d.rp * 2) +
                            al256((int64_t)d.E * d.rp * d.I * 2) + al256((int64_t)d.E * d.H * d.rp * 2);
-    return al256(xq_route_workspace_bytes(d.R, d.E)) + panels + al256(d.R * d.H * 2) + 256;
+    return al256(xq_route_workspace_bytes(d.R, d.E)) + panels + al256(d.R * d.H * 2) + al256(d.R * 4) + 256;
 }
 
 int64_t bwd_workspace(const Dims& d) {
@@ -82,7 +91,7 @@ int64_t bwd_workspace(const Dims& d) {
     const int64_t wide = d.H > d.I ? d.H : d.I;
     const int64_t wg = al256(xq_lora_wgrad_workspace_bytes(d.R, wide, 2 * d.rp <= 64 ? 2 * d.rp : d.rp));
     const int64_t pair = al256((int64_t)d.E * d.H * 2 * d.rp * 4);      // the two A gradients side by side
-    return panels + 3 * al256(d.R * d.H * 2) + al256(d.R * d.I * 2) + al256(d.R * 2 * d.I * 2) + al256(d.R * 4) +
+    return panels + 3 * al256(d.R * d.H * 2) + al256(d.R * d.I * 2) + al256(d.R * 2 * d.I * 2) + 2 * al256(d.R * 4) +
            al256(d.R * d.rp * 2) + al256(d.R * 2 * d.rp * 2) + pair + wg + 256;
 }
 
@@ -126,7 +135,20 @@ extern "C" int xq_grouped_fwd(const xq_weight* gate, const xq_weight* up, const 
         return rc;
     if (R == 0) return XQ_OK;
     bf16_t* xs = (bf16_t*)saved->xs;
-    if ((rc = xq_moe_scatter(hidden, ld_hidden, saved->scatter_index, R, topk, H, xs, H, stream))) return rc;
+    // The pass that first reads the routed rows -- x . A^T of gate (and up) -- takes them from the token matrix through
+    // the inverse of scatter_index and writes the expert-ordered copy xs on its way: no scatter pass of its own.
+    int32_t* token_of_row = cv.take<int32_t>(R * 4);
+    const bool ride = ld_hidden % 8 == 0 && xq_aligned(hidden, 16) && xq_aligned(xs, 16);
+    if (ride) {
+        invert_scatter_kernel<<<dim3((unsigned)xq_cdiv(R, 256)), 256, 0, stream>>>(saved->scatter_index, R, topk, token_of_row);
+        XQ_CHECK_LAUNCH(who);
+    } else if ((rc = xq_moe_scatter(hidden, ld_hidden, saved->scatter_index, R, topk, H, xs, H, stream))) {
+        return rc;
+    }
+    const bf16_t* first_in = ride ? (const bf16_t*)hidden : xs;      // operand of the first pass
+    const int64_t first_ld = ride ? ld_hidden : H;
+    const int32_t* first_map = ride ? token_of_row : nullptr;
+    bf16_t* first_copy = ride ? xs : nullptr;
 
     // bf16 operand layouts of the six factors, one launch.  A factors [E|1, in, r] become the "down" panels
     // [E|1, rp, in] of x . A; B factors [E|1, r, out] become the per-expert right-hand panels [E, out, rp].
@@ -157,9 +179,13 @@ extern "C" int xq_grouped_fwd(const xq_weight* gate, const xq_weight* up, const 
     bf16_t *su_g = (bf16_t*)saved->su_gate, *su_u = (bf16_t*)saved->su_up, *su_d = (bf16_t*)saved->su_down;
     bf16_t *gu = (bf16_t*)saved->gate_up, *h = (bf16_t*)saved->h;       // gu [R, 2I]: gate | up
     if (one_pass) {
-        if ((rc = launch_small_nt(xs, H, R, H, F_gA, 2 * rp, s, su_g, off, toff, E, gAe == 1, stream, rp, su_u, rp))) return rc;
+        if ((rc = launch_small_nt(first_in, first_ld, R, H, F_gA, 2 * rp, s, su_g, off, toff, E, gAe == 1, stream, rp, su_u, rp,
+                                  first_map, first_copy, H)))
+            return rc;
     } else {
-        if ((rc = launch_small_nt(xs, H, R, H, F_gA, rp, s, su_g, off, toff, E, gAe == 1, stream))) return rc;
+        if ((rc = launch_small_nt(first_in, first_ld, R, H, F_gA, rp, s, su_g, off, toff, E, gAe == 1, stream, 0, nullptr, 0,
+                                  first_map, first_copy, H)))
+            return rc;
         if ((rc = launch_small_nt(xs, H, R, H, F_uA, rp, s, su_u, off, toff, E, uAe == 1, stream))) return rc;
     }
     if (fuse_gate_up(gate, up)) {       // both projections in one launch: column tiles past I take the up bank
@@ -240,16 +266,26 @@ extern "C" int xq_grouped_bwd(const xq_weight* gate, const xq_weight* up, const 
     bf16_t* v_d = cv.take<bf16_t>(R * rp * 2);
     bf16_t* v_gu = cv.take<bf16_t>(R * rp2 * 2);          // fused: [R, 2 rp] = v_g | v_u; else v_g [R, rp] then v_u [R, rp]
     float* pair = cv.take<float>((int64_t)E * H * rp2 * 4);
+    int32_t* token_of_row = cv.take<int32_t>(R * 4);
     float* wg = cv.take<float>(0);
     bf16_t *dgate = dgu, *dup = dgu + I;
     bf16_t* v_g = v_gu;
     bf16_t* v_u = fused ? v_gu + rp : v_gu + R * rp;
     const int64_t ld_v = fused ? rp2 : rp;
 
-    if ((rc = xq_moe_scatter(dy, ld_dy, sidx, R, topk, H, g_down, H, stream))) return rc;
+    // as in the forward: the first pass over the routed gradient rows gathers them from dy and writes g_down
+    const bool ride = ld_dy % 8 == 0 && xq_aligned(dy, 16);
+    if (ride) {
+        invert_scatter_kernel<<<dim3((unsigned)xq_cdiv(R, 256)), 256, 0, stream>>>(sidx, R, topk, token_of_row);
+        XQ_CHECK_LAUNCH(who);
+    } else if ((rc = xq_moe_scatter(dy, ld_dy, sidx, R, topk, H, g_down, H, stream))) {
+        return rc;
+    }
 
     // ---- down projection: y = h.W + s*(h.A).B
-    if ((rc = launch_small_nt(g_down, H, R, H, F_dB, rp, s, v_d, off, toff, E, dBe == 1, stream))) return rc;        // s * g . B^T
+    if ((rc = launch_small_nt(ride ? (const bf16_t*)dy : g_down, ride ? ld_dy : H, R, H, F_dB, rp, s, v_d, off, toff, E, dBe == 1, stream,
+                              0, nullptr, 0, ride ? token_of_row : nullptr, ride ? g_down : nullptr, H)))        // s * g . B^T
+        return rc;
     if ((rc = launch_tile_gemm(down, true, g_down, H, R, off, toff, v_d, Lr_dA, rp, nullptr, dh, I, stream, who, nullptr, 0))) return rc;
     if ((rc = launch_tn(g_down, H, H, su_d, rp, r, R, true, grads->dB[2], wg, dBe == 1 ? nullptr : off, E, stream, n_valid))) return rc;   // [E|1, r, H]
     if ((rc = launch_tn(h, I, I, v_d, rp, r, R, false, grads->dA[2], wg, dAe == 1 ? nullptr : off, E, stream, n_valid))) return rc;        // [E|1, I, r]

@@ -58,7 +58,9 @@ int launch_small_nt(const bf16_t* In, int64_t ld_in, int64_t n_rows, int64_t Kc,
                     int r_pad, float scale, bf16_t* T, const int32_t* offsets,
                     const int32_t* tile_offsets, int32_t num_experts, bool shared_f, hipStream_t stream,
                     int64_t ld_t = 0,       // row pitch of T in elements (0: r_pad), to write a column band of a wider matrix
-                    bf16_t* T2 = nullptr, int split = 0);   // result columns from `split` on go to T2 (same pitch): two panels' products from one pass
+                    bf16_t* T2 = nullptr, int split = 0,    // result columns from `split` on go to T2 (same pitch): two panels' products from one pass
+                    const int32_t* row_map = nullptr,       // grouped: product row i is made from row row_map[i] of In, and the
+                    bf16_t* copy_out = nullptr, int64_t ld_copy = 0);   // gathered rows are also written to copy_out [rows, Kc]
 
 // out[c][j] (or out[j][c] when transpose_out) = sum_m P[m][c] * Q[m][j], fp32.
 //   dense: all rows, split over `splits` row ranges, partials in `partial`

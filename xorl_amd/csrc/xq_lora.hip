@@ -165,6 +165,12 @@ struct SmallNtArgs {
     const int32_t* offsets;
     const int32_t* tile_offsets;
     int32_t num_experts;
+    // grouped, optional: row i of the product is made from row row_map[i] of In (rows gathered from a compact matrix),
+    // and the gathered rows are also written to copy_out (row pitch ld_copy) -- the row permutation of a routed
+    // problem rides on the pass that reads the rows first instead of being a pass of its own
+    const int32_t* row_map;
+    bf16_t* copy_out;
+    int64_t ld_copy;
 };
 
 // TR rows per block: 32 (dense; the 4 waves split K) or 128 (grouped; one wave per 32 rows).  FJ = rows of F in
@@ -178,7 +184,7 @@ struct SmallNtArgs {
 // valid ones and their values never used -- so the waits count exactly and the loads of chunk k+2 stay in
 // flight while chunk k is multiplied.
 constexpr int SN_P = 136;   // LDS row pitch in bf16 elements
-template <int TR, int FJ>
+template <int TR, int FJ, bool GATHER = false>
 __global__ void __launch_bounds__(256) small_nt_kernel(SmallNtArgs g) {
     constexpr int NT = (FJ + 7) / 8;
     constexpr int RG = TR / 32, KS = 4 / RG;
@@ -232,12 +238,18 @@ __global__ void __launch_bounds__(256) small_nt_kernel(SmallNtArgs g) {
     const int64_t kspan = g.Kc / KS;  // multiple of 16
     const int64_t kbeg = ks * kspan, kend = kbeg + kspan;
     const bf16_t* xp[8];
+    int32_t orow[GATHER ? 8 : 1];                // GATHER: the rows of copy_out this lane's pieces belong to
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
         int64_t r = wrow0 + j * 4 + crow;
         r = r < row_end ? r : row_end - 1;       // wrow0 may lie past a short segment's end: still a valid row
         r = r < 0 ? 0 : r;
-        xp[j] = g.In + r * g.ld_in;
+        if constexpr (GATHER) {
+            orow[j] = (int32_t)r;
+            xp[j] = g.In + (int64_t)g.row_map[r] * g.ld_in;
+        } else {
+            xp[j] = g.In + r * g.ld_in;
+        }
     }
     u32x4 xr[2][8], fq[FJ];
     auto fetch_x = [&](u32x4* dst, int64_t k) {  // chunk [k, k+128); pieces past kend come from the range's last piece
@@ -258,6 +270,15 @@ __global__ void __launch_bounds__(256) small_nt_kernel(SmallNtArgs g) {
         for (int j = 0; j < 8; ++j) *(u32x4*)(xs + (j * 4 + crow) * SN_P + cpiece) = cur[j];
 #pragma unroll
         for (int j = 0; j < FJ; ++j) *(u32x4*)(fs + (j * 4 + crow) * SN_P + cpiece) = fq[j];
+        if constexpr (GATHER) {
+            // (rows and pieces that were clamped onto valid ones are written again with the same bytes)
+            int64_t kc = k + cpiece;
+            kc = kc < kend ? kc : kend - 8;
+            if (k < kend) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) *(u32x4*)(g.copy_out + (int64_t)orow[j] * g.ld_copy + kc) = cur[j];
+            }
+        }
         fetch_f(k + 128);
         fetch_x(cur, k + 256);
         const int64_t left = kend - k;           // <= 0 for the idle second half of the last pair
@@ -317,36 +338,37 @@ __global__ void __launch_bounds__(256) small_nt_kernel(SmallNtArgs g) {
     }
 }
 
-template <int TR, int FJ>
+template <int TR, int FJ, bool GATHER = false>
 static int launch_small_nt_one(const SmallNtArgs& g, unsigned blocks, hipStream_t stream) {
     constexpr int NT = (FJ + 7) / 8;
     constexpr size_t lds = (size_t)4 * (32 + NT * 32) * SN_P * 2;
     static std::atomic<bool> attr_set{false};   // the attribute call is idempotent: a race only repeats it
     if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute((const void*)small_nt_kernel<TR, FJ>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        hipError_t e = hipFuncSetAttribute((const void*)small_nt_kernel<TR, FJ, GATHER>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) {
             xq_set_error("small_nt: cannot raise the dynamic LDS limit: %s", hipGetErrorString(e));
             return XQ_ERR_LAUNCH;
         }
         attr_set = true;
     }
-    small_nt_kernel<TR, FJ><<<dim3(blocks), 256, lds, stream>>>(g);
+    small_nt_kernel<TR, FJ, GATHER><<<dim3(blocks), 256, lds, stream>>>(g);
     return XQ_OK;
 }
 
-template <int TR>
+template <int TR, bool GATHER = false>
 static int launch_small_nt_rows(const SmallNtArgs& g, unsigned blocks, hipStream_t stream) {
     switch (g.r_pad) {
-        case 16: return launch_small_nt_one<TR, 4>(g, blocks, stream);
-        case 32: return launch_small_nt_one<TR, 8>(g, blocks, stream);
-        case 48: return launch_small_nt_one<TR, 12>(g, blocks, stream);
-        default: return launch_small_nt_one<TR, 16>(g, blocks, stream);
+        case 16: return launch_small_nt_one<TR, 4, GATHER>(g, blocks, stream);
+        case 32: return launch_small_nt_one<TR, 8, GATHER>(g, blocks, stream);
+        case 48: return launch_small_nt_one<TR, 12, GATHER>(g, blocks, stream);
+        default: return launch_small_nt_one<TR, 16, GATHER>(g, blocks, stream);
     }
 }
 
 int launch_small_nt(const bf16_t* In, int64_t ld_in, int64_t n_rows, int64_t Kc, const bf16_t* F, int r_pad,
                     float scale, bf16_t* T, const int32_t* offsets, const int32_t* tile_offsets,
-                    int32_t num_experts, bool shared_f, hipStream_t stream, int64_t ld_t, bf16_t* T2, int split) {
+                    int32_t num_experts, bool shared_f, hipStream_t stream, int64_t ld_t, bf16_t* T2, int split,
+                    const int32_t* row_map, bf16_t* copy_out, int64_t ld_copy) {
     if (ld_t <= 0) ld_t = r_pad;
     if (T2) XQ_REQUIRE(split > 0 && split < r_pad && ld_t >= split && ld_t >= r_pad - split, "small_nt: bad split of the result columns");
     else XQ_REQUIRE(ld_t >= r_pad, "small_nt: output pitch %lld below r_pad %d", (long long)ld_t, r_pad);
@@ -354,10 +376,14 @@ int launch_small_nt(const bf16_t* In, int64_t ld_in, int64_t n_rows, int64_t Kc,
     XQ_REQUIRE(Kc % 64 == 0, "small_nt: contraction length %lld must be a multiple of 64", (long long)Kc);
     XQ_REQUIRE(ld_in % 8 == 0 && xq_aligned(In, 16) && xq_aligned(F, 16), "small_nt: operands must be 16-byte aligned");
     if (n_rows == 0) return XQ_OK;
+    XQ_REQUIRE(!row_map || (offsets && copy_out && ld_copy % 8 == 0 && ld_copy >= Kc && xq_aligned(copy_out, 16)),
+               "small_nt: gathered rows need the grouped form and a 16-byte aligned copy_out");
     SmallNtArgs g{In, ld_in, n_rows, Kc, F, shared_f ? 0 : (int64_t)r_pad * Kc, r_pad, scale, T, ld_t, T2, split, offsets,
-                  tile_offsets, num_experts};
+                  tile_offsets, num_experts, row_map, copy_out, ld_copy};
     int rc;
-    if (offsets) {
+    if (offsets && row_map) {
+        rc = launch_small_nt_rows<128, true>(g, (unsigned)(xq_cdiv(n_rows, 128) + num_experts), stream);
+    } else if (offsets) {
         rc = launch_small_nt_rows<128>(g, (unsigned)(xq_cdiv(n_rows, 128) + num_experts), stream);
     } else {
         g.f_stride = 0;
