@@ -788,12 +788,21 @@ __global__ void __launch_bounds__(2 * T, 2) gemm_256_kernel(G256Args g) {
             // ---- gate / up epilogue: acc[i][0] is the gate, acc[i][1] the up projection of the same 4 x 4 columns
             // per 32-row band: the two projections as their bf16 outputs (a staged row = 32 gate columns | the same 32
             // up columns) are staged and written, then h from the rounded values goes through the same rows
-            uint32_t bg[4][2] = {}, bu[4][2] = {};       // this lane's 16 bias values of either projection, packed bf16
+            if (g.bias || g.bias2) {      // a pass of its own over the accumulators, so that the common case carries none of it
 #pragma unroll
-            for (int q4 = 0; q4 < 4; ++q4) {
-                const int n = min(cur.n0 + wn * 32 + 8 * q4 + 4 * sfh, g.Nout - 4);
-                if (g.bias) { const u32x2 b = *(const u32x2*)(g.bias + n); bg[q4][0] = b[0]; bg[q4][1] = b[1]; }
-                if (g.bias2) { const u32x2 b = *(const u32x2*)(g.bias2 + n); bu[q4][0] = b[0]; bu[q4][1] = b[1]; }
+                for (int j = 0; j < 2; ++j) {
+                    const bf16_t* bp = j == 0 ? g.bias : g.bias2;
+                    if (bp == nullptr) continue;
+#pragma unroll
+                    for (int q4 = 0; q4 < 4; ++q4) {
+                        const u32x2 b = *(const u32x2*)(bp + min(cur.n0 + wn * 32 + 8 * q4 + 4 * sfh, g.Nout - 4));
+#pragma unroll
+                        for (int i = 0; i < TM; ++i) {
+                            acc[i][j][4 * q4] += __uint_as_float(b[0] << 16); acc[i][j][4 * q4 + 1] += __uint_as_float(b[0] & 0xffff0000u);
+                            acc[i][j][4 * q4 + 2] += __uint_as_float(b[1] << 16); acc[i][j][4 * q4 + 3] += __uint_as_float(b[1] & 0xffff0000u);
+                        }
+                    }
+                }
             }
 #pragma unroll
             for (int i = 0; i < TM; ++i) {
@@ -805,8 +814,6 @@ __global__ void __launch_bounds__(2 * T, 2) gemm_256_kernel(G256Args g) {
                     for (int c = 0; c < 4; ++c) {
                         gv[c] = acc[i][0][4 * q4 + c];
                         uv[c] = acc[i][1][4 * q4 + c];
-                        if (g.bias) gv[c] += __uint_as_float((c & 1) ? (bg[q4][c >> 1] & 0xffff0000u) : (bg[q4][c >> 1] << 16));
-                        if (g.bias2) uv[c] += __uint_as_float((c & 1) ? (bu[q4][c >> 1] & 0xffff0000u) : (bu[q4][c >> 1] << 16));
                         gv[c] = round_bf16(gv[c]);
                         uv[c] = round_bf16(uv[c]);
                         hv[c] = round_bf16(gv[c] * sigmoid_f32(gv[c])) * uv[c];
