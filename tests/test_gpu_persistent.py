@@ -111,3 +111,23 @@ def test_routed_experts_bit_equal(hip_device, tile_policy, both_ways, fmt, E, T,
     p, q = both_ways(step)
     _same(p, q, f"{fmt} experts")
     assert float(p[0].float().abs().max()) > 0
+
+
+def test_more_tiles_than_a_block_may_walk(hip_device, both_ways):
+    """131072 x 16384 outputs are 32768 tiles of 256 x 256: more than 64 per block of a one-block-per-CU grid, so the
+    launcher grows the grid (a block keeps a table of at most 64 tiles).  Forward only, a short contraction."""
+    M, N, K, r = 131072, 16384, 64, 16
+    m, _ = make_dense_module("block_fp8", N, K, r, 32, seed=9, device=hip_device)
+    x = gen((M, K), 1.0, 15, torch.bfloat16).to(hip_device)
+
+    def fwd():
+        with torch.no_grad():
+            y = m(x)
+        # a digest instead of the 4 GiB tensor: two launches that differ anywhere differ here
+        v = y.view(torch.int16).to(torch.int32)
+        w = torch.arange(1, N + 1, device=hip_device, dtype=torch.int32)
+        return ((v * w).sum(dim=1, dtype=torch.int64), y[::4099].clone())
+
+    p, q = both_ways(fwd)
+    _same(p, q, "many tiles")
+    assert float(p[1].float().abs().max()) > 0
