@@ -356,6 +356,11 @@ def main():
     ap.add_argument("--unfused", action="store_true",
                     help="config 1 only: call the three QLoRA linears and the SwiGLU kernel one by one instead of the "
                          "fused MLP entry points (same arithmetic; for A/B timing)")
+    ap.add_argument("--reference-path", action="store_true",
+                    help="config 1 only: run the step the way the reference does -- every weight decoded to bf16 once per step "
+                         "(HIP decode kernel) and kept for the backward, library GEMMs (torch -> hipBLASLt) for the base products, "
+                         "the LoRA branch in fp32 torch ops (qlora/modules/linear.py:378-382), autograd for the backward -- "
+                         "to time that organisation on this GPU beside the fused path; no roofline figure")
     ap.add_argument("--no-graph", action="store_true",
                     help="config 4 only: issue the 32 forwards of a step eagerly instead of replaying them as one HIP graph")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -386,11 +391,19 @@ def main():
 
     from xorl_amd.qlora import qlora_mlp_forward
 
+    def reference_linear(m, inp, w):
+        lora = (inp.float() @ m.lora_A.t().float()) @ m.lora_B.t().float() * m.scaling
+        return torch.nn.functional.linear(inp, w) + lora.to(inp.dtype)
+
     def step():
         x.grad = None
         for p in params:
             p.grad = None
-        if args.unfused:          # the three modules and the SwiGLU kernel one by one
+        if args.reference_path:
+            w = {k: m._dequantize_weight().to(torch.bfloat16) for k, m in mods.items()}
+            h = silu_and_mul(reference_linear(mods["gate"], x, w["gate"]), reference_linear(mods["up"], x, w["up"]))
+            y = reference_linear(mods["down"], h, w["down"])
+        elif args.unfused:        # the three modules and the SwiGLU kernel one by one
             y = mods["down"](silu_and_mul(mods["gate"](x), mods["up"](x)))
         else:                     # the same MLP through the library's fused forward / backward (xq_mlp_fwd / xq_mlp_bwd)
             y = qlora_mlp_forward(mods["gate"], mods["up"], mods["down"], x)
@@ -443,6 +456,9 @@ def main():
                      "launches": n.value, "avg_launch_ms": avg_launch_ms},
         "cpu_baseline": cpu,
     }
+    if args.reference_path:
+        out["path"] = "reference organisation: decode to bf16 + library GEMMs + fp32 LoRA branch + autograd (not the product path)"
+        out["roofline"] = None
     print(json.dumps(out))
 
 
