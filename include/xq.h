@@ -104,6 +104,16 @@ int xq_set_tile_policy(int policy);
  * no counterpart in the reference. */
 int xq_set_persistent_tiles(int enabled);
 
+/* xq_linear_fwd with M <= 16 rows runs as ONE launch where the shape and the LoRA operands allow it (FLAT weight,
+ * K % 512 == 0 for block_fp8 / K % 1024 == 0 for the 4-bit formats, K <= 12288; fp32 factors with r <= 16, r % 4 == 0,
+ * 16-byte aligned): whole weight rows per block, the low-rank intermediate formed once per launch and passed between
+ * blocks through device memory that belongs to the library (tied to the call's workspace pointer: calls with different
+ * workspaces may overlap on a device as before).  enabled = 0 keeps every M <= 64 forward on the two-launch
+ * organisation (K split over blocks + epilogue); results of the two agree to rounding, not bit for bit (different
+ * summation orders).  A process-wide switch for tests and A/B measurements (XQ_SKINNY_ROWS=0 in the environment sets
+ * it at load time); no counterpart in the reference. */
+int xq_set_skinny_one_launch(int enabled);
+
 /* ---- decode ------------------------------------------------------------
  * out[e] = decoded weight of expert e, shape [rows, cols], bf16 or fp32.
  * Replaces int4_dequantize / int4_dequantize_gkn

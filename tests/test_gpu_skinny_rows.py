@@ -1,0 +1,169 @@
+"""GPU: the one-launch organisation of the skinny forward (M <= 16: whole weight rows per block, the low-rank intermediate
+formed once per launch and passed between blocks through device memory of the library) against the oracle and against the
+two-launch organisation on the same inputs.  What could go wrong here beyond arithmetic: a stale intermediate from the
+previous launch (the cases change x between calls that share a workspace), slots that are not restored (many calls in a
+row), ragged last blocks, short K ranges per wave, every format's scale addressing."""
+
+import ctypes
+
+import pytest
+import torch
+
+from oracle import recipe as R
+from tests.util_cases import close, gen, make_dense_module
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-2
+
+
+@pytest.fixture
+def organisations():
+    """run(fn) -> (one-launch result, two-launch result); the switch is restored afterwards."""
+    from xorl_amd import _C
+
+    def run(fn):
+        out = []
+        for enabled in (1, 0):
+            _C.check(_C.lib().xq_set_skinny_one_launch(enabled))
+            out.append(fn())
+        _C.check(_C.lib().xq_set_skinny_one_launch(1))
+        return out
+
+    yield run
+    _C.check(_C.lib().xq_set_skinny_one_launch(1))
+
+
+def _forward(m, x, r=None, bias=True):
+    from xorl_amd.functional import qlora_linear
+
+    r = m.r if r is None else r
+    with torch.no_grad():
+        if r == 0:
+            return qlora_linear(x, m._quant_weight(), None, None, 0, 0.0, m.bias if bias else None)
+        return qlora_linear(x, m._quant_weight(), m.lora_A.detach(), m.lora_B.detach(), r, m.scaling, m.bias if bias else None)
+
+
+@pytest.mark.parametrize("fmt,N,K,r,has_bias", [
+    ("block_fp8", 1024, 4096, 16, False),     # kv: 64 blocks of one row group, 4 su parts
+    ("block_fp8", 12288, 4096, 16, True),     # gate/up: 256 blocks of three row groups
+    ("block_fp8", 4096, 12288, 16, False),    # down: 24 load steps per wave, 12 su parts (M <= 1 only: x must fit LDS)
+    ("block_fp8", 12304, 2048, 8, False),     # ragged last block (769 row groups), short K
+    ("block_fp8", 208, 1024, 4, True),        # two load steps per wave, 13 row groups
+    ("block_fp8", 6144, 5120, 12, False),     # 10 steps of a 16-step kernel, two row groups per block
+    ("int4", 4096, 4096, 16, False),
+    ("int4", 12288, 4096, 16, True),
+    ("int4", 1024, 1024, 16, False),          # one load step per wave
+    ("nf4", 12288, 4096, 16, False),
+    ("nf4", 4096, 5120, 8, True),
+    ("nvfp4", 12288, 4096, 16, False),
+    ("nvfp4", 1040, 2048, 16, True),
+])
+def test_one_launch_vs_oracle_and_two_launch(hip_device, organisations, fmt, N, K, r, has_bias):
+    m, w_ref = make_dense_module(fmt, N, K, r, 2 * r, seed=N + K + r, device=hip_device, bias=has_bias)
+    A, B = m.lora_A.detach().cpu(), m.lora_B.detach().cpu()
+    bias = None if m.bias is None else m.bias.detach().cpu()
+    for M in (1, 3, 8, 16):
+        x = gen((M, K), 1.0, 40 + M, torch.bfloat16)
+        xd = x.to(hip_device)
+        one, two = organisations(lambda: _forward(m, xd))
+        ex = R.linear_fwd_bwd_exact(x, w_ref, A, B, m.scaling, bias=bias)
+        assert one.shape == (M, N) and one.dtype == torch.bfloat16
+        close(one.cpu(), ex["y"], TOL)
+        close(two.cpu(), ex["y"], TOL)
+        close(one.cpu(), two.float().cpu(), TOL)
+        # the same bits from a second call
+        assert torch.equal(_forward(m, xd), one)
+    # no low-rank term
+    x = gen((5, K), 1.0, 77, torch.bfloat16)
+    y0 = _forward(m, x.to(hip_device), r=0)
+    ex0 = R.linear_fwd_bwd_exact(x, w_ref, torch.zeros(1, K), torch.zeros(N, 1), 0.0, bias=bias)
+    close(y0.cpu(), ex0["y"], TOL)
+
+
+def test_low_rank_term_alone_follows_x(hip_device):
+    """Weight codes that decode to zero leave y = s (x A^T) B^T: the term on its own scale, for a sequence of different
+    x through ONE workspace (a stale intermediate of the previous launch would show) and with the low-rank term switched
+    off and on again in between."""
+    from xorl_amd import _C
+    from xorl_amd.functional import _workspace_bytes
+
+    N, K, r = 4096, 4096, 16
+    m, _ = make_dense_module("block_fp8", N, K, r, 32, seed=5, device=hip_device)
+    qw = m._quant_weight()
+    qw.packed.zero_()                           # e4m3 byte 0x00 is +0
+    w = qw.c()
+    A, B = m.lora_A.detach().contiguous(), m.lora_B.detach().contiguous()
+    L = _C.lib()
+    wsb = _workspace_bytes(16, N, K, r)
+    ws = torch.empty(wsb, dtype=torch.uint8, device=hip_device)
+    st = _C.stream_ptr(hip_device)
+    for i, M in enumerate((1, 16, 2, 9, 1, 16)):
+        x = gen((M, K), 1.0, 900 + i, torch.bfloat16).to(hip_device)
+        y = torch.empty(M, N, dtype=torch.bfloat16, device=hip_device)
+        with_term = i != 3
+        _C.check(L.xq_linear_fwd(ctypes.byref(w), x.data_ptr(), K, M, A.data_ptr() if with_term else None,
+                                 B.data_ptr() if with_term else None, _C.XQ_DT_F32, r if with_term else 0, ctypes.c_float(m.scaling),
+                                 None, y.data_ptr(), N, None, ws.data_ptr(), wsb, st))
+        su = x.float() @ A.to(torch.bfloat16).float().t()
+        ref = (m.scaling * su) @ B.float().t() if with_term else torch.zeros(M, N, device=hip_device)
+        close(y.float().cpu(), ref.cpu(), TOL)
+
+
+def test_many_workspaces_and_many_calls(hip_device):
+    """More workspaces than the library holds slots, each used several times: slots change hands, every result stays
+    right and identical to the first."""
+    from xorl_amd import _C
+    from xorl_amd.functional import _workspace_bytes
+
+    N, K, r, M = 1024, 4096, 16, 4
+    m, w_ref = make_dense_module("int4", N, K, r, 32, seed=9, device=hip_device)
+    w = m._quant_weight().c()
+    A, B = m.lora_A.detach().contiguous(), m.lora_B.detach().contiguous()
+    L = _C.lib()
+    wsb = _workspace_bytes(M, N, K, r)
+    x = gen((M, K), 1.0, 31, torch.bfloat16)
+    xd = x.to(hip_device)
+    ex = R.linear_fwd_bwd_exact(x, w_ref, A.cpu(), B.cpu(), m.scaling)
+    wss = [torch.empty(wsb, dtype=torch.uint8, device=hip_device) for _ in range(80)]
+    st = _C.stream_ptr(hip_device)
+    first = None
+    for rep in range(3):
+        for ws in wss:
+            y = torch.empty(M, N, dtype=torch.bfloat16, device=hip_device)
+            _C.check(L.xq_linear_fwd(ctypes.byref(w), xd.data_ptr(), K, M, A.data_ptr(), B.data_ptr(), _C.XQ_DT_F32, r,
+                                     ctypes.c_float(m.scaling), None, y.data_ptr(), N, None, ws.data_ptr(), wsb, st))
+            if first is None:
+                first = y
+                close(y.cpu(), ex["y"], TOL)
+            else:
+                assert torch.equal(y, first)
+
+
+def test_one_launch_under_hip_graph_with_changing_input(hip_device):
+    """A captured forward replays against new contents of its input buffer: every replay must use the intermediate of
+    ITS input (the slot is restored inside each launch), and equal the eager result bit for bit."""
+    m, _ = make_dense_module("block_fp8", 4096, 4096, 16, 32, seed=3, device=hip_device)
+    xbuf = gen((8, 4096), 1.0, 1, torch.bfloat16).to(hip_device)
+
+    def step():
+        with torch.no_grad():
+            return m(xbuf)
+
+    step()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = step()
+    for rep in range(4):
+        xbuf.copy_(gen((8, 4096), 1.0, 10 + rep, torch.bfloat16).to(hip_device))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = out.clone()
+        eager = step()
+        torch.cuda.synchronize()
+        assert torch.equal(got, eager), rep

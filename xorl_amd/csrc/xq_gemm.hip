@@ -6,6 +6,7 @@
 #include <stdlib.h>
 #include <mutex>
 #include "xq_lora.h"
+#include "xq_skinny.h"
 
 namespace xq {
 
@@ -376,6 +377,11 @@ using namespace xq;
 extern "C" int xq_set_tile_policy(int policy) {
     XQ_REQUIRE(policy >= 0 && policy <= 3, "xq_set_tile_policy: policy %d not in {0, 1, 2, 3}", policy);
     g_tile_policy = policy;
+    return XQ_OK;
+}
+
+extern "C" int xq_set_skinny_one_launch(int enabled) {
+    set_skinny_rows(enabled ? 1 : 0);
     return XQ_OK;
 }
 

@@ -1,0 +1,56 @@
+// Shared by the two organisations of the skinny-M forward (xq_skinny.hip: K split over blocks, two launches;
+// xq_skinny_rows.hip: whole rows per block, one launch).
+#pragma once
+#include "xq_common.h"
+
+namespace xq {
+
+// decode 8 consecutive K elements (one MFMA operand) of this lane's row
+template <int FMT>
+__device__ __forceinline__ bf16x8 decode8(uint32_t w0, uint32_t w1, float s0, float s1, const float* nf4_lds = nullptr) {
+    uint32_t o[4];
+    if (FMT == XQ_FMT_FP8) {
+        f32x2 a = e4m3x2_to_f32(w0, false), b = e4m3x2_to_f32(w0, true);
+        f32x2 c = e4m3x2_to_f32(w1, false), d = e4m3x2_to_f32(w1, true);
+        o[0] = pack_bf16x2(a[0] * s0, a[1] * s0);
+        o[1] = pack_bf16x2(b[0] * s0, b[1] * s0);
+        o[2] = pack_bf16x2(c[0] * s0, c[1] * s0);
+        o[3] = pack_bf16x2(d[0] * s0, d[1] * s0);
+    } else if (FMT == XQ_FMT_INT4) {
+        // w0 holds 8 nibbles; fma(nib, s, -8s) == fl((nib-8)*s) up to the sign of zero
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            float lo = __builtin_fmaf((float)((w0 >> (8 * i)) & 0xfu), s0, s1);
+            float hi = __builtin_fmaf((float)((w0 >> (8 * i + 4)) & 0xfu), s0, s1);
+            o[i] = pack_bf16x2(lo, hi);
+        }
+    } else if (FMT == XQ_FMT_NF4) {
+        // level[nib] * scale, the levels read from a 64-byte copy of the table in LDS (conflict free for any mix of codes)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            o[i] = pack_bf16x2(nf4_lds[(w0 >> (8 * i)) & 0xfu] * s0, nf4_lds[(w0 >> (8 * i + 4)) & 0xfu] * s0);
+    } else {
+        // v_cvt_scalef32_pk_f32_fp4 with scale 1.0 yields the exact e2m1 values of byte i (low nibble first)
+        f32x2 v0 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w0, 1.0f, 0);
+        f32x2 v1 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w0, 1.0f, 1);
+        f32x2 v2 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w0, 1.0f, 2);
+        f32x2 v3 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w0, 1.0f, 3);
+        o[0] = pack_bf16x2(v0[0] * s0, v0[1] * s0);
+        o[1] = pack_bf16x2(v1[0] * s0, v1[1] * s0);
+        o[2] = pack_bf16x2(v2[0] * s0, v2[1] * s0);
+        o[3] = pack_bf16x2(v3[0] * s0, v3[1] * s0);
+    }
+    u32x4 r = {o[0], o[1], o[2], o[3]};
+    return __builtin_bit_cast(bf16x8, r);
+}
+
+void set_skinny_rows(int enabled);
+
+// ---- one-launch organisation (xq_skinny_rows.hip)
+// true when the shape, format and LoRA operands fit it; the caller falls back to the split organisation otherwise
+bool skinny_rows_supported(const xq_weight* w, int64_t M, const void* lora_A, const void* lora_B, int lora_dtype, int r);
+// `slot_key` names the caller's scratch (its workspace pointer): calls with different keys may overlap on a device
+int launch_skinny_rows(const xq_weight* w, const bf16_t* x, int64_t ldx, int64_t M, const void* lora_A, const void* lora_B, int r,
+                       float scaling, const bf16_t* bias, bf16_t* y, int64_t ldy, const void* slot_key, hipStream_t stream);
+
+}  // namespace xq

@@ -22,8 +22,11 @@
 // Measured per forward on an MI355X, launches back to back (block_fp8, r = 16): 4096->12288 (48 MiB) 15.5 us
 // at M = 1, 22 us at M = 32, 35 us at M = 64; 4096->1024 (4 MiB) 7.3 us at M = 1.  A kernel that only reads
 // the 48 MiB takes 8-9 us.
+#include <stdlib.h>
+
 #include "xq_common.h"
 #include "xq_lora.h"
+#include "xq_skinny.h"
 
 namespace xq {
 
@@ -56,45 +59,6 @@ struct SkinnyEpiArgs {
     bf16_t* y;
     int64_t ldy;
 };
-
-// decode 8 consecutive K elements (one MFMA operand) of this lane's row
-template <int FMT>
-__device__ __forceinline__ bf16x8 decode8(uint32_t w0, uint32_t w1, float s0, float s1, const float* nf4_lds = nullptr) {
-    uint32_t o[4];
-    if (FMT == XQ_FMT_FP8) {
-        f32x2 a = e4m3x2_to_f32(w0, false), b = e4m3x2_to_f32(w0, true);
-        f32x2 c = e4m3x2_to_f32(w1, false), d = e4m3x2_to_f32(w1, true);
-        o[0] = pack_bf16x2(a[0] * s0, a[1] * s0);
-        o[1] = pack_bf16x2(b[0] * s0, b[1] * s0);
-        o[2] = pack_bf16x2(c[0] * s0, c[1] * s0);
-        o[3] = pack_bf16x2(d[0] * s0, d[1] * s0);
-    } else if (FMT == XQ_FMT_INT4) {
-        // w0 holds 8 nibbles; fma(nib, s, -8s) == fl((nib-8)*s) up to the sign of zero
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            float lo = __builtin_fmaf((float)((w0 >> (8 * i)) & 0xfu), s0, s1);
-            float hi = __builtin_fmaf((float)((w0 >> (8 * i + 4)) & 0xfu), s0, s1);
-            o[i] = pack_bf16x2(lo, hi);
-        }
-    } else if (FMT == XQ_FMT_NF4) {
-        // level[nib] * scale, the levels read from a 64-byte copy of the table in LDS (conflict free for any mix of codes)
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-            o[i] = pack_bf16x2(nf4_lds[(w0 >> (8 * i)) & 0xfu] * s0, nf4_lds[(w0 >> (8 * i + 4)) & 0xfu] * s0);
-    } else {
-        // v_cvt_scalef32_pk_f32_fp4 with scale 1.0 yields the exact e2m1 values of byte i (low nibble first)
-        f32x2 v0 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w0, 1.0f, 0);
-        f32x2 v1 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w0, 1.0f, 1);
-        f32x2 v2 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w0, 1.0f, 2);
-        f32x2 v3 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w0, 1.0f, 3);
-        o[0] = pack_bf16x2(v0[0] * s0, v0[1] * s0);
-        o[1] = pack_bf16x2(v1[0] * s0, v1[1] * s0);
-        o[2] = pack_bf16x2(v2[0] * s0, v2[1] * s0);
-        o[3] = pack_bf16x2(v3[0] * s0, v3[1] * s0);
-    }
-    u32x4 r = {o[0], o[1], o[2], o[3]};
-    return __builtin_bit_cast(bf16x8, r);
-}
 
 // 8 consecutive LoRA factor entries (fp32 or bf16 storage) -> one MFMA operand; entries at or
 // beyond `limit` (counted from the first) are zero
@@ -578,6 +542,11 @@ static int launch_skinny_split(const xq_weight* w, const bf16_t* x, int64_t ldx,
     return XQ_OK;
 }
 
+// XQ_SKINNY_ROWS=0 (or xq_set_skinny_rows(0)) keeps every skinny forward on the two-launch organisation: a process-wide
+// test switch, to be set while no other thread is inside the library
+static int g_skinny_rows = [] { const char* e = getenv("XQ_SKINNY_ROWS"); return e ? atoi(e) : 1; }();
+void set_skinny_rows(int enabled) { g_skinny_rows = enabled; }
+
 int launch_skinny(const xq_weight* w, const bf16_t* x, int64_t ldx, int64_t M, const void* lora_A, const void* lora_B,
                   int lora_dtype, int r, float scaling, const bf16_t* bias, bf16_t* y, int64_t ldy, void* workspace,
                   int64_t workspace_bytes, hipStream_t stream) {
@@ -592,7 +561,12 @@ int launch_skinny(const xq_weight* w, const bf16_t* x, int64_t ldx, int64_t M, c
     // region is the whole forward (both launches)
     const double wbytes = (double)xq_packed_bytes_per_expert(w) + (double)xq_scale_bytes_per_expert(w);
     const bool timed = xq_profile_mark_begin(stream, wbytes + 2.0 * M * K + 2.0 * M * N + 4.0 * r * (K + N));
-    const int rc = launch_skinny_split(w, x, ldx, M, lora_A, lora_B, lora_dtype, r, rp, scaling, bias, y, ldy, workspace, stream);
+    // M <= 16: one launch, whole rows per block, where the shape and the LoRA operands fit it and a slot is free
+    int rc = XQ_ERR_UNSUPPORTED;
+    if (g_skinny_rows && skinny_rows_supported(w, M, lora_A, lora_B, lora_dtype, r))
+        rc = launch_skinny_rows(w, x, ldx, M, lora_A, lora_B, r, scaling, bias, y, ldy, workspace, stream);
+    if (rc == XQ_ERR_UNSUPPORTED)
+        rc = launch_skinny_split(w, x, ldx, M, lora_A, lora_B, lora_dtype, r, rp, scaling, bias, y, ldy, workspace, stream);
     if (timed) xq_profile_mark_end(stream);
     if (rc) return rc;
     XQ_CHECK_LAUNCH("skinny forward");

@@ -1,0 +1,622 @@
+// Skinny-M forward for M <= 16 in ONE launch (the decode regime: a handful of tokens against a large packed weight).
+//
+//   y[M, N] = x[M, K] . deq(W)^T + bias + s * (x . A^T) . B^T          (W FLAT [N, K])
+//
+// A block owns 16 G weight rows over the WHOLE of K: its 8 waves split K eight ways, sum their 16 x 16 tiles through LDS
+// and write the outputs themselves -- no fp32 partial tiles in memory, no second launch.  All of a wave's loads are
+// issued up front and unconditionally (clamped, masked), the x slice first (it reaches LDS while the weight bytes
+// stream), and every weight byte is read once, decoded in registers to the exact bf16 value of the reference decoder
+// and fed to v_mfma_f32_16x16x32_bf16 against x fragments (lane (row, quarter) holds 16 or 32 consecutive codes of its
+// row; the K order inside an MFMA is whatever the loads deliver, the x fragments follow the same order).
+//
+// The low-rank intermediate su = x . A^T [M, r] is needed whole by every block but costs r x K factor bytes to form, more
+// than a block's share of the weight.  It is formed once per launch: in each of the first K / 512 blocks the four waves
+// that are last in the load queue contract 512 elements of K before they turn to their weight rows, and publish the
+// 256 sums to a slot in device memory; wave 0 of
+// every block, which is the first to finish its part of the weight stream, collects the parts while the other waves are
+// still streaming.  Nothing on that path waits for an atomic's return value or for an ordering between stores:
+//  * the slot holds a launch count `gen`; every block reads it first thing (one load among its others);
+//  * a published entry is the 8-byte pair (sum, gen + 1), stored whole; a collector takes an entry when its tag is
+//    gen + 1, so what earlier launches left in the slot never passes for this launch's sums and nothing is cleared;
+//  * `gen` moves on once per launch, after every block has read it: each block adds one to `started` when its own read
+//    has returned (no return value asked for), and the last block of the grid, which reads `started` along with the
+//    parts, stores gen + 1 and started = 0 when it finds the whole grid there (it looks again if not).  Both words
+//    exist in 32 copies on different memory lines (block b reads and counts in copy b % 32; the last block sums and
+//    rewrites them all): hundreds of accesses to one location that bypass the caches would take microseconds.
+// Slot accesses are device-scope atomics (they bypass the per-XCD L2s).  Blocks that publish never wait, and they are
+// the first the dispatcher places, so the collectors' wait ends; a limit bounds every wait all the same and turns the
+// block's outputs into NaN.  Sums run in fixed orders (waves ascending, parts ascending): results are identical from
+// call to call.
+//
+// Measured on an MI355X, launches back to back (block_fp8, r = 16, M = 1): 4096->12288 (48 MiB) ~12 us against 15 us for
+// the two-launch organisation, 4096->1024 ~6 us against 7.7 us.
+#include <atomic>
+#include <mutex>
+
+#include "xq_common.h"
+#include "xq_lora.h"
+#include "xq_skinny.h"
+
+namespace xq {
+
+constexpr int kSuPartK = 512;                   // K elements per su part
+constexpr int kSuMaxParts = 32;                 // K <= 16384 with a low-rank term
+constexpr int kSlotCtl = kSuMaxParts * 256 * 2; // word index of the control words
+constexpr int kCtlCopies = 32;                  // `gen` and `started` exist 32 times, 128 bytes apart: block b uses copy b % 32,
+constexpr int kCtlStride = 32;                  // so that a launch's 256 blocks do not queue on one memory location
+constexpr int kSlotWords = kSlotCtl + 2 * kCtlCopies * kCtlStride;   // [parts][256] pairs (sum bits, tag), gen copies, started copies
+constexpr int kSlots = 64;
+constexpr int kRowsSpinLimit = 1 << 20;
+
+struct SkinnyRowsArgs {
+    const bf16_t* x;
+    int64_t ldx;
+    int32_t M, N, K;
+    const uint8_t* packed;
+    const uint8_t* scales;
+    const float* global_scale;
+    int32_t gshift, scale_dtype;   // int4: log2(group)
+    const float* lora_A;           // [r, K] fp32
+    const float* lora_B;           // [N, r] fp32
+    int32_t r;
+    float su_scale;
+    const bf16_t* bias;
+    bf16_t* y;
+    int64_t ldy;
+    int32_t xpitch, slab;          // bytes: LDS row pitch of a wave's x slice, bytes of a wave's LDS area
+    int32_t nsu;                   // su parts (K / 512), 0 without a low-rank term
+    uint32_t* slot;                // [nsu][256] published (sum, tag) pairs, then the copies of gen and of started
+    int32_t spin_limit;
+};
+
+// FMT: weight format; G: 16-row groups per block; NJ: most load steps per wave (a step is one 16-byte load per lane:
+// 64 elements of K per row for fp8, 128 for the 4-bit formats); MR: bound on M (x rows kept in registers on their way
+// to LDS)
+template <int FMT, int G, int NJ, int MR>
+__global__ void __launch_bounds__(512, 1) skinny_rows_kernel(SkinnyRowsArgs g) {
+    constexpr bool F8 = FMT == XQ_FMT_FP8;
+    constexpr int EPS = F8 ? 64 : 128;                 // K elements of a row per load step
+    constexpr int MPS = EPS / 32;                      // MFMAs per step and row group
+    constexpr int EB = F8 ? 1 : 2;                     // elements per byte
+    constexpr int XC = (NJ * EPS + 511) / 512;         // 1 KB pieces of an x row slice
+    constexpr int NSC = FMT == XQ_FMT_NVFP4 ? 2 : 1;   // scale registers per load
+    // every argument in scalar registers after one round trip (lazily placed argument loads cost a round trip each)
+    asm volatile("" ::"s"(g.x), "s"(g.ldx), "s"(g.M), "s"(g.N), "s"(g.K), "s"(g.packed), "s"(g.scales), "s"(g.global_scale),
+                 "s"(g.gshift), "s"(g.scale_dtype), "s"(g.lora_A), "s"(g.lora_B), "s"(g.r), "s"(g.su_scale), "s"(g.bias), "s"(g.y),
+                 "s"(g.ldy), "s"(g.xpitch), "s"(g.slab), "s"(g.nsu), "s"(g.slot), "s"(g.spin_limit));
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int rn = lane & 15, kq = lane >> 4;
+    const int ks = g.K >> 3;                    // K elements per wave
+    const int k0 = wave * ks;
+    const int nj = ks / EPS;                    // load steps of this launch, 1 .. NJ
+    const int n0 = blockIdx.x * (16 * G);
+    const int XP = g.xpitch;
+    unsigned char* slab = smem + wave * g.slab;
+    float* su_tot = (float*)(smem + 8 * g.slab);           // [16 m][16 j], then a flag
+    float* b_tile = su_tot + 272;                           // [64 rows][20]: the block's rows of B, 16 bytes apart in banks
+    float* su_red = b_tile + 64 * 20;                       // [4 waves][256]: the tiles of an su part
+    int* su_flag = (int*)(su_red + 4 * 256);                // [0 .. 3]: wave 4 + w has written its tile; [4]: wave 4 is done with `gen`
+    const bool lora = g.nsu > 0;
+    const bool su_block = (int)blockIdx.x < g.nsu;          // nsu <= gridDim.x (checked on the host)
+    // LDS traffic of the block is ordered by this barrier; __syncthreads() would also wait for every load in flight
+    auto lds_barrier = [&]() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+
+    if (su_block) {
+        // nothing is in flight yet: this barrier costs nothing, and LDS does not start out zero
+        if (tid < 8) su_flag[tid] = 0;
+        lds_barrier();
+    }
+
+    // ---- the slot's launch count.  A block that forms an su part has its publishing wave ask for it first of all (the part
+    // carries it as its tag); everywhere wave 0 asks for it, past the caches, behind its weights (needed when it collects;
+    // loads return in order and this one is slow, so it must not sit in front of them).
+    uint32_t gen = 0;
+    uint32_t* ctl = g.slot + kSlotCtl + (blockIdx.x % kCtlCopies) * kCtlStride;      // this block's copy of gen; started: + kCtlCopies * kCtlStride
+
+    // the operand tie keeps the compiler from moving the add ahead of the point where `gen` is in its register
+    auto count_block = [&]() {
+        uint32_t one = 1u;
+        asm volatile("" : "+v"(one) : "v"(gen));
+        __hip_atomic_fetch_add(ctl + kCtlCopies * kCtlStride, one, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    };
+
+    // ---- a block that forms an su part does so with its waves 4 .. 7: behind the others in the load queue, they would
+    // otherwise sit waiting to issue their weight loads.  Wave 4 + w contracts elements 128 w .. of the part in four
+    // MFMAs, lane (rank rn, quarter kq) holding 8 consecutive elements per MFMA; factor rows and x fragments are its
+    // first loads.
+    const bool su_wave = su_block && wave >= 4;
+    u32x4 fa0[4], fa1[4];
+    bf16x8 fx[4];
+    if (su_wave) {
+        __builtin_amdgcn_s_setprio(3);          // ahead of the other waves' loads: everyone's finish waits for these sums
+        // the publisher tags the sums with it.  This read may come from the XCD's L2: no line of the slot can be there from
+        // before the launch (caches are invalidated between kernels, or results could not pass from one kernel to the
+        // next), and within a launch the word changes only after every block has read it.  A read past the caches takes
+        // microseconds here, and every block's finish waits for the sums.  (Were the value stale after all, the tag
+        // would not be the one the collectors look for: they would give up and write NaN, never take old sums.)
+        if (wave == 4) gen = __hip_atomic_load(ctl, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        const int kb = blockIdx.x * kSuPartK + (wave - 4) * 128 + kq * 8;
+        const float* ap = g.lora_A + (int64_t)(rn < g.r ? rn : 0) * g.K + kb;
+        const bf16_t* xp = g.x + (int64_t)(rn < g.M ? rn : g.M - 1) * g.ldx + kb;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            fa0[u] = *(const u32x4*)(ap + u * 32);
+            fa1[u] = *(const u32x4*)(ap + u * 32 + 4);
+            fx[u] = *(const bf16x8*)(xp + u * 32);
+        }
+        __builtin_amdgcn_s_setprio(0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- x slice [M][ks] of this wave: a load instruction covers 1 KB of one row; rows past M and pieces past the slice
+    // are clamped (loaded, never stored)
+    u32x4 xr[MR][XC];
+    const int ppr = ks >> 3;                    // 16-byte pieces per row of the slice
+#pragma unroll
+    for (int i = 0; i < MR; ++i)
+#pragma unroll
+        for (int c = 0; c < XC; ++c) {
+            const int piece = c * 64 + lane < ppr ? c * 64 + lane : ppr - 1;
+            xr[i][c] = *(const u32x4*)(g.x + (int64_t)(i < g.M ? i : g.M - 1) * g.ldx + k0 + piece * 8);
+        }
+    __builtin_amdgcn_sched_barrier(0);
+
+
+    // ---- su part, before these waves' weight loads are requested: D[j][m] of each wave, the four tiles summed through LDS in
+    // wave order by wave 4, published.  The waves meet through flags in LDS, not a barrier.
+    if (su_wave) {
+        f32x4 su = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            u32x4 t = {pack_bf16x2(__uint_as_float(fa0[u][0]), __uint_as_float(fa0[u][1])), pack_bf16x2(__uint_as_float(fa0[u][2]), __uint_as_float(fa0[u][3])),
+                       pack_bf16x2(__uint_as_float(fa1[u][0]), __uint_as_float(fa1[u][1])), pack_bf16x2(__uint_as_float(fa1[u][2]), __uint_as_float(fa1[u][3]))};
+            if (rn >= g.r) t = u32x4{0, 0, 0, 0};
+            su = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, t), fx[u], su, 0, 0, 0);
+        }
+#pragma unroll
+        for (int q = 0; q < 4; ++q) su_red[(wave - 4) * 256 + q * 64 + lane] = su[q];
+        // the flag goes behind the tile: LDS operations of one wave execute in order.  (A release / acquire pair of the
+        // language would also wait for every global load these waves have in flight -- their x slices.)
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        if (lane == 0) __hip_atomic_store(su_flag + wave - 4, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        if (wave == 4) {
+            int spins = 0;
+            bool all;
+            do {
+                all = lane >= 4 || __hip_atomic_load(su_flag + (lane & 3), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) != 0;
+                all = __all(all);
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                if (!all) {
+                    __builtin_amdgcn_s_sleep(2);
+                    ++spins;
+                }
+            } while (!all && spins < g.spin_limit);
+            // (a wait that hit the limit leaves the part unpublished: the collectors then hit theirs and write NaN)
+            if (all) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    float s = 0.0f;
+#pragma unroll
+                    for (int ww = 0; ww < 4; ++ww) s += su_red[ww * 256 + q * 64 + lane];
+                    __hip_atomic_store((uint64_t*)g.slot + blockIdx.x * 256 + q * 64 + lane, ((uint64_t)(gen + 1) << 32) | __float_as_uint(s),
+                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+            }
+            // wave 0 counts the block in once it has read `gen` itself, and not before this wave has
+            if (lane == 0) __hip_atomic_store(su_flag + 4, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- the block's weight rows, this wave's K range: step j gives lane (row rn, quarter kq) the 16 bytes at element
+    // EPS j + (EPS / 4) kq of its row's slice.  With 16 x rows in registers the last third of the steps is requested once
+    // the x slice has been written to LDS.
+    constexpr int J1 = MR > 8 ? (2 * NJ + 2) / 3 : NJ;
+    u32x4 w[NJ][G];
+    uint32_t sc[NJ][G][NSC];
+    const uint8_t* wp[G];
+    int64_t erow[G];                            // element index of (row, k0 + (EPS / 4) kq), for the per-row scales
+#pragma unroll
+    for (int gi = 0; gi < G; ++gi) {
+        int n = n0 + gi * 16 + rn;
+        n = n < g.N ? n : g.N - 1;
+        erow[gi] = (int64_t)n * g.K + k0 + kq * (EPS / 4);
+        wp[gi] = g.packed + ((int64_t)n * g.K + k0) / EB + kq * 16;
+    }
+    const int scols = (g.K + 127) >> 7;
+    auto load_w = [&](int ja, int jb) {
+#pragma unroll
+        for (int j = ja; j < jb; ++j) {
+            const int jc = j < nj ? j : nj - 1;
+#pragma unroll
+            for (int gi = 0; gi < G; ++gi) {
+                w[j][gi] = *(const u32x4*)(wp[gi] + jc * 64);
+                if (FMT == XQ_FMT_FP8) {
+                    // one scale per 128 x 128 block: the same for the 16 rows of a group and the 64 elements of a step
+                    const int nb = n0 + gi * 16 < g.N ? n0 + gi * 16 : g.N - 16;
+                    sc[j][gi][0] = ((const __attribute__((address_space(4))) uint32_t*)g.scales)[(nb >> 7) * scols + ((k0 + jc * 64) >> 7)];
+                } else if (FMT == XQ_FMT_INT4) {
+                    const int64_t si = (erow[gi] + jc * EPS) >> g.gshift;      // group % 32 == 0: one scale per load
+                    sc[j][gi][0] = g.scale_dtype == XQ_SCALE_F32 ? ((const uint32_t*)g.scales)[si] : (uint32_t)((const uint16_t*)g.scales)[si] << 16;
+                } else if (FMT == XQ_FMT_NF4) {
+                    sc[j][gi][0] = ((const uint32_t*)g.scales)[(erow[gi] + jc * EPS) >> 6];       // fp32, group 64
+                } else {
+                    const int64_t si = (erow[gi] + jc * EPS) >> 4;                                 // two blocks of 16 per load
+                    if (g.scale_dtype == XQ_SCALE_E4M3) {
+                        sc[j][gi][0] = *(const uint16_t*)(g.scales + si);
+                        sc[j][gi][1] = 0;
+                    } else {
+                        const u32x2 t = *(const u32x2*)((const uint32_t*)g.scales + si);
+                        sc[j][gi][0] = t[0];
+                        sc[j][gi][1] = t[1];
+                    }
+                }
+            }
+        }
+    };
+    load_w(0, J1);
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- x slice -> LDS (the wave's own area; LDS operations of one wave execute in order, no barrier)
+#pragma unroll
+    for (int i = 0; i < MR; ++i)
+#pragma unroll
+        for (int c = 0; c < XC; ++c)
+            if (i < g.M && c * 64 + lane < ppr) *(u32x4*)(slab + i * XP + (c * 64 + lane) * 16) = xr[i][c];
+    float* nf4_lds = (float*)(slab + g.slab - 64);          // 16 levels at the end of the wave's area
+    if (FMT == XQ_FMT_NF4 && lane < 16) nf4_lds[lane] = kNf4Level[lane];
+    __builtin_amdgcn_sched_barrier(0);
+    load_w(J1, NJ);
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- what the finish needs, requested behind the weights: the block's rows of B (thread t < 256: row t / 4, ranks
+    // 4 (t % 4) ..), the bias of column tid % 64
+    const int nl = tid & 63;
+    f32x4 bq = {0.0f, 0.0f, 0.0f, 0.0f};
+    const int brow = tid >> 2, bpiece = tid & 3;
+    const bool bvalid = lora && tid < 256 && brow < 16 * G && n0 + brow < g.N && 4 * bpiece < g.r;
+    {
+        const int64_t bn = n0 + brow < g.N ? n0 + brow : g.N - 1;
+        const float* bp = lora ? g.lora_B + bn * g.r + (4 * bpiece < g.r ? 4 * bpiece : 0) : (const float*)g.x;
+        bq = *(const f32x4*)bp;
+    }
+    const int nfin = (nl < 16 * G && n0 + nl < g.N) ? n0 + nl : g.N - 1;
+    const float bias_v = bf16_to_f32((g.bias ? g.bias : g.x)[g.bias ? nfin : 0]);
+    __builtin_amdgcn_sched_barrier(0);
+    if (lora && wave == 0) gen = __hip_atomic_load(ctl, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- decode + multiply, D[n][m] += deq(W)[n][k] x[m][k], in the order the weights arrive
+    const float gsc = FMT == XQ_FMT_NVFP4 ? g.global_scale[0] : 1.0f;
+    const int xm = rn < g.M ? rn : g.M - 1;
+    const unsigned char* xrow = slab + xm * XP + kq * (EPS / 2);
+    f32x4 acc[G];
+#pragma unroll
+    for (int gi = 0; gi < G; ++gi) acc[gi] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+        if (j < nj) {      // wave-uniform
+            bf16x8 xf[MPS];
+#pragma unroll
+            for (int c = 0; c < MPS; ++c) xf[c] = *(const bf16x8*)(xrow + j * (EPS * 2) + c * 16);
+#pragma unroll
+            for (int gi = 0; gi < G; ++gi) {
+#pragma unroll
+                for (int c = 0; c < MPS; ++c) {
+                    bf16x8 wf;
+                    if (FMT == XQ_FMT_FP8) {
+                        wf = decode8<FMT>(w[j][gi][2 * c], w[j][gi][2 * c + 1], __uint_as_float(sc[j][gi][0]), 0.0f);
+                    } else if (FMT == XQ_FMT_INT4) {
+                        const float sv = __uint_as_float(sc[j][gi][0]);
+                        wf = decode8<FMT>(w[j][gi][c], 0u, sv, -8.0f * sv);
+                    } else if (FMT == XQ_FMT_NF4) {
+                        wf = decode8<FMT>(w[j][gi][c], 0u, __uint_as_float(sc[j][gi][0]), 0.0f, nf4_lds);
+                    } else {
+                        float sv;   // block c / 2 of the load's two
+                        if (g.scale_dtype == XQ_SCALE_E4M3) sv = e4m3_to_f32((uint8_t)(sc[j][gi][0] >> (8 * (c >> 1))));
+                        else sv = __uint_as_float(sc[j][gi][c >> 1]);
+                        wf = decode8<FMT>(w[j][gi][c], 0u, sv * gsc, 0.0f);
+                    }
+                    acc[gi] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, xf[c], acc[gi], 0, 0, 0);
+                }
+            }
+        }
+    }
+
+    // this block may be counted once its reads of `gen` have returned: wave 0's has, like the weights requested before it;
+    // in a block that forms an su part wave 4 has read it too and says so when it has published
+    if (lora && wave == 0) {
+        if (su_block) {
+            int spins = 0;
+            while (__hip_atomic_load(su_flag + 4, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) == 0 && spins < g.spin_limit) {
+                __builtin_amdgcn_s_sleep(2);
+                ++spins;
+            }
+        }
+        if (lane == 0) count_block();
+    }
+
+    // ---- the wave's sums -> its own LDS area (its x slice is no longer needed): tile gi, register q, lane; B rows -> LDS
+    float* part = (float*)slab;
+#pragma unroll
+    for (int gi = 0; gi < G; ++gi)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) part[gi * 256 + q * 64 + lane] = acc[gi][q];
+    if (tid < 256) *(f32x4*)(b_tile + brow * 20 + bpiece * 4) = bvalid ? bq : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+
+    // ---- wave 0 (its loads were requested first, so it gets here first) collects the su parts while the other waves are
+    // still streaming: entry q * 64 + l of a part is su[j = 4 (l >> 4) + q][m = l & 15]
+    if (lora && wave == 0) {
+        const bool closer = blockIdx.x == gridDim.x - 1;      // this block moves the launch count on
+        float s[4];
+        int spins = 0;
+        bool missing, open = closer;
+        do {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) s[q] = 0.0f;
+            missing = false;
+            uint32_t started = 0;       // lane l < 32: copy l
+            if (open && lane < kCtlCopies)
+                started = __hip_atomic_load(g.slot + kSlotCtl + (kCtlCopies + lane) * kCtlStride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            for (int p0 = 0; p0 < g.nsu; p0 += 8) {
+                // The first look goes through the caches: the 32 blocks of an XCD then share one fetch of each line, where
+                // 256 blocks' reads past the caches of the same few lines would queue at their memory channels for
+                // microseconds and hold up the weight stream.  What a cached look returns is still judged entry by
+                // entry by its tag; a second look is needed only if this one came before the parts, and goes to memory.
+                uint64_t t[8][4];
+                if (spins == 0) {
+#pragma unroll
+                    for (int u = 0; u < 8; ++u)
+#pragma unroll
+                        for (int q = 0; q < 4; ++q)
+                            t[u][q] = __hip_atomic_load((const uint64_t*)g.slot + (p0 + u < g.nsu ? p0 + u : g.nsu - 1) * 256 + q * 64 + lane,
+                                                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                } else {
+#pragma unroll
+                    for (int u = 0; u < 8; ++u)
+#pragma unroll
+                        for (int q = 0; q < 4; ++q)
+                            t[u][q] = __hip_atomic_load((const uint64_t*)g.slot + (p0 + u < g.nsu ? p0 + u : g.nsu - 1) * 256 + q * 64 + lane,
+                                                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+#pragma unroll
+                for (int u = 0; u < 8; ++u)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        missing |= (uint32_t)(t[u][q] >> 32) != gen + 1;
+                        s[q] += p0 + u < g.nsu ? __uint_as_float((uint32_t)t[u][q]) : 0.0f;
+                    }
+            }
+            missing = __any(missing);
+            if (open) {
+#pragma unroll
+                for (int d = 32; d >= 1; d >>= 1) started += __shfl_xor(started, d, 64);
+                if (started == gridDim.x) {
+                    // every block has read `gen`: the next launch counts from gen + 1
+                    if (lane < kCtlCopies) {
+                        __hip_atomic_store(g.slot + kSlotCtl + lane * kCtlStride, gen + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        __hip_atomic_store(g.slot + kSlotCtl + (kCtlCopies + lane) * kCtlStride, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
+                    open = false;
+                }
+            }
+            if (missing || open) {
+                __builtin_amdgcn_s_sleep(8);
+                ++spins;
+            }
+        } while ((missing || open) && spins < g.spin_limit);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int j = 4 * (lane >> 4) + q, m = lane & 15;
+            su_tot[m * 16 + j] = j < g.r ? s[q] * g.su_scale : 0.0f;
+        }
+        if (lane == 0) ((int*)su_tot)[256] = (missing || open) ? 0 : 1;
+    }
+    lds_barrier();
+
+    // ---- outputs: thread (nl, mg) finishes y[mg][n0 + nl] and y[mg + 8][n0 + nl]: the eight waves' sums in wave order, the
+    // low-rank term rank by rank in fp32, the bias, one rounding
+    const int mg = tid >> 6;
+    const bool nvalid = nl < 16 * G && n0 + nl < g.N;
+    const int gi_f = nl >> 4, nloc = nl & 15;
+    const bool ok = !lora || ((const int*)su_tot)[256] != 0;
+    f32x4 bv[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) bv[q] = *(const f32x4*)(b_tile + nl * 20 + 4 * q);
+#pragma unroll
+    for (int mm = 0; mm < 2; ++mm) {
+        const int m = mg + 8 * mm;
+        if (m < g.M && nvalid) {
+            // D[nloc][m] of a wave's tile sits in register nloc & 3 of lane 16 (nloc >> 2) + m
+            const int idx = gi_f * 256 + (nloc & 3) * 64 + (nloc >> 2) * 16 + m;
+            float o = 0.0f;
+#pragma unroll
+            for (int ww = 0; ww < 8; ++ww) o += ((const float*)(smem + ww * g.slab))[idx];
+            if (lora) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const f32x4 sv = *(const f32x4*)(su_tot + m * 16 + 4 * q);
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) o = __builtin_fmaf(sv[c], bv[q][c], o);
+                }
+            }
+            if (g.bias) o += bias_v;
+            if (!ok) o = __builtin_nanf("");
+            g.y[(int64_t)m * g.ldy + n0 + nl] = to_bf16(o);
+        }
+    }
+}
+
+// ---- slots: device memory that belongs to the library (zero when the code object is loaded).
+// Each device holds its own copy of the array at its own address, reached through hipGetSymbolAddress with that device
+// current.  A slot is tied to the caller's scratch pointer, so calls that may legally overlap (different workspaces)
+// never share one; with more than kSlots scratch pointers in use the least recently used slot changes hands, which is
+// safe as long as fewer than kSlots calls with distinct workspaces are in flight on a device at once.
+static __device__ __align__(256) uint32_t rows_slots[kSlots * kSlotWords];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_slots_mu;
+uint32_t* g_slots_ptr[kMaxDevices] = {};
+const void* g_slot_key[kMaxDevices][kSlots] = {};
+uint64_t g_slot_used[kMaxDevices][kSlots] = {};
+uint64_t g_slot_clock = 0;
+}  // namespace
+
+// the slot of `key` on the current device
+static int rows_slot(const void* key, uint32_t** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        xq_set_error("xq_linear_fwd: cannot identify the current device: %s", hipGetErrorString(e));
+        return XQ_ERR_LAUNCH;
+    }
+    std::lock_guard<std::mutex> lock(g_slots_mu);
+    if (!g_slots_ptr[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(rows_slots));
+        if (e != hipSuccess || !p) {
+            xq_set_error("xq_linear_fwd: hipGetSymbolAddress(rows_slots) failed on device %d: %s", dev, hipGetErrorString(e));
+            return XQ_ERR_LAUNCH;
+        }
+        g_slots_ptr[dev] = (uint32_t*)p;
+    }
+    int s = -1, oldest = 0;
+    for (int i = 0; i < kSlots; ++i) {
+        if (g_slot_used[dev][i] && g_slot_key[dev][i] == key) s = i;
+        if (g_slot_used[dev][i] < g_slot_used[dev][oldest]) oldest = i;    // a never-used slot (0) is older than any used one
+    }
+    if (s < 0) {
+        s = oldest;
+        g_slot_key[dev][s] = key;
+    }
+    g_slot_used[dev][s] = ++g_slot_clock;
+    *out = g_slots_ptr[dev] + (size_t)s * kSlotWords;
+    return XQ_OK;
+}
+
+// geometry of a launch: NJ bound and row groups per block
+struct RowsPlan { int nj, njt, G, MR, xpitch, slab; size_t lds; };
+static bool rows_plan(const xq_weight* w, int64_t M, RowsPlan* p) {
+    const int64_t N = w->rows, K = w->cols;
+    const bool f8 = w->format == XQ_FMT_FP8;
+    const int eps = f8 ? 64 : 128;
+    if (K % (8 * eps) != 0) return false;
+    const int ks = (int)(K >> 3);
+    p->nj = ks / eps;
+    if (f8) p->njt = p->nj <= 4 ? 4 : p->nj <= 8 ? 8 : p->nj <= 16 ? 16 : p->nj <= 24 ? 24 : 0;
+    else p->njt = p->nj <= 4 ? 4 : p->nj <= 8 ? 8 : p->nj <= 12 ? 12 : 0;
+    if (!p->njt) return false;
+    p->MR = M <= 1 ? 1 : M <= 8 ? 8 : 16;
+    // x rows in registers: 16 rows only with slices of at most 1 KB, 8 rows with at most 2 KB (register budget)
+    if (p->MR == 16 && p->njt * eps > 512) return false;
+    if (p->MR == 8 && p->njt * eps > 1024) return false;
+    // as many row groups per block as give about one block per compute unit, within 24 loads per lane
+    const int64_t groups = N / 16;
+    int G = (int)((groups + 255) / 256);
+    const int gmax = p->njt <= 4 ? 3 : p->njt <= 8 ? (f8 ? 3 : 2) : p->njt <= 12 ? 2 : 1;
+    p->G = G < 1 ? 1 : G > gmax ? gmax : G;
+    p->xpitch = ks * 2 + 16;
+    int slab = (int)M * p->xpitch + 64;                       // x slice + the NF4 levels
+    if (slab < (p->G + 1) * 1024) slab = (p->G + 1) * 1024;   // later: the wave's sums
+    p->slab = (slab + 15) & ~15;
+    // more blocks than compute units run in rounds, and a round's fixed costs (x slices, sums through LDS, the su parts
+    // that hold up the blocks which form them) then weigh more than the second launch of the other organisation
+    if (xq_cdiv(groups, p->G) > 256) return false;
+    p->lds = (size_t)8 * p->slab + 272 * 4 + 64 * 20 * 4 + 4 * 256 * 4 + 64;
+    return p->lds <= 160 * 1024;
+}
+
+bool skinny_rows_supported(const xq_weight* w, int64_t M, const void* lora_A, const void* lora_B, int lora_dtype, int r) {
+    if (M < 1 || M > 16 || w->num_experts != 1 || w->rows % 16 != 0) return false;
+    if (w->format != XQ_FMT_FP8 && w->layout != XQ_LAYOUT_FLAT) return false;
+    if (w->format == XQ_FMT_NF4 && (w->group != 64 || w->scale_dtype != XQ_SCALE_F32)) return false;
+    if (w->format == XQ_FMT_INT4 && (w->group < 32 || (w->group & (w->group - 1)) != 0 ||
+                                     (w->scale_dtype != XQ_SCALE_F32 && w->scale_dtype != XQ_SCALE_BF16)))
+        return false;
+    if (w->format == XQ_FMT_NVFP4 && w->scale_dtype != XQ_SCALE_E4M3 && w->scale_dtype != XQ_SCALE_F32) return false;
+    RowsPlan p;
+    if (!rows_plan(w, M, &p)) return false;
+    if (r > 0) {
+        if (lora_dtype != XQ_DT_F32 || r > 16 || r % 4 != 0 || !xq_aligned(lora_A, 16) || !xq_aligned(lora_B, 16)) return false;
+        if (w->cols % kSuPartK != 0 || w->cols / kSuPartK > kSuMaxParts) return false;
+        if (w->cols / kSuPartK > xq_cdiv(w->rows / 16, p.G)) return false;   // a block forms at most one su part
+    }
+    return true;
+}
+
+template <int FMT, int G, int NJ, int MR>
+static int launch_rows_one(const SkinnyRowsArgs& g, unsigned grid, size_t lds, hipStream_t s) {
+    static std::atomic<bool> attr_set{false};   // per instantiation; the attribute call is idempotent: a race only repeats it
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute((const void*)skinny_rows_kernel<FMT, G, NJ, MR>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e != hipSuccess) {
+            xq_set_error("xq_linear_fwd: cannot raise the dynamic LDS limit: %s", hipGetErrorString(e));
+            return XQ_ERR_LAUNCH;
+        }
+        attr_set = true;
+    }
+    skinny_rows_kernel<FMT, G, NJ, MR><<<grid, 512, lds, s>>>(g);
+    return XQ_OK;
+}
+
+template <int FMT, int G, int NJ>
+static int launch_rows_mr(const SkinnyRowsArgs& g, int MR, unsigned grid, size_t lds, hipStream_t s) {
+    constexpr int EPS = FMT == XQ_FMT_FP8 ? 64 : 128;
+    if (MR == 1) return launch_rows_one<FMT, G, NJ, 1>(g, grid, lds, s);
+    if constexpr (NJ * EPS <= 1024) {
+        if (MR == 8) return launch_rows_one<FMT, G, NJ, 8>(g, grid, lds, s);
+    }
+    if constexpr (NJ * EPS <= 512) {
+        if (MR == 16) return launch_rows_one<FMT, G, NJ, 16>(g, grid, lds, s);
+    }
+    XQ_REQUIRE(false, "xq_linear_fwd: internal error: no one-launch skinny kernel for %d x rows, %d steps", MR, NJ);
+}
+
+template <int FMT>
+static int launch_rows_fmt(const SkinnyRowsArgs& g, const RowsPlan& p, unsigned grid, hipStream_t s) {
+#define XQ_ROWS_CASE(GG, NN) \
+    if (p.G == GG && p.njt == NN) return launch_rows_mr<FMT, GG, NN>(g, p.MR, grid, p.lds, s)
+    XQ_ROWS_CASE(1, 4); XQ_ROWS_CASE(2, 4); XQ_ROWS_CASE(3, 4);
+    XQ_ROWS_CASE(1, 8); XQ_ROWS_CASE(2, 8);
+    if constexpr (FMT == XQ_FMT_FP8) {
+        XQ_ROWS_CASE(3, 8); XQ_ROWS_CASE(1, 16); XQ_ROWS_CASE(1, 24);
+    } else {
+        XQ_ROWS_CASE(1, 12); XQ_ROWS_CASE(2, 12);
+    }
+#undef XQ_ROWS_CASE
+    XQ_REQUIRE(false, "xq_linear_fwd: internal error: no one-launch skinny kernel for %d row groups, %d steps", p.G, p.njt);
+}
+
+int launch_skinny_rows(const xq_weight* w, const bf16_t* x, int64_t ldx, int64_t M, const void* lora_A, const void* lora_B, int r,
+                       float scaling, const bf16_t* bias, bf16_t* y, int64_t ldy, const void* slot_key, hipStream_t stream) {
+    RowsPlan p;
+    XQ_REQUIRE(rows_plan(w, M, &p), "xq_linear_fwd: internal error: shape not supported by the one-launch skinny kernel");
+    SkinnyRowsArgs g;
+    g.x = x; g.ldx = ldx; g.M = (int)M; g.N = (int)w->rows; g.K = (int)w->cols;
+    g.packed = (const uint8_t*)w->packed; g.scales = (const uint8_t*)w->scales; g.global_scale = w->global_scale;
+    g.gshift = 0;
+    for (int v = w->group; v > 1; v >>= 1) ++g.gshift;
+    g.scale_dtype = w->scale_dtype;
+    g.lora_A = (const float*)lora_A; g.lora_B = (const float*)lora_B; g.r = r; g.su_scale = scaling;
+    g.bias = bias; g.y = y; g.ldy = ldy;
+    g.xpitch = p.xpitch; g.slab = p.slab;
+    g.nsu = r > 0 ? (int)(w->cols / kSuPartK) : 0;
+    g.slot = nullptr;
+    g.spin_limit = kRowsSpinLimit;
+    if (r > 0) {
+        int rc = rows_slot(slot_key, &g.slot);
+        if (rc) return rc;
+    }
+    const unsigned grid = (unsigned)xq_cdiv(w->rows / 16, p.G);
+    switch (w->format) {
+        case XQ_FMT_FP8: return launch_rows_fmt<XQ_FMT_FP8>(g, p, grid, stream);
+        case XQ_FMT_INT4: return launch_rows_fmt<XQ_FMT_INT4>(g, p, grid, stream);
+        case XQ_FMT_NF4: return launch_rows_fmt<XQ_FMT_NF4>(g, p, grid, stream);
+        default: return launch_rows_fmt<XQ_FMT_NVFP4>(g, p, grid, stream);
+    }
+}
+
+}  // namespace xq
