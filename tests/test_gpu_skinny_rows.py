@@ -57,6 +57,10 @@ def _forward(m, x, r=None, bias=True):
     ("nf4", 4096, 5120, 8, True),
     ("nvfp4", 12288, 4096, 16, False),
     ("nvfp4", 1040, 2048, 16, True),
+    ("block_fp8", 24576, 4096, 16, True),     # fused gate|up: 256 blocks, two rounds of three row groups each
+    ("int4", 24576, 4096, 16, False),
+    ("nf4", 24576, 2048, 8, True),
+    ("nvfp4", 24576, 1024, 16, False),
 ])
 def test_one_launch_vs_oracle_and_two_launch(hip_device, organisations, fmt, N, K, r, has_bias):
     m, w_ref = make_dense_module(fmt, N, K, r, 2 * r, seed=N + K + r, device=hip_device, bias=has_bias)

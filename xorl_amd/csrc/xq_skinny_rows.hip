@@ -12,10 +12,10 @@
 // The low-rank intermediate su = x . A^T [M, r] is needed whole by every block but costs r x K factor bytes to form, more
 // than a block's share of the weight.  It is formed once per launch: in each of the first K / 512 blocks the four waves
 // that are last in the load queue contract 512 elements of K before they turn to their weight rows, and publish the
-// 256 sums to a slot in device memory; wave 0 of
-// every block, which is the first to finish its part of the weight stream, collects the parts while the other waves are
-// still streaming.  Nothing on that path waits for an atomic's return value or for an ordering between stores:
-//  * the slot holds a launch count `gen`; every block reads it first thing (one load among its others);
+// 256 sums to a slot in device memory; wave 0 of every block, which is the first to finish its part of the weight
+// stream, collects the parts while the other waves are still streaming.  Nothing on that path waits for an atomic's
+// return value or for an ordering between stores:
+//  * the slot holds a launch count `gen`, which wave 0 of every block reads (behind its weight loads);
 //  * a published entry is the 8-byte pair (sum, gen + 1), stored whole; a collector takes an entry when its tag is
 //    gen + 1, so what earlier launches left in the slot never passes for this launch's sums and nothing is cleared;
 //  * `gen` moves on once per launch, after every block has read it: each block adds one to `started` when its own read
@@ -23,13 +23,14 @@
 //    parts, stores gen + 1 and started = 0 when it finds the whole grid there (it looks again if not).  Both words
 //    exist in 32 copies on different memory lines (block b reads and counts in copy b % 32; the last block sums and
 //    rewrites them all): hundreds of accesses to one location that bypass the caches would take microseconds.
-// Slot accesses are device-scope atomics (they bypass the per-XCD L2s).  Blocks that publish never wait, and they are
-// the first the dispatcher places, so the collectors' wait ends; a limit bounds every wait all the same and turns the
-// block's outputs into NaN.  Sums run in fixed orders (waves ascending, parts ascending): results are identical from
-// call to call.
+// Slot accesses are device-scope atomics (they bypass the per-XCD L2s) unless said otherwise where they are made.
+// Blocks that publish never wait, and they are the first the dispatcher places, so the collectors' wait ends; a limit
+// bounds every wait all the same and turns the block's outputs into NaN.  Sums run in fixed orders (waves ascending,
+// parts ascending): results are identical from call to call.
 //
-// Measured on an MI355X, launches back to back (block_fp8, r = 16, M = 1): 4096->12288 (48 MiB) ~12 us against 15 us for
-// the two-launch organisation, 4096->1024 ~6 us against 7.7 us.
+// Measured on an MI355X, launches back to back (block_fp8, r = 16, M = 1): 4096->12288 (48 MiB) 12.6 us against 15.3 us
+// for the two-launch organisation (11.5 us without a low-rank term), 4096->4096 7.2 against 8.6, 4096->24576 (96 MiB)
+// 20.0 against 21.6.
 #include <atomic>
 #include <mutex>
 
@@ -69,10 +70,11 @@ struct SkinnyRowsArgs {
     int32_t spin_limit;
 };
 
-// FMT: weight format; G: 16-row groups per block; NJ: most load steps per wave (a step is one 16-byte load per lane:
-// 64 elements of K per row for fp8, 128 for the 4-bit formats); MR: bound on M (x rows kept in registers on their way
-// to LDS)
-template <int FMT, int G, int NJ, int MR>
+// FMT: weight format; G: 16-row groups in flight per block; NJ: most load steps per wave (a step is one 16-byte load
+// per lane: 64 elements of K per row for fp8, 128 for the 4-bit formats); MR: bound on M (x rows kept in registers on
+// their way to LDS); R: rounds -- a block walks R sets of G row groups, each step's registers refilled for the next
+// round as soon as the step has been multiplied, so the weight stream never stops (N % (16 G R) == 0 when R > 1)
+template <int FMT, int G, int NJ, int MR, int R>
 __global__ void __launch_bounds__(512, 1) skinny_rows_kernel(SkinnyRowsArgs g) {
     constexpr bool F8 = FMT == XQ_FMT_FP8;
     constexpr int EPS = F8 ? 64 : 128;                 // K elements of a row per load step
@@ -91,12 +93,12 @@ __global__ void __launch_bounds__(512, 1) skinny_rows_kernel(SkinnyRowsArgs g) {
     const int ks = g.K >> 3;                    // K elements per wave
     const int k0 = wave * ks;
     const int nj = ks / EPS;                    // load steps of this launch, 1 .. NJ
-    const int n0 = blockIdx.x * (16 * G);
+    const int n0 = blockIdx.x * (16 * G * R);
     const int XP = g.xpitch;
     unsigned char* slab = smem + wave * g.slab;
     float* su_tot = (float*)(smem + 8 * g.slab);           // [16 m][16 j], then a flag
-    float* b_tile = su_tot + 272;                           // [64 rows][20]: the block's rows of B, 16 bytes apart in banks
-    float* su_red = b_tile + 64 * 20;                       // [4 waves][256]: the tiles of an su part
+    float* b_tile = su_tot + 272;                           // [96 rows][20]: the block's rows of B, 16 bytes apart in banks
+    float* su_red = b_tile + 96 * 20;                       // [4 waves][256]: the tiles of an su part
     int* su_flag = (int*)(su_red + 4 * 256);                // [0 .. 3]: wave 4 + w has written its tile; [4]: wave 4 is done with `gen`
     const bool lora = g.nsu > 0;
     const bool su_block = (int)blockIdx.x < g.nsu;          // nsu <= gridDim.x (checked on the host)
@@ -226,24 +228,25 @@ __global__ void __launch_bounds__(512, 1) skinny_rows_kernel(SkinnyRowsArgs g) {
         wp[gi] = g.packed + ((int64_t)n * g.K + k0) / EB + kq * 16;
     }
     const int scols = (g.K + 127) >> 7;
-    auto load_w = [&](int ja, int jb) {
+    const int64_t round_bytes = (int64_t)16 * G * g.K / EB;          // from a round's rows to the next round's
+    auto load_w = [&](int ja, int jb, int rr) {
 #pragma unroll
         for (int j = ja; j < jb; ++j) {
             const int jc = j < nj ? j : nj - 1;
 #pragma unroll
             for (int gi = 0; gi < G; ++gi) {
-                w[j][gi] = *(const u32x4*)(wp[gi] + jc * 64);
+                w[j][gi] = *(const u32x4*)(wp[gi] + rr * round_bytes + jc * 64);
                 if (FMT == XQ_FMT_FP8) {
                     // one scale per 128 x 128 block: the same for the 16 rows of a group and the 64 elements of a step
-                    const int nb = n0 + gi * 16 < g.N ? n0 + gi * 16 : g.N - 16;
+                    const int nb = n0 + (rr * G + gi) * 16 < g.N ? n0 + (rr * G + gi) * 16 : g.N - 16;
                     sc[j][gi][0] = ((const __attribute__((address_space(4))) uint32_t*)g.scales)[(nb >> 7) * scols + ((k0 + jc * 64) >> 7)];
                 } else if (FMT == XQ_FMT_INT4) {
-                    const int64_t si = (erow[gi] + jc * EPS) >> g.gshift;      // group % 32 == 0: one scale per load
+                    const int64_t si = (erow[gi] + rr * round_bytes * EB + jc * EPS) >> g.gshift;      // group % 32 == 0: one scale per load
                     sc[j][gi][0] = g.scale_dtype == XQ_SCALE_F32 ? ((const uint32_t*)g.scales)[si] : (uint32_t)((const uint16_t*)g.scales)[si] << 16;
                 } else if (FMT == XQ_FMT_NF4) {
-                    sc[j][gi][0] = ((const uint32_t*)g.scales)[(erow[gi] + jc * EPS) >> 6];       // fp32, group 64
+                    sc[j][gi][0] = ((const uint32_t*)g.scales)[(erow[gi] + rr * round_bytes * EB + jc * EPS) >> 6];       // fp32, group 64
                 } else {
-                    const int64_t si = (erow[gi] + jc * EPS) >> 4;                                 // two blocks of 16 per load
+                    const int64_t si = (erow[gi] + rr * round_bytes * EB + jc * EPS) >> 4;         // two blocks of 16 per load
                     if (g.scale_dtype == XQ_SCALE_E4M3) {
                         sc[j][gi][0] = *(const uint16_t*)(g.scales + si);
                         sc[j][gi][1] = 0;
@@ -256,7 +259,7 @@ __global__ void __launch_bounds__(512, 1) skinny_rows_kernel(SkinnyRowsArgs g) {
             }
         }
     };
-    load_w(0, J1);
+    load_w(0, J1, 0);
     __builtin_amdgcn_sched_barrier(0);
 
     // ---- x slice -> LDS (the wave's own area; LDS operations of one wave execute in order, no barrier)
@@ -268,22 +271,26 @@ __global__ void __launch_bounds__(512, 1) skinny_rows_kernel(SkinnyRowsArgs g) {
     float* nf4_lds = (float*)(slab + g.slab - 64);          // 16 levels at the end of the wave's area
     if (FMT == XQ_FMT_NF4 && lane < 16) nf4_lds[lane] = kNf4Level[lane];
     __builtin_amdgcn_sched_barrier(0);
-    load_w(J1, NJ);
+    load_w(J1, NJ, 0);
     __builtin_amdgcn_sched_barrier(0);
 
-    // ---- what the finish needs, requested behind the weights: the block's rows of B (thread t < 256: row t / 4, ranks
-    // 4 (t % 4) ..), the bias of column tid % 64
+    // ---- what the finish needs, requested behind the weights: the block's rows of B (thread t < 384: row t / 4, ranks
+    // 4 (t % 4) ..), the bias of column tid % 64 of each round
     const int nl = tid & 63;
     f32x4 bq = {0.0f, 0.0f, 0.0f, 0.0f};
     const int brow = tid >> 2, bpiece = tid & 3;
-    const bool bvalid = lora && tid < 256 && brow < 16 * G && n0 + brow < g.N && 4 * bpiece < g.r;
+    const bool bvalid = lora && brow < 16 * G * R && n0 + brow < g.N && 4 * bpiece < g.r;
     {
         const int64_t bn = n0 + brow < g.N ? n0 + brow : g.N - 1;
         const float* bp = lora ? g.lora_B + bn * g.r + (4 * bpiece < g.r ? 4 * bpiece : 0) : (const float*)g.x;
         bq = *(const f32x4*)bp;
     }
-    const int nfin = (nl < 16 * G && n0 + nl < g.N) ? n0 + nl : g.N - 1;
-    const float bias_v = bf16_to_f32((g.bias ? g.bias : g.x)[g.bias ? nfin : 0]);
+    float bias_v[R];
+#pragma unroll
+    for (int rr = 0; rr < R; ++rr) {
+        const int nfin = (nl < 16 * G && n0 + rr * 16 * G + nl < g.N) ? n0 + rr * 16 * G + nl : g.N - 1;
+        bias_v[rr] = bf16_to_f32((g.bias ? g.bias : g.x)[g.bias ? nfin : 0]);
+    }
     __builtin_amdgcn_sched_barrier(0);
     if (lora && wave == 0) gen = __hip_atomic_load(ctl, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __builtin_amdgcn_sched_barrier(0);
@@ -292,9 +299,11 @@ __global__ void __launch_bounds__(512, 1) skinny_rows_kernel(SkinnyRowsArgs g) {
     const float gsc = FMT == XQ_FMT_NVFP4 ? g.global_scale[0] : 1.0f;
     const int xm = rn < g.M ? rn : g.M - 1;
     const unsigned char* xrow = slab + xm * XP + kq * (EPS / 2);
-    f32x4 acc[G];
+    f32x4 acc[R * G];
 #pragma unroll
-    for (int gi = 0; gi < G; ++gi) acc[gi] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    for (int gi = 0; gi < R * G; ++gi) acc[gi] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int rr = 0; rr < R; ++rr)
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
         if (j < nj) {      // wave-uniform
@@ -319,10 +328,11 @@ __global__ void __launch_bounds__(512, 1) skinny_rows_kernel(SkinnyRowsArgs g) {
                         else sv = __uint_as_float(sc[j][gi][c >> 1]);
                         wf = decode8<FMT>(w[j][gi][c], 0u, sv * gsc, 0.0f);
                     }
-                    acc[gi] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, xf[c], acc[gi], 0, 0, 0);
+                    acc[rr * G + gi] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, xf[c], acc[rr * G + gi], 0, 0, 0);
                 }
             }
         }
+        if (rr + 1 < R) load_w(j, j + 1, rr + 1);      // this step's registers are free: the next round's bytes
     }
 
     // this block may be counted once its reads of `gen` have returned: wave 0's has, like the weights requested before it;
@@ -341,10 +351,10 @@ __global__ void __launch_bounds__(512, 1) skinny_rows_kernel(SkinnyRowsArgs g) {
     // ---- the wave's sums -> its own LDS area (its x slice is no longer needed): tile gi, register q, lane; B rows -> LDS
     float* part = (float*)slab;
 #pragma unroll
-    for (int gi = 0; gi < G; ++gi)
+    for (int gi = 0; gi < R * G; ++gi)
 #pragma unroll
         for (int q = 0; q < 4; ++q) part[gi * 256 + q * 64 + lane] = acc[gi][q];
-    if (tid < 256) *(f32x4*)(b_tile + brow * 20 + bpiece * 4) = bvalid ? bq : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    if (tid < 384) *(f32x4*)(b_tile + brow * 20 + bpiece * 4) = bvalid ? bq : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 
     // ---- wave 0 (its loads were requested first, so it gets here first) collects the su parts while the other waves are
     // still streaming: entry q * 64 + l of a part is su[j = 4 (l >> 4) + q][m = l & 15]
@@ -416,35 +426,39 @@ __global__ void __launch_bounds__(512, 1) skinny_rows_kernel(SkinnyRowsArgs g) {
     }
     lds_barrier();
 
-    // ---- outputs: thread (nl, mg) finishes y[mg][n0 + nl] and y[mg + 8][n0 + nl]: the eight waves' sums in wave order, the
-    // low-rank term rank by rank in fp32, the bias, one rounding
+    // ---- outputs: thread (nl, mg) finishes y[mg][n] and y[mg + 8][n] for row n = n0 + 16 G rr + nl of every round: the eight
+    // waves' sums in wave order, the low-rank term rank by rank in fp32, the bias, one rounding
     const int mg = tid >> 6;
-    const bool nvalid = nl < 16 * G && n0 + nl < g.N;
     const int gi_f = nl >> 4, nloc = nl & 15;
     const bool ok = !lora || ((const int*)su_tot)[256] != 0;
-    f32x4 bv[4];
 #pragma unroll
-    for (int q = 0; q < 4; ++q) bv[q] = *(const f32x4*)(b_tile + nl * 20 + 4 * q);
+    for (int rr = 0; rr < R; ++rr) {
+        const int nrow = rr * 16 * G + nl;              // row of the block
+        const bool nvalid = nl < 16 * G && n0 + nrow < g.N;
+        f32x4 bv[4];
 #pragma unroll
-    for (int mm = 0; mm < 2; ++mm) {
-        const int m = mg + 8 * mm;
-        if (m < g.M && nvalid) {
-            // D[nloc][m] of a wave's tile sits in register nloc & 3 of lane 16 (nloc >> 2) + m
-            const int idx = gi_f * 256 + (nloc & 3) * 64 + (nloc >> 2) * 16 + m;
-            float o = 0.0f;
+        for (int q = 0; q < 4; ++q) bv[q] = *(const f32x4*)(b_tile + (nl < 16 * G ? nrow : 0) * 20 + 4 * q);
 #pragma unroll
-            for (int ww = 0; ww < 8; ++ww) o += ((const float*)(smem + ww * g.slab))[idx];
-            if (lora) {
+        for (int mm = 0; mm < 2; ++mm) {
+            const int m = mg + 8 * mm;
+            if (m < g.M && nvalid) {
+                // D[nloc][m] of a wave's tile sits in register nloc & 3 of lane 16 (nloc >> 2) + m
+                const int idx = (rr * G + gi_f) * 256 + (nloc & 3) * 64 + (nloc >> 2) * 16 + m;
+                float o = 0.0f;
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const f32x4 sv = *(const f32x4*)(su_tot + m * 16 + 4 * q);
+                for (int ww = 0; ww < 8; ++ww) o += ((const float*)(smem + ww * g.slab))[idx];
+                if (lora) {
 #pragma unroll
-                    for (int c = 0; c < 4; ++c) o = __builtin_fmaf(sv[c], bv[q][c], o);
+                    for (int q = 0; q < 4; ++q) {
+                        const f32x4 sv = *(const f32x4*)(su_tot + m * 16 + 4 * q);
+#pragma unroll
+                        for (int c = 0; c < 4; ++c) o = __builtin_fmaf(sv[c], bv[q][c], o);
+                    }
                 }
+                if (g.bias) o += bias_v[rr];
+                if (!ok) o = __builtin_nanf("");
+                g.y[(int64_t)m * g.ldy + n0 + nrow] = to_bf16(o);
             }
-            if (g.bias) o += bias_v;
-            if (!ok) o = __builtin_nanf("");
-            g.y[(int64_t)m * g.ldy + n0 + nl] = to_bf16(o);
         }
     }
 }
@@ -498,7 +512,7 @@ static int rows_slot(const void* key, uint32_t** out) {
 }
 
 // geometry of a launch: NJ bound and row groups per block
-struct RowsPlan { int nj, njt, G, MR, xpitch, slab; size_t lds; };
+struct RowsPlan { int nj, njt, G, R, MR, xpitch, slab; size_t lds; };
 static bool rows_plan(const xq_weight* w, int64_t M, RowsPlan* p) {
     const int64_t N = w->rows, K = w->cols;
     const bool f8 = w->format == XQ_FMT_FP8;
@@ -518,14 +532,20 @@ static bool rows_plan(const xq_weight* w, int64_t M, RowsPlan* p) {
     int G = (int)((groups + 255) / 256);
     const int gmax = p->njt <= 4 ? 3 : p->njt <= 8 ? (f8 ? 3 : 2) : p->njt <= 12 ? 2 : 1;
     p->G = G < 1 ? 1 : G > gmax ? gmax : G;
+    // more blocks than compute units would run one after the other, each with its own start-up and finish (that costs
+    // more than the second launch of the other organisation): twice the rows go to one block in two rounds instead,
+    // where the shape allows it
+    p->R = 1;
+    if (xq_cdiv(groups, p->G) > 256) {
+        const bool two_rounds = p->G == 3 && p->njt * eps <= 512 && groups % 6 == 0 && groups / 6 <= 256;
+        if (!two_rounds) return false;
+        p->R = 2;
+    }
     p->xpitch = ks * 2 + 16;
     int slab = (int)M * p->xpitch + 64;                       // x slice + the NF4 levels
-    if (slab < (p->G + 1) * 1024) slab = (p->G + 1) * 1024;   // later: the wave's sums
+    if (slab < (p->G * p->R + 1) * 1024) slab = (p->G * p->R + 1) * 1024;   // later: the wave's sums
     p->slab = (slab + 15) & ~15;
-    // more blocks than compute units run in rounds, and a round's fixed costs (x slices, sums through LDS, the su parts
-    // that hold up the blocks which form them) then weigh more than the second launch of the other organisation
-    if (xq_cdiv(groups, p->G) > 256) return false;
-    p->lds = (size_t)8 * p->slab + 272 * 4 + 64 * 20 * 4 + 4 * 256 * 4 + 64;
+    p->lds = (size_t)8 * p->slab + 272 * 4 + 96 * 20 * 4 + 4 * 256 * 4 + 64;
     return p->lds <= 160 * 1024;
 }
 
@@ -542,52 +562,54 @@ bool skinny_rows_supported(const xq_weight* w, int64_t M, const void* lora_A, co
     if (r > 0) {
         if (lora_dtype != XQ_DT_F32 || r > 16 || r % 4 != 0 || !xq_aligned(lora_A, 16) || !xq_aligned(lora_B, 16)) return false;
         if (w->cols % kSuPartK != 0 || w->cols / kSuPartK > kSuMaxParts) return false;
-        if (w->cols / kSuPartK > xq_cdiv(w->rows / 16, p.G)) return false;   // a block forms at most one su part
+        if (w->cols / kSuPartK > xq_cdiv(w->rows / 16, p.G * p.R)) return false;   // a block forms at most one su part
     }
     return true;
 }
 
-template <int FMT, int G, int NJ, int MR>
+template <int FMT, int G, int NJ, int MR, int R>
 static int launch_rows_one(const SkinnyRowsArgs& g, unsigned grid, size_t lds, hipStream_t s) {
     static std::atomic<bool> attr_set{false};   // per instantiation; the attribute call is idempotent: a race only repeats it
     if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute((const void*)skinny_rows_kernel<FMT, G, NJ, MR>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        hipError_t e = hipFuncSetAttribute((const void*)skinny_rows_kernel<FMT, G, NJ, MR, R>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) {
             xq_set_error("xq_linear_fwd: cannot raise the dynamic LDS limit: %s", hipGetErrorString(e));
             return XQ_ERR_LAUNCH;
         }
         attr_set = true;
     }
-    skinny_rows_kernel<FMT, G, NJ, MR><<<grid, 512, lds, s>>>(g);
+    skinny_rows_kernel<FMT, G, NJ, MR, R><<<grid, 512, lds, s>>>(g);
     return XQ_OK;
 }
 
-template <int FMT, int G, int NJ>
+template <int FMT, int G, int NJ, int R>
 static int launch_rows_mr(const SkinnyRowsArgs& g, int MR, unsigned grid, size_t lds, hipStream_t s) {
     constexpr int EPS = FMT == XQ_FMT_FP8 ? 64 : 128;
-    if (MR == 1) return launch_rows_one<FMT, G, NJ, 1>(g, grid, lds, s);
+    if (MR == 1) return launch_rows_one<FMT, G, NJ, 1, R>(g, grid, lds, s);
     if constexpr (NJ * EPS <= 1024) {
-        if (MR == 8) return launch_rows_one<FMT, G, NJ, 8>(g, grid, lds, s);
+        if (MR == 8) return launch_rows_one<FMT, G, NJ, 8, R>(g, grid, lds, s);
     }
     if constexpr (NJ * EPS <= 512) {
-        if (MR == 16) return launch_rows_one<FMT, G, NJ, 16>(g, grid, lds, s);
+        if (MR == 16) return launch_rows_one<FMT, G, NJ, 16, R>(g, grid, lds, s);
     }
     XQ_REQUIRE(false, "xq_linear_fwd: internal error: no one-launch skinny kernel for %d x rows, %d steps", MR, NJ);
 }
 
 template <int FMT>
 static int launch_rows_fmt(const SkinnyRowsArgs& g, const RowsPlan& p, unsigned grid, hipStream_t s) {
-#define XQ_ROWS_CASE(GG, NN) \
-    if (p.G == GG && p.njt == NN) return launch_rows_mr<FMT, GG, NN>(g, p.MR, grid, p.lds, s)
-    XQ_ROWS_CASE(1, 4); XQ_ROWS_CASE(2, 4); XQ_ROWS_CASE(3, 4);
-    XQ_ROWS_CASE(1, 8); XQ_ROWS_CASE(2, 8);
+    constexpr int EPS = FMT == XQ_FMT_FP8 ? 64 : 128;
+#define XQ_ROWS_CASE(GG, NN, RR) \
+    if (p.G == GG && p.njt == NN && p.R == RR) return launch_rows_mr<FMT, GG, NN, RR>(g, p.MR, grid, p.lds, s)
+    XQ_ROWS_CASE(1, 4, 1); XQ_ROWS_CASE(2, 4, 1); XQ_ROWS_CASE(3, 4, 1); XQ_ROWS_CASE(3, 4, 2);
+    XQ_ROWS_CASE(1, 8, 1); XQ_ROWS_CASE(2, 8, 1);
     if constexpr (FMT == XQ_FMT_FP8) {
-        XQ_ROWS_CASE(3, 8); XQ_ROWS_CASE(1, 16); XQ_ROWS_CASE(1, 24);
+        XQ_ROWS_CASE(3, 8, 1); XQ_ROWS_CASE(3, 8, 2); XQ_ROWS_CASE(1, 16, 1); XQ_ROWS_CASE(1, 24, 1);
     } else {
-        XQ_ROWS_CASE(1, 12); XQ_ROWS_CASE(2, 12);
+        XQ_ROWS_CASE(1, 12, 1); XQ_ROWS_CASE(2, 12, 1);
     }
 #undef XQ_ROWS_CASE
-    XQ_REQUIRE(false, "xq_linear_fwd: internal error: no one-launch skinny kernel for %d row groups, %d steps", p.G, p.njt);
+    (void)EPS;
+    XQ_REQUIRE(false, "xq_linear_fwd: internal error: no one-launch skinny kernel for %d row groups, %d steps, %d rounds", p.G, p.njt, p.R);
 }
 
 int launch_skinny_rows(const xq_weight* w, const bf16_t* x, int64_t ldx, int64_t M, const void* lora_A, const void* lora_B, int r,
@@ -610,7 +632,7 @@ int launch_skinny_rows(const xq_weight* w, const bf16_t* x, int64_t ldx, int64_t
         int rc = rows_slot(slot_key, &g.slot);
         if (rc) return rc;
     }
-    const unsigned grid = (unsigned)xq_cdiv(w->rows / 16, p.G);
+    const unsigned grid = (unsigned)xq_cdiv(w->rows / 16, p.G * p.R);
     switch (w->format) {
         case XQ_FMT_FP8: return launch_rows_fmt<XQ_FMT_FP8>(g, p, grid, stream);
         case XQ_FMT_INT4: return launch_rows_fmt<XQ_FMT_INT4>(g, p, grid, stream);
