@@ -171,3 +171,53 @@ def test_one_launch_under_hip_graph_with_changing_input(hip_device):
         eager = step()
         torch.cuda.synchronize()
         assert torch.equal(got, eager), rep
+
+
+def test_overlapping_calls_on_two_streams(hip_device):
+    """Forwards on two streams, each with its own workspace (so each with its own slot), issued so that they overlap on the
+    device: small grids that leave compute units free for the other stream's kernel.  Every result equals the one the same
+    call gives alone."""
+    from xorl_amd import _C
+    from xorl_amd.functional import _workspace_bytes
+
+    r = 16
+    shapes = [("block_fp8", 1024, 4096, 4), ("int4", 2048, 4096, 1)]
+    L = _C.lib()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    work = []
+    for i, (fmt, N, K, M) in enumerate(shapes):
+        m, _ = make_dense_module(fmt, N, K, r, 32, seed=60 + i, device=hip_device)
+        w = m._quant_weight().c()
+        A, B = m.lora_A.detach().contiguous(), m.lora_B.detach().contiguous()
+        wsb = _workspace_bytes(M, N, K, r)
+        ws = torch.empty(wsb, dtype=torch.uint8, device=hip_device)
+        xs = [gen((M, K), 1.0, 600 + 10 * i + j, torch.bfloat16).to(hip_device) for j in range(6)]
+        ys = [torch.empty(M, N, dtype=torch.bfloat16, device=hip_device) for _ in xs]
+        work.append((m, w, A, B, ws, wsb, xs, ys, N, K, M))
+
+    def call(i, j, y, stream):
+        m, w, A, B, ws, wsb, xs, _, N, K, M = work[i]
+        _C.check(L.xq_linear_fwd(ctypes.byref(w), xs[j].data_ptr(), K, M, A.data_ptr(), B.data_ptr(), _C.XQ_DT_F32, r,
+                                 ctypes.c_float(m.scaling), None, y.data_ptr(), N, None, ws.data_ptr(), wsb, stream))
+
+    # alone, on the current stream
+    alone = []
+    for i in range(2):
+        outs = []
+        for j in range(6):
+            y = torch.empty_like(work[i][7][j])
+            call(i, j, y, _C.stream_ptr(hip_device))
+            outs.append(y)
+        alone.append(outs)
+    torch.cuda.synchronize()
+    # interleaved on two streams, many times over
+    for st in streams:
+        st.wait_stream(torch.cuda.current_stream())
+    for rep in range(20):
+        for j in range(6):
+            for i in range(2):
+                call(i, j, work[i][7][j], ctypes.c_void_p(streams[i].cuda_stream))
+    torch.cuda.synchronize()
+    for i in range(2):
+        for j in range(6):
+            assert torch.equal(work[i][7][j], alone[i][j]), (i, j)
