@@ -48,6 +48,10 @@ constexpr int kCtlStride = 32;                  // so that a launch's 256 blocks
 constexpr int kSlotWords = kSlotCtl + 2 * kCtlCopies * kCtlStride;   // [parts][256] pairs (sum bits, tag), gen copies, started copies
 constexpr int kSlots = 64;
 constexpr int kRowsSpinLimit = 1 << 20;
+#ifndef XQ_ROWS_LOADS_IN_FLIGHT
+#define XQ_ROWS_LOADS_IN_FLIGHT 6
+#endif
+constexpr int kRowsLoadsInFlight = XQ_ROWS_LOADS_IN_FLIGHT;   // 16-byte weight loads per lane kept in flight
 
 struct SkinnyRowsArgs {
     const bf16_t* x;
@@ -213,11 +217,15 @@ __global__ void __launch_bounds__(512, 1) skinny_rows_kernel(SkinnyRowsArgs g) {
     __builtin_amdgcn_sched_barrier(0);
 
     // ---- the block's weight rows, this wave's K range: step j gives lane (row rn, quarter kq) the 16 bytes at element
-    // EPS j + (EPS / 4) kq of its row's slice.  With 16 x rows in registers the last third of the steps is requested once
-    // the x slice has been written to LDS.
-    constexpr int J1 = MR > 8 ? (2 * NJ + 2) / 3 : NJ;
-    u32x4 w[NJ][G];
-    uint32_t sc[NJ][G][NSC];
+    // EPS j + (EPS / 4) kq of its row's slice.  The R NJ steps of a wave form one stream through a ring of DJ step
+    // registers: DJ steps are requested up front, and each step's registers are refilled with the step DJ further on as
+    // soon as it has been multiplied.  About 6 KB per wave in flight (48 KB per CU; 4 to 12 KB measure alike, 24 KB 10 % slower) keeps the memory pipe full (a CU takes loads only
+    // as fast as memory returns them: more would queue in front of the other waves') and lets all eight waves advance
+    // together, so that at the end only the last steps remain to be decoded.
+    constexpr int T = R * NJ;                                   // steps of the stream (those past nj of a round are idle)
+    constexpr int DJ = T < (kRowsLoadsInFlight + G - 1) / G ? T : (kRowsLoadsInFlight + G - 1) / G;
+    u32x4 w[DJ][G];
+    uint32_t sc[DJ][G][NSC];
     const uint8_t* wp[G];
     int64_t erow[G];                            // element index of (row, k0 + (EPS / 4) kq), for the per-row scales
 #pragma unroll
@@ -229,10 +237,10 @@ __global__ void __launch_bounds__(512, 1) skinny_rows_kernel(SkinnyRowsArgs g) {
     }
     const int scols = (g.K + 127) >> 7;
     const int64_t round_bytes = (int64_t)16 * G * g.K / EB;          // from a round's rows to the next round's
-    auto load_w = [&](int ja, int jb, int rr) {
-#pragma unroll
-        for (int j = ja; j < jb; ++j) {
-            const int jc = j < nj ? j : nj - 1;
+    auto load_step = [&](int t) {
+        {
+            const int rr = t / NJ, jj = t % NJ, j = t % DJ;
+            const int jc = jj < nj ? jj : nj - 1;
 #pragma unroll
             for (int gi = 0; gi < G; ++gi) {
                 w[j][gi] = *(const u32x4*)(wp[gi] + rr * round_bytes + jc * 64);
@@ -259,7 +267,8 @@ __global__ void __launch_bounds__(512, 1) skinny_rows_kernel(SkinnyRowsArgs g) {
             }
         }
     };
-    load_w(0, J1, 0);
+#pragma unroll
+    for (int t = 0; t < DJ; ++t) load_step(t);
     __builtin_amdgcn_sched_barrier(0);
 
     // ---- x slice -> LDS (the wave's own area; LDS operations of one wave execute in order, no barrier)
@@ -271,28 +280,27 @@ __global__ void __launch_bounds__(512, 1) skinny_rows_kernel(SkinnyRowsArgs g) {
     float* nf4_lds = (float*)(slab + g.slab - 64);          // 16 levels at the end of the wave's area
     if (FMT == XQ_FMT_NF4 && lane < 16) nf4_lds[lane] = kNf4Level[lane];
     __builtin_amdgcn_sched_barrier(0);
-    load_w(J1, NJ, 0);
-    __builtin_amdgcn_sched_barrier(0);
 
-    // ---- what the finish needs, requested behind the weights: the block's rows of B (thread t < 384: row t / 4, ranks
-    // 4 (t % 4) ..), the bias of column tid % 64 of each round
+    // ---- what the finish needs is requested behind the last weight load (loads return in order, and wave 0's read of the
+    // launch count is slow): the block's rows of B (thread t < 384: row t / 4, ranks 4 (t % 4) ..), the bias of column
+    // tid % 64 of each round, `gen`
     const int nl = tid & 63;
     f32x4 bq = {0.0f, 0.0f, 0.0f, 0.0f};
     const int brow = tid >> 2, bpiece = tid & 3;
     const bool bvalid = lora && brow < 16 * G * R && n0 + brow < g.N && 4 * bpiece < g.r;
-    {
+    float bias_v[R];
+    auto finish_loads = [&]() {
         const int64_t bn = n0 + brow < g.N ? n0 + brow : g.N - 1;
         const float* bp = lora ? g.lora_B + bn * g.r + (4 * bpiece < g.r ? 4 * bpiece : 0) : (const float*)g.x;
         bq = *(const f32x4*)bp;
-    }
-    float bias_v[R];
 #pragma unroll
-    for (int rr = 0; rr < R; ++rr) {
-        const int nfin = (nl < 16 * G && n0 + rr * 16 * G + nl < g.N) ? n0 + rr * 16 * G + nl : g.N - 1;
-        bias_v[rr] = bf16_to_f32((g.bias ? g.bias : g.x)[g.bias ? nfin : 0]);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    if (lora && wave == 0) gen = __hip_atomic_load(ctl, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        for (int rr = 0; rr < R; ++rr) {
+            const int nfin = (nl < 16 * G && n0 + rr * 16 * G + nl < g.N) ? n0 + rr * 16 * G + nl : g.N - 1;
+            bias_v[rr] = bf16_to_f32((g.bias ? g.bias : g.x)[g.bias ? nfin : 0]);
+        }
+        if (lora && wave == 0) gen = __hip_atomic_load(ctl, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    };
+    if (T == DJ) finish_loads();
     __builtin_amdgcn_sched_barrier(0);
 
     // ---- decode + multiply, D[n][m] += deq(W)[n][k] x[m][k], in the order the weights arrive
@@ -303,9 +311,8 @@ __global__ void __launch_bounds__(512, 1) skinny_rows_kernel(SkinnyRowsArgs g) {
 #pragma unroll
     for (int gi = 0; gi < R * G; ++gi) acc[gi] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-    for (int rr = 0; rr < R; ++rr)
-#pragma unroll
-    for (int j = 0; j < NJ; ++j) {
+    for (int t = 0; t < T; ++t) {
+        const int rr = t / NJ, j = t % NJ, sl = t % DJ;
         if (j < nj) {      // wave-uniform
             bf16x8 xf[MPS];
 #pragma unroll
@@ -316,23 +323,25 @@ __global__ void __launch_bounds__(512, 1) skinny_rows_kernel(SkinnyRowsArgs g) {
                 for (int c = 0; c < MPS; ++c) {
                     bf16x8 wf;
                     if (FMT == XQ_FMT_FP8) {
-                        wf = decode8<FMT>(w[j][gi][2 * c], w[j][gi][2 * c + 1], __uint_as_float(sc[j][gi][0]), 0.0f);
+                        wf = decode8<FMT>(w[sl][gi][2 * c], w[sl][gi][2 * c + 1], __uint_as_float(sc[sl][gi][0]), 0.0f);
                     } else if (FMT == XQ_FMT_INT4) {
-                        const float sv = __uint_as_float(sc[j][gi][0]);
-                        wf = decode8<FMT>(w[j][gi][c], 0u, sv, -8.0f * sv);
+                        const float sv = __uint_as_float(sc[sl][gi][0]);
+                        wf = decode8<FMT>(w[sl][gi][c], 0u, sv, -8.0f * sv);
                     } else if (FMT == XQ_FMT_NF4) {
-                        wf = decode8<FMT>(w[j][gi][c], 0u, __uint_as_float(sc[j][gi][0]), 0.0f, nf4_lds);
+                        wf = decode8<FMT>(w[sl][gi][c], 0u, __uint_as_float(sc[sl][gi][0]), 0.0f, nf4_lds);
                     } else {
                         float sv;   // block c / 2 of the load's two
-                        if (g.scale_dtype == XQ_SCALE_E4M3) sv = e4m3_to_f32((uint8_t)(sc[j][gi][0] >> (8 * (c >> 1))));
-                        else sv = __uint_as_float(sc[j][gi][c >> 1]);
-                        wf = decode8<FMT>(w[j][gi][c], 0u, sv * gsc, 0.0f);
+                        if (g.scale_dtype == XQ_SCALE_E4M3) sv = e4m3_to_f32((uint8_t)(sc[sl][gi][0] >> (8 * (c >> 1))));
+                        else sv = __uint_as_float(sc[sl][gi][c >> 1]);
+                        wf = decode8<FMT>(w[sl][gi][c], 0u, sv * gsc, 0.0f);
                     }
                     acc[rr * G + gi] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, xf[c], acc[rr * G + gi], 0, 0, 0);
                 }
             }
         }
-        if (rr + 1 < R) load_w(j, j + 1, rr + 1);      // this step's registers are free: the next round's bytes
+        if (t + DJ < T) load_step(t + DJ);              // this step's registers are free
+        if (t + DJ + 1 == T) finish_loads();
+        __builtin_amdgcn_sched_barrier(0);
     }
 
     // this block may be counted once its reads of `gen` have returned: wave 0's has, like the weights requested before it;
