@@ -1,6 +1,6 @@
-"""GPU: the one-launch organisation of the skinny forward (M <= 16: whole weight rows per block, the low-rank intermediate
-formed once per launch and passed between blocks through device memory of the library) against the oracle and against the
-two-launch organisation on the same inputs.  What could go wrong here beyond arithmetic: a stale intermediate from the
+"""GPU: the one-launch organisation of the skinny forward (whole weight rows per block, the low-rank intermediate formed
+once per launch and passed between blocks through device memory of the library; x slices through LDS for M <= 16,
+streamed for M in 17 .. 64) against the oracle and against the two-launch organisation on the same inputs.  What could go wrong here beyond arithmetic: a stale intermediate from the
 previous launch (the cases change x between calls that share a workspace), slots that are not restored (many calls in a
 row), ragged last blocks, short K ranges per wave, every format's scale addressing."""
 
@@ -66,7 +66,7 @@ def test_one_launch_vs_oracle_and_two_launch(hip_device, organisations, fmt, N, 
     m, w_ref = make_dense_module(fmt, N, K, r, 2 * r, seed=N + K + r, device=hip_device, bias=has_bias)
     A, B = m.lora_A.detach().cpu(), m.lora_B.detach().cpu()
     bias = None if m.bias is None else m.bias.detach().cpu()
-    for M in (1, 3, 8, 16):
+    for M in (1, 3, 8, 16, 17, 32, 40, 64):
         x = gen((M, K), 1.0, 40 + M, torch.bfloat16)
         xd = x.to(hip_device)
         one, two = organisations(lambda: _forward(m, xd))
@@ -98,10 +98,10 @@ def test_low_rank_term_alone_follows_x(hip_device):
     w = qw.c()
     A, B = m.lora_A.detach().contiguous(), m.lora_B.detach().contiguous()
     L = _C.lib()
-    wsb = _workspace_bytes(16, N, K, r)
+    wsb = _workspace_bytes(64, N, K, r)
     ws = torch.empty(wsb, dtype=torch.uint8, device=hip_device)
     st = _C.stream_ptr(hip_device)
-    for i, M in enumerate((1, 16, 2, 9, 1, 16)):
+    for i, M in enumerate((1, 16, 2, 9, 1, 16, 64, 5, 33, 64)):
         x = gen((M, K), 1.0, 900 + i, torch.bfloat16).to(hip_device)
         y = torch.empty(M, N, dtype=torch.bfloat16, device=hip_device)
         with_term = i != 3

@@ -4,8 +4,9 @@
 //
 // A block owns 16 G weight rows over the WHOLE of K: its 8 waves split K eight ways, sum their 16 x 16 tiles through LDS
 // and write the outputs themselves -- no fp32 partial tiles in memory, no second launch.  All of a wave's loads are
-// issued up front and unconditionally (clamped, masked), the x slice first (it reaches LDS while the weight bytes
-// stream), and every weight byte is read once, decoded in registers to the exact bf16 value of the reference decoder
+// unconditional (clamped, masked): the x slice first (it reaches LDS while the weight bytes stream), then the weights
+// as a stream with a few loads per lane in flight; every weight byte is read once, decoded in registers to the exact
+// bf16 value of the reference decoder
 // and fed to v_mfma_f32_16x16x32_bf16 against x fragments (lane (row, quarter) holds 16 or 32 consecutive codes of its
 // row; the K order inside an MFMA is whatever the loads deliver, the x fragments follow the same order).
 //
@@ -28,9 +29,9 @@
 // bounds every wait all the same and turns the block's outputs into NaN.  Sums run in fixed orders (waves ascending,
 // parts ascending): results are identical from call to call.
 //
-// Measured on an MI355X, launches back to back (block_fp8, r = 16, M = 1): 4096->12288 (48 MiB) 12.6 us against 15.3 us
-// for the two-launch organisation (11.5 us without a low-rank term), 4096->4096 7.2 against 8.6, 4096->24576 (96 MiB)
-// 20.0 against 21.6.
+// Measured on an MI355X, launches back to back (block_fp8, r = 16, M = 1): 4096->12288 (48 MiB) 11.4 us against 15.6 us
+// for the two-launch organisation (10.0 us without a low-rank term), 4096->4096 7.4 against 8.8, 4096->24576 (96 MiB)
+// 18.4 against 22.1.
 #include <atomic>
 #include <mutex>
 
