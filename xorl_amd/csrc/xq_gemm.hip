@@ -59,7 +59,7 @@ static int launch_256(const G256Args& f, bool cc, bool grouped, int T, dim3 grid
 }
 
 // compute units of the current device (256 on MI355X), asked once
-static int num_cus() {
+int num_cus() {
     static std::atomic<int> cached{0};
     int c = cached.load(std::memory_order_relaxed);
     if (c > 0) return c;

@@ -96,6 +96,8 @@ int launch_tile_gemm(const xq_weight* w, bool contract_cols, const bf16_t* A, in
                      int r_pad, const bf16_t* bias, bf16_t* C, int64_t ldc, hipStream_t stream, const char* who,
                      float* partial, int64_t partial_bytes, const TwoBanks* two = nullptr);
 
+int num_cus();   // compute units of the current device (xq_gemm.hip)
+
 // skinny-M (M <= 64) forward path, xq_skinny.hip
 bool skinny_supported(const xq_weight* w, int64_t M);
 int64_t skinny_workspace_bytes(int64_t M, int64_t N, int64_t K, int r_pad);

@@ -539,15 +539,16 @@ static bool rows_plan(const xq_weight* w, int64_t M, RowsPlan* p) {
     if (p->MR == 8 && p->njt * eps > 1024) return false;
     // as many row groups per block as give about one block per compute unit, within 24 loads per lane
     const int64_t groups = N / 16;
-    int G = (int)((groups + 255) / 256);
+    const int cus = num_cus();
+    int G = (int)((groups + cus - 1) / cus);
     const int gmax = p->njt <= 4 ? 3 : p->njt <= 8 ? (f8 ? 3 : 2) : p->njt <= 12 ? 2 : 1;
     p->G = G < 1 ? 1 : G > gmax ? gmax : G;
     // more blocks than compute units would run one after the other, each with its own start-up and finish (that costs
     // more than the second launch of the other organisation): twice the rows go to one block in two rounds instead,
     // where the shape allows it
     p->R = 1;
-    if (xq_cdiv(groups, p->G) > 256) {
-        const bool two_rounds = p->G == 3 && p->njt * eps <= 512 && groups % 6 == 0 && groups / 6 <= 256;
+    if (xq_cdiv(groups, p->G) > cus) {
+        const bool two_rounds = p->G == 3 && p->njt * eps <= 512 && groups % 6 == 0 && groups / 6 <= cus;
         if (!two_rounds) return false;
         p->R = 2;
     }
