@@ -7,21 +7,22 @@
 // forward, no atomics, no zeroed buffers, fixed summation orders (deterministic):
 //
 //  1. skinny_split_kernel: a grid of (128-row block) x (K split) tiles.  A block's four waves own 32 weight
-//     rows each and the same K range of at most four 128-element chunks.  ALL loads of a block -- its x slice
-//     and its whole weight tile -- are issued before anything is waited for, so the kernel is one memory round
-//     trip deep, and the number of K splits is chosen so that the whole grid is resident at once (four blocks
-//     per CU at M <= 16, three above).  Weight loads are coalesced (a load instruction covers whole rows of a
-//     chunk) and reach the MFMA layout through a wave-private XOR-swizzled LDS slab; the x slice
-//     [rows, K range] goes through LDS once per block and is shared by the four waves, 32 rows at a time
-//     (M > 32 makes a second pass over the weight registers).  Each block stores its fp32 partial tile to
-//     part[split][M][N]; the first row of blocks carries no weight rows and computes the low-rank
-//     intermediate su = x . A^T for one K split each.
+//     rows each and the same K range of at most four 128-element chunks.  Every load is unconditional and
+//     issued ahead of its use with exactly counted waits: the x slice first, then the weight chunks as a
+//     stream with two chunks in flight (a chunk's registers are requested again once it has been multiplied),
+//     and the number of K splits is chosen so that the whole grid is resident at once (four blocks per CU at
+//     M <= 16, three above).  Weight loads are coalesced (a load instruction covers whole rows of a chunk) and
+//     reach the MFMA layout through a wave-private XOR-swizzled LDS slab; x goes through LDS once per block
+//     and is shared by the four waves: the whole [rows, K range] slice up to 32 rows, chunk by chunk (all 64
+//     rows of 128 elements, two buffers) above, so that a weight chunk is decoded once whatever M is.  Each
+//     block stores its fp32 partial tile to part[split][M][N]; the first row of blocks carries no weight rows
+//     and computes the low-rank intermediate su = x . A^T for one K split each.
 //  2. skinny_epilogue_kernel: sums the splits in order, adds bias and s * su . B^T in fp32 and rounds once
 //     to bf16.
 //
-// Measured per forward on an MI355X, launches back to back (block_fp8, r = 16): 4096->12288 (48 MiB) 15.5 us
-// at M = 1, 22 us at M = 32, 35 us at M = 64; 4096->1024 (4 MiB) 7.3 us at M = 1.  A kernel that only reads
-// the 48 MiB takes 8-9 us.
+// Measured per forward on an MI355X, launches back to back (block_fp8, r = 16): 4096->12288 (48 MiB) 15.6 us
+// at M = 1, 21 us at M = 32, 31 us at M = 64; 4096->1024 (4 MiB) 8 us at M = 1.  A kernel that only reads
+// the 48 MiB takes 8-9 us.  (M <= 16 normally takes the one-launch kernel of xq_skinny_rows.hip instead.)
 #include <stdlib.h>
 
 #include "xq_common.h"
@@ -76,8 +77,10 @@ __device__ __forceinline__ bf16x8 factor_frag(const void* base, int64_t idx, boo
 }
 
 // One block = 128 weight rows x one K split (or, for the leading su blocks, the x . A^T part of one split).
-// MR = 16, 32 or 64 bounds M; at MR = 64 the x rows go through LDS 32 at a time (two passes over the weight
-// registers), so that three blocks still fit a CU.
+// MR = 16, 32 or 64 bounds M.  Up to 32 rows the split's whole x slice is staged in LDS once; at MR = 64 weight
+// blocks take x one 128-element chunk at a time (all 64 rows, two LDS buffers), so that a weight chunk is decoded
+// once and multiplied into both halves of the rows, and three blocks still fit a CU.  (The su blocks at MR = 64
+// stage their x rows 32 at a time.)
 template <int FMT, int MR, int NCH>
 __global__ void __launch_bounds__(256, MR == 16 ? 4 : 3) skinny_split_kernel(SkinnyArgs g) {
     constexpr int TR = MR < 32 ? MR : 32;              // x rows staged at a time
@@ -141,7 +144,7 @@ __global__ void __launch_bounds__(256, MR == 16 ? 4 : 3) skinny_split_kernel(Ski
     // a value the optimiser cannot see through: index arithmetic derived from it inside a loop is redone per
     // iteration instead of being hoisted into (and spilling) registers held across the whole loop
     auto opaque = [](int v) { asm volatile("" : "+v"(v)); return v; };
-    load_x(0, tid);
+    if (MR < 64 || su_block) load_x(0, tid);      // (weight blocks at MR = 64 take x chunk by chunk, see below)
 
     if (su_block) {
         // su part of this split, D[rank][m] (ranks >= r are zero): wave w takes the k16 steps t = w, w+4, ...; the
@@ -229,20 +232,25 @@ __global__ void __launch_bounds__(256, MR == 16 ? 4 : 3) skinny_split_kernel(Ski
     const int nbase = rb * 128 + wave * 32;
     int n = nbase + fr;                                 // the row this lane feeds to the MFMA
     n = n < g.N ? n : g.N - 1;
-    u32x4 w[NCH][NLOAD];
-    uint32_t sc[NCH][NSC];
+    // A single pass over the weights (M <= 32) takes them as a short stream: two chunks in flight, a chunk's registers
+    // refilled with the chunk two further on once it has been multiplied.  A CU accepts loads only as fast as memory
+    // returns them, and with every chunk of its 12 to 16 waves requested at once the waves placed last start late and
+    // have all their decode work left when the stream ends.  (M > 32 takes the same stream with x chunk by chunk, below.)
+    constexpr int DC = NCH > 2 ? 2 : NCH;
+    u32x4 w[DC][NLOAD];
+    uint32_t sc[DC][NSC];
     const bool int4_small_group = FMT == XQ_FMT_INT4 && (g.group & 127) != 0;   // looked up per 8 elements at use
-    {
-        const uint8_t* wp[NLOAD];
+    const uint8_t* wp[NLOAD];
 #pragma unroll
-        for (int i = 0; i < NLOAD; ++i) {
-            int nl = nbase + RPI * i + lrow;
-            nl = nl < g.N ? nl : g.N - 1;
-            wp[i] = g.packed + ((int64_t)nl * g.K) / EB + lpiece * 16;
-        }
-#pragma unroll
-        for (int c = 0; c < NCH; ++c) {
-            const int cc = c_begin + c < c_end ? c_begin + c : c_end - 1;
+    for (int i = 0; i < NLOAD; ++i) {
+        int nl = nbase + RPI * i + lrow;
+        nl = nl < g.N ? nl : g.N - 1;
+        wp[i] = g.packed + ((int64_t)nl * g.K) / EB + lpiece * 16;
+    }
+    auto load_chunk = [&](int c_) {
+        {
+            const int c = c_ % DC;
+            const int cc = c_begin + c_ < c_end ? c_begin + c_ : c_end - 1;
 #pragma unroll
             for (int i = 0; i < NLOAD; ++i) w[c][i] = *(const u32x4*)(wp[i] + (int64_t)cc * (128 / EB));
             if (FMT == XQ_FMT_FP8) sc[c][0] = ((const uint32_t*)g.scales)[(n >> 7) * ((g.K + 127) >> 7) + cc];
@@ -265,6 +273,22 @@ __global__ void __launch_bounds__(256, MR == 16 ? 4 : 3) skinny_split_kernel(Ski
                 }
             }
         }
+    };
+    // M > 32: all 64 x rows of one 128-element chunk at a time, requested just ahead of the chunk's weights (thread t: piece
+    // t % 16 of rows t / 16 + 16 i), so that a chunk is decoded once and multiplied into both halves of the rows
+    u32x4 xcr[4];                                           // one chunk's pieces: requested again as soon as they are in LDS
+    auto load_xc = [&](int c_) {
+        const int cc = c_begin + c_ < c_end ? c_begin + c_ : c_end - 1;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int row = (tid >> 4) + 16 * i;
+            xcr[i] = *(const u32x4*)(g.x + (int64_t)(row < g.M ? row : g.M - 1) * g.ldx + cc * 128 + (tid & 15) * 8);
+        }
+    };
+#pragma unroll
+    for (int c = 0; c < DC; ++c) {
+        if (MR == 64 && c == 0) load_xc(0);
+        load_chunk(c);
     }
 
     // ---- decode + multiply: D[n][m] += deq(W)[n][k] x[m][k].  Each chunk's slab goes through a wave-private LDS
@@ -276,6 +300,88 @@ __global__ void __launch_bounds__(256, MR == 16 ? 4 : 3) skinny_split_kernel(Ski
     unsigned char* wst = smem + (size_t)xrows * XP * 2 + wave * (PPR * 32 * 16);
     float* nf4_lds = (float*)(smem + (size_t)xrows * XP * 2 + 4 * 4096);    // 16 levels behind the slabs
     if (FMT == XQ_FMT_NF4 && tid < 16) nf4_lds[tid] = kNf4Level[tid];        // ordered before its use by stage_x's barrier
+    if constexpr (MR == 64) {
+        constexpr int CXP = 128 + 8;                            // row pitch of an x chunk in LDS, bf16 elements
+        bf16_t* xc = (bf16_t*)smem;                             // [2 buffers][64 rows][CXP]
+        unsigned char* wst2 = smem + 2 * 64 * CXP * 2 + wave * (PPR * 32 * 16);
+        float* nf4_2 = (float*)(smem + 2 * 64 * CXP * 2 + 4 * 4096);
+        if (FMT == XQ_FMT_NF4 && tid < 16) nf4_2[tid] = kNf4Level[tid];     // ordered before its use by the first chunk's barrier
+        const int xrow0 = fr < g.M ? fr : 0, xrow1 = 32 + fr < g.M ? 32 + fr : 0;
+        f32x16 acc0, acc1;
+#pragma unroll
+        for (int q = 0; q < 16; ++q) acc0[q] = acc1[q] = 0.0f;
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) {
+            if (c < nch) {      // block-uniform
+                // x chunk -> buffer c & 1.  Behind this barrier every wave is also done with chunk c - 1, whose buffer
+                // the chunk after this one will overwrite.
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int row = (tid >> 4) + 16 * i;
+                    if (row < g.M) *(u32x4*)(xc + ((c & 1) * 64 + row) * CXP + (tid & 15) * 8) = xcr[i];
+                }
+                if (c + 1 < NCH) load_xc(c + 1);
+                lds_barrier();
+#pragma unroll
+                for (int i = 0; i < NLOAD; ++i) {
+                    const int rl = RPI * i + lrow;
+                    const int sw = FMT == XQ_FMT_FP8 ? (rl >> 1) & 7 : (rl >> 2) & 3;
+                    *(u32x4*)(wst2 + (rl * PPR + (lpiece ^ sw)) * 16) = w[c % DC][i];
+                }
+                __builtin_amdgcn_wave_barrier();
+                const int kc = (c_begin + c) * 128;
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    uint32_t f[4];
+                    if (FMT == XQ_FMT_FP8) {
+                        const u32x4 t = *(const u32x4*)(wst2 + (fr * 8 + ((2 * u + fh) ^ ((fr >> 1) & 7))) * 16);
+                        f[0] = t[0]; f[1] = t[1]; f[2] = t[2]; f[3] = t[3];
+                    } else {
+                        const u32x2 t = *(const u32x2*)(wst2 + (fr * 4 + (u ^ ((fr >> 2) & 3))) * 16 + fh * 8);
+                        f[0] = t[0]; f[1] = t[1];
+                    }
+#pragma unroll
+                    for (int v = 0; v < 2; ++v) {
+                        bf16x8 wf;
+                        if (FMT == XQ_FMT_FP8) {
+                            wf = decode8<FMT>(f[2 * v], f[2 * v + 1], __uint_as_float(sc[c % DC][0]), 0.0f);
+                        } else if (FMT == XQ_FMT_NF4) {
+                            wf = decode8<FMT>(f[v], 0u, __uint_as_float(sc[c % DC][u >> 1]), 0.0f, nf4_2);
+                        } else if (FMT == XQ_FMT_INT4) {
+                            float sv;
+                            if (int4_small_group) sv = load_scale(g.scales, ((int64_t)n * g.K + kc + 32 * u + 16 * fh + 8 * v) / g.group, g.scale_dtype);
+                            else sv = g.scale_dtype == XQ_SCALE_F32 ? __uint_as_float(sc[c % DC][0]) : __uint_as_float(sc[c % DC][0] << 16);
+                            wf = decode8<FMT>(f[v], 0u, sv, -8.0f * sv);
+                        } else {
+                            float sv;
+                            if (g.scale_dtype == XQ_SCALE_E4M3) sv = e4m3_to_f32((uint8_t)(sc[c % DC][u >> 1] >> (8 * (2 * (u & 1) + fh))));
+                            else sv = __uint_as_float(sc[c % DC][u]);
+                            wf = decode8<FMT>(f[v], 0u, sv * gsc, 0.0f);
+                        }
+                        const bf16_t* xb = xc + (c & 1) * 64 * CXP + 32 * u + 16 * fh + 8 * v;
+                        acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf, *(const bf16x8*)(xb + xrow0 * CXP), acc0, 0, 0, 0);
+                        acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf, *(const bf16x8*)(xb + xrow1 * CXP), acc1, 0, 0, 0);
+                    }
+                }
+                __builtin_amdgcn_wave_barrier();
+            }
+            if (c + DC < NCH) load_chunk(c + DC);
+        }
+        float* out = g.partial + (int64_t)split * g.M * g.N;
+#pragma unroll
+        for (int hh = 0; hh < 2; ++hh) {
+            const int m = hh * 32 + fr;
+#pragma unroll
+            for (int q4 = 0; q4 < 4; ++q4) {
+                const int nn = nbase + 8 * q4 + 4 * fh;
+                if (m < g.M && nn < g.N) {
+                    const f32x16& a = hh ? acc1 : acc0;
+                    *(f32x4*)(out + (int64_t)m * g.N + nn) = f32x4{a[q4 * 4], a[q4 * 4 + 1], a[q4 * 4 + 2], a[q4 * 4 + 3]};
+                }
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int h = 0; h < NPASS; ++h) {
         if (h * 32 < g.M) {
@@ -297,7 +403,7 @@ __global__ void __launch_bounds__(256, MR == 16 ? 4 : 3) skinny_split_kernel(Ski
                     for (int i = 0; i < NLOAD; ++i) {
                         const int rl = RPI * i + lrow;
                         const int sw = FMT == XQ_FMT_FP8 ? (rl >> 1) & 7 : (rl >> 2) & 3;
-                        *(u32x4*)(wst + (rl * PPR + (lpiece ^ sw)) * 16) = w[c][i];
+                        *(u32x4*)(wst + (rl * PPR + (lpiece ^ sw)) * 16) = w[c % DC][i];
                     }
                     __builtin_amdgcn_wave_barrier();
                     const int kc = (c_begin + c) * 128;
@@ -315,18 +421,18 @@ __global__ void __launch_bounds__(256, MR == 16 ? 4 : 3) skinny_split_kernel(Ski
                         for (int v = 0; v < 2; ++v) {
                             bf16x8 wf;
                             if (FMT == XQ_FMT_FP8) {
-                                wf = decode8<FMT>(f[2 * v], f[2 * v + 1], __uint_as_float(sc[c][0]), 0.0f);
+                                wf = decode8<FMT>(f[2 * v], f[2 * v + 1], __uint_as_float(sc[c % DC][0]), 0.0f);
                             } else if (FMT == XQ_FMT_NF4) {
-                                wf = decode8<FMT>(f[v], 0u, __uint_as_float(sc[c][u >> 1]), 0.0f, nf4_lds);   // group 64: k = 32u + ..
+                                wf = decode8<FMT>(f[v], 0u, __uint_as_float(sc[c % DC][u >> 1]), 0.0f, nf4_lds);   // group 64: k = 32u + ..
                             } else if (FMT == XQ_FMT_INT4) {
                                 float sv;
                                 if (int4_small_group) sv = load_scale(g.scales, ((int64_t)n * g.K + kc + 32 * u + 16 * fh + 8 * v) / g.group, g.scale_dtype);
-                                else sv = g.scale_dtype == XQ_SCALE_F32 ? __uint_as_float(sc[c][0]) : __uint_as_float(sc[c][0] << 16);
+                                else sv = g.scale_dtype == XQ_SCALE_F32 ? __uint_as_float(sc[c % DC][0]) : __uint_as_float(sc[c % DC][0] << 16);
                                 wf = decode8<FMT>(f[v], 0u, sv, -8.0f * sv);
                             } else {
                                 float sv;   // block scale 2u + fh of the chunk
-                                if (g.scale_dtype == XQ_SCALE_E4M3) sv = e4m3_to_f32((uint8_t)(sc[c][u >> 1] >> (8 * (2 * (u & 1) + fh))));
-                                else sv = __uint_as_float(sc[c][u]);
+                                if (g.scale_dtype == XQ_SCALE_E4M3) sv = e4m3_to_f32((uint8_t)(sc[c % DC][u >> 1] >> (8 * (2 * (u & 1) + fh))));
+                                else sv = __uint_as_float(sc[c % DC][u]);
                                 wf = decode8<FMT>(f[v], 0u, sv * gsc, 0.0f);
                             }
                             const bf16x8 xf = *(const bf16x8*)(xs + xrow * XP + c * 128 + 32 * u + 16 * fh + 8 * v);
@@ -335,6 +441,7 @@ __global__ void __launch_bounds__(256, MR == 16 ? 4 : 3) skinny_split_kernel(Ski
                     }
                     __builtin_amdgcn_wave_barrier();
                 }
+                if (c + DC < NCH) load_chunk(c + DC);      // this chunk's registers are free (single pass only: DC == NCH otherwise)
             }
             // fp32 partial tile: lane (m = 32h + fr) holds 4 consecutive weight rows per register quad
             float* out = g.partial + (int64_t)split * g.M * g.N;
@@ -510,7 +617,8 @@ static int launch_skinny_split(const xq_weight* w, const bf16_t* x, int64_t ldx,
     g.su_part = (float*)((char*)workspace + al256((int64_t)p.splits * M * N * 4));
     g.lora_A = rp ? lora_A : nullptr; g.lora_f32 = lora_dtype == XQ_DT_F32; g.r = r; g.r_pad = rp;
     const dim3 grid((unsigned)p.splits, (unsigned)(p.row_blocks + g.su_blocks));
-    const size_t lds = (size_t)(M < 32 ? M : 32) * g.xp * 2 + 4 * 4096 + 64;   // x slice + the four weight slabs (or the su reduction buffer) + nf4 levels
+    size_t lds = (size_t)(M < 32 ? M : 32) * g.xp * 2 + 4 * 4096 + 64;   // x slice + the four weight slabs (or the su reduction buffer) + nf4 levels
+    if (M > 32 && lds < 2 * 64 * 136 * 2 + 4 * 4096 + 64) lds = 2 * 64 * 136 * 2 + 4 * 4096 + 64;   // two x chunk buffers of 64 rows
 
     SkinnyEpiArgs e;
     e.partial = g.partial; e.su_part = g.su_part; e.splits = p.splits; e.su_parts = rp ? p.splits : 0;
