@@ -457,95 +457,154 @@ __global__ void __launch_bounds__(256, MR == 16 ? 4 : 3) skinny_split_kernel(Ski
 }
 
 // y[m][n..n+3] = sum_s part[s][m][n..] + bias + su_scale * sum_j su[m][j] * B[n][j], su = sum of the su parts.
-// One wave per output row m (up to four rows per block), a lane per 4 consecutive columns; nothing is shared
-// between waves.  Loads are unconditional (indices past the end are clamped, their values masked to zero), so
-// that a wave's su parts, partial tiles and B rows are all in flight together.  Every sum runs in a fixed
-// order: parts p = g, g+4, ... per lane group g, then the four groups; splits ascending.
+// One wave per output row m (up to four rows per block), a lane per 4 consecutive columns.  The block's 256 B rows
+// (64 B per output column and 16 ranks: twice the bytes of a row's partial tiles of eight splits) are fetched once,
+// coalesced, and shared by its waves through LDS.  Loads are unconditional (indices past the end are clamped, their
+// values masked to zero or never stored) and the first batch of each kind is issued before anything is waited for,
+// so that the B rows, partial tiles and su parts are all in flight together.  Every sum runs in a fixed order:
+// parts p = g, g+4, ... per lane group g, then the four groups; splits ascending.
 // RT = 16-rank tiles of the low-rank term (0 = none); VEC = B is fp32 with r % 4 == 0 (16-byte row pieces).
 template <int RT, bool VEC>
 __global__ void __launch_bounds__(256) skinny_epilogue_kernel(SkinnyEpiArgs g) {
     // all arguments in scalar registers after one round trip (see skinny_split_kernel)
     asm volatile("" ::"s"(g.partial), "s"(g.su_part), "s"(g.splits), "s"(g.su_parts), "s"(g.M), "s"(g.N), "s"(g.lora_B),
                  "s"(g.lora_f32), "s"(g.r), "s"(g.r_pad), "s"(g.su_scale), "s"(g.bias), "s"(g.y), "s"(g.ldy));
-    const int lane = threadIdx.x & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int m = blockIdx.y * 4 + wave;
-    if (m >= g.M) return;                                        // wave-uniform
-    int n = (blockIdx.x * 64 + lane) * 4;
+    // B tile of rank tile jt: [64 lanes][16 pieces of 4 ranks] fp32 (piece 4 e + q = ranks 4q .. 4q+3 of the lane's column
+    // e), the pieces of a lane XOR-swizzled with the lane number: conflict-free 16-byte writes and reads
+    __shared__ __attribute__((aligned(16))) float bt[RT > 0 ? RT : 1][64 * 64];
+    const int tid = threadIdx.x, lane = tid & 63, nthreads = blockDim.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int mraw = blockIdx.y * 4 + wave;
+    const int m = mraw < g.M ? mraw : g.M - 1;                   // a wave past M repeats the last row and stores nothing
+    const int n0 = blockIdx.x * 256;
+    int n = n0 + lane * 4;
     const bool nvalid = n < g.N;                                 // N % 4 == 0: a lane's 4 columns are all in or all out
     n = nvalid ? n : 0;
     const int j = lane & 15, pg = lane >> 4;
 
-    // su parts: lane (j, pg) sums parts pg, pg+4, ... of rank j of each tile
+    // ---- issue: B pieces (piece q = 4 ranks of column n0 + q / 4), then the first 16 splits, then the first 32 su parts
+    constexpr int NQ = RT > 0 ? RT * 4 : 1;                       // pieces per thread with 256 threads
+    f32x4 bq[NQ];
+    if (RT > 0) {
+#pragma unroll
+        for (int jt = 0; jt < RT; ++jt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int q = tid + i * nthreads;                 // blocks of fewer than 4 waves go round again below
+                const int col = n0 + (q >> 2) < g.N ? n0 + (q >> 2) : 0, jr = jt * 16 + 4 * (q & 3);
+                f32x4 t = {0.0f, 0.0f, 0.0f, 0.0f};
+                if (VEC) {
+                    t = *(const f32x4*)((const float*)g.lora_B + (int64_t)col * g.r + (jr < g.r ? jr : 0));
+                } else {
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        const int64_t idx = (int64_t)col * g.r + (jr + c < g.r ? jr + c : 0);
+                        t[c] = g.lora_f32 ? ((const float*)g.lora_B)[idx] : bf16_to_f32(((const bf16_t*)g.lora_B)[idx]);
+                    }
+                }
+                bq[jt * 4 + i] = t;
+            }
+    }
+    const float* pp = g.partial + (int64_t)m * g.N + n;
+    const int64_t sstride = (int64_t)g.M * g.N;
+    f32x4 pt[16];
+#pragma unroll
+    for (int u = 0; u < 16; ++u) pt[u] = *(const f32x4*)(pp + (int64_t)(u < g.splits ? u : g.splits - 1) * sstride);
+    const int64_t pstride = (int64_t)g.M * g.r_pad;
+    float st[RT > 0 ? RT : 1][8];
+#pragma unroll
+    for (int jt = 0; jt < RT; ++jt)
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int pi = pg + 4 * u;
+            st[jt][u] = g.su_part[(int64_t)(pi < g.su_parts ? pi : g.su_parts - 1) * pstride + (int64_t)m * g.r_pad + jt * 16 + j];
+        }
+
+    // ---- B pieces -> LDS
+    if (RT > 0) {
+#pragma unroll
+        for (int jt = 0; jt < RT; ++jt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int q = tid + i * nthreads;
+                if (q < 1024) *(f32x4*)(&bt[jt][(q >> 4) * 64 + ((q ^ (q >> 4)) & 15) * 4]) = bq[jt * 4 + i];
+            }
+        // blocks of one or two waves (M < 4): the pieces the first four rounds did not reach
+        for (int q = tid + 4 * nthreads; q < 1024; q += nthreads) {
+            const int col = n0 + (q >> 2) < g.N ? n0 + (q >> 2) : 0;
+#pragma unroll
+            for (int jt = 0; jt < RT; ++jt) {
+                const int jr = jt * 16 + 4 * (q & 3);
+                f32x4 t;
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    const int64_t idx = (int64_t)col * g.r + (jr + c < g.r ? jr + c : 0);
+                    t[c] = g.lora_f32 ? ((const float*)g.lora_B)[idx] : bf16_to_f32(((const bf16_t*)g.lora_B)[idx]);
+                }
+                *(f32x4*)(&bt[jt][(q >> 4) * 64 + ((q ^ (q >> 4)) & 15) * 4]) = t;
+            }
+        }
+        __syncthreads();
+    }
+
+    // ---- su parts: lane (j, pg) sums parts pg, pg+4, ... of rank j of each tile
     float sv[RT > 0 ? RT : 1];
 #pragma unroll
-    for (int jt = 0; jt < RT; ++jt) sv[jt] = 0.0f;
-    const int64_t pstride = (int64_t)g.M * g.r_pad;
-    for (int p0 = 0; p0 < g.su_parts; p0 += 32) {
-        float t[RT > 0 ? RT : 1][8];
+    for (int jt = 0; jt < RT; ++jt) {
+        sv[jt] = 0.0f;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) sv[jt] += pg + 4 * u < g.su_parts ? st[jt][u] : 0.0f;
+    }
+    for (int p0 = 32; p0 < g.su_parts; p0 += 32) {
 #pragma unroll
         for (int jt = 0; jt < RT; ++jt)
 #pragma unroll
             for (int u = 0; u < 8; ++u) {
                 const int pi = p0 + pg + 4 * u;
-                t[jt][u] = g.su_part[(int64_t)(pi < g.su_parts ? pi : g.su_parts - 1) * pstride + (int64_t)m * g.r_pad + jt * 16 + j];
+                st[jt][u] = g.su_part[(int64_t)(pi < g.su_parts ? pi : g.su_parts - 1) * pstride + (int64_t)m * g.r_pad + jt * 16 + j];
             }
 #pragma unroll
         for (int jt = 0; jt < RT; ++jt)
 #pragma unroll
-            for (int u = 0; u < 8; ++u) sv[jt] += p0 + pg + 4 * u < g.su_parts ? t[jt][u] : 0.0f;
+            for (int u = 0; u < 8; ++u) sv[jt] += p0 + pg + 4 * u < g.su_parts ? st[jt][u] : 0.0f;
     }
-    // partial tiles
+    // ---- partial tiles
     f32x4 o = {0.0f, 0.0f, 0.0f, 0.0f};
-    const float* pp = g.partial + (int64_t)m * g.N + n;
-    const int64_t sstride = (int64_t)g.M * g.N;
-    for (int s0 = 0; s0 < g.splits; s0 += 16) {
-        f32x4 t[16];
 #pragma unroll
-        for (int u = 0; u < 16; ++u) t[u] = *(const f32x4*)(pp + (int64_t)(s0 + u < g.splits ? s0 + u : g.splits - 1) * sstride);
+    for (int u = 0; u < 16; ++u) {
+        if (u < g.splits) o += pt[u];                             // wave-uniform
+    }
+    for (int s0 = 16; s0 < g.splits; s0 += 16) {
+#pragma unroll
+        for (int u = 0; u < 16; ++u) pt[u] = *(const f32x4*)(pp + (int64_t)(s0 + u < g.splits ? s0 + u : g.splits - 1) * sstride);
 #pragma unroll
         for (int u = 0; u < 16; ++u) {
-            if (s0 + u < g.splits) o += t[u];                     // wave-uniform
+            if (s0 + u < g.splits) o += pt[u];
         }
     }
-    // low-rank term, 16 ranks at a time
+    // ---- low-rank term, 16 ranks at a time; ranks >= r hold zeros in su (and finite values in the B tile)
 #pragma unroll
     for (int jt = 0; jt < RT; ++jt) {
-        float bv[4][16];
-        if (VEC) {
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const int jr = jt * 16 + 4 * q;              // r % 4 == 0: a group of 4 ranks is all in or all out
-                    const f32x4 t = *(const f32x4*)((const float*)g.lora_B + (int64_t)(n + e) * g.r + (jr < g.r ? jr : 0));
-#pragma unroll
-                    for (int c = 0; c < 4; ++c) bv[e][4 * q + c] = jr < g.r ? t[c] : 0.0f;
-                }
-        } else {
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-#pragma unroll
-                for (int jj = 0; jj < 16; ++jj) {
-                    const int jr = jt * 16 + jj;
-                    const int64_t idx = (int64_t)(n + e) * g.r + (jr < g.r ? jr : 0);
-                    const float t = g.lora_f32 ? ((const float*)g.lora_B)[idx] : bf16_to_f32(((const bf16_t*)g.lora_B)[idx]);
-                    bv[e][jj] = jr < g.r ? t : 0.0f;
-                }
-        }
         float tot = __shfl(sv[jt], j, 64);
         tot += __shfl(sv[jt], 16 + j, 64);
         tot += __shfl(sv[jt], 32 + j, 64);
         tot += __shfl(sv[jt], 48 + j, 64);
         tot *= g.su_scale;                                        // lane l holds su[m][jt*16 + (l & 15)], zero for ranks >= r
+        if (jt * 16 + j >= g.r) tot = 0.0f;
 #pragma unroll
-        for (int jj = 0; jj < 16; ++jj) {
-            const float sj = __shfl(tot, jj, 64);
+        for (int q = 0; q < 4; ++q) {
+            f32x4 bv[4];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) o[e] = __builtin_fmaf(sj, bv[e][jj], o[e]);
+            for (int e = 0; e < 4; ++e) bv[e] = *(const f32x4*)(&bt[jt][lane * 64 + (((e * 4 + q) ^ lane) & 15) * 4]);
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const float sj = __shfl(tot, 4 * q + c, 64);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) o[e] = __builtin_fmaf(sj, bv[e][c], o[e]);
+            }
         }
     }
-    if (!nvalid) return;
+    if (!nvalid || mraw >= g.M) return;
     if (g.bias) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) o[e] += bf16_to_f32(g.bias[n + e]);
