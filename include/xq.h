@@ -150,6 +150,32 @@ int xq_linear_fwd(const xq_weight* w, const void* x, int64_t ldx, int64_t M,
                   const void* bias_bf16, void* y, int64_t ldy, void* su_out,
                   void* workspace, int64_t workspace_bytes, void* stream);
 
+/* Several forwards that share x: y_i = x . deq(W_i)^T + bias_i + s_i * (x . A_i^T) . B_i^T, i < n_jobs <= 4.
+ * Replaces the separate module calls of the reference's attention and MLP blocks
+ * on one input (q_proj / k_proj / v_proj: src/xorl/models/layers/attention/multi_head_attention.py:93-95;
+ * gate_proj / up_proj: src/xorl/models/transformers/qwen3/modeling_qwen3.py:75-76) when a model keeps them as
+ * separate modules (unfuse_for_tp); each forward is the one of qlora/modules/linear.py:369-385.
+ * All weights contract over the same K.  For M <= 16, with weights of one
+ * format that fit the one-launch skinny kernel, all forwards run as ONE launch
+ * (the grid holds each forward's blocks one after the other); otherwise they run
+ * one after the other as xq_linear_fwd(..., su_out = NULL).  Results are
+ * bit-identical to separate xq_linear_fwd calls either way.
+ * workspace: xq_linear_fwd_multi_workspace_bytes(...) bytes, 256-byte aligned. */
+#define XQ_LINEAR_MULTI_MAX 4
+typedef struct xq_linear_job {
+    const xq_weight* w;
+    const void* lora_A;     /* [r, K] in lora_dtype */
+    const void* lora_B;     /* [N, r] in lora_dtype */
+    int32_t r;              /* 0 .. 64 */
+    float scaling;
+    const void* bias_bf16;  /* [N] or NULL */
+    void* y;                /* bf16 [M, N], row stride ldy */
+    int64_t ldy;
+} xq_linear_job;
+int64_t xq_linear_fwd_multi_workspace_bytes(const xq_linear_job* jobs, int n_jobs, int64_t M);
+int xq_linear_fwd_multi(const xq_linear_job* jobs, int n_jobs, const void* x, int64_t ldx, int64_t M, int lora_dtype,
+                        void* workspace, int64_t workspace_bytes, void* stream);
+
 /* xq_linear_fwd for callers that cannot allocate device memory or be handed a
  * workspace: code under HIP-graph capture, tight rollout / serving loops,
  * harnesses that forbid allocation.  No counterpart in the reference (its

@@ -40,6 +40,15 @@ class XqWeight(ctypes.Structure):
     ]
 
 
+class XqLinearJob(ctypes.Structure):
+    """xq_linear_job of include/xq.h: one of the forwards of xq_linear_fwd_multi."""
+    _fields_ = [("w", ctypes.POINTER(XqWeight)), ("lora_A", ctypes.c_void_p), ("lora_B", ctypes.c_void_p), ("r", ctypes.c_int32),
+                ("scaling", ctypes.c_float), ("bias_bf16", ctypes.c_void_p), ("y", ctypes.c_void_p), ("ldy", ctypes.c_int64)]
+
+
+XQ_LINEAR_MULTI_MAX = 4
+
+
 class XqGroupedLora(ctypes.Structure):
     _fields_ = [("A", ctypes.c_void_p * 3), ("B", ctypes.c_void_p * 3), ("A_experts", ctypes.c_int32 * 3),
                 ("B_experts", ctypes.c_int32 * 3), ("dtype", ctypes.c_int32), ("r", ctypes.c_int32),
@@ -85,6 +94,10 @@ _SIGNATURES = {
     "xq_linear_workspace_bytes": (_I64, [_I64, _I64, _I64, _INT]),
     # w, x, ldx, M, A, B, lora_dtype, r, scaling, bias, y, ldy, su_out, ws, ws_bytes, stream
     "xq_linear_fwd": (_INT, [_W, _P, _I64, _I64, _P, _P, _INT, _INT, _F, _P, _P, _I64, _P, _P, _I64, _P]),
+    # jobs, n_jobs, M
+    "xq_linear_fwd_multi_workspace_bytes": (_I64, [_P, _INT, _I64]),
+    # jobs, n_jobs, x, ldx, M, lora_dtype, ws, ws_bytes, stream
+    "xq_linear_fwd_multi": (_INT, [_P, _INT, _P, _I64, _I64, _INT, _P, _I64, _P]),
     "xq_static_scratch_bytes": (_I64, []),
     # w, x, ldx, M, A, B, lora_dtype, r, scaling, bias, y, ldy, stream
     "xq_linear_fwd_static": (_INT, [_W, _P, _I64, _I64, _P, _P, _INT, _INT, _F, _P, _P, _I64, _P]),

@@ -493,6 +493,69 @@ static int static_scratch(void** out, const char* who) {
 
 extern "C" int64_t xq_static_scratch_bytes(void) { return XQ_STATIC_SCRATCH_BYTES; }
 
+extern "C" int64_t xq_linear_fwd_multi_workspace_bytes(const xq_linear_job* jobs, int n_jobs, int64_t M) {
+    int64_t need = 256 * 8;
+    if (!jobs) return need;
+    for (int i = 0; i < n_jobs; ++i) {
+        if (!jobs[i].w) continue;
+        const int64_t b = xq_linear_workspace_bytes(M, jobs[i].w->rows, jobs[i].w->cols, jobs[i].r);
+        if (b > need) need = b;
+    }
+    return need;
+}
+
+extern "C" int xq_linear_fwd_multi(const xq_linear_job* jobs, int n_jobs, const void* x, int64_t ldx, int64_t M, int lora_dtype,
+                                   void* workspace, int64_t workspace_bytes, void* stream_) {
+    XQ_REQUIRE(jobs && n_jobs >= 1 && n_jobs <= XQ_LINEAR_MULTI_MAX, "xq_linear_fwd_multi: %d forwards (1 .. %d are taken)", n_jobs,
+               XQ_LINEAR_MULTI_MAX);
+    XQ_REQUIRE(lora_dtype == XQ_DT_F32 || lora_dtype == XQ_DT_BF16, "xq_linear_fwd_multi: bad lora_dtype");
+    for (int i = 0; i < n_jobs; ++i) {
+        XQ_REQUIRE(jobs[i].w, "xq_linear_fwd_multi: forward %d has no weight", i);
+        int rc = check_dense(jobs[i].w, "xq_linear_fwd_multi");
+        if (rc) return rc;
+        XQ_REQUIRE(jobs[i].w->cols == jobs[0].w->cols, "xq_linear_fwd_multi: forward %d contracts over %lld features, forward 0 over %lld", i,
+                   (long long)jobs[i].w->cols, (long long)jobs[0].w->cols);
+        XQ_REQUIRE(jobs[i].r >= 0 && jobs[i].r <= 64, "xq_linear_fwd_multi: LoRA rank %d out of range [0, 64]", jobs[i].r);
+        XQ_REQUIRE(jobs[i].r == 0 || (jobs[i].lora_A && jobs[i].lora_B), "xq_linear_fwd_multi: LoRA factors are NULL");
+        XQ_REQUIRE(M == 0 || jobs[i].y, "xq_linear_fwd_multi: NULL output pointer");
+        XQ_REQUIRE(M == 0 || (jobs[i].ldy % 8 == 0 && xq_aligned(jobs[i].y, 16)), "xq_linear_fwd_multi: y rows must be 16-byte aligned");
+    }
+    XQ_REQUIRE(M >= 0 && (M == 0 || x), "xq_linear_fwd_multi: NULL activation pointer");
+    if (M == 0) return XQ_OK;
+    hipStream_t stream = (hipStream_t)stream_;
+    XQ_REQUIRE(workspace && xq_aligned(workspace, 256) && workspace_bytes >= xq_linear_fwd_multi_workspace_bytes(jobs, n_jobs, M),
+               "xq_linear_fwd_multi: workspace missing, misaligned or smaller than xq_linear_fwd_multi_workspace_bytes()");
+    // decode shapes that fit the whole-row kernel: every forward in one launch
+    if (g_skinny_enabled && skinny_rows_enabled() && n_jobs > 1 && ldx % 8 == 0 && xq_aligned(x, 16)) {
+        SkinnyRowsJob rj[XQ_LINEAR_MULTI_MAX];
+        double bytes = 2.0 * M * jobs[0].w->cols;
+        bool ok = true;
+        for (int i = 0; i < n_jobs; ++i) {
+            const xq_weight* w = jobs[i].w;
+            rj[i] = SkinnyRowsJob{w, jobs[i].lora_A, jobs[i].lora_B, jobs[i].r, jobs[i].scaling, (const bf16_t*)jobs[i].bias_bf16,
+                                  (bf16_t*)jobs[i].y, jobs[i].ldy};
+            ok = ok && skinny_supported(w, M) && xq_aligned(w->packed, 16);
+            bytes += (double)xq_packed_bytes_per_expert(w) + (double)xq_scale_bytes_per_expert(w) + 2.0 * M * w->rows +
+                     4.0 * jobs[i].r * (w->cols + w->rows);
+        }
+        if (ok && skinny_rows_multi_supported(rj, n_jobs, M, lora_dtype)) {
+            const bool timed = xq_profile_mark_begin(stream, bytes);
+            const int rc = launch_skinny_rows_multi(rj, n_jobs, (const bf16_t*)x, ldx, M, workspace, stream);
+            if (timed) xq_profile_mark_end(stream);
+            if (rc) return rc;
+            XQ_CHECK_LAUNCH("skinny forwards");
+            return XQ_OK;
+        }
+    }
+    // otherwise one after the other (the workspace is reused: the launches are ordered by the stream)
+    for (int i = 0; i < n_jobs; ++i) {
+        const int rc = xq_linear_fwd(jobs[i].w, x, ldx, M, jobs[i].lora_A, jobs[i].lora_B, lora_dtype, jobs[i].r, jobs[i].scaling,
+                                     jobs[i].bias_bf16, jobs[i].y, jobs[i].ldy, nullptr, workspace, workspace_bytes, stream_);
+        if (rc) return rc;
+    }
+    return XQ_OK;
+}
+
 extern "C" int xq_linear_fwd_static(const xq_weight* w, const void* x, int64_t ldx, int64_t M, const void* lora_A,
                                     const void* lora_B, int lora_dtype, int r, float scaling, const void* bias_bf16,
                                     void* y, int64_t ldy, void* stream_) {

@@ -45,6 +45,7 @@ __device__ __forceinline__ bf16x8 decode8(uint32_t w0, uint32_t w1, float s0, fl
 }
 
 void set_skinny_rows(int enabled);
+bool skinny_rows_enabled();
 
 // ---- one-launch organisation (xq_skinny_rows.hip)
 // true when the shape, format and LoRA operands fit it; the caller falls back to the split organisation otherwise
@@ -52,5 +53,21 @@ bool skinny_rows_supported(const xq_weight* w, int64_t M, const void* lora_A, co
 // `slot_key` names the caller's scratch (its workspace pointer): calls with different keys may overlap on a device
 int launch_skinny_rows(const xq_weight* w, const bf16_t* x, int64_t ldx, int64_t M, const void* lora_A, const void* lora_B, int r,
                        float scaling, const bf16_t* bias, bf16_t* y, int64_t ldy, const void* slot_key, hipStream_t stream);
+
+// several forwards that share x (same format, K and M) as one launch of the same kernel; each forward has its own slot,
+// keyed by addresses 256 bytes apart from `slot_key` (the caller's workspace holds at least 256 bytes per forward)
+struct SkinnyRowsJob {
+    const xq_weight* w;
+    const void* lora_A;
+    const void* lora_B;
+    int r;
+    float scaling;
+    const bf16_t* bias;
+    bf16_t* y;
+    int64_t ldy;
+};
+bool skinny_rows_multi_supported(const SkinnyRowsJob* jobs, int n_jobs, int64_t M, int lora_dtype);
+int launch_skinny_rows_multi(const SkinnyRowsJob* jobs, int n_jobs, const bf16_t* x, int64_t ldx, int64_t M, const void* slot_key,
+                             hipStream_t stream);
 
 }  // namespace xq

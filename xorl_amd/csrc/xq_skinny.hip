@@ -713,6 +713,7 @@ static int launch_skinny_split(const xq_weight* w, const bf16_t* x, int64_t ldx,
 // test switch, to be set while no other thread is inside the library
 static int g_skinny_rows = [] { const char* e = getenv("XQ_SKINNY_ROWS"); return e ? atoi(e) : 1; }();
 void set_skinny_rows(int enabled) { g_skinny_rows = enabled; }
+bool skinny_rows_enabled() { return g_skinny_rows != 0; }
 
 int launch_skinny(const xq_weight* w, const bf16_t* x, int64_t ldx, int64_t M, const void* lora_A, const void* lora_B,
                   int lora_dtype, int r, float scaling, const bf16_t* bias, bf16_t* y, int64_t ldy, void* workspace,

@@ -79,8 +79,9 @@ struct SkinnyRowsArgs {
 // per lane: 64 elements of K per row for fp8, 128 for the 4-bit formats); MR: bound on M (x rows kept in registers on
 // their way to LDS); R: rounds -- a block walks R sets of G row groups, each step's registers refilled for the next
 // round as soon as the step has been multiplied, so the weight stream never stops (N % (16 G R) == 0 when R > 1)
+// (`bx` of `nb`: the block's place among the blocks of its forward -- the grid of a launch holds one forward or several)
 template <int FMT, int G, int NJ, int MR, int R>
-__global__ void __launch_bounds__(512, 1) skinny_rows_kernel(SkinnyRowsArgs g) {
+__device__ __forceinline__ void skinny_rows_body(const SkinnyRowsArgs& g, const int bx, const int nb) {
     constexpr bool F8 = FMT == XQ_FMT_FP8;
     constexpr int EPS = F8 ? 64 : 128;                 // K elements of a row per load step
     constexpr int MPS = EPS / 32;                      // MFMAs per step and row group
@@ -98,7 +99,7 @@ __global__ void __launch_bounds__(512, 1) skinny_rows_kernel(SkinnyRowsArgs g) {
     const int ks = g.K >> 3;                    // K elements per wave
     const int k0 = wave * ks;
     const int nj = ks / EPS;                    // load steps of this launch, 1 .. NJ
-    const int n0 = blockIdx.x * (16 * G * R);
+    const int n0 = bx * (16 * G * R);
     const int XP = g.xpitch;
     unsigned char* slab = smem + wave * g.slab;
     float* su_tot = (float*)(smem + 8 * g.slab);           // [16 m][16 j], then a flag
@@ -106,7 +107,7 @@ __global__ void __launch_bounds__(512, 1) skinny_rows_kernel(SkinnyRowsArgs g) {
     float* su_red = b_tile + 96 * 20;                       // [4 waves][256]: the tiles of an su part
     int* su_flag = (int*)(su_red + 4 * 256);                // [0 .. 3]: wave 4 + w has written its tile; [4]: wave 4 is done with `gen`
     const bool lora = g.nsu > 0;
-    const bool su_block = (int)blockIdx.x < g.nsu;          // nsu <= gridDim.x (checked on the host)
+    const bool su_block = bx < g.nsu;          // nsu <= nb (checked on the host)
     // LDS traffic of the block is ordered by this barrier; __syncthreads() would also wait for every load in flight
     auto lds_barrier = [&]() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
 
@@ -120,7 +121,7 @@ __global__ void __launch_bounds__(512, 1) skinny_rows_kernel(SkinnyRowsArgs g) {
     // carries it as its tag); everywhere wave 0 asks for it, past the caches, behind its weights (needed when it collects;
     // loads return in order and this one is slow, so it must not sit in front of them).
     uint32_t gen = 0;
-    uint32_t* ctl = g.slot + kSlotCtl + (blockIdx.x % kCtlCopies) * kCtlStride;      // this block's copy of gen; started: + kCtlCopies * kCtlStride
+    uint32_t* ctl = g.slot + kSlotCtl + (bx % kCtlCopies) * kCtlStride;      // this block's copy of gen; started: + kCtlCopies * kCtlStride
 
     // the operand tie keeps the compiler from moving the add ahead of the point where `gen` is in its register
     auto count_block = [&]() {
@@ -144,7 +145,7 @@ __global__ void __launch_bounds__(512, 1) skinny_rows_kernel(SkinnyRowsArgs g) {
         // microseconds here, and every block's finish waits for the sums.  (Were the value stale after all, the tag
         // would not be the one the collectors look for: they would give up and write NaN, never take old sums.)
         if (wave == 4) gen = __hip_atomic_load(ctl, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-        const int kb = blockIdx.x * kSuPartK + (wave - 4) * 128 + kq * 8;
+        const int kb = bx * kSuPartK + (wave - 4) * 128 + kq * 8;
         const float* ap = g.lora_A + (int64_t)(rn < g.r ? rn : 0) * g.K + kb;
         const bf16_t* xp = g.x + (int64_t)(rn < g.M ? rn : g.M - 1) * g.ldx + kb;
 #pragma unroll
@@ -207,7 +208,7 @@ __global__ void __launch_bounds__(512, 1) skinny_rows_kernel(SkinnyRowsArgs g) {
                     float s = 0.0f;
 #pragma unroll
                     for (int ww = 0; ww < 4; ++ww) s += su_red[ww * 256 + q * 64 + lane];
-                    __hip_atomic_store((uint64_t*)g.slot + blockIdx.x * 256 + q * 64 + lane, ((uint64_t)(gen + 1) << 32) | __float_as_uint(s),
+                    __hip_atomic_store((uint64_t*)g.slot + bx * 256 + q * 64 + lane, ((uint64_t)(gen + 1) << 32) | __float_as_uint(s),
                                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 }
             }
@@ -369,7 +370,7 @@ __global__ void __launch_bounds__(512, 1) skinny_rows_kernel(SkinnyRowsArgs g) {
     // ---- wave 0 (its loads were requested first, so it gets here first) collects the su parts while the other waves are
     // still streaming: entry q * 64 + l of a part is su[j = 4 (l >> 4) + q][m = l & 15]
     if (lora && wave == 0) {
-        const bool closer = blockIdx.x == gridDim.x - 1;      // this block moves the launch count on
+        const bool closer = bx == nb - 1;      // this block moves the launch count on
         float s[4];
         int spins = 0;
         bool missing, open = closer;
@@ -413,7 +414,7 @@ __global__ void __launch_bounds__(512, 1) skinny_rows_kernel(SkinnyRowsArgs g) {
             if (open) {
 #pragma unroll
                 for (int d = 32; d >= 1; d >>= 1) started += __shfl_xor(started, d, 64);
-                if (started == gridDim.x) {
+                if (started == (uint32_t)nb) {
                     // every block has read `gen`: the next launch counts from gen + 1
                     if (lane < kCtlCopies) {
                         __hip_atomic_store(g.slot + kSlotCtl + lane * kCtlStride, gen + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -473,6 +474,26 @@ __global__ void __launch_bounds__(512, 1) skinny_rows_kernel(SkinnyRowsArgs g) {
     }
 }
 
+
+template <int FMT, int G, int NJ, int MR, int R>
+__global__ void __launch_bounds__(512, 1) skinny_rows_kernel(SkinnyRowsArgs g) {
+    skinny_rows_body<FMT, G, NJ, MR, R>(g, (int)blockIdx.x, (int)gridDim.x);
+}
+
+// Several forwards that share x (and format, K and M) in one launch: the grid is the forwards' grids one after the other,
+// each forward with its own weight, factors, outputs and slot; a block finds its forward by its index.
+constexpr int kRowsMaxJobs = 4;
+struct SkinnyRowsBatch {
+    SkinnyRowsArgs job[kRowsMaxJobs];
+    int32_t first[kRowsMaxJobs + 1];    // first block of each forward; entries past the last forward hold the grid size
+};
+template <int FMT, int G, int NJ, int MR, int R>
+__global__ void __launch_bounds__(512, 1) skinny_rows_multi_kernel(SkinnyRowsBatch b) {
+    const int bx = (int)blockIdx.x;
+    const int i = (bx >= b.first[1] ? 1 : 0) + (bx >= b.first[2] ? 1 : 0) + (bx >= b.first[3] ? 1 : 0);   // uniform
+    skinny_rows_body<FMT, G, NJ, MR, R>(b.job[i], bx - b.first[i], b.first[i + 1] - b.first[i]);
+}
+
 // ---- slots: device memory that belongs to the library (zero when the code object is loaded).
 // Each device holds its own copy of the array at its own address, reached through hipGetSymbolAddress with that device
 // current.  A slot is tied to the caller's scratch pointer, so calls that may legally overlap (different workspaces)
@@ -523,8 +544,12 @@ static int rows_slot(const void* key, uint32_t** out) {
 
 // geometry of a launch: NJ bound and row groups per block
 struct RowsPlan { int nj, njt, G, R, MR, xpitch, slab; size_t lds; };
-static bool rows_plan(const xq_weight* w, int64_t M, RowsPlan* p) {
-    const int64_t N = w->rows, K = w->cols;
+static bool rows_plan_multi(const xq_weight* const* ws, int n_w, int64_t M, RowsPlan* p);
+static bool rows_plan(const xq_weight* w, int64_t M, RowsPlan* p) { return rows_plan_multi(&w, 1, M, p); }
+// one geometry for several weights of one format and K that share a launch: each weight's rows are whole blocks
+static bool rows_plan_multi(const xq_weight* const* ws, int n_w, int64_t M, RowsPlan* p) {
+    const xq_weight* w = ws[0];
+    const int64_t K = w->cols;
     const bool f8 = w->format == XQ_FMT_FP8;
     const int eps = f8 ? 64 : 128;
     if (K % (8 * eps) != 0) return false;
@@ -538,7 +563,8 @@ static bool rows_plan(const xq_weight* w, int64_t M, RowsPlan* p) {
     if (p->MR == 16 && p->njt * eps > 512) return false;
     if (p->MR == 8 && p->njt * eps > 1024) return false;
     // as many row groups per block as give about one block per compute unit, within 24 loads per lane
-    const int64_t groups = N / 16;
+    int64_t groups = 0;
+    for (int i = 0; i < n_w; ++i) groups += ws[i]->rows / 16;
     const int cus = num_cus();
     int G = (int)((groups + cus - 1) / cus);
     const int gmax = p->njt <= 4 ? 3 : p->njt <= 8 ? (f8 ? 3 : 2) : p->njt <= 12 ? 2 : 1;
@@ -547,8 +573,14 @@ static bool rows_plan(const xq_weight* w, int64_t M, RowsPlan* p) {
     // more than the second launch of the other organisation): twice the rows go to one block in two rounds instead,
     // where the shape allows it
     p->R = 1;
-    if (xq_cdiv(groups, p->G) > cus) {
-        const bool two_rounds = p->G == 3 && p->njt * eps <= 512 && groups % 6 == 0 && groups / 6 <= cus;
+    int64_t blocks = 0;
+    bool sixes = true;
+    for (int i = 0; i < n_w; ++i) {
+        blocks += xq_cdiv(ws[i]->rows / 16, p->G);
+        sixes = sixes && (ws[i]->rows / 16) % 6 == 0;
+    }
+    if (blocks > cus) {
+        const bool two_rounds = p->G == 3 && p->njt * eps <= 512 && sixes && groups / 6 <= cus;
         if (!two_rounds) return false;
         p->R = 2;
     }
@@ -578,39 +610,43 @@ bool skinny_rows_supported(const xq_weight* w, int64_t M, const void* lora_A, co
     return true;
 }
 
+// `batch` == nullptr: the forward `g` alone; otherwise the forwards of `*batch` as one launch
 template <int FMT, int G, int NJ, int MR, int R>
-static int launch_rows_one(const SkinnyRowsArgs& g, unsigned grid, size_t lds, hipStream_t s) {
-    static std::atomic<bool> attr_set{false};   // per instantiation; the attribute call is idempotent: a race only repeats it
+static int launch_rows_one(const SkinnyRowsArgs& g, const SkinnyRowsBatch* batch, unsigned grid, size_t lds, hipStream_t s) {
+    static std::atomic<bool> attr_set{false};   // per instantiation; the attribute calls are idempotent: a race only repeats them
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute((const void*)skinny_rows_kernel<FMT, G, NJ, MR, R>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e == hipSuccess)
+            e = hipFuncSetAttribute((const void*)skinny_rows_multi_kernel<FMT, G, NJ, MR, R>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) {
             xq_set_error("xq_linear_fwd: cannot raise the dynamic LDS limit: %s", hipGetErrorString(e));
             return XQ_ERR_LAUNCH;
         }
         attr_set = true;
     }
-    skinny_rows_kernel<FMT, G, NJ, MR, R><<<grid, 512, lds, s>>>(g);
+    if (batch) skinny_rows_multi_kernel<FMT, G, NJ, MR, R><<<grid, 512, lds, s>>>(*batch);
+    else skinny_rows_kernel<FMT, G, NJ, MR, R><<<grid, 512, lds, s>>>(g);
     return XQ_OK;
 }
 
 template <int FMT, int G, int NJ, int R>
-static int launch_rows_mr(const SkinnyRowsArgs& g, int MR, unsigned grid, size_t lds, hipStream_t s) {
+static int launch_rows_mr(const SkinnyRowsArgs& g, const SkinnyRowsBatch* batch, int MR, unsigned grid, size_t lds, hipStream_t s) {
     constexpr int EPS = FMT == XQ_FMT_FP8 ? 64 : 128;
-    if (MR == 1) return launch_rows_one<FMT, G, NJ, 1, R>(g, grid, lds, s);
+    if (MR == 1) return launch_rows_one<FMT, G, NJ, 1, R>(g, batch, grid, lds, s);
     if constexpr (NJ * EPS <= 1024) {
-        if (MR == 8) return launch_rows_one<FMT, G, NJ, 8, R>(g, grid, lds, s);
+        if (MR == 8) return launch_rows_one<FMT, G, NJ, 8, R>(g, batch, grid, lds, s);
     }
     if constexpr (NJ * EPS <= 512) {
-        if (MR == 16) return launch_rows_one<FMT, G, NJ, 16, R>(g, grid, lds, s);
+        if (MR == 16) return launch_rows_one<FMT, G, NJ, 16, R>(g, batch, grid, lds, s);
     }
     XQ_REQUIRE(false, "xq_linear_fwd: internal error: no one-launch skinny kernel for %d x rows, %d steps", MR, NJ);
 }
 
 template <int FMT>
-static int launch_rows_fmt(const SkinnyRowsArgs& g, const RowsPlan& p, unsigned grid, hipStream_t s) {
+static int launch_rows_fmt(const SkinnyRowsArgs& g, const SkinnyRowsBatch* batch, const RowsPlan& p, unsigned grid, hipStream_t s) {
     constexpr int EPS = FMT == XQ_FMT_FP8 ? 64 : 128;
 #define XQ_ROWS_CASE(GG, NN, RR) \
-    if (p.G == GG && p.njt == NN && p.R == RR) return launch_rows_mr<FMT, GG, NN, RR>(g, p.MR, grid, p.lds, s)
+    if (p.G == GG && p.njt == NN && p.R == RR) return launch_rows_mr<FMT, GG, NN, RR>(g, batch, p.MR, grid, p.lds, s)
     XQ_ROWS_CASE(1, 4, 1); XQ_ROWS_CASE(2, 4, 1); XQ_ROWS_CASE(3, 4, 1); XQ_ROWS_CASE(3, 4, 2);
     XQ_ROWS_CASE(1, 8, 1); XQ_ROWS_CASE(2, 8, 1);
     if constexpr (FMT == XQ_FMT_FP8) {
@@ -623,11 +659,9 @@ static int launch_rows_fmt(const SkinnyRowsArgs& g, const RowsPlan& p, unsigned 
     XQ_REQUIRE(false, "xq_linear_fwd: internal error: no one-launch skinny kernel for %d row groups, %d steps, %d rounds", p.G, p.njt, p.R);
 }
 
-int launch_skinny_rows(const xq_weight* w, const bf16_t* x, int64_t ldx, int64_t M, const void* lora_A, const void* lora_B, int r,
-                       float scaling, const bf16_t* bias, bf16_t* y, int64_t ldy, const void* slot_key, hipStream_t stream) {
-    RowsPlan p;
-    XQ_REQUIRE(rows_plan(w, M, &p), "xq_linear_fwd: internal error: shape not supported by the one-launch skinny kernel");
-    SkinnyRowsArgs g;
+static int rows_args(const xq_weight* w, const RowsPlan& p, const bf16_t* x, int64_t ldx, int64_t M, const void* lora_A, const void* lora_B,
+                     int r, float scaling, const bf16_t* bias, bf16_t* y, int64_t ldy, const void* slot_key, SkinnyRowsArgs* out) {
+    SkinnyRowsArgs& g = *out;
     g.x = x; g.ldx = ldx; g.M = (int)M; g.N = (int)w->rows; g.K = (int)w->cols;
     g.packed = (const uint8_t*)w->packed; g.scales = (const uint8_t*)w->scales; g.global_scale = w->global_scale;
     g.gshift = 0;
@@ -639,16 +673,71 @@ int launch_skinny_rows(const xq_weight* w, const bf16_t* x, int64_t ldx, int64_t
     g.nsu = r > 0 ? (int)(w->cols / kSuPartK) : 0;
     g.slot = nullptr;
     g.spin_limit = kRowsSpinLimit;
-    if (r > 0) {
-        int rc = rows_slot(slot_key, &g.slot);
-        if (rc) return rc;
-    }
+    if (r > 0) return rows_slot(slot_key, &g.slot);
+    return XQ_OK;
+}
+
+int launch_skinny_rows(const xq_weight* w, const bf16_t* x, int64_t ldx, int64_t M, const void* lora_A, const void* lora_B, int r,
+                       float scaling, const bf16_t* bias, bf16_t* y, int64_t ldy, const void* slot_key, hipStream_t stream) {
+    RowsPlan p;
+    XQ_REQUIRE(rows_plan(w, M, &p), "xq_linear_fwd: internal error: shape not supported by the one-launch skinny kernel");
+    SkinnyRowsArgs g;
+    const int rc = rows_args(w, p, x, ldx, M, lora_A, lora_B, r, scaling, bias, y, ldy, slot_key, &g);
+    if (rc) return rc;
     const unsigned grid = (unsigned)xq_cdiv(w->rows / 16, p.G * p.R);
     switch (w->format) {
-        case XQ_FMT_FP8: return launch_rows_fmt<XQ_FMT_FP8>(g, p, grid, stream);
-        case XQ_FMT_INT4: return launch_rows_fmt<XQ_FMT_INT4>(g, p, grid, stream);
-        case XQ_FMT_NF4: return launch_rows_fmt<XQ_FMT_NF4>(g, p, grid, stream);
-        default: return launch_rows_fmt<XQ_FMT_NVFP4>(g, p, grid, stream);
+        case XQ_FMT_FP8: return launch_rows_fmt<XQ_FMT_FP8>(g, nullptr, p, grid, stream);
+        case XQ_FMT_INT4: return launch_rows_fmt<XQ_FMT_INT4>(g, nullptr, p, grid, stream);
+        case XQ_FMT_NF4: return launch_rows_fmt<XQ_FMT_NF4>(g, nullptr, p, grid, stream);
+        default: return launch_rows_fmt<XQ_FMT_NVFP4>(g, nullptr, p, grid, stream);
+    }
+}
+
+// ---- several forwards that share x as one launch
+bool skinny_rows_multi_supported(const SkinnyRowsJob* jobs, int n_jobs, int64_t M, int lora_dtype) {
+    if (n_jobs < 2 || n_jobs > kRowsMaxJobs) return false;
+    const xq_weight* ws[kRowsMaxJobs];
+    for (int i = 0; i < n_jobs; ++i) {
+        const xq_weight* w = jobs[i].w;
+        ws[i] = w;
+        if (w->format != jobs[0].w->format || w->cols != jobs[0].w->cols || w->group != jobs[0].w->group ||
+            w->scale_dtype != jobs[0].w->scale_dtype || w->layout != jobs[0].w->layout)
+            return false;
+        if (!skinny_rows_supported(w, M, jobs[i].lora_A, jobs[i].lora_B, lora_dtype, jobs[i].r)) return false;
+    }
+    RowsPlan p;
+    if (!rows_plan_multi(ws, n_jobs, M, &p)) return false;
+    for (int i = 0; i < n_jobs; ++i)
+        if (jobs[i].r > 0 && ws[i]->cols / kSuPartK > xq_cdiv(ws[i]->rows / 16, p.G * p.R)) return false;   // a block forms at most one su part
+    return true;
+}
+
+int launch_skinny_rows_multi(const SkinnyRowsJob* jobs, int n_jobs, const bf16_t* x, int64_t ldx, int64_t M, const void* slot_key,
+                             hipStream_t stream) {
+    const xq_weight* ws[kRowsMaxJobs];
+    for (int i = 0; i < n_jobs; ++i) ws[i] = jobs[i].w;
+    RowsPlan p;
+    XQ_REQUIRE(rows_plan_multi(ws, n_jobs, M, &p), "xq_linear_fwd_multi: internal error: shapes not supported by the one-launch skinny kernel");
+    SkinnyRowsBatch b;
+    int first = 0;
+    for (int i = 0; i < kRowsMaxJobs; ++i) {
+        b.first[i] = first;
+        if (i >= n_jobs) {
+            b.job[i] = b.job[0];
+            continue;
+        }
+        // each forward has a slot of its own: its key is a distinct address inside the caller's workspace
+        const int rc = rows_args(ws[i], p, x, ldx, M, jobs[i].lora_A, jobs[i].lora_B, jobs[i].r, jobs[i].scaling, jobs[i].bias, jobs[i].y,
+                                 jobs[i].ldy, (const char*)slot_key + 256 * i, &b.job[i]);
+        if (rc) return rc;
+        first += (int)xq_cdiv(ws[i]->rows / 16, p.G * p.R);
+    }
+    b.first[kRowsMaxJobs] = first;
+    switch (ws[0]->format) {
+        case XQ_FMT_FP8: return launch_rows_fmt<XQ_FMT_FP8>(b.job[0], &b, p, (unsigned)first, stream);
+        case XQ_FMT_INT4: return launch_rows_fmt<XQ_FMT_INT4>(b.job[0], &b, p, (unsigned)first, stream);
+        case XQ_FMT_NF4: return launch_rows_fmt<XQ_FMT_NF4>(b.job[0], &b, p, (unsigned)first, stream);
+        default: return launch_rows_fmt<XQ_FMT_NVFP4>(b.job[0], &b, p, (unsigned)first, stream);
     }
 }
 

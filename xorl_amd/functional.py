@@ -263,6 +263,53 @@ def qlora_linear(x: Tensor, qw: QuantWeight, lora_A: Optional[Tensor], lora_B: O
     return QLoRALinearFunction.apply(x, lora_A, lora_B, bias, qw, r, scaling, training)
 
 
+def qlora_linear_multi(x: Tensor, jobs) -> list:
+    """Forward-only: several QLoRA linears on one input, ``[qlora_linear(x, *job) for job in jobs]`` as one library call
+    (xq_linear_fwd_multi): the separate q_proj / k_proj / v_proj or gate_proj / up_proj calls of a model that keeps
+    them unfused (reference: models/layers/attention/multi_head_attention.py:93-95, modeling_qwen3.py:75-76).
+
+    ``jobs``: up to 4 tuples ``(qw, lora_A, lora_B, r, scaling, bias)`` with the arguments of :func:`qlora_linear`
+    (r <= 64, factors of one dtype).  At decode sizes (at most 16 rows of x) weights of one format run as ONE launch;
+    results are bit-identical to the separate calls either way.  No autograd: call it under ``torch.no_grad()``."""
+    if not 1 <= len(jobs) <= _C.XQ_LINEAR_MULTI_MAX:
+        raise _C.XqError(f"qlora_linear_multi takes 1..{_C.XQ_LINEAR_MULTI_MAX} forwards, got {len(jobs)}")
+    if x.dtype != torch.bfloat16:
+        raise _C.XqError(f"activations must be bf16, got {x.dtype}")
+    if torch.is_grad_enabled() and any(t is not None and t.requires_grad for j in jobs for t in (x, j[1], j[2], j[5])):
+        raise _C.XqError("qlora_linear_multi is forward-only: call it under torch.no_grad()")
+    x2 = _as_2d(x)
+    M, K = x2.shape
+    dev = x.device
+    arr = (_C.XqLinearJob * len(jobs))()
+    keep, ys, lora_dt = [], [], None
+    for i, (qw, lora_A, lora_B, r, scaling, bias) in enumerate(jobs):
+        if qw.cols != K:
+            raise _C.XqError(f"input width {K} != in_features {qw.cols} of forward {i}")
+        if r > MAX_FUSED_RANK:
+            raise _C.XqError(f"qlora_linear_multi: rank {r} of forward {i} exceeds {MAX_FUSED_RANK}")
+        A = lora_A.detach()[:r].contiguous() if (lora_A is not None and r) else None
+        B = lora_B.detach()[:, :r].contiguous() if (lora_B is not None and r) else None
+        if A is not None:
+            if lora_dt is None:
+                lora_dt = _lora_dt(A)
+            elif lora_dt != _lora_dt(A):
+                raise _C.XqError("qlora_linear_multi: the forwards' LoRA factors must share one dtype")
+        b = bias.detach().to(torch.bfloat16).contiguous() if bias is not None else None
+        y = torch.empty(M, qw.rows, dtype=torch.bfloat16, device=dev)
+        cw = qw.c()
+        keep += [A, B, b, cw]
+        arr[i].w = ctypes.pointer(cw)
+        arr[i].lora_A, arr[i].lora_B, arr[i].r, arr[i].scaling = _C.ptr(A), _C.ptr(B), (r if A is not None else 0), float(scaling)
+        arr[i].bias_bf16, arr[i].y, arr[i].ldy = _C.ptr(b), y.data_ptr(), qw.rows
+        ys.append(y)
+    L = _C.lib()
+    ws_bytes = L.xq_linear_fwd_multi_workspace_bytes(arr, len(jobs), M)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    _C.check(L.xq_linear_fwd_multi(arr, len(jobs), x2.data_ptr(), _ld(x2), M, lora_dt if lora_dt is not None else _C.XQ_DT_F32,
+                                   ws.data_ptr(), ws_bytes, _C.stream_ptr(dev)))
+    return [y.reshape(*x.shape[:-1], y.shape[1]) for y in ys]
+
+
 # ---------------------------------------------------------------------------
 # dense SwiGLU MLP of three QLoRA linears (xq_mlp_fwd / xq_mlp_bwd)
 # ---------------------------------------------------------------------------

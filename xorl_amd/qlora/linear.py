@@ -795,6 +795,31 @@ def qlora_mlp_forward(gate_proj: "QLoRALinear", up_proj: "QLoRALinear", down_pro
                      r, s, gate_proj.bias, up_proj.bias, down_proj.bias)
 
 
+def qlora_linears_forward(modules, x: Tensor) -> list:
+    """`[m(x) for m in modules]` for QLoRA linears that share their input -- the separate q_proj / k_proj / v_proj calls
+    of the reference's attention block (models/layers/attention/multi_head_attention.py:93-95) and the gate_proj /
+    up_proj calls of its unfused MLP (models/transformers/qwen3/modeling_qwen3.py:75-76).  Without autograd (decode,
+    rollout) up to four modules go to the library as ONE call, which at decode sizes is one kernel launch
+    (xq_linear_fwd_multi); in every other case the modules are called one by one.  The results are the same bits."""
+    from ..functional import qlora_linear_multi
+    from .._C import XQ_LINEAR_MULTI_MAX
+
+    mods = list(modules)
+    needs_grad = torch.is_grad_enabled() and (x.requires_grad or any(
+        p.requires_grad for m in mods for p in (m.lora_A, m.lora_B, m.bias) if p is not None))
+    one_call = (1 < len(mods) <= XQ_LINEAR_MULTI_MAX and not needs_grad and not torch.compiler.is_compiling()
+                and all(isinstance(m, QLoRALinear) for m in mods)
+                and all(m.active_r <= MAX_FUSED_RANK and m.in_features == mods[0].in_features for m in mods)
+                and len({m.lora_A.dtype for m in mods}) == 1
+                and not any(m.enable_aqn and m.training for m in mods)
+                and not any(_is_dtensor(m.packed_weight_f32.data) or _is_dtensor(m.lora_A) for m in mods)
+                and x.dtype == torch.bfloat16 and x.is_cuda)
+    if not one_call:
+        return [m(x) for m in mods]
+    return qlora_linear_multi(x, [(m._forward_quant_weight(), m.lora_A, m.lora_B, m.active_r, m._active_scaling(), m.bias)
+                                  for m in mods])
+
+
 def deregister_qlora_weights_from_fsdp(model: nn.Module, param_names: tuple = ("weight",)) -> int:
     """Drop QLoRALinear parameters from FSDP2 parameter groups so no mixed
     precision cast ever touches the packed bytes; they stay sharded DTensors
