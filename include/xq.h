@@ -114,6 +114,18 @@ int xq_set_persistent_tiles(int enabled);
  * it at load time); no counterpart in the reference. */
 int xq_set_skinny_one_launch(int enabled);
 
+/* Test switch (process-wide, no counterpart in the reference): how many times a bounded wait of the one-launch skinny
+ * kernel looks before it gives up (limit <= 0 restores the default, about a second of waiting).  The waits are for other
+ * blocks of the same launch (the published parts of x . A^T; the count of blocks that have read the launch count).  A
+ * block whose wait gives up writes NaN to its outputs and ends like every other block; if it is the block that closes the
+ * launch it marks the library's slot for this workspace failed, and every later forward through that slot writes NaN
+ * (never values made from another launch's sums) until xq_skinny_reset().  A small limit forces those paths from the host
+ * without any kernel hanging or faulting. */
+int xq_set_skinny_spin_limit(int limit);
+/* Clears the library's slots on the current device (launch counts, failure marks, published parts).  Synchronises the
+ * device before and after: call it with no forward in flight.  No counterpart in the reference. */
+int xq_skinny_reset(void);
+
 /* ---- decode ------------------------------------------------------------
  * out[e] = decoded weight of expert e, shape [rows, cols], bf16 or fp32.
  * Replaces int4_dequantize / int4_dequantize_gkn

@@ -221,3 +221,52 @@ def test_overlapping_calls_on_two_streams(hip_device):
     for i in range(2):
         for j in range(6):
             assert torch.equal(work[i][7][j], alone[i][j]), (i, j)
+
+
+def test_bounded_waits_give_up_and_the_slot_recovers(hip_device):
+    """With the waits cut to a single look (forced from the host) every kernel still ends; a block either has all it
+    waited for, and writes the right outputs, or gives up and writes NaN, never values made from stale sums.  Once the
+    closing block of a launch has given up the slot is marked failed and every forward through it writes NaN, also after
+    the limit is back to normal, until the host clears the slots; then results are exact again."""
+    from xorl_amd import _C
+    from xorl_amd.functional import _workspace_bytes
+
+    N, K, r = 12288, 4096, 16
+    m, _ = make_dense_module("block_fp8", N, K, r, 32, seed=9, device=hip_device)
+    w = m._quant_weight().c()
+    A, B = m.lora_A.detach().contiguous(), m.lora_B.detach().contiguous()
+    L = _C.lib()
+    M = 8
+    wsb = _workspace_bytes(M, N, K, r)
+    ws = torch.empty(wsb, dtype=torch.uint8, device=hip_device)        # one workspace = one slot throughout
+    y = torch.empty(M, N, dtype=torch.bfloat16, device=hip_device)
+
+    def call(x, rank=r):
+        _C.check(L.xq_linear_fwd(ctypes.byref(w), x.data_ptr(), K, M, A.data_ptr(), B.data_ptr(), _C.XQ_DT_F32, rank, ctypes.c_float(m.scaling),
+                                 None, y.data_ptr(), N, None, ws.data_ptr(), wsb, _C.stream_ptr(hip_device)))
+        torch.cuda.synchronize()
+        return y.clone()
+
+    xs = [gen((M, K), 1.0, 300 + i, torch.bfloat16).to(hip_device) for i in range(6)]
+    want = [call(x) for x in xs]
+    assert all(torch.isfinite(t.float()).all() for t in want)
+    no_lora = call(xs[0], 0)
+    try:
+        _C.check(L.xq_set_skinny_spin_limit(1))
+        n_bad = 0
+        for x, ref in zip(xs, want):
+            got = call(x)
+            bad = torch.isnan(got.float())
+            assert torch.equal(got[~bad], ref[~bad])                    # what is not NaN is right: nothing stale was summed
+            cols = bad.any(dim=0)                                       # a block gives up as a whole: all rows of x
+            assert torch.equal(bad, cols.unsqueeze(0).expand_as(bad))
+            n_bad += int(bad.sum())
+        assert n_bad > 0                                                # (a single look does not find 256 blocks in step)
+    finally:
+        _C.check(L.xq_set_skinny_spin_limit(0))
+    # the mark stays: NaN everywhere with the normal limit too; a forward without a low-rank term does not use the slot
+    assert torch.isnan(call(xs[0]).float()).all()
+    assert torch.equal(call(xs[0], 0), no_lora)
+    _C.check(L.xq_skinny_reset())
+    for x, ref in zip(xs, want):
+        assert torch.equal(call(x), ref)

@@ -122,6 +122,8 @@ _SIGNATURES = {
     "xq_set_tile_policy": (_INT, [_INT]),
     "xq_set_persistent_tiles": (_INT, [_INT]),
     "xq_set_skinny_one_launch": (_INT, [_INT]),
+    "xq_set_skinny_spin_limit": (_INT, [_INT]),
+    "xq_skinny_reset": (_INT, []),
     "xq_route_workspace_bytes": (_I64, [_I64, _I32]),
     # selected, n_routed, E, counts, offsets, scatter_index, tile_offsets, ws, ws_bytes, stream
     "xq_route_build": (_INT, [_P, _I64, _I32, _P, _P, _P, _P, _P, _I64, _P]),

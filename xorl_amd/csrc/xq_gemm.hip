@@ -385,6 +385,13 @@ extern "C" int xq_set_skinny_one_launch(int enabled) {
     return XQ_OK;
 }
 
+extern "C" int xq_set_skinny_spin_limit(int limit) {
+    set_skinny_rows_spin_limit(limit);
+    return XQ_OK;
+}
+
+extern "C" int xq_skinny_reset(void) { return reset_skinny_rows_slots(); }
+
 extern "C" int xq_set_persistent_tiles(int enabled) {
     g_persist = enabled != 0;
     return XQ_OK;

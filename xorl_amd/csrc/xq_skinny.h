@@ -46,6 +46,8 @@ __device__ __forceinline__ bf16x8 decode8(uint32_t w0, uint32_t w1, float s0, fl
 
 void set_skinny_rows(int enabled);
 bool skinny_rows_enabled();
+void set_skinny_rows_spin_limit(int limit);   // <= 0: the default
+int reset_skinny_rows_slots();                 // clears the current device's slots (synchronises the device)
 
 // ---- one-launch organisation (xq_skinny_rows.hip)
 // true when the shape, format and LoRA operands fit it; the caller falls back to the split organisation otherwise

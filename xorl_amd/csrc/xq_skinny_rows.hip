@@ -26,8 +26,11 @@
 //    rewrites them all): hundreds of accesses to one location that bypass the caches would take microseconds.
 // Slot accesses are device-scope atomics (they bypass the per-XCD L2s) unless said otherwise where they are made.
 // Blocks that publish never wait, and they are the first the dispatcher places, so the collectors' wait ends; a limit
-// bounds every wait all the same and turns the block's outputs into NaN.  Sums run in fixed orders (waves ascending,
-// parts ascending): results are identical from call to call.
+// bounds every wait all the same and turns the block's outputs into NaN.  A last block that gives up stores a mark in
+// place of the launch count; every block that reads the mark -- late blocks of that launch, all blocks of later launches
+// on the slot -- publishes nothing and writes NaN until the host clears the slots (reset_skinny_rows_slots): a failed
+// launch never lets stale sums through.  Sums run in fixed orders (waves ascending, parts ascending): results are
+// identical from call to call.
 //
 // Measured on an MI355X, launches back to back (block_fp8, r = 16, M = 1): 4096->12288 (48 MiB) 11.4 us against 15.6 us
 // for the two-launch organisation (10.0 us without a low-rank term), 4096->4096 7.4 against 8.8, 4096->24576 (96 MiB)
@@ -49,6 +52,7 @@ constexpr int kCtlStride = 32;                  // so that a launch's 256 blocks
 constexpr int kSlotWords = kSlotCtl + 2 * kCtlCopies * kCtlStride;   // [parts][256] pairs (sum bits, tag), gen copies, started copies
 constexpr int kSlots = 64;
 constexpr int kRowsSpinLimit = 1 << 20;
+constexpr uint32_t kGenPoison = 0xFFFFFFFFu;   // launch count of a slot in which a wait has given up: see the closer below
 #ifndef XQ_ROWS_LOADS_IN_FLIGHT
 #define XQ_ROWS_LOADS_IN_FLIGHT 6
 #endif
@@ -201,8 +205,9 @@ __device__ __forceinline__ void skinny_rows_body(const SkinnyRowsArgs& g, const 
                     ++spins;
                 }
             } while (!all && spins < g.spin_limit);
-            // (a wait that hit the limit leaves the part unpublished: the collectors then hit theirs and write NaN)
-            if (all) {
+            // (a wait that hit the limit, or a slot that is marked failed, leaves the part unpublished: the collectors then
+            // hit their limit, or see the mark, and write NaN)
+            if (all && gen != kGenPoison) {
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
                     float s = 0.0f;
@@ -349,14 +354,16 @@ __device__ __forceinline__ void skinny_rows_body(const SkinnyRowsArgs& g, const 
     // this block may be counted once its reads of `gen` have returned: wave 0's has, like the weights requested before it;
     // in a block that forms an su part wave 4 has read it too and says so when it has published
     if (lora && wave == 0) {
+        bool publisher_done = true;
         if (su_block) {
             int spins = 0;
-            while (__hip_atomic_load(su_flag + 4, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) == 0 && spins < g.spin_limit) {
+            while (!(publisher_done = __hip_atomic_load(su_flag + 4, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) != 0) && spins < g.spin_limit) {
                 __builtin_amdgcn_s_sleep(2);
                 ++spins;
             }
         }
-        if (lane == 0) count_block();
+        // (a block whose publishing wave is that late is never counted: the closer then gives up and marks the slot failed)
+        if (lane == 0 && publisher_done) count_block();
     }
 
     // ---- the wave's sums -> its own LDS area (its x slice is no longer needed): tile gi, register q, lane; B rows -> LDS
@@ -373,8 +380,9 @@ __device__ __forceinline__ void skinny_rows_body(const SkinnyRowsArgs& g, const 
         const bool closer = bx == nb - 1;      // this block moves the launch count on
         float s[4];
         int spins = 0;
-        bool missing, open = closer;
-        do {
+        const bool failed_slot = gen == kGenPoison;
+        bool missing = failed_slot, open = closer && !failed_slot;
+        if (!failed_slot) do {
 #pragma unroll
             for (int q = 0; q < 4; ++q) s[q] = 0.0f;
             missing = false;
@@ -417,7 +425,8 @@ __device__ __forceinline__ void skinny_rows_body(const SkinnyRowsArgs& g, const 
                 if (started == (uint32_t)nb) {
                     // every block has read `gen`: the next launch counts from gen + 1
                     if (lane < kCtlCopies) {
-                        __hip_atomic_store(g.slot + kSlotCtl + lane * kCtlStride, gen + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        __hip_atomic_store(g.slot + kSlotCtl + lane * kCtlStride, gen + 1 == kGenPoison ? 0u : gen + 1, __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_AGENT);
                         __hip_atomic_store(g.slot + kSlotCtl + (kCtlCopies + lane) * kCtlStride, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     }
                     open = false;
@@ -428,6 +437,12 @@ __device__ __forceinline__ void skinny_rows_body(const SkinnyRowsArgs& g, const 
                 ++spins;
             }
         } while ((missing || open) && spins < g.spin_limit);
+        // A closer that gave up cannot tell which blocks have yet to read the launch count, so no value it could store
+        // would keep this launch's late parts and the next launch's apart.  It marks the slot failed instead: every block
+        // that reads the mark (late blocks of this launch, all blocks of later launches) publishes nothing and writes
+        // NaN, until the host clears the library's slots (reset_skinny_rows_slots).  Never values from stale sums.
+        if (open && lane < kCtlCopies)
+            __hip_atomic_store(g.slot + kSlotCtl + lane * kCtlStride, kGenPoison, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
             const int j = 4 * (lane >> 4) + q, m = lane & 15;
@@ -510,6 +525,11 @@ uint64_t g_slot_used[kMaxDevices][kSlots] = {};
 uint64_t g_slot_clock = 0;
 }  // namespace
 
+// looks of a bounded wait before it gives up: a process-wide test switch (a small value forces the give-up paths, in which
+// every kernel still ends and the outputs concerned are NaN)
+static std::atomic<int> g_rows_spin_limit{kRowsSpinLimit};
+void set_skinny_rows_spin_limit(int limit) { g_rows_spin_limit = limit > 0 ? limit : kRowsSpinLimit; }
+
 // the slot of `key` on the current device
 static int rows_slot(const void* key, uint32_t** out) {
     int dev = -1;
@@ -539,6 +559,31 @@ static int rows_slot(const void* key, uint32_t** out) {
     }
     g_slot_used[dev][s] = ++g_slot_clock;
     *out = g_slots_ptr[dev] + (size_t)s * kSlotWords;
+    return XQ_OK;
+}
+
+// Clears the slots of the current device (launch counts, marks of failed waits, published parts): for a host that has
+// seen NaN outputs after a forced or real give-up.  Waits for the device before and after; no forward may be in flight.
+int reset_skinny_rows_slots() {
+    uint32_t* slot = nullptr;
+    int rc = rows_slot(nullptr, &slot);       // resolves the array's address on this device (the null key takes a slot like any other)
+    if (rc) return rc;
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e == hipSuccess) e = hipDeviceSynchronize();
+    if (e == hipSuccess) {
+        std::lock_guard<std::mutex> lock(g_slots_mu);
+        e = hipMemset(g_slots_ptr[dev], 0, sizeof(uint32_t) * (size_t)kSlots * kSlotWords);
+        for (int i = 0; i < kSlots; ++i) {
+            g_slot_key[dev][i] = nullptr;
+            g_slot_used[dev][i] = 0;
+        }
+    }
+    if (e == hipSuccess) e = hipDeviceSynchronize();
+    if (e != hipSuccess) {
+        xq_set_error("xq_skinny_reset: %s", hipGetErrorString(e));
+        return XQ_ERR_LAUNCH;
+    }
     return XQ_OK;
 }
 
@@ -672,7 +717,7 @@ static int rows_args(const xq_weight* w, const RowsPlan& p, const bf16_t* x, int
     g.xpitch = p.xpitch; g.slab = p.slab;
     g.nsu = r > 0 ? (int)(w->cols / kSuPartK) : 0;
     g.slot = nullptr;
-    g.spin_limit = kRowsSpinLimit;
+    g.spin_limit = g_rows_spin_limit.load();
     if (r > 0) return rows_slot(slot_key, &g.slot);
     return XQ_OK;
 }
