@@ -470,6 +470,16 @@ int xq_mlp_bwd(const xq_weight* gate, const xq_weight* up, const xq_weight* down
                void* dx, int64_t lddx, const xq_mlp_grads* grads, void* workspace, int64_t workspace_bytes,
                void* stream);
 
+/* The same MLP forward when nothing is kept for a backward (inference, rollout: the reference's Qwen3MLP.forward under
+ * torch.no_grad(), modeling_qwen3.py:60-81).  Each projection takes the kernel that suits the row count: up to 64 rows
+ * the weight-streaming kernels (gate and up as one launch up to 16 rows), above that the tile kernels; the rounding
+ * points are those of the separate module calls.  The intermediate gate|up and h live in the workspace
+ * (xq_mlp_infer_workspace_bytes(...) bytes, 256-byte aligned). */
+int64_t xq_mlp_infer_workspace_bytes(int64_t M, int64_t hidden, int64_t intermediate, int r);
+int xq_mlp_fwd_infer(const xq_weight* gate, const xq_weight* up, const xq_weight* down, const xq_mlp_lora* lora,
+                     const void* x, int64_t ldx, int64_t M, void* y, int64_t ldy, void* workspace,
+                     int64_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

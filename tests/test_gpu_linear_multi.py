@@ -181,3 +181,31 @@ def test_module_helper(hip_device):
         close(y.detach().float().cpu(), w.double().cpu(), TOL)
     sum(y.float().sum() for y in ys).backward()
     assert xg.grad is not None and all(m.lora_A.grad is not None for m in mods)
+
+
+@pytest.mark.parametrize("fmt", ["block_fp8", "int4"])
+def test_mlp_forward_without_autograd_is_the_module_calls(hip_device, fmt):
+    """qlora_mlp_forward under no_grad is one library call (xq_mlp_fwd_infer); its output is, bit for bit, the three
+    module calls around the SwiGLU kernel, at decode sizes (weight-streaming kernels) and above (tile kernels), and it
+    matches the fp64 program."""
+    from xorl_amd.functional import silu_and_mul
+    from xorl_amd.qlora import qlora_mlp_forward
+
+    H, I, r = 1024, 3072, 8
+    (g, wg), (u, wu), (d, wd) = (make_dense_module(fmt, N, K, r, 16, seed=50 + i, device=hip_device)
+                                 for i, (N, K) in enumerate(((I, H), (I, H), (H, I))))
+    loras = {k: (m.lora_A.detach().cpu(), m.lora_B.detach().cpu()) for k, m in (("gate", g), ("up", u), ("down", d))}
+    for M in (1, 8, 16, 40, 64, 300):
+        x = gen((M, H), 1.0, 60 + M, torch.bfloat16)
+        xd = x.to(hip_device)
+        with torch.no_grad():
+            got = qlora_mlp_forward(g, u, d, xd)
+            want = d(silu_and_mul(g(xd), u(xd)))
+        assert got.shape == (M, H) and torch.equal(got, want)
+        close(got.cpu(), R.mlp_fwd_bwd_exact(x, wg, wu, wd, loras, g.scaling)["y"], 2e-2)
+    # with a bias on every projection (no oracle program for it: the module calls are the reference)
+    (g, _), (u, _), (d, _) = (make_dense_module(fmt, N, K, r, 16, seed=70 + i, device=hip_device, bias=True)
+                              for i, (N, K) in enumerate(((I, H), (I, H), (H, I))))
+    xd = gen((5, H), 1.0, 99, torch.bfloat16).to(hip_device)
+    with torch.no_grad():
+        assert torch.equal(qlora_mlp_forward(g, u, d, xd), d(silu_and_mul(g(xd), u(xd))))

@@ -149,6 +149,9 @@ _SIGNATURES = {
                               ctypes.POINTER(XqGroupedSaved), _P, _I64, _P, _INT, ctypes.POINTER(XqGroupedGrads), _P, _I64,
                               _P]),
     "xq_mlp_workspace_bytes": (_I64, [_I64, _I64, _I64, _INT, _INT]),
+    "xq_mlp_infer_workspace_bytes": (_I64, [_I64, _I64, _I64, _INT]),
+    # gate, up, down, lora, x, ldx, M, y, ldy, ws, ws_bytes, stream
+    "xq_mlp_fwd_infer": (_INT, [_W, _W, _W, ctypes.POINTER(XqMlpLora), _P, _I64, _I64, _P, _I64, _P, _I64, _P]),
     # gate, up, down, lora, x, ldx, M, y, ldy, saved, ws, ws_bytes, stream
     "xq_mlp_fwd": (_INT, [_W, _W, _W, ctypes.POINTER(XqMlpLora), _P, _I64, _I64, _P, _I64, ctypes.POINTER(XqMlpSaved), _P,
                           _I64, _P]),

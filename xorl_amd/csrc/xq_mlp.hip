@@ -181,6 +181,47 @@ extern "C" int xq_mlp_fwd(const xq_weight* gate, const xq_weight* up, const xq_w
                             who, part, part_bytes);
 }
 
+// ---- forward only: nothing is kept for a backward, so each projection is free to take the kernel that suits the row
+// count -- at decode sizes the weight-streaming kernels (gate and up as one launch), not the tile kernels above
+static int64_t infer_linear_ws(int64_t M, int64_t H, int64_t I, int r) {
+    const int64_t a = xq_linear_workspace_bytes(M, I, H, r), b = xq_linear_workspace_bytes(M, H, I, r);
+    return al256((a > b ? a : b) > 2048 ? (a > b ? a : b) : 2048);
+}
+
+extern "C" int64_t xq_mlp_infer_workspace_bytes(int64_t M, int64_t hidden, int64_t intermediate, int r) {
+    if (M < 0 || r < 0) return 0;
+    return al256(M * 2 * intermediate * 2) + al256(M * intermediate * 2) + infer_linear_ws(M, hidden, intermediate, r) + 256;
+}
+
+extern "C" int xq_mlp_fwd_infer(const xq_weight* gate, const xq_weight* up, const xq_weight* down, const xq_mlp_lora* lora,
+                                const void* x, int64_t ldx, int64_t M, void* y, int64_t ldy, void* workspace,
+                                int64_t workspace_bytes, void* stream) {
+    static const char* who = "xq_mlp_fwd_infer";
+    XQ_REQUIRE(workspace && xq_aligned(workspace, 256), "%s: workspace missing or misaligned", who);
+    Dims d;
+    Carve cv{(uint8_t*)workspace, 0};
+    // (the argument checks are those of xq_mlp_fwd; the buffers it would keep for a backward live in the workspace here)
+    xq_mlp_saved tmp{workspace, workspace, workspace, workspace};
+    int rc = check_call(gate, up, down, lora, M, &tmp, who, &d);
+    if (rc) return rc;
+    if (M == 0) return XQ_OK;
+    XQ_REQUIRE(x && y, "%s: NULL activation pointer", who);
+    XQ_REQUIRE(workspace_bytes >= xq_mlp_infer_workspace_bytes(M, d.H, d.I, d.r),
+               "%s: workspace smaller than xq_mlp_infer_workspace_bytes()", who);
+    bf16_t* gu = cv.take<bf16_t>(M * 2 * d.I * 2);
+    bf16_t* h = cv.take<bf16_t>(M * d.I * 2);
+    void* ws = cv.take<uint8_t>(0);
+    const int64_t ws_bytes = workspace_bytes - cv.used;
+    xq_linear_job jobs[2] = {
+        {gate, lora->A[0], lora->B[0], d.r, lora->scaling, lora->bias[0], gu, 2 * d.I},
+        {up, lora->A[1], lora->B[1], d.r, lora->scaling, lora->bias[1], gu + d.I, 2 * d.I},
+    };
+    if ((rc = xq_linear_fwd_multi(jobs, 2, x, ldx, M, lora->dtype, ws, ws_bytes, stream))) return rc;
+    if ((rc = xq_silu_mul_fwd(gu, gu + d.I, 2 * d.I, nullptr, h, d.I, M, d.I, stream))) return rc;
+    return xq_linear_fwd(down, h, d.I, M, lora->A[2], lora->B[2], lora->dtype, d.r, lora->scaling, lora->bias[2], y, ldy, nullptr, ws,
+                         ws_bytes, stream);
+}
+
 extern "C" int xq_mlp_bwd(const xq_weight* gate, const xq_weight* up, const xq_weight* down, const xq_mlp_lora* lora,
                           const void* x_, int64_t ldx, const void* dy_, int64_t lddy, int64_t M, const xq_mlp_saved* saved,
                           void* dx, int64_t lddx, const xq_mlp_grads* grads, void* workspace, int64_t workspace_bytes,

@@ -498,6 +498,43 @@ class QLoRAMLPFunction(torch.autograd.Function):
         return (dx.reshape(ctx.shape) if need_dx else None, *out, *gb, None, None, None, None, None)
 
 
+_MLP_INFER_WS: dict = {}
+
+
+def qlora_mlp_infer(x: Tensor, qw_gate: QuantWeight, qw_up: QuantWeight, qw_down: QuantWeight, gate_A: Optional[Tensor],
+                    gate_B: Optional[Tensor], up_A: Optional[Tensor], up_B: Optional[Tensor], down_A: Optional[Tensor],
+                    down_B: Optional[Tensor], r: int, scaling: float, bias_gate: Optional[Tensor] = None,
+                    bias_up: Optional[Tensor] = None, bias_down: Optional[Tensor] = None) -> Tensor:
+    """:func:`qlora_mlp` without autograd, as one library call (xq_mlp_fwd_infer): at decode sizes gate and up share one
+    launch of the weight-streaming kernel and nothing is kept for a backward.  Same rounding points as the modules."""
+    if r > MAX_FUSED_RANK:
+        raise _C.XqError(f"the fused MLP takes LoRA ranks up to {MAX_FUSED_RANK}, got {r}")
+    if x.dtype != torch.bfloat16:
+        raise _C.XqError(f"activations must be bf16, got {x.dtype}")
+    _C.require_hip(x)
+    x2 = _as_2d(x)
+    M, H = x2.shape
+    I = qw_gate.rows
+    if qw_gate.cols != H:
+        raise _C.XqError(f"input width {H} != in_features {qw_gate.cols}")
+    factors = [None if t is None or r == 0 else t.detach()[:r].contiguous() for t in (gate_A, None, up_A, None, down_A, None)]
+    for i, t in ((1, gate_B), (3, up_B), (5, down_B)):
+        factors[i] = None if t is None or r == 0 else t.detach()[:, :r].contiguous()
+    biases = [None if b is None else b.detach().to(torch.bfloat16).contiguous() for b in (bias_gate, bias_up, bias_down)]
+    L = _mlp_lora_struct(factors, biases, r if factors[0] is not None else 0, float(scaling))
+    key = (M, H, I, r)
+    n = _MLP_INFER_WS.get(key)
+    if n is None:
+        n = _MLP_INFER_WS[key] = _C.lib().xq_mlp_infer_workspace_bytes(M, H, I, r)
+    dev = x.device
+    ws = torch.empty(n, dtype=torch.uint8, device=dev)
+    y = torch.empty(M, H, dtype=torch.bfloat16, device=dev)
+    cg, cu, cd = qw_gate.c(), qw_up.c(), qw_down.c()
+    _C.check(_C.lib().xq_mlp_fwd_infer(ctypes.byref(cg), ctypes.byref(cu), ctypes.byref(cd), ctypes.byref(L), x2.data_ptr(), _ld(x2), M,
+                                       y.data_ptr(), H, ws.data_ptr(), n, _C.stream_ptr(dev)))
+    return y.reshape(*x.shape[:-1], H)
+
+
 def qlora_mlp(x: Tensor, qw_gate: QuantWeight, qw_up: QuantWeight, qw_down: QuantWeight, gate_A: Optional[Tensor],
               gate_B: Optional[Tensor], up_A: Optional[Tensor], up_B: Optional[Tensor], down_A: Optional[Tensor],
               down_B: Optional[Tensor], r: int, scaling: float, bias_gate: Optional[Tensor] = None,

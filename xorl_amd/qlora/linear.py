@@ -776,7 +776,7 @@ def qlora_mlp_forward(gate_proj: "QLoRALinear", up_proj: "QLoRALinear", down_pro
     backward of the library when the three modules allow it: same active LoRA rank (<= 64) and scaling, plain
     (unsharded) state, no quantization noise.  Otherwise the three modules and the SwiGLU kernel are called one by
     one; both ways give the same rounding points."""
-    from ..functional import qlora_mlp, silu_and_mul
+    from ..functional import qlora_mlp, qlora_mlp_infer, silu_and_mul
 
     mods = (gate_proj, up_proj, down_proj)
     r, s = gate_proj.active_r, gate_proj._active_scaling()
@@ -790,6 +790,13 @@ def qlora_mlp_forward(gate_proj: "QLoRALinear", up_proj: "QLoRALinear", down_pro
                and x.dtype == torch.bfloat16 and x.is_cuda)
     if not fusable:
         return down_proj(silu_and_mul(gate_proj(x), up_proj(x)))
+    needs_grad = torch.is_grad_enabled() and (x.requires_grad or any(
+        p is not None and p.requires_grad for m in mods for p in (m.lora_A, m.lora_B, m.bias)))
+    if not needs_grad and not torch.compiler.is_compiling():
+        # inference / rollout: one library call that keeps nothing for a backward (weight-streaming kernels at decode sizes)
+        return qlora_mlp_infer(x, gate_proj._forward_quant_weight(), up_proj._forward_quant_weight(), down_proj._forward_quant_weight(),
+                               gate_proj.lora_A, gate_proj.lora_B, up_proj.lora_A, up_proj.lora_B, down_proj.lora_A, down_proj.lora_B,
+                               r, s, gate_proj.bias, up_proj.bias, down_proj.bias)
     return qlora_mlp(x, gate_proj._forward_quant_weight(), up_proj._forward_quant_weight(), down_proj._forward_quant_weight(),
                      gate_proj.lora_A, gate_proj.lora_B, up_proj.lora_A, up_proj.lora_B, down_proj.lora_A, down_proj.lora_B,
                      r, s, gate_proj.bias, up_proj.bias, down_proj.bias)
