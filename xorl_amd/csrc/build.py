@@ -18,6 +18,8 @@ FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
     # packed fp32 VALU forms are kept out of the generated code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # the first 16 dwords of a kernel's scalar arguments arrive in registers with the wave (where the platform does it)
+    "-mllvm", "-amdgpu-kernarg-preload-count=16",
     "-Wall", "-Wno-unused-function",
 ]
 

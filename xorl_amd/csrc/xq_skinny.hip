@@ -81,15 +81,27 @@ __device__ __forceinline__ bf16x8 factor_frag(const void* base, int64_t idx, boo
 // blocks take x one 128-element chunk at a time (all 64 rows, two LDS buffers), so that a weight chunk is decoded
 // once and multiplied into both halves of the rows, and three blocks still fit a CU.  (The su blocks at MR = 64
 // stage their x rows 32 at a time.)
+// The arguments that the first loads need are the leading scalars: the hardware hands a kernel's first 14 argument dwords
+// to each wave in registers (where the platform supports it; otherwise they are fetched like the rest), so those loads do
+// not wait for a round trip to the argument block.  fmt_bits = group | scale_dtype << 24, split_bits = splits |
+// su_blocks << 16, chunk_bits = chunk_q | chunk_rem << 16; `rest` carries the other fields (its copies of these are unused).
 template <int FMT, int MR, int NCH>
-__global__ void __launch_bounds__(256, MR == 16 ? 4 : 3) skinny_split_kernel(SkinnyArgs g) {
+__global__ void __launch_bounds__(256, MR == 16 ? 4 : 3)
+skinny_split_kernel(const bf16_t* x_, int32_t ldx_, int32_t M_, int32_t N_, int32_t K_, const uint8_t* packed_, const uint8_t* scales_,
+                    int32_t fmt_bits, int32_t split_bits, int32_t chunk_bits, int32_t xp_, SkinnyArgs rest) {
     constexpr int TR = MR < 32 ? MR : 32;              // x rows staged at a time
     constexpr int NPASS = MR / TR;
-    // Pin every argument in scalar registers here: otherwise the argument loads are placed lazily, each batch
-    // with its own wait, and several memory round trips pass before the first weight load is issued.
-    asm volatile("" ::"s"(g.x), "s"(g.ldx), "s"(g.M), "s"(g.N), "s"(g.K), "s"(g.packed), "s"(g.scales), "s"(g.global_scale),
-                 "s"(g.group), "s"(g.scale_dtype), "s"(g.splits), "s"(g.su_blocks), "s"(g.chunk_q), "s"(g.chunk_rem),
-                 "s"(g.xp), "s"(g.partial), "s"(g.su_part), "s"(g.lora_A), "s"(g.lora_f32), "s"(g.r), "s"(g.r_pad));
+    SkinnyArgs g = rest;
+    g.x = x_; g.ldx = ldx_; g.M = M_; g.N = N_; g.K = K_; g.packed = packed_; g.scales = scales_;
+    g.group = fmt_bits & 0xFFFFFF; g.scale_dtype = fmt_bits >> 24;
+    g.splits = split_bits & 0xFFFF; g.su_blocks = split_bits >> 16;
+    g.chunk_q = chunk_bits & 0xFFFF; g.chunk_rem = chunk_bits >> 16;
+    g.xp = xp_;
+    // The other arguments are pinned in scalar registers in one go once the first loads are out (left to the compiler,
+    // argument loads are placed lazily, each batch with its own wait).
+    auto pin_rest = [&]() {
+        asm volatile("" ::"s"(g.global_scale), "s"(g.partial), "s"(g.su_part), "s"(g.lora_A), "s"(g.lora_f32), "s"(g.r), "s"(g.r_pad));
+    };
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     bf16_t* xs = (bf16_t*)smem;                                  // [min(M, 32) rows][xp]; fragment rows past M read row 0:
     const int XP = g.xp;                                         // they feed only output columns >= M, which are never stored
@@ -147,6 +159,7 @@ __global__ void __launch_bounds__(256, MR == 16 ? 4 : 3) skinny_split_kernel(Ski
     if (MR < 64 || su_block) load_x(0, tid);      // (weight blocks at MR = 64 take x chunk by chunk, see below)
 
     if (su_block) {
+        pin_rest();
         // su part of this split, D[rank][m] (ranks >= r are zero): wave w takes the k16 steps t = w, w+4, ...; the
         // four sums meet in LDS (behind the x slice) in wave order.  The factor rows are fetched with unconditional
         // 16-byte loads (rows and steps past the end clamped, their values masked), the first rank tile's together
@@ -290,6 +303,7 @@ __global__ void __launch_bounds__(256, MR == 16 ? 4 : 3) skinny_split_kernel(Ski
         if (MR == 64 && c == 0) load_xc(0);
         load_chunk(c);
     }
+    pin_rest();
 
     // ---- decode + multiply: D[n][m] += deq(W)[n][k] x[m][k].  Each chunk's slab goes through a wave-private LDS
     // staging area (XOR-swizzled 16-byte pieces: writes and fragment reads are conflict free) to reach the
@@ -464,11 +478,15 @@ __global__ void __launch_bounds__(256, MR == 16 ? 4 : 3) skinny_split_kernel(Ski
 // so that the B rows, partial tiles and su parts are all in flight together.  Every sum runs in a fixed order:
 // parts p = g, g+4, ... per lane group g, then the four groups; splits ascending.
 // RT = 16-rank tiles of the low-rank term (0 = none); VEC = B is fp32 with r % 4 == 0 (16-byte row pieces).
+// (leading scalars: see skinny_split_kernel; count_bits = splits | su_parts << 16, rank_bits = lora_f32 | r << 8 | r_pad << 16)
 template <int RT, bool VEC>
-__global__ void __launch_bounds__(256) skinny_epilogue_kernel(SkinnyEpiArgs g) {
-    // all arguments in scalar registers after one round trip (see skinny_split_kernel)
-    asm volatile("" ::"s"(g.partial), "s"(g.su_part), "s"(g.splits), "s"(g.su_parts), "s"(g.M), "s"(g.N), "s"(g.lora_B),
-                 "s"(g.lora_f32), "s"(g.r), "s"(g.r_pad), "s"(g.su_scale), "s"(g.bias), "s"(g.y), "s"(g.ldy));
+__global__ void __launch_bounds__(256)
+skinny_epilogue_kernel(const float* partial_, const float* su_part_, const void* lora_B_, bf16_t* y_, int32_t ldy_, int32_t M_, int32_t N_,
+                       int32_t count_bits, int32_t rank_bits, SkinnyEpiArgs rest) {
+    SkinnyEpiArgs g = rest;
+    g.partial = partial_; g.su_part = su_part_; g.lora_B = lora_B_; g.y = y_; g.ldy = ldy_; g.M = M_; g.N = N_;
+    g.splits = count_bits & 0xFFFF; g.su_parts = count_bits >> 16;
+    g.lora_f32 = rank_bits & 255; g.r = (rank_bits >> 8) & 255; g.r_pad = rank_bits >> 16;
     // B tile of rank tile jt: [64 lanes][16 pieces of 4 ranks] fp32 (piece 4 e + q = ranks 4q .. 4q+3 of the lane's column
     // e), the pieces of a lane XOR-swizzled with the lane number: conflict-free 16-byte writes and reads
     __shared__ __attribute__((aligned(16))) float bt[RT > 0 ? RT : 1][64 * 64];
@@ -520,6 +538,7 @@ __global__ void __launch_bounds__(256) skinny_epilogue_kernel(SkinnyEpiArgs g) {
             st[jt][u] = g.su_part[(int64_t)(pi < g.su_parts ? pi : g.su_parts - 1) * pstride + (int64_t)m * g.r_pad + jt * 16 + j];
         }
 
+    asm volatile("" ::"s"(g.su_scale), "s"(g.bias));        // the arguments that did not come with the wave, in one go
     // ---- B pieces -> LDS
     if (RT > 0) {
 #pragma unroll
@@ -646,9 +665,14 @@ bool skinny_supported(const xq_weight* w, int64_t M) {
 template <int FMT, int NCH>
 static int launch_split_one(const SkinnyArgs& g, dim3 grid, size_t lds, hipStream_t s) {
     // at most 32 rows of 1040 B + the slabs = 49 KB: below the default dynamic LDS limit
-    if (g.M <= 16) skinny_split_kernel<FMT, 16, NCH><<<grid, 256, lds, s>>>(g);
-    else if (g.M <= 32) skinny_split_kernel<FMT, 32, NCH><<<grid, 256, lds, s>>>(g);
-    else skinny_split_kernel<FMT, 64, NCH><<<grid, 256, lds, s>>>(g);
+    XQ_REQUIRE(g.ldx < (1ll << 31) && g.group < (1 << 24) && g.splits < (1 << 16) && g.chunk_q < (1 << 16),
+               "xq_linear_fwd: internal error: skinny launch arguments out of range");
+    const int32_t fmt_bits = g.group | g.scale_dtype << 24, split_bits = g.splits | g.su_blocks << 16, chunk_bits = g.chunk_q | g.chunk_rem << 16;
+#define XQ_SPLIT_ARGS g.x, (int32_t)g.ldx, g.M, g.N, g.K, g.packed, g.scales, fmt_bits, split_bits, chunk_bits, g.xp, g
+    if (g.M <= 16) skinny_split_kernel<FMT, 16, NCH><<<grid, 256, lds, s>>>(XQ_SPLIT_ARGS);
+    else if (g.M <= 32) skinny_split_kernel<FMT, 32, NCH><<<grid, 256, lds, s>>>(XQ_SPLIT_ARGS);
+    else skinny_split_kernel<FMT, 64, NCH><<<grid, 256, lds, s>>>(XQ_SPLIT_ARGS);
+#undef XQ_SPLIT_ARGS
     return XQ_OK;
 }
 
@@ -693,19 +717,23 @@ static int launch_skinny_split(const xq_weight* w, const bf16_t* x, int64_t ldx,
     const int waves = M < 4 ? (int)M : 4;
     const dim3 egrid((unsigned)xq_cdiv(N, 256), (unsigned)xq_cdiv(M, 4));
     const bool vec = g.lora_f32 && r % 4 == 0 && xq_aligned(lora_B, 16);
+    XQ_REQUIRE(ldy < (1ll << 31) && p.splits < (1 << 16), "xq_linear_fwd: internal error: skinny epilogue arguments out of range");
+    const int32_t count_bits = e.splits | e.su_parts << 16, rank_bits = e.lora_f32 | e.r << 8 | e.r_pad << 16;
+#define XQ_EPI_ARGS e.partial, e.su_part, e.lora_B, e.y, (int32_t)e.ldy, e.M, e.N, count_bits, rank_bits, e
 #define XQ_EPI(RT)                                                                                      \
     do {                                                                                                \
-        if (vec) skinny_epilogue_kernel<RT, true><<<egrid, waves * 64, 0, stream>>>(e);                 \
-        else skinny_epilogue_kernel<RT, false><<<egrid, waves * 64, 0, stream>>>(e);                    \
+        if (vec) skinny_epilogue_kernel<RT, true><<<egrid, waves * 64, 0, stream>>>(XQ_EPI_ARGS);       \
+        else skinny_epilogue_kernel<RT, false><<<egrid, waves * 64, 0, stream>>>(XQ_EPI_ARGS);          \
     } while (0)
     switch (rp >> 4) {
-        case 0: skinny_epilogue_kernel<0, false><<<egrid, waves * 64, 0, stream>>>(e); break;
+        case 0: skinny_epilogue_kernel<0, false><<<egrid, waves * 64, 0, stream>>>(XQ_EPI_ARGS); break;
         case 1: XQ_EPI(1); break;
         case 2: XQ_EPI(2); break;
         case 3: XQ_EPI(3); break;
         default: XQ_EPI(4); break;
     }
 #undef XQ_EPI
+#undef XQ_EPI_ARGS
     return XQ_OK;
 }
 

@@ -35,6 +35,8 @@
 // Measured on an MI355X, launches back to back (block_fp8, r = 16, M = 1): 4096->12288 (48 MiB) 11.4 us against 15.6 us
 // for the two-launch organisation (10.0 us without a low-rank term), 4096->4096 7.4 against 8.8, 4096->24576 (96 MiB)
 // 18.4 against 22.1.
+#include <stdlib.h>
+
 #include <atomic>
 #include <mutex>
 
@@ -84,7 +86,7 @@ struct SkinnyRowsArgs {
 // their way to LDS); R: rounds -- a block walks R sets of G row groups, each step's registers refilled for the next
 // round as soon as the step has been multiplied, so the weight stream never stops (N % (16 G R) == 0 when R > 1)
 // (`bx` of `nb`: the block's place among the blocks of its forward -- the grid of a launch holds one forward or several)
-template <int FMT, int G, int NJ, int MR, int R>
+template <int FMT, int G, int NJ, int MR, int R, bool PRE = false>
 __device__ __forceinline__ void skinny_rows_body(const SkinnyRowsArgs& g, const int bx, const int nb) {
     constexpr bool F8 = FMT == XQ_FMT_FP8;
     constexpr int EPS = F8 ? 64 : 128;                 // K elements of a row per load step
@@ -93,9 +95,10 @@ __device__ __forceinline__ void skinny_rows_body(const SkinnyRowsArgs& g, const 
     constexpr int XC = (NJ * EPS + 511) / 512;         // 1 KB pieces of an x row slice
     constexpr int NSC = FMT == XQ_FMT_NVFP4 ? 2 : 1;   // scale registers per load
     // every argument in scalar registers after one round trip (lazily placed argument loads cost a round trip each)
-    asm volatile("" ::"s"(g.x), "s"(g.ldx), "s"(g.M), "s"(g.N), "s"(g.K), "s"(g.packed), "s"(g.scales), "s"(g.global_scale),
-                 "s"(g.gshift), "s"(g.scale_dtype), "s"(g.lora_A), "s"(g.lora_B), "s"(g.r), "s"(g.su_scale), "s"(g.bias), "s"(g.y),
-                 "s"(g.ldy), "s"(g.xpitch), "s"(g.slab), "s"(g.nsu), "s"(g.slot), "s"(g.spin_limit));
+    if constexpr (!PRE)
+        asm volatile("" ::"s"(g.x), "s"(g.ldx), "s"(g.M), "s"(g.N), "s"(g.K), "s"(g.packed), "s"(g.scales), "s"(g.global_scale),
+                     "s"(g.gshift), "s"(g.scale_dtype), "s"(g.lora_A), "s"(g.lora_B), "s"(g.r), "s"(g.su_scale), "s"(g.bias), "s"(g.y),
+                     "s"(g.ldy), "s"(g.xpitch), "s"(g.slab), "s"(g.nsu), "s"(g.slot), "s"(g.spin_limit));
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -277,6 +280,9 @@ __device__ __forceinline__ void skinny_rows_body(const SkinnyRowsArgs& g, const 
 #pragma unroll
     for (int t = 0; t < DJ; ++t) load_step(t);
     __builtin_amdgcn_sched_barrier(0);
+    // (PRE: the arguments the loads above need arrived in registers with the wave; the others are fetched now, in one go)
+    if constexpr (PRE)
+        asm volatile("" ::"s"(g.global_scale), "s"(g.lora_B), "s"(g.r), "s"(g.su_scale), "s"(g.bias), "s"(g.y), "s"(g.ldy), "s"(g.spin_limit));
 
     // ---- x slice -> LDS (the wave's own area; LDS operations of one wave execute in order, no barrier)
 #pragma unroll
@@ -495,6 +501,23 @@ __global__ void __launch_bounds__(512, 1) skinny_rows_kernel(SkinnyRowsArgs g) {
     skinny_rows_body<FMT, G, NJ, MR, R>(g, (int)blockIdx.x, (int)gridDim.x);
 }
 
+// The same kernel with the arguments its first loads need as leading scalars: the hardware hands a kernel's first 16
+// argument dwords to each wave in registers (where the platform supports it; otherwise they are fetched like the rest),
+// so the wave's first loads do not wait for a round trip to the argument block.
+template <int FMT, int G, int NJ, int MR, int R>
+__global__ void __launch_bounds__(512, 1) skinny_rows_kernel_p(const bf16_t* x, int32_t ldx, int32_t M, int32_t N, int32_t K,
+                                                               const uint8_t* packed, const uint8_t* scales, uint32_t* slot,
+                                                               const float* lora_A, int32_t nsu, int32_t fmt_bits, SkinnyRowsArgs rest) {
+    SkinnyRowsArgs g = rest;
+    g.x = x; g.ldx = ldx; g.M = M; g.N = N; g.K = K; g.packed = packed; g.scales = scales; g.slot = slot; g.lora_A = lora_A;
+    g.nsu = nsu; g.gshift = fmt_bits & 255; g.scale_dtype = fmt_bits >> 8;
+    g.xpitch = (K >> 3) * 2 + 16;
+    int slab = M * g.xpitch + 64;
+    slab = slab < (G * R + 1) * 1024 ? (G * R + 1) * 1024 : slab;
+    g.slab = (slab + 15) & ~15;
+    skinny_rows_body<FMT, G, NJ, MR, R, true>(g, (int)blockIdx.x, (int)gridDim.x);
+}
+
 // Several forwards that share x (and format, K and M) in one launch: the grid is the forwards' grids one after the other,
 // each forward with its own weight, factors, outputs and slot; a block finds its forward by its index.
 constexpr int kRowsMaxJobs = 4;
@@ -663,13 +686,20 @@ static int launch_rows_one(const SkinnyRowsArgs& g, const SkinnyRowsBatch* batch
         hipError_t e = hipFuncSetAttribute((const void*)skinny_rows_kernel<FMT, G, NJ, MR, R>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e == hipSuccess)
             e = hipFuncSetAttribute((const void*)skinny_rows_multi_kernel<FMT, G, NJ, MR, R>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e == hipSuccess)
+            e = hipFuncSetAttribute((const void*)skinny_rows_kernel_p<FMT, G, NJ, MR, R>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) {
             xq_set_error("xq_linear_fwd: cannot raise the dynamic LDS limit: %s", hipGetErrorString(e));
             return XQ_ERR_LAUNCH;
         }
         attr_set = true;
     }
+    // XQ_ROWS_PRELOAD=0 launches the form that fetches every argument itself (A/B measurements)
+    static const bool preload = [] { const char* e = getenv("XQ_ROWS_PRELOAD"); return e ? atoi(e) != 0 : true; }();
     if (batch) skinny_rows_multi_kernel<FMT, G, NJ, MR, R><<<grid, 512, lds, s>>>(*batch);
+    else if (preload && g.ldx < (1ll << 31))
+        skinny_rows_kernel_p<FMT, G, NJ, MR, R><<<grid, 512, lds, s>>>(g.x, (int32_t)g.ldx, g.M, g.N, g.K, g.packed, g.scales, g.slot, g.lora_A,
+                                                                         g.nsu, g.gshift | g.scale_dtype << 8, g);
     else skinny_rows_kernel<FMT, G, NJ, MR, R><<<grid, 512, lds, s>>>(g);
     return XQ_OK;
 }
