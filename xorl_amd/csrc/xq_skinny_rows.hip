@@ -525,11 +525,16 @@ struct SkinnyRowsBatch {
     SkinnyRowsArgs job[kRowsMaxJobs];
     int32_t first[kRowsMaxJobs + 1];    // first block of each forward; entries past the last forward hold the grid size
 };
+// (the boundaries between the forwards are leading scalars, with the wave from the start: the one fetch of the block's own
+// argument set does not wait for another fetch to tell it which set that is)
 template <int FMT, int G, int NJ, int MR, int R>
-__global__ void __launch_bounds__(512, 1) skinny_rows_multi_kernel(SkinnyRowsBatch b) {
+__global__ void __launch_bounds__(512, 1) skinny_rows_multi_kernel(int32_t first1, int32_t first2, int32_t first3, int32_t first4,
+                                                                   SkinnyRowsBatch b) {
     const int bx = (int)blockIdx.x;
-    const int i = (bx >= b.first[1] ? 1 : 0) + (bx >= b.first[2] ? 1 : 0) + (bx >= b.first[3] ? 1 : 0);   // uniform
-    skinny_rows_body<FMT, G, NJ, MR, R>(b.job[i], bx - b.first[i], b.first[i + 1] - b.first[i]);
+    const int i = (bx >= first1 ? 1 : 0) + (bx >= first2 ? 1 : 0) + (bx >= first3 ? 1 : 0);   // uniform
+    const int lo = i == 0 ? 0 : i == 1 ? first1 : i == 2 ? first2 : first3;
+    const int hi = i == 0 ? first1 : i == 1 ? first2 : i == 2 ? first3 : first4;
+    skinny_rows_body<FMT, G, NJ, MR, R>(b.job[i], bx - lo, hi - lo);
 }
 
 // ---- slots: device memory that belongs to the library (zero when the code object is loaded).
@@ -696,7 +701,7 @@ static int launch_rows_one(const SkinnyRowsArgs& g, const SkinnyRowsBatch* batch
     }
     // XQ_ROWS_PRELOAD=0 launches the form that fetches every argument itself (A/B measurements)
     static const bool preload = [] { const char* e = getenv("XQ_ROWS_PRELOAD"); return e ? atoi(e) != 0 : true; }();
-    if (batch) skinny_rows_multi_kernel<FMT, G, NJ, MR, R><<<grid, 512, lds, s>>>(*batch);
+    if (batch) skinny_rows_multi_kernel<FMT, G, NJ, MR, R><<<grid, 512, lds, s>>>(batch->first[1], batch->first[2], batch->first[3], batch->first[4], *batch);
     else if (preload && g.ldx < (1ll << 31))
         skinny_rows_kernel_p<FMT, G, NJ, MR, R><<<grid, 512, lds, s>>>(g.x, (int32_t)g.ldx, g.M, g.N, g.K, g.packed, g.scales, g.slot, g.lora_A,
                                                                          g.nsu, g.gshift | g.scale_dtype << 8, g);
