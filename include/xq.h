@@ -162,6 +162,19 @@ int xq_linear_fwd(const xq_weight* w, const void* x, int64_t ldx, int64_t M,
                   const void* bias_bf16, void* y, int64_t ldy, void* su_out,
                   void* workspace, int64_t workspace_bytes, void* stream);
 
+/* h[M, I] = silu(gate) * up for a weight that holds gate | up stacked, W [2 I, K] (one QLoRA linear: the reference's
+ * default gate_up_proj module, qlora/utils.py:33-37, followed by fused_silu_and_mul, ops/fused_silu_and_mul.py:22-60;
+ * call site models/transformers/qwen3/modeling_qwen3.py:62-70): the forward of xq_linear_fwd on all 2 I rows and the
+ * SwiGLU arithmetic of xq_silu_mul_fwd on its rounded outputs (same rounding points, bit-identical to the two calls).
+ * For M <= 16, where the weight takes the one-launch skinny kernel in two rounds (I % 48 == 0, K <= 4096 at one byte
+ * per weight), one launch: a block holds the gate rows and the up rows of its columns and writes h directly.
+ * Otherwise the two calls run one after the other inside this one (gate | up goes through the workspace).
+ * workspace: xq_linear_fwd_swiglu_workspace_bytes(M, 2 I, K, r) bytes, 256-byte aligned. */
+int64_t xq_linear_fwd_swiglu_workspace_bytes(int64_t M, int64_t N2, int64_t K, int r);
+int xq_linear_fwd_swiglu(const xq_weight* w, const void* x, int64_t ldx, int64_t M,
+                         const void* lora_A, const void* lora_B, int lora_dtype, int r, float scaling,
+                         const void* bias_bf16, void* h, int64_t ldh, void* workspace, int64_t workspace_bytes, void* stream);
+
 /* Several forwards that share x: y_i = x . deq(W_i)^T + bias_i + s_i * (x . A_i^T) . B_i^T, i < n_jobs <= 4.
  * Replaces the separate module calls of the reference's attention and MLP blocks
  * on one input (q_proj / k_proj / v_proj: src/xorl/models/layers/attention/multi_head_attention.py:93-95;

@@ -209,3 +209,41 @@ def test_mlp_forward_without_autograd_is_the_module_calls(hip_device, fmt):
     xd = gen((5, H), 1.0, 99, torch.bfloat16).to(hip_device)
     with torch.no_grad():
         assert torch.equal(qlora_mlp_forward(g, u, d, xd), d(silu_and_mul(g(xd), u(xd))))
+
+
+@pytest.mark.parametrize("fmt,I,K,r,has_bias", [
+    ("block_fp8", 12288, 4096, 16, False),     # Qwen3-8B gate | up: one launch (two rounds of three row groups) up to 16 rows
+    ("block_fp8", 1536, 2048, 8, True),        # 4 steps of the fp8 kernel
+    ("int4", 12288, 4096, 16, True),
+    ("nf4", 6144, 2048, 8, False),
+    ("nvfp4", 12288, 4096, 16, False),
+    ("block_fp8", 1024, 1024, 4, True),        # I not a multiple of 48: the two calls inside the one
+])
+def test_gate_up_with_swiglu_finish(hip_device, fmt, I, K, r, has_bias):
+    """xq_linear_fwd_swiglu / qlora_gate_up_silu: h = silu(gate) * up from the stacked weight, bit for bit the module call
+    followed by the SwiGLU kernel, at decode sizes (one launch) and above, and against the fp64 program."""
+    from xorl_amd.functional import silu_and_mul
+    from xorl_amd.qlora import qlora_gate_up_silu
+
+    m, w_ref = make_dense_module(fmt, 2 * I, K, r, 2 * r, seed=I + K, device=hip_device, bias=has_bias)
+    A, B = m.lora_A.detach().cpu(), m.lora_B.detach().cpu()
+    bias = None if m.bias is None else m.bias.detach().cpu()
+    for M in (1, 7, 16, 24, 64):
+        x = gen((M, K), 1.0, 500 + M, torch.bfloat16)
+        xd = x.to(hip_device)
+        with torch.no_grad():
+            got = qlora_gate_up_silu(m, xd)
+            gate, up = m(xd).chunk(2, dim=-1)
+            want = silu_and_mul(gate, up)
+        assert got.shape == (M, I) and got.dtype == torch.bfloat16
+        assert torch.equal(got, want)
+        y = R.linear_fwd_bwd_exact(x, w_ref, A, B, m.scaling, bias=bias)["y"]
+        g64, u64 = y[:, :I], y[:, I:]
+        close(got.cpu(), g64 * torch.sigmoid(g64) * u64, 2e-2)
+        with torch.no_grad():
+            assert torch.equal(qlora_gate_up_silu(m, xd), got)        # the same bits from a second call
+    # decode sizes take one region of the library's launch counter, the two calls two
+    if I % 48 == 0:
+        xd = gen((4, K), 1.0, 3, torch.bfloat16).to(hip_device)
+        with torch.no_grad():
+            assert _launches(lambda: qlora_gate_up_silu(m, xd)) == 1

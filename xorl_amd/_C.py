@@ -94,6 +94,9 @@ _SIGNATURES = {
     "xq_linear_workspace_bytes": (_I64, [_I64, _I64, _I64, _INT]),
     # w, x, ldx, M, A, B, lora_dtype, r, scaling, bias, y, ldy, su_out, ws, ws_bytes, stream
     "xq_linear_fwd": (_INT, [_W, _P, _I64, _I64, _P, _P, _INT, _INT, _F, _P, _P, _I64, _P, _P, _I64, _P]),
+    "xq_linear_fwd_swiglu_workspace_bytes": (_I64, [_I64, _I64, _I64, _INT]),
+    # w, x, ldx, M, A, B, lora_dtype, r, scaling, bias, h, ldh, ws, ws_bytes, stream
+    "xq_linear_fwd_swiglu": (_INT, [_W, _P, _I64, _I64, _P, _P, _INT, _INT, _F, _P, _P, _I64, _P, _I64, _P]),
     # jobs, n_jobs, M
     "xq_linear_fwd_multi_workspace_bytes": (_I64, [_P, _INT, _I64]),
     # jobs, n_jobs, x, ldx, M, lora_dtype, ws, ws_bytes, stream

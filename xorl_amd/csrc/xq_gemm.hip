@@ -500,6 +500,47 @@ static int static_scratch(void** out, const char* who) {
 
 extern "C" int64_t xq_static_scratch_bytes(void) { return XQ_STATIC_SCRATCH_BYTES; }
 
+extern "C" int64_t xq_linear_fwd_swiglu_workspace_bytes(int64_t M, int64_t N2, int64_t K, int r) {
+    if (M < 0 || N2 < 0) return 0;
+    return align256(xq_linear_workspace_bytes(M, N2, K, r)) + align256(M * N2 * 2) + 256;
+}
+
+extern "C" int xq_linear_fwd_swiglu(const xq_weight* w, const void* x, int64_t ldx, int64_t M, const void* lora_A, const void* lora_B,
+                                    int lora_dtype, int r, float scaling, const void* bias_bf16, void* h, int64_t ldh, void* workspace,
+                                    int64_t workspace_bytes, void* stream_) {
+    int rc = check_dense(w, "xq_linear_fwd_swiglu");
+    if (rc) return rc;
+    const int64_t N2 = w->rows, K = w->cols, I = N2 / 2;
+    XQ_REQUIRE(N2 % 16 == 0, "xq_linear_fwd_swiglu: the weight holds gate | up, [2 I, K] with I %% 8 == 0; got %lld rows", (long long)N2);
+    XQ_REQUIRE(M >= 0 && (M == 0 || (x && h)), "xq_linear_fwd_swiglu: NULL activation pointer");
+    XQ_REQUIRE(r >= 0 && r <= 64, "xq_linear_fwd_swiglu: LoRA rank %d out of range [0, 64]", r);
+    XQ_REQUIRE(r == 0 || (lora_A && lora_B), "xq_linear_fwd_swiglu: LoRA factors are NULL");
+    XQ_REQUIRE(lora_dtype == XQ_DT_F32 || lora_dtype == XQ_DT_BF16, "xq_linear_fwd_swiglu: bad lora_dtype");
+    if (M == 0) return XQ_OK;
+    XQ_REQUIRE(ldh % 8 == 0 && xq_aligned(h, 16), "xq_linear_fwd_swiglu: h rows must be 16-byte aligned");
+    XQ_REQUIRE(workspace && xq_aligned(workspace, 256) && workspace_bytes >= xq_linear_fwd_swiglu_workspace_bytes(M, N2, K, r),
+               "xq_linear_fwd_swiglu: workspace missing, misaligned or smaller than xq_linear_fwd_swiglu_workspace_bytes()");
+    hipStream_t stream = (hipStream_t)stream_;
+    // decode sizes: one launch that holds a column's gate and up rows in the same block
+    if (g_skinny_enabled && skinny_rows_enabled() && skinny_supported(w, M) && ldx % 8 == 0 && ldx < (1ll << 31) && xq_aligned(x, 16) &&
+        xq_aligned(w->packed, 16) && skinny_rows_swiglu_supported(w, M, lora_A, lora_B, lora_dtype, r)) {
+        const double bytes = (double)xq_packed_bytes_per_expert(w) + (double)xq_scale_bytes_per_expert(w) + 2.0 * M * K + 2.0 * M * I +
+                             4.0 * r * (K + N2);
+        const bool timed = xq_profile_mark_begin(stream, bytes);
+        rc = launch_skinny_rows_swiglu(w, (const bf16_t*)x, ldx, M, lora_A, lora_B, r, scaling, (const bf16_t*)bias_bf16, (bf16_t*)h, ldh,
+                                       workspace, stream);
+        if (timed) xq_profile_mark_end(stream);
+        if (rc) return rc;
+        XQ_CHECK_LAUNCH("skinny forward with SwiGLU");
+        return XQ_OK;
+    }
+    // otherwise the forward into the workspace, then the elementwise kernel
+    const int64_t lin = align256(xq_linear_workspace_bytes(M, N2, K, r));
+    bf16_t* gu = (bf16_t*)((uint8_t*)workspace + lin);
+    if ((rc = xq_linear_fwd(w, x, ldx, M, lora_A, lora_B, lora_dtype, r, scaling, bias_bf16, gu, N2, nullptr, workspace, lin, stream_))) return rc;
+    return xq_silu_mul_fwd(gu, gu + I, N2, nullptr, h, ldh, M, I, stream_);
+}
+
 extern "C" int64_t xq_linear_fwd_multi_workspace_bytes(const xq_linear_job* jobs, int n_jobs, int64_t M) {
     int64_t need = 256 * 8;
     if (!jobs) return need;

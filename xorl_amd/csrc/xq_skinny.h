@@ -56,6 +56,11 @@ bool skinny_rows_supported(const xq_weight* w, int64_t M, const void* lora_A, co
 int launch_skinny_rows(const xq_weight* w, const bf16_t* x, int64_t ldx, int64_t M, const void* lora_A, const void* lora_B, int r,
                        float scaling, const bf16_t* bias, bf16_t* y, int64_t ldy, const void* slot_key, hipStream_t stream);
 
+// gate | up as one weight [2 I, K] with the SwiGLU finish: h [M, I] = silu(gate) * up in one launch
+bool skinny_rows_swiglu_supported(const xq_weight* w, int64_t M, const void* lora_A, const void* lora_B, int lora_dtype, int r);
+int launch_skinny_rows_swiglu(const xq_weight* w, const bf16_t* x, int64_t ldx, int64_t M, const void* lora_A, const void* lora_B, int r,
+                              float scaling, const bf16_t* bias, bf16_t* h, int64_t ldh, const void* slot_key, hipStream_t stream);
+
 // several forwards that share x (same format, K and M) as one launch of the same kernel; each forward has its own slot,
 // keyed by addresses 256 bytes apart from `slot_key` (the caller's workspace holds at least 256 bytes per forward)
 struct SkinnyRowsJob {

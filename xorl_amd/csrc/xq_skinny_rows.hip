@@ -86,8 +86,12 @@ struct SkinnyRowsArgs {
 // their way to LDS); R: rounds -- a block walks R sets of G row groups, each step's registers refilled for the next
 // round as soon as the step has been multiplied, so the weight stream never stops (N % (16 G R) == 0 when R > 1)
 // (`bx` of `nb`: the block's place among the blocks of its forward -- the grid of a launch holds one forward or several)
-template <int FMT, int G, int NJ, int MR, int R, bool PRE = false>
+// GU (two rounds only): the weight is gate | up stacked, [2 I, K]; round 0 walks the block's gate rows and round 1 the up rows
+// of the same columns, I rows further on, and the finish writes h[m][n] = bf16(bf16(silu(gate)) * up) from the two rounded
+// outputs (ops/fused_silu_and_mul.py:22-60) to y [M, I] instead of the two outputs themselves.
+template <int FMT, int G, int NJ, int MR, int R, bool PRE = false, bool GU = false>
 __device__ __forceinline__ void skinny_rows_body(const SkinnyRowsArgs& g, const int bx, const int nb) {
+    static_assert(!GU || R == 2, "the SwiGLU finish pairs the two rounds of a block");
     constexpr bool F8 = FMT == XQ_FMT_FP8;
     constexpr int EPS = F8 ? 64 : 128;                 // K elements of a row per load step
     constexpr int MPS = EPS / 32;                      // MFMAs per step and row group
@@ -106,7 +110,9 @@ __device__ __forceinline__ void skinny_rows_body(const SkinnyRowsArgs& g, const 
     const int ks = g.K >> 3;                    // K elements per wave
     const int k0 = wave * ks;
     const int nj = ks / EPS;                    // load steps of this launch, 1 .. NJ
-    const int n0 = bx * (16 * G * R);
+    const int n0 = bx * (16 * G * (GU ? 1 : R));
+    const int rstride = GU ? g.N >> 1 : 16 * G;        // rows from a round's rows to the next round's
+    const int nlim = GU ? g.N >> 1 : g.N;              // end of the rows that round 0 may walk
     const int XP = g.xpitch;
     unsigned char* slab = smem + wave * g.slab;
     float* su_tot = (float*)(smem + 8 * g.slab);           // [16 m][16 j], then a flag
@@ -241,12 +247,12 @@ __device__ __forceinline__ void skinny_rows_body(const SkinnyRowsArgs& g, const 
 #pragma unroll
     for (int gi = 0; gi < G; ++gi) {
         int n = n0 + gi * 16 + rn;
-        n = n < g.N ? n : g.N - 1;
+        n = n < nlim ? n : nlim - 1;
         erow[gi] = (int64_t)n * g.K + k0 + kq * (EPS / 4);
         wp[gi] = g.packed + ((int64_t)n * g.K + k0) / EB + kq * 16;
     }
     const int scols = (g.K + 127) >> 7;
-    const int64_t round_bytes = (int64_t)16 * G * g.K / EB;          // from a round's rows to the next round's
+    const int64_t round_bytes = (int64_t)rstride * g.K / EB;         // from a round's rows to the next round's
     auto load_step = [&](int t) {
         {
             const int rr = t / NJ, jj = t % NJ, j = t % DJ;
@@ -256,7 +262,7 @@ __device__ __forceinline__ void skinny_rows_body(const SkinnyRowsArgs& g, const 
                 w[j][gi] = *(const u32x4*)(wp[gi] + rr * round_bytes + jc * 64);
                 if (FMT == XQ_FMT_FP8) {
                     // one scale per 128 x 128 block: the same for the 16 rows of a group and the 64 elements of a step
-                    const int nb = n0 + (rr * G + gi) * 16 < g.N ? n0 + (rr * G + gi) * 16 : g.N - 16;
+                    const int nb = n0 + rr * rstride + gi * 16 < g.N ? n0 + rr * rstride + gi * 16 : g.N - 16;
                     sc[j][gi][0] = ((const __attribute__((address_space(4))) uint32_t*)g.scales)[(nb >> 7) * scols + ((k0 + jc * 64) >> 7)];
                 } else if (FMT == XQ_FMT_INT4) {
                     const int64_t si = (erow[gi] + rr * round_bytes * EB + jc * EPS) >> g.gshift;      // group % 32 == 0: one scale per load
@@ -300,15 +306,16 @@ __device__ __forceinline__ void skinny_rows_body(const SkinnyRowsArgs& g, const 
     const int nl = tid & 63;
     f32x4 bq = {0.0f, 0.0f, 0.0f, 0.0f};
     const int brow = tid >> 2, bpiece = tid & 3;
-    const bool bvalid = lora && brow < 16 * G * R && n0 + brow < g.N && 4 * bpiece < g.r;
+    const int brow_n = n0 + (brow / (16 * G)) * rstride + brow % (16 * G);     // the weight row of the block's row `brow`
+    const bool bvalid = lora && brow < 16 * G * R && brow_n < g.N && 4 * bpiece < g.r;
     float bias_v[R];
     auto finish_loads = [&]() {
-        const int64_t bn = n0 + brow < g.N ? n0 + brow : g.N - 1;
+        const int64_t bn = brow_n < g.N ? brow_n : g.N - 1;
         const float* bp = lora ? g.lora_B + bn * g.r + (4 * bpiece < g.r ? 4 * bpiece : 0) : (const float*)g.x;
         bq = *(const f32x4*)bp;
 #pragma unroll
         for (int rr = 0; rr < R; ++rr) {
-            const int nfin = (nl < 16 * G && n0 + rr * 16 * G + nl < g.N) ? n0 + rr * 16 * G + nl : g.N - 1;
+            const int nfin = (nl < 16 * G && n0 + rr * rstride + nl < g.N) ? n0 + rr * rstride + nl : g.N - 1;
             bias_v[rr] = bf16_to_f32((g.bias ? g.bias : g.x)[g.bias ? nfin : 0]);
         }
         if (lora && wave == 0) gen = __hip_atomic_load(ctl, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -463,10 +470,11 @@ __device__ __forceinline__ void skinny_rows_body(const SkinnyRowsArgs& g, const 
     const int mg = tid >> 6;
     const int gi_f = nl >> 4, nloc = nl & 15;
     const bool ok = !lora || ((const int*)su_tot)[256] != 0;
+    float gate_v[2] = {0.0f, 0.0f};                     // GU: the rounded gate outputs of round 0, until round 1 has the up outputs
 #pragma unroll
     for (int rr = 0; rr < R; ++rr) {
         const int nrow = rr * 16 * G + nl;              // row of the block
-        const bool nvalid = nl < 16 * G && n0 + nrow < g.N;
+        const bool nvalid = nl < 16 * G && n0 + rr * rstride + nl < g.N && n0 + nl < nlim;
         f32x4 bv[4];
 #pragma unroll
         for (int q = 0; q < 4; ++q) bv[q] = *(const f32x4*)(b_tile + (nl < 16 * G ? nrow : 0) * 20 + 4 * q);
@@ -489,7 +497,12 @@ __device__ __forceinline__ void skinny_rows_body(const SkinnyRowsArgs& g, const 
                 }
                 if (g.bias) o += bias_v[rr];
                 if (!ok) o = __builtin_nanf("");
-                g.y[(int64_t)m * g.ldy + n0 + nrow] = to_bf16(o);
+                if constexpr (GU) {
+                    if (rr == 0) gate_v[mm] = round_bf16(o);
+                    else g.y[(int64_t)m * g.ldy + n0 + nl] = to_bf16(round_bf16(gate_v[mm] * sigmoid_f32(gate_v[mm])) * round_bf16(o));
+                } else {
+                    g.y[(int64_t)m * g.ldy + n0 + nrow] = to_bf16(o);
+                }
             }
         }
     }
@@ -504,7 +517,7 @@ __global__ void __launch_bounds__(512, 1) skinny_rows_kernel(SkinnyRowsArgs g) {
 // The same kernel with the arguments its first loads need as leading scalars: the hardware hands a kernel's first 16
 // argument dwords to each wave in registers (where the platform supports it; otherwise they are fetched like the rest),
 // so the wave's first loads do not wait for a round trip to the argument block.
-template <int FMT, int G, int NJ, int MR, int R>
+template <int FMT, int G, int NJ, int MR, int R, bool GU = false>
 __global__ void __launch_bounds__(512, 1) skinny_rows_kernel_p(const bf16_t* x, int32_t ldx, int32_t M, int32_t N, int32_t K,
                                                                const uint8_t* packed, const uint8_t* scales, uint32_t* slot,
                                                                const float* lora_A, int32_t nsu, int32_t fmt_bits, SkinnyRowsArgs rest) {
@@ -515,7 +528,7 @@ __global__ void __launch_bounds__(512, 1) skinny_rows_kernel_p(const bf16_t* x, 
     int slab = M * g.xpitch + 64;
     slab = slab < (G * R + 1) * 1024 ? (G * R + 1) * 1024 : slab;
     g.slab = (slab + 15) & ~15;
-    skinny_rows_body<FMT, G, NJ, MR, R, true>(g, (int)blockIdx.x, (int)gridDim.x);
+    skinny_rows_body<FMT, G, NJ, MR, R, true, GU>(g, (int)blockIdx.x, (int)gridDim.x);
 }
 
 // Several forwards that share x (and format, K and M) in one launch: the grid is the forwards' grids one after the other,
@@ -771,6 +784,56 @@ int launch_skinny_rows(const xq_weight* w, const bf16_t* x, int64_t ldx, int64_t
         case XQ_FMT_NF4: return launch_rows_fmt<XQ_FMT_NF4>(g, nullptr, p, grid, stream);
         default: return launch_rows_fmt<XQ_FMT_NVFP4>(g, nullptr, p, grid, stream);
     }
+}
+
+// ---- gate | up with the SwiGLU finish: h = silu(gate) * up from one weight [2 I, K] in one launch
+template <int FMT, int NJ, int MR>
+static int launch_rows_gu_one(const SkinnyRowsArgs& g, unsigned grid, size_t lds, hipStream_t s) {
+    static std::atomic<bool> attr_set{false};
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute((const void*)skinny_rows_kernel_p<FMT, 3, NJ, MR, 2, true>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e != hipSuccess) {
+            xq_set_error("xq_linear_fwd_swiglu: cannot raise the dynamic LDS limit: %s", hipGetErrorString(e));
+            return XQ_ERR_LAUNCH;
+        }
+        attr_set = true;
+    }
+    skinny_rows_kernel_p<FMT, 3, NJ, MR, 2, true><<<grid, 512, lds, s>>>(g.x, (int32_t)g.ldx, g.M, g.N, g.K, g.packed, g.scales, g.slot, g.lora_A, g.nsu,
+                                                                          g.gshift | g.scale_dtype << 8, g);
+    return XQ_OK;
+}
+
+template <int FMT, int NJ>
+static int launch_rows_gu_mr(const SkinnyRowsArgs& g, int MR, unsigned grid, size_t lds, hipStream_t s) {
+    if (MR == 1) return launch_rows_gu_one<FMT, NJ, 1>(g, grid, lds, s);
+    if (MR == 8) return launch_rows_gu_one<FMT, NJ, 8>(g, grid, lds, s);
+    return launch_rows_gu_one<FMT, NJ, 16>(g, grid, lds, s);
+}
+
+// true when w [2 I, K] takes the one-launch kernel in two rounds of three row groups, so that a block can hold the gate and
+// the up rows of the same 48 columns
+bool skinny_rows_swiglu_supported(const xq_weight* w, int64_t M, const void* lora_A, const void* lora_B, int lora_dtype, int r) {
+    if (w->rows % 2 != 0 || !skinny_rows_supported(w, M, lora_A, lora_B, lora_dtype, r)) return false;
+    RowsPlan p;
+    if (!rows_plan(w, M, &p)) return false;
+    return p.R == 2 && p.G == 3 && (w->rows / 2) % 48 == 0 && (w->format == XQ_FMT_FP8 ? p.njt <= 8 : p.njt <= 4);
+}
+
+int launch_skinny_rows_swiglu(const xq_weight* w, const bf16_t* x, int64_t ldx, int64_t M, const void* lora_A, const void* lora_B, int r,
+                              float scaling, const bf16_t* bias, bf16_t* h, int64_t ldh, const void* slot_key, hipStream_t stream) {
+    RowsPlan p;
+    XQ_REQUIRE(rows_plan(w, M, &p) && p.R == 2 && p.G == 3 && ldx < (1ll << 31),
+               "xq_linear_fwd_swiglu: internal error: shape not supported by the one-launch skinny kernel");
+    SkinnyRowsArgs g;
+    const int rc = rows_args(w, p, x, ldx, M, lora_A, lora_B, r, scaling, bias, h, ldh, slot_key, &g);
+    if (rc) return rc;
+    const unsigned grid = (unsigned)(w->rows / 2 / 48);
+#define XQ_GU_CASE(F, NN) \
+    if (w->format == F && p.njt == NN) return launch_rows_gu_mr<F, NN>(g, p.MR, grid, p.lds, stream)
+    XQ_GU_CASE(XQ_FMT_FP8, 4); XQ_GU_CASE(XQ_FMT_FP8, 8);
+    XQ_GU_CASE(XQ_FMT_INT4, 4); XQ_GU_CASE(XQ_FMT_NF4, 4); XQ_GU_CASE(XQ_FMT_NVFP4, 4);
+#undef XQ_GU_CASE
+    XQ_REQUIRE(false, "xq_linear_fwd_swiglu: internal error: no kernel for %d load steps", p.njt);
 }
 
 // ---- several forwards that share x as one launch

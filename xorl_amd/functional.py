@@ -263,6 +263,40 @@ def qlora_linear(x: Tensor, qw: QuantWeight, lora_A: Optional[Tensor], lora_B: O
     return QLoRALinearFunction.apply(x, lora_A, lora_B, bias, qw, r, scaling, training)
 
 
+def qlora_linear_swiglu(x: Tensor, qw: QuantWeight, lora_A: Optional[Tensor], lora_B: Optional[Tensor], r: int, scaling: float,
+                        bias: Optional[Tensor] = None) -> Tensor:
+    """Forward-only: ``silu_and_mul(*qlora_linear(x, qw, ...).chunk(2, dim=-1))`` for a weight that holds gate | up stacked
+    ([2 I, K]: the reference's default ``gate_up_proj`` module, qlora/utils.py:33-37, followed by ``fused_silu_and_mul``,
+    models/transformers/qwen3/modeling_qwen3.py:62-70) as one library call (xq_linear_fwd_swiglu); at decode sizes one
+    kernel launch that writes h [.., I] directly.  Bit-identical to the two calls.  No autograd."""
+    if x.dtype != torch.bfloat16:
+        raise _C.XqError(f"activations must be bf16, got {x.dtype}")
+    if r > MAX_FUSED_RANK:
+        raise _C.XqError(f"qlora_linear_swiglu: rank {r} exceeds {MAX_FUSED_RANK}")
+    if torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in (x, lora_A, lora_B, bias)):
+        raise _C.XqError("qlora_linear_swiglu is forward-only: call it under torch.no_grad()")
+    if qw.rows % 2:
+        raise _C.XqError(f"qlora_linear_swiglu: the weight must hold gate | up, got {qw.rows} rows")
+    _C.require_hip(x)
+    x2 = _as_2d(x)
+    M, K = x2.shape
+    if qw.cols != K:
+        raise _C.XqError(f"input width {K} != in_features {qw.cols}")
+    I = qw.rows // 2
+    dev = x.device
+    A = lora_A.detach()[:r].contiguous() if (lora_A is not None and r) else None
+    B = lora_B.detach()[:, :r].contiguous() if (lora_B is not None and r) else None
+    b = bias.detach().to(torch.bfloat16).contiguous() if bias is not None else None
+    L = _C.lib()
+    ws_bytes = L.xq_linear_fwd_swiglu_workspace_bytes(M, qw.rows, K, r)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    h = torch.empty(M, I, dtype=torch.bfloat16, device=dev)
+    cw = qw.c()
+    _C.check(L.xq_linear_fwd_swiglu(ctypes.byref(cw), x2.data_ptr(), _ld(x2), M, _C.ptr(A), _C.ptr(B), _lora_dt(A), r if A is not None else 0,
+                                    float(scaling), _C.ptr(b), h.data_ptr(), I, ws.data_ptr(), ws_bytes, _C.stream_ptr(dev)))
+    return h.reshape(*x.shape[:-1], I)
+
+
 def qlora_linear_multi(x: Tensor, jobs) -> list:
     """Forward-only: several QLoRA linears on one input, ``[qlora_linear(x, *job) for job in jobs]`` as one library call
     (xq_linear_fwd_multi): the separate q_proj / k_proj / v_proj or gate_proj / up_proj calls of a model that keeps

@@ -8,6 +8,7 @@ from .linear import (
     NvFP4QLoRALinear,
     QLoRALinear,
     deregister_qlora_weights_from_fsdp,
+    qlora_gate_up_silu,
     qlora_linears_forward,
     qlora_mlp_forward,
 )
@@ -20,6 +21,7 @@ __all__ = [
     "Int4QLoRALinear",
     "NF4QLoRALinear",
     "deregister_qlora_weights_from_fsdp",
+    "qlora_gate_up_silu",
     "qlora_linears_forward",
     "qlora_mlp_forward",
 ]

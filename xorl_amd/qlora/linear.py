@@ -802,6 +802,26 @@ def qlora_mlp_forward(gate_proj: "QLoRALinear", up_proj: "QLoRALinear", down_pro
                      r, s, gate_proj.bias, up_proj.bias, down_proj.bias)
 
 
+def qlora_gate_up_silu(gate_up_proj: "QLoRALinear", x: Tensor) -> Tensor:
+    """`fused_silu_and_mul(gate_up_proj(x))` -- the first half of the reference's Qwen3MLP.forward with its default fused
+    module (models/transformers/qwen3/modeling_qwen3.py:62-70).  Without autograd this is one library call, at decode
+    sizes one kernel launch that writes h directly (xq_linear_fwd_swiglu); otherwise the module call and the SwiGLU
+    kernel.  The same bits either way."""
+    from ..functional import qlora_linear_swiglu, silu_and_mul
+
+    m = gate_up_proj
+    needs_grad = torch.is_grad_enabled() and (x.requires_grad or any(
+        p is not None and p.requires_grad for p in (m.lora_A, m.lora_B, m.bias)))
+    one_call = (isinstance(m, QLoRALinear) and not needs_grad and not torch.compiler.is_compiling() and m.active_r <= MAX_FUSED_RANK
+                and m.out_features % 2 == 0 and not (m.enable_aqn and m.training)
+                and not (_is_dtensor(m.packed_weight_f32.data) or _is_dtensor(m.lora_A))
+                and x.dtype == torch.bfloat16 and x.is_cuda)
+    if not one_call:
+        gate, up = m(x).chunk(2, dim=-1)
+        return silu_and_mul(gate, up)
+    return qlora_linear_swiglu(x, m._forward_quant_weight(), m.lora_A, m.lora_B, m.active_r, m._active_scaling(), m.bias)
+
+
 def qlora_linears_forward(modules, x: Tensor) -> list:
     """`[m(x) for m in modules]` for QLoRA linears that share their input -- the separate q_proj / k_proj / v_proj calls
     of the reference's attention block (models/layers/attention/multi_head_attention.py:93-95) and the gate_proj /
