@@ -172,7 +172,7 @@ static int launch_tile_gemm_t(const xq_weight* w, bool contract_cols, const bf16
                               const int32_t* offsets, const int32_t* tile_offsets, const bf16_t* su, const bf16_t* lora_right,
                               int r_pad, const bf16_t* bias, bf16_t* C, int64_t ldc, hipStream_t stream, const char* who,
                               int force_T, int force_split, float* partial, int64_t partial_bytes,
-                              const TwoBanks* two = nullptr) {
+                              const TwoBanks* two = nullptr, const int32_t* a_rows = nullptr) {
     TileArgs g;
     g.A = A; g.lda = lda; g.C = C; g.ldc = ldc;
     g.packed = (const uint8_t*)w->packed;
@@ -243,7 +243,7 @@ static int launch_tile_gemm_t(const xq_weight* w, bool contract_cols, const bf16
         const int64_t tiles_n = xq_cdiv(g.Nout, T);
         if (fmt_ok && g_tile_policy != 1 && tiles_m * tiles_n < (1ll << 31)) {
             G256Args f;
-            f.A = A; f.lda = lda; f.C = C; f.ldc = ldc;
+            f.A = A; f.lda = lda; f.a_rows = a_rows; f.C = C; f.ldc = ldc;
             f.W = g.packed; f.scales = g.scales; f.global_scale = g.global_scale;
             f.packed_stride = g.packed_stride; f.scale_stride = g.scale_stride;
             f.wrows = g.wrows; f.wcols = g.wcols; f.gshift = gshift; f.scale_dtype = g.scale_dtype;
@@ -285,6 +285,7 @@ static int launch_tile_gemm_t(const xq_weight* w, bool contract_cols, const bf16
             return XQ_OK;
         }
     }
+    XQ_REQUIRE(!a_rows, "%s: internal error: a row map needs the pipelined tile kernel (see tile_gemm_takes_row_map)", who);
     unsigned mt = (unsigned)(xq_cdiv(n_rows, BM) + (offsets ? w->num_experts : 0));
     dim3 grid(mt, (unsigned)xq_cdiv(g.Nout, BN));
     const bool timed = xq_profile_mark_begin(stream, 2.0 * (double)n_rows * g.Nout * ((double)g.Kc + g.r_pad));
@@ -352,9 +353,21 @@ int launch_gate_up_swiglu(const xq_weight* wg, const xq_weight* wu, const bf16_t
 int launch_tile_gemm(const xq_weight* w, bool contract_cols, const bf16_t* A, int64_t lda, int64_t n_rows,
                      const int32_t* offsets, const int32_t* tile_offsets, const bf16_t* su, const bf16_t* lora_right,
                      int r_pad, const bf16_t* bias, bf16_t* C, int64_t ldc, hipStream_t stream, const char* who,
-                     float* partial, int64_t partial_bytes, const TwoBanks* two) {
+                     float* partial, int64_t partial_bytes, const TwoBanks* two, const int32_t* a_rows) {
+    XQ_REQUIRE(!a_rows || offsets, "%s: a row map goes with a grouped launch", who);
     return launch_tile_gemm_t(w, contract_cols, A, lda, n_rows, offsets, tile_offsets, su, lora_right, r_pad, bias, C, ldc,
-                              stream, who, 0, 1, partial, partial_bytes, two);
+                              stream, who, 0, 1, partial, partial_bytes, two, a_rows);
+}
+
+// whether a grouped launch over this bank runs on the pipelined tile kernel, which can read its activation rows through
+// a row map (the conditions of launch_tile_gemm_t)
+bool tile_gemm_takes_row_map(const xq_weight* w) {
+    if (g_tile_policy == 1) return false;
+    if (w->format == XQ_FMT_FP8) return true;
+    int gshift = 0;
+    while ((1 << gshift) < w->group) ++gshift;
+    return (1 << gshift) == w->group && w->group >= 16 && w->layout == XQ_LAYOUT_GKN && w->cols % 16 == 0 && w->rows >= 2 &&
+           xq_aligned(w->scales, 16) && xq_scale_bytes_per_expert(w) % 16 == 0;
 }
 
 static inline int64_t align256(int64_t b) { return (b + 255) & ~(int64_t)255; }

@@ -63,6 +63,8 @@ __device__ __forceinline__ int swz(int r, int c) { return r * 64 + ((c ^ ((r >> 
 struct G256Args {
     const bf16_t* A;
     int64_t lda;
+    const int32_t* a_rows;     // grouped, optional: row i of the problem is row a_rows[i] of A (the routed rows of a compact
+                               // [tokens, K] matrix are read in place instead of from an expert-ordered copy)
     bf16_t* C;
     int64_t ldc;
     const uint8_t* W;          // packed codes (expert 0)
@@ -562,6 +564,9 @@ __global__ void __launch_bounds__(2 * T, 2) gemm_256_kernel(G256Args g) {
             const int u = tv + p * NT;
             int64_t r = t.row0 + (u >> 3);
             r = r < t.row_end ? r : t.row_end - 1;
+            if constexpr (GROUPED) {
+                if (g.a_rows) r = g.a_rows[r];
+            }
             a_src[p] = g.A + r * g.lda + (u & 7) * 8 + kt0 * F8_BK;
         }
 #pragma unroll

@@ -273,8 +273,12 @@ extern "C" int xq_grouped_bwd(const xq_weight* gate, const xq_weight* up, const 
     bf16_t* v_u = fused ? v_gu + rp : v_gu + R * rp;
     const int64_t ld_v = fused ? rp2 : rp;
 
-    // as in the forward: the first pass over the routed gradient rows gathers them from dy and writes g_down
+    // The routed gradient rows are rows of dy, each of them topk times: with 16-byte aligned rows nothing expert-ordered is
+    // written for them -- the passes that read them (s * g . B^T, the dgrad launch, the B gradient) go through the inverse of
+    // scatter_index to dy itself, 1 / topk of the bytes and mostly cache hits.  (A bank that takes the generic tile kernel
+    // still gets its copy, written by the first pass on its way.)
     const bool ride = ld_dy % 8 == 0 && xq_aligned(dy, 16);
+    const bool in_place = ride && tile_gemm_takes_row_map(down);
     if (ride) {
         invert_scatter_kernel<<<dim3((unsigned)xq_cdiv(R, 256)), 256, 0, stream>>>(sidx, R, topk, token_of_row);
         XQ_CHECK_LAUNCH(who);
@@ -284,10 +288,13 @@ extern "C" int xq_grouped_bwd(const xq_weight* gate, const xq_weight* up, const 
 
     // ---- down projection: y = h.W + s*(h.A).B
     if ((rc = launch_small_nt(ride ? (const bf16_t*)dy : g_down, ride ? ld_dy : H, R, H, F_dB, rp, s, v_d, off, toff, E, dBe == 1, stream,
-                              0, nullptr, 0, ride ? token_of_row : nullptr, ride ? g_down : nullptr, H)))        // s * g . B^T
+                              0, nullptr, 0, ride ? token_of_row : nullptr, ride && !in_place ? g_down : nullptr, H)))        // s * g . B^T
         return rc;
-    if ((rc = launch_tile_gemm(down, true, g_down, H, R, off, toff, v_d, Lr_dA, rp, nullptr, dh, I, stream, who, nullptr, 0))) return rc;
-    if ((rc = launch_tn(g_down, H, H, su_d, rp, r, R, true, grads->dB[2], wg, dBe == 1 ? nullptr : off, E, stream, n_valid))) return rc;   // [E|1, r, H]
+    const bf16_t* gd = in_place ? (const bf16_t*)dy : g_down;      // the routed gradient rows: dy through the map, or the copy
+    const int64_t ld_gd = in_place ? ld_dy : H;
+    const int32_t* gd_rows = in_place ? token_of_row : nullptr;
+    if ((rc = launch_tile_gemm(down, true, gd, ld_gd, R, off, toff, v_d, Lr_dA, rp, nullptr, dh, I, stream, who, nullptr, 0, nullptr, gd_rows))) return rc;
+    if ((rc = launch_tn(gd, ld_gd, H, su_d, rp, r, R, true, grads->dB[2], wg, dBe == 1 ? nullptr : off, E, stream, n_valid, 0, gd_rows))) return rc;   // [E|1, r, H]
     if ((rc = launch_tn(h, I, I, v_d, rp, r, R, false, grads->dA[2], wg, dAe == 1 ? nullptr : off, E, stream, n_valid))) return rc;        // [E|1, I, r]
 
     // ---- SwiGLU + routing weight

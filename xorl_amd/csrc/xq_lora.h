@@ -60,7 +60,7 @@ int launch_small_nt(const bf16_t* In, int64_t ld_in, int64_t n_rows, int64_t Kc,
                     int64_t ld_t = 0,       // row pitch of T in elements (0: r_pad), to write a column band of a wider matrix
                     bf16_t* T2 = nullptr, int split = 0,    // result columns from `split` on go to T2 (same pitch): two panels' products from one pass
                     const int32_t* row_map = nullptr,       // grouped: product row i is made from row row_map[i] of In, and the
-                    bf16_t* copy_out = nullptr, int64_t ld_copy = 0);   // gathered rows are also written to copy_out [rows, Kc]
+                    bf16_t* copy_out = nullptr, int64_t ld_copy = 0);   // gathered rows are also written to copy_out [rows, Kc] (if given)
 
 // out[c][j] (or out[j][c] when transpose_out) = sum_m P[m][c] * Q[m][j], fp32.
 //   dense: all rows, split over `splits` row ranges, partials in `partial`
@@ -72,7 +72,8 @@ int launch_tn(const bf16_t* P, int64_t ldp, int64_t width, const bf16_t* Q, int 
               int64_t n_rows, bool transpose_out, float* out, float* partial,
               const int32_t* offsets, int32_t num_experts, hipStream_t stream,
               const int32_t* row_limit = nullptr,    // dense form: contract only rows below *row_limit (device value)
-              int64_t ldq = 0);                      // row pitch of Q in elements (0: r_pad), for a column band of a wider matrix
+              int64_t ldq = 0,                       // row pitch of Q in elements (0: r_pad), for a column band of a wider matrix
+              const int32_t* p_rows = nullptr);      // optional: row m of the contraction is row p_rows[m] of P (Q rows stay in order)
 
 int launch_zero_fill(void* p, int64_t bytes, hipStream_t stream);
 
@@ -94,7 +95,9 @@ int launch_gate_up_swiglu(const xq_weight* wg, const xq_weight* wu, const bf16_t
 int launch_tile_gemm(const xq_weight* w, bool contract_cols, const bf16_t* A, int64_t lda, int64_t n_rows,
                      const int32_t* offsets, const int32_t* tile_offsets, const bf16_t* su, const bf16_t* lora_right,
                      int r_pad, const bf16_t* bias, bf16_t* C, int64_t ldc, hipStream_t stream, const char* who,
-                     float* partial, int64_t partial_bytes, const TwoBanks* two = nullptr);
+                     float* partial, int64_t partial_bytes, const TwoBanks* two = nullptr,
+                     const int32_t* a_rows = nullptr);   // grouped, optional: row i of the problem is row a_rows[i] of A
+bool tile_gemm_takes_row_map(const xq_weight* w);        // ... which only the pipelined tile kernel does
 
 int num_cus();   // compute units of the current device (xq_gemm.hip)
 

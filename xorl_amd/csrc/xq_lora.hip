@@ -274,7 +274,7 @@ __global__ void __launch_bounds__(256) small_nt_kernel(SmallNtArgs g) {
             // (rows and pieces that were clamped onto valid ones are written again with the same bytes)
             int64_t kc = k + cpiece;
             kc = kc < kend ? kc : kend - 8;
-            if (k < kend) {
+            if (g.copy_out && k < kend) {
 #pragma unroll
                 for (int j = 0; j < 8; ++j) *(u32x4*)(g.copy_out + (int64_t)orow[j] * g.ld_copy + kc) = cur[j];
             }
@@ -376,8 +376,8 @@ int launch_small_nt(const bf16_t* In, int64_t ld_in, int64_t n_rows, int64_t Kc,
     XQ_REQUIRE(Kc % 64 == 0, "small_nt: contraction length %lld must be a multiple of 64", (long long)Kc);
     XQ_REQUIRE(ld_in % 8 == 0 && xq_aligned(In, 16) && xq_aligned(F, 16), "small_nt: operands must be 16-byte aligned");
     if (n_rows == 0) return XQ_OK;
-    XQ_REQUIRE(!row_map || (offsets && copy_out && ld_copy % 8 == 0 && ld_copy >= Kc && xq_aligned(copy_out, 16)),
-               "small_nt: gathered rows need the grouped form and a 16-byte aligned copy_out");
+    XQ_REQUIRE(!row_map || (offsets && (!copy_out || (ld_copy % 8 == 0 && ld_copy >= Kc && xq_aligned(copy_out, 16)))),
+               "small_nt: gathered rows need the grouped form, and a copy of them a 16-byte aligned copy_out");
     SmallNtArgs g{In, ld_in, n_rows, Kc, F, shared_f ? 0 : (int64_t)r_pad * Kc, r_pad, scale, T, ld_t, T2, split, offsets,
                   tile_offsets, num_experts, row_map, copy_out, ld_copy};
     int rc;
@@ -408,6 +408,7 @@ struct TnArgs {
     const int32_t* offsets;  // grouped
     const int32_t* row_limit;  // dense, optional (device): only rows below *row_limit are contracted
     int64_t ldq;               // row pitch of Q in elements
+    const int32_t* p_rows;     // optional: row m of the contraction is row p_rows[m] of P
 };
 
 constexpr int TN_PP = 128 + 16;  // Ps pitch (bf16 elements): 288 B rows
@@ -431,13 +432,24 @@ __device__ __forceinline__ void tn_accumulate(const TnArgs& g, int64_t c0, int64
     const int qr = q_thread ? tid / qchunks : 0, qc = q_thread ? (tid % qchunks) * 8 : 0;
     const u32x4 z = {0, 0, 0, 0};
     const int64_t last = m_end - 1;
-    struct Tile { u32x4 p0, p1, q; };
+    struct Tile { u32x4 p0, p1, q; int32_t i0, i1; };
+    // with a row map, the P rows of tile m are named by entries fetched one stage earlier (with the data of tile m - 64):
+    // the data loads then follow their indices without a round trip of their own in the steady state
+    auto fetch_rows = [&](Tile& t, int64_t m) {
+        if (g.p_rows) {
+            const int64_t r0 = m + pr < m_end ? m + pr : last, r1 = m + pr + 16 < m_end ? m + pr + 16 : last;
+            t.i0 = g.p_rows[r0];
+            t.i1 = g.p_rows[r1];
+        }
+    };
     auto fetch = [&](Tile& t, int64_t m) {
-        const int64_t r0 = m + pr < m_end ? m + pr : last, r1 = m + pr + 16 < m_end ? m + pr + 16 : last;
+        int64_t r0 = m + pr < m_end ? m + pr : last, r1 = m + pr + 16 < m_end ? m + pr + 16 : last;
         const int64_t rq = m + qr < m_end ? m + qr : last;
+        if (g.p_rows) { r0 = t.i0; r1 = t.i1; }
         t.p0 = *(const u32x4*)(g.P + r0 * g.ldp + pcol);
         t.p1 = *(const u32x4*)(g.P + r1 * g.ldp + pcol);
         t.q = *(const u32x4*)(g.Q + rq * g.ldq + qc);
+        fetch_rows(t, m + 64);
     };
     auto tile = [&](Tile& t, int64_t m, int buf) {     // multiply tile m out of LDS buffer `buf`, refill t with tile m + 64
         bf16_t* ps = Ps + buf * (32 * TN_PP);
@@ -459,6 +471,8 @@ __device__ __forceinline__ void tn_accumulate(const TnArgs& g, int64_t c0, int64
         }
     };
     Tile ta, tb;
+    fetch_rows(ta, m_begin);
+    fetch_rows(tb, m_begin + 32);
     fetch(ta, m_begin);
     fetch(tb, m_begin + 32);
     for (int64_t m = m_begin; m < m_end; m += 64) {
@@ -609,13 +623,13 @@ int64_t tn_partial_bytes(int64_t n_rows, int64_t width, int r_pad) {
 
 int launch_tn(const bf16_t* P, int64_t ldp, int64_t width, const bf16_t* Q, int r_pad, int r_out, int64_t n_rows,
               bool transpose_out, float* out, float* partial, const int32_t* offsets, int32_t num_experts,
-              hipStream_t stream, const int32_t* row_limit, int64_t ldq) {
+              hipStream_t stream, const int32_t* row_limit, int64_t ldq, const int32_t* p_rows) {
     if (ldq <= 0) ldq = r_pad;
     XQ_REQUIRE(ldq >= r_pad && ldq % 8 == 0, "tn: Q pitch %lld must be a multiple of 8 and at least r_pad", (long long)ldq);
     XQ_REQUIRE(r_pad > 0 && r_pad <= 64 && r_pad % 16 == 0 && r_out <= r_pad, "tn: bad rank (r_pad %d, r_out %d)", r_pad, r_out);
     XQ_REQUIRE(width % 8 == 0 && ldp % 8 == 0 && xq_aligned(P, 16) && xq_aligned(Q, 16), "tn: operands must be 16-byte aligned, width %% 8 == 0");
     if (width == 0 || r_out == 0) return XQ_OK;
-    TnArgs g{P, ldp, width, Q, r_pad, r_out, n_rows, 0, transpose_out ? 1 : 0, out, offsets, offsets ? nullptr : row_limit, ldq};
+    TnArgs g{P, ldp, width, Q, r_pad, r_out, n_rows, 0, transpose_out ? 1 : 0, out, offsets, offsets ? nullptr : row_limit, ldq, p_rows};
     unsigned col_tiles = (unsigned)xq_cdiv(width, 128);
     XQ_REQUIRE(partial != nullptr, "tn: partial workspace is NULL");
     if (offsets) {
