@@ -393,6 +393,11 @@ int xq_grouped_lora_wgrad(const void* P, int64_t ldp, int64_t p_width, const voi
  * rows, r_pad = r rounded up to 16): xs bf16 [R, H] (token rows in expert order), gate_up bf16 [R, 2 I] (the
  * gate projection in columns [0, I), the up projection in [I, 2 I)), h bf16 [R, I], w_row fp32 [R], su_gate / su_up / su_down bf16 [R, r_pad], scatter_index int32 [R], offsets int32
  * [E + 1], tile_offsets int32 [2 (E + 1)], counts int32 [E].  A forward-only caller passes scratch for them.
+ * xs may be NULL where xq_grouped_in_place(gate, up, down) returns 1 (banks that run on the pipelined tile kernel) and
+ * the rows of hidden are 16-byte aligned: the routed rows are rows of hidden, each topk times, so the forward then
+ * writes no expert-ordered copy of them and reads hidden through the routing instead; the backward of such a forward
+ * is given the same hidden states as x_tokens (row stride ld_x_tokens, in elements) -- R * H * 2 bytes less to keep
+ * per layer.  (The backward treats dy the same way whatever xs is.)
  * Factor gradients are fp32, shaped like the factors, overwritten (exact zeros for experts without rows).
  * hidden, out, dy, dx are bf16 [n_tokens, H] with row strides in elements; routing_w [n_tokens, topk] fp32 or
  * bf16, selected int32 [n_tokens, topk]; dx / d_routing may be NULL.  Expert ids outside [0, E) drop their copy.
@@ -420,6 +425,8 @@ typedef struct xq_grouped_saved {
     int32_t* offsets;
     int32_t* tile_offsets;
     int32_t* counts;
+    const void* x_tokens;      /* backward, when xs is NULL: the forward's hidden [n_tokens, H] bf16 */
+    int64_t ld_x_tokens;
 } xq_grouped_saved;
 
 typedef struct xq_grouped_grads {
@@ -429,6 +436,7 @@ typedef struct xq_grouped_grads {
 
 int64_t xq_grouped_workspace_bytes(int64_t n_tokens, int32_t topk, int32_t num_experts, int64_t hidden,
                                    int64_t intermediate, int r, int backward);
+int xq_grouped_in_place(const xq_weight* gate, const xq_weight* up, const xq_weight* down);
 int xq_grouped_fwd(const xq_weight* gate, const xq_weight* up, const xq_weight* down, const xq_grouped_lora* lora,
                    const void* hidden, int64_t ld_hidden, int64_t n_tokens, const void* routing_w, int rw_dtype,
                    const int32_t* selected, int32_t topk, void* out, int64_t ld_out,

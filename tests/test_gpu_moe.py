@@ -680,3 +680,36 @@ def test_grouped_low_rank_entry_points(hip_device):
             close(g[e], ref, 1e-2, rows="none")
     g1 = MF._wgrad(P.to(hip_device), t.to(hip_device), r, None, E, True).cpu()          # one product over all rows, [1, r, width]
     close(g1[0], t[:, :r].double().t() @ P.double(), 1e-2, rows="none")
+
+
+@pytest.mark.parametrize("fmt,hybrid", [("block_fp8", True), ("block_fp8", False), ("nvfp4", True), ("nf4", False)])
+def test_routed_rows_read_in_place_equal_the_copy(hip_device, fmt, hybrid):
+    """Where the banks run on the pipelined tile kernel the forward keeps no expert-ordered copy of the routed rows (and the
+    backward none of the routed gradient rows): the launches read the token matrices through the routing.  Same values in
+    the same order: outputs and every gradient are the bits of the form that writes the copies."""
+    import xorl_amd.moe_functional as MF
+
+    E, T, H, I, r, topk = 12, 1500, 256, 512, 16, 4
+    m, _ = _make_experts(fmt, E, H, I, r, hybrid, seed=31, device=hip_device)
+    rw, sel = _zipf_routing(T, E, topk, seed=3)
+    x = gen((T, H), 1.0, 4, torch.bfloat16).to(hip_device)
+    dy = gen((T, H), 1.0, 5, torch.bfloat16).to(hip_device)
+    res = []
+    try:
+        for in_place in (True, False):
+            MF.READ_ROUTED_ROWS_IN_PLACE = in_place
+            xd = x.clone().requires_grad_(True)
+            rwd = rw.to(hip_device).requires_grad_(True)
+            for p in m.parameters():
+                p.grad = None
+            y = m(xd, rwd, sel.to(hip_device))
+            saved_xs = y.grad_fn.saved_tensors[0] if hasattr(y.grad_fn, "saved_tensors") else None
+            y.backward(dy)
+            grads = [getattr(m, f"{k}_proj_lora_{ab}").grad.clone() for k in ("gate", "up", "down") for ab in "AB"]
+            res.append((y.detach(), xd.grad, rwd.grad, grads, saved_xs))
+    finally:
+        MF.READ_ROUTED_ROWS_IN_PLACE = True
+    (y0, dx0, drw0, g0, xs0), (y1, dx1, drw1, g1, xs1) = res
+    assert torch.equal(y0, y1) and torch.equal(dx0, dx1) and torch.equal(drw0, drw1)
+    for a, b in zip(g0, g1):
+        assert torch.equal(a, b)

@@ -57,7 +57,8 @@ class XqGroupedLora(ctypes.Structure):
 
 class XqGroupedSaved(ctypes.Structure):
     _fields_ = [(n, ctypes.c_void_p) for n in ("xs", "gate_up", "h", "w_row", "su_gate", "su_up", "su_down",
-                                               "scatter_index", "offsets", "tile_offsets", "counts")]
+                                               "scatter_index", "offsets", "tile_offsets", "counts", "x_tokens")] + [
+                                                   ("ld_x_tokens", ctypes.c_int64)]
 
 
 class XqGroupedGrads(ctypes.Structure):
@@ -144,6 +145,7 @@ _SIGNATURES = {
     # P, ldp, p_width, Q, r_pad, r_out, n_rows, offsets, E, transpose_out, out, ws, row_limit, stream
     "xq_grouped_lora_wgrad": (_INT, [_P, _I64, _I64, _P, _INT, _INT, _I64, _P, _I32, _INT, _P, _P, _P, _P]),
     "xq_grouped_workspace_bytes": (_I64, [_I64, _I32, _I32, _I64, _I64, _INT, _INT]),
+    "xq_grouped_in_place": (_INT, [_W, _W, _W]),
     # gate, up, down, lora, hidden, ld_hidden, n_tokens, routing_w, rw_dtype, selected, topk, out, ld_out, saved, ws, ws_bytes, stream
     "xq_grouped_fwd": (_INT, [_W, _W, _W, ctypes.POINTER(XqGroupedLora), _P, _I64, _I64, _P, _INT, _P, _I32, _P, _I64,
                               ctypes.POINTER(XqGroupedSaved), _P, _I64, _P]),

@@ -72,7 +72,7 @@ int check_call(const xq_weight* gate, const xq_weight* up, const xq_weight* down
     d->E = E; d->topk = topk; d->r = lora->r; d->rp = r_pad_of(lora->r);
     d->T = n_tokens; d->R = n_tokens * topk; d->H = H; d->I = I;
     if (d->R > 0)
-        XQ_REQUIRE(saved->xs && saved->gate_up && saved->h && saved->w_row && saved->su_gate && saved->su_up &&
+        XQ_REQUIRE(saved->gate_up && saved->h && saved->w_row && saved->su_gate && saved->su_up &&
                        saved->su_down && saved->scatter_index,
                    "%s: a buffer of xq_grouped_saved is NULL", who);
     XQ_REQUIRE(saved->offsets && saved->tile_offsets && saved->counts, "%s: a routing buffer of xq_grouped_saved is NULL", who);
@@ -102,6 +102,11 @@ bool fuse_gate_up(const xq_weight* gate, const xq_weight* up) { return two_banks
 }  // namespace xq
 
 using namespace xq;
+
+extern "C" int xq_grouped_in_place(const xq_weight* gate, const xq_weight* up, const xq_weight* down) {
+    (void)down;
+    return gate && up && tile_gemm_takes_row_map(gate) && tile_gemm_takes_row_map(up) ? 1 : 0;
+}
 
 extern "C" int64_t xq_grouped_workspace_bytes(int64_t n_tokens, int32_t topk, int32_t num_experts, int64_t hidden,
                                               int64_t intermediate, int r, int backward) {
@@ -137,8 +142,13 @@ extern "C" int xq_grouped_fwd(const xq_weight* gate, const xq_weight* up, const 
     bf16_t* xs = (bf16_t*)saved->xs;
     // The pass that first reads the routed rows -- x . A^T of gate (and up) -- takes them from the token matrix through
     // the inverse of scatter_index and writes the expert-ordered copy xs on its way: no scatter pass of its own.
+    // With saved->xs == NULL no copy is written at all: the projection launches read the token matrix through the same
+    // map (the routed rows are rows of it, each topk times), and so does the backward (saved->x_tokens).
     int32_t* token_of_row = cv.take<int32_t>(R * 4);
     const bool ride = ld_hidden % 8 == 0 && xq_aligned(hidden, 16) && xq_aligned(xs, 16);
+    const bool in_place = xs == nullptr;
+    XQ_REQUIRE(!in_place || (ride && tile_gemm_takes_row_map(gate) && tile_gemm_takes_row_map(up)),
+               "%s: saved->xs may be NULL only where xq_grouped_in_place() says so, with 16-byte aligned rows of hidden", who);
     if (ride) {
         invert_scatter_kernel<<<dim3((unsigned)xq_cdiv(R, 256)), 256, 0, stream>>>(saved->scatter_index, R, topk, token_of_row);
         XQ_CHECK_LAUNCH(who);
@@ -149,6 +159,9 @@ extern "C" int xq_grouped_fwd(const xq_weight* gate, const xq_weight* up, const 
     const int64_t first_ld = ride ? ld_hidden : H;
     const int32_t* first_map = ride ? token_of_row : nullptr;
     bf16_t* first_copy = ride ? xs : nullptr;
+    const bf16_t* xr = in_place ? (const bf16_t*)hidden : xs;         // the routed rows for the passes after the first
+    const int64_t ld_xr = in_place ? ld_hidden : H;
+    const int32_t* xr_rows = in_place ? token_of_row : nullptr;
 
     // bf16 operand layouts of the six factors, one launch.  A factors [E|1, in, r] become the "down" panels
     // [E|1, rp, in] of x . A; B factors [E|1, r, out] become the per-expert right-hand panels [E, out, rp].
@@ -186,14 +199,14 @@ extern "C" int xq_grouped_fwd(const xq_weight* gate, const xq_weight* up, const 
         if ((rc = launch_small_nt(first_in, first_ld, R, H, F_gA, rp, s, su_g, off, toff, E, gAe == 1, stream, 0, nullptr, 0,
                                   first_map, first_copy, H)))
             return rc;
-        if ((rc = launch_small_nt(xs, H, R, H, F_uA, rp, s, su_u, off, toff, E, uAe == 1, stream))) return rc;
+        if ((rc = launch_small_nt(xr, ld_xr, R, H, F_uA, rp, s, su_u, off, toff, E, uAe == 1, stream, 0, nullptr, 0, xr_rows, nullptr, 0))) return rc;
     }
     if (fuse_gate_up(gate, up)) {       // both projections in one launch: column tiles past I take the up bank
         const TwoBanks two{up, su_u, Lr_uB};
-        if ((rc = launch_tile_gemm(gate, false, xs, H, R, off, toff, su_g, Lr_gB, rp, nullptr, gu, 2 * I, stream, who, nullptr, 0, &two))) return rc;
+        if ((rc = launch_tile_gemm(gate, false, xr, ld_xr, R, off, toff, su_g, Lr_gB, rp, nullptr, gu, 2 * I, stream, who, nullptr, 0, &two, xr_rows))) return rc;
     } else {
-        if ((rc = launch_tile_gemm(gate, false, xs, H, R, off, toff, su_g, Lr_gB, rp, nullptr, gu, 2 * I, stream, who, nullptr, 0))) return rc;
-        if ((rc = launch_tile_gemm(up, false, xs, H, R, off, toff, su_u, Lr_uB, rp, nullptr, gu + I, 2 * I, stream, who, nullptr, 0))) return rc;
+        if ((rc = launch_tile_gemm(gate, false, xr, ld_xr, R, off, toff, su_g, Lr_gB, rp, nullptr, gu, 2 * I, stream, who, nullptr, 0, nullptr, xr_rows))) return rc;
+        if ((rc = launch_tile_gemm(up, false, xr, ld_xr, R, off, toff, su_u, Lr_uB, rp, nullptr, gu + I, 2 * I, stream, who, nullptr, 0, nullptr, xr_rows))) return rc;
     }
     if ((rc = xq_moe_scatter_scalar(routing_w, rw_dtype, saved->scatter_index, R, saved->w_row, stream))) return rc;
     if ((rc = xq_silu_mul_fwd(gu, gu + I, 2 * I, saved->w_row, h, I, R, I, stream))) return rc;
@@ -232,6 +245,10 @@ extern "C" int xq_grouped_bwd(const xq_weight* gate, const xq_weight* up, const 
     const int32_t *off = saved->offsets, *toff = saved->tile_offsets, *sidx = saved->scatter_index;
     const int32_t* n_valid = off + E;     // rows that belong to an expert (all of them unless an id was out of range)
     const bf16_t *xs = (const bf16_t*)saved->xs, *gu = (const bf16_t*)saved->gate_up;
+    // the forward kept no expert-ordered copy of the routed rows: they are read from the token matrix through the map
+    const bool x_in_place = xs == nullptr;
+    XQ_REQUIRE(!x_in_place || (saved->x_tokens && saved->ld_x_tokens % 8 == 0 && xq_aligned(saved->x_tokens, 16)),
+               "%s: saved->xs is NULL and saved->x_tokens does not name the forward's hidden states (16-byte aligned rows)", who);
     const bf16_t *h = (const bf16_t*)saved->h, *su_g = (const bf16_t*)saved->su_gate, *su_u = (const bf16_t*)saved->su_up;
     const bf16_t* su_d = (const bf16_t*)saved->su_down;
     const int gBe = lora->B_experts[0], uBe = lora->B_experts[1], dBe = lora->B_experts[2];
@@ -279,6 +296,13 @@ extern "C" int xq_grouped_bwd(const xq_weight* gate, const xq_weight* up, const 
     // still gets its copy, written by the first pass on its way.)
     const bool ride = ld_dy % 8 == 0 && xq_aligned(dy, 16);
     const bool in_place = ride && tile_gemm_takes_row_map(down);
+    if (x_in_place && !ride) {
+        invert_scatter_kernel<<<dim3((unsigned)xq_cdiv(R, 256)), 256, 0, stream>>>(sidx, R, topk, token_of_row);
+        XQ_CHECK_LAUNCH(who);
+    }
+    const bf16_t* xr = x_in_place ? (const bf16_t*)saved->x_tokens : xs;
+    const int64_t ld_xr = x_in_place ? saved->ld_x_tokens : H;
+    const int32_t* xr_rows = x_in_place ? token_of_row : nullptr;
     if (ride) {
         invert_scatter_kernel<<<dim3((unsigned)xq_cdiv(R, 256)), 256, 0, stream>>>(sidx, R, topk, token_of_row);
         XQ_CHECK_LAUNCH(who);
@@ -316,13 +340,13 @@ extern "C" int xq_grouped_bwd(const xq_weight* gate, const xq_weight* up, const 
     // gradients of the two A factors, [E|1, H, r] = x^T . v: both contract the same rows of x, so with v_g | v_u side
     // by side they share one pass over them
     if (fused) {
-        if ((rc = launch_tn(xs, H, H, v_gu, rp2, rp2, R, false, pair, wg, gAe == 1 ? nullptr : off, E, stream, n_valid))) return rc;
+        if ((rc = launch_tn(xr, ld_xr, H, v_gu, rp2, rp2, R, false, pair, wg, gAe == 1 ? nullptr : off, E, stream, n_valid, 0, xr_rows))) return rc;
         const int64_t rows = (int64_t)gAe * H;
         split_pair_kernel<<<dim3((unsigned)xq_cdiv(rows * r, 256)), 256, 0, stream>>>(pair, rows, rp, r, grads->dA[0], grads->dA[1]);
         XQ_CHECK_LAUNCH(who);
     } else {
-        if ((rc = launch_tn(xs, H, H, v_g, rp, r, R, false, grads->dA[0], wg, gAe == 1 ? nullptr : off, E, stream, n_valid))) return rc;
-        if ((rc = launch_tn(xs, H, H, v_u, rp, r, R, false, grads->dA[1], wg, uAe == 1 ? nullptr : off, E, stream, n_valid))) return rc;
+        if ((rc = launch_tn(xr, ld_xr, H, v_g, rp, r, R, false, grads->dA[0], wg, gAe == 1 ? nullptr : off, E, stream, n_valid, 0, xr_rows))) return rc;
+        if ((rc = launch_tn(xr, ld_xr, H, v_u, rp, r, R, false, grads->dA[1], wg, uAe == 1 ? nullptr : off, E, stream, n_valid, 0, xr_rows))) return rc;
     }
     if (!dx) return XQ_OK;
     return xq_moe_gather(dx_g, fused ? nullptr : dx_u, H, sidx, d.T, topk, H, dx, ld_dx, stream);

@@ -152,11 +152,19 @@ def _lora_struct(factors, r: int, scaling: float) -> _C.XqGroupedLora:
     return L
 
 
-def _saved_struct(saved) -> _C.XqGroupedSaved:
+# Test switch: False keeps the expert-ordered copy of the routed rows (saved xs [R, H]) even where the banks can read the
+# token matrix in place.
+READ_ROUTED_ROWS_IN_PLACE = True
+
+
+def _saved_struct(saved, x_tokens: Optional[Tensor] = None) -> _C.XqGroupedSaved:
+    """saved[0] (xs) with no elements: the routed rows are read in place from the token matrix (`x_tokens` in the backward)."""
     S = _C.XqGroupedSaved()
     for name, t in zip(("xs", "gate_up", "h", "w_row", "su_gate", "su_up", "su_down", "scatter_index", "offsets",
                         "tile_offsets", "counts"), saved):
-        setattr(S, name, t.data_ptr())
+        setattr(S, name, t.data_ptr() if t.numel() else None)
+    if x_tokens is not None and x_tokens.numel():
+        S.x_tokens, S.ld_x_tokens = x_tokens.data_ptr(), (x_tokens.stride(0) if x_tokens.shape[0] > 1 else x_tokens.shape[1])
     return S
 
 
@@ -168,7 +176,7 @@ def _workspace(dev, T: int, topk: int, E: int, H: int, I: int, r: int, backward:
     return torch.empty(n, dtype=torch.uint8, device=dev)
 
 
-def _moe_fwd_impl(hidden2: Tensor, rw: Tensor, sel: Tensor, factors, banks, r: int, scaling: float):
+def _moe_fwd_impl(hidden2: Tensor, rw: Tensor, sel: Tensor, factors, banks, r: int, scaling: float, allow_in_place: bool = True):
     """xq_grouped_fwd.  hidden2 bf16 [T, H]; rw [T, topk] fp32 / bf16; sel int32 [T, topk]; factors the six active
     LoRA views, contiguous; banks three QuantWeight.  -> (out [T, H], the eleven tensors the backward reads)."""
     qg, qu, qd = banks
@@ -177,12 +185,16 @@ def _moe_fwd_impl(hidden2: Tensor, rw: Tensor, sel: Tensor, factors, banks, r: i
     R, rp, dev = T * topk, _r_pad(r), hidden2.device
     bf = lambda *shape: torch.empty(*shape, dtype=torch.bfloat16, device=dev)
     i32 = lambda n: torch.empty(n, dtype=torch.int32, device=dev)
-    saved = (bf(R, H), bf(R, 2 * I), bf(R, I), torch.empty(R, dtype=torch.float32, device=dev), bf(R, rp), bf(R, rp),
-             bf(R, rp), i32(R), i32(E + 1), i32(2 * (E + 1)), i32(E))
+    wg, wu, wd = qg.c(), qu.c(), qd.c()
+    # where the banks allow it the routed rows are read in place from hidden2 (no [R, H] copy kept for the backward)
+    # (not under torch.compile: the traced op has one output signature, with the copy)
+    in_place = (allow_in_place and READ_ROUTED_ROWS_IN_PLACE and R > 0 and hidden2.data_ptr() % 16 == 0 and (T == 1 or hidden2.stride(0) % 8 == 0)
+                and bool(_C.lib().xq_grouped_in_place(ctypes.byref(wg), ctypes.byref(wu), ctypes.byref(wd))))
+    saved = (bf(0, H) if in_place else bf(R, H), bf(R, 2 * I), bf(R, I), torch.empty(R, dtype=torch.float32, device=dev), bf(R, rp),
+             bf(R, rp), bf(R, rp), i32(R), i32(E + 1), i32(2 * (E + 1)), i32(E))
     out = bf(T, H)
     ws = _workspace(dev, T, topk, E, H, I, r, False)
     lora, S = _lora_struct(factors, r, scaling), _saved_struct(saved)
-    wg, wu, wd = qg.c(), qu.c(), qd.c()
     _C.check(_C.lib().xq_grouped_fwd(ctypes.byref(wg), ctypes.byref(wu), ctypes.byref(wd), ctypes.byref(lora),
                                      hidden2.data_ptr(), hidden2.stride(0) if T > 1 else H, T, rw.data_ptr(),
                                      _C.XQ_DT_F32 if rw.dtype == torch.float32 else _C.XQ_DT_BF16, sel.data_ptr(), topk,
@@ -191,7 +203,7 @@ def _moe_fwd_impl(hidden2: Tensor, rw: Tensor, sel: Tensor, factors, banks, r: i
 
 
 def _moe_bwd_impl(dy2: Tensor, saved, factors, banks, r: int, scaling: float, T: int, topk: int, rw_dtype: torch.dtype,
-                  need_dx: bool, need_drw: bool):
+                  need_dx: bool, need_drw: bool, hidden2: Optional[Tensor] = None):
     """xq_grouped_bwd -> (dx [T, H] or empty, d_routing [T, topk] or empty, six fp32 factor gradients)."""
     qg, qu, qd = banks
     E, H, I = qg.num_experts, qg.rows, qg.cols
@@ -204,7 +216,7 @@ def _moe_bwd_impl(dy2: Tensor, saved, factors, banks, r: int, scaling: float, T:
     for p in range(3):
         G.dA[p], G.dB[p] = grads[2 * p].data_ptr(), grads[2 * p + 1].data_ptr()
     ws = _workspace(dev, T, topk, E, H, I, r, True)
-    lora, S = _lora_struct(factors, r, scaling), _saved_struct(saved)
+    lora, S = _lora_struct(factors, r, scaling), _saved_struct(saved, hidden2)
     wg, wu, wd = qg.c(), qu.c(), qd.c()
     _C.check(_C.lib().xq_grouped_bwd(ctypes.byref(wg), ctypes.byref(wu), ctypes.byref(wd), ctypes.byref(lora),
                                      dy2.data_ptr(), dy2.stride(0) if T > 1 else H, T, topk, ctypes.byref(S),
@@ -224,7 +236,7 @@ def _moe_fwd_op(hidden: Tensor, rw: Tensor, sel: Tensor, gA: Tensor, gB: Tensor,
     banks = (_rebuild_bank(g_packed, g_scales, g_gs, fmt, layout, sd, H, I, group, E),
              _rebuild_bank(u_packed, u_scales, u_gs, fmt, layout, sd, H, I, group, E),
              _rebuild_bank(d_packed, d_scales, d_gs, fmt, layout, sd, I, H, group, E))
-    out, saved = _moe_fwd_impl(hidden, rw, sel, (gA, gB, uA, uB, dA, dB), banks, r, scaling)
+    out, saved = _moe_fwd_impl(hidden, rw, sel, (gA, gB, uA, uB, dA, dB), banks, r, scaling, allow_in_place=False)
     return [out, *saved]
 
 
@@ -240,7 +252,7 @@ def _(hidden, rw, sel, gA, gB, uA, uB, dA, dB, g_packed, g_scales, g_gs, u_packe
 
 
 @torch.library.custom_op("xq::moe_bwd", mutates_args=(), device_types="cuda")
-def _moe_bwd_op(dy: Tensor, saved: List[Tensor], gA: Tensor, gB: Tensor, uA: Tensor, uB: Tensor, dA: Tensor, dB: Tensor,
+def _moe_bwd_op(dy: Tensor, hidden: Tensor, saved: List[Tensor], gA: Tensor, gB: Tensor, uA: Tensor, uB: Tensor, dA: Tensor, dB: Tensor,
                 g_packed: Tensor, g_scales: Tensor, g_gs: Optional[Tensor], u_packed: Tensor, u_scales: Tensor,
                 u_gs: Optional[Tensor], d_packed: Tensor, d_scales: Tensor, d_gs: Optional[Tensor], fmt: str,
                 layout: int, scale_code: int, group: int, E: int, H: int, I: int, r: int, scaling: float, T: int,
@@ -250,12 +262,12 @@ def _moe_bwd_op(dy: Tensor, saved: List[Tensor], gA: Tensor, gB: Tensor, uA: Ten
              _rebuild_bank(u_packed, u_scales, u_gs, fmt, layout, sd, H, I, group, E),
              _rebuild_bank(d_packed, d_scales, d_gs, fmt, layout, sd, I, H, group, E))
     dx, drw, grads = _moe_bwd_impl(dy, tuple(saved), (gA, gB, uA, uB, dA, dB), banks, r, scaling, T, topk,
-                                   _CODE_TO_DT[rw_code], need_dx, need_drw)
+                                   _CODE_TO_DT[rw_code], need_dx, need_drw, hidden)
     return [dx, drw, *grads]
 
 
 @_moe_bwd_op.register_fake
-def _(dy, saved, gA, gB, uA, uB, dA, dB, g_packed, g_scales, g_gs, u_packed, u_scales, u_gs, d_packed, d_scales, d_gs,
+def _(dy, hidden, saved, gA, gB, uA, uB, dA, dB, g_packed, g_scales, g_gs, u_packed, u_scales, u_gs, d_packed, d_scales, d_gs,
       fmt, layout, scale_code, group, E, H, I, r, scaling, T, topk, rw_code, need_dx, need_drw):
     rw_dt = _CODE_TO_DT[rw_code]
     return [dy.new_empty((T, H) if need_dx else (0,), dtype=torch.bfloat16),
@@ -306,12 +318,12 @@ class MoeExpertsQLoRAFunction(torch.autograd.Function):
             out, saved = _moe_fwd_impl(hidden2, rw, sel, factors, banks, r, s)
         ctx.qw = banks
         ctx.meta = (E, T, topk, H, I, r, s, shape, routing_weights.dtype, routing_weights.shape)
-        ctx.save_for_backward(*saved, *factors)
+        ctx.save_for_backward(*saved, *factors, hidden2)
         return out.reshape(shape)
 
     @staticmethod
     def backward(ctx, dy):
-        saved, factors = ctx.saved_tensors[:11], ctx.saved_tensors[11:]
+        saved, factors, hidden2 = ctx.saved_tensors[:11], ctx.saved_tensors[11:17], ctx.saved_tensors[17]
         qw_gate, qw_up, qw_down = ctx.qw
         E, T, topk, H, I, r, s, shape, rw_dtype, rw_shape = ctx.meta
         dy2 = dy.reshape(-1, H).to(torch.bfloat16)
@@ -319,12 +331,12 @@ class MoeExpertsQLoRAFunction(torch.autograd.Function):
         need_dx, need_drw = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         kernel_rw_dt = rw_dtype if rw_dtype in (torch.float32, torch.bfloat16) else torch.float32
         if torch.compiler.is_compiling():
-            res = _moe_bwd_op(dy2, list(saved), *factors, *_bank_args(qw_gate), *_bank_args(qw_up), *_bank_args(qw_down),
+            res = _moe_bwd_op(dy2, hidden2, list(saved), *factors, *_bank_args(qw_gate), *_bank_args(qw_up), *_bank_args(qw_down),
                               qw_gate.fmt, qw_gate.layout, _DT_TO_CODE[qw_gate.scale_dtype], qw_gate.group, E, H, I, r, s,
                               T, topk, _DT_TO_CODE[kernel_rw_dt], need_dx, need_drw)
             dx, drw, grads = res[0], res[1], res[2:]
         else:
-            dx, drw, grads = _moe_bwd_impl(dy2, saved, factors, ctx.qw, r, s, T, topk, kernel_rw_dt, need_dx, need_drw)
+            dx, drw, grads = _moe_bwd_impl(dy2, saved, factors, ctx.qw, r, s, T, topk, kernel_rw_dt, need_dx, need_drw, hidden2)
         dx = dx.reshape(shape) if need_dx else None
         drw = drw.reshape(rw_shape).to(rw_dtype) if need_drw else None
         gs = [g.to(f.dtype) for g, f in zip(grads, factors)]
