@@ -216,13 +216,16 @@ template <int FMT>
 __device__ __forceinline__ void decode8_4bit(uint32_t w, float s, uint32_t* out4, const float* nf4_lds) {
     float v[8];
     if (FMT == XQ_FMT_INT4) {
-        const float m8s = -8.0f * s;
+        // the nibbles become floats two at a time through the fp8 converter: a byte 0x0n read as e4m3 is n * 2^-9 for
+        // every n in 0..15, and (n * 2^-9) * (512 s) is n * s exactly
+        const float m8s = -8.0f * s, s512 = s * 512.0f;
         const uint32_t even = w & 0x0f0f0f0fu, odd = (w >> 4) & 0x0f0f0f0fu;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            v[2 * i] = __builtin_fmaf((float)((even >> (8 * i)) & 0xffu), s, m8s);
-            v[2 * i + 1] = __builtin_fmaf((float)((odd >> (8 * i)) & 0xffu), s, m8s);
-        }
+        const f32x2 e01 = e4m3x2_to_f32(even, false), e23 = e4m3x2_to_f32(even, true);
+        const f32x2 o01 = e4m3x2_to_f32(odd, false), o23 = e4m3x2_to_f32(odd, true);
+        v[0] = __builtin_fmaf(e01[0], s512, m8s); v[1] = __builtin_fmaf(o01[0], s512, m8s);
+        v[2] = __builtin_fmaf(e01[1], s512, m8s); v[3] = __builtin_fmaf(o01[1], s512, m8s);
+        v[4] = __builtin_fmaf(e23[0], s512, m8s); v[5] = __builtin_fmaf(o23[0], s512, m8s);
+        v[6] = __builtin_fmaf(e23[1], s512, m8s); v[7] = __builtin_fmaf(o23[1], s512, m8s);
     } else if (FMT == XQ_FMT_NF4) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) v[i] = nf4_lds[(w >> (4 * i)) & 0xfu] * s;

@@ -17,13 +17,17 @@ __device__ __forceinline__ bf16x8 decode8(uint32_t w0, uint32_t w1, float s0, fl
         o[2] = pack_bf16x2(c[0] * s0, c[1] * s0);
         o[3] = pack_bf16x2(d[0] * s0, d[1] * s0);
     } else if (FMT == XQ_FMT_INT4) {
-        // w0 holds 8 nibbles; fma(nib, s, -8s) == fl((nib-8)*s) up to the sign of zero
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            float lo = __builtin_fmaf((float)((w0 >> (8 * i)) & 0xfu), s0, s1);
-            float hi = __builtin_fmaf((float)((w0 >> (8 * i + 4)) & 0xfu), s0, s1);
-            o[i] = pack_bf16x2(lo, hi);
-        }
+        // w0 holds 8 nibbles; fma(nib, s, -8s) == fl((nib-8)*s) up to the sign of zero.  The nibbles become floats two
+        // at a time through the fp8 converter: a byte 0x0n read as e4m3 is n * 2^-9 for every n in 0..15 (the subnormals
+        // run without a gap into the first binade), and (n * 2^-9) * (512 s) is n * s exactly.
+        const uint32_t ev = w0 & 0x0f0f0f0fu, od = (w0 >> 4) & 0x0f0f0f0fu;     // nibbles 0 2 4 6 / 1 3 5 7, one per byte
+        const float s512 = s0 * 512.0f;
+        const f32x2 e01 = e4m3x2_to_f32(ev, false), e23 = e4m3x2_to_f32(ev, true);
+        const f32x2 o01 = e4m3x2_to_f32(od, false), o23 = e4m3x2_to_f32(od, true);
+        o[0] = pack_bf16x2(__builtin_fmaf(e01[0], s512, s1), __builtin_fmaf(o01[0], s512, s1));
+        o[1] = pack_bf16x2(__builtin_fmaf(e01[1], s512, s1), __builtin_fmaf(o01[1], s512, s1));
+        o[2] = pack_bf16x2(__builtin_fmaf(e23[0], s512, s1), __builtin_fmaf(o23[0], s512, s1));
+        o[3] = pack_bf16x2(__builtin_fmaf(e23[1], s512, s1), __builtin_fmaf(o23[1], s512, s1));
     } else if (FMT == XQ_FMT_NF4) {
         // level[nib] * scale, the levels read from a 64-byte copy of the table in LDS (conflict free for any mix of codes)
 #pragma unroll

@@ -242,6 +242,14 @@ __device__ __forceinline__ void skinny_rows_body(const SkinnyRowsArgs& g, const 
     constexpr int DJ = T < (kRowsLoadsInFlight + G - 1) / G ? T : (kRowsLoadsInFlight + G - 1) / G;
     u32x4 w[DJ][G];
     uint32_t sc[DJ][G][NSC];
+    // int4 with one bf16 scale per 128 elements (a step): a lane's scales of four consecutive steps are 8 contiguous bytes,
+    // and one load per four steps fetches them.  A 2-byte load per step and row group is a vector memory instruction that
+    // touches 16 cache lines like the step's weight load itself -- as many instructions again as the weights take, and
+    // the kernel runs at the pace of its memory instructions.  (Needs whole groups of four steps per wave, all in use.)
+    constexpr bool I4 = FMT == XQ_FMT_INT4;
+    const bool vs = I4 && g.gshift == 7 && g.scale_dtype == XQ_SCALE_BF16 && nj == NJ && (NJ & 3) == 0 && (g.K & 511) == 0 &&
+                    (ks & 511) == 0 && ((uintptr_t)g.scales & 7) == 0;
+    u32x2 scv[I4 ? R : 1][I4 ? G : 1][I4 ? (NJ + 3) / 4 : 1];
     const uint8_t* wp[G];
     int64_t erow[G];                            // element index of (row, k0 + (EPS / 4) kq), for the per-row scales
 #pragma unroll
@@ -265,8 +273,14 @@ __device__ __forceinline__ void skinny_rows_body(const SkinnyRowsArgs& g, const 
                     const int nb = n0 + rr * rstride + gi * 16 < g.N ? n0 + rr * rstride + gi * 16 : g.N - 16;
                     sc[j][gi][0] = ((const __attribute__((address_space(4))) uint32_t*)g.scales)[(nb >> 7) * scols + ((k0 + jc * 64) >> 7)];
                 } else if (FMT == XQ_FMT_INT4) {
-                    const int64_t si = (erow[gi] + rr * round_bytes * EB + jc * EPS) >> g.gshift;      // group % 32 == 0: one scale per load
-                    sc[j][gi][0] = g.scale_dtype == XQ_SCALE_F32 ? ((const uint32_t*)g.scales)[si] : (uint32_t)((const uint16_t*)g.scales)[si] << 16;
+                    if (vs) {
+                        if (jj % 4 == 0)
+                            scv[I4 ? rr : 0][I4 ? gi : 0][I4 ? jj / 4 : 0] =
+                                *(const u32x2*)((const uint16_t*)g.scales + ((erow[gi] + rr * round_bytes * EB) >> 7) + jj);
+                    } else {
+                        const int64_t si = (erow[gi] + rr * round_bytes * EB + jc * EPS) >> g.gshift;      // group % 32 == 0: one scale per load
+                        sc[j][gi][0] = g.scale_dtype == XQ_SCALE_F32 ? ((const uint32_t*)g.scales)[si] : (uint32_t)((const uint16_t*)g.scales)[si] << 16;
+                    }
                 } else if (FMT == XQ_FMT_NF4) {
                     sc[j][gi][0] = ((const uint32_t*)g.scales)[(erow[gi] + rr * round_bytes * EB + jc * EPS) >> 6];       // fp32, group 64
                 } else {
@@ -345,7 +359,13 @@ __device__ __forceinline__ void skinny_rows_body(const SkinnyRowsArgs& g, const 
                     if (FMT == XQ_FMT_FP8) {
                         wf = decode8<FMT>(w[sl][gi][2 * c], w[sl][gi][2 * c + 1], __uint_as_float(sc[sl][gi][0]), 0.0f);
                     } else if (FMT == XQ_FMT_INT4) {
-                        const float sv = __uint_as_float(sc[sl][gi][0]);
+                        float sv;
+                        if (vs) {
+                            const uint32_t v = scv[I4 ? rr : 0][I4 ? gi : 0][I4 ? j / 4 : 0][(j >> 1) & 1];
+                            sv = __uint_as_float((j & 1) ? (v & 0xffff0000u) : (v << 16));
+                        } else {
+                            sv = __uint_as_float(sc[sl][gi][0]);
+                        }
                         wf = decode8<FMT>(w[sl][gi][c], 0u, sv, -8.0f * sv);
                     } else if (FMT == XQ_FMT_NF4) {
                         wf = decode8<FMT>(w[sl][gi][c], 0u, __uint_as_float(sc[sl][gi][0]), 0.0f, nf4_lds);
