@@ -43,7 +43,7 @@ BF16_MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense bf16, published
 MEASURED_TRAFFIC = {
     # gemm_256_kernel<int4, T=128> in 4 K splits + splitk_reduce_kernel: mean of the forward and dgrad launches
     # (64 MiB of it are the fp32 partial sums written and read back)
-    0: (109.6 * 2 ** 20, "profiles/gemm_128_int4_linear_m512.txt", 0.04486),
+    0: (109.6 * 2 ** 20, "profiles/gemm_128_int4_linear_m512.txt", 0.04315),
     # gemm_256_kernel<fp8>: mean over the 4 launches of a step (gate|up forward with the SwiGLU epilogue, down
     # forward, d_h, dx as one sum over the gate and up weights)
     1: (1408.3 * 2 ** 20, "profiles/gemm_256_fp8_mlp_m8192.txt", 1.12517),
@@ -56,7 +56,7 @@ MEASURED_TRAFFIC = {
     # skinny_rows_kernel (M <= 16) and skinny_split_kernel + skinny_epilogue_kernel (M = 32, 64): mean per forward
     # over the 32 cases (includes the fp32 partial tiles of the two-launch cases written and read back: 23.3 MiB of
     # it are algorithmic)
-    4: (39.7 * 2 ** 20, "profiles/skinny_kernels_decode_shapes.txt", 0.01767),
+    4: (39.7 * 2 ** 20, "profiles/skinny_kernels_decode_shapes.txt", 0.01688),
     # merge_prep_kernel + merge_kernel<fp8>: mean per call (re-quantise 96 MiB, publish 144 MiB algorithmic)
     5: (134.4 * 2 ** 20, "profiles/merge_kernel_fp8_mlp_weights.txt", 0.04168),
     # gemm_256_kernel<nf4>: mean of the forward and dgrad launches
