@@ -250,6 +250,14 @@ __device__ __forceinline__ void skinny_rows_body(const SkinnyRowsArgs& g, const 
     const bool vs = I4 && g.gshift == 7 && g.scale_dtype == XQ_SCALE_BF16 && nj == NJ && (NJ & 3) == 0 && (g.K & 511) == 0 &&
                     (ks & 511) == 0 && ((uintptr_t)g.scales & 7) == 0;
     u32x2 scv[I4 ? R : 1][I4 ? G : 1][I4 ? (NJ + 3) / 4 : 1];
+    // nvfp4 with e4m3 block scales and nf4 (fp32, group 64) hold 8 scale bytes per row and step, two of them (nf4: one fp32)
+    // for each of the row's four lanes.  Lane kq fetches the 8 bytes of step 4 q + kq -- one load per four steps -- and the four
+    // lanes of a row then exchange: a 4 x 4 transpose over the wave's four 16-lane rows leaves each lane with its own piece
+    // of each of the four steps.
+    constexpr bool P8 = FMT == XQ_FMT_NVFP4 || FMT == XQ_FMT_NF4;
+    const bool vs4 = P8 && (FMT == XQ_FMT_NF4 || g.scale_dtype == XQ_SCALE_E4M3) && ((uintptr_t)g.scales & 7) == 0;
+    u32x2 scx[P8 ? R : 1][P8 ? G : 1][P8 ? (NJ + 3) / 4 : 1];
+    uint32_t sx[P8 ? G : 1][4];        // this lane's scale piece for each step of the current group of four
     const uint8_t* wp[G];
     int64_t erow[G];                            // element index of (row, k0 + (EPS / 4) kq), for the per-row scales
 #pragma unroll
@@ -280,6 +288,13 @@ __device__ __forceinline__ void skinny_rows_body(const SkinnyRowsArgs& g, const 
                     } else {
                         const int64_t si = (erow[gi] + rr * round_bytes * EB + jc * EPS) >> g.gshift;      // group % 32 == 0: one scale per load
                         sc[j][gi][0] = g.scale_dtype == XQ_SCALE_F32 ? ((const uint32_t*)g.scales)[si] : (uint32_t)((const uint16_t*)g.scales)[si] << 16;
+                    }
+                } else if (vs4) {
+                    // (byte offset of a row's scales = element index / 16 in both formats; steps past the last are clamped onto it)
+                    if (jj % 4 == 0) {
+                        const int js = jj + kq < nj ? jj + kq : nj - 1;
+                        scx[P8 ? rr : 0][P8 ? gi : 0][P8 ? jj / 4 : 0] =
+                            *(const u32x2*)(g.scales + (((erow[gi] & ~(int64_t)127) + rr * round_bytes * EB + (int64_t)js * EPS) >> 4));
                     }
                 } else if (FMT == XQ_FMT_NF4) {
                     sc[j][gi][0] = ((const uint32_t*)g.scales)[(erow[gi] + rr * round_bytes * EB + jc * EPS) >> 6];       // fp32, group 64
@@ -351,6 +366,23 @@ __device__ __forceinline__ void skinny_rows_body(const SkinnyRowsArgs& g, const 
             bf16x8 xf[MPS];
 #pragma unroll
             for (int c = 0; c < MPS; ++c) xf[c] = *(const bf16x8*)(xrow + j * (EPS * 2) + c * 16);
+            if constexpr (P8) {
+                if (vs4 && j % 4 == 0) {
+                    // register k of lane row r <- what lane row k fetched for lane row r: upper / lower halves of the wave swap
+                    // between registers two apart (v_permlane32_swap), then odd / even 16-lane rows between neighbours
+                    // (v_permlane16_swap)
+#pragma unroll
+                    for (int gi = 0; gi < G; ++gi) {
+                        const u32x2 d = scx[rr][gi][j / 4];
+                        uint32_t x0 = d[0], x1 = FMT == XQ_FMT_NF4 ? d[0] : d[0] >> 16, x2 = d[1], x3 = FMT == XQ_FMT_NF4 ? d[1] : d[1] >> 16;
+                        const auto p02 = __builtin_amdgcn_permlane32_swap(x0, x2, false, false);
+                        const auto p13 = __builtin_amdgcn_permlane32_swap(x1, x3, false, false);
+                        const auto q01 = __builtin_amdgcn_permlane16_swap(p02[0], p13[0], false, false);
+                        const auto q23 = __builtin_amdgcn_permlane16_swap(p02[1], p13[1], false, false);
+                        sx[gi][0] = q01[0]; sx[gi][1] = q01[1]; sx[gi][2] = q23[0]; sx[gi][3] = q23[1];
+                    }
+                }
+            }
 #pragma unroll
             for (int gi = 0; gi < G; ++gi) {
 #pragma unroll
@@ -368,10 +400,14 @@ __device__ __forceinline__ void skinny_rows_body(const SkinnyRowsArgs& g, const 
                         }
                         wf = decode8<FMT>(w[sl][gi][c], 0u, sv, -8.0f * sv);
                     } else if (FMT == XQ_FMT_NF4) {
-                        wf = decode8<FMT>(w[sl][gi][c], 0u, __uint_as_float(sc[sl][gi][0]), 0.0f, nf4_lds);
+                        uint32_t sb;
+                        if (vs4) sb = sx[P8 ? gi : 0][j & 3];
+                        else sb = sc[sl][gi][0];
+                        wf = decode8<FMT>(w[sl][gi][c], 0u, __uint_as_float(sb), 0.0f, nf4_lds);
                     } else {
                         float sv;   // block c / 2 of the load's two
-                        if (g.scale_dtype == XQ_SCALE_E4M3) sv = e4m3_to_f32((uint8_t)(sc[sl][gi][0] >> (8 * (c >> 1))));
+                        if (vs4) sv = e4m3_to_f32((uint8_t)(sx[P8 ? gi : 0][j & 3] >> (8 * (c >> 1))));
+                        else if (g.scale_dtype == XQ_SCALE_E4M3) sv = e4m3_to_f32((uint8_t)(sc[sl][gi][0] >> (8 * (c >> 1))));
                         else sv = __uint_as_float(sc[sl][gi][c >> 1]);
                         wf = decode8<FMT>(w[sl][gi][c], 0u, sv * gsc, 0.0f);
                     }
