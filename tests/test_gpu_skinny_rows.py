@@ -61,6 +61,13 @@ def _forward(m, x, r=None, bias=True):
     ("int4", 24576, 4096, 16, False),
     ("nf4", 24576, 2048, 8, True),
     ("nvfp4", 24576, 1024, 16, False),
+    # scale loads that cover four load steps at a time: two and three groups of four (int4), a last group of one step
+    # (nvfp4, nf4: five steps per wave), three whole groups (nvfp4)
+    ("int4", 2048, 8192, 16, False),
+    ("int4", 1024, 12288, 8, True),
+    ("nvfp4", 2048, 5120, 16, False),
+    ("nvfp4", 1024, 12288, 8, False),
+    ("nf4", 1024, 8192, 16, False),
 ])
 def test_one_launch_vs_oracle_and_two_launch(hip_device, organisations, fmt, N, K, r, has_bias):
     m, w_ref = make_dense_module(fmt, N, K, r, 2 * r, seed=N + K + r, device=hip_device, bias=has_bias)
