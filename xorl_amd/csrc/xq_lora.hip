@@ -394,6 +394,197 @@ int launch_small_nt(const bf16_t* In, int64_t ld_in, int64_t n_rows, int64_t Kc,
     return XQ_OK;
 }
 
+// ------------------------------------------------------------------ SwiGLU backward + its two low-rank products
+// One pass over (gate, up, dh): writes dgate | dup (the elementwise kernel's arithmetic, ops/moe/lora.py:855-917 with no
+// routing weight) and forms Tg = s * dgate . Fg^T and Tu = s * dup . Fu^T from the values on their way out -- the two
+// products no longer read dgate | dup back.  Dense rows; organisation and summation order of small_nt_kernel<32, FJ>
+// (32 rows per block, the four waves split the columns, 128 columns at a time through wave-private LDS tiles), so Tg
+// and Tu are the bits the two small_nt launches produce.
+struct SiluNtArgs {
+    const bf16_t* gate;
+    const bf16_t* up;
+    int64_t ld_gu;
+    const bf16_t* dh;
+    int64_t ld_dh;
+    bf16_t* dgate;
+    bf16_t* dup;
+    int64_t ld_out;
+    int64_t n_rows, Kc;        // rows; columns of gate / up / dh (the contraction length of the two products)
+    const bf16_t* Fg;          // [r_pad][Kc]
+    const bf16_t* Fu;
+    int r_pad;
+    float scale;
+    bf16_t* Tg;                // [n_rows][ld_t]
+    bf16_t* Tu;
+    int64_t ld_t;
+};
+
+template <int FJ>
+__global__ void __launch_bounds__(256) silu_bwd_nt_kernel(SiluNtArgs g) {
+    static_assert(FJ <= 8, "one MFMA column tile per product");
+    constexpr int WTILE = (32 + 32) * SN_P;      // bf16 elements per wave: value tile + factor tile
+    extern __shared__ __attribute__((aligned(16))) bf16_t sn_lds[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int64_t row0 = (int64_t)blockIdx.x * 32, row_end = g.n_rows;
+    if (row0 >= row_end) return;
+    bf16_t* xs = sn_lds + wave * WTILE;          // [32][SN_P]
+    bf16_t* fs = xs + 32 * SN_P;                 // [32][SN_P]
+    const int fr = lane & 31, fk = (lane >> 5) * 8;
+    const int crow = lane >> 4, cpiece = (lane & 15) * 8;
+    const int frows = g.r_pad;
+    const int64_t kspan = g.Kc / 4;              // multiple of 16
+    const int64_t kbeg = wave * kspan, kend = kbeg + kspan;
+    const int64_t rbase = row0 + crow;           // this lane's rows: rbase + 4 j, clamped onto the last row
+    auto row_of = [&](int j) { const int64_t r = rbase + j * 4; return r < row_end ? r : row_end - 1; };
+    u32x4 gq[8], uq[8], dq[8], fq[FJ];
+    // every load is unconditional: rows past the end and pieces past the wave's columns are clamped onto valid ones
+    auto fetch = [&](int64_t k) {
+        int64_t kc = k + cpiece;
+        kc = kc < kend ? kc : kend - 8;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int64_t r = row_of(j);
+            gq[j] = *(const u32x4*)(g.gate + r * g.ld_gu + kc);
+            uq[j] = *(const u32x4*)(g.up + r * g.ld_gu + kc);
+            dq[j] = *(const u32x4*)(g.dh + r * g.ld_dh + kc);
+        }
+    };
+    auto fetch_f = [&](const bf16_t* F, int64_t k) {
+        int64_t kc = k + cpiece;
+        kc = kc < kend ? kc : kend - 8;
+#pragma unroll
+        for (int j = 0; j < FJ; ++j) fq[j] = *(const u32x4*)(F + (int64_t)(j * 4 + crow) * g.Kc + kc);
+    };
+    auto stage_f = [&]() {
+#pragma unroll
+        for (int j = 0; j < FJ; ++j) *(u32x4*)(fs + (j * 4 + crow) * SN_P + cpiece) = fq[j];
+    };
+    f32x16 acc_g, acc_u;
+#pragma unroll
+    for (int q = 0; q < 16; ++q) acc_g[q] = acc_u[q] = 0.0f;
+    auto multiply = [&](f32x16& acc, int nsteps) {
+#pragma unroll
+        for (int st = 0; st < 8; ++st) {
+            if (st < nsteps) {                   // uniform
+                const bf16x8 a = *(const bf16x8*)(xs + fr * SN_P + st * 16 + fk);
+                const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+                const bf16x8 b = fr < frows ? *(const bf16x8*)(fs + fr * SN_P + st * 16 + fk) : zero8;
+                acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc, 0, 0, 0);
+            }
+        }
+    };
+    // The factor chunks (from L2) are requested ahead of the value chunks and go to the LDS tile as soon as the MFMAs that
+    // read its previous contents are issued (LDS operations of one wave execute in order), so their registers are free
+    // while a chunk's values are worked out.
+    fetch_f(g.Fg, kbeg);
+    fetch(kbeg);
+    stage_f();
+    for (int64_t k = kbeg; k < kend; k += 128) {
+        const int64_t kc = k + cpiece;
+        const bool mine = kc < kend;             // this lane's piece lies in the wave's columns
+        fetch_f(g.Fu, k);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            u32x4 og, ou;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                float rg[2], ru[2];
+#pragma unroll
+                for (int hlf = 0; hlf < 2; ++hlf) {
+                    const float gv = bf16_to_f32((bf16_t)(gq[j][i] >> (16 * hlf))), uv = bf16_to_f32((bf16_t)(uq[j][i] >> (16 * hlf)));
+                    const float d = bf16_to_f32((bf16_t)(dq[j][i] >> (16 * hlf)));
+                    const float sg = sigmoid_f32(gv);
+                    const float a = round_bf16(gv * sg);
+                    rg[hlf] = round_bf16(d * uv) * (sg * (1.0f + gv * (1.0f - sg)));
+                    ru[hlf] = a * d;
+                }
+                og[i] = pack_bf16x2(rg[0], rg[1]);
+                ou[i] = pack_bf16x2(ru[0], ru[1]);
+            }
+            if (rbase + j * 4 < row_end && mine) {
+                const int64_t r = rbase + j * 4;
+                *(u32x4*)(g.dgate + r * g.ld_out + kc) = og;
+                *(u32x4*)(g.dup + r * g.ld_out + kc) = ou;
+            }
+            *(u32x4*)(xs + (j * 4 + crow) * SN_P + cpiece) = og;
+            uq[j] = ou;                          // waits in registers for its turn in the tile
+        }
+        const int64_t left = kend - k;
+        const int nsteps = (int)((left < 128 ? left : 128) >> 4);
+        multiply(acc_g, nsteps);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) *(u32x4*)(xs + (j * 4 + crow) * SN_P + cpiece) = uq[j];
+        stage_f();                               // the up factor's chunk
+        fetch_f(g.Fg, k + 128);                  // (past the last chunk: clamped, never used)
+        fetch(k + 128);
+        multiply(acc_u, nsteps);
+        stage_f();                               // the gate factor's next chunk
+    }
+
+    // the four waves' sums meet in LDS, in wave order (as in small_nt_kernel)
+    float* red = (float*)sn_lds;                 // [3 waves][2 products][16][64] floats, over the (now dead) tiles
+    __syncthreads();
+    if (wave > 0) {
+#pragma unroll
+        for (int q = 0; q < 16; ++q) {
+            red[(((wave - 1) * 2 + 0) * 16 + q) * 64 + lane] = acc_g[q];
+            red[(((wave - 1) * 2 + 1) * 16 + q) * 64 + lane] = acc_u[q];
+        }
+    }
+    __syncthreads();
+    if (wave > 0) return;
+#pragma unroll
+    for (int s = 1; s < 4; ++s)
+#pragma unroll
+        for (int q = 0; q < 16; ++q) {
+            acc_g[q] += red[(((s - 1) * 2 + 0) * 16 + q) * 64 + lane];
+            acc_u[q] += red[(((s - 1) * 2 + 1) * 16 + q) * 64 + lane];
+        }
+    const int rgrp = (lane >> 5) * 4;
+    if (fr < g.r_pad) {
+#pragma unroll
+        for (int q = 0; q < 16; ++q) {
+            const int64_t row = row0 + (q & 3) + rgrp + 8 * (q >> 2);
+            if (row < row_end) {
+                g.Tg[row * g.ld_t + fr] = to_bf16(acc_g[q] * g.scale);
+                g.Tu[row * g.ld_t + fr] = to_bf16(acc_u[q] * g.scale);
+            }
+        }
+    }
+}
+
+template <int FJ>
+static int launch_silu_bwd_nt_one(const SiluNtArgs& g, hipStream_t stream) {
+    constexpr size_t lds = (size_t)4 * (32 + 32) * SN_P * 2;
+    static std::atomic<bool> attr_set{false};   // the attribute call is idempotent: a race only repeats it
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute((const void*)silu_bwd_nt_kernel<FJ>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) {
+            xq_set_error("silu_bwd_nt: cannot raise the dynamic LDS limit: %s", hipGetErrorString(e));
+            return XQ_ERR_LAUNCH;
+        }
+        attr_set = true;
+    }
+    silu_bwd_nt_kernel<FJ><<<dim3((unsigned)xq_cdiv(g.n_rows, 32)), 256, lds, stream>>>(g);
+    XQ_CHECK_LAUNCH("silu_bwd_nt");
+    return XQ_OK;
+}
+
+bool silu_bwd_nt_supported(int64_t cols, int r_pad) { return (r_pad == 16 || r_pad == 32) && cols % 64 == 0 && cols >= 512; }
+
+int launch_silu_bwd_nt(const bf16_t* gate, const bf16_t* up, int64_t ld_gu, const bf16_t* dh, int64_t ld_dh, bf16_t* dgate,
+                       bf16_t* dup, int64_t ld_out, int64_t n_rows, int64_t cols, const bf16_t* Fg, const bf16_t* Fu, int r_pad,
+                       float scale, bf16_t* Tg, bf16_t* Tu, int64_t ld_t, hipStream_t stream) {
+    XQ_REQUIRE(silu_bwd_nt_supported(cols, r_pad), "silu_bwd_nt: %lld columns with r_pad %d are not handled here", (long long)cols, r_pad);
+    XQ_REQUIRE(ld_gu % 8 == 0 && ld_dh % 8 == 0 && ld_out % 8 == 0 && ld_t >= r_pad, "silu_bwd_nt: row pitches must be multiples of 8");
+    XQ_REQUIRE(xq_aligned(gate, 16) && xq_aligned(up, 16) && xq_aligned(dh, 16) && xq_aligned(dgate, 16) && xq_aligned(dup, 16) &&
+                   xq_aligned(Fg, 16) && xq_aligned(Fu, 16),
+               "silu_bwd_nt: operands must be 16-byte aligned");
+    if (n_rows == 0) return XQ_OK;
+    SiluNtArgs g{gate, up, ld_gu, dh, ld_dh, dgate, dup, ld_out, n_rows, cols, Fg, Fu, r_pad, scale, Tg, Tu, ld_t};
+    return r_pad == 16 ? launch_silu_bwd_nt_one<4>(g, stream) : launch_silu_bwd_nt_one<8>(g, stream);
+}
+
 // ------------------------------------------------------------------ tn (weight-gradient shape)
 struct TnArgs {
     const bf16_t* P;

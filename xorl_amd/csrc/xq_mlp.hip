@@ -53,6 +53,9 @@ __global__ void __launch_bounds__(256) add_rows_kernel(bf16_t* a, int64_t lda, c
 }
 
 static const int g_mlp_gu = [] { const char* e = getenv("XQ_MLP_GU"); return e ? atoi(e) : 1; }();
+// XQ_MLP_SILU_NT=0: the SwiGLU backward and the two low-rank products of its outputs as three launches (A/B measurements;
+// same bits either way)
+static const int g_mlp_silu_nt = [] { const char* e = getenv("XQ_MLP_SILU_NT"); return e ? atoi(e) : 1; }();
 bool fuse_gate_up_fwd(const xq_weight* gate, const xq_weight* up) { return g_mlp_gu && gate->format == XQ_FMT_FP8 && up->format == XQ_FMT_FP8; }
 
 // Where the two low-rank intermediates lie in su_gate_up (M * 2 * rp elements): as the column bands [0, rp) and
@@ -288,15 +291,23 @@ extern "C" int xq_mlp_bwd(const xq_weight* gate, const xq_weight* up, const xq_w
         if ((rc = launch_tn(dy, lddy, H, su_d, rp, r, M, false, grads->dB[2], part, nullptr, 1, stream))) return rc;       // [H, r]
         if ((rc = launch_tn(h, I, I, v_d, rp, r, M, true, grads->dA[2], part, nullptr, 1, stream))) return rc;             // [r, I]
     }
-    // ---- SwiGLU
-    if ((rc = xq_silu_mul_bwd(gu, gu + I, 2 * I, dh, I, nullptr, dgate, dup, 2 * I, nullptr, M, I, stream))) return rc;
-    // ---- gate / up
+    // ---- SwiGLU, and s * dgate . B_g^T, s * dup . B_u^T: one pass over (gate, up, dh) where the rank allows, so that the
+    // two products do not read dgate | dup back
     const int64_t ld_v = fused ? rp2 : rp;
     bf16_t* v_g = v_gu;
     bf16_t* v_u = fused ? v_gu + rp : v_gu + M * rp;
+    const bool one_pass = rp && g_mlp_silu_nt && silu_bwd_nt_supported(I, rp);
+    if (one_pass) {
+        if ((rc = launch_silu_bwd_nt(gu, gu + I, 2 * I, dh, I, dgate, dup, 2 * I, M, I, Bt_g, Bt_u, rp, s, v_g, v_u, ld_v, stream))) return rc;
+    } else if ((rc = xq_silu_mul_bwd(gu, gu + I, 2 * I, dh, I, nullptr, dgate, dup, 2 * I, nullptr, M, I, stream))) {
+        return rc;
+    }
+    // ---- gate / up
     if (rp) {
-        if ((rc = launch_small_nt(dgate, 2 * I, M, I, Bt_g, rp, s, v_g, nullptr, nullptr, 1, true, stream, ld_v))) return rc;
-        if ((rc = launch_small_nt(dup, 2 * I, M, I, Bt_u, rp, s, v_u, nullptr, nullptr, 1, true, stream, ld_v))) return rc;
+        if (!one_pass) {
+            if ((rc = launch_small_nt(dgate, 2 * I, M, I, Bt_g, rp, s, v_g, nullptr, nullptr, 1, true, stream, ld_v))) return rc;
+            if ((rc = launch_small_nt(dup, 2 * I, M, I, Bt_u, rp, s, v_u, nullptr, nullptr, 1, true, stream, ld_v))) return rc;
+        }
         const SuLayout sl = su_layout(gate, up, rp, M);
         if ((rc = launch_tn(dgate, 2 * I, I, su_gu, rp, r, M, false, grads->dB[0], part, nullptr, 1, stream, nullptr, sl.pitch))) return rc;        // [I, r]
         if ((rc = launch_tn(dup, 2 * I, I, su_gu + sl.up_offset, rp, r, M, false, grads->dB[1], part, nullptr, 1, stream, nullptr, sl.pitch))) return rc;
