@@ -321,13 +321,19 @@ extern "C" int xq_grouped_bwd(const xq_weight* gate, const xq_weight* up, const 
     if ((rc = launch_tn(gd, ld_gd, H, su_d, rp, r, R, true, grads->dB[2], wg, dBe == 1 ? nullptr : off, E, stream, n_valid, 0, gd_rows))) return rc;   // [E|1, r, H]
     if ((rc = launch_tn(h, I, I, v_d, rp, r, R, false, grads->dA[2], wg, dAe == 1 ? nullptr : off, E, stream, n_valid))) return rc;        // [E|1, I, r]
 
-    // ---- SwiGLU + routing weight
-    if ((rc = xq_silu_mul_bwd(gu, gu + I, 2 * I, dh, I, saved->w_row, dgate, dup, 2 * I, d_w_row, R, I, stream))) return rc;
+    // ---- SwiGLU + routing weight, and s * dgate . B_g^T, s * dup . B_u^T of the up / gate projections (y = x.W + s*(x.A).B):
+    // one pass over (gate, up, dh) where the rank allows, so that the two products do not read dgate | dup back
+    static const bool silu_nt = [] { const char* e = getenv("XQ_MLP_SILU_NT"); return e ? atoi(e) != 0 : true; }();
+    if (silu_nt && silu_bwd_nt_supported(I, rp)) {
+        if ((rc = launch_silu_bwd_nt(gu, gu + I, 2 * I, dh, I, dgate, dup, 2 * I, R, I, F_gB, F_uB, rp, s, v_g, v_u, ld_v, stream, off, toff, E,
+                                     gBe == 1, uBe == 1, saved->w_row, d_w_row)))
+            return rc;
+    } else {
+        if ((rc = xq_silu_mul_bwd(gu, gu + I, 2 * I, dh, I, saved->w_row, dgate, dup, 2 * I, d_w_row, R, I, stream))) return rc;
+        if ((rc = launch_small_nt(dup, 2 * I, R, I, F_uB, rp, s, v_u, off, toff, E, uBe == 1, stream, ld_v))) return rc;
+        if ((rc = launch_small_nt(dgate, 2 * I, R, I, F_gB, rp, s, v_g, off, toff, E, gBe == 1, stream, ld_v))) return rc;
+    }
     if (d_routing && (rc = xq_moe_gather_scalar(d_w_row, sidx, R, d_routing, rw_dtype, stream))) return rc;
-
-    // ---- up / gate projections: y = x.W + s*(x.A).B
-    if ((rc = launch_small_nt(dup, 2 * I, R, I, F_uB, rp, s, v_u, off, toff, E, uBe == 1, stream, ld_v))) return rc;
-    if ((rc = launch_small_nt(dgate, 2 * I, R, I, F_gB, rp, s, v_g, off, toff, E, gBe == 1, stream, ld_v))) return rc;
     if (fused) {
         const TwoBanks two{up, nullptr, nullptr};
         if ((rc = launch_tile_gemm(gate, true, dgu, 2 * I, R, off, toff, v_gu, Lr_guA, rp2, nullptr, dx_g, H, stream, who, nullptr, 0, &two))) return rc;

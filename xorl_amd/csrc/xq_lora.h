@@ -62,13 +62,17 @@ int launch_small_nt(const bf16_t* In, int64_t ld_in, int64_t n_rows, int64_t Kc,
                     const int32_t* row_map = nullptr,       // grouped: product row i is made from row row_map[i] of In, and the
                     bf16_t* copy_out = nullptr, int64_t ld_copy = 0);   // gathered rows are also written to copy_out [rows, Kc] (if given)
 
-// SwiGLU backward and the two low-rank products of its outputs in one pass (dense rows, r_pad 16 or 32): dgate | dup as
-// xq_silu_mul_bwd writes them without a routing weight, Tg = scale * dgate . Fg^T, Tu = scale * dup . Fu^T as two
+// SwiGLU backward and the two low-rank products of its outputs in one pass (r_pad 16 or 32): dgate | dup as
+// xq_silu_mul_bwd writes them, Tg = scale * dgate . Fg^T, Tu = scale * dup . Fu^T as two
 // launch_small_nt calls on them would (same bits)
 bool silu_bwd_nt_supported(int64_t cols, int r_pad);
 int launch_silu_bwd_nt(const bf16_t* gate, const bf16_t* up, int64_t ld_gu, const bf16_t* dh, int64_t ld_dh, bf16_t* dgate,
                        bf16_t* dup, int64_t ld_out, int64_t n_rows, int64_t cols, const bf16_t* Fg, const bf16_t* Fu, int r_pad,
-                       float scale, bf16_t* Tg, bf16_t* Tu, int64_t ld_t, hipStream_t stream);
+                       float scale, bf16_t* Tg, bf16_t* Tu, int64_t ld_t, hipStream_t stream,
+                       // routed rows in expert order (offsets != NULL): a factor pair per expert ([E][r_pad][cols]) unless
+                       // shared, the rows' routing weights applied and (d_row_w != NULL) their gradients written
+                       const int32_t* offsets = nullptr, const int32_t* tile_offsets = nullptr, int32_t num_experts = 1,
+                       bool shared_fg = true, bool shared_fu = true, const float* row_w = nullptr, float* d_row_w = nullptr);
 
 // out[c][j] (or out[j][c] when transpose_out) = sum_m P[m][c] * Q[m][j], fp32.
 //   dense: all rows, split over `splits` row ranges, partials in `partial`

@@ -417,32 +417,85 @@ struct SiluNtArgs {
     bf16_t* Tg;                // [n_rows][ld_t]
     bf16_t* Tu;
     int64_t ld_t;
+    // routed rows (GROUPED): rows in expert order, a factor pair per expert (stride 0: shared), the routing weight of a row
+    // applied as the elementwise kernel applies it, and its gradient
+    const int32_t* offsets;
+    const int32_t* tile_offsets;
+    int32_t num_experts;
+    int64_t fg_stride, fu_stride;
+    const float* row_w;
+    float* d_row_w;
 };
 
-template <int FJ>
-__global__ void __launch_bounds__(256) silu_bwd_nt_kernel(SiluNtArgs g) {
+// GROUPED: routed rows in expert order, organisation of small_nt_kernel<128, FJ> (a block = a 128-row tile of one expert, a
+// wave = 32 rows over all columns, the expert's own factor pair), the routing weight applied and its gradient formed as
+// the elementwise kernel does (the sum over a row runs in another order here: 16 lanes' partial sums, then a butterfly).
+template <int FJ, bool GROUPED>
+__global__ void __launch_bounds__(256, 2) silu_bwd_nt_kernel(SiluNtArgs g) {
     static_assert(FJ <= 8, "one MFMA column tile per product");
-    constexpr int WTILE = (32 + 32) * SN_P;      // bf16 elements per wave: value tile + factor tile
+    // 64 columns at a time (where small_nt_kernel takes 128: the same MFMA steps in the same order): three operands' pieces
+    // are 12 KB per wave in flight, and two blocks share a compute unit
+    constexpr int CW = 64, P = CW + 8;           // columns of a chunk; LDS row pitch (144 B: the 16 lanes of a read phase hit distinct banks)
+    constexpr int NL = 32 * CW / 512;            // 16-byte loads per lane and operand chunk (a load instruction covers 512 / CW rows)
+    constexpr int RPI = 512 / CW;                // rows per load instruction
+    constexpr int FL = (FJ * 4 + RPI - 1) / RPI; // loads per lane of a factor chunk (FJ * 4 rows)
+    constexpr int WTILE = (32 + 32) * P;         // bf16 elements per wave: value tile + factor tile
     extern __shared__ __attribute__((aligned(16))) bf16_t sn_lds[];
+    __shared__ int sh_info[3];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int64_t row0 = (int64_t)blockIdx.x * 32, row_end = g.n_rows;
-    if (row0 >= row_end) return;
-    bf16_t* xs = sn_lds + wave * WTILE;          // [32][SN_P]
-    bf16_t* fs = xs + 32 * SN_P;                 // [32][SN_P]
+    int e = 0;
+    int64_t row0, row_end;
+    if constexpr (GROUPED) {
+        // the expert whose tile range holds this block's tile: one look per thread, all loads in flight together
+        if (tid == 0) sh_info[0] = -1;
+        __syncthreads();
+        const int t = blockIdx.x;
+        for (int x = tid; x < g.num_experts; x += 256) {
+            const int lo = g.tile_offsets[x], hi = g.tile_offsets[x + 1];
+            const int o0 = g.offsets[x], o1 = g.offsets[x + 1];
+            if (lo <= t && t < hi) {
+                sh_info[0] = x;
+                sh_info[1] = o0 + (t - lo) * 128;
+                sh_info[2] = o1;
+            }
+        }
+        __syncthreads();
+        e = sh_info[0];
+        if (e < 0) return;
+        row0 = sh_info[1] + wave * 32;
+        row_end = sh_info[2];
+        if (row0 >= row_end) return;             // (no block barrier from here on in this form)
+    } else {
+        row0 = (int64_t)blockIdx.x * 32;
+        row_end = g.n_rows;
+        if (row0 >= row_end) return;
+    }
+    const bf16_t* Fg = g.Fg + (int64_t)e * g.fg_stride;
+    const bf16_t* Fu = g.Fu + (int64_t)e * g.fu_stride;
+    bf16_t* xs = sn_lds + wave * WTILE;          // [32][P]
+    bf16_t* fs = xs + 32 * P;                    // [32][P]
     const int fr = lane & 31, fk = (lane >> 5) * 8;
-    const int crow = lane >> 4, cpiece = (lane & 15) * 8;
+    const int crow = lane / (CW / 8), cpiece = (lane % (CW / 8)) * 8;
     const int frows = g.r_pad;
-    const int64_t kspan = g.Kc / 4;              // multiple of 16
-    const int64_t kbeg = wave * kspan, kend = kbeg + kspan;
-    const int64_t rbase = row0 + crow;           // this lane's rows: rbase + 4 j, clamped onto the last row
-    auto row_of = [&](int j) { const int64_t r = rbase + j * 4; return r < row_end ? r : row_end - 1; };
-    u32x4 gq[8], uq[8], dq[8], fq[FJ];
+    const int64_t kspan = GROUPED ? g.Kc : g.Kc / 4;        // multiple of 16
+    const int64_t kbeg = GROUPED ? 0 : wave * kspan, kend = kbeg + kspan;
+    const int64_t rbase = row0 + crow;           // this lane's rows: rbase + RPI j, clamped onto the last row
+    auto row_of = [&](int j) { const int64_t r = rbase + j * RPI; return r < row_end ? r : row_end - 1; };
+    float rw[GROUPED ? NL : 1], wsum[GROUPED ? NL : 1];
+    if constexpr (GROUPED) {
+#pragma unroll
+        for (int j = 0; j < NL; ++j) {
+            rw[j] = g.row_w[row_of(j)];
+            wsum[j] = 0.0f;
+        }
+    }
+    u32x4 gq[NL], uq[NL], dq[NL], fq[FL];
     // every load is unconditional: rows past the end and pieces past the wave's columns are clamped onto valid ones
     auto fetch = [&](int64_t k) {
         int64_t kc = k + cpiece;
         kc = kc < kend ? kc : kend - 8;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
+        for (int j = 0; j < NL; ++j) {
             const int64_t r = row_of(j);
             gq[j] = *(const u32x4*)(g.gate + r * g.ld_gu + kc);
             uq[j] = *(const u32x4*)(g.up + r * g.ld_gu + kc);
@@ -453,22 +506,23 @@ __global__ void __launch_bounds__(256) silu_bwd_nt_kernel(SiluNtArgs g) {
         int64_t kc = k + cpiece;
         kc = kc < kend ? kc : kend - 8;
 #pragma unroll
-        for (int j = 0; j < FJ; ++j) fq[j] = *(const u32x4*)(F + (int64_t)(j * 4 + crow) * g.Kc + kc);
+        for (int j = 0; j < FL; ++j) fq[j] = *(const u32x4*)(F + (int64_t)(j * RPI + crow < FJ * 4 ? j * RPI + crow : FJ * 4 - 1) * g.Kc + kc);
     };
     auto stage_f = [&]() {
 #pragma unroll
-        for (int j = 0; j < FJ; ++j) *(u32x4*)(fs + (j * 4 + crow) * SN_P + cpiece) = fq[j];
+        for (int j = 0; j < FL; ++j)
+            if (j * RPI + crow < 32) *(u32x4*)(fs + (j * RPI + crow) * P + cpiece) = fq[j];
     };
     f32x16 acc_g, acc_u;
 #pragma unroll
     for (int q = 0; q < 16; ++q) acc_g[q] = acc_u[q] = 0.0f;
     auto multiply = [&](f32x16& acc, int nsteps) {
 #pragma unroll
-        for (int st = 0; st < 8; ++st) {
+        for (int st = 0; st < CW / 16; ++st) {
             if (st < nsteps) {                   // uniform
-                const bf16x8 a = *(const bf16x8*)(xs + fr * SN_P + st * 16 + fk);
+                const bf16x8 a = *(const bf16x8*)(xs + fr * P + st * 16 + fk);
                 const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
-                const bf16x8 b = fr < frows ? *(const bf16x8*)(fs + fr * SN_P + st * 16 + fk) : zero8;
+                const bf16x8 b = fr < frows ? *(const bf16x8*)(fs + fr * P + st * 16 + fk) : zero8;
                 acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc, 0, 0, 0);
             }
         }
@@ -476,15 +530,15 @@ __global__ void __launch_bounds__(256) silu_bwd_nt_kernel(SiluNtArgs g) {
     // The factor chunks (from L2) are requested ahead of the value chunks and go to the LDS tile as soon as the MFMAs that
     // read its previous contents are issued (LDS operations of one wave execute in order), so their registers are free
     // while a chunk's values are worked out.
-    fetch_f(g.Fg, kbeg);
+    fetch_f(Fg, kbeg);
     fetch(kbeg);
     stage_f();
-    for (int64_t k = kbeg; k < kend; k += 128) {
+    for (int64_t k = kbeg; k < kend; k += CW) {
         const int64_t kc = k + cpiece;
         const bool mine = kc < kend;             // this lane's piece lies in the wave's columns
-        fetch_f(g.Fu, k);
+        fetch_f(Fu, k);
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
+        for (int j = 0; j < NL; ++j) {
             u32x4 og, ou;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
@@ -495,32 +549,58 @@ __global__ void __launch_bounds__(256) silu_bwd_nt_kernel(SiluNtArgs g) {
                     const float d = bf16_to_f32((bf16_t)(dq[j][i] >> (16 * hlf)));
                     const float sg = sigmoid_f32(gv);
                     const float a = round_bf16(gv * sg);
-                    rg[hlf] = round_bf16(d * uv) * (sg * (1.0f + gv * (1.0f - sg)));
-                    ru[hlf] = a * d;
+                    float dp = d;
+                    if constexpr (GROUPED) {
+                        dp = round_bf16(d * rw[j]);
+                        if (mine) wsum[j] += d * round_bf16(a * uv);
+                    }
+                    rg[hlf] = round_bf16(dp * uv) * (sg * (1.0f + gv * (1.0f - sg)));
+                    ru[hlf] = a * dp;
                 }
                 og[i] = pack_bf16x2(rg[0], rg[1]);
                 ou[i] = pack_bf16x2(ru[0], ru[1]);
             }
-            if (rbase + j * 4 < row_end && mine) {
-                const int64_t r = rbase + j * 4;
+            if (rbase + j * RPI < row_end && mine) {
+                const int64_t r = rbase + j * RPI;
                 *(u32x4*)(g.dgate + r * g.ld_out + kc) = og;
                 *(u32x4*)(g.dup + r * g.ld_out + kc) = ou;
             }
-            *(u32x4*)(xs + (j * 4 + crow) * SN_P + cpiece) = og;
+            *(u32x4*)(xs + (j * RPI + crow) * P + cpiece) = og;
             uq[j] = ou;                          // waits in registers for its turn in the tile
         }
         const int64_t left = kend - k;
-        const int nsteps = (int)((left < 128 ? left : 128) >> 4);
+        const int nsteps = (int)((left < CW ? left : CW) >> 4);
         multiply(acc_g, nsteps);
 #pragma unroll
-        for (int j = 0; j < 8; ++j) *(u32x4*)(xs + (j * 4 + crow) * SN_P + cpiece) = uq[j];
+        for (int j = 0; j < NL; ++j) *(u32x4*)(xs + (j * RPI + crow) * P + cpiece) = uq[j];
         stage_f();                               // the up factor's chunk
-        fetch_f(g.Fg, k + 128);                  // (past the last chunk: clamped, never used)
-        fetch(k + 128);
+        fetch_f(Fg, k + CW);                    // (past the last chunk: clamped, never used)
+        fetch(k + CW);
         multiply(acc_u, nsteps);
         stage_f();                               // the gate factor's next chunk
     }
 
+    const int rgrp = (lane >> 5) * 4;
+    if constexpr (GROUPED) {
+#pragma unroll
+        for (int j = 0; j < NL; ++j) {
+            float v = wsum[j];
+#pragma unroll
+            for (int o = 1; o < CW / 8; o <<= 1) v += __shfl_xor(v, o, 64);
+            if (g.d_row_w && lane % (CW / 8) == 0 && rbase + j * RPI < row_end) g.d_row_w[rbase + j * RPI] = v;
+        }
+        if (fr < g.r_pad) {
+#pragma unroll
+            for (int q = 0; q < 16; ++q) {
+                const int64_t row = row0 + (q & 3) + rgrp + 8 * (q >> 2);
+                if (row < row_end) {
+                    g.Tg[row * g.ld_t + fr] = to_bf16(acc_g[q] * g.scale);
+                    g.Tu[row * g.ld_t + fr] = to_bf16(acc_u[q] * g.scale);
+                }
+            }
+        }
+        return;
+    }
     // the four waves' sums meet in LDS, in wave order (as in small_nt_kernel)
     float* red = (float*)sn_lds;                 // [3 waves][2 products][16][64] floats, over the (now dead) tiles
     __syncthreads();
@@ -540,7 +620,6 @@ __global__ void __launch_bounds__(256) silu_bwd_nt_kernel(SiluNtArgs g) {
             acc_g[q] += red[(((s - 1) * 2 + 0) * 16 + q) * 64 + lane];
             acc_u[q] += red[(((s - 1) * 2 + 1) * 16 + q) * 64 + lane];
         }
-    const int rgrp = (lane >> 5) * 4;
     if (fr < g.r_pad) {
 #pragma unroll
         for (int q = 0; q < 16; ++q) {
@@ -553,19 +632,19 @@ __global__ void __launch_bounds__(256) silu_bwd_nt_kernel(SiluNtArgs g) {
     }
 }
 
-template <int FJ>
-static int launch_silu_bwd_nt_one(const SiluNtArgs& g, hipStream_t stream) {
-    constexpr size_t lds = (size_t)4 * (32 + 32) * SN_P * 2;
+template <int FJ, bool GROUPED>
+static int launch_silu_bwd_nt_one(const SiluNtArgs& g, unsigned blocks, hipStream_t stream) {
+    constexpr size_t lds = (size_t)4 * (32 + 32) * (64 + 8) * 2;
     static std::atomic<bool> attr_set{false};   // the attribute call is idempotent: a race only repeats it
     if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute((const void*)silu_bwd_nt_kernel<FJ>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        hipError_t e = hipFuncSetAttribute((const void*)silu_bwd_nt_kernel<FJ, GROUPED>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) {
             xq_set_error("silu_bwd_nt: cannot raise the dynamic LDS limit: %s", hipGetErrorString(e));
             return XQ_ERR_LAUNCH;
         }
         attr_set = true;
     }
-    silu_bwd_nt_kernel<FJ><<<dim3((unsigned)xq_cdiv(g.n_rows, 32)), 256, lds, stream>>>(g);
+    silu_bwd_nt_kernel<FJ, GROUPED><<<dim3(blocks), 256, lds, stream>>>(g);
     XQ_CHECK_LAUNCH("silu_bwd_nt");
     return XQ_OK;
 }
@@ -574,15 +653,25 @@ bool silu_bwd_nt_supported(int64_t cols, int r_pad) { return (r_pad == 16 || r_p
 
 int launch_silu_bwd_nt(const bf16_t* gate, const bf16_t* up, int64_t ld_gu, const bf16_t* dh, int64_t ld_dh, bf16_t* dgate,
                        bf16_t* dup, int64_t ld_out, int64_t n_rows, int64_t cols, const bf16_t* Fg, const bf16_t* Fu, int r_pad,
-                       float scale, bf16_t* Tg, bf16_t* Tu, int64_t ld_t, hipStream_t stream) {
+                       float scale, bf16_t* Tg, bf16_t* Tu, int64_t ld_t, hipStream_t stream, const int32_t* offsets,
+                       const int32_t* tile_offsets, int32_t num_experts, bool shared_fg, bool shared_fu, const float* row_w,
+                       float* d_row_w) {
     XQ_REQUIRE(silu_bwd_nt_supported(cols, r_pad), "silu_bwd_nt: %lld columns with r_pad %d are not handled here", (long long)cols, r_pad);
     XQ_REQUIRE(ld_gu % 8 == 0 && ld_dh % 8 == 0 && ld_out % 8 == 0 && ld_t >= r_pad, "silu_bwd_nt: row pitches must be multiples of 8");
     XQ_REQUIRE(xq_aligned(gate, 16) && xq_aligned(up, 16) && xq_aligned(dh, 16) && xq_aligned(dgate, 16) && xq_aligned(dup, 16) &&
                    xq_aligned(Fg, 16) && xq_aligned(Fu, 16),
                "silu_bwd_nt: operands must be 16-byte aligned");
+    XQ_REQUIRE(!offsets || (tile_offsets && row_w && num_experts >= 1), "silu_bwd_nt: the routed form needs tile offsets and row weights");
     if (n_rows == 0) return XQ_OK;
-    SiluNtArgs g{gate, up, ld_gu, dh, ld_dh, dgate, dup, ld_out, n_rows, cols, Fg, Fu, r_pad, scale, Tg, Tu, ld_t};
-    return r_pad == 16 ? launch_silu_bwd_nt_one<4>(g, stream) : launch_silu_bwd_nt_one<8>(g, stream);
+    SiluNtArgs g{gate, up, ld_gu, dh, ld_dh, dgate, dup, ld_out, n_rows, cols, Fg, Fu, r_pad, scale, Tg, Tu, ld_t,
+                 offsets, tile_offsets, num_experts, offsets && !shared_fg ? (int64_t)r_pad * cols : 0,
+                 offsets && !shared_fu ? (int64_t)r_pad * cols : 0, row_w, d_row_w};
+    if (offsets) {
+        const unsigned blocks = (unsigned)(xq_cdiv(n_rows, 128) + num_experts);
+        return r_pad == 16 ? launch_silu_bwd_nt_one<4, true>(g, blocks, stream) : launch_silu_bwd_nt_one<8, true>(g, blocks, stream);
+    }
+    const unsigned blocks = (unsigned)xq_cdiv(n_rows, 32);
+    return r_pad == 16 ? launch_silu_bwd_nt_one<4, false>(g, blocks, stream) : launch_silu_bwd_nt_one<8, false>(g, blocks, stream);
 }
 
 // ------------------------------------------------------------------ tn (weight-gradient shape)
