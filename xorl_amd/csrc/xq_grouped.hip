@@ -209,8 +209,14 @@ extern "C" int xq_grouped_fwd(const xq_weight* gate, const xq_weight* up, const 
         if ((rc = launch_tile_gemm(up, false, xr, ld_xr, R, off, toff, su_u, Lr_uB, rp, nullptr, gu + I, 2 * I, stream, who, nullptr, 0, nullptr, xr_rows))) return rc;
     }
     if ((rc = xq_moe_scatter_scalar(routing_w, rw_dtype, saved->scatter_index, R, saved->w_row, stream))) return rc;
-    if ((rc = xq_silu_mul_fwd(gu, gu + I, 2 * I, saved->w_row, h, I, R, I, stream))) return rc;
-    if ((rc = launch_small_nt(h, I, R, I, F_dA, rp, s, su_d, off, toff, E, dAe == 1, stream))) return rc;
+    // SwiGLU (times the row's routing weight) and s * h . A_d^T of the down projection: one pass where the rank allows
+    static const bool silu_nt = [] { const char* e = getenv("XQ_MLP_SILU_NT"); return e ? atoi(e) != 0 : true; }();
+    if (silu_nt && silu_bwd_nt_supported(I, rp)) {
+        if ((rc = launch_silu_fwd_nt(gu, gu + I, 2 * I, h, I, R, I, F_dA, rp, s, su_d, rp, stream, off, toff, E, dAe == 1, saved->w_row))) return rc;
+    } else {
+        if ((rc = xq_silu_mul_fwd(gu, gu + I, 2 * I, saved->w_row, h, I, R, I, stream))) return rc;
+        if ((rc = launch_small_nt(h, I, R, I, F_dA, rp, s, su_d, off, toff, E, dAe == 1, stream))) return rc;
+    }
     if ((rc = launch_tile_gemm(down, false, h, I, R, off, toff, su_d, Lr_dB, rp, nullptr, down_out, H, stream, who, nullptr, 0))) return rc;
     return xq_moe_gather(down_out, nullptr, H, saved->scatter_index, d.T, topk, H, out, ld_out, stream);
 }

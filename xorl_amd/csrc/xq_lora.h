@@ -74,6 +74,13 @@ int launch_silu_bwd_nt(const bf16_t* gate, const bf16_t* up, int64_t ld_gu, cons
                        const int32_t* offsets = nullptr, const int32_t* tile_offsets = nullptr, int32_t num_experts = 1,
                        bool shared_fg = true, bool shared_fu = true, const float* row_w = nullptr, float* d_row_w = nullptr);
 
+// the forward in the same organisation: h = SwiGLU(gate, up) as xq_silu_mul_fwd writes it (routed rows: times the row's
+// weight) and T = scale * h . F^T as launch_small_nt on h would (same bits)
+int launch_silu_fwd_nt(const bf16_t* gate, const bf16_t* up, int64_t ld_gu, bf16_t* h, int64_t ld_h, int64_t n_rows, int64_t cols,
+                       const bf16_t* F, int r_pad, float scale, bf16_t* T, int64_t ld_t, hipStream_t stream,
+                       const int32_t* offsets = nullptr, const int32_t* tile_offsets = nullptr, int32_t num_experts = 1,
+                       bool shared_f = true, const float* row_w = nullptr);
+
 // out[c][j] (or out[j][c] when transpose_out) = sum_m P[m][c] * Q[m][j], fp32.
 //   dense: all rows, split over `splits` row ranges, partials in `partial`
 //          ([splits][width][r_pad] fp32) reduced in fixed order (deterministic);

@@ -430,7 +430,10 @@ struct SiluNtArgs {
 // GROUPED: routed rows in expert order, organisation of small_nt_kernel<128, FJ> (a block = a 128-row tile of one expert, a
 // wave = 32 rows over all columns, the expert's own factor pair), the routing weight applied and its gradient formed as
 // the elementwise kernel does (the sum over a row runs in another order here: 16 lanes' partial sums, then a butterfly).
-template <int FJ, bool GROUPED>
+// FWD: the forward pass in the same organisation -- h = bf16(bf16(silu(gate)) * up) (routed: then rounded and times the row's
+// weight), the elementwise forward kernel's arithmetic, written through `dgate`, and Tg = scale * h . Fg^T from the values
+// on their way out (dh, dup, Fu, Tu, d_row_w unused).
+template <int FJ, bool GROUPED, bool FWD = false>
 __global__ void __launch_bounds__(256, 2) silu_bwd_nt_kernel(SiluNtArgs g) {
     static_assert(FJ <= 8, "one MFMA column tile per product");
     // 64 columns at a time (where small_nt_kernel takes 128: the same MFMA steps in the same order): three operands' pieces
@@ -499,7 +502,7 @@ __global__ void __launch_bounds__(256, 2) silu_bwd_nt_kernel(SiluNtArgs g) {
             const int64_t r = row_of(j);
             gq[j] = *(const u32x4*)(g.gate + r * g.ld_gu + kc);
             uq[j] = *(const u32x4*)(g.up + r * g.ld_gu + kc);
-            dq[j] = *(const u32x4*)(g.dh + r * g.ld_dh + kc);
+            if constexpr (!FWD) dq[j] = *(const u32x4*)(g.dh + r * g.ld_dh + kc);
         }
     };
     auto fetch_f = [&](const bf16_t* F, int64_t k) {
@@ -533,6 +536,36 @@ __global__ void __launch_bounds__(256, 2) silu_bwd_nt_kernel(SiluNtArgs g) {
     fetch_f(Fg, kbeg);
     fetch(kbeg);
     stage_f();
+    if constexpr (FWD) {
+        for (int64_t k = kbeg; k < kend; k += CW) {
+            const int64_t kc = k + cpiece;
+            const bool mine = kc < kend;
+#pragma unroll
+            for (int j = 0; j < NL; ++j) {
+                u32x4 oh;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    float res[2];
+#pragma unroll
+                    for (int hlf = 0; hlf < 2; ++hlf) {
+                        const float gv = bf16_to_f32((bf16_t)(gq[j][i] >> (16 * hlf))), uv = bf16_to_f32((bf16_t)(uq[j][i] >> (16 * hlf)));
+                        const float a = round_bf16(gv * sigmoid_f32(gv));
+                        float v = a * uv;
+                        if constexpr (GROUPED) v = round_bf16(v) * rw[j];
+                        res[hlf] = v;
+                    }
+                    oh[i] = pack_bf16x2(res[0], res[1]);
+                }
+                if (rbase + j * RPI < row_end && mine) *(u32x4*)(g.dgate + (rbase + j * RPI) * g.ld_out + kc) = oh;
+                *(u32x4*)(xs + (j * RPI + crow) * P + cpiece) = oh;
+            }
+            fetch_f(Fg, k + CW);                // (past the last chunk: clamped, never used)
+            fetch(k + CW);
+            const int64_t left = kend - k;
+            multiply(acc_g, (int)((left < CW ? left : CW) >> 4));
+            stage_f();
+        }
+    } else
     for (int64_t k = kbeg; k < kend; k += CW) {
         const int64_t kc = k + cpiece;
         const bool mine = kc < kend;             // this lane's piece lies in the wave's columns
@@ -587,7 +620,7 @@ __global__ void __launch_bounds__(256, 2) silu_bwd_nt_kernel(SiluNtArgs g) {
             float v = wsum[j];
 #pragma unroll
             for (int o = 1; o < CW / 8; o <<= 1) v += __shfl_xor(v, o, 64);
-            if (g.d_row_w && lane % (CW / 8) == 0 && rbase + j * RPI < row_end) g.d_row_w[rbase + j * RPI] = v;
+            if (!FWD && g.d_row_w && lane % (CW / 8) == 0 && rbase + j * RPI < row_end) g.d_row_w[rbase + j * RPI] = v;
         }
         if (fr < g.r_pad) {
 #pragma unroll
@@ -595,7 +628,7 @@ __global__ void __launch_bounds__(256, 2) silu_bwd_nt_kernel(SiluNtArgs g) {
                 const int64_t row = row0 + (q & 3) + rgrp + 8 * (q >> 2);
                 if (row < row_end) {
                     g.Tg[row * g.ld_t + fr] = to_bf16(acc_g[q] * g.scale);
-                    g.Tu[row * g.ld_t + fr] = to_bf16(acc_u[q] * g.scale);
+                    if constexpr (!FWD) g.Tu[row * g.ld_t + fr] = to_bf16(acc_u[q] * g.scale);
                 }
             }
         }
@@ -626,25 +659,25 @@ __global__ void __launch_bounds__(256, 2) silu_bwd_nt_kernel(SiluNtArgs g) {
             const int64_t row = row0 + (q & 3) + rgrp + 8 * (q >> 2);
             if (row < row_end) {
                 g.Tg[row * g.ld_t + fr] = to_bf16(acc_g[q] * g.scale);
-                g.Tu[row * g.ld_t + fr] = to_bf16(acc_u[q] * g.scale);
+                if constexpr (!FWD) g.Tu[row * g.ld_t + fr] = to_bf16(acc_u[q] * g.scale);
             }
         }
     }
 }
 
-template <int FJ, bool GROUPED>
+template <int FJ, bool GROUPED, bool FWD = false>
 static int launch_silu_bwd_nt_one(const SiluNtArgs& g, unsigned blocks, hipStream_t stream) {
     constexpr size_t lds = (size_t)4 * (32 + 32) * (64 + 8) * 2;
     static std::atomic<bool> attr_set{false};   // the attribute call is idempotent: a race only repeats it
     if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute((const void*)silu_bwd_nt_kernel<FJ, GROUPED>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        hipError_t e = hipFuncSetAttribute((const void*)silu_bwd_nt_kernel<FJ, GROUPED, FWD>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) {
             xq_set_error("silu_bwd_nt: cannot raise the dynamic LDS limit: %s", hipGetErrorString(e));
             return XQ_ERR_LAUNCH;
         }
         attr_set = true;
     }
-    silu_bwd_nt_kernel<FJ, GROUPED><<<dim3(blocks), 256, lds, stream>>>(g);
+    silu_bwd_nt_kernel<FJ, GROUPED, FWD><<<dim3(blocks), 256, lds, stream>>>(g);
     XQ_CHECK_LAUNCH("silu_bwd_nt");
     return XQ_OK;
 }
@@ -672,6 +705,24 @@ int launch_silu_bwd_nt(const bf16_t* gate, const bf16_t* up, int64_t ld_gu, cons
     }
     const unsigned blocks = (unsigned)xq_cdiv(n_rows, 32);
     return r_pad == 16 ? launch_silu_bwd_nt_one<4, false>(g, blocks, stream) : launch_silu_bwd_nt_one<8, false>(g, blocks, stream);
+}
+
+int launch_silu_fwd_nt(const bf16_t* gate, const bf16_t* up, int64_t ld_gu, bf16_t* h, int64_t ld_h, int64_t n_rows, int64_t cols,
+                       const bf16_t* F, int r_pad, float scale, bf16_t* T, int64_t ld_t, hipStream_t stream, const int32_t* offsets,
+                       const int32_t* tile_offsets, int32_t num_experts, bool shared_f, const float* row_w) {
+    XQ_REQUIRE(silu_bwd_nt_supported(cols, r_pad), "silu_fwd_nt: %lld columns with r_pad %d are not handled here", (long long)cols, r_pad);
+    XQ_REQUIRE(ld_gu % 8 == 0 && ld_h % 8 == 0 && ld_t >= r_pad, "silu_fwd_nt: row pitches must be multiples of 8");
+    XQ_REQUIRE(xq_aligned(gate, 16) && xq_aligned(up, 16) && xq_aligned(h, 16) && xq_aligned(F, 16), "silu_fwd_nt: operands must be 16-byte aligned");
+    XQ_REQUIRE(!offsets || (tile_offsets && row_w && num_experts >= 1), "silu_fwd_nt: the routed form needs tile offsets and row weights");
+    if (n_rows == 0) return XQ_OK;
+    SiluNtArgs g{gate, up, ld_gu, nullptr, 0, h, nullptr, ld_h, n_rows, cols, F, F, r_pad, scale, T, nullptr, ld_t,
+                 offsets, tile_offsets, num_experts, offsets && !shared_f ? (int64_t)r_pad * cols : 0, 0, row_w, nullptr};
+    if (offsets) {
+        const unsigned blocks = (unsigned)(xq_cdiv(n_rows, 128) + num_experts);
+        return r_pad == 16 ? launch_silu_bwd_nt_one<4, true, true>(g, blocks, stream) : launch_silu_bwd_nt_one<8, true, true>(g, blocks, stream);
+    }
+    const unsigned blocks = (unsigned)xq_cdiv(n_rows, 32);
+    return r_pad == 16 ? launch_silu_bwd_nt_one<4, false, true>(g, blocks, stream) : launch_silu_bwd_nt_one<8, false, true>(g, blocks, stream);
 }
 
 // ------------------------------------------------------------------ tn (weight-gradient shape)

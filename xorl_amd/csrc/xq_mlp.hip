@@ -170,6 +170,7 @@ extern "C" int xq_mlp_fwd(const xq_weight* gate, const xq_weight* up, const xq_w
     float* part = cv.take<float>(0);
     const int64_t part_bytes = workspace_bytes - cv.used;
     const bf16_t *bias_g = (const bf16_t*)lora->bias[0], *bias_u = (const bf16_t*)lora->bias[1], *bias_d = (const bf16_t*)lora->bias[2];
+    bool h_product_done = false;
     if (fused) {
         if ((rc = launch_gate_up_swiglu(gate, up, x, ldx, M, rp ? su_gu : nullptr, rp ? su_gu + sl.up_offset : nullptr, sl.pitch, Bl_g, Bl_u,
                                         rp, bias_g, bias_u, gu, 2 * I, h, I, stream)))
@@ -177,9 +178,15 @@ extern "C" int xq_mlp_fwd(const xq_weight* gate, const xq_weight* up, const xq_w
     } else {
         if ((rc = launch_tile_gemm(gate, true, x, ldx, M, nullptr, nullptr, rp ? su_gu : nullptr, Bl_g, rp, bias_g, gu, 2 * I, stream, who, part, part_bytes))) return rc;
         if ((rc = launch_tile_gemm(up, true, x, ldx, M, nullptr, nullptr, rp ? su_gu + sl.up_offset : nullptr, Bl_u, rp, bias_u, gu + I, 2 * I, stream, who, part, part_bytes))) return rc;
-        if ((rc = xq_silu_mul_fwd(gu, gu + I, 2 * I, nullptr, h, I, M, I, stream))) return rc;
+        // SwiGLU, and s * h . A_d^T of the down projection from the values on their way out where the rank allows
+        if (rp && g_mlp_silu_nt && silu_bwd_nt_supported(I, rp)) {
+            if ((rc = launch_silu_fwd_nt(gu, gu + I, 2 * I, h, I, M, I, A_d, rp, s, su_d, rp, stream))) return rc;
+            h_product_done = true;
+        } else if ((rc = xq_silu_mul_fwd(gu, gu + I, 2 * I, nullptr, h, I, M, I, stream))) {
+            return rc;
+        }
     }
-    if (rp && (rc = launch_small_nt(h, I, M, I, A_d, rp, s, su_d, nullptr, nullptr, 1, true, stream))) return rc;
+    if (rp && !h_product_done && (rc = launch_small_nt(h, I, M, I, A_d, rp, s, su_d, nullptr, nullptr, 1, true, stream))) return rc;
     return launch_tile_gemm(down, true, h, I, M, nullptr, nullptr, rp ? su_d : nullptr, Bl_d, rp, bias_d, (bf16_t*)y, ldy, stream,
                             who, part, part_bytes);
 }
