@@ -46,13 +46,13 @@ MEASURED_TRAFFIC = {
     0: (109.6 * 2 ** 20, "profiles/gemm_128_int4_linear_m512.txt", 0.04315),
     # gemm_256_kernel<fp8>: mean over the 4 launches of a step (gate|up forward with the SwiGLU epilogue, down
     # forward, d_h, dx as one sum over the gate and up weights)
-    1: (1408.3 * 2 ** 20, "profiles/gemm_256_fp8_mlp_m8192.txt", 1.12517),
+    1: (1405.3 * 2 ** 20, "profiles/gemm_256_fp8_mlp_m8192.txt", 1.05903),
     # gemm_256_kernel<nvfp4>, 256x256 tiles (whole rounds; trailing rows in K splits) and 128x128 tiles
     # (+ splitk_reduce_kernel): mean over the 12 launches of a step, fp32 partial sums included
     2: (185.7 * 2 ** 20, "profiles/gemm_256_nvfp4_attn_m4096.txt", 0.14304),
     # gemm_256_kernel<fp8, grouped>: mean over the 4 launches of a step (gate|up forward over two banks, down
     # forward, d_h, dx as one sum over both banks)
-    3: (1342.5 * 2 ** 20, "profiles/gemm_256_fp8_grouped_moe_e128.txt", 0.71589),
+    3: (1343.0 * 2 ** 20, "profiles/gemm_256_fp8_grouped_moe_e128.txt", 0.71449),
     # skinny_rows_kernel (M <= 16) and skinny_split_kernel + skinny_epilogue_kernel (M = 32, 64): mean per forward
     # over the 32 cases (includes the fp32 partial tiles of the two-launch cases written and read back: 23.3 MiB of
     # it are algorithmic)
@@ -62,7 +62,7 @@ MEASURED_TRAFFIC = {
     # gemm_256_kernel<nf4>: mean of the forward and dgrad launches
     6: (748.2 * 2 ** 20, "profiles/gemm_256_nf4_mlp_m8192.txt", 0.84180),
     # gemm_256_kernel<nvfp4 GKN, grouped>: mean over the 6 launches of a step
-    7: (894.6 * 2 ** 20, "profiles/gemm_256_nvfp4_gkn_grouped_moe_e128.txt", 0.52816),
+    7: (893.9 * 2 ** 20, "profiles/gemm_256_nvfp4_gkn_grouped_moe_e128.txt", 0.52825),
     # merge_prep_kernel + merge_kernel<nvfp4>: mean per call over amax / re-quantise / publish of the four weights
     9: (59.0 * 2 ** 20, "profiles/merge_kernel_nvfp4_attn_weights.txt", 0.03500),
 }
