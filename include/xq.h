@@ -104,6 +104,14 @@ int xq_set_tile_policy(int policy);
  * no counterpart in the reference. */
 int xq_set_persistent_tiles(int enabled);
 
+/* xq_mlp_fwd on block-fp8 weights runs gate and up either as two launches followed by one pass that writes h = SwiGLU and
+ * forms the down projection's low-rank intermediate on the way (enabled = 0, the default), or as ONE launch over both weights
+ * with the SwiGLU in its epilogue (enabled = 1).  Same outputs and saved activations bit for bit; the saved low-rank
+ * intermediates of gate and up are laid out differently, so the switch must not change between a forward and its backward.
+ * A process-wide switch for tests and A/B measurements (XQ_MLP_GU in the environment sets it at load time); no counterpart
+ * in the reference. */
+int xq_set_mlp_gate_up_fused(int enabled);
+
 /* xq_linear_fwd with M <= 16 rows runs as ONE launch where the shape and the LoRA operands allow it (FLAT weight,
  * K % 512 == 0 for block_fp8 / K % 1024 == 0 for the 4-bit formats, K <= 12288; fp32 factors with r <= 16, r % 4 == 0,
  * 16-byte aligned): whole weight rows per block, the low-rank intermediate formed once per launch and passed between

@@ -70,6 +70,42 @@ def test_fused_mlp_vs_oracle_and_modules(hip_device, tile_policy, fmt, M, H, I, 
         assert torch.equal(qlora_mlp_forward(mods["gate"], mods["up"], mods["down"], x.to(hip_device)), fused["y"])
 
 
+@pytest.mark.parametrize("tile_policy", [0, 2], indirect=True)
+@pytest.mark.parametrize("M,H,I,r,bias", [(300, 256, 512, 16, False), (1100, 512, 1024, 32, True), (2100, 512, 1536, 16, False)])
+def test_gate_up_as_one_launch_or_two(hip_device, tile_policy, M, H, I, r, bias):
+    """Block-fp8 gate and up as ONE launch with the SwiGLU in its epilogue, or as two launches followed by the pass that
+    writes h and forms the down projection's low-rank intermediate (the default): same bits everywhere, and the
+    one-launch form against the oracle."""
+    from xorl_amd import _C
+    from xorl_amd.qlora import qlora_mlp_forward
+
+    mods, w_ref = _mods("block_fp8", H, I, r, hip_device, bias=bias, seed=M + 1)
+    x = gen((M, H), 1.0, 81, torch.bfloat16)
+    dy = gen((M, H), 1.0, 82, torch.bfloat16)
+    got = {}
+    try:
+        for fused in (1, 0):
+            _C.check(_C.lib().xq_set_mlp_gate_up_fused(fused))
+            _zero(mods)
+            xd = x.to(hip_device).requires_grad_(True)
+            y = qlora_mlp_forward(mods["gate"], mods["up"], mods["down"], xd)
+            y.backward(dy.to(hip_device))
+            got[fused] = {"y": y.detach().clone(), "dx": xd.grad.clone(), **_grads(mods)}
+    finally:
+        _C.check(_C.lib().xq_set_mlp_gate_up_fused(0))
+    for name in got[0]:
+        assert torch.equal(got[0][name], got[1][name]), name
+    if bias:        # (the oracle's MLP program has no bias terms)
+        return
+    loras = {k: (m.lora_A.detach().cpu(), m.lora_B.detach().cpu()) for k, m in mods.items()}
+    ex = R.mlp_fwd_bwd_exact(x, w_ref["gate"], w_ref["up"], w_ref["down"], loras, mods["gate"].scaling, dy)
+    close(got[1]["y"].cpu(), ex["y"], TOL)
+    close(got[1]["dx"].cpu(), ex["dx"], TOL)
+    for k in ("gate", "up", "down"):
+        close(got[1][f"dA_{k}"].cpu(), ex[f"dA_{k}"], TOL)
+        close(got[1][f"dB_{k}"].cpu(), ex[f"dB_{k}"], TOL)
+
+
 def test_fused_mlp_bias_no_lora_and_fallbacks(hip_device):
     from xorl_amd.qlora import qlora_mlp_forward
 

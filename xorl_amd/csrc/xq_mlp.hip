@@ -9,6 +9,7 @@
 //             and the two A gradients come from one pass over x.
 // Other formats (and shapes the fused forms do not take) run the same program launch by launch.
 #include "xq_lora.h"
+#include <atomic>
 #include <stdlib.h>
 
 namespace xq {
@@ -52,7 +53,12 @@ __global__ void __launch_bounds__(256) add_rows_kernel(bf16_t* a, int64_t lda, c
     *(u32x4*)(a + m * lda + c) = o;
 }
 
-static const int g_mlp_gu = [] { const char* e = getenv("XQ_MLP_GU"); return e ? atoi(e) : 1; }();
+// gate and up of a block-fp8 MLP as ONE launch with the SwiGLU in its epilogue (1), or as two launches followed by the pass
+// that writes h and forms s * h . A_d^T on the way (0, the default: the two plain launches run at a higher rate than the
+// launch with the wide epilogue, and the step is level or slightly shorter).  XQ_MLP_GU in the environment sets it at load
+// time, xq_set_mlp_gate_up_fused() at run time; the layout of the saved low-rank intermediates follows it, so it must not
+// change between a forward and its backward.
+static std::atomic<int> g_mlp_gu{[] { const char* e = getenv("XQ_MLP_GU"); return e ? atoi(e) : 0; }()};
 // XQ_MLP_SILU_NT=0: the SwiGLU backward and the two low-rank products of its outputs as three launches (A/B measurements;
 // same bits either way)
 static const int g_mlp_silu_nt = [] { const char* e = getenv("XQ_MLP_SILU_NT"); return e ? atoi(e) : 1; }();
@@ -116,6 +122,11 @@ int64_t bwd_workspace(const Dims& d) {
 }  // namespace xq
 
 using namespace xq;
+
+extern "C" int xq_set_mlp_gate_up_fused(int enabled) {
+    g_mlp_gu = enabled != 0;
+    return XQ_OK;
+}
 
 extern "C" int64_t xq_mlp_workspace_bytes(int64_t M, int64_t hidden, int64_t intermediate, int r, int backward) {
     if (M < 0 || r < 0) return 0;
