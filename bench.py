@@ -134,7 +134,7 @@ def cpu_baseline(mods, rows: int, warmups: int = 2, runs: int = 5):
         "unit": "TFLOP/s",
         "cores": os.cpu_count(),
         "kind": "port",
-        "sample": f"{rows} of {M} token rows of the same MLP, decode+fwd+bwd, torch CPU ops on the oracle decode: "
+        "sample": f"{'all ' if rows == M else ''}{rows} of {M} token rows of the same MLP, decode+fwd+bwd, torch CPU ops on the oracle decode: "
                   f"median of {runs} runs after {warmups} warm-ups, {dt:.2f} s per run "
                   f"(min {min(times):.2f}, max {max(times):.2f})",
     }
@@ -330,12 +330,13 @@ def calibrate_copy(dev):
     del src, dst
 
 
-def traffic_of(args, live_avg_launch_ms):
+def traffic_of(args, live_avg_launch_ms, cfg=None):
     """-> (traffic bytes or None, provenance text).  The committed counter figure of this config, unless the run's
     own average launch duration says that it times something else than the counters measured."""
-    if args.traffic_bytes is not None:
+    cfg = args.config if cfg is None else cfg
+    if args.traffic_bytes is not None and cfg == args.config:
         return args.traffic_bytes, "--traffic-bytes"
-    entry = MEASURED_TRAFFIC.get(args.config)
+    entry = MEASURED_TRAFFIC.get(cfg)
     if entry is None:
         return None, "no counter run committed for this config"
     nbytes, profile, ref_ms = entry
@@ -350,8 +351,12 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--cpu-rows", type=int, default=4096,
-                    help="token rows of the CPU baseline sample (0 = skip); 2 warm-ups + 5 timed runs, ~12 s at 4096 rows")
+    ap.add_argument("--cpu-rows", type=int, default=M,
+                    help="token rows of the CPU baseline (0 = skip); default: the whole workload, 2 warm-ups + 5 timed runs "
+                         "of about 4.5 s each")
+    ap.add_argument("--no-secondary", action="store_true",
+                    help="config 1 only: skip the `secondary` measurements (configs[4] decode shapes against the HBM "
+                         "roofline, configs[3] grouped experts against the MFMA roofline) that the default run appends")
     ap.add_argument("--config", type=int, default=1,
                     help="BASELINE.json configs index; 1 (default) is the headline workload, the others report the "
                          "same JSON for their own workload (no CPU baseline)")
@@ -461,17 +466,22 @@ def main():
     if args.reference_path:
         out["path"] = "reference organisation: decode to bf16 + library GEMMs + fp32 LoRA branch + autograd (not the product path)"
         out["roofline"] = None
+    elif not args.unfused and not args.no_secondary:
+        del mods, x, dy, params
+        torch.cuda.empty_cache()
+        out["secondary"] = secondary_measurements(args, dev)
     print(json.dumps(out))
 
 
-def run_other(args, dev):
+def measure_other(args, dev, cfg, steps, warmup):
+    """One of the other workloads, measured like the headline one -> the dict of its JSON line."""
     from xorl_amd import _C
 
-    step, work, is_bytes, workload, kernel = other_config(args.config, dev)
+    step, work, is_bytes, workload, kernel = other_config(cfg, dev)
     L = _C.lib()
     if args.calibrate_copy:
         calibrate_copy(dev)
-    use_graph = args.config == 4 and not args.no_graph
+    use_graph = cfg == 4 and not args.no_graph
     if use_graph:
         # the decode-regime step is 32 launch-bound forwards: replay it as one HIP graph (what a serving loop
         # does).  Captured after an eager warm-up on a side stream; every replay runs the same kernels on the
@@ -491,19 +501,19 @@ def run_other(args, dev):
         workload += "; the step is replayed as one HIP graph"
     else:
         run = step
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         run()
     torch.cuda.synchronize()
     if not use_graph:
         L.xq_profile_enable(1)
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         run()
     torch.cuda.synchronize()
-    dt = (time.perf_counter() - t0) / args.steps
+    dt = (time.perf_counter() - t0) / steps
     if use_graph:
         L.xq_profile_enable(1)
-        for _ in range(args.steps):
+        for _ in range(steps):
             step()
         torch.cuda.synchronize()
     n, ms, fl = ctypes.c_int(0), ctypes.c_double(0), ctypes.c_double(0)
@@ -512,15 +522,116 @@ def run_other(args, dev):
     scale, unit, peak = (1e9, "GB/s", 8000.0) if is_bytes else (1e12, "TFLOP/s", BF16_MFMA_PEAK_TFLOPS)
     achieved = fl.value / (ms.value * 1e-3) / scale if ms.value > 0 else 0.0
     avg_launch_ms = ms.value / max(n.value, 1)
-    traffic, traffic_source = traffic_of(args, avg_launch_ms)
-    print(json.dumps({
-        "metric": METRIC, "value": work / dt / scale, "unit": unit, "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": dt * 1e3, "higher_is_better": True, "scaling": "weak",
+    traffic, traffic_source = traffic_of(args, avg_launch_ms, cfg)
+    return {
+        "metric": METRIC, "value": work / dt / scale, "unit": unit, "n_gpus": 1, "steps": steps,
+        "warmup": warmup, "ms_per_step": dt * 1e3, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic", "config": {"workload": workload},
         "roofline": {"bound": "hbm" if is_bytes else "mfma", "achieved": achieved, "peak": peak, "unit": unit,
                      "frac": achieved / peak, "traffic": traffic, "traffic_source": traffic_source, "kernel": kernel,
                      "launches": n.value, "avg_launch_ms": avg_launch_ms},
-        "cpu_baseline": None}))
+        "cpu_baseline": None}
+
+
+def run_other(args, dev):
+    print(json.dumps(measure_other(args, dev, args.config, args.steps, args.warmup)))
+
+
+# ---- configs[4] case by case: microseconds and GB/s of every (format, projection, M) forward
+DECODE_SHAPES = {"q": (4096, 4096), "kv": (1024, 4096), "gate_up": (12288, 4096), "down": (4096, 12288),
+                 "gate|up fused": (24576, 4096)}       # the last one is the reference's default fused module, not a configs[4] case
+COLD_FOOTPRINT = 640 << 20      # bytes of weight copies a case rotates through: 2.5 x the 256 MB memory-side cache
+
+
+def decode_case_table(dev, reps: int = 24, replays: int = 5):
+    """Every configs[4] forward on its own: `reps` forwards back to back as one HIP graph (launch boundaries included, no
+    host time), timed with events on the launch stream, median of `replays` replays.  Two figures per case: "cold" rotates
+    through copies of the weight whose total size exceeds the 256 MB memory-side cache, so every byte comes from HBM as it
+    does in a model whose layers do not fit that cache (this is the roofline figure); "hot" replays one weight, which
+    that cache may serve."""
+    from xorl_amd.functional import QuantWeight, qlora_linear
+
+    rows = []
+    g = torch.Generator(device=dev).manual_seed(7)
+    # one memory pool for all the graphs: the forwards' workspaces then sit at the same few addresses in every graph, and
+    # the library's per-workspace slots (which stay with a captured workspace for good) are not used up case by case
+    pool = torch.cuda.graph_pool_handle()
+    for fmt in ("int4", "block_fp8"):
+        for name, (N, K) in DECODE_SHAPES.items():
+            m = dense_module(fmt, N, K, 16, 32, 60, dev)
+            qw = m._quant_weight()
+            wbytes = qw.packed.numel() * qw.packed.element_size() + qw.scales.numel() * qw.scales.element_size()
+            n_copies = max(2, -(-COLD_FOOTPRINT // wbytes))
+            copies = [qw] + [QuantWeight(qw.fmt, qw.layout, qw.packed.clone(), qw.scales.clone(), qw.scale_dtype, qw.rows, qw.cols,
+                                         qw.group, global_scale=qw.global_scale) for _ in range(n_copies - 1)]
+            A, B, sc = m.lora_A.detach(), m.lora_B.detach(), m.scaling
+            for Mtok in (1, 8, 32, 64):
+                x = torch.randn(Mtok, K, generator=g, device=dev).to(torch.bfloat16)
+                algo = wbytes + 2 * Mtok * K + 2 * Mtok * N + 4 * 16 * (K + N)
+                us = {}
+                for mode, ws in (("cold", copies), ("hot", copies[:1])):
+                    def run():
+                        with torch.no_grad():
+                            for i in range(reps):
+                                qlora_linear(x, ws[i % len(ws)], A, B, 16, sc)
+                    side = torch.cuda.Stream()
+                    side.wait_stream(torch.cuda.current_stream())
+                    with torch.cuda.stream(side):
+                        run()
+                    torch.cuda.current_stream().wait_stream(side)
+                    torch.cuda.synchronize()
+                    graph = torch.cuda.CUDAGraph()
+                    with torch.cuda.graph(graph, pool=pool):
+                        run()
+                    graph.replay()
+                    torch.cuda.synchronize()
+                    times = []
+                    for _ in range(replays):
+                        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                        e0.record()
+                        graph.replay()
+                        e1.record()
+                        e1.synchronize()
+                        times.append(e0.elapsed_time(e1) * 1e3 / reps)
+                    us[mode] = sorted(times)[len(times) // 2]
+                    del graph
+                rows.append({"format": fmt, "proj": name, "N": N, "K": K, "M": Mtok, "bytes": algo,
+                             "us": round(us["cold"], 2), "GBps": round(algo / us["cold"] / 1e3, 1),
+                             "frac": round(algo / us["cold"] / 1e3 / 8000.0, 4),
+                             "us_hot": round(us["hot"], 2), "GBps_hot": round(algo / us["hot"] / 1e3, 1)})
+            del copies, m, qw
+            torch.cuda.empty_cache()
+    return rows
+
+
+def secondary_measurements(args, dev):
+    """The other two regimes of the path, measured in the same run as the headline line: configs[4] (skinny M, HBM
+    roofline; per case and over the 32 BASELINE cases) and configs[3] (grouped experts, MFMA roofline)."""
+    out = []
+    table = decode_case_table(dev)
+    base = [r for r in table if r["proj"] != "gate|up fused"]
+    tot_b, tot_us = sum(r["bytes"] for r in base), sum(r["us"] for r in base)
+    agg = tot_b / tot_us / 1e3
+    c4 = measure_other(args, dev, 4, 20, 5)
+    out.append({
+        "workload": "configs[4]: skinny-M forward, M in {1,8,32,64} x {q, kv, gate/up, down of Qwen3-8B} x {int4, block_fp8}, r=16; "
+                    "`cases` times every forward on its own (24 back to back in one HIP graph, weights rotating through "
+                    f"{COLD_FOOTPRINT >> 20} MiB of copies so that they come from HBM; *_hot: one weight replayed, which the 256 MB "
+                    "memory-side cache may serve); `achieved` is the 32 BASELINE cases' bytes over the sum of their times; "
+                    "`graph_step` replays the 32 forwards on one set of weights as one HIP graph",
+        "bound": "hbm", "achieved": agg, "peak": 8000.0, "unit": "GB/s", "frac": agg / 8000.0,
+        "traffic": c4["roofline"]["traffic"], "traffic_source": c4["roofline"]["traffic_source"],
+        "kernel": c4["roofline"]["kernel"],
+        "graph_step": {"value": c4["value"], "unit": "GB/s", "ms_per_step": c4["ms_per_step"],
+                       "eager_per_forward_achieved": c4["roofline"]["achieved"], "avg_forward_ms": c4["roofline"]["avg_launch_ms"]},
+        "cases": table,
+    })
+    torch.cuda.empty_cache()
+    c3 = measure_other(args, dev, 3, 10, 3)
+    out.append({"workload": c3["config"]["workload"], "value": c3["value"], "unit": "TFLOP/s", "ms_per_step": c3["ms_per_step"],
+                **c3["roofline"]})
+    torch.cuda.empty_cache()
+    return out
 
 
 if __name__ == "__main__":

@@ -107,10 +107,12 @@ int xq_set_persistent_tiles(int enabled);
 /* xq_mlp_fwd on block-fp8 weights runs gate and up either as two launches followed by one pass that writes h = SwiGLU and
  * forms the down projection's low-rank intermediate on the way (enabled = 0, the default), or as ONE launch over both weights
  * with the SwiGLU in its epilogue (enabled = 1).  Same outputs and saved activations bit for bit; the saved low-rank
- * intermediates of gate and up are laid out differently, so the switch must not change between a forward and its backward.
+ * intermediates of gate and up are laid out differently, which xq_mlp_saved::gate_up_fused records for the backward: the
+ * switch is only the default of a forward whose struct does not say (a negative field) and may change at any time.
  * A process-wide switch for tests and A/B measurements (XQ_MLP_GU in the environment sets it at load time); no counterpart
  * in the reference. */
 int xq_set_mlp_gate_up_fused(int enabled);
+int xq_get_mlp_gate_up_fused(void);   /* the current default: 0 or 1 */
 
 /* xq_linear_fwd with M <= 16 rows runs as ONE launch where the shape and the LoRA operands allow it (FLAT weight,
  * K % 512 == 0 for block_fp8 / K % 1024 == 0 for the 4-bit formats, K <= 12288; fp32 factors with r <= 16, r % 4 == 0,
@@ -133,6 +135,16 @@ int xq_set_skinny_spin_limit(int limit);
 /* Clears the library's slots on the current device (launch counts, failure marks, published parts).  Synchronises the
  * device before and after: call it with no forward in flight.  No counterpart in the reference. */
 int xq_skinny_reset(void);
+/* What the one-launch skinny forwards on the current device have reported since the last call.  *gave_up: blocks whose
+ * bounded wait gave up (each wrote NaN to its outputs); *failed_slots: slots marked failed (every forward through such a
+ * slot writes NaN).  Either pointer may be NULL.  The call waits for `stream`, reads a few words back and, if anything was
+ * found, waits for the whole device and clears the marks and the count, so that later forwards are exact again: a host
+ * calls it where it waits for results anyway (before it reads sampled tokens, say) and treats a non-zero report as "the
+ * forwards since the last call may hold NaN".  The slots are a fixed pool (256 per device) keyed by workspace pointer: a
+ * slot that a HIP-graph capture recorded stays with its workspace for good, another one changes hands only after the
+ * stream of its last launch has run dry, and a forward that can get no slot runs the two-launch organisation instead.
+ * No counterpart in the reference. */
+int xq_skinny_status(int* gave_up, int* failed_slots, void* stream);
 
 /* ---- decode ------------------------------------------------------------
  * out[e] = decoded weight of expert e, shape [rows, cols], bf16 or fp32.
@@ -483,6 +495,13 @@ typedef struct xq_mlp_saved {
     void* h;
     void* su_gate_up;
     void* su_down;
+    /* How the forward ran gate and up, which fixes the layout of su_gate_up.  On entry to xq_mlp_fwd: < 0 lets the
+     * process-wide default decide (xq_set_mlp_gate_up_fused), 0 asks for two launches, 1 for one launch with the SwiGLU in
+     * its epilogue (block-fp8 gate and up only; otherwise two).  On return: 0 or 1, what was done.  xq_mlp_bwd reads it --
+     * hand it the struct the forward filled (or the same value) -- and rejects anything else; the process-wide switch
+     * plays no part in a backward. */
+    int32_t gate_up_fused;
+    int32_t reserved;
 } xq_mlp_saved;
 
 typedef struct xq_mlp_grads {
@@ -492,7 +511,7 @@ typedef struct xq_mlp_grads {
 
 int64_t xq_mlp_workspace_bytes(int64_t M, int64_t hidden, int64_t intermediate, int r, int backward);
 int xq_mlp_fwd(const xq_weight* gate, const xq_weight* up, const xq_weight* down, const xq_mlp_lora* lora,
-               const void* x, int64_t ldx, int64_t M, void* y, int64_t ldy, const xq_mlp_saved* saved,
+               const void* x, int64_t ldx, int64_t M, void* y, int64_t ldy, xq_mlp_saved* saved,
                void* workspace, int64_t workspace_bytes, void* stream);
 int xq_mlp_bwd(const xq_weight* gate, const xq_weight* up, const xq_weight* down, const xq_mlp_lora* lora,
                const void* x, int64_t ldx, const void* dy, int64_t lddy, int64_t M, const xq_mlp_saved* saved,

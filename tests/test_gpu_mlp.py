@@ -158,3 +158,51 @@ def test_fused_mlp_under_torch_compile(hip_device, backend):
     got = run(torch.compile(qlora_mlp_forward, backend=backend, fullgraph=True))
     for a, b in zip(ref, got):
         assert torch.equal(a, b)
+
+
+def test_gate_up_form_travels_with_the_saved_state(hip_device):
+    """The form a forward ran gate and up in (one launch or two) fixes the layout of the saved low-rank intermediates;
+    it travels to the backward in xq_mlp_saved, so flipping the process-wide default between a forward and its backward
+    changes nothing: every gradient equals the undisturbed step's bit for bit, in both directions of the flip."""
+    from xorl_amd import _C
+    from xorl_amd.qlora import qlora_mlp_forward
+
+    M, H, I, r = 384, 512, 768, 16
+    mods, _ = _mods("block_fp8", H, I, r, hip_device, bias=False, seed=77)
+    x = gen((M, H), 1.0, 91, torch.bfloat16)
+    dy = gen((M, H), 1.0, 92, torch.bfloat16)
+    L = _C.lib()
+
+    def step(fwd_mode, bwd_mode):
+        _zero(mods)
+        _C.check(L.xq_set_mlp_gate_up_fused(fwd_mode))
+        xd = x.to(hip_device).requires_grad_(True)
+        y = qlora_mlp_forward(mods["gate"], mods["up"], mods["down"], xd)
+        _C.check(L.xq_set_mlp_gate_up_fused(bwd_mode))
+        y.backward(dy.to(hip_device))
+        return {"y": y.detach().clone(), "dx": xd.grad.clone(), **_grads(mods)}
+
+    try:
+        base = step(0, 0)
+        for fwd_mode, bwd_mode in ((0, 1), (1, 0), (1, 1)):
+            got = step(fwd_mode, bwd_mode)
+            for name in base:
+                assert torch.equal(got[name], base[name]), (fwd_mode, bwd_mode, name)
+    finally:
+        _C.check(L.xq_set_mlp_gate_up_fused(0))
+
+
+def test_mlp_backward_rejects_a_saved_state_without_its_form(hip_device):
+    """xq_mlp_bwd takes the form from the struct the forward filled; a struct that does not say (negative) is an argument error."""
+    import ctypes
+    from xorl_amd import _C
+    from xorl_amd import functional as F
+
+    M, H, I, r = 128, 256, 256, 16
+    mods, _ = _mods("block_fp8", H, I, r, hip_device, bias=False, seed=5)
+    banks = tuple(mods[k]._forward_quant_weight() for k in ("gate", "up", "down"))
+    factors = tuple(t.detach().contiguous() for k in ("gate", "up", "down") for t in (mods[k].lora_A, mods[k].lora_B))
+    x = gen((M, H), 1.0, 3, torch.bfloat16).to(hip_device)
+    y, saved = F._mlp_fwd_impl(x, factors, (None, None, None), banks, r, 2.0, 0)
+    with pytest.raises(ValueError, match="gate_up_fused"):
+        F._mlp_bwd_impl(torch.ones_like(y), x, saved, factors, banks, r, 2.0, True, -1)

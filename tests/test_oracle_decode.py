@@ -305,9 +305,16 @@ def test_fp8_decode_against_reference_held_restatement(shape):
     assert np.array_equal(b16, _bf16_bits(ref))
     p2, b2 = NP.fp8_decode(wb, s, R, Cc)
     assert np.array_equal(p2.view(np.uint32), p.view(np.uint32)) and np.array_equal(b2, b16)
-    # transposed scale grid must fail on a non-square case
+    # a scale grid indexed the other way round (block (k, n) in place of (n, k)) must change the result: decoding the
+    # transposed matrix with the transposed grid gives the transpose, with the untransposed grid (same element count,
+    # read in the wrong order) it does not
     if s.shape[0] != s.shape[1]:
-        assert s.T.shape != s.shape
+        wt = np.ascontiguousarray(wb.T)
+        pt, _ = C.fp8_decode(wt, np.ascontiguousarray(s.T), Cc, R)
+        assert np.array_equal(pt.view(np.uint32), np.ascontiguousarray(p.T).view(np.uint32))
+        if min(s.shape) > 1:      # (a grid of one row or column reads the same in either order)
+            wrong, _ = C.fp8_decode(wt, s.reshape(s.shape[1], s.shape[0]), Cc, R)
+            assert not np.array_equal(wrong.view(np.uint32), pt.view(np.uint32))
 
 
 def test_fp8_closed_form_fixture():

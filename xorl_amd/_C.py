@@ -71,7 +71,8 @@ class XqMlpLora(ctypes.Structure):
 
 
 class XqMlpSaved(ctypes.Structure):
-    _fields_ = [(n, ctypes.c_void_p) for n in ("gate_up", "h", "su_gate_up", "su_down")]
+    _fields_ = [(n, ctypes.c_void_p) for n in ("gate_up", "h", "su_gate_up", "su_down")] + [
+        ("gate_up_fused", ctypes.c_int32), ("reserved", ctypes.c_int32)]
 
 
 class XqMlpGrads(ctypes.Structure):
@@ -126,9 +127,12 @@ _SIGNATURES = {
     "xq_set_tile_policy": (_INT, [_INT]),
     "xq_set_persistent_tiles": (_INT, [_INT]),
     "xq_set_mlp_gate_up_fused": (_INT, [_INT]),
+    "xq_get_mlp_gate_up_fused": (_INT, []),
     "xq_set_skinny_one_launch": (_INT, [_INT]),
     "xq_set_skinny_spin_limit": (_INT, [_INT]),
     "xq_skinny_reset": (_INT, []),
+    # gave_up, failed_slots, stream
+    "xq_skinny_status": (_INT, [_P, _P, _P]),
     "xq_route_workspace_bytes": (_I64, [_I64, _I32]),
     # selected, n_routed, E, counts, offsets, scatter_index, tile_offsets, ws, ws_bytes, stream
     "xq_route_build": (_INT, [_P, _I64, _I32, _P, _P, _P, _P, _P, _I64, _P]),

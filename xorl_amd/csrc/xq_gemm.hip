@@ -405,6 +405,14 @@ extern "C" int xq_set_skinny_spin_limit(int limit) {
 
 extern "C" int xq_skinny_reset(void) { return reset_skinny_rows_slots(); }
 
+extern "C" int xq_skinny_status(int* gave_up, int* failed_slots, void* stream) {
+    int a = 0, b = 0;
+    const int rc = skinny_rows_status(&a, &b, (hipStream_t)stream);
+    if (gave_up) *gave_up = a;
+    if (failed_slots) *failed_slots = b;
+    return rc;
+}
+
 extern "C" int xq_set_persistent_tiles(int enabled) {
     g_persist = enabled != 0;
     return XQ_OK;
@@ -542,10 +550,12 @@ extern "C" int xq_linear_fwd_swiglu(const xq_weight* w, const void* x, int64_t l
         const bool timed = xq_profile_mark_begin(stream, bytes);
         rc = launch_skinny_rows_swiglu(w, (const bf16_t*)x, ldx, M, lora_A, lora_B, r, scaling, (const bf16_t*)bias_bf16, (bf16_t*)h, ldh,
                                        workspace, stream);
-        if (timed) xq_profile_mark_end(stream);
-        if (rc) return rc;
-        XQ_CHECK_LAUNCH("skinny forward with SwiGLU");
-        return XQ_OK;
+        if (rc != XQ_ERR_UNSUPPORTED) {      // (unsupported: no slot for the low-rank exchange could be had; nothing was launched)
+            if (timed) xq_profile_mark_end(stream);
+            if (rc) return rc;
+            XQ_CHECK_LAUNCH("skinny forward with SwiGLU");
+            return XQ_OK;
+        }
     }
     // otherwise the forward into the workspace, then the elementwise kernel
     const int64_t lin = align256(xq_linear_workspace_bytes(M, N2, K, r));
@@ -602,10 +612,12 @@ extern "C" int xq_linear_fwd_multi(const xq_linear_job* jobs, int n_jobs, const 
         if (ok && skinny_rows_multi_supported(rj, n_jobs, M, lora_dtype)) {
             const bool timed = xq_profile_mark_begin(stream, bytes);
             const int rc = launch_skinny_rows_multi(rj, n_jobs, (const bf16_t*)x, ldx, M, workspace, stream);
-            if (timed) xq_profile_mark_end(stream);
-            if (rc) return rc;
-            XQ_CHECK_LAUNCH("skinny forwards");
-            return XQ_OK;
+            if (rc != XQ_ERR_UNSUPPORTED) {  // (unsupported: no slots for the low-rank exchange could be had; nothing was launched)
+                if (timed) xq_profile_mark_end(stream);
+                if (rc) return rc;
+                XQ_CHECK_LAUNCH("skinny forwards");
+                return XQ_OK;
+            }
         }
     }
     // otherwise one after the other (the workspace is reused: the launches are ordered by the stream)

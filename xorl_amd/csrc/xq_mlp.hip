@@ -56,21 +56,24 @@ __global__ void __launch_bounds__(256) add_rows_kernel(bf16_t* a, int64_t lda, c
 // gate and up of a block-fp8 MLP as ONE launch with the SwiGLU in its epilogue (1), or as two launches followed by the pass
 // that writes h and forms s * h . A_d^T on the way (0, the default: the two plain launches run at a higher rate than the
 // launch with the wide epilogue, and the step is level or slightly shorter).  XQ_MLP_GU in the environment sets it at load
-// time, xq_set_mlp_gate_up_fused() at run time; the layout of the saved low-rank intermediates follows it, so it must not
-// change between a forward and its backward.
+// time, xq_set_mlp_gate_up_fused() at run time.  It is only the default of a forward: xq_mlp_saved::gate_up_fused carries the
+// form a forward used (or was asked for) to its backward, which lays out the saved low-rank intermediates by that field.
 static std::atomic<int> g_mlp_gu{[] { const char* e = getenv("XQ_MLP_GU"); return e ? atoi(e) : 0; }()};
 // XQ_MLP_SILU_NT=0: the SwiGLU backward and the two low-rank products of its outputs as three launches (A/B measurements;
 // same bits either way)
 static const int g_mlp_silu_nt = [] { const char* e = getenv("XQ_MLP_SILU_NT"); return e ? atoi(e) : 1; }();
-bool fuse_gate_up_fwd(const xq_weight* gate, const xq_weight* up) { return g_mlp_gu && gate->format == XQ_FMT_FP8 && up->format == XQ_FMT_FP8; }
+// `asked`: xq_mlp_saved::gate_up_fused on entry to the forward (< 0: the process-wide default decides)
+bool fuse_gate_up_fwd(const xq_weight* gate, const xq_weight* up, int asked) {
+    return (asked < 0 ? g_mlp_gu.load() != 0 : asked != 0) && gate->format == XQ_FMT_FP8 && up->format == XQ_FMT_FP8;
+}
 
 // Where the two low-rank intermediates lie in su_gate_up (M * 2 * rp elements): as the column bands [0, rp) and
 // [rp, 2 rp) of one [M, 2 rp] matrix when the fused gate / up launch reads them, else as two packed [M, rp] matrices.
 struct SuLayout {
     int64_t up_offset, pitch;
 };
-SuLayout su_layout(const xq_weight* gate, const xq_weight* up, int rp, int64_t M) {
-    if (fuse_gate_up_fwd(gate, up)) return {rp, 2 * (int64_t)rp};
+SuLayout su_layout(bool fused_fwd, int rp, int64_t M) {
+    if (fused_fwd) return {rp, 2 * (int64_t)rp};
     return {M * rp, rp};
 }
 
@@ -128,6 +131,8 @@ extern "C" int xq_set_mlp_gate_up_fused(int enabled) {
     return XQ_OK;
 }
 
+extern "C" int xq_get_mlp_gate_up_fused(void) { return g_mlp_gu.load() != 0; }
+
 extern "C" int64_t xq_mlp_workspace_bytes(int64_t M, int64_t hidden, int64_t intermediate, int r, int backward) {
     if (M < 0 || r < 0) return 0;
     Dims d{M, hidden, intermediate, r, r_pad_of(r)};
@@ -135,12 +140,14 @@ extern "C" int64_t xq_mlp_workspace_bytes(int64_t M, int64_t hidden, int64_t int
 }
 
 extern "C" int xq_mlp_fwd(const xq_weight* gate, const xq_weight* up, const xq_weight* down, const xq_mlp_lora* lora,
-                          const void* x_, int64_t ldx, int64_t M, void* y, int64_t ldy, const xq_mlp_saved* saved,
+                          const void* x_, int64_t ldx, int64_t M, void* y, int64_t ldy, xq_mlp_saved* saved,
                           void* workspace, int64_t workspace_bytes, void* stream_) {
     static const char* who = "xq_mlp_fwd";
     Dims d;
     int rc = check_call(gate, up, down, lora, M, saved, who, &d);
     if (rc) return rc;
+    const bool fused = fuse_gate_up_fwd(gate, up, saved->gate_up_fused);
+    saved->gate_up_fused = fused ? 1 : 0;       // what the backward must be told
     if (M == 0) return XQ_OK;
     XQ_REQUIRE(x_ && y, "%s: NULL activation pointer", who);
     XQ_REQUIRE(workspace && xq_aligned(workspace, 256) && workspace_bytes >= fwd_workspace(d),
@@ -155,8 +162,7 @@ extern "C" int xq_mlp_fwd(const xq_weight* gate, const xq_weight* up, const xq_w
     bf16_t *su_gu = (bf16_t*)saved->su_gate_up, *su_d = (bf16_t*)saved->su_down;
     Carve cv{(uint8_t*)workspace, 0};
     bf16_t *A_gu = nullptr, *Bl_g = nullptr, *Bl_u = nullptr, *A_d = nullptr, *Bl_d = nullptr;
-    const bool fused = fuse_gate_up_fwd(gate, up);
-    const SuLayout sl = su_layout(gate, up, rp, M);
+    const SuLayout sl = su_layout(fused, rp, M);
     const bool one_pass = fused && rp > 0 && 2 * rp <= 64;      // both low-rank intermediates from one pass over x
     if (rp) {
         // panels: [A_g ; A_u] as [2 rp, H] (the rows of x . A^T), B as [out, rp] right-hand panels
@@ -222,7 +228,7 @@ extern "C" int xq_mlp_fwd_infer(const xq_weight* gate, const xq_weight* up, cons
     Dims d;
     Carve cv{(uint8_t*)workspace, 0};
     // (the argument checks are those of xq_mlp_fwd; the buffers it would keep for a backward live in the workspace here)
-    xq_mlp_saved tmp{workspace, workspace, workspace, workspace};
+    xq_mlp_saved tmp{workspace, workspace, workspace, workspace, 0, 0};
     int rc = check_call(gate, up, down, lora, M, &tmp, who, &d);
     if (rc) return rc;
     if (M == 0) return XQ_OK;
@@ -253,6 +259,9 @@ extern "C" int xq_mlp_bwd(const xq_weight* gate, const xq_weight* up, const xq_w
     if (rc) return rc;
     const int r = d.r, rp = d.rp;
     const int64_t H = d.H, I = d.I;
+    XQ_REQUIRE(saved->gate_up_fused == 0 || (saved->gate_up_fused == 1 && gate->format == XQ_FMT_FP8 && up->format == XQ_FMT_FP8),
+               "%s: xq_mlp_saved::gate_up_fused is %d: pass the struct the forward filled (0 or 1; 1 only for block-fp8 gate and up)", who,
+               saved->gate_up_fused);
     XQ_REQUIRE(rp == 0 || grads, "%s: grads is NULL", who);
     if (rp) for (int p = 0; p < 3; ++p) XQ_REQUIRE(grads->dA[p] && grads->dB[p], "%s: a factor gradient buffer is NULL", who);
     hipStream_t stream = (hipStream_t)stream_;
@@ -326,7 +335,7 @@ extern "C" int xq_mlp_bwd(const xq_weight* gate, const xq_weight* up, const xq_w
             if ((rc = launch_small_nt(dgate, 2 * I, M, I, Bt_g, rp, s, v_g, nullptr, nullptr, 1, true, stream, ld_v))) return rc;
             if ((rc = launch_small_nt(dup, 2 * I, M, I, Bt_u, rp, s, v_u, nullptr, nullptr, 1, true, stream, ld_v))) return rc;
         }
-        const SuLayout sl = su_layout(gate, up, rp, M);
+        const SuLayout sl = su_layout(saved->gate_up_fused == 1, rp, M);
         if ((rc = launch_tn(dgate, 2 * I, I, su_gu, rp, r, M, false, grads->dB[0], part, nullptr, 1, stream, nullptr, sl.pitch))) return rc;        // [I, r]
         if ((rc = launch_tn(dup, 2 * I, I, su_gu + sl.up_offset, rp, r, M, false, grads->dB[1], part, nullptr, 1, stream, nullptr, sl.pitch))) return rc;
         if (fused) {       // [2 rp, H] = [v_g | v_u]^T . x, then its two bands

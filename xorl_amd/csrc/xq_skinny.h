@@ -52,6 +52,7 @@ void set_skinny_rows(int enabled);
 bool skinny_rows_enabled();
 void set_skinny_rows_spin_limit(int limit);   // <= 0: the default
 int reset_skinny_rows_slots();                 // clears the current device's slots (synchronises the device)
+int skinny_rows_status(int* gave_up, int* failed_slots, hipStream_t stream);   // reads and clears the failure reports (synchronises the stream)
 
 // ---- one-launch organisation (xq_skinny_rows.hip)
 // true when the shape, format and LoRA operands fit it; the caller falls back to the split organisation otherwise

@@ -52,7 +52,7 @@ constexpr int kSlotCtl = kSuMaxParts * 256 * 2; // word index of the control wor
 constexpr int kCtlCopies = 32;                  // `gen` and `started` exist 32 times, 128 bytes apart: block b uses copy b % 32,
 constexpr int kCtlStride = 32;                  // so that a launch's 256 blocks do not queue on one memory location
 constexpr int kSlotWords = kSlotCtl + 2 * kCtlCopies * kCtlStride;   // [parts][256] pairs (sum bits, tag), gen copies, started copies
-constexpr int kSlots = 64;
+constexpr int kSlots = 256;
 constexpr int kRowsSpinLimit = 1 << 20;
 constexpr uint32_t kGenPoison = 0xFFFFFFFFu;   // launch count of a slot in which a wait has given up: see the closer below
 #ifndef XQ_ROWS_LOADS_IN_FLIGHT
@@ -79,6 +79,7 @@ struct SkinnyRowsArgs {
     int32_t nsu;                   // su parts (K / 512), 0 without a low-rank term
     uint32_t* slot;                // [nsu][256] published (sum, tag) pairs, then the copies of gen and of started
     int32_t spin_limit;
+    uint32_t* fail;                // the device's count of blocks whose wait gave up (they wrote NaN): read by skinny_rows_status
 };
 
 // FMT: weight format; G: 16-row groups in flight per block; NJ: most load steps per wave (a step is one 16-byte load
@@ -512,6 +513,8 @@ __device__ __forceinline__ void skinny_rows_body(const SkinnyRowsArgs& g, const 
         // NaN, until the host clears the library's slots (reset_skinny_rows_slots).  Never values from stale sums.
         if (open && lane < kCtlCopies)
             __hip_atomic_store(g.slot + kSlotCtl + lane * kCtlStride, kGenPoison, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        // a block that is about to write NaN says so where the host can see it (no return value asked for)
+        if ((missing || open) && lane == 0) __hip_atomic_fetch_add(g.fail, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
             const int j = 4 * (lane >> 4) + q, m = lane & 15;
@@ -609,16 +612,23 @@ __global__ void __launch_bounds__(512, 1) skinny_rows_multi_kernel(int32_t first
 // ---- slots: device memory that belongs to the library (zero when the code object is loaded).
 // Each device holds its own copy of the array at its own address, reached through hipGetSymbolAddress with that device
 // current.  A slot is tied to the caller's scratch pointer, so calls that may legally overlap (different workspaces)
-// never share one; with more than kSlots scratch pointers in use the least recently used slot changes hands, which is
-// safe as long as fewer than kSlots calls with distinct workspaces are in flight on a device at once.
-static __device__ __align__(256) uint32_t rows_slots[kSlots * kSlotWords];
+// never share one.  A slot changes hands only when nothing can still refer to it: a slot used by a launch that was
+// recorded into a HIP graph stays with its key for good (the graph holds its address), and another slot is taken over
+// only once the stream of its last launch has run dry.  When no slot can be had that way the caller takes the
+// two-launch organisation, which needs none.  The word behind the slots counts the blocks whose bounded wait gave up.
+static __device__ __align__(256) uint32_t rows_slots[kSlots * kSlotWords + 64];
 
 namespace {
 constexpr int kMaxDevices = 64;
+struct SlotHost {
+    const void* key;
+    uint64_t used;          // 0: never used
+    hipStream_t stream;     // stream of the last launch through the slot
+    bool pinned;            // a captured launch refers to it
+};
 std::mutex g_slots_mu;
 uint32_t* g_slots_ptr[kMaxDevices] = {};
-const void* g_slot_key[kMaxDevices][kSlots] = {};
-uint64_t g_slot_used[kMaxDevices][kSlots] = {};
+SlotHost g_slot[kMaxDevices][kSlots] = {};
 uint64_t g_slot_clock = 0;
 }  // namespace
 
@@ -627,15 +637,14 @@ uint64_t g_slot_clock = 0;
 static std::atomic<int> g_rows_spin_limit{kRowsSpinLimit};
 void set_skinny_rows_spin_limit(int limit) { g_rows_spin_limit = limit > 0 ? limit : kRowsSpinLimit; }
 
-// the slot of `key` on the current device
-static int rows_slot(const void* key, uint32_t** out) {
+// the slot array of the current device (address resolved once per device); g_slots_mu held by the caller
+static int rows_slots_base(int* dev_out, uint32_t** base) {
     int dev = -1;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
         xq_set_error("xq_linear_fwd: cannot identify the current device: %s", hipGetErrorString(e));
         return XQ_ERR_LAUNCH;
     }
-    std::lock_guard<std::mutex> lock(g_slots_mu);
     if (!g_slots_ptr[dev]) {
         void* p = nullptr;
         e = hipGetSymbolAddress(&p, HIP_SYMBOL(rows_slots));
@@ -645,42 +654,118 @@ static int rows_slot(const void* key, uint32_t** out) {
         }
         g_slots_ptr[dev] = (uint32_t*)p;
     }
-    int s = -1, oldest = 0;
-    for (int i = 0; i < kSlots; ++i) {
-        if (g_slot_used[dev][i] && g_slot_key[dev][i] == key) s = i;
-        if (g_slot_used[dev][i] < g_slot_used[dev][oldest]) oldest = i;    // a never-used slot (0) is older than any used one
-    }
-    if (s < 0) {
-        s = oldest;
-        g_slot_key[dev][s] = key;
-    }
-    g_slot_used[dev][s] = ++g_slot_clock;
-    *out = g_slots_ptr[dev] + (size_t)s * kSlotWords;
+    *dev_out = dev;
+    *base = g_slots_ptr[dev];
     return XQ_OK;
 }
 
-// Clears the slots of the current device (launch counts, marks of failed waits, published parts): for a host that has
-// seen NaN outputs after a forced or real give-up.  Waits for the device before and after; no forward may be in flight.
-int reset_skinny_rows_slots() {
-    uint32_t* slot = nullptr;
-    int rc = rows_slot(nullptr, &slot);       // resolves the array's address on this device (the null key takes a slot like any other)
-    if (rc) return rc;
+// The slot of `key` on the current device for a launch on `stream`, and the device's failure counter.
+// XQ_ERR_UNSUPPORTED (no message): every slot belongs to another key and none of them can be shown to be idle.
+static int rows_slot(const void* key, hipStream_t stream, uint32_t** out, uint32_t** fail) {
+    std::lock_guard<std::mutex> lock(g_slots_mu);
     int dev = 0;
-    hipError_t e = hipGetDevice(&dev);
-    if (e == hipSuccess) e = hipDeviceSynchronize();
-    if (e == hipSuccess) {
-        std::lock_guard<std::mutex> lock(g_slots_mu);
-        e = hipMemset(g_slots_ptr[dev], 0, sizeof(uint32_t) * (size_t)kSlots * kSlotWords);
-        for (int i = 0; i < kSlots; ++i) {
-            g_slot_key[dev][i] = nullptr;
-            g_slot_used[dev][i] = 0;
+    uint32_t* base = nullptr;
+    int rc = rows_slots_base(&dev, &base);
+    if (rc) return rc;
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &cap) != hipSuccess) {
+        (void)hipGetLastError();
+        cap = hipStreamCaptureStatusNone;
+    }
+    const bool capturing = cap != hipStreamCaptureStatusNone;
+    SlotHost* tab = g_slot[dev];
+    int s = -1;
+    for (int i = 0; i < kSlots && s < 0; ++i)
+        if (tab[i].used && tab[i].key == key) s = i;
+    for (int i = 0; i < kSlots && s < 0; ++i)
+        if (!tab[i].used) s = i;
+    if (s < 0) {
+        // Least recently used first.  A slot whose last launch went to this same stream can be taken over at once: the
+        // stream runs its launches one after the other.  One last used on another stream only when that stream has run
+        // dry (a host-side look, no work is enqueued; not while capturing: queries are not capture-safe everywhere).
+        for (int tries = 0; tries < 8 && s < 0; ++tries) {
+            int oldest = -1;
+            for (int i = 0; i < kSlots; ++i)
+                if (!tab[i].pinned && (oldest < 0 || tab[i].used < tab[oldest].used)) oldest = i;
+            if (oldest < 0) break;
+            if (tab[oldest].stream == stream) {
+                s = oldest;
+            } else if (!capturing) {
+                const hipError_t q = hipStreamQuery(tab[oldest].stream);
+                if (q == hipSuccess) s = oldest;
+                else if (q != hipErrorNotReady) (void)hipGetLastError();
+            }
+            if (s < 0) tab[oldest].used = ++g_slot_clock;      // busy elsewhere: look at the next oldest
         }
+    }
+    if (s < 0) return XQ_ERR_UNSUPPORTED;
+    tab[s].key = key;
+    tab[s].used = ++g_slot_clock;
+    tab[s].stream = stream;
+    tab[s].pinned = tab[s].pinned || capturing;
+    *out = base + (size_t)s * kSlotWords;
+    *fail = base + (size_t)kSlots * kSlotWords;
+    return XQ_OK;
+}
+
+// Clears the slots of the current device (launch counts, marks of failed waits, published parts, the failure count): for
+// a host that has seen NaN outputs after a forced or real give-up.  Waits for the device before and after; no forward may
+// be in flight, and graphs that captured a one-launch forward keep their slots' addresses (the cleared slot works on).
+int reset_skinny_rows_slots() {
+    std::lock_guard<std::mutex> lock(g_slots_mu);
+    int dev = 0;
+    uint32_t* base = nullptr;
+    int rc = rows_slots_base(&dev, &base);
+    if (rc) return rc;
+    hipError_t e = hipDeviceSynchronize();
+    if (e == hipSuccess) e = hipMemset(base, 0, sizeof(uint32_t) * ((size_t)kSlots * kSlotWords + 64));
+    if (e == hipSuccess) {
+        for (int i = 0; i < kSlots; ++i)
+            if (!g_slot[dev][i].pinned) g_slot[dev][i] = SlotHost{};
     }
     if (e == hipSuccess) e = hipDeviceSynchronize();
     if (e != hipSuccess) {
         xq_set_error("xq_skinny_reset: %s", hipGetErrorString(e));
         return XQ_ERR_LAUNCH;
     }
+    return XQ_OK;
+}
+
+// What the one-launch forwards of the current device have reported since the last call: blocks whose bounded wait gave up
+// (each wrote NaN outputs) and slots marked failed (every forward through such a slot writes NaN).  Waits for `stream`,
+// reads a few words back, and, when anything was found, waits for the whole device, clears the marks and the count, so
+// that later forwards are exact again.  Costs one stream synchronisation: for the points where the host waits anyway.
+int skinny_rows_status(int* gave_up, int* failed_slots, hipStream_t stream) {
+    *gave_up = 0;
+    *failed_slots = 0;
+    std::lock_guard<std::mutex> lock(g_slots_mu);
+    int dev = 0;
+    uint32_t* base = nullptr;
+    int rc = rows_slots_base(&dev, &base);
+    if (rc) return rc;
+    uint32_t count = 0, gens[kSlots];
+    hipError_t e = hipStreamSynchronize(stream);
+    if (e == hipSuccess) e = hipMemcpy(&count, base + (size_t)kSlots * kSlotWords, 4, hipMemcpyDeviceToHost);
+    if (e == hipSuccess)
+        e = hipMemcpy2D(gens, 4, base + kSlotCtl, sizeof(uint32_t) * (size_t)kSlotWords, 4, kSlots, hipMemcpyDeviceToHost);
+    int bad = 0;
+    if (e == hipSuccess) {
+        for (int i = 0; i < kSlots; ++i) bad += gens[i] == kGenPoison;
+        if (bad || count) {
+            e = hipDeviceSynchronize();
+            for (int i = 0; i < kSlots && e == hipSuccess; ++i)
+                if (gens[i] == kGenPoison)      // the whole slot: parts of the failed launch must not meet a launch count that starts over
+                    e = hipMemset(base + (size_t)i * kSlotWords, 0, sizeof(uint32_t) * (size_t)kSlotWords);
+            if (e == hipSuccess) e = hipMemset(base + (size_t)kSlots * kSlotWords, 0, 4);
+            if (e == hipSuccess) e = hipDeviceSynchronize();
+        }
+    }
+    if (e != hipSuccess) {
+        xq_set_error("xq_skinny_status: %s", hipGetErrorString(e));
+        return XQ_ERR_LAUNCH;
+    }
+    *gave_up = (int)(count > 0x7fffffffu ? 0x7fffffffu : count);
+    *failed_slots = bad;
     return XQ_OK;
 }
 
@@ -809,7 +894,8 @@ static int launch_rows_fmt(const SkinnyRowsArgs& g, const SkinnyRowsBatch* batch
 }
 
 static int rows_args(const xq_weight* w, const RowsPlan& p, const bf16_t* x, int64_t ldx, int64_t M, const void* lora_A, const void* lora_B,
-                     int r, float scaling, const bf16_t* bias, bf16_t* y, int64_t ldy, const void* slot_key, SkinnyRowsArgs* out) {
+                     int r, float scaling, const bf16_t* bias, bf16_t* y, int64_t ldy, const void* slot_key, hipStream_t stream,
+                     SkinnyRowsArgs* out) {
     SkinnyRowsArgs& g = *out;
     g.x = x; g.ldx = ldx; g.M = (int)M; g.N = (int)w->rows; g.K = (int)w->cols;
     g.packed = (const uint8_t*)w->packed; g.scales = (const uint8_t*)w->scales; g.global_scale = w->global_scale;
@@ -822,7 +908,8 @@ static int rows_args(const xq_weight* w, const RowsPlan& p, const bf16_t* x, int
     g.nsu = r > 0 ? (int)(w->cols / kSuPartK) : 0;
     g.slot = nullptr;
     g.spin_limit = g_rows_spin_limit.load();
-    if (r > 0) return rows_slot(slot_key, &g.slot);
+    g.fail = nullptr;
+    if (r > 0) return rows_slot(slot_key, stream, &g.slot, &g.fail);
     return XQ_OK;
 }
 
@@ -831,7 +918,7 @@ int launch_skinny_rows(const xq_weight* w, const bf16_t* x, int64_t ldx, int64_t
     RowsPlan p;
     XQ_REQUIRE(rows_plan(w, M, &p), "xq_linear_fwd: internal error: shape not supported by the one-launch skinny kernel");
     SkinnyRowsArgs g;
-    const int rc = rows_args(w, p, x, ldx, M, lora_A, lora_B, r, scaling, bias, y, ldy, slot_key, &g);
+    const int rc = rows_args(w, p, x, ldx, M, lora_A, lora_B, r, scaling, bias, y, ldy, slot_key, stream, &g);
     if (rc) return rc;
     const unsigned grid = (unsigned)xq_cdiv(w->rows / 16, p.G * p.R);
     switch (w->format) {
@@ -881,7 +968,7 @@ int launch_skinny_rows_swiglu(const xq_weight* w, const bf16_t* x, int64_t ldx, 
     XQ_REQUIRE(rows_plan(w, M, &p) && p.R == 2 && p.G == 3 && ldx < (1ll << 31),
                "xq_linear_fwd_swiglu: internal error: shape not supported by the one-launch skinny kernel");
     SkinnyRowsArgs g;
-    const int rc = rows_args(w, p, x, ldx, M, lora_A, lora_B, r, scaling, bias, h, ldh, slot_key, &g);
+    const int rc = rows_args(w, p, x, ldx, M, lora_A, lora_B, r, scaling, bias, h, ldh, slot_key, stream, &g);
     if (rc) return rc;
     const unsigned grid = (unsigned)(w->rows / 2 / 48);
 #define XQ_GU_CASE(F, NN) \
@@ -927,7 +1014,7 @@ int launch_skinny_rows_multi(const SkinnyRowsJob* jobs, int n_jobs, const bf16_t
         }
         // each forward has a slot of its own: its key is a distinct address inside the caller's workspace
         const int rc = rows_args(ws[i], p, x, ldx, M, jobs[i].lora_A, jobs[i].lora_B, jobs[i].r, jobs[i].scaling, jobs[i].bias, jobs[i].y,
-                                 jobs[i].ldy, (const char*)slot_key + 256 * i, &b.job[i]);
+                                 jobs[i].ldy, (const char*)slot_key + 256 * i, stream, &b.job[i]);
         if (rc) return rc;
         first += (int)xq_cdiv(ws[i]->rows / 16, p.G * p.R);
     }

@@ -91,6 +91,41 @@ def _workspace_bytes(M: int, N: int, K: int, r: int) -> int:
     return v
 
 
+# ---- failure reports of the one-launch decode kernel (M <= 16 with a LoRA term).  Its blocks pass the low-rank
+# intermediate to each other through device memory with bounded waits; a wait that gives up writes NaN and counts itself
+# in device memory, where xq_skinny_status() finds it.  Reading the count waits for the stream, so it is done where the
+# host waits anyway: by the caller (`skinny_status()` next to its own synchronisation) and, as a backstop, here after
+# every SKINNY_CHECK_EVERY forward-only calls of at most 16 rows.
+SKINNY_CHECK_EVERY = 1024
+_skinny_calls = 0
+
+
+def skinny_status(device=None, raise_on_failure: bool = True) -> Tuple[int, int]:
+    """(blocks whose wait gave up, slots marked failed) reported by the one-launch decode forwards on `device` since the
+    last call; waits for the current stream.  Anything non-zero means forwards since the last call may hold NaN: the
+    library has then already cleared the marks (later forwards are exact again) and this raises ``RuntimeError`` unless
+    told not to."""
+    dev = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    gave_up, failed = ctypes.c_int(0), ctypes.c_int(0)
+    with torch.cuda.device(dev):
+        _C.check(_C.lib().xq_skinny_status(ctypes.byref(gave_up), ctypes.byref(failed), _C.stream_ptr(dev)))
+    if raise_on_failure and (gave_up.value or failed.value):
+        raise RuntimeError(f"xorl_amd: {gave_up.value} block(s) of one-launch decode forwards gave up waiting and wrote NaN "
+                           f"({failed.value} exchange slot(s) were marked failed) since the last check; the marks are cleared, "
+                           "repeat the affected forwards")
+    return gave_up.value, failed.value
+
+
+def _note_decode_forward(dev, M: int) -> None:
+    global _skinny_calls
+    if M > 16:
+        return
+    _skinny_calls += 1
+    if _skinny_calls >= SKINNY_CHECK_EVERY and not torch.cuda.is_current_stream_capturing():
+        _skinny_calls = 0
+        skinny_status(dev)
+
+
 def _linear_fwd_impl(x: Tensor, packed: Tensor, scales: Tensor, global_scale: Optional[Tensor],
                      lora_A: Optional[Tensor], lora_B: Optional[Tensor], bias: Optional[Tensor],
                      fmt: str, scale_dt: torch.dtype, group: int, N: int, K: int, r: int,
@@ -119,6 +154,8 @@ def _linear_fwd_impl(x: Tensor, packed: Tensor, scales: Tensor, global_scale: Op
     _C.check(_C.lib().xq_linear_fwd(ctypes.byref(w), x2.data_ptr(), _ld(x2), M, _C.ptr(A), _C.ptr(B), _lora_dt(A), r,
                                     scaling, _C.ptr(b), y.data_ptr(), N, su.data_ptr() if (rp and want_su) else None,
                                     ws.data_ptr(), ws_bytes, _C.stream_ptr(dev)))
+    if not want_su:
+        _note_decode_forward(dev, M)
     return y.reshape(*x.shape[:-1], N), su
 
 
@@ -294,6 +331,7 @@ def qlora_linear_swiglu(x: Tensor, qw: QuantWeight, lora_A: Optional[Tensor], lo
     cw = qw.c()
     _C.check(L.xq_linear_fwd_swiglu(ctypes.byref(cw), x2.data_ptr(), _ld(x2), M, _C.ptr(A), _C.ptr(B), _lora_dt(A), r if A is not None else 0,
                                     float(scaling), _C.ptr(b), h.data_ptr(), I, ws.data_ptr(), ws_bytes, _C.stream_ptr(dev)))
+    _note_decode_forward(dev, M)
     return h.reshape(*x.shape[:-1], I)
 
 
@@ -341,6 +379,7 @@ def qlora_linear_multi(x: Tensor, jobs) -> list:
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     _C.check(L.xq_linear_fwd_multi(arr, len(jobs), x2.data_ptr(), _ld(x2), M, lora_dt if lora_dt is not None else _C.XQ_DT_F32,
                                    ws.data_ptr(), ws_bytes, _C.stream_ptr(dev)))
+    _note_decode_forward(dev, M)
     return [y.reshape(*x.shape[:-1], y.shape[1]) for y in ys]
 
 
@@ -361,10 +400,24 @@ def _mlp_lora_struct(factors, biases, r: int, scaling: float) -> _C.XqMlpLora:
     return L
 
 
-def _mlp_saved_struct(saved) -> _C.XqMlpSaved:
+def _mlp_saved_struct(saved, gu: int) -> _C.XqMlpSaved:
     S = _C.XqMlpSaved()
     S.gate_up, S.h, S.su_gate_up, S.su_down = (t.data_ptr() for t in saved)
+    S.gate_up_fused = gu
     return S
+
+
+def _mlp_gate_up_mode(qg: QuantWeight, qu: QuantWeight) -> int:
+    """How a forward on these weights runs gate and up right now: 1 = one launch with the SwiGLU in its epilogue, 0 = two
+    launches (xq_mlp_saved::gate_up_fused).  Read once per forward and handed to the forward AND its backward, so the pair
+    agrees whatever xq_set_mlp_gate_up_fused() is called with in between."""
+    return int(bool(_mlp_gate_up_default()) and qg.fmt == "block_fp8" and qu.fmt == "block_fp8")
+
+
+@torch.compiler.assume_constant_result
+def _mlp_gate_up_default() -> int:
+    # (a constant of the traced graph under torch.compile: forward and backward of one trace get the same value)
+    return int(_C.lib().xq_get_mlp_gate_up_fused())
 
 
 def _mlp_workspace(dev, M: int, H: int, I: int, r: int, backward: bool) -> Tensor:
@@ -375,7 +428,7 @@ def _mlp_workspace(dev, M: int, H: int, I: int, r: int, backward: bool) -> Tenso
     return torch.empty(n, dtype=torch.uint8, device=dev)
 
 
-def _mlp_fwd_impl(x2: Tensor, factors, biases, banks, r: int, scaling: float):
+def _mlp_fwd_impl(x2: Tensor, factors, biases, banks, r: int, scaling: float, gu: int):
     """xq_mlp_fwd.  x2 bf16 [M, H]; factors (gA, gB, uA, uB, dA, dB) active views, contiguous (None at r == 0);
     biases three bf16 vectors or None; banks (gate, up, down) QuantWeight.  -> (y [M, H], four saved tensors)."""
     qg, qu, qd = banks
@@ -385,15 +438,17 @@ def _mlp_fwd_impl(x2: Tensor, factors, biases, banks, r: int, scaling: float):
     saved = (bf(M, 2 * I), bf(M, I), bf(M, 2 * rp), bf(M, rp))
     y = bf(M, H)
     ws = _mlp_workspace(dev, M, H, I, r, False)
-    lora, S = _mlp_lora_struct(factors, biases, r, scaling), _mlp_saved_struct(saved)
+    lora, S = _mlp_lora_struct(factors, biases, r, scaling), _mlp_saved_struct(saved, gu)
     wg, wu, wd = qg.c(), qu.c(), qd.c()
     _C.check(_C.lib().xq_mlp_fwd(ctypes.byref(wg), ctypes.byref(wu), ctypes.byref(wd), ctypes.byref(lora), x2.data_ptr(),
                                  _ld(x2), M, y.data_ptr(), H, ctypes.byref(S), ws.data_ptr(), ws.numel(),
                                  _C.stream_ptr(dev)))
+    if S.gate_up_fused != gu:
+        raise RuntimeError(f"xq_mlp_fwd ran gate and up in form {S.gate_up_fused}, asked for {gu}")
     return y, saved
 
 
-def _mlp_bwd_impl(dy2: Tensor, x2: Tensor, saved, factors, banks, r: int, scaling: float, need_dx: bool):
+def _mlp_bwd_impl(dy2: Tensor, x2: Tensor, saved, factors, banks, r: int, scaling: float, need_dx: bool, gu: int):
     """xq_mlp_bwd -> (dx [M, H] or empty, six fp32 factor gradients (empty at r == 0))."""
     qg, qu, qd = banks
     I, H = qg.rows, qg.cols
@@ -404,7 +459,7 @@ def _mlp_bwd_impl(dy2: Tensor, x2: Tensor, saved, factors, banks, r: int, scalin
     for p in range(3):
         G.dA[p], G.dB[p] = (grads[2 * p].data_ptr(), grads[2 * p + 1].data_ptr()) if r else (None, None)
     ws = _mlp_workspace(dev, M, H, I, r, True)
-    lora, S = _mlp_lora_struct(factors, (None, None, None), r, scaling), _mlp_saved_struct(saved)
+    lora, S = _mlp_lora_struct(factors, (None, None, None), r, scaling), _mlp_saved_struct(saved, gu)
     wg, wu, wd = qg.c(), qu.c(), qd.c()
     _C.check(_C.lib().xq_mlp_bwd(ctypes.byref(wg), ctypes.byref(wu), ctypes.byref(wd), ctypes.byref(lora), x2.data_ptr(),
                                  _ld(x2), dy2.data_ptr(), _ld(dy2), M, ctypes.byref(S), dx.data_ptr() if need_dx else None,
@@ -425,17 +480,17 @@ def _mlp_fwd_op(x: Tensor, factors: List[Tensor], biases: List[Optional[Tensor]]
                 g_packed: Tensor, g_scales: Tensor, g_gs: Optional[Tensor], g_fmt: str, g_code: int, g_group: int,
                 u_packed: Tensor, u_scales: Tensor, u_gs: Optional[Tensor], u_fmt: str, u_code: int, u_group: int,
                 d_packed: Tensor, d_scales: Tensor, d_gs: Optional[Tensor], d_fmt: str, d_code: int, d_group: int,
-                H: int, I: int, r: int, scaling: float) -> List[Tensor]:
+                H: int, I: int, r: int, scaling: float, gu: int) -> List[Tensor]:
     banks = (_qw_from(g_packed, g_scales, g_gs, g_fmt, g_code, g_group, I, H),
              _qw_from(u_packed, u_scales, u_gs, u_fmt, u_code, u_group, I, H),
              _qw_from(d_packed, d_scales, d_gs, d_fmt, d_code, d_group, H, I))
-    y, saved = _mlp_fwd_impl(x, tuple(factors) if r else (None,) * 6, tuple(biases), banks, r, scaling)
+    y, saved = _mlp_fwd_impl(x, tuple(factors) if r else (None,) * 6, tuple(biases), banks, r, scaling, gu)
     return [y, *saved]
 
 
 @_mlp_fwd_op.register_fake
 def _(x, factors, biases, g_packed, g_scales, g_gs, g_fmt, g_code, g_group, u_packed, u_scales, u_gs, u_fmt, u_code, u_group,
-      d_packed, d_scales, d_gs, d_fmt, d_code, d_group, H, I, r, scaling):
+      d_packed, d_scales, d_gs, d_fmt, d_code, d_group, H, I, r, scaling, gu):
     M, rp = x.shape[0], max(_r_pad(r), 16)
     return [x.new_empty(M, H), x.new_empty(M, 2 * I), x.new_empty(M, I), x.new_empty(M, 2 * rp), x.new_empty(M, rp)]
 
@@ -445,17 +500,17 @@ def _mlp_bwd_op(dy: Tensor, x: Tensor, saved: List[Tensor], factors: List[Tensor
                 g_packed: Tensor, g_scales: Tensor, g_gs: Optional[Tensor], g_fmt: str, g_code: int, g_group: int,
                 u_packed: Tensor, u_scales: Tensor, u_gs: Optional[Tensor], u_fmt: str, u_code: int, u_group: int,
                 d_packed: Tensor, d_scales: Tensor, d_gs: Optional[Tensor], d_fmt: str, d_code: int, d_group: int,
-                H: int, I: int, r: int, scaling: float, need_dx: bool) -> List[Tensor]:
+                H: int, I: int, r: int, scaling: float, need_dx: bool, gu: int) -> List[Tensor]:
     banks = (_qw_from(g_packed, g_scales, g_gs, g_fmt, g_code, g_group, I, H),
              _qw_from(u_packed, u_scales, u_gs, u_fmt, u_code, u_group, I, H),
              _qw_from(d_packed, d_scales, d_gs, d_fmt, d_code, d_group, H, I))
-    dx, grads = _mlp_bwd_impl(dy, x, tuple(saved), tuple(factors) if r else (None,) * 6, banks, r, scaling, need_dx)
+    dx, grads = _mlp_bwd_impl(dy, x, tuple(saved), tuple(factors) if r else (None,) * 6, banks, r, scaling, need_dx, gu)
     return [dx, *grads]
 
 
 @_mlp_bwd_op.register_fake
 def _(dy, x, saved, factors, g_packed, g_scales, g_gs, g_fmt, g_code, g_group, u_packed, u_scales, u_gs, u_fmt, u_code,
-      u_group, d_packed, d_scales, d_gs, d_fmt, d_code, d_group, H, I, r, scaling, need_dx):
+      u_group, d_packed, d_scales, d_gs, d_fmt, d_code, d_group, H, I, r, scaling, need_dx, gu):
     out = [x.new_empty(x.shape if need_dx else (0,))]
     if r:
         out += [x.new_empty(f.shape, dtype=torch.float32) for f in factors]
@@ -485,15 +540,17 @@ class QLoRAMLPFunction(torch.autograd.Function):
             factors = (None,) * 6
         biases = tuple(None if b is None else b.to(torch.bfloat16).contiguous() for b in (bias_g, bias_u, bias_d))
         s = float(scaling)
+        gu = _mlp_gate_up_mode(qg, qu)
         if torch.compiler.is_compiling():
-            res = _mlp_fwd_op(x2, list(factors) if r else [], list(biases), *_qw_args(qg), *_qw_args(qu), *_qw_args(qd), H, I, r, s)
+            res = _mlp_fwd_op(x2, list(factors) if r else [], list(biases), *_qw_args(qg), *_qw_args(qu), *_qw_args(qd), H, I, r, s, gu)
             y, saved = res[0], tuple(res[1:])
         else:
-            y, saved = _mlp_fwd_impl(x2, factors, biases, (qg, qu, qd), r, s)
-        ctx.banks, ctx.r, ctx.s, ctx.shape = (qg, qu, qd), r, s, x.shape
+            y, saved = _mlp_fwd_impl(x2, factors, biases, (qg, qu, qd), r, s, gu)
+        ctx.banks, ctx.r, ctx.s, ctx.shape, ctx.gu = (qg, qu, qd), r, s, x.shape, gu
         ctx.param_shapes = tuple(None if p is None else p.shape for p in params)
         ctx.param_dtypes = tuple(None if p is None else p.dtype for p in params)
         ctx.n_factors = 6 if r else 0
+        ctx.bias_d_dtype = x.dtype if bias_d is None else bias_d.dtype
         ctx.save_for_backward(x2, *saved, *(factors if r else ()))
         return y.reshape(*x.shape[:-1], H)
 
@@ -507,10 +564,10 @@ class QLoRAMLPFunction(torch.autograd.Function):
         need_dx = ctx.needs_input_grad[0]
         if torch.compiler.is_compiling():
             res = _mlp_bwd_op(dy2, x2, list(saved), list(factors) if r else [], *_qw_args(qg), *_qw_args(qu), *_qw_args(qd),
-                              H, I, r, ctx.s, need_dx)
+                              H, I, r, ctx.s, need_dx, ctx.gu)
             dx, grads = res[0], res[1:]
         else:
-            dx, grads = _mlp_bwd_impl(dy2, x2, saved, factors, ctx.banks, r, ctx.s, need_dx)
+            dx, grads = _mlp_bwd_impl(dy2, x2, saved, factors, ctx.banks, r, ctx.s, need_dx, ctx.gu)
         out = []
         for i, (g, shape, dt) in enumerate(zip(grads, ctx.param_shapes, ctx.param_dtypes)):
             if shape is None or not r or not ctx.needs_input_grad[1 + i]:
@@ -526,7 +583,7 @@ class QLoRAMLPFunction(torch.autograd.Function):
             out.append(g.to(dt))
         gb = [None, None, None]
         if ctx.needs_input_grad[9]:        # the down projection's bias sees dy itself
-            gb[2] = dy2.float().sum(0).to(dy.dtype)
+            gb[2] = dy2.float().sum(0).to(ctx.bias_d_dtype)
         if ctx.needs_input_grad[7] or ctx.needs_input_grad[8]:
             raise NotImplementedError("trainable gate / up biases are not part of the fused MLP path (frozen in QLoRA)")
         return (dx.reshape(ctx.shape) if need_dx else None, *out, *gb, None, None, None, None, None)
@@ -566,6 +623,7 @@ def qlora_mlp_infer(x: Tensor, qw_gate: QuantWeight, qw_up: QuantWeight, qw_down
     cg, cu, cd = qw_gate.c(), qw_up.c(), qw_down.c()
     _C.check(_C.lib().xq_mlp_fwd_infer(ctypes.byref(cg), ctypes.byref(cu), ctypes.byref(cd), ctypes.byref(L), x2.data_ptr(), _ld(x2), M,
                                        y.data_ptr(), H, ws.data_ptr(), n, _C.stream_ptr(dev)))
+    _note_decode_forward(dev, M)
     return y.reshape(*x.shape[:-1], H)
 
 

@@ -779,9 +779,12 @@ def qlora_mlp_forward(gate_proj: "QLoRALinear", up_proj: "QLoRALinear", down_pro
     from ..functional import qlora_mlp, qlora_mlp_infer, silu_and_mul
 
     mods = (gate_proj, up_proj, down_proj)
+    if not all(isinstance(m, QLoRALinear) for m in mods):
+        return down_proj(silu_and_mul(gate_proj(x), up_proj(x)))
     r, s = gate_proj.active_r, gate_proj._active_scaling()
-    fusable = (all(isinstance(m, QLoRALinear) for m in mods)
-               and all(m.active_r == r and m._active_scaling() == s for m in mods) and r <= MAX_FUSED_RANK
+    fusable = (all(m.active_r == r and m._active_scaling() == s for m in mods) and r <= MAX_FUSED_RANK
+               # (the fused backward forms no gradient for a gate / up bias: a trainable one takes the module path)
+               and not any(m.bias is not None and m.bias.requires_grad for m in (gate_proj, up_proj))
                and not any(m.enable_aqn and m.training for m in mods)
                and not any(_is_dtensor(m.packed_weight_f32.data) or _is_dtensor(m.lora_A) for m in mods)
                and gate_proj.out_features == up_proj.out_features == down_proj.in_features
