@@ -104,9 +104,18 @@ int xq_set_tile_policy(int policy);
  * no counterpart in the reference. */
 int xq_set_persistent_tiles(int enabled);
 
+/* Dense block-fp8 products on 256 x 256 tiles (forward, dgrad; unsplit) run on the kernel that loads both operand tiles
+ * straight into LDS, keeps the weight tile as e4m3 bytes there and multiplies with v_mfma_f32_16x16x32_bf16 (enabled = 1,
+ * the default), or on the tile kernel that every other format and the expert banks use (enabled = 0).  Both decode to the
+ * reference's bf16 values bit for bit; their sums run in different orders, so outputs agree to rounding.  A process-wide
+ * switch for tests and A/B measurements (XQ_FP8_DIRECT in the environment sets it at load time); no counterpart in the
+ * reference. */
+int xq_set_fp8_direct_tiles(int enabled);
+
 /* xq_mlp_fwd on block-fp8 weights runs gate and up either as two launches followed by one pass that writes h = SwiGLU and
  * forms the down projection's low-rank intermediate on the way (enabled = 0, the default), or as ONE launch over both weights
- * with the SwiGLU in its epilogue (enabled = 1).  Same outputs and saved activations bit for bit; the saved low-rank
+ * with the SwiGLU in its epilogue (enabled = 1).  Same outputs and saved activations bit for bit when the plain launches run on
+ * the same tile kernel (xq_set_fp8_direct_tiles(0)), to rounding otherwise (other summation order); the saved low-rank
  * intermediates of gate and up are laid out differently, which xq_mlp_saved::gate_up_fused records for the backward: the
  * switch is only the default of a forward whose struct does not say (a negative field) and may change at any time.
  * A process-wide switch for tests and A/B measurements (XQ_MLP_GU in the environment sets it at load time); no counterpart

@@ -84,6 +84,9 @@ def test_gate_up_as_one_launch_or_two(hip_device, tile_policy, M, H, I, r, bias)
     dy = gen((M, H), 1.0, 82, torch.bfloat16)
     got = {}
     try:
+        # (the one-launch form lives in the tile kernel that all formats share: the bit-for-bit comparison keeps the two plain
+        # launches on that kernel too; with the block-fp8 kernel of its own for them the sums run in another order)
+        _C.check(_C.lib().xq_set_fp8_direct_tiles(0))
         for fused in (1, 0):
             _C.check(_C.lib().xq_set_mlp_gate_up_fused(fused))
             _zero(mods)
@@ -91,10 +94,19 @@ def test_gate_up_as_one_launch_or_two(hip_device, tile_policy, M, H, I, r, bias)
             y = qlora_mlp_forward(mods["gate"], mods["up"], mods["down"], xd)
             y.backward(dy.to(hip_device))
             got[fused] = {"y": y.detach().clone(), "dx": xd.grad.clone(), **_grads(mods)}
+        _C.check(_C.lib().xq_set_fp8_direct_tiles(1))
+        _C.check(_C.lib().xq_set_mlp_gate_up_fused(0))
+        _zero(mods)
+        xd = x.to(hip_device).requires_grad_(True)
+        y = qlora_mlp_forward(mods["gate"], mods["up"], mods["down"], xd)
+        y.backward(dy.to(hip_device))
+        direct = {"y": y.detach().clone(), "dx": xd.grad.clone(), **_grads(mods)}
     finally:
         _C.check(_C.lib().xq_set_mlp_gate_up_fused(0))
+        _C.check(_C.lib().xq_set_fp8_direct_tiles(1))
     for name in got[0]:
         assert torch.equal(got[0][name], got[1][name]), name
+        assert R.max_rel_err(direct[name].float().cpu(), got[0][name].double().cpu()) <= 2 ** -7, name     # same decoded operands, other summation order
     if bias:        # (the oracle's MLP program has no bias terms)
         return
     loras = {k: (m.lora_A.detach().cpu(), m.lora_B.detach().cpu()) for k, m in mods.items()}

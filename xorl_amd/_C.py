@@ -126,6 +126,7 @@ _SIGNATURES = {
     "xq_silu_mul_bwd": (_INT, [_P, _P, _I64, _P, _I64, _P, _P, _P, _I64, _P, _I64, _I64, _P]),
     "xq_set_tile_policy": (_INT, [_INT]),
     "xq_set_persistent_tiles": (_INT, [_INT]),
+    "xq_set_fp8_direct_tiles": (_INT, [_INT]),
     "xq_set_mlp_gate_up_fused": (_INT, [_INT]),
     "xq_get_mlp_gate_up_fused": (_INT, []),
     "xq_set_skinny_one_launch": (_INT, [_INT]),

@@ -3,6 +3,7 @@
 #include <algorithm>
 #include <atomic>
 #include "xq_gemm_256.h"
+#include "xq_gemm_dtl.h"
 #include <stdlib.h>
 #include <mutex>
 #include "xq_lora.h"
@@ -42,6 +43,23 @@ static int launch_256_one(const G256Args& f, dim3 grid, hipStream_t s, const cha
         attr_set = true;
     }
     gemm_256_kernel<FMT, CC, GROUPED, T, SPLIT256><<<grid, Geo<T>::NT, Geo<T>::lds_bytes(CC), s>>>(f);
+    return XQ_OK;
+}
+
+// Dense block-fp8 launches on large unsplit tiles run gemm_dtl16_kernel (1, the default) or gemm_256_kernel (0): a
+// process-wide switch for tests and A/B measurements, XQ_FP8_DIRECT in the environment sets it at load time.
+static std::atomic<int> g_fp8_direct{[] { const char* e = getenv("XQ_FP8_DIRECT"); return e ? atoi(e) : 1; }()};
+
+static int launch_dtl16(const G256Args& f, bool cc, dim3 grid, hipStream_t s, const char* who) {
+    static std::atomic<bool> attr_set{false};
+    if (!attr_set) {
+        int rc = raise_lds_limit(gemm_dtl16_kernel<true, 8>, GeoDtl::lds_total(), who);
+        if (!rc) rc = raise_lds_limit(gemm_dtl16_kernel<false, 8>, GeoDtl::lds_total(), who);
+        if (rc) return rc;
+        attr_set = true;
+    }
+    if (cc) gemm_dtl16_kernel<true, 8><<<grid, 512, GeoDtl::lds_total(), s>>>(f);
+    else gemm_dtl16_kernel<false, 8><<<grid, 512, GeoDtl::lds_total(), s>>>(f);
     return XQ_OK;
 }
 
@@ -270,7 +288,13 @@ static int launch_tile_gemm_t(const xq_weight* w, bool contract_cols, const bf16
             dim3 grid(persistent ? persistent_grid(tiles_m * tiles_n) : (unsigned)(tiles_m * tiles_n), (unsigned)ksplit);
             const bool timed = xq_profile_mark_begin(stream, 2.0 * (double)n_rows * g.Nout * ((double)g.Kc + g.r_pad));
             int rc;
-            if (w->format == XQ_FMT_FP8) rc = launch_256<XQ_FMT_FP8>(f, contract_cols, grouped, T, grid, stream, who);
+            // dense block-fp8 on large unsplit tiles: the kernel that brings both operand tiles straight into LDS and decodes
+            // after the fragment read (xq_gemm_dtl.h), one block per tile
+            const int nk_all = g.Kc / BK;
+            if (g_fp8_direct && w->format == XQ_FMT_FP8 && T == 256 && !grouped && ksplit == 1 && nk_all >= 3 &&
+                nk_all <= 2 * GeoDtl::SCL_MAX && (!two || (f.nk1 % 2 == 0 && f.nk1 >= 2)))
+                rc = launch_dtl16(f, contract_cols, dim3((unsigned)(tiles_m * tiles_n)), stream, who);
+            else if (w->format == XQ_FMT_FP8) rc = launch_256<XQ_FMT_FP8>(f, contract_cols, grouped, T, grid, stream, who);
             else if (w->format == XQ_FMT_INT4) rc = launch_256<XQ_FMT_INT4>(f, contract_cols, grouped, T, grid, stream, who);
             else if (w->format == XQ_FMT_NF4) rc = launch_256<XQ_FMT_NF4>(f, contract_cols, grouped, T, grid, stream, who);
             else rc = launch_256<XQ_FMT_NVFP4>(f, contract_cols, grouped, T, grid, stream, who);
@@ -411,6 +435,11 @@ extern "C" int xq_skinny_status(int* gave_up, int* failed_slots, void* stream) {
     if (gave_up) *gave_up = a;
     if (failed_slots) *failed_slots = b;
     return rc;
+}
+
+extern "C" int xq_set_fp8_direct_tiles(int enabled) {
+    g_fp8_direct = enabled != 0;
+    return XQ_OK;
 }
 
 extern "C" int xq_set_persistent_tiles(int enabled) {
