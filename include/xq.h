@@ -439,7 +439,10 @@ typedef struct xq_grouped_lora {
     int32_t dtype;      /* XQ_DT_* of all six factors */
     int32_t r;
     float scaling;
-    int32_t reserved;
+    /* > 0: the gate pre-activation is clamped to [-swiglu_limit, swiglu_limit] before the SiLU, and the gate gradient is zero
+     * where the unclamped value lies outside that range (the swiglu_limit argument of the reference's expert functions,
+     * ops/moe/lora.py:545-547,638,863,917-919; ops/moe/triton.py:127-141).  0: no clamp. */
+    float swiglu_limit;
 } xq_grouped_lora;
 
 typedef struct xq_grouped_saved {

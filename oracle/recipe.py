@@ -141,6 +141,7 @@ def moe_fwd_bwd(
     scaling: float,
     dy: Optional[torch.Tensor] = None,
     dtype: torch.dtype = torch.float64,
+    swiglu_limit: float = 0.0,
 ):
     """The grouped LoRA MLP of ops/moe/lora.py:525-713 as a per-expert loop
     (the form of eager_ep_compute_lora, backend/eager.py:187-242), with the
@@ -175,6 +176,11 @@ def moe_fwd_bwd(
             return inp @ W[e] + ((inp @ Ae) @ Be) * scaling
         g = proj(xe, Wg, "gate")
         u = proj(xe, Wu, "up")
+        if swiglu_limit > 0:
+            # ops/moe/triton.py:127-141: the gate pre-activation clamped before the SiLU (lora.py:638), the gate gradient
+            # zero where the unclamped value lies outside [-limit, limit] (lora.py:917-919) -- which is what autograd gives
+            # for clamp, the bounds themselves passing the gradient
+            g = g.clamp(-swiglu_limit, swiglu_limit)
         h = F.silu(g) * u
         h = h * RW[tok, slot].unsqueeze(1)
         d = proj(h, Wd, "down")

@@ -127,6 +127,62 @@ def test_moe_fwd_bwd_vs_oracle(hip_device, tile_policy, fmt, E, T, H, I, r, topk
                 assert torch.count_nonzero(t[empty.to(t.device)]) == 0
 
 
+@pytest.mark.parametrize("E,T,H,I,r,topk,hybrid", [(6, 300, 128, 192, 8, 2, True), (4, 900, 256, 512, 16, 2, False)])
+def test_moe_swiglu_limit_vs_oracle(hip_device, E, T, H, I, r, topk, hybrid):
+    """The gate-only SwiGLU clamp (ops/moe/triton.py:127-141, ops/moe/lora.py:638,863,917-919): the gate pre-activation
+    clamped to [-limit, limit] before the SiLU, its gradient zero outside.  The mask is a discontinuity, so the data are
+    built to make it the same on both sides: inputs in {-1, 0, 1}, gate weights multiples of 1/8 with every 128 x 128 block
+    reaching 1.75 (block scale 2^-8: the e4m3 codes hold them exactly), a zero gate B factor -- the gate pre-activations are
+    then exact multiples of 1/8 in the kernels and in the float64 program alike, and the limit sits between two of them."""
+    from xorl_amd.qlora import BlockFP8QLoRAMoeExperts
+
+    limit = 4.0625
+    g = torch.Generator().manual_seed(E * 1000 + T)
+    ints = lambda *shape, lo, hi: torch.randint(lo, hi + 1, shape, generator=g).float()
+    wg = ints(E, H, I, lo=-14, hi=14) / 8.0
+    wg[:, ::128, ::128] = 1.75                      # every scale block holds the value that makes its scale 2^-8
+    m = BlockFP8QLoRAMoeExperts(E, E, I, H, r=r, lora_alpha=2 * r, hybrid_shared=hybrid)
+    m.load_weights(wg, gen((E, H, I), 0.05, 5), gen((E, I, H), 0.05, 6))
+    m.swiglu_limit = limit
+    with torch.no_grad():
+        for i, name in enumerate(("gate_proj", "up_proj", "down_proj")):
+            A, B = getattr(m, f"{name}_lora_A"), getattr(m, f"{name}_lora_B")
+            A.copy_(gen(tuple(A.shape), 0.05, 30 + i))
+            B.copy_(gen(tuple(B.shape), 0.05, 40 + i) if name != "gate_proj" else torch.zeros_like(B))
+    m = m.to(hip_device)
+    banks = {p: m.dequantize_all_experts(p, *m._proj_dims(p)).to(torch.bfloat16).cpu() for p in ("gate", "up", "down")}
+    assert torch.equal(banks["gate"].float(), wg)                    # the gate bank came through the codes exactly
+    rw, sel = _zipf_routing(T, E, topk, seed=7)
+    rw = rw.to(torch.bfloat16)
+    x = ints(T, H, lo=-1, hi=1).to(torch.bfloat16)
+    dy = gen((T, H), 1.0, 9, torch.bfloat16)
+    # the construction does what it is for: a good share of the gate values on each side of the limit, none on it
+    gates = torch.cat([x.double()[(sel == e).any(1)] @ wg[e].double() for e in range(E)])
+    share = (gates.abs() > limit).double().mean().item()
+    assert 0.05 < share < 0.95 and (gates.abs() - limit).abs().min() >= 0.0625
+    lora = {k: (getattr(m, f"{k}_proj_lora_A").detach().cpu(), getattr(m, f"{k}_proj_lora_B").detach().cpu())
+            for k in ("gate", "up", "down")}
+    got = {}
+    for lim in (limit, 0.0):
+        m.swiglu_limit = lim
+        for p in m.parameters():
+            p.grad = None
+        xd = x.to(hip_device).requires_grad_(True)
+        rwd = rw.to(hip_device).requires_grad_(True)
+        y = m(xd, rwd, sel.to(hip_device))
+        y.backward(dy.to(hip_device))
+        got[lim] = y.detach().cpu()
+        ex = R.moe_fwd_bwd(x, rw, sel, banks["gate"], banks["up"], banks["down"], lora, m.scaling, dy, swiglu_limit=lim)
+        close(y.cpu(), ex["y"], TOL)
+        close(xd.grad.cpu(), ex["dx"], TOL)
+        close(rwd.grad.cpu(), ex["d_routing"], 2e-2, rows="none")
+        for k in ("gate", "up", "down"):
+            gA, gB = getattr(m, f"{k}_proj_lora_A").grad.cpu(), getattr(m, f"{k}_proj_lora_B").grad.cpu()
+            close(gA, ex[f"dA_{k}"], TOL, rows="first")
+            close(gB, ex[f"dB_{k}"], TOL, rows="first")
+    assert not torch.equal(got[limit], got[0.0])                     # the clamp changes the result
+
+
 def test_moe_zero_lora_equals_base(hip_device):
     m, banks = _make_experts("block_fp8", 8, 128, 128, 8, True, seed=40, device=hip_device)
     rw, sel = _zipf_routing(200, 8, 2, seed=41)

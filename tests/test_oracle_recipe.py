@@ -156,6 +156,49 @@ def test_grouped_program_against_per_token_brute_force():
         assert torch.count_nonzero(res[f"dB_{k}"][E - 1]) == 0
 
 
+def test_grouped_swiglu_limit_against_the_reference_rule():
+    """swiglu_limit in the oracle's grouped program against the reference's two rules written out by hand
+    (ops/moe/triton.py:127-141): forward silu(clamp(gate, -L, L)) * up per (token, slot); backward the gate gradient
+    silu'(clamped gate) * (dh * up), zeroed where the UNCLAMPED gate lies outside [-L, L] with the bounds themselves inside."""
+    hidden, rw, sel, wg, wu, wd, lora, dy = _moe_case(seed=7)
+    L = 0.6                                     # inside the spread of this case's gate values
+    res = R.moe_fwd_bwd(hidden, rw, sel, wg, wu, wd, lora, 0.5, dy, swiglu_limit=L)
+    plain = R.moe_fwd_bwd(hidden, rw, sel, wg, wu, wd, lora, 0.5, dy)
+    T, H = hidden.shape
+    y = torch.zeros(T, H, dtype=torch.float64)
+    d_rw = torch.zeros(rw.shape, dtype=torch.float64)
+    clamped = total = 0
+    W = lambda t: t.to(torch.bfloat16).double()
+    for t in range(T):
+        for j in range(sel.shape[1]):
+            e = int(sel[t, j])
+            x = hidden[t].double()
+            def p(v, Wb, key):
+                A, B = lora[key]
+                return v @ W(Wb)[e] + ((v @ A[e].double()) @ B[e].double()) * 0.5
+            g, u = p(x, wg, "gate"), p(x, wu, "up")
+            gc = torch.minimum(torch.maximum(g, torch.tensor(-L, dtype=torch.float64)), torch.tensor(L, dtype=torch.float64))
+            clamped += int((g.abs() > L).sum()); total += g.numel()
+            a = gc * torch.sigmoid(gc)
+            h = a * u
+            y[t] += p(h * rw[t, j].double(), wd, "down")
+            # routing-weight gradient: dy . d(down(h * w))/dw, with down linear: = (down-projected h) . dy
+            d_rw[t, j] = (p(h, wd, "down") * dy[t].double()).sum()
+    assert 0.1 < clamped / total < 0.9
+    assert torch.allclose(res["y"], y, rtol=1e-12, atol=1e-12)
+    assert torch.allclose(res["d_routing"], d_rw, rtol=1e-10, atol=1e-12)
+    assert not torch.allclose(res["y"], plain["y"])
+    # the mask rule on its own: autograd through clamp = silu_backward at the clamped value times the inclusive mask
+    g = torch.tensor([-2.0, -L, -L / 2, 0.0, L, 1.5 * L], dtype=torch.float64, requires_grad=True)
+    F.silu(g.clamp(-L, L)).sum().backward()
+    gd = g.detach()
+    gc = gd.clamp(-L, L)
+    sig = torch.sigmoid(gc)
+    mask = ((gd >= -L) & (gd <= L)).double()
+    assert torch.equal(mask, torch.tensor([0.0, 1.0, 1.0, 1.0, 1.0, 0.0], dtype=torch.float64))
+    assert torch.allclose(g.grad, mask * sig * (1 + gc * (1 - sig)), rtol=1e-14, atol=0)
+
+
 def test_grouped_zero_lora_equals_base_and_shared_factor_grads_sum():
     hidden, rw, sel, wg, wu, wd, lora, dy = _moe_case(seed=4)
     zero = {k: (A, torch.zeros_like(B)) for k, (A, B) in lora.items()}

@@ -52,7 +52,7 @@ XQ_LINEAR_MULTI_MAX = 4
 class XqGroupedLora(ctypes.Structure):
     _fields_ = [("A", ctypes.c_void_p * 3), ("B", ctypes.c_void_p * 3), ("A_experts", ctypes.c_int32 * 3),
                 ("B_experts", ctypes.c_int32 * 3), ("dtype", ctypes.c_int32), ("r", ctypes.c_int32),
-                ("scaling", ctypes.c_float), ("reserved", ctypes.c_int32)]
+                ("scaling", ctypes.c_float), ("swiglu_limit", ctypes.c_float)]
 
 
 class XqGroupedSaved(ctypes.Structure):

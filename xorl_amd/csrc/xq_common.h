@@ -67,6 +67,15 @@ __device__ __forceinline__ float bf16_to_f32(bf16_t h) { return __uint_as_float(
 // product that is rounded to bf16, and the SwiGLU epilogue of the gate / up launch pays for every instruction here
 __device__ __forceinline__ float sigmoid_f32(float x) { return __builtin_amdgcn_rcpf(1.0f + __expf(-x)); }
 __device__ __forceinline__ float round_bf16(float x) { return bf16_to_f32(to_bf16(x)); }
+// The gate pre-activation under a SwiGLU limit (ops/moe/triton.py:127-131, a clamp on the bf16 tensor: the bounds are
+// rounded to bf16 with the result); limit <= 0 leaves it alone.  The gate gradient is masked where the unclamped
+// value lies outside [-limit, limit] (ops/moe/triton.py:134-141: the bounds themselves are inside).
+__device__ __forceinline__ float swiglu_clamp(float g, float limit) {
+    return limit > 0.0f ? round_bf16(fminf(fmaxf(g, -limit), limit)) : g;
+}
+__device__ __forceinline__ float swiglu_mask(float g, float limit) {
+    return (limit > 0.0f && !(g >= -limit && g <= limit)) ? 0.0f : 1.0f;
+}
 
 // e4m3fn (OCP) byte pair -> two fp32: v_cvt_pk_f32_fp8.  hi selects the upper
 // 16 bits of the dword.

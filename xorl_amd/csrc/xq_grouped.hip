@@ -131,6 +131,7 @@ extern "C" int xq_grouped_fwd(const xq_weight* gate, const xq_weight* up, const 
     const int E = d.E, rp = d.rp;
     const int64_t R = d.R, H = d.H, I = d.I;
     const float s = lora->scaling;
+    const float limit = lora->swiglu_limit > 0.0f ? lora->swiglu_limit : 0.0f;
     Carve cv{(uint8_t*)workspace, 0};
     void* route_ws = cv.take<uint8_t>(xq_route_workspace_bytes(R, E));
     const int64_t route_ws_bytes = al256(xq_route_workspace_bytes(R, E));
@@ -212,9 +213,9 @@ extern "C" int xq_grouped_fwd(const xq_weight* gate, const xq_weight* up, const 
     // SwiGLU (times the row's routing weight) and s * h . A_d^T of the down projection: one pass where the rank allows
     static const bool silu_nt = [] { const char* e = getenv("XQ_MLP_SILU_NT"); return e ? atoi(e) != 0 : true; }();
     if (silu_nt && silu_bwd_nt_supported(I, rp)) {
-        if ((rc = launch_silu_fwd_nt(gu, gu + I, 2 * I, h, I, R, I, F_dA, rp, s, su_d, rp, stream, off, toff, E, dAe == 1, saved->w_row))) return rc;
+        if ((rc = launch_silu_fwd_nt(gu, gu + I, 2 * I, h, I, R, I, F_dA, rp, s, su_d, rp, stream, off, toff, E, dAe == 1, saved->w_row, limit))) return rc;
     } else {
-        if ((rc = xq_silu_mul_fwd(gu, gu + I, 2 * I, saved->w_row, h, I, R, I, stream))) return rc;
+        if ((rc = silu_mul_fwd_limit(gu, gu + I, 2 * I, saved->w_row, h, I, R, I, limit, stream))) return rc;
         if ((rc = launch_small_nt(h, I, R, I, F_dA, rp, s, su_d, off, toff, E, dAe == 1, stream))) return rc;
     }
     if ((rc = launch_tile_gemm(down, false, h, I, R, off, toff, su_d, Lr_dB, rp, nullptr, down_out, H, stream, who, nullptr, 0))) return rc;
@@ -238,6 +239,7 @@ extern "C" int xq_grouped_bwd(const xq_weight* gate, const xq_weight* up, const 
     const int E = d.E, r = d.r, rp = d.rp;
     const int64_t R = d.R, H = d.H, I = d.I;
     const float s = lora->scaling;
+    const float limit = lora->swiglu_limit > 0.0f ? lora->swiglu_limit : 0.0f;
     if (R == 0) {      // no rows: every factor gradient is zero
         for (int p = 0; p < 3; ++p) {
             const int64_t in = p == 2 ? I : H, outw = p == 2 ? H : I;
@@ -332,10 +334,10 @@ extern "C" int xq_grouped_bwd(const xq_weight* gate, const xq_weight* up, const 
     static const bool silu_nt = [] { const char* e = getenv("XQ_MLP_SILU_NT"); return e ? atoi(e) != 0 : true; }();
     if (silu_nt && silu_bwd_nt_supported(I, rp)) {
         if ((rc = launch_silu_bwd_nt(gu, gu + I, 2 * I, dh, I, dgate, dup, 2 * I, R, I, F_gB, F_uB, rp, s, v_g, v_u, ld_v, stream, off, toff, E,
-                                     gBe == 1, uBe == 1, saved->w_row, d_w_row)))
+                                     gBe == 1, uBe == 1, saved->w_row, d_w_row, limit)))
             return rc;
     } else {
-        if ((rc = xq_silu_mul_bwd(gu, gu + I, 2 * I, dh, I, saved->w_row, dgate, dup, 2 * I, d_w_row, R, I, stream))) return rc;
+        if ((rc = silu_mul_bwd_limit(gu, gu + I, 2 * I, dh, I, saved->w_row, dgate, dup, 2 * I, d_w_row, R, I, limit, stream))) return rc;
         if ((rc = launch_small_nt(dup, 2 * I, R, I, F_uB, rp, s, v_u, off, toff, E, uBe == 1, stream, ld_v))) return rc;
         if ((rc = launch_small_nt(dgate, 2 * I, R, I, F_gB, rp, s, v_g, off, toff, E, gBe == 1, stream, ld_v))) return rc;
     }

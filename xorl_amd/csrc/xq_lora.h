@@ -72,14 +72,21 @@ int launch_silu_bwd_nt(const bf16_t* gate, const bf16_t* up, int64_t ld_gu, cons
                        // routed rows in expert order (offsets != NULL): a factor pair per expert ([E][r_pad][cols]) unless
                        // shared, the rows' routing weights applied and (d_row_w != NULL) their gradients written
                        const int32_t* offsets = nullptr, const int32_t* tile_offsets = nullptr, int32_t num_experts = 1,
-                       bool shared_fg = true, bool shared_fu = true, const float* row_w = nullptr, float* d_row_w = nullptr);
+                       bool shared_fg = true, bool shared_fu = true, const float* row_w = nullptr, float* d_row_w = nullptr,
+                       float swiglu_limit = 0.0f);     // > 0: the gate pre-activation is clamped to [-limit, limit], its gradient masked outside
 
 // the forward in the same organisation: h = SwiGLU(gate, up) as xq_silu_mul_fwd writes it (routed rows: times the row's
 // weight) and T = scale * h . F^T as launch_small_nt on h would (same bits)
 int launch_silu_fwd_nt(const bf16_t* gate, const bf16_t* up, int64_t ld_gu, bf16_t* h, int64_t ld_h, int64_t n_rows, int64_t cols,
                        const bf16_t* F, int r_pad, float scale, bf16_t* T, int64_t ld_t, hipStream_t stream,
                        const int32_t* offsets = nullptr, const int32_t* tile_offsets = nullptr, int32_t num_experts = 1,
-                       bool shared_f = true, const float* row_w = nullptr);
+                       bool shared_f = true, const float* row_w = nullptr, float swiglu_limit = 0.0f);
+
+// xq_silu_mul_fwd / xq_silu_mul_bwd with a SwiGLU limit on the gate pre-activation (ops/moe/triton.py:127-141; <= 0: none)
+int silu_mul_fwd_limit(const void* gate, const void* up, int64_t ld_in, const float* row_w, void* h, int64_t ld_h, int64_t rows,
+                       int64_t cols, float limit, void* stream);
+int silu_mul_bwd_limit(const void* gate, const void* up, int64_t ld_in, const void* dh, int64_t ld_dh, const float* row_w, void* dgate,
+                       void* dup, int64_t ld_out, float* d_row_w, int64_t rows, int64_t cols, float limit, void* stream);
 
 // out[c][j] (or out[j][c] when transpose_out) = sum_m P[m][c] * Q[m][j], fp32.
 //   dense: all rows, split over `splits` row ranges, partials in `partial`

@@ -425,6 +425,7 @@ struct SiluNtArgs {
     int64_t fg_stride, fu_stride;
     const float* row_w;
     float* d_row_w;
+    float limit;               // SwiGLU limit on the gate pre-activation (<= 0: none)
 };
 
 // GROUPED: routed rows in expert order, organisation of small_nt_kernel<128, FJ> (a block = a 128-row tile of one expert, a
@@ -548,7 +549,7 @@ __global__ void __launch_bounds__(256, 2) silu_bwd_nt_kernel(SiluNtArgs g) {
                     float res[2];
 #pragma unroll
                     for (int hlf = 0; hlf < 2; ++hlf) {
-                        const float gv = bf16_to_f32((bf16_t)(gq[j][i] >> (16 * hlf))), uv = bf16_to_f32((bf16_t)(uq[j][i] >> (16 * hlf)));
+                        const float gv = swiglu_clamp(bf16_to_f32((bf16_t)(gq[j][i] >> (16 * hlf))), g.limit), uv = bf16_to_f32((bf16_t)(uq[j][i] >> (16 * hlf)));
                         const float a = round_bf16(gv * sigmoid_f32(gv));
                         float v = a * uv;
                         if constexpr (GROUPED) v = round_bf16(v) * rw[j];
@@ -578,7 +579,8 @@ __global__ void __launch_bounds__(256, 2) silu_bwd_nt_kernel(SiluNtArgs g) {
                 float rg[2], ru[2];
 #pragma unroll
                 for (int hlf = 0; hlf < 2; ++hlf) {
-                    const float gv = bf16_to_f32((bf16_t)(gq[j][i] >> (16 * hlf))), uv = bf16_to_f32((bf16_t)(uq[j][i] >> (16 * hlf)));
+                    const float g_raw = bf16_to_f32((bf16_t)(gq[j][i] >> (16 * hlf))), uv = bf16_to_f32((bf16_t)(uq[j][i] >> (16 * hlf)));
+                    const float gv = swiglu_clamp(g_raw, g.limit), open = swiglu_mask(g_raw, g.limit);
                     const float d = bf16_to_f32((bf16_t)(dq[j][i] >> (16 * hlf)));
                     const float sg = sigmoid_f32(gv);
                     const float a = round_bf16(gv * sg);
@@ -587,7 +589,7 @@ __global__ void __launch_bounds__(256, 2) silu_bwd_nt_kernel(SiluNtArgs g) {
                         dp = round_bf16(d * rw[j]);
                         if (mine) wsum[j] += d * round_bf16(a * uv);
                     }
-                    rg[hlf] = round_bf16(dp * uv) * (sg * (1.0f + gv * (1.0f - sg)));
+                    rg[hlf] = round_bf16(dp * uv) * (sg * (1.0f + gv * (1.0f - sg))) * open;
                     ru[hlf] = a * dp;
                 }
                 og[i] = pack_bf16x2(rg[0], rg[1]);
@@ -688,7 +690,7 @@ int launch_silu_bwd_nt(const bf16_t* gate, const bf16_t* up, int64_t ld_gu, cons
                        bf16_t* dup, int64_t ld_out, int64_t n_rows, int64_t cols, const bf16_t* Fg, const bf16_t* Fu, int r_pad,
                        float scale, bf16_t* Tg, bf16_t* Tu, int64_t ld_t, hipStream_t stream, const int32_t* offsets,
                        const int32_t* tile_offsets, int32_t num_experts, bool shared_fg, bool shared_fu, const float* row_w,
-                       float* d_row_w) {
+                       float* d_row_w, float swiglu_limit) {
     XQ_REQUIRE(silu_bwd_nt_supported(cols, r_pad), "silu_bwd_nt: %lld columns with r_pad %d are not handled here", (long long)cols, r_pad);
     XQ_REQUIRE(ld_gu % 8 == 0 && ld_dh % 8 == 0 && ld_out % 8 == 0 && ld_t >= r_pad, "silu_bwd_nt: row pitches must be multiples of 8");
     XQ_REQUIRE(xq_aligned(gate, 16) && xq_aligned(up, 16) && xq_aligned(dh, 16) && xq_aligned(dgate, 16) && xq_aligned(dup, 16) &&
@@ -698,7 +700,7 @@ int launch_silu_bwd_nt(const bf16_t* gate, const bf16_t* up, int64_t ld_gu, cons
     if (n_rows == 0) return XQ_OK;
     SiluNtArgs g{gate, up, ld_gu, dh, ld_dh, dgate, dup, ld_out, n_rows, cols, Fg, Fu, r_pad, scale, Tg, Tu, ld_t,
                  offsets, tile_offsets, num_experts, offsets && !shared_fg ? (int64_t)r_pad * cols : 0,
-                 offsets && !shared_fu ? (int64_t)r_pad * cols : 0, row_w, d_row_w};
+                 offsets && !shared_fu ? (int64_t)r_pad * cols : 0, row_w, d_row_w, swiglu_limit};
     if (offsets) {
         const unsigned blocks = (unsigned)(xq_cdiv(n_rows, 128) + num_experts);
         return r_pad == 16 ? launch_silu_bwd_nt_one<4, true>(g, blocks, stream) : launch_silu_bwd_nt_one<8, true>(g, blocks, stream);
@@ -709,14 +711,14 @@ int launch_silu_bwd_nt(const bf16_t* gate, const bf16_t* up, int64_t ld_gu, cons
 
 int launch_silu_fwd_nt(const bf16_t* gate, const bf16_t* up, int64_t ld_gu, bf16_t* h, int64_t ld_h, int64_t n_rows, int64_t cols,
                        const bf16_t* F, int r_pad, float scale, bf16_t* T, int64_t ld_t, hipStream_t stream, const int32_t* offsets,
-                       const int32_t* tile_offsets, int32_t num_experts, bool shared_f, const float* row_w) {
+                       const int32_t* tile_offsets, int32_t num_experts, bool shared_f, const float* row_w, float swiglu_limit) {
     XQ_REQUIRE(silu_bwd_nt_supported(cols, r_pad), "silu_fwd_nt: %lld columns with r_pad %d are not handled here", (long long)cols, r_pad);
     XQ_REQUIRE(ld_gu % 8 == 0 && ld_h % 8 == 0 && ld_t >= r_pad, "silu_fwd_nt: row pitches must be multiples of 8");
     XQ_REQUIRE(xq_aligned(gate, 16) && xq_aligned(up, 16) && xq_aligned(h, 16) && xq_aligned(F, 16), "silu_fwd_nt: operands must be 16-byte aligned");
     XQ_REQUIRE(!offsets || (tile_offsets && row_w && num_experts >= 1), "silu_fwd_nt: the routed form needs tile offsets and row weights");
     if (n_rows == 0) return XQ_OK;
     SiluNtArgs g{gate, up, ld_gu, nullptr, 0, h, nullptr, ld_h, n_rows, cols, F, F, r_pad, scale, T, nullptr, ld_t,
-                 offsets, tile_offsets, num_experts, offsets && !shared_f ? (int64_t)r_pad * cols : 0, 0, row_w, nullptr};
+                 offsets, tile_offsets, num_experts, offsets && !shared_f ? (int64_t)r_pad * cols : 0, 0, row_w, nullptr, swiglu_limit};
     if (offsets) {
         const unsigned blocks = (unsigned)(xq_cdiv(n_rows, 128) + num_experts);
         return r_pad == 16 ? launch_silu_bwd_nt_one<4, true, true>(g, blocks, stream) : launch_silu_bwd_nt_one<8, true, true>(g, blocks, stream);

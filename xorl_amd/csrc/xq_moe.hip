@@ -12,7 +12,7 @@ namespace {
 // h = bf16(bf16(bf16(silu(g)) * u) * w_row)
 __global__ void __launch_bounds__(256) silu_mul_fwd_kernel(const bf16_t* gate, const bf16_t* up, int64_t ld_in,
                                                            const float* row_w, bf16_t* h, int64_t ld_h, int64_t rows,
-                                                           int64_t cols8) {
+                                                           int64_t cols8, float limit) {
     int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (t >= rows * cols8) return;
     int64_t r = t / cols8, c = (t - r * cols8) * 8;
@@ -25,6 +25,7 @@ __global__ void __launch_bounds__(256) silu_mul_fwd_kernel(const bf16_t* gate, c
 #pragma unroll
         for (int hlf = 0; hlf < 2; ++hlf) {
             float g = bf16_to_f32((bf16_t)(gv[i] >> (16 * hlf))), u = bf16_to_f32((bf16_t)(uv[i] >> (16 * hlf)));
+            g = swiglu_clamp(g, limit);
             float a = round_bf16(g * sigmoid_f32(g));
             float v = a * u;
             if (row_w) v = round_bf16(v) * w;
@@ -41,7 +42,7 @@ __global__ void __launch_bounds__(256) silu_mul_fwd_kernel(const bf16_t* gate, c
 __global__ void __launch_bounds__(256) silu_mul_bwd_kernel(const bf16_t* gate, const bf16_t* up, int64_t ld_in,
                                                            const bf16_t* dh, int64_t ld_dh, const float* row_w,
                                                            bf16_t* dgate, bf16_t* dup, int64_t ld_out, float* d_row_w,
-                                                           int64_t rows, int64_t cols) {
+                                                           int64_t rows, int64_t cols, float limit) {
     // one block per row (cols/8 vector steps striding over the row) so the row-weight gradient is a block reduction
     __shared__ float red[4];
     const int64_t r = blockIdx.x;
@@ -58,11 +59,13 @@ __global__ void __launch_bounds__(256) silu_mul_bwd_kernel(const bf16_t* gate, c
             for (int hlf = 0; hlf < 2; ++hlf) {
                 float g = bf16_to_f32((bf16_t)(gv[i] >> (16 * hlf))), u = bf16_to_f32((bf16_t)(uv[i] >> (16 * hlf)));
                 float d = bf16_to_f32((bf16_t)(dv[i] >> (16 * hlf)));
+                const float open = swiglu_mask(g, limit);
+                g = swiglu_clamp(g, limit);
                 float s = sigmoid_f32(g);
                 float a = round_bf16(g * s);
                 float dp = row_w ? round_bf16(d * w) : d;
                 wsum += d * round_bf16(a * u);
-                rg[hlf] = round_bf16(dp * u) * (s * (1.0f + g * (1.0f - s)));
+                rg[hlf] = round_bf16(dp * u) * (s * (1.0f + g * (1.0f - s))) * open;
                 ru[hlf] = a * dp;
             }
             og[i] = pack_bf16x2(rg[0], rg[1]);
@@ -306,22 +309,22 @@ __global__ void __launch_bounds__(256) moe_gather_kernel(const bf16_t* rows, con
 
 }  // namespace
 
-extern "C" int xq_silu_mul_fwd(const void* gate, const void* up, int64_t ld_in, const float* row_w, void* h,
-                               int64_t ld_h, int64_t rows, int64_t cols, void* stream) {
+namespace xq {
+int silu_mul_fwd_limit(const void* gate, const void* up, int64_t ld_in, const float* row_w, void* h, int64_t ld_h, int64_t rows,
+                       int64_t cols, float limit, void* stream) {
     XQ_REQUIRE(cols % 8 == 0 && ld_in % 8 == 0 && ld_h % 8 == 0, "xq_silu_mul_fwd: cols and strides must be multiples of 8");
     if (rows == 0 || cols == 0) return XQ_OK;   // an empty batch has no storage to point at
     XQ_REQUIRE(gate && up && h, "xq_silu_mul_fwd: NULL pointer");
     XQ_REQUIRE(xq_aligned(gate, 16) && xq_aligned(up, 16) && xq_aligned(h, 16), "xq_silu_mul_fwd: pointers must be 16-byte aligned");
     int64_t total = rows * (cols / 8);
     silu_mul_fwd_kernel<<<dim3((unsigned)xq_cdiv(total, 256)), 256, 0, (hipStream_t)stream>>>(
-        (const bf16_t*)gate, (const bf16_t*)up, ld_in, row_w, (bf16_t*)h, ld_h, rows, cols / 8);
+        (const bf16_t*)gate, (const bf16_t*)up, ld_in, row_w, (bf16_t*)h, ld_h, rows, cols / 8, limit);
     XQ_CHECK_LAUNCH("xq_silu_mul_fwd");
     return XQ_OK;
 }
 
-extern "C" int xq_silu_mul_bwd(const void* gate, const void* up, int64_t ld_in, const void* dh, int64_t ld_dh,
-                               const float* row_w, void* dgate, void* dup, int64_t ld_out, float* d_row_w,
-                               int64_t rows, int64_t cols, void* stream) {
+int silu_mul_bwd_limit(const void* gate, const void* up, int64_t ld_in, const void* dh, int64_t ld_dh, const float* row_w, void* dgate,
+                       void* dup, int64_t ld_out, float* d_row_w, int64_t rows, int64_t cols, float limit, void* stream) {
     XQ_REQUIRE(cols % 8 == 0 && ld_in % 8 == 0 && ld_dh % 8 == 0 && ld_out % 8 == 0, "xq_silu_mul_bwd: cols and strides must be multiples of 8");
     if (rows == 0 || cols == 0) return XQ_OK;   // an empty batch has no storage to point at
     XQ_REQUIRE(gate && up && dh && dgate && dup, "xq_silu_mul_bwd: NULL pointer");
@@ -329,9 +332,21 @@ extern "C" int xq_silu_mul_bwd(const void* gate, const void* up, int64_t ld_in, 
                "xq_silu_mul_bwd: pointers must be 16-byte aligned");
     silu_mul_bwd_kernel<<<dim3((unsigned)rows), 256, 0, (hipStream_t)stream>>>(
         (const bf16_t*)gate, (const bf16_t*)up, ld_in, (const bf16_t*)dh, ld_dh, row_w, (bf16_t*)dgate, (bf16_t*)dup,
-        ld_out, d_row_w, rows, cols);
+        ld_out, d_row_w, rows, cols, limit);
     XQ_CHECK_LAUNCH("xq_silu_mul_bwd");
     return XQ_OK;
+}
+}  // namespace xq
+
+extern "C" int xq_silu_mul_fwd(const void* gate, const void* up, int64_t ld_in, const float* row_w, void* h,
+                               int64_t ld_h, int64_t rows, int64_t cols, void* stream) {
+    return xq::silu_mul_fwd_limit(gate, up, ld_in, row_w, h, ld_h, rows, cols, 0.0f, stream);
+}
+
+extern "C" int xq_silu_mul_bwd(const void* gate, const void* up, int64_t ld_in, const void* dh, int64_t ld_dh,
+                               const float* row_w, void* dgate, void* dup, int64_t ld_out, float* d_row_w,
+                               int64_t rows, int64_t cols, void* stream) {
+    return xq::silu_mul_bwd_limit(gate, up, ld_in, dh, ld_dh, row_w, dgate, dup, ld_out, d_row_w, rows, cols, 0.0f, stream);
 }
 
 extern "C" int64_t xq_route_workspace_bytes(int64_t n_routed, int32_t num_experts) {

@@ -138,7 +138,7 @@ def _rebuild_bank(packed, scales, gs, fmt, layout, scale_dt, rows, cols, group, 
     return QuantWeight(fmt, layout, packed, scales, scale_dt, rows, cols, group, global_scale=gs, num_experts=E)
 
 
-def _lora_struct(factors, r: int, scaling: float) -> _C.XqGroupedLora:
+def _lora_struct(factors, r: int, scaling: float, swiglu_limit: float = 0.0) -> _C.XqGroupedLora:
     gA, gB, uA, uB, dA, dB = factors
     dt = gA.dtype
     if dt not in (torch.float32, torch.bfloat16) or any(f.dtype != dt for f in factors):
@@ -148,7 +148,7 @@ def _lora_struct(factors, r: int, scaling: float) -> _C.XqGroupedLora:
         L.A[p], L.B[p] = A.data_ptr(), B.data_ptr()
         L.A_experts[p], L.B_experts[p] = A.shape[0], B.shape[0]
     L.dtype = _C.XQ_DT_F32 if dt == torch.float32 else _C.XQ_DT_BF16
-    L.r, L.scaling = r, scaling
+    L.r, L.scaling, L.swiglu_limit = r, scaling, max(float(swiglu_limit), 0.0)
     return L
 
 
@@ -176,7 +176,8 @@ def _workspace(dev, T: int, topk: int, E: int, H: int, I: int, r: int, backward:
     return torch.empty(n, dtype=torch.uint8, device=dev)
 
 
-def _moe_fwd_impl(hidden2: Tensor, rw: Tensor, sel: Tensor, factors, banks, r: int, scaling: float, allow_in_place: bool = True):
+def _moe_fwd_impl(hidden2: Tensor, rw: Tensor, sel: Tensor, factors, banks, r: int, scaling: float, allow_in_place: bool = True,
+                  swiglu_limit: float = 0.0):
     """xq_grouped_fwd.  hidden2 bf16 [T, H]; rw [T, topk] fp32 / bf16; sel int32 [T, topk]; factors the six active
     LoRA views, contiguous; banks three QuantWeight.  -> (out [T, H], the eleven tensors the backward reads)."""
     qg, qu, qd = banks
@@ -194,7 +195,7 @@ def _moe_fwd_impl(hidden2: Tensor, rw: Tensor, sel: Tensor, factors, banks, r: i
              bf(R, rp), bf(R, rp), i32(R), i32(E + 1), i32(2 * (E + 1)), i32(E))
     out = bf(T, H)
     ws = _workspace(dev, T, topk, E, H, I, r, False)
-    lora, S = _lora_struct(factors, r, scaling), _saved_struct(saved)
+    lora, S = _lora_struct(factors, r, scaling, swiglu_limit), _saved_struct(saved)
     _C.check(_C.lib().xq_grouped_fwd(ctypes.byref(wg), ctypes.byref(wu), ctypes.byref(wd), ctypes.byref(lora),
                                      hidden2.data_ptr(), hidden2.stride(0) if T > 1 else H, T, rw.data_ptr(),
                                      _C.XQ_DT_F32 if rw.dtype == torch.float32 else _C.XQ_DT_BF16, sel.data_ptr(), topk,
@@ -203,7 +204,7 @@ def _moe_fwd_impl(hidden2: Tensor, rw: Tensor, sel: Tensor, factors, banks, r: i
 
 
 def _moe_bwd_impl(dy2: Tensor, saved, factors, banks, r: int, scaling: float, T: int, topk: int, rw_dtype: torch.dtype,
-                  need_dx: bool, need_drw: bool, hidden2: Optional[Tensor] = None):
+                  need_dx: bool, need_drw: bool, hidden2: Optional[Tensor] = None, swiglu_limit: float = 0.0):
     """xq_grouped_bwd -> (dx [T, H] or empty, d_routing [T, topk] or empty, six fp32 factor gradients)."""
     qg, qu, qd = banks
     E, H, I = qg.num_experts, qg.rows, qg.cols
@@ -216,7 +217,7 @@ def _moe_bwd_impl(dy2: Tensor, saved, factors, banks, r: int, scaling: float, T:
     for p in range(3):
         G.dA[p], G.dB[p] = grads[2 * p].data_ptr(), grads[2 * p + 1].data_ptr()
     ws = _workspace(dev, T, topk, E, H, I, r, True)
-    lora, S = _lora_struct(factors, r, scaling), _saved_struct(saved, hidden2)
+    lora, S = _lora_struct(factors, r, scaling, swiglu_limit), _saved_struct(saved, hidden2)
     wg, wu, wd = qg.c(), qu.c(), qd.c()
     _C.check(_C.lib().xq_grouped_bwd(ctypes.byref(wg), ctypes.byref(wu), ctypes.byref(wd), ctypes.byref(lora),
                                      dy2.data_ptr(), dy2.stride(0) if T > 1 else H, T, topk, ctypes.byref(S),
@@ -231,18 +232,19 @@ def _moe_fwd_op(hidden: Tensor, rw: Tensor, sel: Tensor, gA: Tensor, gB: Tensor,
                 dB: Tensor, g_packed: Tensor, g_scales: Tensor, g_gs: Optional[Tensor], u_packed: Tensor,
                 u_scales: Tensor, u_gs: Optional[Tensor], d_packed: Tensor, d_scales: Tensor, d_gs: Optional[Tensor],
                 fmt: str, layout: int, scale_code: int, group: int, E: int, H: int, I: int, r: int,
-                scaling: float) -> List[Tensor]:
+                scaling: float, swiglu_limit: float = 0.0) -> List[Tensor]:
     sd = _CODE_TO_DT[scale_code]
     banks = (_rebuild_bank(g_packed, g_scales, g_gs, fmt, layout, sd, H, I, group, E),
              _rebuild_bank(u_packed, u_scales, u_gs, fmt, layout, sd, H, I, group, E),
              _rebuild_bank(d_packed, d_scales, d_gs, fmt, layout, sd, I, H, group, E))
-    out, saved = _moe_fwd_impl(hidden, rw, sel, (gA, gB, uA, uB, dA, dB), banks, r, scaling, allow_in_place=False)
+    out, saved = _moe_fwd_impl(hidden, rw, sel, (gA, gB, uA, uB, dA, dB), banks, r, scaling, allow_in_place=False,
+                               swiglu_limit=swiglu_limit)
     return [out, *saved]
 
 
 @_moe_fwd_op.register_fake
 def _(hidden, rw, sel, gA, gB, uA, uB, dA, dB, g_packed, g_scales, g_gs, u_packed, u_scales, u_gs, d_packed, d_scales,
-      d_gs, fmt, layout, scale_code, group, E, H, I, r, scaling):
+      d_gs, fmt, layout, scale_code, group, E, H, I, r, scaling, swiglu_limit=0.0):
     T, topk = sel.shape
     R, rp = T * topk, _r_pad(r)
     bf = lambda *shape: hidden.new_empty(*shape, dtype=torch.bfloat16)
@@ -256,19 +258,19 @@ def _moe_bwd_op(dy: Tensor, hidden: Tensor, saved: List[Tensor], gA: Tensor, gB:
                 g_packed: Tensor, g_scales: Tensor, g_gs: Optional[Tensor], u_packed: Tensor, u_scales: Tensor,
                 u_gs: Optional[Tensor], d_packed: Tensor, d_scales: Tensor, d_gs: Optional[Tensor], fmt: str,
                 layout: int, scale_code: int, group: int, E: int, H: int, I: int, r: int, scaling: float, T: int,
-                topk: int, rw_code: int, need_dx: bool, need_drw: bool) -> List[Tensor]:
+                topk: int, rw_code: int, need_dx: bool, need_drw: bool, swiglu_limit: float = 0.0) -> List[Tensor]:
     sd = _CODE_TO_DT[scale_code]
     banks = (_rebuild_bank(g_packed, g_scales, g_gs, fmt, layout, sd, H, I, group, E),
              _rebuild_bank(u_packed, u_scales, u_gs, fmt, layout, sd, H, I, group, E),
              _rebuild_bank(d_packed, d_scales, d_gs, fmt, layout, sd, I, H, group, E))
     dx, drw, grads = _moe_bwd_impl(dy, tuple(saved), (gA, gB, uA, uB, dA, dB), banks, r, scaling, T, topk,
-                                   _CODE_TO_DT[rw_code], need_dx, need_drw, hidden)
+                                   _CODE_TO_DT[rw_code], need_dx, need_drw, hidden, swiglu_limit)
     return [dx, drw, *grads]
 
 
 @_moe_bwd_op.register_fake
 def _(dy, hidden, saved, gA, gB, uA, uB, dA, dB, g_packed, g_scales, g_gs, u_packed, u_scales, u_gs, d_packed, d_scales, d_gs,
-      fmt, layout, scale_code, group, E, H, I, r, scaling, T, topk, rw_code, need_dx, need_drw):
+      fmt, layout, scale_code, group, E, H, I, r, scaling, T, topk, rw_code, need_dx, need_drw, swiglu_limit=0.0):
     rw_dt = _CODE_TO_DT[rw_code]
     return [dy.new_empty((T, H) if need_dx else (0,), dtype=torch.bfloat16),
             dy.new_empty((T, topk) if need_drw else (0,), dtype=rw_dt),
@@ -287,7 +289,8 @@ class MoeExpertsQLoRAFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, hidden, routing_weights, selected_experts, gA, gB, uA, uB, dA, dB,
-                qw_gate: QuantWeight, qw_up: QuantWeight, qw_down: QuantWeight, num_experts: int, scaling: float):
+                qw_gate: QuantWeight, qw_up: QuantWeight, qw_down: QuantWeight, num_experts: int, scaling: float,
+                swiglu_limit: float = 0.0):
         _C.require_hip(hidden, routing_weights, selected_experts)
         if hidden.dtype != torch.bfloat16:
             raise _C.XqError(f"hidden states must be bf16, got {hidden.dtype}")
@@ -310,13 +313,15 @@ class MoeExpertsQLoRAFunction(torch.autograd.Function):
         r = gA.shape[-1]
         factors = tuple(f.contiguous() for f in (gA, gB, uA, uB, dA, dB))
         s = float(scaling)
+        lim = max(float(swiglu_limit or 0.0), 0.0)
         if torch.compiler.is_compiling():
             res = _moe_fwd_op(hidden2, rw, sel, *factors, *_bank_args(qw_gate), *_bank_args(qw_up), *_bank_args(qw_down),
-                              qw_gate.fmt, qw_gate.layout, _DT_TO_CODE[qw_gate.scale_dtype], qw_gate.group, E, H, I, r, s)
+                              qw_gate.fmt, qw_gate.layout, _DT_TO_CODE[qw_gate.scale_dtype], qw_gate.group, E, H, I, r, s, lim)
             out, saved = res[0], tuple(res[1:])
         else:
-            out, saved = _moe_fwd_impl(hidden2, rw, sel, factors, banks, r, s)
+            out, saved = _moe_fwd_impl(hidden2, rw, sel, factors, banks, r, s, swiglu_limit=lim)
         ctx.qw = banks
+        ctx.swiglu_limit = lim
         ctx.meta = (E, T, topk, H, I, r, s, shape, routing_weights.dtype, routing_weights.shape)
         ctx.save_for_backward(*saved, *factors, hidden2)
         return out.reshape(shape)
@@ -333,14 +338,15 @@ class MoeExpertsQLoRAFunction(torch.autograd.Function):
         if torch.compiler.is_compiling():
             res = _moe_bwd_op(dy2, hidden2, list(saved), *factors, *_bank_args(qw_gate), *_bank_args(qw_up), *_bank_args(qw_down),
                               qw_gate.fmt, qw_gate.layout, _DT_TO_CODE[qw_gate.scale_dtype], qw_gate.group, E, H, I, r, s,
-                              T, topk, _DT_TO_CODE[kernel_rw_dt], need_dx, need_drw)
+                              T, topk, _DT_TO_CODE[kernel_rw_dt], need_dx, need_drw, ctx.swiglu_limit)
             dx, drw, grads = res[0], res[1], res[2:]
         else:
-            dx, drw, grads = _moe_bwd_impl(dy2, saved, factors, ctx.qw, r, s, T, topk, kernel_rw_dt, need_dx, need_drw, hidden2)
+            dx, drw, grads = _moe_bwd_impl(dy2, saved, factors, ctx.qw, r, s, T, topk, kernel_rw_dt, need_dx, need_drw, hidden2,
+                                           ctx.swiglu_limit)
         dx = dx.reshape(shape) if need_dx else None
         drw = drw.reshape(rw_shape).to(rw_dtype) if need_drw else None
         gs = [g.to(f.dtype) for g, f in zip(grads, factors)]
-        return (dx, drw, None, *gs, None, None, None, None, None)
+        return (dx, drw, None, *gs, None, None, None, None, None, None)
 
 
 def moe_experts_qlora_forward(num_experts: int, routing_weights: Tensor, selected_experts: Tensor,
@@ -351,11 +357,10 @@ def moe_experts_qlora_forward(num_experts: int, routing_weights: Tensor, selecte
     """Entry with the argument order of the reference's MOE_EXPERT_BACKENDS_LORA callables
     (models/layers/moe/backend/__init__.py:421-445), except that the three base banks are
     packed QuantWeight descriptors instead of dequantized [E, K, N] tensors."""
-    if swiglu_limit:
-        raise NotImplementedError("swiglu_limit clamping is not part of the packed-bank expert path")
     return MoeExpertsQLoRAFunction.apply(hidden_states, routing_weights, selected_experts, gate_proj_lora_A,
                                          gate_proj_lora_B, up_proj_lora_A, up_proj_lora_B, down_proj_lora_A,
-                                         down_proj_lora_B, gate_proj, up_proj, down_proj, num_experts, scaling)
+                                         down_proj_lora_B, gate_proj, up_proj, down_proj, num_experts, scaling,
+                                         float(swiglu_limit or 0.0))
 
 
 def moe_experts_qlora_ep_compute(permute_tokens: Tensor, cumsum: Tensor, gate_proj: QuantWeight, up_proj: QuantWeight,
@@ -370,8 +375,6 @@ def moe_experts_qlora_ep_compute(permute_tokens: Tensor, cumsum: Tensor, gate_pr
 
     The rows run through the routed program as a top-1 problem with unit weights: the stable sort by expert is
     then the identity and the weight multiplication exact."""
-    if swiglu_limit:
-        raise NotImplementedError("swiglu_limit clamping is not part of the packed-bank expert path")
     E = gate_proj.num_experts
     R = permute_tokens.shape[0]
     if cumsum.numel() < E:
@@ -388,7 +391,7 @@ def moe_experts_qlora_ep_compute(permute_tokens: Tensor, cumsum: Tensor, gate_pr
         raise _C.XqError(f"cumsum ends at {int(ends[-1])} but {R} rows were passed")
     ones = torch.ones(R, 1, dtype=torch.float32, device=dev)
     return MoeExpertsQLoRAFunction.apply(permute_tokens, ones, expert_of_row.to(torch.int32).unsqueeze(1), *factors,
-                                         gate_proj, up_proj, down_proj, E, scaling)
+                                         gate_proj, up_proj, down_proj, E, scaling, float(swiglu_limit or 0.0))
 
 
 # registry entries a maintainer adds beside "triton" / "native" / "quack"

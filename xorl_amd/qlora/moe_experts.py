@@ -115,11 +115,16 @@ class QLoRAMoeExperts(LoraModule, nn.Module):
                 raise TypeError(f"{type(module).__name__} holds no [num_experts, in, out] expert weights")
             gate = fused
             total, hidden, inter = fused.shape[0], fused.shape[1], fused.shape[2] // 2
-        for attr, want in (("gated", True), ("swiglu_limit", 0.0), ("gate_up_bias", None), ("down_bias", None)):
+        for attr, want in (("gated", True), ("gate_up_bias", None), ("down_bias", None)):
             have = getattr(module, attr, want)
-            if have is not None and have != want and not (attr == "swiglu_limit" and not have):
-                raise ValueError(f"expert adapters need gated SiLU experts without clamping or biases; "
+            if have is not None and have != want:
+                raise ValueError(f"expert adapters need gated SiLU experts without biases; "
                                  f"{type(module).__name__}.{attr} = {have!r}")
+        # a gate-only SwiGLU clamp (lora/expert_adapter_contract.py:39-57: the DeepSeek-V4 program) is carried over: the routed
+        # kernels clamp the gate pre-activation and mask its gradient (ops/moe/triton.py:127-141)
+        limit = float(getattr(module, "swiglu_limit", 0.0) or 0.0)
+        if limit < 0:
+            raise ValueError(f"{type(module).__name__}.swiglu_limit = {limit!r} must not be negative")
         required = {"nvfp4": 16, "block_fp8": 128, "nf4": 64}
         if quant_format not in required:
             raise ValueError(f"Expert QLoRA formats: {sorted(required)}; got {quant_format!r}")
@@ -128,12 +133,14 @@ class QLoRAMoeExperts(LoraModule, nn.Module):
                              f"got {quant_group_size}")
         if cls is QLoRAMoeExperts:
             cls = {"block_fp8": BlockFP8QLoRAMoeExperts, "nf4": NF4QLoRAMoeExperts, "nvfp4": NvFP4QLoRAMoeExperts}[quant_format]
-        return cls(num_local_experts=total if num_local_experts is None else num_local_experts, num_experts=total,
-                   intermediate_size=getattr(module, "intermediate_size", inter),
-                   hidden_size=getattr(module, "hidden_dim", hidden), r=r, lora_alpha=lora_alpha,
-                   act_fn=getattr(module, "act_fn", None), hidden_act=getattr(module, "hidden_act", "silu"),
-                   expert_offset=expert_offset, device=gate.device, hybrid_shared=hybrid_shared,
-                   target_modules=target_modules, use_rslora=use_rslora)
+        new = cls(num_local_experts=total if num_local_experts is None else num_local_experts, num_experts=total,
+                  intermediate_size=getattr(module, "intermediate_size", inter),
+                  hidden_size=getattr(module, "hidden_dim", hidden), r=r, lora_alpha=lora_alpha,
+                  act_fn=getattr(module, "act_fn", None), hidden_act=getattr(module, "hidden_act", "silu"),
+                  expert_offset=expert_offset, device=gate.device, hybrid_shared=hybrid_shared,
+                  target_modules=target_modules, use_rslora=use_rslora)
+        new.swiglu_limit = limit
+        return new
 
     # ------------------------------------------------------------------ LoRA params
     def _create_lora_params(self, name, A_experts, B_experts, r, in_features, out_features, device=None):
@@ -331,7 +338,8 @@ class QLoRAMoeExperts(LoraModule, nn.Module):
             num_experts=self.num_local_experts, routing_weights=routing_weights, selected_experts=selected_experts,
             hidden_states=hidden_states, gate_proj=self._bank("gate"), up_proj=self._bank("up"),
             down_proj=self._bank("down"), gate_proj_lora_A=gA, gate_proj_lora_B=gB, up_proj_lora_A=uA,
-            up_proj_lora_B=uB, down_proj_lora_A=dA, down_proj_lora_B=dB, scaling=self._active_scaling())
+            up_proj_lora_B=uB, down_proj_lora_A=dA, down_proj_lora_B=dB, scaling=self._active_scaling(),
+            swiglu_limit=float(self.swiglu_limit or 0.0))
 
     def compute_dispatched(self, permute_tokens: Tensor, cumsum: Tensor, expert_scores: Tensor = None) -> Tensor:
         """The compute step of an expert-parallel forward (moe_experts.py:652-698): rows already grouped by local
@@ -341,7 +349,8 @@ class QLoRAMoeExperts(LoraModule, nn.Module):
         uA, uB = self._active_lora_views("up_proj")
         dA, dB = self._active_lora_views("down_proj")
         out = moe_experts_qlora_ep_compute(permute_tokens, cumsum, self._bank("gate"), self._bank("up"),
-                                           self._bank("down"), gA, gB, uA, uB, dA, dB, self._active_scaling())
+                                           self._bank("down"), gA, gB, uA, uB, dA, dB, self._active_scaling(),
+                                           float(self.swiglu_limit or 0.0))
         if expert_scores is not None:
             out = out * expert_scores.unsqueeze(1).to(out.dtype)
         return out
