@@ -317,6 +317,20 @@ int xq_merge_requant_nf4(const xq_weight* w, const void* lora_A, const void* lor
                          float scaling, void* codes_out, float* scales_out, void* workspace,
                          int64_t workspace_bytes, void* stream);
 
+/* int4 counterpart for a flat int4 weight with 128-element groups
+ * (in_features % 128 == 0): W' = bf16(bf16(deq(W)) + bf16(delta)) as
+ * xq_merge_dense forms it, re-encoded per group in the same pass.
+ * symmetric = 0: the rule of ops/quantize/int4_quantize.py:12-41
+ * (scale = max(absmax, 1e-12) * 2/15 in fp32, code = clamp(trunc(x * (1 /
+ * scale) + 8.5), 0, 15)), scales_out fp32 [N, K/128].  symmetric = 1: scale =
+ * bf16(absmax / 7), code = clamp(rne(x / scale), -7, 7) + 8, scales_out bf16
+ * [N, K/128] -- the rule of the int4 benchmark workload, which the reference
+ * has no module for.  codes_out [N, K/2] and scales_out may be the weight's
+ * own buffers when the scale type stays the same. */
+int xq_merge_requant_int4(const xq_weight* w, const void* lora_A, const void* lora_B, int lora_dtype, int r,
+                          float scaling, int symmetric, void* codes_out, void* scales_out, void* workspace,
+                          int64_t workspace_bytes, void* stream);
+
 /* ---- SwiGLU between gate/up and down ------------------------------------
  * Replaces fused_silu_and_mul (ops/fused_silu_and_mul.py:22-60 and its
  * backward): h = bf16(silu_fp32(gate)) * up, two roundings.  With row_w

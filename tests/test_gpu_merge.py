@@ -194,3 +194,48 @@ def test_merge_errors(hip_device):
         merge_requant_fp8(m._quant_weight(), m.lora_A, m.lora_B, 8, 2.0)      # block_fp8 only
     with pytest.raises(ValueError):
         m.merged_weight(torch.float16)
+
+
+@pytest.mark.parametrize("symmetric", [True, False])
+@pytest.mark.parametrize("N,K,r", [(384, 256, 0), (200, 384, 16), (1024, 512, 64)])
+def test_merge_requant_int4(hip_device, N, K, r, symmetric):
+    """Fused int4 merge + re-quantise (128-element groups) against the oracle's C quantizers applied to the merged
+    values the publish kernel writes -- the reference codec's rule (ops/quantize/int4_quantize.py:12-41, fp32 scales)
+    and the symmetric absmax/7 rule (bf16 scales): codes and scales byte for byte; then the module method."""
+    from xorl_amd.functional import merge_dense, merge_requant_int4
+    from xorl_amd.qlora import Int4QLoRALinear
+
+    rr = max(r, 8)
+    lin = torch.nn.Linear(K, N, bias=False)
+    with torch.no_grad():
+        lin.weight.copy_(gen((N, K), 0.02, 5 * N + K))
+        lin.weight[3].zero_()                          # a group of zeros: scale 0 (symmetric) or the 1e-12 floor
+    m = Int4QLoRALinear.from_module(lin, r=rr, lora_alpha=4 * rr, symmetric=symmetric).to(hip_device)
+    with torch.no_grad():
+        m.lora_A.copy_(gen((rr, K), 0.16, 5 * N + K + 1).to(hip_device))
+        m.lora_B.copy_(gen((N, rr), 0.16, 5 * N + K + 2).to(hip_device))
+        m.lora_B[3].zero_()
+        if r == 0:
+            m.lora_B.zero_()
+    s = m._active_scaling()
+    qw = m._quant_weight()
+    merged = merge_dense(qw, m.lora_A, m.lora_B, r, s, torch.bfloat16).cpu()
+    assert r == 0 or float((merged.float() - m._dequantize_weight().cpu().float()).abs().max()) > 0
+    assert torch.count_nonzero(merged[3]) == 0
+    codes, scales = merge_requant_int4(qw, m.lora_A, m.lora_B, r, s, symmetric)
+    if symmetric:
+        want_codes, want_scales = C.int4_quantize_sym_flat(merged.float().numpy(), 128)
+        assert scales.dtype == torch.bfloat16
+        got_scales = scales.cpu().view(torch.int16).numpy().view(np.uint16)
+    else:
+        want_codes, want_scales = C.int4_quantize_flat(merged.float().numpy(), 128)
+        assert scales.dtype == torch.float32
+        got_scales, want_scales = scales.cpu().numpy().view(np.uint32), np.asarray(want_scales).view(np.uint32)
+    assert np.array_equal(got_scales.reshape(-1), np.asarray(want_scales).reshape(-1))
+    assert np.array_equal(codes.cpu().numpy().reshape(-1), np.asarray(want_codes).reshape(-1))
+    m.merge_weights()
+    assert torch.count_nonzero(m.lora_B) == 0
+    assert torch.equal(m._read_packed_weight_uint8().reshape(-1).cpu(), codes.cpu().reshape(-1))
+    assert m._scale_dtypes["weight_scales"] == scales.dtype
+    w_new = m._dequantize_weight().cpu().float()
+    assert (w_new - merged.float()).abs().mean() / merged.float().abs().mean() < 0.16   # 15 or 16 levels per group: mean error ~ absmax / 28

@@ -564,7 +564,12 @@ def test_expert_merge_weights_matches_reference_arithmetic(hip_device, fmt, hybr
     deq(W) + delta.to(deq dtype) -- a bf16 add for nvfp4 / nf4 (their decoders return bf16), an fp32 add for
     block_fp8 --, nvfp4 blends each expert's fresh amax into the running one (lerp by ema_decay) and re-quantises
     against it.  The module's new packed bytes, scales, global scales and running amax must equal, byte for byte,
-    the oracle's quantizer applied to that sum built from the oracle's decode; merging twice exercises the blend."""
+    the oracle's quantizer applied to that sum built from the oracle's decode; merging twice exercises the blend.
+    block_fp8 banks go through the dense fused merge pass expert by expert, which forms the update itself: there the
+    quantizer is checked bit for bit on the pass's own fp32 sums and to neighbouring codes on the oracle's."""
+    from xorl_amd import _C
+    from xorl_amd import functional as Fn
+
     E, H, I, r = 4, 128, 256, 8
     m, banks = _make_experts(fmt, E, H, I, r, hybrid, seed=80, device=hip_device)
     dt = torch.float32 if fmt == "block_fp8" else torch.bfloat16
@@ -612,7 +617,17 @@ def test_expert_merge_weights_matches_reference_arithmetic(hip_device, fmt, hybr
             for e in range(E):
                 x = merged[e].float().numpy()
                 if fmt == "block_fp8":
-                    per.append(C.fp8_quantize(x, 128, 1.0))
+                    # the fused pass forms the update itself (split-bf16 MFMA products, fp32 sums): its own fp32 sums, read
+                    # through the publish mode of the same kernel, are within 3e-5 of the oracle's (the update dominates the sum
+                    # here, and a split-bf16 product drops the lo x lo terms: 2^-16 relative), and the bank must hold
+                    # the oracle quantizer applied to them bit for bit
+                    qw = Fn.QuantWeight("block_fp8", _C.XQ_LAYOUT_FLAT, getattr(m, f"{p}_packed")[e],
+                                        getattr(m, f"{p}_block_scales")[e], torch.float32, K, N, 128)
+                    A, B = m._active_lora_views(f"{p}_proj")
+                    own = Fn.merge_dense(qw, B[e if B.shape[0] > 1 else 0], A[e if A.shape[0] > 1 else 0], m.active_r,
+                                         m._active_scaling(), torch.float32).cpu()
+                    assert R.max_rel_err(own, merged[e]) <= 3e-5, (round_, p, e)
+                    per.append(C.fp8_quantize(own.numpy(), 128, 1.0) + C.fp8_quantize(x, 128, 1.0))
                 elif fmt == "nf4":
                     per.append(C.nf4_quantize_gkn(x, 64))
                 else:
@@ -630,6 +645,12 @@ def test_expert_merge_weights_matches_reference_arithmetic(hip_device, fmt, hybr
                 if fmt == "block_fp8":
                     s = getattr(m, f"{p}_block_scales")[e].cpu().contiguous().view(torch.float32).numpy()
                     assert np.array_equal(s.view(np.uint32).ravel(), per[e][1].view(np.uint32).ravel()), (round_, p, e)
+                    # against the oracle's own sums: scales to 5e-5, codes equal or neighbours (a sum on a rounding edge)
+                    assert np.allclose(s.ravel(), per[e][3].ravel(), rtol=5e-5, atol=0)
+                    gb, wb = got_packed[e].ravel().astype(np.int32), per[e][2].ravel().astype(np.int32)
+                    assert float((gb != wb).mean()) <= 5e-3
+                    sg, sw = np.where(gb & 0x80, -(gb & 0x7f), gb & 0x7f), np.where(wb & 0x80, -(wb & 0x7f), wb & 0x7f)
+                    assert bool(((np.abs(sg - sw) <= 1) | ((np.abs(sg) <= 1) & (np.abs(sw) <= 1))).all())
                 elif fmt == "nf4":
                     s = getattr(m, f"{p}_scales")[e].cpu().contiguous().view(torch.float32).numpy()
                     assert np.array_equal(s.view(np.uint32).ravel(), per[e][1].view(np.uint32).ravel()), (round_, p, e)

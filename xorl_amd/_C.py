@@ -120,6 +120,8 @@ _SIGNATURES = {
     "xq_merge_requant_nvfp4": (_INT, [_W, _P, _P, _INT, _INT, _F, _P, _P, _P, _P, _P, _I64, _P]),
     # w, A, B, lora_dtype, r, scaling, codes_out, scales_out, workspace, workspace_bytes, stream
     "xq_merge_requant_nf4": (_INT, [_W, _P, _P, _INT, _INT, _F, _P, _P, _P, _I64, _P]),
+    # w, A, B, lora_dtype, r, scaling, symmetric, codes_out, scales_out, workspace, workspace_bytes, stream
+    "xq_merge_requant_int4": (_INT, [_W, _P, _P, _INT, _INT, _F, _INT, _P, _P, _P, _I64, _P]),
     # gate, up, ld_in, row_w, h, ld_h, rows, cols, stream
     "xq_silu_mul_fwd": (_INT, [_P, _P, _I64, _P, _P, _I64, _I64, _I64, _P]),
     # gate, up, ld_in, dh, ld_dh, row_w, dgate, dup, ld_out, d_row_w, rows, cols, stream

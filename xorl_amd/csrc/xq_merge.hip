@@ -45,10 +45,13 @@ struct MergeArgs {
     const bf16_t* Ah;    // ([Kpad][r_pad], row = k)
     const bf16_t* Al;
     int32_t mode;        // 0: bf16 out (publish arithmetic), 1: fp32 out, 2: block-fp8 requantise,
-                         // 3: absmax of the mode-0 values only, 4 / 5: nvfp4 / nf4 requantise of the mode-0 values
+                         // 3: absmax of the mode-0 values only, 4 / 5: nvfp4 / nf4 requantise of the mode-0 values,
+                         // 6 / 7: int4 requantise of the mode-0 values, 128-element groups along K (6: scale =
+                         // bf16(absmax / 7), codes rne(x / scale) in [-7, 7] + 8; 7: the reference's rule, fp32 scales)
     void* out;           // mode 0/1: [N, K]
     uint8_t* packed_out; // mode 2: [N, K] e4m3 bytes    } both may alias the inputs: a block reads its tile and its
     float* scales_out;   // mode 2: [ceil(N/128), ceil(K/128)] } scale before it writes them, and touches no other
+                         // mode 5: [N, K/64] fp32; mode 6: [N, K/128] bf16; mode 7: [N, K/128] fp32
     float* amax_out;     // mode 3: one float, zeroed before the launch; receives max |value| over the matrix
     const float* gamax;  // mode 4: the tensor-level amax the scales are derived from (one float on the device)
     uint8_t* codes_out;  // mode 4 / 5: [N, K/2] code pairs     } may alias the inputs (tile-local, read before written);
@@ -108,7 +111,8 @@ __global__ void __launch_bounds__(256) merge_prep_kernel(MergeArgs g, int npad, 
     }
 }
 
-// REQ: the block-fp8 re-quantise mode (results are held in registers until the tile's absmax is known).
+// REQ: the block-fp8 re-quantise mode (results are held in registers until the tile's absmax is known) and, for an
+// int4 weight, the int4 one (held until the row's 128-element group, which is the tile's whole row, is known).
 // 512 threads per tile: 32 result registers per thread in that mode, so that two blocks (16 waves) fit a CU.
 template <int FMT, int RP, bool REQ>
 __global__ void __launch_bounds__(512, 4) merge_kernel(MergeArgs g) {
@@ -311,6 +315,42 @@ __global__ void __launch_bounds__(512, 4) merge_kernel(MergeArgs g) {
             }
         }
     }
+    if constexpr (REQ && FMT == XQ_FMT_INT4) {
+        // ---- 3a. int4, one group per tile row: the four lanes of a row hold its 128 values
+        float ga = amax;
+        ga = fmaxf(ga, __shfl_xor(ga, 1, 64));
+        ga = fmaxf(ga, __shfl_xor(ga, 2, 64));
+        if (n >= g.N) return;
+        const int64_t gi = (n * g.K + k0) >> 7;
+        uint32_t pk[4] = {0u, 0u, 0u, 0u};
+        if (g.mode == 6) {
+            // scale = bf16(absmax / 7); code = clamp(rne(x / scale), -7, 7) + 8, all zero codes (8) for a zero group
+            const bf16_t sb = to_bf16(ga / 7.0f);
+            const float sc = bf16_to_f32(sb);
+            if ((tid & 3) == 0) ((bf16_t*)g.scales_out)[gi] = sb;
+#pragma unroll
+            for (int i = 0; i < 32; ++i) {
+                const float q = sc > 0.0f ? __builtin_amdgcn_fmed3f(__builtin_rintf(m[i] / sc), -7.0f, 7.0f) : 0.0f;
+                pk[i >> 3] |= (uint32_t)((int)q + 8) << (4 * (i & 7));
+            }
+        } else {
+            // ops/quantize/int4_quantize.py:12-41: scale = max(absmax, 1e-12) * (2/15); code = clamp(trunc(x * (1 / scale)
+            // + 8.5), 0, 15) with the product and the sum rounded separately
+            const float sc = fmaxf(ga, 1e-12f) * (float)(2.0 / 15.0), inv = 1.0f / sc;
+            if ((tid & 3) == 0) g.scales_out[gi] = sc;
+#pragma unroll
+            for (int i = 0; i < 32; ++i) {
+                const int q = (int)__fadd_rn(__fmul_rn(m[i], inv), 8.5f);
+                pk[i >> 3] |= (uint32_t)(q < 0 ? 0 : q > 15 ? 15 : q) << (4 * (i & 7));
+            }
+        }
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int k = k0 + h * 64 + rcol;
+            if (k < g.K) *(u32x2*)(g.codes_out + ((n * g.K + k) >> 1)) = u32x2{pk[2 * h], pk[2 * h + 1]};
+        }
+        return;
+    }
     if (!REQ) {
         if (g.mode == 3) {       // tile absmax -> one atomic per block (values are non-negative: integer order = float order)
 #pragma unroll
@@ -448,7 +488,8 @@ static int launch_merge(const xq_weight* w, const void* A, const void* B, int lo
         merge_prep_kernel<<<dim3((unsigned)xq_cdiv((npad + kpad) * g.r_pad, 256)), 256, 0, stream>>>(g, (int)npad, (int)kpad);
     if (w->format == XQ_FMT_FP8) rc = mode == 2 ? launch_merge_fmt<XQ_FMT_FP8, true>(g, grid, stream, who)
                                                 : launch_merge_fmt<XQ_FMT_FP8, false>(g, grid, stream, who);
-    else if (w->format == XQ_FMT_INT4) rc = launch_merge_fmt<XQ_FMT_INT4, false>(g, grid, stream, who);
+    else if (w->format == XQ_FMT_INT4) rc = mode >= 6 ? launch_merge_fmt<XQ_FMT_INT4, true>(g, grid, stream, who)
+                                                      : launch_merge_fmt<XQ_FMT_INT4, false>(g, grid, stream, who);
     else if (w->format == XQ_FMT_NF4) rc = launch_merge_fmt<XQ_FMT_NF4, false>(g, grid, stream, who);
     else rc = launch_merge_fmt<XQ_FMT_NVFP4, false>(g, grid, stream, who);
     if (timed) xq_profile_mark_end(stream);
@@ -498,6 +539,19 @@ extern "C" int xq_merge_requant_nvfp4(const xq_weight* w, const void* lora_A, co
     nv.gamax = global_amax; nv.codes_out = (uint8_t*)codes_out; nv.bscale_out = (uint8_t*)block_scales_out; nv.gscale_out = global_scale_out;
     return launch_merge(w, lora_A, lora_B, lora_dtype, r, scaling, 4, nullptr, nullptr, nullptr, workspace, workspace_bytes,
                         (hipStream_t)stream, "xq_merge_requant_nvfp4", nv);
+}
+
+extern "C" int xq_merge_requant_int4(const xq_weight* w, const void* lora_A, const void* lora_B, int lora_dtype, int r,
+                                     float scaling, int symmetric, void* codes_out, void* scales_out, void* workspace,
+                                     int64_t workspace_bytes, void* stream) {
+    XQ_REQUIRE(w && w->format == XQ_FMT_INT4 && w->layout == XQ_LAYOUT_FLAT && w->group == 128 && w->cols % 128 == 0,
+               "xq_merge_requant_int4: the weight must be flat int4 with 128-element groups and in_features %% 128 == 0");
+    XQ_REQUIRE(codes_out && scales_out && xq_aligned(codes_out, 8) && xq_aligned(scales_out, 4),
+               "xq_merge_requant_int4: NULL or misaligned output");
+    Nvfp4Out nv;
+    nv.codes_out = (uint8_t*)codes_out;
+    return launch_merge(w, lora_A, lora_B, lora_dtype, r, scaling, symmetric ? 6 : 7, nullptr, nullptr, (float*)scales_out,
+                        workspace, workspace_bytes, (hipStream_t)stream, "xq_merge_requant_int4", nv);
 }
 
 extern "C" int xq_merge_requant_nf4(const xq_weight* w, const void* lora_A, const void* lora_B, int lora_dtype, int r,

@@ -800,6 +800,32 @@ def merge_requant_nvfp4(qw: QuantWeight, lora_A: Optional[Tensor], lora_B: Optio
     return codes, bscales.view(torch.float8_e4m3fn), gscale
 
 
+def merge_requant_int4(qw: QuantWeight, lora_A: Optional[Tensor], lora_B: Optional[Tensor], r: int, scaling: float,
+                       symmetric: bool, codes_out: Optional[Tensor] = None,
+                       scales_out: Optional[Tensor] = None) -> Tuple[Tensor, Tensor]:
+    """Flat int4 with 128-element groups only: Q(bf16(deq(W)) + bf16(scaling * B @ A)) in one pass over the packed
+    bytes.  `symmetric` picks the quantizer: False = ops/quantize/int4_quantize.py:12-41 (fp32 scales), True =
+    scale bf16(absmax / 7), codes rne(x / scale) + 8 (bf16 scales).  Returns (codes uint8 [N, K/2], scales [N, K/128]);
+    pass the weight's own buffers to update in place."""
+    _C.require_hip(qw.packed, lora_A, lora_B)
+    if qw.fmt != "int4":
+        raise _C.XqError(f"merge_requant_int4: the weight must be int4, got {qw.fmt}")
+    dev = qw.packed.device
+    A = lora_A[:r].contiguous() if r > 0 else None
+    B = lora_B[:, :r].contiguous() if r > 0 else None
+    if codes_out is None:
+        codes_out = torch.empty(qw.rows, qw.cols // 2, dtype=torch.uint8, device=dev)
+    if scales_out is None:
+        scales_out = torch.empty(qw.rows, qw.cols // 128, dtype=torch.bfloat16 if symmetric else torch.float32, device=dev)
+    ws_bytes = _C.lib().xq_merge_workspace_bytes(qw.rows, qw.cols, r)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    w = qw.c()
+    _C.check(_C.lib().xq_merge_requant_int4(ctypes.byref(w), _C.ptr(A), _C.ptr(B), _lora_dt(A), r, float(scaling),
+                                            1 if symmetric else 0, codes_out.data_ptr(), scales_out.data_ptr(),
+                                            ws.data_ptr(), ws_bytes, _C.stream_ptr(dev)))
+    return codes_out, scales_out
+
+
 def merge_requant_nf4(qw: QuantWeight, lora_A: Optional[Tensor], lora_B: Optional[Tensor], r: int, scaling: float,
                       codes_out: Optional[Tensor] = None, scales_out: Optional[Tensor] = None) -> Tuple[Tensor, Tensor]:
     """NF4 only: nf4_quantize(deq(W) + scaling * B @ A) in one pass over the packed bytes (merge_weights +

@@ -668,6 +668,26 @@ class Int4QLoRALinear(QLoRALinear):
         self.weight_scales = self._to_uint8(scales)
         self._aqn_step_cache = None
 
+    def merge_weights(self, ema_decay: float = 0.1) -> None:
+        """Decode, add the LoRA update and re-encode with fresh group scales (this module's own rule, symmetric or the
+        reference codec's) in one fused pass over the bytes; sharded (DTensor) state, group sizes other than 128 and
+        ranks beyond the fused kernels' take the generic path."""
+        from ..functional import merge_requant_int4
+
+        sdt = torch.bfloat16 if self.symmetric else torch.float32
+        if (_is_dtensor(self.packed_weight_f32) or _is_dtensor(self.lora_A) or self.active_r > MAX_FUSED_RANK
+                or not self.packed_weight_f32.is_cuda or self.quant_group_size != 128 or self.in_features % 128
+                or self._scale_dtypes.get("weight_scales") != sdt):
+            return super().merge_weights(ema_decay)
+        with torch.no_grad():
+            codes, scales = merge_requant_int4(self._quant_weight(), self.lora_A, self.lora_B, self.active_r,
+                                               self._active_scaling(), self.symmetric)
+            self._write_packed_weight(codes.reshape(-1))
+            self.weight_scales = self._to_uint8(scales)
+            self._aqn_step_cache = None
+            nn.init.kaiming_uniform_(self.lora_A, a=math.sqrt(5))
+            self.lora_B.zero_()
+
     def _quant_weight(self) -> QuantWeight:
         return QuantWeight("int4", _C.XQ_LAYOUT_FLAT, self._read_packed_weight_uint8(), self.weight_scales,
                            self._scale_dtypes["weight_scales"], self.out_features, self.in_features,

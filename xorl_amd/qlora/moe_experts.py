@@ -433,6 +433,29 @@ class BlockFP8QLoRAMoeExperts(QLoRAMoeExperts):
                            getattr(self, f"{proj_name}_block_scales"), torch.float32, K, N, 128,
                            num_experts=self.num_local_experts)
 
+    def merge_weights(self, ema_decay: float = 0.1, experts_per_step: int = 16) -> None:
+        """Each expert's [K, N] slice is decoded, updated and re-encoded with fresh 128x128 block scales by the dense
+        fused merge pass, in place in the bank (moe_experts.py:1134-1146): an expert's slice is a flat block-fp8
+        matrix of K rows, and its update A_e [K, r] @ B_e [r, N] is that pass's (lora_B @ lora_A) with the factors'
+        roles exchanged.  No decoded bank is ever held.  Ranks beyond the fused pass take the generic path."""
+        from ..functional import MAX_FUSED_RANK, merge_requant_fp8
+
+        packed0 = getattr(self, "gate_packed")
+        if self.active_r > MAX_FUSED_RANK or packed0 is None or not packed0.is_cuda:
+            return super().merge_weights(ema_decay, experts_per_step)
+        with torch.no_grad():
+            s = self._active_scaling()
+            for name in ("gate", "up", "down"):
+                K, N = self._proj_dims(name)
+                packed = getattr(self, f"{name}_packed")
+                scales = getattr(self, f"{name}_block_scales")
+                A, B = self._active_lora_views(f"{name}_proj")       # [E|1, K, r], [E|1, r, N]
+                for e in range(self.num_local_experts):
+                    qw = QuantWeight("block_fp8", _C.XQ_LAYOUT_FLAT, packed[e], scales[e], torch.float32, K, N, 128)
+                    merge_requant_fp8(qw, B[e if B.shape[0] > 1 else 0], A[e if A.shape[0] > 1 else 0],
+                                      self.active_r, s, packed_out=packed[e], scales_out=scales[e])
+        self.reset_lora_parameters()
+
     @torch.compiler.disable
     def dequantize_all_experts(self, proj_name: str, K: int, N: int) -> Tensor:
         import ctypes
