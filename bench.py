@@ -44,9 +44,9 @@ MEASURED_TRAFFIC = {
     # gemm_256_kernel<int4, T=128> in 4 K splits + splitk_reduce_kernel: mean of the forward and dgrad launches
     # (64 MiB of it are the fp32 partial sums written and read back)
     0: (109.6 * 2 ** 20, "profiles/gemm_128_int4_linear_m512.txt", 0.04315),
-    # gemm_256_kernel<fp8>: mean over the 5 launches of a step (gate, up and down
+    # gemm_dtl16_kernel (dense block-fp8, 256x256 tiles): mean over the 5 launches of a step (gate, up and down
     # forward, d_h, dx as one sum over the gate and up weights)
-    1: (1079.3 * 2 ** 20, "profiles/gemm_256_fp8_mlp_m8192.txt", 0.84558),
+    1: (1070.2 * 2 ** 20, "profiles/gemm_dtl16_fp8_mlp_m8192.txt", 0.7876),
     # gemm_256_kernel<nvfp4>, 256x256 tiles (whole rounds; trailing rows in K splits) and 128x128 tiles
     # (+ splitk_reduce_kernel): mean over the 12 launches of a step, fp32 partial sums included
     2: (185.7 * 2 ** 20, "profiles/gemm_256_nvfp4_attn_m4096.txt", 0.14304),
@@ -455,10 +455,10 @@ def main():
                    "tokens": M, "hidden": H, "intermediate": I, "lora_r": R, "format": "block_fp8"},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": BF16_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / BF16_MFMA_PEAK_TFLOPS, "traffic": traffic, "traffic_source": traffic_source,
-                     "kernel": "gemm_256_kernel<fp8, contract_cols true|false, dense> (fused fp8 dequant-GEMM: gate, up "
-                               "and down forward, down dgrad, gate+up dgrad as one sum)"
+                     "kernel": "gemm_dtl16_kernel<contract_cols true|false, 8 waves> (dense fused block-fp8 dequant-GEMM, "
+                               "256x256x64 tiles: gate, up and down forward, down dgrad, gate+up dgrad as one sum)"
                                if not args.unfused else
-                               "gemm_256_kernel<fp8, contract_cols true|false, dense> (fused fp8 dequant-GEMM, "
+                               "gemm_dtl16_kernel<contract_cols true|false, 8 waves> (dense fused block-fp8 dequant-GEMM, "
                                "forward and dgrad launches)",
                      "launches": n.value, "avg_launch_ms": avg_launch_ms},
         "cpu_baseline": cpu,

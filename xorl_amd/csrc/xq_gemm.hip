@@ -46,20 +46,27 @@ static int launch_256_one(const G256Args& f, dim3 grid, hipStream_t s, const cha
     return XQ_OK;
 }
 
-// Dense block-fp8 launches on large unsplit tiles run gemm_dtl16_kernel (1, the default) or gemm_256_kernel (0): a
+// Block-fp8 launches on large unsplit tiles (dense and expert banks) run gemm_dtl16_kernel (1, the default) or gemm_256_kernel (0): a
 // process-wide switch for tests and A/B measurements, XQ_FP8_DIRECT in the environment sets it at load time.
 static std::atomic<int> g_fp8_direct{[] { const char* e = getenv("XQ_FP8_DIRECT"); return e ? atoi(e) : 1; }()};
 
-static int launch_dtl16(const G256Args& f, bool cc, dim3 grid, hipStream_t s, const char* who) {
+static int launch_dtl16(const G256Args& f, bool cc, bool grouped, dim3 grid, hipStream_t s, const char* who) {
     static std::atomic<bool> attr_set{false};
     if (!attr_set) {
-        int rc = raise_lds_limit(gemm_dtl16_kernel<true, 8>, GeoDtl::lds_total(), who);
-        if (!rc) rc = raise_lds_limit(gemm_dtl16_kernel<false, 8>, GeoDtl::lds_total(), who);
+        int rc = raise_lds_limit(gemm_dtl16_kernel<true, 8, false>, GeoDtl::lds_total(), who);
+        if (!rc) rc = raise_lds_limit(gemm_dtl16_kernel<false, 8, false>, GeoDtl::lds_total(), who);
+        if (!rc) rc = raise_lds_limit(gemm_dtl16_kernel<true, 8, true>, GeoDtl::lds_total(), who);
+        if (!rc) rc = raise_lds_limit(gemm_dtl16_kernel<false, 8, true>, GeoDtl::lds_total(), who);
         if (rc) return rc;
         attr_set = true;
     }
-    if (cc) gemm_dtl16_kernel<true, 8><<<grid, 512, GeoDtl::lds_total(), s>>>(f);
-    else gemm_dtl16_kernel<false, 8><<<grid, 512, GeoDtl::lds_total(), s>>>(f);
+    if (grouped) {
+        if (cc) gemm_dtl16_kernel<true, 8, true><<<grid, 512, GeoDtl::lds_total(), s>>>(f);
+        else gemm_dtl16_kernel<false, 8, true><<<grid, 512, GeoDtl::lds_total(), s>>>(f);
+    } else {
+        if (cc) gemm_dtl16_kernel<true, 8, false><<<grid, 512, GeoDtl::lds_total(), s>>>(f);
+        else gemm_dtl16_kernel<false, 8, false><<<grid, 512, GeoDtl::lds_total(), s>>>(f);
+    }
     return XQ_OK;
 }
 
@@ -288,12 +295,15 @@ static int launch_tile_gemm_t(const xq_weight* w, bool contract_cols, const bf16
             dim3 grid(persistent ? persistent_grid(tiles_m * tiles_n) : (unsigned)(tiles_m * tiles_n), (unsigned)ksplit);
             const bool timed = xq_profile_mark_begin(stream, 2.0 * (double)n_rows * g.Nout * ((double)g.Kc + g.r_pad));
             int rc;
-            // dense block-fp8 on large unsplit tiles: the kernel that brings both operand tiles straight into LDS and decodes
-            // after the fragment read (xq_gemm_dtl.h), one block per tile
+            // block-fp8 on large unsplit tiles, dense or expert banks: the kernel that brings both operand tiles straight into LDS
+            // and decodes after the fragment read (xq_gemm_dtl.h), one block per tile
             const int nk_all = g.Kc / BK;
-            if (g_fp8_direct && w->format == XQ_FMT_FP8 && T == 256 && !grouped && ksplit == 1 && nk_all >= 3 &&
-                nk_all <= 2 * GeoDtl::SCL_MAX && (!two || (f.nk1 % 2 == 0 && f.nk1 >= 2)))
-                rc = launch_dtl16(f, contract_cols, dim3((unsigned)(tiles_m * tiles_n)), stream, who);
+            // (two matrices: the second one starts on a scale-block boundary of the contraction, or -- two banks side by side
+            // in a forward -- on a tile boundary of the columns)
+            const bool two_ok = !two || ((grouped && !contract_cols) ? f.ncols1 % 256 == 0 : (f.nk1 % 2 == 0 && f.nk1 >= 2));
+            if (g_fp8_direct && w->format == XQ_FMT_FP8 && T == 256 && ksplit == 1 && nk_all >= 3 &&
+                nk_all <= 2 * GeoDtl::SCL_MAX && two_ok && (!grouped || g.wcols % 16 == 0))
+                rc = launch_dtl16(f, contract_cols, grouped, dim3((unsigned)(tiles_m * tiles_n)), stream, who);
             else if (w->format == XQ_FMT_FP8) rc = launch_256<XQ_FMT_FP8>(f, contract_cols, grouped, T, grid, stream, who);
             else if (w->format == XQ_FMT_INT4) rc = launch_256<XQ_FMT_INT4>(f, contract_cols, grouped, T, grid, stream, who);
             else if (w->format == XQ_FMT_NF4) rc = launch_256<XQ_FMT_NF4>(f, contract_cols, grouped, T, grid, stream, who);

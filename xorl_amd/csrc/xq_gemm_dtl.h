@@ -64,7 +64,13 @@ __device__ __forceinline__ u32x2 dtl_decode4(uint32_t w, float sc) {
 // with its 256 accumulator registers (one wave per SIMD): every weight value is then decoded by exactly one wave -- half
 // the conversions per MFMA of the eight-wave form, whose column blocks are shared by two waves -- and an activation
 // fragment feeds the same four MFMAs.
-template <bool CC, int NW>
+//
+// GROUPED: the rows are in expert order and W is a bank of matrices of one shape (G256Args: offsets, tile_prefix,
+// packed_stride, scale_stride, a_rows); a block finds the expert of its row tile, reads and writes that expert's rows only,
+// and is gone if the launch holds fewer row tiles than its grid covers.  !CC is a bank's forward (optionally over two
+// banks side by side: column tiles from ncols1 on take the second bank), CC its dgrad (optionally one sum over two banks:
+// K-steps from nk1 on read the second one).
+template <bool CC, int NW, bool GROUPED = false>
 __global__ void __launch_bounds__(NW * 64, NW == 8 ? 2 : 1) gemm_dtl16_kernel(G256Args g) {
     using D = GeoDtl;
     constexpr int T = 256, TN = 4, NT = NW * 64;
@@ -79,19 +85,62 @@ __global__ void __launch_bounds__(NW * 64, NW == 8 ? 2 : 1) gemm_dtl16_kernel(G2
 
     int pid_m, pid_n;
     {
-        const int nb = g.tiles_m * g.tiles_n;
+        // (grouped: the grid covers an upper bound of the row tiles; the order is laid over the tiles there are, so that
+        // the blocks with nothing to do are not all one XCD's)
+        const int nb = (GROUPED ? g.tile_prefix[g.num_experts] : g.tiles_m) * g.tiles_n;
         const int b = blockIdx.x, per = nb >> 3;
+        if (GROUPED && b >= nb) return;
         const int logical = (b < per * 8) ? (b & 7) * per + (b >> 3) : b;
-        constexpr int GM = 4;
-        const int width = GM * g.tiles_n;
-        const int grp = logical / width, first_m = grp * GM;
-        const int gsz = min(g.tiles_m - first_m, GM);
-        const int in = logical - grp * width;
-        pid_m = first_m + in % gsz;
-        pid_n = in / gsz;
+        if constexpr (GROUPED) {
+            pid_m = logical / g.tiles_n;      // all column tiles of a row tile side by side: an XCD stays on one expert's matrix
+            pid_n = logical - pid_m * g.tiles_n;
+        } else {
+            constexpr int GM = 4;
+            const int width = GM * g.tiles_n;
+            const int grp = logical / width, first_m = grp * GM;
+            const int gsz = min(g.tiles_m - first_m, GM);
+            const int in = logical - grp * width;
+            pid_m = first_m + in % gsz;
+            pid_n = in / gsz;
+        }
     }
-    const int64_t row0 = (int64_t)pid_m * T;
+    // the tile: expert, rows it may read and write, output columns (n0) and the same columns within their bank (n0w)
+    int e = 0;
+    int64_t row0 = (int64_t)pid_m * T, row_end = g.M;
+    if constexpr (GROUPED) {
+        // thread t looks at expert t (t + NT, ...): one memory round trip instead of a search's chain of dependent loads
+        __shared__ int sh_tile[3];
+        if (tid == 0) sh_tile[0] = -1;
+        __syncthreads();
+        for (int t = tid; t < g.num_experts; t += NT) {
+            const int lo = g.tile_prefix[t], hi = g.tile_prefix[t + 1];
+            if (lo <= pid_m && pid_m < hi) {
+                sh_tile[0] = t;
+                sh_tile[1] = g.offsets[t] + (pid_m - lo) * T;
+                sh_tile[2] = g.offsets[t + 1];
+            }
+        }
+        __syncthreads();
+        e = __builtin_amdgcn_readfirstlane(sh_tile[0]);
+        if (e < 0) return;                    // (cannot happen for a row tile below tile_prefix[num_experts])
+        row0 = __builtin_amdgcn_readfirstlane(sh_tile[1]);
+        row_end = __builtin_amdgcn_readfirstlane(sh_tile[2]);
+    }
     const int n0 = pid_n * T;
+    int n0w = n0, bank_width = g.Nout;
+    const uint8_t* Wb = g.W + (int64_t)e * g.packed_stride;
+    const float* Sb = (const float*)(g.scales + (int64_t)e * g.scale_stride);
+    const float* Sb2 = g.W2 != nullptr ? (const float*)(g.scales2 + (int64_t)e * g.scale_stride) : nullptr;
+    const bf16_t* su_b = g.su;
+    const bf16_t* lr_b = g.lora_right;
+    if constexpr (GROUPED && !CC) {
+        if (g.W2 != nullptr) {
+            bank_width = g.ncols1;
+            if (n0 >= g.ncols1) {
+                Wb = g.W2 + (int64_t)e * g.packed_stride; Sb = Sb2; su_b = g.su2; lr_b = g.lora_right2; n0w = n0 - g.ncols1;
+            }
+        }
+    }
     const int nk = g.Kc / D::BK;
     const int scols = (g.wcols + 127) >> 7;
 
@@ -102,7 +151,10 @@ __global__ void __launch_bounds__(NW * 64, NW == 8 ? 2 : 1) gemm_dtl16_kernel(G2
     for (int p = 0; p < AP; ++p) {
         const int rt = (wave * AP + p) * 8 + (lane >> 3);
         int64_t r = row0 + rt;
-        r = r < g.M ? r : g.M - 1;
+        r = r < row_end ? r : row_end - 1;
+        if constexpr (GROUPED) {
+            if (g.a_rows) r = g.a_rows[r];
+        }
         a_src[p] = g.A + r * g.lda + (((lane & 7) ^ ((rt >> 1) & 7)) << 3);
     }
     const uint8_t* w_src[WP];
@@ -110,19 +162,20 @@ __global__ void __launch_bounds__(NW * 64, NW == 8 ? 2 : 1) gemm_dtl16_kernel(G2
     for (int q = 0; q < WP; ++q) {
         if (CC) {
             const int rt = (wave * WP + q) * 16 + (lane >> 2);
-            const int wr = min(n0 + rt, g.wrows - 1);
-            w_src[q] = g.W + (int64_t)wr * g.wcols + (((lane & 3) ^ ((rt >> 2) & 3)) << 4);
+            const int wr = min(n0w + rt, g.wrows - 1);
+            w_src[q] = Wb + (int64_t)wr * g.wcols + (((lane & 3) ^ ((rt >> 2) & 3)) << 4);
         } else {
             const int kr = (wave * WP + q) * 4 + (lane >> 4);
-            const int wc = min(n0 + (((lane & 15) ^ (kr & 7)) << 4), g.wcols - 16);
-            w_src[q] = g.W + (int64_t)kr * g.wcols + wc;
+            const int wc = min(n0w + (((lane & 15) ^ (kr & 7)) << 4), g.wcols - 16);
+            w_src[q] = Wb + (int64_t)kr * g.wcols + wc;
         }
     }
     const int64_t w_kstep = CC ? D::BK : (int64_t)D::BK * g.wcols;
-    // contraction over two matrices of one shape (dense dgrad of gate and up as one sum, G256Args::W2): K-steps from nk1 on
-    // read the second matrix, from its first row block
-    const int nk1 = (!CC && g.W2 != nullptr) ? g.nk1 : (1 << 30);
-    const int64_t w2_delta = (!CC && g.W2 != nullptr) ? (g.W2 - g.W) - (int64_t)nk1 * w_kstep : 0;
+    // contraction over two matrices of one shape (dgrad of gate and up as one sum, G256Args::W2; dense: !CC, banks: CC):
+    // K-steps from nk1 on read the second matrix (the same expert's), from its first K-step
+    constexpr bool TWO_K = GROUPED ? CC : !CC;
+    const int nk1 = (TWO_K && g.W2 != nullptr) ? g.nk1 : (1 << 30);
+    const int64_t w2_delta = (TWO_K && g.W2 != nullptr) ? (g.W2 - g.W) - (int64_t)nk1 * w_kstep : 0;
     auto issue_part = [&](int kt, int stage, int part) {
         unsigned char* a = dsm + stage * D::STAGE_BYTES + wave * (AP * 1024);
         unsigned char* w = dsm + stage * D::STAGE_BYTES + D::A_STAGE_BYTES + wave * (WP * 1024);
@@ -139,15 +192,13 @@ __global__ void __launch_bounds__(NW * 64, NW == 8 ? 2 : 1) gemm_dtl16_kernel(G2
         const int nkb = (nk + 1) >> 1;
         for (int i = tid; i < 2 * nkb; i += NT) {
             const int blk = i / nkb, kb = i - blk * nkb;
-            const int nn = n0 + blk * 128;
+            const int nn = n0w + blk * 128;
+            const bool second = 2 * kb >= nk1;                      // (nk1 is even: the matrices change on a scale-block boundary)
+            const float* sp = second ? Sb2 : Sb;
+            const int kb1 = second ? kb - (nk1 >> 1) : kb;
             float v;
-            if (CC) {
-                v = ((const float*)g.scales)[(min(nn, g.wrows - 1) >> 7) * scols + kb];
-            } else {
-                const bool second = 2 * kb >= nk1;                  // (nk1 is even: the matrices change on a scale-block boundary)
-                const float* sp = second ? (const float*)g.scales2 : (const float*)g.scales;
-                v = sp[(int64_t)(second ? kb - (nk1 >> 1) : kb) * scols + (min(nn, g.wcols - 1) >> 7)];
-            }
+            if (CC) v = sp[(min(nn, g.wrows - 1) >> 7) * scols + kb1];
+            else v = sp[(int64_t)kb1 * scols + (min(nn, g.wcols - 1) >> 7)];
             s_lds[blk * D::SCL_MAX + kb] = v;
         }
         __syncthreads();
@@ -336,15 +387,16 @@ __global__ void __launch_bounds__(NW * 64, NW == 8 ? 2 : 1) gemm_dtl16_kernel(G2
     __syncthreads();
     if (g.r_pad > 0) {
         const int rp = g.r_pad, steps = (rp + 31) >> 5, cpr = steps << 2, have = rp >> 3;
+        const bf16_t* lr = lr_b + (int64_t)e * bank_width * rp;
         for (int idx = tid; idx < T * cpr; idx += NT) {
             const int r = idx / cpr, c = idx - r * cpr;
             int64_t row = row0 + r;
-            row = row < g.M ? row : g.M - 1;
-            int n = n0 + r;
-            n = n < g.Nout ? n : g.Nout - 1;
+            row = row < row_end ? row : row_end - 1;
+            int n = n0w + r;
+            n = n < bank_width ? n : bank_width - 1;
             const u32x4 z = {0, 0, 0, 0};
-            *(u32x4*)(As + swz(r, c)) = c < have ? *(const u32x4*)(g.su + row * g.ld_su + c * 8) : z;
-            *(u32x4*)(Bs + swz(r, c)) = c < have ? *(const u32x4*)(g.lora_right + (int64_t)n * rp + c * 8) : z;
+            *(u32x4*)(As + swz(r, c)) = c < have ? *(const u32x4*)(su_b + row * g.ld_su + c * 8) : z;
+            *(u32x4*)(Bs + swz(r, c)) = c < have ? *(const u32x4*)(lr + (int64_t)n * rp + c * 8) : z;
         }
         __syncthreads();
         for (int ks = 0; ks < steps; ++ks) {
@@ -389,7 +441,7 @@ __global__ void __launch_bounds__(NW * 64, NW == 8 ? 2 : 1) gemm_dtl16_kernel(G2
             } else {
                 const int64_t row = row0 + wm * RW + i * 16 + s16;
                 const int n = n0 + wn * 64 + j * 16 + 4 * sg;
-                if (row < g.M && n < g.Nout) *(u32x2*)(g.C + row * g.ldc + n) = v;
+                if (row < row_end && n < g.Nout) *(u32x2*)(g.C + row * g.ldc + n) = v;
             }
         }
     }
@@ -400,7 +452,7 @@ __global__ void __launch_bounds__(NW * 64, NW == 8 ? 2 : 1) gemm_dtl16_kernel(G2
             const u32x4 v = *(const u32x4*)(stg + swz(rl, ch));
             const int64_t row = row0 + wm * RW + rl;
             const int n = n0 + wn * 64 + ch * 8;
-            if (row < g.M && n < g.Nout) *(u32x4*)(g.C + row * g.ldc + n) = v;
+            if (row < row_end && n < g.Nout) *(u32x4*)(g.C + row * g.ldc + n) = v;
         }
     }
 }
