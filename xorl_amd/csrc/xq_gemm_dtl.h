@@ -143,6 +143,10 @@ __global__ void __launch_bounds__(NW * 64, NW == 8 ? 2 : 1) gemm_dtl16_kernel(G2
     }
     const int nk = g.Kc / D::BK;
     const int scols = (g.wcols + 127) >> 7;
+    // 16-row tiles of this wave's sub-tile that hold rows of the problem: the MFMAs of the others are skipped (their sums
+    // would never be stored), so the last tile of an expert -- or of a dense matrix -- costs what its rows cost rounded up to
+    // 16, not to 256: the two waves of a SIMD share its matrix pipe, and one of them leaving it alone hands it to the other
+    const int mt = __builtin_amdgcn_readfirstlane((int)max((int64_t)0, min((int64_t)TM, (row_end - row0 - wm * RW + 15) >> 4)));
 
     // ---- direct-to-LDS sources (the stage layouts of gemm_dtl_kernel): a wave brings in the 8 AP activation rows from
     // wave * 8 AP on and the 16 WP weight rows (CC; !CC: 4 WP k rows) from wave * 16 WP (4 WP) on
@@ -317,6 +321,7 @@ __global__ void __launch_bounds__(NW * 64, NW == 8 ? 2 : 1) gemm_dtl16_kernel(G2
                 }
             }
             // the chunk's four MFMAs
+            if (i < mt)
 #pragma unroll
             for (int j = 0; j < TN; ++j) {
                 if constexpr (NW == 4) {
