@@ -543,12 +543,45 @@ DECODE_SHAPES = {"q": (4096, 4096), "kv": (1024, 4096), "gate_up": (12288, 4096)
 COLD_FOOTPRINT = 640 << 20      # bytes of weight copies a case rotates through: 2.5 x the 256 MB memory-side cache
 
 
+def _graph_time_us(run, pool, reps: int, replays: int) -> float:
+    """`run()` (which makes `reps` launches) captured as one HIP graph after an eager warm-up on a side stream; the median
+    over `replays` replays of the time per launch, events on the launch stream."""
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, pool=pool):
+        run()
+    graph.replay()
+    torch.cuda.synchronize()
+    times = []
+    for _ in range(replays):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        graph.replay()
+        e1.record()
+        e1.synchronize()
+        times.append(e0.elapsed_time(e1) * 1e3 / reps)
+    del graph
+    return sorted(times)[len(times) // 2]
+
+
+def _read_probe(t, out):
+    from xorl_amd import _C
+
+    _C.check(_C.lib().xq_read_probe(t.data_ptr(), t.numel() * t.element_size(), out.data_ptr(), _C.stream_ptr(t.device)))
+
+
 def decode_case_table(dev, reps: int = 24, replays: int = 5):
     """Every configs[4] forward on its own: `reps` forwards back to back as one HIP graph (launch boundaries included, no
     host time), timed with events on the launch stream, median of `replays` replays.  Two figures per case: "cold" rotates
     through copies of the weight whose total size exceeds the 256 MB memory-side cache, so every byte comes from HBM as it
     does in a model whose layers do not fit that cache (this is the roofline figure); "hot" replays one weight, which
-    that cache may serve."""
+    that cache may serve.  `read_probe_*`: a kernel that only reads the weight's packed bytes, timed the same way -- the
+    measured ceiling for a one-shot read of that size, launch boundary included."""
     from xorl_amd.functional import QuantWeight, qlora_linear
 
     rows = []
@@ -556,6 +589,7 @@ def decode_case_table(dev, reps: int = 24, replays: int = 5):
     # one memory pool for all the graphs: the forwards' workspaces then sit at the same few addresses in every graph, and
     # the library's per-workspace slots (which stay with a captured workspace for good) are not used up case by case
     pool = torch.cuda.graph_pool_handle()
+    probe_out = torch.zeros(1, dtype=torch.int32, device=dev)
     for fmt in ("int4", "block_fp8"):
         for name, (N, K) in DECODE_SHAPES.items():
             m = dense_module(fmt, N, K, 16, 32, 60, dev)
@@ -565,6 +599,12 @@ def decode_case_table(dev, reps: int = 24, replays: int = 5):
             copies = [qw] + [QuantWeight(qw.fmt, qw.layout, qw.packed.clone(), qw.scales.clone(), qw.scale_dtype, qw.rows, qw.cols,
                                          qw.group, global_scale=qw.global_scale) for _ in range(n_copies - 1)]
             A, B, sc = m.lora_A.detach(), m.lora_B.detach(), m.scaling
+            # the measured ceiling for this weight: a kernel that only reads the packed bytes, in the same kind of graph
+            read_us = {}
+            for mode, ws in (("cold", copies), ("hot", copies[:1])):
+                read_us[mode] = _graph_time_us(lambda: [_read_probe(ws[i % len(ws)].packed, probe_out) for i in range(reps)], pool, reps,
+                                               replays)
+            pbytes = qw.packed.numel() * qw.packed.element_size()
             for Mtok in (1, 8, 32, 64):
                 x = torch.randn(Mtok, K, generator=g, device=dev).to(torch.bfloat16)
                 algo = wbytes + 2 * Mtok * K + 2 * Mtok * N + 4 * 16 * (K + N)
@@ -574,31 +614,13 @@ def decode_case_table(dev, reps: int = 24, replays: int = 5):
                         with torch.no_grad():
                             for i in range(reps):
                                 qlora_linear(x, ws[i % len(ws)], A, B, 16, sc)
-                    side = torch.cuda.Stream()
-                    side.wait_stream(torch.cuda.current_stream())
-                    with torch.cuda.stream(side):
-                        run()
-                    torch.cuda.current_stream().wait_stream(side)
-                    torch.cuda.synchronize()
-                    graph = torch.cuda.CUDAGraph()
-                    with torch.cuda.graph(graph, pool=pool):
-                        run()
-                    graph.replay()
-                    torch.cuda.synchronize()
-                    times = []
-                    for _ in range(replays):
-                        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                        e0.record()
-                        graph.replay()
-                        e1.record()
-                        e1.synchronize()
-                        times.append(e0.elapsed_time(e1) * 1e3 / reps)
-                    us[mode] = sorted(times)[len(times) // 2]
-                    del graph
+                    us[mode] = _graph_time_us(run, pool, reps, replays)
                 rows.append({"format": fmt, "proj": name, "N": N, "K": K, "M": Mtok, "bytes": algo,
                              "us": round(us["cold"], 2), "GBps": round(algo / us["cold"] / 1e3, 1),
                              "frac": round(algo / us["cold"] / 1e3 / 8000.0, 4),
-                             "us_hot": round(us["hot"], 2), "GBps_hot": round(algo / us["hot"] / 1e3, 1)})
+                             "us_hot": round(us["hot"], 2), "GBps_hot": round(algo / us["hot"] / 1e3, 1),
+                             "read_probe_us": round(read_us["cold"], 2), "read_probe_GBps": round(pbytes / read_us["cold"] / 1e3, 1),
+                             "read_probe_us_hot": round(read_us["hot"], 2)})
             del copies, m, qw
             torch.cuda.empty_cache()
     return rows
@@ -617,7 +639,8 @@ def secondary_measurements(args, dev):
         "workload": "configs[4]: skinny-M forward, M in {1,8,32,64} x {q, kv, gate/up, down of Qwen3-8B} x {int4, block_fp8}, r=16; "
                     "`cases` times every forward on its own (24 back to back in one HIP graph, weights rotating through "
                     f"{COLD_FOOTPRINT >> 20} MiB of copies so that they come from HBM; *_hot: one weight replayed, which the 256 MB "
-                    "memory-side cache may serve); `achieved` is the 32 BASELINE cases' bytes over the sum of their times; "
+                    "memory-side cache may serve; read_probe_*: a kernel that only reads the packed bytes, timed the same way); `achieved` is "
+                    "the 32 BASELINE cases' bytes over the sum of their times; "
                     "`graph_step` replays the 32 forwards on one set of weights as one HIP graph",
         "bound": "hbm", "achieved": agg, "peak": 8000.0, "unit": "GB/s", "frac": agg / 8000.0,
         "traffic": c4["roofline"]["traffic"], "traffic_source": c4["roofline"]["traffic_source"],

@@ -86,6 +86,13 @@ const char* xq_last_error(void);
 int xq_profile_enable(int on);
 int xq_profile_collect(int* n_launches, double* total_ms, double* total_flops);
 
+/* A plain streaming read of `bytes` bytes (a multiple of 16, 16-byte
+ * aligned) that does nothing else; `out` is one device word it practically
+ * never writes.  For the benchmark: timed next to the weight-streaming
+ * forwards it gives the measured ceiling for a read of that size.  No
+ * counterpart in the reference. */
+int xq_read_probe(const void* data, int64_t bytes, uint32_t* out, void* stream);
+
 /* Kernel selection of the fused dequant-GEMM entry points (dense and grouped),
  * for tests and A/B measurements; no counterpart in the reference.
  *   0 (default): by problem size.  Block-fp8 and FLAT int4/nvfp4 weights with a

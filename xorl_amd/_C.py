@@ -126,6 +126,8 @@ _SIGNATURES = {
     "xq_silu_mul_fwd": (_INT, [_P, _P, _I64, _P, _P, _I64, _I64, _I64, _P]),
     # gate, up, ld_in, dh, ld_dh, row_w, dgate, dup, ld_out, d_row_w, rows, cols, stream
     "xq_silu_mul_bwd": (_INT, [_P, _P, _I64, _P, _I64, _P, _P, _P, _I64, _P, _I64, _I64, _P]),
+    # data, bytes, out, stream
+    "xq_read_probe": (_INT, [_P, _I64, _P, _P]),
     "xq_set_tile_policy": (_INT, [_INT]),
     "xq_set_persistent_tiles": (_INT, [_INT]),
     "xq_set_fp8_direct_tiles": (_INT, [_INT]),

@@ -2,6 +2,8 @@
 #include <stdarg.h>
 #include <stdio.h>
 
+#include <algorithm>
+
 #include "xq_common.h"
 
 static thread_local char g_err[512] = "";
@@ -112,5 +114,38 @@ extern "C" int xq_profile_collect(int* n_launches, double* total_ms, double* tot
     if (total_ms) *total_ms = ms;
     if (total_flops) *total_flops = fl;
     g_prof.count = 0;
+    return XQ_OK;
+}
+
+// ---- a plain streaming read of `bytes` bytes: what the memory system gives a kernel that does nothing else.  The
+// benchmark times it next to the weight-streaming forwards (same bytes, same place in a HIP graph), so that their HBM
+// fraction can be read against a measured ceiling for a read of that size rather than against the data-sheet peak alone.
+namespace {
+__global__ void __launch_bounds__(256) read_probe_kernel(const u32x4* __restrict__ p, int64_t n16, uint32_t* __restrict__ out) {
+    const int64_t stride = (int64_t)gridDim.x * 256;
+    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    u32x4 a = {0, 0, 0, 0};
+    for (; i + 3 * stride < n16; i += 4 * stride) {            // four loads per lane in flight
+        const u32x4 v0 = __builtin_nontemporal_load(p + i), v1 = __builtin_nontemporal_load(p + i + stride);
+        const u32x4 v2 = __builtin_nontemporal_load(p + i + 2 * stride), v3 = __builtin_nontemporal_load(p + i + 3 * stride);
+        a[0] ^= v0[0] ^ v1[0] ^ v2[0] ^ v3[0]; a[1] ^= v0[1] ^ v1[1] ^ v2[1] ^ v3[1];
+        a[2] ^= v0[2] ^ v1[2] ^ v2[2] ^ v3[2]; a[3] ^= v0[3] ^ v1[3] ^ v2[3] ^ v3[3];
+    }
+    for (; i < n16; i += stride) {
+        const u32x4 v = __builtin_nontemporal_load(p + i);
+        a[0] ^= v[0]; a[1] ^= v[1]; a[2] ^= v[2]; a[3] ^= v[3];
+    }
+    const uint32_t x = a[0] ^ a[1] ^ a[2] ^ a[3];
+    if (x == 0x9e3779b9u) out[0] = x;                          // keeps the loads; practically never taken
+}
+}  // namespace
+
+extern "C" int xq_read_probe(const void* data, int64_t bytes, uint32_t* out, void* stream) {
+    XQ_REQUIRE(data && out && xq_aligned(data, 16) && bytes >= 0, "xq_read_probe: NULL or misaligned buffer");
+    const int64_t n16 = bytes >> 4;
+    if (n16 == 0) return XQ_OK;
+    const int64_t blocks = std::min<int64_t>(xq_cdiv(n16, 256 * 4), 8 * 256);
+    read_probe_kernel<<<dim3((unsigned)std::max<int64_t>(blocks, 1)), 256, 0, (hipStream_t)stream>>>((const u32x4*)data, n16, out);
+    XQ_CHECK_LAUNCH("xq_read_probe");
     return XQ_OK;
 }

@@ -197,7 +197,8 @@ static int launch_tile_gemm_t(const xq_weight* w, bool contract_cols, const bf16
                               const int32_t* offsets, const int32_t* tile_offsets, const bf16_t* su, const bf16_t* lora_right,
                               int r_pad, const bf16_t* bias, bf16_t* C, int64_t ldc, hipStream_t stream, const char* who,
                               int force_T, int force_split, float* partial, int64_t partial_bytes,
-                              const TwoBanks* two = nullptr, const int32_t* a_rows = nullptr) {
+                              const TwoBanks* two = nullptr, const int32_t* a_rows = nullptr, int64_t a_span_rows = 0) {
+    const int64_t a_rows_span = a_rows ? a_span_rows : n_rows;      // rows of A that the launch may touch (0: not known)
     TileArgs g;
     g.A = A; g.lda = lda; g.C = C; g.ldc = ldc;
     g.packed = (const uint8_t*)w->packed;
@@ -302,7 +303,9 @@ static int launch_tile_gemm_t(const xq_weight* w, bool contract_cols, const bf16
             // in a forward -- on a tile boundary of the columns)
             const bool two_ok = !two || ((grouped && !contract_cols) ? f.ncols1 % 256 == 0 : (f.nk1 % 2 == 0 && f.nk1 >= 2));
             if (g_fp8_direct && w->format == XQ_FMT_FP8 && T == 256 && ksplit == 1 && nk_all >= 3 &&
-                nk_all <= 2 * GeoDtl::SCL_MAX && two_ok && (!grouped || g.wcols % 16 == 0))
+                nk_all <= 2 * GeoDtl::SCL_MAX && two_ok && (!grouped || g.wcols % 16 == 0) &&
+                // (its lanes address their operands by 32-bit byte offsets from a base)
+                a_rows_span > 0 && a_rows_span * lda * 2 < (1ll << 32) && (int64_t)g.wrows * g.wcols < (1ll << 32))
                 rc = launch_dtl16(f, contract_cols, grouped, dim3((unsigned)(tiles_m * tiles_n)), stream, who);
             else if (w->format == XQ_FMT_FP8) rc = launch_256<XQ_FMT_FP8>(f, contract_cols, grouped, T, grid, stream, who);
             else if (w->format == XQ_FMT_INT4) rc = launch_256<XQ_FMT_INT4>(f, contract_cols, grouped, T, grid, stream, who);
@@ -387,10 +390,10 @@ int launch_gate_up_swiglu(const xq_weight* wg, const xq_weight* wu, const bf16_t
 int launch_tile_gemm(const xq_weight* w, bool contract_cols, const bf16_t* A, int64_t lda, int64_t n_rows,
                      const int32_t* offsets, const int32_t* tile_offsets, const bf16_t* su, const bf16_t* lora_right,
                      int r_pad, const bf16_t* bias, bf16_t* C, int64_t ldc, hipStream_t stream, const char* who,
-                     float* partial, int64_t partial_bytes, const TwoBanks* two, const int32_t* a_rows) {
+                     float* partial, int64_t partial_bytes, const TwoBanks* two, const int32_t* a_rows, int64_t a_span_rows) {
     XQ_REQUIRE(!a_rows || offsets, "%s: a row map goes with a grouped launch", who);
     return launch_tile_gemm_t(w, contract_cols, A, lda, n_rows, offsets, tile_offsets, su, lora_right, r_pad, bias, C, ldc,
-                              stream, who, 0, 1, partial, partial_bytes, two, a_rows);
+                              stream, who, 0, 1, partial, partial_bytes, two, a_rows, a_span_rows);
 }
 
 // whether a grouped launch over this bank runs on the pipelined tile kernel, which can read its activation rows through

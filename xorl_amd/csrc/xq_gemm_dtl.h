@@ -150,7 +150,10 @@ __global__ void __launch_bounds__(NW * 64, NW == 8 ? 2 : 1) gemm_dtl16_kernel(G2
 
     // ---- direct-to-LDS sources (the stage layouts of gemm_dtl_kernel): a wave brings in the 8 AP activation rows from
     // wave * 8 AP on and the 16 WP weight rows (CC; !CC: 4 WP k rows) from wave * 16 WP (4 WP) on
-    const bf16_t* a_src[AP];
+    // A lane's source is (a base every lane shares, advanced from K-step to K-step in scalar registers) + (a 32-bit byte
+    // offset of its own, fixed for the tile): the address costs no vector instruction per load.  (The host sends launches
+    // whose activation matrix or weight matrix spans 4 GiB or more to gemm_256_kernel.)
+    uint32_t a_off[AP];
 #pragma unroll
     for (int p = 0; p < AP; ++p) {
         const int rt = (wave * AP + p) * 8 + (lane >> 3);
@@ -159,19 +162,19 @@ __global__ void __launch_bounds__(NW * 64, NW == 8 ? 2 : 1) gemm_dtl16_kernel(G2
         if constexpr (GROUPED) {
             if (g.a_rows) r = g.a_rows[r];
         }
-        a_src[p] = g.A + r * g.lda + (((lane & 7) ^ ((rt >> 1) & 7)) << 3);
+        a_off[p] = (uint32_t)((r * g.lda + (((lane & 7) ^ ((rt >> 1) & 7)) << 3)) * 2);
     }
-    const uint8_t* w_src[WP];
+    uint32_t w_off[WP];
 #pragma unroll
     for (int q = 0; q < WP; ++q) {
         if (CC) {
             const int rt = (wave * WP + q) * 16 + (lane >> 2);
             const int wr = min(n0w + rt, g.wrows - 1);
-            w_src[q] = Wb + (int64_t)wr * g.wcols + (((lane & 3) ^ ((rt >> 2) & 3)) << 4);
+            w_off[q] = (uint32_t)((int64_t)wr * g.wcols + (((lane & 3) ^ ((rt >> 2) & 3)) << 4));
         } else {
             const int kr = (wave * WP + q) * 4 + (lane >> 4);
             const int wc = min(n0w + (((lane & 15) ^ (kr & 7)) << 4), g.wcols - 16);
-            w_src[q] = Wb + (int64_t)kr * g.wcols + wc;
+            w_off[q] = (uint32_t)((int64_t)kr * g.wcols + wc);
         }
     }
     const int64_t w_kstep = CC ? D::BK : (int64_t)D::BK * g.wcols;
@@ -180,14 +183,20 @@ __global__ void __launch_bounds__(NW * 64, NW == 8 ? 2 : 1) gemm_dtl16_kernel(G2
     constexpr bool TWO_K = GROUPED ? CC : !CC;
     const int nk1 = (TWO_K && g.W2 != nullptr) ? g.nk1 : (1 << 30);
     const int64_t w2_delta = (TWO_K && g.W2 != nullptr) ? (g.W2 - g.W) - (int64_t)nk1 * w_kstep : 0;
+    // (written out: the compiler's form of this load takes a 64-bit address per lane.  M0 -- the LDS base of the load -- is
+    // written here and used nowhere else in the kernel: the compiler is not told, it has no use for M0 in this kernel.)
+    const uint32_t dma_lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)dsm;
     auto issue_part = [&](int kt, int stage, int part) {
-        unsigned char* a = dsm + stage * D::STAGE_BYTES + wave * (AP * 1024);
-        unsigned char* w = dsm + stage * D::STAGE_BYTES + D::A_STAGE_BYTES + wave * (WP * 1024);
+        const uint32_t a = dma_lds0 + stage * D::STAGE_BYTES + wave * (AP * 1024);
+        const uint32_t w = dma_lds0 + stage * D::STAGE_BYTES + D::A_STAGE_BYTES + wave * (WP * 1024);
         if (part < AP) {
-            __builtin_amdgcn_global_load_lds(XQ_GLB_PTR(a_src[part] + kt * D::BK), XQ_LDS_PTR(a + part * 1024), 16, 0, 0);
+            const unsigned char* base = (const unsigned char*)(g.A + kt * D::BK);
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                         :: "s"(a + part * 1024), "v"(a_off[part]), "s"(base) : "memory");
         } else {
-            const int64_t off = kt * w_kstep + (kt >= nk1 ? w2_delta : 0);
-            __builtin_amdgcn_global_load_lds(XQ_GLB_PTR(w_src[part - AP] + off), XQ_LDS_PTR(w + (part - AP) * 1024), 16, 0, 0);
+            const unsigned char* base = Wb + (kt * w_kstep + (kt >= nk1 ? w2_delta : 0));
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                         :: "s"(w + (part - AP) * 1024), "v"(w_off[part - AP]), "s"(base) : "memory");
         }
     };
 
@@ -287,8 +296,8 @@ __global__ void __launch_bounds__(NW * 64, NW == 8 ? 2 : 1) gemm_dtl16_kernel(G2
     };
 
     int stage = 0;
-    auto iteration = [&](int kt, auto MORE_, auto HAVE2_) {
-        constexpr bool MORE = decltype(MORE_)::value, HAVE2 = decltype(HAVE2_)::value;
+    auto iteration = [&](int kt, auto MORE_, auto HAVE2_, auto SKIP_) {
+        constexpr bool MORE = decltype(MORE_)::value, HAVE2 = decltype(HAVE2_)::value, SKIP = decltype(SKIP_)::value;
         const uint32_t so = (uint32_t)stage * D::STAGE_BYTES;
         const int nstage = stage == 2 ? 0 : stage + 1;
         const int pstage = stage == 0 ? 2 : stage - 1;        // stage of K-step kt + 2 (free since the last barrier)
@@ -321,7 +330,7 @@ __global__ void __launch_bounds__(NW * 64, NW == 8 ? 2 : 1) gemm_dtl16_kernel(G2
                 }
             }
             // the chunk's four MFMAs
-            if (i < mt)
+            if (!SKIP || i < mt)
 #pragma unroll
             for (int j = 0; j < TN; ++j) {
                 if constexpr (NW == 4) {
@@ -377,10 +386,15 @@ __global__ void __launch_bounds__(NW * 64, NW == 8 ? 2 : 1) gemm_dtl16_kernel(G2
     {
         using Tt = std::integral_constant<bool, true>;
         using Ff = std::integral_constant<bool, false>;
-        int kt = 0;
-        for (; kt + 2 < nk; ++kt) iteration(kt, Tt{}, Tt{});
-        iteration(kt, Tt{}, Ff{});
-        iteration(kt + 1, Ff{}, Ff{});
+        // (two copies of the loop: the one for whole tiles carries no test of the row tiles)
+        auto run = [&](auto SKIP_) {
+            int kt = 0;
+            for (; kt + 2 < nk; ++kt) iteration(kt, Tt{}, Tt{}, SKIP_);
+            iteration(kt, Tt{}, Ff{}, SKIP_);
+            iteration(kt + 1, Ff{}, Ff{}, SKIP_);
+        };
+        if (mt == TM) run(Ff{});
+        else run(Tt{});
     }
 #undef XQ_DTL_READ_A
 #undef XQ_DTL_READ_W

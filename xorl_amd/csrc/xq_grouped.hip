@@ -204,10 +204,10 @@ extern "C" int xq_grouped_fwd(const xq_weight* gate, const xq_weight* up, const 
     }
     if (fuse_gate_up(gate, up)) {       // both projections in one launch: column tiles past I take the up bank
         const TwoBanks two{up, su_u, Lr_uB};
-        if ((rc = launch_tile_gemm(gate, false, xr, ld_xr, R, off, toff, su_g, Lr_gB, rp, nullptr, gu, 2 * I, stream, who, nullptr, 0, &two, xr_rows))) return rc;
+        if ((rc = launch_tile_gemm(gate, false, xr, ld_xr, R, off, toff, su_g, Lr_gB, rp, nullptr, gu, 2 * I, stream, who, nullptr, 0, &two, xr_rows, d.T))) return rc;
     } else {
-        if ((rc = launch_tile_gemm(gate, false, xr, ld_xr, R, off, toff, su_g, Lr_gB, rp, nullptr, gu, 2 * I, stream, who, nullptr, 0, nullptr, xr_rows))) return rc;
-        if ((rc = launch_tile_gemm(up, false, xr, ld_xr, R, off, toff, su_u, Lr_uB, rp, nullptr, gu + I, 2 * I, stream, who, nullptr, 0, nullptr, xr_rows))) return rc;
+        if ((rc = launch_tile_gemm(gate, false, xr, ld_xr, R, off, toff, su_g, Lr_gB, rp, nullptr, gu, 2 * I, stream, who, nullptr, 0, nullptr, xr_rows, d.T))) return rc;
+        if ((rc = launch_tile_gemm(up, false, xr, ld_xr, R, off, toff, su_u, Lr_uB, rp, nullptr, gu + I, 2 * I, stream, who, nullptr, 0, nullptr, xr_rows, d.T))) return rc;
     }
     if ((rc = xq_moe_scatter_scalar(routing_w, rw_dtype, saved->scatter_index, R, saved->w_row, stream))) return rc;
     // SwiGLU (times the row's routing weight) and s * h . A_d^T of the down projection: one pass where the rank allows
@@ -325,7 +325,7 @@ extern "C" int xq_grouped_bwd(const xq_weight* gate, const xq_weight* up, const 
     const bf16_t* gd = in_place ? (const bf16_t*)dy : g_down;      // the routed gradient rows: dy through the map, or the copy
     const int64_t ld_gd = in_place ? ld_dy : H;
     const int32_t* gd_rows = in_place ? token_of_row : nullptr;
-    if ((rc = launch_tile_gemm(down, true, gd, ld_gd, R, off, toff, v_d, Lr_dA, rp, nullptr, dh, I, stream, who, nullptr, 0, nullptr, gd_rows))) return rc;
+    if ((rc = launch_tile_gemm(down, true, gd, ld_gd, R, off, toff, v_d, Lr_dA, rp, nullptr, dh, I, stream, who, nullptr, 0, nullptr, gd_rows, d.T))) return rc;
     if ((rc = launch_tn(gd, ld_gd, H, su_d, rp, r, R, true, grads->dB[2], wg, dBe == 1 ? nullptr : off, E, stream, n_valid, 0, gd_rows))) return rc;   // [E|1, r, H]
     if ((rc = launch_tn(h, I, I, v_d, rp, r, R, false, grads->dA[2], wg, dAe == 1 ? nullptr : off, E, stream, n_valid))) return rc;        // [E|1, I, r]
 

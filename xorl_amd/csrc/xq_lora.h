@@ -122,7 +122,8 @@ int launch_tile_gemm(const xq_weight* w, bool contract_cols, const bf16_t* A, in
                      const int32_t* offsets, const int32_t* tile_offsets, const bf16_t* su, const bf16_t* lora_right,
                      int r_pad, const bf16_t* bias, bf16_t* C, int64_t ldc, hipStream_t stream, const char* who,
                      float* partial, int64_t partial_bytes, const TwoBanks* two = nullptr,
-                     const int32_t* a_rows = nullptr);   // grouped, optional: row i of the problem is row a_rows[i] of A
+                     const int32_t* a_rows = nullptr,    // grouped, optional: row i of the problem is row a_rows[i] of A,
+                     int64_t a_span_rows = 0);           // ... which has this many rows (0: not known)
 bool tile_gemm_takes_row_map(const xq_weight* w);        // ... which only the pipelined tile kernel does
 
 int num_cus();   // compute units of the current device (xq_gemm.hip)
