@@ -46,13 +46,13 @@ MEASURED_TRAFFIC = {
     0: (109.6 * 2 ** 20, "profiles/gemm_128_int4_linear_m512.txt", 0.04315),
     # gemm_dtl16_kernel (dense block-fp8, 256x256 tiles): mean over the 5 launches of a step (gate, up and down
     # forward, d_h, dx as one sum over the gate and up weights)
-    1: (1070.2 * 2 ** 20, "profiles/gemm_dtl16_fp8_mlp_m8192.txt", 0.7876),
+    1: (1070.5 * 2 ** 20, "profiles/gemm_dtl16_fp8_mlp_m8192.txt", 0.7717),
     # gemm_256_kernel<nvfp4>, 256x256 tiles (whole rounds; trailing rows in K splits) and 128x128 tiles
     # (+ splitk_reduce_kernel): mean over the 12 launches of a step, fp32 partial sums included
     2: (185.7 * 2 ** 20, "profiles/gemm_256_nvfp4_attn_m4096.txt", 0.14304),
-    # gemm_256_kernel<fp8, grouped>: mean over the 4 launches of a step (gate|up forward over two banks, down
+    # gemm_dtl16_kernel<.., grouped>: mean over the 4 launches of a step (gate|up forward over two banks, down
     # forward, d_h, dx as one sum over both banks)
-    3: (1343.0 * 2 ** 20, "profiles/gemm_256_fp8_grouped_moe_e128.txt", 0.71449),
+    3: (1395.0 * 2 ** 20, "profiles/gemm_dtl16_fp8_grouped_moe_e128.txt", 0.6417),
     # skinny_rows_kernel (M <= 16) and skinny_split_kernel + skinny_epilogue_kernel (M = 32, 64): mean per forward
     # over the 32 cases (includes the fp32 partial tiles of the two-launch cases written and read back: 23.3 MiB of
     # it are algorithmic)
@@ -233,6 +233,8 @@ def other_config(cfg: int, dev):
                 f"grouped {fmt_name} QLoRA Qwen3-30B-A3B experts, E=128, hidden 2048, intermediate 768, "
                 f"top-8 of 16384 tokens, Zipf(1.1) counts (max {int(counts.max())}, {int((counts == 0).sum())} empty), "
                 f"per-expert r=16, fwd+bwd",
+                (f"gemm_dtl16_kernel<contract_cols true|false, 8 waves, grouped> (fused block-fp8 dequant grouped GEMM, "
+                 f"forward and dgrad launches)") if cfg == 3 else
                 f"gemm_256_kernel<{kfmt}, grouped> (fused dequant grouped GEMM, forward and dgrad launches)")
     if cfg == 4:
         shapes = {"q": (4096, 4096), "kv": (1024, 4096), "gate_up": (12288, 4096), "down": (4096, 12288)}
