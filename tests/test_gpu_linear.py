@@ -457,3 +457,30 @@ def test_weight_descriptor_checks_scale_storage(hip_device):
         _C.make_weight("nvfp4", _C.XQ_LAYOUT_GKN, torch.zeros(4, K // 2, N, dtype=torch.uint8, device=hip_device),
                        torch.zeros(4, K // 16, N, dtype=torch.uint8, device=hip_device), torch.float8_e4m3fn, K, N, 16,
                        global_scale=torch.ones(3, device=hip_device), num_experts=4)
+
+
+def test_activation_rows_that_span_4gib(hip_device):
+    """The block-fp8 kernel for large tiles addresses a lane's activation row by a 32-bit byte offset from a base all lanes
+    share; a launch whose rows span 4 GiB or more (here: a column slice of a [2304, 932072] bf16 matrix) must take the kernel
+    with 64-bit lane addresses instead.  Same forward as on the contiguous copy to rounding (another summation order),
+    and equal to the oracle."""
+    from xorl_amd.functional import qlora_linear
+
+    M, K, N, r = 2304, 512, 4096, 16
+    ld = ((1 << 32) // (2 * M) + 8) // 8 * 8
+    assert M * ld * 2 >= 1 << 32
+    m, w_ref = make_dense_module("block_fp8", N, K, r, 2 * r, seed=77, device=hip_device)
+    x = gen((M, K), 1.0, 78, torch.bfloat16)
+    parent = torch.zeros(M, ld, dtype=torch.bfloat16, device=hip_device)
+    parent[:, :K] = x.to(hip_device)
+    view = parent[:, :K]
+    assert view.stride(0) == ld and (view[-1].data_ptr() - view.data_ptr()) >= (1 << 32) - 2 * ld
+    with torch.no_grad():
+        y_view = qlora_linear(view, m._quant_weight(), m.lora_A, m.lora_B, r, m.scaling)
+        y_copy = qlora_linear(view.contiguous(), m._quant_weight(), m.lora_A, m.lora_B, r, m.scaling)
+    torch.cuda.synchronize()
+    del parent, view
+    ex = R.linear_fwd_bwd_exact(x, w_ref, m.lora_A.detach().cpu(), m.lora_B.detach().cpu(), m.scaling)
+    close(y_view.cpu(), ex["y"], TOL)
+    close(y_copy.cpu(), ex["y"], TOL)
+    assert R.max_rel_err(y_view.cpu().float(), y_copy.cpu().float()) <= 2 ** -7
