@@ -1,0 +1,188 @@
+"""GPU: one activation row (M = 1) through the dot-product kernel -- whole weight rows streamed by waves, decoded to the
+reference decoder's bf16 values and multiplied without matrix cores -- against the oracle and against the MFMA kernel on
+the same inputs (xq_set_skinny_gemv(0)).  Beyond arithmetic the cases aim at: blocks of one wave (rows of 1 KB), ragged
+last blocks, a weight with fewer blocks than parts of the low-rank intermediate (falls back), the slot shared with the
+other kernel when M alternates on one workspace, waits that give up."""
+
+import ctypes
+
+import pytest
+import torch
+
+from oracle import recipe as R
+from tests.util_cases import close, gen, make_dense_module
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-2
+
+
+@pytest.fixture
+def kernels():
+    """run(fn) -> (dot-product kernel's result, MFMA kernel's result); the switch is restored afterwards."""
+    from xorl_amd import _C
+
+    def run(fn):
+        out = []
+        for on in (1, 0):
+            _C.check(_C.lib().xq_set_skinny_gemv(on))
+            out.append(fn())
+        _C.check(_C.lib().xq_set_skinny_gemv(1))
+        return out
+
+    yield run
+    _C.check(_C.lib().xq_set_skinny_gemv(1))
+
+
+def _forward(m, x, r):
+    from xorl_amd.functional import qlora_linear
+
+    with torch.no_grad():
+        if r == 0:
+            return qlora_linear(x, m._quant_weight(), None, None, 0, 0.0, m.bias)
+        return qlora_linear(x, m._quant_weight(), m.lora_A.detach(), m.lora_B.detach(), r, m.scaling, m.bias)
+
+
+@pytest.mark.parametrize("fmt,N,K,r,has_bias", [
+    ("block_fp8", 4096, 4096, 16, False),     # q/o: 4 waves per block, one group of 4 rows per block
+    ("block_fp8", 12288, 4096, 16, True),     # gate/up: two groups per block
+    ("block_fp8", 24576, 4096, 16, False),    # fused gate|up: four groups per block
+    ("block_fp8", 4096, 12288, 16, False),    # down: 12 waves per block, 24 parts of the intermediate
+    ("block_fp8", 8208, 16384, 8, False),     # the longest row (16 waves), 32 parts, 8 and 7 groups per block
+    ("block_fp8", 1040, 1024, 4, True),       # one wave per block
+    ("block_fp8", 50016, 1024, 16, False),    # one wave per block, 3 and 2 groups per block
+    ("block_fp8", 25008, 2048, 12, True),     # two waves per block, 3 and 2 groups per block
+    ("block_fp8", 16, 1024, 16, False),       # four blocks, two parts
+    ("block_fp8", 4096, 5120, 0, True),       # no low-rank term
+    ("int4", 4096, 4096, 16, False),          # 4-bit formats stay on the MFMA kernel whatever the switch says
+])
+def test_dot_product_kernel_vs_oracle_and_mfma_kernel(hip_device, kernels, fmt, N, K, r, has_bias):
+    m, w_ref = make_dense_module(fmt, N, K, max(r, 1), 2 * max(r, 1), seed=N + K + r, device=hip_device, bias=has_bias)
+    A = m.lora_A.detach().cpu() if r else torch.zeros(1, K)
+    B = m.lora_B.detach().cpu() if r else torch.zeros(N, 1)
+    bias = None if m.bias is None else m.bias.detach().cpu()
+    for call in range(3):                                   # x changes between calls that share a workspace
+        x = gen((1, K), 1.0, 70 + call, torch.bfloat16)
+        xd = x.to(hip_device)
+        dot, mfma = kernels(lambda: _forward(m, xd, r))
+        ex = R.linear_fwd_bwd_exact(x, w_ref, A, B, m.scaling if r else 0.0, bias=bias)
+        assert torch.isfinite(dot.float()).all()
+        close(dot.cpu(), ex["y"], TOL)
+        close(mfma.cpu(), ex["y"], TOL)
+        # the two kernels round the same decoded weights and differ in the order of fp32 sums only
+        close(dot.cpu(), mfma.float().cpu(), 4e-3)
+
+
+def test_one_workspace_alternating_between_the_kernels(hip_device, fmt="block_fp8"):
+    """M = 1 (dot-product kernel) and M = 8 (MFMA kernel) take turns on one workspace, hence one slot: each launch must
+    see its own parts of the low-rank intermediate only.  The low-rank term dominates the output here, so that a stale or
+    foreign part would show."""
+    from xorl_amd import _C
+    from xorl_amd.functional import _workspace_bytes
+
+    N, K, r = 4096, 4096, 16
+    m, w_ref = make_dense_module(fmt, N, K, r, 32, seed=11, device=hip_device)
+    with torch.no_grad():
+        m.lora_A.mul_(20.0)
+        m.lora_B.mul_(20.0)
+    A, B = m.lora_A.detach().contiguous(), m.lora_B.detach().contiguous()
+    w = m._quant_weight().c()
+    L = _C.lib()
+    wsb = _workspace_bytes(8, N, K, r)
+    ws = torch.empty(wsb, dtype=torch.uint8, device=hip_device)
+    for i in range(24):
+        M = 1 if i % 3 != 2 else 8
+        x = gen((M, K), 1.0, 500 + i, torch.bfloat16)
+        xd = x.to(hip_device)
+        y = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=hip_device)
+        _C.check(L.xq_linear_fwd(ctypes.byref(w), xd.data_ptr(), K, M, A.data_ptr(), B.data_ptr(), _C.XQ_DT_F32, r,
+                                 ctypes.c_float(m.scaling), None, y.data_ptr(), N, None, ws.data_ptr(), wsb, _C.stream_ptr(hip_device)))
+        ex = R.linear_fwd_bwd_exact(x, w_ref, A.cpu(), B.cpu(), m.scaling)
+        close(y.cpu(), ex["y"], TOL)
+
+
+def test_dot_product_kernel_under_hip_graph(hip_device):
+    """Captured once, replayed with x changing and eager calls on the same workspace in between: every replay gives the
+    eager call's bits."""
+    from xorl_amd import _C
+    from xorl_amd.functional import _workspace_bytes
+
+    N, K, r = 12288, 4096, 16
+    m, _ = make_dense_module("block_fp8", N, K, r, 32, seed=13, device=hip_device)
+    A, B = m.lora_A.detach().contiguous(), m.lora_B.detach().contiguous()
+    w = m._quant_weight().c()
+    L = _C.lib()
+    wsb = _workspace_bytes(1, N, K, r)
+    ws = torch.empty(wsb, dtype=torch.uint8, device=hip_device)
+    x = torch.zeros(1, K, dtype=torch.bfloat16, device=hip_device)
+    y = torch.zeros(1, N, dtype=torch.bfloat16, device=hip_device)
+
+    def call():
+        _C.check(L.xq_linear_fwd(ctypes.byref(w), x.data_ptr(), K, 1, A.data_ptr(), B.data_ptr(), _C.XQ_DT_F32, r, ctypes.c_float(m.scaling),
+                                 None, y.data_ptr(), N, None, ws.data_ptr(), wsb, _C.stream_ptr(hip_device)))
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        call()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call()
+    for i in range(5):
+        x.copy_(gen((1, K), 1.0, 800 + i, torch.bfloat16).to(hip_device))
+        y.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = y.clone()
+        y.fill_(float("nan"))
+        call()
+        torch.cuda.synchronize()
+        assert torch.isfinite(got.float()).all()
+        assert torch.equal(got, y), i
+
+
+def test_bounded_waits_in_the_dot_product_kernel(hip_device):
+    """The waits cut to a single look from the host: every kernel ends; an output is right or NaN, never made from stale
+    sums; a slot that was marked failed recovers through the status call."""
+    from xorl_amd import _C
+    from xorl_amd.functional import _workspace_bytes, skinny_status
+
+    N, K, r = 12288, 4096, 16
+    m, _ = make_dense_module("block_fp8", N, K, r, 32, seed=17, device=hip_device)
+    with torch.no_grad():
+        m.lora_A.mul_(20.0)
+        m.lora_B.mul_(20.0)
+    w = m._quant_weight().c()
+    A, B = m.lora_A.detach().contiguous(), m.lora_B.detach().contiguous()
+    L = _C.lib()
+    wsb = _workspace_bytes(1, N, K, r)
+    ws = torch.empty(wsb, dtype=torch.uint8, device=hip_device)
+    y = torch.empty(1, N, dtype=torch.bfloat16, device=hip_device)
+
+    def call(x):
+        _C.check(L.xq_linear_fwd(ctypes.byref(w), x.data_ptr(), K, 1, A.data_ptr(), B.data_ptr(), _C.XQ_DT_F32, r, ctypes.c_float(m.scaling),
+                                 None, y.data_ptr(), N, None, ws.data_ptr(), wsb, _C.stream_ptr(hip_device)))
+        torch.cuda.synchronize()
+        return y.clone()
+
+    xs = [gen((1, K), 1.0, 600 + i, torch.bfloat16).to(hip_device) for i in range(6)]
+    try:
+        want = [call(x) for x in xs]
+        assert all(torch.isfinite(t.float()).all() for t in want)
+        assert skinny_status(hip_device) == (0, 0)
+        try:
+            _C.check(L.xq_set_skinny_spin_limit(1))
+            for x, ref in zip(xs, want):
+                got = call(x)
+                bad = torch.isnan(got.float())
+                assert torch.equal(got[~bad], ref[~bad])
+        finally:
+            _C.check(L.xq_set_skinny_spin_limit(0))
+        skinny_status(hip_device, raise_on_failure=False)       # clears a failed mark, if the closing block gave up
+        assert skinny_status(hip_device) == (0, 0)
+        for x, ref in zip(xs, want):
+            assert torch.equal(call(x), ref)
+    finally:
+        _C.check(L.xq_set_skinny_spin_limit(0))
+        skinny_status(hip_device, raise_on_failure=False)

@@ -135,6 +135,7 @@ _SIGNATURES = {
     "xq_get_mlp_gate_up_fused": (_INT, []),
     "xq_set_skinny_one_launch": (_INT, [_INT]),
     "xq_set_skinny_spin_limit": (_INT, [_INT]),
+    "xq_set_skinny_gemv": (_INT, [_INT]),
     "xq_skinny_reset": (_INT, []),
     # gave_up, failed_slots, stream
     "xq_skinny_status": (_INT, [_P, _P, _P]),

@@ -435,6 +435,11 @@ extern "C" int xq_set_skinny_one_launch(int enabled) {
     return XQ_OK;
 }
 
+extern "C" int xq_set_skinny_gemv(int enabled) {
+    set_skinny_gemv(enabled);
+    return XQ_OK;
+}
+
 extern "C" int xq_set_skinny_spin_limit(int limit) {
     set_skinny_rows_spin_limit(limit);
     return XQ_OK;

@@ -915,6 +915,7 @@ static int rows_args(const xq_weight* w, const RowsPlan& p, const bf16_t* x, int
 
 int launch_skinny_rows(const xq_weight* w, const bf16_t* x, int64_t ldx, int64_t M, const void* lora_A, const void* lora_B, int r,
                        float scaling, const bf16_t* bias, bf16_t* y, int64_t ldy, const void* slot_key, hipStream_t stream) {
+    if (skinny_gemv_supported(w, M, lora_A, lora_B, XQ_DT_F32, r)) return launch_skinny_gemv(w, x, lora_A, lora_B, r, scaling, bias, y, slot_key, stream);
     RowsPlan p;
     XQ_REQUIRE(rows_plan(w, M, &p), "xq_linear_fwd: internal error: shape not supported by the one-launch skinny kernel");
     SkinnyRowsArgs g;
@@ -927,6 +928,357 @@ int launch_skinny_rows(const xq_weight* w, const bf16_t* x, int64_t ldx, int64_t
         case XQ_FMT_NF4: return launch_rows_fmt<XQ_FMT_NF4>(g, nullptr, p, grid, stream);
         default: return launch_rows_fmt<XQ_FMT_NVFP4>(g, nullptr, p, grid, stream);
     }
+}
+
+// ---------------------------------------------------------------- M = 1, block fp8: dot products instead of MFMA tiles
+// One token against a packed weight needs no matrix cores, and the organisation above -- 8 waves per CU, a load instruction
+// that takes 64 bytes of each of 16 rows -- is what keeps it from the rate of a plain read when the bytes come from HBM
+// (8 waves per CU pull at most ~6 TB/s however deep their queues; a linear read by 32 waves per CU reaches 6.9).  Here the
+// waves stream 1 KB pieces of whole rows: a row is shared by K / 1024 waves (a "set"; wave w of it owns the bytes 1024 w ..
+// of every row the set works on, so a load instruction is one contiguous KB of one row), rows go through a set in groups of
+// RB, the next group's RB loads of a lane in flight while it works on the current one.  A lane decodes its 16 weights of a
+// row to the reference decoder's bf16 values (decode8) and multiplies them with its x elements -- the same for every row,
+// held in registers as bf16 pairs -- by v_dot2c_f32_bf16 (exact products, fp32 sums); the lanes' sums of a row meet by
+// lane-permuting adds, the waves' through LDS in wave order.
+// A block is as many sets as make up to 8 waves, two blocks to a CU, plus one more wave that does not stream: it takes the
+// block's part in the low-rank exchange (the slots and the launch-count protocol of the kernel above: parts of z = A x
+// published with the launch's tag, collected by every block, the last block moves the launch count on), fetches the B rows
+// and bias, and finishes the block's rows (at most 64) when the sets are through.  The parts of z (16 ranks x 512 elements
+// each) are formed by K / 512 blocks of their own at the head of the grid, which do nothing else and are gone after a few
+// microseconds.  So no streaming wave ever waits for anything but its own weights -- under a saturated memory system any
+// dependent load costs ~3 us, and a block that is late by that makes the launch late by that -- and the parts of z are
+// read once per block: ~500 readers of the same few lines, not thousands.  (A part's entry for rank j sits at pair j of the
+// part's 256; tags keep launches of the two kernels on one slot apart.)
+// The 4-bit formats stay on the MFMA kernel: their decode is ~3 instructions per weight, which as dot products is more
+// time than the read (measured: slower than the MFMA kernel in every case).
+constexpr int kGemvRows = 4;                        // rows per group: with the next group's, 8 loads of a lane in flight
+constexpr int kGemvSlots = 64 / kGemvRows;          // groups of rows per block at most (all its sets together)
+
+// acc += w.lo * x.lo + w.hi * x.hi on bf16 pairs (exact products, one fp32 sum).  Written as the instruction: the
+// compiler's builtin for it, fed with elements of vectors, came out with one register pair for all four pairs of a vector.
+__device__ __forceinline__ void dot2_bf16(float& acc, uint32_t w, uint32_t x) {
+    asm("v_dot2c_f32_bf16 %0, %1, %2" : "+v"(acc) : "v"(w), "v"(x));
+}
+// the value of the lane that a DPP control names (all lanes active here)
+template <int CTRL>
+__device__ __forceinline__ float lane_perm(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float read_lane(float v, int l) { return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), l)); }
+
+struct GemvArgs {
+    const bf16_t* x;
+    int32_t N, K;
+    const uint8_t* packed;
+    const float* scales;           // [ceil(N / 128), ceil(K / 128)]
+    const float* lora_A;           // [r, K] fp32
+    const float* lora_B;           // [N, r] fp32
+    int32_t r;
+    float su_scale;
+    const bf16_t* bias;
+    bf16_t* y;
+    int32_t nsu;                   // parts of z (K / 512), 0 without a low-rank term
+    int32_t nw, sets, gmax;        // waves of a set, sets of a block, groups of a set at most (sets * gmax <= kGemvSlots)
+    uint32_t* slot;
+    int32_t spin_limit;
+    uint32_t* fail;
+};
+
+// (registers held to what lets 6 waves share a SIMD: left to itself the compiler spends the 128 that blocks of up to 16 waves
+// allow on decoding all rows of a group at once)
+template <int RB>
+__global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(6, 8))) skinny_gemv_kernel(GemvArgs g) {
+    __shared__ float red[kGemvSlots][RB][16];         // [set * gmax + group of the set][row][wave of the set]
+    __shared__ float zpart[16][17];                   // a block that forms a part of z: [k slice][rank]
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int nb = gridDim.x;
+    const bool lora = g.nsu > 0;
+
+    // ---- the first K / 512 blocks of a launch with a low-rank term form the parts of z and nothing else (they are gone
+    // after a few microseconds; a block that streamed as well would be late by a memory latency under load, and the
+    // launch with it): 256 threads contract 512 elements of K for the 16 ranks, thread (slice, rank) a run of 32 elements;
+    // the slices are summed in order by the threads of slice 0 and published with the launch's tag
+    if ((int)blockIdx.x < g.nsu) {
+        const int part = blockIdx.x;
+        if (wave >= 4) return;
+        // (the launch count through this XCD's L2: no line of the slot can be there from before the launch, and within a
+        // launch the word changes only after every block has read it; the block is counted in once it has been read)
+        uint32_t gen = 0;
+        if (wave == 0) {
+            gen = __hip_atomic_load(g.slot + kSlotCtl + (part % kCtlCopies) * kCtlStride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            if (lane == 0) {
+                uint32_t one = 1u;
+                asm volatile("" : "+v"(one) : "v"(gen));
+                __hip_atomic_fetch_add(g.slot + kSlotCtl + (kCtlCopies + part % kCtlCopies) * kCtlStride, one, __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+        const int j = tid & 15, sl = tid >> 4;
+        const int kb = part * kSuPartK + sl * 32;
+        const float* ap = g.lora_A + (int64_t)(j < g.r ? j : 0) * g.K + kb;
+        const bf16_t* xp = g.x + kb;
+        float a = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 32; e += 8) {
+            const f32x4 a0 = *(const f32x4*)(ap + e), a1 = *(const f32x4*)(ap + e + 4);
+            const u32x4 xx = *(const u32x4*)(xp + e);
+            // (the factor rounded to bf16 first, as in the other kernels: exact products, fp32 sums)
+            a = __builtin_fmaf(round_bf16(a0[0]), __uint_as_float(xx[0] << 16), a); a = __builtin_fmaf(round_bf16(a0[1]), __uint_as_float(xx[0] & 0xffff0000u), a);
+            a = __builtin_fmaf(round_bf16(a0[2]), __uint_as_float(xx[1] << 16), a); a = __builtin_fmaf(round_bf16(a0[3]), __uint_as_float(xx[1] & 0xffff0000u), a);
+            a = __builtin_fmaf(round_bf16(a1[0]), __uint_as_float(xx[2] << 16), a); a = __builtin_fmaf(round_bf16(a1[1]), __uint_as_float(xx[2] & 0xffff0000u), a);
+            a = __builtin_fmaf(round_bf16(a1[2]), __uint_as_float(xx[3] << 16), a); a = __builtin_fmaf(round_bf16(a1[3]), __uint_as_float(xx[3] & 0xffff0000u), a);
+        }
+        zpart[sl][j] = j < g.r ? a : 0.0f;
+        // (the four waves that are left meet at a named point of their own: the block's other waves have ended)
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+        if (tid < 16) {
+            float z = 0.0f;
+            for (int q = 0; q < 16; ++q) z += zpart[q][tid];
+            if (gen != kGenPoison)                    // a slot that is marked failed gets nothing
+                __hip_atomic_store((uint64_t*)g.slot + part * 256 + tid, ((uint64_t)(gen + 1) << 32) | __float_as_uint(z), __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+        }
+        return;
+    }
+
+    const int bx = blockIdx.x - g.nsu, nbs = nb - g.nsu;   // this block among those that stream
+    const int nstream = g.sets * g.nw;                // streaming waves; wave `nstream` is the one that does not stream
+    const bool streamer = wave < nstream;
+    const int st = wave / g.nw, ws = wave - st * g.nw;
+    const int ngroups = (g.N + RB - 1) / RB;
+    const int nvb = nbs * g.sets;                     // sets of the launch; set v takes the groups v, v + nvb, ...
+
+    // (the two kinds of waves go separate ways from here, each with the block's barrier in its own path, so that neither
+    // carries the other's registers)
+    if (streamer) {
+        const int v = bx * g.sets + st;
+        const int gcount = v < ngroups ? (ngroups - v + nvb - 1) / nvb : 0;   // at most gmax (host)
+        const int kbase = (ws * 64 + lane) * 16;      // first element of this lane's piece of a row
+        const int sc_cols = (g.K + 127) >> 7;
+        // a group's pieces and scales (one scale per lane and row: 16 elements lie in one 128-block)
+        auto issue = [&](u32x4 (&w)[RB], float (&sc)[RB], int grp) {
+#pragma unroll
+            for (int i = 0; i < RB; ++i) {
+                const int n = grp * RB + i < g.N ? grp * RB + i : g.N - 1;
+                w[i] = __builtin_nontemporal_load((const u32x4*)(g.packed + (int64_t)n * g.K + kbase));
+                sc[i] = g.scales[(n >> 7) * sc_cols + (kbase >> 7)];
+            }
+        };
+        // ---- the groups of this wave's set: the next one's loads go out, then the current one is decoded and multiplied,
+        // summed over the wave's lanes (fixed order: within 16 lanes by lane-permuting adds, then the four 16s in order)
+        // and left in LDS for the finish
+        u32x4 xv[2];
+        auto work = [&](const u32x4 (&w)[RB], const float (&sc)[RB], int gi) {
+            float a[RB];
+#pragma unroll
+            for (int i = 0; i < RB; ++i) {
+                a[i] = 0.0f;
+#pragma unroll
+                for (int c = 0; c < 2; ++c) {
+                    const u32x4 wp = __builtin_bit_cast(u32x4, decode8<XQ_FMT_FP8>(w[i][2 * c], w[i][2 * c + 1], sc[i], 0.0f));
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) dot2_bf16(a[i], wp[e], xv[c][e]);
+                }
+            }
+            // (a dot instruction's result may be read by another kind of instruction only some cycles later; the compiler
+            // keeps that distance for its own instructions and cannot see into the asm above)
+            asm volatile("s_nop 3" ::: "memory");
+#pragma unroll
+            for (int i = 0; i < RB; ++i) {
+                float t = a[i];
+                t += lane_perm<0xB1>(t);              // neighbours in a quad
+                t += lane_perm<0x4E>(t);              // the quad's halves
+                t += lane_perm<0x141>(t);             // lanes 0-7 mirrored: the other quad of the 8
+                t += lane_perm<0x140>(t);             // lanes 0-15 mirrored: the other 8 of the 16
+                const float sum = (read_lane(t, 0) + read_lane(t, 16)) + (read_lane(t, 32) + read_lane(t, 48));
+                if (lane == 0) red[st * g.gmax + gi][i][ws] = sum;
+            }
+        };
+        if (gcount > 0) {
+            u32x4 wa[RB], wb[RB];
+            float sa[RB], sb[RB];
+            issue(wa, sa, v);
+            xv[0] = *(const u32x4*)(g.x + kbase);
+            xv[1] = *(const u32x4*)(g.x + kbase + 8);
+            // (the steps are written out by the state of the two buffers, so that no step waits for more than its own loads)
+            int gi = 0;
+            while (gi + 2 < gcount) {
+                issue(wb, sb, v + (gi + 1) * nvb);
+                work(wa, sa, gi);
+                issue(wa, sa, v + (gi + 2) * nvb);
+                work(wb, sb, gi + 1);
+                gi += 2;
+            }
+            if (gi + 1 < gcount) {
+                issue(wb, sb, v + (gi + 1) * nvb);
+                work(wa, sa, gi);
+                work(wb, sb, gi + 1);
+            } else {
+                work(wa, sa, gi);
+            }
+        }
+        __syncthreads();
+        return;
+    }
+
+    // ---- the last wave.  First the slot's launch count (its block's copy) and the B rows and bias of the rows it will
+    // finish: lane t finishes row t % RB of the block's group slot t / RB = set * gmax + group of the set.  The block is
+    // counted in once the count has been read.
+    const int f_slot = lane / RB, f_i = lane - f_slot * RB;
+    const int f_set = f_slot / g.gmax, f_gi = f_slot - f_set * g.gmax;
+    const int f_group = bx * g.sets + f_set + f_gi * nvb;
+    const int fn = f_group * RB + f_i;
+    const bool finisher = f_set < g.sets && f_group < ngroups && fn < g.N;
+    uint32_t gen = 0;
+    f32x4 brow[4];
+    float bias_v = 0.0f;
+    if (lora) {
+        // (past the caches: it is not needed before the first look at the parts has returned)
+        gen = __hip_atomic_load(g.slot + kSlotCtl + (blockIdx.x % kCtlCopies) * kCtlStride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        brow[q] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        if (finisher && lora && 4 * q < g.r) brow[q] = *(const f32x4*)(g.lora_B + (int64_t)fn * g.r + 4 * q);
+    }
+    if (finisher && g.bias) bias_v = bf16_to_f32(g.bias[fn]);
+    if (lora && lane == 0) {
+        uint32_t one = 1u;
+        asm volatile("" : "+v"(one) : "v"(gen));       // (the add may not move ahead of the point where `gen` is in its register)
+        __hip_atomic_fetch_add(g.slot + kSlotCtl + (kCtlCopies + blockIdx.x % kCtlCopies) * kCtlStride, one, __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+    }
+    // ---- while the sets stream: collect all parts -- lane (q, j) takes rank j of the parts q, q + 4, ... -- looking past
+    // the caches until they carry this launch's tag
+    float zv = 0.0f;                                  // lane j < 16 (and the lanes 16 apart): z[j] * scaling
+    bool whole = true;
+    if (lora) {
+        const bool closer = (int)blockIdx.x == nb - 1;
+        const bool failed_slot = gen == kGenPoison;
+        bool missing = failed_slot, open = closer && !failed_slot;
+        float z = 0.0f;
+        int spins = 0;
+        if (!failed_slot) for (;;) {
+            uint64_t zt[kSuMaxParts / 4];
+#pragma unroll
+            for (int u = 0; u < kSuMaxParts / 4; ++u) {
+                const int p = 4 * u + (lane >> 4);
+                zt[u] = 0;
+                if (4 * u < g.nsu)
+                    zt[u] = __hip_atomic_load((const uint64_t*)g.slot + (p < g.nsu ? p : g.nsu - 1) * 256 + (lane & 15), __ATOMIC_RELAXED,
+                                              __HIP_MEMORY_SCOPE_AGENT);
+            }
+            uint32_t started = 0;
+            if (open && lane < kCtlCopies)
+                started = __hip_atomic_load(g.slot + kSlotCtl + (kCtlCopies + lane) * kCtlStride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            z = 0.0f;
+            missing = false;
+#pragma unroll
+            for (int u = 0; u < kSuMaxParts / 4; ++u) {
+                const bool have = 4 * u + (lane >> 4) < g.nsu;
+                missing |= have && (uint32_t)(zt[u] >> 32) != gen + 1;
+                z += have ? __uint_as_float((uint32_t)zt[u]) : 0.0f;
+            }
+            missing = __any(missing);
+            if (open) {
+#pragma unroll
+                for (int d = 32; d >= 1; d >>= 1) started += __shfl_xor(started, d, 64);
+                if (started == (uint32_t)nb) {
+                    if (lane < kCtlCopies) {
+                        __hip_atomic_store(g.slot + kSlotCtl + lane * kCtlStride, gen + 1 == kGenPoison ? 0u : gen + 1, __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_AGENT);
+                        __hip_atomic_store(g.slot + kSlotCtl + (kCtlCopies + lane) * kCtlStride, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
+                    open = false;
+                }
+            }
+            if (!(missing || open) || ++spins >= g.spin_limit) break;
+            __builtin_amdgcn_s_sleep(8);
+        }
+        // (a closer that gave up marks the slot failed; a block that is about to write NaN says so: as in the kernel above)
+        if (open && lane < kCtlCopies)
+            __hip_atomic_store(g.slot + kSlotCtl + lane * kCtlStride, kGenPoison, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if ((missing || open) && lane == 0) __hip_atomic_fetch_add(g.fail, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        z += __shfl_xor(z, 16, 64);                   // the four lanes of a rank: (q0 + q1) + (q2 + q3)
+        z += __shfl_xor(z, 32, 64);
+        zv = (lane & 15) < g.r ? z * g.su_scale : 0.0f;
+        whole = !(missing || open);
+    }
+    __syncthreads();
+
+    // ---- outputs: the waves' sums in wave order, the low-rank term rank by rank, the bias
+    float o = 0.0f;
+    if (finisher)
+        for (int ww = 0; ww < g.nw; ++ww) o += red[f_slot][f_i][ww];
+    if (lora) {
+#pragma unroll
+        for (int j = 0; j < 16; ++j) o = __builtin_fmaf(read_lane(zv, j), brow[j >> 2][j & 3], o);
+        if (!whole) o = __builtin_nanf("");
+    }
+    if (g.bias) o += bias_v;
+    if (finisher) g.y[fn] = to_bf16(o);
+}
+
+static std::atomic<int> g_skinny_gemv{[] { const char* e = getenv("XQ_SKINNY_GEMV"); return e ? atoi(e) : 1; }()};
+void set_skinny_gemv(int on) { g_skinny_gemv = on != 0; }
+
+// a launch's shape: sets of K / 1024 waves, as many to a block as make up to 8 streaming waves; as many blocks as the CUs
+// hold at once (20 of a CU's 24 waves: two blocks of 9 waves, one of 13; the rest is room for the blocks that form z)
+// where the weight has that many groups of rows, more blocks where a block's sets would otherwise get more than
+// kGemvSlots groups
+struct GemvPlan {
+    int nw, sets, gmax;
+    unsigned blocks;
+};
+static GemvPlan gemv_plan(const xq_weight* w) {
+    GemvPlan p;
+    p.nw = (int)(w->cols / 1024);
+    p.sets = 8 / p.nw > 1 ? 8 / p.nw : 1;
+    const int64_t ngroups = xq_cdiv(w->rows, kGemvRows);
+    const int gcap = kGemvSlots / p.sets;             // groups of a set at most
+    const int64_t fill = 256 * (20 / (p.sets * p.nw + 1) > 1 ? 20 / (p.sets * p.nw + 1) : 1);
+    int64_t nb = xq_cdiv(ngroups, p.sets) < fill ? xq_cdiv(ngroups, p.sets) : fill;
+    if (xq_cdiv(ngroups, (int64_t)p.sets * gcap) > nb) nb = xq_cdiv(ngroups, (int64_t)p.sets * gcap);
+    p.blocks = (unsigned)nb;
+    p.gmax = (int)xq_cdiv(ngroups, nb * p.sets);
+    return p;
+}
+
+bool skinny_gemv_supported(const xq_weight* w, int64_t M, const void* lora_A, const void* lora_B, int lora_dtype, int r) {
+    if (!g_skinny_gemv || M != 1 || w->num_experts != 1 || w->layout != XQ_LAYOUT_FLAT) return false;
+    if (w->format != XQ_FMT_FP8 || w->scale_dtype != XQ_SCALE_F32) return false;
+    if (w->cols % 1024 != 0 || w->cols / 1024 > 15 || w->rows < 1 || w->rows >= (1ll << 30)) return false;
+    if (!xq_aligned(w->packed, 16)) return false;
+    if (r > 0) {
+        if (lora_dtype != XQ_DT_F32 || r > 16 || r % 4 != 0 || !xq_aligned(lora_A, 16) || !xq_aligned(lora_B, 16)) return false;
+        if (w->cols / kSuPartK > kSuMaxParts) return false;
+    }
+    return true;
+}
+
+int launch_skinny_gemv(const xq_weight* w, const bf16_t* x, const void* lora_A, const void* lora_B, int r, float scaling,
+                       const bf16_t* bias, bf16_t* y, const void* slot_key, hipStream_t stream) {
+    const GemvPlan p = gemv_plan(w);
+    XQ_REQUIRE(p.sets * p.gmax <= kGemvSlots && p.sets * p.nw >= 4 && (p.sets * p.nw + 1) * 64 <= 1024,
+               "xq_linear_fwd: internal error: dot-product launch out of range");
+    GemvArgs g;
+    g.x = x; g.N = (int)w->rows; g.K = (int)w->cols;
+    g.packed = (const uint8_t*)w->packed; g.scales = (const float*)w->scales;
+    g.lora_A = (const float*)lora_A; g.lora_B = (const float*)lora_B; g.r = r; g.su_scale = scaling;
+    g.bias = bias; g.y = y;
+    g.nsu = r > 0 ? (int)(w->cols / kSuPartK) : 0;
+    g.nw = p.nw; g.sets = p.sets; g.gmax = p.gmax;
+    g.slot = nullptr; g.fail = nullptr;
+    g.spin_limit = g_rows_spin_limit.load();
+    if (r > 0) {
+        const int rc = rows_slot(slot_key, stream, &g.slot, &g.fail);
+        if (rc) return rc;
+    }
+    skinny_gemv_kernel<kGemvRows><<<p.blocks + (unsigned)g.nsu, (unsigned)((p.sets * p.nw + 1) * 64), 0, stream>>>(g);
+    return XQ_OK;
 }
 
 // ---- gate | up with the SwiGLU finish: h = silu(gate) * up from one weight [2 I, K] in one launch
