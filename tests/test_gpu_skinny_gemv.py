@@ -51,9 +51,16 @@ def _forward(m, x, r):
     ("block_fp8", 1040, 1024, 4, True),       # one wave per block
     ("block_fp8", 50016, 1024, 16, False),    # one wave per block, 3 and 2 groups per block
     ("block_fp8", 25008, 2048, 12, True),     # two waves per block, 3 and 2 groups per block
-    ("block_fp8", 16, 1024, 16, False),       # four blocks, two parts
+    ("block_fp8", 16, 1024, 16, False),       # one block, sets of one group, two parts
+    ("block_fp8", 11024, 4096, 16, True),     # 11 rows per set (groups of 4, 4, 3), the last sets shorter or empty
+    ("int4", 12304, 2048, 16, False),         # one wave per set, 4 rows per set and sets left without rows
     ("block_fp8", 4096, 5120, 0, True),       # no low-rank term
-    ("int4", 4096, 4096, 16, False),          # 4-bit formats stay on the MFMA kernel whatever the switch says
+    ("int4", 4096, 4096, 16, False),          # 2 KB rows: two waves per set, four sets
+    ("int4", 12288, 4096, 16, True),
+    ("int4", 4096, 12288, 16, False),         # 6 waves per set, one set
+    ("int4", 1024, 2048, 8, True),            # one wave per set
+    ("int4", 2048, 8192, 0, False),
+    ("nf4", 4096, 4096, 16, False),           # the other 4-bit formats stay on the MFMA kernel whatever the switch says
 ])
 def test_dot_product_kernel_vs_oracle_and_mfma_kernel(hip_device, kernels, fmt, N, K, r, has_bias):
     m, w_ref = make_dense_module(fmt, N, K, max(r, 1), 2 * max(r, 1), seed=N + K + r, device=hip_device, bias=has_bias)
@@ -72,7 +79,8 @@ def test_dot_product_kernel_vs_oracle_and_mfma_kernel(hip_device, kernels, fmt, 
         close(dot.cpu(), mfma.float().cpu(), 4e-3)
 
 
-def test_one_workspace_alternating_between_the_kernels(hip_device, fmt="block_fp8"):
+@pytest.mark.parametrize("fmt", ["block_fp8", "int4"])
+def test_one_workspace_alternating_between_the_kernels(hip_device, fmt):
     """M = 1 (dot-product kernel) and M = 8 (MFMA kernel) take turns on one workspace, hence one slot: each launch must
     see its own parts of the low-rank intermediate only.  The low-rank term dominates the output here, so that a stale or
     foreign part would show."""

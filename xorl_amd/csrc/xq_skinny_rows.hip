@@ -43,6 +43,7 @@
 #include "xq_common.h"
 #include "xq_lora.h"
 #include "xq_skinny.h"
+#include <type_traits>
 
 namespace xq {
 
@@ -930,13 +931,13 @@ int launch_skinny_rows(const xq_weight* w, const bf16_t* x, int64_t ldx, int64_t
     }
 }
 
-// ---------------------------------------------------------------- M = 1, block fp8: dot products instead of MFMA tiles
+// ---------------------------------------------------------------- M = 1, block fp8 and int4: dot products instead of MFMA tiles
 // One token against a packed weight needs no matrix cores, and the organisation above -- 8 waves per CU, a load instruction
 // that takes 64 bytes of each of 16 rows -- is what keeps it from the rate of a plain read when the bytes come from HBM
 // (8 waves per CU pull at most ~6 TB/s however deep their queues; a linear read by 32 waves per CU reaches 6.9).  Here the
 // waves stream 1 KB pieces of whole rows: a row is shared by K / 1024 waves (a "set"; wave w of it owns the bytes 1024 w ..
 // of every row the set works on, so a load instruction is one contiguous KB of one row), rows go through a set in groups of
-// RB, the next group's RB loads of a lane in flight while it works on the current one.  A lane decodes its 16 weights of a
+// RB, the next group's RB loads of a lane in flight while it works on the current one.  A lane decodes its 16 weights (fp8) of a
 // row to the reference decoder's bf16 values (decode8) and multiplies them with its x elements -- the same for every row,
 // held in registers as bf16 pairs -- by v_dot2c_f32_bf16 (exact products, fp32 sums); the lanes' sums of a row meet by
 // lane-permuting adds, the waves' through LDS in wave order.
@@ -949,8 +950,10 @@ int launch_skinny_rows(const xq_weight* w, const bf16_t* x, int64_t ldx, int64_t
 // dependent load costs ~3 us, and a block that is late by that makes the launch late by that -- and the parts of z are
 // read once per block: ~500 readers of the same few lines, not thousands.  (A part's entry for rank j sits at pair j of the
 // part's 256; tags keep launches of the two kernels on one slot apart.)
-// The 4-bit formats stay on the MFMA kernel: their decode is ~3 instructions per weight, which as dot products is more
-// time than the read (measured: slower than the MFMA kernel in every case).
+// int4 takes the same kernel with 32 weights per lane and load (rows of 2 KB per wave): its time is the decode's -- as
+// many instructions per weight as block fp8, twice as many per byte -- so it is level with the MFMA kernel on the large
+// shapes and ahead where that kernel's organisation fits badly (q, kv, down: -15 %).  nf4 and nvfp4 stay on the MFMA
+// kernel.
 constexpr int kGemvRows = 4;                        // rows per group: with the next group's, 8 loads of a lane in flight
 constexpr int kGemvSlots = 64 / kGemvRows;          // groups of rows per block at most (all its sets together)
 
@@ -970,7 +973,8 @@ struct GemvArgs {
     const bf16_t* x;
     int32_t N, K;
     const uint8_t* packed;
-    const float* scales;           // [ceil(N / 128), ceil(K / 128)]
+    const uint8_t* scales;         // fp8: fp32 [ceil(N / 128), ceil(K / 128)]; int4: one per group along K
+    int32_t gshift, scale_dtype;   // int4: log2 of the group size, the scales' type
     const float* lora_A;           // [r, K] fp32
     const float* lora_B;           // [N, r] fp32
     int32_t r;
@@ -978,7 +982,7 @@ struct GemvArgs {
     const bf16_t* bias;
     bf16_t* y;
     int32_t nsu;                   // parts of z (K / 512), 0 without a low-rank term
-    int32_t nw, sets, gmax;        // waves of a set, sets of a block, groups of a set at most (sets * gmax <= kGemvSlots)
+    int32_t nw, sets, gmax, rps;   // waves of a set, sets of a block, groups of a set at most (sets * gmax <= kGemvSlots), rows of a set
     uint32_t* slot;
     int32_t spin_limit;
     uint32_t* fail;
@@ -986,8 +990,10 @@ struct GemvArgs {
 
 // (registers held to what lets 6 waves share a SIMD: left to itself the compiler spends the 128 that blocks of up to 16 waves
 // allow on decoding all rows of a group at once)
-template <int RB>
-__global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(6, 8))) skinny_gemv_kernel(GemvArgs g) {
+template <int FMT, int RB>
+__global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(FMT == XQ_FMT_FP8 ? 6 : 5, 8))) skinny_gemv_kernel(GemvArgs g) {
+    constexpr bool F8 = FMT == XQ_FMT_FP8;
+    constexpr int EPL = F8 ? 16 : 32;                 // weights of a row per lane (one 16-byte load)
     __shared__ float red[kGemvSlots][RB][16];         // [set * gmax + group of the set][row][wave of the set]
     __shared__ float zpart[16][17];                   // a block that forms a part of z: [k slice][rank]
     const int tid = threadIdx.x, lane = tid & 63;
@@ -1048,37 +1054,61 @@ __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(6, 8)
     const int nstream = g.sets * g.nw;                // streaming waves; wave `nstream` is the one that does not stream
     const bool streamer = wave < nstream;
     const int st = wave / g.nw, ws = wave - st * g.nw;
-    const int ngroups = (g.N + RB - 1) / RB;
-    const int nvb = nbs * g.sets;                     // sets of the launch; set v takes the groups v, v + nvb, ...
+    // set v of the launch's nbs * sets takes the rows v * rps .. (v + 1) * rps - 1, in groups of RB (the last one may be short)
 
     // (the two kinds of waves go separate ways from here, each with the block's barrier in its own path, so that neither
     // carries the other's registers)
     if (streamer) {
         const int v = bx * g.sets + st;
-        const int gcount = v < ngroups ? (ngroups - v + nvb - 1) / nvb : 0;   // at most gmax (host)
-        const int kbase = (ws * 64 + lane) * 16;      // first element of this lane's piece of a row
+        const int row0 = v * g.rps;
+        const int nrows = row0 < g.N ? (g.N - row0 < g.rps ? g.N - row0 : g.rps) : 0;
+        const int gcount = (nrows + RB - 1) / RB;     // at most gmax (host)
+        const int kbase = (ws * 64 + lane) * EPL;     // first element of this lane's piece of a row
         const int sc_cols = (g.K + 127) >> 7;
-        // a group's pieces and scales (one scale per lane and row: 16 elements lie in one 128-block)
-        auto issue = [&](u32x4 (&w)[RB], float (&sc)[RB], int grp) {
+        const int64_t row_bytes = F8 ? g.K : g.K >> 1;
+        // a group's pieces and scales (one scale per lane and row: the lane's elements lie in one 128-block, or in one
+        // group of at least 32)
+        // (an int4 scale is fetched as the aligned 32-bit word that holds it, fp32 or bf16, and picked apart when it is
+        // used: a conversion next to the load would wait for every load in flight)
+        const bool s32 = g.scale_dtype == XQ_SCALE_F32;
+        // (a row past the set's last one stands for that one: the same lines again, nothing more from memory)
+        auto issue = [&](u32x4 (&w)[RB], float (&sc)[RB], int gi) {
 #pragma unroll
             for (int i = 0; i < RB; ++i) {
-                const int n = grp * RB + i < g.N ? grp * RB + i : g.N - 1;
-                w[i] = __builtin_nontemporal_load((const u32x4*)(g.packed + (int64_t)n * g.K + kbase));
-                sc[i] = g.scales[(n >> 7) * sc_cols + (kbase >> 7)];
+                const int n = row0 + (gi * RB + i < nrows ? gi * RB + i : nrows - 1);
+                w[i] = __builtin_nontemporal_load((const u32x4*)(g.packed + (int64_t)n * row_bytes + (ws * 64 + lane) * 16));
+                if (F8) {
+                    sc[i] = ((const float*)g.scales)[(n >> 7) * sc_cols + (kbase >> 7)];
+                } else {
+                    const int64_t si = ((int64_t)n * g.K + kbase) >> g.gshift;
+                    sc[i] = *(const float*)(g.scales + ((s32 ? si << 2 : si << 1) & ~(int64_t)3));
+                }
             }
+        };
+        // the scale of row i of a group from what `issue` fetched (int4 with bf16 scales: the half that the index names)
+        auto scale_of = [&](float raw, int gi, int i) -> float {
+            if (F8 || s32) return raw;
+            const int n = row0 + (gi * RB + i < nrows ? gi * RB + i : nrows - 1);
+            const int64_t si = ((int64_t)n * g.K + kbase) >> g.gshift;
+            const uint32_t u = __float_as_uint(raw);
+            return __uint_as_float((si & 1) ? u & 0xffff0000u : u << 16);
         };
         // ---- the groups of this wave's set: the next one's loads go out, then the current one is decoded and multiplied,
         // summed over the wave's lanes (fixed order: within 16 lanes by lane-permuting adds, then the four 16s in order)
         // and left in LDS for the finish
-        u32x4 xv[2];
-        auto work = [&](const u32x4 (&w)[RB], const float (&sc)[RB], int gi) {
+        u32x4 xv[EPL / 8];
+        auto work_rows = [&](auto whole, const u32x4 (&w)[RB], const float (&sc)[RB], int gi) {
             float a[RB];
 #pragma unroll
             for (int i = 0; i < RB; ++i) {
                 a[i] = 0.0f;
+                if (!decltype(whole)::value && gi * RB + i >= nrows) continue;     // (wave-uniform: a short last group)
+                const float sv = scale_of(sc[i], gi, i);
 #pragma unroll
-                for (int c = 0; c < 2; ++c) {
-                    const u32x4 wp = __builtin_bit_cast(u32x4, decode8<XQ_FMT_FP8>(w[i][2 * c], w[i][2 * c + 1], sc[i], 0.0f));
+                for (int c = 0; c < EPL / 8; ++c) {
+                    u32x4 wp;
+                    if constexpr (F8) wp = __builtin_bit_cast(u32x4, decode8<FMT>(w[i][2 * c], w[i][2 * c + 1], sv, 0.0f));
+                    else wp = __builtin_bit_cast(u32x4, decode8<FMT>(w[i][c], 0u, sv, -8.0f * sv));
 #pragma unroll
                     for (int e = 0; e < 4; ++e) dot2_bf16(a[i], wp[e], xv[c][e]);
                 }
@@ -1097,23 +1127,27 @@ __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(6, 8)
                 if (lane == 0) red[st * g.gmax + gi][i][ws] = sum;
             }
         };
+        auto work = [&](const u32x4 (&w)[RB], const float (&sc)[RB], int gi) {
+            if (gi * RB + RB <= nrows) work_rows(std::true_type{}, w, sc, gi);
+            else work_rows(std::false_type{}, w, sc, gi);
+        };
         if (gcount > 0) {
             u32x4 wa[RB], wb[RB];
             float sa[RB], sb[RB];
-            issue(wa, sa, v);
-            xv[0] = *(const u32x4*)(g.x + kbase);
-            xv[1] = *(const u32x4*)(g.x + kbase + 8);
+            issue(wa, sa, 0);
+#pragma unroll
+            for (int c = 0; c < EPL / 8; ++c) xv[c] = *(const u32x4*)(g.x + kbase + 8 * c);
             // (the steps are written out by the state of the two buffers, so that no step waits for more than its own loads)
             int gi = 0;
             while (gi + 2 < gcount) {
-                issue(wb, sb, v + (gi + 1) * nvb);
+                issue(wb, sb, gi + 1);
                 work(wa, sa, gi);
-                issue(wa, sa, v + (gi + 2) * nvb);
+                issue(wa, sa, gi + 2);
                 work(wb, sb, gi + 1);
                 gi += 2;
             }
             if (gi + 1 < gcount) {
-                issue(wb, sb, v + (gi + 1) * nvb);
+                issue(wb, sb, gi + 1);
                 work(wa, sa, gi);
                 work(wb, sb, gi + 1);
             } else {
@@ -1129,9 +1163,9 @@ __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(6, 8)
     // counted in once the count has been read.
     const int f_slot = lane / RB, f_i = lane - f_slot * RB;
     const int f_set = f_slot / g.gmax, f_gi = f_slot - f_set * g.gmax;
-    const int f_group = bx * g.sets + f_set + f_gi * nvb;
-    const int fn = f_group * RB + f_i;
-    const bool finisher = f_set < g.sets && f_group < ngroups && fn < g.N;
+    const int f_row = f_gi * RB + f_i;                // row within the set's range
+    const int fn = (bx * g.sets + f_set) * g.rps + f_row;
+    const bool finisher = f_set < g.sets && f_row < g.rps && fn < g.N;
     uint32_t gen = 0;
     f32x4 brow[4];
     float bias_v = 0.0f;
@@ -1230,31 +1264,37 @@ void set_skinny_gemv(int on) { g_skinny_gemv = on != 0; }
 // where the weight has that many groups of rows, more blocks where a block's sets would otherwise get more than
 // kGemvSlots groups
 struct GemvPlan {
-    int nw, sets, gmax;
+    int nw, sets, gmax, rps;
     unsigned blocks;
 };
 static GemvPlan gemv_plan(const xq_weight* w) {
     GemvPlan p;
-    p.nw = (int)(w->cols / 1024);
+    p.nw = (int)((w->format == XQ_FMT_FP8 ? w->cols : w->cols / 2) / 1024);
     p.sets = 8 / p.nw > 1 ? 8 / p.nw : 1;
-    const int64_t ngroups = xq_cdiv(w->rows, kGemvRows);
-    const int gcap = kGemvSlots / p.sets;             // groups of a set at most
+    const int cap = (kGemvSlots / p.sets) * kGemvRows;     // rows of a set at most
     const int64_t fill = 256 * (20 / (p.sets * p.nw + 1) > 1 ? 20 / (p.sets * p.nw + 1) : 1);
-    int64_t nb = xq_cdiv(ngroups, p.sets) < fill ? xq_cdiv(ngroups, p.sets) : fill;
-    if (xq_cdiv(ngroups, (int64_t)p.sets * gcap) > nb) nb = xq_cdiv(ngroups, (int64_t)p.sets * gcap);
+    int64_t nb = xq_cdiv(w->rows, (int64_t)p.sets * kGemvRows) < fill ? xq_cdiv(w->rows, (int64_t)p.sets * kGemvRows) : fill;
+    if (xq_cdiv(w->rows, (int64_t)p.sets * cap) > nb) nb = xq_cdiv(w->rows, (int64_t)p.sets * cap);
     p.blocks = (unsigned)nb;
-    p.gmax = (int)xq_cdiv(ngroups, nb * p.sets);
+    p.rps = (int)xq_cdiv(w->rows, nb * p.sets);            // the rows dealt evenly: a set's range is at most one row longer than another's
+    p.gmax = (int)xq_cdiv(p.rps, kGemvRows);
     return p;
 }
 
 bool skinny_gemv_supported(const xq_weight* w, int64_t M, const void* lora_A, const void* lora_B, int lora_dtype, int r) {
     if (!g_skinny_gemv || M != 1 || w->num_experts != 1 || w->layout != XQ_LAYOUT_FLAT) return false;
-    if (w->format != XQ_FMT_FP8 || w->scale_dtype != XQ_SCALE_F32) return false;
-    if (w->cols % 1024 != 0 || w->cols / 1024 > 15 || w->rows < 1 || w->rows >= (1ll << 30)) return false;
+    if (w->format == XQ_FMT_FP8 ? w->scale_dtype != XQ_SCALE_F32
+                                : w->format != XQ_FMT_INT4 || w->group < 32 || (w->group & (w->group - 1)) != 0 ||
+                                      (w->scale_dtype != XQ_SCALE_F32 && w->scale_dtype != XQ_SCALE_BF16))
+        return false;
+    // (bf16 scales are read as the aligned words that hold them: the array must end on a word)
+    if (w->format == XQ_FMT_INT4 && (w->rows * w->cols / w->group) % 2 != 0) return false;
+    const int64_t row_bytes = w->format == XQ_FMT_FP8 ? w->cols : w->cols / 2;
+    if (row_bytes % 1024 != 0 || row_bytes / 1024 > 15 || w->rows < 1 || w->rows >= (1ll << 30)) return false;
     if (!xq_aligned(w->packed, 16)) return false;
     if (r > 0) {
         if (lora_dtype != XQ_DT_F32 || r > 16 || r % 4 != 0 || !xq_aligned(lora_A, 16) || !xq_aligned(lora_B, 16)) return false;
-        if (w->cols / kSuPartK > kSuMaxParts) return false;
+        if (w->cols % kSuPartK != 0 || w->cols / kSuPartK > kSuMaxParts) return false;
     }
     return true;
 }
@@ -1266,18 +1306,23 @@ int launch_skinny_gemv(const xq_weight* w, const bf16_t* x, const void* lora_A, 
                "xq_linear_fwd: internal error: dot-product launch out of range");
     GemvArgs g;
     g.x = x; g.N = (int)w->rows; g.K = (int)w->cols;
-    g.packed = (const uint8_t*)w->packed; g.scales = (const float*)w->scales;
+    g.packed = (const uint8_t*)w->packed; g.scales = (const uint8_t*)w->scales;
+    g.gshift = 0;
+    for (int v = w->group; v > 1; v >>= 1) ++g.gshift;
+    g.scale_dtype = w->scale_dtype;
     g.lora_A = (const float*)lora_A; g.lora_B = (const float*)lora_B; g.r = r; g.su_scale = scaling;
     g.bias = bias; g.y = y;
     g.nsu = r > 0 ? (int)(w->cols / kSuPartK) : 0;
-    g.nw = p.nw; g.sets = p.sets; g.gmax = p.gmax;
+    g.nw = p.nw; g.sets = p.sets; g.gmax = p.gmax; g.rps = p.rps;
     g.slot = nullptr; g.fail = nullptr;
     g.spin_limit = g_rows_spin_limit.load();
     if (r > 0) {
         const int rc = rows_slot(slot_key, stream, &g.slot, &g.fail);
         if (rc) return rc;
     }
-    skinny_gemv_kernel<kGemvRows><<<p.blocks + (unsigned)g.nsu, (unsigned)((p.sets * p.nw + 1) * 64), 0, stream>>>(g);
+    const unsigned grid = p.blocks + (unsigned)g.nsu, threads = (unsigned)((p.sets * p.nw + 1) * 64);
+    if (w->format == XQ_FMT_FP8) skinny_gemv_kernel<XQ_FMT_FP8, kGemvRows><<<grid, threads, 0, stream>>>(g);
+    else skinny_gemv_kernel<XQ_FMT_INT4, kGemvRows><<<grid, threads, 0, stream>>>(g);
     return XQ_OK;
 }
 
