@@ -53,10 +53,10 @@ MEASURED_TRAFFIC = {
     # gemm_dtl16_kernel<.., grouped>: mean over the 4 launches of a step (gate|up forward over two banks, down
     # forward, d_h, dx as one sum over both banks)
     3: (1395.0 * 2 ** 20, "profiles/gemm_dtl16_fp8_grouped_moe_e128.txt", 0.6417),
-    # skinny_rows_kernel (M <= 16) and skinny_split_kernel + skinny_epilogue_kernel (M = 32, 64): mean per forward
-    # over the 32 cases (includes the fp32 partial tiles of the two-launch cases written and read back: 23.3 MiB of
-    # it are algorithmic)
-    4: (39.7 * 2 ** 20, "profiles/skinny_kernels_decode_shapes.txt", 0.01688),
+    # skinny_gemv_kernel (M = 1), skinny_rows_kernel (M <= 16) and skinny_split_kernel + skinny_epilogue_kernel
+    # (M = 32, 64): mean per forward over the 32 cases (includes the fp32 partial tiles of the two-launch cases
+    # written and read back: 23.3 MiB of it are algorithmic)
+    4: (39.3 * 2 ** 20, "profiles/skinny_kernels_decode_shapes.txt", 0.01721),
     # merge_prep_kernel + merge_kernel<fp8>: mean per call (re-quantise 96 MiB, publish 144 MiB algorithmic)
     5: (134.4 * 2 ** 20, "profiles/merge_kernel_fp8_mlp_weights.txt", 0.04168),
     # gemm_256_kernel<nf4>: mean of the forward and dgrad launches
@@ -254,9 +254,9 @@ def other_config(cfg: int, dev):
         return (step, total, True,
                 "configs[4]: skinny-M forward, M in {1,8,32,64} x {q 4096->4096, kv 4096->1024, gate/up 4096->12288, "
                 "down 12288->4096} x {int4, block_fp8}, r=16 (32 forwards per step)",
-                "skinny_rows_kernel<int4|fp8> (M <= 16, one launch) and skinny_split_kernel<int4|fp8> + "
-                "skinny_epilogue_kernel (M = 32, 64) (weight-streaming fused dequant-GEMV/GEMM; the timed region is "
-                "the whole forward)")
+                "skinny_gemv_kernel<int4|fp8> (M = 1, dot products), skinny_rows_kernel<int4|fp8> (M <= 16, one launch) "
+                "and skinny_split_kernel<int4|fp8> + skinny_epilogue_kernel (M = 32, 64) (weight-streaming fused "
+                "dequant-GEMV/GEMM; the timed region is the whole forward)")
     if cfg == 5:
         # not a BASELINE config: the merge / re-quantise pass over configs[1]'s three block_fp8 weights (r = 32)
         from xorl_amd.functional import merge_dense, merge_requant_fp8

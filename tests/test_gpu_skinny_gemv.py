@@ -56,7 +56,7 @@ def _forward(m, x, r):
     ("int4", 12304, 2048, 16, False),         # one wave per set, 4 rows per set and sets left without rows
     ("block_fp8", 4096, 5120, 0, True),       # no low-rank term
     ("int4", 4096, 4096, 16, False),          # 2 KB rows: two waves per set, four sets
-    ("int4", 12288, 4096, 16, True),
+    ("int4", 12288, 4096, 16, True),          # many short rows: stays on the MFMA kernel
     ("int4", 4096, 12288, 16, False),         # 6 waves per set, one set
     ("int4", 1024, 2048, 8, True),            # one wave per set
     ("int4", 2048, 8192, 0, False),

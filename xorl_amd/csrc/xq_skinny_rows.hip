@@ -951,9 +951,9 @@ int launch_skinny_rows(const xq_weight* w, const bf16_t* x, int64_t ldx, int64_t
 // read once per block: ~500 readers of the same few lines, not thousands.  (A part's entry for rank j sits at pair j of the
 // part's 256; tags keep launches of the two kernels on one slot apart.)
 // int4 takes the same kernel with 32 weights per lane and load (rows of 2 KB per wave): its time is the decode's -- as
-// many instructions per weight as block fp8, twice as many per byte -- so it is level with the MFMA kernel on the large
-// shapes and ahead where that kernel's organisation fits badly (q, kv, down: -15 %).  nf4 and nvfp4 stay on the MFMA
-// kernel.
+// many instructions per weight as block fp8, twice as many per byte -- so it is level with the MFMA kernel on weights of
+// many short rows (those stay on that kernel) and ahead where that kernel's organisation fits badly (q, kv, down: -15 %).
+// nf4 and nvfp4 stay on the MFMA kernel.
 constexpr int kGemvRows = 4;                        // rows per group: with the next group's, 8 loads of a lane in flight
 constexpr int kGemvSlots = 64 / kGemvRows;          // groups of rows per block at most (all its sets together)
 
@@ -1289,6 +1289,9 @@ bool skinny_gemv_supported(const xq_weight* w, int64_t M, const void* lora_A, co
         return false;
     // (bf16 scales are read as the aligned words that hold them: the array must end on a word)
     if (w->format == XQ_FMT_INT4 && (w->rows * w->cols / w->group) % 2 != 0) return false;
+    // int4 is decode-bound in either kernel; this one is ahead where the other's organisation fits badly -- few rows (q, kv)
+    // or long ones (down: -15 %) -- and 3 % behind on many short rows (gate/up [12288, 4096], [24576, 4096]), which stay there
+    if (w->format == XQ_FMT_INT4 && w->rows > 4096 && w->cols < 8192) return false;
     const int64_t row_bytes = w->format == XQ_FMT_FP8 ? w->cols : w->cols / 2;
     if (row_bytes % 1024 != 0 || row_bytes / 1024 > 15 || w->rows < 1 || w->rows >= (1ll << 30)) return false;
     if (!xq_aligned(w->packed, 16)) return false;
