@@ -12,7 +12,7 @@ import pytest
 import torch
 
 from oracle import recipe as R
-from tests.util_cases import close, gen, make_dense_module, single_rows_on_the_mfma_kernel
+from tests.util_cases import close, gen, make_dense_module
 
 pytestmark = pytest.mark.gpu
 TOL = 1e-2
@@ -26,10 +26,9 @@ def _job(m, r=None, bias=True):
 
 
 def _separate(x, jobs):
-    """The forwards one by one, on the kernel that the joint launch uses."""
     from xorl_amd.functional import qlora_linear
 
-    with torch.no_grad(), single_rows_on_the_mfma_kernel():
+    with torch.no_grad():
         return [qlora_linear(x, qw, A, B, r, s, b) for qw, A, B, r, s, b in jobs]
 
 
@@ -201,9 +200,7 @@ def test_mlp_forward_without_autograd_is_the_module_calls(hip_device, fmt):
         xd = x.to(hip_device)
         with torch.no_grad():
             got = qlora_mlp_forward(g, u, d, xd)
-            with single_rows_on_the_mfma_kernel():       # gate and up share a launch of that kernel; down is a call of its own
-                gate, up = g(xd), u(xd)
-            want = d(silu_and_mul(gate, up))
+            want = d(silu_and_mul(g(xd), u(xd)))
         assert got.shape == (M, H) and torch.equal(got, want)
         close(got.cpu(), R.mlp_fwd_bwd_exact(x, wg, wu, wd, loras, g.scaling)["y"], 2e-2)
     # with a bias on every projection (no oracle program for it: the module calls are the reference)
@@ -236,8 +233,7 @@ def test_gate_up_with_swiglu_finish(hip_device, fmt, I, K, r, has_bias):
         xd = x.to(hip_device)
         with torch.no_grad():
             got = qlora_gate_up_silu(m, xd)
-            with single_rows_on_the_mfma_kernel():
-                gate, up = m(xd).chunk(2, dim=-1)
+            gate, up = m(xd).chunk(2, dim=-1)
             want = silu_and_mul(gate, up)
         assert got.shape == (M, I) and got.dtype == torch.bfloat16
         assert torch.equal(got, want)

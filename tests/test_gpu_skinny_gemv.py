@@ -108,6 +108,35 @@ def test_one_workspace_alternating_between_the_kernels(hip_device, fmt):
         close(y.cpu(), ex["y"], TOL)
 
 
+def test_joint_launches_on_either_kernel(hip_device, kernels):
+    """q + k + v in one launch and gate | up with the SwiGLU finish, one row: the dot-product kernel's results against the
+    MFMA kernel's (same decoded weights, other summation order) and against the separate calls (same bits on either)."""
+    from xorl_amd.functional import qlora_linear, qlora_linear_multi, silu_and_mul
+    from xorl_amd.qlora import qlora_gate_up_silu
+
+    K = 4096
+    mods = [make_dense_module("block_fp8", N, K, 16, 32, seed=N + i, device=hip_device, bias=(i == 1))[0] for i, N in enumerate((4096, 1024, 1024))]
+    jobs = [(m._quant_weight(), m.lora_A.detach(), m.lora_B.detach(), 16, m.scaling, m.bias) for m in mods]
+    gu, _ = make_dense_module("block_fp8", 2 * 3072, K, 16, 32, seed=77, device=hip_device)
+    for call in range(2):
+        x = gen((1, K), 1.0, 40 + call, torch.bfloat16).to(hip_device)
+
+        def joint():
+            with torch.no_grad():
+                ys = qlora_linear_multi(x, jobs)
+                sep = [qlora_linear(x, *j) for j in jobs]
+                h = qlora_gate_up_silu(gu, x)
+                gate, up = gu(x).chunk(2, dim=-1)
+                return ys, sep, h, silu_and_mul(gate, up)
+
+        (ys1, sep1, h1, hs1), (ys0, sep0, h0, hs0) = kernels(joint)
+        for a, b, c, d in zip(ys1, sep1, ys0, sep0):
+            assert torch.equal(a, b) and torch.equal(c, d)
+            close(a.cpu(), c.float().cpu(), 4e-3)
+        assert torch.equal(h1, hs1) and torch.equal(h0, hs0)
+        close(h1.cpu(), h0.float().cpu(), 8e-3)
+
+
 def test_dot_product_kernel_under_hip_graph(hip_device):
     """Captured once, replayed with x changing and eager calls on the same workspace in between: every replay gives the
     eager call's bits."""

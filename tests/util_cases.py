@@ -92,21 +92,3 @@ def oracle_decode_dense(m) -> torch.Tensor:
         s = m.weight_scales.cpu().contiguous().view(torch.float32).numpy()
         return bits_to_bf16(NP.nf4_decode_flat(packed, s, N, K, m.quant_group_size))
     raise ValueError(m.quant_format)
-
-
-class single_rows_on_the_mfma_kernel:
-    """Context: one activation row against a block-fp8 weight takes the kernel of the larger row counts instead of the
-    dot-product kernel, for tests that compare a joint launch with separate calls bit for bit (the two kernels sum in
-    different orders: same values to rounding, not the same bits)."""
-
-    def __enter__(self):
-        from xorl_amd import _C
-
-        _C.check(_C.lib().xq_set_skinny_gemv(0))
-
-    def __exit__(self, *exc):
-        from xorl_amd import _C
-
-        _C.check(_C.lib().xq_set_skinny_gemv(1))
-        return False
-

@@ -54,7 +54,7 @@ void set_skinny_rows_spin_limit(int limit);   // <= 0: the default
 void set_skinny_gemv(int on);                  // M = 1 on the dot-product kernel (default) or on the MFMA kernel
 bool skinny_gemv_supported(const xq_weight* w, int64_t M, const void* lora_A, const void* lora_B, int lora_dtype, int r);
 int launch_skinny_gemv(const xq_weight* w, const bf16_t* x, const void* lora_A, const void* lora_B, int r, float scaling,
-                       const bf16_t* bias, bf16_t* y, const void* slot_key, hipStream_t stream);
+                       const bf16_t* bias, bf16_t* y, const void* slot_key, hipStream_t stream, bool swiglu);
 int reset_skinny_rows_slots();                 // clears the current device's slots (synchronises the device)
 int skinny_rows_status(int* gave_up, int* failed_slots, hipStream_t stream);   // reads and clears the failure reports (synchronises the stream)
 

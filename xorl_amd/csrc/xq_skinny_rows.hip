@@ -916,7 +916,7 @@ static int rows_args(const xq_weight* w, const RowsPlan& p, const bf16_t* x, int
 
 int launch_skinny_rows(const xq_weight* w, const bf16_t* x, int64_t ldx, int64_t M, const void* lora_A, const void* lora_B, int r,
                        float scaling, const bf16_t* bias, bf16_t* y, int64_t ldy, const void* slot_key, hipStream_t stream) {
-    if (skinny_gemv_supported(w, M, lora_A, lora_B, XQ_DT_F32, r)) return launch_skinny_gemv(w, x, lora_A, lora_B, r, scaling, bias, y, slot_key, stream);
+    if (skinny_gemv_supported(w, M, lora_A, lora_B, XQ_DT_F32, r)) return launch_skinny_gemv(w, x, lora_A, lora_B, r, scaling, bias, y, slot_key, stream, false);
     RowsPlan p;
     XQ_REQUIRE(rows_plan(w, M, &p), "xq_linear_fwd: internal error: shape not supported by the one-launch skinny kernel");
     SkinnyRowsArgs g;
@@ -953,7 +953,8 @@ int launch_skinny_rows(const xq_weight* w, const bf16_t* x, int64_t ldx, int64_t
 // int4 takes the same kernel with 32 weights per lane and load (rows of 2 KB per wave): its time is the decode's -- as
 // many instructions per weight as block fp8, twice as many per byte -- so it is level with the MFMA kernel on weights of
 // many short rows (those stay on that kernel) and ahead where that kernel's organisation fits badly (q, kv, down: -15 %).
-// nf4 and nvfp4 stay on the MFMA kernel.
+// nf4 and nvfp4 stay on the MFMA kernel.  Several forwards on one x (xq_linear_fwd_multi) and gate | up with the SwiGLU
+// finish (xq_linear_fwd_swiglu) take the same body: see skinny_gemv_multi_kernel and the GU form below.
 constexpr int kGemvRows = 4;                        // rows per group: with the next group's, 8 loads of a lane in flight
 constexpr int kGemvSlots = 64 / kGemvRows;          // groups of rows per block at most (all its sets together)
 
@@ -990,23 +991,28 @@ struct GemvArgs {
 
 // (registers held to what lets 6 waves share a SIMD: left to itself the compiler spends the 128 that blocks of up to 16 waves
 // allow on decoding all rows of a group at once)
-template <int FMT, int RB>
-__global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(FMT == XQ_FMT_FP8 ? 6 : 5, 8))) skinny_gemv_kernel(GemvArgs g) {
+// `blk` of `nb`: this block among those of its forward (a launch may hold several forwards, one after the other).
+// GU: the weight is gate | up stacked, [2 I, K]; the rows are walked as gate 0, up 0, gate 1, up 1, ... so that the two
+// rows of a column meet in neighbouring lanes of the finish, which writes h [I] = bf16(bf16(silu(gate)) * up) from the two
+// rounded outputs (the arithmetic of the SwiGLU kernel, ops/fused_silu_and_mul.py:22-60) instead of the outputs themselves.
+template <int FMT, int RB, bool GU>
+__device__ __forceinline__ void skinny_gemv_body(const GemvArgs& g, const int blk, const int nb) {
     constexpr bool F8 = FMT == XQ_FMT_FP8;
     constexpr int EPL = F8 ? 16 : 32;                 // weights of a row per lane (one 16-byte load)
     __shared__ float red[kGemvSlots][RB][16];         // [set * gmax + group of the set][row][wave of the set]
     __shared__ float zpart[16][17];                   // a block that forms a part of z: [k slice][rank]
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int nb = gridDim.x;
     const bool lora = g.nsu > 0;
+    // row of the weight for row j of the walk
+    auto weight_row = [&](int j) { return GU ? ((j & 1) ? (g.N >> 1) + (j >> 1) : (j >> 1)) : j; };
 
     // ---- the first K / 512 blocks of a launch with a low-rank term form the parts of z and nothing else (they are gone
     // after a few microseconds; a block that streamed as well would be late by a memory latency under load, and the
     // launch with it): 256 threads contract 512 elements of K for the 16 ranks, thread (slice, rank) a run of 32 elements;
     // the slices are summed in order by the threads of slice 0 and published with the launch's tag
-    if ((int)blockIdx.x < g.nsu) {
-        const int part = blockIdx.x;
+    if (blk < g.nsu) {
+        const int part = blk;
         if (wave >= 4) return;
         // (the launch count through this XCD's L2: no line of the slot can be there from before the launch, and within a
         // launch the word changes only after every block has read it; the block is counted in once it has been read)
@@ -1050,7 +1056,7 @@ __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(FMT =
         return;
     }
 
-    const int bx = blockIdx.x - g.nsu, nbs = nb - g.nsu;   // this block among those that stream
+    const int bx = blk - g.nsu;                      // this block among those that stream
     const int nstream = g.sets * g.nw;                // streaming waves; wave `nstream` is the one that does not stream
     const bool streamer = wave < nstream;
     const int st = wave / g.nw, ws = wave - st * g.nw;
@@ -1075,7 +1081,7 @@ __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(FMT =
         auto issue = [&](u32x4 (&w)[RB], float (&sc)[RB], int gi) {
 #pragma unroll
             for (int i = 0; i < RB; ++i) {
-                const int n = row0 + (gi * RB + i < nrows ? gi * RB + i : nrows - 1);
+                const int n = weight_row(row0 + (gi * RB + i < nrows ? gi * RB + i : nrows - 1));
                 w[i] = __builtin_nontemporal_load((const u32x4*)(g.packed + (int64_t)n * row_bytes + (ws * 64 + lane) * 16));
                 if (F8) {
                     sc[i] = ((const float*)g.scales)[(n >> 7) * sc_cols + (kbase >> 7)];
@@ -1088,7 +1094,7 @@ __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(FMT =
         // the scale of row i of a group from what `issue` fetched (int4 with bf16 scales: the half that the index names)
         auto scale_of = [&](float raw, int gi, int i) -> float {
             if (F8 || s32) return raw;
-            const int n = row0 + (gi * RB + i < nrows ? gi * RB + i : nrows - 1);
+            const int n = weight_row(row0 + (gi * RB + i < nrows ? gi * RB + i : nrows - 1));
             const int64_t si = ((int64_t)n * g.K + kbase) >> g.gshift;
             const uint32_t u = __float_as_uint(raw);
             return __uint_as_float((si & 1) ? u & 0xffff0000u : u << 16);
@@ -1164,14 +1170,15 @@ __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(FMT =
     const int f_slot = lane / RB, f_i = lane - f_slot * RB;
     const int f_set = f_slot / g.gmax, f_gi = f_slot - f_set * g.gmax;
     const int f_row = f_gi * RB + f_i;                // row within the set's range
-    const int fn = (bx * g.sets + f_set) * g.rps + f_row;
-    const bool finisher = f_set < g.sets && f_row < g.rps && fn < g.N;
+    const int fj = (bx * g.sets + f_set) * g.rps + f_row;          // row of the walk
+    const bool finisher = f_set < g.sets && f_row < g.rps && fj < g.N;
+    const int fn = weight_row(finisher ? fj : 0);     // row of the weight
     uint32_t gen = 0;
     f32x4 brow[4];
     float bias_v = 0.0f;
     if (lora) {
         // (past the caches: it is not needed before the first look at the parts has returned)
-        gen = __hip_atomic_load(g.slot + kSlotCtl + (blockIdx.x % kCtlCopies) * kCtlStride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        gen = __hip_atomic_load(g.slot + kSlotCtl + (blk % kCtlCopies) * kCtlStride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
@@ -1182,7 +1189,7 @@ __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(FMT =
     if (lora && lane == 0) {
         uint32_t one = 1u;
         asm volatile("" : "+v"(one) : "v"(gen));       // (the add may not move ahead of the point where `gen` is in its register)
-        __hip_atomic_fetch_add(g.slot + kSlotCtl + (kCtlCopies + blockIdx.x % kCtlCopies) * kCtlStride, one, __ATOMIC_RELAXED,
+        __hip_atomic_fetch_add(g.slot + kSlotCtl + (kCtlCopies + blk % kCtlCopies) * kCtlStride, one, __ATOMIC_RELAXED,
                                __HIP_MEMORY_SCOPE_AGENT);
     }
     // ---- while the sets stream: collect all parts -- lane (q, j) takes rank j of the parts q, q + 4, ... -- looking past
@@ -1190,7 +1197,7 @@ __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(FMT =
     float zv = 0.0f;                                  // lane j < 16 (and the lanes 16 apart): z[j] * scaling
     bool whole = true;
     if (lora) {
-        const bool closer = (int)blockIdx.x == nb - 1;
+        const bool closer = blk == nb - 1;
         const bool failed_slot = gen == kGenPoison;
         bool missing = failed_slot, open = closer && !failed_slot;
         float z = 0.0f;
@@ -1253,7 +1260,40 @@ __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(FMT =
         if (!whole) o = __builtin_nanf("");
     }
     if (g.bias) o += bias_v;
-    if (finisher) g.y[fn] = to_bf16(o);
+    if constexpr (GU) {
+        // (RB and the sets' ranges are even: lane t even holds a column's gate, lane t + 1 its up)
+        const float up = lane_perm<0xB1>(o);
+        const float gate = round_bf16(o);
+        if (finisher && !(lane & 1)) g.y[fj >> 1] = to_bf16(round_bf16(gate * sigmoid_f32(gate)) * round_bf16(up));
+    } else {
+        if (finisher) g.y[fn] = to_bf16(o);
+    }
+}
+
+template <int FMT, int RB, bool GU>
+__global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(FMT == XQ_FMT_FP8 ? 6 : 5, 8))) skinny_gemv_kernel(GemvArgs g) {
+    skinny_gemv_body<FMT, RB, GU>(g, (int)blockIdx.x, (int)gridDim.x);
+}
+
+// several forwards on one x (same format and K, hence the same block shape) in one grid: first the blocks that form the
+// parts of z, forward by forward (so that none of them waits behind another forward's rows for a CU), then the streaming
+// blocks, forward by forward; a block finds its forward by its index (the boundaries are leading scalars, with the wave
+// from the start).  p1 .. p4, s1 .. s4: blocks of either kind before the second, third, fourth forward and in all.
+struct GemvBatch {
+    GemvArgs job[kRowsMaxJobs];
+};
+template <int FMT, int RB>
+__global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(FMT == XQ_FMT_FP8 ? 6 : 5, 8)))
+skinny_gemv_multi_kernel(int32_t p1, int32_t p2, int32_t p3, int32_t p4, int32_t s1, int32_t s2, int32_t s3, int32_t s4, GemvBatch b) {
+    const int bx = (int)blockIdx.x;
+    const bool forms_z = bx < p4;
+    const int c = forms_z ? bx : bx - p4;             // index among the blocks of its kind
+    const int f1 = forms_z ? p1 : s1, f2 = forms_z ? p2 : s2, f3 = forms_z ? p3 : s3;
+    const int i = (c >= f1 ? 1 : 0) + (c >= f2 ? 1 : 0) + (c >= f3 ? 1 : 0);   // uniform
+    const int plo = i == 0 ? 0 : i == 1 ? p1 : i == 2 ? p2 : p3, phi = i == 0 ? p1 : i == 1 ? p2 : i == 2 ? p3 : p4;
+    const int slo = i == 0 ? 0 : i == 1 ? s1 : i == 2 ? s2 : s3, shi = i == 0 ? s1 : i == 1 ? s2 : i == 2 ? s3 : s4;
+    const int nsu = phi - plo;                        // this forward's blocks that form z come first in its own count
+    skinny_gemv_body<FMT, RB, false>(b.job[i], forms_z ? c - plo : nsu + (c - slo), nsu + (shi - slo));
 }
 
 static std::atomic<int> g_skinny_gemv{[] { const char* e = getenv("XQ_SKINNY_GEMV"); return e ? atoi(e) : 1; }()};
@@ -1267,16 +1307,20 @@ struct GemvPlan {
     int nw, sets, gmax, rps;
     unsigned blocks;
 };
-static GemvPlan gemv_plan(const xq_weight* w) {
+// `share`: this forward's part of the blocks that the CUs hold at once (1 for a launch of its own; in a joint launch the
+// forwards split them by their rows).  `even`: ranges of an even number of rows (gate | up walked in pairs).
+static GemvPlan gemv_plan(const xq_weight* w, double share = 1.0, bool even = false) {
     GemvPlan p;
     p.nw = (int)((w->format == XQ_FMT_FP8 ? w->cols : w->cols / 2) / 1024);
     p.sets = 8 / p.nw > 1 ? 8 / p.nw : 1;
     const int cap = (kGemvSlots / p.sets) * kGemvRows;     // rows of a set at most
-    const int64_t fill = 256 * (20 / (p.sets * p.nw + 1) > 1 ? 20 / (p.sets * p.nw + 1) : 1);
+    int64_t fill = (int64_t)(256 * (20 / (p.sets * p.nw + 1) > 1 ? 20 / (p.sets * p.nw + 1) : 1) * share + 0.5);
+    if (fill < 1) fill = 1;
     int64_t nb = xq_cdiv(w->rows, (int64_t)p.sets * kGemvRows) < fill ? xq_cdiv(w->rows, (int64_t)p.sets * kGemvRows) : fill;
     if (xq_cdiv(w->rows, (int64_t)p.sets * cap) > nb) nb = xq_cdiv(w->rows, (int64_t)p.sets * cap);
     p.blocks = (unsigned)nb;
     p.rps = (int)xq_cdiv(w->rows, nb * p.sets);            // the rows dealt evenly: a set's range is at most one row longer than another's
+    if (even) p.rps += p.rps & 1;                          // (cap is even)
     p.gmax = (int)xq_cdiv(p.rps, kGemvRows);
     return p;
 }
@@ -1302,12 +1346,11 @@ bool skinny_gemv_supported(const xq_weight* w, int64_t M, const void* lora_A, co
     return true;
 }
 
-int launch_skinny_gemv(const xq_weight* w, const bf16_t* x, const void* lora_A, const void* lora_B, int r, float scaling,
-                       const bf16_t* bias, bf16_t* y, const void* slot_key, hipStream_t stream) {
-    const GemvPlan p = gemv_plan(w);
+static int gemv_args(const xq_weight* w, const GemvPlan& p, const bf16_t* x, const void* lora_A, const void* lora_B, int r, float scaling,
+                     const bf16_t* bias, bf16_t* y, const void* slot_key, hipStream_t stream, GemvArgs* out) {
     XQ_REQUIRE(p.sets * p.gmax <= kGemvSlots && p.sets * p.nw >= 4 && (p.sets * p.nw + 1) * 64 <= 1024,
                "xq_linear_fwd: internal error: dot-product launch out of range");
-    GemvArgs g;
+    GemvArgs& g = *out;
     g.x = x; g.N = (int)w->rows; g.K = (int)w->cols;
     g.packed = (const uint8_t*)w->packed; g.scales = (const uint8_t*)w->scales;
     g.gshift = 0;
@@ -1319,13 +1362,58 @@ int launch_skinny_gemv(const xq_weight* w, const bf16_t* x, const void* lora_A, 
     g.nw = p.nw; g.sets = p.sets; g.gmax = p.gmax; g.rps = p.rps;
     g.slot = nullptr; g.fail = nullptr;
     g.spin_limit = g_rows_spin_limit.load();
-    if (r > 0) {
-        const int rc = rows_slot(slot_key, stream, &g.slot, &g.fail);
-        if (rc) return rc;
-    }
+    if (r > 0) return rows_slot(slot_key, stream, &g.slot, &g.fail);
+    return XQ_OK;
+}
+
+// swiglu: w is gate | up [2 I, K] and y is h [I]
+int launch_skinny_gemv(const xq_weight* w, const bf16_t* x, const void* lora_A, const void* lora_B, int r, float scaling,
+                       const bf16_t* bias, bf16_t* y, const void* slot_key, hipStream_t stream, bool swiglu) {
+    const GemvPlan p = gemv_plan(w, 1.0, swiglu);
+    GemvArgs g;
+    const int rc = gemv_args(w, p, x, lora_A, lora_B, r, scaling, bias, y, slot_key, stream, &g);
+    if (rc) return rc;
     const unsigned grid = p.blocks + (unsigned)g.nsu, threads = (unsigned)((p.sets * p.nw + 1) * 64);
-    if (w->format == XQ_FMT_FP8) skinny_gemv_kernel<XQ_FMT_FP8, kGemvRows><<<grid, threads, 0, stream>>>(g);
-    else skinny_gemv_kernel<XQ_FMT_INT4, kGemvRows><<<grid, threads, 0, stream>>>(g);
+    if (w->format == XQ_FMT_FP8) {
+        if (swiglu) skinny_gemv_kernel<XQ_FMT_FP8, kGemvRows, true><<<grid, threads, 0, stream>>>(g);
+        else skinny_gemv_kernel<XQ_FMT_FP8, kGemvRows, false><<<grid, threads, 0, stream>>>(g);
+    } else {
+        if (swiglu) skinny_gemv_kernel<XQ_FMT_INT4, kGemvRows, true><<<grid, threads, 0, stream>>>(g);
+        else skinny_gemv_kernel<XQ_FMT_INT4, kGemvRows, false><<<grid, threads, 0, stream>>>(g);
+    }
+    return XQ_OK;
+}
+
+// several forwards (same format and K) in one grid; each has its own slot, keyed 256 bytes apart inside the caller's workspace
+static int launch_skinny_gemv_multi(const SkinnyRowsJob* jobs, int n_jobs, const bf16_t* x, const void* slot_key, hipStream_t stream) {
+    int64_t rows = 0;
+    for (int i = 0; i < n_jobs; ++i) rows += jobs[i].w->rows;
+    GemvBatch b;
+    int32_t pf[kRowsMaxJobs + 1], sf[kRowsMaxJobs + 1];   // blocks that form z / that stream, before each forward
+    int pat = 0, sat = 0;
+    unsigned threads = 0;
+    for (int i = 0; i < kRowsMaxJobs; ++i) {
+        pf[i] = pat;
+        sf[i] = sat;
+        if (i >= n_jobs) {
+            b.job[i] = b.job[0];
+            continue;
+        }
+        const GemvPlan p = gemv_plan(jobs[i].w, (double)jobs[i].w->rows / (double)rows);
+        const int rc = gemv_args(jobs[i].w, p, x, jobs[i].lora_A, jobs[i].lora_B, jobs[i].r, jobs[i].scaling, jobs[i].bias, jobs[i].y,
+                                 (const char*)slot_key + 256 * i, stream, &b.job[i]);
+        if (rc) return rc;
+        pat += b.job[i].nsu;
+        sat += (int)p.blocks;
+        threads = (unsigned)((p.sets * p.nw + 1) * 64);
+    }
+    pf[kRowsMaxJobs] = pat;
+    sf[kRowsMaxJobs] = sat;
+    const unsigned grid = (unsigned)(pat + sat);
+    if (jobs[0].w->format == XQ_FMT_FP8)
+        skinny_gemv_multi_kernel<XQ_FMT_FP8, kGemvRows><<<grid, threads, 0, stream>>>(pf[1], pf[2], pf[3], pf[4], sf[1], sf[2], sf[3], sf[4], b);
+    else
+        skinny_gemv_multi_kernel<XQ_FMT_INT4, kGemvRows><<<grid, threads, 0, stream>>>(pf[1], pf[2], pf[3], pf[4], sf[1], sf[2], sf[3], sf[4], b);
     return XQ_OK;
 }
 
@@ -1364,6 +1452,8 @@ bool skinny_rows_swiglu_supported(const xq_weight* w, int64_t M, const void* lor
 
 int launch_skinny_rows_swiglu(const xq_weight* w, const bf16_t* x, int64_t ldx, int64_t M, const void* lora_A, const void* lora_B, int r,
                               float scaling, const bf16_t* bias, bf16_t* h, int64_t ldh, const void* slot_key, hipStream_t stream) {
+    if (w->rows % 2 == 0 && skinny_gemv_supported(w, M, lora_A, lora_B, XQ_DT_F32, r))
+        return launch_skinny_gemv(w, x, lora_A, lora_B, r, scaling, bias, h, slot_key, stream, true);
     RowsPlan p;
     XQ_REQUIRE(rows_plan(w, M, &p) && p.R == 2 && p.G == 3 && ldx < (1ll << 31),
                "xq_linear_fwd_swiglu: internal error: shape not supported by the one-launch skinny kernel");
@@ -1402,6 +1492,9 @@ int launch_skinny_rows_multi(const SkinnyRowsJob* jobs, int n_jobs, const bf16_t
                              hipStream_t stream) {
     const xq_weight* ws[kRowsMaxJobs];
     for (int i = 0; i < n_jobs; ++i) ws[i] = jobs[i].w;
+    bool dots = true;                                  // one row, every forward on the dot-product kernel
+    for (int i = 0; i < n_jobs; ++i) dots = dots && skinny_gemv_supported(ws[i], M, jobs[i].lora_A, jobs[i].lora_B, XQ_DT_F32, jobs[i].r);
+    if (dots) return launch_skinny_gemv_multi(jobs, n_jobs, x, slot_key, stream);
     RowsPlan p;
     XQ_REQUIRE(rows_plan_multi(ws, n_jobs, M, &p), "xq_linear_fwd_multi: internal error: shapes not supported by the one-launch skinny kernel");
     SkinnyRowsBatch b;
