@@ -1118,10 +1118,11 @@ __device__ __forceinline__ void skinny_gemv_body(const GemvArgs& g, const int bl
 #pragma unroll
                     for (int e = 0; e < 4; ++e) dot2_bf16(a[i], wp[e], xv[c][e]);
                 }
+                // (a dot instruction's result may be read, or its register written, by another kind of instruction only
+                // 3 - 4 cycles later; the compiler keeps that distance for its own instructions and cannot see into
+                // the asm above: the wait is tied to the sum, so that whatever uses it comes behind)
+                asm volatile("s_nop 3" : "+v"(a[i]));
             }
-            // (a dot instruction's result may be read by another kind of instruction only some cycles later; the compiler
-            // keeps that distance for its own instructions and cannot see into the asm above)
-            asm volatile("s_nop 3" ::: "memory");
 #pragma unroll
             for (int i = 0; i < RB; ++i) {
                 float t = a[i];
