@@ -108,6 +108,39 @@ def test_one_workspace_alternating_between_the_kernels(hip_device, fmt):
         close(y.cpu(), ex["y"], TOL)
 
 
+@pytest.mark.parametrize("N,K,group,symmetric", [(4096, 4096, 128, True), (1024, 8192, 32, True), (2048, 2048, 64, True),
+                                                     (4096, 4096, 128, False), (1024, 4096, 32, False)])
+def test_int4_scale_types_and_groups(hip_device, kernels, N, K, group, symmetric):
+    """int4 with bf16 scales (the symmetric rule's storage) and fp32 scales (the reference codec's rule), groups of 32 to
+    128: the dot-product kernel against the oracle's decode and, to rounding, against the MFMA kernel."""
+    from tests.util_cases import oracle_decode_dense
+    from xorl_amd.functional import qlora_linear
+    from xorl_amd.qlora.linear import Int4QLoRALinear
+
+    m = Int4QLoRALinear(K, N, r=16, lora_alpha=32, quant_group_size=group, symmetric=symmetric)
+    with torch.no_grad():
+        m._init_from_weight(gen((N, K), 0.02, N + K + group))
+        m.lora_A.copy_(gen((16, K), 0.02, 1))
+        m.lora_B.copy_(gen((N, 16), 0.02, 2))
+    w_ref = oracle_decode_dense(m)
+    m = m.to(hip_device)
+    qw = m._quant_weight()
+    assert qw.scale_dtype == (torch.bfloat16 if symmetric else torch.float32) and qw.group == group
+    A, B = m.lora_A.detach(), m.lora_B.detach()
+    x = gen((1, K), 1.0, 9, torch.bfloat16)
+    xd = x.to(hip_device)
+
+    def forward():
+        with torch.no_grad():
+            return qlora_linear(xd, qw, A, B, 16, m.scaling)
+
+    dot, mfma = kernels(forward)
+    close(dot.cpu(), mfma.float().cpu(), 4e-3)
+    ex = R.linear_fwd_bwd_exact(x, w_ref, A.cpu(), B.cpu(), m.scaling)
+    close(dot.cpu(), ex["y"], TOL)
+    close(mfma.cpu(), ex["y"], TOL)
+
+
 def test_joint_launches_on_either_kernel(hip_device, kernels):
     """q + k + v in one launch and gate | up with the SwiGLU finish, one row: the dot-product kernel's results against the
     MFMA kernel's (same decoded weights, other summation order) and against the separate calls (same bits on either)."""
