@@ -46,13 +46,13 @@ MEASURED_TRAFFIC = {
     0: (109.6 * 2 ** 20, "profiles/gemm_128_int4_linear_m512.txt", 0.04315),
     # gemm_dtl16_kernel (dense block-fp8, 256x256 tiles): mean over the 5 launches of a step (gate, up and down
     # forward, d_h, dx as one sum over the gate and up weights)
-    1: (1070.5 * 2 ** 20, "profiles/gemm_dtl16_fp8_mlp_m8192.txt", 0.7717),
+    1: (1070.4 * 2 ** 20, "profiles/gemm_dtl16_fp8_mlp_m8192.txt", 0.7509),
     # gemm_256_kernel<nvfp4>, 256x256 tiles (whole rounds; trailing rows in K splits) and 128x128 tiles
     # (+ splitk_reduce_kernel): mean over the 12 launches of a step, fp32 partial sums included
     2: (185.7 * 2 ** 20, "profiles/gemm_256_nvfp4_attn_m4096.txt", 0.14304),
     # gemm_dtl16_kernel<.., grouped>: mean over the 4 launches of a step (gate|up forward over two banks, down
     # forward, d_h, dx as one sum over both banks)
-    3: (1395.0 * 2 ** 20, "profiles/gemm_dtl16_fp8_grouped_moe_e128.txt", 0.6417),
+    3: (1402.4 * 2 ** 20, "profiles/gemm_dtl16_fp8_grouped_moe_e128.txt", 0.6325),
     # skinny_gemv_kernel (M = 1), skinny_rows_kernel (M <= 16) and skinny_split_kernel + skinny_epilogue_kernel
     # (M = 32, 64): mean per forward over the 32 cases (includes the fp32 partial tiles of the two-launch cases
     # written and read back: 23.3 MiB of it are algorithmic)
