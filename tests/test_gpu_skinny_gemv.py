@@ -170,6 +170,54 @@ def test_joint_launches_on_either_kernel(hip_device, kernels):
         close(h1.cpu(), h0.float().cpu(), 8e-3)
 
 
+def test_overlapping_dot_product_forwards_on_two_streams(hip_device):
+    """One-row forwards on two streams, each with its own workspace (hence its own slot), small enough to run side by side
+    on the device: every result equals the one the same call gives alone."""
+    from xorl_amd import _C
+    from xorl_amd.functional import _workspace_bytes
+
+    r = 16
+    shapes = [("block_fp8", 1024, 4096), ("block_fp8", 2048, 2048), ("int4", 1024, 4096)]
+    L = _C.lib()
+    streams = [torch.cuda.Stream() for _ in shapes]
+    work = []
+    for i, (fmt, N, K) in enumerate(shapes):
+        m, _ = make_dense_module(fmt, N, K, r, 32, seed=80 + i, device=hip_device)
+        w = m._quant_weight().c()
+        A, B = m.lora_A.detach().contiguous(), m.lora_B.detach().contiguous()
+        wsb = _workspace_bytes(1, N, K, r)
+        ws = torch.empty(wsb, dtype=torch.uint8, device=hip_device)
+        xs = [gen((1, K), 1.0, 700 + 10 * i + j, torch.bfloat16).to(hip_device) for j in range(6)]
+        ys = [torch.empty(1, N, dtype=torch.bfloat16, device=hip_device) for _ in xs]
+        work.append((m, w, A, B, ws, wsb, xs, ys, N, K))
+
+    def call(i, j, y, stream):
+        m, w, A, B, ws, wsb, xs, _, N, K = work[i]
+        _C.check(L.xq_linear_fwd(ctypes.byref(w), xs[j].data_ptr(), K, 1, A.data_ptr(), B.data_ptr(), _C.XQ_DT_F32, r,
+                                 ctypes.c_float(m.scaling), None, y.data_ptr(), N, None, ws.data_ptr(), wsb, stream))
+
+    alone = []
+    for i in range(len(shapes)):
+        outs = []
+        for j in range(6):
+            y = torch.empty_like(work[i][7][j])
+            call(i, j, y, _C.stream_ptr(hip_device))
+            outs.append(y)
+        alone.append(outs)
+    torch.cuda.synchronize()
+    assert all(torch.isfinite(y.float()).all() for outs in alone for y in outs)
+    for st in streams:
+        st.wait_stream(torch.cuda.current_stream())
+    for rep in range(20):
+        for j in range(6):
+            for i in range(len(shapes)):
+                call(i, j, work[i][7][j], ctypes.c_void_p(streams[i].cuda_stream))
+    torch.cuda.synchronize()
+    for i in range(len(shapes)):
+        for j in range(6):
+            assert torch.equal(work[i][7][j], alone[i][j]), (i, j)
+
+
 def test_dot_product_kernel_under_hip_graph(hip_device):
     """Captured once, replayed with x changing and eager calls on the same workspace in between: every replay gives the
     eager call's bits."""
