@@ -1315,9 +1315,18 @@ static GemvPlan gemv_plan(const xq_weight* w, double share = 1.0, bool even = fa
     p.nw = (int)((w->format == XQ_FMT_FP8 ? w->cols : w->cols / 2) / 1024);
     p.sets = 8 / p.nw > 1 ? 8 / p.nw : 1;
     const int cap = (kGemvSlots / p.sets) * kGemvRows;     // rows of a set at most
-    int64_t fill = (int64_t)(256 * (20 / (p.sets * p.nw + 1) > 1 ? 20 / (p.sets * p.nw + 1) : 1) * share + 0.5);
+    // blocks: what the CUs hold at once at most (two blocks of 9 waves each, one of 13), fewer where the sets would get
+    // less than two groups of rows each (a block that lasts two steps hides its wait for the low-rank parts behind the
+    // second; measured on block-fp8 [4096, 4096]: 7.0 us against 8.3 with one step per set; int4, whose time is its
+    // decode, wants all the blocks it can have) but not fewer than one per CU, nor more than there are groups
+    const int per_cu = 20 / (p.sets * p.nw + 1) > 1 ? 20 / (p.sets * p.nw + 1) : 1;
+    int64_t fill = (int64_t)(256 * per_cu * share + 0.5), floor_ = (int64_t)(256 * share + 0.5);
     if (fill < 1) fill = 1;
-    int64_t nb = xq_cdiv(w->rows, (int64_t)p.sets * kGemvRows) < fill ? xq_cdiv(w->rows, (int64_t)p.sets * kGemvRows) : fill;
+    if (floor_ < 1) floor_ = 1;
+    const int64_t two_steps = xq_cdiv(w->rows, (int64_t)p.sets * 2 * kGemvRows);
+    int64_t nb = w->format != XQ_FMT_FP8 ? fill : two_steps > floor_ ? two_steps : floor_;
+    if (nb > fill) nb = fill;
+    if (nb > xq_cdiv(w->rows, (int64_t)p.sets * kGemvRows)) nb = xq_cdiv(w->rows, (int64_t)p.sets * kGemvRows);
     if (xq_cdiv(w->rows, (int64_t)p.sets * cap) > nb) nb = xq_cdiv(w->rows, (int64_t)p.sets * cap);
     p.blocks = (unsigned)nb;
     p.rps = (int)xq_cdiv(w->rows, nb * p.sets);            // the rows dealt evenly: a set's range is at most one row longer than another's
