@@ -56,7 +56,7 @@ MEASURED_TRAFFIC = {
     # skinny_gemv_kernel (M = 1), skinny_rows_kernel (M <= 16) and skinny_split_kernel + skinny_epilogue_kernel
     # (M = 32, 64): mean per forward over the 32 cases (includes the fp32 partial tiles of the two-launch cases
     # written and read back: 23.3 MiB of it are algorithmic)
-    4: (39.3 * 2 ** 20, "profiles/skinny_kernels_decode_shapes.txt", 0.01721),
+    4: (39.3 * 2 ** 20, "profiles/skinny_kernels_decode_shapes.txt", 0.01712),
     # merge_prep_kernel + merge_kernel<fp8>: mean per call (re-quantise 96 MiB, publish 144 MiB algorithmic)
     5: (134.4 * 2 ** 20, "profiles/merge_kernel_fp8_mlp_weights.txt", 0.04168),
     # gemm_256_kernel<nf4>: mean of the forward and dgrad launches
