@@ -139,13 +139,13 @@ int xq_get_mlp_gate_up_fused(void);   /* the current default: 0 or 1 */
  * summation orders).  A process-wide switch for tests and A/B measurements (XQ_SKINNY_ROWS=0 in the environment sets
  * it at load time); no counterpart in the reference. */
 int xq_set_skinny_one_launch(int enabled);
-/* One token (M = 1) against a FLAT block-fp8 or int4 weight whose rows are whole KBs (in_features % 1024 == 0, int4:
- * % 2048 and only shapes on which it is the faster kernel -- at most 4096 rows, or rows of 8192 elements and more; at
- * most 15 KB per row) runs a kernel of its own inside the one-launch path: no matrix cores, waves that stream
- * whole rows (block fp8: the rate of a plain read from HBM), same slots and same failure rules.  enabled = 0 sends those
- * forwards to the kernel of the larger row counts (results agree to rounding: same decoded values, other summation
- * order).  Process-wide switch for tests and A/B measurements (XQ_SKINNY_GEMV=0 in the environment); no counterpart in
- * the reference. */
+/* One token (M = 1) against a FLAT block-fp8, nvfp4 (e4m3 block scales) or int4 weight whose rows are whole KBs
+ * (in_features % 1024 == 0, the 4-bit formats: % 2048; at most 15 KB per row; int4 only on shapes on which it is the
+ * faster kernel -- at most 4096 rows, or rows of 8192 elements and more) runs a kernel of its own inside the one-launch
+ * path: no matrix cores, waves that stream whole rows (block fp8: the rate of a plain read from HBM), same slots and same
+ * failure rules.  enabled = 0 sends those forwards to the kernel of the larger row counts (results agree to rounding: same
+ * decoded values, other summation order).  Process-wide switch for tests and A/B measurements (XQ_SKINNY_GEMV=0 in the
+ * environment); no counterpart in the reference. */
 int xq_set_skinny_gemv(int enabled);
 
 /* Test switch (process-wide, no counterpart in the reference): how many times a bounded wait of the one-launch skinny

@@ -1,4 +1,4 @@
-"""GPU: one activation row (M = 1) through the dot-product kernel -- whole weight rows streamed by waves, decoded to the
+"""GPU: one activation row (M = 1; block fp8, int4, nvfp4) through the dot-product kernel -- whole weight rows streamed by waves, decoded to the
 reference decoder's bf16 values and multiplied without matrix cores -- against the oracle and against the MFMA kernel on
 the same inputs (xq_set_skinny_gemv(0)).  Beyond arithmetic the cases aim at: blocks of one wave (rows of 1 KB), ragged
 last blocks, a weight with fewer blocks than parts of the low-rank intermediate (falls back), the slot shared with the
@@ -60,7 +60,12 @@ def _forward(m, x, r):
     ("int4", 4096, 12288, 16, False),         # 6 waves per set, one set
     ("int4", 1024, 2048, 8, True),            # one wave per set
     ("int4", 2048, 8192, 0, False),
-    ("nf4", 4096, 4096, 16, False),           # the other 4-bit formats stay on the MFMA kernel whatever the switch says
+    ("nvfp4", 4096, 4096, 16, False),         # e2m1 codes, two e4m3 block scales per lane and row, the tensor's global scale
+    ("nvfp4", 12288, 4096, 16, True),
+    ("nvfp4", 4096, 12288, 8, False),
+    ("nvfp4", 1040, 2048, 16, True),          # one wave per set
+    ("nvfp4", 2048, 6144, 0, True),           # three waves per set, two sets
+    ("nf4", 4096, 4096, 16, False),           # nf4 stays on the MFMA kernel whatever the switch says
 ])
 def test_dot_product_kernel_vs_oracle_and_mfma_kernel(hip_device, kernels, fmt, N, K, r, has_bias):
     m, w_ref = make_dense_module(fmt, N, K, max(r, 1), 2 * max(r, 1), seed=N + K + r, device=hip_device, bias=has_bias)
@@ -79,7 +84,7 @@ def test_dot_product_kernel_vs_oracle_and_mfma_kernel(hip_device, kernels, fmt, 
         close(dot.cpu(), mfma.float().cpu(), 4e-3)
 
 
-@pytest.mark.parametrize("fmt", ["block_fp8", "int4"])
+@pytest.mark.parametrize("fmt", ["block_fp8", "int4", "nvfp4"])
 def test_one_workspace_alternating_between_the_kernels(hip_device, fmt):
     """M = 1 (dot-product kernel) and M = 8 (MFMA kernel) take turns on one workspace, hence one slot: each launch must
     see its own parts of the low-rank intermediate only.  The low-rank term dominates the output here, so that a stale or
@@ -177,7 +182,7 @@ def test_overlapping_dot_product_forwards_on_two_streams(hip_device):
     from xorl_amd.functional import _workspace_bytes
 
     r = 16
-    shapes = [("block_fp8", 1024, 4096), ("block_fp8", 2048, 2048), ("int4", 1024, 4096)]
+    shapes = [("block_fp8", 1024, 4096), ("block_fp8", 2048, 2048), ("int4", 1024, 4096), ("nvfp4", 1024, 4096)]
     L = _C.lib()
     streams = [torch.cuda.Stream() for _ in shapes]
     work = []

@@ -931,7 +931,7 @@ int launch_skinny_rows(const xq_weight* w, const bf16_t* x, int64_t ldx, int64_t
     }
 }
 
-// ---------------------------------------------------------------- M = 1, block fp8 and int4: dot products instead of MFMA tiles
+// ---------------------------------------------------------------- M = 1, block fp8, int4, nvfp4: dot products instead of MFMA tiles
 // One token against a packed weight needs no matrix cores, and the organisation above -- 8 waves per CU, a load instruction
 // that takes 64 bytes of each of 16 rows -- is what keeps it from the rate of a plain read when the bytes come from HBM
 // (8 waves per CU pull at most ~6 TB/s however deep their queues; a linear read by 32 waves per CU reaches 6.9).  Here the
@@ -950,11 +950,13 @@ int launch_skinny_rows(const xq_weight* w, const bf16_t* x, int64_t ldx, int64_t
 // dependent load costs ~3 us, and a block that is late by that makes the launch late by that -- and the parts of z are
 // read once per block: ~500 readers of the same few lines, not thousands.  (A part's entry for rank j sits at pair j of the
 // part's 256; tags keep launches of the two kernels on one slot apart.)
-// int4 takes the same kernel with 32 weights per lane and load (rows of 2 KB per wave): its time is the decode's -- as
-// many instructions per weight as block fp8, twice as many per byte -- so it is level with the MFMA kernel on weights of
-// many short rows (those stay on that kernel) and ahead where that kernel's organisation fits badly (q, kv, down: -15 %).
-// nf4 and nvfp4 stay on the MFMA kernel.  Several forwards on one x (xq_linear_fwd_multi) and gate | up with the SwiGLU
-// finish (xq_linear_fwd_swiglu) take the same body: see skinny_gemv_multi_kernel and the GU form below.
+// int4 and nvfp4 take the same kernel with 32 weights per lane and load (rows of 2 KB per wave; nvfp4: the lane's two e4m3
+// block scales come as one word, the tensor's global scale is a scalar).  Their time is the decode's -- as many
+// instructions per weight as block fp8, twice as many per byte.  nvfp4 is ahead of the MFMA kernel on every shape
+// measured (-8 % on many short rows to -30 % on few); int4 is level with it on weights of many short rows (those stay
+// on that kernel) and ahead where that kernel's organisation fits badly (q, kv, down: -15 %).  nf4 stays on the MFMA
+// kernel.  Several forwards on one x (xq_linear_fwd_multi) and gate | up with the SwiGLU finish (xq_linear_fwd_swiglu)
+// take the same body: see skinny_gemv_multi_kernel and the GU form below.
 constexpr int kGemvRows = 4;                        // rows per group: with the next group's, 8 loads of a lane in flight
 constexpr int kGemvSlots = 64 / kGemvRows;          // groups of rows per block at most (all its sets together)
 
@@ -974,7 +976,8 @@ struct GemvArgs {
     const bf16_t* x;
     int32_t N, K;
     const uint8_t* packed;
-    const uint8_t* scales;         // fp8: fp32 [ceil(N / 128), ceil(K / 128)]; int4: one per group along K
+    const uint8_t* scales;         // fp8: fp32 [ceil(N / 128), ceil(K / 128)]; int4: one per group along K; nvfp4: e4m3, one per 16
+    const float* global_scale;     // nvfp4: the tensor's second-level scale
     int32_t gshift, scale_dtype;   // int4: log2 of the group size, the scales' type
     const float* lora_A;           // [r, K] fp32
     const float* lora_B;           // [N, r] fp32
@@ -997,7 +1000,7 @@ struct GemvArgs {
 // rounded outputs (the arithmetic of the SwiGLU kernel, ops/fused_silu_and_mul.py:22-60) instead of the outputs themselves.
 template <int FMT, int RB, bool GU>
 __device__ __forceinline__ void skinny_gemv_body(const GemvArgs& g, const int blk, const int nb) {
-    constexpr bool F8 = FMT == XQ_FMT_FP8;
+    constexpr bool F8 = FMT == XQ_FMT_FP8, NV = FMT == XQ_FMT_NVFP4;
     constexpr int EPL = F8 ? 16 : 32;                 // weights of a row per lane (one 16-byte load)
     __shared__ float red[kGemvSlots][RB][16];         // [set * gmax + group of the set][row][wave of the set]
     __shared__ float zpart[16][17];                   // a block that forms a part of z: [k slice][rank]
@@ -1085,6 +1088,10 @@ __device__ __forceinline__ void skinny_gemv_body(const GemvArgs& g, const int bl
                 w[i] = __builtin_nontemporal_load((const u32x4*)(g.packed + (int64_t)n * row_bytes + (ws * 64 + lane) * 16));
                 if (F8) {
                     sc[i] = ((const float*)g.scales)[(n >> 7) * sc_cols + (kbase >> 7)];
+                } else if (NV) {
+                    // (the lane's two e4m3 scales, one per 16 weights, inside the aligned word that holds them)
+                    const int64_t si = ((int64_t)n * g.K + kbase) >> 4;
+                    sc[i] = *(const float*)(g.scales + (si & ~(int64_t)3));
                 } else {
                     const int64_t si = ((int64_t)n * g.K + kbase) >> g.gshift;
                     sc[i] = *(const float*)(g.scales + ((s32 ? si << 2 : si << 1) & ~(int64_t)3));
@@ -1092,13 +1099,16 @@ __device__ __forceinline__ void skinny_gemv_body(const GemvArgs& g, const int bl
             }
         };
         // the scale of row i of a group from what `issue` fetched (int4 with bf16 scales: the half that the index names)
+        // (nvfp4: the two scale bytes in the low half of the result's bits)
         auto scale_of = [&](float raw, int gi, int i) -> float {
-            if (F8 || s32) return raw;
+            if (F8 || (!NV && s32)) return raw;
             const int n = weight_row(row0 + (gi * RB + i < nrows ? gi * RB + i : nrows - 1));
-            const int64_t si = ((int64_t)n * g.K + kbase) >> g.gshift;
             const uint32_t u = __float_as_uint(raw);
+            if (NV) return __uint_as_float(u >> (8 * (int)((((int64_t)n * g.K + kbase) >> 4) & 2)));
+            const int64_t si = ((int64_t)n * g.K + kbase) >> g.gshift;
             return __uint_as_float((si & 1) ? u & 0xffff0000u : u << 16);
         };
+        const float gsc = NV ? g.global_scale[0] : 1.0f;
         // ---- the groups of this wave's set: the next one's loads go out, then the current one is decoded and multiplied,
         // summed over the wave's lanes (fixed order: within 16 lanes by lane-permuting adds, then the four 16s in order)
         // and left in LDS for the finish
@@ -1114,6 +1124,8 @@ __device__ __forceinline__ void skinny_gemv_body(const GemvArgs& g, const int bl
                 for (int c = 0; c < EPL / 8; ++c) {
                     u32x4 wp;
                     if constexpr (F8) wp = __builtin_bit_cast(u32x4, decode8<FMT>(w[i][2 * c], w[i][2 * c + 1], sv, 0.0f));
+                    else if constexpr (NV)
+                        wp = __builtin_bit_cast(u32x4, decode8<FMT>(w[i][c], 0u, e4m3_to_f32((uint8_t)(__float_as_uint(sv) >> (8 * (c >> 1)))) * gsc, 0.0f));
                     else wp = __builtin_bit_cast(u32x4, decode8<FMT>(w[i][c], 0u, sv, -8.0f * sv));
 #pragma unroll
                     for (int e = 0; e < 4; ++e) dot2_bf16(a[i], wp[e], xv[c][e]);
@@ -1337,10 +1349,14 @@ static GemvPlan gemv_plan(const xq_weight* w, double share = 1.0, bool even = fa
 
 bool skinny_gemv_supported(const xq_weight* w, int64_t M, const void* lora_A, const void* lora_B, int lora_dtype, int r) {
     if (!g_skinny_gemv || M != 1 || w->num_experts != 1 || w->layout != XQ_LAYOUT_FLAT) return false;
-    if (w->format == XQ_FMT_FP8 ? w->scale_dtype != XQ_SCALE_F32
-                                : w->format != XQ_FMT_INT4 || w->group < 32 || (w->group & (w->group - 1)) != 0 ||
-                                      (w->scale_dtype != XQ_SCALE_F32 && w->scale_dtype != XQ_SCALE_BF16))
+    if (w->format == XQ_FMT_FP8) {
+        if (w->scale_dtype != XQ_SCALE_F32) return false;
+    } else if (w->format == XQ_FMT_NVFP4) {
+        if (w->scale_dtype != XQ_SCALE_E4M3 || w->group != 16 || !w->global_scale) return false;
+    } else if (w->format != XQ_FMT_INT4 || w->group < 32 || (w->group & (w->group - 1)) != 0 ||
+               (w->scale_dtype != XQ_SCALE_F32 && w->scale_dtype != XQ_SCALE_BF16)) {
         return false;
+    }
     // (bf16 scales are read as the aligned words that hold them: the array must end on a word)
     if (w->format == XQ_FMT_INT4 && (w->rows * w->cols / w->group) % 2 != 0) return false;
     // int4 is decode-bound in either kernel; this one is ahead where the other's organisation fits badly -- few rows (q, kv)
@@ -1362,7 +1378,7 @@ static int gemv_args(const xq_weight* w, const GemvPlan& p, const bf16_t* x, con
                "xq_linear_fwd: internal error: dot-product launch out of range");
     GemvArgs& g = *out;
     g.x = x; g.N = (int)w->rows; g.K = (int)w->cols;
-    g.packed = (const uint8_t*)w->packed; g.scales = (const uint8_t*)w->scales;
+    g.packed = (const uint8_t*)w->packed; g.scales = (const uint8_t*)w->scales; g.global_scale = w->global_scale;
     g.gshift = 0;
     for (int v = w->group; v > 1; v >>= 1) ++g.gshift;
     g.scale_dtype = w->scale_dtype;
@@ -1387,6 +1403,9 @@ int launch_skinny_gemv(const xq_weight* w, const bf16_t* x, const void* lora_A, 
     if (w->format == XQ_FMT_FP8) {
         if (swiglu) skinny_gemv_kernel<XQ_FMT_FP8, kGemvRows, true><<<grid, threads, 0, stream>>>(g);
         else skinny_gemv_kernel<XQ_FMT_FP8, kGemvRows, false><<<grid, threads, 0, stream>>>(g);
+    } else if (w->format == XQ_FMT_NVFP4) {
+        if (swiglu) skinny_gemv_kernel<XQ_FMT_NVFP4, kGemvRows, true><<<grid, threads, 0, stream>>>(g);
+        else skinny_gemv_kernel<XQ_FMT_NVFP4, kGemvRows, false><<<grid, threads, 0, stream>>>(g);
     } else {
         if (swiglu) skinny_gemv_kernel<XQ_FMT_INT4, kGemvRows, true><<<grid, threads, 0, stream>>>(g);
         else skinny_gemv_kernel<XQ_FMT_INT4, kGemvRows, false><<<grid, threads, 0, stream>>>(g);
@@ -1422,6 +1441,8 @@ static int launch_skinny_gemv_multi(const SkinnyRowsJob* jobs, int n_jobs, const
     const unsigned grid = (unsigned)(pat + sat);
     if (jobs[0].w->format == XQ_FMT_FP8)
         skinny_gemv_multi_kernel<XQ_FMT_FP8, kGemvRows><<<grid, threads, 0, stream>>>(pf[1], pf[2], pf[3], pf[4], sf[1], sf[2], sf[3], sf[4], b);
+    else if (jobs[0].w->format == XQ_FMT_NVFP4)
+        skinny_gemv_multi_kernel<XQ_FMT_NVFP4, kGemvRows><<<grid, threads, 0, stream>>>(pf[1], pf[2], pf[3], pf[4], sf[1], sf[2], sf[3], sf[4], b);
     else
         skinny_gemv_multi_kernel<XQ_FMT_INT4, kGemvRows><<<grid, threads, 0, stream>>>(pf[1], pf[2], pf[3], pf[4], sf[1], sf[2], sf[3], sf[4], b);
     return XQ_OK;
