@@ -139,7 +139,7 @@ int xq_get_mlp_gate_up_fused(void);   /* the current default: 0 or 1 */
  * summation orders).  A process-wide switch for tests and A/B measurements (XQ_SKINNY_ROWS=0 in the environment sets
  * it at load time); no counterpart in the reference. */
 int xq_set_skinny_one_launch(int enabled);
-/* One token (M = 1) against a FLAT block-fp8, nvfp4 (e4m3 block scales) or int4 weight whose rows are whole KBs
+/* One token (M = 1) against a FLAT block-fp8, nvfp4 (e4m3 block scales), nf4 (groups of 64) or int4 weight whose rows are whole KBs
  * (in_features % 1024 == 0, the 4-bit formats: % 2048; at most 15 KB per row; int4 only on shapes on which it is the
  * faster kernel -- at most 4096 rows, or rows of 8192 elements and more) runs a kernel of its own inside the one-launch
  * path: no matrix cores, waves that stream whole rows (block fp8: the rate of a plain read from HBM), same slots and same

@@ -1,4 +1,4 @@
-"""GPU: one activation row (M = 1; block fp8, int4, nvfp4) through the dot-product kernel -- whole weight rows streamed by waves, decoded to the
+"""GPU: one activation row (M = 1; block fp8, int4, nvfp4, nf4) through the dot-product kernel -- whole weight rows streamed by waves, decoded to the
 reference decoder's bf16 values and multiplied without matrix cores -- against the oracle and against the MFMA kernel on
 the same inputs (xq_set_skinny_gemv(0)).  Beyond arithmetic the cases aim at: blocks of one wave (rows of 1 KB), ragged
 last blocks, a weight with fewer blocks than parts of the low-rank intermediate (falls back), the slot shared with the
@@ -65,7 +65,10 @@ def _forward(m, x, r):
     ("nvfp4", 4096, 12288, 8, False),
     ("nvfp4", 1040, 2048, 16, True),          # one wave per set
     ("nvfp4", 2048, 6144, 0, True),           # three waves per set, two sets
-    ("nf4", 4096, 4096, 16, False),           # nf4 stays on the MFMA kernel whatever the switch says
+    ("nf4", 4096, 4096, 16, False),           # levels looked up in a per-wave table in LDS, fp32 scales per 64
+    ("nf4", 12288, 4096, 16, True),
+    ("nf4", 4096, 12288, 8, False),
+    ("nf4", 1040, 2048, 0, True),             # one wave per set
 ])
 def test_dot_product_kernel_vs_oracle_and_mfma_kernel(hip_device, kernels, fmt, N, K, r, has_bias):
     m, w_ref = make_dense_module(fmt, N, K, max(r, 1), 2 * max(r, 1), seed=N + K + r, device=hip_device, bias=has_bias)
@@ -84,7 +87,7 @@ def test_dot_product_kernel_vs_oracle_and_mfma_kernel(hip_device, kernels, fmt, 
         close(dot.cpu(), mfma.float().cpu(), 4e-3)
 
 
-@pytest.mark.parametrize("fmt", ["block_fp8", "int4", "nvfp4"])
+@pytest.mark.parametrize("fmt", ["block_fp8", "int4", "nvfp4", "nf4"])
 def test_one_workspace_alternating_between_the_kernels(hip_device, fmt):
     """M = 1 (dot-product kernel) and M = 8 (MFMA kernel) take turns on one workspace, hence one slot: each launch must
     see its own parts of the low-rank intermediate only.  The low-rank term dominates the output here, so that a stale or

@@ -931,7 +931,7 @@ int launch_skinny_rows(const xq_weight* w, const bf16_t* x, int64_t ldx, int64_t
     }
 }
 
-// ---------------------------------------------------------------- M = 1, block fp8, int4, nvfp4: dot products instead of MFMA tiles
+// ---------------------------------------------------------------- M = 1, every format: dot products instead of MFMA tiles
 // One token against a packed weight needs no matrix cores, and the organisation above -- 8 waves per CU, a load instruction
 // that takes 64 bytes of each of 16 rows -- is what keeps it from the rate of a plain read when the bytes come from HBM
 // (8 waves per CU pull at most ~6 TB/s however deep their queues; a linear read by 32 waves per CU reaches 6.9).  Here the
@@ -950,13 +950,13 @@ int launch_skinny_rows(const xq_weight* w, const bf16_t* x, int64_t ldx, int64_t
 // dependent load costs ~3 us, and a block that is late by that makes the launch late by that -- and the parts of z are
 // read once per block: ~500 readers of the same few lines, not thousands.  (A part's entry for rank j sits at pair j of the
 // part's 256; tags keep launches of the two kernels on one slot apart.)
-// int4 and nvfp4 take the same kernel with 32 weights per lane and load (rows of 2 KB per wave; nvfp4: the lane's two e4m3
-// block scales come as one word, the tensor's global scale is a scalar).  Their time is the decode's -- as many
-// instructions per weight as block fp8, twice as many per byte.  nvfp4 is ahead of the MFMA kernel on every shape
-// measured (-8 % on many short rows to -30 % on few); int4 is level with it on weights of many short rows (those stay
-// on that kernel) and ahead where that kernel's organisation fits badly (q, kv, down: -15 %).  nf4 stays on the MFMA
-// kernel.  Several forwards on one x (xq_linear_fwd_multi) and gate | up with the SwiGLU finish (xq_linear_fwd_swiglu)
-// take the same body: see skinny_gemv_multi_kernel and the GU form below.
+// The 4-bit formats take the same kernel with 32 weights per lane and load (rows of 2 KB per wave; nvfp4: the lane's two
+// e4m3 block scales come as one word, the tensor's global scale is a scalar; nf4: the 16 levels in a per-wave table in
+// LDS).  Their time is the decode's -- as many instructions per weight as block fp8, twice as many per byte.  nvfp4 and nf4
+// are ahead of the MFMA kernel on every shape measured (-8 % on many short rows to -30 % on few, nf4 -16 to -34 %); int4 is
+// level with it on weights of many short rows (those stay on that kernel) and ahead where that kernel's organisation
+// fits badly (q, kv, down: -15 %).  Several forwards on one x (xq_linear_fwd_multi) and gate | up with the SwiGLU finish
+// (xq_linear_fwd_swiglu) take the same body: see skinny_gemv_multi_kernel and the GU form below.
 constexpr int kGemvRows = 4;                        // rows per group: with the next group's, 8 loads of a lane in flight
 constexpr int kGemvSlots = 64 / kGemvRows;          // groups of rows per block at most (all its sets together)
 
@@ -1000,10 +1000,11 @@ struct GemvArgs {
 // rounded outputs (the arithmetic of the SwiGLU kernel, ops/fused_silu_and_mul.py:22-60) instead of the outputs themselves.
 template <int FMT, int RB, bool GU>
 __device__ __forceinline__ void skinny_gemv_body(const GemvArgs& g, const int blk, const int nb) {
-    constexpr bool F8 = FMT == XQ_FMT_FP8, NV = FMT == XQ_FMT_NVFP4;
+    constexpr bool F8 = FMT == XQ_FMT_FP8, NV = FMT == XQ_FMT_NVFP4, NF = FMT == XQ_FMT_NF4;
     constexpr int EPL = F8 ? 16 : 32;                 // weights of a row per lane (one 16-byte load)
     __shared__ float red[kGemvSlots][RB][16];         // [set * gmax + group of the set][row][wave of the set]
     __shared__ float zpart[16][17];                   // a block that forms a part of z: [k slice][rank]
+    __shared__ float nf4_tab[NF ? 16 : 1][16];        // nf4: the 16 levels, a copy per wave (16 banks: any mix of codes reads it at full rate)
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const bool lora = g.nsu > 0;
@@ -1068,6 +1069,8 @@ __device__ __forceinline__ void skinny_gemv_body(const GemvArgs& g, const int bl
     // (the two kinds of waves go separate ways from here, each with the block's barrier in its own path, so that neither
     // carries the other's registers)
     if (streamer) {
+        // (written and read by this wave only: LDS operations of a wave execute in order)
+        if (NF && lane < 16) nf4_tab[wave][lane] = kNf4Level[lane];
         const int v = bx * g.sets + st;
         const int row0 = v * g.rps;
         const int nrows = row0 < g.N ? (g.N - row0 < g.rps ? g.N - row0 : g.rps) : 0;
@@ -1088,6 +1091,8 @@ __device__ __forceinline__ void skinny_gemv_body(const GemvArgs& g, const int bl
                 w[i] = __builtin_nontemporal_load((const u32x4*)(g.packed + (int64_t)n * row_bytes + (ws * 64 + lane) * 16));
                 if (F8) {
                     sc[i] = ((const float*)g.scales)[(n >> 7) * sc_cols + (kbase >> 7)];
+                } else if (NF) {
+                    sc[i] = ((const float*)g.scales)[((int64_t)n * g.K + kbase) >> 6];
                 } else if (NV) {
                     // (the lane's two e4m3 scales, one per 16 weights, inside the aligned word that holds them)
                     const int64_t si = ((int64_t)n * g.K + kbase) >> 4;
@@ -1101,7 +1106,7 @@ __device__ __forceinline__ void skinny_gemv_body(const GemvArgs& g, const int bl
         // the scale of row i of a group from what `issue` fetched (int4 with bf16 scales: the half that the index names)
         // (nvfp4: the two scale bytes in the low half of the result's bits)
         auto scale_of = [&](float raw, int gi, int i) -> float {
-            if (F8 || (!NV && s32)) return raw;
+            if (F8 || NF || (!NV && s32)) return raw;
             const int n = weight_row(row0 + (gi * RB + i < nrows ? gi * RB + i : nrows - 1));
             const uint32_t u = __float_as_uint(raw);
             if (NV) return __uint_as_float(u >> (8 * (int)((((int64_t)n * g.K + kbase) >> 4) & 2)));
@@ -1124,6 +1129,7 @@ __device__ __forceinline__ void skinny_gemv_body(const GemvArgs& g, const int bl
                 for (int c = 0; c < EPL / 8; ++c) {
                     u32x4 wp;
                     if constexpr (F8) wp = __builtin_bit_cast(u32x4, decode8<FMT>(w[i][2 * c], w[i][2 * c + 1], sv, 0.0f));
+                    else if constexpr (NF) wp = __builtin_bit_cast(u32x4, decode8<FMT>(w[i][c], 0u, sv, 0.0f, nf4_tab[wave]));
                     else if constexpr (NV)
                         wp = __builtin_bit_cast(u32x4, decode8<FMT>(w[i][c], 0u, e4m3_to_f32((uint8_t)(__float_as_uint(sv) >> (8 * (c >> 1)))) * gsc, 0.0f));
                     else wp = __builtin_bit_cast(u32x4, decode8<FMT>(w[i][c], 0u, sv, -8.0f * sv));
@@ -1351,6 +1357,8 @@ bool skinny_gemv_supported(const xq_weight* w, int64_t M, const void* lora_A, co
     if (!g_skinny_gemv || M != 1 || w->num_experts != 1 || w->layout != XQ_LAYOUT_FLAT) return false;
     if (w->format == XQ_FMT_FP8) {
         if (w->scale_dtype != XQ_SCALE_F32) return false;
+    } else if (w->format == XQ_FMT_NF4) {
+        if (w->scale_dtype != XQ_SCALE_F32 || w->group != 64) return false;
     } else if (w->format == XQ_FMT_NVFP4) {
         if (w->scale_dtype != XQ_SCALE_E4M3 || w->group != 16 || !w->global_scale) return false;
     } else if (w->format != XQ_FMT_INT4 || w->group < 32 || (w->group & (w->group - 1)) != 0 ||
@@ -1403,6 +1411,9 @@ int launch_skinny_gemv(const xq_weight* w, const bf16_t* x, const void* lora_A, 
     if (w->format == XQ_FMT_FP8) {
         if (swiglu) skinny_gemv_kernel<XQ_FMT_FP8, kGemvRows, true><<<grid, threads, 0, stream>>>(g);
         else skinny_gemv_kernel<XQ_FMT_FP8, kGemvRows, false><<<grid, threads, 0, stream>>>(g);
+    } else if (w->format == XQ_FMT_NF4) {
+        if (swiglu) skinny_gemv_kernel<XQ_FMT_NF4, kGemvRows, true><<<grid, threads, 0, stream>>>(g);
+        else skinny_gemv_kernel<XQ_FMT_NF4, kGemvRows, false><<<grid, threads, 0, stream>>>(g);
     } else if (w->format == XQ_FMT_NVFP4) {
         if (swiglu) skinny_gemv_kernel<XQ_FMT_NVFP4, kGemvRows, true><<<grid, threads, 0, stream>>>(g);
         else skinny_gemv_kernel<XQ_FMT_NVFP4, kGemvRows, false><<<grid, threads, 0, stream>>>(g);
@@ -1441,6 +1452,8 @@ static int launch_skinny_gemv_multi(const SkinnyRowsJob* jobs, int n_jobs, const
     const unsigned grid = (unsigned)(pat + sat);
     if (jobs[0].w->format == XQ_FMT_FP8)
         skinny_gemv_multi_kernel<XQ_FMT_FP8, kGemvRows><<<grid, threads, 0, stream>>>(pf[1], pf[2], pf[3], pf[4], sf[1], sf[2], sf[3], sf[4], b);
+    else if (jobs[0].w->format == XQ_FMT_NF4)
+        skinny_gemv_multi_kernel<XQ_FMT_NF4, kGemvRows><<<grid, threads, 0, stream>>>(pf[1], pf[2], pf[3], pf[4], sf[1], sf[2], sf[3], sf[4], b);
     else if (jobs[0].w->format == XQ_FMT_NVFP4)
         skinny_gemv_multi_kernel<XQ_FMT_NVFP4, kGemvRows><<<grid, threads, 0, stream>>>(pf[1], pf[2], pf[3], pf[4], sf[1], sf[2], sf[3], sf[4], b);
     else
