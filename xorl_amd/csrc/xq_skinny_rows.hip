@@ -970,6 +970,16 @@ template <int CTRL>
 __device__ __forceinline__ float lane_perm(float v) {
     return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
 }
+// v + the same lanes of the other 16-lane rows: the rows swap in pairs (v_permlane16_swap), then the wave's halves
+// (v_permlane32_swap); every lane ends with the sum of the four lanes 16 apart, added as (r0 + r1) + (r2 + r3)
+__device__ __forceinline__ float sum_rows_of_16(float v) {
+    const uint32_t u = __float_as_uint(v);
+    auto p = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    const float h = __uint_as_float(p[0]) + __uint_as_float(p[1]);
+    const uint32_t hu = __float_as_uint(h);
+    auto q = __builtin_amdgcn_permlane32_swap(hu, hu, false, false);
+    return __uint_as_float(q[0]) + __uint_as_float(q[1]);
+}
 __device__ __forceinline__ float read_lane(float v, int l) { return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), l)); }
 
 struct GemvArgs {
@@ -1141,16 +1151,23 @@ __device__ __forceinline__ void skinny_gemv_body(const GemvArgs& g, const int bl
                 // the asm above: the wait is tied to the sum, so that whatever uses it comes behind)
                 asm volatile("s_nop 3" : "+v"(a[i]));
             }
-#pragma unroll
-            for (int i = 0; i < RB; ++i) {
-                float t = a[i];
-                t += lane_perm<0xB1>(t);              // neighbours in a quad
-                t += lane_perm<0x4E>(t);              // the quad's halves
-                t += lane_perm<0x141>(t);             // lanes 0-7 mirrored: the other quad of the 8
-                t += lane_perm<0x140>(t);             // lanes 0-15 mirrored: the other 8 of the 16
-                const float sum = (read_lane(t, 0) + read_lane(t, 16)) + (read_lane(t, 32) + read_lane(t, 48));
-                if (lane == 0) red[st * g.gmax + gi][i][ws] = sum;
-            }
+            // the four rows' sums over 16 lanes each, all four at once: neighbours swap the rows they do not keep (lane l keeps
+            // row l & 1 of rows 0 | 1 and of rows 2 | 3), the quad's halves likewise (lane l ends with row l & 3 summed over its
+            // quad), then the four quads of the 16 lanes by two rotations and the four 16-lane rows by two swaps -- a fixed order,
+            // 7 adds instead of 4 x 7
+            static_assert(RB == 4, "the lanes' row exchange is written for groups of four rows");
+            const bool o1 = (lane & 1) != 0, o2 = (lane & 2) != 0;
+            float k01 = o1 ? a[1] : a[0], s01 = o1 ? a[0] : a[1];
+            float k23 = o1 ? a[3] : a[2], s23 = o1 ? a[2] : a[3];
+            k01 += lane_perm<0xB1>(s01);
+            k23 += lane_perm<0xB1>(s23);
+            float kk = o2 ? k23 : k01;
+            const float ss = o2 ? k01 : k23;
+            kk += lane_perm<0x4E>(ss);
+            kk += lane_perm<0x124>(kk);               // the quad four lanes on (rotation within 16 lanes)
+            kk += lane_perm<0x128>(kk);               // and the pair of quads eight lanes on
+            kk = sum_rows_of_16(kk);
+            if (lane < 4) red[st * g.gmax + gi][lane][ws] = kk;
         };
         auto work = [&](const u32x4 (&w)[RB], const float (&sc)[RB], int gi) {
             if (gi * RB + RB <= nrows) work_rows(std::true_type{}, w, sc, gi);
