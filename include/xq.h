@@ -507,6 +507,25 @@ int xq_grouped_bwd(const xq_weight* gate, const xq_weight* up, const xq_weight* 
                    void* dx, int64_t ld_dx, void* d_routing, int rw_dtype, const xq_grouped_grads* grads,
                    void* workspace, int64_t workspace_bytes, void* stream);
 
+/* The same forward for a handful of tokens with nothing kept for a backward (decode, rollout: the reference runs
+ * _MoeExpertsLoRAFunction.forward, ops/moe/lora.py:525-713, under no_grad for these too, through the same grouped
+ * GEMMs).  Same arguments as xq_grouped_fwd without `saved`, same result up to the summation order inside a dot
+ * product (same rounding points: bf16 gate / up / h / down rows, bf16 low-rank intermediates and factors).  With few
+ * tokens an expert sees one or two rows and the time is the bytes of the touched experts: each touched expert's three
+ * matrices are streamed once, multiplied on the vector unit, in five launches on `stream`.
+ * xq_grouped_infer_supported() says whether a call fits: block-fp8 banks (fp32 scales) that make an MLP, hidden and
+ * intermediate sizes multiples of 256, at most 1024 experts, 1..512 routed copies (n_tokens * topk), topk <= 16,
+ * r in 1..64.  Other calls return XQ_ERR_ARG here: the caller takes xq_grouped_fwd for them.
+ * workspace: xq_grouped_infer_workspace_bytes() bytes, 256-byte aligned. */
+int xq_grouped_infer_supported(const xq_weight* gate, const xq_weight* up, const xq_weight* down, int64_t n_tokens,
+                               int32_t topk, int r);
+int64_t xq_grouped_infer_workspace_bytes(int64_t n_tokens, int32_t topk, int32_t num_experts, int64_t hidden,
+                                         int64_t intermediate, int r);
+int xq_grouped_fwd_infer(const xq_weight* gate, const xq_weight* up, const xq_weight* down, const xq_grouped_lora* lora,
+                         const void* hidden, int64_t ld_hidden, int64_t n_tokens, const void* routing_w, int rw_dtype,
+                         const int32_t* selected, int32_t topk, void* out, int64_t ld_out, void* workspace,
+                         int64_t workspace_bytes, void* stream);
+
 /* ---- the dense SwiGLU MLP in two calls ---------------------------------------
  * y = down(silu(gate(x)) * up(x)) over three QLoRA linears: the reference's Qwen3MLP.forward
  * (models/transformers/qwen3/modeling_qwen3.py:60-81) on QLoRALinear modules (qlora/modules/linear.py:369-385) with

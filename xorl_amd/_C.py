@@ -164,6 +164,11 @@ _SIGNATURES = {
     "xq_grouped_bwd": (_INT, [_W, _W, _W, ctypes.POINTER(XqGroupedLora), _P, _I64, _I64, _I32,
                               ctypes.POINTER(XqGroupedSaved), _P, _I64, _P, _INT, ctypes.POINTER(XqGroupedGrads), _P, _I64,
                               _P]),
+    "xq_grouped_infer_supported": (_INT, [_W, _W, _W, _I64, _I32, _INT]),
+    "xq_grouped_infer_workspace_bytes": (_I64, [_I64, _I32, _I32, _I64, _I64, _INT]),
+    # gate, up, down, lora, hidden, ld_hidden, n_tokens, routing_w, rw_dtype, selected, topk, out, ld_out, ws, ws_bytes, stream
+    "xq_grouped_fwd_infer": (_INT, [_W, _W, _W, ctypes.POINTER(XqGroupedLora), _P, _I64, _I64, _P, _INT, _P, _I32, _P, _I64,
+                                    _P, _I64, _P]),
     "xq_mlp_workspace_bytes": (_I64, [_I64, _I64, _I64, _INT, _INT]),
     "xq_mlp_infer_workspace_bytes": (_I64, [_I64, _I64, _I64, _INT]),
     # gate, up, down, lora, x, ldx, M, y, ldy, ws, ws_bytes, stream

@@ -1,0 +1,664 @@
+// xq_grouped_fwd_infer: the routed SwiGLU expert MLP with LoRA on block-fp8 expert banks for a handful of tokens
+// (decode / rollout), nothing kept for a backward.  The program is the forward of the reference's
+// _MoeExpertsLoRAFunction (ops/moe/lora.py:525-713) with the rounding points of xq_grouped_fwd; what differs is the
+// organisation.  With few tokens an expert sees one or two rows, so the time is the touched experts' bytes: every
+// touched expert's three matrices are streamed once from HBM by blocks that each own 256 output columns and a range
+// of the contraction dimension, multiply on the vector unit (v_dot2c_f32_bf16 on bf16 pairs: a bank matrix is
+// [K, N] with N contiguous, so a lane keeps 16 output columns and walks down K -- no transposition, no matrix cores,
+// which a one-row operand would leave idle) and store fp32 partial sums; two small kernels between and after the
+// two streaming launches add the partial sums and the low-rank terms, apply SwiGLU and the routing weight and sum a
+// token's top-k copies.  Five launches (four for one token, which needs no routing launch), all sums in a fixed order (deterministic), nothing zeroed, no atomics on
+// memory.
+//
+//   decode_route_kernel   : the touched experts' rows in units of 2 or 4 (stable order of the routed copies) -- one block
+//   decode_stream_kernel  : gate | up partial sums [bank][K slice][row][I] + x . A partial sums (blocks of their own)
+//   decode_mid_kernel     : h = bf16(bf16(bf16(silu(g)) u) w), g / u = bf16(sum of slices + su . B), su = bf16(s x . A)
+//   decode_stream_kernel  : down partial sums [K slice][row][H] + h . A_d partial sums
+//   decode_final_kernel   : out[t] = bf16(sum over the token's copies of bf16(sum of slices + su_d . B_d))
+#include "xq_lora.h"
+
+namespace xq {
+namespace {
+
+constexpr int kDecMaxPairs = 512;       // routed copies (tokens x top-k) per call
+constexpr int kDecMaxExperts = 1024;
+constexpr int kDecMaxTopk = 16;
+constexpr int kDecTile = 256;           // output columns of a block
+constexpr int kDecChunk = 128;          // contraction rows per step of a block: one row of scale blocks
+constexpr int kDecMaxChunks = 16;       // chunks per K slice at most (the slice's x rows are staged in LDS)
+
+inline int64_t al256(int64_t b) { return (b + 255) & ~(int64_t)255; }
+inline int r_pad_of(int r) { return ((r + 15) / 16) * 16; }
+
+// routing lists in device memory: head[0] units, head[1] rows; a unit is up to MR consecutive rows of one expert
+// (units in ascending expert order): unit[4 u] = {expert, first row, row count, 0} and unit_token[4 u + m] the token of
+// its row m; per row row_info[2 row] = {the routed copy it is (token * topk + slot) or -1 past the last row, its expert}; per copy
+// pair_info[2 copy] = {its row or -1, its expert}.  What a block needs first sits behind one index, so that its loads
+// go out together instead of one after the other's result.
+// With one row per unit (direct: the one-token call) there is nothing to sort: a unit is a routed copy, its row the
+// copy's number, and the kernels read the expert ids where the caller has them -- no routing launch.
+struct DecLists {
+    int32_t* base;
+    int32_t R;
+    const int32_t* selected;      // direct: [R] expert ids (NULL otherwise)
+    int32_t E, topk;
+    __host__ __device__ int32_t* head() const { return base; }
+    __host__ __device__ int32_t* unit() const { return base + 4; }
+    __host__ __device__ int32_t* unit_token() const { return base + 4 + 4 * R; }
+    __host__ __device__ int32_t* row_info() const { return base + 4 + 8 * R; }
+    __host__ __device__ int32_t* pair_info() const { return base + 4 + 10 * R; }
+    static int64_t bytes(int64_t R) { return (4 + 12 * R) * 4; }
+};
+
+__global__ void __launch_bounds__(512) decode_route_kernel(const int32_t* selected, int R, int E, int lg, int topk, int units_max, DecLists L) {
+    const int MR = 1 << lg;                          // rows per unit: 2 or 4
+    __shared__ __attribute__((aligned(16))) int32_t s_sel[kDecMaxPairs];
+    __shared__ __attribute__((aligned(16))) int32_t s_cnt[kDecMaxExperts], s_begin[kDecMaxExperts], s_unit[kDecMaxExperts];
+    const int t = threadIdx.x;
+    for (int e = t; e < kDecMaxExperts; e += 512) s_cnt[e] = 0;
+    int mine = -1;
+    if (t < R) {
+        const int v = selected[t];
+        mine = v >= 0 && v < E ? v : -1;             // ids outside [0, E) drop their copy
+    }
+    s_sel[t] = mine;
+    __syncthreads();
+    int rank = 0;                                    // earlier copies of the same expert: the stable order
+    if (mine >= 0) {
+        int p = 0;
+        for (; p + 4 <= t; p += 4) {                 // four at a time: one LDS read
+            const int4 v = *(const int4*)&s_sel[p];
+            rank += (v.x == mine ? 1 : 0) + (v.y == mine ? 1 : 0) + (v.z == mine ? 1 : 0) + (v.w == mine ? 1 : 0);
+        }
+        for (; p < t; ++p) rank += s_sel[p] == mine ? 1 : 0;
+        atomicAdd(&s_cnt[mine], 1);
+    }
+    __syncthreads();
+    for (int e = t; e < E; e += 512) {
+        int b = 0, idx = 0, e2 = 0;
+        for (; e2 + 4 <= e; e2 += 4) {
+            const int4 c = *(const int4*)&s_cnt[e2];
+            b += c.x + c.y + c.z + c.w;
+            idx += ((c.x + MR - 1) >> lg) + ((c.y + MR - 1) >> lg) + ((c.z + MR - 1) >> lg) + ((c.w + MR - 1) >> lg);
+        }
+        for (; e2 < e; ++e2) {
+            const int c = s_cnt[e2];
+            b += c;
+            idx += (c + MR - 1) >> lg;
+        }
+        s_begin[e] = b;
+        s_unit[e] = idx;
+        const int c = s_cnt[e];
+        for (int q = 0; q * MR < c; ++q) {
+            int32_t* u = L.unit() + 4 * (idx + q);
+            u[0] = e;
+            u[1] = b + q * MR;
+            u[2] = c - q * MR < MR ? c - q * MR : MR;
+            u[3] = 0;
+        }
+        if (e == E - 1) {
+            s_sel[0] = idx + ((c + MR - 1) >> lg);   // units, rows (s_sel has been read: the barrier above)
+            s_sel[1] = b + c;
+        }
+    }
+    __syncthreads();
+    // the grid is laid out for units_max units and R rows: the others say so themselves (no rows / no copy)
+    for (int u = s_sel[0] + t; u < units_max; u += 512) *(int4*)(L.unit() + 4 * u) = int4{0, 0, 0, 0};
+    for (int rr = s_sel[1] + t; rr < R; rr += 512) L.row_info()[2 * rr] = -1;
+
+    if (t < R) {
+        if (mine >= 0) {
+            const int rr = s_begin[mine] + rank;
+            L.row_info()[2 * rr] = t;
+            L.row_info()[2 * rr + 1] = mine;
+            L.pair_info()[2 * t] = rr;
+            L.pair_info()[2 * t + 1] = mine;
+            const int u = s_unit[mine] + (rank >> lg), m = rank & (MR - 1);
+            L.unit_token()[4 * u + m] = t / topk;
+            // rows past a unit's own are staged as copies of its first
+            if (m == 0)
+                for (int q = 1; q < 4; ++q)
+                    if (rank + q >= s_cnt[mine] || q >= MR) L.unit_token()[4 * u + q] = t / topk;
+        } else {
+            L.pair_info()[2 * t] = -1;
+            L.pair_info()[2 * t + 1] = 0;
+        }
+    }
+}
+
+// acc += w.lo * x.lo + w.hi * x.hi on bf16 pairs (exact products, one fp32 sum); written as the instruction (the
+// compiler's builtin for it has come out with wrong operand registers when fed with elements of vectors)
+__device__ __forceinline__ void dec_dot2(float& acc, uint32_t w, uint32_t x) {
+    asm("v_dot2c_f32_bf16 %0, %1, %2" : "+v"(acc) : "v"(w), "v"(x));
+}
+
+// sum over s < ns of p[s * stride] in ascending order, the loads sixteen at a time (slices past the end are read again
+// from the last one and left out): a loop of dependent round trips would cost a memory latency per slice
+__device__ __forceinline__ float sum_slices(const float* p, int64_t stride, int ns) {
+    float v = 0.0f;
+    for (int s0 = 0; s0 < ns; s0 += 16) {
+        float t[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) t[u] = p[(int64_t)(s0 + u < ns ? s0 + u : ns - 1) * stride];
+#pragma unroll
+        for (int u = 0; u < 16; ++u)
+            if (s0 + u < ns) v += t[u];
+    }
+    return v;
+}
+// sixteen ranks of a column of a B factor as the bf16 values the training forward multiplies with (ranks past r are
+// read again from the last one; the sum leaves them out)
+// (the storage type is tested once, not per element: a branch around every load would make each wait for the one before)
+__device__ __forceinline__ void load_b16(float (&b)[16], const void* B, int64_t b0, int64_t ld, int j0, int r, bool f32) {
+    if (f32) {
+        float raw[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) raw[u] = ((const float*)B)[b0 + (int64_t)(j0 + u < r ? j0 + u : r - 1) * ld];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) b[u] = round_bf16(raw[u]);
+    } else {
+        bf16_t raw[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) raw[u] = ((const bf16_t*)B)[b0 + (int64_t)(j0 + u < r ? j0 + u : r - 1) * ld];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) b[u] = bf16_to_f32(raw[u]);
+    }
+}
+__device__ __forceinline__ float fma_b16(float v, const float* su, const float (&b)[16], int j0, int r) {
+#pragma unroll
+    for (int u = 0; u < 16; ++u)
+        if (j0 + u < r) v += su[j0 + u] * b[u];
+    return v;
+}
+
+struct DecStream {
+    const uint8_t* packed[2];       // one bank (down) or two (gate, up): [E][K][N] e4m3 bytes
+    const float* scales[2];         // [E][K / 128][ceil(N / 128)]
+    int32_t n_banks, K, N, sn;
+    const bf16_t* x;                // the rows that are multiplied: token rows (by_token) or rows in expert order
+    int64_t ldx;
+    int32_t by_token, topk;
+    int32_t cps, n_slices, n_tiles; // chunks per K slice, slices, column tiles (blockIdx.x == n_tiles: the low-rank unit)
+    float* part;                    // [n_banks][n_slices][R][N]
+    const void* A[2];               // LoRA A [E | 1][K][r], fp32 or bf16
+    int32_t A_shared[2];
+    int32_t lora_f32, r, rp;
+    float* su_part;                 // [n_banks][n_slices][R][rp]
+    int32_t R;
+    DecLists L;
+};
+
+// One block: one unit (up to MR rows of one touched expert), one bank, one K slice, and either 256 output columns
+// of the bank matrix or the x . A part of the slice.  An expert with more than MR rows is several units: their blocks
+// read the same bytes at about the same time, which the caches serve.  Wave w owns rows 32 w .. +31 of every 128-row
+// chunk, lane (kq = lane / 16, c = lane % 16) the row pairs 8 s + 2 kq, + 1 (s = 0..3) and columns 16 c .. + 15: a
+// load instruction covers four rows' 256-byte segments, a chunk is 8 loads per lane, and the next chunk's 8 are in
+// flight while one is multiplied (the first chunk's are issued before the x rows are staged).  The two rows of a pair
+// are decoded to the reference's bf16 weights (e4m3 x block scale, rounded) and packed column by column, so that one
+// v_dot2c per output column and x row multiplies both with the x pair of those two k, which sits in LDS as it does in
+// memory.  (The register count is held down by the attribute: left alone the compiler spends every register a
+// 256-thread block may have on decoding ahead.)
+template <int MR>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MR == 1 ? 4 : MR == 2 ? 3 : 2, 8))) decode_stream_kernel(DecStream g) {
+    __shared__ __attribute__((aligned(16))) bf16_t xs[MR][kDecMaxChunks * kDecChunk];
+    __shared__ __attribute__((aligned(16))) float red[16 * kDecTile];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int tile = blockIdx.x, slice = blockIdx.y;
+    const int li = (int)blockIdx.z / g.n_banks, bank = (int)blockIdx.z % g.n_banks;
+    int4 unit;
+    if (g.L.selected) {
+        const int v = g.L.selected[li];
+        unit = int4{v, li, v >= 0 && v < g.L.E ? 1 : 0, 0};
+    } else {
+        unit = *(const int4*)(g.L.unit() + 4 * li);
+    }
+    const int e = __builtin_amdgcn_readfirstlane(unit.x);
+    const int row0 = __builtin_amdgcn_readfirstlane(unit.y), mc = __builtin_amdgcn_readfirstlane(unit.z);
+    if (mc == 0) return;
+    const int c_begin = slice * g.cps;
+    const int nch = min(g.cps, g.K / kDecChunk - c_begin);           // >= 1: the launcher leaves no slice empty
+    const int k0 = c_begin * kDecChunk, klen = nch * kDecChunk;
+    const int64_t out_row0 = ((int64_t)bank * g.n_slices + slice) * g.R + row0;
+    const bool lora_unit = tile == g.n_tiles;
+    const int kq = lane >> 4, c = lane & 15;
+    const int n0 = tile * kDecTile;
+    const uint8_t* wbase = g.packed[bank] + ((int64_t)e * g.K + k0 + wave * 32) * g.N + n0;
+    const uint32_t woff = (uint32_t)(2 * kq * g.N + c * 16);
+    const float* sbase = g.scales[bank] + ((int64_t)e * (g.K / kDecChunk) + c_begin) * g.sn + (n0 >> 7);
+    const uint32_t soff = (uint32_t)(c >> 3);
+
+    u32x4 wa[8], wb[8];
+    float sa, sb;
+    auto issue = [&](u32x4(&w)[8], float& sc, int ch) {
+        const uint8_t* p = wbase + (int64_t)ch * kDecChunk * g.N;
+        sc = (sbase + (int64_t)ch * g.sn)[soff];
+#pragma unroll
+        for (int st = 0; st < 4; ++st) {
+            w[2 * st] = __builtin_nontemporal_load((const u32x4*)(p + (int64_t)(8 * st) * g.N + woff));
+            w[2 * st + 1] = __builtin_nontemporal_load((const u32x4*)(p + (int64_t)(8 * st + 1) * g.N + woff));
+        }
+    };
+    if (!lora_unit) issue(wa, sa, 0);                                // block-uniform; nothing below waits for it by count
+
+    // the unit's x rows, this slice's columns
+    const int ppr = klen >> 3;                                       // 16-byte pieces per row
+    for (int p = tid; p < MR * ppr; p += 256) {
+        const int m = p / ppr, piece = p - m * ppr;
+        const int64_t xrow = !g.by_token ? row0 + (m < mc ? m : 0) : g.L.selected ? li / g.topk : g.L.unit_token()[4 * li + m];
+        *(u32x4*)(&xs[m][piece * 8]) = *(const u32x4*)(g.x + xrow * g.ldx + k0 + piece * 8);
+    }
+    __syncthreads();
+
+    if (lora_unit) {
+        // su part [m][j] = sum over the slice's k of x[m][k] * bf16(A[k][j]): thread (kk = tid / 16, j = tid % 16) takes
+        // k = kk, kk + 16, ...; the 16 sums of a rank meet in LDS in order
+        const int64_t a_base = ((int64_t)(g.A_shared[bank] ? 0 : e) * g.K + k0) * g.r;
+        for (int jc = 0; jc < g.rp; jc += 16) {
+            const int j = jc + (tid & 15), kk = tid >> 4;
+            const int jl = j < g.r ? j : 0;
+            float a_acc[MR];
+#pragma unroll
+            for (int m = 0; m < MR; ++m) a_acc[m] = 0.0f;
+            for (int k = kk; k < klen; k += 64) {                    // klen is a multiple of 128: four loads at a time
+                float a[4];
+                if (g.lora_f32) {                                    // tested once per batch, not per load
+                    float raw[4];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) raw[u] = ((const float*)g.A[bank])[a_base + (int64_t)(k + 16 * u) * g.r + jl];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) a[u] = round_bf16(raw[u]);
+                } else {
+                    bf16_t raw[4];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) raw[u] = ((const bf16_t*)g.A[bank])[a_base + (int64_t)(k + 16 * u) * g.r + jl];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) a[u] = bf16_to_f32(raw[u]);
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u)
+#pragma unroll
+                    for (int m = 0; m < MR; ++m) a_acc[m] += bf16_to_f32(xs[m][k + 16 * u]) * a[u];
+            }
+#pragma unroll
+            for (int m = 0; m < MR; ++m) red[(kk * MR + m) * 16 + (tid & 15)] = j < g.r ? a_acc[m] : 0.0f;
+            __syncthreads();
+            if (tid < MR * 16) {
+                const int m = tid >> 4, jj = tid & 15;
+                float v = 0.0f;
+                for (int q = 0; q < 16; ++q) v += red[(q * MR + m) * 16 + jj];
+                if (m < mc) g.su_part[(out_row0 + m) * g.rp + jc + jj] = v;
+            }
+            __syncthreads();
+        }
+        return;
+    }
+
+    float acc[MR][16];
+#pragma unroll
+    for (int m = 0; m < MR; ++m)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) acc[m][j] = 0.0f;
+    auto work = [&](const u32x4(&w)[8], float sc, int ch) {
+        const uint32_t* xw = (const uint32_t*)&xs[0][0] + ((ch * kDecChunk + wave * 32 + 2 * kq) >> 1);
+#pragma unroll
+        for (int st = 0; st < 4; ++st) {
+            uint32_t pk[16];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const f32x2 a01 = e4m3x2_to_f32(w[2 * st][q], false), a23 = e4m3x2_to_f32(w[2 * st][q], true);
+                const f32x2 b01 = e4m3x2_to_f32(w[2 * st + 1][q], false), b23 = e4m3x2_to_f32(w[2 * st + 1][q], true);
+                pk[4 * q + 0] = pack_bf16x2(a01[0] * sc, b01[0] * sc);
+                pk[4 * q + 1] = pack_bf16x2(a01[1] * sc, b01[1] * sc);
+                pk[4 * q + 2] = pack_bf16x2(a23[0] * sc, b23[0] * sc);
+                pk[4 * q + 3] = pack_bf16x2(a23[1] * sc, b23[1] * sc);
+            }
+#pragma unroll
+            for (int m = 0; m < MR; ++m) {                           // rows past the unit's own hold copies of its first: no branch here
+                const uint32_t xp = xw[m * (kDecMaxChunks * kDecChunk / 2) + 4 * st];
+#pragma unroll
+                for (int j = 0; j < 16; ++j) dec_dot2(acc[m][j], pk[j], xp);
+            }
+            __builtin_amdgcn_sched_barrier(0);                       // one step's decoded pairs live at a time
+        }
+        // A dot result must not be read by another kind of instruction for three wait states, and the compiler does not
+        // see the hazard of an instruction written in assembly: a register copy that it places at the end of a block (the
+        // sums are carried through branches and loops) would read the last step's sums too early.  Nothing crosses the
+        // two scheduling barriers.
+        asm volatile("s_nop 3");
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    // no load sits under a condition that its wait does not share: the waits then count exactly
+    int ch = 0;
+    while (ch + 2 < nch) {
+        issue(wb, sb, ch + 1);
+        work(wa, sa, ch);
+        issue(wa, sa, ch + 2);
+        work(wb, sb, ch + 1);
+        ch += 2;
+    }
+    if (nch - ch == 2) {
+        issue(wb, sb, ch + 1);
+        work(wa, sa, ch);
+        work(wb, sb, ch + 1);
+    } else {
+        work(wa, sa, ch);
+    }
+
+    // the 16 partial sums of a column (4 waves x 4 row groups of a lane's 16) meet in LDS, one x row at a time
+#pragma unroll
+    for (int m = 0; m < MR; ++m) {
+        if (m < mc) {                                                // uniform
+            if (m > 0) __syncthreads();
+            float* dst = red + (wave * 4 + kq) * kDecTile + c * 16;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) *(f32x4*)(dst + 4 * q) = f32x4{acc[m][4 * q], acc[m][4 * q + 1], acc[m][4 * q + 2], acc[m][4 * q + 3]};
+            __syncthreads();
+            float v = 0.0f;
+#pragma unroll
+            for (int q = 0; q < 16; ++q) v += red[q * kDecTile + tid];
+            g.part[(out_row0 + m) * g.N + n0 + tid] = v;
+        }
+    }
+}
+
+struct DecMid {
+    const float* part;          // [2][ns][R][I]
+    const float* su_part;       // [2][ns][R][rp]
+    int32_t ns, R, I, r, rp;
+    const void* B[2];           // LoRA B [E | 1][r][I]
+    int32_t B_shared[2];
+    int32_t lora_f32;
+    float scaling, limit;
+    const void* routing_w;      // [T * topk]
+    int32_t rw_f32;
+    bf16_t* h;                  // [R][I], rows in expert order
+    DecLists L;
+};
+
+// one row, 256 columns: gate and up from their slices and low-rank terms, SwiGLU, the routing weight.  Everything
+// that depends only on the row is requested before anything is waited for.
+__global__ void __launch_bounds__(256) decode_mid_kernel(DecMid g) {
+    __shared__ float su_s[2 * 64];
+    const int rr = blockIdx.x, tid = threadIdx.x;
+    int2 info;
+    if (g.L.selected) {
+        const int v = g.L.selected[rr];
+        info = int2{v >= 0 && v < g.L.E ? rr : -1, v};
+    } else {
+        info = *(const int2*)(g.L.row_info() + 2 * rr);
+    }
+    const int pair = info.x, e = info.y;
+    if (pair < 0) return;
+    const int col = blockIdx.y * 256 + tid;
+    const int64_t slice_stride = (int64_t)g.R * g.I;
+    float b[2][16], gu[2];
+    int64_t b0[2];
+#pragma unroll
+    for (int bank = 0; bank < 2; ++bank) {
+        b0[bank] = (int64_t)(g.B_shared[bank] ? 0 : e) * g.r * g.I + col;
+        load_b16(b[bank], g.B[bank], b0[bank], g.I, 0, g.r, g.lora_f32);
+    }
+    const float w = g.rw_f32 ? ((const float*)g.routing_w)[pair] : bf16_to_f32(((const bf16_t*)g.routing_w)[pair]);
+#pragma unroll
+    for (int bank = 0; bank < 2; ++bank) gu[bank] = sum_slices(g.part + ((int64_t)bank * g.ns * g.R + rr) * g.I + col, slice_stride, g.ns);
+    if (tid < 2 * g.rp) {
+        const int bank = tid / g.rp, j = tid - bank * g.rp;
+        su_s[bank * 64 + j] = round_bf16(g.scaling * sum_slices(g.su_part + ((int64_t)bank * g.ns * g.R + rr) * g.rp + j, (int64_t)g.R * g.rp, g.ns));
+    }
+    __syncthreads();
+#pragma unroll
+    for (int bank = 0; bank < 2; ++bank) {
+        float v = fma_b16(gu[bank], su_s + bank * 64, b[bank], 0, g.r);
+        for (int j0 = 16; j0 < g.r; j0 += 16) {
+            load_b16(b[bank], g.B[bank], b0[bank], g.I, j0, g.r, g.lora_f32);
+            v = fma_b16(v, su_s + bank * 64, b[bank], j0, g.r);
+        }
+        gu[bank] = round_bf16(v);
+    }
+    const float gv = swiglu_clamp(gu[0], g.limit);
+    const float a = round_bf16(gv * sigmoid_f32(gv));
+    g.h[(int64_t)rr * g.I + col] = to_bf16(round_bf16(a * gu[1]) * w);
+}
+
+struct DecFinal {
+    const float* part;          // [ns][R][H]
+    const float* su_part;       // [ns][R][rp]
+    int32_t ns, R, H, r, rp, topk;
+    const void* B;              // LoRA B of down [E | 1][r][H]
+    int32_t B_shared, lora_f32;
+    float scaling;
+    bf16_t* out;
+    int64_t ld_out;
+    DecLists L;
+};
+
+// one token, 256 columns: its copies' down projections (slices + low-rank term, rounded to bf16 each) summed in slot
+// order.  Four groups of 256 threads take the slots four at a time; the rounded rows meet in LDS.
+__global__ void __launch_bounds__(1024) decode_final_kernel(DecFinal g) {
+    __shared__ float su_s[kDecMaxTopk * 64];
+    __shared__ float d_s[kDecMaxTopk * 256];
+    constexpr int NS = kDecMaxTopk / 4;                              // slots of a group at most
+    const int t = blockIdx.x, tid = threadIdx.x;
+    const int grp = tid >> 8, cl = tid & 255, col = blockIdx.y * 256 + cl;
+    int rrs[NS], es[NS];
+#pragma unroll
+    for (int i = 0; i < NS; ++i) {
+        const int slot = grp + 4 * i;
+        int2 info = int2{-1, 0};
+        if (slot < g.topk) {
+            const int p = t * g.topk + slot;
+            if (g.L.selected) {
+                const int v = g.L.selected[p];
+                info = int2{v >= 0 && v < g.L.E ? p : -1, v};
+            } else {
+                info = *(const int2*)(g.L.pair_info() + 2 * p);
+            }
+        }
+        rrs[i] = info.x;
+        es[i] = info.y;
+    }
+    for (int q = tid; q < g.topk * g.rp; q += 1024) {
+        const int slot = q / g.rp, j = q - slot * g.rp;
+        const int p = t * g.topk + slot;
+        int rr;
+        if (g.L.selected) {
+            const int v = g.L.selected[p];
+            rr = v >= 0 && v < g.L.E ? p : -1;
+        } else {
+            rr = g.L.pair_info()[2 * p];
+        }
+        su_s[slot * 64 + j] = rr >= 0 ? round_bf16(g.scaling * sum_slices(g.su_part + (int64_t)rr * g.rp + j, (int64_t)g.R * g.rp, g.ns)) : 0.0f;
+    }
+    float v[NS], b[NS][16];
+    int64_t b0[NS];
+#pragma unroll
+    for (int i = 0; i < NS; ++i) {                                   // a group's threads share rrs[i]: uniform branches
+        b0[i] = (int64_t)(g.B_shared ? 0 : es[i]) * g.r * g.H + col;
+        v[i] = 0.0f;
+        if (rrs[i] >= 0) {
+            load_b16(b[i], g.B, b0[i], g.H, 0, g.r, g.lora_f32);
+            v[i] = sum_slices(g.part + (int64_t)rrs[i] * g.H + col, (int64_t)g.R * g.H, g.ns);
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < NS; ++i) {
+        const int slot = grp + 4 * i;
+        if (slot < g.topk) {
+            float d = 0.0f;
+            if (rrs[i] >= 0) {
+                d = fma_b16(v[i], su_s + slot * 64, b[i], 0, g.r);
+                for (int j0 = 16; j0 < g.r; j0 += 16) {
+                    load_b16(b[i], g.B, b0[i], g.H, j0, g.r, g.lora_f32);
+                    d = fma_b16(d, su_s + slot * 64, b[i], j0, g.r);
+                }
+                d = round_bf16(d);
+            }
+            d_s[slot * 256 + cl] = d;
+        }
+    }
+    __syncthreads();
+    if (grp == 0) {
+        float acc = 0.0f;
+        for (int slot = 0; slot < g.topk; ++slot) acc += d_s[slot * 256 + cl];     // dropped copies hold zeros
+        g.out[(int64_t)t * g.ld_out + col] = to_bf16(acc);
+    }
+}
+
+struct DecPlan {
+    int ns_gu, cps_gu, ns_d, cps_d, units;
+};
+
+// K slices: enough blocks to fill the chip when few experts are touched (the grid is laid out for min(R, E) experts;
+// blocks of experts that are not touched leave at once), slices of at most kDecMaxChunks chunks
+void slices_for(int chunks, int blocks_per_slice, int* ns, int* cps) {
+    int want = (int)xq_cdiv(1024, blocks_per_slice);
+    const int least = (int)xq_cdiv(chunks, kDecMaxChunks);
+    if (want < least) want = least;
+    if (want > chunks) want = chunks;
+    *cps = (int)xq_cdiv(chunks, want);
+    *ns = (int)xq_cdiv(chunks, *cps);
+}
+
+// units at most: every unit holds a row, and an expert's last unit alone may hold fewer than MR
+DecPlan plan_for(int64_t R, int E, int64_t H, int64_t I, int MR) {
+    DecPlan p;
+    const int64_t most = E + R / MR;
+    p.units = (int)(R < most ? R : most);
+    slices_for((int)(H / kDecChunk), p.units * 2 * (int)(I / kDecTile), &p.ns_gu, &p.cps_gu);
+    slices_for((int)(I / kDecChunk), p.units * (int)(H / kDecTile), &p.ns_d, &p.cps_d);
+    return p;
+}
+
+inline int rows_per_unit(int64_t n_tokens) { return n_tokens == 1 ? 1 : n_tokens <= 4 ? 2 : 4; }
+
+int64_t infer_workspace(int64_t R, int E, int64_t H, int64_t I, int rp, int MR) {
+    const DecPlan p = plan_for(R, E, H, I, MR);
+    return al256(DecLists::bytes(R)) + al256(2ll * p.ns_gu * R * I * 4) + al256(2ll * p.ns_gu * R * rp * 4) + al256(R * I * 2) +
+           al256((int64_t)p.ns_d * R * H * 4) + al256((int64_t)p.ns_d * R * rp * 4) + 256;
+}
+
+bool infer_supported(const xq_weight* gate, const xq_weight* up, const xq_weight* down, int64_t n_tokens, int32_t topk, int r) {
+    if (!gate || !up || !down) return false;
+    const xq_weight* w[3] = {gate, up, down};
+    for (int i = 0; i < 3; ++i)
+        if (w[i]->format != XQ_FMT_FP8 || w[i]->scale_dtype != XQ_SCALE_F32 || !xq_aligned(w[i]->packed, 16) || !w[i]->scales) return false;
+    const int64_t H = gate->rows, I = gate->cols;
+    if (up->rows != H || up->cols != I || down->rows != I || down->cols != H) return false;
+    if (H % kDecTile || I % kDecTile) return false;
+    const int E = gate->num_experts;
+    if (E < 1 || E > kDecMaxExperts || up->num_experts != E || down->num_experts != E) return false;
+    if (topk < 1 || topk > kDecMaxTopk || n_tokens < 1 || n_tokens * topk > kDecMaxPairs) return false;
+    return r >= 1 && r <= 64;
+}
+
+}  // namespace
+}  // namespace xq
+
+using namespace xq;
+
+extern "C" int xq_grouped_infer_supported(const xq_weight* gate, const xq_weight* up, const xq_weight* down, int64_t n_tokens,
+                                          int32_t topk, int r) {
+    return infer_supported(gate, up, down, n_tokens, topk, r) ? 1 : 0;
+}
+
+extern "C" int64_t xq_grouped_infer_workspace_bytes(int64_t n_tokens, int32_t topk, int32_t num_experts, int64_t hidden,
+                                                    int64_t intermediate, int r) {
+    if (n_tokens < 1 || topk < 1 || num_experts < 1 || r < 1 || hidden < kDecChunk || intermediate < kDecChunk) return 0;
+    return infer_workspace(n_tokens * topk, num_experts, hidden, intermediate, r_pad_of(r), rows_per_unit(n_tokens));
+}
+
+extern "C" int xq_grouped_fwd_infer(const xq_weight* gate, const xq_weight* up, const xq_weight* down, const xq_grouped_lora* lora,
+                                    const void* hidden, int64_t ld_hidden, int64_t n_tokens, const void* routing_w, int rw_dtype,
+                                    const int32_t* selected, int32_t topk, void* out, int64_t ld_out, void* workspace,
+                                    int64_t workspace_bytes, void* stream_) {
+    static const char* who = "xq_grouped_fwd_infer";
+    XQ_REQUIRE(gate && up && down && lora, "%s: NULL descriptor", who);
+    int rc;
+    if ((rc = xq_validate_weight(gate, who)) || (rc = xq_validate_weight(up, who)) || (rc = xq_validate_weight(down, who))) return rc;
+    XQ_REQUIRE(infer_supported(gate, up, down, n_tokens, topk, lora->r),
+               "%s: takes block-fp8 banks that make an MLP (hidden and intermediate sizes multiples of %d, at most %d experts), "
+               "1 to %d routed copies (tokens x top-k, top-k <= %d) and ranks 1..64; see xq_grouped_infer_supported()",
+               who, kDecTile, kDecMaxExperts, kDecMaxPairs, kDecMaxTopk);
+    XQ_REQUIRE(lora->dtype == XQ_DT_F32 || lora->dtype == XQ_DT_BF16, "%s: bad lora dtype", who);
+    const int E = gate->num_experts;
+    for (int p = 0; p < 3; ++p) {
+        XQ_REQUIRE(lora->A[p] && lora->B[p], "%s: LoRA factor %d is NULL", who, p);
+        XQ_REQUIRE((lora->A_experts[p] == 1 || lora->A_experts[p] == E) && (lora->B_experts[p] == 1 || lora->B_experts[p] == E),
+                   "%s: a LoRA factor holds 1 (shared) or %d matrices", who, E);
+    }
+    XQ_REQUIRE(rw_dtype == XQ_DT_F32 || rw_dtype == XQ_DT_BF16, "%s: routing weights are fp32 or bf16", who);
+    XQ_REQUIRE(hidden && routing_w && selected && out, "%s: NULL tensor", who);
+    const int64_t H = gate->rows, I = gate->cols, R = n_tokens * topk;
+    XQ_REQUIRE(xq_aligned(hidden, 16) && (n_tokens == 1 || ld_hidden % 8 == 0) && ld_hidden >= H && ld_out >= H,
+               "%s: rows of hidden must be 16-byte aligned; row strides at least the hidden size", who);
+    const int r = lora->r, rp = r_pad_of(r);
+    const int MR = rows_per_unit(n_tokens);
+    XQ_REQUIRE(workspace && xq_aligned(workspace, 256) && workspace_bytes >= infer_workspace(R, E, H, I, rp, MR),
+               "%s: workspace missing, misaligned or smaller than xq_grouped_infer_workspace_bytes()", who);
+    hipStream_t stream = (hipStream_t)stream_;
+    const DecPlan pl = plan_for(R, E, H, I, MR);
+    uint8_t* ws = (uint8_t*)workspace;
+    int64_t used = 0;
+    auto take = [&](int64_t bytes) { uint8_t* p = ws + used; used += al256(bytes); return p; };
+    DecLists L{(int32_t*)take(DecLists::bytes(R)), (int32_t)R, MR == 1 ? selected : nullptr, E, topk};
+    float* part_gu = (float*)take(2ll * pl.ns_gu * R * I * 4);
+    float* su_gu = (float*)take(2ll * pl.ns_gu * R * rp * 4);
+    bf16_t* h = (bf16_t*)take(R * I * 2);
+    float* part_d = (float*)take((int64_t)pl.ns_d * R * H * 4);
+    float* su_d = (float*)take((int64_t)pl.ns_d * R * rp * 4);
+
+    if (MR > 1) {
+        decode_route_kernel<<<dim3(1), 512, 0, stream>>>(selected, (int)R, E, MR == 2 ? 1 : 2, topk, pl.units, L);
+        XQ_CHECK_LAUNCH(who);
+    }
+
+    const int lora_f32 = lora->dtype == XQ_DT_F32;
+    DecStream s1{};
+    s1.packed[0] = (const uint8_t*)gate->packed; s1.packed[1] = (const uint8_t*)up->packed;
+    s1.scales[0] = (const float*)gate->scales; s1.scales[1] = (const float*)up->scales;
+    s1.n_banks = 2; s1.K = (int)H; s1.N = (int)I; s1.sn = (int)xq_cdiv(I, 128);
+    s1.x = (const bf16_t*)hidden; s1.ldx = ld_hidden; s1.by_token = 1; s1.topk = topk;
+    s1.cps = pl.cps_gu; s1.n_slices = pl.ns_gu; s1.n_tiles = (int)(I / kDecTile);
+    s1.part = part_gu;
+    s1.A[0] = lora->A[0]; s1.A[1] = lora->A[1];
+    s1.A_shared[0] = lora->A_experts[0] == 1 && E > 1; s1.A_shared[1] = lora->A_experts[1] == 1 && E > 1;
+    s1.lora_f32 = lora_f32; s1.r = r; s1.rp = rp; s1.su_part = su_gu; s1.R = (int)R; s1.L = L;
+    const dim3 g1((unsigned)(s1.n_tiles + 1), (unsigned)pl.ns_gu, (unsigned)(pl.units * 2));
+    if (MR == 1) decode_stream_kernel<1><<<g1, 256, 0, stream>>>(s1);
+    else if (MR == 2) decode_stream_kernel<2><<<g1, 256, 0, stream>>>(s1);
+    else decode_stream_kernel<4><<<g1, 256, 0, stream>>>(s1);
+    XQ_CHECK_LAUNCH(who);
+
+    DecMid md{};
+    md.part = part_gu; md.su_part = su_gu; md.ns = pl.ns_gu; md.R = (int)R; md.I = (int)I; md.r = r; md.rp = rp;
+    md.B[0] = lora->B[0]; md.B[1] = lora->B[1];
+    md.B_shared[0] = lora->B_experts[0] == 1 && E > 1; md.B_shared[1] = lora->B_experts[1] == 1 && E > 1;
+    md.lora_f32 = lora_f32; md.scaling = lora->scaling; md.limit = lora->swiglu_limit > 0.0f ? lora->swiglu_limit : 0.0f;
+    md.routing_w = routing_w; md.rw_f32 = rw_dtype == XQ_DT_F32; md.h = h; md.L = L;
+    decode_mid_kernel<<<dim3((unsigned)R, (unsigned)(I / 256)), 256, 0, stream>>>(md);
+    XQ_CHECK_LAUNCH(who);
+
+    DecStream s2{};
+    s2.packed[0] = (const uint8_t*)down->packed; s2.scales[0] = (const float*)down->scales;
+    s2.n_banks = 1; s2.K = (int)I; s2.N = (int)H; s2.sn = (int)xq_cdiv(H, 128);
+    s2.x = h; s2.ldx = I; s2.by_token = 0; s2.topk = topk;
+    s2.cps = pl.cps_d; s2.n_slices = pl.ns_d; s2.n_tiles = (int)(H / kDecTile);
+    s2.part = part_d;
+    s2.A[0] = lora->A[2]; s2.A_shared[0] = lora->A_experts[2] == 1 && E > 1;
+    s2.lora_f32 = lora_f32; s2.r = r; s2.rp = rp; s2.su_part = su_d; s2.R = (int)R; s2.L = L;
+    const dim3 g2((unsigned)(s2.n_tiles + 1), (unsigned)pl.ns_d, (unsigned)pl.units);
+    if (MR == 1) decode_stream_kernel<1><<<g2, 256, 0, stream>>>(s2);
+    else if (MR == 2) decode_stream_kernel<2><<<g2, 256, 0, stream>>>(s2);
+    else decode_stream_kernel<4><<<g2, 256, 0, stream>>>(s2);
+    XQ_CHECK_LAUNCH(who);
+
+    DecFinal fn{};
+    fn.part = part_d; fn.su_part = su_d; fn.ns = pl.ns_d; fn.R = (int)R; fn.H = (int)H; fn.r = r; fn.rp = rp; fn.topk = topk;
+    fn.B = lora->B[2]; fn.B_shared = lora->B_experts[2] == 1 && E > 1; fn.lora_f32 = lora_f32; fn.scaling = lora->scaling;
+    fn.out = (bf16_t*)out; fn.ld_out = ld_out; fn.L = L;
+    decode_final_kernel<<<dim3((unsigned)n_tokens, (unsigned)(H / 256)), 1024, 0, stream>>>(fn);
+    XQ_CHECK_LAUNCH(who);
+    return XQ_OK;
+}

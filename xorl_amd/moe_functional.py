@@ -349,6 +349,51 @@ class MoeExpertsQLoRAFunction(torch.autograd.Function):
         return (dx, drw, None, *gs, None, None, None, None, None, None)
 
 
+# Test switch: False sends forwards that need no gradient through xq_grouped_fwd as well.
+DECODE_PATH = True
+
+
+def _moe_infer(hidden: Tensor, routing_weights: Tensor, selected_experts: Tensor, factors, banks, num_experts: int,
+               scaling: float, swiglu_limit: float) -> Optional[Tensor]:
+    """xq_grouped_fwd_infer: the forward for a handful of tokens when nothing is differentiated (block-fp8 banks; the
+    touched experts' bytes streamed once).  None where the call does not fit it."""
+    qg, qu, qd = banks
+    H = qg.rows
+    if (hidden.dtype != torch.bfloat16 or not hidden.is_cuda or hidden.numel() == 0 or hidden.shape[-1] != H
+            or any(qw.num_experts != num_experts for qw in banks)):
+        return None
+    shape = hidden.shape
+    hidden2 = _as_2d(hidden.reshape(-1, H))
+    T, topk = hidden2.shape[0], selected_experts.shape[-1]
+    r = factors[0].shape[-1]
+    wg, wu, wd = qg.c(), qu.c(), qd.c()
+    L = _C.lib()
+    if not L.xq_grouped_infer_supported(ctypes.byref(wg), ctypes.byref(wu), ctypes.byref(wd), T, topk, r):
+        return None
+    if hidden2.data_ptr() % 16 or (T > 1 and hidden2.stride(0) % 8):
+        return None
+    _C.require_hip(hidden, routing_weights, selected_experts)
+    sel = selected_experts.reshape(T, topk).to(torch.int32).contiguous()
+    rw = routing_weights.reshape(T, topk)
+    if rw.dtype not in (torch.float32, torch.bfloat16):
+        rw = rw.float()
+    rw = rw.contiguous()
+    factors = tuple(f.detach().contiguous() for f in factors)
+    dev = hidden2.device
+    lora = _lora_struct(factors, r, float(scaling), swiglu_limit)
+    key = ("infer", T, topk, num_experts, H, qg.cols, r)
+    n = _WS.get(key)
+    if n is None:
+        n = _WS[key] = L.xq_grouped_infer_workspace_bytes(T, topk, num_experts, H, qg.cols, r)
+    ws = torch.empty(n, dtype=torch.uint8, device=dev)
+    out = torch.empty(T, H, dtype=torch.bfloat16, device=dev)
+    _C.check(L.xq_grouped_fwd_infer(ctypes.byref(wg), ctypes.byref(wu), ctypes.byref(wd), ctypes.byref(lora),
+                                    hidden2.data_ptr(), hidden2.stride(0) if T > 1 else H, T, rw.data_ptr(),
+                                    _C.XQ_DT_F32 if rw.dtype == torch.float32 else _C.XQ_DT_BF16, sel.data_ptr(), topk,
+                                    out.data_ptr(), H, ws.data_ptr(), ws.numel(), _s(dev)))
+    return out.reshape(shape)
+
+
 def moe_experts_qlora_forward(num_experts: int, routing_weights: Tensor, selected_experts: Tensor,
                               hidden_states: Tensor, gate_proj: QuantWeight, up_proj: QuantWeight,
                               down_proj: QuantWeight, gate_proj_lora_A: Tensor, gate_proj_lora_B: Tensor,
@@ -356,7 +401,17 @@ def moe_experts_qlora_forward(num_experts: int, routing_weights: Tensor, selecte
                               down_proj_lora_B: Tensor, scaling: float, swiglu_limit: float = 0.0) -> Tensor:
     """Entry with the argument order of the reference's MOE_EXPERT_BACKENDS_LORA callables
     (models/layers/moe/backend/__init__.py:421-445), except that the three base banks are
-    packed QuantWeight descriptors instead of dequantized [E, K, N] tensors."""
+    packed QuantWeight descriptors instead of dequantized [E, K, N] tensors.
+
+    A forward of a handful of tokens that nothing is differentiated through (decode, rollout) takes the
+    weight-streaming form xq_grouped_fwd_infer where the banks allow it."""
+    factors = (gate_proj_lora_A, gate_proj_lora_B, up_proj_lora_A, up_proj_lora_B, down_proj_lora_A, down_proj_lora_B)
+    if DECODE_PATH and not torch.compiler.is_compiling() and not (
+            torch.is_grad_enabled() and any(t.requires_grad for t in (hidden_states, routing_weights, *factors))):
+        out = _moe_infer(hidden_states, routing_weights, selected_experts, factors, (gate_proj, up_proj, down_proj),
+                         num_experts, scaling, float(swiglu_limit or 0.0))
+        if out is not None:
+            return out
     return MoeExpertsQLoRAFunction.apply(hidden_states, routing_weights, selected_experts, gate_proj_lora_A,
                                          gate_proj_lora_B, up_proj_lora_A, up_proj_lora_B, down_proj_lora_A,
                                          down_proj_lora_B, gate_proj, up_proj, down_proj, num_experts, scaling,
