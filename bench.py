@@ -628,6 +628,46 @@ def decode_case_table(dev, reps: int = 24, replays: int = 5):
     return rows
 
 
+def routed_decode_table(dev, sets: int = 16, replays: int = 5):
+    """The routed expert MLP of configs[3]'s banks for a handful of tokens with nothing to differentiate: the
+    weight-streaming form (xq_grouped_fwd_infer) beside the training forward (xq_grouped_fwd) on the same calls, `sets`
+    forwards with different routings per HIP graph so that the touched experts come from HBM."""
+    import xorl_amd.moe_functional as MF
+    from xorl_amd.qlora import BlockFP8QLoRAMoeExperts
+
+    E, Hd, I, topk, r = 128, 2048, 768, 8, 16
+    m = BlockFP8QLoRAMoeExperts(E, E, I, Hd, r=r, lora_alpha=2 * r, hybrid_shared=False).to(dev)
+    g = torch.Generator(device=dev).manual_seed(50)
+    w = lambda *shape: torch.randn(*shape, generator=g, device=dev) * 0.02
+    m.load_weights(w(E, Hd, I), w(E, Hd, I), w(E, I, Hd))
+    m = m.to(dev)
+    pool = torch.cuda.graph_pool_handle()
+    rows = []
+    for T in (1, 4, 16, 64):
+        calls = []
+        for i in range(sets):
+            rw, sel = zipf_routing(max(T, 8), E, topk, seed=3 + i, device=dev)
+            calls.append((torch.randn(T, Hd, generator=g, device=dev).to(torch.bfloat16), rw[:T].contiguous(), sel[:T].contiguous()))
+        touched = sum(int(torch.unique(c[2]).numel()) for c in calls) / sets
+        nbytes = touched * 3 * (Hd * I + (Hd // 128) * (I // 128) * 4)
+        us = {}
+        for name, on in (("streaming", True), ("training_forward", False)):
+            MF.DECODE_PATH = on
+
+            def run():
+                with torch.no_grad():
+                    for c in calls:
+                        m(*c)
+            us[name] = _graph_time_us(run, pool, sets, replays)
+        MF.DECODE_PATH = True
+        rows.append({"tokens": T, "experts_touched": touched, "bytes": nbytes, "us": us["streaming"],
+                     "GBps": nbytes / us["streaming"] / 1e3, "frac": nbytes / us["streaming"] / 1e3 / 8000.0,
+                     "us_training_forward": us["training_forward"]})
+    del m
+    torch.cuda.empty_cache()
+    return rows
+
+
 def secondary_measurements(args, dev):
     """The other two regimes of the path, measured in the same run as the headline line: configs[4] (skinny M, HBM
     roofline; per case and over the 32 BASELINE cases) and configs[3] (grouped experts, MFMA roofline)."""
@@ -656,6 +696,12 @@ def secondary_measurements(args, dev):
     out.append({"workload": c3["config"]["workload"], "value": c3["value"], "unit": "TFLOP/s", "ms_per_step": c3["ms_per_step"],
                 **c3["roofline"]})
     torch.cuda.empty_cache()
+    out.append({"workload": "not a BASELINE config: the routed expert MLP of configs[3]'s banks (E=128, hidden 2048, intermediate 768, "
+                            "top-8, r=16, block_fp8) for 1-64 tokens, forward only, nothing differentiated; per forward, 16 "
+                            "routings per HIP graph (touched experts from HBM); `bytes` = packed bytes of the touched experts",
+                "bound": "hbm", "peak": 8000.0, "unit": "GB/s",
+                "kernel": "decode_stream_kernel (+ decode_route / decode_mid / decode_final), xq_grouped_fwd_infer",
+                "cases": routed_decode_table(dev)})
     return out
 
 
