@@ -1,5 +1,5 @@
 """GPU parity: the routed expert MLP for a handful of tokens with nothing to differentiate (xq_grouped_fwd_infer: the
-touched experts' block-fp8 matrices streamed once, five launches) against the float64 per-expert oracle program and
+touched experts' block-fp8 or nvfp4 matrices streamed once, four or five launches) against the float64 per-expert oracle program and
 against the training forward (xq_grouped_fwd) on the same inputs."""
 
 import ctypes
@@ -49,6 +49,7 @@ def _both_paths(m, x, rw, sel, device):
     return y.cpu(), y_train.cpu()
 
 
+@pytest.mark.parametrize("fmt", ["block_fp8", "nvfp4"])
 @pytest.mark.parametrize("E,T,H,I,r,topk,hybrid,rw_dtype", [
     (8, 1, 256, 512, 16, 2, False, torch.bfloat16),        # one token: one row per expert, the one-row form
     (16, 1, 1024, 768, 16, 8, False, torch.float32),       # 8 experts of 16, K slices of one chunk
@@ -59,8 +60,8 @@ def _both_paths(m, x, rw, sel, device):
     (8, 1, 4096, 256, 16, 2, False, torch.float32),        # one-row form, K slices of two chunks
     (12, 4, 2048, 768, 16, 8, False, torch.bfloat16),      # two-row form, K slices of three chunks and a last one of one
 ])
-def test_decode_forward_vs_oracle(hip_device, E, T, H, I, r, topk, hybrid, rw_dtype):
-    m, banks = _make_experts("block_fp8", E, H, I, r, hybrid, seed=3 * E + T, device=hip_device)
+def test_decode_forward_vs_oracle(hip_device, fmt, E, T, H, I, r, topk, hybrid, rw_dtype):
+    m, banks = _make_experts(fmt, E, H, I, r, hybrid, seed=3 * E + T, device=hip_device)
     rw, sel = _zipf_routing(T, E, topk, seed=11)
     rw = rw.to(rw_dtype)
     x = gen((T, H), 1.0, 12, torch.bfloat16)
@@ -74,9 +75,10 @@ def test_decode_forward_vs_oracle(hip_device, E, T, H, I, r, topk, hybrid, rw_dt
     assert torch.equal(y, y2)
 
 
-def test_decode_forward_bf16_factors_and_swiglu_limit(hip_device):
+@pytest.mark.parametrize("fmt", ["block_fp8", "nvfp4"])
+def test_decode_forward_bf16_factors_and_swiglu_limit(hip_device, fmt):
     E, T, H, I, r, topk = 8, 4, 512, 256, 16, 2
-    m, banks = _make_experts("block_fp8", E, H, I, r, False, seed=91, device=hip_device)
+    m, banks = _make_experts(fmt, E, H, I, r, False, seed=91, device=hip_device)
     with torch.no_grad():
         for name in ("gate_proj", "up_proj", "down_proj"):
             for f in ("A", "B"):
@@ -128,7 +130,7 @@ def test_decode_form_declines_what_it_does_not_take(hip_device):
     import xorl_amd.moe_functional as MF
     from xorl_amd import _C
 
-    # hidden size not a multiple of 256; nvfp4 banks; more than 512 routed copies; a forward that is differentiated
+    # hidden size not a multiple of 256; NF4 banks; more than 512 routed copies; a forward that is differentiated
     m, _ = _make_experts("block_fp8", 4, 128, 256, 8, False, seed=60, device=hip_device)
     rw, sel = _zipf_routing(2, 4, 2, seed=61)
     x = gen((2, 128), 1.0, 62, torch.bfloat16).to(hip_device)
@@ -138,7 +140,7 @@ def test_decode_form_declines_what_it_does_not_take(hip_device):
     assert MF._moe_infer(*args(m, x, rw, sel)) is None
     wg, wu, wd = (m._bank(p).c() for p in ("gate", "up", "down"))
     assert _C.lib().xq_grouped_infer_supported(ctypes.byref(wg), ctypes.byref(wu), ctypes.byref(wd), 2, 2, 8) == 0
-    m4, _ = _make_experts("nvfp4", 4, 256, 256, 8, False, seed=63, device=hip_device)
+    m4, _ = _make_experts("nf4", 4, 256, 256, 8, False, seed=63, device=hip_device)
     x4 = gen((2, 256), 1.0, 64, torch.bfloat16).to(hip_device)
     assert MF._moe_infer(*args(m4, x4, rw, sel)) is None
     m8, _ = _make_experts("block_fp8", 4, 256, 256, 8, False, seed=65, device=hip_device)

@@ -1,4 +1,4 @@
-// xq_grouped_fwd_infer: the routed SwiGLU expert MLP with LoRA on block-fp8 expert banks for a handful of tokens
+// xq_grouped_fwd_infer: the routed SwiGLU expert MLP with LoRA on block-fp8 or nvfp4 expert banks for a handful of tokens
 // (decode / rollout), nothing kept for a backward.  The program is the forward of the reference's
 // _MoeExpertsLoRAFunction (ops/moe/lora.py:525-713) with the rounding points of xq_grouped_fwd; what differs is the
 // organisation.  With few tokens an expert sees one or two rows, so the time is the touched experts' bytes: every
@@ -172,8 +172,10 @@ __device__ __forceinline__ float fma_b16(float v, const float* su, const float (
 }
 
 struct DecStream {
-    const uint8_t* packed[2];       // one bank (down) or two (gate, up): [E][K][N] e4m3 bytes
-    const float* scales[2];         // [E][K / 128][ceil(N / 128)]
+    const uint8_t* packed[2];       // one bank (down) or two (gate, up): block fp8 [E][K][N] e4m3 bytes; nvfp4 [E][K / 2][N]
+                                    // bytes, rows 2 p (low nibble) and 2 p + 1 of a column in one byte
+    const void* scales[2];          // block fp8: fp32 [E][K / 128][ceil(N / 128)]; nvfp4: e4m3 [E][K / 16][N]
+    const float* gs[2];             // nvfp4: the experts' global scales
     int32_t n_banks, K, N, sn;
     const bf16_t* x;                // the rows that are multiplied: token rows (by_token) or rows in expert order
     int64_t ldx;
@@ -198,8 +200,13 @@ struct DecStream {
 // v_dot2c per output column and x row multiplies both with the x pair of those two k, which sits in LDS as it does in
 // memory.  (The register count is held down by the attribute: left alone the compiler spends every register a
 // 256-thread block may have on decoding ahead.)
-template <int MR>
+// nvfp4 banks (FMT = XQ_FMT_NVFP4) hold the two rows of a pair in one byte, which is the operand layout as it is: a
+// lane's 16-byte load is its 16 columns of one row pair, a chunk 4 weight loads and 2 loads of e4m3 block scales (16
+// columns x the wave's two 16-row groups) per lane; a byte becomes its two e2m1 values by one conversion, each times
+// fl(block scale x global scale), rounded to bf16 -- the reference decoder's values.
+template <int MR, int FMT>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MR == 1 ? 4 : MR == 2 ? 3 : 2, 8))) decode_stream_kernel(DecStream g) {
+    constexpr bool NV = FMT == XQ_FMT_NVFP4;
     __shared__ __attribute__((aligned(16))) bf16_t xs[MR][kDecMaxChunks * kDecChunk];
     __shared__ __attribute__((aligned(16))) float red[16 * kDecTile];
     const int tid = threadIdx.x, lane = tid & 63;
@@ -223,20 +230,35 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MR == 
     const bool lora_unit = tile == g.n_tiles;
     const int kq = lane >> 4, c = lane & 15;
     const int n0 = tile * kDecTile;
-    const uint8_t* wbase = g.packed[bank] + ((int64_t)e * g.K + k0 + wave * 32) * g.N + n0;
-    const uint32_t woff = (uint32_t)(2 * kq * g.N + c * 16);
-    const float* sbase = g.scales[bank] + ((int64_t)e * (g.K / kDecChunk) + c_begin) * g.sn + (n0 >> 7);
-    const uint32_t soff = (uint32_t)(c >> 3);
+    const uint8_t* wbase = NV ? g.packed[bank] + ((int64_t)e * (g.K >> 1) + ((k0 + wave * 32) >> 1)) * g.N + n0
+                              : g.packed[bank] + ((int64_t)e * g.K + k0 + wave * 32) * g.N + n0;
+    const uint32_t woff = (uint32_t)((NV ? kq : 2 * kq) * g.N + c * 16);
+    // block fp8: the lane's block scale of a chunk; nvfp4: the 16 columns' e4m3 scales of the wave's two 16-row groups
+    const uint8_t* sbase = NV ? (const uint8_t*)g.scales[bank] + ((int64_t)e * (g.K >> 4) + c_begin * 8 + wave * 2) * g.N + n0
+                              : (const uint8_t*)((const float*)g.scales[bank] + ((int64_t)e * (g.K / kDecChunk) + c_begin) * g.sn + (n0 >> 7));
+    const uint32_t soff = (uint32_t)(NV ? c * 16 : (c >> 3) * 4);
+    const float gsc = NV ? g.gs[bank][e] : 1.0f;
 
+    // a chunk's loads: block fp8 w[0..7] the eight rows and sc the block scale; nvfp4 w[0..3] the four row pairs, w[4..5]
+    // the scale bytes
     u32x4 wa[8], wb[8];
     float sa, sb;
     auto issue = [&](u32x4(&w)[8], float& sc, int ch) {
-        const uint8_t* p = wbase + (int64_t)ch * kDecChunk * g.N;
-        sc = (sbase + (int64_t)ch * g.sn)[soff];
+        if (NV) {
+            const uint8_t* p = wbase + (int64_t)ch * (kDecChunk / 2) * g.N;
+            const uint8_t* sp = sbase + (int64_t)ch * 8 * g.N;
+            w[4] = *(const u32x4*)(sp + soff);
+            w[5] = *(const u32x4*)(sp + g.N + soff);
 #pragma unroll
-        for (int st = 0; st < 4; ++st) {
-            w[2 * st] = __builtin_nontemporal_load((const u32x4*)(p + (int64_t)(8 * st) * g.N + woff));
-            w[2 * st + 1] = __builtin_nontemporal_load((const u32x4*)(p + (int64_t)(8 * st + 1) * g.N + woff));
+            for (int st = 0; st < 4; ++st) w[st] = __builtin_nontemporal_load((const u32x4*)(p + (int64_t)(4 * st) * g.N + woff));
+        } else {
+            const uint8_t* p = wbase + (int64_t)ch * kDecChunk * g.N;
+            sc = *(const float*)(sbase + (int64_t)ch * g.sn * 4 + soff);
+#pragma unroll
+            for (int st = 0; st < 4; ++st) {
+                w[2 * st] = __builtin_nontemporal_load((const u32x4*)(p + (int64_t)(8 * st) * g.N + woff));
+                w[2 * st + 1] = __builtin_nontemporal_load((const u32x4*)(p + (int64_t)(8 * st + 1) * g.N + woff));
+            }
         }
     };
     if (!lora_unit) issue(wa, sa, 0);                                // block-uniform; nothing below waits for it by count
@@ -301,17 +323,42 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MR == 
         for (int j = 0; j < 16; ++j) acc[m][j] = 0.0f;
     auto work = [&](const u32x4(&w)[8], float sc, int ch) {
         const uint32_t* xw = (const uint32_t*)&xs[0][0] + ((ch * kDecChunk + wave * 32 + 2 * kq) >> 1);
+        float scl[16];                                               // nvfp4: the 16 columns' scales of the current 16-row group
 #pragma unroll
         for (int st = 0; st < 4; ++st) {
             uint32_t pk[16];
+            if (NV) {
+                if ((st & 1) == 0) {
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const f32x2 a01 = e4m3x2_to_f32(w[2 * st][q], false), a23 = e4m3x2_to_f32(w[2 * st][q], true);
-                const f32x2 b01 = e4m3x2_to_f32(w[2 * st + 1][q], false), b23 = e4m3x2_to_f32(w[2 * st + 1][q], true);
-                pk[4 * q + 0] = pack_bf16x2(a01[0] * sc, b01[0] * sc);
-                pk[4 * q + 1] = pack_bf16x2(a01[1] * sc, b01[1] * sc);
-                pk[4 * q + 2] = pack_bf16x2(a23[0] * sc, b23[0] * sc);
-                pk[4 * q + 3] = pack_bf16x2(a23[1] * sc, b23[1] * sc);
+                    for (int q = 0; q < 4; ++q) {
+                        const f32x2 s01 = e4m3x2_to_f32(w[4 + (st >> 1)][q], false), s23 = e4m3x2_to_f32(w[4 + (st >> 1)][q], true);
+                        scl[4 * q + 0] = s01[0] * gsc;
+                        scl[4 * q + 1] = s01[1] * gsc;
+                        scl[4 * q + 2] = s23[0] * gsc;
+                        scl[4 * q + 3] = s23[1] * gsc;
+                    }
+                }
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const f32x2 v0 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w[st][q], 1.0f, 0);
+                    const f32x2 v1 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w[st][q], 1.0f, 1);
+                    const f32x2 v2 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w[st][q], 1.0f, 2);
+                    const f32x2 v3 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w[st][q], 1.0f, 3);
+                    pk[4 * q + 0] = pack_bf16x2(v0[0] * scl[4 * q + 0], v0[1] * scl[4 * q + 0]);
+                    pk[4 * q + 1] = pack_bf16x2(v1[0] * scl[4 * q + 1], v1[1] * scl[4 * q + 1]);
+                    pk[4 * q + 2] = pack_bf16x2(v2[0] * scl[4 * q + 2], v2[1] * scl[4 * q + 2]);
+                    pk[4 * q + 3] = pack_bf16x2(v3[0] * scl[4 * q + 3], v3[1] * scl[4 * q + 3]);
+                }
+            } else {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const f32x2 a01 = e4m3x2_to_f32(w[2 * st][q], false), a23 = e4m3x2_to_f32(w[2 * st][q], true);
+                    const f32x2 b01 = e4m3x2_to_f32(w[2 * st + 1][q], false), b23 = e4m3x2_to_f32(w[2 * st + 1][q], true);
+                    pk[4 * q + 0] = pack_bf16x2(a01[0] * sc, b01[0] * sc);
+                    pk[4 * q + 1] = pack_bf16x2(a01[1] * sc, b01[1] * sc);
+                    pk[4 * q + 2] = pack_bf16x2(a23[0] * sc, b23[0] * sc);
+                    pk[4 * q + 3] = pack_bf16x2(a23[1] * sc, b23[1] * sc);
+                }
             }
 #pragma unroll
             for (int m = 0; m < MR; ++m) {                           // rows past the unit's own hold copies of its first: no branch here
@@ -506,6 +553,17 @@ __global__ void __launch_bounds__(1024) decode_final_kernel(DecFinal g) {
     }
 }
 
+template <int FMT>
+void launch_stream_fmt(int MR, dim3 grid, const DecStream& a, hipStream_t stream) {
+    if (MR == 1) decode_stream_kernel<1, FMT><<<grid, 256, 0, stream>>>(a);
+    else if (MR == 2) decode_stream_kernel<2, FMT><<<grid, 256, 0, stream>>>(a);
+    else decode_stream_kernel<4, FMT><<<grid, 256, 0, stream>>>(a);
+}
+void launch_stream(int fmt, int MR, dim3 grid, const DecStream& a, hipStream_t stream) {
+    if (fmt == XQ_FMT_NVFP4) launch_stream_fmt<XQ_FMT_NVFP4>(MR, grid, a, stream);
+    else launch_stream_fmt<XQ_FMT_FP8>(MR, grid, a, stream);
+}
+
 struct DecPlan {
     int ns_gu, cps_gu, ns_d, cps_d, units;
 };
@@ -542,8 +600,18 @@ int64_t infer_workspace(int64_t R, int E, int64_t H, int64_t I, int rp, int MR) 
 bool infer_supported(const xq_weight* gate, const xq_weight* up, const xq_weight* down, int64_t n_tokens, int32_t topk, int r) {
     if (!gate || !up || !down) return false;
     const xq_weight* w[3] = {gate, up, down};
-    for (int i = 0; i < 3; ++i)
-        if (w[i]->format != XQ_FMT_FP8 || w[i]->scale_dtype != XQ_SCALE_F32 || !xq_aligned(w[i]->packed, 16) || !w[i]->scales) return false;
+    for (int i = 0; i < 3; ++i) {
+        if (w[i]->format != gate->format || !xq_aligned(w[i]->packed, 16) || !w[i]->scales) return false;
+        if (w[i]->format == XQ_FMT_FP8) {
+            if (w[i]->scale_dtype != XQ_SCALE_F32) return false;
+        } else if (w[i]->format == XQ_FMT_NVFP4) {
+            if (w[i]->layout != XQ_LAYOUT_GKN || w[i]->scale_dtype != XQ_SCALE_E4M3 || w[i]->group != 16 || !w[i]->global_scale ||
+                !xq_aligned(w[i]->scales, 16))
+                return false;
+        } else {
+            return false;
+        }
+    }
     const int64_t H = gate->rows, I = gate->cols;
     if (up->rows != H || up->cols != I || down->rows != I || down->cols != H) return false;
     if (H % kDecTile || I % kDecTile) return false;
@@ -578,7 +646,7 @@ extern "C" int xq_grouped_fwd_infer(const xq_weight* gate, const xq_weight* up, 
     int rc;
     if ((rc = xq_validate_weight(gate, who)) || (rc = xq_validate_weight(up, who)) || (rc = xq_validate_weight(down, who))) return rc;
     XQ_REQUIRE(infer_supported(gate, up, down, n_tokens, topk, lora->r),
-               "%s: takes block-fp8 banks that make an MLP (hidden and intermediate sizes multiples of %d, at most %d experts), "
+               "%s: takes block-fp8 or nvfp4 (e4m3 block scales) banks of one format that make an MLP (hidden and intermediate sizes multiples of %d, at most %d experts), "
                "1 to %d routed copies (tokens x top-k, top-k <= %d) and ranks 1..64; see xq_grouped_infer_supported()",
                who, kDecTile, kDecMaxExperts, kDecMaxPairs, kDecMaxTopk);
     XQ_REQUIRE(lora->dtype == XQ_DT_F32 || lora->dtype == XQ_DT_BF16, "%s: bad lora dtype", who);
@@ -617,7 +685,8 @@ extern "C" int xq_grouped_fwd_infer(const xq_weight* gate, const xq_weight* up, 
     const int lora_f32 = lora->dtype == XQ_DT_F32;
     DecStream s1{};
     s1.packed[0] = (const uint8_t*)gate->packed; s1.packed[1] = (const uint8_t*)up->packed;
-    s1.scales[0] = (const float*)gate->scales; s1.scales[1] = (const float*)up->scales;
+    s1.scales[0] = gate->scales; s1.scales[1] = up->scales;
+    s1.gs[0] = gate->global_scale; s1.gs[1] = up->global_scale;
     s1.n_banks = 2; s1.K = (int)H; s1.N = (int)I; s1.sn = (int)xq_cdiv(I, 128);
     s1.x = (const bf16_t*)hidden; s1.ldx = ld_hidden; s1.by_token = 1; s1.topk = topk;
     s1.cps = pl.cps_gu; s1.n_slices = pl.ns_gu; s1.n_tiles = (int)(I / kDecTile);
@@ -626,9 +695,7 @@ extern "C" int xq_grouped_fwd_infer(const xq_weight* gate, const xq_weight* up, 
     s1.A_shared[0] = lora->A_experts[0] == 1 && E > 1; s1.A_shared[1] = lora->A_experts[1] == 1 && E > 1;
     s1.lora_f32 = lora_f32; s1.r = r; s1.rp = rp; s1.su_part = su_gu; s1.R = (int)R; s1.L = L;
     const dim3 g1((unsigned)(s1.n_tiles + 1), (unsigned)pl.ns_gu, (unsigned)(pl.units * 2));
-    if (MR == 1) decode_stream_kernel<1><<<g1, 256, 0, stream>>>(s1);
-    else if (MR == 2) decode_stream_kernel<2><<<g1, 256, 0, stream>>>(s1);
-    else decode_stream_kernel<4><<<g1, 256, 0, stream>>>(s1);
+    launch_stream(gate->format, MR, g1, s1, stream);
     XQ_CHECK_LAUNCH(who);
 
     DecMid md{};
@@ -641,7 +708,7 @@ extern "C" int xq_grouped_fwd_infer(const xq_weight* gate, const xq_weight* up, 
     XQ_CHECK_LAUNCH(who);
 
     DecStream s2{};
-    s2.packed[0] = (const uint8_t*)down->packed; s2.scales[0] = (const float*)down->scales;
+    s2.packed[0] = (const uint8_t*)down->packed; s2.scales[0] = down->scales; s2.gs[0] = down->global_scale;
     s2.n_banks = 1; s2.K = (int)I; s2.N = (int)H; s2.sn = (int)xq_cdiv(H, 128);
     s2.x = h; s2.ldx = I; s2.by_token = 0; s2.topk = topk;
     s2.cps = pl.cps_d; s2.n_slices = pl.ns_d; s2.n_tiles = (int)(H / kDecTile);
@@ -649,9 +716,7 @@ extern "C" int xq_grouped_fwd_infer(const xq_weight* gate, const xq_weight* up, 
     s2.A[0] = lora->A[2]; s2.A_shared[0] = lora->A_experts[2] == 1 && E > 1;
     s2.lora_f32 = lora_f32; s2.r = r; s2.rp = rp; s2.su_part = su_d; s2.R = (int)R; s2.L = L;
     const dim3 g2((unsigned)(s2.n_tiles + 1), (unsigned)pl.ns_d, (unsigned)pl.units);
-    if (MR == 1) decode_stream_kernel<1><<<g2, 256, 0, stream>>>(s2);
-    else if (MR == 2) decode_stream_kernel<2><<<g2, 256, 0, stream>>>(s2);
-    else decode_stream_kernel<4><<<g2, 256, 0, stream>>>(s2);
+    launch_stream(gate->format, MR, g2, s2, stream);
     XQ_CHECK_LAUNCH(who);
 
     DecFinal fn{};
