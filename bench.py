@@ -378,6 +378,9 @@ def main():
     ap.add_argument("--traffic-bytes", type=float, default=None,
                     help="HBM bytes per launch of the roofline kernel from such counter runs (reported as "
                          "roofline.traffic; default: the committed measurement of that config, else null)")
+    ap.add_argument("--routed-decode", choices=("block_fp8", "nvfp4"), default=None,
+                    help="not a BASELINE config: only the routed expert MLP of configs[3]'s banks (in this format) for 1-64 "
+                         "tokens, forward only -- the table that the default run carries as its third `secondary` entry")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs the QLoRA path on ONE GPU; --gpus must be 1 "
@@ -389,6 +392,11 @@ def main():
     from xorl_amd.functional import silu_and_mul
 
     dev = torch.device("cuda:0")
+    if args.routed_decode:
+        print(json.dumps({"metric": "routed expert MLP forward for a handful of tokens (not a BASELINE config)", "unit": "GB/s",
+                          "n_gpus": 1, "data": "synthetic", "config": {"workload": ROUTED_DECODE_WORKLOAD + "; " + args.routed_decode},
+                          "cases": routed_decode_table(dev, fmt=args.routed_decode)}))
+        return
     if args.config != 1:
         return run_other(args, dev)
     mods_cpu = build_modules()
@@ -628,15 +636,21 @@ def decode_case_table(dev, reps: int = 24, replays: int = 5):
     return rows
 
 
-def routed_decode_table(dev, sets: int = 16, replays: int = 5):
+ROUTED_DECODE_WORKLOAD = ("the routed expert MLP of configs[3]'s banks (E=128, hidden 2048, intermediate 768, top-8, r=16) for 1-64 "
+                          "tokens, forward only, nothing differentiated; per forward, 16 routings per HIP graph (touched experts "
+                          "from HBM); `bytes` = packed bytes of the touched experts")
+
+
+def routed_decode_table(dev, sets: int = 16, replays: int = 5, fmt: str = "block_fp8"):
     """The routed expert MLP of configs[3]'s banks for a handful of tokens with nothing to differentiate: the
     weight-streaming form (xq_grouped_fwd_infer) beside the training forward (xq_grouped_fwd) on the same calls, `sets`
     forwards with different routings per HIP graph so that the touched experts come from HBM."""
     import xorl_amd.moe_functional as MF
-    from xorl_amd.qlora import BlockFP8QLoRAMoeExperts
+    from xorl_amd.qlora import BlockFP8QLoRAMoeExperts, NvFP4QLoRAMoeExperts
 
     E, Hd, I, topk, r = 128, 2048, 768, 8, 16
-    m = BlockFP8QLoRAMoeExperts(E, E, I, Hd, r=r, lora_alpha=2 * r, hybrid_shared=False).to(dev)
+    cls = NvFP4QLoRAMoeExperts if fmt == "nvfp4" else BlockFP8QLoRAMoeExperts
+    m = cls(E, E, I, Hd, r=r, lora_alpha=2 * r, hybrid_shared=False).to(dev)
     g = torch.Generator(device=dev).manual_seed(50)
     w = lambda *shape: torch.randn(*shape, generator=g, device=dev) * 0.02
     m.load_weights(w(E, Hd, I), w(E, Hd, I), w(E, I, Hd))
@@ -649,7 +663,7 @@ def routed_decode_table(dev, sets: int = 16, replays: int = 5):
             rw, sel = zipf_routing(max(T, 8), E, topk, seed=3 + i, device=dev)
             calls.append((torch.randn(T, Hd, generator=g, device=dev).to(torch.bfloat16), rw[:T].contiguous(), sel[:T].contiguous()))
         touched = sum(int(torch.unique(c[2]).numel()) for c in calls) / sets
-        nbytes = touched * 3 * (Hd * I + (Hd // 128) * (I // 128) * 4)
+        nbytes = touched * 3 * ((Hd * I // 2 + Hd * I // 16 + 4) if fmt == "nvfp4" else (Hd * I + (Hd // 128) * (I // 128) * 4))
         us = {}
         for name, on in (("streaming", True), ("training_forward", False)):
             MF.DECODE_PATH = on
@@ -696,9 +710,7 @@ def secondary_measurements(args, dev):
     out.append({"workload": c3["config"]["workload"], "value": c3["value"], "unit": "TFLOP/s", "ms_per_step": c3["ms_per_step"],
                 **c3["roofline"]})
     torch.cuda.empty_cache()
-    out.append({"workload": "not a BASELINE config: the routed expert MLP of configs[3]'s banks (E=128, hidden 2048, intermediate 768, "
-                            "top-8, r=16, block_fp8) for 1-64 tokens, forward only, nothing differentiated; per forward, 16 "
-                            "routings per HIP graph (touched experts from HBM); `bytes` = packed bytes of the touched experts",
+    out.append({"workload": "not a BASELINE config: " + ROUTED_DECODE_WORKLOAD + "; block_fp8",
                 "bound": "hbm", "peak": 8000.0, "unit": "GB/s",
                 "kernel": "decode_stream_kernel (+ decode_route / decode_mid / decode_final), xq_grouped_fwd_infer",
                 "cases": routed_decode_table(dev)})
