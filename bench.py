@@ -378,7 +378,7 @@ def main():
     ap.add_argument("--traffic-bytes", type=float, default=None,
                     help="HBM bytes per launch of the roofline kernel from such counter runs (reported as "
                          "roofline.traffic; default: the committed measurement of that config, else null)")
-    ap.add_argument("--routed-decode", choices=("block_fp8", "nvfp4"), default=None,
+    ap.add_argument("--routed-decode", choices=("block_fp8", "nvfp4", "nf4"), default=None,
                     help="not a BASELINE config: only the routed expert MLP of configs[3]'s banks (in this format) for 1-64 "
                          "tokens, forward only -- the table that the default run carries as its third `secondary` entry")
     args = ap.parse_args()
@@ -646,10 +646,11 @@ def routed_decode_table(dev, sets: int = 16, replays: int = 5, fmt: str = "block
     weight-streaming form (xq_grouped_fwd_infer) beside the training forward (xq_grouped_fwd) on the same calls, `sets`
     forwards with different routings per HIP graph so that the touched experts come from HBM."""
     import xorl_amd.moe_functional as MF
-    from xorl_amd.qlora import BlockFP8QLoRAMoeExperts, NvFP4QLoRAMoeExperts
+    from xorl_amd.qlora import BlockFP8QLoRAMoeExperts, NF4QLoRAMoeExperts, NvFP4QLoRAMoeExperts
 
     E, Hd, I, topk, r = 128, 2048, 768, 8, 16
-    cls = NvFP4QLoRAMoeExperts if fmt == "nvfp4" else BlockFP8QLoRAMoeExperts
+    cls = {"nvfp4": NvFP4QLoRAMoeExperts, "nf4": NF4QLoRAMoeExperts}.get(fmt, BlockFP8QLoRAMoeExperts)
+    per_expert = {"nvfp4": Hd * I // 2 + Hd * I // 16 + 4, "nf4": Hd * I // 2 + Hd * I // 64 * 4}.get(fmt, Hd * I + (Hd // 128) * (I // 128) * 4)
     m = cls(E, E, I, Hd, r=r, lora_alpha=2 * r, hybrid_shared=False).to(dev)
     g = torch.Generator(device=dev).manual_seed(50)
     w = lambda *shape: torch.randn(*shape, generator=g, device=dev) * 0.02
@@ -663,7 +664,7 @@ def routed_decode_table(dev, sets: int = 16, replays: int = 5, fmt: str = "block
             rw, sel = zipf_routing(max(T, 8), E, topk, seed=3 + i, device=dev)
             calls.append((torch.randn(T, Hd, generator=g, device=dev).to(torch.bfloat16), rw[:T].contiguous(), sel[:T].contiguous()))
         touched = sum(int(torch.unique(c[2]).numel()) for c in calls) / sets
-        nbytes = touched * 3 * ((Hd * I // 2 + Hd * I // 16 + 4) if fmt == "nvfp4" else (Hd * I + (Hd // 128) * (I // 128) * 4))
+        nbytes = touched * 3 * per_expert
         us = {}
         for name, on in (("streaming", True), ("training_forward", False)):
             MF.DECODE_PATH = on

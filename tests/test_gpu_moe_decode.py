@@ -1,5 +1,5 @@
 """GPU parity: the routed expert MLP for a handful of tokens with nothing to differentiate (xq_grouped_fwd_infer: the
-touched experts' block-fp8 or nvfp4 matrices streamed once, four or five launches) against the float64 per-expert oracle program and
+touched experts' block-fp8, nvfp4 or NF4 matrices streamed once, four or five launches) against the float64 per-expert oracle program and
 against the training forward (xq_grouped_fwd) on the same inputs."""
 
 import ctypes
@@ -13,6 +13,7 @@ from tests.util_cases import close, gen
 
 pytestmark = pytest.mark.gpu
 TOL = 1e-2
+SAME = 8e-3     # streaming form against training forward
 
 
 def _lora_of(m):
@@ -49,7 +50,7 @@ def _both_paths(m, x, rw, sel, device):
     return y.cpu(), y_train.cpu()
 
 
-@pytest.mark.parametrize("fmt", ["block_fp8", "nvfp4"])
+@pytest.mark.parametrize("fmt", ["block_fp8", "nvfp4", "nf4"])
 @pytest.mark.parametrize("E,T,H,I,r,topk,hybrid,rw_dtype", [
     (8, 1, 256, 512, 16, 2, False, torch.bfloat16),        # one token: one row per expert, the one-row form
     (16, 1, 1024, 768, 16, 8, False, torch.float32),       # 8 experts of 16, K slices of one chunk
@@ -68,14 +69,15 @@ def test_decode_forward_vs_oracle(hip_device, fmt, E, T, H, I, r, topk, hybrid, 
     y, y_train = _both_paths(m, x, rw, sel, hip_device)
     ex = R.moe_fwd_bwd(x, rw, sel, banks["gate"], banks["up"], banks["down"], _lora_of(m), m.scaling)
     close(y, ex["y"], TOL)
-    # same rounding points as the training forward: the two differ by summation order inside the dot products only
-    assert R.max_rel_err(y.float(), y_train.float()) <= 4e-3
+    # same rounding points as the training forward: the two differ by summation order inside the dot products only, which
+    # can move a bf16 intermediate or output by an ulp (up to 2^-7 of the value)
+    assert R.max_rel_err(y.float(), y_train.float()) <= SAME
     # and the call is deterministic
     y2, _ = _both_paths(m, x, rw, sel, hip_device)
     assert torch.equal(y, y2)
 
 
-@pytest.mark.parametrize("fmt", ["block_fp8", "nvfp4"])
+@pytest.mark.parametrize("fmt", ["block_fp8", "nvfp4", "nf4"])
 def test_decode_forward_bf16_factors_and_swiglu_limit(hip_device, fmt):
     E, T, H, I, r, topk = 8, 4, 512, 256, 16, 2
     m, banks = _make_experts(fmt, E, H, I, r, False, seed=91, device=hip_device)
@@ -93,7 +95,7 @@ def test_decode_forward_bf16_factors_and_swiglu_limit(hip_device, fmt):
         y, y_train = _both_paths(m, x, rw, sel, hip_device)
         ex = R.moe_fwd_bwd(x, rw, sel, banks["gate"], banks["up"], banks["down"], lora, m.scaling, swiglu_limit=lim)
         close(y, ex["y"], TOL)
-        assert R.max_rel_err(y.float(), y_train.float()) <= 4e-3
+        assert R.max_rel_err(y.float(), y_train.float()) <= SAME
         outs[lim] = y
     assert not torch.equal(outs[0.0], outs[0.75])          # the clamp took part
 
@@ -116,7 +118,7 @@ def test_decode_forward_drops_bad_ids_and_takes_repeated_experts(hip_device):
     rw0[~ok] = 0
     ex = R.moe_fwd_bwd(x, rw0, sel.clamp(0, E - 1), banks["gate"], banks["up"], banks["down"], _lora_of(m), m.scaling)
     close(y, ex["y"], TOL)
-    assert R.max_rel_err(y.float(), y_train.float()) <= 4e-3
+    assert R.max_rel_err(y.float(), y_train.float()) <= SAME
     # a token whose copies are all dropped gets zeros
     sel2 = sel.clone()
     sel2[5] = -3
@@ -130,7 +132,8 @@ def test_decode_form_declines_what_it_does_not_take(hip_device):
     import xorl_amd.moe_functional as MF
     from xorl_amd import _C
 
-    # hidden size not a multiple of 256; NF4 banks; more than 512 routed copies; a forward that is differentiated
+    # hidden size not a multiple of 256; a scale group size outside the forms built; more than 512 routed copies; a forward
+    # that is differentiated
     m, _ = _make_experts("block_fp8", 4, 128, 256, 8, False, seed=60, device=hip_device)
     rw, sel = _zipf_routing(2, 4, 2, seed=61)
     x = gen((2, 128), 1.0, 62, torch.bfloat16).to(hip_device)
@@ -142,7 +145,10 @@ def test_decode_form_declines_what_it_does_not_take(hip_device):
     assert _C.lib().xq_grouped_infer_supported(ctypes.byref(wg), ctypes.byref(wu), ctypes.byref(wd), 2, 2, 8) == 0
     m4, _ = _make_experts("nf4", 4, 256, 256, 8, False, seed=63, device=hip_device)
     x4 = gen((2, 256), 1.0, 64, torch.bfloat16).to(hip_device)
-    assert MF._moe_infer(*args(m4, x4, rw, sel)) is None
+    assert MF._moe_infer(*args(m4, x4, rw, sel)) is not None          # NF4 banks with fp32 scales per 64 rows are taken ...
+    w4 = [m4._bank(p).c() for p in ("gate", "up", "down")]
+    w4[1].group = 32                                                  # ... other group sizes are not
+    assert _C.lib().xq_grouped_infer_supported(ctypes.byref(w4[0]), ctypes.byref(w4[1]), ctypes.byref(w4[2]), 2, 2, 8) == 0
     m8, _ = _make_experts("block_fp8", 4, 256, 256, 8, False, seed=65, device=hip_device)
     rw_big, sel_big = _zipf_routing(300, 4, 2, seed=66)
     x_big = gen((300, 256), 1.0, 67, torch.bfloat16).to(hip_device)

@@ -1,4 +1,4 @@
-// xq_grouped_fwd_infer: the routed SwiGLU expert MLP with LoRA on block-fp8 or nvfp4 expert banks for a handful of tokens
+// xq_grouped_fwd_infer: the routed SwiGLU expert MLP with LoRA on block-fp8, nvfp4 or nf4 expert banks for a handful of tokens
 // (decode / rollout), nothing kept for a backward.  The program is the forward of the reference's
 // _MoeExpertsLoRAFunction (ops/moe/lora.py:525-713) with the rounding points of xq_grouped_fwd; what differs is the
 // organisation.  With few tokens an expert sees one or two rows, so the time is the touched experts' bytes: every
@@ -174,7 +174,7 @@ __device__ __forceinline__ float fma_b16(float v, const float* su, const float (
 struct DecStream {
     const uint8_t* packed[2];       // one bank (down) or two (gate, up): block fp8 [E][K][N] e4m3 bytes; nvfp4 [E][K / 2][N]
                                     // bytes, rows 2 p (low nibble) and 2 p + 1 of a column in one byte
-    const void* scales[2];          // block fp8: fp32 [E][K / 128][ceil(N / 128)]; nvfp4: e4m3 [E][K / 16][N]
+    const void* scales[2];          // block fp8: fp32 [E][K / 128][ceil(N / 128)]; nvfp4: e4m3 [E][K / 16][N]; nf4: fp32 [E][K / 64][N]
     const float* gs[2];             // nvfp4: the experts' global scales
     int32_t n_banks, K, N, sn;
     const bf16_t* x;                // the rows that are multiplied: token rows (by_token) or rows in expert order
@@ -203,16 +203,21 @@ struct DecStream {
 // nvfp4 banks (FMT = XQ_FMT_NVFP4) hold the two rows of a pair in one byte, which is the operand layout as it is: a
 // lane's 16-byte load is its 16 columns of one row pair, a chunk 4 weight loads and 2 loads of e4m3 block scales (16
 // columns x the wave's two 16-row groups) per lane; a byte becomes its two e2m1 values by one conversion, each times
-// fl(block scale x global scale), rounded to bf16 -- the reference decoder's values.
+// fl(block scale x global scale), rounded to bf16 -- the reference decoder's values.  NF4 banks (FMT = XQ_FMT_NF4,
+// fp32 scales per 64 rows and column) have the same byte layout: the wave's 32 rows lie in one scale group, so a chunk
+// is 4 weight loads and 4 loads of the 16 columns' scales; the 16 levels are read from a copy of the table in LDS,
+// one copy per wave (16 banks: any mix of codes reads it at full rate).
 template <int MR, int FMT>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MR == 1 ? 4 : MR == 2 ? 3 : 2, 8))) decode_stream_kernel(DecStream g) {
-    constexpr bool NV = FMT == XQ_FMT_NVFP4;
+    constexpr bool NV = FMT == XQ_FMT_NVFP4, NF = FMT == XQ_FMT_NF4, P4 = NV || NF;
+    __shared__ float nf4_tab[NF ? 4 : 1][16];
     __shared__ __attribute__((aligned(16))) bf16_t xs[MR][kDecMaxChunks * kDecChunk];
     __shared__ __attribute__((aligned(16))) float red[16 * kDecTile];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int tile = blockIdx.x, slice = blockIdx.y;
     const int li = (int)blockIdx.z / g.n_banks, bank = (int)blockIdx.z % g.n_banks;
+    if (NF && tid < 64) nf4_tab[tid >> 4][tid & 15] = kNf4Level[tid & 15];    // ordered before its use by the barrier behind the x rows
     int4 unit;
     if (g.L.selected) {
         const int v = g.L.selected[li];
@@ -230,21 +235,30 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MR == 
     const bool lora_unit = tile == g.n_tiles;
     const int kq = lane >> 4, c = lane & 15;
     const int n0 = tile * kDecTile;
-    const uint8_t* wbase = NV ? g.packed[bank] + ((int64_t)e * (g.K >> 1) + ((k0 + wave * 32) >> 1)) * g.N + n0
+    const uint8_t* wbase = P4 ? g.packed[bank] + ((int64_t)e * (g.K >> 1) + ((k0 + wave * 32) >> 1)) * g.N + n0
                               : g.packed[bank] + ((int64_t)e * g.K + k0 + wave * 32) * g.N + n0;
-    const uint32_t woff = (uint32_t)((NV ? kq : 2 * kq) * g.N + c * 16);
+    const uint32_t woff = (uint32_t)((P4 ? kq : 2 * kq) * g.N + c * 16);
     // block fp8: the lane's block scale of a chunk; nvfp4: the 16 columns' e4m3 scales of the wave's two 16-row groups
+    // nf4: the 16 columns' fp32 scales of the wave's 64-row group
     const uint8_t* sbase = NV ? (const uint8_t*)g.scales[bank] + ((int64_t)e * (g.K >> 4) + c_begin * 8 + wave * 2) * g.N + n0
+                         : NF ? (const uint8_t*)((const float*)g.scales[bank] + ((int64_t)e * (g.K >> 6) + c_begin * 2 + (wave >> 1)) * g.N + n0)
                               : (const uint8_t*)((const float*)g.scales[bank] + ((int64_t)e * (g.K / kDecChunk) + c_begin) * g.sn + (n0 >> 7));
-    const uint32_t soff = (uint32_t)(NV ? c * 16 : (c >> 3) * 4);
+    const uint32_t soff = (uint32_t)(NV ? c * 16 : NF ? c * 64 : (c >> 3) * 4);
     const float gsc = NV ? g.gs[bank][e] : 1.0f;
 
     // a chunk's loads: block fp8 w[0..7] the eight rows and sc the block scale; nvfp4 w[0..3] the four row pairs, w[4..5]
-    // the scale bytes
+    // the scale bytes; nf4 w[0..3] the four row pairs, w[4..7] the 16 scales
     u32x4 wa[8], wb[8];
     float sa, sb;
     auto issue = [&](u32x4(&w)[8], float& sc, int ch) {
-        if (NV) {
+        if (NF) {
+            const uint8_t* p = wbase + (int64_t)ch * (kDecChunk / 2) * g.N;
+            const uint8_t* sp = sbase + (int64_t)ch * 2 * g.N * 4 + soff;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) w[4 + q] = *(const u32x4*)(sp + 16 * q);
+#pragma unroll
+            for (int st = 0; st < 4; ++st) w[st] = __builtin_nontemporal_load((const u32x4*)(p + (int64_t)(4 * st) * g.N + woff));
+        } else if (NV) {
             const uint8_t* p = wbase + (int64_t)ch * (kDecChunk / 2) * g.N;
             const uint8_t* sp = sbase + (int64_t)ch * 8 * g.N;
             w[4] = *(const u32x4*)(sp + soff);
@@ -327,7 +341,18 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MR == 
 #pragma unroll
         for (int st = 0; st < 4; ++st) {
             uint32_t pk[16];
-            if (NV) {
+            if (NF) {
+                const float* tab = nf4_tab[wave];
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+#pragma unroll
+                    for (int b = 0; b < 4; ++b) {
+                        const uint32_t byte = (w[st][q] >> (8 * b)) & 0xffu;
+                        const float sv = __uint_as_float(w[4 + q][b]);
+                        pk[4 * q + b] = pack_bf16x2(tab[byte & 15u] * sv, tab[byte >> 4] * sv);
+                    }
+                }
+            } else if (NV) {
                 if ((st & 1) == 0) {
 #pragma unroll
                     for (int q = 0; q < 4; ++q) {
@@ -561,6 +586,7 @@ void launch_stream_fmt(int MR, dim3 grid, const DecStream& a, hipStream_t stream
 }
 void launch_stream(int fmt, int MR, dim3 grid, const DecStream& a, hipStream_t stream) {
     if (fmt == XQ_FMT_NVFP4) launch_stream_fmt<XQ_FMT_NVFP4>(MR, grid, a, stream);
+    else if (fmt == XQ_FMT_NF4) launch_stream_fmt<XQ_FMT_NF4>(MR, grid, a, stream);
     else launch_stream_fmt<XQ_FMT_FP8>(MR, grid, a, stream);
 }
 
@@ -608,6 +634,8 @@ bool infer_supported(const xq_weight* gate, const xq_weight* up, const xq_weight
             if (w[i]->layout != XQ_LAYOUT_GKN || w[i]->scale_dtype != XQ_SCALE_E4M3 || w[i]->group != 16 || !w[i]->global_scale ||
                 !xq_aligned(w[i]->scales, 16))
                 return false;
+        } else if (w[i]->format == XQ_FMT_NF4) {
+            if (w[i]->layout != XQ_LAYOUT_GKN || w[i]->scale_dtype != XQ_SCALE_F32 || w[i]->group != 64 || !xq_aligned(w[i]->scales, 16)) return false;
         } else {
             return false;
         }
@@ -646,7 +674,7 @@ extern "C" int xq_grouped_fwd_infer(const xq_weight* gate, const xq_weight* up, 
     int rc;
     if ((rc = xq_validate_weight(gate, who)) || (rc = xq_validate_weight(up, who)) || (rc = xq_validate_weight(down, who))) return rc;
     XQ_REQUIRE(infer_supported(gate, up, down, n_tokens, topk, lora->r),
-               "%s: takes block-fp8 or nvfp4 (e4m3 block scales) banks of one format that make an MLP (hidden and intermediate sizes multiples of %d, at most %d experts), "
+               "%s: takes block-fp8, nvfp4 (e4m3 block scales) or nf4 (fp32 scales, group 64) banks of one format that make an MLP (hidden and intermediate sizes multiples of %d, at most %d experts), "
                "1 to %d routed copies (tokens x top-k, top-k <= %d) and ranks 1..64; see xq_grouped_infer_supported()",
                who, kDecTile, kDecMaxExperts, kDecMaxPairs, kDecMaxTopk);
     XQ_REQUIRE(lora->dtype == XQ_DT_F32 || lora->dtype == XQ_DT_BF16, "%s: bad lora dtype", who);
