@@ -194,3 +194,42 @@ def test_decode_forward_in_a_hip_graph(hip_device):
         torch.cuda.synchronize()
         ex = R.moe_fwd_bwd(x2, rw2, sel2, banks["gate"], banks["up"], banks["down"], _lora_of(m), m.scaling)
         close(out.cpu(), ex["y"], TOL)
+
+
+def test_dispatched_rows_take_the_streaming_form(hip_device):
+    """compute_dispatched (rows already grouped by expert, no routing scores) under no_grad with a handful of rows: the same
+    streaming forward as a top-1 problem with unit weights; equal to the training form's result to rounding and to the
+    oracle program."""
+    import xorl_amd.moe_functional as MF
+
+    E, H, I, r = 8, 512, 256, 16
+    m, banks = _make_experts("block_fp8", E, H, I, r, False, seed=33, device=hip_device)
+    counts = torch.tensor([3, 0, 1, 6, 0, 2, 0, 5])
+    R_ = int(counts.sum())
+    x = gen((R_, H), 1.0, 34, torch.bfloat16)
+    cumsum = counts.cumsum(0).to(hip_device)
+    calls = []
+    real = MF._moe_infer
+
+    def spy(*a, **k):
+        out = real(*a, **k)
+        calls.append(out is not None)
+        return out
+
+    MF._moe_infer = spy
+    try:
+        with torch.no_grad():
+            y = m.compute_dispatched(x.to(hip_device), cumsum).cpu()
+    finally:
+        MF._moe_infer = real
+    assert calls == [True]
+    MF.DECODE_PATH = False
+    try:
+        with torch.no_grad():
+            y_train = m.compute_dispatched(x.to(hip_device), cumsum).cpu()
+    finally:
+        MF.DECODE_PATH = True
+    sel = torch.repeat_interleave(torch.arange(E), counts).int().unsqueeze(1)
+    ex = R.moe_fwd_bwd(x, torch.ones(R_, 1), sel, banks["gate"], banks["up"], banks["down"], _lora_of(m), m.scaling)
+    close(y, ex["y"], TOL)
+    assert R.max_rel_err(y.float(), y_train.float()) <= SAME

@@ -445,6 +445,13 @@ def moe_experts_qlora_ep_compute(permute_tokens: Tensor, cumsum: Tensor, gate_pr
     if int(ends[-1]) != R:
         raise _C.XqError(f"cumsum ends at {int(ends[-1])} but {R} rows were passed")
     ones = torch.ones(R, 1, dtype=torch.float32, device=dev)
+    if DECODE_PATH and not torch.compiler.is_compiling() and not (
+            torch.is_grad_enabled() and any(t.requires_grad for t in (permute_tokens, *factors))):
+        # a handful of rows with nothing to differentiate: the weight-streaming forward (top-1, unit weights)
+        out = _moe_infer(permute_tokens, ones, expert_of_row.to(torch.int32).unsqueeze(1), factors, (gate_proj, up_proj, down_proj),
+                         E, scaling, float(swiglu_limit or 0.0))
+        if out is not None:
+            return out
     return MoeExpertsQLoRAFunction.apply(permute_tokens, ones, expert_of_row.to(torch.int32).unsqueeze(1), *factors,
                                          gate_proj, up_proj, down_proj, E, scaling, float(swiglu_limit or 0.0))
 
