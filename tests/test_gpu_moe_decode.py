@@ -233,3 +233,16 @@ def test_dispatched_rows_take_the_streaming_form(hip_device):
     ex = R.moe_fwd_bwd(x, torch.ones(R_, 1), sel, banks["gate"], banks["up"], banks["down"], _lora_of(m), m.scaling)
     close(y, ex["y"], TOL)
     assert R.max_rel_err(y.float(), y_train.float()) <= SAME
+
+
+def test_decode_forward_many_experts_and_widest_topk(hip_device):
+    """More experts than the routing block has threads (its loops over experts take several rounds), the widest top-k the
+    form takes, a rank below 16, one expert alone, and two tokens (the two-row form with mostly one-row units)."""
+    for E, T, H, I, r, topk in [(520, 5, 256, 256, 4, 16), (1, 3, 256, 256, 8, 1), (9, 2, 256, 512, 16, 8)]:
+        m, banks = _make_experts("block_fp8", E, H, I, r, False, seed=E + 7, device=hip_device)
+        rw, sel = _zipf_routing(T, E, topk, seed=E + 8, empty=0 if E == 1 else 1)
+        x = gen((T, H), 1.0, E + 9, torch.bfloat16)
+        y, y_train = _both_paths(m, x, rw, sel, hip_device)
+        ex = R.moe_fwd_bwd(x, rw, sel, banks["gate"], banks["up"], banks["down"], _lora_of(m), m.scaling)
+        close(y, ex["y"], TOL)
+        assert R.max_rel_err(y.float(), y_train.float()) <= SAME
