@@ -59,7 +59,8 @@ def _both_paths(m, x, rw, sel, device):
     (6, 64, 256, 256, 24, 2, True, torch.float32),         # r not a multiple of 16; up to dozens of rows per expert
     (40, 64, 512, 512, 64, 8, False, torch.bfloat16),      # 512 routed copies (the most), r = 64
     (8, 1, 4096, 256, 16, 2, False, torch.float32),        # one-row form, K slices of two chunks
-    (12, 4, 2048, 768, 16, 8, False, torch.bfloat16),      # two-row form, K slices of three chunks and a last one of one
+    (40, 64, 2048, 256, 16, 8, False, torch.float32),      # four-row form, K slices of four chunks (the streaming loop proper)
+    (12, 4, 2048, 768, 16, 8, False, torch.bfloat16),      # one-row form on four tokens, K slices of three chunks and a last one of one
 ])
 def test_decode_forward_vs_oracle(hip_device, fmt, E, T, H, I, r, topk, hybrid, rw_dtype):
     m, banks = _make_experts(fmt, E, H, I, r, hybrid, seed=3 * E + T, device=hip_device)
@@ -237,7 +238,7 @@ def test_dispatched_rows_take_the_streaming_form(hip_device):
 
 def test_decode_forward_many_experts_and_widest_topk(hip_device):
     """More experts than the routing block has threads (its loops over experts take several rounds), the widest top-k the
-    form takes, a rank below 16, one expert alone, and two tokens (the two-row form with mostly one-row units)."""
+    form takes, a rank below 16, one expert alone, and two tokens."""
     for E, T, H, I, r, topk in [(520, 5, 256, 256, 4, 16), (1, 3, 256, 256, 8, 1), (9, 2, 256, 512, 16, 8)]:
         m, banks = _make_experts("block_fp8", E, H, I, r, False, seed=E + 7, device=hip_device)
         rw, sel = _zipf_routing(T, E, topk, seed=E + 8, empty=0 if E == 1 else 1)

@@ -7,10 +7,10 @@
 // [K, N] with N contiguous, so a lane keeps 16 output columns and walks down K -- no transposition, no matrix cores,
 // which a one-row operand would leave idle) and store fp32 partial sums; two small kernels between and after the
 // two streaming launches add the partial sums and the low-rank terms, apply SwiGLU and the routing weight and sum a
-// token's top-k copies.  Five launches (four for one token, which needs no routing launch), all sums in a fixed order (deterministic), nothing zeroed, no atomics on
+// token's top-k copies.  Five launches (four for up to four tokens, which need no routing launch), all sums in a fixed order (deterministic), nothing zeroed, no atomics on
 // memory.
 //
-//   decode_route_kernel   : the touched experts' rows in units of 2 or 4 (stable order of the routed copies) -- one block
+//   decode_route_kernel   : the touched experts' rows in units of 4 (stable order of the routed copies) -- one block
 //   decode_stream_kernel  : gate | up partial sums [bank][K slice][row][I] + x . A partial sums (blocks of their own)
 //   decode_mid_kernel     : h = bf16(bf16(bf16(silu(g)) u) w), g / u = bf16(sum of slices + su . B), su = bf16(s x . A)
 //   decode_stream_kernel  : down partial sums [K slice][row][H] + h . A_d partial sums
@@ -35,7 +35,7 @@ inline int r_pad_of(int r) { return ((r + 15) / 16) * 16; }
 // its row m; per row row_info[2 row] = {the routed copy it is (token * topk + slot) or -1 past the last row, its expert}; per copy
 // pair_info[2 copy] = {its row or -1, its expert}.  What a block needs first sits behind one index, so that its loads
 // go out together instead of one after the other's result.
-// With one row per unit (direct: the one-token call) there is nothing to sort: a unit is a routed copy, its row the
+// With one row per unit (direct: calls of up to four tokens) there is nothing to sort: a unit is a routed copy, its row the
 // copy's number, and the kernels read the expert ids where the caller has them -- no routing launch.
 struct DecLists {
     int32_t* base;
@@ -51,7 +51,7 @@ struct DecLists {
 };
 
 __global__ void __launch_bounds__(512) decode_route_kernel(const int32_t* selected, int R, int E, int lg, int topk, int units_max, DecLists L) {
-    const int MR = 1 << lg;                          // rows per unit: 2 or 4
+    const int MR = 1 << lg;                          // rows per unit
     __shared__ __attribute__((aligned(16))) int32_t s_sel[kDecMaxPairs];
     __shared__ __attribute__((aligned(16))) int32_t s_cnt[kDecMaxExperts], s_begin[kDecMaxExperts], s_unit[kDecMaxExperts];
     const int t = threadIdx.x;
@@ -208,7 +208,7 @@ struct DecStream {
 // is 4 weight loads and 4 loads of the 16 columns' scales; the 16 levels are read from a copy of the table in LDS,
 // one copy per wave (16 banks: any mix of codes reads it at full rate).
 template <int MR, int FMT>
-__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MR == 1 ? 4 : MR == 2 ? 3 : 2, 8))) decode_stream_kernel(DecStream g) {
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MR == 1 ? 4 : 2, 8))) decode_stream_kernel(DecStream g) {
     constexpr bool NV = FMT == XQ_FMT_NVFP4, NF = FMT == XQ_FMT_NF4, P4 = NV || NF;
     __shared__ float nf4_tab[NF ? 4 : 1][16];
     __shared__ __attribute__((aligned(16))) bf16_t xs[MR][kDecMaxChunks * kDecChunk];
@@ -581,7 +581,6 @@ __global__ void __launch_bounds__(1024) decode_final_kernel(DecFinal g) {
 template <int FMT>
 void launch_stream_fmt(int MR, dim3 grid, const DecStream& a, hipStream_t stream) {
     if (MR == 1) decode_stream_kernel<1, FMT><<<grid, 256, 0, stream>>>(a);
-    else if (MR == 2) decode_stream_kernel<2, FMT><<<grid, 256, 0, stream>>>(a);
     else decode_stream_kernel<4, FMT><<<grid, 256, 0, stream>>>(a);
 }
 void launch_stream(int fmt, int MR, dim3 grid, const DecStream& a, hipStream_t stream) {
@@ -615,7 +614,9 @@ DecPlan plan_for(int64_t R, int E, int64_t H, int64_t I, int MR) {
     return p;
 }
 
-inline int rows_per_unit(int64_t n_tokens) { return n_tokens == 1 ? 1 : n_tokens <= 4 ? 2 : 4; }
+// up to four tokens run one row per unit with no routing launch (measured at four tokens: 50.0 us against 53.8 with units
+// of two rows behind a routing launch); more tokens are grouped four rows to a unit
+inline int rows_per_unit(int64_t n_tokens) { return n_tokens <= 4 ? 1 : 4; }
 
 int64_t infer_workspace(int64_t R, int E, int64_t H, int64_t I, int rp, int MR) {
     const DecPlan p = plan_for(R, E, H, I, MR);
@@ -706,7 +707,7 @@ extern "C" int xq_grouped_fwd_infer(const xq_weight* gate, const xq_weight* up, 
     float* su_d = (float*)take((int64_t)pl.ns_d * R * rp * 4);
 
     if (MR > 1) {
-        decode_route_kernel<<<dim3(1), 512, 0, stream>>>(selected, (int)R, E, MR == 2 ? 1 : 2, topk, pl.units, L);
+        decode_route_kernel<<<dim3(1), 512, 0, stream>>>(selected, (int)R, E, 2, topk, pl.units, L);
         XQ_CHECK_LAUNCH(who);
     }
 
