@@ -514,10 +514,17 @@ skinny_epilogue_kernel(const float* partial_, const float* su_part_, const void*
                 if (VEC) {
                     t = *(const f32x4*)((const float*)g.lora_B + (int64_t)col * g.r + (jr < g.r ? jr : 0));
                 } else {
+                    // (the storage type is tested around the four loads, not around each: a branch per load would make
+                    // every load wait for the one before)
+                    if (g.lora_f32) {
 #pragma unroll
-                    for (int c = 0; c < 4; ++c) {
-                        const int64_t idx = (int64_t)col * g.r + (jr + c < g.r ? jr + c : 0);
-                        t[c] = g.lora_f32 ? ((const float*)g.lora_B)[idx] : bf16_to_f32(((const bf16_t*)g.lora_B)[idx]);
+                        for (int c = 0; c < 4; ++c) t[c] = ((const float*)g.lora_B)[(int64_t)col * g.r + (jr + c < g.r ? jr + c : 0)];
+                    } else {
+                        bf16_t raw[4];
+#pragma unroll
+                        for (int c = 0; c < 4; ++c) raw[c] = ((const bf16_t*)g.lora_B)[(int64_t)col * g.r + (jr + c < g.r ? jr + c : 0)];
+#pragma unroll
+                        for (int c = 0; c < 4; ++c) t[c] = bf16_to_f32(raw[c]);
                     }
                 }
                 bq[jt * 4 + i] = t;
@@ -555,10 +562,15 @@ skinny_epilogue_kernel(const float* partial_, const float* su_part_, const void*
             for (int jt = 0; jt < RT; ++jt) {
                 const int jr = jt * 16 + 4 * (q & 3);
                 f32x4 t;
+                if (g.lora_f32) {
 #pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    const int64_t idx = (int64_t)col * g.r + (jr + c < g.r ? jr + c : 0);
-                    t[c] = g.lora_f32 ? ((const float*)g.lora_B)[idx] : bf16_to_f32(((const bf16_t*)g.lora_B)[idx]);
+                    for (int c = 0; c < 4; ++c) t[c] = ((const float*)g.lora_B)[(int64_t)col * g.r + (jr + c < g.r ? jr + c : 0)];
+                } else {
+                    bf16_t raw[4];
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) raw[c] = ((const bf16_t*)g.lora_B)[(int64_t)col * g.r + (jr + c < g.r ? jr + c : 0)];
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) t[c] = bf16_to_f32(raw[c]);
                 }
                 *(f32x4*)(&bt[jt][(q >> 4) * 64 + ((q ^ (q >> 4)) & 15) * 4]) = t;
             }
