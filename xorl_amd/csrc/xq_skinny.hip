@@ -61,21 +61,6 @@ struct SkinnyEpiArgs {
     int64_t ldy;
 };
 
-// 8 consecutive LoRA factor entries (fp32 or bf16 storage) -> one MFMA operand; entries at or
-// beyond `limit` (counted from the first) are zero
-__device__ __forceinline__ bf16x8 factor_frag(const void* base, int64_t idx, bool f32, int limit) {
-    uint32_t o[4];
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-        float lo = 0.0f, hi = 0.0f;
-        if (2 * e < limit) lo = f32 ? ((const float*)base)[idx + 2 * e] : bf16_to_f32(((const bf16_t*)base)[idx + 2 * e]);
-        if (2 * e + 1 < limit) hi = f32 ? ((const float*)base)[idx + 2 * e + 1] : bf16_to_f32(((const bf16_t*)base)[idx + 2 * e + 1]);
-        o[e] = pack_bf16x2(lo, hi);
-    }
-    u32x4 r = {o[0], o[1], o[2], o[3]};
-    return __builtin_bit_cast(bf16x8, r);
-}
-
 // One block = 128 weight rows x one K split (or, for the leading su blocks, the x . A^T part of one split).
 // MR = 16, 32 or 64 bounds M.  Up to 32 rows the split's whole x slice is staged in LDS once; at MR = 64 weight
 // blocks take x one 128-element chunk at a time (all 64 rows, two LDS buffers), so that a weight chunk is decoded
