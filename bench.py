@@ -658,7 +658,7 @@ def routed_decode_table(dev, sets: int = 16, replays: int = 5, fmt: str = "block
     m = m.to(dev)
     pool = torch.cuda.graph_pool_handle()
     rows = []
-    for T in (1, 4, 16, 64):
+    for T in (1, 4, 8, 16, 64):
         calls = []
         for i in range(sets):
             rw, sel = zipf_routing(max(T, 8), E, topk, seed=3 + i, device=dev)

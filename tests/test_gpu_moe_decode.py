@@ -55,6 +55,7 @@ def _both_paths(m, x, rw, sel, device):
     (8, 1, 256, 512, 16, 2, False, torch.bfloat16),        # one token: one row per expert, the one-row form
     (16, 1, 1024, 768, 16, 8, False, torch.float32),       # 8 experts of 16, K slices of one chunk
     (16, 3, 512, 256, 8, 4, True, torch.bfloat16),         # shared A / B factors where the module shares them
+    (16, 9, 512, 256, 8, 4, True, torch.float32),          # the fewest tokens that are grouped four rows to a unit
     (16, 16, 1024, 768, 16, 8, False, torch.bfloat16),     # four-row form, experts of several units, K slices of two chunks
     (6, 64, 256, 256, 24, 2, True, torch.float32),         # r not a multiple of 16; up to dozens of rows per expert
     (40, 64, 512, 512, 64, 8, False, torch.bfloat16),      # 512 routed copies (the most), r = 64
