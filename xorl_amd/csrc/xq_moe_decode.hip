@@ -30,9 +30,9 @@ constexpr int kDecMaxChunks = 16;       // chunks per K slice at most (the slice
 inline int64_t al256(int64_t b) { return (b + 255) & ~(int64_t)255; }
 inline int r_pad_of(int r) { return ((r + 15) / 16) * 16; }
 
-// routing lists in device memory: head[0] units, head[1] rows; a unit is up to MR consecutive rows of one expert
-// (units in ascending expert order): unit[4 u] = {expert, first row, row count, 0} and unit_token[4 u + m] the token of
-// its row m; per row row_info[2 row] = {the routed copy it is (token * topk + slot) or -1 past the last row, its expert}; per copy
+// routing lists in device memory: a unit is up to MR consecutive rows of one expert (units in ascending expert order):
+// unit[4 u] = {expert, first row, row count, 0} (all zero past the last unit) and unit_token[4 u + m] the token of its
+// row m; per row row_info[2 row] = {the routed copy it is (token * topk + slot) or -1 past the last row, its expert}; per copy
 // pair_info[2 copy] = {its row or -1, its expert}.  What a block needs first sits behind one index, so that its loads
 // go out together instead of one after the other's result.
 // With one row per unit (direct: calls of up to eight tokens) there is nothing to sort: a unit is a routed copy, its row the
@@ -42,7 +42,6 @@ struct DecLists {
     int32_t R;
     const int32_t* selected;      // direct: [R] expert ids (NULL otherwise)
     int32_t E, topk;
-    __host__ __device__ int32_t* head() const { return base; }
     __host__ __device__ int32_t* unit() const { return base + 4; }
     __host__ __device__ int32_t* unit_token() const { return base + 4 + 4 * R; }
     __host__ __device__ int32_t* row_info() const { return base + 4 + 8 * R; }
@@ -593,8 +592,8 @@ struct DecPlan {
     int ns_gu, cps_gu, ns_d, cps_d, units;
 };
 
-// K slices: enough blocks to fill the chip when few experts are touched (the grid is laid out for min(R, E) experts;
-// blocks of experts that are not touched leave at once), slices of at most kDecMaxChunks chunks
+// K slices: enough blocks to fill the chip when few experts are touched (the grid is laid out for the most units that the
+// call can have; blocks of units that do not exist leave at once), slices of at most kDecMaxChunks chunks
 void slices_for(int chunks, int blocks_per_slice, int* ns, int* cps) {
     int want = (int)xq_cdiv(1024, blocks_per_slice);
     const int least = (int)xq_cdiv(chunks, kDecMaxChunks);
