@@ -10,7 +10,7 @@
 // token's top-k copies.  Five launches (four for up to eight tokens, which need no routing launch), all sums in a fixed order (deterministic), nothing zeroed, no atomics on
 // memory.
 //
-//   decode_route_kernel   : the touched experts' rows in units of 4 (stable order of the routed copies) -- one block
+//   decode_route_kernel   : the touched experts' rows in units of 4 -- one block
 //   decode_stream_kernel  : gate | up partial sums [bank][K slice][row][I] + x . A partial sums (blocks of their own)
 //   decode_mid_kernel     : h = bf16(bf16(bf16(silu(g)) u) w), g / u = bf16(sum of slices + su . B), su = bf16(s x . A)
 //   decode_stream_kernel  : down partial sums [K slice][row][H] + h . A_d partial sums
@@ -51,7 +51,7 @@ struct DecLists {
 
 __global__ void __launch_bounds__(512) decode_route_kernel(const int32_t* selected, int R, int E, int lg, int topk, int units_max, DecLists L) {
     const int MR = 1 << lg;                          // rows per unit
-    __shared__ __attribute__((aligned(16))) int32_t s_sel[kDecMaxPairs];
+    __shared__ int32_t s_tot[2];
     __shared__ __attribute__((aligned(16))) int32_t s_cnt[kDecMaxExperts], s_begin[kDecMaxExperts], s_unit[kDecMaxExperts];
     const int t = threadIdx.x;
     for (int e = t; e < kDecMaxExperts; e += 512) s_cnt[e] = 0;
@@ -60,18 +60,12 @@ __global__ void __launch_bounds__(512) decode_route_kernel(const int32_t* select
         const int v = selected[t];
         mine = v >= 0 && v < E ? v : -1;             // ids outside [0, E) drop their copy
     }
-    s_sel[t] = mine;
     __syncthreads();
-    int rank = 0;                                    // earlier copies of the same expert: the stable order
-    if (mine >= 0) {
-        int p = 0;
-        for (; p + 4 <= t; p += 4) {                 // four at a time: one LDS read
-            const int4 v = *(const int4*)&s_sel[p];
-            rank += (v.x == mine ? 1 : 0) + (v.y == mine ? 1 : 0) + (v.z == mine ? 1 : 0) + (v.w == mine ? 1 : 0);
-        }
-        for (; p < t; ++p) rank += s_sel[p] == mine ? 1 : 0;
-        atomicAdd(&s_cnt[mine], 1);
-    }
+    // a copy's place among its expert's rows: whichever the counter hands out.  The places differ from run to run, the
+    // result does not: a row's arithmetic depends neither on its place in a unit nor on the unit's other rows, and a
+    // token's copies are summed in slot order.
+    int rank = 0;
+    if (mine >= 0) rank = atomicAdd(&s_cnt[mine], 1);
     __syncthreads();
     for (int e = t; e < E; e += 512) {
         int b = 0, idx = 0, e2 = 0;
@@ -96,14 +90,14 @@ __global__ void __launch_bounds__(512) decode_route_kernel(const int32_t* select
             u[3] = 0;
         }
         if (e == E - 1) {
-            s_sel[0] = idx + ((c + MR - 1) >> lg);   // units, rows (s_sel has been read: the barrier above)
-            s_sel[1] = b + c;
+            s_tot[0] = idx + ((c + MR - 1) >> lg);   // units, rows
+            s_tot[1] = b + c;
         }
     }
     __syncthreads();
     // the grid is laid out for units_max units and R rows: the others say so themselves (no rows / no copy)
-    for (int u = s_sel[0] + t; u < units_max; u += 512) *(int4*)(L.unit() + 4 * u) = int4{0, 0, 0, 0};
-    for (int rr = s_sel[1] + t; rr < R; rr += 512) L.row_info()[2 * rr] = -1;
+    for (int u = s_tot[0] + t; u < units_max; u += 512) *(int4*)(L.unit() + 4 * u) = int4{0, 0, 0, 0};
+    for (int rr = s_tot[1] + t; rr < R; rr += 512) L.row_info()[2 * rr] = -1;
 
     if (t < R) {
         if (mine >= 0) {
