@@ -230,7 +230,9 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MR == 
     const int n0 = tile * kDecTile;
     const uint8_t* wbase = P4 ? g.packed[bank] + ((int64_t)e * (g.K >> 1) + ((k0 + wave * 32) >> 1)) * g.N + n0
                               : g.packed[bank] + ((int64_t)e * g.K + k0 + wave * 32) * g.N + n0;
-    const uint32_t woff = (uint32_t)((P4 ? kq : 2 * kq) * g.N + c * 16);
+    // MR = 1: a lane owns row pairs (dot products); MR = 4: four consecutive rows (the contraction depth of the 4x4x4 MFMA)
+    constexpr bool MF = MR == 4;
+    const uint32_t woff = (uint32_t)((MF ? (P4 ? 2 * kq : 4 * kq) : (P4 ? kq : 2 * kq)) * g.N + c * 16);
     // block fp8: the lane's block scale of a chunk; nvfp4: the 16 columns' e4m3 scales of the wave's two 16-row groups
     // nf4: the 16 columns' fp32 scales of the wave's 64-row group
     const uint8_t* sbase = NV ? (const uint8_t*)g.scales[bank] + ((int64_t)e * (g.K >> 4) + c_begin * 8 + wave * 2) * g.N + n0
@@ -250,21 +252,28 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MR == 
 #pragma unroll
             for (int q = 0; q < 4; ++q) w[4 + q] = *(const u32x4*)(sp + 16 * q);
 #pragma unroll
-            for (int st = 0; st < 4; ++st) w[st] = __builtin_nontemporal_load((const u32x4*)(p + (int64_t)(4 * st) * g.N + woff));
+            for (int st = 0; st < 4; ++st)
+                w[st] = __builtin_nontemporal_load((const u32x4*)(p + (int64_t)(MF ? 8 * (st >> 1) + (st & 1) : 4 * st) * g.N + woff));
         } else if (NV) {
             const uint8_t* p = wbase + (int64_t)ch * (kDecChunk / 2) * g.N;
             const uint8_t* sp = sbase + (int64_t)ch * 8 * g.N;
             w[4] = *(const u32x4*)(sp + soff);
             w[5] = *(const u32x4*)(sp + g.N + soff);
 #pragma unroll
-            for (int st = 0; st < 4; ++st) w[st] = __builtin_nontemporal_load((const u32x4*)(p + (int64_t)(4 * st) * g.N + woff));
+            for (int st = 0; st < 4; ++st)
+                w[st] = __builtin_nontemporal_load((const u32x4*)(p + (int64_t)(MF ? 8 * (st >> 1) + (st & 1) : 4 * st) * g.N + woff));
         } else {
             const uint8_t* p = wbase + (int64_t)ch * kDecChunk * g.N;
             sc = *(const float*)(sbase + (int64_t)ch * g.sn * 4 + soff);
+            if (MF) {
 #pragma unroll
-            for (int st = 0; st < 4; ++st) {
-                w[2 * st] = __builtin_nontemporal_load((const u32x4*)(p + (int64_t)(8 * st) * g.N + woff));
-                w[2 * st + 1] = __builtin_nontemporal_load((const u32x4*)(p + (int64_t)(8 * st + 1) * g.N + woff));
+                for (int i = 0; i < 8; ++i) w[i] = __builtin_nontemporal_load((const u32x4*)(p + (int64_t)(16 * (i >> 2) + (i & 3)) * g.N + woff));
+            } else {
+#pragma unroll
+                for (int st = 0; st < 4; ++st) {
+                    w[2 * st] = __builtin_nontemporal_load((const u32x4*)(p + (int64_t)(8 * st) * g.N + woff));
+                    w[2 * st + 1] = __builtin_nontemporal_load((const u32x4*)(p + (int64_t)(8 * st + 1) * g.N + woff));
+                }
             }
         }
     };
@@ -328,7 +337,69 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MR == 
     for (int m = 0; m < MR; ++m)
 #pragma unroll
         for (int j = 0; j < 16; ++j) acc[m][j] = 0.0f;
+    // MR = 4: the unit's four x rows times four consecutive weight rows of a column are one block of v_mfma_f32_4x4x4_16b_bf16
+    // (16 blocks of 4 lanes: lane j of a block gives 4 k of its column as B and 4 k of x row j as A, and receives the
+    // block's four rows of its column).  A lane's 16 columns take 16 such instructions per 4 weight rows, where dot products
+    // would take 128 vector instructions -- and they run beside the decode, on the matrix pipe.
+    typedef short s16x4 __attribute__((ext_vector_type(4)));
+    f32x4 accq[MF ? 16 : 1];
+    if (MF) {
+#pragma unroll
+        for (int j = 0; j < 16; ++j) accq[j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+    auto work4 = [&](const u32x4(&w)[8], float sc, int ch) {
+        const bf16_t* xa = &xs[c & 3][ch * kDecChunk + wave * 32 + 4 * kq];
+#pragma unroll
+        for (int qs = 0; qs < 2; ++qs) {                             // rows 16 qs + 4 kq .. + 3 of the wave's 32
+            const s16x4 av = __builtin_bit_cast(s16x4, *(const u32x2*)(xa + 16 * qs));
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {                            // columns 4 q .. 4 q + 3 of the lane's 16
+                float v[4][4];                                       // [row][column]
+                if (NF) {
+                    const float* tab = nf4_tab[wave];
+#pragma unroll
+                    for (int h = 0; h < 2; ++h)
+#pragma unroll
+                        for (int b = 0; b < 4; ++b) {
+                            const uint32_t byte = (w[2 * qs + h][q] >> (8 * b)) & 0xffu;
+                            const float sv = __uint_as_float(w[4 + q][b]);
+                            v[2 * h][b] = tab[byte & 15u] * sv;
+                            v[2 * h + 1][b] = tab[byte >> 4] * sv;
+                        }
+                } else if (NV) {
+                    const f32x2 s01 = e4m3x2_to_f32(w[4 + qs][q], false), s23 = e4m3x2_to_f32(w[4 + qs][q], true);
+                    const float sv[4] = {s01[0] * gsc, s01[1] * gsc, s23[0] * gsc, s23[1] * gsc};
+#pragma unroll
+                    for (int h = 0; h < 2; ++h) {
+                        const f32x2 v0 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w[2 * qs + h][q], 1.0f, 0);
+                        const f32x2 v1 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w[2 * qs + h][q], 1.0f, 1);
+                        const f32x2 v2 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w[2 * qs + h][q], 1.0f, 2);
+                        const f32x2 v3 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w[2 * qs + h][q], 1.0f, 3);
+                        v[2 * h][0] = v0[0] * sv[0]; v[2 * h + 1][0] = v0[1] * sv[0];
+                        v[2 * h][1] = v1[0] * sv[1]; v[2 * h + 1][1] = v1[1] * sv[1];
+                        v[2 * h][2] = v2[0] * sv[2]; v[2 * h + 1][2] = v2[1] * sv[2];
+                        v[2 * h][3] = v3[0] * sv[3]; v[2 * h + 1][3] = v3[1] * sv[3];
+                    }
+                } else {
+#pragma unroll
+                    for (int rr = 0; rr < 4; ++rr) {
+                        const f32x2 a01 = e4m3x2_to_f32(w[4 * qs + rr][q], false), a23 = e4m3x2_to_f32(w[4 * qs + rr][q], true);
+                        v[rr][0] = a01[0] * sc; v[rr][1] = a01[1] * sc; v[rr][2] = a23[0] * sc; v[rr][3] = a23[1] * sc;
+                    }
+                }
+#pragma unroll
+                for (int b = 0; b < 4; ++b) {
+                    const u32x2 bw = {pack_bf16x2(v[0][b], v[1][b]), pack_bf16x2(v[2][b], v[3][b])};
+                    accq[4 * q + b] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(av, __builtin_bit_cast(s16x4, bw), accq[4 * q + b], 0, 0, 0);
+                }
+            }
+        }
+    };
     auto work = [&](const u32x4(&w)[8], float sc, int ch) {
+        if constexpr (MF) {
+            work4(w, sc, ch);
+            return;
+        }
         const uint32_t* xw = (const uint32_t*)&xs[0][0] + ((ch * kDecChunk + wave * 32 + 2 * kq) >> 1);
         float scl[16];                                               // nvfp4: the 16 columns' scales of the current 16-row group
 #pragma unroll
@@ -410,6 +481,12 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MR == 
         work(wa, sa, ch);
     }
 
+    if (MF) {
+#pragma unroll
+        for (int m = 0; m < MR; ++m)
+#pragma unroll
+            for (int j = 0; j < 16; ++j) acc[m][j] = accq[j][m];
+    }
     // the 16 partial sums of a column (4 waves x 4 row groups of a lane's 16) meet in LDS, one x row at a time
 #pragma unroll
     for (int m = 0; m < MR; ++m) {
