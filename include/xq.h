@@ -512,7 +512,7 @@ int xq_grouped_bwd(const xq_weight* gate, const xq_weight* up, const xq_weight* 
  * GEMMs).  Same arguments as xq_grouped_fwd without `saved`, same result up to the summation order inside a dot
  * product (same rounding points: bf16 gate / up / h / down rows, bf16 low-rank intermediates and factors).  With few
  * tokens an expert sees one or two rows and the time is the bytes of the touched experts: each touched expert's three
- * matrices are streamed once, multiplied on the vector unit, in five launches on `stream` (four for up to eight tokens).
+ * matrices are streamed once, multiplied on the vector unit, in five launches on `stream` (four for up to four tokens).
  * xq_grouped_infer_supported() says whether a call fits: three banks of one format, block fp8 (fp32 scales), nvfp4
  * (GKN, e4m3 block scales, group 16) or nf4 (GKN, fp32 scales, group 64), that make an MLP, hidden and intermediate sizes multiples of 256, at most 1024 experts, 1..512 routed copies (n_tokens * topk), topk <= 16,
  * r in 1..64.  Other calls return XQ_ERR_ARG here: the caller takes xq_grouped_fwd for them.

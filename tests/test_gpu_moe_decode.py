@@ -55,13 +55,13 @@ def _both_paths(m, x, rw, sel, device):
     (8, 1, 256, 512, 16, 2, False, torch.bfloat16),        # one token: one row per expert, the one-row form
     (16, 1, 1024, 768, 16, 8, False, torch.float32),       # 8 experts of 16, K slices of one chunk
     (16, 3, 512, 256, 8, 4, True, torch.bfloat16),         # shared A / B factors where the module shares them
-    (16, 9, 512, 256, 8, 4, True, torch.float32),          # the fewest tokens that are grouped four rows to a unit
+    (16, 5, 512, 256, 8, 4, True, torch.float32),          # the fewest tokens that are grouped four rows to a unit
     (16, 16, 1024, 768, 16, 8, False, torch.bfloat16),     # four-row form, experts of several units, K slices of two chunks
     (6, 64, 256, 256, 24, 2, True, torch.float32),         # r not a multiple of 16; up to dozens of rows per expert
     (40, 64, 512, 512, 64, 8, False, torch.bfloat16),      # 512 routed copies (the most), r = 64
     (8, 1, 4096, 256, 16, 2, False, torch.float32),        # one-row form, K slices of two chunks
     (40, 64, 2048, 256, 16, 8, False, torch.float32),      # four-row form, K slices of four chunks (the streaming loop proper)
-    (12, 4, 2048, 768, 16, 8, False, torch.bfloat16),      # one-row form on four tokens, K slices of three chunks and a last one of one
+    (12, 4, 2048, 768, 16, 8, False, torch.bfloat16),      # one-row form on four tokens (the most it takes), K slices of three chunks and a last one of one
 ])
 def test_decode_forward_vs_oracle(hip_device, fmt, E, T, H, I, r, topk, hybrid, rw_dtype):
     m, banks = _make_experts(fmt, E, H, I, r, hybrid, seed=3 * E + T, device=hip_device)

@@ -3,12 +3,13 @@
 // _MoeExpertsLoRAFunction (ops/moe/lora.py:525-713) with the rounding points of xq_grouped_fwd; what differs is the
 // organisation.  With few tokens an expert sees one or two rows, so the time is the touched experts' bytes: every
 // touched expert's three matrices are streamed once from HBM by blocks that each own 256 output columns and a range
-// of the contraction dimension, multiply on the vector unit (v_dot2c_f32_bf16 on bf16 pairs: a bank matrix is
-// [K, N] with N contiguous, so a lane keeps 16 output columns and walks down K -- no transposition, no matrix cores,
-// which a one-row operand would leave idle) and store fp32 partial sums; two small kernels between and after the
-// two streaming launches add the partial sums and the low-rank terms, apply SwiGLU and the routing weight and sum a
-// token's top-k copies.  Five launches (four for up to eight tokens, which need no routing launch), all sums in a fixed order (deterministic), nothing zeroed, no atomics on
-// memory.
+// of the contraction dimension and store fp32 partial sums.  A bank matrix is [K, N] with N contiguous, so a lane keeps
+// 16 output columns and walks down K -- no transposition.  One row of a unit is multiplied on the vector unit
+// (v_dot2c_f32_bf16 on bf16 pairs of two weight rows: a one-row operand would leave the matrix cores idle), four rows
+// by v_mfma_f32_4x4x4_16b_bf16 (four weight rows of a column against the unit's four x rows).  Two small kernels
+// between and after the two streaming launches add the partial sums and the low-rank terms, apply SwiGLU and the routing
+// weight and sum a token's top-k copies.  Five launches (four for up to four tokens, which need no routing launch), all
+// sums in a fixed order (deterministic), nothing zeroed, no atomics on memory.
 //
 //   decode_route_kernel   : the touched experts' rows in units of 4 -- one block
 //   decode_stream_kernel  : gate | up partial sums [bank][K slice][row][I] + x . A partial sums (blocks of their own)
@@ -35,7 +36,7 @@ inline int r_pad_of(int r) { return ((r + 15) / 16) * 16; }
 // row m; per row row_info[2 row] = {the routed copy it is (token * topk + slot) or -1 past the last row, its expert}; per copy
 // pair_info[2 copy] = {its row or -1, its expert}.  What a block needs first sits behind one index, so that its loads
 // go out together instead of one after the other's result.
-// With one row per unit (direct: calls of up to eight tokens) there is nothing to sort: a unit is a routed copy, its row the
+// With one row per unit (direct: calls of up to four tokens) there is nothing to sort: a unit is a routed copy, its row the
 // copy's number, and the kernels read the expert ids where the caller has them -- no routing launch.
 struct DecLists {
     int32_t* base;
@@ -684,9 +685,10 @@ DecPlan plan_for(int64_t R, int E, int64_t H, int64_t I, int MR) {
     return p;
 }
 
-// up to eight tokens run one row per unit with no routing launch (measured on 128 experts, top-8: 50.0 us against 53.8 at
-// four tokens, 69.1 against 76.9 at eight; at sixteen 113 against 100); more tokens are grouped four rows to a unit
-inline int rows_per_unit(int64_t n_tokens) { return n_tokens <= 8 ? 1 : 4; }
+// up to four tokens run one row per unit with no routing launch (measured on 128 experts, top-8, block fp8 / nvfp4: 50.6 /
+// 46.1 us against 54.8 / 48.8 at four tokens; at eight 68.4 / 62.1 against 66.7 / 58.0); more tokens are grouped four
+// rows to a unit
+inline int rows_per_unit(int64_t n_tokens) { return n_tokens <= 4 ? 1 : 4; }
 
 int64_t infer_workspace(int64_t R, int E, int64_t H, int64_t I, int rp, int MR) {
     const DecPlan p = plan_for(R, E, H, I, MR);
